@@ -1,0 +1,175 @@
+"""ctypes binding of the CPU oracle (``libpmetal_oracle.so``).
+
+Test infrastructure only: the test-suite, the smoke check and the benchmark's
+CPU-baseline leg import this; the product package never does.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libpmetal_oracle.so")
+
+TYPE_F32, TYPE_F16, TYPE_Q8_0, TYPE_Q4K, TYPE_Q6K = 0, 1, 8, 12, 14
+ORDER_REF, ORDER_GGML = 0, 1
+OK, ERR_UNSUPPORTED_TYPE, ERR_INVALID_SIZE, ERR_INVALID_SHAPE, ERR_SHAPE_TOO_LARGE = 0, 2, 3, 6, 7
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with gcc (a no-op when the library is newer than its sources)."""
+    srcs = [os.path.join(HERE, f) for f in ("pmetal_oracle.c", "pmetal_oracle.h", "Makefile")]
+    stale = force or not os.path.exists(LIB_PATH) or any(
+        os.path.getmtime(s) > os.path.getmtime(LIB_PATH) for s in srcs
+    )
+    if stale:
+        subprocess.run(["make", "-C", HERE, "-B", "libpmetal_oracle.so"], check=True, capture_output=True)
+    return LIB_PATH
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            build()
+        L = C.CDLL(LIB_PATH)
+        f32p, u8p, i8p, i32p = (C.POINTER(C.c_float), C.POINTER(C.c_uint8), C.POINTER(C.c_int8),
+                                C.POINTER(C.c_int32))
+        L.pmo_f32_to_f16.argtypes, L.pmo_f32_to_f16.restype = [C.c_float], C.c_uint16
+        L.pmo_f16_to_f32.argtypes, L.pmo_f16_to_f32.restype = [C.c_uint16], C.c_float
+        L.pmo_f32_to_bf16.argtypes, L.pmo_f32_to_bf16.restype = [C.c_float], C.c_uint16
+        L.pmo_bf16_to_f32.argtypes, L.pmo_bf16_to_f32.restype = [C.c_uint16], C.c_float
+        L.pmo_nearest_int.argtypes, L.pmo_nearest_int.restype = [C.c_float], C.c_int32
+        L.pmo_make_qkx1_quants.argtypes = [C.c_int32, C.c_int32, f32p, C.c_int32, f32p, f32p]
+        L.pmo_make_qkx1_quants.restype = None
+        L.pmo_make_qx_quants.argtypes = [C.c_int32, C.c_int32, f32p, C.c_int32, i8p]
+        L.pmo_make_qx_quants.restype = C.c_float
+        L.pmo_get_scale_min_k4.argtypes = [C.c_int32, u8p, u8p, u8p]
+        L.pmo_get_scale_min_k4.restype = None
+        for name in ("pmo_type_size", "pmo_block_size"):
+            getattr(L, name).argtypes, getattr(L, name).restype = [C.c_uint32], C.c_size_t
+        L.pmo_tensor_size.argtypes, L.pmo_tensor_size.restype = [C.c_uint32, C.c_size_t], C.c_size_t
+        for name in ("pmo_quantize_q8_0", "pmo_quantize_q4k", "pmo_quantize_q6k"):
+            getattr(L, name).argtypes, getattr(L, name).restype = [f32p, C.c_size_t, u8p], None
+        L.pmo_dequantize_q8_0.argtypes, L.pmo_dequantize_q8_0.restype = [u8p, C.c_size_t, f32p], None
+        L.pmo_dequantize_q6k.argtypes, L.pmo_dequantize_q6k.restype = [u8p, C.c_size_t, f32p], None
+        L.pmo_dequantize_q4k.argtypes = [u8p, C.c_size_t, f32p, C.c_uint32]
+        L.pmo_dequantize_q4k.restype = None
+        L.pmo_quantize.argtypes = [C.c_uint32, f32p, C.c_size_t, u8p, C.c_size_t]
+        L.pmo_quantize.restype = C.c_int32
+        L.pmo_dequantize.argtypes = [C.c_uint32, u8p, C.c_size_t, i32p, C.c_size_t, f32p, C.c_size_t,
+                                     C.c_uint32]
+        L.pmo_dequantize.restype = C.c_int32
+        L.pmo_use_more_bits.argtypes, L.pmo_use_more_bits.restype = [C.c_size_t, C.c_size_t], C.c_int32
+        L.pmo_is_quantizable_gguf_tensor.argtypes = [C.c_char_p, C.c_size_t]
+        L.pmo_is_quantizable_gguf_tensor.restype = C.c_int32
+        L.pmo_q4km_tensor_type.argtypes = [C.c_char_p, C.c_size_t, C.c_size_t]
+        L.pmo_q4km_tensor_type.restype = C.c_uint32
+        for name in ("pmo_qmatvec_f64", "pmo_qmatvec_f32"):
+            getattr(L, name).argtypes = [C.c_uint32, u8p, C.c_size_t, C.c_size_t, f32p, f32p, C.c_uint32]
+            getattr(L, name).restype = C.c_int32
+        L.pmo_qmatmul_f64.argtypes = [C.c_uint32, u8p, C.c_size_t, C.c_size_t, f32p, C.c_size_t, f32p,
+                                      C.c_uint32]
+        L.pmo_qmatmul_f64.restype = C.c_int32
+        _lib = L
+    return _lib
+
+
+def _f32p(a):
+    return a.ctypes.data_as(C.POINTER(C.c_float))
+
+
+def _u8p(a):
+    return a.ctypes.data_as(C.POINTER(C.c_uint8))
+
+
+def tensor_size(t: int, n: int) -> int:
+    return lib().pmo_tensor_size(t, n)
+
+
+def quantize(t: int, x: np.ndarray) -> np.ndarray:
+    """quantize.rs:17 ``quantize(data, dtype)``: flat f32 -> block bytes."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+    out = np.zeros(tensor_size(t, x.size), dtype=np.uint8)
+    rc = lib().pmo_quantize(t, _f32p(x), x.size, _u8p(out), out.size)
+    if rc != OK:
+        raise ValueError(f"oracle quantize failed with code {rc}")
+    return out
+
+
+def dequantize(t: int, data: np.ndarray, shape, order: int = ORDER_REF) -> np.ndarray:
+    """dequant.rs:92 ``dequantize(data, dtype, shape)``; raises ValueError(code) like DequantError."""
+    data = np.ascontiguousarray(data, dtype=np.uint8).reshape(-1)
+    shp = np.asarray(list(shape), dtype=np.int32)
+    n = 1
+    for d in shape:
+        n *= max(int(d), 0)
+    # an absurd shape is rejected by the validation before dst is touched; do not try to allocate it
+    out = np.empty(n if n < (1 << 40) else 0, dtype=np.float32)
+    rc = lib().pmo_dequantize(t, _u8p(data), data.size, shp.ctypes.data_as(C.POINTER(C.c_int32)), shp.size,
+                              _f32p(out), out.size, order)
+    if rc != OK:
+        raise ValueError(rc)
+    return out
+
+
+def make_qkx1_quants(nmax: int, ntry: int, x: np.ndarray):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    s, m = C.c_float(), C.c_float()
+    lib().pmo_make_qkx1_quants(nmax, ntry, _f32p(x), x.size, C.byref(s), C.byref(m))
+    return np.float32(s.value), np.float32(m.value)
+
+
+def make_qx_quants(n: int, nmax: int, x: np.ndarray, rmse_type: int):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    ls = np.zeros(n, dtype=np.int8)
+    s = lib().pmo_make_qx_quants(n, nmax, _f32p(x), rmse_type, ls.ctypes.data_as(C.POINTER(C.c_int8)))
+    return np.float32(s), ls
+
+
+def get_scale_min_k4(j: int, q: np.ndarray):
+    q = np.ascontiguousarray(q, dtype=np.uint8)
+    sc, m = C.c_uint8(), C.c_uint8()
+    lib().pmo_get_scale_min_k4(j, _u8p(q), C.byref(sc), C.byref(m))
+    return sc.value, m.value
+
+
+def qmatvec(t: int, w: np.ndarray, n_rows: int, k: int, x: np.ndarray, order: int = ORDER_REF,
+            acc: str = "f64") -> np.ndarray:
+    w = np.ascontiguousarray(w, dtype=np.uint8).reshape(-1)
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    assert w.size == n_rows * tensor_size(t, k) and x.size == k
+    y = np.empty(n_rows, dtype=np.float32)
+    fn = lib().pmo_qmatvec_f64 if acc == "f64" else lib().pmo_qmatvec_f32
+    rc = fn(t, _u8p(w), n_rows, k, _f32p(x), _f32p(y), order)
+    if rc != OK:
+        raise ValueError(rc)
+    return y
+
+
+def qmatmul(t: int, w: np.ndarray, n_rows: int, k: int, x: np.ndarray, order: int = ORDER_REF) -> np.ndarray:
+    w = np.ascontiguousarray(w, dtype=np.uint8).reshape(-1)
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, k)
+    y = np.empty((x.shape[0], n_rows), dtype=np.float32)
+    rc = lib().pmo_qmatmul_f64(t, _u8p(w), n_rows, k, _f32p(x), x.shape[0], _f32p(y), order)
+    if rc != OK:
+        raise ValueError(rc)
+    return y
+
+
+def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    """half::bf16::from_f32 (RNE) on an array, vectorised; returns uint16 bit patterns."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    rounded = ((u.astype(np.uint64) + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    return np.where(nan, ((u >> 16) | 0x40).astype(np.uint16), rounded)
+
+
+def bf16_bits_to_f32(h: np.ndarray) -> np.ndarray:
+    return (np.ascontiguousarray(h, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)

@@ -1,0 +1,743 @@
+/*
+ * pmetal_oracle.c -- CPU restatement of PMetal's GGUF block-quantized weight
+ * path (Q8_0, Q4_K, Q6_K).  TEST INFRASTRUCTURE ONLY: see pmetal_oracle.h.
+ *
+ * Build: gcc -O2 -ffp-contract=off -fno-fast-math (see Makefile).  Every float
+ * operation below is a single IEEE binary32 operation in the order the
+ * reference performs it; Rust never contracts a*b+c into an fma, so neither
+ * may the compiler here.
+ *
+ * Parity status per function (what pins it without running the Rust):
+ *   f16/bf16 conversion ... numpy float16 (all 65536 f16 values, sampled and
+ *                           boundary f32 values); IEEE definition.
+ *   nearest_int ........... reference KATs quantize.rs:862-868.
+ *   get_scale_min_k4 ...... reference KATs quantize.rs:1035-1047,
+ *                           k_quants.rs:1386-1396; pack/unpack identity.
+ *   make_qkx1_quants ...... closed forms (reference tests quantize.rs:998-1017)
+ *                           + independent numpy-float32 twin. Restatement-pinned.
+ *   make_qx_quants ........ closed forms + invariants + numpy twin.
+ *                           Restatement-pinned.
+ *   quantize_q8_0 ......... fully determined by IEEE ops: numpy twin is exact.
+ *   quantize_q4k/q6k ...... block sizes, reference round-trip bounds
+ *                           (k_quants.rs:1446-1509), invariants, numpy twin.
+ *                           Restatement-pinned (bytes never compared with Rust).
+ *   dequantize_* .......... reference KATs (dequant.rs:1016-1036,
+ *                           k_quants.rs:1368-1383) + hand-built blocks + numpy.
+ *   recipe ................ reference KATs commands/quantize.rs:1561-1608.
+ */
+#include "pmetal_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define QK_K 256
+#define K_SCALE_SIZE 12
+
+/* ------------------------------------------------------------------------- */
+/* half 2.7.1: f16::from_f32 / to_f32, bf16::from_f32 / to_f32               */
+/* (call sites k_quants.rs:928-929, :1097, :359-360, :475; quantize.rs:285;  */
+/*  dequant.rs:482).  IEEE round-to-nearest-even, subnormals kept,           */
+/*  overflow -> inf, NaN kept as a quiet NaN.                                */
+/* ------------------------------------------------------------------------- */
+
+static uint32_t f32_bits(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    return u;
+}
+
+static float bits_f32(uint32_t u) {
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+uint16_t pmo_f32_to_f16(float f) {
+    uint32_t x = f32_bits(f);
+    uint32_t sign = (x >> 16) & 0x8000u;
+    uint32_t exp = (x >> 23) & 0xFFu;
+    uint32_t man = x & 0x007FFFFFu;
+    if (exp == 0xFFu) {
+        uint32_t nan_bit = man ? 0x0200u : 0u;
+        return (uint16_t)(sign | 0x7C00u | nan_bit | (man >> 13));
+    }
+    int32_t half_exp = (int32_t)exp - 127 + 15;
+    if (half_exp >= 0x1F) return (uint16_t)(sign | 0x7C00u);
+    if (half_exp <= 0) {
+        if (14 - half_exp > 24) return (uint16_t)sign;
+        uint32_t m = man | 0x00800000u;
+        uint32_t shift = (uint32_t)(14 - half_exp);
+        uint32_t half_man = m >> shift;
+        uint32_t round_bit = 1u << (shift - 1);
+        /* round to nearest, ties to even */
+        if ((m & round_bit) && (m & (3u * round_bit - 1u))) half_man += 1;
+        return (uint16_t)(sign | half_man);
+    }
+    uint32_t out = sign | ((uint32_t)half_exp << 10) | (man >> 13);
+    uint32_t round_bit = 0x00001000u;
+    if ((man & round_bit) && (man & (3u * round_bit - 1u))) out += 1; /* may carry into exp: correct */
+    return (uint16_t)out;
+}
+
+float pmo_f16_to_f32(uint16_t h) {
+    uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+    uint32_t exp = ((uint32_t)h >> 10) & 0x1Fu;
+    uint32_t man = (uint32_t)h & 0x03FFu;
+    if (exp == 0x1Fu) return bits_f32(sign | 0x7F800000u | (man ? (0x00400000u | (man << 13)) : 0u));
+    if (exp == 0) {
+        if (man == 0) return bits_f32(sign);
+        /* subnormal: value = man * 2^-24, exact in f32 */
+        float v = (float)man * 5.9604644775390625e-08f;
+        return sign ? -v : v;
+    }
+    return bits_f32(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
+uint16_t pmo_f32_to_bf16(float f) {
+    uint32_t x = f32_bits(f);
+    if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((x >> 16) | 0x0040u);
+    uint32_t round_bit = 0x00008000u;
+    if ((x & round_bit) && (x & (3u * round_bit - 1u))) return (uint16_t)((x >> 16) + 1u);
+    return (uint16_t)(x >> 16);
+}
+
+float pmo_bf16_to_f32(uint16_t h) { return bits_f32((uint32_t)h << 16); }
+
+/* ------------------------------------------------------------------------- */
+/* Rust core semantics                                                       */
+/* ------------------------------------------------------------------------- */
+
+/* `v as i32` for f32: saturating, NaN -> 0. */
+static int32_t f32_as_i32(float v) {
+    if (v != v) return 0;
+    if (v >= 2147483648.0f) return INT32_MAX;
+    if (v <= -2147483648.0f) return INT32_MIN;
+    return (int32_t)v;
+}
+
+/* f32::total_cmp: -1, 0, +1 */
+static int total_cmp(float a, float b) {
+    int32_t l = (int32_t)f32_bits(a);
+    int32_t r = (int32_t)f32_bits(b);
+    l ^= (int32_t)(((uint32_t)(l >> 31)) >> 1);
+    r ^= (int32_t)(((uint32_t)(r >> 31)) >> 1);
+    return (l > r) - (l < r);
+}
+
+static int32_t clamp_i32(int32_t v, int32_t lo, int32_t hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+/* quantize.rs:566-570: `v.round() as i32` -- half away from zero, saturating. */
+int32_t pmo_nearest_int(float v) { return f32_as_i32(roundf(v)); }
+
+/* ------------------------------------------------------------------------- */
+/* quantize.rs:583-644 make_qkx1_quants                                      */
+/* ------------------------------------------------------------------------- */
+void pmo_make_qkx1_quants(int32_t nmax, int32_t ntry, const float *x, int32_t n, float *scale_out,
+                          float *min_out) {
+    uint8_t l[QK_K];
+    memset(l, 0, sizeof l);
+
+    /* :588-593 min_by/max_by with total_cmp (first minimum, last maximum). */
+    float min = x[0], max = x[0];
+    for (int32_t i = 1; i < n; i++) {
+        if (total_cmp(min, x[i]) > 0) min = x[i];
+        if (total_cmp(max, x[i]) <= 0) max = x[i];
+    }
+    /* :596 */
+    if (max == min) {
+        *scale_out = 0.0f;
+        *min_out = 0.0f;
+        return;
+    }
+    /* :601 */
+    min = fminf(min, 0.0f);
+    /* :604-605 */
+    float iscale = (float)nmax / (max - min);
+    float scale = 1.0f / iscale;
+
+    for (int32_t t = 0; t < ntry; t++) {
+        float sumlx = 0.0f;
+        int32_t suml2 = 0;
+        int did_change = 0;
+        /* :612-621 */
+        for (int32_t i = 0; i < n; i++) {
+            int32_t li = clamp_i32(pmo_nearest_int(iscale * (x[i] - min)), 0, nmax);
+            uint8_t cl = (uint8_t)li;
+            if (cl != l[i]) {
+                l[i] = cl;
+                did_change = 1;
+            }
+            sumlx += (x[i] - min) * (float)li;
+            suml2 += li * li;
+        }
+        /* :622-624 */
+        if (suml2 == 0) break;
+        /* :625 */
+        scale = sumlx / (float)suml2;
+        /* :627-632 Iterator::sum::<f32>: sequential; Rust >= 1.83 (the reference
+         * pins rust-version 1.89) folds from -0.0. */
+        float sum = -0.0f;
+        for (int32_t i = 0; i < n; i++) sum += x[i] - scale * (float)l[i];
+        /* :634-637 */
+        min = sum / (float)n;
+        if (min > 0.0f) min = 0.0f;
+        /* :638-641 */
+        iscale = 1.0f / scale;
+        if (!did_change) break;
+    }
+    *scale_out = scale;
+    *min_out = -min;
+}
+
+/* ------------------------------------------------------------------------- */
+/* quantize.rs:738-841 make_qx_quants                                        */
+/* ------------------------------------------------------------------------- */
+float pmo_make_qx_quants(int32_t n, int32_t nmax, const float *x, int32_t rmse_type, int8_t *ls) {
+    memset(ls, 0, (size_t)n);
+
+    /* :742-750 */
+    float max = 0.0f, amax = 0.0f;
+    for (int32_t i = 0; i < n; i++) {
+        float ax = fabsf(x[i]);
+        if (ax > amax) {
+            amax = ax;
+            max = x[i];
+        }
+    }
+    /* :752-754 */
+    if (amax == 0.0f) return 0.0f;
+    /* :756 */
+    float iscale = -(float)nmax / max;
+
+    /* :758-764 */
+    if (rmse_type == 0) {
+        for (int32_t i = 0; i < n; i++) {
+            int32_t l = pmo_nearest_int(iscale * x[i]);
+            ls[i] = (int8_t)(nmax + clamp_i32(l, -nmax, nmax - 1));
+        }
+        return 1.0f / iscale;
+    }
+
+    int32_t weight_type = rmse_type % 2;
+    float sumlx = 0.0f, suml2 = 0.0f;
+    /* :770-776 */
+    for (int32_t i = 0; i < n; i++) {
+        int32_t l = clamp_i32(pmo_nearest_int(iscale * x[i]), -nmax, nmax - 1);
+        ls[i] = (int8_t)(l + nmax);
+        float w = weight_type == 1 ? x[i] * x[i] : 1.0f;
+        sumlx += w * x[i] * (float)l;
+        suml2 += w * (float)(l * l);
+    }
+    /* :778-779 */
+    float scale = sumlx / suml2;
+    float best = scale * sumlx;
+
+    /* :782-810 */
+    for (int32_t t = 0; t < 3; t++) {
+        float iscale2 = 1.0f / scale;
+        float slx = 0.0f, sl2 = 0.0f;
+        int changed = 0;
+        for (int32_t i = 0; i < n; i++) {
+            int32_t l = clamp_i32(pmo_nearest_int(iscale2 * x[i]), -nmax, nmax - 1);
+            if (l + nmax != (int32_t)ls[i]) changed = 1;
+            float w = weight_type == 1 ? x[i] * x[i] : 1.0f;
+            slx += w * x[i] * (float)l;
+            sl2 += w * (float)(l * l);
+        }
+        if (!changed || sl2 == 0.0f || slx * slx <= best * sl2) break;
+        for (int32_t i = 0; i < n; i++) {
+            int32_t l = pmo_nearest_int(iscale2 * x[i]);
+            ls[i] = (int8_t)(nmax + clamp_i32(l, -nmax, nmax - 1));
+        }
+        sumlx = slx;
+        suml2 = sl2;
+        scale = sumlx / suml2;
+        best = scale * sumlx;
+    }
+
+    /* :813-838 */
+    for (int32_t t = 0; t < 5; t++) {
+        int32_t n_changed = 0;
+        for (int32_t i = 0; i < n; i++) {
+            float w = weight_type == 1 ? x[i] * x[i] : 1.0f;
+            int32_t l = (int32_t)ls[i] - nmax;
+            float slx = sumlx - w * x[i] * (float)l;
+            if (slx > 0.0f) {
+                float sl2 = suml2 - w * (float)(l * l);
+                int32_t new_l = clamp_i32(pmo_nearest_int(x[i] * sl2 / slx), -nmax, nmax - 1);
+                if (new_l != l) {
+                    slx += w * x[i] * (float)new_l;
+                    sl2 += w * (float)(new_l * new_l);
+                    if (sl2 > 0.0f && slx * slx * suml2 > sumlx * sumlx * sl2) {
+                        ls[i] = (int8_t)(nmax + new_l);
+                        sumlx = slx;
+                        suml2 = sl2;
+                        scale = sumlx / suml2;
+                        n_changed += 1;
+                    }
+                }
+            }
+        }
+        if (n_changed == 0) break;
+    }
+    return scale;
+}
+
+/* quantize.rs:844-855 */
+void pmo_get_scale_min_k4(int32_t j, const uint8_t *q, uint8_t *sc, uint8_t *m) {
+    if (j < 4) {
+        *sc = q[j] & 63;
+        *m = q[j + 4] & 63;
+    } else {
+        *sc = (uint8_t)((q[j + 4] & 0xF) | ((q[j - 4] >> 6) << 4));
+        *m = (uint8_t)((q[j + 4] >> 4) | ((q[j] >> 6) << 4));
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* types.rs:102-187                                                          */
+/* ------------------------------------------------------------------------- */
+size_t pmo_type_size(uint32_t t) {
+    switch (t) {
+    case PMO_TYPE_F32: return 4;
+    case PMO_TYPE_F16: return 2;
+    case PMO_TYPE_Q8_0: return 34;
+    case PMO_TYPE_Q4K: return 144;
+    case PMO_TYPE_Q6K: return 210;
+    default: return 0;
+    }
+}
+
+size_t pmo_block_size(uint32_t t) {
+    switch (t) {
+    case PMO_TYPE_F32:
+    case PMO_TYPE_F16: return 1;
+    case PMO_TYPE_Q8_0: return 32;
+    case PMO_TYPE_Q4K:
+    case PMO_TYPE_Q6K: return 256;
+    default: return 0;
+    }
+}
+
+size_t pmo_tensor_size(uint32_t t, size_t n) {
+    size_t bs = pmo_block_size(t);
+    if (bs == 0) return 0;
+    size_t n_blocks = n / bs + (n % bs != 0);
+    return n_blocks * pmo_type_size(t);
+}
+
+/* ------------------------------------------------------------------------- */
+/* quantize.rs:268-300 quantize_q8_0                                         */
+/* ------------------------------------------------------------------------- */
+void pmo_quantize_q8_0(const float *x, size_t n, uint8_t *dst) {
+    size_t n_blocks = n / 32 + (n % 32 != 0);
+    for (size_t b = 0; b < n_blocks; b++) {
+        size_t start = b * 32;
+        size_t end = start + 32 < n ? start + 32 : n;
+        float amax = 0.0f;
+        for (size_t i = start; i < end; i++) amax = fmaxf(amax, fabsf(x[i])); /* acc.max(x.abs()) */
+        float scale = amax / 127.0f;
+        float iscale = amax == 0.0f ? 0.0f : 127.0f / amax;
+        uint16_t d = pmo_f32_to_f16(scale);
+        uint8_t *out = dst + b * 34;
+        out[0] = (uint8_t)(d & 0xFF);
+        out[1] = (uint8_t)(d >> 8);
+        for (size_t i = 0; i < 32; i++) {
+            int8_t v = 0;
+            if (start + i < end) v = (int8_t)clamp_i32(pmo_nearest_int(x[start + i] * iscale), -127, 127);
+            out[2 + i] = (uint8_t)v;
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* k_quants.rs:876-955 quantize_q4k                                          */
+/* ------------------------------------------------------------------------- */
+void pmo_quantize_q4k(const float *xs, size_t n, uint8_t *dst) {
+    size_t n_blocks = n / QK_K + (n % QK_K != 0);
+    memset(dst, 0, n_blocks * 144); /* :878-886; f16::from_f32(0.0) = 0x0000 */
+    for (size_t b = 0; b < n_blocks; b++) {
+        size_t start = b * QK_K;
+        if (start + QK_K > n) continue; /* :890-892 trailing partial block stays zero */
+        const float *x = xs + start;
+        uint8_t *blk = dst + b * 144;
+        uint8_t *bscales = blk + 4;
+        uint8_t *qs = blk + 16;
+
+        float mins[8], scales[8];
+        for (int j = 0; j < 8; j++) pmo_make_qkx1_quants(15, 5, x + 32 * j, 32, &scales[j], &mins[j]);
+
+        /* :904-905 fold(0.0, |max, val| val.max(max)) */
+        float max_scale = 0.0f, max_min = 0.0f;
+        for (int j = 0; j < 8; j++) max_scale = fmaxf(scales[j], max_scale);
+        for (int j = 0; j < 8; j++) max_min = fmaxf(mins[j], max_min);
+
+        float inv_scale = max_scale > 0.0f ? 63.0f / max_scale : 0.0f;
+        float inv_min = max_min > 0.0f ? 63.0f / max_min : 0.0f;
+
+        /* :915-926 */
+        for (int j = 0; j < 8; j++) {
+            int32_t a = pmo_nearest_int(inv_scale * scales[j]);
+            int32_t c = pmo_nearest_int(inv_min * mins[j]);
+            uint8_t ls = (uint8_t)(a < 63 ? a : 63);
+            uint8_t lm = (uint8_t)(c < 63 ? c : 63);
+            if (j < 4) {
+                bscales[j] = ls;
+                bscales[j + 4] = lm;
+            } else {
+                bscales[j + 4] = (uint8_t)((ls & 0xF) | ((lm & 0xF) << 4));
+                bscales[j - 4] |= (uint8_t)((ls >> 4) << 6);
+                bscales[j] |= (uint8_t)((lm >> 4) << 6);
+            }
+        }
+
+        /* :928-929 */
+        uint16_t d16 = pmo_f32_to_f16(max_scale / 63.0f);
+        uint16_t dmin16 = pmo_f32_to_f16(max_min / 63.0f);
+        blk[0] = (uint8_t)(d16 & 0xFF);
+        blk[1] = (uint8_t)(d16 >> 8);
+        blk[2] = (uint8_t)(dmin16 & 0xFF);
+        blk[3] = (uint8_t)(dmin16 >> 8);
+        float df = pmo_f16_to_f32(d16), dminf = pmo_f16_to_f32(dmin16);
+
+        /* :932-943 */
+        uint8_t l[QK_K];
+        memset(l, 0, sizeof l);
+        for (int j = 0; j < 8; j++) {
+            uint8_t sc, m;
+            pmo_get_scale_min_k4(j, bscales, &sc, &m);
+            float d = df * (float)sc;
+            if (d != 0.0f) {
+                float dm = dminf * (float)m;
+                for (int ii = 0; ii < 32; ii++) {
+                    int32_t lv = pmo_nearest_int((x[32 * j + ii] + dm) / d);
+                    l[32 * j + ii] = (uint8_t)clamp_i32(lv, 0, 15);
+                }
+            }
+        }
+        /* :946-951 */
+        for (int j = 0; j < QK_K; j += 64)
+            for (int lv = 0; lv < 32; lv++)
+                qs[(j / 64) * 32 + lv] = (uint8_t)(l[j + lv] | (l[j + lv + 32] << 4));
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* k_quants.rs:1056-1134 quantize_q6k                                        */
+/* ------------------------------------------------------------------------- */
+void pmo_quantize_q6k(const float *xs, size_t n, uint8_t *dst) {
+    size_t n_blocks = n / QK_K + (n % QK_K != 0);
+    memset(dst, 0, n_blocks * 210);
+    for (size_t b = 0; b < n_blocks; b++) {
+        size_t start = b * QK_K;
+        if (start + QK_K > n) continue; /* :1070-1072 */
+        const float *x = xs + start;
+        uint8_t *blk = dst + b * 210;
+        uint8_t *ql = blk, *qh = blk + 128;
+        int8_t *bscales = (int8_t *)(blk + 192);
+
+        int8_t l[QK_K];
+        float scales_f[16];
+        float max_scale = 0.0f, max_abs_scale = 0.0f;
+
+        /* :1082-1094 */
+        for (int ib = 0; ib < 16; ib++) {
+            float scale = pmo_make_qx_quants(16, 32, x + 16 * ib, 1, l + 16 * ib);
+            scales_f[ib] = scale;
+            float abs_scale = fabsf(scale);
+            if (abs_scale > max_abs_scale) {
+                max_abs_scale = abs_scale;
+                max_scale = scale;
+            }
+        }
+        /* :1096-1097 (all-zero block: iscale = -inf, d = f16(-0.0) = 0x8000) */
+        float iscale = -128.0f / max_scale;
+        uint16_t d16 = pmo_f32_to_f16(1.0f / iscale);
+        blk[208] = (uint8_t)(d16 & 0xFF);
+        blk[209] = (uint8_t)(d16 >> 8);
+        float df = pmo_f16_to_f32(d16);
+
+        /* :1100-1102 `.min(127) as i8` (i32 -> i8 wraps) */
+        for (int j = 0; j < 16; j++) {
+            int32_t v = pmo_nearest_int(iscale * scales_f[j]);
+            if (v > 127) v = 127;
+            bscales[j] = (int8_t)(uint8_t)(uint32_t)v;
+        }
+        /* :1105-1113 */
+        for (int j = 0; j < 16; j++) {
+            float d = df * (float)bscales[j];
+            if (d != 0.0f) {
+                for (int ii = 0; ii < 16; ii++) {
+                    int32_t ll = clamp_i32(pmo_nearest_int(x[16 * j + ii] / d), -32, 31);
+                    l[16 * j + ii] = (int8_t)(ll + 32);
+                }
+            }
+        }
+        /* :1116-1130 */
+        for (int j = 0; j < QK_K; j += 128) {
+            for (int li = 0; li < 32; li++) {
+                uint8_t a = (uint8_t)l[j + li], c = (uint8_t)l[j + li + 32];
+                uint8_t e = (uint8_t)l[j + li + 64], g = (uint8_t)l[j + li + 96];
+                ql[j / 2 + li] = (uint8_t)((a & 0xF) | ((e & 0xF) << 4));
+                ql[j / 2 + li + 32] = (uint8_t)((c & 0xF) | ((g & 0xF) << 4));
+                qh[j / 4 + li] = (uint8_t)((a >> 4) | ((c >> 4) << 2) | ((e >> 4) << 4) | ((g >> 4) << 6));
+            }
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* dequant.rs:466-495 dequantize_q8_0 (body)                                 */
+/* ------------------------------------------------------------------------- */
+void pmo_dequantize_q8_0(const uint8_t *src, size_t n, float *dst) {
+    size_t n_blocks = n / 32 + (n % 32 != 0);
+    for (size_t b = 0; b < n_blocks; b++) {
+        const uint8_t *blk = src + b * 34;
+        float scale = pmo_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+        for (size_t i = 0; i < 32 && b * 32 + i < n; i++) dst[b * 32 + i] = (float)(int8_t)blk[2 + i] * scale;
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* k_quants.rs:358-404 dequantize_q4k + :515-560 dequantize_q4k_bytes        */
+/* ------------------------------------------------------------------------- */
+static void dequantize_q4k_block(const uint8_t *blk, float *out, uint32_t order) {
+    float d = pmo_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+    float dmin = pmo_f16_to_f32((uint16_t)(blk[2] | (blk[3] << 8)));
+    const uint8_t *scales = blk + 4;
+    const uint8_t *qs = blk + 16;
+    int idx = 0, is = 0;
+    for (int j = 0; j < QK_K; j += 64) {
+        uint8_t sc1, m1, sc2, m2;
+        pmo_get_scale_min_k4(is, scales, &sc1, &m1);
+        float d1 = d * (float)sc1, dm1 = dmin * (float)m1;
+        pmo_get_scale_min_k4(is + 1, scales, &sc2, &m2);
+        float d2 = d * (float)sc2, dm2 = dmin * (float)m2;
+        const uint8_t *q = qs + j / 2;
+        if (order == PMO_ORDER_REF) {
+            /* :380-400: 16 low, 16 high of bytes 0..15 with (d1, dm1); then bytes 16..31 with (d2, dm2) */
+            for (int l = 0; l < 16; l++) out[idx++] = d1 * (float)(q[l] & 0xF) - dm1;
+            for (int l = 0; l < 16; l++) out[idx++] = d1 * (float)(q[l] >> 4) - dm1;
+            for (int l = 0; l < 16; l++) out[idx++] = d2 * (float)(q[16 + l] & 0xF) - dm2;
+            for (int l = 0; l < 16; l++) out[idx++] = d2 * (float)(q[16 + l] >> 4) - dm2;
+        } else {
+            /* the inverse of the quantizer's packing, k_quants.rs:946-951 */
+            for (int l = 0; l < 32; l++) out[idx++] = d1 * (float)(q[l] & 0xF) - dm1;
+            for (int l = 0; l < 32; l++) out[idx++] = d2 * (float)(q[l] >> 4) - dm2;
+        }
+        is += 2;
+    }
+}
+
+void pmo_dequantize_q4k(const uint8_t *src, size_t n, float *dst, uint32_t order) {
+    size_t n_blocks = n / QK_K + (n % QK_K != 0);
+    float tmp[QK_K];
+    for (size_t b = 0; b < n_blocks; b++) {
+        dequantize_q4k_block(src + b * 144, tmp, order);
+        size_t cnt = n - b * QK_K < QK_K ? n - b * QK_K : QK_K;
+        memcpy(dst + b * QK_K, tmp, cnt * sizeof(float));
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* k_quants.rs:474-496 dequantize_q6k + :614-660 dequantize_q6k_bytes        */
+/* ------------------------------------------------------------------------- */
+static void dequantize_q6k_block(const uint8_t *blk, float *out) {
+    float d = pmo_f16_to_f32((uint16_t)(blk[208] | (blk[209] << 8)));
+    for (int n = 0; n < QK_K; n += 128) {
+        int c = n / 128;
+        float *ys = out + n;
+        const int8_t *sc = (const int8_t *)(blk + 192 + 8 * c);
+        const uint8_t *ql = blk + 64 * c;
+        const uint8_t *qh = blk + 128 + 32 * c;
+        for (int l = 0; l < 32; l++) {
+            int is = l / 16;
+            int8_t q1 = (int8_t)((int8_t)((ql[l] & 0xF) | ((qh[l] & 3) << 4)) - 32);
+            int8_t q2 = (int8_t)((int8_t)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32);
+            int8_t q3 = (int8_t)((int8_t)((ql[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32);
+            int8_t q4 = (int8_t)((int8_t)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32);
+            ys[l] = d * (float)sc[is] * (float)q1;
+            ys[l + 32] = d * (float)sc[is + 2] * (float)q2;
+            ys[l + 64] = d * (float)sc[is + 4] * (float)q3;
+            ys[l + 96] = d * (float)sc[is + 6] * (float)q4;
+        }
+    }
+}
+
+void pmo_dequantize_q6k(const uint8_t *src, size_t n, float *dst) {
+    size_t n_blocks = n / QK_K + (n % QK_K != 0);
+    float tmp[QK_K];
+    for (size_t b = 0; b < n_blocks; b++) {
+        dequantize_q6k_block(src + b * 210, tmp);
+        size_t cnt = n - b * QK_K < QK_K ? n - b * QK_K : QK_K;
+        memcpy(dst + b * QK_K, tmp, cnt * sizeof(float));
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* quantize.rs:17-87 and dequant.rs:92-132, :184-216                         */
+/* ------------------------------------------------------------------------- */
+int32_t pmo_quantize(uint32_t t, const float *x, size_t n, uint8_t *dst, size_t dst_len) {
+    if (t != PMO_TYPE_Q8_0 && t != PMO_TYPE_Q4K && t != PMO_TYPE_Q6K) return PMO_ERR_UNSUPPORTED_TYPE;
+    if (dst_len != pmo_tensor_size(t, n)) return PMO_ERR_INVALID_SIZE;
+    if (t == PMO_TYPE_Q8_0) pmo_quantize_q8_0(x, n, dst);
+    else if (t == PMO_TYPE_Q4K) pmo_quantize_q4k(x, n, dst);
+    else pmo_quantize_q6k(x, n, dst);
+    return PMO_OK;
+}
+
+int32_t pmo_dequantize(uint32_t t, const uint8_t *src, size_t src_len, const int32_t *shape, size_t ndim,
+                       float *dst, size_t dst_cap, uint32_t order) {
+    if (t != PMO_TYPE_Q8_0 && t != PMO_TYPE_Q4K && t != PMO_TYPE_Q6K) return PMO_ERR_UNSUPPORTED_TYPE;
+    /* dequant.rs:193-206 shape_n_elements */
+    for (size_t i = 0; i < ndim; i++)
+        if (shape[i] < 0) return PMO_ERR_INVALID_SHAPE;
+    size_t n = 1;
+    for (size_t i = 0; i < ndim; i++) {
+        size_t dim = (size_t)shape[i];
+        if (dim != 0 && n > SIZE_MAX / dim) return PMO_ERR_SHAPE_TOO_LARGE;
+        n *= dim;
+    }
+    /* dequant.rs:208-216 validate_data_size */
+    if (src_len != pmo_tensor_size(t, n)) return PMO_ERR_INVALID_SIZE;
+    if (dst_cap < n) return PMO_ERR_INVALID_SIZE;
+    if (t == PMO_TYPE_Q8_0) pmo_dequantize_q8_0(src, n, dst);
+    else if (t == PMO_TYPE_Q4K) pmo_dequantize_q4k(src, n, dst, order);
+    else pmo_dequantize_q6k(src, n, dst);
+    return PMO_OK;
+}
+
+/* ------------------------------------------------------------------------- */
+/* crates/pmetal/src/commands/quantize.rs:955-1137 (method q4_k_m)           */
+/* ------------------------------------------------------------------------- */
+int32_t pmo_use_more_bits(size_t layer, size_t n_layers) {
+    if (n_layers == 0) return 0;
+    size_t sat = layer >= n_layers / 8 ? layer - n_layers / 8 : 0; /* saturating_sub */
+    return layer < n_layers / 8 || layer >= 7 * n_layers / 8 || sat % 3 == 2;
+}
+
+static int ends_with(const char *s, const char *suffix) {
+    size_t a = strlen(s), b = strlen(suffix);
+    return a >= b && memcmp(s + a - b, suffix, b) == 0;
+}
+
+int32_t pmo_is_quantizable_gguf_tensor(const char *name, size_t ndim) {
+    static const char *const deny[] = {
+        "_norm.weight", "norm.weight", "ffn_gate_inp.weight", "router", "altup", "laurel",
+        "per_layer_model_proj", "pos_embd", "token_types", "ssm_conv1d", "shortconv.conv.weight",
+        "attn_rel_b.weight", ".position_embd", ".rel_pos", ".patch_embd", ".patch_merger"};
+    if (!(ndim == 2 || ndim == 3) || !ends_with(name, ".weight")) return 0;
+    char lower[512];
+    size_t len = strlen(name);
+    if (len >= sizeof lower) len = sizeof lower - 1;
+    for (size_t i = 0; i < len; i++) {
+        char c = name[i];
+        lower[i] = (c >= 'A' && c <= 'Z') ? (char)(c + 32) : c;
+    }
+    lower[len] = 0;
+    for (size_t i = 0; i < sizeof deny / sizeof deny[0]; i++)
+        if (strstr(lower, deny[i])) return 0;
+    return 1;
+}
+
+/* parse_layer_from_gguf_name :982-986: "blk.<n>.rest" */
+static int parse_layer(const char *name, size_t *layer) {
+    if (strncmp(name, "blk.", 4) != 0) return 0;
+    const char *p = name + 4;
+    const char *dot = strchr(p, '.');
+    if (!dot || dot == p) return 0;
+    size_t v = 0;
+    const char *q = p;
+    if (*q == '+') q++; /* usize::from_str accepts a leading '+' */
+    if (q == dot) return 0;
+    for (; q < dot; q++) {
+        if (*q < '0' || *q > '9') return 0;
+        v = v * 10 + (size_t)(*q - '0');
+    }
+    *layer = v;
+    return 1;
+}
+
+uint32_t pmo_q4km_tensor_type(const char *name, size_t ndim, size_t n_layers) {
+    if (!pmo_is_quantizable_gguf_tensor(name, ndim)) return PMO_TYPE_F16; /* :1015-1017 */
+    uint32_t dtype = PMO_TYPE_Q4K;                                        /* :1019-1023 */
+    size_t layer = 0;
+    if (!parse_layer(name, &layer)) layer = 0; /* :1034 */
+    if (strcmp(name, "output.weight") == 0 || strcmp(name, "token_embd.weight") == 0)
+        return PMO_TYPE_Q6K; /* :1036-1055 */
+    if (strstr(name, "attn_v.weight")) { /* :1058-1090, arm Q4KM :1075-1081 */
+        if (pmo_use_more_bits(layer, n_layers)) dtype = PMO_TYPE_Q6K;
+    } else if (strstr(name, "ffn_down.weight") || strstr(name, "ffn_down_exps.weight")) {
+        if (pmo_use_more_bits(layer, n_layers)) dtype = PMO_TYPE_Q6K; /* :1104-1110 */
+    } else if (strstr(name, "attn_output.weight")) {
+        /* :1120-1126: q4_k_m keeps the default */
+    } else if (strstr(name, "attn_qkv.weight")) {
+        /* :1127-1133: q4_k_m -> Q5K, a type outside this path; reported as its GgmlType id 13 */
+        dtype = 13;
+    }
+    return dtype;
+}
+
+/* ------------------------------------------------------------------------- */
+/* dequantize-then-matmul (definition of the fused kernels' expected output) */
+/* ------------------------------------------------------------------------- */
+static int32_t dequant_row(uint32_t t, const uint8_t *w, size_t row, size_t k, float *tmp, uint32_t order) {
+    size_t row_bytes = pmo_tensor_size(t, k);
+    if (t == PMO_TYPE_Q8_0) pmo_dequantize_q8_0(w + row * row_bytes, k, tmp);
+    else if (t == PMO_TYPE_Q4K) pmo_dequantize_q4k(w + row * row_bytes, k, tmp, order);
+    else if (t == PMO_TYPE_Q6K) pmo_dequantize_q6k(w + row * row_bytes, k, tmp);
+    else return PMO_ERR_UNSUPPORTED_TYPE;
+    return PMO_OK;
+}
+
+int32_t pmo_qmatvec_f64(uint32_t t, const uint8_t *w, size_t n_rows, size_t k, const float *x, float *y,
+                        uint32_t order) {
+    size_t bs = pmo_block_size(t);
+    if (bs <= 1 || k % bs != 0) return PMO_ERR_INVALID_SHAPE;
+    float *tmp = (float *)malloc(k * sizeof(float));
+    if (!tmp) return PMO_ERR_SHAPE_TOO_LARGE;
+    for (size_t r = 0; r < n_rows; r++) {
+        dequant_row(t, w, r, k, tmp, order);
+        double acc = 0.0;
+        for (size_t i = 0; i < k; i++) acc += (double)tmp[i] * (double)x[i];
+        y[r] = (float)acc;
+    }
+    free(tmp);
+    return PMO_OK;
+}
+
+int32_t pmo_qmatvec_f32(uint32_t t, const uint8_t *w, size_t n_rows, size_t k, const float *x, float *y,
+                        uint32_t order) {
+    size_t bs = pmo_block_size(t);
+    if (bs <= 1 || k % bs != 0) return PMO_ERR_INVALID_SHAPE;
+    float *tmp = (float *)malloc(k * sizeof(float));
+    if (!tmp) return PMO_ERR_SHAPE_TOO_LARGE;
+    for (size_t r = 0; r < n_rows; r++) {
+        dequant_row(t, w, r, k, tmp, order);
+        float acc = 0.0f;
+        for (size_t i = 0; i < k; i++) acc += tmp[i] * x[i];
+        y[r] = acc;
+    }
+    free(tmp);
+    return PMO_OK;
+}
+
+int32_t pmo_qmatmul_f64(uint32_t t, const uint8_t *w, size_t n_rows, size_t k, const float *x, size_t m_rows,
+                        float *y, uint32_t order) {
+    size_t bs = pmo_block_size(t);
+    if (bs <= 1 || k % bs != 0) return PMO_ERR_INVALID_SHAPE;
+    float *tmp = (float *)malloc(k * sizeof(float));
+    if (!tmp) return PMO_ERR_SHAPE_TOO_LARGE;
+    for (size_t r = 0; r < n_rows; r++) {
+        dequant_row(t, w, r, k, tmp, order);
+        for (size_t m = 0; m < m_rows; m++) {
+            const float *xr = x + m * k;
+            double acc = 0.0;
+            for (size_t i = 0; i < k; i++) acc += (double)tmp[i] * (double)xr[i];
+            y[m * n_rows + r] = (float)acc;
+        }
+    }
+    free(tmp);
+    return PMO_OK;
+}

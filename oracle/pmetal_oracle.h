@@ -1,0 +1,115 @@
+/*
+ * pmetal_oracle.h -- CPU restatement of PMetal's GGUF block-quantized weight path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This is the checker the HIP kernels are compared
+ * against; nothing in the shipped library links, loads or calls it.  Only the
+ * test-suite, the smoke check and the benchmark's CPU-baseline leg use it.
+ *
+ * Every function follows one function of the reference (Epistates/pmetal,
+ * crate pmetal-gguf) and cites it as file:line relative to the reference root.
+ * The reference is Rust and cannot be compiled in this environment, so the
+ * oracle is pinned by the reference's own known-answer tests, by closed forms
+ * and by an independent numpy-float32 re-derivation (see tests/).  The bytes of
+ * quantize_q4k / quantize_q6k on general inputs are therefore pinned by the
+ * fidelity of this restatement and the independent twin only, never by running
+ * the Rust: "restatement-pinned".
+ */
+#ifndef PMETAL_ORACLE_H
+#define PMETAL_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* GgmlType ids, crates/pmetal-gguf/src/types.rs:16-97 (only the path's types). */
+enum {
+    PMO_TYPE_F32 = 0,
+    PMO_TYPE_F16 = 1,
+    PMO_TYPE_Q8_0 = 8,
+    PMO_TYPE_Q4K = 12,
+    PMO_TYPE_Q6K = 14,
+};
+
+/* Error classes mirroring DequantError (dequant.rs:37-70) and
+ * PMetalError::Quantization (quantize.rs:82-85). */
+enum {
+    PMO_OK = 0,
+    PMO_ERR_UNSUPPORTED_TYPE = 2,
+    PMO_ERR_INVALID_SIZE = 3,
+    PMO_ERR_INVALID_SHAPE = 6,
+    PMO_ERR_SHAPE_TOO_LARGE = 7,
+};
+
+/* Q4_K element order used by dequantize / matvec:
+ *   REF  = the order the reference's dequantize_q4k emits (k_quants.rs:365-403);
+ *   GGML = the order its own quantizer packs (k_quants.rs:946-951). */
+enum { PMO_ORDER_REF = 0, PMO_ORDER_GGML = 1 };
+
+/* half 2.7.1 conversions (Cargo.lock:2429-2432): IEEE binary16 / bfloat16, RNE. */
+uint16_t pmo_f32_to_f16(float f);
+float pmo_f16_to_f32(uint16_t h);
+uint16_t pmo_f32_to_bf16(float f);
+float pmo_bf16_to_f32(uint16_t h);
+
+/* quantize.rs:566-570 */
+int32_t pmo_nearest_int(float v);
+/* quantize.rs:583-644; n <= 256 */
+void pmo_make_qkx1_quants(int32_t nmax, int32_t ntry, const float *x, int32_t n,
+                          float *scale_out, float *min_out);
+/* quantize.rs:738-841; n <= 256; ls receives n values in [0, 2*nmax) */
+float pmo_make_qx_quants(int32_t n, int32_t nmax, const float *x, int32_t rmse_type, int8_t *ls);
+/* quantize.rs:844-855 */
+void pmo_get_scale_min_k4(int32_t j, const uint8_t *q, uint8_t *sc, uint8_t *m);
+
+/* types.rs:102-187 */
+size_t pmo_type_size(uint32_t ggml_type);  /* 0 if not one of the path's types */
+size_t pmo_block_size(uint32_t ggml_type); /* 0 if not one of the path's types */
+size_t pmo_tensor_size(uint32_t ggml_type, size_t n_elements);
+
+/* quantize.rs:268-300, k_quants.rs:876-955, k_quants.rs:1056-1134.
+ * dst must hold pmo_tensor_size(type, n) bytes. */
+void pmo_quantize_q8_0(const float *x, size_t n, uint8_t *dst);
+void pmo_quantize_q4k(const float *x, size_t n, uint8_t *dst);
+void pmo_quantize_q6k(const float *x, size_t n, uint8_t *dst);
+
+/* dequant.rs:466-495, k_quants.rs:358-404 + 515-560, k_quants.rs:474-496 + 614-660.
+ * src holds pmo_tensor_size(type, n) bytes; dst receives n floats. */
+void pmo_dequantize_q8_0(const uint8_t *src, size_t n, float *dst);
+void pmo_dequantize_q4k(const uint8_t *src, size_t n, float *dst, uint32_t order);
+void pmo_dequantize_q6k(const uint8_t *src, size_t n, float *dst);
+
+/* quantize.rs:17-87 (dispatcher) and dequant.rs:92-132 + 184-216 (dispatcher and
+ * validation).  Return a PMO_* code. */
+int32_t pmo_quantize(uint32_t ggml_type, const float *x, size_t n, uint8_t *dst, size_t dst_len);
+int32_t pmo_dequantize(uint32_t ggml_type, const uint8_t *src, size_t src_len, const int32_t *shape,
+                       size_t ndim, float *dst, size_t dst_cap, uint32_t order);
+
+/* crates/pmetal/src/commands/quantize.rs:988-993 */
+int32_t pmo_use_more_bits(size_t layer, size_t n_layers);
+/* crates/pmetal/src/commands/quantize.rs:955-980 */
+int32_t pmo_is_quantizable_gguf_tensor(const char *gguf_name, size_t ndim);
+/* crates/pmetal/src/commands/quantize.rs:999-1137 restricted to method q4_k_m:
+ * returns the GgmlType id chosen for the tensor. */
+uint32_t pmo_q4km_tensor_type(const char *gguf_name, size_t ndim, size_t n_layers);
+
+/* Not a reference function: "reference dequantize, then matmul", the definition
+ * the fused GEMV/GEMM kernels are checked against.  W is [n_rows, k] quantized
+ * row-major; x is f32 [k]; y[n] = sum_k W[n,k]*x[k] accumulated in double and
+ * rounded once.  The _f32 variant accumulates sequentially in float (what a
+ * plain f32 CPU matmul after the reference's dequantize would do) and is the
+ * function the CPU baseline times. */
+int32_t pmo_qmatvec_f64(uint32_t ggml_type, const uint8_t *w, size_t n_rows, size_t k,
+                        const float *x, float *y, uint32_t order);
+int32_t pmo_qmatvec_f32(uint32_t ggml_type, const uint8_t *w, size_t n_rows, size_t k,
+                        const float *x, float *y, uint32_t order);
+/* Y[m, n] = sum_k X[m,k] * W[n,k]; X f32 [m_rows, k] row-major, Y f32 [m_rows, n_rows]. */
+int32_t pmo_qmatmul_f64(uint32_t ggml_type, const uint8_t *w, size_t n_rows, size_t k,
+                        const float *x, size_t m_rows, float *y, uint32_t order);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
