@@ -1,0 +1,177 @@
+/*
+ * pmetal_hip.h -- C ABI of libpmetal_hip.so: PMetal's GGUF block-quantized weight
+ * path (Q8_0, Q4_K, Q6_K) as hand-written HIP kernels for MI355X (gfx950).
+ *
+ * This is the surface a Rust `-sys` crate binds (plain pointers and sizes, no
+ * C++ or framework types).  Every entry point names the reference interface it
+ * stands in for as file:line under the reference tree (Epistates/pmetal).
+ *
+ * Conventions
+ *  - Return value: 0 on success, otherwise one of the PMETAL_HIP_ERR_* classes; the
+ *    failing call also stores a message in a thread-local slot (the pattern of
+ *    crates/pmetal-bridge/cpp/bridge/common.h:41-58).  Nothing throws or aborts
+ *    across the ABI.
+ *  - Ownership: the caller owns every buffer it passes and every device allocation
+ *    it requested; the library keeps no caller pointer after a call returns.
+ *  - Device pointers must be 16-byte aligned (hipMalloc and torch allocations are;
+ *    GGUF tensor data is 32-byte aligned in the file).
+ *  - `stream` is a hipStream_t passed as void*; NULL is the default stream.  Device
+ *    entry points are asynchronous on that stream; host-pointer entry points
+ *    synchronise before returning.
+ *  - Tensors are flat row-major [rows, k]; blocks run along k.
+ *  - There is no CPU fallback: without a usable HIP device every compute entry
+ *    point fails with PMETAL_HIP_ERR_NO_DEVICE.
+ */
+#ifndef PMETAL_HIP_H
+#define PMETAL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* GgmlType ids: crates/pmetal-gguf/src/types.rs:16-97. */
+#define PMETAL_GGML_TYPE_F32 0u
+#define PMETAL_GGML_TYPE_F16 1u
+#define PMETAL_GGML_TYPE_Q8_0 8u
+#define PMETAL_GGML_TYPE_Q4K 12u
+#define PMETAL_GGML_TYPE_Q5K 13u /* named by the recipe only; no kernels */
+#define PMETAL_GGML_TYPE_Q6K 14u
+
+/* Error classes.  1-3, 6, 7 map onto DequantError (crates/pmetal-gguf/src/dequant.rs:37-70)
+ * and PMetalError::Quantization (crates/pmetal-core/src/error.rs:50-52). */
+#define PMETAL_HIP_OK 0
+#define PMETAL_HIP_ERR_INVALID_ARG 1      /* null pointer, misalignment, bad enum        */
+#define PMETAL_HIP_ERR_UNSUPPORTED_TYPE 2 /* DequantError::UnsupportedType / Quantization */
+#define PMETAL_HIP_ERR_INVALID_SIZE 3     /* DequantError::InvalidSize                    */
+#define PMETAL_HIP_ERR_HIP_RUNTIME 4      /* a HIP call failed; message has hipGetErrorString */
+#define PMETAL_HIP_ERR_NO_DEVICE 5
+#define PMETAL_HIP_ERR_INVALID_SHAPE 6   /* DequantError::InvalidShape                   */
+#define PMETAL_HIP_ERR_SHAPE_TOO_LARGE 7 /* DequantError::ShapeTooLarge                  */
+
+/* Q4_K element order for dequantize / GEMV / GEMM.
+ *  REF : the order the reference's dequantize_q4k emits (k_quants.rs:365-403); default,
+ *        bit-compatible with what `load_gguf` (weight_format.rs:299) hands to the model.
+ *  GGML: the inverse of the packing done by the reference's quantize_q4k
+ *        (k_quants.rs:946-951), i.e. what llama.cpp/Candle decode.                     */
+#define PMETAL_HIP_ORDER_REF 0u
+#define PMETAL_HIP_ORDER_GGML 1u
+
+/* Activation / output element types. */
+#define PMETAL_HIP_DTYPE_F32 0u
+#define PMETAL_HIP_DTYPE_BF16 1u
+
+/* ---- lifecycle and errors (crates/pmetal-bridge/cpp/bridge/common.h:41-58) ---------- */
+int32_t pmetal_hip_device_count(void);
+/* Selects `device` for the calling thread and loads the kernels. */
+int32_t pmetal_hip_init(int32_t device);
+int32_t pmetal_hip_last_error_code(void);
+/* NUL-terminated, never NULL, valid until the next call on this thread. */
+const char *pmetal_hip_last_error_message(void);
+void pmetal_hip_clear_error(void);
+
+/* ---- sizes (crates/pmetal-gguf/src/types.rs:102-187) -------------------------------- */
+size_t pmetal_hip_type_size(uint32_t ggml_type);  /* bytes per block; 0 if unsupported  */
+size_t pmetal_hip_block_size(uint32_t ggml_type); /* elements per block; 0 if unsupported */
+size_t pmetal_hip_tensor_size(uint32_t ggml_type, size_t n_elements);
+/* dequant.rs:178-206 expected_byte_size_checked: validates `shape`, returns the byte size
+ * through *out_bytes and the element count through *out_elements (either may be NULL). */
+int32_t pmetal_hip_expected_byte_size(uint32_t ggml_type, const int32_t *shape, size_t ndim,
+                                      size_t *out_bytes, size_t *out_elements);
+/* dequant.rs:135 is_supported / quantize.rs:17-87 arms, restricted to this path. */
+int32_t pmetal_hip_is_supported(uint32_t ggml_type);
+
+/* ---- device memory ------------------------------------------------------------------ */
+void *pmetal_hip_alloc(size_t bytes); /* NULL on failure (error slot set) */
+int32_t pmetal_hip_free(void *dptr);
+int32_t pmetal_hip_h2d(void *dst_dev, const void *src_host, size_t bytes);
+int32_t pmetal_hip_d2h(void *dst_host, const void *src_dev, size_t bytes);
+int32_t pmetal_hip_memset(void *dst_dev, int value, size_t bytes, void *stream);
+int32_t pmetal_hip_sync(void *stream);
+
+/* ---- events (timing on the stream the kernels run on) -------------------------------- */
+void *pmetal_hip_event_create(void);
+int32_t pmetal_hip_event_record(void *event, void *stream);
+int32_t pmetal_hip_event_elapsed_ms(void *start, void *stop, float *ms); /* syncs on stop */
+int32_t pmetal_hip_event_destroy(void *event);
+
+/* ---- quantize: pmetal_gguf::quantize::quantize(data, dtype) -> Vec<u8> ---------------
+ * crates/pmetal-gguf/src/quantize.rs:17-87; kernels follow quantize_q8_0 (:268-300),
+ * quantize_q4k (k_quants.rs:876-955), quantize_q6k (k_quants.rs:1056-1134).
+ * Output bytes are bit-identical to the reference CPU path.  dst_len must equal
+ * pmetal_hip_tensor_size(type, n).  A trailing partial 256-super-block is emitted as
+ * zero bytes (k_quants.rs:890-892); Q8_0 zero-pads inside its last block.            */
+int32_t pmetal_hip_quantize(uint32_t ggml_type, const float *src_host, size_t n, uint8_t *dst_host,
+                            size_t dst_len);
+int32_t pmetal_hip_quantize_dev(uint32_t ggml_type, const float *src_dev, size_t n, uint8_t *dst_dev,
+                                size_t dst_len, void *stream);
+
+/* ---- dequantize: pmetal_gguf::dequant::dequantize(data, dtype, shape) -> Vec<f32> ----
+ * crates/pmetal-gguf/src/dequant.rs:92-132 with its validation (:184-216); kernels follow
+ * dequantize_q8_0 (:466-495), dequantize_q4k (k_quants.rs:358-404, :515-560),
+ * dequantize_q6k (k_quants.rs:474-496, :614-660).  Values are bit-identical to the
+ * reference.  dst_len is the capacity of dst in floats and must be >= the element count.
+ * The host variant mirrors MlxMetalBridge::dequantize_q4_0 (crates/pmetal-mlx/src/
+ * bridge.rs:65-84): host bytes in, synchronous.                                         */
+int32_t pmetal_hip_dequantize(uint32_t ggml_type, const uint8_t *src_host, size_t src_len,
+                              const int32_t *shape, size_t ndim, float *dst_host, size_t dst_len,
+                              uint32_t order);
+int32_t pmetal_hip_dequantize_dev(uint32_t ggml_type, const uint8_t *src_dev, size_t src_len, float *dst_dev,
+                                  size_t n, uint32_t order, void *stream);
+
+/* ---- quantized linear ------------------------------------------------------------------
+ * Stand in for InlineArray::quantized_matmul(x, w, .., transpose = true, ..)
+ * (crates/pmetal-bridge/src/inline_array/quantized.rs:55-108, C side
+ * crates/pmetal-bridge/cpp/bridge/quantized.h:19-22) and LayerWeight::matmul_from
+ * (crates/pmetal-bridge/src/qwen3_native/weights.rs:66-84) for GGUF-typed weights:
+ *   y[n]    = sum_k W[n,k] * x[k]                      (qgemv, one token)
+ *   Y[m, n] = sum_k X[m,k] * W[n,k]                    (qgemm, m tokens)
+ * with W = reference dequantize of the packed blocks (order as given), fp32 accumulation,
+ * max relative error <= 1e-3 against dequantize-then-f32-matmul.
+ * W: [n, k] packed row-major, k a multiple of the block size.  x/X: f32 or bf16.
+ * y/Y: f32 (qgemv) or f32/bf16 (qgemm), row-major [m, n].                               */
+int32_t pmetal_hip_qgemv(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, int64_t k, const void *x_dev,
+                         uint32_t x_dtype, float *y_dev, uint32_t order, void *stream);
+int32_t pmetal_hip_qgemm(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, int64_t k, const void *x_dev,
+                         uint32_t x_dtype, int64_t m, void *y_dev, uint32_t y_dtype, uint32_t order,
+                         void *stream);
+/* Dispatch by m: m == 1 -> qgemv (f32 output only), otherwise qgemm. */
+int32_t pmetal_hip_qlinear(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, int64_t k, const void *x_dev,
+                           uint32_t x_dtype, int64_t m, void *y_dev, uint32_t y_dtype, uint32_t order,
+                           void *stream);
+
+/* One decode step's worth of batch-1 projections, launched back to back on one stream
+ * (the per-token loop over LayerWeight::matmul_from, weights.rs:66-84). */
+typedef struct pmetal_hip_linear_desc {
+    uint32_t ggml_type;
+    uint32_t x_dtype;
+    uint32_t order;
+    uint32_t reserved;
+    int64_t n;
+    int64_t k;
+    const uint8_t *w_dev;
+    const void *x_dev;
+    float *y_dev;
+} pmetal_hip_linear_desc;
+int32_t pmetal_hip_qgemv_batch(const pmetal_hip_linear_desc *descs, size_t count, void *stream);
+
+/* ---- Q4_K_M recipe (crates/pmetal/src/commands/quantize.rs) --------------------------- */
+int32_t pmetal_hip_use_more_bits(size_t layer, size_t n_layers);                   /* :988-993  */
+int32_t pmetal_hip_is_quantizable_gguf_tensor(const char *gguf_name, size_t ndim); /* :955-980  */
+/* llama_style_tensor_type (:999-1137) for method q4_k_m: GgmlType id for the tensor. */
+uint32_t pmetal_hip_q4km_tensor_type(const char *gguf_name, size_t ndim, size_t n_layers);
+
+/* ---- synthetic tensors for benchmarks (no reference counterpart) ---------------------- */
+/* Fills dst_dev[n] with N(0, std^2) from a counter-based generator keyed by (seed, index);
+ * a fraction `outlier_rate` of elements is replaced by +-outlier_mag.                    */
+int32_t pmetal_hip_fill_normal_f32(float *dst_dev, size_t n, uint64_t seed, float std, float outlier_rate,
+                                   float outlier_mag, void *stream);
+/* f32 -> bf16 (round to nearest even), device to device. */
+int32_t pmetal_hip_f32_to_bf16_dev(const float *src_dev, uint16_t *dst_dev, size_t n, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PMETAL_HIP_H */

@@ -125,6 +125,24 @@ static int total_cmp(float a, float b) {
     return (l > r) - (l < r);
 }
 
+/* f32::max / f32::min (IEEE 754-2008 maxNum / minNum: a NaN operand is ignored).  For the pair
+ * (-0.0, +0.0) IEEE leaves the result open; the reference only runs on Apple Silicon (MLX/Metal),
+ * whose FMAXNM / FMINNM order -0.0 below +0.0, so that is what is restated here (the C library's
+ * own max would return its first argument instead). */
+static float rust_max(float a, float b) {
+    if (a != a) return b;
+    if (b != b) return a;
+    if (a == b) return bits_f32(f32_bits(a) & f32_bits(b)); /* +0 wins over -0 */
+    return a > b ? a : b;
+}
+
+static float rust_min(float a, float b) {
+    if (a != a) return b;
+    if (b != b) return a;
+    if (a == b) return bits_f32(f32_bits(a) | f32_bits(b)); /* -0 wins over +0 */
+    return a < b ? a : b;
+}
+
 static int32_t clamp_i32(int32_t v, int32_t lo, int32_t hi) { return v < lo ? lo : (v > hi ? hi : v); }
 
 /* quantize.rs:566-570: `v.round() as i32` -- half away from zero, saturating. */
@@ -151,7 +169,7 @@ void pmo_make_qkx1_quants(int32_t nmax, int32_t ntry, const float *x, int32_t n,
         return;
     }
     /* :601 */
-    min = fminf(min, 0.0f);
+    min = rust_min(min, 0.0f);
     /* :604-605 */
     float iscale = (float)nmax / (max - min);
     float scale = 1.0f / iscale;
@@ -336,7 +354,7 @@ void pmo_quantize_q8_0(const float *x, size_t n, uint8_t *dst) {
         size_t start = b * 32;
         size_t end = start + 32 < n ? start + 32 : n;
         float amax = 0.0f;
-        for (size_t i = start; i < end; i++) amax = fmaxf(amax, fabsf(x[i])); /* acc.max(x.abs()) */
+        for (size_t i = start; i < end; i++) amax = rust_max(amax, fabsf(x[i])); /* acc.max(x.abs()) */
         float scale = amax / 127.0f;
         float iscale = amax == 0.0f ? 0.0f : 127.0f / amax;
         uint16_t d = pmo_f32_to_f16(scale);
@@ -370,8 +388,8 @@ void pmo_quantize_q4k(const float *xs, size_t n, uint8_t *dst) {
 
         /* :904-905 fold(0.0, |max, val| val.max(max)) */
         float max_scale = 0.0f, max_min = 0.0f;
-        for (int j = 0; j < 8; j++) max_scale = fmaxf(scales[j], max_scale);
-        for (int j = 0; j < 8; j++) max_min = fmaxf(mins[j], max_min);
+        for (int j = 0; j < 8; j++) max_scale = rust_max(scales[j], max_scale);
+        for (int j = 0; j < 8; j++) max_min = rust_max(mins[j], max_min);
 
         float inv_scale = max_scale > 0.0f ? 63.0f / max_scale : 0.0f;
         float inv_min = max_min > 0.0f ? 63.0f / max_min : 0.0f;

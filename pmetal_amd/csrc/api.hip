@@ -1,0 +1,478 @@
+// extern "C" surface of libpmetal_hip.so (declared in include/pmetal_hip.h).
+//
+// Host-side argument validation mirrors the reference's dispatchers
+// (crates/pmetal-gguf/src/quantize.rs:17-87, crates/pmetal-gguf/src/dequant.rs:92-132 and :184-216)
+// so that a Rust caller sees the same error classes; failures are reported through a return code
+// plus a thread-local message slot, the pattern of crates/pmetal-bridge/cpp/bridge/common.h:41-58.
+// There is no CPU fallback anywhere in this file: without a HIP device every compute call fails.
+#include "../../include/pmetal_hip.h"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+
+#include "internal.hpp"
+
+namespace {
+
+thread_local int32_t g_err_code = 0;
+thread_local char g_err_msg[512] = {0};
+
+int32_t fail(int32_t code, const char *fmt, ...) {
+    g_err_code = code;
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err_msg, sizeof g_err_msg, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int32_t ok() {
+    g_err_code = 0;
+    g_err_msg[0] = 0;
+    return PMETAL_HIP_OK;
+}
+
+int32_t hip_fail(hipError_t e, const char *what) {
+    (void)hipGetLastError();  // do not let a sticky error leak into the next call
+    if (e == hipErrorNoDevice || e == hipErrorInvalidDevice || e == hipErrorInsufficientDriver)
+        return fail(PMETAL_HIP_ERR_NO_DEVICE, "%s: %s", what, hipGetErrorString(e));
+    return fail(PMETAL_HIP_ERR_HIP_RUNTIME, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define HIP_TRY(expr)                                      \
+    do {                                                   \
+        hipError_t _e = (expr);                            \
+        if (_e != hipSuccess) return hip_fail(_e, #expr);  \
+    } while (0)
+
+bool path_type(uint32_t t) {
+    return t == PMETAL_GGML_TYPE_Q8_0 || t == PMETAL_GGML_TYPE_Q4K || t == PMETAL_GGML_TYPE_Q6K;
+}
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// One-time check that a usable device exists; compute entry points call it first.
+int32_t require_device() {
+    static std::once_flag once;
+    static hipError_t status = hipSuccess;
+    static int count = 0;
+    std::call_once(once, [] {
+        status = hipGetDeviceCount(&count);
+        if (status != hipSuccess) (void)hipGetLastError();
+    });
+    if (status != hipSuccess) return hip_fail(status, "hipGetDeviceCount");
+    if (count <= 0) return fail(PMETAL_HIP_ERR_NO_DEVICE, "no HIP device is visible");
+    return PMETAL_HIP_OK;
+}
+
+// dequant.rs:193-206 shape_n_elements
+int32_t shape_elements(const int32_t *shape, size_t ndim, size_t *out) {
+    if (ndim > 0 && !shape) return fail(PMETAL_HIP_ERR_INVALID_ARG, "shape is NULL");
+    for (size_t i = 0; i < ndim; i++)
+        if (shape[i] < 0) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "dimensions must be non-negative");
+    size_t n = 1;
+    for (size_t i = 0; i < ndim; i++) {
+        const size_t dim = (size_t)shape[i];
+        if (dim != 0 && n > SIZE_MAX / dim) return fail(PMETAL_HIP_ERR_SHAPE_TOO_LARGE, "shape is too large");
+        n *= dim;
+    }
+    *out = n;
+    return PMETAL_HIP_OK;
+}
+
+struct DevBuf {
+    void *p = nullptr;
+    ~DevBuf() {
+        if (p) (void)hipFree(p);
+    }
+};
+
+// qgemm scratch, grown on demand and kept per thread so concurrent callers do not share it.
+struct Workspace {
+    void *p = nullptr;
+    size_t bytes = 0;
+    int device = -1;
+};
+thread_local Workspace g_ws;
+
+int32_t workspace(size_t bytes, void **out) {
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    if (g_ws.p && (g_ws.bytes < bytes || g_ws.device != dev)) {
+        HIP_TRY(hipDeviceSynchronize());
+        HIP_TRY(hipFree(g_ws.p));
+        g_ws = Workspace{};
+    }
+    if (!g_ws.p && bytes) {
+        HIP_TRY(hipMalloc(&g_ws.p, bytes));
+        g_ws.bytes = bytes;
+        g_ws.device = dev;
+    }
+    *out = g_ws.p;
+    return PMETAL_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t pmetal_hip_device_count(void) {
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) {
+        hip_fail(e, "hipGetDeviceCount");
+        return 0;
+    }
+    ok();
+    return n;
+}
+
+int32_t pmetal_hip_init(int32_t device) {
+    if (int32_t rc = require_device()) return rc;
+    int n = 0;
+    HIP_TRY(hipGetDeviceCount(&n));
+    if (device < 0 || device >= n) return fail(PMETAL_HIP_ERR_INVALID_ARG, "device %d out of range [0, %d)", device, n);
+    HIP_TRY(hipSetDevice(device));
+    HIP_TRY(hipFree(nullptr));  // forces context creation and code-object load
+    return ok();
+}
+
+int32_t pmetal_hip_last_error_code(void) { return g_err_code; }
+const char *pmetal_hip_last_error_message(void) { return g_err_msg; }
+void pmetal_hip_clear_error(void) { ok(); }
+
+// ---- sizes: types.rs:102-187 ----
+size_t pmetal_hip_type_size(uint32_t t) {
+    switch (t) {
+    case PMETAL_GGML_TYPE_Q8_0: return 34;
+    case PMETAL_GGML_TYPE_Q4K: return 144;
+    case PMETAL_GGML_TYPE_Q6K: return 210;
+    default: return 0;
+    }
+}
+
+size_t pmetal_hip_block_size(uint32_t t) {
+    switch (t) {
+    case PMETAL_GGML_TYPE_Q8_0: return 32;
+    case PMETAL_GGML_TYPE_Q4K:
+    case PMETAL_GGML_TYPE_Q6K: return 256;
+    default: return 0;
+    }
+}
+
+size_t pmetal_hip_tensor_size(uint32_t t, size_t n) {
+    const size_t bs = pmetal_hip_block_size(t);
+    if (!bs) return 0;
+    return (n / bs + (n % bs != 0)) * pmetal_hip_type_size(t);
+}
+
+int32_t pmetal_hip_is_supported(uint32_t t) { return path_type(t) ? 1 : 0; }
+
+int32_t pmetal_hip_expected_byte_size(uint32_t t, const int32_t *shape, size_t ndim, size_t *out_bytes,
+                                      size_t *out_elements) {
+    if (!path_type(t)) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "unsupported GGML type %u", t);
+    size_t n = 0;
+    if (int32_t rc = shape_elements(shape, ndim, &n)) return rc;
+    const size_t bs = pmetal_hip_block_size(t), ts = pmetal_hip_type_size(t);
+    const size_t blocks = n / bs + (n % bs != 0);
+    if (blocks > SIZE_MAX / ts) return fail(PMETAL_HIP_ERR_SHAPE_TOO_LARGE, "shape is too large");
+    if (out_bytes) *out_bytes = blocks * ts;
+    if (out_elements) *out_elements = n;
+    return ok();
+}
+
+// ---- memory ----
+void *pmetal_hip_alloc(size_t bytes) {
+    if (require_device()) return nullptr;
+    void *p = nullptr;
+    hipError_t e = hipMalloc(&p, bytes ? bytes : 1);
+    if (e != hipSuccess) {
+        hip_fail(e, "hipMalloc");
+        return nullptr;
+    }
+    ok();
+    return p;
+}
+
+int32_t pmetal_hip_free(void *p) {
+    if (!p) return ok();
+    HIP_TRY(hipFree(p));
+    return ok();
+}
+
+int32_t pmetal_hip_h2d(void *dst, const void *src, size_t bytes) {
+    if (bytes && (!dst || !src)) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
+    if (bytes) HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+    return ok();
+}
+
+int32_t pmetal_hip_d2h(void *dst, const void *src, size_t bytes) {
+    if (bytes && (!dst || !src)) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
+    if (bytes) HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+    return ok();
+}
+
+int32_t pmetal_hip_memset(void *dst, int value, size_t bytes, void *stream) {
+    if (bytes && !dst) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
+    if (bytes) HIP_TRY(hipMemsetAsync(dst, value, bytes, (hipStream_t)stream));
+    return ok();
+}
+
+int32_t pmetal_hip_sync(void *stream) {
+    if (int32_t rc = require_device()) return rc;
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    return ok();
+}
+
+// ---- events ----
+void *pmetal_hip_event_create(void) {
+    if (require_device()) return nullptr;
+    hipEvent_t ev = nullptr;
+    hipError_t e = hipEventCreate(&ev);
+    if (e != hipSuccess) {
+        hip_fail(e, "hipEventCreate");
+        return nullptr;
+    }
+    ok();
+    return ev;
+}
+
+int32_t pmetal_hip_event_record(void *event, void *stream) {
+    if (!event) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL event");
+    HIP_TRY(hipEventRecord((hipEvent_t)event, (hipStream_t)stream));
+    return ok();
+}
+
+int32_t pmetal_hip_event_elapsed_ms(void *start, void *stop, float *ms) {
+    if (!start || !stop || !ms) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL argument");
+    HIP_TRY(hipEventSynchronize((hipEvent_t)stop));
+    HIP_TRY(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return ok();
+}
+
+int32_t pmetal_hip_event_destroy(void *event) {
+    if (!event) return ok();
+    HIP_TRY(hipEventDestroy((hipEvent_t)event));
+    return ok();
+}
+
+// ---- quantize ----
+int32_t pmetal_hip_quantize_dev(uint32_t t, const float *src, size_t n, uint8_t *dst, size_t dst_len, void *stream) {
+    if (!path_type(t))
+        return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "Quantization to GGML type %u not yet implemented", t);
+    const size_t expected = pmetal_hip_tensor_size(t, n);
+    if (dst_len != expected)
+        return fail(PMETAL_HIP_ERR_INVALID_SIZE, "Invalid data size: expected %zu bytes, got %zu", expected, dst_len);
+    if (n == 0) return ok();
+    if (!src || !dst) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
+    if (!aligned16(src) || !aligned16(dst)) return fail(PMETAL_HIP_ERR_INVALID_ARG, "device pointers must be 16-byte aligned");
+    if (int32_t rc = require_device()) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    hipError_t e;
+    if (t == PMETAL_GGML_TYPE_Q8_0) e = pmh::launch_quantize_q8_0(src, n, dst, s);
+    else if (t == PMETAL_GGML_TYPE_Q4K) e = pmh::launch_quantize_q4k(src, n, dst, s);
+    else e = pmh::launch_quantize_q6k(src, n, dst, s);
+    if (e != hipSuccess) return hip_fail(e, "quantize kernel launch");
+    return ok();
+}
+
+int32_t pmetal_hip_quantize(uint32_t t, const float *src, size_t n, uint8_t *dst, size_t dst_len) {
+    if (!path_type(t))
+        return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "Quantization to GGML type %u not yet implemented", t);
+    const size_t expected = pmetal_hip_tensor_size(t, n);
+    if (dst_len != expected)
+        return fail(PMETAL_HIP_ERR_INVALID_SIZE, "Invalid data size: expected %zu bytes, got %zu", expected, dst_len);
+    if (n == 0) return ok();
+    if (!src || !dst) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
+    if (int32_t rc = require_device()) return rc;
+    DevBuf din, dout;
+    HIP_TRY(hipMalloc(&din.p, n * sizeof(float)));
+    HIP_TRY(hipMalloc(&dout.p, expected));
+    HIP_TRY(hipMemcpy(din.p, src, n * sizeof(float), hipMemcpyHostToDevice));
+    if (int32_t rc = pmetal_hip_quantize_dev(t, (const float *)din.p, n, (uint8_t *)dout.p, expected, nullptr)) return rc;
+    HIP_TRY(hipMemcpy(dst, dout.p, expected, hipMemcpyDeviceToHost));  // synchronises the null stream
+    return ok();
+}
+
+// ---- dequantize ----
+int32_t pmetal_hip_dequantize_dev(uint32_t t, const uint8_t *src, size_t src_len, float *dst, size_t n, uint32_t order,
+                                  void *stream) {
+    if (!path_type(t)) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "Unsupported quantization type: %u", t);
+    if (order > PMETAL_HIP_ORDER_GGML) return fail(PMETAL_HIP_ERR_INVALID_ARG, "order must be 0 (REF) or 1 (GGML)");
+    const size_t expected = pmetal_hip_tensor_size(t, n);
+    if (src_len != expected)
+        return fail(PMETAL_HIP_ERR_INVALID_SIZE, "Invalid data size: expected %zu bytes, got %zu", expected, src_len);
+    if (n == 0) return ok();
+    if (!src || !dst) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
+    if (!aligned16(src) || !aligned16(dst)) return fail(PMETAL_HIP_ERR_INVALID_ARG, "device pointers must be 16-byte aligned");
+    if (int32_t rc = require_device()) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    hipError_t e;
+    if (t == PMETAL_GGML_TYPE_Q8_0) e = pmh::launch_dequantize_q8_0(src, n, dst, s);
+    else if (t == PMETAL_GGML_TYPE_Q4K) e = pmh::launch_dequantize_q4k(src, n, dst, order, s);
+    else e = pmh::launch_dequantize_q6k(src, n, dst, s);
+    if (e != hipSuccess) return hip_fail(e, "dequantize kernel launch");
+    return ok();
+}
+
+int32_t pmetal_hip_dequantize(uint32_t t, const uint8_t *src, size_t src_len, const int32_t *shape, size_t ndim,
+                              float *dst, size_t dst_len, uint32_t order) {
+    if (!path_type(t)) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "Unsupported quantization type: %u", t);
+    if (order > PMETAL_HIP_ORDER_GGML) return fail(PMETAL_HIP_ERR_INVALID_ARG, "order must be 0 (REF) or 1 (GGML)");
+    size_t n = 0;
+    if (int32_t rc = shape_elements(shape, ndim, &n)) return rc;
+    const size_t bs = pmetal_hip_block_size(t), ts = pmetal_hip_type_size(t);
+    const size_t blocks = n / bs + (n % bs != 0);
+    if (blocks > SIZE_MAX / ts) return fail(PMETAL_HIP_ERR_SHAPE_TOO_LARGE, "shape is too large");
+    const size_t expected = blocks * ts;
+    if (src_len != expected)
+        return fail(PMETAL_HIP_ERR_INVALID_SIZE, "Invalid data size: expected %zu bytes, got %zu", expected, src_len);
+    if (dst_len < n) return fail(PMETAL_HIP_ERR_INVALID_SIZE, "output holds %zu floats, need %zu", dst_len, n);
+    if (n == 0) return ok();
+    if (!src || !dst) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
+    if (int32_t rc = require_device()) return rc;
+    DevBuf din, dout;
+    HIP_TRY(hipMalloc(&din.p, expected));
+    HIP_TRY(hipMalloc(&dout.p, n * sizeof(float)));
+    HIP_TRY(hipMemcpy(din.p, src, expected, hipMemcpyHostToDevice));
+    if (int32_t rc = pmetal_hip_dequantize_dev(t, (const uint8_t *)din.p, expected, (float *)dout.p, n, order, nullptr))
+        return rc;
+    HIP_TRY(hipMemcpy(dst, dout.p, n * sizeof(float), hipMemcpyDeviceToHost));
+    return ok();
+}
+
+// ---- quantized linear ----
+static int32_t check_linear(uint32_t t, const void *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype,
+                            const void *y, uint32_t order) {
+    if (!path_type(t)) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "Unsupported quantization type: %u", t);
+    if (order > PMETAL_HIP_ORDER_GGML) return fail(PMETAL_HIP_ERR_INVALID_ARG, "order must be 0 (REF) or 1 (GGML)");
+    if (x_dtype > PMETAL_HIP_DTYPE_BF16) return fail(PMETAL_HIP_ERR_INVALID_ARG, "x_dtype must be 0 (f32) or 1 (bf16)");
+    if (n <= 0 || k <= 0) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "n and k must be positive (n=%lld, k=%lld)", (long long)n, (long long)k);
+    const int64_t bs = (int64_t)pmetal_hip_block_size(t);
+    if (k % bs != 0) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "k=%lld is not a multiple of the block size %lld", (long long)k, (long long)bs);
+    if (n > 0x7FFFFFFF || k / bs > 0x7FFFFFF) return fail(PMETAL_HIP_ERR_SHAPE_TOO_LARGE, "n or k too large");
+    if (!w || !x || !y) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
+    if (!aligned16(w) || !aligned16(x) || !aligned16(y))
+        return fail(PMETAL_HIP_ERR_INVALID_ARG, "device pointers must be 16-byte aligned");
+    return require_device();
+}
+
+int32_t pmetal_hip_qgemv(uint32_t t, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, float *y,
+                         uint32_t order, void *stream) {
+    if (int32_t rc = check_linear(t, w, n, k, x, x_dtype, y, order)) return rc;
+    hipError_t e = pmh::launch_qgemv(t, w, n, k, x, x_dtype, y, order, (hipStream_t)stream);
+    if (e == hipErrorInvalidValue)
+        return fail(PMETAL_HIP_ERR_SHAPE_TOO_LARGE, "k=%lld does not fit the activation staging buffer", (long long)k);
+    if (e != hipSuccess) return hip_fail(e, "qgemv kernel launch");
+    return ok();
+}
+
+int32_t pmetal_hip_qgemv_batch(const pmetal_hip_linear_desc *descs, size_t count, void *stream) {
+    if (count && !descs) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL descriptor array");
+    for (size_t i = 0; i < count; i++) {
+        const pmetal_hip_linear_desc &d = descs[i];
+        if (int32_t rc = pmetal_hip_qgemv(d.ggml_type, d.w_dev, d.n, d.k, d.x_dev, d.x_dtype, d.y_dev, d.order, stream))
+            return rc;
+    }
+    return ok();
+}
+
+int32_t pmetal_hip_qgemm(uint32_t t, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, int64_t m,
+                         void *y, uint32_t y_dtype, uint32_t order, void *stream) {
+    if (int32_t rc = check_linear(t, w, n, k, x, x_dtype, y, order)) return rc;
+    if (y_dtype > PMETAL_HIP_DTYPE_BF16) return fail(PMETAL_HIP_ERR_INVALID_ARG, "y_dtype must be 0 (f32) or 1 (bf16)");
+    if (m <= 0 || m > 0x7FFFFFFF) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "m must be in [1, 2^31)");
+    if (t == PMETAL_GGML_TYPE_Q8_0) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "qgemm supports Q4_K and Q6_K weights");
+    void *ws = nullptr;
+    if (int32_t rc = workspace(pmh::qgemm_workspace_bytes(m, k), &ws)) return rc;
+    hipError_t e = pmh::launch_qgemm(t, w, n, k, x, x_dtype, m, y, y_dtype, order, ws, (hipStream_t)stream);
+    if (e == hipErrorNotSupported) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "qgemm: configuration not supported");
+    if (e != hipSuccess) return hip_fail(e, "qgemm kernel launch");
+    return ok();
+}
+
+int32_t pmetal_hip_qlinear(uint32_t t, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, int64_t m,
+                           void *y, uint32_t y_dtype, uint32_t order, void *stream) {
+    if (m == 1 && y_dtype == PMETAL_HIP_DTYPE_F32)
+        return pmetal_hip_qgemv(t, w, n, k, x, x_dtype, (float *)y, order, stream);
+    return pmetal_hip_qgemm(t, w, n, k, x, x_dtype, m, y, y_dtype, order, stream);
+}
+
+// ---- Q4_K_M recipe: crates/pmetal/src/commands/quantize.rs ----
+int32_t pmetal_hip_use_more_bits(size_t layer, size_t n_layers) {  // :988-993
+    if (n_layers == 0) return 0;
+    const size_t eighth = n_layers / 8;
+    const size_t rel = layer >= eighth ? layer - eighth : 0;
+    return (layer < eighth || layer >= 7 * n_layers / 8 || rel % 3 == 2) ? 1 : 0;
+}
+
+int32_t pmetal_hip_is_quantizable_gguf_tensor(const char *name, size_t ndim) {  // :955-980
+    if (!name) return 0;
+    const size_t len = strlen(name);
+    if (!(ndim == 2 || ndim == 3) || len < 7 || strcmp(name + len - 7, ".weight") != 0) return 0;
+    std::string lower(name);
+    for (char &c : lower)
+        if (c >= 'A' && c <= 'Z') c = (char)(c - 'A' + 'a');
+    static const char *const kDense[] = {"_norm.weight", "norm.weight", "ffn_gate_inp.weight", "router", "altup",
+                                         "laurel", "per_layer_model_proj", "pos_embd", "token_types", "ssm_conv1d",
+                                         "shortconv.conv.weight", "attn_rel_b.weight", ".position_embd", ".rel_pos",
+                                         ".patch_embd", ".patch_merger"};
+    for (const char *pat : kDense)
+        if (lower.find(pat) != std::string::npos) return 0;
+    return 1;
+}
+
+uint32_t pmetal_hip_q4km_tensor_type(const char *name, size_t ndim, size_t n_layers) {  // :999-1137, method q4_k_m
+    if (!name || !pmetal_hip_is_quantizable_gguf_tensor(name, ndim)) return PMETAL_GGML_TYPE_F16;
+    const std::string s(name);
+    if (s == "output.weight" || s == "token_embd.weight") return PMETAL_GGML_TYPE_Q6K;
+    size_t layer = 0;  // parse_layer_from_gguf_name :982-986, default 0
+    if (s.rfind("blk.", 0) == 0) {
+        const size_t dot = s.find('.', 4);
+        if (dot != std::string::npos && dot > 4) {
+            size_t i = 4, v = 0;
+            if (s[i] == '+' && dot > 5) i++;
+            bool digits = true;
+            for (size_t q = i; q < dot; q++) {
+                if (s[q] < '0' || s[q] > '9') {
+                    digits = false;
+                    break;
+                }
+                v = v * 10 + (size_t)(s[q] - '0');
+            }
+            if (digits) layer = v;
+        }
+    }
+    const bool more = pmetal_hip_use_more_bits(layer, n_layers) != 0;
+    if (s.find("attn_v.weight") != std::string::npos) return more ? PMETAL_GGML_TYPE_Q6K : PMETAL_GGML_TYPE_Q4K;
+    if (s.find("ffn_down.weight") != std::string::npos || s.find("ffn_down_exps.weight") != std::string::npos)
+        return more ? PMETAL_GGML_TYPE_Q6K : PMETAL_GGML_TYPE_Q4K;
+    if (s.find("attn_output.weight") != std::string::npos) return PMETAL_GGML_TYPE_Q4K;
+    if (s.find("attn_qkv.weight") != std::string::npos) return PMETAL_GGML_TYPE_Q5K;
+    return PMETAL_GGML_TYPE_Q4K;
+}
+
+// ---- synthetic tensors ----
+int32_t pmetal_hip_fill_normal_f32(float *dst, size_t n, uint64_t seed, float std, float outlier_rate, float outlier_mag,
+                                   void *stream) {
+    if (n == 0) return ok();
+    if (!dst) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
+    if (int32_t rc = require_device()) return rc;
+    hipError_t e = pmh::launch_fill_normal(dst, n, seed, std, outlier_rate, outlier_mag, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "fill kernel launch");
+    return ok();
+}
+
+int32_t pmetal_hip_f32_to_bf16_dev(const float *src, uint16_t *dst, size_t n, void *stream) {
+    if (n == 0) return ok();
+    if (!src || !dst) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
+    if (int32_t rc = require_device()) return rc;
+    hipError_t e = pmh::launch_f32_to_bf16(src, dst, n, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "convert kernel launch");
+    return ok();
+}
+
+}  // extern "C"

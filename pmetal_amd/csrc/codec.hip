@@ -1,0 +1,612 @@
+// Bit-exact f32 <-> {Q8_0, Q4_K, Q6_K} kernels for gfx950.
+//
+// The results must equal the reference CPU path bit for bit, so this file is compiled with
+// -ffp-contract=off: every `a * b + c` below is two roundings, as in the Rust it follows
+// (Rust never fuses).  Divisions are IEEE-correct (hipcc's default
+// -fhip-fp32-correctly-rounded-divide-sqrt), rounding is half-away-from-zero done exactly, and
+// every float sum of the two scale searches is accumulated sequentially in element order by ONE
+// lane -- a tree or cross-lane reduction would change the bits.  Only min/max, which are
+// order-independent, are reduced across lanes.
+//
+// Reference functions followed (paths under crates/pmetal-gguf/src/):
+//   quantize.rs:268-300 quantize_q8_0        quantize.rs:583-644 make_qkx1_quants
+//   quantize.rs:738-841 make_qx_quants       k_quants.rs:876-955 quantize_q4k
+//   k_quants.rs:1056-1134 quantize_q6k       dequant.rs:466-495 dequantize_q8_0
+//   k_quants.rs:358-404 dequantize_q4k       k_quants.rs:474-496 dequantize_q6k
+#include "internal.hpp"
+
+#pragma clang fp contract(off)
+
+namespace {
+
+typedef uint32_t u32_a2 __attribute__((aligned(2)));  // dword at a 2-byte aligned address
+typedef uint32_t u32_a1 __attribute__((aligned(1)));
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+}
+
+// half::f16::from_f32: IEEE round-to-nearest-even (v_cvt_f16_f32; f16 denormals are on by default).
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+}
+
+// f32::round: half away from zero.  v - trunc(v) is exact, so this is too.
+__device__ __forceinline__ float round_half_away(float v) {
+    float t = __builtin_truncf(v);
+    float diff = v - t;
+    return (__builtin_fabsf(diff) >= 0.5f) ? t + __builtin_copysignf(1.0f, v) : t;
+}
+
+// clamp(nearest_int(v), lo, hi) with Rust's `as i32` (NaN -> 0, saturating); needs lo <= 0 <= hi.
+__device__ __forceinline__ float clamp_round(float v, float lo, float hi) {
+    float r = round_half_away(v);
+    r = (r != r) ? 0.0f : r;
+    return __builtin_fminf(__builtin_fmaxf(r, lo), hi);
+}
+
+// `v as i32` for f32.
+__device__ __forceinline__ int f32_as_i32(float v) {
+    if (v != v) return 0;
+    if (v >= 2147483648.0f) return 2147483647;
+    if (v <= -2147483648.0f) return -2147483647 - 1;
+    return (int)v;
+}
+
+// f32::total_cmp key: integer order of the keys is the total order of the floats.
+__device__ __forceinline__ int total_key(float v) {
+    int b = __builtin_bit_cast(int, v);
+    return b ^ (int)(((unsigned)(b >> 31)) >> 1);
+}
+
+// -------------------------------------------------------------------------------------------
+// Q8_0 quantize (quantize.rs:268-300).  One lane per 4 elements, 8 lanes per 32-element block.
+// -------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_quantize_q8_0(const float *__restrict__ x, size_t n,
+                                                        uint8_t *__restrict__ dst, size_t n_blocks) {
+    const size_t tid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t blk = tid >> 3;
+    const int j = (int)(tid & 7);
+    const size_t e = tid * 4;
+    float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (e + 3 < n) {
+        float4 t = *reinterpret_cast<const float4 *>(x + e);
+        v[0] = t.x, v[1] = t.y, v[2] = t.z, v[3] = t.w;
+    } else {
+#pragma unroll
+        for (int c = 0; c < 3; c++)
+            if (e + c < n) v[c] = x[e + c];
+    }
+    // amax = fold(0.0, max(|x|)): order-independent, NaN ignored by fmaxf as by f32::max.
+    float a = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v[0]), __builtin_fabsf(v[1])),
+                              __builtin_fmaxf(__builtin_fabsf(v[2]), __builtin_fabsf(v[3])));
+    a = __builtin_fmaxf(a, 0.0f);  // a block of NaNs only folds to 0.0
+    a = __builtin_fmaxf(a, __shfl_xor(a, 1));
+    a = __builtin_fmaxf(a, __shfl_xor(a, 2));
+    a = __builtin_fmaxf(a, __shfl_xor(a, 4));
+    const float scale = a / 127.0f;
+    const float iscale = (a == 0.0f) ? 0.0f : 127.0f / a;
+    uint32_t packed = 0;
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        int q = (int)clamp_round(v[c] * iscale, -127.0f, 127.0f);
+        if (e + c >= n) q = 0;  // zero-pad the partial last block (quantize.rs:293)
+        packed |= ((uint32_t)q & 0xFFu) << (8 * c);
+    }
+    if (blk < n_blocks) {
+        uint8_t *out = dst + blk * 34;
+        *reinterpret_cast<u32_a2 *>(out + 2 + 4 * j) = packed;
+        if (j == 0) *reinterpret_cast<uint16_t *>(out) = (uint16_t)f32_to_f16_bits(scale);
+    }
+}
+
+// -------------------------------------------------------------------------------------------
+// Q8_0 dequantize (dequant.rs:466-495): out = (q as f32) * f16->f32(d).  One lane per 4 outputs.
+// -------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_dequantize_q8_0(const uint8_t *__restrict__ src, size_t n,
+                                                          float *__restrict__ dst) {
+    const size_t tid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t e = tid * 4;
+    if (e >= n) return;
+    const uint8_t *blk = src + (tid >> 3) * 34;
+    const float d = f16_bits_to_f32(*reinterpret_cast<const uint16_t *>(blk));
+    const uint32_t q = *reinterpret_cast<const u32_a2 *>(blk + 2 + 4 * (tid & 7));
+    float o[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) o[c] = (float)(int8_t)(q >> (8 * c)) * d;
+    if (e + 3 < n) {
+        *reinterpret_cast<float4 *>(dst + e) = make_float4(o[0], o[1], o[2], o[3]);
+    } else {
+        for (int c = 0; c < 4 && e + c < n; c++) dst[e + c] = o[c];
+    }
+}
+
+// get_scale_min_k4 (quantize.rs:844-855) on the 12 scale bytes held as three dwords.
+__device__ __forceinline__ void scale_min_k4(int j, uint32_t s0, uint32_t s1, uint32_t s2, uint32_t &sc,
+                                             uint32_t &m) {
+    const int sh = 8 * (j & 3);
+    const uint32_t a = (s0 >> sh) & 0xFFu, b = (s1 >> sh) & 0xFFu, c = (s2 >> sh) & 0xFFu;
+    if (j < 4) {
+        sc = a & 63u;
+        m = b & 63u;
+    } else {
+        sc = (c & 0xFu) | ((a >> 6) << 4);
+        m = (c >> 4) | ((b >> 6) << 4);
+    }
+}
+
+// -------------------------------------------------------------------------------------------
+// Q4_K dequantize (k_quants.rs:358-404 + :515-560).  One lane per 4 outputs, one wave per
+// super-block; out = (d*sc) * nibble - (dmin*m), each operation rounded.
+// ORDER 0: the reference's emission order; ORDER 1: inverse of the quantizer's packing.
+// -------------------------------------------------------------------------------------------
+template <int ORDER>
+__global__ __launch_bounds__(256) void k_dequantize_q4k(const uint8_t *__restrict__ src, size_t n,
+                                                         float *__restrict__ dst) {
+    const size_t tid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t e = tid * 4;
+    if (e >= n) return;
+    const uint8_t *blk = src + (tid >> 6) * 144;
+    const int i = (int)(tid & 63);
+    const int c = i >> 4;       // 64-element chunk
+    const int p = (i & 15) * 4; // position inside the chunk
+    int byte, hi, sb;
+    if (ORDER == 0) {
+        byte = 32 * c + (p & 15) + 16 * (p >> 5);
+        hi = (p >> 4) & 1;
+        sb = 2 * c + (p >> 5);
+    } else {
+        byte = 32 * c + (p & 31);
+        hi = p >> 5;
+        sb = 2 * c + (p >> 5);
+    }
+    const uint4 hdr = *reinterpret_cast<const uint4 *>(blk);
+    const float d = f16_bits_to_f32(hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(hdr.x >> 16);
+    uint32_t sc, m;
+    scale_min_k4(sb, hdr.y, hdr.z, hdr.w, sc, m);
+    const float d1 = d * (float)sc;
+    const float dm1 = dmin * (float)m;
+    uint32_t q = *reinterpret_cast<const uint32_t *>(blk + 16 + byte);
+    q = hi ? (q >> 4) : q;
+    float o[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) o[t] = d1 * (float)((q >> (8 * t)) & 0xFu) - dm1;
+    if (e + 3 < n) {
+        *reinterpret_cast<float4 *>(dst + e) = make_float4(o[0], o[1], o[2], o[3]);
+    } else {
+        for (int t = 0; t < 4 && e + t < n; t++) dst[e + t] = o[t];
+    }
+}
+
+// -------------------------------------------------------------------------------------------
+// Q6_K dequantize (k_quants.rs:474-496 + :614-660): out = (d * sc) * q, left-associated.
+// -------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_dequantize_q6k(const uint8_t *__restrict__ src, size_t n,
+                                                         float *__restrict__ dst) {
+    const size_t tid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t e = tid * 4;
+    if (e >= n) return;
+    const uint8_t *blk = src + (tid >> 6) * 210;
+    const int i = (int)(tid & 63);
+    const int h = i >> 5;         // 128-element half
+    const int g = (i >> 3) & 3;   // 32-element group inside the half
+    const int l = (i & 7) * 4;    // 0..28
+    const uint32_t qlw = *reinterpret_cast<const u32_a2 *>(blk + 64 * h + 32 * (g & 1) + l);
+    const uint32_t qhw = *reinterpret_cast<const u32_a2 *>(blk + 128 + 32 * h + l);
+    const float sc = (float)(int8_t)blk[192 + 8 * h + 2 * g + (l >> 4)];
+    const float d = f16_bits_to_f32(*reinterpret_cast<const uint16_t *>(blk + 208));
+    const float dsc = d * sc;
+    const uint32_t nib = (g >= 2) ? (qlw >> 4) : qlw;
+    const uint32_t hi2 = qhw >> (2 * g);
+    float o[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        int q = (int)(((nib >> (8 * t)) & 0xFu) | (((hi2 >> (8 * t)) & 3u) << 4)) - 32;
+        o[t] = dsc * (float)q;
+    }
+    if (e + 3 < n) {
+        *reinterpret_cast<float4 *>(dst + e) = make_float4(o[0], o[1], o[2], o[3]);
+    } else {
+        for (int t = 0; t < 4 && e + t < n; t++) dst[e + t] = o[t];
+    }
+}
+
+// -------------------------------------------------------------------------------------------
+// Q4_K quantize (k_quants.rs:876-955).  One wave per 8 super-blocks: lane L owns sub-block L
+// (32 elements) of the 64 sub-blocks, runs make_qkx1_quants (quantize.rs:583-644) sequentially in
+// registers, then the 8 lanes of a super-block agree on d/dmin, pack the 6-bit scales, requantize
+// and emit 16 bytes of nibbles each.
+// -------------------------------------------------------------------------------------------
+constexpr int kQ4kLdsStride = 33;  // 32 floats + 1 pad: lanes read column-wise without bank conflicts
+
+__global__ __launch_bounds__(64) void k_quantize_q4k(const float *__restrict__ x, size_t n_sb,
+                                                      uint8_t *__restrict__ dst) {
+    __shared__ float xs[64 * kQ4kLdsStride];
+    const int lane = threadIdx.x;
+    const size_t sb0 = (size_t)blockIdx.x * 8;
+    const size_t n_valid = (n_sb - sb0 < 8 ? n_sb - sb0 : 8) * 256;  // floats this wave may read
+    const float *src = x + sb0 * 256;
+#pragma unroll
+    for (int it = 0; it < 8; it++) {
+        const int idx = it * 64 + lane;  // float4 index inside the 2048-float tile
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if ((size_t)idx * 4 < n_valid) v = *reinterpret_cast<const float4 *>(src + idx * 4);
+        float *p = xs + (idx >> 3) * kQ4kLdsStride + (idx & 7) * 4;
+        p[0] = v.x, p[1] = v.y, p[2] = v.z, p[3] = v.w;
+    }
+    __syncthreads();
+    float xv[32];
+#pragma unroll
+    for (int i = 0; i < 32; i++) xv[i] = xs[lane * kQ4kLdsStride + i];
+
+    // ---- make_qkx1_quants(15, 5, xv) ----
+    float mn = xv[0], mx = xv[0];
+#pragma unroll
+    for (int i = 1; i < 32; i++) {
+        if (total_key(mn) > total_key(xv[i])) mn = xv[i];
+        if (total_key(mx) <= total_key(xv[i])) mx = xv[i];
+    }
+    float scale = 0.0f, neg_min = 0.0f;  // returned (scale, -min)
+    if (!(mx == mn)) {
+        float minv = __builtin_fminf(mn, 0.0f);
+        float iscale = 15.0f / (mx - minv);
+        scale = 1.0f / iscale;
+        uint32_t lp[8] = {0, 0, 0, 0, 0, 0, 0, 0};  // previous quants, 4 per dword
+        for (int t = 0; t < 5; t++) {
+            float lf[32];
+            float sumlx = 0.0f, suml2 = 0.0f;  // suml2 is an integer <= 7200: exact in f32
+            bool changed = false;
+#pragma unroll
+            for (int w = 0; w < 8; w++) {
+                uint32_t word = 0;
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    const int i = 4 * w + c;
+                    const float xm = xv[i] - minv;
+                    const float v = iscale * xm;
+                    // clamp(nearest_int(v), 0, 15): for v < 0 any rounding clamps to 0
+                    const float tr = __builtin_truncf(v);
+                    float r = (v - tr >= 0.5f) ? tr + 1.0f : tr;
+                    r = __builtin_fminf(__builtin_fmaxf(r, 0.0f), 15.0f);  // NaN -> 0
+                    lf[i] = r;
+                    sumlx += xm * r;
+                    suml2 += r * r;
+                    word |= (uint32_t)r << (8 * c);
+                }
+                changed |= (word != lp[w]);
+                lp[w] = word;
+            }
+            if (suml2 == 0.0f) break;
+            scale = sumlx / suml2;
+            float sum = -0.0f;  // Iterator::sum::<f32> folds from -0.0
+#pragma unroll
+            for (int i = 0; i < 32; i++) sum += xv[i] - scale * lf[i];
+            minv = sum / 32.0f;
+            if (minv > 0.0f) minv = 0.0f;
+            iscale = 1.0f / scale;
+            if (!changed) break;
+        }
+        neg_min = -minv;
+    }
+
+    // ---- super-block level (k_quants.rs:904-929): the 8 lanes of a super-block cooperate ----
+    float max_scale = scale, max_min = neg_min;
+#pragma unroll
+    for (int off = 1; off < 8; off <<= 1) {
+        max_scale = __builtin_fmaxf(max_scale, __shfl_xor(max_scale, off));
+        max_min = __builtin_fmaxf(max_min, __shfl_xor(max_min, off));
+    }
+    // fold(0.0, max): the fold starts from +0.0, and +0.0 orders above -0.0 on the reference's target
+    max_scale = __builtin_fmaxf(max_scale, 0.0f);
+    max_min = __builtin_fmaxf(max_min, 0.0f);
+    if (max_scale == 0.0f) max_scale = 0.0f;
+    if (max_min == 0.0f) max_min = 0.0f;
+    const float inv_scale = max_scale > 0.0f ? 63.0f / max_scale : 0.0f;
+    const float inv_min = max_min > 0.0f ? 63.0f / max_min : 0.0f;
+    int a = f32_as_i32(round_half_away(inv_scale * scale));
+    int b = f32_as_i32(round_half_away(inv_min * neg_min));
+    const uint32_t ls8 = (uint32_t)(a < 63 ? a : 63) & 0xFFu;  // `.min(63) as u8`
+    const uint32_t lm8 = (uint32_t)(b < 63 ? b : 63) & 0xFFu;
+    const int j = lane & 7;
+    // partner sub-block j^4 supplies / receives the two high bits
+    const uint32_t ls8_p = __shfl_xor(ls8, 4), lm8_p = __shfl_xor(lm8, 4);
+    // bytes of the 12-byte scale field this lane produces (k_quants.rs:915-926)
+    //   j < 4 : scales[j]   = ls_j | (ls_{j+4} >> 4) << 6 ; scales[j+4] = lm_j | (lm_{j+4} >> 4) << 6
+    //   j >= 4: scales[j+4] = (ls_j & 0xF) | (lm_j & 0xF) << 4
+    uint32_t byte_a, byte_b = 0;
+    uint32_t sc, m;  // get_scale_min_k4(j, scales)
+    if (j < 4) {
+        byte_a = (ls8 | ((ls8_p >> 4) << 6)) & 0xFFu;
+        byte_b = (lm8 | ((lm8_p >> 4) << 6)) & 0xFFu;
+        sc = byte_a & 63u;
+        m = byte_b & 63u;
+    } else {
+        byte_a = ((ls8 & 0xFu) | ((lm8 & 0xFu) << 4)) & 0xFFu;
+        const uint32_t lo_a = (ls8_p | ((ls8 >> 4) << 6)) & 0xFFu;  // scales[j-4]
+        const uint32_t lo_b = (lm8_p | ((lm8 >> 4) << 6)) & 0xFFu;  // scales[j]
+        sc = (byte_a & 0xFu) | ((lo_a >> 6) << 4);
+        m = (byte_a >> 4) | ((lo_b >> 6) << 4);
+    }
+    const uint32_t d16 = f32_to_f16_bits(max_scale / 63.0f);
+    const uint32_t dmin16 = f32_to_f16_bits(max_min / 63.0f);
+
+    // ---- requantize with the decoded f16 scales (k_quants.rs:932-943) ----
+    uint32_t lb[8] = {0, 0, 0, 0, 0, 0, 0, 0};  // 32 quants, one per byte
+    const float dq = f16_bits_to_f32(d16) * (float)sc;
+    if (dq != 0.0f) {
+        const float dm = f16_bits_to_f32(dmin16) * (float)m;
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const float r = clamp_round((xv[4 * w + c] + dm) / dq, 0.0f, 15.0f);
+                lb[w] |= (uint32_t)r << (8 * c);
+            }
+        }
+    }
+    // ---- pack (k_quants.rs:946-951): qs[32c + l] = L[64c + l] | L[64c + l + 32] << 4 ----
+    // Even sub-block 2c supplies the low nibbles, odd 2c+1 the high ones.  The even lane emits bytes
+    // l = 0..15 of the pair, the odd lane bytes 16..31.
+    const bool odd = lane & 1;
+    uint32_t outw[4];
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+        const uint32_t send = odd ? lb[w] : lb[4 + w];
+        const uint32_t recv = __shfl_xor(send, 1);
+        outw[w] = odd ? (recv | (lb[4 + w] << 4)) : (lb[w] | (recv << 4));
+    }
+    const size_t sb = sb0 + (lane >> 3);
+    if (sb < n_sb) {
+        uint8_t *blk = dst + sb * 144;
+        *reinterpret_cast<uint4 *>(blk + 16 + 16 * j) = make_uint4(outw[0], outw[1], outw[2], outw[3]);
+        if (j < 4) {
+            blk[4 + j] = (uint8_t)byte_a;
+            blk[8 + j] = (uint8_t)byte_b;
+        } else {
+            blk[8 + j] = (uint8_t)byte_a;
+        }
+        if (j == 0) *reinterpret_cast<uint32_t *>(blk) = d16 | (dmin16 << 16);
+    }
+}
+
+// -------------------------------------------------------------------------------------------
+// Q6_K quantize (k_quants.rs:1056-1134).  One wave per 4 super-blocks: lane L owns the 16-element
+// sub-block L of the 64, runs make_qx_quants(16, 32, x, 1) (quantize.rs:738-841) sequentially,
+// then the 16 lanes of a super-block pick max_scale, requantize and assemble ql/qh through LDS.
+// -------------------------------------------------------------------------------------------
+constexpr int kQ6kLdsStride = 17;
+
+__global__ __launch_bounds__(64) void k_quantize_q6k(const float *__restrict__ x, size_t n_sb,
+                                                      uint8_t *__restrict__ dst) {
+    __shared__ float xs[64 * kQ6kLdsStride];
+    __shared__ uint32_t lbuf[4 * 64];   // final 6-bit values, one per byte, 256 per super-block
+    __shared__ __attribute__((aligned(16))) uint16_t obuf[4 * 105];  // the 4 output blocks (210 bytes each)
+    const int lane = threadIdx.x;
+    const size_t sb0 = (size_t)blockIdx.x * 4;
+    const size_t n_here = n_sb - sb0 < 4 ? n_sb - sb0 : 4;
+    const size_t n_valid = n_here * 256;
+    const float *src = x + sb0 * 256;
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int idx = it * 64 + lane;  // float4 index inside the 1024-float tile
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if ((size_t)idx * 4 < n_valid) v = *reinterpret_cast<const float4 *>(src + idx * 4);
+        float *p = xs + (idx >> 2) * kQ6kLdsStride + (idx & 3) * 4;
+        p[0] = v.x, p[1] = v.y, p[2] = v.z, p[3] = v.w;
+    }
+    __syncthreads();
+    float xv[16], wx[16], w[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        xv[i] = xs[lane * kQ6kLdsStride + i];
+        w[i] = xv[i] * xv[i];
+        wx[i] = w[i] * xv[i];
+    }
+
+    // ---- make_qx_quants(16, 32, xv, rmse_type = 1) ----
+    float l[16];  // signed quants l in [-32, 31]; ls = l + 32
+    float maxv = 0.0f, amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const float ax = __builtin_fabsf(xv[i]);
+        if (ax > amax) {
+            amax = ax;
+            maxv = xv[i];
+        }
+    }
+    float scale = 0.0f;
+    bool zero_block = (amax == 0.0f);  // returns (0.0, ls = all zero): l + 32 == 0
+#pragma unroll
+    for (int i = 0; i < 16; i++) l[i] = -32.0f;
+    if (!zero_block) {
+        const float iscale0 = -32.0f / maxv;
+        float sumlx = 0.0f, suml2 = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            l[i] = clamp_round(iscale0 * xv[i], -32.0f, 31.0f);
+            sumlx += wx[i] * l[i];
+            suml2 += w[i] * (l[i] * l[i]);
+        }
+        scale = sumlx / suml2;
+        float best = scale * sumlx;
+        for (int t = 0; t < 3; t++) {
+            const float isc = 1.0f / scale;
+            float slx = 0.0f, sl2 = 0.0f;
+            bool changed = false;
+            float nl[16];
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                nl[i] = clamp_round(isc * xv[i], -32.0f, 31.0f);
+                changed |= (nl[i] != l[i]);
+                slx += wx[i] * nl[i];
+                sl2 += w[i] * (nl[i] * nl[i]);
+            }
+            if (!changed || sl2 == 0.0f || slx * slx <= best * sl2) break;
+#pragma unroll
+            for (int i = 0; i < 16; i++) l[i] = nl[i];
+            sumlx = slx;
+            suml2 = sl2;
+            scale = sumlx / suml2;
+            best = scale * sumlx;
+        }
+        for (int t = 0; t < 5; t++) {
+            int n_changed = 0;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                float slx = sumlx - wx[i] * l[i];
+                if (slx > 0.0f) {
+                    float sl2 = suml2 - w[i] * (l[i] * l[i]);
+                    const float new_l = clamp_round(xv[i] * sl2 / slx, -32.0f, 31.0f);
+                    if (new_l != l[i]) {
+                        slx += wx[i] * new_l;
+                        sl2 += w[i] * (new_l * new_l);
+                        if (sl2 > 0.0f && slx * slx * suml2 > sumlx * sumlx * sl2) {
+                            l[i] = new_l;
+                            sumlx = slx;
+                            suml2 = sl2;
+                            scale = sumlx / suml2;
+                            n_changed++;
+                        }
+                    }
+                }
+            }
+            if (n_changed == 0) break;
+        }
+    }
+
+    // ---- super-block level (k_quants.rs:1082-1102) ----
+    // max_scale = scale of the first sub-block attaining the largest |scale| (strict > in a forward
+    // scan); |scale| of NaN never wins.
+    const float abs_scale = __builtin_fabsf(scale);
+    float gmax = (abs_scale == abs_scale) ? abs_scale : 0.0f;
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) gmax = __builtin_fmaxf(gmax, __shfl_xor(gmax, off));
+    const unsigned long long hit = __ballot(abs_scale == gmax && gmax > 0.0f);
+    const int grp = lane & ~15;
+    const unsigned long long ghit = (hit >> grp) & 0xFFFFull;
+    const int first = ghit ? (__builtin_ctzll(ghit) + grp) : lane;
+    float max_scale = __shfl(scale, first);
+    if (!ghit) max_scale = 0.0f;
+    const float iscale = -128.0f / max_scale;
+    const uint32_t d16 = f32_to_f16_bits(1.0f / iscale);
+    int sq = f32_as_i32(round_half_away(iscale * scale));
+    sq = sq < 127 ? sq : 127;
+    const int8_t s8 = (int8_t)(uint8_t)(uint32_t)sq;  // `.min(127) as i8` wraps
+
+    // ---- requantize (k_quants.rs:1105-1113) ----
+    const float dq = f16_bits_to_f32(d16) * (float)s8;
+    uint32_t lw[4] = {0, 0, 0, 0};
+    if (dq != 0.0f) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const float ll = clamp_round(xv[i] / dq, -32.0f, 31.0f);
+            lw[i >> 2] |= (uint32_t)(int)(ll + 32.0f) << (8 * (i & 3));
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const float keep = zero_block ? 0.0f : l[i] + 32.0f;  // make_qx_quants' own ls
+            lw[i >> 2] |= (uint32_t)(int)keep << (8 * (i & 3));
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < 4; q++) lbuf[lane * 4 + q] = lw[q];
+    __syncthreads();
+
+    // ---- pack ql / qh (k_quants.rs:1116-1130) into obuf; 16 lanes per super-block ----
+    const int sbl = lane >> 4;  // local super-block
+    const int t = lane & 15;
+    const uint32_t *L32 = lbuf + sbl * 64;
+    uint16_t *ob = obuf + sbl * 105;
+#pragma unroll
+    for (int r = 0; r < 2; r++) {
+        const int q = t * 2 + r;  // ql dword 0..31: bytes 4q..4q+3
+        const int base = 32 * (q >> 4) + (q & 15);
+        const uint32_t lo = L32[base], hi = L32[base + 16];
+        const uint32_t v = (lo & 0x0F0F0F0Fu) | ((hi & 0x0F0F0F0Fu) << 4);
+        ob[2 * q] = (uint16_t)v;
+        ob[2 * q + 1] = (uint16_t)(v >> 16);
+    }
+    {
+        const int p = t;  // qh dword 0..15
+        const int base = 32 * (p >> 3) + (p & 7);
+        const uint32_t a4 = (L32[base] >> 4) & 0x03030303u, b4 = (L32[base + 8] >> 4) & 0x03030303u;
+        const uint32_t c4 = (L32[base + 16] >> 4) & 0x03030303u, e4 = (L32[base + 24] >> 4) & 0x03030303u;
+        const uint32_t v = a4 | (b4 << 2) | (c4 << 4) | (e4 << 6);
+        ob[64 + 2 * p] = (uint16_t)v;
+        ob[64 + 2 * p + 1] = (uint16_t)(v >> 16);
+    }
+    {
+        // scales: 16 signed bytes; two lanes share a u16
+        const uint32_t mine = (uint32_t)(uint8_t)s8;
+        const uint32_t other = __shfl_xor(mine, 1);
+        if ((t & 1) == 0) ob[96 + (t >> 1)] = (uint16_t)(mine | (other << 8));
+        if (t == 0) ob[104] = (uint16_t)d16;
+    }
+    __syncthreads();
+    // ---- coalesced store of the n_here * 210 bytes (the tile starts 8-byte aligned) ----
+    uint8_t *out = dst + sb0 * 210;
+    const uint32_t *ob32 = reinterpret_cast<const uint32_t *>(obuf);
+    const int n_u16 = (int)n_here * 105;
+    for (int i = lane; i < n_u16 / 2; i += 64) reinterpret_cast<uint32_t *>(out)[i] = ob32[i];
+    if ((n_u16 & 1) && lane == 0) reinterpret_cast<uint16_t *>(out)[n_u16 - 1] = obuf[n_u16 - 1];
+}
+
+inline unsigned grid_for(size_t work_items, size_t per_block) {
+    return (unsigned)((work_items + per_block - 1) / per_block);
+}
+
+}  // namespace
+
+namespace pmh {
+
+hipError_t launch_quantize_q8_0(const float *x, size_t n, uint8_t *dst, hipStream_t s) {
+    const size_t n_blocks = (n + 31) / 32;
+    if (n_blocks == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_quantize_q8_0, dim3(grid_for(n_blocks * 8, 256)), dim3(256), 0, s, x, n, dst, n_blocks);
+    return hipGetLastError();
+}
+
+hipError_t launch_quantize_q4k(const float *x, size_t n, uint8_t *dst, hipStream_t s) {
+    const size_t n_sb = n / 256;  // full super-blocks; a trailing partial one is zero bytes
+    if (n % 256) {
+        hipError_t e = launch_zero_bytes(dst + n_sb * 144, 144, s);
+        if (e != hipSuccess) return e;
+    }
+    if (n_sb == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_quantize_q4k, dim3(grid_for(n_sb, 8)), dim3(64), 0, s, x, n_sb, dst);
+    return hipGetLastError();
+}
+
+hipError_t launch_quantize_q6k(const float *x, size_t n, uint8_t *dst, hipStream_t s) {
+    const size_t n_sb = n / 256;
+    if (n % 256) {
+        hipError_t e = launch_zero_bytes(dst + n_sb * 210, 210, s);
+        if (e != hipSuccess) return e;
+    }
+    if (n_sb == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_quantize_q6k, dim3(grid_for(n_sb, 4)), dim3(64), 0, s, x, n_sb, dst);
+    return hipGetLastError();
+}
+
+hipError_t launch_dequantize_q8_0(const uint8_t *src, size_t n, float *dst, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_dequantize_q8_0, dim3(grid_for((n + 3) / 4, 256)), dim3(256), 0, s, src, n, dst);
+    return hipGetLastError();
+}
+
+hipError_t launch_dequantize_q4k(const uint8_t *src, size_t n, float *dst, uint32_t order, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    const dim3 grid(grid_for((n + 3) / 4, 256));
+    if (order == kOrderRef) hipLaunchKernelGGL(k_dequantize_q4k<0>, grid, dim3(256), 0, s, src, n, dst);
+    else hipLaunchKernelGGL(k_dequantize_q4k<1>, grid, dim3(256), 0, s, src, n, dst);
+    return hipGetLastError();
+}
+
+hipError_t launch_dequantize_q6k(const uint8_t *src, size_t n, float *dst, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_dequantize_q6k, dim3(grid_for((n + 3) / 4, 256)), dim3(256), 0, s, src, n, dst);
+    return hipGetLastError();
+}
+
+}  // namespace pmh

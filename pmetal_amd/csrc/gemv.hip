@@ -1,0 +1,380 @@
+// Dequant-fused GEMV  y[n] = sum_k W[n,k] * x[k]  for Q6_K and Q8_0 weights on gfx950, and the
+// dispatch over weight types (Q4_K lives in gemv_q4k.hip).
+//
+// W is the packed GGUF block stream, row-major [n, k]; the value of a weight is what the
+// reference's dequantize yields (k_quants.rs:474-496 for Q6_K, dequant.rs:466-495 for Q8_0).  The
+// reference has no fused kernel: it dequantizes on the CPU at load
+// (crates/pmetal-models/src/weight_format.rs:299) and multiplies dense; these kernels are checked
+// against exactly that (dequantize, then matmul), to 1e-3.
+//
+//  * A "team" of T lanes walks one weight row at a time; for Q6_K 8 lanes share a 210-byte
+//    super-block, for Q8_0 one lane owns a 34-byte block.  Blocks are only 2-byte aligned, so the
+//    loads are unaligned dword loads, which the hardware supports.
+//  * Q6_K quants are assembled in registers into bf16 pairs: OR-ing the integer q' = q + 32 (shifted
+//    by one) into the mantissa of bf16(64.0) gives exactly 64 + q', and one v_dot2c_f32_bf16
+//    multiplies two of them with two activations, accumulating in fp32.  The offsets are removed
+//    with per-group sums of x computed once.
+//  * x is staged once per workgroup in LDS, already permuted into the pair order the unpacking
+//    produces, laid out so that consecutive lanes read consecutive 16-byte words.  f32 activations
+//    are split exactly into three bf16 planes (hi + mid + lo) and run through the same path thrice.
+//  * The team's partial sums are reduced with DPP (quad_perm, row_half_mirror, row_mirror) and, for
+//    teams wider than a 16-lane row, ds_bpermute; lane 0 of the team stores y[row].
+#include "gemv_common.hpp"
+
+namespace {
+
+using namespace pmh::gemv;
+
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef uint32_t u32_a2 __attribute__((aligned(2)));
+typedef uint16_t u16_a2 __attribute__((aligned(2)));
+struct __attribute__((packed, aligned(2))) u32x2_a2 {
+    uint32_t x, y;
+};
+struct __attribute__((packed, aligned(2))) u32x4_a2 {
+    uint32_t x, y, z, w;
+};
+
+// Integer -> bf16 without a conversion: OR the integer into the mantissa of a power of two whose ulp is
+// <= 1.  bf16(16.0) has ulp 1/8, so 0x4180 | (q << 3) is exactly 16 + q for q < 16; bf16(64.0) has ulp
+// 1/2, so 0x4280 | (q << 1) is exactly 64 + q for q < 64.  The smallest usable offset keeps the
+// cancellation error of "dot - offset * sum(x)" small.
+constexpr uint32_t kBf16_64 = 0x42804280u;
+
+__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c,
+                                           false);
+}
+
+// Split an f32 into three bf16 terms hi + mid + lo; 3 x 8 significant bits hold all 24 bits of the
+// f32, so the sum is exact (barring underflow of the low terms).
+__device__ __forceinline__ void split3(float f, uint32_t &h, uint32_t &m, uint32_t &l) {
+    h = bf16_rne(f);
+    const float r1 = f - bf16_to_f32(h);
+    m = bf16_rne(r1);
+    l = bf16_rne(r1 - bf16_to_f32(m));
+}
+
+// Load NE (8 or 16) consecutive activations starting at element `e` as PLANES planes of NE/2 packed
+// bf16 pairs p[i] = elem 2i | elem 2i+1 << 16 (bf16 input: one plane; f32 input: three planes whose
+// sum is the input), and return their f32 sum.
+template <bool XF32, int NE>
+__device__ __forceinline__ float load_x(const void *xg, size_t e, uint32_t (&pl)[3][NE / 2]) {
+    float sum = 0.0f;
+    if (XF32) {
+        const float4 *p = reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(xg) + e);
+#pragma unroll
+        for (int q = 0; q < NE / 4; q++) {
+            const float4 v = p[q];
+            const float f[4] = {v.x, v.y, v.z, v.w};
+            uint32_t h[4], m[4], l[4];
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                split3(f[c], h[c], m[c], l[c]);
+                sum += f[c];
+            }
+            pl[0][2 * q] = h[0] | (h[1] << 16), pl[0][2 * q + 1] = h[2] | (h[3] << 16);
+            pl[1][2 * q] = m[0] | (m[1] << 16), pl[1][2 * q + 1] = m[2] | (m[3] << 16);
+            pl[2][2 * q] = l[0] | (l[1] << 16), pl[2][2 * q + 1] = l[2] | (l[3] << 16);
+        }
+    } else {
+        const uint4 *p = reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(xg) + e);
+#pragma unroll
+        for (int q = 0; q < NE / 8; q++) {
+            const uint4 a = p[q];
+            pl[0][4 * q] = a.x, pl[0][4 * q + 1] = a.y, pl[0][4 * q + 2] = a.z, pl[0][4 * q + 3] = a.w;
+        }
+#pragma unroll
+        for (int i = 0; i < NE / 2; i++) {
+            pl[1][i] = pl[2][i] = 0;
+            sum += bf16_to_f32(pl[0][i] & 0xFFFFu) + bf16_to_f32(pl[0][i] >> 16);
+        }
+    }
+    return sum;
+}
+
+// From packed (e0|e1), (e2|e3) make the pairs the unpacking produces: (e0|e2) and (e1|e3).
+__device__ __forceinline__ void even_odd_pairs(uint32_t p0, uint32_t p1, uint32_t &ev, uint32_t &od) {
+    ev = (p0 & 0xFFFFu) | (p1 << 16);
+    od = (p0 >> 16) | (p1 & 0xFFFF0000u);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Q6_K (210-byte super-blocks, only 2-byte aligned).  Lane t of a super-block: half h = t / 4,
+// l in [8(t%4), 8(t%4)+8); for each of the 4 groups g it owns elements 128h + 32g + l.
+// LDS: xl[PLANES][4][slots] uint4 (index g: pairs (l0,l2) (l1,l3) (l4,l6) (l5,l7)) then xs[slots]
+// float4 (per-group sums of x).
+// ------------------------------------------------------------------------------------------------
+template <int PLANES, bool XF32>
+__device__ __forceinline__ void stage_x_q6k(const void *xg, int spr, uint4 *xl, float4 *xs) {
+    const int slots = spr * 8;
+    for (int slot = threadIdx.x; slot < slots; slot += blockDim.x) {
+        const int s = slot >> 3, t = slot & 7;
+        const int base = 128 * (t >> 2) + 8 * (t & 3);
+        float sums[4];
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            uint32_t pl[3][4];
+            sums[g] = load_x<XF32, 8>(xg, (size_t)s * 256 + base + 32 * g, pl);
+#pragma unroll
+            for (int p = 0; p < PLANES; p++) {
+                uint4 v;
+                even_odd_pairs(pl[p][0], pl[p][1], v.x, v.y);
+                even_odd_pairs(pl[p][2], pl[p][3], v.z, v.w);
+                xl[(p * 4 + g) * slots + slot] = v;
+            }
+        }
+        xs[slot] = make_float4(sums[0], sums[1], sums[2], sums[3]);
+    }
+}
+
+template <int PLANES>
+__device__ __forceinline__ float q6k_lane(const uint8_t *blk, const int t, const uint4 *xl, const int slots,
+                                          const int slot, const float4 xsum) {
+    const int h = t >> 2, lq = (t & 3) * 8;
+    const u32x2_a2 qla = *reinterpret_cast<const u32x2_a2 *>(blk + 64 * h + lq);
+    const u32x2_a2 qlb = *reinterpret_cast<const u32x2_a2 *>(blk + 64 * h + 32 + lq);
+    const u32x2_a2 qh = *reinterpret_cast<const u32x2_a2 *>(blk + 128 + 32 * h + lq);
+    const u32x2_a2 sc8 = *reinterpret_cast<const u32x2_a2 *>(blk + 192 + 8 * h);
+    const float d = f16_bits_to_f32(*reinterpret_cast<const u16_a2 *>(blk + 208));
+    const uint32_t la[2] = {qla.x, qla.y}, lb[2] = {qlb.x, qlb.y}, hh[2] = {qh.x, qh.y};
+    const float xs4[4] = {xsum.x, xsum.y, xsum.z, xsum.w};
+    const int shalf = lq >> 4;  // which of the two 16-element scale slots of a group
+    float total = 0.0f;
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        uint32_t v[2];
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+            const uint32_t nib = ((g & 1) ? lb[r] : la[r]) >> (g >= 2 ? 4 : 0);
+            const uint32_t hi2 = g == 0 ? (hh[r] << 4) : g == 1 ? (hh[r] << 2) : g == 2 ? hh[r] : (hh[r] >> 2);
+            v[r] = (nib & 0x0F0F0F0Fu) | (hi2 & 0x30303030u);  // four 6-bit values q + 32
+        }
+        const uint32_t a0 = ((v[0] << 1) & 0x007E007Eu) | kBf16_64, b0 = ((v[0] >> 7) & 0x007E007Eu) | kBf16_64;
+        const uint32_t a1 = ((v[1] << 1) & 0x007E007Eu) | kBf16_64, b1 = ((v[1] >> 7) & 0x007E007Eu) | kBf16_64;
+        float dot = 0.0f;
+#pragma unroll
+        for (int p = 0; p < PLANES; p++) {
+            const uint4 xv = xl[(p * 4 + g) * slots + slot];
+            dot = dot2(a0, xv.x, dot);
+            dot = dot2(b0, xv.y, dot);
+            dot = dot2(a1, xv.z, dot);
+            dot = dot2(b1, xv.w, dot);
+        }
+        const int si = 2 * g + shalf;  // scale byte inside this half's 8
+        const uint32_t sw = si < 4 ? sc8.x : sc8.y;
+        const float sc = (float)(int8_t)(sw >> (8 * (si & 3)));
+        total += sc * (dot - 96.0f * xs4[g]);  // stored value is q + 32 and the bf16 trick adds 64
+    }
+    return d * total;
+}
+
+template <int T, bool XF32>
+__global__ __launch_bounds__(256) void k_qgemv_q6k(const uint8_t *__restrict__ W, const void *__restrict__ xg,
+                                                    float *__restrict__ y, int n_rows, int spr) {
+    constexpr int PLANES = XF32 ? 3 : 1;
+    constexpr int SEG = T / 8;
+    extern __shared__ uint4 smem[];
+    const int slots = spr * 8;
+    uint4 *xl = smem;
+    float4 *xs = reinterpret_cast<float4 *>(xl + PLANES * 4 * slots);
+    stage_x_q6k<PLANES, XF32>(xg, spr, xl, xs);
+    __syncthreads();
+
+    const int lt = threadIdx.x & (T - 1);
+    const int t = lt & 7;
+    const int team = blockIdx.x * (256 / T) + threadIdx.x / T;
+    const int n_teams = gridDim.x * (256 / T);
+    const int iters = spr / SEG;
+    const size_t row_bytes = (size_t)spr * 210;
+    const size_t lane_off = (size_t)(lt >> 3) * 210;
+
+    for (int row = team; row < n_rows; row += 2 * n_teams) {
+        const int row1 = row + n_teams;
+        const bool has1 = row1 < n_rows;
+        const uint8_t *p0 = W + (size_t)row * row_bytes + lane_off;
+        const uint8_t *p1 = W + (size_t)(has1 ? row1 : row) * row_bytes + lane_off;
+        float acc0 = 0.0f, acc1 = 0.0f;
+        for (int it = 0; it < iters; it++) {
+            const size_t o = (size_t)it * SEG * 210;
+            const int slot = it * T + lt;
+            const float4 xsum = xs[slot];
+            acc0 += q6k_lane<PLANES>(p0 + o, t, xl, slots, slot, xsum);
+            acc1 += q6k_lane<PLANES>(p1 + o, t, xl, slots, slot, xsum);
+        }
+        acc0 = team_sum<T>(acc0);
+        acc1 = team_sum<T>(acc1);
+        if (lt == 0) {
+            y[row] = acc0;
+            if (has1) y[row1] = acc1;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Q8_0 (34-byte blocks of 32, 2-byte aligned).  One lane per block; 8-bit quants do not fit the
+// bf16 mantissa trick, so each is sign-extended, converted and multiplied in fp32 with x held as f32
+// in LDS (at 8.5 bits per weight the VALU budget per byte is twice that of Q4_K).
+// LDS: xf[8][blocks] float4 (elements 32b + 4q .. +3).
+// ------------------------------------------------------------------------------------------------
+template <bool XF32>
+__device__ __forceinline__ void stage_x_q8_0(const void *xg, int bpr, float4 *xf) {
+    for (int b = threadIdx.x; b < bpr; b += blockDim.x) {
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            float4 v;
+            if (XF32) {
+                v = reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(xg) + (size_t)b * 32)[q];
+            } else {
+                const uint2 u =
+                    reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(xg) + (size_t)b * 32)[q];
+                v = make_float4(bf16_to_f32(u.x & 0xFFFFu), bf16_to_f32(u.x >> 16), bf16_to_f32(u.y & 0xFFFFu),
+                                bf16_to_f32(u.y >> 16));
+            }
+            xf[q * bpr + b] = v;
+        }
+    }
+}
+
+__device__ __forceinline__ float q8_0_lane(const uint8_t *blk, const float4 *xf, const int bpr, const int b) {
+    const float d = f16_bits_to_f32(*reinterpret_cast<const u16_a2 *>(blk));
+    const u32x4_a2 qa = *reinterpret_cast<const u32x4_a2 *>(blk + 2);
+    const u32x4_a2 qb = *reinterpret_cast<const u32x4_a2 *>(blk + 18);
+    const uint32_t w[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+    float acc = 0.0f;
+#pragma unroll
+    for (int q = 0; q < 8; q++) {
+        const float4 xv = xf[q * bpr + b];
+        acc += (float)(int8_t)(w[q]) * xv.x;
+        acc += (float)(int8_t)(w[q] >> 8) * xv.y;
+        acc += (float)(int8_t)(w[q] >> 16) * xv.z;
+        acc += (float)(int8_t)(w[q] >> 24) * xv.w;
+    }
+    return d * acc;
+}
+
+template <int T, bool XF32>
+__global__ __launch_bounds__(256) void k_qgemv_q8_0(const uint8_t *__restrict__ W, const void *__restrict__ xg,
+                                                     float *__restrict__ y, int n_rows, int bpr) {
+    extern __shared__ uint4 smem[];
+    float4 *xf = reinterpret_cast<float4 *>(smem);
+    stage_x_q8_0<XF32>(xg, bpr, xf);
+    __syncthreads();
+
+    const int lt = threadIdx.x & (T - 1);
+    const int team = blockIdx.x * (256 / T) + threadIdx.x / T;
+    const int n_teams = gridDim.x * (256 / T);
+    const int iters = bpr / T;
+    const size_t row_bytes = (size_t)bpr * 34;
+
+    for (int row = team; row < n_rows; row += 2 * n_teams) {
+        const int row1 = row + n_teams;
+        const bool has1 = row1 < n_rows;
+        const uint8_t *p0 = W + (size_t)row * row_bytes;
+        const uint8_t *p1 = W + (size_t)(has1 ? row1 : row) * row_bytes;
+        float acc0 = 0.0f, acc1 = 0.0f;
+        for (int it = 0; it < iters; it++) {
+            const int b = it * T + lt;
+            acc0 += q8_0_lane(p0 + (size_t)b * 34, xf, bpr, b);
+            acc1 += q8_0_lane(p1 + (size_t)b * 34, xf, bpr, b);
+        }
+        acc0 = team_sum<T>(acc0);
+        acc1 = team_sum<T>(acc1);
+        if (lt == 0) {
+            y[row] = acc0;
+            if (has1) y[row1] = acc1;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------------------
+int rows_per_team() {
+    static const int v = [] {
+        const char *e = std::getenv("PMETAL_HIP_GEMV_ROWS_PER_TEAM");
+        const int r = e ? std::atoi(e) : 0;
+        return r > 0 ? r : 4;
+    }();
+    return v;
+}
+
+unsigned grid_for_rows(int64_t n, int teams_per_wg) {
+    const int64_t per_wg = (int64_t)teams_per_wg * rows_per_team();
+    int64_t g = (n + per_wg - 1) / per_wg;
+    if (g < 1) g = 1;
+    if (g > (1 << 20)) g = 1 << 20;
+    return (unsigned)g;
+}
+
+template <typename Kern>
+hipError_t launch(Kern kern, unsigned grid, size_t lds, hipStream_t s, const uint8_t *w, const void *x, float *y,
+                  int n, int units) {
+    if (lds > kMaxLds) return hipErrorInvalidValue;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, s, w, x, y, n, units);
+    return hipGetLastError();
+}
+
+template <bool XF32>
+hipError_t launch_q6k(int team, unsigned grid, size_t lds, hipStream_t s, const uint8_t *w, const void *x, float *y,
+                      int n, int spr) {
+    switch (team) {
+    case 8: return launch(k_qgemv_q6k<8, XF32>, grid, lds, s, w, x, y, n, spr);
+    case 16: return launch(k_qgemv_q6k<16, XF32>, grid, lds, s, w, x, y, n, spr);
+    case 32: return launch(k_qgemv_q6k<32, XF32>, grid, lds, s, w, x, y, n, spr);
+    default: return launch(k_qgemv_q6k<64, XF32>, grid, lds, s, w, x, y, n, spr);
+    }
+}
+
+template <bool XF32>
+hipError_t launch_q8_0(int team, unsigned grid, size_t lds, hipStream_t s, const uint8_t *w, const void *x,
+                       float *y, int n, int bpr) {
+    switch (team) {
+    case 1: return launch(k_qgemv_q8_0<1, XF32>, grid, lds, s, w, x, y, n, bpr);
+    case 2: return launch(k_qgemv_q8_0<2, XF32>, grid, lds, s, w, x, y, n, bpr);
+    case 4: return launch(k_qgemv_q8_0<4, XF32>, grid, lds, s, w, x, y, n, bpr);
+    case 8: return launch(k_qgemv_q8_0<8, XF32>, grid, lds, s, w, x, y, n, bpr);
+    case 16: return launch(k_qgemv_q8_0<16, XF32>, grid, lds, s, w, x, y, n, bpr);
+    case 32: return launch(k_qgemv_q8_0<32, XF32>, grid, lds, s, w, x, y, n, bpr);
+    default: return launch(k_qgemv_q8_0<64, XF32>, grid, lds, s, w, x, y, n, bpr);
+    }
+}
+
+}  // namespace
+
+namespace pmh {
+
+// Preconditions (checked by the C ABI layer): n > 0, k > 0 a multiple of the block size, n and
+// k / block below 2^31, pointers 16-byte aligned, type/order/x_dtype valid.  Returns
+// hipErrorInvalidValue when the staged activations do not fit the 160 KiB of LDS.
+hipError_t launch_qgemv(uint32_t type, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype,
+                        float *y, uint32_t order, hipStream_t s) {
+    const bool xf32 = x_dtype == kDtypeF32;
+    const int planes = xf32 ? 3 : 1;
+    if (type == kTypeQ4K) return launch_qgemv_q4k(w, n, k, x, x_dtype, y, order, s);
+    if (type == kTypeQ6K) {
+        const int spr = (int)(k / 256);
+        const int team = 8 * pow2_divisor(spr, 8);
+        const size_t slots = (size_t)spr * 8;
+        const size_t lds = slots * 64 * planes + slots * 16;
+        const unsigned grid = grid_for_rows(n, 256 / team);
+        return xf32 ? launch_q6k<true>(team, grid, lds, s, w, x, y, (int)n, spr)
+                    : launch_q6k<false>(team, grid, lds, s, w, x, y, (int)n, spr);
+    }
+    if (type == kTypeQ8_0) {
+        const int bpr = (int)(k / 32);
+        const int team = pow2_divisor(bpr, 64);
+        const size_t lds = (size_t)bpr * 128;
+        const unsigned grid = grid_for_rows(n, 256 / team);
+        return xf32 ? launch_q8_0<true>(team, grid, lds, s, w, x, y, (int)n, bpr)
+                    : launch_q8_0<false>(team, grid, lds, s, w, x, y, (int)n, bpr);
+    }
+    return hipErrorInvalidValue;
+}
+
+}  // namespace pmh

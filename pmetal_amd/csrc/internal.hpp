@@ -1,0 +1,38 @@
+// Internal declarations shared by the translation units of libpmetal_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace pmh {
+
+constexpr uint32_t kTypeQ8_0 = 8, kTypeQ4K = 12, kTypeQ6K = 14;
+constexpr uint32_t kOrderRef = 0, kOrderGgml = 1;
+constexpr uint32_t kDtypeF32 = 0, kDtypeBf16 = 1;
+
+// ---- codec.hip: bit-exact quantize / dequantize (compiled without fp contraction) ----
+hipError_t launch_quantize_q8_0(const float *x, size_t n, uint8_t *dst, hipStream_t s);
+hipError_t launch_quantize_q4k(const float *x, size_t n, uint8_t *dst, hipStream_t s);
+hipError_t launch_quantize_q6k(const float *x, size_t n, uint8_t *dst, hipStream_t s);
+hipError_t launch_dequantize_q8_0(const uint8_t *src, size_t n, float *dst, hipStream_t s);
+hipError_t launch_dequantize_q4k(const uint8_t *src, size_t n, float *dst, uint32_t order, hipStream_t s);
+hipError_t launch_dequantize_q6k(const uint8_t *src, size_t n, float *dst, hipStream_t s);
+
+// ---- gemv.hip: dequant-fused y = W x ----
+hipError_t launch_qgemv(uint32_t type, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype,
+                        float *y, uint32_t order, hipStream_t s);
+
+// ---- gemm.hip: dequant-fused Y = X W^T ----
+// Bytes of device workspace qgemm needs for (m, k); the caller provides it.
+size_t qgemm_workspace_bytes(int64_t m, int64_t k);
+hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype,
+                        int64_t m, void *y, uint32_t y_dtype, uint32_t order, void *workspace, hipStream_t s);
+
+// ---- util.hip ----
+hipError_t launch_fill_normal(float *dst, size_t n, uint64_t seed, float std, float outlier_rate,
+                              float outlier_mag, hipStream_t s);
+hipError_t launch_f32_to_bf16(const float *src, uint16_t *dst, size_t n, hipStream_t s);
+hipError_t launch_zero_bytes(uint8_t *dst, size_t bytes, hipStream_t s);
+
+}  // namespace pmh

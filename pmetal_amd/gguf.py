@@ -1,0 +1,191 @@
+"""Host-side mirror of the reference's quantize / dequantize / quantized-linear API over the C ABI.
+
+Names, argument meaning and error behaviour follow the Rust interface the kernels stand in for:
+
+* ``GgmlType``        -- crates/pmetal-gguf/src/types.rs:16-187
+* ``quantize``        -- crates/pmetal-gguf/src/quantize.rs:17 ``quantize(data, dtype) -> Vec<u8>``
+* ``dequantize``      -- crates/pmetal-gguf/src/dequant.rs:92 ``dequantize(data, dtype, shape) -> Vec<f32>``
+* ``DequantError``    -- crates/pmetal-gguf/src/dequant.rs:37-70
+* ``GgufLinear``      -- the GGUF-typed counterpart of ``LayerWeight::matmul_from``
+  (crates/pmetal-bridge/src/qwen3_native/weights.rs:66-84)
+* ``use_more_bits`` / ``q4km_tensor_type`` -- crates/pmetal/src/commands/quantize.rs:988-1137
+
+Everything computes on the GPU through ``libpmetal_hip.so``; nothing here falls back to the CPU.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import enum
+
+import numpy as np
+
+from . import _lib
+
+
+class GgmlType(enum.IntEnum):
+    F32 = 0
+    F16 = 1
+    Q8_0 = 8
+    Q4K = 12
+    Q5K = 13
+    Q6K = 14
+
+    def type_size(self) -> int:
+        return _lib.load().pmetal_hip_type_size(int(self))
+
+    def block_size(self) -> int:
+        return _lib.load().pmetal_hip_block_size(int(self))
+
+    def tensor_size(self, n_elements: int) -> int:
+        return _lib.load().pmetal_hip_tensor_size(int(self), n_elements)
+
+
+ORDER_REF, ORDER_GGML = 0, 1
+DTYPE_F32, DTYPE_BF16 = 0, 1
+
+
+class PMetalHipError(RuntimeError):
+    """A failed call; ``code`` is the PMETAL_HIP_ERR_* class."""
+
+    def __init__(self, code: int, message: str):
+        super().__init__(f"[pmetal_hip {code}] {message}")
+        self.code = code
+        self.message = message
+
+
+class QuantizationError(PMetalHipError):
+    """PMetalError::Quantization (crates/pmetal-core/src/error.rs:50-52)."""
+
+
+class DequantError(PMetalHipError):
+    """DequantError (dequant.rs:37-70); ``kind`` names the variant."""
+    KINDS = {2: "UnsupportedType", 3: "InvalidSize", 6: "InvalidShape", 7: "ShapeTooLarge"}
+
+    @property
+    def kind(self) -> str:
+        return self.KINDS.get(self.code, "Other")
+
+
+class NoDeviceError(PMetalHipError):
+    pass
+
+
+def check(rc: int, ctx: str = "") -> None:
+    if rc == 0:
+        return
+    msg = _lib.load().pmetal_hip_last_error_message().decode("utf-8", "replace")
+    if rc == 5:
+        raise NoDeviceError(rc, msg)
+    if ctx == "quantize" and rc in (2, 3):
+        raise QuantizationError(rc, msg)
+    if rc in DequantError.KINDS:
+        raise DequantError(rc, msg)
+    raise PMetalHipError(rc, msg)
+
+
+def init(device: int = 0) -> None:
+    check(_lib.load().pmetal_hip_init(device))
+
+
+def device_count() -> int:
+    return _lib.load().pmetal_hip_device_count()
+
+
+def quantize(data, dtype: int) -> np.ndarray:
+    """``quantize(data: &[f32], dtype) -> Vec<u8>``; bytes bit-identical to the reference CPU path."""
+    lib = _lib.load()
+    x = np.ascontiguousarray(data, dtype=np.float32).reshape(-1)
+    out = np.empty(lib.pmetal_hip_tensor_size(int(dtype), x.size), dtype=np.uint8)
+    check(lib.pmetal_hip_quantize(int(dtype), x.ctypes.data, x.size, out.ctypes.data, out.size), "quantize")
+    return out
+
+
+def dequantize(data, dtype: int, shape, order: int = ORDER_REF) -> np.ndarray:
+    """``dequantize(data: &[u8], dtype, shape: &[i32]) -> Vec<f32>`` (flat, row-major)."""
+    lib = _lib.load()
+    raw = np.ascontiguousarray(data, dtype=np.uint8).reshape(-1)
+    shp = (C.c_int32 * max(len(shape), 1))(*[int(d) for d in shape])
+    nbytes, nelem = C.c_size_t(), C.c_size_t()
+    check(lib.pmetal_hip_expected_byte_size(int(dtype), shp, len(shape), C.byref(nbytes), C.byref(nelem)))
+    if raw.size != nbytes.value:  # reported by the library itself, before any allocation here
+        check(lib.pmetal_hip_dequantize(int(dtype), raw.ctypes.data, raw.size, shp, len(shape), None, 0, order))
+    out = np.empty(nelem.value, dtype=np.float32)
+    check(lib.pmetal_hip_dequantize(int(dtype), raw.ctypes.data, raw.size, shp, len(shape), out.ctypes.data, out.size,
+                                    order))
+    return out
+
+
+def use_more_bits(layer: int, n_layers: int) -> bool:
+    return bool(_lib.load().pmetal_hip_use_more_bits(layer, n_layers))
+
+
+def q4km_tensor_type(gguf_name: str, ndim: int, n_layers: int) -> GgmlType:
+    return GgmlType(_lib.load().pmetal_hip_q4km_tensor_type(gguf_name.encode(), ndim, n_layers))
+
+
+class DeviceBuffer:
+    """A device allocation owned by the caller (freed on ``free()`` / garbage collection)."""
+
+    def __init__(self, nbytes: int):
+        self.nbytes = int(nbytes)
+        self.ptr = _lib.load().pmetal_hip_alloc(self.nbytes)
+        if not self.ptr:
+            check(_lib.load().pmetal_hip_last_error_code() or 4)
+
+    @classmethod
+    def from_host(cls, arr: np.ndarray) -> "DeviceBuffer":
+        arr = np.ascontiguousarray(arr)
+        buf = cls(arr.nbytes)
+        check(_lib.load().pmetal_hip_h2d(buf.ptr, arr.ctypes.data, arr.nbytes))
+        return buf
+
+    def to_host(self, dtype, count: int | None = None) -> np.ndarray:
+        dt = np.dtype(dtype)
+        n = self.nbytes // dt.itemsize if count is None else count
+        out = np.empty(n, dtype=dt)
+        check(_lib.load().pmetal_hip_d2h(out.ctypes.data, self.ptr, out.nbytes))
+        return out
+
+    def free(self) -> None:
+        if getattr(self, "ptr", None):
+            _lib.load().pmetal_hip_free(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def _dev_ptr(obj) -> int:
+    if isinstance(obj, DeviceBuffer):
+        return obj.ptr
+    if hasattr(obj, "data_ptr"):  # a torch tensor on the GPU
+        return int(obj.data_ptr())
+    return int(obj)
+
+
+class GgufLinear:
+    """A GGUF-quantized weight ``[n, k]`` resident on the device; ``forward`` is ``x @ W^T``.
+
+    Mirrors ``LayerWeight::matmul_from``: one token goes through the fused GEMV, several through the
+    fused GEMM.  ``w`` are the packed block bytes (host array or device buffer)."""
+
+    def __init__(self, dtype: int, n: int, k: int, w, order: int = ORDER_REF):
+        self.dtype, self.n, self.k, self.order = GgmlType(dtype), int(n), int(k), order
+        expected = self.dtype.tensor_size(self.n * self.k)
+        if isinstance(w, np.ndarray):
+            if w.size != expected:
+                raise DequantError(3, f"Invalid data size: expected {expected} bytes, got {w.size}")
+            w = DeviceBuffer.from_host(np.ascontiguousarray(w, dtype=np.uint8))
+        self.w = w
+
+    def forward(self, x, m: int = 1, x_dtype: int = DTYPE_BF16, y=None, y_dtype: int = DTYPE_F32, stream=None):
+        """``x``: device buffer of ``[m, k]`` activations; returns the device buffer of ``[m, n]`` outputs."""
+        lib = _lib.load()
+        if y is None:
+            y = DeviceBuffer(m * self.n * (4 if y_dtype == DTYPE_F32 else 2))
+        check(lib.pmetal_hip_qlinear(int(self.dtype), _dev_ptr(self.w), self.n, self.k, _dev_ptr(x), x_dtype, m,
+                                     _dev_ptr(y), y_dtype, self.order, stream))
+        return y

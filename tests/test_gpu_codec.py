@@ -1,0 +1,123 @@
+"""GPU parity: quantize / dequantize through the C ABI must equal the CPU oracle bit for bit."""
+import numpy as np
+import pytest
+
+import pmetal_amd as pm
+from gpu_util import Q4K, Q6K, Q8_0, first_mismatch, gpu_dequantize_dev, gpu_quantize_dev, weights
+
+pytestmark = pytest.mark.gpu
+BLOCK = {Q8_0: 34, Q4K: 144, Q6K: 210}
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _device():
+    pm.init(0)
+
+
+def edge_inputs(block_elems):
+    """Inputs the reference tests and the format's corner cases call for."""
+    rng = np.random.default_rng(99)
+    ramp = ((np.arange(256) - 128.0) * 0.01).astype(np.float32)
+    cases = {
+        "ramp": ramp,
+        "zeros": np.zeros(512, np.float32),
+        "constant": np.full(512, 0.37, np.float32),
+        "all_positive": np.abs(weights(1, 1024)) + np.float32(0.01),
+        "all_negative": -np.abs(weights(2, 1024)) - np.float32(0.01),
+        "tiny": weights(3, 1024, std=1e-30),
+        "denormal": (rng.standard_normal(512) * 1e-41).astype(np.float32),
+        "huge": weights(4, 1024, std=1e30),
+        "mixed_scale": (weights(5, 2048) * np.repeat(10.0 ** rng.integers(-6, 6, 2048 // 16), 16)).astype(np.float32),
+        "one_hot": np.eye(1, 768, 300, dtype=np.float32).reshape(-1) * 3.0,
+        "signed_zero": np.where(np.arange(512) % 2 == 0, np.float32(0.0), np.float32(-0.0)).astype(np.float32),
+        "half_ties": (np.arange(512) % 31 - 15).astype(np.float32) * np.float32(0.5),
+        "ragged": weights(6, 256 * 3 + 77),
+        "short": weights(7, 5),
+        "one_block_plus_one": weights(8, block_elems + 1),
+    }
+    return cases
+
+
+@pytest.mark.parametrize("t", [Q8_0, Q4K, Q6K])
+def test_quantize_edge_cases_bit_exact(oracle, t):
+    for name, x in edge_inputs(32 if t == Q8_0 else 256).items():
+        want = oracle.quantize(t, x)
+        got = gpu_quantize_dev(t, x)
+        assert np.array_equal(got, want), f"{name}: {first_mismatch(got, want, BLOCK[t])}"
+
+
+@pytest.mark.parametrize("t", [Q8_0, Q4K, Q6K])
+def test_quantize_empty(oracle, t):
+    assert gpu_quantize_dev(t, np.zeros(0, np.float32)).size == 0
+    assert pm.quantize(np.zeros(0, np.float32), t).size == 0
+
+
+@pytest.mark.parametrize("t,n,outl", [(Q8_0, 3072 * 1024, 0.0), (Q4K, 1 << 21, 0.0), (Q4K, 1 << 21, 1e-3),
+                                      (Q6K, 1 << 21, 0.0), (Q6K, 1 << 21, 1e-3)])
+def test_quantize_random_bit_exact(oracle, t, n, outl):
+    x = weights(100 + t, n, outliers=outl)
+    want = oracle.quantize(t, x)
+    got = gpu_quantize_dev(t, x)
+    assert np.array_equal(got, want), first_mismatch(got, want, BLOCK[t])
+
+
+@pytest.mark.parametrize("t", [Q8_0, Q4K, Q6K])
+def test_quantize_host_pointer_entry_point(oracle, t):
+    x = weights(7 + t, 256 * 40 + (13 if t == Q8_0 else 0))
+    assert np.array_equal(pm.quantize(x, t), oracle.quantize(t, x))
+
+
+@pytest.mark.parametrize("t", [Q8_0, Q4K, Q6K])
+def test_dequantize_quantized_weights_bit_exact(oracle, t):
+    x = weights(200 + t, 1 << 20, outliers=1e-3)
+    raw = oracle.quantize(t, x)
+    orders = (0, 1) if t == Q4K else (0,)
+    for order in orders:
+        want = oracle.dequantize(t, raw, [x.size], order=order)
+        got = gpu_dequantize_dev(t, raw, x.size, order)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), f"order {order}"
+    # host-pointer entry point with a 2-D shape, as load_gguf calls it
+    got = pm.dequantize(raw, t, [1 << 10, 1 << 10])
+    assert np.array_equal(got.view(np.uint32), oracle.dequantize(t, raw, [1 << 10, 1 << 10]).view(np.uint32))
+
+
+@pytest.mark.parametrize("t", [Q8_0, Q4K, Q6K])
+def test_dequantize_arbitrary_bytes_and_ragged_tail(oracle, t):
+    # every bit pattern of scales / quants, including f16 subnormals, infinities and NaNs in d
+    rng = np.random.default_rng(300 + t)
+    be = 32 if t == Q8_0 else 256
+    nblocks = 4096
+    raw = rng.integers(0, 256, nblocks * BLOCK[t], dtype=np.uint8)
+    for n in (nblocks * be, nblocks * be - 3, nblocks * be - be + 1):
+        r = raw[: pm.GgmlType(t).tensor_size(n)]
+        for order in ((0, 1) if t == Q4K else (0,)):
+            want = oracle.dequantize(t, r, [n], order=order)
+            got = gpu_dequantize_dev(t, r, n, order)
+            nan = np.isnan(want)
+            assert np.array_equal(np.isnan(got), nan)
+            assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+
+
+def test_reference_roundtrip_bounds_on_gpu(oracle):
+    # the reference's own round-trip tests (k_quants.rs:1446-1509), run through the GPU path
+    ramp = ((np.arange(256) - 128.0) * 0.01).astype(np.float32)
+    for t, rmse_max, err_max in ((Q4K, 0.15, 0.5), (Q6K, 0.1, 0.3)):
+        back = pm.dequantize(pm.quantize(ramp, t), t, [256])
+        assert np.sqrt(np.mean((back - ramp) ** 2)) < rmse_max and np.max(np.abs(back - ramp)) < err_max
+    back = pm.dequantize(pm.quantize(ramp, Q8_0), Q8_0, [256])
+    assert np.max(np.abs(back - ramp)) < 0.01
+
+
+def test_errors_match_reference_classes():
+    with pytest.raises(pm.DequantError) as e:
+        pm.dequantize(np.zeros(10, np.uint8), Q4K, [256])
+    assert e.value.kind == "InvalidSize"
+    with pytest.raises(pm.DequantError) as e:
+        pm.dequantize(np.zeros(0, np.uint8), Q4K, [-1])
+    assert e.value.kind == "InvalidShape"
+    with pytest.raises(pm.DequantError) as e:
+        pm.dequantize(np.zeros(0, np.uint8), 99, [0])
+    assert e.value.kind == "UnsupportedType"
+    with pytest.raises(pm.QuantizationError):
+        pm.quantize(np.zeros(32, np.float32), 2)  # Q4_0: outside this path
+    assert pm.dequantize(np.zeros(0, np.uint8), Q6K, [0, 7]).size == 0
