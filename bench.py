@@ -137,12 +137,38 @@ def bench_gemv(args, n, k, t=Q4K, copies=16):
     }, (t, n, k)
 
 
+def bench_gemm(args, m, n, k, t=Q4K):
+    pm, _lib, lib = load()
+    timer = Timer(pm, lib)
+    w = device_weights(pm, lib, t, n * k, 2000)
+    x = pm.DeviceBuffer.from_host(bf16_bits(np.random.default_rng(2).standard_normal(m * k)))
+    y = pm.DeviceBuffer(2 * m * n)
+
+    def step():
+        pm.check(lib.pmetal_hip_qgemm(t, w.ptr, n, k, x.ptr, pm.DTYPE_BF16, m, y.ptr, pm.DTYPE_BF16, 0, None))
+
+    ev_ms, wall_ms = timer.run(step, args.steps, args.warmup)
+    flops = 2.0 * m * n * k
+    us = ev_ms * 1e3 / args.steps
+    tflops = flops / (us * 1e-6) / 1e12
+    return {
+        "value": tflops, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
+        "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tflops / BF16_PEAK_TFLOPS, 4), "traffic": None, "kernel": "k_qgemm_q4k (+ k_prep_x)",
+                     "flops_per_launch": flops, "us_per_launch": round(us, 3)},
+        "extra": {},
+    }, (t, n, k)
+
+
 WORKLOADS = {
     "gemv_q4k_14336x4096": dict(kind="gemv", n=14336, k=4096, metric="Q4_K GEMV GB/s @14336x4096", unit="GB/s",
                                 dtype="bf16 x, 4-bit weights, fp32 accumulate"),
     "gemv_q4k_4096x14336": dict(kind="gemv", n=4096, k=14336, metric="Q4_K GEMV GB/s @4096x14336", unit="GB/s",
                                 dtype="bf16 x, 4-bit weights, fp32 accumulate"),
 }
+for _m in (16, 64, 128, 512, 2048):
+    WORKLOADS[f"gemm_q4k_m{_m}"] = dict(kind="gemm", m=_m, n=14336, k=4096, metric=f"Q4_K GEMM TFLOPS @M={_m},K=4096,N=14336",
+                                        unit="TFLOP/s", dtype="bf16 x (exact in f16), integer f16 weight tiles, fp32 accumulate")
 
 
 def main():
@@ -156,18 +182,22 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)")
     wl = WORKLOADS[args.workload]
-    res, (t, n, k) = bench_gemv(args, wl["n"], wl["k"])
+    if wl["kind"] == "gemm":
+        res, (t, n, k) = bench_gemm(args, wl["m"], wl["n"], wl["k"])
+    else:
+        res, (t, n, k) = bench_gemv(args, wl["n"], wl["k"])
     out = {
         "metric": wl["metric"], "value": round(res["value"], 1), "unit": wl["unit"], "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(res["ms_per_step"], 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": wl["dtype"],
         "data": "synthetic: N(0,0.02) f32 weights generated and quantized on the device, x ~ N(0,1) bf16",
         "config": {"workload": args.workload, "element_order": "REF",
-                   "step": "16 back-to-back GEMVs over 16 distinct weight tensors (528 MB, HBM-resident)"},
+                   "step": ("one GEMM launch (activation pre-pass + MFMA kernel)" if wl["kind"] == "gemm" else
+                            "16 back-to-back GEMVs over 16 distinct weight tensors (528 MB, HBM-resident)")},
         "roofline": res["roofline"], "extra": res["extra"],
     }
     out["extra"]["event_ms_per_step"] = round(res["event_ms_per_step"], 5)
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and wl["kind"] == "gemv":
         out["cpu_baseline"] = cpu_baseline_gemv(t, n, k)
     print(json.dumps(out), flush=True)
 

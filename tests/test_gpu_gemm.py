@@ -1,0 +1,113 @@
+"""GPU parity: dequant-fused Q4_K GEMM against dequantize-then-matmul (f64 accumulation).
+
+Tolerance: max relative error <= 1e-3 (BASELINE.json's north_star), element-wise over outputs with
+|y| > 1e-3 * max|y| and normwise (max|dy| / max|y|), as for the GEMV."""
+import numpy as np
+import pytest
+
+import pmetal_amd as pm
+from gpu_util import Q4K, Q6K, Q8_0, rel_errors, weights
+from pmetal_amd import _lib
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _device():
+    pm.init(0)
+
+
+def gpu_qgemm(t, wq, n, k, x_bits, m, y_dtype=pm.DTYPE_F32, order=0, x_dtype=pm.DTYPE_BF16):
+    lib = _lib.load()
+    dw = pm.DeviceBuffer.from_host(np.ascontiguousarray(wq, dtype=np.uint8))
+    dx = pm.DeviceBuffer.from_host(x_bits)
+    ysz = 4 if y_dtype == pm.DTYPE_F32 else 2
+    dy = pm.DeviceBuffer(m * n * ysz)
+    pm.check(lib.pmetal_hip_memset(dy.ptr, 0xFF, m * n * ysz, None))
+    pm.check(lib.pmetal_hip_qgemm(t, dw.ptr, n, k, dx.ptr, x_dtype, m, dy.ptr, y_dtype, order, None))
+    pm.check(lib.pmetal_hip_sync(None))
+    if y_dtype == pm.DTYPE_F32:
+        return dy.to_host(np.float32).reshape(m, n)
+    return (dy.to_host(np.uint16).astype(np.uint32) << 16).view(np.float32).reshape(m, n)
+
+
+def reference(oracle, t, wq, n, k, x_f32, order):
+    w = oracle.dequantize(t, wq, [n, k], order=order).reshape(n, k).astype(np.float64)
+    return (x_f32.astype(np.float64) @ w.T).astype(np.float32)
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 128, 256), (16, 128, 512), (64, 256, 1024), (128, 384, 4096), (33, 200, 768),
+                                   (130, 129, 256), (512, 512, 2048)])
+def test_qgemm_q4k_matches_dequantize_then_matmul(oracle, m, n, k):
+    wq = oracle.quantize(Q4K, weights(m + n + k, n * k, outliers=1e-3))
+    x = np.random.default_rng(m * 7 + k).standard_normal((m, k)).astype(np.float32)
+    bits = oracle.f32_to_bf16_bits(x.reshape(-1)).reshape(m, k)
+    xr = oracle.bf16_bits_to_f32(bits.reshape(-1)).reshape(m, k)
+    for order in (0, 1):
+        want = reference(oracle, Q4K, wq, n, k, xr, order)
+        got = gpu_qgemm(Q4K, wq, n, k, bits, m, order=order)
+        elem, norm = rel_errors(got.reshape(-1), want.reshape(-1))
+        print(f"Q4_K GEMM m={m} n={n} k={k} order={order}: elem {elem:.2e} norm {norm:.2e}")
+        assert elem <= TOL and norm <= TOL
+
+
+def test_qgemm_bf16_output_and_large_activations(oracle):
+    m, n, k = 64, 256, 1024
+    wq = oracle.quantize(Q4K, weights(5, n * k))
+    x = np.random.default_rng(6).standard_normal((m, k)).astype(np.float32)
+    x[3] *= 1e6   # a row far outside the f16 range: handled by the per-row power-of-two scale
+    x[5] *= 1e-6
+    x[7] = 0.0
+    bits = oracle.f32_to_bf16_bits(x.reshape(-1)).reshape(m, k)
+    xr = oracle.bf16_bits_to_f32(bits.reshape(-1)).reshape(m, k)
+    want = reference(oracle, Q4K, wq, n, k, xr, 0)
+    got = gpu_qgemm(Q4K, wq, n, k, bits, m)
+    for row in range(m):  # per row: the rows have wildly different magnitudes
+        elem, norm = rel_errors(got[row], want[row])
+        assert elem <= TOL and norm <= TOL, (row, elem, norm)
+    got16 = gpu_qgemm(Q4K, wq, n, k, bits, m, y_dtype=pm.DTYPE_BF16)
+    for row in (0, 3, 5, 63):
+        scale = np.max(np.abs(want[row])) or 1.0
+        assert np.max(np.abs(got16[row] - want[row])) / scale <= 2.0 ** -8  # bf16 rounding of the output
+
+
+def test_qgemm_config2_full_size(oracle):
+    # BASELINE config 2: M = 512, K = 4096, N = 14336, bf16 activations ~ N(0, 1)
+    m, n, k = 512, 14336, 4096
+    wq = pm.quantize(weights(31, n * k), Q4K)
+    x = np.random.default_rng(32).standard_normal((m, k)).astype(np.float32)
+    bits = oracle.f32_to_bf16_bits(x.reshape(-1)).reshape(m, k)
+    xr = oracle.bf16_bits_to_f32(bits.reshape(-1)).reshape(m, k)
+    want = reference(oracle, Q4K, wq, n, k, xr, 0)
+    got = gpu_qgemm(Q4K, wq, n, k, bits, m)
+    elem, norm = rel_errors(got.reshape(-1), want.reshape(-1))
+    print(f"Q4_K GEMM 512x14336x4096: elem {elem:.2e} norm {norm:.2e}")
+    assert elem <= TOL and norm <= TOL
+
+
+def test_qgemm_agrees_with_qgemv_and_qlinear_dispatch(oracle):
+    from gpu_util import gpu_qgemv
+    lib = _lib.load()
+    n, k = 512, 2048
+    wq = oracle.quantize(Q4K, weights(41, n * k))
+    bits = oracle.f32_to_bf16_bits(np.random.default_rng(42).standard_normal(k).astype(np.float32))
+    y_gemv = gpu_qgemv(Q4K, wq, n, k, bits, pm.DTYPE_BF16)
+    y_gemm = gpu_qgemm(Q4K, wq, n, k, bits.reshape(1, k), 1).reshape(-1)
+    elem, norm = rel_errors(y_gemm, y_gemv)
+    assert norm <= 1e-5
+    lin = pm.GgufLinear(Q4K, n, k, wq)
+    y1 = lin.forward(pm.DeviceBuffer.from_host(bits), m=1).to_host(np.float32)
+    assert np.array_equal(y1, y_gemv)  # m == 1 dispatches to the GEMV
+    xb = np.tile(bits, (4, 1))
+    y4 = lin.forward(pm.DeviceBuffer.from_host(xb), m=4).to_host(np.float32).reshape(4, n)
+    assert np.allclose(y4[2], y_gemv, rtol=1e-4, atol=1e-5)
+
+
+def test_qgemm_argument_errors():
+    lib = _lib.load()
+    buf = pm.DeviceBuffer(1 << 16)
+    assert lib.pmetal_hip_qgemm(Q4K, buf.ptr, 4, 256, buf.ptr, 1, 0, buf.ptr, 0, 0, None) == 6   # m == 0
+    assert lib.pmetal_hip_qgemm(Q4K, buf.ptr, 4, 100, buf.ptr, 1, 4, buf.ptr, 0, 0, None) == 6   # k % 256
+    assert lib.pmetal_hip_qgemm(Q8_0, buf.ptr, 4, 256, buf.ptr, 1, 4, buf.ptr, 0, 0, None) == 2  # no Q8_0 GEMM
+    assert lib.pmetal_hip_qgemm(Q4K, buf.ptr, 4, 256, buf.ptr, 1, 4, buf.ptr, 7, 0, None) == 1   # y_dtype
