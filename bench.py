@@ -28,6 +28,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled against a streaming
+# kernel of known size (summary and commands: profiles/qgemv_q4k_14336x4096.md)
+MEASURED_TRAFFIC = {"gemv_q4k_14336x4096": 33232404}
 BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16/fp16 MFMA, published
 Q8_0, Q4K, Q6K = 8, 12, 14
 
@@ -160,12 +163,109 @@ def bench_gemm(args, m, n, k, t=Q4K):
     }, (t, n, k)
 
 
+def qwen3_06b_linears(pm):
+    """(gguf name, n, k, type) of every batch-1 projection of a Qwen3-0.6B-shaped decoder, Q4_K_M recipe."""
+    out = []
+    for layer in range(28):
+        for name, n, k in (("attn_q", 2048, 1024), ("attn_k", 1024, 1024), ("attn_v", 1024, 1024),
+                           ("attn_output", 1024, 2048), ("ffn_gate", 3072, 1024), ("ffn_up", 3072, 1024),
+                           ("ffn_down", 1024, 3072)):
+            gg = f"blk.{layer}.{name}.weight"
+            out.append((gg, n, k, int(pm.q4km_tensor_type(gg, 2, 28))))
+    out.append(("output.weight", 151936, 1024, int(pm.q4km_tensor_type("output.weight", 2, 28))))
+    return out
+
+
+def llama3_8b_tensors(pm):
+    """(gguf name, n, k, type) of every quantized tensor of a Llama-3-8B-shaped model, Q4_K_M recipe."""
+    out = [("token_embd.weight", 128256, 4096, int(pm.q4km_tensor_type("token_embd.weight", 2, 32)))]
+    for layer in range(32):
+        for name, n, k in (("attn_q", 4096, 4096), ("attn_k", 1024, 4096), ("attn_v", 1024, 4096),
+                           ("attn_output", 4096, 4096), ("ffn_gate", 14336, 4096), ("ffn_up", 14336, 4096),
+                           ("ffn_down", 4096, 14336)):
+            gg = f"blk.{layer}.{name}.weight"
+            out.append((gg, n, k, int(pm.q4km_tensor_type(gg, 2, 32))))
+    out.append(("output.weight", 128256, 4096, int(pm.q4km_tensor_type("output.weight", 2, 32))))
+    return out
+
+
+def bench_decode(args):
+    """All batch-1 linear projections of one token of a random-init Qwen3-0.6B-shaped stack (linears only)."""
+    pm, _lib, lib = load()
+    timer = Timer(pm, lib)
+    lins = qwen3_06b_linears(pm)
+    descs = (_lib.LinearDesc * len(lins))()
+    keep, total_bytes = [], 0
+    xs = {k: pm.DeviceBuffer.from_host(bf16_bits(np.random.default_rng(k).standard_normal(k))) for k in (1024, 2048, 3072)}
+    for i, (name, n, k, t) in enumerate(lins):
+        w = device_weights(pm, lib, t, n * k, 3000 + i)
+        y = pm.DeviceBuffer(4 * n)
+        keep.append((w, y))
+        descs[i] = _lib.LinearDesc(t, pm.DTYPE_BF16, 0, 0, n, k, w.ptr, xs[k].ptr, y.ptr)
+        total_bytes += gemv_bytes(t, n, k, 2)
+
+    def step():
+        pm.check(lib.pmetal_hip_qgemv_batch(descs, len(lins), None))
+
+    ev_ms, wall_ms = timer.run(step, args.steps, args.warmup)
+    tok_s = args.steps / (ev_ms * 1e-3)
+    gbs = total_bytes * tok_s / 1e9
+    return {
+        "value": tok_s, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "k_qgemv_q4k / k_qgemv_q6k (197 launches)",
+                     "bytes_per_step": total_bytes},
+        "extra": {"launches_per_token": len(lins), "q6k_tensors": sum(1 for l in lins if l[3] == Q6K)},
+    }, (Q4K, 0, 0)
+
+
+def bench_quantize(args):
+    """f32 -> Q4_K_M over a random-init Llama-3-8B-shaped weight set resident in HBM (32 GB in, 5 GB out)."""
+    pm, _lib, lib = load()
+    timer = Timer(pm, lib)
+    tensors = llama3_8b_tensors(pm)
+    n_total = sum(n * k for _, n, k, _ in tensors)
+    out_total = sum(lib.pmetal_hip_tensor_size(t, n * k) for _, n, k, t in tensors)
+    src = pm.DeviceBuffer(4 * n_total)
+    dst = pm.DeviceBuffer(out_total + 256 * len(tensors))
+    jobs, so, do = [], 0, 0
+    for i, (name, n, k, t) in enumerate(tensors):
+        ne = n * k
+        pm.check(lib.pmetal_hip_fill_normal_f32(src.ptr + 4 * so, ne, 7000 + i, 0.02, 1e-3, 0.5, None))
+        nb = lib.pmetal_hip_tensor_size(t, ne)
+        jobs.append((t, src.ptr + 4 * so, ne, dst.ptr + do, nb))
+        so += ne
+        do += (nb + 255) // 256 * 256
+    pm.check(lib.pmetal_hip_sync(None))
+
+    def step():
+        for t, sp, ne, dp, nb in jobs:
+            pm.check(lib.pmetal_hip_quantize_dev(t, sp, ne, dp, nb, None), "quantize")
+
+    ev_ms, wall_ms = timer.run(step, args.steps, args.warmup)
+    gbs_in = 4.0 * n_total * args.steps / (ev_ms * 1e-3) / 1e9
+    gbs_total = (4.0 * n_total + out_total) * args.steps / (ev_ms * 1e-3) / 1e9
+    q6 = sum(n * k for _, n, k, t in tensors if t == Q6K)
+    return {
+        "value": gbs_in, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
+        "roofline": {"bound": "hbm", "achieved": round(gbs_total, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs_total / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "k_quantize_q4k / k_quantize_q6k", "bytes_per_step": 4 * n_total + out_total},
+        "extra": {"elements": n_total, "q6k_fraction": round(q6 / n_total, 4), "tensors": len(tensors),
+                  "output_bytes": out_total},
+    }, (Q4K, 0, 0)
+
+
 WORKLOADS = {
     "gemv_q4k_14336x4096": dict(kind="gemv", n=14336, k=4096, metric="Q4_K GEMV GB/s @14336x4096", unit="GB/s",
                                 dtype="bf16 x, 4-bit weights, fp32 accumulate"),
     "gemv_q4k_4096x14336": dict(kind="gemv", n=4096, k=14336, metric="Q4_K GEMV GB/s @4096x14336", unit="GB/s",
                                 dtype="bf16 x, 4-bit weights, fp32 accumulate"),
 }
+WORKLOADS["decode_qwen3_0.6b_q4km"] = dict(kind="decode", metric="Q4_K_M decode linears tokens/s (Qwen3-0.6B shape)", unit="tokens/s",
+                                           dtype="bf16 x, 4-/6-bit weights, fp32 accumulate")
+WORKLOADS["quantize_llama3_8b_q4km"] = dict(kind="quantize", metric="f32->Q4_K_M quantize GB/s of f32 consumed (Llama-3-8B shape)",
+                                            unit="GB/s", dtype="f32 -> 4-/6-bit blocks, bit-exact f32 search")
 for _m in (16, 64, 128, 512, 2048):
     WORKLOADS[f"gemm_q4k_m{_m}"] = dict(kind="gemm", m=_m, n=14336, k=4096, metric=f"Q4_K GEMM TFLOPS @M={_m},K=4096,N=14336",
                                         unit="TFLOP/s", dtype="bf16 x (exact in f16), integer f16 weight tiles, fp32 accumulate")
@@ -178,25 +278,44 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="gemv_q4k_14336x4096", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run a plain streaming kernel of known size (f32 -> bf16 over 2^24 elements: 64 MiB read, "
+                         "32 MiB written) so that profiler byte counters can be scaled against it")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)")
     wl = WORKLOADS[args.workload]
     if wl["kind"] == "gemm":
         res, (t, n, k) = bench_gemm(args, wl["m"], wl["n"], wl["k"])
+    elif wl["kind"] == "decode":
+        res, (t, n, k) = bench_decode(args)
+    elif wl["kind"] == "quantize":
+        res, (t, n, k) = bench_quantize(args)
     else:
         res, (t, n, k) = bench_gemv(args, wl["n"], wl["k"])
     out = {
         "metric": wl["metric"], "value": round(res["value"], 1), "unit": wl["unit"], "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(res["ms_per_step"], 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": wl["dtype"],
-        "data": "synthetic: N(0,0.02) f32 weights generated and quantized on the device, x ~ N(0,1) bf16",
+        "data": ("synthetic: N(0,0.02) f32 with 0.1% outliers at +-0.5, generated on the device" if wl["kind"] == "quantize"
+                 else "synthetic: N(0,0.02) f32 weights generated and quantized on the device, x ~ N(0,1) bf16"),
         "config": {"workload": args.workload, "element_order": "REF",
-                   "step": ("one GEMM launch (activation pre-pass + MFMA kernel)" if wl["kind"] == "gemm" else
-                            "16 back-to-back GEMVs over 16 distinct weight tensors (528 MB, HBM-resident)")},
+                   "step": {"gemm": "one GEMM launch (activation pre-pass + MFMA kernel)",
+                            "gemv": "16 back-to-back GEMVs over 16 distinct weight tensors (528 MB, HBM-resident)",
+                            "decode": "all 197 batch-1 projections of one token, back to back on one stream",
+                            "quantize": "all 226 tensors of the model, f32 resident in HBM"}[wl["kind"]]},
         "roofline": res["roofline"], "extra": res["extra"],
     }
     out["extra"]["event_ms_per_step"] = round(res["event_ms_per_step"], 5)
+    out["roofline"]["traffic"] = MEASURED_TRAFFIC.get(args.workload)
+    if args.calibrate:
+        pm, _lib, lib = load()
+        n_cal = 1 << 24
+        src, dst = pm.DeviceBuffer(4 * n_cal), pm.DeviceBuffer(2 * n_cal)
+        pm.check(lib.pmetal_hip_fill_normal_f32(src.ptr, n_cal, 1, 1.0, 0.0, 0.0, None))
+        for _ in range(5):
+            pm.check(lib.pmetal_hip_f32_to_bf16_dev(src.ptr, dst.ptr, n_cal, None))
+        pm.check(lib.pmetal_hip_sync(None))
     if not args.no_cpu_baseline and wl["kind"] == "gemv":
         out["cpu_baseline"] = cpu_baseline_gemv(t, n, k)
     print(json.dumps(out), flush=True)
