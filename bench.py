@@ -258,17 +258,17 @@ def bench_quantize(args):
 
 WORKLOADS = {
     "gemv_q4k_14336x4096": dict(kind="gemv", n=14336, k=4096, metric="Q4_K GEMV GB/s @14336x4096", unit="GB/s",
-                                dtype="bf16 x, 4-bit weights, fp32 accumulate"),
+                                dtype="bf16"),
     "gemv_q4k_4096x14336": dict(kind="gemv", n=4096, k=14336, metric="Q4_K GEMV GB/s @4096x14336", unit="GB/s",
-                                dtype="bf16 x, 4-bit weights, fp32 accumulate"),
+                                dtype="bf16"),
 }
 WORKLOADS["decode_qwen3_0.6b_q4km"] = dict(kind="decode", metric="Q4_K_M decode linears tokens/s (Qwen3-0.6B shape)", unit="tokens/s",
-                                           dtype="bf16 x, 4-/6-bit weights, fp32 accumulate")
+                                           dtype="bf16")
 WORKLOADS["quantize_llama3_8b_q4km"] = dict(kind="quantize", metric="f32->Q4_K_M quantize GB/s of f32 consumed (Llama-3-8B shape)",
-                                            unit="GB/s", dtype="f32 -> 4-/6-bit blocks, bit-exact f32 search")
+                                            unit="GB/s", dtype="f32")
 for _m in (16, 64, 128, 512, 2048):
     WORKLOADS[f"gemm_q4k_m{_m}"] = dict(kind="gemm", m=_m, n=14336, k=4096, metric=f"Q4_K GEMM TFLOPS @M={_m},K=4096,N=14336",
-                                        unit="TFLOP/s", dtype="bf16 x (exact in f16), integer f16 weight tiles, fp32 accumulate")
+                                        unit="TFLOP/s", dtype="f16")
 
 
 def main():

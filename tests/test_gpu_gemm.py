@@ -111,3 +111,16 @@ def test_qgemm_argument_errors():
     assert lib.pmetal_hip_qgemm(Q4K, buf.ptr, 4, 100, buf.ptr, 1, 4, buf.ptr, 0, 0, None) == 6   # k % 256
     assert lib.pmetal_hip_qgemm(Q8_0, buf.ptr, 4, 256, buf.ptr, 1, 4, buf.ptr, 0, 0, None) == 2  # no Q8_0 GEMM
     assert lib.pmetal_hip_qgemm(Q4K, buf.ptr, 4, 256, buf.ptr, 1, 4, buf.ptr, 7, 0, None) == 1   # y_dtype
+
+
+@pytest.mark.parametrize("t", [Q6K, Q8_0])
+def test_qlinear_runs_rowwise_gemv_for_types_without_gemm(oracle, t):
+    n, k, m = 96, 512, 3
+    wq = oracle.quantize(t, weights(51, n * k))
+    x = np.random.default_rng(52).standard_normal((m, k)).astype(np.float32)
+    bits = oracle.f32_to_bf16_bits(x.reshape(-1)).reshape(m, k)
+    lin = pm.GgufLinear(t, n, k, wq)
+    y = lin.forward(pm.DeviceBuffer.from_host(bits), m=m).to_host(np.float32).reshape(m, n)
+    want = reference(oracle, t, wq, n, k, oracle.bf16_bits_to_f32(bits.reshape(-1)).reshape(m, k), 0)
+    elem, norm = rel_errors(y.reshape(-1), want.reshape(-1))
+    assert elem <= TOL and norm <= TOL
