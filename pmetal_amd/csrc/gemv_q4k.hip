@@ -41,15 +41,23 @@ using namespace pmh::gemv;
 //   REF  order: lowbase = 32j,               highbase = lowbase + 16   (both in sub-block j)
 //   GGML order: lowbase = 64(j/2) + 16(j%2), highbase = lowbase + 32   (sub-blocks 2(j/2), 2(j/2)+1)
 
+// Four consecutive activations as they lie in memory (f32: 16 bytes, bf16: 8 bytes in .x/.y); unpacking is
+// kept apart from the load so that a wave can go on issuing loads while these are in flight.
 template <bool XF32>
-__device__ __forceinline__ void load_x4(const void *xg, size_t e, float (&v)[4]) {
+__device__ __forceinline__ uint4 load_x4_raw(const void *xg, size_t e) {
+    if (XF32) return *reinterpret_cast<const uint4 *>(reinterpret_cast<const float *>(xg) + e);
+    const uint2 u = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(xg) + e);
+    return make_uint4(u.x, u.y, 0u, 0u);
+}
+
+template <bool XF32>
+__device__ __forceinline__ void unpack_x4(const uint4 r, float (&v)[4]) {
     if (XF32) {
-        const float4 f = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(xg) + e);
-        v[0] = f.x, v[1] = f.y, v[2] = f.z, v[3] = f.w;
+        v[0] = __builtin_bit_cast(float, r.x), v[1] = __builtin_bit_cast(float, r.y);
+        v[2] = __builtin_bit_cast(float, r.z), v[3] = __builtin_bit_cast(float, r.w);
     } else {
-        const uint2 u = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(xg) + e);
-        v[0] = bf16_to_f32(u.x & 0xFFFFu), v[1] = bf16_to_f32(u.x >> 16);
-        v[2] = bf16_to_f32(u.y & 0xFFFFu), v[3] = bf16_to_f32(u.y >> 16);
+        v[0] = bf16_to_f32(r.x & 0xFFFFu), v[1] = bf16_to_f32(r.x >> 16);
+        v[2] = bf16_to_f32(r.y & 0xFFFFu), v[3] = bf16_to_f32(r.y >> 16);
     }
 }
 
@@ -139,42 +147,56 @@ __device__ __forceinline__ void stage_convert(int idx, const float (&lo)[4], con
 }
 
 // Per-lane constants for the branch-free get_scale_min_k4 (crates/pmetal-gguf/src/quantize.rs:844-855).
-// With a, b, c the bytes (j & 3) of the three scale dwords:
+// With a, b, c the bytes (j & 3) of the three scale dwords y, z, w of the header:
 //   j <  4: sc = a & 63,                   m = b & 63
 //   j >= 4: sc = (c & 15) | (a >> 6) << 4, m = (c >> 4) | (b >> 6) << 4
-// both are (c' & cm) | ((a >> sa) & am) with c' = c resp. c >> 4.
+// Both are  bfe(c-word, off_c, wid_c) | bfe(a-word, off_a, wid_a) << shl  with per-lane field positions
+// (a zero-width field reads as 0).
 struct ScaleSel {
-    uint32_t sh;     // 8 * (j & 3)
-    uint32_t sh_ab;  // sh + (j < 4 ? 0 : 2)
-    uint32_t am;     // j < 4 ? 63 : 0x30
-    uint32_t cm;     // j < 4 ? 0 : 15
+    uint32_t off_a;  // 8 (j & 3) + (j < 4 ? 0 : 6)
+    uint32_t wid_a;  // j < 4 ? 6 : 2
+    uint32_t off_c;  // 8 (j & 3)
+    uint32_t wid_c;  // j < 4 ? 0 : 4
+    uint32_t shl;    // j < 4 ? 0 : 4
 };
 
 __device__ __forceinline__ ScaleSel scale_sel(int j) {
     ScaleSel s;
-    s.sh = 8u * (j & 3);
-    s.sh_ab = s.sh + (j < 4 ? 0u : 2u);
-    s.am = j < 4 ? 63u : 0x30u;
-    s.cm = j < 4 ? 0u : 15u;
+    s.off_c = 8u * (j & 3);
+    s.off_a = s.off_c + (j < 4 ? 0u : 6u);
+    s.wid_a = j < 4 ? 6u : 2u;
+    s.wid_c = j < 4 ? 0u : 4u;
+    s.shl = j < 4 ? 0u : 4u;
     return s;
 }
 
 __device__ __forceinline__ void scale_min(const uint4 hdr, const ScaleSel &s, float &sc, float &m) {
-    const uint32_t c = hdr.w >> s.sh;
-    sc = (float)((c & s.cm) | ((hdr.y >> s.sh_ab) & s.am));
-    m = (float)(((c >> 4) & s.cm) | ((hdr.z >> s.sh_ab) & s.am));
+    const uint32_t a = __builtin_amdgcn_ubfe(hdr.y, s.off_a, s.wid_a);
+    const uint32_t b = __builtin_amdgcn_ubfe(hdr.z, s.off_a, s.wid_a);
+    const uint32_t c0 = __builtin_amdgcn_ubfe(hdr.w, s.off_c, s.wid_c);
+    const uint32_t c1 = __builtin_amdgcn_ubfe(hdr.w, s.off_c + 4u, s.wid_c);
+    sc = (float)((a << s.shl) | c0);
+    m = (float)((b << s.shl) | c1);
 }
 
 // sum over the 32 nibbles of (q * X) with X = sum_k 16^k digit_k - 2^P, as fp32
 template <int NDIG>
 __device__ __forceinline__ float combine(const uint32_t (&acc)[NDIG], uint32_t accq) {
+    if (NDIG == 5) {
+        // 2^P = 8 * 16^4: the offset comes off the top digit sum, and the whole signed sum fits 32 bits
+        // (|sum| <= 32 * 15 * 2^19 < 2^28): one integer chain, one rounding.
+        int t = (int)acc[4] - 8 * (int)accq;
+#pragma unroll
+        for (int k = 3; k >= 0; k--) t = (t << 4) + (int)acc[k];
+        return (float)t;
+    }
     constexpr int P = 4 * NDIG - 1;
     // the low four digit sums fit an integer exactly; the rest is folded in fp32
     uint32_t t = acc[3];
 #pragma unroll
     for (int k = 2; k >= 0; k--) t = (t << 4) + acc[k];
     float f = (float)t;
-    if (NDIG > 4) f += 65536.0f * (float)(NDIG > 5 ? acc[4] + (acc[5] << 4) : acc[4]);
+    f += 65536.0f * (float)(NDIG > 5 ? acc[4] + (acc[5] << 4) : acc[4]);
     return f - (float)(1 << P) * (float)accq;
 }
 
@@ -183,7 +205,9 @@ template <int ORDER, int NDIG>
 __device__ __forceinline__ float lane_dot(const uint4 hdr, const uint4 qv, const ScaleSel &s0, const ScaleSel &s1,
                                           const uint4 (&xdig)[NDIG], const float4 xm) {
     const uint32_t w[4] = {qv.x, qv.y, qv.z, qv.w};
-    const float d = f16_bits_to_f32(hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(hdr.x >> 16);
+    // fma with an f16 operand converted in place
+    const float d = (float)__builtin_bit_cast(_Float16, (uint16_t)(hdr.x & 0xFFFFu));
+    const float dmin = (float)__builtin_bit_cast(_Float16, (uint16_t)(hdr.x >> 16));
     if (ORDER == 0) {
         uint32_t acc[NDIG], accq = 0;
 #pragma unroll
@@ -198,7 +222,9 @@ __device__ __forceinline__ float lane_dot(const uint4 hdr, const uint4 qv, const
         for (int i = 0; i < 4; i++) accq = __builtin_amdgcn_udot8(w[i], 0x11111111u, accq, false);
         float sc, m;
         scale_min(hdr, s0, sc, m);
-        return (d * sc) * (xm.x * combine<NDIG>(acc, accq)) - (dmin * m) * xm.w;
+        const float u = sc * (xm.x * combine<NDIG>(acc, accq));
+        const float v = m * xm.w;
+        return __builtin_fmaf(d, u, -(dmin * v));
     } else {
         // low nibbles belong to sub-block 2(j/2), high nibbles to 2(j/2)+1: separate sums
         uint32_t wl[4], wh[4];
@@ -229,43 +255,240 @@ __device__ __forceinline__ float lane_dot(const uint4 hdr, const uint4 qv, const
     }
 }
 
-// Tasks in flight per team.  When a row is one or two tasks long (ITERS = 1, 2) every task of a team uses
-// the same one or two x slots, which are then held in registers for the whole kernel; the registers that
-// takes are paid for with a shallower prefetch.
-template <int ITERS>
-struct Depth {
-    static constexpr int value = ITERS == 0 ? 8 : 4;
-};
-
 #ifdef PMH_TRACE
-__device__ unsigned long long *g_trace;  // [workgroup][wave][8] timestamps, set by the harness
-#define PMH_STAMP(slot)                                                                              \
-    do {                                                                                             \
-        if ((threadIdx.x & 63) == 0)                                                                 \
-            g_trace[((size_t)blockIdx.x * 16 + (threadIdx.x >> 6)) * 8 + (slot)] = __builtin_readcyclecounter(); \
+// experiment hook: per-wave cycle stamps kept in registers and written out when the kernel ends
+__device__ unsigned long long *g_trace;  // [workgroup][wave][8], set by the harness
+#define PMH_STAMP_DECL unsigned long long pmh_st[8] = {0, 0, 0, 0, 0, 0, 0, 0}, pmh_rt[2] = {0, 0}
+#define PMH_STAMP(slot) pmh_st[slot] = __builtin_readcyclecounter()
+#define PMH_RT(slot) pmh_rt[slot >> 2] = __builtin_amdgcn_s_memrealtime()
+#define PMH_STAMP_FLUSH                                                                     \
+    do {                                                                                    \
+        if ((threadIdx.x & 63) == 0)                                                        \
+            for (int q = 0; q < 8; q++)                                                     \
+                g_trace[((size_t)blockIdx.x * 16 + (threadIdx.x >> 6)) * 8 + q] =           \
+                    q == 5 ? pmh_rt[0] : q == 7 ? pmh_rt[1] : pmh_st[q];                    \
     } while (0)
 #else
+#define PMH_STAMP_DECL
 #define PMH_STAMP(slot)
+#define PMH_RT(slot)
+#define PMH_STAMP_FLUSH
 #endif
 
-template <int ORDER, bool XF32, int T, int ITERS>
+// Conversion of x into LDS in two steps, so that the first pass of activation loads can be requested before
+// the weight loads queue up behind it: stage_x_begin loads, stage_x_finish converts (and runs the further
+// passes a long row needs).  All threads of the workgroup take part; the caller places the barrier.
+#ifndef PMH_STAGE_PRE
+#define PMH_STAGE_PRE 2
+#endif
+constexpr int kStagePre = PMH_STAGE_PRE;  // passes of activation loads requested up front
+
+template <int ORDER, bool XF32>
+__device__ __forceinline__ void stage_x_begin(const void *xg, int slots, int nthreads, uint4 (&r_lo)[kStagePre],
+                                              uint4 (&r_hi)[kStagePre]) {
+#pragma unroll
+    for (int ps = 0; ps < kStagePre; ps++) {
+        r_lo[ps] = r_hi[ps] = make_uint4(0u, 0u, 0u, 0u);
+        const int idx = threadIdx.x + ps * nthreads;
+        if (idx < slots * 4) {
+            size_t e_lo, e_hi;
+            stage_offsets<ORDER>(idx, e_lo, e_hi);
+            r_lo[ps] = load_x4_raw<XF32>(xg, e_lo);
+            r_hi[ps] = load_x4_raw<XF32>(xg, e_hi);
+        }
+    }
+}
+
+template <int ORDER, int NDIG, bool XF32>
+__device__ __forceinline__ void stage_x_finish(const void *xg, int slots, int nthreads, const uint4 (&r_lo)[kStagePre],
+                                               const uint4 (&r_hi)[kStagePre], uint4 *xd, float4 *xm) {
+    const int stage_total = slots * 4;
+    float x_lo[4], x_hi[4];
+#pragma unroll
+    for (int ps = 0; ps < kStagePre; ps++) {
+        const int idx = threadIdx.x + ps * nthreads;
+        if (idx < stage_total) {
+            unpack_x4<XF32>(r_lo[ps], x_lo);
+            unpack_x4<XF32>(r_hi[ps], x_hi);
+            stage_convert<NDIG, XF32>(idx, x_lo, x_hi, slots, xd, xm);
+        }
+    }
+    for (int idx = threadIdx.x + kStagePre * nthreads; idx < stage_total; idx += nthreads) {
+        size_t e_lo, e_hi;
+        stage_offsets<ORDER>(idx, e_lo, e_hi);
+        unpack_x4<XF32>(load_x4_raw<XF32>(xg, e_lo), x_lo);
+        unpack_x4<XF32>(load_x4_raw<XF32>(xg, e_hi), x_hi);
+        stage_convert<NDIG, XF32>(idx, x_lo, x_hi, slots, xd, xm);
+    }
+}
+
+// ---- kernel A: one wave per (row group, k-chunk) ------------------------------------------------
+// A team of T lanes covers a chunk of T/8 super-blocks of a row; a row is KS = (k/256) / (T/8) chunks.
+// The workgroup has KS * G waves: wave (g, h) takes chunk h of the rows of row group g, 64/T rows per task,
+// so every task of a wave needs the same x digits, which stay in registers.  Up to kDepth tasks are in
+// flight per wave; every load is issued unconditionally (tasks past the end read the first bytes of W, all
+// lanes the same address) so that the number of outstanding loads is known at every wait.  Each lane's
+// partial sum goes to LDS; after a barrier the workgroup adds up the partials of each of its rows.
+constexpr int kDepth = 8;  // tasks in flight per wave
+#ifndef PMH_KPRE
+#define PMH_KPRE 2
+#endif
+constexpr int kPre = PMH_KPRE;  // of which this many are requested before x is converted
+
+// Row stride of the partial sums in LDS.  The final summation puts `red` lanes on a row (lane p adds every
+// red-th partial), 64 / red rows side by side in a wave: a stride of `red` floats past a multiple of 64 keeps
+// those rows in different banks.
+__host__ __device__ constexpr int part_stride(int slots, int red) { return ((slots + 63) / 64) * 64 + (red & 63); }
+
+template <int ORDER, bool XF32, int T, bool SINGLE>
+__global__ __launch_bounds__(1024) void k_qgemv_q4k_chunk(const uint8_t *__restrict__ W, const void *__restrict__ xg,
+                                                           float *__restrict__ y, int n_rows, int spr,
+                                                           int rows_per_wg, int rows_per_wave, int n_nominal, int red,
+                                                           int nthreads) {
+    constexpr int NDIG = XF32 ? 6 : 5;
+    constexpr int SEG = T / 8;   // super-blocks a team covers
+    constexpr int RPT = 64 / T;  // rows per task
+    extern __shared__ uint4 smem[];
+    const int slots = spr * 8;
+    uint4 *xd = smem;
+    float4 *xm = reinterpret_cast<float4 *>(xd + NDIG * slots);
+    float *part = reinterpret_cast<float *>(xm + slots);  // [group][n_nominal * RPT][part_stride(slots)]
+    const int ps = part_stride(slots, red);
+
+    PMH_STAMP_DECL;
+    PMH_STAMP(0);
+    PMH_RT(0);
+    const int lane = threadIdx.x & 63;
+    const int lt = lane & (T - 1), tm = lane / T, j = lane & 7;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int ks = spr / SEG;
+    const int h = wave % ks, g = wave / ks;
+    const int wg_r0 = blockIdx.x * rows_per_wg;
+    const int wg_r1 = wg_r0 + rows_per_wg < n_rows ? wg_r0 + rows_per_wg : n_rows;
+    const int wave_r0 = wg_r0 + g * rows_per_wave;
+    const int wave_r1 = wave_r0 + rows_per_wave < wg_r1 ? wave_r0 + rows_per_wave : wg_r1;
+    const int rows_here = wave_r1 > wave_r0 ? wave_r1 - wave_r0 : 0;
+    const int nt_wave = (rows_here + RPT - 1) / RPT;  // real tasks of this wave (wave-uniform)
+
+    const uint32_t rowbytes = (uint32_t)spr * 144u;
+    const uint32_t chunk_off = (uint32_t)(h * SEG + (lt >> 3)) * 144u;
+    const uint32_t chunk_qoff = chunk_off + 16u + 16u * (uint32_t)j;
+    auto issue = [&](int t, uint4 &h4, uint4 &q4) {
+        const bool real = t < nt_wave;  // wave-uniform
+        int row = wave_r0 + t * RPT + tm;
+        if (RPT > 1) row = row < wave_r1 ? row : wave_r1 - 1;  // a ragged last task re-reads the last row
+        const uint32_t ro = real ? (uint32_t)row * rowbytes : 0u;
+        h4 = *reinterpret_cast<const uint4 *>(W + (ro + (real ? chunk_off : 0u)));
+        q4 = *reinterpret_cast<const uint4 *>(W + (ro + (real ? chunk_qoff : 0u)));
+    };
+
+    uint4 x_lo[kStagePre], x_hi[kStagePre];
+    stage_x_begin<ORDER, XF32>(xg, slots, nthreads, x_lo, x_hi);
+    uint4 bh[kDepth], bq[kDepth];
+#pragma unroll
+    for (int i = 0; i < kPre; i++) issue(i, bh[i], bq[i]);
+    PMH_STAMP(1);
+    stage_x_finish<ORDER, NDIG, XF32>(xg, slots, nthreads, x_lo, x_hi, xd, xm);
+    PMH_STAMP(2);
+    __syncthreads();
+    PMH_STAMP(3);
+
+    const ScaleSel s0 = scale_sel(ORDER == 0 ? j : 2 * (j >> 1));
+    const ScaleSel s1 = scale_sel(ORDER == 0 ? j : 2 * (j >> 1) + 1);
+    uint4 xr[NDIG];
+#pragma unroll
+    for (int k = 0; k < NDIG; k++) xr[k] = xd[k * slots + h * T + lt];
+    const float4 xmr = xm[h * T + lt];
+
+    // partial sums: row (g, t * RPT + tm) of the padded layout, column h * T + lt
+    const int npad = n_nominal * RPT;
+    float *pp = part + (size_t)(g * npad + tm) * ps + h * T + lt;
+    const int pstride = RPT * ps;  // floats between consecutive tasks
+
+    auto consume = [&](int t, const uint4 &h4, const uint4 &q4) {
+        if (t < nt_wave) pp[(size_t)t * pstride] = lane_dot<ORDER, NDIG>(h4, q4, s0, s1, xr, xmr);
+    };
+
+    // First round: the ring fills up while the first tasks are consumed (two requests per task consumed),
+    // so no wave sits in front of the load unit with nothing to compute.
+    int issued = kPre;
+#pragma unroll
+    for (int i = 0; i < kDepth; i++) {
+        consume(i, bh[i], bq[i]);
+        const int upto = SINGLE ? (kPre + 2 * (i + 1) < kDepth ? kPre + 2 * (i + 1) : kDepth)
+                                : (kPre + 2 * (i + 1) < kDepth + i + 1 ? kPre + 2 * (i + 1) : kDepth + i + 1);
+#pragma unroll
+        for (; issued < upto; issued++) issue(issued, bh[issued % kDepth], bq[issued % kDepth]);
+    }
+    PMH_STAMP(4);
+    if (!SINGLE) {
+        // steady rounds: consume task t, refill its buffer with task t + kDepth
+        int base = kDepth;
+        for (; base + kDepth < n_nominal; base += kDepth) {
+#pragma unroll
+            for (int i = 0; i < kDepth; i++) {
+                consume(base + i, bh[i], bq[i]);
+                issue(base + kDepth + i, bh[i], bq[i]);
+            }
+        }
+        // last round: nothing left to request
+#pragma unroll
+        for (int i = 0; i < kDepth; i++) consume(base + i, bh[i], bq[i]);
+    }
+    PMH_STAMP(5);
+    __syncthreads();
+
+    // Row totals: `red` lanes per row (a power of two from 8 to 64 that divides slots), lane p adding every
+    // red-th partial, then a sum over the lanes of the row.
+    const int wg_rows = wg_r1 - wg_r0;
+    const int per_thread = slots / red;
+    const int red_shift = 31 - __builtin_clz(red);
+    for (int idx0 = 0; idx0 < wg_rows * red; idx0 += nthreads) {
+        const int idx = idx0 + threadIdx.x;
+        int rl = idx >> red_shift;
+        const bool ok = rl < wg_rows;
+        rl = ok ? rl : wg_rows - 1;
+        const int grp = rl / rows_per_wave, loc = rl - grp * rows_per_wave;
+        const int p = idx & (red - 1);
+        const float *src = part + (size_t)(grp * npad + loc) * ps + p;
+        float t0 = 0.0f, t1 = 0.0f, t2 = 0.0f, t3 = 0.0f;
+        int i = 0;
+        for (; i + 8 <= per_thread; i += 8) {  // eight reads in flight
+            const float *q = src + (size_t)i * red;
+            const float a0 = q[0], a1 = q[red], a2 = q[2 * red], a3 = q[3 * red];
+            const float a4 = q[4 * red], a5 = q[5 * red], a6 = q[6 * red], a7 = q[7 * red];
+            t0 += a0 + a4, t1 += a1 + a5, t2 += a2 + a6, t3 += a3 + a7;
+        }
+        for (; i < per_thread; i++) t0 += src[(size_t)i * red];
+        const float sum = team_sum_rt((t0 + t1) + (t2 + t3), red);
+        if (ok && p == 0) y[wg_r0 + rl] = sum;
+    }
+    PMH_STAMP(6);
+    PMH_RT(7);
+    PMH_STAMP_FLUSH;
+}
+
+// ---- kernel B: general shapes -------------------------------------------------------------------
+// A team of T lanes walks a contiguous chunk of rows as one linear stream of tasks, T/8 * 144 bytes apart,
+// re-reading its x digits from LDS for every task and reducing with DPP at the end of every row.
+constexpr int kRing = 8;
+
+template <int ORDER, bool XF32, int T>
 __global__ __launch_bounds__(1024) void k_qgemv_q4k(const uint8_t *__restrict__ W, const void *__restrict__ xg,
                                                      float *__restrict__ y, int n_rows, int spr, int rows_per_wg,
-                                                     int per_team) {
+                                                     int per_team, int nthreads) {
     constexpr int NDIG = XF32 ? 6 : 5;
-    constexpr int SEG = T / 8;        // super-blocks a team covers per task
-    constexpr int STRIDE = SEG * 144; // bytes between a lane's consecutive tasks
-    constexpr int kDepth = Depth<ITERS>::value;
+    constexpr int SEG = T / 8;         // super-blocks a team covers per task
+    constexpr int STRIDE = SEG * 144;  // bytes between a lane's consecutive tasks
     extern __shared__ uint4 smem[];
     const int slots = spr * 8;
     uint4 *xd = smem;
     float4 *xm = reinterpret_cast<float4 *>(xd + NDIG * slots);
 
-    PMH_STAMP(0);
     const int lane = threadIdx.x & 63;
     const int lt = lane & (T - 1);
     const int j = lane & 7;
-    const int iters = ITERS ? ITERS : spr / SEG;  // tasks per row
+    const int iters = spr / SEG;  // tasks per row
     constexpr int kTeamsPerWave = 64 / T;
     // with full-wave teams everything about a team is wave-uniform: keep it in scalar registers
     auto uni = [](int v) { return T == 64 ? __builtin_amdgcn_readfirstlane(v) : v; };
@@ -279,85 +502,47 @@ __global__ __launch_bounds__(1024) void k_qgemv_q4k(const uint8_t *__restrict__ 
     const int n_tasks = (r1 > r0 ? r1 - r0 : 0) * iters;  // this team's tasks
     const int n_nominal = per_team * iters;               // workgroup-uniform upper bound
 
-    // The first pass of activation loads goes out before the weight loads queue up behind it.
-    const int stage_total = slots * 4;
-    float x_lo[4], x_hi[4];
-    if ((int)threadIdx.x < stage_total) {
-        size_t e_lo, e_hi;
-        stage_offsets<ORDER>(threadIdx.x, e_lo, e_hi);
-        load_x4<XF32>(xg, e_lo, x_lo);
-        load_x4<XF32>(xg, e_hi, x_hi);
-    }
-
     // A team's tasks are one linear stream: task t of the team starts STRIDE * t bytes after its first.
     const uint8_t *ph = W + (size_t)(n_tasks > 0 ? r0 : 0) * spr * 144 + (size_t)(lt >> 3) * 144;
     const uint8_t *pq = ph + 16 + 16 * j;
 
-    // kDepth tasks are in flight per team.  They are requested before x is converted, so the memory system
-    // streams while the staging runs, and each buffer is refilled as soon as it has been consumed.  (The
-    // load unit takes one 1 KiB wave-load per ~32 cycles and a wave stuck issuing loads cannot start
-    // converting x, so a deeper initial burst does not pay.)
-    uint4 bh[kDepth], bq[kDepth];
+    // kRing tasks are in flight per team.  They are requested before x is converted, so the memory system
+    // streams while the staging runs, and each buffer is refilled as soon as it has been consumed.
+    uint4 x_lo[kStagePre], x_hi[kStagePre];
+    stage_x_begin<ORDER, XF32>(xg, slots, nthreads, x_lo, x_hi);
+    uint4 bh[kRing], bq[kRing];
 #pragma unroll
-    for (int i = 0; i < kDepth; i++) {
+    for (int i = 0; i < kRing; i++) {
         if (i < n_tasks) {
             bh[i] = *reinterpret_cast<const uint4 *>(ph + i * STRIDE);
             bq[i] = *reinterpret_cast<const uint4 *>(pq + i * STRIDE);
         }
     }
-    PMH_STAMP(1);
-
-    if ((int)threadIdx.x < stage_total) stage_convert<NDIG, XF32>(threadIdx.x, x_lo, x_hi, slots, xd, xm);
-    for (int idx = threadIdx.x + blockDim.x; idx < stage_total; idx += blockDim.x) {  // long rows: more passes
-        size_t e_lo, e_hi;
-        stage_offsets<ORDER>(idx, e_lo, e_hi);
-        load_x4<XF32>(xg, e_lo, x_lo);
-        load_x4<XF32>(xg, e_hi, x_hi);
-        stage_convert<NDIG, XF32>(idx, x_lo, x_hi, slots, xd, xm);
-    }
-    PMH_STAMP(2);
+    stage_x_finish<ORDER, NDIG, XF32>(xg, slots, nthreads, x_lo, x_hi, xd, xm);
     __syncthreads();
-    PMH_STAMP(3);
 
     const ScaleSel s0 = scale_sel(ORDER == 0 ? j : 2 * (j >> 1));
     const ScaleSel s1 = scale_sel(ORDER == 0 ? j : 2 * (j >> 1) + 1);
-    // register-resident x: slot (it * T + lt) for it < ITERS
-    uint4 xr[ITERS ? ITERS : 1][NDIG];
-    float4 xmr[ITERS ? ITERS : 1];
-    if (ITERS) {
-#pragma unroll
-        for (int t = 0; t < ITERS; t++) {
-#pragma unroll
-            for (int k = 0; k < NDIG; k++) xr[t][k] = xd[k * slots + t * T + lt];
-            xmr[t] = xm[t * T + lt];
-        }
-    }
     float acc = 0.0f;
     int it = 0;  // position inside the row: the same for every team of the workgroup
     int row = r0;
-    for (int first = 0; first < n_nominal; first += kDepth) {
+    for (int first = 0; first < n_nominal; first += kRing) {
 #pragma unroll
-        for (int i = 0; i < kDepth; i++) {
+        for (int i = 0; i < kRing; i++) {
             if (first + i < n_nominal) {
                 const bool valid = first + i < n_tasks;
                 if (valid) {
-                    if (ITERS) {  // kDepth is a multiple of ITERS, so the position in the row is static
-                        acc += lane_dot<ORDER, NDIG>(bh[i], bq[i], s0, s1, xr[i % (ITERS ? ITERS : 1)],
-                                                     xmr[i % (ITERS ? ITERS : 1)]);
-                    } else {
-                        const int slot = it * T + lt;
-                        uint4 xdig[NDIG];
+                    const int slot = it * T + lt;
+                    uint4 xdig[NDIG];
 #pragma unroll
-                        for (int k = 0; k < NDIG; k++) xdig[k] = xd[k * slots + slot];
-                        acc += lane_dot<ORDER, NDIG>(bh[i], bq[i], s0, s1, xdig, xm[slot]);
-                    }
+                    for (int k = 0; k < NDIG; k++) xdig[k] = xd[k * slots + slot];
+                    acc += lane_dot<ORDER, NDIG>(bh[i], bq[i], s0, s1, xdig, xm[slot]);
                 }
-                if (first + i + kDepth < n_tasks) {  // refill this buffer with the task kDepth ahead
-                    bh[i] = *reinterpret_cast<const uint4 *>(ph + (size_t)(i + kDepth) * STRIDE);
-                    bq[i] = *reinterpret_cast<const uint4 *>(pq + (size_t)(i + kDepth) * STRIDE);
+                if (first + i + kRing < n_tasks) {  // refill this buffer with the task kRing ahead
+                    bh[i] = *reinterpret_cast<const uint4 *>(ph + (size_t)(i + kRing) * STRIDE);
+                    bq[i] = *reinterpret_cast<const uint4 *>(pq + (size_t)(i + kRing) * STRIDE);
                 }
-                const bool row_end = ITERS ? (i % (ITERS ? ITERS : 1) == ITERS - 1) : (++it == iters);
-                if (row_end) {
+                if (++it == iters) {
                     const float total = team_sum_last<T>(acc);
                     if (lt == T - 1 && valid) y[row] = total;
                     row++;
@@ -366,36 +551,47 @@ __global__ __launch_bounds__(1024) void k_qgemv_q4k(const uint8_t *__restrict__ 
                 }
             }
         }
-        ph += kDepth * STRIDE;
-        pq += kDepth * STRIDE;
-        PMH_STAMP(4 + ((first / kDepth) & 3));
+        ph += kRing * STRIDE;
+        pq += kRing * STRIDE;
     }
 }
 
+template <typename Kern, typename... Args>
+hipError_t launch_with_lds(Kern kern, dim3 grid, dim3 block, size_t lds, hipStream_t s, Args... args) {
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(kern, grid, block, lds, s, args...);
+    return hipGetLastError();
+}
+
 template <int ORDER, bool XF32>
-hipError_t launch_cfg(int T, dim3 grid, dim3 block, size_t lds, hipStream_t s, const uint8_t *w, const void *x,
-                      float *y, int n, int spr, int rows_per_wg, int per_team) {
-    auto go = [&](auto kern) -> hipError_t {
-        if (lds > 64 * 1024) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e != hipSuccess) return e;
-        }
-        hipLaunchKernelGGL(kern, grid, block, lds, s, w, x, y, n, spr, rows_per_wg, per_team);
-        return hipGetLastError();
-    };
-    const int iters = spr / (T / 8);
-    const bool xreg = iters <= 2 && !XF32 && ORDER == 0;  // the headline path keeps x in registers
+hipError_t launch_chunk(int T, bool single, dim3 grid, dim3 block, size_t lds, hipStream_t s, const uint8_t *w,
+                        const void *x, float *y, int n, int spr, int rows_per_wg, int rows_per_wave, int n_nominal, int red) {
+#define PMH_GO(TT)                                                                                                  \
+    return single ? launch_with_lds(k_qgemv_q4k_chunk<ORDER, XF32, TT, true>, grid, block, lds, s, w, x, y, n, spr, \
+                                    rows_per_wg, rows_per_wave, n_nominal, red, (int)block.x)                       \
+                  : launch_with_lds(k_qgemv_q4k_chunk<ORDER, XF32, TT, false>, grid, block, lds, s, w, x, y, n, spr, \
+                                    rows_per_wg, rows_per_wave, n_nominal, red, (int)block.x)
     switch (T) {
-    case 8: return go(k_qgemv_q4k<ORDER, XF32, 8, 0>);
-    case 16: return go(k_qgemv_q4k<ORDER, XF32, 16, 0>);
-    case 32:
-        if (xreg && iters == 1) return go(k_qgemv_q4k<ORDER, XF32, 32, 1>);
-        return go(k_qgemv_q4k<ORDER, XF32, 32, 0>);
-    default:
-        if (xreg && iters == 1) return go(k_qgemv_q4k<ORDER, XF32, 64, 1>);
-        if (xreg && iters == 2) return go(k_qgemv_q4k<ORDER, XF32, 64, 2>);
-        return go(k_qgemv_q4k<ORDER, XF32, 64, 0>);
+    case 8: PMH_GO(8);
+    case 16: PMH_GO(16);
+    case 32: PMH_GO(32);
+    default: PMH_GO(64);
+    }
+#undef PMH_GO
+}
+
+template <int ORDER, bool XF32>
+hipError_t launch_general(int T, dim3 grid, dim3 block, size_t lds, hipStream_t s, const uint8_t *w, const void *x,
+                          float *y, int n, int spr, int rows_per_wg, int per_team) {
+    switch (T) {
+    case 8: return launch_with_lds(k_qgemv_q4k<ORDER, XF32, 8>, grid, block, lds, s, w, x, y, n, spr, rows_per_wg, per_team, (int)block.x);
+    case 16: return launch_with_lds(k_qgemv_q4k<ORDER, XF32, 16>, grid, block, lds, s, w, x, y, n, spr, rows_per_wg, per_team, (int)block.x);
+    case 32: return launch_with_lds(k_qgemv_q4k<ORDER, XF32, 32>, grid, block, lds, s, w, x, y, n, spr, rows_per_wg, per_team, (int)block.x);
+    default: return launch_with_lds(k_qgemv_q4k<ORDER, XF32, 64>, grid, block, lds, s, w, x, y, n, spr, rows_per_wg, per_team, (int)block.x);
     }
 }
 
@@ -410,17 +606,50 @@ hipError_t launch_qgemv_q4k(const uint8_t *w, int64_t n, int64_t k, const void *
     const int spr = (int)(k / 256);
     const int T = 8 * gemv::pow2_divisor(spr, 8);
     const size_t slots = (size_t)spr * 8;
-    const size_t lds = slots * 16 * (xf32 ? 6 : 5) + slots * 16;
-    if (lds > gemv::kMaxLds) return hipErrorInvalidValue;
+    const size_t lds_x = slots * 16 * (xf32 ? 6 : 5) + slots * 16;
+    if (lds_x > gemv::kMaxLds) return hipErrorInvalidValue;
 
-    // Workgroups own contiguous chunks of rows, about `wgs_per_cu` per compute unit (x is staged once
-    // per workgroup), up to 16 waves each; the wave count is the largest that keeps the busiest team's
-    // row count minimal.
+    // Workgroups own contiguous chunks of rows, about `wgs_per_cu` per compute unit (x is staged once per
+    // workgroup).
     const int64_t wgs_per_cu = gemv::tuning("PMETAL_HIP_GEMV_WGS_PER_CU", 1);
     const int64_t want = (int64_t)gemv::compute_units() * (wgs_per_cu > 0 ? wgs_per_cu : 1);
     int64_t n_wg = n < want ? n : want;
     const int64_t rows_per_wg = (n + n_wg - 1) / n_wg;
     n_wg = (n + rows_per_wg - 1) / rows_per_wg;
+    const dim3 grid((unsigned)n_wg);
+
+    // Kernel A when a row is at most 16 chunks, offsets fit 32 bits, the partial sums fit in LDS and there is
+    // enough work per compute unit to pay for its second barrier (measured crossover: about 12 MiB of weights).
+    const int ks = spr / (T / 8), rpt = 64 / T;
+    const uint64_t w_bytes = (uint64_t)n * (uint64_t)spr * 144u;
+    const int64_t mode = gemv::tuning("PMETAL_HIP_GEMV_KERNEL", 0);  // 0 = choose, 1 = kernel A, 2 = kernel B
+    const bool want_a = mode == 1 || (mode == 0 && w_bytes >= (12ull << 20));
+    if (want_a && ks <= 16 && w_bytes < (1ull << 32)) {
+        const int64_t max_waves = gemv::tuning("PMETAL_HIP_GEMV_WAVES", 16);
+        int64_t groups = (max_waves >= ks && max_waves <= 16 ? max_waves : 16) / ks;
+        const int64_t max_groups = (rows_per_wg + rpt - 1) / rpt;
+        if (groups > max_groups) groups = max_groups;
+        const int64_t rows_per_wave = (rows_per_wg + groups - 1) / groups;
+        groups = (rows_per_wg + rows_per_wave - 1) / rows_per_wave;
+        const int64_t n_nominal = (rows_per_wave + rpt - 1) / rpt;
+        const int64_t threads = ks * groups * 64;
+        int red = 8;  // lanes per row in the final summation: as many as the workgroup has to spare, at most T
+        const int64_t red_cap = gemv::tuning("PMETAL_HIP_GEMV_RED", 64);
+        while (red < red_cap && red * 2 <= T && rows_per_wg * red * 2 <= threads) red *= 2;
+        const size_t lds = lds_x + (size_t)groups * (size_t)n_nominal * rpt * part_stride((int)slots, red) * 4;
+        if (lds <= 128 * 1024) {
+            const dim3 block((unsigned)threads);
+            const bool single = n_nominal <= kDepth;
+            const int a_n = (int)n, a_rpw = (int)rows_per_wg, a_rpv = (int)rows_per_wave, a_nn = (int)n_nominal;
+            if (order == kOrderRef)
+                return xf32 ? launch_chunk<0, true>(T, single, grid, block, lds, s, w, x, y, a_n, spr, a_rpw, a_rpv, a_nn, red)
+                            : launch_chunk<0, false>(T, single, grid, block, lds, s, w, x, y, a_n, spr, a_rpw, a_rpv, a_nn, red);
+            return xf32 ? launch_chunk<1, true>(T, single, grid, block, lds, s, w, x, y, a_n, spr, a_rpw, a_rpv, a_nn, red)
+                        : launch_chunk<1, false>(T, single, grid, block, lds, s, w, x, y, a_n, spr, a_rpw, a_rpv, a_nn, red);
+        }
+    }
+
+    // Kernel B: up to 16 waves; the wave count is the largest that keeps the busiest team's row count minimal.
     const int teams_per_wave = 64 / T;
     int best_waves = 16;
     int64_t best_cost = INT64_MAX;
@@ -429,15 +658,13 @@ hipError_t launch_qgemv_q4k(const uint8_t *w, int64_t n, int64_t k, const void *
         const int64_t per_team = (rows_per_wg + teams - 1) / teams;
         if (per_team < best_cost) best_cost = per_team, best_waves = waves;
     }
-    const int forced = (int)gemv::tuning("PMETAL_HIP_GEMV_WAVES", 0);
-    if (forced >= 1 && forced <= 16) best_waves = forced;
     const int per_team = (int)((rows_per_wg + (int64_t)best_waves * teams_per_wave - 1) / ((int64_t)best_waves * teams_per_wave));
-    const dim3 grid((unsigned)n_wg), block((unsigned)best_waves * 64);
+    const dim3 block((unsigned)best_waves * 64);
     if (order == kOrderRef)
-        return xf32 ? launch_cfg<0, true>(T, grid, block, lds, s, w, x, y, (int)n, spr, (int)rows_per_wg, per_team)
-                    : launch_cfg<0, false>(T, grid, block, lds, s, w, x, y, (int)n, spr, (int)rows_per_wg, per_team);
-    return xf32 ? launch_cfg<1, true>(T, grid, block, lds, s, w, x, y, (int)n, spr, (int)rows_per_wg, per_team)
-                : launch_cfg<1, false>(T, grid, block, lds, s, w, x, y, (int)n, spr, (int)rows_per_wg, per_team);
+        return xf32 ? launch_general<0, true>(T, grid, block, lds_x, s, w, x, y, (int)n, spr, (int)rows_per_wg, per_team)
+                    : launch_general<0, false>(T, grid, block, lds_x, s, w, x, y, (int)n, spr, (int)rows_per_wg, per_team);
+    return xf32 ? launch_general<1, true>(T, grid, block, lds_x, s, w, x, y, (int)n, spr, (int)rows_per_wg, per_team)
+                : launch_general<1, false>(T, grid, block, lds_x, s, w, x, y, (int)n, spr, (int)rows_per_wg, per_team);
 }
 
 }  // namespace pmh
