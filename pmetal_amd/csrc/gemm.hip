@@ -12,18 +12,22 @@
 //     B tile  = sc * q             an integer <= 63 * 15 = 945          (f16 holds integers to 2048)
 //     A tile  = x * 2^-e_m         bf16 activations are exact in f16 once a per-row power of two keeps
 //                                  them below 2^10 (a pre-pass does that and sums x per 32-element block)
-// and the per-super-block factors are applied to the fp32 partial sums:
-//     Y[m,n] = 2^e_m * sum_SB ( d[n,SB] * P_SB[m,n] - dmin[n,SB] * Q_SB[m,n] )
-//     P_SB = sum_{k in SB} A[m,k] * B[n,k]            16 x v_mfma_f32_32x32x16_f16 per 32x32 block
-//     Q_SB = sum_{j<8} m[n,j] * xsum[m,j]             one more MFMA: xsum as f16 hi + lo, m exact
-// so the only roundings are the fp32 accumulations.
+// and the per-super-block factor d is applied to the fp32 partial sums:
+//     Y[m,n] = 2^e_m * sum_SB ( d[n,SB] * P_SB[m,n] + R_SB[m,n] )
+//     P_SB = sum_{k in SB} A[m,k] * B[n,k]              16 x v_mfma_f32_32x32x16_f16 per 32x32 block
+//     R_SB = - sum_{j<8} (dmin[n,SB] * m[n,j]) * xsum[m,j]
+// R_SB also runs on the matrix core, straight into the accumulators: dmin * m (17 significant bits) and the
+// block sums xsum are each split exactly into an f16 head and tail, and the four cross products of the
+// eight sub-blocks make one K = 32 product (two more MFMAs per block and super-block).  The only roundings
+// are the fp32 accumulations.
 //
-// Tiling: a workgroup of 256 threads (4 waves) computes a BM x 128 tile of Y (BM = 128, or 64 / 32 for
-// short activation batches); for BM = 128 the waves form a 2 x 2 grid and each owns 2 x 2 MFMA blocks.  K advances two 32-element sub-blocks per stage: every thread dequantizes
-// 32 weights (one 16-byte piece, both nibble planes) into the B tile and copies 4 x 8 activations into the
-// A tile (a wave reads 8 rows x 128 contiguous bytes per load); both tiles are stored in LDS in MFMA
-// operand order ([k-step][k-group][row] items of 16 bytes) so the operand reads are conflict-free
-// ds_read_b128.  Global loads run two stages ahead in registers, the LDS stages are double buffered.
+// Tiling: a workgroup of 8, 4 or 2 waves computes a 256 x 128, 128 x 128 or 64 x 32 tile of Y (by the number
+// of activation rows); every wave owns 2 x 2 (or one) MFMA blocks.  K advances 64 elements per stage.  The pre-pass
+// stores the activations as 16-byte items (8 consecutive k of one row) in [k / 8][m] order, so that a wave
+// copies 64 consecutive items from global memory to LDS: coalesced reads, conflict-free writes, and the
+// items lie in LDS exactly as the MFMA A operand wants them ([k-step][k-group][row]).  The B tile is
+// dequantized by the whole workgroup once per stage into the same operand order.  Global loads run two
+// stages ahead in registers, the LDS stages are double buffered, one barrier per stage.
 #include "internal.hpp"
 
 namespace {
@@ -31,9 +35,9 @@ namespace {
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // 16 bytes in registers
 
-constexpr int BN = 128;  // workgroup tile width (weight rows); the height BM is a template parameter
-constexpr int kThreads = 256;
+constexpr int kMPad = 256; // the pre-pass pads the activation rows to a multiple of this
 
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
     return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
@@ -42,74 +46,108 @@ __device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
 __device__ __forceinline__ float bf16_to_f32(uint32_t h) { return __builtin_bit_cast(float, h << 16); }
 
 // ------------------------------------------------------------------------------------------------
-// Pre-pass over the activations: one workgroup per row m.
-//   xs[m][k]            = f16( x[m][k] * 2^-e_m )          exact
-//   xsum[m][sb][0 / 1]  = hi / lo f16 split of sum_{k in 32-block sb} xs[m][k]
-//   rowscale[m]         = 2^e_m
-// e_m normalises the row maximum into [2^9, 2^10): block sums (< 2^15) fit f16 and small rows stay out of
-// the f16 subnormal range.
+// Pre-pass 1: one wave per row m (rows up to Mp, a multiple of 4): rowscale[m] = 2^e_m with the row maximum * 2^-e_m in [2^9, 2^10),
+// so that block sums (< 2^15) fit f16 and small rows stay out of the f16 subnormal range.
 // ------------------------------------------------------------------------------------------------
 template <bool XF32>
-__global__ __launch_bounds__(256) void k_prep_x(const void *__restrict__ xg, int64_t k, _Float16 *__restrict__ xs,
-                                                 _Float16 *__restrict__ xsum, float *__restrict__ rowscale) {
-    __shared__ float red[4];
-    const int64_t m = blockIdx.x;
-    const int tid = threadIdx.x;
-    auto load = [&](int64_t i) -> float {
-        if (XF32) return reinterpret_cast<const float *>(xg)[m * k + i];
-        return bf16_to_f32(reinterpret_cast<const uint16_t *>(xg)[m * k + i]);
-    };
+__global__ __launch_bounds__(256) void k_prep_scale(const void *__restrict__ xg, int64_t k, int M,
+                                                     float *__restrict__ rowscale) {
+    // one wave per row, 16-byte loads (k is a multiple of 256)
+    const int64_t m = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
     float amax = 0.0f;
-    for (int64_t i = tid; i < k; i += 256) amax = __builtin_fmaxf(amax, __builtin_fabsf(load(i)));
-    for (int off = 32; off > 0; off >>= 1) amax = __builtin_fmaxf(amax, __shfl_xor(amax, off));
-    if ((tid & 63) == 0) red[tid >> 6] = amax;
-    __syncthreads();
-    amax = __builtin_fmaxf(__builtin_fmaxf(red[0], red[1]), __builtin_fmaxf(red[2], red[3]));
-    // 2^e with amax * 2^-e < 2^10, so that the sum of a 32-element block (< 2^15) also fits f16
-    const int eb = (int)((__builtin_bit_cast(uint32_t, amax) >> 23) & 0xFFu);  // amax in [2^(eb-127), 2^(eb-126))
-    int e = eb - 126 - 10;  // also scales small rows up, out of the f16 subnormal range
-    e = e < -126 ? -126 : (e > 126 ? 126 : e);
-    if (eb == 255) e = 0;  // inf / NaN: let them through
-    const float down = __builtin_bit_cast(float, (uint32_t)(127 - e) << 23);
-    if (tid == 0) rowscale[m] = __builtin_bit_cast(float, (uint32_t)(127 + e) << 23);
-    // 32-element blocks: 8 lanes per block, 4 elements per lane
-    const int64_t n_sb = k / 32;
-    for (int64_t blk = tid >> 3; blk < n_sb; blk += 32) {
-        const int part = tid & 7;
-        float s = 0.0f;
-        _Float16 out[4];
+    if (m < M) {
+        if (XF32) {
+            const float4 *row = reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(xg) + m * k);
+            for (int64_t i = lane; i < k / 4; i += 64) {
+                const float4 v = row[i];
+                amax = __builtin_fmaxf(__builtin_fmaxf(amax, __builtin_fmaxf(__builtin_fabsf(v.x), __builtin_fabsf(v.y))),
+                                       __builtin_fmaxf(__builtin_fabsf(v.z), __builtin_fabsf(v.w)));
+            }
+        } else {
+            const uint4 *row = reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(xg) + m * k);
+            for (int64_t i = lane; i < k / 8; i += 64) {
+                const uint4 v = row[i];
+                const uint32_t r[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            const _Float16 h = (_Float16)(load(blk * 32 + part * 4 + c) * down);
-            out[c] = h;
-            s += (float)h;
-        }
-        *reinterpret_cast<uint2 *>(xs + m * k + blk * 32 + part * 4) = *reinterpret_cast<const uint2 *>(out);
-        s += __shfl_xor(s, 1);
-        s += __shfl_xor(s, 2);
-        s += __shfl_xor(s, 4);
-        if (part == 0) {
-            const _Float16 hi = (_Float16)s;
-            const _Float16 lo = (_Float16)(s - (float)hi);
-            xsum[(m * n_sb + blk) * 2] = hi;
-            xsum[(m * n_sb + blk) * 2 + 1] = lo;
+                for (int q = 0; q < 4; q++)
+                    amax = __builtin_fmaxf(amax, __builtin_fmaxf(__builtin_fabsf(bf16_to_f32(r[q] & 0xFFFFu)),
+                                                                 __builtin_fabsf(bf16_to_f32(r[q] >> 16))));
+            }
         }
     }
+    for (int off = 32; off > 0; off >>= 1) amax = __builtin_fmaxf(amax, __shfl_xor(amax, off));
+    const int eb = (int)((__builtin_bit_cast(uint32_t, amax) >> 23) & 0xFFu);  // amax in [2^(eb-127), 2^(eb-126))
+    int e = eb - 126 - 10;
+    e = e < -126 ? -126 : (e > 126 ? 126 : e);
+    if (eb == 255) e = 0;  // inf / NaN: let them through
+    if (lane == 0) rowscale[m] = __builtin_bit_cast(float, (uint32_t)(127 + e) << 23);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Pre-pass 2: grid (Mp / 64, k / 256), 256 threads; lane = row, wave w = sub-blocks 2w and 2w + 1 of the
+// super-block.
+//   xs   [k / 8][Mp]               items of 8 f16: x[m][8c .. 8c+7] * 2^-e_m   (rows >= M are zero)
+//   xsum [k / 256][2][2][Mp]       items of 8 f16 for the R_SB product, item (t, g) of row m =
+//                                  (h_j, l_j, h_j, l_j, h_j+1, l_j+1, h_j+1, l_j+1),  j = 4 t + 2 g,
+//                                  h + l = sum of the 32 scaled activations of sub-block j (exact split)
+// ------------------------------------------------------------------------------------------------
+template <bool XF32>
+__global__ __launch_bounds__(256) void k_prep_tiles(const void *__restrict__ xg, int64_t k, int M, int Mp,
+                                                     const float *__restrict__ rowscale, uint4 *__restrict__ xs,
+                                                     uint4 *__restrict__ xsum) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int m = blockIdx.x * 64 + lane;
+    const int64_t sb = blockIdx.y;
+    const bool live = m < M;
+    const float down = live ? 1.0f / rowscale[m] : 0.0f;  // exact: a power of two
+    _Float16 hl[4];
+#pragma unroll
+    for (int s = 0; s < 2; s++) {
+        const int64_t k0 = sb * 256 + (2 * w + s) * 32;
+        float sum = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            float v[8];
+            if (!live) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) v[i] = 0.0f;
+            } else if (XF32) {
+                const float4 a = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(xg) + (int64_t)m * k + k0 + 8 * c);
+                const float4 b = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(xg) + (int64_t)m * k + k0 + 8 * c + 4);
+                v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
+            } else {
+                const uint4 u = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(xg) + (int64_t)m * k + k0 + 8 * c);
+                const uint32_t r[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+                for (int i = 0; i < 4; i++) v[2 * i] = bf16_to_f32(r[i] & 0xFFFFu), v[2 * i + 1] = bf16_to_f32(r[i] >> 16);
+            }
+            half8_t h;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                h[i] = (_Float16)(v[i] * down);
+                sum += (float)h[i];
+            }
+            xs[(size_t)(k0 / 8 + c) * Mp + m] = __builtin_bit_cast(uint4, h);
+        }
+        hl[2 * s] = (_Float16)sum;
+        hl[2 * s + 1] = (_Float16)(sum - (float)hl[2 * s]);
+    }
+    half8_t item = {hl[0], hl[1], hl[0], hl[1], hl[2], hl[3], hl[2], hl[3]};
+    // j = 2 w = 4 t + 2 g
+    xsum[((size_t)sb * 4 + w) * Mp + m] = __builtin_bit_cast(uint4, item);
 }
 
 // ------------------------------------------------------------------------------------------------
 // main kernel
 // ------------------------------------------------------------------------------------------------
-// K advances 64 elements (two sub-blocks) per stage.  LDS stage: A then B tile, each
-// [4 MFMA k-steps][2 k-groups][128 rows] items of 8 f16 (16 bytes) = 16 KiB; two stages.
-constexpr int BK = 64;
-constexpr int kItemsB = 4 * 2 * BN;  // uint4 items of the B tile per stage
-
 // 16 nibbles (one plane of a 16-byte piece) times the integer scale -> 16 exact f16 values.
 // 0x6400 | q is the f16 1024 + q; (1024 + q) * sc - 1024 * sc is exact in a packed f16 fma.
-__device__ __forceinline__ void dequant16(const uint4 piece, const int plane, const float sc, uint4 &lo8, uint4 &hi8) {
-    const half2_t sc2 = {(_Float16)sc, (_Float16)sc};
-    const half2_t off2 = {(_Float16)(-1024.0f * sc), (_Float16)(-1024.0f * sc)};  // exact: sc <= 63
+__device__ __forceinline__ void dequant16(const uint4 piece, const int plane, const uint32_t sc, uint4 &lo8, uint4 &hi8) {
+    const _Float16 s = (_Float16)(float)sc;
+    const half2_t sc2 = {s, s};
+    const _Float16 o = (_Float16)(-1024.0f * (float)sc);  // exact: sc <= 63
+    const half2_t off2 = {o, o};
     const uint32_t w[4] = {piece.x, piece.y, piece.z, piece.w};
     uint32_t out[8];
 #pragma unroll
@@ -128,206 +166,259 @@ __device__ __forceinline__ void dequant16(const uint4 piece, const int plane, co
     hi8 = make_uint4(out[4], out[5], out[6], out[7]);
 }
 
-// (scale, min) of sub-block j from the 12 scale bytes (quantize.rs:844-855).
+// (scale, min) of sub-block j from the 12 scale bytes (quantize.rs:844-855); j is a compile-time constant
+// wherever this is called, so the branch folds.
 __device__ __forceinline__ void scale_min_u(const uint4 hdr, const int j, uint32_t &sc, uint32_t &mn) {
     const int sh = 8 * (j & 3);
-    const uint32_t a = (hdr.y >> sh) & 0xFFu, b = (hdr.z >> sh) & 0xFFu, c = (hdr.w >> sh) & 0xFFu;
     if (j < 4) {
-        sc = a & 63u;
-        mn = b & 63u;
+        sc = (hdr.y >> sh) & 63u;
+        mn = (hdr.z >> sh) & 63u;
     } else {
-        sc = (c & 0xFu) | ((a >> 6) << 4);
-        mn = (c >> 4) | ((b >> 6) << 4);
+        const uint32_t c = hdr.w >> sh;
+        sc = (c & 0xFu) | (((hdr.y >> (sh + 6)) & 3u) << 4);
+        mn = ((c >> 4) & 0xFu) | (((hdr.z >> (sh + 6)) & 3u) << 4);
     }
 }
 
-// The 4 waves form a WAVES_M x (4 / WAVES_M) grid; each wave owns BLK_M x BLK_N MFMA blocks of 32 x 32:
-//   BM = 128: 2 x 2 waves of 2 x 2 blocks      BM = 64: 1 x 4 waves of 2 x 1      BM = 32: 1 x 4 waves of 1 x 1
-template <int ORDER, bool YBF16, int WAVES_M, int BLK_M>
-__global__ __launch_bounds__(kThreads, 2) void k_qgemm_q4k(const uint8_t *__restrict__ W,
-                                                            const _Float16 *__restrict__ xs,
-                                                            const _Float16 *__restrict__ xsum,
-                                                            const float *__restrict__ rowscale, void *__restrict__ yg,
-                                                            int M, int N, int spr) {
-    constexpr int WAVES_N = 4 / WAVES_M;
-    constexpr int BLK_N = BN / 32 / WAVES_N;
-    constexpr int BM = WAVES_M * BLK_M * 32;
-    constexpr int RA = BM / 32;  // A-tile rows copied per thread and stage
-    __shared__ uint4 lds_a[2][8 * BM];  // [stage][(k-step, k-group) = chunk][row]
-    __shared__ uint4 lds_b[2][kItemsB];
+// -(dmin * mn) split exactly into an f16 head and tail (dmin has 11 significant bits, mn 6).
+__device__ __forceinline__ void neg_min_split(const float dmin, const uint32_t mn, _Float16 &h, _Float16 &l) {
+    const float p = -(dmin * (float)mn);  // exact in fp32
+    h = (_Float16)p;
+    l = (_Float16)(p - (float)h);
+}
+
+// Workgroup = WM x WN waves, every wave owns NB x NB MFMA blocks of 32 x 32:
+//   <4, 2, 2>: 256 x 128 tile, 512 threads      <2, 2, 2>: 128 x 128, 256 threads      <2, 1, 1>: 64 x 32, 128 threads
+template <int WM, int WN, int NB>
+struct Tile {
+    static constexpr int BM = 32 * NB * WM, BN = 32 * NB * WN, kThreads = 64 * WM * WN;
+    static constexpr int kUnits = kThreads / BN;   // threads per weight row
+    static constexpr int kBTasks = 4 / kUnits;     // (piece, plane) tasks per thread and stage
+    static constexpr int kPieces = kBTasks == 4 ? 2 : 1;
+    static constexpr int kAItems = 8 * BM / kThreads;  // A items per thread and stage
+    static constexpr size_t kLdsBytes = (size_t)(2 * 8 * BM + 2 * 8 * BN + 4 * BN) * 16 + BN * 4;
+    static_assert(kUnits == 1 || kUnits == 2 || kUnits == 4, "a weight row is staged by 1, 2 or 4 threads");
+    static_assert(8 * BM % kThreads == 0, "the A tile must divide among the threads");
+};
+
+template <int ORDER, bool YBF16, int WM, int WN, int NB>
+__global__ __launch_bounds__(64 * WM * WN, NB == 1 ? 2 : 512 / (64 * WM * WN)) void k_qgemm_q4k(
+    const uint8_t *__restrict__ W, const uint4 *__restrict__ xs, const uint4 *__restrict__ xsum,
+    const float *__restrict__ rowscale, void *__restrict__ yg, int M, int Mp, int N, int spr) {
+    using TL = Tile<WM, WN, NB>;
+    constexpr int BM = TL::BM, BN = TL::BN, kThreads = TL::kThreads, kUnits = TL::kUnits, kBTasks = TL::kBTasks,
+                  kPieces = TL::kPieces, kAItems = TL::kAItems;
+    // LDS: two stages of the A tile [8 chunks][BM] and the B tile [4 k-steps][2 k-groups][BN] (16-byte items),
+    // the B operand of the R product [2][2][BN] and d [BN] of the current super-block.
+    extern __shared__ uint4 smem[];
+    uint4 *lds_a = smem;
+    uint4 *lds_b = lds_a + 2 * 8 * BM;
+    uint4 *lds_r = lds_b + 2 * 8 * BN;
+    float *lds_d = reinterpret_cast<float *>(lds_r + 4 * BN);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WAVES_N, wn = wave % WAVES_N;  // wave position in the grid
+    const int wm = wave / WN, wn = wave % WN;  // wave position in the WM x WN grid
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-    const int K = spr * 256;
     const size_t row_bytes = (size_t)spr * 144;
 
     // ---- loader roles ----
-    // A: thread (row = tid / 8 + 32 r, chunk c = tid % 8) copies 8 f16 at k = 8 c: a wave reads 8 rows x 128 B
-    const int ac = tid & 7, ar = tid >> 3;
-    const _Float16 *xrow[RA];
-#pragma unroll
-    for (int r = 0; r < RA; r++) {
-        const int row = m0 + ar + 32 * r;
-        xrow[r] = xs + (size_t)(row < M ? row : M - 1) * K + 8 * ac;  // rows past M are computed and dropped
-    }
-    // B: thread (n = tid / 2, w = tid % 2) dequantizes both nibble planes of one 16-byte piece per stage
-    const int bn = tid >> 1, bw = tid & 1;
+    // A: item idx = tid + i * kThreads (i < kAItems) -> chunk = idx / BM, row = idx % BM: a wave copies 64
+    //    consecutive items.
+    // B: weight row bn = tid % BN, unit bu = tid / BN; (piece, plane) task q = bu * kBTasks + t,
+    //    piece = q / 2, plane = q % 2.
+    const int bn = tid % BN, bu = tid / BN;
     const uint8_t *wrow = W + (size_t)(n0 + bn < N ? n0 + bn : N - 1) * row_bytes;
 
-    struct Fetch {
-        uint4 a[RA], hdr, piece;
-    };
-    auto fetch = [&](int step, Fetch &f) {
+    // One stage's global data in registers: the A items of this thread, and for B the super-block header and
+    // one or two 16-byte pieces.  Steps past the end re-read the last one, so every load is unconditional.
+    const int last_step = spr * 4 - 1;
+    auto fetch_a = [&](int step, u32x4 (&fa)[kAItems]) __attribute__((always_inline)) {
+        step = step < last_step ? step : last_step;
 #pragma unroll
-        for (int r = 0; r < RA; r++) f.a[r] = *reinterpret_cast<const uint4 *>(xrow[r] + (size_t)step * BK);
+        for (int i = 0; i < kAItems; i++) {
+            const int idx = tid + i * kThreads;
+            fa[i] = *reinterpret_cast<const u32x4 *>(xs + (size_t)(step * 8 + idx / BM) * Mp + m0 + idx % BM);
+        }
+    };
+    auto fetch_b = [&](int step, u32x4 &fhdr, u32x4 (&fpc)[kPieces]) __attribute__((always_inline)) {
+        step = step < last_step ? step : last_step;
         const uint8_t *blk = wrow + (size_t)(step >> 2) * 144;
-        f.hdr = *reinterpret_cast<const uint4 *>(blk);
+        fhdr = *reinterpret_cast<const u32x4 *>(blk);
         // the stage covers sub-blocks 2c and 2c+1, c = step % 4, which are pieces 2c and 2c+1 in both orders
-        f.piece = *reinterpret_cast<const uint4 *>(blk + 16 + 16 * (2 * (step & 3) + bw));
-    };
-    auto stage_in = [&](int stage, int step, const Fetch &f) {
-#pragma unroll
-        for (int r = 0; r < RA; r++) lds_a[stage][ac * BM + ar + 32 * r] = f.a[r];  // item [ks = c / 2][g = c % 2][row]
         const int c = step & 3;
+        if (kPieces == 2) {
 #pragma unroll
-        for (int p = 0; p < 2; p++) {
-            // nibble plane p of this piece:
+            for (int q = 0; q < kPieces; q++) fpc[q] = *reinterpret_cast<const u32x4 *>(blk + 16 + 16 * (2 * c + q));
+        } else {
+            const int pc = (bu * kBTasks) >> 1;
+            fpc[0] = *reinterpret_cast<const u32x4 *>(blk + 16 + 16 * (2 * c + pc));
+        }
+    };
+    auto stage_a = [&](int stage, const u32x4 (&fa)[kAItems]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < kAItems; i++) *reinterpret_cast<u32x4 *>(lds_a + stage * 8 * BM + tid + i * kThreads) = fa[i];
+    };
+    // c = step % 4 is a compile-time constant at every call
+    auto stage_b = [&](int stage, int c, const u32x4 &fhdr, const u32x4 (&fpc)[kPieces]) __attribute__((always_inline)) {
+        uint4 *dst = lds_b + stage * 8 * BN;
+        const uint4 hdr4 = make_uint4(fhdr.x, fhdr.y, fhdr.z, fhdr.w);
+        uint32_t sc0, sc1, mn;
+        scale_min_u(hdr4, 2 * c, sc0, mn);
+        scale_min_u(hdr4, 2 * c + 1, sc1, mn);
+#pragma unroll
+        for (int t = 0; t < kBTasks; t++) {
+            const int q = bu * kBTasks + t;
+            const int bw = q >> 1, p = q & 1;
+            // nibble plane p of piece bw:
             //   REF : elements 16 p .. + 15 of sub-block 2c + bw  -> k = 32 bw + 16 p + b, scale 2c + bw
             //   GGML: elements 16 bw .. + 15 of sub-block 2c + p  -> k = 32 p + 16 bw + b, scale 2c + p
-            const int sub = ORDER == 0 ? 2 * c + bw : 2 * c + p;
             const int ks = ORDER == 0 ? 2 * bw + p : 2 * p + bw;
-            uint32_t sc, mn;
-            scale_min_u(f.hdr, sub, sc, mn);
+            const uint32_t sc = (ORDER == 0 ? bw : p) ? sc1 : sc0;
+            const u32x4 pc4 = fpc[kPieces == 2 ? bw : 0];
             uint4 b0, b1;
-            dequant16(f.piece, p, (float)sc, b0, b1);
-            lds_b[stage][(ks * 2 + 0) * BN + bn] = b0;
-            lds_b[stage][(ks * 2 + 1) * BN + bn] = b1;
+            dequant16(make_uint4(pc4.x, pc4.y, pc4.z, pc4.w), p, sc, b0, b1);
+            dst[(ks * 2 + 0) * BN + bn] = b0;
+            dst[(ks * 2 + 1) * BN + bn] = b1;
+        }
+        if (c == 1) {
+            // once per super-block (while its second stage is being staged, one barrier after the previous
+            // super-block's R product has been issued): d and the B operand of the R product for this column.
+            // item (t, g) = (-h_j, -h_j, -l_j, -l_j, -h_j+1, -h_j+1, -l_j+1, -l_j+1), j = 4 t + 2 g, against
+            // the activations' (h, l, h, l, ...): all four cross products.
+            const float dmin = f16_bits_to_f32(hdr4.x >> 16);
+            if (bu == 0) lds_d[bn] = f16_bits_to_f32(hdr4.x & 0xFFFFu);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                if (r % kUnits == bu) {
+                    uint32_t sc, mn0, mn1;
+                    scale_min_u(hdr4, 2 * r, sc, mn0);
+                    scale_min_u(hdr4, 2 * r + 1, sc, mn1);
+                    _Float16 h0, l0, h1, l1;
+                    neg_min_split(dmin, mn0, h0, l0);
+                    neg_min_split(dmin, mn1, h1, l1);
+                    const half8_t item = {h0, h0, l0, l0, h1, h1, l1, l1};
+                    lds_r[r * BN + bn] = __builtin_bit_cast(uint4, item);
+                }
+            }
         }
     };
 
-    // ---- accumulators: BLK_M x BLK_N blocks of 32 x 32 per wave ----
-    float16_t acc[BLK_M][BLK_N], part[BLK_M][BLK_N];
+    // ---- accumulators: NB x NB blocks of 32 x 32 per wave ----
+    float16_t acc[NB][NB], part[NB][NB];
 #pragma unroll
-    for (int i = 0; i < BLK_M; i++)
+    for (int i = 0; i < NB; i++)
 #pragma unroll
-        for (int jx = 0; jx < BLK_N; jx++)
+        for (int jx = 0; jx < NB; jx++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][jx][r] = 0.0f, part[i][jx][r] = 0.0f;
 
     const int col = lane & 31, kgrp = lane >> 5;
-    // columns this lane owns in the two n-blocks of its wave, and their weight rows (for d, dmin, mins)
-    int ncol[BLK_N];
-    const uint8_t *nrow[BLK_N];
-#pragma unroll
-    for (int jx = 0; jx < BLK_N; jx++) {
-        ncol[jx] = n0 + (wn * BLK_N + jx) * 32 + col;
-        nrow[jx] = W + (size_t)(ncol[jx] < N ? ncol[jx] : N - 1) * row_bytes;
-    }
-    // rows this lane feeds as A operand in the min-term MFMA
-    int mrow[BLK_M];
-#pragma unroll
-    for (int i = 0; i < BLK_M; i++) {
-        const int r = m0 + (wm * BLK_M + i) * 32 + col;
-        mrow[i] = r < M ? r : M - 1;
-    }
 
-    // Global loads run two stages ahead of the MFMAs (two register sets), the dequantization into LDS one
-    // stage ahead (two LDS stages).
-    const int n_steps = spr * 4;
-    Fetch f0, f1;
-    fetch(0, f0);
-    if (1 < n_steps) fetch(1, f1);
-    stage_in(0, 0, f0);
-    if (2 < n_steps) fetch(2, f0);
-    __syncthreads();
+    // A operand of the R product: requested one step before it is used
+    u32x4 xsv[2][NB];
+    auto fetch_xsum = [&](int sb) __attribute__((always_inline)) {
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int i = 0; i < NB; i++)
+                xsv[t][i] = *reinterpret_cast<const u32x4 *>(xsum + ((size_t)sb * 4 + t * 2 + kgrp) * Mp + m0 + (wm * NB + i) * 32 + col);
+    };
 
-    auto compute = [&](int step) {
-        const int stage = step & 1;
+    // c = step % 4 is a compile-time constant at every call
+    auto compute = [&](int stage, int c, int sb) __attribute__((always_inline)) {
+        const uint4 *sa = lds_a + stage * 8 * BM, *sbp = lds_b + stage * 8 * BN;
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
-            half8_t av[BLK_M], bv[BLK_N];
+            half8_t av[NB], bv[NB];
 #pragma unroll
-            for (int i = 0; i < BLK_M; i++)
-                av[i] = __builtin_bit_cast(half8_t, lds_a[stage][(ks * 2 + kgrp) * BM + (wm * BLK_M + i) * 32 + col]);
+            for (int i = 0; i < NB; i++) av[i] = __builtin_bit_cast(half8_t, sa[(ks * 2 + kgrp) * BM + (wm * NB + i) * 32 + col]);
 #pragma unroll
-            for (int jx = 0; jx < BLK_N; jx++)
-                bv[jx] = __builtin_bit_cast(half8_t, lds_b[stage][(ks * 2 + kgrp) * BN + (wn * BLK_N + jx) * 32 + col]);
+            for (int jx = 0; jx < NB; jx++) bv[jx] = __builtin_bit_cast(half8_t, sbp[(ks * 2 + kgrp) * BN + (wn * NB + jx) * 32 + col]);
 #pragma unroll
-            for (int i = 0; i < BLK_M; i++)
+            for (int i = 0; i < NB; i++)
 #pragma unroll
-                for (int jx = 0; jx < BLK_N; jx++)
-                    part[i][jx] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bv[jx], part[i][jx], 0, 0, 0);
-        }
-        if ((step & 3) == 3) {
-            // ---- end of a super-block: fold P and the min term into the accumulators ----
-            const int sb = step >> 2;
-            float dd[BLK_N], dm[BLK_N];
-            half8_t mv[BLK_N];
+                for (int jx = 0; jx < NB; jx++) {
+                    if (c == 0 && ks == 0) {  // first product of a super-block starts from zero
+                        float16_t z;
 #pragma unroll
-            for (int jx = 0; jx < BLK_N; jx++) {
-                const uint4 h = *reinterpret_cast<const uint4 *>(nrow[jx] + (size_t)sb * 144);
-                dd[jx] = f16_bits_to_f32(h.x & 0xFFFFu);
-                dm[jx] = f16_bits_to_f32(h.x >> 16);
-                // B' operand of the min term: column n, k' = 8 kgrp .. + 7 -> mins m_0..m_7 (hi and lo half)
-#pragma unroll
-                for (int t = 0; t < 8; t++) {
-                    uint32_t sc, mn;
-                    scale_min_u(h, t, sc, mn);
-                    mv[jx][t] = (_Float16)(float)mn;
-                }
-            }
-            half8_t sv[BLK_M];  // A' operand: row m; k-group 0 -> hi parts of the 8 sums, k-group 1 -> lo parts
-#pragma unroll
-            for (int i = 0; i < BLK_M; i++) {
-                const _Float16 *p = xsum + ((size_t)mrow[i] * (spr * 8) + (size_t)sb * 8) * 2;
-                const half8_t a = *reinterpret_cast<const half8_t *>(p);      // hi0 lo0 hi1 lo1 hi2 lo2 hi3 lo3
-                const half8_t b = *reinterpret_cast<const half8_t *>(p + 8);  // hi4 lo4 ...
-#pragma unroll
-                for (int t = 0; t < 4; t++) {
-                    sv[i][t] = kgrp ? a[2 * t + 1] : a[2 * t];
-                    sv[i][4 + t] = kgrp ? b[2 * t + 1] : b[2 * t];
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < BLK_M; i++)
-#pragma unroll
-                for (int jx = 0; jx < BLK_N; jx++) {
-                    float16_t q;
-#pragma unroll
-                    for (int r = 0; r < 16; r++) q[r] = 0.0f;
-                    q = __builtin_amdgcn_mfma_f32_32x32x16_f16(sv[i], mv[jx], q, 0, 0, 0);
-#pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        acc[i][jx][r] += dd[jx] * part[i][jx][r] - dm[jx] * q[r];
-                        part[i][jx][r] = 0.0f;
+                        for (int r = 0; r < 16; r++) z[r] = 0.0f;
+                        part[i][jx] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bv[jx], z, 0, 0, 0);
+                    } else {
+                        part[i][jx] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bv[jx], part[i][jx], 0, 0, 0);
                     }
                 }
         }
+        if (c == 3) {
+            // ---- end of a super-block: R product into the accumulators, then acc += d * P ----
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                half8_t sv[NB], mv[NB];
+#pragma unroll
+                for (int i = 0; i < NB; i++) sv[i] = __builtin_bit_cast(half8_t, xsv[t][i]);
+#pragma unroll
+                for (int jx = 0; jx < NB; jx++) mv[jx] = __builtin_bit_cast(half8_t, lds_r[(t * 2 + kgrp) * BN + (wn * NB + jx) * 32 + col]);
+#pragma unroll
+                for (int i = 0; i < NB; i++)
+#pragma unroll
+                    for (int jx = 0; jx < NB; jx++)
+                        acc[i][jx] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sv[i], mv[jx], acc[i][jx], 0, 0, 0);
+            }
+#pragma unroll
+            for (int jx = 0; jx < NB; jx++) {
+                const float dd = lds_d[(wn * NB + jx) * 32 + col];
+#pragma unroll
+                for (int i = 0; i < NB; i++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[i][jx][r] = __builtin_fmaf(dd, part[i][jx][r], acc[i][jx][r]);
+            }
+        }
     };
 
-    for (int step = 0; step < n_steps; step += 2) {
-        // even step: stage step + 1 comes from f1, then f1 is refilled for step + 3
-        if (step + 1 < n_steps) stage_in(1, step + 1, f1);
-        if (step + 3 < n_steps) fetch(step + 3, f1);
-        compute(step);
-        __syncthreads();
-        if (step + 1 < n_steps) {
-            if (step + 2 < n_steps) stage_in(0, step + 2, f0);
-            if (step + 4 < n_steps) fetch(step + 4, f0);
-            compute(step + 1);
-            __syncthreads();
-        }
+    // Global loads run ahead of the LDS staging in register sets; with four steps per loop trip the set a step
+    // uses is a compile-time constant.  Large tiles (registers are scarce): B two steps ahead in two sets, A
+    // requested at the start of a step and stored to LDS at its end, behind the MFMAs.  The small tile (short
+    // steps, few waves per compute unit to hide latency): both four steps ahead in four sets.
+    // Two LDS stages; one barrier per step; c = step % 4 and the LDS stage are compile-time constants.
+    constexpr int DA = NB == 1 ? 4 : 1, DB = NB == 1 ? 4 : 2;
+    u32x4 fa[DA][kAItems], fh[DB], fp[DB][kPieces];
+#pragma unroll
+    for (int i = 0; i < DA; i++) fetch_a(i, fa[i]);
+#pragma unroll
+    for (int i = 0; i < DB; i++) fetch_b(i, fh[i], fp[i]);
+    stage_a(0, fa[0]);
+    stage_b(0, 0, fh[0], fp[0]);
+    if (DA > 1) fetch_a(DA, fa[0]);
+    fetch_b(DB, fh[0], fp[0]);
+    __syncthreads();
+#define PMH_STEP(C)                                                                                      \
+    if ((C) == 2) fetch_xsum(sb);                                                                        \
+    if (DA == 1) {                                                                                       \
+        fetch_a(step + (C) + 1, fa[0]);                                                                  \
+        __builtin_amdgcn_sched_barrier(0); /* keep the requests a whole step ahead of their use */       \
+    }                                                                                                    \
+    stage_b(((C) + 1) & 1, ((C) + 1) & 3, fh[((C) + 1) % DB], fp[((C) + 1) % DB]);                       \
+    fetch_b(step + (C) + 1 + DB, fh[((C) + 1) % DB], fp[((C) + 1) % DB]);                                \
+    compute((C) & 1, C, sb);                                                                             \
+    stage_a(((C) + 1) & 1, fa[((C) + 1) % DA]);                                                          \
+    if (DA > 1) fetch_a(step + (C) + 1 + DA, fa[((C) + 1) % DA]);                                        \
+    __syncthreads();
+    for (int sb = 0; sb < spr; sb++) {
+        const int step = sb * 4;
+        PMH_STEP(0)
+        PMH_STEP(1)
+        PMH_STEP(2)
+        PMH_STEP(3)
     }
+#undef PMH_STEP
 
     // ---- epilogue: C layout of v_mfma_f32_32x32x*: lane holds column (lane & 31), rows 8 (r / 4) + 4 (lane / 32) + r % 4
 #pragma unroll
-    for (int i = 0; i < BLK_M; i++)
+    for (int i = 0; i < NB; i++)
 #pragma unroll
-        for (int jx = 0; jx < BLK_N; jx++) {
-            const int n = ncol[jx];
+        for (int jx = 0; jx < NB; jx++) {
+            const int n = n0 + (wn * NB + jx) * 32 + col;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const int m = m0 + (wm * BLK_M + i) * 32 + 8 * (r >> 2) + 4 * kgrp + (r & 3);
+                const int m = m0 + (wm * NB + i) * 32 + 8 * (r >> 2) + 4 * kgrp + (r & 3);
                 if (m < M && n < N) {
                     const float v = acc[i][jx][r] * rowscale[m];
                     if (YBF16) {
@@ -346,55 +437,66 @@ __global__ __launch_bounds__(kThreads, 2) void k_qgemm_q4k(const uint8_t *__rest
 
 namespace pmh {
 
-// workspace: xs [m, k] f16, xsum [m, k/32, 2] f16, rowscale [m] f32 (each 256-byte aligned)
+// workspace: xs [k/8][Mp] items, xsum [k/256][4][Mp] items, rowscale [Mp] f32 (each 256-byte aligned)
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+static int64_t padded_rows(int64_t m) { return (m + kMPad - 1) / kMPad * kMPad; }
 
 size_t qgemm_workspace_bytes(int64_t m, int64_t k) {
-    return align256((size_t)m * k * 2) + align256((size_t)m * (k / 32) * 4) + align256((size_t)m * 4);
+    const size_t mp = (size_t)padded_rows(m);
+    return align256(mp * (size_t)k * 2) + align256(mp * (size_t)(k / 256) * 4 * 16) + align256(mp * 4);
+}
+
+template <int ORDER, bool YBF16, int WM, int WN, int NB>
+static hipError_t launch_tile(hipStream_t s, const uint8_t *w, const uint4 *xs, const uint4 *xsum, const float *rowscale,
+                              void *y, int64_t m, int64_t mp, int64_t n, int spr) {
+    using TL = Tile<WM, WN, NB>;
+    auto kern = k_qgemm_q4k<ORDER, YBF16, WM, WN, NB>;
+    if (TL::kLdsBytes > 64 * 1024) {
+        hipError_t a = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)TL::kLdsBytes);
+        if (a != hipSuccess) return a;
+    }
+    const dim3 grid((unsigned)((n + TL::BN - 1) / TL::BN), (unsigned)((m + TL::BM - 1) / TL::BM));
+    hipLaunchKernelGGL(kern, grid, dim3(TL::kThreads), TL::kLdsBytes, s, w, xs, xsum, rowscale, y, (int)m, (int)mp, (int)n, spr);
+    return hipGetLastError();
+}
+
+template <int ORDER, bool YBF16>
+static hipError_t launch_shape(hipStream_t s, const uint8_t *w, const uint4 *xs, const uint4 *xsum, const float *rowscale,
+                               void *y, int64_t m, int64_t mp, int64_t n, int spr) {
+    // tile by m: short activation batches use small tiles, so that less of the MFMA work is padding and the
+    // weight matrix spreads over enough workgroups to pull it from HBM at speed
+    if (m <= 64) return launch_tile<ORDER, YBF16, 2, 1, 1>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
+    if (m <= 256) return launch_tile<ORDER, YBF16, 2, 2, 2>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
+    return launch_tile<ORDER, YBF16, 4, 2, 2>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
 }
 
 hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype,
                         int64_t m, void *y, uint32_t y_dtype, uint32_t order, void *workspace, hipStream_t s) {
     if (type != kTypeQ4K) return hipErrorNotSupported;
     if (k % 256 != 0 || m <= 0 || n <= 0) return hipErrorInvalidValue;
+    const int64_t mp = padded_rows(m);
     uint8_t *ws = reinterpret_cast<uint8_t *>(workspace);
-    _Float16 *xs = reinterpret_cast<_Float16 *>(ws);
-    _Float16 *xsum = reinterpret_cast<_Float16 *>(ws + align256((size_t)m * k * 2));
-    float *rowscale = reinterpret_cast<float *>(ws + align256((size_t)m * k * 2) + align256((size_t)m * (k / 32) * 4));
-    if (x_dtype == kDtypeF32) hipLaunchKernelGGL(k_prep_x<true>, dim3((unsigned)m), dim3(256), 0, s, x, k, xs, xsum, rowscale);
-    else hipLaunchKernelGGL(k_prep_x<false>, dim3((unsigned)m), dim3(256), 0, s, x, k, xs, xsum, rowscale);
+    uint4 *xs = reinterpret_cast<uint4 *>(ws);
+    uint4 *xsum = reinterpret_cast<uint4 *>(ws + align256((size_t)mp * k * 2));
+    float *rowscale = reinterpret_cast<float *>(ws + align256((size_t)mp * k * 2) + align256((size_t)mp * (k / 256) * 64));
+    const dim3 pgrid((unsigned)(mp / 64), (unsigned)(k / 256));
+    if (x_dtype == kDtypeF32) {
+        hipLaunchKernelGGL(k_prep_scale<true>, dim3((unsigned)((mp + 3) / 4)), dim3(256), 0, s, x, k, (int)m, rowscale);
+        hipLaunchKernelGGL(k_prep_tiles<true>, pgrid, dim3(256), 0, s, x, k, (int)m, (int)mp, rowscale, xs, xsum);
+    } else {
+        hipLaunchKernelGGL(k_prep_scale<false>, dim3((unsigned)((mp + 3) / 4)), dim3(256), 0, s, x, k, (int)m, rowscale);
+        hipLaunchKernelGGL(k_prep_tiles<false>, pgrid, dim3(256), 0, s, x, k, (int)m, (int)mp, rowscale, xs, xsum);
+    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     const int spr = (int)(k / 256);
     const bool ybf = y_dtype == kDtypeBf16;
-    auto go = [&](auto kern, int bm) {
-        const dim3 grid((unsigned)((n + BN - 1) / BN), (unsigned)((m + bm - 1) / bm));
-        hipLaunchKernelGGL(kern, grid, dim3(kThreads), 0, s, w, xs, xsum, rowscale, y, (int)m, (int)n, spr);
-    };
-    // tile height by m: short activation batches use a flatter tile so that less of the MFMA work is padding
-    const int shape = m <= 32 ? 0 : (m <= 64 ? 1 : 2);
-    if (order == kOrderRef) {
-        if (ybf) {
-            if (shape == 0) go(k_qgemm_q4k<0, true, 1, 1>, 32);
-            else if (shape == 1) go(k_qgemm_q4k<0, true, 1, 2>, 64);
-            else go(k_qgemm_q4k<0, true, 2, 2>, 128);
-        } else {
-            if (shape == 0) go(k_qgemm_q4k<0, false, 1, 1>, 32);
-            else if (shape == 1) go(k_qgemm_q4k<0, false, 1, 2>, 64);
-            else go(k_qgemm_q4k<0, false, 2, 2>, 128);
-        }
-    } else {
-        if (ybf) {
-            if (shape == 0) go(k_qgemm_q4k<1, true, 1, 1>, 32);
-            else if (shape == 1) go(k_qgemm_q4k<1, true, 1, 2>, 64);
-            else go(k_qgemm_q4k<1, true, 2, 2>, 128);
-        } else {
-            if (shape == 0) go(k_qgemm_q4k<1, false, 1, 1>, 32);
-            else if (shape == 1) go(k_qgemm_q4k<1, false, 1, 2>, 64);
-            else go(k_qgemm_q4k<1, false, 2, 2>, 128);
-        }
-    }
-    return hipGetLastError();
+    if (order == kOrderRef)
+        return ybf ? launch_shape<0, true>(s, w, xs, xsum, rowscale, y, m, mp, n, spr)
+                   : launch_shape<0, false>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
+    return ybf ? launch_shape<1, true>(s, w, xs, xsum, rowscale, y, m, mp, n, spr)
+               : launch_shape<1, false>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
 }
 
 }  // namespace pmh
