@@ -85,8 +85,9 @@ __global__ __launch_bounds__(256) void k_prep_scale(const void *__restrict__ xg,
 }
 
 // ------------------------------------------------------------------------------------------------
-// Pre-pass 2: grid (Mp / 64, k / 256), 256 threads; lane = row, wave w = sub-blocks 2w and 2w + 1 of the
-// super-block.
+// Pre-pass 2: grid (Mp / 32, k / 256), 256 threads.  Thread (row = tid / 8, c8 = tid % 8) converts the 8
+// activations of chunk c8 of every 64-element group of the super-block: 8 lanes read 128 contiguous bytes
+// of a row, and for one chunk the 8 rows of a wave write 128 contiguous bytes.
 //   xs   [k / 8][Mp]               items of 8 f16: x[m][8c .. 8c+7] * 2^-e_m   (rows >= M are zero)
 //   xsum [k / 256][2][2][Mp]       items of 8 f16 for the R_SB product, item (t, g) of row m =
 //                                  (h_j, l_j, h_j, l_j, h_j+1, l_j+1, h_j+1, l_j+1),  j = 4 t + 2 g,
@@ -96,46 +97,48 @@ template <bool XF32>
 __global__ __launch_bounds__(256) void k_prep_tiles(const void *__restrict__ xg, int64_t k, int M, int Mp,
                                                      const float *__restrict__ rowscale, uint4 *__restrict__ xs,
                                                      uint4 *__restrict__ xsum) {
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    const int m = blockIdx.x * 64 + lane;
+    const int c8 = threadIdx.x & 7;
+    const int m = blockIdx.x * 32 + (threadIdx.x >> 3);
     const int64_t sb = blockIdx.y;
     const bool live = m < M;
     const float down = live ? 1.0f / rowscale[m] : 0.0f;  // exact: a power of two
-    _Float16 hl[4];
 #pragma unroll
-    for (int s = 0; s < 2; s++) {
-        const int64_t k0 = sb * 256 + (2 * w + s) * 32;
+    for (int it = 0; it < 4; it++) {  // 64 elements per trip: sub-blocks 2 it (c8 < 4) and 2 it + 1
+        const int64_t k0 = sb * 256 + it * 64 + c8 * 8;
+        float v[8];
+        if (!live) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[i] = 0.0f;
+        } else if (XF32) {
+            const float4 a = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(xg) + (int64_t)m * k + k0);
+            const float4 b = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(xg) + (int64_t)m * k + k0 + 4);
+            v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
+        } else {
+            const uint4 u = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(xg) + (int64_t)m * k + k0);
+            const uint32_t r[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) v[2 * i] = bf16_to_f32(r[i] & 0xFFFFu), v[2 * i + 1] = bf16_to_f32(r[i] >> 16);
+        }
+        half8_t h;
         float sum = 0.0f;
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            float v[8];
-            if (!live) {
-#pragma unroll
-                for (int i = 0; i < 8; i++) v[i] = 0.0f;
-            } else if (XF32) {
-                const float4 a = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(xg) + (int64_t)m * k + k0 + 8 * c);
-                const float4 b = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(xg) + (int64_t)m * k + k0 + 8 * c + 4);
-                v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
-            } else {
-                const uint4 u = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(xg) + (int64_t)m * k + k0 + 8 * c);
-                const uint32_t r[4] = {u.x, u.y, u.z, u.w};
-#pragma unroll
-                for (int i = 0; i < 4; i++) v[2 * i] = bf16_to_f32(r[i] & 0xFFFFu), v[2 * i + 1] = bf16_to_f32(r[i] >> 16);
-            }
-            half8_t h;
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                h[i] = (_Float16)(v[i] * down);
-                sum += (float)h[i];
-            }
-            xs[(size_t)(k0 / 8 + c) * Mp + m] = __builtin_bit_cast(uint4, h);
+        for (int i = 0; i < 8; i++) {
+            h[i] = (_Float16)(v[i] * down);
+            sum += (float)h[i];
         }
-        hl[2 * s] = (_Float16)sum;
-        hl[2 * s + 1] = (_Float16)(sum - (float)hl[2 * s]);
+        xs[(size_t)(k0 / 8) * Mp + m] = __builtin_bit_cast(uint4, h);
+        // sub-block sums: over the 4 lanes of a chunk quad (exact: every partial sum is a multiple of the
+        // row's f16 grid and stays below 2^15 of it), then the pair (2 it, 2 it + 1) meets in lane c8 = 0
+        sum += __shfl_xor(sum, 1);
+        sum += __shfl_xor(sum, 2);
+        const float other = __shfl_down(sum, 4);
+        if (c8 == 0) {
+            const _Float16 h0 = (_Float16)sum, h1 = (_Float16)other;
+            const _Float16 l0 = (_Float16)(sum - (float)h0), l1 = (_Float16)(other - (float)h1);
+            const half8_t item = {h0, l0, h0, l0, h1, l1, h1, l1};
+            xsum[((size_t)sb * 4 + it) * Mp + m] = __builtin_bit_cast(uint4, item);  // j = 2 it = 4 t + 2 g
+        }
     }
-    half8_t item = {hl[0], hl[1], hl[0], hl[1], hl[2], hl[3], hl[2], hl[3]};
-    // j = 2 w = 4 t + 2 g
-    xsum[((size_t)sb * 4 + w) * Mp + m] = __builtin_bit_cast(uint4, item);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -480,7 +483,7 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
     uint4 *xs = reinterpret_cast<uint4 *>(ws);
     uint4 *xsum = reinterpret_cast<uint4 *>(ws + align256((size_t)mp * k * 2));
     float *rowscale = reinterpret_cast<float *>(ws + align256((size_t)mp * k * 2) + align256((size_t)mp * (k / 256) * 64));
-    const dim3 pgrid((unsigned)(mp / 64), (unsigned)(k / 256));
+    const dim3 pgrid((unsigned)(mp / 32), (unsigned)(k / 256));
     if (x_dtype == kDtypeF32) {
         hipLaunchKernelGGL(k_prep_scale<true>, dim3((unsigned)((mp + 3) / 4)), dim3(256), 0, s, x, k, (int)m, rowscale);
         hipLaunchKernelGGL(k_prep_tiles<true>, pgrid, dim3(256), 0, s, x, k, (int)m, (int)mp, rowscale, xs, xsum);
