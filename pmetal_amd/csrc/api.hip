@@ -372,10 +372,37 @@ int32_t pmetal_hip_qgemv(uint32_t t, const uint8_t *w, int64_t n, int64_t k, con
 
 int32_t pmetal_hip_qgemv_batch(const pmetal_hip_linear_desc *descs, size_t count, void *stream) {
     if (count && !descs) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL descriptor array");
-    for (size_t i = 0; i < count; i++) {
+    size_t i = 0;
+    while (i < count) {
         const pmetal_hip_linear_desc &d = descs[i];
-        if (int32_t rc = pmetal_hip_qgemv(d.ggml_type, d.w_dev, d.n, d.k, d.x_dev, d.x_dtype, d.y_dev, d.order, stream))
-            return rc;
+        // Consecutive small Q4_K projections of the same activation vector (q / k / v, gate / up) share a launch.
+        size_t j = i + 1;
+        if (d.ggml_type == PMETAL_GGML_TYPE_Q4K && d.k > 0 && d.k % 256 == 0 && d.n > 0 && pmh::qgemv_q4k_groupable(d.n, d.k)) {
+            while (j < count && j - i < (size_t)pmh::kMaxGemvGroup) {
+                const pmetal_hip_linear_desc &e = descs[j];
+                if (e.ggml_type != d.ggml_type || e.k != d.k || e.x_dev != d.x_dev || e.x_dtype != d.x_dtype ||
+                    e.order != d.order || e.n <= 0 || !pmh::qgemv_q4k_groupable(e.n, e.k))
+                    break;
+                j++;
+            }
+        }
+        if (j - i < 2) {
+            if (int32_t rc = pmetal_hip_qgemv(d.ggml_type, d.w_dev, d.n, d.k, d.x_dev, d.x_dtype, d.y_dev, d.order, stream))
+                return rc;
+            i++;
+            continue;
+        }
+        const uint8_t *w[pmh::kMaxGemvGroup];
+        float *y[pmh::kMaxGemvGroup];
+        int64_t n[pmh::kMaxGemvGroup];
+        for (size_t g = i; g < j; g++) {
+            const pmetal_hip_linear_desc &e = descs[g];
+            if (int32_t rc = check_linear(e.ggml_type, e.w_dev, e.n, e.k, e.x_dev, e.x_dtype, e.y_dev, e.order)) return rc;
+            w[g - i] = e.w_dev, y[g - i] = e.y_dev, n[g - i] = e.n;
+        }
+        hipError_t err = pmh::launch_qgemv_q4k_group(w, n, y, (int)(j - i), d.k, d.x_dev, d.x_dtype, d.order, (hipStream_t)stream);
+        if (err != hipSuccess) return hip_fail(err, "grouped qgemv kernel launch");
+        i = j;
     }
     return ok();
 }

@@ -128,16 +128,29 @@ __device__ __forceinline__ void stage_x_q6k(const void *xg, int spr, uint4 *xl, 
     }
 }
 
-template <int PLANES>
-__device__ __forceinline__ float q6k_lane(const uint8_t *blk, const int t, const uint4 *xl, const int slots,
-                                          const int slot, const float4 xsum) {
+// One lane's share of a Q6_K super-block as it lies in memory (loaded ahead of its use).
+struct Q6Raw {
+    u32x2_a2 qla, qlb, qh, sc8;
+    uint32_t d;
+};
+
+__device__ __forceinline__ Q6Raw q6k_load(const uint8_t *blk, const int t) {
     const int h = t >> 2, lq = (t & 3) * 8;
-    const u32x2_a2 qla = *reinterpret_cast<const u32x2_a2 *>(blk + 64 * h + lq);
-    const u32x2_a2 qlb = *reinterpret_cast<const u32x2_a2 *>(blk + 64 * h + 32 + lq);
-    const u32x2_a2 qh = *reinterpret_cast<const u32x2_a2 *>(blk + 128 + 32 * h + lq);
-    const u32x2_a2 sc8 = *reinterpret_cast<const u32x2_a2 *>(blk + 192 + 8 * h);
-    const float d = f16_bits_to_f32(*reinterpret_cast<const u16_a2 *>(blk + 208));
-    const uint32_t la[2] = {qla.x, qla.y}, lb[2] = {qlb.x, qlb.y}, hh[2] = {qh.x, qh.y};
+    Q6Raw r;
+    r.qla = *reinterpret_cast<const u32x2_a2 *>(blk + 64 * h + lq);
+    r.qlb = *reinterpret_cast<const u32x2_a2 *>(blk + 64 * h + 32 + lq);
+    r.qh = *reinterpret_cast<const u32x2_a2 *>(blk + 128 + 32 * h + lq);
+    r.sc8 = *reinterpret_cast<const u32x2_a2 *>(blk + 192 + 8 * h);
+    r.d = *reinterpret_cast<const u16_a2 *>(blk + 208);
+    return r;
+}
+
+template <int PLANES>
+__device__ __forceinline__ float q6k_lane(const Q6Raw &raw, const int t, const uint4 *xl, const int slots,
+                                          const int slot, const float4 xsum) {
+    const int lq = (t & 3) * 8;
+    const float d = f16_bits_to_f32(raw.d);
+    const uint32_t la[2] = {raw.qla.x, raw.qla.y}, lb[2] = {raw.qlb.x, raw.qlb.y}, hh[2] = {raw.qh.x, raw.qh.y};
     const float xs4[4] = {xsum.x, xsum.y, xsum.z, xsum.w};
     const int shalf = lq >> 4;  // which of the two 16-element scale slots of a group
     float total = 0.0f;
@@ -162,13 +175,16 @@ __device__ __forceinline__ float q6k_lane(const uint8_t *blk, const int t, const
             dot = dot2(b1, xv.w, dot);
         }
         const int si = 2 * g + shalf;  // scale byte inside this half's 8
-        const uint32_t sw = si < 4 ? sc8.x : sc8.y;
+        const uint32_t sw = si < 4 ? raw.sc8.x : raw.sc8.y;
         const float sc = (float)(int8_t)(sw >> (8 * (si & 3)));
         total += sc * (dot - 96.0f * xs4[g]);  // stored value is q + 32 and the bf16 trick adds 64
     }
     return d * total;
 }
 
+// A team of T lanes walks two rows at a time; the two lanes' shares of the next task (the next chunk of the
+// row pair, or the first chunk of the next pair) are requested before the current one is multiplied, and the
+// first request goes out before x is converted.
 template <int T, bool XF32>
 __global__ __launch_bounds__(256) void k_qgemv_q6k(const uint8_t *__restrict__ W, const void *__restrict__ xg,
                                                     float *__restrict__ y, int n_rows, int spr) {
@@ -178,8 +194,6 @@ __global__ __launch_bounds__(256) void k_qgemv_q6k(const uint8_t *__restrict__ W
     const int slots = spr * 8;
     uint4 *xl = smem;
     float4 *xs = reinterpret_cast<float4 *>(xl + PLANES * 4 * slots);
-    stage_x_q6k<PLANES, XF32>(xg, spr, xl, xs);
-    __syncthreads();
 
     const int lt = threadIdx.x & (T - 1);
     const int t = lt & 7;
@@ -189,25 +203,37 @@ __global__ __launch_bounds__(256) void k_qgemv_q6k(const uint8_t *__restrict__ W
     const size_t row_bytes = (size_t)spr * 210;
     const size_t lane_off = (size_t)(lt >> 3) * 210;
 
-    for (int row = team; row < n_rows; row += 2 * n_teams) {
-        const int row1 = row + n_teams;
-        const bool has1 = row1 < n_rows;
-        const uint8_t *p0 = W + (size_t)row * row_bytes + lane_off;
-        const uint8_t *p1 = W + (size_t)(has1 ? row1 : row) * row_bytes + lane_off;
-        float acc0 = 0.0f, acc1 = 0.0f;
-        for (int it = 0; it < iters; it++) {
-            const size_t o = (size_t)it * SEG * 210;
-            const int slot = it * T + lt;
-            const float4 xsum = xs[slot];
-            acc0 += q6k_lane<PLANES>(p0 + o, t, xl, slots, slot, xsum);
-            acc1 += q6k_lane<PLANES>(p1 + o, t, xl, slots, slot, xsum);
+    // task (row, it): rows row and row + n_teams, chunk it; a row past the end is replaced by the last row
+    auto block_ptr = [&](int row, int it) -> const uint8_t * {
+        const int r = row < n_rows ? row : n_rows - 1;
+        return W + (size_t)r * row_bytes + lane_off + (size_t)it * SEG * 210;
+    };
+    int row = team, it = 0;
+    Q6Raw c0 = q6k_load(block_ptr(row, 0), t), c1 = q6k_load(block_ptr(row + n_teams, 0), t);
+
+    stage_x_q6k<PLANES, XF32>(xg, spr, xl, xs);
+    __syncthreads();
+
+    float acc0 = 0.0f, acc1 = 0.0f;
+    while (row < n_rows) {
+        int nrow = row, nit = it + 1;
+        if (nit == iters) nit = 0, nrow = row + 2 * n_teams;
+        const Q6Raw n0 = q6k_load(block_ptr(nrow, nit), t), n1 = q6k_load(block_ptr(nrow + n_teams, nit), t);
+        const int slot = it * T + lt;
+        const float4 xsum = xs[slot];
+        acc0 += q6k_lane<PLANES>(c0, t, xl, slots, slot, xsum);
+        acc1 += q6k_lane<PLANES>(c1, t, xl, slots, slot, xsum);
+        if (nit == 0) {
+            acc0 = team_sum<T>(acc0);
+            acc1 = team_sum<T>(acc1);
+            if (lt == 0) {
+                y[row] = acc0;
+                if (row + n_teams < n_rows) y[row + n_teams] = acc1;
+            }
+            acc0 = acc1 = 0.0f;
         }
-        acc0 = team_sum<T>(acc0);
-        acc1 = team_sum<T>(acc1);
-        if (lt == 0) {
-            y[row] = acc0;
-            if (has1) y[row1] = acc1;
-        }
+        c0 = n0, c1 = n1;
+        row = nrow, it = nit;
     }
 }
 
@@ -299,8 +325,13 @@ int rows_per_team() {
     return v;
 }
 
+// Rows per team: rows_per_team() when that still leaves a workgroup for every compute unit, fewer otherwise
+// (a small matrix is spread over the whole chip rather than streamed by a few workgroups).
 unsigned grid_for_rows(int64_t n, int teams_per_wg) {
-    const int64_t per_wg = (int64_t)teams_per_wg * rows_per_team();
+    int64_t r = rows_per_team();
+    const int64_t cus = compute_units();
+    while (r > 1 && (n + teams_per_wg * r - 1) / (teams_per_wg * r) < cus) r /= 2;
+    const int64_t per_wg = (int64_t)teams_per_wg * r;
     int64_t g = (n + per_wg - 1) / per_wg;
     if (g < 1) g = 1;
     if (g > (1 << 20)) g = 1 << 20;

@@ -96,7 +96,4 @@ inline int compute_units() {
 
 }  // namespace gemv
 
-hipError_t launch_qgemv_q4k(const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, float *y,
-                            uint32_t order, hipStream_t s);
-
 }  // namespace pmh

@@ -473,10 +473,26 @@ __global__ __launch_bounds__(1024) void k_qgemv_q4k_chunk(const uint8_t *__restr
 // re-reading its x digits from LDS for every task and reducing with DPP at the end of every row.
 constexpr int kRing = 8;
 
+// Up to kMaxGroup weight matrices that share k and the activation vector (the q / k / v or the gate / up
+// projections of a decoder layer) go through one launch: x is converted once per workgroup instead of once
+// per matrix and launch.  Workgroups [wg_begin[g], wg_begin[g + 1]) belong to matrix g.
+struct GemvGroup {
+    const uint8_t *w[pmh::kMaxGemvGroup];
+    float *y[pmh::kMaxGemvGroup];
+    int n[pmh::kMaxGemvGroup];
+    int wg_begin[pmh::kMaxGemvGroup + 1];
+};
+
 template <int ORDER, bool XF32, int T>
-__global__ __launch_bounds__(1024) void k_qgemv_q4k(const uint8_t *__restrict__ W, const void *__restrict__ xg,
-                                                     float *__restrict__ y, int n_rows, int spr, int rows_per_wg,
-                                                     int per_team, int nthreads) {
+__global__ __launch_bounds__(1024) void k_qgemv_q4k(const GemvGroup grp, const void *__restrict__ xg, int spr,
+                                                     int rows_per_wg, int per_team, int nthreads) {
+    int g = 0;
+#pragma unroll
+    for (int i = 1; i < pmh::kMaxGemvGroup; i++) g += (int)blockIdx.x >= grp.wg_begin[i] ? 1 : 0;
+    const uint8_t *__restrict__ W = grp.w[g];
+    float *__restrict__ y = grp.y[g];
+    const int n_rows = grp.n[g];
+    const int wg_index = (int)blockIdx.x - grp.wg_begin[g];
     constexpr int NDIG = XF32 ? 6 : 5;
     constexpr int SEG = T / 8;         // super-blocks a team covers per task
     constexpr int STRIDE = SEG * 144;  // bytes between a lane's consecutive tasks
@@ -495,7 +511,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q4k(const uint8_t *__restrict__ 
     const int team = uni((int)(threadIdx.x >> 6) * kTeamsPerWave + lane / T);
 
     // contiguous chunk of rows for this workgroup, then `per_team` of them for this team
-    const int wg_r0 = blockIdx.x * rows_per_wg;
+    const int wg_r0 = wg_index * rows_per_wg;
     const int wg_r1 = wg_r0 + rows_per_wg < n_rows ? wg_r0 + rows_per_wg : n_rows;
     const int r0 = wg_r0 + team * per_team;
     const int r1 = r0 + per_team < wg_r1 ? r0 + per_team : wg_r1;
@@ -585,14 +601,58 @@ hipError_t launch_chunk(int T, bool single, dim3 grid, dim3 block, size_t lds, h
 }
 
 template <int ORDER, bool XF32>
-hipError_t launch_general(int T, dim3 grid, dim3 block, size_t lds, hipStream_t s, const uint8_t *w, const void *x,
-                          float *y, int n, int spr, int rows_per_wg, int per_team) {
+hipError_t launch_general(int T, dim3 grid, dim3 block, size_t lds, hipStream_t s, const GemvGroup &grp, const void *x,
+                          int spr, int rows_per_wg, int per_team) {
     switch (T) {
-    case 8: return launch_with_lds(k_qgemv_q4k<ORDER, XF32, 8>, grid, block, lds, s, w, x, y, n, spr, rows_per_wg, per_team, (int)block.x);
-    case 16: return launch_with_lds(k_qgemv_q4k<ORDER, XF32, 16>, grid, block, lds, s, w, x, y, n, spr, rows_per_wg, per_team, (int)block.x);
-    case 32: return launch_with_lds(k_qgemv_q4k<ORDER, XF32, 32>, grid, block, lds, s, w, x, y, n, spr, rows_per_wg, per_team, (int)block.x);
-    default: return launch_with_lds(k_qgemv_q4k<ORDER, XF32, 64>, grid, block, lds, s, w, x, y, n, spr, rows_per_wg, per_team, (int)block.x);
+    case 8: return launch_with_lds(k_qgemv_q4k<ORDER, XF32, 8>, grid, block, lds, s, grp, x, spr, rows_per_wg, per_team, (int)block.x);
+    case 16: return launch_with_lds(k_qgemv_q4k<ORDER, XF32, 16>, grid, block, lds, s, grp, x, spr, rows_per_wg, per_team, (int)block.x);
+    case 32: return launch_with_lds(k_qgemv_q4k<ORDER, XF32, 32>, grid, block, lds, s, grp, x, spr, rows_per_wg, per_team, (int)block.x);
+    default: return launch_with_lds(k_qgemv_q4k<ORDER, XF32, 64>, grid, block, lds, s, grp, x, spr, rows_per_wg, per_team, (int)block.x);
     }
+}
+
+// Kernel B over a group of matrices: up to 16 waves; the wave count is the largest that keeps the busiest
+// team's row count minimal.
+hipError_t launch_group_general(const uint8_t *const *w, const int64_t *n, float *const *y, int count, int64_t k,
+                                const void *x, bool xf32, uint32_t order, hipStream_t s) {
+    const int spr = (int)(k / 256);
+    const int T = 8 * pow2_divisor(spr, 8);
+    const size_t slots = (size_t)spr * 8;
+    const size_t lds_x = slots * 16 * (xf32 ? 6 : 5) + slots * 16;
+    if (lds_x > kMaxLds) return hipErrorInvalidValue;
+    int64_t total = 0;
+    for (int i = 0; i < count; i++) total += n[i];
+    const int64_t want = compute_units();
+    int64_t n_wg = total < want ? total : want;
+    const int64_t rows_per_wg = (total + n_wg - 1) / n_wg;
+    GemvGroup grp{};
+    int begin = 0;
+    for (int i = 0; i < pmh::kMaxGemvGroup; i++) {
+        grp.wg_begin[i] = begin;
+        if (i < count) {
+            grp.w[i] = w[i], grp.y[i] = y[i], grp.n[i] = (int)n[i];
+            begin += (int)((n[i] + rows_per_wg - 1) / rows_per_wg);
+        } else {
+            grp.w[i] = w[0], grp.y[i] = y[0], grp.n[i] = 0;
+        }
+    }
+    grp.wg_begin[pmh::kMaxGemvGroup] = begin;
+    const dim3 grid((unsigned)begin);
+    const int teams_per_wave = 64 / T;
+    int best_waves = 16;
+    int64_t best_cost = INT64_MAX;
+    for (int waves = 16; waves >= 1; waves--) {  // ties go to more waves: more bytes in flight
+        const int64_t teams = (int64_t)waves * teams_per_wave;
+        const int64_t per_team = (rows_per_wg + teams - 1) / teams;
+        if (per_team < best_cost) best_cost = per_team, best_waves = waves;
+    }
+    const int per_team = (int)((rows_per_wg + (int64_t)best_waves * teams_per_wave - 1) / ((int64_t)best_waves * teams_per_wave));
+    const dim3 block((unsigned)best_waves * 64);
+    if (order == pmh::kOrderRef)
+        return xf32 ? launch_general<0, true>(T, grid, block, lds_x, s, grp, x, spr, (int)rows_per_wg, per_team)
+                    : launch_general<0, false>(T, grid, block, lds_x, s, grp, x, spr, (int)rows_per_wg, per_team);
+    return xf32 ? launch_general<1, true>(T, grid, block, lds_x, s, grp, x, spr, (int)rows_per_wg, per_team)
+                : launch_general<1, false>(T, grid, block, lds_x, s, grp, x, spr, (int)rows_per_wg, per_team);
 }
 
 }  // namespace
@@ -649,22 +709,16 @@ hipError_t launch_qgemv_q4k(const uint8_t *w, int64_t n, int64_t k, const void *
         }
     }
 
-    // Kernel B: up to 16 waves; the wave count is the largest that keeps the busiest team's row count minimal.
-    const int teams_per_wave = 64 / T;
-    int best_waves = 16;
-    int64_t best_cost = INT64_MAX;
-    for (int waves = 16; waves >= 1; waves--) {  // ties go to more waves: more bytes in flight
-        const int64_t teams = (int64_t)waves * teams_per_wave;
-        const int64_t per_team = (rows_per_wg + teams - 1) / teams;
-        if (per_team < best_cost) best_cost = per_team, best_waves = waves;
-    }
-    const int per_team = (int)((rows_per_wg + (int64_t)best_waves * teams_per_wave - 1) / ((int64_t)best_waves * teams_per_wave));
-    const dim3 block((unsigned)best_waves * 64);
-    if (order == kOrderRef)
-        return xf32 ? launch_general<0, true>(T, grid, block, lds_x, s, w, x, y, (int)n, spr, (int)rows_per_wg, per_team)
-                    : launch_general<0, false>(T, grid, block, lds_x, s, w, x, y, (int)n, spr, (int)rows_per_wg, per_team);
-    return xf32 ? launch_general<1, true>(T, grid, block, lds_x, s, w, x, y, (int)n, spr, (int)rows_per_wg, per_team)
-                : launch_general<1, false>(T, grid, block, lds_x, s, w, x, y, (int)n, spr, (int)rows_per_wg, per_team);
+    return launch_group_general(&w, &n, &y, 1, k, x, xf32, order, s);
+}
+
+// Matrices that kernel A would not take anyway (small ones), sharing k, x, x_dtype and order, in one launch.
+bool qgemv_q4k_groupable(int64_t n, int64_t k) { return (uint64_t)n * (uint64_t)(k / 256) * 144u < (12ull << 20); }
+
+hipError_t launch_qgemv_q4k_group(const uint8_t *const *w, const int64_t *n, float *const *y, int count, int64_t k,
+                                  const void *x, uint32_t x_dtype, uint32_t order, hipStream_t s) {
+    if (count < 1 || count > kMaxGemvGroup) return hipErrorInvalidValue;
+    return launch_group_general(w, n, y, count, k, x, x_dtype == kDtypeF32, order, s);
 }
 
 }  // namespace pmh

@@ -23,6 +23,17 @@ hipError_t launch_dequantize_q6k(const uint8_t *src, size_t n, float *dst, hipSt
 hipError_t launch_qgemv(uint32_t type, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype,
                         float *y, uint32_t order, hipStream_t s);
 
+// ---- gemv_q4k.hip ----
+constexpr int kMaxGemvGroup = 4;
+
+hipError_t launch_qgemv_q4k(const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, float *y,
+                            uint32_t order, hipStream_t s);
+// Several small Q4_K matrices with the same k, x, x_dtype and order in one launch (count <= kMaxGemvGroup);
+// qgemv_q4k_groupable tells whether a matrix is small enough to go into a group.
+bool qgemv_q4k_groupable(int64_t n, int64_t k);
+hipError_t launch_qgemv_q4k_group(const uint8_t *const *w, const int64_t *n, float *const *y, int count, int64_t k,
+                                  const void *x, uint32_t x_dtype, uint32_t order, hipStream_t s);
+
 // ---- gemm.hip: dequant-fused Y = X W^T ----
 // Bytes of device workspace qgemm needs for (m, k); the caller provides it.
 size_t qgemm_workspace_bytes(int64_t m, int64_t k);

@@ -112,6 +112,34 @@ def test_qgemv_batch_runs_a_decode_step(oracle):
         assert elem <= TOL and norm <= TOL
 
 
+@pytest.mark.parametrize("order", [0, 1])
+def test_qgemv_batch_groups_projections_of_one_activation(oracle, order):
+    """q / k / v-like projections that share x go through one grouped launch; the rows must come out exactly as
+    from separate launches (and a fifth matrix starts a new group, a different x ends one)."""
+    from pmetal_amd import _lib
+    lib = _lib.load()
+    k = 1024
+    bits = oracle.f32_to_bf16_bits(np.random.default_rng(70).standard_normal(k).astype(np.float32))
+    other = oracle.f32_to_bf16_bits(np.random.default_rng(71).standard_normal(k).astype(np.float32))
+    dx, dx2 = pm.DeviceBuffer.from_host(bits), pm.DeviceBuffer.from_host(other)
+    rows = [2048, 1024, 1000, 37, 515, 96]
+    xs_of = [dx, dx, dx, dx, dx, dx2]
+    descs = (_lib.LinearDesc * len(rows))()
+    keep, singles = [], []
+    for i, n in enumerate(rows):
+        wq = oracle.quantize(Q4K, weights(80 + i, n * k))
+        dw, dy = pm.DeviceBuffer.from_host(wq), pm.DeviceBuffer(4 * n)
+        pm.check(lib.pmetal_hip_memset(dy.ptr, 0xFF, 4 * n, None))
+        keep.append((dw, dy))
+        descs[i] = _lib.LinearDesc(Q4K, pm.DTYPE_BF16, order, 0, n, k, dw.ptr, xs_of[i].ptr, dy.ptr)
+        x_bits = bits if xs_of[i] is dx else other
+        singles.append(gpu_qgemv(Q4K, wq, n, k, x_bits, pm.DTYPE_BF16, order))
+    pm.check(lib.pmetal_hip_qgemv_batch(descs, len(rows), None))
+    pm.check(lib.pmetal_hip_sync(None))
+    for (dw, dy), single in zip(keep, singles):
+        assert np.array_equal(dy.to_host(np.float32), single)
+
+
 def test_qgemv_argument_errors():
     from pmetal_amd import _lib
     lib = _lib.load()
