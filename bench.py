@@ -30,7 +30,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled against a streaming
 # kernel of known size (summary and commands: profiles/qgemv_q4k_14336x4096.md)
-MEASURED_TRAFFIC = {"gemv_q4k_14336x4096": 33232404}
+MEASURED_TRAFFIC = {"gemv_q4k_14336x4096": 33299335}
 BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16/fp16 MFMA, published
 Q8_0, Q4K, Q6K = 8, 12, 14
 
@@ -134,7 +134,7 @@ def bench_gemv(args, n, k, t=Q4K, copies=16):
         "value": gbs, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "k_qgemv_q4k", "bytes_per_launch": bytes_per_launch,
+                     "kernel": "k_qgemv_q4k_chunk", "bytes_per_launch": bytes_per_launch,
                      "us_per_launch": round(us_per_launch, 3)},
         "extra": {"cache_resident_GBps": round(cached_gbs, 1), "weight_copies": copies},
     }, (t, n, k)
@@ -157,7 +157,7 @@ def bench_gemm(args, m, n, k, t=Q4K):
     return {
         "value": tflops, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(tflops / BF16_PEAK_TFLOPS, 4), "traffic": None, "kernel": "k_qgemm_q4k (+ k_prep_x)",
+                     "frac": round(tflops / BF16_PEAK_TFLOPS, 4), "traffic": None, "kernel": "k_qgemm_q4k (+ k_prep_scale, k_prep_tiles)",
                      "flops_per_launch": flops, "us_per_launch": round(us, 3)},
         "extra": {},
     }, (t, n, k)
@@ -213,7 +213,7 @@ def bench_decode(args):
     return {
         "value": tok_s, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "k_qgemv_q4k / k_qgemv_q6k (197 launches)",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "k_qgemv_q4k / k_qgemv_q6k (197 projections in 127 launches)",
                      "bytes_per_step": total_bytes},
         "extra": {"launches_per_token": len(lins), "q6k_tensors": sum(1 for l in lins if l[3] == Q6K)},
     }, (Q4K, 0, 0)
