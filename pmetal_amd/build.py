@@ -25,8 +25,10 @@ COMMON = [
 # per-file extra flags
 EXTRA = {
     "codec.hip": ["-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt", "-fno-gpu-flush-denormals-to-zero"],
-    "gemv.hip": [],
-    "gemv_q4k.hip": [],
+    # the first 16 dwords of kernel arguments arrive in scalar registers with the wave (no argument fetch
+    # in front of the first load of these latency-bound kernels)
+    "gemv.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
+    "gemv_q4k.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
     "gemm.hip": [],
     "util.hip": [],
     "api.hip": [],

@@ -483,16 +483,23 @@ struct GemvGroup {
     int wg_begin[pmh::kMaxGemvGroup + 1];
 };
 
+// The arguments come as scalars, the ones needed first up front: the leading 16 dwords of the kernel-argument
+// segment are preloaded into scalar registers at wave launch (the translation unit is built with
+// -amdgpu-kernarg-preload-count=16), so the first weight request does not wait for an argument fetch.
 template <int ORDER, bool XF32, int T>
-__global__ __launch_bounds__(1024) void k_qgemv_q4k(const GemvGroup grp, const void *__restrict__ xg, int spr,
-                                                     int rows_per_wg, int per_team, int nthreads) {
-    int g = 0;
-#pragma unroll
-    for (int i = 1; i < pmh::kMaxGemvGroup; i++) g += (int)blockIdx.x >= grp.wg_begin[i] ? 1 : 0;
-    const uint8_t *__restrict__ W = grp.w[g];
-    float *__restrict__ y = grp.y[g];
-    const int n_rows = grp.n[g];
-    const int wg_index = (int)blockIdx.x - grp.wg_begin[g];
+__global__ __launch_bounds__(1024) void k_qgemv_q4k(const void *__restrict__ xg, const uint8_t *__restrict__ w0,
+                                                     const uint8_t *__restrict__ w1, const uint8_t *__restrict__ w2,
+                                                     const uint8_t *__restrict__ w3, int wg_b1, int wg_b2, int wg_b3,
+                                                     int spr, int rows_per_wg, int per_team, int n0, int n1, int n2,
+                                                     int n3, float *__restrict__ y0, float *__restrict__ y1,
+                                                     float *__restrict__ y2, float *__restrict__ y3, int nthreads) {
+    static_assert(pmh::kMaxGemvGroup == 4, "the argument list spells out four group members");
+    const int bx = (int)blockIdx.x;
+    const int g = (bx >= wg_b1 ? 1 : 0) + (bx >= wg_b2 ? 1 : 0) + (bx >= wg_b3 ? 1 : 0);
+    const uint8_t *__restrict__ W = g == 0 ? w0 : g == 1 ? w1 : g == 2 ? w2 : w3;
+    float *__restrict__ y = g == 0 ? y0 : g == 1 ? y1 : g == 2 ? y2 : y3;
+    const int n_rows = g == 0 ? n0 : g == 1 ? n1 : g == 2 ? n2 : n3;
+    const int wg_index = bx - (g == 0 ? 0 : g == 1 ? wg_b1 : g == 2 ? wg_b2 : wg_b3);
     constexpr int NDIG = XF32 ? 6 : 5;
     constexpr int SEG = T / 8;         // super-blocks a team covers per task
     constexpr int STRIDE = SEG * 144;  // bytes between a lane's consecutive tasks
@@ -603,11 +610,16 @@ hipError_t launch_chunk(int T, bool single, dim3 grid, dim3 block, size_t lds, h
 template <int ORDER, bool XF32>
 hipError_t launch_general(int T, dim3 grid, dim3 block, size_t lds, hipStream_t s, const GemvGroup &grp, const void *x,
                           int spr, int rows_per_wg, int per_team) {
+    auto go = [&](auto kern) {
+        return launch_with_lds(kern, grid, block, lds, s, x, grp.w[0], grp.w[1], grp.w[2], grp.w[3], grp.wg_begin[1],
+                               grp.wg_begin[2], grp.wg_begin[3], spr, rows_per_wg, per_team, grp.n[0], grp.n[1], grp.n[2],
+                               grp.n[3], grp.y[0], grp.y[1], grp.y[2], grp.y[3], (int)block.x);
+    };
     switch (T) {
-    case 8: return launch_with_lds(k_qgemv_q4k<ORDER, XF32, 8>, grid, block, lds, s, grp, x, spr, rows_per_wg, per_team, (int)block.x);
-    case 16: return launch_with_lds(k_qgemv_q4k<ORDER, XF32, 16>, grid, block, lds, s, grp, x, spr, rows_per_wg, per_team, (int)block.x);
-    case 32: return launch_with_lds(k_qgemv_q4k<ORDER, XF32, 32>, grid, block, lds, s, grp, x, spr, rows_per_wg, per_team, (int)block.x);
-    default: return launch_with_lds(k_qgemv_q4k<ORDER, XF32, 64>, grid, block, lds, s, grp, x, spr, rows_per_wg, per_team, (int)block.x);
+    case 8: return go(k_qgemv_q4k<ORDER, XF32, 8>);
+    case 16: return go(k_qgemv_q4k<ORDER, XF32, 16>);
+    case 32: return go(k_qgemv_q4k<ORDER, XF32, 32>);
+    default: return go(k_qgemv_q4k<ORDER, XF32, 64>);
     }
 }
 
