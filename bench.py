@@ -157,7 +157,7 @@ def bench_gemm(args, m, n, k, t=Q4K):
     return {
         "value": tflops, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(tflops / BF16_PEAK_TFLOPS, 4), "traffic": None, "kernel": "k_qgemm_q4k (+ k_prep_scale, k_prep_tiles)",
+                     "frac": round(tflops / BF16_PEAK_TFLOPS, 4), "traffic": None, "kernel": "k_qgemm (+ k_prep_scale, k_prep_tiles)",
                      "flops_per_launch": flops, "us_per_launch": round(us, 3)},
         "extra": {},
     }, (t, n, k)
@@ -268,7 +268,9 @@ WORKLOADS["quantize_llama3_8b_q4km"] = dict(kind="quantize", metric="f32->Q4_K_M
                                             unit="GB/s", dtype="f32")
 for _m in (16, 64, 128, 512, 2048):
     WORKLOADS[f"gemm_q4k_m{_m}"] = dict(kind="gemm", m=_m, n=14336, k=4096, metric=f"Q4_K GEMM TFLOPS @M={_m},K=4096,N=14336",
-                                        unit="TFLOP/s", dtype="f16")
+                                        unit="TFLOP/s", dtype="f16", type=Q4K)
+WORKLOADS["gemm_q6k_m512"] = dict(kind="gemm", m=512, n=14336, k=4096, metric="Q6_K GEMM TFLOPS @M=512,K=4096,N=14336",
+                                  unit="TFLOP/s", dtype="f16", type=Q6K)
 
 
 def main():
@@ -286,7 +288,7 @@ def main():
         sys.exit("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)")
     wl = WORKLOADS[args.workload]
     if wl["kind"] == "gemm":
-        res, (t, n, k) = bench_gemm(args, wl["m"], wl["n"], wl["k"])
+        res, (t, n, k) = bench_gemm(args, wl["m"], wl["n"], wl["k"], wl["type"])
     elif wl["kind"] == "decode":
         res, (t, n, k) = bench_decode(args)
     elif wl["kind"] == "quantize":

@@ -425,9 +425,8 @@ int32_t pmetal_hip_qlinear(uint32_t t, const uint8_t *w, int64_t n, int64_t k, c
                            void *y, uint32_t y_dtype, uint32_t order, void *stream) {
     if (m == 1 && y_dtype == PMETAL_HIP_DTYPE_F32)
         return pmetal_hip_qgemv(t, w, n, k, x, x_dtype, (float *)y, order, stream);
-    if (t != PMETAL_GGML_TYPE_Q4K && (t == PMETAL_GGML_TYPE_Q6K || t == PMETAL_GGML_TYPE_Q8_0) &&
-        y_dtype == PMETAL_HIP_DTYPE_F32 && m > 1 && n > 0 && k > 0 && x && y) {
-        // No fused GEMM for these types yet: one fused GEMV per activation row, back to back on the stream.
+    if (t == PMETAL_GGML_TYPE_Q8_0 && y_dtype == PMETAL_HIP_DTYPE_F32 && m > 1 && n > 0 && k > 0 && x && y) {
+        // No fused GEMM for Q8_0: one fused GEMV per activation row, back to back on the stream.
         const size_t x_row = (size_t)k * (x_dtype == PMETAL_HIP_DTYPE_F32 ? 4 : 2);
         for (int64_t r = 0; r < m; r++) {
             const int32_t rc = pmetal_hip_qgemv(t, w, n, k, (const uint8_t *)x + (size_t)r * x_row, x_dtype,

@@ -183,6 +183,51 @@ __device__ __forceinline__ void scale_min_u(const uint4 hdr, const int j, uint32
     }
 }
 
+// 16 bytes / 4 bytes / 2 bytes at an address that is only 2-byte aligned (Q6_K super-blocks are 210 bytes)
+struct __attribute__((packed, aligned(2))) u32x4_a2 {
+    uint32_t x, y, z, w;
+};
+struct __attribute__((packed, aligned(2))) u32_a2 {
+    uint32_t v;
+};
+typedef uint16_t u16_a2 __attribute__((aligned(2)));
+
+__device__ __forceinline__ u32x4 load16_a2(const uint8_t *p) {
+    const u32x4_a2 t = *reinterpret_cast<const u32x4_a2 *>(p);
+    return u32x4{t.x, t.y, t.z, t.w};
+}
+
+// Q6_K: 16 six-bit quants (low nibbles in ql shifted by ql_shift, top two bits in qh at qh_shift) of one
+// 16-element scale group.  sc * (q - 32) can reach 4096 and would not always be exact in f16, so the value is
+// split where the storage splits it, q - 32 = 16 (hi2 - 2) + nib, into two exact tiles:
+//     B1 = (16 sc) * (hi2 - 2)   |.| <= 2048 * 2, a multiple of 16        B2 = sc * nib   |.| <= 1920
+// multiplied one after the other into the same accumulator.  (0x6400 | v is the f16 1024 + v.)
+__device__ __forceinline__ void dequant16_q6(const u32x4 ql, const u32x4 qh, const int ql_shift, const int qh_shift,
+                                             const int sc, uint4 &b1lo, uint4 &b1hi, uint4 &b2lo, uint4 &b2hi) {
+    const _Float16 s1 = (_Float16)(float)(16 * sc), s2 = (_Float16)(float)sc;  // exact: |sc| <= 128
+    const half2_t s1v = {s1, s1}, s2v = {s2, s2};
+    const half2_t m1026 = {(_Float16)-1026.0f, (_Float16)-1026.0f}, m1024 = {(_Float16)-1024.0f, (_Float16)-1024.0f};
+    const uint32_t lw[4] = {ql.x, ql.y, ql.z, ql.w}, hw[4] = {qh.x, qh.y, qh.z, qh.w};
+    uint32_t o1[8], o2[8];
+#pragma unroll
+    for (int d = 0; d < 4; d++) {
+        const uint32_t nib = (lw[d] >> ql_shift) & 0x0F0F0F0Fu;
+        const uint32_t hi2 = (hw[d] >> qh_shift) & 0x03030303u;
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const uint32_t sel = half ? 0x04030402u : 0x04010400u;  // bytes (b0, b1) resp. (b2, b3) -> 0x64bb pairs
+            const half2_t n2 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, nib, sel));
+            const half2_t h2 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, hi2, sel));
+            o2[2 * d + half] = __builtin_bit_cast(uint32_t, (n2 + m1024) * s2v);  // both steps exact
+            o1[2 * d + half] = __builtin_bit_cast(uint32_t, (h2 + m1026) * s1v);
+        }
+    }
+    b1lo = make_uint4(o1[0], o1[1], o1[2], o1[3]);
+    b1hi = make_uint4(o1[4], o1[5], o1[6], o1[7]);
+    b2lo = make_uint4(o2[0], o2[1], o2[2], o2[3]);
+    b2hi = make_uint4(o2[4], o2[5], o2[6], o2[7]);
+}
+
 // -(dmin * mn) split exactly into an f16 head and tail (dmin has 11 significant bits, mn 6).
 __device__ __forceinline__ void neg_min_split(const float dmin, const uint32_t mn, _Float16 &h, _Float16 &l) {
     const float p = -(dmin * (float)mn);  // exact in fp32
@@ -192,36 +237,40 @@ __device__ __forceinline__ void neg_min_split(const float dmin, const uint32_t m
 
 // Workgroup = WM x WN waves, every wave owns NB x NB MFMA blocks of 32 x 32:
 //   <4, 2, 2>: 256 x 128 tile, 512 threads      <2, 2, 2>: 128 x 128, 256 threads      <2, 1, 1>: 64 x 32, 128 threads
-template <int WM, int WN, int NB>
+template <int QT, int WM, int WN, int NB>
 struct Tile {
     static constexpr int BM = 32 * NB * WM, BN = 32 * NB * WN, kThreads = 64 * WM * WN;
     static constexpr int kUnits = kThreads / BN;   // threads per weight row
     static constexpr int kBTasks = 4 / kUnits;     // (piece, plane) tasks per thread and stage
-    static constexpr int kPieces = kBTasks == 4 ? 2 : 1;
+    // 16-byte pieces of weight data per thread and stage: Q4_K one or two quant pieces; Q6_K ql + qh per task
+    static constexpr int kPieces = QT == 14 ? 2 * kBTasks : (kBTasks == 4 ? 2 : 1);
+    static constexpr int kBItems = (QT == 14 ? 16 : 8) * BN;  // items of one B stage (Q6_K: two tiles)
+    static constexpr int kBlockBytes = QT == 14 ? 210 : 144;
     static constexpr int kAItems = 8 * BM / kThreads;  // A items per thread and stage
-    static constexpr size_t kLdsBytes = (size_t)(2 * 8 * BM + 2 * 8 * BN + 4 * BN) * 16 + BN * 4;
+    static constexpr size_t kLdsBytes = (size_t)(2 * 8 * BM + 2 * kBItems + 4 * BN) * 16 + BN * 4;
     static_assert(kUnits == 1 || kUnits == 2 || kUnits == 4, "a weight row is staged by 1, 2 or 4 threads");
     static_assert(8 * BM % kThreads == 0, "the A tile must divide among the threads");
 };
 
-template <int ORDER, bool YBF16, int WM, int WN, int NB>
-__global__ __launch_bounds__(64 * WM * WN, NB == 1 ? 2 : 512 / (64 * WM * WN)) void k_qgemm_q4k(
+template <int QT, int ORDER, bool YBF16, int WM, int WN, int NB>
+__global__ __launch_bounds__(64 * WM * WN, NB == 1 ? 2 : 512 / (64 * WM * WN)) void k_qgemm(
     const uint8_t *__restrict__ W, const uint4 *__restrict__ xs, const uint4 *__restrict__ xsum,
     const float *__restrict__ rowscale, void *__restrict__ yg, int M, int Mp, int N, int spr) {
-    using TL = Tile<WM, WN, NB>;
+    using TL = Tile<QT, WM, WN, NB>;
     constexpr int BM = TL::BM, BN = TL::BN, kThreads = TL::kThreads, kUnits = TL::kUnits, kBTasks = TL::kBTasks,
-                  kPieces = TL::kPieces, kAItems = TL::kAItems;
+                  kPieces = TL::kPieces, kAItems = TL::kAItems, kBItems = TL::kBItems;
+    constexpr bool kQ6 = QT == 14;
     // LDS: two stages of the A tile [8 chunks][BM] and the B tile [4 k-steps][2 k-groups][BN] (16-byte items),
     // the B operand of the R product [2][2][BN] and d [BN] of the current super-block.
     extern __shared__ uint4 smem[];
     uint4 *lds_a = smem;
     uint4 *lds_b = lds_a + 2 * 8 * BM;
-    uint4 *lds_r = lds_b + 2 * 8 * BN;
+    uint4 *lds_r = lds_b + 2 * kBItems;
     float *lds_d = reinterpret_cast<float *>(lds_r + 4 * BN);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;  // wave position in the WM x WN grid
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-    const size_t row_bytes = (size_t)spr * 144;
+    const size_t row_bytes = (size_t)spr * TL::kBlockBytes;
 
     // ---- loader roles ----
     // A: item idx = tid + i * kThreads (i < kAItems) -> chunk = idx / BM, row = idx % BM: a wave copies 64
@@ -244,16 +293,30 @@ __global__ __launch_bounds__(64 * WM * WN, NB == 1 ? 2 : 512 / (64 * WM * WN)) v
     };
     auto fetch_b = [&](int step, u32x4 &fhdr, u32x4 (&fpc)[kPieces]) __attribute__((always_inline)) {
         step = step < last_step ? step : last_step;
-        const uint8_t *blk = wrow + (size_t)(step >> 2) * 144;
-        fhdr = *reinterpret_cast<const u32x4 *>(blk);
-        // the stage covers sub-blocks 2c and 2c+1, c = step % 4, which are pieces 2c and 2c+1 in both orders
+        const uint8_t *blk = wrow + (size_t)(step >> 2) * TL::kBlockBytes;
         const int c = step & 3;
-        if (kPieces == 2) {
+        if constexpr (kQ6) {
+            // stage c covers elements 64 c .. + 63 of the super-block: half h = c / 2, the low (c even) or high
+            // nibbles of ql bytes 64 h .. + 63 in natural order, qh bytes 32 h + (k % 32) at bit 2 (2 (c % 2) + k / 32),
+            // scales 4 c .. 4 c + 3 (crates/pmetal-gguf/src/k_quants.rs:484-494).  Task = one 16-element scale group.
+            const int h = c >> 1;
 #pragma unroll
-            for (int q = 0; q < kPieces; q++) fpc[q] = *reinterpret_cast<const u32x4 *>(blk + 16 + 16 * (2 * c + q));
+            for (int t = 0; t < kBTasks; t++) {
+                const int ks = bu * kBTasks + t;
+                fpc[t] = load16_a2(blk + 64 * h + 16 * ks);
+                fpc[kBTasks + t] = load16_a2(blk + 128 + 32 * h + 16 * (ks & 1));
+            }
+            fhdr = u32x4{reinterpret_cast<const u32_a2 *>(blk + 192 + 4 * c)->v, *reinterpret_cast<const u16_a2 *>(blk + 208), 0u, 0u};
         } else {
-            const int pc = (bu * kBTasks) >> 1;
-            fpc[0] = *reinterpret_cast<const u32x4 *>(blk + 16 + 16 * (2 * c + pc));
+            fhdr = *reinterpret_cast<const u32x4 *>(blk);
+            // the stage covers sub-blocks 2c and 2c+1, which are pieces 2c and 2c+1 in both orders
+            if (kPieces == 2) {
+#pragma unroll
+                for (int q = 0; q < kPieces; q++) fpc[q] = *reinterpret_cast<const u32x4 *>(blk + 16 + 16 * (2 * c + q));
+            } else {
+                const int pc = (bu * kBTasks) >> 1;
+                fpc[0] = *reinterpret_cast<const u32x4 *>(blk + 16 + 16 * (2 * c + pc));
+            }
         }
     };
     auto stage_a = [&](int stage, const u32x4 (&fa)[kAItems]) __attribute__((always_inline)) {
@@ -262,44 +325,60 @@ __global__ __launch_bounds__(64 * WM * WN, NB == 1 ? 2 : 512 / (64 * WM * WN)) v
     };
     // c = step % 4 is a compile-time constant at every call
     auto stage_b = [&](int stage, int c, const u32x4 &fhdr, const u32x4 (&fpc)[kPieces]) __attribute__((always_inline)) {
-        uint4 *dst = lds_b + stage * 8 * BN;
-        const uint4 hdr4 = make_uint4(fhdr.x, fhdr.y, fhdr.z, fhdr.w);
-        uint32_t sc0, sc1, mn;
-        scale_min_u(hdr4, 2 * c, sc0, mn);
-        scale_min_u(hdr4, 2 * c + 1, sc1, mn);
+        if constexpr (kQ6) {
+            uint4 *dst1 = lds_b + stage * kBItems, *dst2 = dst1 + 8 * BN;
 #pragma unroll
-        for (int t = 0; t < kBTasks; t++) {
-            const int q = bu * kBTasks + t;
-            const int bw = q >> 1, p = q & 1;
-            // nibble plane p of piece bw:
-            //   REF : elements 16 p .. + 15 of sub-block 2c + bw  -> k = 32 bw + 16 p + b, scale 2c + bw
-            //   GGML: elements 16 bw .. + 15 of sub-block 2c + p  -> k = 32 p + 16 bw + b, scale 2c + p
-            const int ks = ORDER == 0 ? 2 * bw + p : 2 * p + bw;
-            const uint32_t sc = (ORDER == 0 ? bw : p) ? sc1 : sc0;
-            const u32x4 pc4 = fpc[kPieces == 2 ? bw : 0];
-            uint4 b0, b1;
-            dequant16(make_uint4(pc4.x, pc4.y, pc4.z, pc4.w), p, sc, b0, b1);
-            dst[(ks * 2 + 0) * BN + bn] = b0;
-            dst[(ks * 2 + 1) * BN + bn] = b1;
-        }
-        if (c == 1) {
-            // once per super-block (while its second stage is being staged, one barrier after the previous
-            // super-block's R product has been issued): d and the B operand of the R product for this column.
-            // item (t, g) = (-h_j, -h_j, -l_j, -l_j, -h_j+1, -h_j+1, -l_j+1, -l_j+1), j = 4 t + 2 g, against
-            // the activations' (h, l, h, l, ...): all four cross products.
-            const float dmin = f16_bits_to_f32(hdr4.x >> 16);
-            if (bu == 0) lds_d[bn] = f16_bits_to_f32(hdr4.x & 0xFFFFu);
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                if (r % kUnits == bu) {
-                    uint32_t sc, mn0, mn1;
-                    scale_min_u(hdr4, 2 * r, sc, mn0);
-                    scale_min_u(hdr4, 2 * r + 1, sc, mn1);
-                    _Float16 h0, l0, h1, l1;
-                    neg_min_split(dmin, mn0, h0, l0);
-                    neg_min_split(dmin, mn1, h1, l1);
-                    const half8_t item = {h0, h0, l0, l0, h1, h1, l1, l1};
-                    lds_r[r * BN + bn] = __builtin_bit_cast(uint4, item);
+            for (int t = 0; t < kBTasks; t++) {
+                const int ks = bu * kBTasks + t;
+                const int sc = (int)(int8_t)(fhdr.x >> (8 * ks));
+                uint4 b1lo, b1hi, b2lo, b2hi;
+                dequant16_q6(fpc[t], fpc[kBTasks + t], 4 * (c & 1), 2 * (2 * (c & 1) + (ks >> 1)), sc, b1lo, b1hi, b2lo, b2hi);
+                dst1[(ks * 2 + 0) * BN + bn] = b1lo;
+                dst1[(ks * 2 + 1) * BN + bn] = b1hi;
+                dst2[(ks * 2 + 0) * BN + bn] = b2lo;
+                dst2[(ks * 2 + 1) * BN + bn] = b2hi;
+            }
+            if (c == 1 && bu == 0) lds_d[bn] = f16_bits_to_f32(fhdr.y);
+        } else {
+            uint4 *dst = lds_b + stage * kBItems;
+            const uint4 hdr4 = make_uint4(fhdr.x, fhdr.y, fhdr.z, fhdr.w);
+            uint32_t sc0, sc1, mn;
+            scale_min_u(hdr4, 2 * c, sc0, mn);
+            scale_min_u(hdr4, 2 * c + 1, sc1, mn);
+    #pragma unroll
+            for (int t = 0; t < kBTasks; t++) {
+                const int q = bu * kBTasks + t;
+                const int bw = q >> 1, p = q & 1;
+                // nibble plane p of piece bw:
+                //   REF : elements 16 p .. + 15 of sub-block 2c + bw  -> k = 32 bw + 16 p + b, scale 2c + bw
+                //   GGML: elements 16 bw .. + 15 of sub-block 2c + p  -> k = 32 p + 16 bw + b, scale 2c + p
+                const int ks = ORDER == 0 ? 2 * bw + p : 2 * p + bw;
+                const uint32_t sc = (ORDER == 0 ? bw : p) ? sc1 : sc0;
+                const u32x4 pc4 = fpc[kPieces == 2 ? bw : 0];
+                uint4 b0, b1;
+                dequant16(make_uint4(pc4.x, pc4.y, pc4.z, pc4.w), p, sc, b0, b1);
+                dst[(ks * 2 + 0) * BN + bn] = b0;
+                dst[(ks * 2 + 1) * BN + bn] = b1;
+            }
+            if (c == 1) {
+                // once per super-block (while its second stage is being staged, one barrier after the previous
+                // super-block's R product has been issued): d and the B operand of the R product for this column.
+                // item (t, g) = (-h_j, -h_j, -l_j, -l_j, -h_j+1, -h_j+1, -l_j+1, -l_j+1), j = 4 t + 2 g, against
+                // the activations' (h, l, h, l, ...): all four cross products.
+                const float dmin = f16_bits_to_f32(hdr4.x >> 16);
+                if (bu == 0) lds_d[bn] = f16_bits_to_f32(hdr4.x & 0xFFFFu);
+    #pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    if (r % kUnits == bu) {
+                        uint32_t sc, mn0, mn1;
+                        scale_min_u(hdr4, 2 * r, sc, mn0);
+                        scale_min_u(hdr4, 2 * r + 1, sc, mn1);
+                        _Float16 h0, l0, h1, l1;
+                        neg_min_split(dmin, mn0, h0, l0);
+                        neg_min_split(dmin, mn1, h1, l1);
+                        const half8_t item = {h0, h0, l0, l0, h1, h1, l1, l1};
+                        lds_r[r * BN + bn] = __builtin_bit_cast(uint4, item);
+                    }
                 }
             }
         }
@@ -328,14 +407,17 @@ __global__ __launch_bounds__(64 * WM * WN, NB == 1 ? 2 : 512 / (64 * WM * WN)) v
 
     // c = step % 4 is a compile-time constant at every call
     auto compute = [&](int stage, int c, int sb) __attribute__((always_inline)) {
-        const uint4 *sa = lds_a + stage * 8 * BM, *sbp = lds_b + stage * 8 * BN;
+        const uint4 *sa = lds_a + stage * 8 * BM, *sbp = lds_b + stage * kBItems;
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
-            half8_t av[NB], bv[NB];
+            half8_t av[NB], bv[NB], bw[NB];
 #pragma unroll
             for (int i = 0; i < NB; i++) av[i] = __builtin_bit_cast(half8_t, sa[(ks * 2 + kgrp) * BM + (wm * NB + i) * 32 + col]);
 #pragma unroll
-            for (int jx = 0; jx < NB; jx++) bv[jx] = __builtin_bit_cast(half8_t, sbp[(ks * 2 + kgrp) * BN + (wn * NB + jx) * 32 + col]);
+            for (int jx = 0; jx < NB; jx++) {
+                bv[jx] = __builtin_bit_cast(half8_t, sbp[(ks * 2 + kgrp) * BN + (wn * NB + jx) * 32 + col]);
+                if (kQ6) bw[jx] = __builtin_bit_cast(half8_t, sbp[8 * BN + (ks * 2 + kgrp) * BN + (wn * NB + jx) * 32 + col]);
+            }
 #pragma unroll
             for (int i = 0; i < NB; i++)
 #pragma unroll
@@ -348,12 +430,13 @@ __global__ __launch_bounds__(64 * WM * WN, NB == 1 ? 2 : 512 / (64 * WM * WN)) v
                     } else {
                         part[i][jx] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bv[jx], part[i][jx], 0, 0, 0);
                     }
+                    if (kQ6) part[i][jx] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bw[jx], part[i][jx], 0, 0, 0);
                 }
         }
         if (c == 3) {
-            // ---- end of a super-block: R product into the accumulators, then acc += d * P ----
+            // ---- end of a super-block: R product into the accumulators (Q4_K), then acc += d * P ----
 #pragma unroll
-            for (int t = 0; t < 2; t++) {
+            for (int t = 0; t < (kQ6 ? 0 : 2); t++) {
                 half8_t sv[NB], mv[NB];
 #pragma unroll
                 for (int i = 0; i < NB; i++) sv[i] = __builtin_bit_cast(half8_t, xsv[t][i]);
@@ -393,7 +476,7 @@ __global__ __launch_bounds__(64 * WM * WN, NB == 1 ? 2 : 512 / (64 * WM * WN)) v
     fetch_b(DB, fh[0], fp[0]);
     __syncthreads();
 #define PMH_STEP(C)                                                                                      \
-    if ((C) == 2) fetch_xsum(sb);                                                                        \
+    if ((C) == 2 && !kQ6) fetch_xsum(sb);                                                                        \
     if (DA == 1) {                                                                                       \
         fetch_a(step + (C) + 1, fa[0]);                                                                  \
         __builtin_amdgcn_sched_barrier(0); /* keep the requests a whole step ahead of their use */       \
@@ -449,11 +532,11 @@ size_t qgemm_workspace_bytes(int64_t m, int64_t k) {
     return align256(mp * (size_t)k * 2) + align256(mp * (size_t)(k / 256) * 4 * 16) + align256(mp * 4);
 }
 
-template <int ORDER, bool YBF16, int WM, int WN, int NB>
+template <int QT, int ORDER, bool YBF16, int WM, int WN, int NB>
 static hipError_t launch_tile(hipStream_t s, const uint8_t *w, const uint4 *xs, const uint4 *xsum, const float *rowscale,
                               void *y, int64_t m, int64_t mp, int64_t n, int spr) {
-    using TL = Tile<WM, WN, NB>;
-    auto kern = k_qgemm_q4k<ORDER, YBF16, WM, WN, NB>;
+    using TL = Tile<QT, WM, WN, NB>;
+    auto kern = k_qgemm<QT, ORDER, YBF16, WM, WN, NB>;
     if (TL::kLdsBytes > 64 * 1024) {
         hipError_t a = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)TL::kLdsBytes);
@@ -464,19 +547,19 @@ static hipError_t launch_tile(hipStream_t s, const uint8_t *w, const uint4 *xs, 
     return hipGetLastError();
 }
 
-template <int ORDER, bool YBF16>
+template <int QT, int ORDER, bool YBF16>
 static hipError_t launch_shape(hipStream_t s, const uint8_t *w, const uint4 *xs, const uint4 *xsum, const float *rowscale,
                                void *y, int64_t m, int64_t mp, int64_t n, int spr) {
     // tile by m: short activation batches use small tiles, so that less of the MFMA work is padding and the
     // weight matrix spreads over enough workgroups to pull it from HBM at speed
-    if (m <= 64) return launch_tile<ORDER, YBF16, 2, 1, 1>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
-    if (m <= 256) return launch_tile<ORDER, YBF16, 2, 2, 2>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
-    return launch_tile<ORDER, YBF16, 4, 2, 2>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
+    if (m <= 64) return launch_tile<QT, ORDER, YBF16, 2, 1, 1>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
+    if (m <= 256) return launch_tile<QT, ORDER, YBF16, 2, 2, 2>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
+    return launch_tile<QT, ORDER, YBF16, 4, 2, 2>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
 }
 
 hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype,
                         int64_t m, void *y, uint32_t y_dtype, uint32_t order, void *workspace, hipStream_t s) {
-    if (type != kTypeQ4K) return hipErrorNotSupported;
+    if (type != kTypeQ4K && type != kTypeQ6K) return hipErrorNotSupported;
     if (k % 256 != 0 || m <= 0 || n <= 0) return hipErrorInvalidValue;
     const int64_t mp = padded_rows(m);
     uint8_t *ws = reinterpret_cast<uint8_t *>(workspace);
@@ -495,11 +578,14 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
     if (e != hipSuccess) return e;
     const int spr = (int)(k / 256);
     const bool ybf = y_dtype == kDtypeBf16;
+    if (type == kTypeQ6K)  // one element order
+        return ybf ? launch_shape<14, 0, true>(s, w, xs, xsum, rowscale, y, m, mp, n, spr)
+                   : launch_shape<14, 0, false>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
     if (order == kOrderRef)
-        return ybf ? launch_shape<0, true>(s, w, xs, xsum, rowscale, y, m, mp, n, spr)
-                   : launch_shape<0, false>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
-    return ybf ? launch_shape<1, true>(s, w, xs, xsum, rowscale, y, m, mp, n, spr)
-               : launch_shape<1, false>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
+        return ybf ? launch_shape<12, 0, true>(s, w, xs, xsum, rowscale, y, m, mp, n, spr)
+                   : launch_shape<12, 0, false>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
+    return ybf ? launch_shape<12, 1, true>(s, w, xs, xsum, rowscale, y, m, mp, n, spr)
+               : launch_shape<12, 1, false>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
 }
 
 }  // namespace pmh

@@ -113,7 +113,30 @@ def test_qgemm_argument_errors():
     assert lib.pmetal_hip_qgemm(Q4K, buf.ptr, 4, 256, buf.ptr, 1, 4, buf.ptr, 7, 0, None) == 1   # y_dtype
 
 
-@pytest.mark.parametrize("t", [Q6K, Q8_0])
+@pytest.mark.parametrize("m,n,k", [(1, 128, 256), (16, 128, 512), (64, 256, 1024), (128, 384, 4096), (33, 200, 768),
+                                   (130, 129, 256), (300, 512, 2048), (512, 1024, 2048)])
+def test_qgemm_q6k_matches_dequantize_then_matmul(oracle, m, n, k):
+    wq = oracle.quantize(Q6K, weights(60 + m, n * k))
+    x = np.random.default_rng(61 + m).standard_normal((m, k)).astype(np.float32)
+    bits = oracle.f32_to_bf16_bits(x.reshape(-1)).reshape(m, k)
+    xb = oracle.bf16_bits_to_f32(bits.reshape(-1)).reshape(m, k)
+    want = reference(oracle, Q6K, wq, n, k, xb, 0)
+    got = gpu_qgemm(Q6K, wq, n, k, bits, m)
+    elem, norm = rel_errors(got.reshape(-1), want.reshape(-1))
+    print(f"Q6_K GEMM m={m} n={n} k={k}: elem {elem:.2e} norm {norm:.2e}")
+    assert elem <= TOL and norm <= TOL
+    if m == 16:  # extreme scales: every |sc| = 128 sub-block and the all-zero super-block (d = -0)
+        w = weights(62, n * k)
+        w[: 256] = 0.0
+        w[256:512] = np.where(np.arange(256) % 2 == 0, 1.0, -1.0).astype(np.float32)
+        wq = oracle.quantize(Q6K, w)
+        want = reference(oracle, Q6K, wq, n, k, xb, 0)
+        got = gpu_qgemm(Q6K, wq, n, k, bits, m)
+        elem, norm = rel_errors(got.reshape(-1), want.reshape(-1))
+        assert elem <= TOL and norm <= TOL
+
+
+@pytest.mark.parametrize("t", [Q8_0])
 def test_qlinear_runs_rowwise_gemv_for_types_without_gemm(oracle, t):
     n, k, m = 96, 512, 3
     wq = oracle.quantize(t, weights(51, n * k))
