@@ -255,33 +255,10 @@ __device__ __forceinline__ float lane_dot(const uint4 hdr, const uint4 qv, const
     }
 }
 
-#ifdef PMH_TRACE
-// experiment hook: per-wave cycle stamps kept in registers and written out when the kernel ends
-__device__ unsigned long long *g_trace;  // [workgroup][wave][8], set by the harness
-#define PMH_STAMP_DECL unsigned long long pmh_st[8] = {0, 0, 0, 0, 0, 0, 0, 0}, pmh_rt[2] = {0, 0}
-#define PMH_STAMP(slot) pmh_st[slot] = __builtin_readcyclecounter()
-#define PMH_RT(slot) pmh_rt[slot >> 2] = __builtin_amdgcn_s_memrealtime()
-#define PMH_STAMP_FLUSH                                                                     \
-    do {                                                                                    \
-        if ((threadIdx.x & 63) == 0)                                                        \
-            for (int q = 0; q < 8; q++)                                                     \
-                g_trace[((size_t)blockIdx.x * 16 + (threadIdx.x >> 6)) * 8 + q] =           \
-                    q == 5 ? pmh_rt[0] : q == 7 ? pmh_rt[1] : pmh_st[q];                    \
-    } while (0)
-#else
-#define PMH_STAMP_DECL
-#define PMH_STAMP(slot)
-#define PMH_RT(slot)
-#define PMH_STAMP_FLUSH
-#endif
-
 // Conversion of x into LDS in two steps, so that the first pass of activation loads can be requested before
 // the weight loads queue up behind it: stage_x_begin loads, stage_x_finish converts (and runs the further
 // passes a long row needs).  All threads of the workgroup take part; the caller places the barrier.
-#ifndef PMH_STAGE_PRE
-#define PMH_STAGE_PRE 2
-#endif
-constexpr int kStagePre = PMH_STAGE_PRE;  // passes of activation loads requested up front
+constexpr int kStagePre = 2;  // passes of activation loads requested up front
 
 template <int ORDER, bool XF32>
 __device__ __forceinline__ void stage_x_begin(const void *xg, int slots, int nthreads, uint4 (&r_lo)[kStagePre],
@@ -330,10 +307,7 @@ __device__ __forceinline__ void stage_x_finish(const void *xg, int slots, int nt
 // lanes the same address) so that the number of outstanding loads is known at every wait.  Each lane's
 // partial sum goes to LDS; after a barrier the workgroup adds up the partials of each of its rows.
 constexpr int kDepth = 8;  // tasks in flight per wave
-#ifndef PMH_KPRE
-#define PMH_KPRE 2
-#endif
-constexpr int kPre = PMH_KPRE;  // of which this many are requested before x is converted
+constexpr int kPre = 2;  // of which this many are requested before x is converted
 
 // Row stride of the partial sums in LDS.  The final summation puts `red` lanes on a row (lane p adds every
 // red-th partial), 64 / red rows side by side in a wave: a stride of `red` floats past a multiple of 64 keeps
@@ -354,10 +328,6 @@ __global__ __launch_bounds__(1024) void k_qgemv_q4k_chunk(const uint8_t *__restr
     float4 *xm = reinterpret_cast<float4 *>(xd + NDIG * slots);
     float *part = reinterpret_cast<float *>(xm + slots);  // [group][n_nominal * RPT][part_stride(slots)]
     const int ps = part_stride(slots, red);
-
-    PMH_STAMP_DECL;
-    PMH_STAMP(0);
-    PMH_RT(0);
     const int lane = threadIdx.x & 63;
     const int lt = lane & (T - 1), tm = lane / T, j = lane & 7;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -387,11 +357,8 @@ __global__ __launch_bounds__(1024) void k_qgemv_q4k_chunk(const uint8_t *__restr
     uint4 bh[kDepth], bq[kDepth];
 #pragma unroll
     for (int i = 0; i < kPre; i++) issue(i, bh[i], bq[i]);
-    PMH_STAMP(1);
     stage_x_finish<ORDER, NDIG, XF32>(xg, slots, nthreads, x_lo, x_hi, xd, xm);
-    PMH_STAMP(2);
     __syncthreads();
-    PMH_STAMP(3);
 
     const ScaleSel s0 = scale_sel(ORDER == 0 ? j : 2 * (j >> 1));
     const ScaleSel s1 = scale_sel(ORDER == 0 ? j : 2 * (j >> 1) + 1);
@@ -420,7 +387,6 @@ __global__ __launch_bounds__(1024) void k_qgemv_q4k_chunk(const uint8_t *__restr
 #pragma unroll
         for (; issued < upto; issued++) issue(issued, bh[issued % kDepth], bq[issued % kDepth]);
     }
-    PMH_STAMP(4);
     if (!SINGLE) {
         // steady rounds: consume task t, refill its buffer with task t + kDepth
         int base = kDepth;
@@ -435,7 +401,6 @@ __global__ __launch_bounds__(1024) void k_qgemv_q4k_chunk(const uint8_t *__restr
 #pragma unroll
         for (int i = 0; i < kDepth; i++) consume(base + i, bh[i], bq[i]);
     }
-    PMH_STAMP(5);
     __syncthreads();
 
     // Row totals: `red` lanes per row (a power of two from 8 to 64 that divides slots), lane p adding every
@@ -463,9 +428,6 @@ __global__ __launch_bounds__(1024) void k_qgemv_q4k_chunk(const uint8_t *__restr
         const float sum = team_sum_rt((t0 + t1) + (t2 + t3), red);
         if (ok && p == 0) y[wg_r0 + rl] = sum;
     }
-    PMH_STAMP(6);
-    PMH_RT(7);
-    PMH_STAMP_FLUSH;
 }
 
 // ---- kernel B: general shapes -------------------------------------------------------------------
@@ -681,10 +643,9 @@ hipError_t launch_qgemv_q4k(const uint8_t *w, int64_t n, int64_t k, const void *
     const size_t lds_x = slots * 16 * (xf32 ? 6 : 5) + slots * 16;
     if (lds_x > gemv::kMaxLds) return hipErrorInvalidValue;
 
-    // Workgroups own contiguous chunks of rows, about `wgs_per_cu` per compute unit (x is staged once per
+    // Workgroups own contiguous chunks of rows, one per compute unit (x is staged once per
     // workgroup).
-    const int64_t wgs_per_cu = gemv::tuning("PMETAL_HIP_GEMV_WGS_PER_CU", 1);
-    const int64_t want = (int64_t)gemv::compute_units() * (wgs_per_cu > 0 ? wgs_per_cu : 1);
+    const int64_t want = gemv::compute_units();
     int64_t n_wg = n < want ? n : want;
     const int64_t rows_per_wg = (n + n_wg - 1) / n_wg;
     n_wg = (n + rows_per_wg - 1) / rows_per_wg;
@@ -694,11 +655,10 @@ hipError_t launch_qgemv_q4k(const uint8_t *w, int64_t n, int64_t k, const void *
     // enough work per compute unit to pay for its second barrier (measured crossover: about 12 MiB of weights).
     const int ks = spr / (T / 8), rpt = 64 / T;
     const uint64_t w_bytes = (uint64_t)n * (uint64_t)spr * 144u;
-    const int64_t mode = gemv::tuning("PMETAL_HIP_GEMV_KERNEL", 0);  // 0 = choose, 1 = kernel A, 2 = kernel B
+    static const int64_t mode = gemv::tuning("PMETAL_HIP_GEMV_KERNEL", 0);  // 0 = choose, 1 = kernel A, 2 = kernel B
     const bool want_a = mode == 1 || (mode == 0 && w_bytes >= (12ull << 20));
     if (want_a && ks <= 16 && w_bytes < (1ull << 32)) {
-        const int64_t max_waves = gemv::tuning("PMETAL_HIP_GEMV_WAVES", 16);
-        int64_t groups = (max_waves >= ks && max_waves <= 16 ? max_waves : 16) / ks;
+        int64_t groups = 16 / ks;
         const int64_t max_groups = (rows_per_wg + rpt - 1) / rpt;
         if (groups > max_groups) groups = max_groups;
         const int64_t rows_per_wave = (rows_per_wg + groups - 1) / groups;
@@ -706,8 +666,7 @@ hipError_t launch_qgemv_q4k(const uint8_t *w, int64_t n, int64_t k, const void *
         const int64_t n_nominal = (rows_per_wave + rpt - 1) / rpt;
         const int64_t threads = ks * groups * 64;
         int red = 8;  // lanes per row in the final summation: as many as the workgroup has to spare, at most T
-        const int64_t red_cap = gemv::tuning("PMETAL_HIP_GEMV_RED", 64);
-        while (red < red_cap && red * 2 <= T && rows_per_wg * red * 2 <= threads) red *= 2;
+        while (red < 64 && red * 2 <= T && rows_per_wg * red * 2 <= threads) red *= 2;
         const size_t lds = lds_x + (size_t)groups * (size_t)n_nominal * rpt * part_stride((int)slots, red) * 4;
         if (lds <= 128 * 1024) {
             const dim3 block((unsigned)threads);

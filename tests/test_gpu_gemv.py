@@ -47,6 +47,29 @@ def test_qgemv_matches_dequantize_then_matmul(oracle, t, n, k, x_dtype):
         assert elem <= TOL and norm <= TOL
 
 
+# Shapes of 12 MiB and more take the chunk-owner kernel: ragged row counts (the last workgroup, wave and task are
+# short), 32-lane teams (k / 256 = 12), a row count below the number of compute units times the waves, and a
+# row of 16 chunks (k = 32768).
+BIG_CASES = [(6001, 4096), (7301, 3072), (3001, 8192), (16385, 1536), (800, 32768)]
+
+
+@pytest.mark.parametrize("n,k", BIG_CASES)
+@pytest.mark.parametrize("x_dtype", [pm.DTYPE_BF16, pm.DTYPE_F32])
+def test_qgemv_q4k_large_ragged_shapes(oracle, n, k, x_dtype):
+    # quantized bytes generated directly (every byte pattern is a valid block; d and dmin kept small and finite)
+    rng = np.random.default_rng(n + k)
+    raw = rng.integers(0, 256, size=(n * (k // 256), 144), dtype=np.uint8)
+    raw[:, 0:4] = np.frombuffer(np.array([0.01, 0.02], np.float16).tobytes(), np.uint8)
+    raw = raw.reshape(-1)
+    x_dev, x_ref = activations(oracle, n, k, x_dtype)
+    for order in (0, 1):
+        want = oracle.qmatvec(Q4K, raw, n, k, x_ref, order=order)
+        got = gpu_qgemv(Q4K, raw, n, k, x_dev, x_dtype, order)
+        elem, norm = rel_errors(got, want)
+        print(f"Q4_K {n}x{k} x_dtype {x_dtype} order {order}: elem {elem:.2e} norm {norm:.2e}")
+        assert elem <= TOL and norm <= TOL
+
+
 def test_qgemv_config0_q8_0_round_trip_and_gemv(oracle):
     # BASELINE config 0: 3072x1024 N(0, 0.02), Q8_0 round trip, then y = W x with f32 x ~ N(0, 1)
     n, k = 3072, 1024
