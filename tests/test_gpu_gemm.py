@@ -38,7 +38,7 @@ def reference(oracle, t, wq, n, k, x_f32, order):
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 128, 256), (16, 128, 512), (64, 256, 1024), (128, 384, 4096), (33, 200, 768),
-                                   (130, 129, 256), (512, 512, 2048)])
+                                   (130, 129, 256), (512, 512, 2048), (257, 160, 512), (300, 100, 768)])
 def test_qgemm_q4k_matches_dequantize_then_matmul(oracle, m, n, k):
     wq = oracle.quantize(Q4K, weights(m + n + k, n * k, outliers=1e-3))
     x = np.random.default_rng(m * 7 + k).standard_normal((m, k)).astype(np.float32)
@@ -70,6 +70,28 @@ def test_qgemm_bf16_output_and_large_activations(oracle):
     for row in (0, 3, 5, 63):
         scale = np.max(np.abs(want[row])) or 1.0
         assert np.max(np.abs(got16[row] - want[row])) / scale <= 2.0 ** -8  # bf16 rounding of the output
+
+
+@pytest.mark.parametrize("t", [Q4K, Q6K])
+@pytest.mark.parametrize("m", [24, 200, 300])
+def test_qgemm_f32_activations(oracle, t, m):
+    """f32 activations are rounded once to f16 at the row's power-of-two scale (11 significant bits; a bf16 cast
+    would keep 8): against the unrounded reference the result holds the 1e-3 bound norm-wise, and element-wise
+    against the reference fed the same rounded activations."""
+    n, k = 320, 1024
+    wq = oracle.quantize(t, weights(90 + m, n * k))
+    x = np.random.default_rng(91 + m).standard_normal((m, k)).astype(np.float32)
+    x[1] *= 3e4
+    got = gpu_qgemm(t, wq, n, k, x, m, x_dtype=pm.DTYPE_F32)
+    want = reference(oracle, t, wq, n, k, x, 0)
+    # the kernel's rounding: x * 2^-e to f16 with the row maximum in [2^9, 2^10), then back
+    e = np.floor(np.log2(np.max(np.abs(x), axis=1, keepdims=True))) - 9
+    xr = (np.ldexp(x, (-e).astype(np.int32)).astype(np.float16).astype(np.float32) * np.exp2(e)).astype(np.float32)
+    want_r = reference(oracle, t, wq, n, k, xr, 0)
+    for row in range(m):
+        _, norm = rel_errors(got[row], want[row])
+        elem_r, norm_r = rel_errors(got[row], want_r[row])
+        assert norm <= TOL and elem_r <= TOL and norm_r <= TOL, (row, norm, elem_r, norm_r)
 
 
 def test_qgemm_config2_full_size(oracle):
