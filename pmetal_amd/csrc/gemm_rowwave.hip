@@ -1,0 +1,609 @@
+// Dequant-fused Q4_K GEMM  Y[m,n] = sum_k X[m,k] * W[n,k]  on the gfx950 matrix cores, every wave owning its
+// weight rows.
+//
+// W is the packed GGUF stream [n, k] of 144-byte super-blocks; a weight's value is what the reference's
+// dequantize_q4k yields (crates/pmetal-gguf/src/k_quants.rs:358-404; element order REF or GGML as for the
+// GEMV).  The reference has no fused kernel (it dequantizes on the CPU at load,
+// crates/pmetal-models/src/weight_format.rs:299-303, and multiplies densely); this kernel is checked against
+// exactly that, dequantize-then-matmul, to 1e-3.
+//
+// A wave owns 32 weight rows and dequantizes them straight into MFMA operand registers (no shared weight tile
+// in LDS, no LDS writes by the waves at all); only the activations are shared by the waves of a workgroup.  A
+// launch is cut along N, M and, for short activation batches, K into enough workgroups to fill the machine.
+// The arithmetic is exact up to the fp32 accumulation (see gemm.hip, which keeps the same scheme for Q6_K):
+// integer tiles sc * q in f16, activations scaled per row by a power of two into the f16 range, the
+// per-super-block factor d applied to the fp32 partial sums, the min term as a K = 32 MFMA product of exact
+// head + tail splits.
+//
+// Data movement uses direct global -> LDS loads only (no staging registers, no ds_write):
+//   * activations: a pre-pass writes 16-byte items (8 f16) in the order the MFMA wants them,
+//     xs[(2 sb + h) * 18 + grp][Mp], per half super-block h 16 operand groups (k-step t, lane half g) and two
+//     groups of sub-block sums; a workgroup copies the 18 x BM items of a half super-block into one of two
+//     LDS stages while it computes on the other (one barrier per half super-block);
+//   * weights: each wave copies the 64 quant bytes per row of a half super-block (coalesced: four lanes per
+//     row) two half super-blocks ahead, and the 16-byte headers one super-block ahead, into its private LDS
+//     region; then every lane (row n = lane % 32, half g = lane / 32) reads back the 32 bytes it multiplies:
+//     dword t of them holds the eight 4-bit quants of MFMA k-step t.  Which k they are is a property of the
+//     element order, matched by the pre-pass:
+//         GGML: k = 64 (2h + g) + 4t + e (low nibbles, sub-block 4h+2g), + 32 (high nibbles, sub-block 4h+2g+1)
+//         REF : k = 32 (4h + 2g + t/4) + 4 (t%4) + e (low), + 16 (high), both sub-block 4h + 2g + t/4
+// With a K split (grid.z > 1) the workgroups write fp32 partial tiles and a small kernel adds them in a fixed
+// order, so the result does not depend on scheduling.
+//
+// What bounds it: every matrix instruction reads its 1 KiB activation fragment from LDS (a wave cannot reuse a
+// fragment for a second group of weight rows without doubling the dequantization work per matrix instruction,
+// which measured slower), so a 128-row workgroup is bound by the LDS read rate at about 60 % of the matrix
+// peak.
+#include "internal.hpp"
+
+namespace {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kGroups = 18;    // 16-byte items per activation row and half super-block
+constexpr int kBlockBytes = 144;
+
+#define PMH_GPTR(p) ((const __attribute__((address_space(1))) void *)(p))
+#define PMH_LPTR(p) ((__attribute__((address_space(3))) void *)(p))
+
+// 16 bytes per lane from global memory to LDS: lane l lands at dst + 16 l (dst is wave-uniform).
+__device__ __forceinline__ void dma16(const void *src, uint4 *dst) {
+    __builtin_amdgcn_global_load_lds(PMH_GPTR(src), PMH_LPTR(dst), 16, 0, 0);
+}
+
+// Workgroup barrier that leaves the newest `keep` vector-memory requests in flight.  (__syncthreads() carries a
+// release fence, which waits for every direct-to-LDS copy.)  The copies that the other waves will read are older
+// than those, and this wave's own LDS reads have returned (lgkmcnt(0)) before another wave may refill a stage.
+template <int KEEP>
+__device__ __forceinline__ void barrier_keep() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0x0070 | KEEP);  // vmcnt(KEEP) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+}
+__device__ __forceinline__ float bf16_to_f32(uint32_t h) { return __builtin_bit_cast(float, h << 16); }
+
+// ------------------------------------------------------------------------------------------------
+// Pre-pass: one workgroup per activation row m < Mp.  rowscale[m] = 2^e with the row maximum * 2^-e in
+// [2^9, 2^10) (bf16 activations are then exact in f16 and block sums stay below 2^15); rows >= M are zero.
+// One thread per operand item: chunk u = 64 elements = sub-blocks 2u, 2u+1 (u = 4 sb + 2 h + g), k-step t.
+// ------------------------------------------------------------------------------------------------
+template <bool XF32, int ORDER>
+__global__ __launch_bounds__(256) void k_prep_rw(const void *__restrict__ xg, int64_t k, int M, int Mp,
+                                                  float *__restrict__ rowscale, uint4 *__restrict__ xs) {
+    const int m = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
+    const bool live = m < M;
+    __shared__ float red[4];
+    float amax = 0.0f;
+    if (live) {
+        if (XF32) {
+            const float4 *row = reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(xg) + (int64_t)m * k);
+            for (int64_t i = tid; i < k / 4; i += 256) {
+                const float4 v = row[i];
+                amax = __builtin_fmaxf(__builtin_fmaxf(amax, __builtin_fmaxf(__builtin_fabsf(v.x), __builtin_fabsf(v.y))),
+                                       __builtin_fmaxf(__builtin_fabsf(v.z), __builtin_fabsf(v.w)));
+            }
+        } else {
+            const uint4 *row = reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(xg) + (int64_t)m * k);
+            for (int64_t i = tid; i < k / 8; i += 256) {
+                const uint4 v = row[i];
+                const uint32_t r[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                    amax = __builtin_fmaxf(amax, __builtin_fmaxf(__builtin_fabsf(bf16_to_f32(r[q] & 0xFFFFu)),
+                                                                 __builtin_fabsf(bf16_to_f32(r[q] >> 16))));
+            }
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) amax = __builtin_fmaxf(amax, __shfl_xor(amax, off));
+    if (lane == 0) red[tid >> 6] = amax;
+    __syncthreads();
+    amax = __builtin_fmaxf(__builtin_fmaxf(red[0], red[1]), __builtin_fmaxf(red[2], red[3]));
+    const int eb = (int)((__builtin_bit_cast(uint32_t, amax) >> 23) & 0xFFu);  // amax in [2^(eb-127), 2^(eb-126))
+    int e = eb - 126 - 10;
+    e = e < -126 ? -126 : (e > 126 ? 126 : e);
+    if (eb == 255) e = 0;  // inf / NaN: let them through
+    const float up = __builtin_bit_cast(float, (uint32_t)(127 + e) << 23);
+    if (tid == 0) rowscale[m] = up;
+    const float down = live ? 1.0f / up : 0.0f;  // exact: a power of two
+
+    for (int64_t q = tid; q < k / 8; q += 256) {
+        const int64_t u = q >> 3;
+        const int t = (int)(q & 7);
+        const int64_t lo = ORDER == 0 ? 64 * u + 32 * (t >> 2) + 4 * (t & 3) : 64 * u + 4 * t;
+        const int64_t hi = lo + (ORDER == 0 ? 16 : 32);
+        float v[8];
+        if (!live) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[i] = 0.0f;
+        } else if (XF32) {
+            const float *row = reinterpret_cast<const float *>(xg) + (int64_t)m * k;
+            const float4 a = *reinterpret_cast<const float4 *>(row + lo), b = *reinterpret_cast<const float4 *>(row + hi);
+            v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
+        } else {
+            const uint16_t *row = reinterpret_cast<const uint16_t *>(xg) + (int64_t)m * k;
+            const uint2 a = *reinterpret_cast<const uint2 *>(row + lo), b = *reinterpret_cast<const uint2 *>(row + hi);
+            v[0] = bf16_to_f32(a.x & 0xFFFFu), v[1] = bf16_to_f32(a.x >> 16), v[2] = bf16_to_f32(a.y & 0xFFFFu), v[3] = bf16_to_f32(a.y >> 16);
+            v[4] = bf16_to_f32(b.x & 0xFFFFu), v[5] = bf16_to_f32(b.x >> 16), v[6] = bf16_to_f32(b.y & 0xFFFFu), v[7] = bf16_to_f32(b.y >> 16);
+        }
+        half8_t h;
+        float slo = 0.0f, shi = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            h[i] = (_Float16)(v[i] * down);
+            if (i < 4) slo += (float)h[i];
+            else shi += (float)h[i];
+        }
+        const int64_t sb = u >> 2;
+        const int hh = (int)(u >> 1) & 1, g = (int)u & 1;
+        const size_t base = (size_t)((sb * 2 + hh) * kGroups) * Mp + m;
+        xs[base + (size_t)(t * 2 + g) * Mp] = __builtin_bit_cast(uint4, h);
+        // sums of the two sub-blocks of the chunk over its 8 k-steps (8 consecutive lanes)
+        float s0, s1;
+        if (ORDER == 0) {  // sub-block 2u: k-steps 0..3 (low and high nibbles), 2u+1: k-steps 4..7
+            float s = slo + shi;
+            s += __shfl_xor(s, 1);
+            s += __shfl_xor(s, 2);
+            s0 = s;
+            s1 = __shfl_down(s, 4);
+        } else {  // sub-block 2u: the low nibbles of all k-steps, 2u+1: the high nibbles
+            slo += __shfl_xor(slo, 1), shi += __shfl_xor(shi, 1);
+            slo += __shfl_xor(slo, 2), shi += __shfl_xor(shi, 2);
+            slo += __shfl_xor(slo, 4), shi += __shfl_xor(shi, 4);
+            s0 = slo, s1 = shi;
+        }
+        if (t == 0) {  // exact head + tail split of each sum; item (H0, L0, H0, L0, H1, L1, H1, L1)
+            const _Float16 h0 = (_Float16)s0, h1 = (_Float16)s1;
+            const _Float16 l0 = (_Float16)(s0 - (float)h0), l1 = (_Float16)(s1 - (float)h1);
+            const half8_t item = {h0, l0, h0, l0, h1, l1, h1, l1};
+            xs[base + (size_t)(16 + g) * Mp] = __builtin_bit_cast(uint4, item);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// main kernel
+// ------------------------------------------------------------------------------------------------
+// per-thread constants of the copy roles; a wave owns NR groups of 32 weight rows
+template <int MB, int NR, int NW>
+struct Lane {
+    static constexpr int BM = 32 * MB, kThreads = 64 * NW;
+    static constexpr int kARounds = (kGroups * BM + kThreads - 1) / kThreads;
+    int wave, col, g;
+    uint32_t q_off[NR][2];     // byte offset of this lane's quant piece of round r from the workgroup's first row
+    uint32_t h_off[NR];        // ... of this lane's header
+    uint32_t a_off[kARounds];  // item offset of this lane's activation item of round i from (group 0, row m0)
+};
+
+template <int MB, int NR>
+struct Acc {
+    float16_t acc[NR][MB], part[NR][MB];
+    u32x4 hdr[NR];  // headers of the current super-block: d | dmin << 16, then the 12 scale bytes
+};
+
+// 8 quants of one dword (low nibbles, then high nibbles) times their integer scales -> 8 exact f16 values.
+// 0x6400 | q is the f16 1024 + q; (1024 + q) * sc - 1024 * sc is exact in a packed f16 fma.
+__device__ __forceinline__ half8_t dequant8(const uint32_t w, const half2_t sc_lo, const half2_t off_lo, const half2_t sc_hi,
+                                            const half2_t off_hi) {
+    const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
+    const half2_t r0 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, lo, 0x04010400u)), sc_lo, off_lo);
+    const half2_t r1 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, lo, 0x04030402u)), sc_lo, off_lo);
+    const half2_t r2 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, hi, 0x04010400u)), sc_hi, off_hi);
+    const half2_t r3 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, hi, 0x04030402u)), sc_hi, off_hi);
+    return half8_t{r0[0], r0[1], r1[0], r1[1], r2[0], r2[1], r3[0], r3[1]};
+}
+
+// The same in four pieces, so that the pieces can be placed between matrix instructions.  k-step t selects the
+// scales: GGML order multiplies the low nibbles by the first and the high nibbles by the second sub-block scale,
+// REF order both by the scale of sub-block t / 4.
+struct Dq {
+    uint32_t lo, hi;
+    half2_t r[4];
+    __device__ __forceinline__ half8_t value() const { return half8_t{r[0][0], r[0][1], r[1][0], r[1][1], r[2][0], r[2][1], r[3][0], r[3][1]}; }
+};
+template <int ORDER>
+__device__ __forceinline__ void dq_chunk(const int c, const int t, const uint32_t w, const half2_t (&sc2)[2], const half2_t (&off2)[2], Dq &d) {
+    const int lo_s = ORDER == 0 ? (t >> 2) : 0, hi_s = ORDER == 0 ? (t >> 2) : 1;
+    if (c == 0) {
+        d.lo = w & 0x0F0F0F0Fu;
+        d.r[0] = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, d.lo, 0x04010400u)), sc2[lo_s], off2[lo_s]);
+    } else if (c == 1) {
+        d.r[1] = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, d.lo, 0x04030402u)), sc2[lo_s], off2[lo_s]);
+        d.hi = (w >> 4) & 0x0F0F0F0Fu;
+    } else if (c == 2) {
+        d.r[2] = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, d.hi, 0x04010400u)), sc2[hi_s], off2[hi_s]);
+    } else {
+        d.r[3] = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, d.hi, 0x04030402u)), sc2[hi_s], off2[hi_s]);
+    }
+}
+
+// -(dmin * mn) split exactly into an f16 head and tail (dmin has 11 significant bits, mn 6).
+__device__ __forceinline__ void neg_min_split(const float dmin, const uint32_t mn, _Float16 &h, _Float16 &l) {
+    const float p = -(dmin * (float)mn);  // exact in fp32
+    h = (_Float16)p;
+    l = (_Float16)(p - (float)h);
+}
+
+// One half super-block H of one wave.  The restrict qualifiers say what the copies in flight cannot touch:
+// operand reads from a_cur / q_cur need not wait for the direct loads into a_nxt / q_nxt / hb.
+//   a_cur / a_nxt: activation stages (18 x BM items)      q_cur / q_nxt: this wave's quant pieces (NR x 128 items)
+//   hb: this wave's headers (NR x 64 items)
+//   xs_nxt: item (group 0, row m0) of the next half super-block    wq_nxt / wh_nxt: first row of the workgroup at
+//   the next half's quant bytes / the next super-block's header
+template <int ORDER, int MB, int NR, int NW, int H>
+__device__ __forceinline__ void rw_half(const uint4 *__restrict__ a_cur, uint4 *__restrict__ a_nxt,
+                                        const uint4 *__restrict__ q_cur, uint4 *__restrict__ q_nxt, uint4 *__restrict__ hb,
+                                        const uint4 *__restrict__ xs_nxt, const uint8_t *__restrict__ wq_nxt,
+                                        const uint8_t *__restrict__ wh_nxt, const Lane<MB, NR, NW> &L, Acc<MB, NR> &R) {
+    constexpr int BM = 32 * MB, kThreads = 64 * NW;
+    const int col = L.col, g = L.g;
+    if (H == 0) {
+#pragma unroll
+        for (int rg = 0; rg < NR; rg++) {
+            const uint4 hv = hb[rg * 64 + col];
+            R.hdr[rg] = u32x4{hv.x, hv.y, hv.z, hv.w};
+        }
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the headers are in registers before their buffer is refilled
+#pragma unroll
+        for (int rg = 0; rg < NR; rg++) dma16(wh_nxt + L.h_off[rg], hb + rg * 64);
+    }
+    // copies for the next half super-block
+#pragma unroll
+    for (int i = 0; i < Lane<MB, NR, NW>::kARounds; i++)
+        if (i * kThreads + L.wave * 64 < kGroups * BM) dma16(xs_nxt + L.a_off[i], a_nxt + i * kThreads + L.wave * 64);
+#pragma unroll
+    for (int rg = 0; rg < NR; rg++)
+#pragma unroll
+        for (int r = 0; r < 2; r++) dma16(wq_nxt + L.q_off[rg][r], q_nxt + rg * 128 + r * 64);
+    __builtin_amdgcn_sched_barrier(0);  // the copies are requested before anything else of this half
+
+    // scales and mins of sub-blocks j0 = 4 H + 2 g and j0 + 1 (6-bit fields, crates/pmetal/src/commands/quantize.rs:844-855)
+    const uint32_t sh = 16u * (uint32_t)g;
+    half2_t sc2[NR][2], off2[NR][2];
+    uint32_t mn[NR][2];
+    uint32_t qd[NR][8];
+    // this lane's 32 quant bytes per row group: pieces 2g and 2g+1 of row col (the copy swizzles the four pieces of
+    // a row by (row / 4) % 4 so that 16 consecutive rows read conflict-free)
+    const int sw = (col >> 2) & 3;
+#pragma unroll
+    for (int rg = 0; rg < NR; rg++) {
+        const uint4 qa = q_cur[rg * 128 + col * 4 + ((2 * g) ^ sw)], qb = q_cur[rg * 128 + col * 4 + ((2 * g + 1) ^ sw)];
+        qd[rg][0] = qa.x, qd[rg][1] = qa.y, qd[rg][2] = qa.z, qd[rg][3] = qa.w;
+        qd[rg][4] = qb.x, qd[rg][5] = qb.y, qd[rg][6] = qb.z, qd[rg][7] = qb.w;
+        uint32_t sc0, sc1;
+        if (H == 0) {
+            const uint32_t yv = R.hdr[rg].y >> sh, zv = R.hdr[rg].z >> sh;
+            sc0 = yv & 63u, sc1 = (yv >> 8) & 63u;
+            mn[rg][0] = zv & 63u, mn[rg][1] = (zv >> 8) & 63u;
+        } else {
+            const uint32_t wv = R.hdr[rg].w >> sh, yv = R.hdr[rg].y >> sh, zv = R.hdr[rg].z >> sh;
+            sc0 = (wv & 0xFu) | ((yv >> 2) & 0x30u), sc1 = ((wv >> 8) & 0xFu) | ((yv >> 10) & 0x30u);
+            mn[rg][0] = ((wv >> 4) & 0xFu) | ((zv >> 2) & 0x30u), mn[rg][1] = ((wv >> 12) & 0xFu) | ((zv >> 10) & 0x30u);
+        }
+        const _Float16 s0 = (_Float16)(float)sc0, s1 = (_Float16)(float)sc1;
+        const _Float16 o0 = (_Float16)(-1024.0f * (float)sc0), o1 = (_Float16)(-1024.0f * (float)sc1);  // exact: sc <= 63
+        sc2[rg][0] = half2_t{s0, s0}, sc2[rg][1] = half2_t{s1, s1};
+        off2[rg][0] = half2_t{o0, o0}, off2[rg][1] = half2_t{o1, o1};
+    }
+
+    // min term of sub-blocks j0, j0 + 1: (-h, -h, -l, -l) against the activations' (H, L, H, L): all four cross
+    // products of the exact head + tail splits, straight into the accumulators (after the eight k-steps)
+    half8_t br[NR];
+#pragma unroll
+    for (int rg = 0; rg < NR; rg++) {
+        const float dmin = f16_bits_to_f32(R.hdr[rg].x >> 16);
+        _Float16 h0, l0, h1, l1;
+        neg_min_split(dmin, mn[rg][0], h0, l0);
+        neg_min_split(dmin, mn[rg][1], h1, l1);
+        br[rg] = half8_t{h0, h0, l0, l0, h1, h1, l1, l1};
+    }
+
+    // Software pipeline, written in issue order (a wave issues in order, so the order here is the schedule):
+    // the activation fragments of k-step t + 1 are requested before the products of k-step t, and the weights of
+    // k-step t + 1 are dequantized in pieces between those products.
+    constexpr int kSlots = MB * NR, kChunks = 4 * NR;
+    half8_t af[2][MB];
+    Dq dq[NR];
+#pragma unroll
+    for (int i = 0; i < MB; i++) af[0][i] = __builtin_bit_cast(half8_t, a_cur[g * BM + 32 * i + col]);
+#pragma unroll
+    for (int rg = 0; rg < NR; rg++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) dq_chunk<ORDER>(c, 0, qd[rg][0], sc2[rg], off2[rg], dq[rg]);
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+        half8_t b[NR];
+#pragma unroll
+        for (int rg = 0; rg < NR; rg++) b[rg] = dq[rg].value();
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < MB; i++)
+#pragma unroll
+            for (int rg = 0; rg < NR; rg++) {
+                const half8_t a = af[t & 1][i];
+                if (H == 0 && t == 0) {  // first product of a super-block starts from zero
+                    float16_t z;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) z[r] = 0.0f;
+                    R.part[rg][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b[rg], z, 0, 0, 0);
+                } else {
+                    R.part[rg][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b[rg], R.part[rg][i], 0, 0, 0);
+                }
+                if (t < 7) {
+                    const int slot = i * NR + rg;
+#pragma unroll
+                    for (int ch = slot * kChunks / kSlots; ch < (slot + 1) * kChunks / kSlots; ch++)
+                        dq_chunk<ORDER>(ch % 4, t + 1, qd[ch / 4][t + 1], sc2[ch / 4], off2[ch / 4], dq[ch / 4]);
+                }
+                if (i == 0 && rg == 0) {
+                    // the next step's fragments are requested behind the first product of this step: the wait in
+                    // front of that product then covers only fragments requested a whole step ago
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int ii = 0; ii < MB; ii++)
+                        af[(t + 1) & 1][ii] = __builtin_bit_cast(half8_t, a_cur[(t < 7 ? (t + 1) * 2 + g : 16 + g) * BM + 32 * ii + col]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+    }
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+#pragma unroll
+        for (int rg = 0; rg < NR; rg++) R.acc[rg][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[0][i], br[rg], R.acc[rg][i], 0, 0, 0);
+    if (H == 1) {
+#pragma unroll
+        for (int rg = 0; rg < NR; rg++) {
+            const float d = f16_bits_to_f32(R.hdr[rg].x & 0xFFFFu);
+#pragma unroll
+            for (int i = 0; i < MB; i++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) R.acc[rg][i][r] = __builtin_fmaf(d, R.part[rg][i][r], R.acc[rg][i][r]);
+        }
+    }
+}
+
+// grid (ceil(N / (32 NR NW)), Mp / BM, splits); workgroup z works on super-blocks [z * chunk, min(spr, (z + 1) * chunk)).
+// mode 0: y f32 [M][N], 1: y bf16, 2: fp32 partial tiles [splits][Mp][N] (not yet scaled by rowscale)
+//
+// Copies in flight: the activation stage of the next half super-block (it comes from L2) and the quant pieces of
+// the next two (they come from HBM): three quant stages per wave, rotated.  Within a half super-block the
+// activation copies are requested before the quant copies, so waiting until only the 2 NR newest requests are
+// outstanding leaves exactly the quant copies for the half after next in flight.
+template <int ORDER, int MB, int NR, int NW>
+__global__ __launch_bounds__(64 * NW, MB * NR <= 1 && NW <= 8 ? 2 : 1) void k_qgemm_rw(
+    const uint8_t *__restrict__ W, const uint4 *__restrict__ xs, const float *__restrict__ rowscale, void *__restrict__ yg,
+    float *__restrict__ partial, int M, int Mp, int N, int spr, int chunk, int mode) {
+    constexpr int BM = 32 * MB, kThreads = 64 * NW, kRows = 32 * NR * NW;
+    extern __shared__ uint4 smem[];
+    uint4 *a0 = smem, *a1 = a0 + kGroups * BM, *qbase = a1 + kGroups * BM, *hb = qbase + 3 * NW * NR * 128;
+    const int tid = threadIdx.x;
+    Lane<MB, NR, NW> L;
+    L.wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    L.col = lane & 31, L.g = lane >> 5;
+    const int n0 = blockIdx.x * kRows, m0 = blockIdx.y * BM;
+    const int nw0 = n0 + 32 * NR * L.wave;  // first weight row of this wave
+    const int sb0 = blockIdx.z * chunk;
+    const int cnt = spr - sb0 < chunk ? spr - sb0 : chunk;
+    const uint32_t row_bytes = (uint32_t)spr * kBlockBytes;
+    auto row_off = [&](int row) {  // byte offset of a row of this wave from the workgroup's first row; rows past N repeat the last
+        int n = nw0 + row;
+        n = n < N ? n : N - 1;
+        return (uint32_t)(n - n0) * row_bytes;
+    };
+#pragma unroll
+    for (int rg = 0; rg < NR; rg++) {
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+            const int row = 16 * r + (lane >> 2);
+            L.q_off[rg][r] = row_off(32 * rg + row) + 16u * (uint32_t)((lane & 3) ^ ((row >> 2) & 3));
+        }
+        L.h_off[rg] = row_off(32 * rg + (lane & 31));
+    }
+#pragma unroll
+    for (int i = 0; i < Lane<MB, NR, NW>::kARounds; i++) {
+        const int idx = tid + i * kThreads;
+        L.a_off[i] = (uint32_t)((idx / BM) * Mp + idx % BM);
+    }
+    // this wave's three quant stages (rotated: qa is read, qb is next, qc receives the copies) and its headers
+    uint4 *qa = qbase + L.wave * (NR * 128), *qb = qa + NW * NR * 128, *qc = qb + NW * NR * 128;
+    uint4 *hw = hb + L.wave * (NR * 64);
+    const uint8_t *wblk = W + (size_t)n0 * row_bytes;
+
+    Acc<MB, NR> R;
+#pragma unroll
+    for (int rg = 0; rg < NR; rg++)
+#pragma unroll
+        for (int i = 0; i < MB; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) R.acc[rg][i][r] = 0.0f, R.part[rg][i][r] = 0.0f;
+
+    // prologue: headers, both halves' quant pieces and the first activation stage of super-block sb0
+    {
+        const uint8_t *blk = wblk + (size_t)sb0 * kBlockBytes;
+#pragma unroll
+        for (int rg = 0; rg < NR; rg++) {
+            dma16(blk + L.h_off[rg], hw + rg * 64);
+#pragma unroll
+            for (int r = 0; r < 2; r++) {
+                dma16(blk + 16 + L.q_off[rg][r], qa + rg * 128 + r * 64);
+                dma16(blk + 16 + 64 + L.q_off[rg][r], qb + rg * 128 + r * 64);
+            }
+        }
+        const uint4 *xa = xs + (size_t)(sb0 * 2 * kGroups) * Mp + m0;
+#pragma unroll
+        for (int i = 0; i < Lane<MB, NR, NW>::kARounds; i++)
+            if (i * kThreads + L.wave * 64 < kGroups * BM) dma16(xa + L.a_off[i], a0 + i * kThreads + L.wave * 64);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();
+
+    for (int s = 0; s < cnt; s++) {
+        const int sb = sb0 + s;
+        const int sbn = sb + 1 < spr ? sb + 1 : spr - 1;  // the copies for "the next super-block" stay inside the matrix
+        const uint8_t *blkn = wblk + (size_t)sbn * kBlockBytes;
+        rw_half<ORDER, MB, NR, NW, 0>(a0, a1, qa, qc, hw, xs + (size_t)((sb * 2 + 1) * kGroups) * Mp + m0, blkn + 16, blkn, L, R);
+        barrier_keep<2 * NR>();
+        rw_half<ORDER, MB, NR, NW, 1>(a1, a0, qb, qa, hw, xs + (size_t)(sbn * 2 * kGroups) * Mp + m0, blkn + 16 + 64, nullptr, L, R);
+        barrier_keep<2 * NR>();
+        // two half super-blocks on: (qa, qb, qc) <- (qc, qa, qb)
+        uint4 *t = qc;
+        qc = qb, qb = qa, qa = t;
+    }
+    // C layout of v_mfma_f32_32x32x*: lane holds column (lane & 31), rows 8 (r / 4) + 4 (lane / 32) + r % 4
+#pragma unroll
+    for (int rg = 0; rg < NR; rg++) {
+        const int n = nw0 + 32 * rg + L.col;
+        if (n >= N) continue;
+#pragma unroll
+        for (int i = 0; i < MB; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = m0 + 32 * i + 8 * (r >> 2) + 4 * L.g + (r & 3);
+                if (m >= M) continue;
+                if (mode == 2) {
+                    partial[((size_t)blockIdx.z * Mp + m) * N + n] = R.acc[rg][i][r];
+                } else {
+                    const float v = R.acc[rg][i][r] * rowscale[m];
+                    if (mode == 1) {
+                        uint32_t u = __builtin_bit_cast(uint32_t, v);
+                        u = ((u & 0x7FFFFFFFu) > 0x7F800000u) ? ((u >> 16) | 0x40u) : ((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+                        reinterpret_cast<uint16_t *>(yg)[(size_t)m * N + n] = (uint16_t)u;
+                    } else {
+                        reinterpret_cast<float *>(yg)[(size_t)m * N + n] = v;
+                    }
+                }
+            }
+    }
+}
+
+// y[m][n] = rowscale[m] * (partial[0][m][n] + partial[1][m][n] + ...), added in this order
+template <bool YBF16>
+__global__ __launch_bounds__(256) void k_rw_reduce(const float *__restrict__ partial, int splits, int M, int Mp, int N,
+                                                    const float *__restrict__ rowscale, void *__restrict__ yg) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)M * N) return;
+    const int m = (int)(idx / N);
+    const size_t plane = (size_t)Mp * N;
+    float s = partial[idx];
+    for (int z = 1; z < splits; z++) s += partial[(size_t)z * plane + idx];
+    const float v = s * rowscale[m];
+    if (YBF16) {
+        uint32_t u = __builtin_bit_cast(uint32_t, v);
+        u = ((u & 0x7FFFFFFFu) > 0x7F800000u) ? ((u >> 16) | 0x40u) : ((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+        reinterpret_cast<uint16_t *>(yg)[idx] = (uint16_t)u;
+    } else {
+        reinterpret_cast<float *>(yg)[idx] = v;
+    }
+}
+
+template <int MB, int NR, int NW>
+constexpr size_t rw_lds_bytes() {
+    return (size_t)(2 * kGroups * 32 * MB + NW * NR * (3 * 128 + 64)) * 16;
+}
+
+}  // namespace
+
+namespace pmh {
+
+static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+bool qgemm_rowwave_fits(uint32_t type, int64_t m, int64_t n, int64_t k) {
+    // byte offsets inside a workgroup's rows and item offsets inside the activation copy are 32-bit
+    return type == kTypeQ4K && m >= 1 && m <= (int64_t)1 << 22 && n >= 1 && k >= 256 && k % 256 == 0 && k <= (int64_t)1 << 22 && n <= 0x7FFFFF00;
+}
+
+RowwavePlan qgemm_rowwave_plan(int64_t m, int64_t n, int64_t k) {
+    RowwavePlan p;
+    p.mb = m <= 32 ? 1 : (m <= 64 ? 2 : 4);
+    p.mp = (m + 32 * p.mb - 1) / (32 * p.mb) * (32 * p.mb);
+    p.nw = p.mb == 2 ? 16 : 8;
+    const int64_t spr = k / 256;
+    const int64_t rows = 32 * p.nw;
+    const int64_t base = (n + rows - 1) / rows * (p.mp / (32 * p.mb));
+    // K split: more workgroups fill more of the machine, but every split writes and re-reads an fp32 tile of Y.
+    // Estimated time = (time on a full machine) / (fraction of workgroup slots in use) + partial-tile traffic;
+    // rates as measured on MI355X (about 700 TFLOP/s of this kernel, 4 TB/s for the weight stream and for the
+    // partial tiles, 3 us for the extra launch).
+    const double slots = p.mb == 1 ? 512.0 : 256.0;  // workgroups resident at once
+    const double flops = 2.0 * (double)p.mp * (double)n * (double)k, wbytes = (double)n * (double)k * 0.5625;
+    const double t_full = flops / 7.0e14 > wbytes / 4.0e12 ? flops / 7.0e14 : wbytes / 4.0e12;
+    double best = 0.0;
+    p.splits = 1, p.chunk = (int)spr;
+    for (int64_t want = 1; want <= spr; want *= 2) {
+        const int64_t chunk = (spr + want - 1) / want, splits = (spr + chunk - 1) / chunk;
+        const double groups = (double)(base * splits);
+        const double rounds = (double)(int64_t)((groups + slots - 1) / slots);
+        const double t = t_full * rounds * slots / groups +
+                         (splits > 1 ? (double)splits * (double)m * (double)n * 8.0 / 4.0e12 + 3.0e-6 : 0.0);
+        if (want == 1 || t < best) best = t, p.splits = (int)splits, p.chunk = (int)chunk;
+    }
+    return p;
+}
+
+size_t qgemm_rowwave_workspace_bytes(int64_t m, int64_t n, int64_t k) {
+    const RowwavePlan p = qgemm_rowwave_plan(m, n, k);
+    const size_t xs = align256((size_t)(k / 256) * 2 * kGroups * p.mp * 16);
+    const size_t part = p.splits > 1 ? align256((size_t)p.splits * p.mp * n * 4) : 0;
+    return xs + align256((size_t)p.mp * 4) + part;
+}
+
+template <int ORDER, int MB, int NR, int NW>
+static hipError_t launch_rw(hipStream_t s, const uint8_t *w, const uint4 *xs, const float *rowscale, void *y, float *partial,
+                            int64_t m, int64_t n, int spr, const RowwavePlan &p, int mode) {
+    auto kern = k_qgemm_rw<ORDER, MB, NR, NW>;
+    constexpr size_t lds = rw_lds_bytes<MB, NR, NW>();
+    constexpr int kRows = 32 * NR * NW;
+    if (lds > 64 * 1024) {
+        hipError_t a = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (a != hipSuccess) return a;
+    }
+    const dim3 grid((unsigned)((n + kRows - 1) / kRows), (unsigned)(p.mp / (32 * MB)), (unsigned)p.splits);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * NW), lds, s, w, xs, rowscale, y, partial, (int)m, (int)p.mp, (int)n, spr, p.chunk, mode);
+    return hipGetLastError();
+}
+
+hipError_t launch_qgemm_rowwave(const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, int64_t m, void *y,
+                                uint32_t y_dtype, uint32_t order, void *workspace, hipStream_t s) {
+    if (!qgemm_rowwave_fits(kTypeQ4K, m, n, k)) return hipErrorInvalidValue;
+    const RowwavePlan p = qgemm_rowwave_plan(m, n, k);
+    const int spr = (int)(k / 256);
+    uint8_t *ws = reinterpret_cast<uint8_t *>(workspace);
+    uint4 *xs = reinterpret_cast<uint4 *>(ws);
+    const size_t xs_bytes = align256((size_t)spr * 2 * kGroups * p.mp * 16);
+    float *rowscale = reinterpret_cast<float *>(ws + xs_bytes);
+    float *partial = reinterpret_cast<float *>(ws + xs_bytes + align256((size_t)p.mp * 4));
+    const bool xf32 = x_dtype == kDtypeF32, ref = order == kOrderRef;
+    if (xf32 && ref) hipLaunchKernelGGL((k_prep_rw<true, 0>), dim3((unsigned)p.mp), dim3(256), 0, s, x, k, (int)m, (int)p.mp, rowscale, xs);
+    else if (xf32) hipLaunchKernelGGL((k_prep_rw<true, 1>), dim3((unsigned)p.mp), dim3(256), 0, s, x, k, (int)m, (int)p.mp, rowscale, xs);
+    else if (ref) hipLaunchKernelGGL((k_prep_rw<false, 0>), dim3((unsigned)p.mp), dim3(256), 0, s, x, k, (int)m, (int)p.mp, rowscale, xs);
+    else hipLaunchKernelGGL((k_prep_rw<false, 1>), dim3((unsigned)p.mp), dim3(256), 0, s, x, k, (int)m, (int)p.mp, rowscale, xs);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const bool ybf = y_dtype == kDtypeBf16;
+    const int mode = p.splits > 1 ? 2 : (ybf ? 1 : 0);
+#define PMH_RW_CASE(O, B, R, NWV) launch_rw<O, B, R, NWV>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
+    if (p.mb == 1) {
+        e = ref ? PMH_RW_CASE(0, 1, 1, 8) : PMH_RW_CASE(1, 1, 1, 8);
+    } else if (p.mb == 2) {
+        e = ref ? PMH_RW_CASE(0, 2, 1, 16) : PMH_RW_CASE(1, 2, 1, 16);
+    } else {
+        e = ref ? PMH_RW_CASE(0, 4, 1, 8) : PMH_RW_CASE(1, 4, 1, 8);
+    }
+#undef PMH_RW_CASE
+    if (e != hipSuccess || p.splits == 1) return e;
+    const size_t total = (size_t)m * n;
+    const dim3 rgrid((unsigned)((total + 255) / 256));
+    if (ybf) hipLaunchKernelGGL(k_rw_reduce<true>, rgrid, dim3(256), 0, s, partial, p.splits, (int)m, (int)p.mp, (int)n, rowscale, y);
+    else hipLaunchKernelGGL(k_rw_reduce<false>, rgrid, dim3(256), 0, s, partial, p.splits, (int)m, (int)p.mp, (int)n, rowscale, y);
+    return hipGetLastError();
+}
+
+}  // namespace pmh

@@ -40,6 +40,20 @@ size_t qgemm_workspace_bytes(int64_t m, int64_t k);
 hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype,
                         int64_t m, void *y, uint32_t y_dtype, uint32_t order, void *workspace, hipStream_t s);
 
+// ---- gemm_rowwave.hip: Q4_K GEMM for short activation batches (every wave owns 32 weight rows) ----
+struct RowwavePlan {
+    int mb;      // 32-row activation blocks per workgroup (1, 2 or 4)
+    int nw;      // waves per workgroup (8 or 16)
+    int mp;      // activation rows padded to a multiple of 32 mb
+    int splits;  // workgroups along K (more than one: partial tiles plus a reduction kernel)
+    int chunk;   // super-blocks per split
+};
+bool qgemm_rowwave_fits(uint32_t type, int64_t m, int64_t n, int64_t k);
+RowwavePlan qgemm_rowwave_plan(int64_t m, int64_t n, int64_t k);
+size_t qgemm_rowwave_workspace_bytes(int64_t m, int64_t n, int64_t k);
+hipError_t launch_qgemm_rowwave(const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, int64_t m, void *y,
+                                uint32_t y_dtype, uint32_t order, void *workspace, hipStream_t s);
+
 // ---- util.hip ----
 hipError_t launch_fill_normal(float *dst, size_t n, uint64_t seed, float std, float outlier_rate,
                               float outlier_mag, hipStream_t s);

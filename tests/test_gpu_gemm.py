@@ -126,6 +126,22 @@ def test_qgemm_agrees_with_qgemv_and_qlinear_dispatch(oracle):
     assert np.allclose(y4[2], y_gemv, rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("m,n,k", [(2, 96, 512), (5, 1000, 1024), (40, 260, 2048), (96, 700, 1024), (384, 1024, 1024)])
+def test_qgemm_q4k_k_split_is_deterministic_and_ragged_rows(oracle, m, n, k):
+    """Short batches split K over several workgroups and add fp32 partial tiles in a fixed order: two runs give the
+    same bits; n is not a multiple of the 32 rows a wave owns."""
+    wq = oracle.quantize(Q4K, weights(300 + m, n * k))
+    x = np.random.default_rng(301 + m).standard_normal((m, k)).astype(np.float32)
+    bits = oracle.f32_to_bf16_bits(x.reshape(-1)).reshape(m, k)
+    xr = oracle.bf16_bits_to_f32(bits.reshape(-1)).reshape(m, k)
+    want = reference(oracle, Q4K, wq, n, k, xr, 1)
+    got = gpu_qgemm(Q4K, wq, n, k, bits, m, order=1)
+    again = gpu_qgemm(Q4K, wq, n, k, bits, m, order=1)
+    assert np.array_equal(got, again)
+    elem, norm = rel_errors(got.reshape(-1), want.reshape(-1))
+    assert elem <= TOL and norm <= TOL
+
+
 def test_qgemm_argument_errors():
     lib = _lib.load()
     buf = pm.DeviceBuffer(1 << 16)
