@@ -1,4 +1,7 @@
-// Dequant-fused Q4_K GEMM  Y[m,n] = sum_k X[m,k] * W[n,k]  (prefill) on the gfx950 matrix cores.
+// Dequant-fused GEMM  Y[m,n] = sum_k X[m,k] * W[n,k]  (prefill) on the gfx950 matrix cores, large-tile design:
+// one dequantized weight tile per workgroup, shared through LDS.  It serves Q6_K, and Q4_K shapes outside the
+// limits of the kernel in gemm_rowwave.hip (where every wave owns its weight rows), which is the faster one.
+// The text below describes Q4_K; the Q6_K differences are noted at dequant16_q6.
 //
 // W is the packed GGUF stream [n, k] of 144-byte super-blocks; a weight's value is what the reference's
 // dequantize_q4k yields (crates/pmetal-gguf/src/k_quants.rs:358-404; element order REF or GGML as for the
