@@ -32,8 +32,8 @@
 //
 // What bounds it: every matrix instruction reads its 1 KiB activation fragment from LDS (a wave cannot reuse a
 // fragment for a second group of weight rows without doubling the dequantization work per matrix instruction,
-// which measured slower), so a 128-row workgroup is bound by the LDS read rate at about 60 % of the matrix
-// peak.
+// which measured slower, as did one wave per SIMD with a 128 x 64 tile), so a 128-row workgroup is bound by the
+// LDS read rate at about 60 % of the matrix peak.
 #include "internal.hpp"
 
 namespace {
@@ -522,9 +522,9 @@ bool qgemm_rowwave_fits(uint32_t type, int64_t m, int64_t n, int64_t k) {
 
 RowwavePlan qgemm_rowwave_plan(int64_t m, int64_t n, int64_t k) {
     RowwavePlan p;
-    p.mb = m <= 32 ? 1 : (m <= 64 ? 2 : 4);
+    p.mb = m <= 64 ? 1 : 4;  // 32 activation rows per workgroup (more workgroups along M) or 128
     p.mp = (m + 32 * p.mb - 1) / (32 * p.mb) * (32 * p.mb);
-    p.nw = p.mb == 2 ? 16 : 8;
+    p.nw = 8;
     const int64_t spr = k / 256;
     const int64_t rows = 32 * p.nw;
     const int64_t base = (n + rows - 1) / rows * (p.mp / (32 * p.mb));
@@ -532,7 +532,7 @@ RowwavePlan qgemm_rowwave_plan(int64_t m, int64_t n, int64_t k) {
     // Estimated time = (time on a full machine) / (fraction of workgroup slots in use) + partial-tile traffic;
     // rates as measured on MI355X (about 700 TFLOP/s of this kernel, 4 TB/s for the weight stream and for the
     // partial tiles, 3 us for the extra launch).
-    const double slots = p.mb == 1 ? 512.0 : 256.0;  // workgroups resident at once
+    const double slots = 256.0;  // one workgroup per compute unit keeps the weight stream busy
     const double flops = 2.0 * (double)p.mp * (double)n * (double)k, wbytes = (double)n * (double)k * 0.5625;
     const double t_full = flops / 7.0e14 > wbytes / 4.0e12 ? flops / 7.0e14 : wbytes / 4.0e12;
     double best = 0.0;
@@ -592,8 +592,6 @@ hipError_t launch_qgemm_rowwave(const uint8_t *w, int64_t n, int64_t k, const vo
 #define PMH_RW_CASE(O, B, R, NWV) launch_rw<O, B, R, NWV>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
     if (p.mb == 1) {
         e = ref ? PMH_RW_CASE(0, 1, 1, 8) : PMH_RW_CASE(1, 1, 1, 8);
-    } else if (p.mb == 2) {
-        e = ref ? PMH_RW_CASE(0, 2, 1, 16) : PMH_RW_CASE(1, 2, 1, 16);
     } else {
         e = ref ? PMH_RW_CASE(0, 4, 1, 8) : PMH_RW_CASE(1, 4, 1, 8);
     }
