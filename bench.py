@@ -47,21 +47,22 @@ class Timer:
     def __init__(self, pm, lib):
         self.pm, self.lib = pm, lib
         self.e0, self.e1 = lib.pmetal_hip_event_create(), lib.pmetal_hip_event_create()
+        self.stream = None  # the stream fn() launches on: the events are recorded there
 
     def run(self, fn, steps, warmup):
         """W untimed + exactly K timed calls of fn(); returns (event_ms, wall_ms)."""
-        pm, lib = self.pm, self.lib
+        pm, lib, st = self.pm, self.lib, self.stream
         for _ in range(warmup):
             fn()
-        pm.check(lib.pmetal_hip_sync(None))
+        pm.check(lib.pmetal_hip_sync(st))
         t0 = time.perf_counter()
-        pm.check(lib.pmetal_hip_event_record(self.e0, None))
+        pm.check(lib.pmetal_hip_event_record(self.e0, st))
         for _ in range(steps):
             fn()
-        pm.check(lib.pmetal_hip_event_record(self.e1, None))
+        pm.check(lib.pmetal_hip_event_record(self.e1, st))
         ms = C.c_float()
         pm.check(lib.pmetal_hip_event_elapsed_ms(self.e0, self.e1, C.byref(ms)))
-        pm.check(lib.pmetal_hip_sync(None))
+        pm.check(lib.pmetal_hip_sync(st))
         return float(ms.value), (time.perf_counter() - t0) * 1e3
 
 
@@ -208,7 +209,18 @@ def bench_decode(args):
     def step():
         pm.check(lib.pmetal_hip_qgemv_batch(descs, len(lins), None))
 
-    ev_ms, wall_ms = timer.run(step, args.steps, args.warmup)
+    eager_ms, _ = timer.run(step, args.steps, args.warmup)
+    # the same launches recorded once and replayed with one submission per token (a HIP graph)
+    stream = lib.pmetal_hip_stream_create()
+    pm.check(lib.pmetal_hip_record_begin(stream))
+    pm.check(lib.pmetal_hip_qgemv_batch(descs, len(lins), stream))
+    rec = lib.pmetal_hip_record_end(stream)
+    if not rec:
+        raise RuntimeError(lib.pmetal_hip_last_error_message())
+    timer.stream = stream
+    ev_ms, wall_ms = timer.run(lambda: pm.check(lib.pmetal_hip_replay(rec, stream)), args.steps, args.warmup)
+    timer.stream = None
+    pm.check(lib.pmetal_hip_recording_destroy(rec))
     tok_s = args.steps / (ev_ms * 1e-3)
     gbs = total_bytes * tok_s / 1e9
     return {
@@ -216,7 +228,8 @@ def bench_decode(args):
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "k_qgemv_q4k / k_qgemv_q6k (197 projections in 127 launches)",
                      "bytes_per_step": total_bytes},
-        "extra": {"launches_per_token": len(lins), "q6k_tensors": sum(1 for l in lins if l[3] == Q6K)},
+        "extra": {"launches_per_token": len(lins), "q6k_tensors": sum(1 for l in lins if l[3] == Q6K),
+                  "submission": "one recorded sequence per token", "eager_tokens_per_s": round(args.steps / (eager_ms * 1e-3), 1)},
     }, (Q4K, 0, 0)
 
 

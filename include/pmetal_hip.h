@@ -91,6 +91,22 @@ int32_t pmetal_hip_d2h(void *dst_host, const void *src_dev, size_t bytes);
 int32_t pmetal_hip_memset(void *dst_dev, int value, size_t bytes, void *stream);
 int32_t pmetal_hip_sync(void *stream);
 
+/* ---- streams and recorded launch sequences ---------------------------------------------
+ * No counterpart in the reference's FFI: there MLX evaluates its lazily built graph and owns the
+ * scheduling.  A decode step is some 130 small launches, and issuing them one by one from the host
+ * costs more than running them; a recording replays the whole sequence with one submission (a HIP
+ * graph).  Between record_begin and record_end every kernel launch issued on `stream` through this
+ * library is recorded instead of run.  Record only launch-type calls (qgemv, qgemv_batch,
+ * quantize_dev, dequantize_dev, f32_to_bf16_dev, and qgemm / qlinear once a call of the same or a
+ * larger shape has run, so that their scratch buffer exists); pmetal_hip_memset refuses to be
+ * recorded.  A recording holds the pointers it was recorded with.                            */
+void *pmetal_hip_stream_create(void); /* NULL on failure (error slot set) */
+int32_t pmetal_hip_stream_destroy(void *stream);
+int32_t pmetal_hip_record_begin(void *stream); /* `stream` must come from pmetal_hip_stream_create */
+void *pmetal_hip_record_end(void *stream);     /* the recording, NULL on failure */
+int32_t pmetal_hip_replay(void *recording, void *stream);
+int32_t pmetal_hip_recording_destroy(void *recording);
+
 /* ---- events (timing on the stream the kernels run on) -------------------------------- */
 void *pmetal_hip_event_create(void);
 int32_t pmetal_hip_event_record(void *event, void *stream);

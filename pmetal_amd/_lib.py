@@ -35,6 +35,12 @@ SYMBOLS = [
     ("pmetal_hip_d2h", _i32, [_vp, _vp, _sz]),
     ("pmetal_hip_memset", _i32, [_vp, C.c_int, _sz, _vp]),
     ("pmetal_hip_sync", _i32, [_vp]),
+    ("pmetal_hip_stream_create", _vp, []),
+    ("pmetal_hip_stream_destroy", _i32, [_vp]),
+    ("pmetal_hip_record_begin", _i32, [_vp]),
+    ("pmetal_hip_record_end", _vp, [_vp]),
+    ("pmetal_hip_replay", _i32, [_vp, _vp]),
+    ("pmetal_hip_recording_destroy", _i32, [_vp]),
     ("pmetal_hip_event_create", _vp, []),
     ("pmetal_hip_event_record", _i32, [_vp, _vp]),
     ("pmetal_hip_event_elapsed_ms", _i32, [_vp, _vp, C.POINTER(_f32)]),

@@ -217,6 +217,12 @@ int32_t pmetal_hip_d2h(void *dst, const void *src, size_t bytes) {
 
 int32_t pmetal_hip_memset(void *dst, int value, size_t bytes, void *stream) {
     if (bytes && !dst) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
+    if (stream) {  // a memset node in a recording has replayed wrongly on this hardware: keep it out
+        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+        HIP_TRY(hipStreamIsCapturing((hipStream_t)stream, &st));
+        if (st != hipStreamCaptureStatusNone)
+            return fail(PMETAL_HIP_ERR_INVALID_ARG, "pmetal_hip_memset cannot be recorded");
+    }
     if (bytes) HIP_TRY(hipMemsetAsync(dst, value, bytes, (hipStream_t)stream));
     return ok();
 }
@@ -224,6 +230,66 @@ int32_t pmetal_hip_memset(void *dst, int value, size_t bytes, void *stream) {
 int32_t pmetal_hip_sync(void *stream) {
     if (int32_t rc = require_device()) return rc;
     HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    return ok();
+}
+
+// ---- streams and recordings ----
+void *pmetal_hip_stream_create(void) {
+    if (require_device()) return nullptr;
+    hipStream_t st = nullptr;
+    hipError_t e = hipStreamCreateWithFlags(&st, hipStreamNonBlocking);  // default priority
+    if (e != hipSuccess) {
+        hip_fail(e, "hipStreamCreateWithFlags");
+        return nullptr;
+    }
+    ok();
+    return st;
+}
+
+int32_t pmetal_hip_stream_destroy(void *stream) {
+    if (!stream) return ok();
+    HIP_TRY(hipStreamDestroy((hipStream_t)stream));
+    return ok();
+}
+
+int32_t pmetal_hip_record_begin(void *stream) {
+    if (!stream) return fail(PMETAL_HIP_ERR_INVALID_ARG, "recording needs a stream from pmetal_hip_stream_create");
+    if (int32_t rc = require_device()) return rc;
+    HIP_TRY(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
+    return ok();
+}
+
+void *pmetal_hip_record_end(void *stream) {
+    if (!stream) {
+        fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL stream");
+        return nullptr;
+    }
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture((hipStream_t)stream, &graph);
+    if (e != hipSuccess || !graph) {
+        hip_fail(e != hipSuccess ? e : hipErrorUnknown, "hipStreamEndCapture");
+        return nullptr;
+    }
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) {
+        hip_fail(e, "hipGraphInstantiate");
+        return nullptr;
+    }
+    ok();
+    return exec;
+}
+
+int32_t pmetal_hip_replay(void *recording, void *stream) {
+    if (!recording) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL recording");
+    HIP_TRY(hipGraphLaunch((hipGraphExec_t)recording, (hipStream_t)stream));
+    return ok();
+}
+
+int32_t pmetal_hip_recording_destroy(void *recording) {
+    if (!recording) return ok();
+    HIP_TRY(hipGraphExecDestroy((hipGraphExec_t)recording));
     return ok();
 }
 
