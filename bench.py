@@ -159,7 +159,7 @@ def bench_gemm(args, m, n, k, t=Q4K):
         "value": tflops, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / BF16_PEAK_TFLOPS, 4), "traffic": None,
-                     "kernel": "k_qgemm_rw (+ k_prep_rw, k_rw_reduce when K is split)" if t == Q4K else "k_qgemm (+ k_prep_scale, k_prep_tiles)",
+                     "kernel": ("k_qgemm_rw" if t == Q4K else "k_qgemm_rw_q6") + " (+ k_prep_rw, k_rw_reduce when K is split)",
                      "flops_per_launch": flops, "us_per_launch": round(us, 3)},
         "extra": {},
     }, (t, n, k)

@@ -30,7 +30,6 @@ EXTRA = {
     "gemv.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
     "gemv_q4k.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
     "gemm.hip": [],
-    "gemm_rowwave.hip": [],
     "util.hip": [],
     "api.hip": [],
 }

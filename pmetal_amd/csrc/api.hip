@@ -479,13 +479,11 @@ int32_t pmetal_hip_qgemm(uint32_t t, const uint8_t *w, int64_t n, int64_t k, con
     if (y_dtype > PMETAL_HIP_DTYPE_BF16) return fail(PMETAL_HIP_ERR_INVALID_ARG, "y_dtype must be 0 (f32) or 1 (bf16)");
     if (m <= 0 || m > 0x7FFFFFFF) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "m must be in [1, 2^31)");
     if (t == PMETAL_GGML_TYPE_Q8_0) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "qgemm supports Q4_K and Q6_K weights");
-    // short activation batches of Q4_K go to the kernel in which every wave owns its weight rows
-    const bool rowwave = pmh::qgemm_rowwave_fits(t, m, n, k);
+    if (!pmh::qgemm_fits(t, m, n, k))
+        return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qgemm: m and k must be at most 2^22 (m = %lld, k = %lld)", (long long)m, (long long)k);
     void *ws = nullptr;
-    if (int32_t rc = workspace(rowwave ? pmh::qgemm_rowwave_workspace_bytes(m, n, k) : pmh::qgemm_workspace_bytes(m, k), &ws))
-        return rc;
-    hipError_t e = rowwave ? pmh::launch_qgemm_rowwave(w, n, k, x, x_dtype, m, y, y_dtype, order, ws, (hipStream_t)stream)
-                           : pmh::launch_qgemm(t, w, n, k, x, x_dtype, m, y, y_dtype, order, ws, (hipStream_t)stream);
+    if (int32_t rc = workspace(pmh::qgemm_workspace_bytes(m, n, k), &ws)) return rc;
+    hipError_t e = pmh::launch_qgemm(t, w, n, k, x, x_dtype, m, y, y_dtype, order, ws, (hipStream_t)stream);
     if (e == hipErrorNotSupported) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "qgemm: configuration not supported");
     if (e != hipSuccess) return hip_fail(e, "qgemm kernel launch");
     return ok();

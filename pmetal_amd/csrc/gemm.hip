@@ -1,36 +1,40 @@
-// Dequant-fused GEMM  Y[m,n] = sum_k X[m,k] * W[n,k]  (prefill) on the gfx950 matrix cores, large-tile design:
-// one dequantized weight tile per workgroup, shared through LDS.  It serves Q6_K, and Q4_K shapes outside the
-// limits of the kernel in gemm_rowwave.hip (where every wave owns its weight rows), which is the faster one.
-// The text below describes Q4_K; the Q6_K differences are noted at dequant16_q6.
+// Dequant-fused Q4_K and Q6_K GEMM  Y[m,n] = sum_k X[m,k] * W[n,k]  on the gfx950 matrix cores, every wave owning
+// its weight rows.  The text below describes Q4_K; the Q6_K kernel further down notes its differences.
 //
 // W is the packed GGUF stream [n, k] of 144-byte super-blocks; a weight's value is what the reference's
 // dequantize_q4k yields (crates/pmetal-gguf/src/k_quants.rs:358-404; element order REF or GGML as for the
 // GEMV).  The reference has no fused kernel (it dequantizes on the CPU at load,
-// crates/pmetal-models/src/weight_format.rs:299-303, and multiplies densely); this kernel is checked
-// against exactly that, dequantize-then-matmul, to 1e-3.
+// crates/pmetal-models/src/weight_format.rs:299-303, and multiplies densely); this kernel is checked against
+// exactly that, dequantize-then-matmul, to 1e-3.
 //
-// Why the tiles are exact integers in f16 and not rounded bf16 weights: rounding d*sc*q - dmin*m to bf16
-// (8 significant bits) leaves a relative error of about 1e-3 per product, which fails the 1e-3 gate.
-// Instead the MFMA multiplies quantities that are exact in f16:
-//     B tile  = sc * q             an integer <= 63 * 15 = 945          (f16 holds integers to 2048)
-//     A tile  = x * 2^-e_m         bf16 activations are exact in f16 once a per-row power of two keeps
-//                                  them below 2^10 (a pre-pass does that and sums x per 32-element block)
-// and the per-super-block factor d is applied to the fp32 partial sums:
-//     Y[m,n] = 2^e_m * sum_SB ( d[n,SB] * P_SB[m,n] + R_SB[m,n] )
-//     P_SB = sum_{k in SB} A[m,k] * B[n,k]              16 x v_mfma_f32_32x32x16_f16 per 32x32 block
-//     R_SB = - sum_{j<8} (dmin[n,SB] * m[n,j]) * xsum[m,j]
-// R_SB also runs on the matrix core, straight into the accumulators: dmin * m (17 significant bits) and the
-// block sums xsum are each split exactly into an f16 head and tail, and the four cross products of the
-// eight sub-blocks make one K = 32 product (two more MFMAs per block and super-block).  The only roundings
-// are the fp32 accumulations.
+// A wave owns 32 weight rows and dequantizes them straight into MFMA operand registers (no shared weight tile
+// in LDS, no LDS writes by the waves at all); only the activations are shared by the waves of a workgroup.  A
+// launch is cut along N, M and, for short activation batches, K into enough workgroups to fill the machine.
+// The arithmetic is exact up to the fp32 accumulation: rounding d*sc*q - dmin*m to f16 or bf16 leaves a relative
+// error per product that fails the element-wise 1e-3 gate on small outputs, so the MFMA multiplies integer tiles
+// sc * q in f16 (<= 63 * 15 = 945; f16 holds integers to 2048) with activations scaled per row by a power of two
+// into the f16 range (bf16 activations are exact there), the per-super-block factor d is applied to the fp32
+// partial sums, and the min term is a K = 32 MFMA product of exact head + tail splits.
 //
-// Tiling: a workgroup of 8, 4 or 2 waves computes a 256 x 128, 128 x 128 or 64 x 32 tile of Y (by the number
-// of activation rows); every wave owns 2 x 2 (or one) MFMA blocks.  K advances 64 elements per stage.  The pre-pass
-// stores the activations as 16-byte items (8 consecutive k of one row) in [k / 8][m] order, so that a wave
-// copies 64 consecutive items from global memory to LDS: coalesced reads, conflict-free writes, and the
-// items lie in LDS exactly as the MFMA A operand wants them ([k-step][k-group][row]).  The B tile is
-// dequantized by the whole workgroup once per stage into the same operand order.  Global loads run two
-// stages ahead in registers, the LDS stages are double buffered, one barrier per stage.
+// Data movement uses direct global -> LDS loads only (no staging registers, no ds_write):
+//   * activations: a pre-pass writes 16-byte items (8 f16) in the order the MFMA wants them,
+//     xs[(2 sb + h) * 18 + grp][Mp], per half super-block h 16 operand groups (k-step t, lane half g) and two
+//     groups of sub-block sums; a workgroup copies the 18 x BM items of a half super-block into one of two
+//     LDS stages while it computes on the other (one barrier per half super-block);
+//   * weights: each wave copies the 64 quant bytes per row of a half super-block (coalesced: four lanes per
+//     row) two half super-blocks ahead, and the 16-byte headers one super-block ahead, into its private LDS
+//     region; then every lane (row n = lane % 32, half g = lane / 32) reads back the 32 bytes it multiplies:
+//     dword t of them holds the eight 4-bit quants of MFMA k-step t.  Which k they are is a property of the
+//     element order, matched by the pre-pass:
+//         GGML: k = 64 (2h + g) + 4t + e (low nibbles, sub-block 4h+2g), + 32 (high nibbles, sub-block 4h+2g+1)
+//         REF : k = 32 (4h + 2g + t/4) + 4 (t%4) + e (low), + 16 (high), both sub-block 4h + 2g + t/4
+// With a K split (grid.z > 1) the workgroups write fp32 partial tiles and a small kernel adds them in a fixed
+// order, so the result does not depend on scheduling.
+//
+// What bounds it: every matrix instruction reads its 1 KiB activation fragment from LDS (a wave cannot reuse a
+// fragment for a second group of weight rows without doubling the dequantization work per matrix instruction,
+// which measured slower, as did one wave per SIMD with a 128 x 64 tile), so a 128-row workgroup is bound by the
+// LDS read rate at about 60 % of the matrix peak.
 #include "internal.hpp"
 
 namespace {
@@ -38,38 +42,59 @@ namespace {
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // 16 bytes in registers
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kMPad = 256; // the pre-pass pads the activation rows to a multiple of this
+constexpr int kGroups = 18;    // 16-byte items per activation row and half super-block
+constexpr int kBlockBytes = 144;
+
+#define PMH_GPTR(p) ((const __attribute__((address_space(1))) void *)(p))
+#define PMH_LPTR(p) ((__attribute__((address_space(3))) void *)(p))
+
+// 16 bytes per lane from global memory to LDS: lane l lands at dst + 16 l (dst is wave-uniform).
+__device__ __forceinline__ void dma16(const void *src, uint4 *dst) {
+    __builtin_amdgcn_global_load_lds(PMH_GPTR(src), PMH_LPTR(dst), 16, 0, 0);
+}
+
+// Workgroup barrier that leaves the newest `keep` vector-memory requests in flight.  (__syncthreads() carries a
+// release fence, which waits for every direct-to-LDS copy.)  The copies that the other waves will read are older
+// than those, and this wave's own LDS reads have returned (lgkmcnt(0)) before another wave may refill a stage.
+template <int KEEP>
+__device__ __forceinline__ void barrier_keep() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0x0070 | KEEP);  // vmcnt(KEEP) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
 
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
     return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
 }
-
 __device__ __forceinline__ float bf16_to_f32(uint32_t h) { return __builtin_bit_cast(float, h << 16); }
 
 // ------------------------------------------------------------------------------------------------
-// Pre-pass 1: one wave per row m (rows up to Mp, a multiple of 4): rowscale[m] = 2^e_m with the row maximum * 2^-e_m in [2^9, 2^10),
-// so that block sums (< 2^15) fit f16 and small rows stay out of the f16 subnormal range.
+// Pre-pass: one workgroup per activation row m < Mp.  rowscale[m] = 2^e with the row maximum * 2^-e in
+// [2^9, 2^10) (bf16 activations are then exact in f16 and block sums stay below 2^15); rows >= M are zero.
+// One thread per operand item: chunk u = 64 elements = sub-blocks 2u, 2u+1 (u = 4 sb + 2 h + g), k-step t.
+// ORDER 0 / 1: Q4_K element orders REF / GGML; ORDER 2: the Q6_K layout (no block sums).
 // ------------------------------------------------------------------------------------------------
-template <bool XF32>
-__global__ __launch_bounds__(256) void k_prep_scale(const void *__restrict__ xg, int64_t k, int M,
-                                                     float *__restrict__ rowscale) {
-    // one wave per row, 16-byte loads (k is a multiple of 256)
-    const int64_t m = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int lane = threadIdx.x & 63;
+template <bool XF32, int ORDER>
+__global__ __launch_bounds__(256) void k_prep_rw(const void *__restrict__ xg, int64_t k, int M, int Mp,
+                                                  float *__restrict__ rowscale, uint4 *__restrict__ xs) {
+    const int m = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
+    const bool live = m < M;
+    __shared__ float red[4];
     float amax = 0.0f;
-    if (m < M) {
+    if (live) {
         if (XF32) {
-            const float4 *row = reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(xg) + m * k);
-            for (int64_t i = lane; i < k / 4; i += 64) {
+            const float4 *row = reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(xg) + (int64_t)m * k);
+            for (int64_t i = tid; i < k / 4; i += 256) {
                 const float4 v = row[i];
                 amax = __builtin_fmaxf(__builtin_fmaxf(amax, __builtin_fmaxf(__builtin_fabsf(v.x), __builtin_fabsf(v.y))),
                                        __builtin_fmaxf(__builtin_fabsf(v.z), __builtin_fabsf(v.w)));
             }
         } else {
-            const uint4 *row = reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(xg) + m * k);
-            for (int64_t i = lane; i < k / 8; i += 64) {
+            const uint4 *row = reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(xg) + (int64_t)m * k);
+            for (int64_t i = tid; i < k / 8; i += 256) {
                 const uint4 v = row[i];
                 const uint32_t r[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
@@ -80,66 +105,77 @@ __global__ __launch_bounds__(256) void k_prep_scale(const void *__restrict__ xg,
         }
     }
     for (int off = 32; off > 0; off >>= 1) amax = __builtin_fmaxf(amax, __shfl_xor(amax, off));
+    if (lane == 0) red[tid >> 6] = amax;
+    __syncthreads();
+    amax = __builtin_fmaxf(__builtin_fmaxf(red[0], red[1]), __builtin_fmaxf(red[2], red[3]));
     const int eb = (int)((__builtin_bit_cast(uint32_t, amax) >> 23) & 0xFFu);  // amax in [2^(eb-127), 2^(eb-126))
     int e = eb - 126 - 10;
     e = e < -126 ? -126 : (e > 126 ? 126 : e);
     if (eb == 255) e = 0;  // inf / NaN: let them through
-    if (lane == 0) rowscale[m] = __builtin_bit_cast(float, (uint32_t)(127 + e) << 23);
-}
+    const float up = __builtin_bit_cast(float, (uint32_t)(127 + e) << 23);
+    if (tid == 0) rowscale[m] = up;
+    const float down = live ? 1.0f / up : 0.0f;  // exact: a power of two
 
-// ------------------------------------------------------------------------------------------------
-// Pre-pass 2: grid (Mp / 32, k / 256), 256 threads.  Thread (row = tid / 8, c8 = tid % 8) converts the 8
-// activations of chunk c8 of every 64-element group of the super-block: 8 lanes read 128 contiguous bytes
-// of a row, and for one chunk the 8 rows of a wave write 128 contiguous bytes.
-//   xs   [k / 8][Mp]               items of 8 f16: x[m][8c .. 8c+7] * 2^-e_m   (rows >= M are zero)
-//   xsum [k / 256][2][2][Mp]       items of 8 f16 for the R_SB product, item (t, g) of row m =
-//                                  (h_j, l_j, h_j, l_j, h_j+1, l_j+1, h_j+1, l_j+1),  j = 4 t + 2 g,
-//                                  h + l = sum of the 32 scaled activations of sub-block j (exact split)
-// ------------------------------------------------------------------------------------------------
-template <bool XF32>
-__global__ __launch_bounds__(256) void k_prep_tiles(const void *__restrict__ xg, int64_t k, int M, int Mp,
-                                                     const float *__restrict__ rowscale, uint4 *__restrict__ xs,
-                                                     uint4 *__restrict__ xsum) {
-    const int c8 = threadIdx.x & 7;
-    const int m = blockIdx.x * 32 + (threadIdx.x >> 3);
-    const int64_t sb = blockIdx.y;
-    const bool live = m < M;
-    const float down = live ? 1.0f / rowscale[m] : 0.0f;  // exact: a power of two
-#pragma unroll
-    for (int it = 0; it < 4; it++) {  // 64 elements per trip: sub-blocks 2 it (c8 < 4) and 2 it + 1
-        const int64_t k0 = sb * 256 + it * 64 + c8 * 8;
+    for (int64_t q = tid; q < k / 8; q += 256) {
+        // the item's two runs of four elements (lo, hi), its half super-block and its operand group
+        int64_t lo, hi, half;
+        int t, g;
+        if (ORDER == 2) {  // Q6_K: half = 128 elements; low nibbles at 32 g + 4 t, high nibbles 64 further
+            half = q >> 4;
+            t = (int)(q & 15) >> 1, g = (int)q & 1;
+            lo = 128 * half + 32 * g + 4 * t;
+            hi = lo + 64;
+        } else {
+            const int64_t u = q >> 3;
+            t = (int)(q & 7), g = (int)u & 1;
+            half = u >> 1;
+            lo = ORDER == 0 ? 64 * u + 32 * (t >> 2) + 4 * (t & 3) : 64 * u + 4 * t;
+            hi = lo + (ORDER == 0 ? 16 : 32);
+        }
         float v[8];
         if (!live) {
 #pragma unroll
             for (int i = 0; i < 8; i++) v[i] = 0.0f;
         } else if (XF32) {
-            const float4 a = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(xg) + (int64_t)m * k + k0);
-            const float4 b = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(xg) + (int64_t)m * k + k0 + 4);
+            const float *row = reinterpret_cast<const float *>(xg) + (int64_t)m * k;
+            const float4 a = *reinterpret_cast<const float4 *>(row + lo), b = *reinterpret_cast<const float4 *>(row + hi);
             v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
         } else {
-            const uint4 u = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(xg) + (int64_t)m * k + k0);
-            const uint32_t r[4] = {u.x, u.y, u.z, u.w};
-#pragma unroll
-            for (int i = 0; i < 4; i++) v[2 * i] = bf16_to_f32(r[i] & 0xFFFFu), v[2 * i + 1] = bf16_to_f32(r[i] >> 16);
+            const uint16_t *row = reinterpret_cast<const uint16_t *>(xg) + (int64_t)m * k;
+            const uint2 a = *reinterpret_cast<const uint2 *>(row + lo), b = *reinterpret_cast<const uint2 *>(row + hi);
+            v[0] = bf16_to_f32(a.x & 0xFFFFu), v[1] = bf16_to_f32(a.x >> 16), v[2] = bf16_to_f32(a.y & 0xFFFFu), v[3] = bf16_to_f32(a.y >> 16);
+            v[4] = bf16_to_f32(b.x & 0xFFFFu), v[5] = bf16_to_f32(b.x >> 16), v[6] = bf16_to_f32(b.y & 0xFFFFu), v[7] = bf16_to_f32(b.y >> 16);
         }
         half8_t h;
-        float sum = 0.0f;
+        float slo = 0.0f, shi = 0.0f;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             h[i] = (_Float16)(v[i] * down);
-            sum += (float)h[i];
+            if (i < 4) slo += (float)h[i];
+            else shi += (float)h[i];
         }
-        xs[(size_t)(k0 / 8) * Mp + m] = __builtin_bit_cast(uint4, h);
-        // sub-block sums: over the 4 lanes of a chunk quad (exact: every partial sum is a multiple of the
-        // row's f16 grid and stays below 2^15 of it), then the pair (2 it, 2 it + 1) meets in lane c8 = 0
-        sum += __shfl_xor(sum, 1);
-        sum += __shfl_xor(sum, 2);
-        const float other = __shfl_down(sum, 4);
-        if (c8 == 0) {
-            const _Float16 h0 = (_Float16)sum, h1 = (_Float16)other;
-            const _Float16 l0 = (_Float16)(sum - (float)h0), l1 = (_Float16)(other - (float)h1);
+        const size_t base = (size_t)(half * kGroups) * Mp + m;
+        xs[base + (size_t)(t * 2 + g) * Mp] = __builtin_bit_cast(uint4, h);
+        if (ORDER == 2) continue;  // Q6_K has no min term: no block sums
+        // sums of the two sub-blocks of the chunk over its 8 k-steps (8 consecutive lanes)
+        float s0, s1;
+        if (ORDER == 0) {  // sub-block 2u: k-steps 0..3 (low and high nibbles), 2u+1: k-steps 4..7
+            float s = slo + shi;
+            s += __shfl_xor(s, 1);
+            s += __shfl_xor(s, 2);
+            s0 = s;
+            s1 = __shfl_down(s, 4);
+        } else {  // sub-block 2u: the low nibbles of all k-steps, 2u+1: the high nibbles
+            slo += __shfl_xor(slo, 1), shi += __shfl_xor(shi, 1);
+            slo += __shfl_xor(slo, 2), shi += __shfl_xor(shi, 2);
+            slo += __shfl_xor(slo, 4), shi += __shfl_xor(shi, 4);
+            s0 = slo, s1 = shi;
+        }
+        if (t == 0) {  // exact head + tail split of each sum; item (H0, L0, H0, L0, H1, L1, H1, L1)
+            const _Float16 h0 = (_Float16)s0, h1 = (_Float16)s1;
+            const _Float16 l0 = (_Float16)(s0 - (float)h0), l1 = (_Float16)(s1 - (float)h1);
             const half8_t item = {h0, l0, h0, l0, h1, l1, h1, l1};
-            xsum[((size_t)sb * 4 + it) * Mp + m] = __builtin_bit_cast(uint4, item);  // j = 2 it = 4 t + 2 g
+            xs[base + (size_t)(16 + g) * Mp] = __builtin_bit_cast(uint4, item);
         }
     }
 }
@@ -147,88 +183,57 @@ __global__ __launch_bounds__(256) void k_prep_tiles(const void *__restrict__ xg,
 // ------------------------------------------------------------------------------------------------
 // main kernel
 // ------------------------------------------------------------------------------------------------
-// 16 nibbles (one plane of a 16-byte piece) times the integer scale -> 16 exact f16 values.
+// per-thread constants of the copy roles; a wave owns NR groups of 32 weight rows
+template <int MB, int NR, int NW>
+struct Lane {
+    static constexpr int BM = 32 * MB, kThreads = 64 * NW;
+    static constexpr int kARounds = (kGroups * BM + kThreads - 1) / kThreads;
+    int wave, col, g;
+    uint32_t q_off[NR][2];     // byte offset of this lane's quant piece of round r from the workgroup's first row
+    uint32_t h_off[NR];        // ... of this lane's header
+    uint32_t a_off[kARounds];  // item offset of this lane's activation item of round i from (group 0, row m0)
+};
+
+template <int MB, int NR>
+struct Acc {
+    float16_t acc[NR][MB], part[NR][MB];
+    u32x4 hdr[NR];  // headers of the current super-block: d | dmin << 16, then the 12 scale bytes
+};
+
+// 8 quants of one dword (low nibbles, then high nibbles) times their integer scales -> 8 exact f16 values.
 // 0x6400 | q is the f16 1024 + q; (1024 + q) * sc - 1024 * sc is exact in a packed f16 fma.
-__device__ __forceinline__ void dequant16(const uint4 piece, const int plane, const uint32_t sc, uint4 &lo8, uint4 &hi8) {
-    const _Float16 s = (_Float16)(float)sc;
-    const half2_t sc2 = {s, s};
-    const _Float16 o = (_Float16)(-1024.0f * (float)sc);  // exact: sc <= 63
-    const half2_t off2 = {o, o};
-    const uint32_t w[4] = {piece.x, piece.y, piece.z, piece.w};
-    uint32_t out[8];
-#pragma unroll
-    for (int d = 0; d < 4; d++) {
-        const uint32_t nib = (plane ? (w[d] >> 4) : w[d]) & 0x0F0F0F0Fu;  // 4 quants, one per byte
-        // bytes (b0, b1) and (b2, b3) -> f16 pairs 0x64bb
-        const uint32_t p0 = __builtin_amdgcn_perm(0x64646464u, nib, 0x04010400u);
-        const uint32_t p1 = __builtin_amdgcn_perm(0x64646464u, nib, 0x04030402u);
-        // must be a fused multiply-add: the product alone is not representable in f16
-        const half2_t r0 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, p0), sc2, off2);
-        const half2_t r1 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, p1), sc2, off2);
-        out[2 * d] = __builtin_bit_cast(uint32_t, r0);
-        out[2 * d + 1] = __builtin_bit_cast(uint32_t, r1);
-    }
-    lo8 = make_uint4(out[0], out[1], out[2], out[3]);
-    hi8 = make_uint4(out[4], out[5], out[6], out[7]);
+__device__ __forceinline__ half8_t dequant8(const uint32_t w, const half2_t sc_lo, const half2_t off_lo, const half2_t sc_hi,
+                                            const half2_t off_hi) {
+    const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
+    const half2_t r0 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, lo, 0x04010400u)), sc_lo, off_lo);
+    const half2_t r1 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, lo, 0x04030402u)), sc_lo, off_lo);
+    const half2_t r2 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, hi, 0x04010400u)), sc_hi, off_hi);
+    const half2_t r3 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, hi, 0x04030402u)), sc_hi, off_hi);
+    return half8_t{r0[0], r0[1], r1[0], r1[1], r2[0], r2[1], r3[0], r3[1]};
 }
 
-// (scale, min) of sub-block j from the 12 scale bytes (quantize.rs:844-855); j is a compile-time constant
-// wherever this is called, so the branch folds.
-__device__ __forceinline__ void scale_min_u(const uint4 hdr, const int j, uint32_t &sc, uint32_t &mn) {
-    const int sh = 8 * (j & 3);
-    if (j < 4) {
-        sc = (hdr.y >> sh) & 63u;
-        mn = (hdr.z >> sh) & 63u;
+// The same in four pieces, so that the pieces can be placed between matrix instructions.  k-step t selects the
+// scales: GGML order multiplies the low nibbles by the first and the high nibbles by the second sub-block scale,
+// REF order both by the scale of sub-block t / 4.
+struct Dq {
+    uint32_t lo, hi;
+    half2_t r[4];
+    __device__ __forceinline__ half8_t value() const { return half8_t{r[0][0], r[0][1], r[1][0], r[1][1], r[2][0], r[2][1], r[3][0], r[3][1]}; }
+};
+template <int ORDER>
+__device__ __forceinline__ void dq_chunk(const int c, const int t, const uint32_t w, const half2_t (&sc2)[2], const half2_t (&off2)[2], Dq &d) {
+    const int lo_s = ORDER == 0 ? (t >> 2) : 0, hi_s = ORDER == 0 ? (t >> 2) : 1;
+    if (c == 0) {
+        d.lo = w & 0x0F0F0F0Fu;
+        d.r[0] = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, d.lo, 0x04010400u)), sc2[lo_s], off2[lo_s]);
+    } else if (c == 1) {
+        d.r[1] = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, d.lo, 0x04030402u)), sc2[lo_s], off2[lo_s]);
+        d.hi = (w >> 4) & 0x0F0F0F0Fu;
+    } else if (c == 2) {
+        d.r[2] = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, d.hi, 0x04010400u)), sc2[hi_s], off2[hi_s]);
     } else {
-        const uint32_t c = hdr.w >> sh;
-        sc = (c & 0xFu) | (((hdr.y >> (sh + 6)) & 3u) << 4);
-        mn = ((c >> 4) & 0xFu) | (((hdr.z >> (sh + 6)) & 3u) << 4);
+        d.r[3] = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, d.hi, 0x04030402u)), sc2[hi_s], off2[hi_s]);
     }
-}
-
-// 16 bytes / 4 bytes / 2 bytes at an address that is only 2-byte aligned (Q6_K super-blocks are 210 bytes)
-struct __attribute__((packed, aligned(2))) u32x4_a2 {
-    uint32_t x, y, z, w;
-};
-struct __attribute__((packed, aligned(2))) u32_a2 {
-    uint32_t v;
-};
-typedef uint16_t u16_a2 __attribute__((aligned(2)));
-
-__device__ __forceinline__ u32x4 load16_a2(const uint8_t *p) {
-    const u32x4_a2 t = *reinterpret_cast<const u32x4_a2 *>(p);
-    return u32x4{t.x, t.y, t.z, t.w};
-}
-
-// Q6_K: 16 six-bit quants (low nibbles in ql shifted by ql_shift, top two bits in qh at qh_shift) of one
-// 16-element scale group.  sc * (q - 32) can reach 4096 and would not always be exact in f16, so the value is
-// split where the storage splits it, q - 32 = 16 (hi2 - 2) + nib, into two exact tiles:
-//     B1 = (16 sc) * (hi2 - 2)   |.| <= 2048 * 2, a multiple of 16        B2 = sc * nib   |.| <= 1920
-// multiplied one after the other into the same accumulator.  (0x6400 | v is the f16 1024 + v.)
-__device__ __forceinline__ void dequant16_q6(const u32x4 ql, const u32x4 qh, const int ql_shift, const int qh_shift,
-                                             const int sc, uint4 &b1lo, uint4 &b1hi, uint4 &b2lo, uint4 &b2hi) {
-    const _Float16 s1 = (_Float16)(float)(16 * sc), s2 = (_Float16)(float)sc;  // exact: |sc| <= 128
-    const half2_t s1v = {s1, s1}, s2v = {s2, s2};
-    const half2_t m1026 = {(_Float16)-1026.0f, (_Float16)-1026.0f}, m1024 = {(_Float16)-1024.0f, (_Float16)-1024.0f};
-    const uint32_t lw[4] = {ql.x, ql.y, ql.z, ql.w}, hw[4] = {qh.x, qh.y, qh.z, qh.w};
-    uint32_t o1[8], o2[8];
-#pragma unroll
-    for (int d = 0; d < 4; d++) {
-        const uint32_t nib = (lw[d] >> ql_shift) & 0x0F0F0F0Fu;
-        const uint32_t hi2 = (hw[d] >> qh_shift) & 0x03030303u;
-#pragma unroll
-        for (int half = 0; half < 2; half++) {
-            const uint32_t sel = half ? 0x04030402u : 0x04010400u;  // bytes (b0, b1) resp. (b2, b3) -> 0x64bb pairs
-            const half2_t n2 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, nib, sel));
-            const half2_t h2 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, hi2, sel));
-            o2[2 * d + half] = __builtin_bit_cast(uint32_t, (n2 + m1024) * s2v);  // both steps exact
-            o1[2 * d + half] = __builtin_bit_cast(uint32_t, (h2 + m1026) * s1v);
-        }
-    }
-    b1lo = make_uint4(o1[0], o1[1], o1[2], o1[3]);
-    b1hi = make_uint4(o1[4], o1[5], o1[6], o1[7]);
-    b2lo = make_uint4(o2[0], o2[1], o2[2], o2[3]);
-    b2hi = make_uint4(o2[4], o2[5], o2[6], o2[7]);
 }
 
 // -(dmin * mn) split exactly into an f16 head and tail (dmin has 11 significant bits, mn 6).
@@ -238,279 +243,248 @@ __device__ __forceinline__ void neg_min_split(const float dmin, const uint32_t m
     l = (_Float16)(p - (float)h);
 }
 
-// Workgroup = WM x WN waves, every wave owns NB x NB MFMA blocks of 32 x 32:
-//   <4, 2, 2>: 256 x 128 tile, 512 threads      <2, 2, 2>: 128 x 128, 256 threads      <2, 1, 1>: 64 x 32, 128 threads
-template <int QT, int WM, int WN, int NB>
-struct Tile {
-    static constexpr int BM = 32 * NB * WM, BN = 32 * NB * WN, kThreads = 64 * WM * WN;
-    static constexpr int kUnits = kThreads / BN;   // threads per weight row
-    static constexpr int kBTasks = 4 / kUnits;     // (piece, plane) tasks per thread and stage
-    // 16-byte pieces of weight data per thread and stage: Q4_K one or two quant pieces; Q6_K ql + qh per task
-    static constexpr int kPieces = QT == 14 ? 2 * kBTasks : (kBTasks == 4 ? 2 : 1);
-    static constexpr int kBItems = (QT == 14 ? 16 : 8) * BN;  // items of one B stage (Q6_K: two tiles)
-    static constexpr int kBlockBytes = QT == 14 ? 210 : 144;
-    static constexpr int kAItems = 8 * BM / kThreads;  // A items per thread and stage
-    static constexpr size_t kLdsBytes = (size_t)(2 * 8 * BM + 2 * kBItems + 4 * BN) * 16 + BN * 4;
-    static_assert(kUnits == 1 || kUnits == 2 || kUnits == 4, "a weight row is staged by 1, 2 or 4 threads");
-    static_assert(8 * BM % kThreads == 0, "the A tile must divide among the threads");
-};
-
-template <int QT, int ORDER, bool YBF16, int WM, int WN, int NB>
-__global__ __launch_bounds__(64 * WM * WN, NB == 1 ? 2 : 512 / (64 * WM * WN)) void k_qgemm(
-    const uint8_t *__restrict__ W, const uint4 *__restrict__ xs, const uint4 *__restrict__ xsum,
-    const float *__restrict__ rowscale, void *__restrict__ yg, int M, int Mp, int N, int spr) {
-    using TL = Tile<QT, WM, WN, NB>;
-    constexpr int BM = TL::BM, BN = TL::BN, kThreads = TL::kThreads, kUnits = TL::kUnits, kBTasks = TL::kBTasks,
-                  kPieces = TL::kPieces, kAItems = TL::kAItems, kBItems = TL::kBItems;
-    constexpr bool kQ6 = QT == 14;
-    // LDS: two stages of the A tile [8 chunks][BM] and the B tile [4 k-steps][2 k-groups][BN] (16-byte items),
-    // the B operand of the R product [2][2][BN] and d [BN] of the current super-block.
-    extern __shared__ uint4 smem[];
-    uint4 *lds_a = smem;
-    uint4 *lds_b = lds_a + 2 * 8 * BM;
-    uint4 *lds_r = lds_b + 2 * kBItems;
-    float *lds_d = reinterpret_cast<float *>(lds_r + 4 * BN);
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WN, wn = wave % WN;  // wave position in the WM x WN grid
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-    const size_t row_bytes = (size_t)spr * TL::kBlockBytes;
-
-    // ---- loader roles ----
-    // A: item idx = tid + i * kThreads (i < kAItems) -> chunk = idx / BM, row = idx % BM: a wave copies 64
-    //    consecutive items.
-    // B: weight row bn = tid % BN, unit bu = tid / BN; (piece, plane) task q = bu * kBTasks + t,
-    //    piece = q / 2, plane = q % 2.
-    const int bn = tid % BN, bu = tid / BN;
-    const uint8_t *wrow = W + (size_t)(n0 + bn < N ? n0 + bn : N - 1) * row_bytes;
-
-    // One stage's global data in registers: the A items of this thread, and for B the super-block header and
-    // one or two 16-byte pieces.  Steps past the end re-read the last one, so every load is unconditional.
-    const int last_step = spr * 4 - 1;
-    auto fetch_a = [&](int step, u32x4 (&fa)[kAItems]) __attribute__((always_inline)) {
-        step = step < last_step ? step : last_step;
+// One half super-block H of one wave.  The restrict qualifiers say what the copies in flight cannot touch:
+// operand reads from a_cur / q_cur need not wait for the direct loads into a_nxt / q_nxt / hb.
+//   a_cur / a_nxt: activation stages (18 x BM items)      q_cur / q_nxt: this wave's quant pieces (NR x 128 items)
+//   hb: this wave's headers (NR x 64 items)
+//   xs_nxt: item (group 0, row m0) of the next half super-block    wq_nxt / wh_nxt: first row of the workgroup at
+//   the next half's quant bytes / the next super-block's header
+template <int ORDER, int MB, int NR, int NW, int H>
+__device__ __forceinline__ void rw_half(const uint4 *__restrict__ a_cur, uint4 *__restrict__ a_nxt,
+                                        const uint4 *__restrict__ q_cur, uint4 *__restrict__ q_nxt, uint4 *__restrict__ hb,
+                                        const uint4 *__restrict__ xs_nxt, const uint8_t *__restrict__ wq_nxt,
+                                        const uint8_t *__restrict__ wh_nxt, const Lane<MB, NR, NW> &L, Acc<MB, NR> &R) {
+    constexpr int BM = 32 * MB, kThreads = 64 * NW;
+    const int col = L.col, g = L.g;
+    if (H == 0) {
 #pragma unroll
-        for (int i = 0; i < kAItems; i++) {
-            const int idx = tid + i * kThreads;
-            fa[i] = *reinterpret_cast<const u32x4 *>(xs + (size_t)(step * 8 + idx / BM) * Mp + m0 + idx % BM);
+        for (int rg = 0; rg < NR; rg++) {
+            const uint4 hv = hb[rg * 64 + col];
+            R.hdr[rg] = u32x4{hv.x, hv.y, hv.z, hv.w};
         }
-    };
-    auto fetch_b = [&](int step, u32x4 &fhdr, u32x4 (&fpc)[kPieces]) __attribute__((always_inline)) {
-        step = step < last_step ? step : last_step;
-        const uint8_t *blk = wrow + (size_t)(step >> 2) * TL::kBlockBytes;
-        const int c = step & 3;
-        if constexpr (kQ6) {
-            // stage c covers elements 64 c .. + 63 of the super-block: half h = c / 2, the low (c even) or high
-            // nibbles of ql bytes 64 h .. + 63 in natural order, qh bytes 32 h + (k % 32) at bit 2 (2 (c % 2) + k / 32),
-            // scales 4 c .. 4 c + 3 (crates/pmetal-gguf/src/k_quants.rs:484-494).  Task = one 16-element scale group.
-            const int h = c >> 1;
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the headers are in registers before their buffer is refilled
 #pragma unroll
-            for (int t = 0; t < kBTasks; t++) {
-                const int ks = bu * kBTasks + t;
-                fpc[t] = load16_a2(blk + 64 * h + 16 * ks);
-                fpc[kBTasks + t] = load16_a2(blk + 128 + 32 * h + 16 * (ks & 1));
-            }
-            fhdr = u32x4{reinterpret_cast<const u32_a2 *>(blk + 192 + 4 * c)->v, *reinterpret_cast<const u16_a2 *>(blk + 208), 0u, 0u};
-        } else {
-            fhdr = *reinterpret_cast<const u32x4 *>(blk);
-            // the stage covers sub-blocks 2c and 2c+1, which are pieces 2c and 2c+1 in both orders
-            if (kPieces == 2) {
-#pragma unroll
-                for (int q = 0; q < kPieces; q++) fpc[q] = *reinterpret_cast<const u32x4 *>(blk + 16 + 16 * (2 * c + q));
-            } else {
-                const int pc = (bu * kBTasks) >> 1;
-                fpc[0] = *reinterpret_cast<const u32x4 *>(blk + 16 + 16 * (2 * c + pc));
-            }
-        }
-    };
-    auto stage_a = [&](int stage, const u32x4 (&fa)[kAItems]) __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < kAItems; i++) *reinterpret_cast<u32x4 *>(lds_a + stage * 8 * BM + tid + i * kThreads) = fa[i];
-    };
-    // c = step % 4 is a compile-time constant at every call
-    auto stage_b = [&](int stage, int c, const u32x4 &fhdr, const u32x4 (&fpc)[kPieces]) __attribute__((always_inline)) {
-        if constexpr (kQ6) {
-            uint4 *dst1 = lds_b + stage * kBItems, *dst2 = dst1 + 8 * BN;
-#pragma unroll
-            for (int t = 0; t < kBTasks; t++) {
-                const int ks = bu * kBTasks + t;
-                const int sc = (int)(int8_t)(fhdr.x >> (8 * ks));
-                uint4 b1lo, b1hi, b2lo, b2hi;
-                dequant16_q6(fpc[t], fpc[kBTasks + t], 4 * (c & 1), 2 * (2 * (c & 1) + (ks >> 1)), sc, b1lo, b1hi, b2lo, b2hi);
-                dst1[(ks * 2 + 0) * BN + bn] = b1lo;
-                dst1[(ks * 2 + 1) * BN + bn] = b1hi;
-                dst2[(ks * 2 + 0) * BN + bn] = b2lo;
-                dst2[(ks * 2 + 1) * BN + bn] = b2hi;
-            }
-            if (c == 1 && bu == 0) lds_d[bn] = f16_bits_to_f32(fhdr.y);
-        } else {
-            uint4 *dst = lds_b + stage * kBItems;
-            const uint4 hdr4 = make_uint4(fhdr.x, fhdr.y, fhdr.z, fhdr.w);
-            uint32_t sc0, sc1, mn;
-            scale_min_u(hdr4, 2 * c, sc0, mn);
-            scale_min_u(hdr4, 2 * c + 1, sc1, mn);
-    #pragma unroll
-            for (int t = 0; t < kBTasks; t++) {
-                const int q = bu * kBTasks + t;
-                const int bw = q >> 1, p = q & 1;
-                // nibble plane p of piece bw:
-                //   REF : elements 16 p .. + 15 of sub-block 2c + bw  -> k = 32 bw + 16 p + b, scale 2c + bw
-                //   GGML: elements 16 bw .. + 15 of sub-block 2c + p  -> k = 32 p + 16 bw + b, scale 2c + p
-                const int ks = ORDER == 0 ? 2 * bw + p : 2 * p + bw;
-                const uint32_t sc = (ORDER == 0 ? bw : p) ? sc1 : sc0;
-                const u32x4 pc4 = fpc[kPieces == 2 ? bw : 0];
-                uint4 b0, b1;
-                dequant16(make_uint4(pc4.x, pc4.y, pc4.z, pc4.w), p, sc, b0, b1);
-                dst[(ks * 2 + 0) * BN + bn] = b0;
-                dst[(ks * 2 + 1) * BN + bn] = b1;
-            }
-            if (c == 1) {
-                // once per super-block (while its second stage is being staged, one barrier after the previous
-                // super-block's R product has been issued): d and the B operand of the R product for this column.
-                // item (t, g) = (-h_j, -h_j, -l_j, -l_j, -h_j+1, -h_j+1, -l_j+1, -l_j+1), j = 4 t + 2 g, against
-                // the activations' (h, l, h, l, ...): all four cross products.
-                const float dmin = f16_bits_to_f32(hdr4.x >> 16);
-                if (bu == 0) lds_d[bn] = f16_bits_to_f32(hdr4.x & 0xFFFFu);
-    #pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    if (r % kUnits == bu) {
-                        uint32_t sc, mn0, mn1;
-                        scale_min_u(hdr4, 2 * r, sc, mn0);
-                        scale_min_u(hdr4, 2 * r + 1, sc, mn1);
-                        _Float16 h0, l0, h1, l1;
-                        neg_min_split(dmin, mn0, h0, l0);
-                        neg_min_split(dmin, mn1, h1, l1);
-                        const half8_t item = {h0, h0, l0, l0, h1, h1, l1, l1};
-                        lds_r[r * BN + bn] = __builtin_bit_cast(uint4, item);
-                    }
-                }
-            }
-        }
-    };
-
-    // ---- accumulators: NB x NB blocks of 32 x 32 per wave ----
-    float16_t acc[NB][NB], part[NB][NB];
-#pragma unroll
-    for (int i = 0; i < NB; i++)
-#pragma unroll
-        for (int jx = 0; jx < NB; jx++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][jx][r] = 0.0f, part[i][jx][r] = 0.0f;
-
-    const int col = lane & 31, kgrp = lane >> 5;
-
-    // A operand of the R product: requested one step before it is used
-    u32x4 xsv[2][NB];
-    auto fetch_xsum = [&](int sb) __attribute__((always_inline)) {
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-            for (int i = 0; i < NB; i++)
-                xsv[t][i] = *reinterpret_cast<const u32x4 *>(xsum + ((size_t)sb * 4 + t * 2 + kgrp) * Mp + m0 + (wm * NB + i) * 32 + col);
-    };
-
-    // c = step % 4 is a compile-time constant at every call
-    auto compute = [&](int stage, int c, int sb) __attribute__((always_inline)) {
-        const uint4 *sa = lds_a + stage * 8 * BM, *sbp = lds_b + stage * kBItems;
-#pragma unroll
-        for (int ks = 0; ks < 4; ks++) {
-            half8_t av[NB], bv[NB], bw[NB];
-#pragma unroll
-            for (int i = 0; i < NB; i++) av[i] = __builtin_bit_cast(half8_t, sa[(ks * 2 + kgrp) * BM + (wm * NB + i) * 32 + col]);
-#pragma unroll
-            for (int jx = 0; jx < NB; jx++) {
-                bv[jx] = __builtin_bit_cast(half8_t, sbp[(ks * 2 + kgrp) * BN + (wn * NB + jx) * 32 + col]);
-                if (kQ6) bw[jx] = __builtin_bit_cast(half8_t, sbp[8 * BN + (ks * 2 + kgrp) * BN + (wn * NB + jx) * 32 + col]);
-            }
-#pragma unroll
-            for (int i = 0; i < NB; i++)
-#pragma unroll
-                for (int jx = 0; jx < NB; jx++) {
-                    if (c == 0 && ks == 0) {  // first product of a super-block starts from zero
-                        float16_t z;
-#pragma unroll
-                        for (int r = 0; r < 16; r++) z[r] = 0.0f;
-                        part[i][jx] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bv[jx], z, 0, 0, 0);
-                    } else {
-                        part[i][jx] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bv[jx], part[i][jx], 0, 0, 0);
-                    }
-                    if (kQ6) part[i][jx] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bw[jx], part[i][jx], 0, 0, 0);
-                }
-        }
-        if (c == 3) {
-            // ---- end of a super-block: R product into the accumulators (Q4_K), then acc += d * P ----
-#pragma unroll
-            for (int t = 0; t < (kQ6 ? 0 : 2); t++) {
-                half8_t sv[NB], mv[NB];
-#pragma unroll
-                for (int i = 0; i < NB; i++) sv[i] = __builtin_bit_cast(half8_t, xsv[t][i]);
-#pragma unroll
-                for (int jx = 0; jx < NB; jx++) mv[jx] = __builtin_bit_cast(half8_t, lds_r[(t * 2 + kgrp) * BN + (wn * NB + jx) * 32 + col]);
-#pragma unroll
-                for (int i = 0; i < NB; i++)
-#pragma unroll
-                    for (int jx = 0; jx < NB; jx++)
-                        acc[i][jx] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sv[i], mv[jx], acc[i][jx], 0, 0, 0);
-            }
-#pragma unroll
-            for (int jx = 0; jx < NB; jx++) {
-                const float dd = lds_d[(wn * NB + jx) * 32 + col];
-#pragma unroll
-                for (int i = 0; i < NB; i++)
-#pragma unroll
-                    for (int r = 0; r < 16; r++) acc[i][jx][r] = __builtin_fmaf(dd, part[i][jx][r], acc[i][jx][r]);
-            }
-        }
-    };
-
-    // Global loads run ahead of the LDS staging in register sets; with four steps per loop trip the set a step
-    // uses is a compile-time constant.  Large tiles (registers are scarce): B two steps ahead in two sets, A
-    // requested at the start of a step and stored to LDS at its end, behind the MFMAs.  The small tile (short
-    // steps, few waves per compute unit to hide latency): both four steps ahead in four sets.
-    // Two LDS stages; one barrier per step; c = step % 4 and the LDS stage are compile-time constants.
-    constexpr int DA = NB == 1 ? 4 : 1, DB = NB == 1 ? 4 : 2;
-    u32x4 fa[DA][kAItems], fh[DB], fp[DB][kPieces];
-#pragma unroll
-    for (int i = 0; i < DA; i++) fetch_a(i, fa[i]);
-#pragma unroll
-    for (int i = 0; i < DB; i++) fetch_b(i, fh[i], fp[i]);
-    stage_a(0, fa[0]);
-    stage_b(0, 0, fh[0], fp[0]);
-    if (DA > 1) fetch_a(DA, fa[0]);
-    fetch_b(DB, fh[0], fp[0]);
-    __syncthreads();
-#define PMH_STEP(C)                                                                                      \
-    if ((C) == 2 && !kQ6) fetch_xsum(sb);                                                                        \
-    if (DA == 1) {                                                                                       \
-        fetch_a(step + (C) + 1, fa[0]);                                                                  \
-        __builtin_amdgcn_sched_barrier(0); /* keep the requests a whole step ahead of their use */       \
-    }                                                                                                    \
-    stage_b(((C) + 1) & 1, ((C) + 1) & 3, fh[((C) + 1) % DB], fp[((C) + 1) % DB]);                       \
-    fetch_b(step + (C) + 1 + DB, fh[((C) + 1) % DB], fp[((C) + 1) % DB]);                                \
-    compute((C) & 1, C, sb);                                                                             \
-    stage_a(((C) + 1) & 1, fa[((C) + 1) % DA]);                                                          \
-    if (DA > 1) fetch_a(step + (C) + 1 + DA, fa[((C) + 1) % DA]);                                        \
-    __syncthreads();
-    for (int sb = 0; sb < spr; sb++) {
-        const int step = sb * 4;
-        PMH_STEP(0)
-        PMH_STEP(1)
-        PMH_STEP(2)
-        PMH_STEP(3)
+        for (int rg = 0; rg < NR; rg++) dma16(wh_nxt + L.h_off[rg], hb + rg * 64);
     }
-#undef PMH_STEP
+    // copies for the next half super-block
+#pragma unroll
+    for (int i = 0; i < Lane<MB, NR, NW>::kARounds; i++)
+        if (i * kThreads + L.wave * 64 < kGroups * BM) dma16(xs_nxt + L.a_off[i], a_nxt + i * kThreads + L.wave * 64);
+#pragma unroll
+    for (int rg = 0; rg < NR; rg++)
+#pragma unroll
+        for (int r = 0; r < 2; r++) dma16(wq_nxt + L.q_off[rg][r], q_nxt + rg * 128 + r * 64);
+    __builtin_amdgcn_sched_barrier(0);  // the copies are requested before anything else of this half
 
-    // ---- epilogue: C layout of v_mfma_f32_32x32x*: lane holds column (lane & 31), rows 8 (r / 4) + 4 (lane / 32) + r % 4
+    // scales and mins of sub-blocks j0 = 4 H + 2 g and j0 + 1 (6-bit fields, crates/pmetal/src/commands/quantize.rs:844-855)
+    const uint32_t sh = 16u * (uint32_t)g;
+    half2_t sc2[NR][2], off2[NR][2];
+    uint32_t mn[NR][2];
+    uint32_t qd[NR][8];
+    // this lane's 32 quant bytes per row group: pieces 2g and 2g+1 of row col (the copy swizzles the four pieces of
+    // a row by (row / 4) % 4 so that 16 consecutive rows read conflict-free)
+    const int sw = (col >> 2) & 3;
 #pragma unroll
-    for (int i = 0; i < NB; i++)
+    for (int rg = 0; rg < NR; rg++) {
+        const uint4 qa = q_cur[rg * 128 + col * 4 + ((2 * g) ^ sw)], qb = q_cur[rg * 128 + col * 4 + ((2 * g + 1) ^ sw)];
+        qd[rg][0] = qa.x, qd[rg][1] = qa.y, qd[rg][2] = qa.z, qd[rg][3] = qa.w;
+        qd[rg][4] = qb.x, qd[rg][5] = qb.y, qd[rg][6] = qb.z, qd[rg][7] = qb.w;
+        uint32_t sc0, sc1;
+        if (H == 0) {
+            const uint32_t yv = R.hdr[rg].y >> sh, zv = R.hdr[rg].z >> sh;
+            sc0 = yv & 63u, sc1 = (yv >> 8) & 63u;
+            mn[rg][0] = zv & 63u, mn[rg][1] = (zv >> 8) & 63u;
+        } else {
+            const uint32_t wv = R.hdr[rg].w >> sh, yv = R.hdr[rg].y >> sh, zv = R.hdr[rg].z >> sh;
+            sc0 = (wv & 0xFu) | ((yv >> 2) & 0x30u), sc1 = ((wv >> 8) & 0xFu) | ((yv >> 10) & 0x30u);
+            mn[rg][0] = ((wv >> 4) & 0xFu) | ((zv >> 2) & 0x30u), mn[rg][1] = ((wv >> 12) & 0xFu) | ((zv >> 10) & 0x30u);
+        }
+        const _Float16 s0 = (_Float16)(float)sc0, s1 = (_Float16)(float)sc1;
+        const _Float16 o0 = (_Float16)(-1024.0f * (float)sc0), o1 = (_Float16)(-1024.0f * (float)sc1);  // exact: sc <= 63
+        sc2[rg][0] = half2_t{s0, s0}, sc2[rg][1] = half2_t{s1, s1};
+        off2[rg][0] = half2_t{o0, o0}, off2[rg][1] = half2_t{o1, o1};
+    }
+
+    // min term of sub-blocks j0, j0 + 1: (-h, -h, -l, -l) against the activations' (H, L, H, L): all four cross
+    // products of the exact head + tail splits, straight into the accumulators (after the eight k-steps)
+    half8_t br[NR];
 #pragma unroll
-        for (int jx = 0; jx < NB; jx++) {
-            const int n = n0 + (wn * NB + jx) * 32 + col;
+    for (int rg = 0; rg < NR; rg++) {
+        const float dmin = f16_bits_to_f32(R.hdr[rg].x >> 16);
+        _Float16 h0, l0, h1, l1;
+        neg_min_split(dmin, mn[rg][0], h0, l0);
+        neg_min_split(dmin, mn[rg][1], h1, l1);
+        br[rg] = half8_t{h0, h0, l0, l0, h1, h1, l1, l1};
+    }
+
+    // Software pipeline, written in issue order (a wave issues in order, so the order here is the schedule):
+    // the activation fragments of k-step t + 1 are requested before the products of k-step t, and the weights of
+    // k-step t + 1 are dequantized in pieces between those products.
+    constexpr int kSlots = MB * NR, kChunks = 4 * NR;
+    half8_t af[2][MB];
+    Dq dq[NR];
+#pragma unroll
+    for (int i = 0; i < MB; i++) af[0][i] = __builtin_bit_cast(half8_t, a_cur[g * BM + 32 * i + col]);
+#pragma unroll
+    for (int rg = 0; rg < NR; rg++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) dq_chunk<ORDER>(c, 0, qd[rg][0], sc2[rg], off2[rg], dq[rg]);
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+        half8_t b[NR];
+#pragma unroll
+        for (int rg = 0; rg < NR; rg++) b[rg] = dq[rg].value();
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < MB; i++)
+#pragma unroll
+            for (int rg = 0; rg < NR; rg++) {
+                const half8_t a = af[t & 1][i];
+                if (H == 0 && t == 0) {  // first product of a super-block starts from zero
+                    float16_t z;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) z[r] = 0.0f;
+                    R.part[rg][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b[rg], z, 0, 0, 0);
+                } else {
+                    R.part[rg][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b[rg], R.part[rg][i], 0, 0, 0);
+                }
+                if (t < 7) {
+                    const int slot = i * NR + rg;
+#pragma unroll
+                    for (int ch = slot * kChunks / kSlots; ch < (slot + 1) * kChunks / kSlots; ch++)
+                        dq_chunk<ORDER>(ch % 4, t + 1, qd[ch / 4][t + 1], sc2[ch / 4], off2[ch / 4], dq[ch / 4]);
+                }
+                if (i == 0 && rg == 0) {
+                    // the next step's fragments are requested behind the first product of this step: the wait in
+                    // front of that product then covers only fragments requested a whole step ago
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int ii = 0; ii < MB; ii++)
+                        af[(t + 1) & 1][ii] = __builtin_bit_cast(half8_t, a_cur[(t < 7 ? (t + 1) * 2 + g : 16 + g) * BM + 32 * ii + col]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+    }
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+#pragma unroll
+        for (int rg = 0; rg < NR; rg++) R.acc[rg][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[0][i], br[rg], R.acc[rg][i], 0, 0, 0);
+    if (H == 1) {
+#pragma unroll
+        for (int rg = 0; rg < NR; rg++) {
+            const float d = f16_bits_to_f32(R.hdr[rg].x & 0xFFFFu);
+#pragma unroll
+            for (int i = 0; i < MB; i++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) R.acc[rg][i][r] = __builtin_fmaf(d, R.part[rg][i][r], R.acc[rg][i][r]);
+        }
+    }
+}
+
+// grid (ceil(N / (32 NR NW)), Mp / BM, splits); workgroup z works on super-blocks [z * chunk, min(spr, (z + 1) * chunk)).
+// mode 0: y f32 [M][N], 1: y bf16, 2: fp32 partial tiles [splits][Mp][N] (not yet scaled by rowscale)
+//
+// Copies in flight: the activation stage of the next half super-block (it comes from L2) and the quant pieces of
+// the next two (they come from HBM): three quant stages per wave, rotated.  Within a half super-block the
+// activation copies are requested before the quant copies, so waiting until only the 2 NR newest requests are
+// outstanding leaves exactly the quant copies for the half after next in flight.
+template <int ORDER, int MB, int NR, int NW>
+__global__ __launch_bounds__(64 * NW, MB * NR <= 1 && NW <= 8 ? 2 : 1) void k_qgemm_rw(
+    const uint8_t *__restrict__ W, const uint4 *__restrict__ xs, const float *__restrict__ rowscale, void *__restrict__ yg,
+    float *__restrict__ partial, int M, int Mp, int N, int spr, int chunk, int mode) {
+    constexpr int BM = 32 * MB, kThreads = 64 * NW, kRows = 32 * NR * NW;
+    extern __shared__ uint4 smem[];
+    uint4 *a0 = smem, *a1 = a0 + kGroups * BM, *qbase = a1 + kGroups * BM, *hb = qbase + 3 * NW * NR * 128;
+    const int tid = threadIdx.x;
+    Lane<MB, NR, NW> L;
+    L.wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    L.col = lane & 31, L.g = lane >> 5;
+    const int n0 = blockIdx.x * kRows, m0 = blockIdx.y * BM;
+    const int nw0 = n0 + 32 * NR * L.wave;  // first weight row of this wave
+    const int sb0 = blockIdx.z * chunk;
+    const int cnt = spr - sb0 < chunk ? spr - sb0 : chunk;
+    const uint32_t row_bytes = (uint32_t)spr * kBlockBytes;
+    auto row_off = [&](int row) {  // byte offset of a row of this wave from the workgroup's first row; rows past N repeat the last
+        int n = nw0 + row;
+        n = n < N ? n : N - 1;
+        return (uint32_t)(n - n0) * row_bytes;
+    };
+#pragma unroll
+    for (int rg = 0; rg < NR; rg++) {
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+            const int row = 16 * r + (lane >> 2);
+            L.q_off[rg][r] = row_off(32 * rg + row) + 16u * (uint32_t)((lane & 3) ^ ((row >> 2) & 3));
+        }
+        L.h_off[rg] = row_off(32 * rg + (lane & 31));
+    }
+#pragma unroll
+    for (int i = 0; i < Lane<MB, NR, NW>::kARounds; i++) {
+        const int idx = tid + i * kThreads;
+        L.a_off[i] = (uint32_t)((idx / BM) * Mp + idx % BM);
+    }
+    // this wave's three quant stages (rotated: qa is read, qb is next, qc receives the copies) and its headers
+    uint4 *qa = qbase + L.wave * (NR * 128), *qb = qa + NW * NR * 128, *qc = qb + NW * NR * 128;
+    uint4 *hw = hb + L.wave * (NR * 64);
+    const uint8_t *wblk = W + (size_t)n0 * row_bytes;
+
+    Acc<MB, NR> R;
+#pragma unroll
+    for (int rg = 0; rg < NR; rg++)
+#pragma unroll
+        for (int i = 0; i < MB; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) R.acc[rg][i][r] = 0.0f, R.part[rg][i][r] = 0.0f;
+
+    // prologue: headers, both halves' quant pieces and the first activation stage of super-block sb0
+    {
+        const uint8_t *blk = wblk + (size_t)sb0 * kBlockBytes;
+#pragma unroll
+        for (int rg = 0; rg < NR; rg++) {
+            dma16(blk + L.h_off[rg], hw + rg * 64);
+#pragma unroll
+            for (int r = 0; r < 2; r++) {
+                dma16(blk + 16 + L.q_off[rg][r], qa + rg * 128 + r * 64);
+                dma16(blk + 16 + 64 + L.q_off[rg][r], qb + rg * 128 + r * 64);
+            }
+        }
+        const uint4 *xa = xs + (size_t)(sb0 * 2 * kGroups) * Mp + m0;
+#pragma unroll
+        for (int i = 0; i < Lane<MB, NR, NW>::kARounds; i++)
+            if (i * kThreads + L.wave * 64 < kGroups * BM) dma16(xa + L.a_off[i], a0 + i * kThreads + L.wave * 64);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();
+
+    for (int s = 0; s < cnt; s++) {
+        const int sb = sb0 + s;
+        const int sbn = sb + 1 < spr ? sb + 1 : spr - 1;  // the copies for "the next super-block" stay inside the matrix
+        const uint8_t *blkn = wblk + (size_t)sbn * kBlockBytes;
+        rw_half<ORDER, MB, NR, NW, 0>(a0, a1, qa, qc, hw, xs + (size_t)((sb * 2 + 1) * kGroups) * Mp + m0, blkn + 16, blkn, L, R);
+        barrier_keep<2 * NR>();
+        rw_half<ORDER, MB, NR, NW, 1>(a1, a0, qb, qa, hw, xs + (size_t)(sbn * 2 * kGroups) * Mp + m0, blkn + 16 + 64, nullptr, L, R);
+        barrier_keep<2 * NR>();
+        // two half super-blocks on: (qa, qb, qc) <- (qc, qa, qb)
+        uint4 *t = qc;
+        qc = qb, qb = qa, qa = t;
+    }
+    // C layout of v_mfma_f32_32x32x*: lane holds column (lane & 31), rows 8 (r / 4) + 4 (lane / 32) + r % 4
+#pragma unroll
+    for (int rg = 0; rg < NR; rg++) {
+        const int n = nw0 + 32 * rg + L.col;
+        if (n >= N) continue;
+#pragma unroll
+        for (int i = 0; i < MB; i++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const int m = m0 + (wm * NB + i) * 32 + 8 * (r >> 2) + 4 * kgrp + (r & 3);
-                if (m < M && n < N) {
-                    const float v = acc[i][jx][r] * rowscale[m];
-                    if (YBF16) {
+                const int m = m0 + 32 * i + 8 * (r >> 2) + 4 * L.g + (r & 3);
+                if (m >= M) continue;
+                if (mode == 2) {
+                    partial[((size_t)blockIdx.z * Mp + m) * N + n] = R.acc[rg][i][r];
+                } else {
+                    const float v = R.acc[rg][i][r] * rowscale[m];
+                    if (mode == 1) {
                         uint32_t u = __builtin_bit_cast(uint32_t, v);
                         u = ((u & 0x7FFFFFFFu) > 0x7F800000u) ? ((u >> 16) | 0x40u) : ((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
                         reinterpret_cast<uint16_t *>(yg)[(size_t)m * N + n] = (uint16_t)u;
@@ -519,76 +493,395 @@ __global__ __launch_bounds__(64 * WM * WN, NB == 1 ? 2 : 512 / (64 * WM * WN)) v
                     }
                 }
             }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Q6_K (crates/pmetal-gguf/src/k_quants.rs:474-496: 210-byte super-blocks: ql[128] low nibbles, qh[64] top two
+// bits, 16 int8 scales, f16 d; value d * sc * (q - 32)).  Same structure as the Q4_K kernel, with these differences:
+//   * sc * (q - 32) can reach 4096 and is not always exact in f16, so it is split where the storage splits it,
+//     q - 32 = 16 (hi2 - 2) + nib, into two exact tiles  B1 = (16 sc) (hi2 - 2)  and  B2 = sc * nib  that multiply
+//     the same activation fragment one after the other (a fragment read from LDS feeds two matrix instructions);
+//   * no min term; one scale per 16 elements;
+//   * a half super-block of a row is 64 bytes of ql and 32 of qh; lane (n, g) multiplies ql bytes 32 g .. 32 g + 31
+//     (dword t: low nibbles = elements 32 g + 4 t + e of the half, high nibbles 64 further) with the qh bytes
+//     4 t + e (two-bit field g for the low, 2 + g for the high nibbles);
+//   * super-blocks are only 2-byte aligned; the direct-to-LDS loads take such addresses.
+// ------------------------------------------------------------------------------------------------
+constexpr int kQ6Bytes = 210, kQ6Groups = 16, kQ6Stage = 192;  // LDS items of a wave's quant stage: 128 ql + 64 qh
+
+template <int MB>
+struct LaneQ6 {
+    static constexpr int BM = 32 * MB, kThreads = 512;
+    static constexpr int kARounds = kQ6Groups * BM / kThreads;
+    static_assert(kQ6Groups * BM % kThreads == 0, "the activation stage must divide among the threads");
+    int wave, col, g;
+    uint32_t ql_off[2], qh_off, h_off;  // byte offsets of this lane's pieces from the workgroup's first row
+    uint32_t a_off[kARounds];
+};
+
+template <int MB>
+struct AccQ6 {
+    float16_t acc[MB], part[MB];
+    u32x4 sc;    // the 16 int8 scales of the current super-block
+    uint32_t d;  // f16 bits of d
+};
+
+// The two operands of one k-step, built in eight pieces that are placed between matrix instructions.
+struct Dq6 {
+    uint32_t nlo, nhi, hlo, hhi;
+    half2_t r1[4], r2[4];
+    __device__ __forceinline__ half8_t b1() const { return half8_t{r1[0][0], r1[0][1], r1[1][0], r1[1][1], r1[2][0], r1[2][1], r1[3][0], r1[3][1]}; }
+    __device__ __forceinline__ half8_t b2() const { return half8_t{r2[0][0], r2[0][1], r2[1][0], r2[1][1], r2[2][0], r2[2][1], r2[3][0], r2[3][1]}; }
+};
+// qlw: the ql dword of the k-step; qhw: its qh dword already shifted by 2 g; s2 / s1: (sc, sc) and (16 sc, 16 sc)
+// of the low-nibble and of the high-nibble elements.  0x6400 | v is the f16 1024 + v; both steps of each value are exact.
+__device__ __forceinline__ void dq6_chunk(const int c, const uint32_t qlw, const uint32_t qhw, const half2_t (&s2)[2],
+                                          const half2_t (&s1)[2], Dq6 &d) {
+    const half2_t m1024 = {(_Float16)-1024.0f, (_Float16)-1024.0f}, m1026 = {(_Float16)-1026.0f, (_Float16)-1026.0f};
+    const uint32_t sel = (c & 1) ? 0x04030402u : 0x04010400u;  // bytes (b0, b1) resp. (b2, b3) -> 0x64bb pairs
+    if (c == 0) d.nlo = qlw & 0x0F0F0F0Fu;
+    if (c == 2) d.nhi = (qlw >> 4) & 0x0F0F0F0Fu;
+    if (c == 4) d.hlo = qhw & 0x03030303u;
+    if (c == 6) d.hhi = (qhw >> 4) & 0x03030303u;
+    if (c < 4) {
+        const uint32_t v = c < 2 ? d.nlo : d.nhi;
+        d.r2[c] = (__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, v, sel)) + m1024) * s2[c >> 1];
+    } else {
+        const uint32_t v = c < 6 ? d.hlo : d.hhi;
+        d.r1[c - 4] = (__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, v, sel)) + m1026) * s1[(c - 4) >> 1];
+    }
+}
+
+template <int MB, int H>
+__device__ __forceinline__ void rw_half_q6(const uint4 *__restrict__ a_cur, uint4 *__restrict__ a_nxt,
+                                           const uint4 *__restrict__ q_cur, uint4 *__restrict__ q_nxt, uint4 *__restrict__ hb,
+                                           const uint4 *__restrict__ xs_nxt, const uint8_t *__restrict__ wq_nxt,
+                                           const uint8_t *__restrict__ wh_nxt, const LaneQ6<MB> &L, AccQ6<MB> &R) {
+    constexpr int BM = 32 * MB, kThreads = 512;
+    const int col = L.col, g = L.g;
+    if (H == 0) {
+        const uint4 sv = hb[col], dv = hb[32 + col];  // bytes 192..207 and 194..209 of the super-block
+        R.sc = u32x4{sv.x, sv.y, sv.z, sv.w};
+        R.d = dv.w >> 16;
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the header is in registers before its buffer is refilled
+        dma16(wh_nxt + L.h_off, hb);
+    }
+#pragma unroll
+    for (int i = 0; i < LaneQ6<MB>::kARounds; i++) dma16(xs_nxt + L.a_off[i], a_nxt + i * kThreads + L.wave * 64);
+    // quant pieces two half super-blocks ahead: ql bytes 64 H .., qh bytes 128 + 32 H .. of that super-block
+#pragma unroll
+    for (int r = 0; r < 2; r++) dma16(wq_nxt + 64 * H + L.ql_off[r], q_nxt + r * 64);
+    dma16(wq_nxt + 32 * H + L.qh_off, q_nxt + 128);
+    __builtin_amdgcn_sched_barrier(0);  // the copies are requested before anything else of this half
+
+    // this lane's 32 ql bytes and the 32 qh bytes of its row (pieces swizzled by the copy for conflict-free reads)
+    const int sw = (col >> 2) & 3, sw2 = (col >> 3) & 1;
+    const uint4 qa = q_cur[col * 4 + ((2 * g) ^ sw)], qb = q_cur[col * 4 + ((2 * g + 1) ^ sw)];
+    const uint4 ha = q_cur[128 + col * 2 + sw2], hc = q_cur[128 + col * 2 + (1 ^ sw2)];
+    const uint32_t qd[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+    const uint32_t hs = 2u * (uint32_t)g;
+    const uint32_t hd[8] = {ha.x >> hs, ha.y >> hs, ha.z >> hs, ha.w >> hs, hc.x >> hs, hc.y >> hs, hc.z >> hs, hc.w >> hs};
+    // scales 8 H + 2 g + t / 4 (low nibbles) and 8 H + 4 + 2 g + t / 4 (high nibbles)
+    const uint32_t wlo = (H == 0 ? R.sc.x : R.sc.z) >> (16u * (uint32_t)g), whi = (H == 0 ? R.sc.y : R.sc.w) >> (16u * (uint32_t)g);
+    half2_t s2[2][2], s1[2][2];  // [k-step / 4][low, high]
+#pragma unroll
+    for (int th = 0; th < 2; th++) {
+        const float fl = (float)(int)(int8_t)(wlo >> (8 * th)), fh = (float)(int)(int8_t)(whi >> (8 * th));
+        const _Float16 l2 = (_Float16)fl, h2 = (_Float16)fh, l1 = (_Float16)(16.0f * fl), h1 = (_Float16)(16.0f * fh);  // exact: |sc| <= 128
+        s2[th][0] = half2_t{l2, l2}, s2[th][1] = half2_t{h2, h2};
+        s1[th][0] = half2_t{l1, l1}, s1[th][1] = half2_t{h1, h1};
+    }
+
+    // software pipeline in issue order, as in the Q4_K kernel; every fragment feeds two matrix instructions
+    constexpr int kSlots = 2 * MB;
+    half8_t af[2][MB];
+    Dq6 dq;
+#pragma unroll
+    for (int i = 0; i < MB; i++) af[0][i] = __builtin_bit_cast(half8_t, a_cur[g * BM + 32 * i + col]);
+#pragma unroll
+    for (int c = 0; c < 8; c++) dq6_chunk(c, qd[0], hd[0], s2[0], s1[0], dq);
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+        const half8_t b1 = dq.b1(), b2 = dq.b2();
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int slot = 0; slot < kSlots; slot++) {
+            const int i = slot >> 1;
+            const half8_t a = af[t & 1][i];
+            if (H == 0 && t == 0 && (slot & 1) == 0) {  // first product of a super-block starts from zero
+                float16_t z;
+#pragma unroll
+                for (int r = 0; r < 16; r++) z[r] = 0.0f;
+                R.part[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b1, z, 0, 0, 0);
+            } else {
+                R.part[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, (slot & 1) ? b2 : b1, R.part[i], 0, 0, 0);
+            }
+            if (t < 7) {
+#pragma unroll
+                for (int ch = slot * 8 / kSlots; ch < (slot + 1) * 8 / kSlots; ch++)
+                    dq6_chunk(ch, qd[t + 1], hd[t + 1], s2[(t + 1) >> 2], s1[(t + 1) >> 2], dq);
+                if (slot == 0) {
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int ii = 0; ii < MB; ii++)
+                        af[(t + 1) & 1][ii] = __builtin_bit_cast(half8_t, a_cur[((t + 1) * 2 + g) * BM + 32 * ii + col]);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
+    }
+    if (H == 1) {
+        const float d = f16_bits_to_f32(R.d);
+#pragma unroll
+        for (int i = 0; i < MB; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) R.acc[i][r] = __builtin_fmaf(d, R.part[i][r], R.acc[i][r]);
+    }
+}
+
+// grid and modes as for k_qgemm_rw; 8 waves = 256 weight rows per workgroup
+template <int MB>
+__global__ __launch_bounds__(512, 1) void k_qgemm_rw_q6(const uint8_t *__restrict__ W, const uint4 *__restrict__ xs,
+                                                         const float *__restrict__ rowscale, void *__restrict__ yg,
+                                                         float *__restrict__ partial, int M, int Mp, int N, int spr, int chunk,
+                                                         int mode) {
+    constexpr int BM = 32 * MB, kThreads = 512, NW = 8;
+    extern __shared__ uint4 smem[];
+    uint4 *a0 = smem, *a1 = a0 + kQ6Groups * BM, *qbase = a1 + kQ6Groups * BM, *hb = qbase + 3 * NW * kQ6Stage;
+    const int tid = threadIdx.x;
+    LaneQ6<MB> L;
+    L.wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    L.col = lane & 31, L.g = lane >> 5;
+    const int n0 = blockIdx.x * 256, m0 = blockIdx.y * BM;
+    const int nw0 = n0 + 32 * L.wave;
+    const int sb0 = blockIdx.z * chunk;
+    const int cnt = spr - sb0 < chunk ? spr - sb0 : chunk;
+    const uint32_t row_bytes = (uint32_t)spr * kQ6Bytes;
+    auto row_off = [&](int row) {  // rows past N repeat the last
+        int n = nw0 + row;
+        n = n < N ? n : N - 1;
+        return (uint32_t)(n - n0) * row_bytes;
+    };
+#pragma unroll
+    for (int r = 0; r < 2; r++) {
+        const int row = 16 * r + (lane >> 2);
+        L.ql_off[r] = row_off(row) + 16u * (uint32_t)((lane & 3) ^ ((row >> 2) & 3));
+    }
+    {
+        const int row = lane >> 1;
+        L.qh_off = row_off(row) + 128u + 16u * (uint32_t)((lane & 1) ^ ((row >> 3) & 1));
+    }
+    L.h_off = row_off(lane & 31) + (lane < 32 ? 192u : 194u);
+#pragma unroll
+    for (int i = 0; i < LaneQ6<MB>::kARounds; i++) {
+        const int idx = tid + i * kThreads;
+        L.a_off[i] = (uint32_t)((idx / BM) * Mp + idx % BM);
+    }
+    uint4 *qa = qbase + L.wave * kQ6Stage, *qb = qa + NW * kQ6Stage, *qc = qb + NW * kQ6Stage;
+    uint4 *hw = hb + L.wave * 64;
+    const uint8_t *wblk = W + (size_t)n0 * row_bytes;
+
+    AccQ6<MB> R;
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) R.acc[i][r] = 0.0f, R.part[i][r] = 0.0f;
+
+    {
+        const uint8_t *blk = wblk + (size_t)sb0 * kQ6Bytes;
+        dma16(blk + L.h_off, hw);
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+            dma16(blk + L.ql_off[r], qa + r * 64);
+            dma16(blk + 64 + L.ql_off[r], qb + r * 64);
+        }
+        dma16(blk + L.qh_off, qa + 128);
+        dma16(blk + 32 + L.qh_off, qb + 128);
+        const uint4 *xa = xs + (size_t)(sb0 * 2 * kGroups) * Mp + m0;
+#pragma unroll
+        for (int i = 0; i < LaneQ6<MB>::kARounds; i++) dma16(xa + L.a_off[i], a0 + i * kThreads + L.wave * 64);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();
+
+    for (int s = 0; s < cnt; s++) {
+        const int sb = sb0 + s;
+        const int sbn = sb + 1 < spr ? sb + 1 : spr - 1;
+        const uint8_t *blkn = wblk + (size_t)sbn * kQ6Bytes;
+        rw_half_q6<MB, 0>(a0, a1, qa, qc, hw, xs + (size_t)((sb * 2 + 1) * kGroups) * Mp + m0, blkn, blkn, L, R);
+        barrier_keep<3>();
+        rw_half_q6<MB, 1>(a1, a0, qb, qa, hw, xs + (size_t)(sbn * 2 * kGroups) * Mp + m0, blkn, nullptr, L, R);
+        barrier_keep<3>();
+        uint4 *t = qc;
+        qc = qb, qb = qa, qa = t;
+    }
+
+    const int n = nw0 + L.col;
+    if (n >= N) return;
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int m = m0 + 32 * i + 8 * (r >> 2) + 4 * L.g + (r & 3);
+            if (m >= M) continue;
+            if (mode == 2) {
+                partial[((size_t)blockIdx.z * Mp + m) * N + n] = R.acc[i][r];
+            } else {
+                const float v = R.acc[i][r] * rowscale[m];
+                if (mode == 1) {
+                    uint32_t u = __builtin_bit_cast(uint32_t, v);
+                    u = ((u & 0x7FFFFFFFu) > 0x7F800000u) ? ((u >> 16) | 0x40u) : ((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+                    reinterpret_cast<uint16_t *>(yg)[(size_t)m * N + n] = (uint16_t)u;
+                } else {
+                    reinterpret_cast<float *>(yg)[(size_t)m * N + n] = v;
+                }
+            }
+        }
+}
+
+// y[m][n] = rowscale[m] * (partial[0][m][n] + partial[1][m][n] + ...), added in this order
+template <bool YBF16>
+__global__ __launch_bounds__(256) void k_rw_reduce(const float *__restrict__ partial, int splits, int M, int Mp, int N,
+                                                    const float *__restrict__ rowscale, void *__restrict__ yg) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)M * N) return;
+    const int m = (int)(idx / N);
+    const size_t plane = (size_t)Mp * N;
+    float s = partial[idx];
+    for (int z = 1; z < splits; z++) s += partial[(size_t)z * plane + idx];
+    const float v = s * rowscale[m];
+    if (YBF16) {
+        uint32_t u = __builtin_bit_cast(uint32_t, v);
+        u = ((u & 0x7FFFFFFFu) > 0x7F800000u) ? ((u >> 16) | 0x40u) : ((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+        reinterpret_cast<uint16_t *>(yg)[idx] = (uint16_t)u;
+    } else {
+        reinterpret_cast<float *>(yg)[idx] = v;
+    }
+}
+
+template <int MB, int NR, int NW>
+constexpr size_t rw_lds_bytes() {
+    return (size_t)(2 * kGroups * 32 * MB + NW * NR * (3 * 128 + 64)) * 16;
 }
 
 }  // namespace
 
 namespace pmh {
 
-// workspace: xs [k/8][Mp] items, xsum [k/256][4][Mp] items, rowscale [Mp] f32 (each 256-byte aligned)
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
-static int64_t padded_rows(int64_t m) { return (m + kMPad - 1) / kMPad * kMPad; }
 
-size_t qgemm_workspace_bytes(int64_t m, int64_t k) {
-    const size_t mp = (size_t)padded_rows(m);
-    return align256(mp * (size_t)k * 2) + align256(mp * (size_t)(k / 256) * 4 * 16) + align256(mp * 4);
+bool qgemm_fits(uint32_t type, int64_t m, int64_t n, int64_t k) {
+    // byte offsets inside a workgroup's rows and item offsets inside the activation copy are 32-bit
+    return (type == kTypeQ4K || type == kTypeQ6K) && m >= 1 && m <= (int64_t)1 << 22 && n >= 1 && k >= 256 && k % 256 == 0 && k <= (int64_t)1 << 22 && n <= 0x7FFFFF00;
 }
 
-template <int QT, int ORDER, bool YBF16, int WM, int WN, int NB>
-static hipError_t launch_tile(hipStream_t s, const uint8_t *w, const uint4 *xs, const uint4 *xsum, const float *rowscale,
-                              void *y, int64_t m, int64_t mp, int64_t n, int spr) {
-    using TL = Tile<QT, WM, WN, NB>;
-    auto kern = k_qgemm<QT, ORDER, YBF16, WM, WN, NB>;
-    if (TL::kLdsBytes > 64 * 1024) {
-        hipError_t a = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)TL::kLdsBytes);
+GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k) {
+    GemmPlan p;
+    p.mb = m <= 64 ? 1 : 4;  // 32 activation rows per workgroup (more workgroups along M) or 128
+    p.mp = (m + 32 * p.mb - 1) / (32 * p.mb) * (32 * p.mb);
+    p.nw = 8;
+    const int64_t spr = k / 256;
+    const int64_t rows = 32 * p.nw;
+    const int64_t base = (n + rows - 1) / rows * (p.mp / (32 * p.mb));
+    // K split: more workgroups fill more of the machine, but every split writes and re-reads an fp32 tile of Y.
+    // Estimated time = (time on a full machine) / (fraction of workgroup slots in use) + partial-tile traffic;
+    // rates as measured on MI355X (about 700 TFLOP/s of this kernel, 4 TB/s for the weight stream and for the
+    // partial tiles, 3 us for the extra launch).
+    const double slots = 256.0;  // one workgroup per compute unit keeps the weight stream busy
+    const double flops = 2.0 * (double)p.mp * (double)n * (double)k, wbytes = (double)n * (double)k * 0.5625;
+    const double t_full = flops / 7.0e14 > wbytes / 4.0e12 ? flops / 7.0e14 : wbytes / 4.0e12;
+    double best = 0.0;
+    p.splits = 1, p.chunk = (int)spr;
+    for (int64_t want = 1; want <= spr; want *= 2) {
+        const int64_t chunk = (spr + want - 1) / want, splits = (spr + chunk - 1) / chunk;
+        const double groups = (double)(base * splits);
+        const double rounds = (double)(int64_t)((groups + slots - 1) / slots);
+        const double t = t_full * rounds * slots / groups +
+                         (splits > 1 ? (double)splits * (double)m * (double)n * 8.0 / 4.0e12 + 3.0e-6 : 0.0);
+        if (want == 1 || t < best) best = t, p.splits = (int)splits, p.chunk = (int)chunk;
+    }
+    return p;
+}
+
+size_t qgemm_workspace_bytes(int64_t m, int64_t n, int64_t k) {
+    const GemmPlan p = qgemm_plan(m, n, k);
+    const size_t xs = align256((size_t)(k / 256) * 2 * kGroups * p.mp * 16);
+    const size_t part = p.splits > 1 ? align256((size_t)p.splits * p.mp * n * 4) : 0;
+    return xs + align256((size_t)p.mp * 4) + part;
+}
+
+template <int ORDER, int MB, int NR, int NW>
+static hipError_t launch_rw(hipStream_t s, const uint8_t *w, const uint4 *xs, const float *rowscale, void *y, float *partial,
+                            int64_t m, int64_t n, int spr, const GemmPlan &p, int mode) {
+    auto kern = k_qgemm_rw<ORDER, MB, NR, NW>;
+    constexpr size_t lds = rw_lds_bytes<MB, NR, NW>();
+    constexpr int kRows = 32 * NR * NW;
+    if (lds > 64 * 1024) {
+        hipError_t a = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (a != hipSuccess) return a;
     }
-    const dim3 grid((unsigned)((n + TL::BN - 1) / TL::BN), (unsigned)((m + TL::BM - 1) / TL::BM));
-    hipLaunchKernelGGL(kern, grid, dim3(TL::kThreads), TL::kLdsBytes, s, w, xs, xsum, rowscale, y, (int)m, (int)mp, (int)n, spr);
+    const dim3 grid((unsigned)((n + kRows - 1) / kRows), (unsigned)(p.mp / (32 * MB)), (unsigned)p.splits);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * NW), lds, s, w, xs, rowscale, y, partial, (int)m, (int)p.mp, (int)n, spr, p.chunk, mode);
     return hipGetLastError();
 }
 
-template <int QT, int ORDER, bool YBF16>
-static hipError_t launch_shape(hipStream_t s, const uint8_t *w, const uint4 *xs, const uint4 *xsum, const float *rowscale,
-                               void *y, int64_t m, int64_t mp, int64_t n, int spr) {
-    // tile by m: short activation batches use small tiles, so that less of the MFMA work is padding and the
-    // weight matrix spreads over enough workgroups to pull it from HBM at speed
-    if (m <= 64) return launch_tile<QT, ORDER, YBF16, 2, 1, 1>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
-    if (m <= 256) return launch_tile<QT, ORDER, YBF16, 2, 2, 2>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
-    return launch_tile<QT, ORDER, YBF16, 4, 2, 2>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
+template <int MB>
+static hipError_t launch_rw_q6(hipStream_t s, const uint8_t *w, const uint4 *xs, const float *rowscale, void *y, float *partial,
+                               int64_t m, int64_t n, int spr, const GemmPlan &p, int mode) {
+    auto kern = k_qgemm_rw_q6<MB>;
+    constexpr size_t lds = (size_t)(2 * kQ6Groups * 32 * MB + 8 * (3 * kQ6Stage + 64)) * 16;
+    hipError_t a = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (a != hipSuccess) return a;
+    const dim3 grid((unsigned)((n + 255) / 256), (unsigned)(p.mp / (32 * MB)), (unsigned)p.splits);
+    hipLaunchKernelGGL(kern, grid, dim3(512), lds, s, w, xs, rowscale, y, partial, (int)m, (int)p.mp, (int)n, spr, p.chunk, mode);
+    return hipGetLastError();
 }
 
 hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype,
-                        int64_t m, void *y, uint32_t y_dtype, uint32_t order, void *workspace, hipStream_t s) {
-    if (type != kTypeQ4K && type != kTypeQ6K) return hipErrorNotSupported;
-    if (k % 256 != 0 || m <= 0 || n <= 0) return hipErrorInvalidValue;
-    const int64_t mp = padded_rows(m);
+                                int64_t m, void *y, uint32_t y_dtype, uint32_t order, void *workspace, hipStream_t s) {
+    if (!qgemm_fits(type, m, n, k)) return hipErrorInvalidValue;
+    const GemmPlan p = qgemm_plan(m, n, k);
+    const int spr = (int)(k / 256);
     uint8_t *ws = reinterpret_cast<uint8_t *>(workspace);
     uint4 *xs = reinterpret_cast<uint4 *>(ws);
-    uint4 *xsum = reinterpret_cast<uint4 *>(ws + align256((size_t)mp * k * 2));
-    float *rowscale = reinterpret_cast<float *>(ws + align256((size_t)mp * k * 2) + align256((size_t)mp * (k / 256) * 64));
-    const dim3 pgrid((unsigned)(mp / 32), (unsigned)(k / 256));
-    if (x_dtype == kDtypeF32) {
-        hipLaunchKernelGGL(k_prep_scale<true>, dim3((unsigned)((mp + 3) / 4)), dim3(256), 0, s, x, k, (int)m, rowscale);
-        hipLaunchKernelGGL(k_prep_tiles<true>, pgrid, dim3(256), 0, s, x, k, (int)m, (int)mp, rowscale, xs, xsum);
+    const size_t xs_bytes = align256((size_t)spr * 2 * kGroups * p.mp * 16);
+    float *rowscale = reinterpret_cast<float *>(ws + xs_bytes);
+    float *partial = reinterpret_cast<float *>(ws + xs_bytes + align256((size_t)p.mp * 4));
+    const bool xf32 = x_dtype == kDtypeF32, q6 = type == kTypeQ6K, ref = order == kOrderRef;
+    const int xorder = q6 ? 2 : (ref ? 0 : 1);  // the element order the pre-pass lays the activations out for
+#define PMH_PREP(F, O) hipLaunchKernelGGL((k_prep_rw<F, O>), dim3((unsigned)p.mp), dim3(256), 0, s, x, k, (int)m, (int)p.mp, rowscale, xs)
+    if (xf32) {
+        if (xorder == 0) PMH_PREP(true, 0);
+        else if (xorder == 1) PMH_PREP(true, 1);
+        else PMH_PREP(true, 2);
     } else {
-        hipLaunchKernelGGL(k_prep_scale<false>, dim3((unsigned)((mp + 3) / 4)), dim3(256), 0, s, x, k, (int)m, rowscale);
-        hipLaunchKernelGGL(k_prep_tiles<false>, pgrid, dim3(256), 0, s, x, k, (int)m, (int)mp, rowscale, xs, xsum);
+        if (xorder == 0) PMH_PREP(false, 0);
+        else if (xorder == 1) PMH_PREP(false, 1);
+        else PMH_PREP(false, 2);
     }
+#undef PMH_PREP
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    const int spr = (int)(k / 256);
     const bool ybf = y_dtype == kDtypeBf16;
-    if (type == kTypeQ6K)  // one element order
-        return ybf ? launch_shape<14, 0, true>(s, w, xs, xsum, rowscale, y, m, mp, n, spr)
-                   : launch_shape<14, 0, false>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
-    if (order == kOrderRef)
-        return ybf ? launch_shape<12, 0, true>(s, w, xs, xsum, rowscale, y, m, mp, n, spr)
-                   : launch_shape<12, 0, false>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
-    return ybf ? launch_shape<12, 1, true>(s, w, xs, xsum, rowscale, y, m, mp, n, spr)
-               : launch_shape<12, 1, false>(s, w, xs, xsum, rowscale, y, m, mp, n, spr);
+    const int mode = p.splits > 1 ? 2 : (ybf ? 1 : 0);
+#define PMH_RW_CASE(O, B, R, NWV) launch_rw<O, B, R, NWV>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
+    if (q6) {
+        e = p.mb == 1 ? launch_rw_q6<1>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
+                      : launch_rw_q6<4>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode);
+    } else if (p.mb == 1) {
+        e = ref ? PMH_RW_CASE(0, 1, 1, 8) : PMH_RW_CASE(1, 1, 1, 8);
+    } else {
+        e = ref ? PMH_RW_CASE(0, 4, 1, 8) : PMH_RW_CASE(1, 4, 1, 8);
+    }
+#undef PMH_RW_CASE
+    if (e != hipSuccess || p.splits == 1) return e;
+    const size_t total = (size_t)m * n;
+    const dim3 rgrid((unsigned)((total + 255) / 256));
+    if (ybf) hipLaunchKernelGGL(k_rw_reduce<true>, rgrid, dim3(256), 0, s, partial, p.splits, (int)m, (int)p.mp, (int)n, rowscale, y);
+    else hipLaunchKernelGGL(k_rw_reduce<false>, rgrid, dim3(256), 0, s, partial, p.splits, (int)m, (int)p.mp, (int)n, rowscale, y);
+    return hipGetLastError();
 }
 
 }  // namespace pmh

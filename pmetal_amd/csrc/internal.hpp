@@ -34,25 +34,20 @@ bool qgemv_q4k_groupable(int64_t n, int64_t k);
 hipError_t launch_qgemv_q4k_group(const uint8_t *const *w, const int64_t *n, float *const *y, int count, int64_t k,
                                   const void *x, uint32_t x_dtype, uint32_t order, hipStream_t s);
 
-// ---- gemm.hip: dequant-fused Y = X W^T ----
-// Bytes of device workspace qgemm needs for (m, k); the caller provides it.
-size_t qgemm_workspace_bytes(int64_t m, int64_t k);
-hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype,
-                        int64_t m, void *y, uint32_t y_dtype, uint32_t order, void *workspace, hipStream_t s);
-
-// ---- gemm_rowwave.hip: Q4_K GEMM for short activation batches (every wave owns 32 weight rows) ----
-struct RowwavePlan {
-    int mb;      // 32-row activation blocks per workgroup (1, 2 or 4)
-    int nw;      // waves per workgroup (8 or 16)
+// ---- gemm.hip: dequant-fused Y = X W^T for Q4_K and Q6_K (every wave owns 32 weight rows) ----
+struct GemmPlan {
+    int mb;      // 32-row activation blocks per workgroup (1 or 4)
     int mp;      // activation rows padded to a multiple of 32 mb
+    int nw;      // waves per workgroup
     int splits;  // workgroups along K (more than one: partial tiles plus a reduction kernel)
     int chunk;   // super-blocks per split
 };
-bool qgemm_rowwave_fits(uint32_t type, int64_t m, int64_t n, int64_t k);
-RowwavePlan qgemm_rowwave_plan(int64_t m, int64_t n, int64_t k);
-size_t qgemm_rowwave_workspace_bytes(int64_t m, int64_t n, int64_t k);
-hipError_t launch_qgemm_rowwave(const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, int64_t m, void *y,
-                                uint32_t y_dtype, uint32_t order, void *workspace, hipStream_t s);
+bool qgemm_fits(uint32_t type, int64_t m, int64_t n, int64_t k);
+GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k);
+// Bytes of device workspace qgemm needs for (m, n, k); the caller provides it.
+size_t qgemm_workspace_bytes(int64_t m, int64_t n, int64_t k);
+hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype,
+                        int64_t m, void *y, uint32_t y_dtype, uint32_t order, void *workspace, hipStream_t s);
 
 // ---- util.hip ----
 hipError_t launch_fill_normal(float *dst, size_t n, uint64_t seed, float std, float outlier_rate,
