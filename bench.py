@@ -152,6 +152,13 @@ def bench_gemm(args, m, n, k, t=Q4K):
         pm.check(lib.pmetal_hip_qgemm(t, w.ptr, n, k, x.ptr, pm.DTYPE_BF16, m, y.ptr, pm.DTYPE_BF16, 0, None))
 
     ev_ms, wall_ms = timer.run(step, args.steps, args.warmup)
+    # what the matrix cores of this machine sustain in a register-only MFMA loop (no memory, no LDS) of about the
+    # same length, with operands that vary: the ceiling any kernel here works under (the published peak assumes
+    # the top clock, which a matrix loop does not hold)
+    sink = pm.DeviceBuffer(4)
+    probe_iters = 20000
+    p_ms, _ = timer.run(lambda: pm.check(lib.pmetal_hip_mfma_probe_f16(probe_iters, 1, 256, sink.ptr, None)), 3, 1)
+    sustained = 3 * 256 * 8 * probe_iters * 4 * 32768.0 / (p_ms * 1e-3) / 1e12
     flops = 2.0 * m * n * k
     us = ev_ms * 1e3 / args.steps
     tflops = flops / (us * 1e-6) / 1e12
@@ -161,7 +168,7 @@ def bench_gemm(args, m, n, k, t=Q4K):
                      "frac": round(tflops / BF16_PEAK_TFLOPS, 4), "traffic": None,
                      "kernel": ("k_qgemm_rw" if t == Q4K else "k_qgemm_rw_q6") + " (+ k_prep_rw, k_rw_reduce when K is split)",
                      "flops_per_launch": flops, "us_per_launch": round(us, 3)},
-        "extra": {},
+        "extra": {"mfma_loop_sustained_TFLOPs": round(sustained, 1), "frac_of_sustained": round(tflops / sustained, 4)},
     }, (t, n, k)
 
 

@@ -188,6 +188,16 @@ int32_t pmetal_hip_fill_normal_f32(float *dst_dev, size_t n, uint64_t seed, floa
 /* f32 -> bf16 (round to nearest even), device to device. */
 int32_t pmetal_hip_f32_to_bf16_dev(const float *src_dev, uint16_t *dst_dev, size_t n, void *stream);
 
+
+/* ---- measurement aid (no reference counterpart) ---------------------------------------
+ * Launches a register-only loop of `iters` x 4 v_mfma_f32_32x32x16_f16 per wave on `workgroups`
+ * workgroups of 8 waves (131072 flops per matrix instruction and wave; no memory traffic), so that a
+ * caller can time what the matrix cores of this machine sustain: the published peak assumes the top
+ * clock, which a long matrix loop does not hold.  vary = 0: all operands 1.0; vary = 1: operands
+ * differ per lane and change over time.  `sink_dev` is a 4-byte device buffer (never written in
+ * practice).                                                                                */
+int32_t pmetal_hip_mfma_probe_f16(int32_t iters, int32_t vary, int32_t workgroups, float *sink_dev, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -580,4 +580,14 @@ int32_t pmetal_hip_f32_to_bf16_dev(const float *src, uint16_t *dst, size_t n, vo
     return ok();
 }
 
+// ---- measurement aid ----
+int32_t pmetal_hip_mfma_probe_f16(int32_t iters, int32_t vary, int32_t workgroups, float *sink, void *stream) {
+    if (iters < 0 || workgroups < 1 || workgroups > 65536) return fail(PMETAL_HIP_ERR_INVALID_ARG, "iters >= 0, 1 <= workgroups <= 65536");
+    if (!sink) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
+    if (int32_t rc = require_device()) return rc;
+    hipError_t e = pmh::launch_mfma_probe(iters, vary != 0, workgroups, sink, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "probe kernel launch");
+    return ok();
+}
+
 }  // extern "C"

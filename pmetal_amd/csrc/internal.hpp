@@ -54,5 +54,6 @@ hipError_t launch_fill_normal(float *dst, size_t n, uint64_t seed, float std, fl
                               float outlier_mag, hipStream_t s);
 hipError_t launch_f32_to_bf16(const float *src, uint16_t *dst, size_t n, hipStream_t s);
 hipError_t launch_zero_bytes(uint8_t *dst, size_t bytes, hipStream_t s);
+hipError_t launch_mfma_probe(int iters, int vary, int workgroups, float *sink, hipStream_t s);
 
 }  // namespace pmh

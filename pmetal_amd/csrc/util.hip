@@ -1,4 +1,5 @@
-// Small utility kernels: zero fill, f32 -> bf16, synthetic normal tensors for benchmarks.
+// Small utility kernels: zero fill, f32 -> bf16, synthetic normal tensors for benchmarks, and a probe of the
+// matrix-core rate the machine sustains.
 #include "internal.hpp"
 
 namespace {
@@ -52,6 +53,34 @@ __global__ __launch_bounds__(256) void k_fill_normal(float *__restrict__ dst, si
     }
 }
 
+// Register-only loop of v_mfma_f32_32x32x16_f16: 8 waves per workgroup (two per SIMD), four independent
+// accumulators per wave, no memory traffic.  With `vary` the operands differ per lane and one of them changes sign
+// every trip (one extra VALU instruction per four matrix instructions); without it they are all 1.0.
+typedef _Float16 probe_half8 __attribute__((ext_vector_type(8)));
+typedef float probe_float16 __attribute__((ext_vector_type(16)));
+__global__ __launch_bounds__(512) void k_mfma_probe(int iters, int vary, float *__restrict__ sink) {
+    probe_half8 a, b;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        a[i] = (_Float16)(vary ? (float)((threadIdx.x * 37 + i * 11) % 97) * 0.37f - 17.0f : 1.0f);
+        b[i] = (_Float16)(vary ? (float)((threadIdx.x * 13 + i * 7) % 89) * 0.21f - 9.0f : 1.0f);
+    }
+    probe_float16 c0, c1, c2, c3;
+#pragma unroll
+    for (int i = 0; i < 16; i++) c0[i] = 0.0f, c1[i] = 0.0f, c2[i] = 0.0f, c3[i] = 0.0f;
+    for (int i = 0; i < iters; i++) {
+        c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c0, 0, 0, 0);
+        c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c1, 0, 0, 0);
+        c2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c2, 0, 0, 0);
+        c3 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c3, 0, 0, 0);
+        if (vary) a[i & 7] = -a[i & 7];
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) s += c0[i] + c1[i] + c2[i] + c3[i];
+    if (s == 1.2345f) sink[0] = s;  // keeps the loop alive; practically never true
+}
+
 inline unsigned capped_grid(size_t items) {
     size_t g = (items + 255) / 256;
     return (unsigned)(g < 1 ? 1 : (g > 65536 ? 65536 : g));
@@ -78,6 +107,11 @@ hipError_t launch_fill_normal(float *dst, size_t n, uint64_t seed, float std, fl
     if (n == 0) return hipSuccess;
     hipLaunchKernelGGL(k_fill_normal, dim3(capped_grid((n + 1) / 2)), dim3(256), 0, s, dst, n, seed, std,
                        outlier_rate, outlier_mag);
+    return hipGetLastError();
+}
+
+hipError_t launch_mfma_probe(int iters, int vary, int workgroups, float *sink, hipStream_t s) {
+    hipLaunchKernelGGL(k_mfma_probe, dim3((unsigned)workgroups), dim3(512), 0, s, iters, vary, sink);
     return hipGetLastError();
 }
 
