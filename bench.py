@@ -108,6 +108,63 @@ def cpu_baseline_gemv(t, n, k, budget_s=12.0):
             "sample": f"{reps} x (dequantize + f32 matvec) of {rows}x{k} rows of the same shape, {dt:.1f} s"}
 
 
+def cpu_baseline_quantize(budget_s=12.0):
+    """Oracle: the reference's quantizers, one thread, on f32 tensors in the model's Q4_K : Q6_K element ratio."""
+    from oracle import binding as oracle
+    oracle.build()
+    rng = np.random.default_rng(6)
+    x4 = (rng.standard_normal(3 << 18) * 0.02).astype(np.float32)   # 786432 elements to Q4_K
+    x6 = (rng.standard_normal(1 << 18) * 0.02).astype(np.float32)   # 262144 elements to Q6_K (the recipe's 26 %)
+    oracle.quantize(Q4K, x4[:4096]), oracle.quantize(Q6K, x6[:4096])
+    reps, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < budget_s:
+        oracle.quantize(Q4K, x4)
+        oracle.quantize(Q6K, x6)
+        reps += 1
+    dt = time.perf_counter() - t0
+    return {"value": round(4.0 * (x4.size + x6.size) * reps / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{reps} x (786432 elements to Q4_K + 262144 to Q6_K), {dt:.1f} s"}
+
+
+def cpu_baseline_gemm(t, m, n, k, budget_s=12.0):
+    """Oracle: reference dequantize + f32 matmul (row by row, sequential dot products), one thread, on a slice."""
+    from oracle import binding as oracle
+    oracle.build()
+    rows, mm = min(n, 256), min(m, 64)
+    rng = np.random.default_rng(7)
+    wq = oracle.quantize(t, (rng.standard_normal(rows * k) * 0.02).astype(np.float32))
+    x = oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(rng.standard_normal(mm * k).astype(np.float32))).reshape(mm, k)
+    oracle.qmatmul(t, wq, rows, k, x[:1])
+    reps, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < budget_s:
+        oracle.qmatmul(t, wq, rows, k, x)
+        reps += 1
+    dt = time.perf_counter() - t0
+    return {"value": round(2.0 * mm * rows * k * reps / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": f"{reps} x (dequantize + matmul) of {mm} x {rows} x {k}, {dt:.1f} s"}
+
+
+def cpu_baseline_decode(pm, budget_s=15.0):
+    """Oracle: dequantize + f32 matvec, one thread, over the projections of the first two layers of the stack."""
+    from oracle import binding as oracle
+    oracle.build()
+    lins = [l for l in qwen3_06b_linears(pm) if l[0].startswith(("blk.0.", "blk.1."))]
+    rng = np.random.default_rng(8)
+    ws = [(t, oracle.quantize(t, (rng.standard_normal(n * k) * 0.02).astype(np.float32)), n, k) for _, n, k, t in lins]
+    xs = {k: oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(rng.standard_normal(k).astype(np.float32))) for k in (1024, 2048, 3072)}
+    reps, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < budget_s:
+        for t, wq, n, k in ws:
+            oracle.qmatvec(t, wq, n, k, xs[k], acc="f32")
+        reps += 1
+    dt = time.perf_counter() - t0
+    sample_bytes = sum(gemv_bytes(t, n, k, 2) for t, _, n, k in ws)
+    total_bytes = sum(gemv_bytes(t, n, k, 2) for _, n, k, t in qwen3_06b_linears(pm))
+    return {"value": round(reps / dt * sample_bytes / total_bytes, 4), "unit": "tokens/s", "cores": 1, "kind": "port",
+            "sample": f"{reps} x the 14 projections of layers 0-1 ({sample_bytes} of {total_bytes} weight bytes per token), "
+                      f"scaled by bytes, {dt:.1f} s"}
+
+
 def bench_gemv(args, n, k, t=Q4K, copies=16):
     pm, _lib, lib = load()
     timer = Timer(pm, lib)
@@ -339,8 +396,15 @@ def main():
         for _ in range(5):
             pm.check(lib.pmetal_hip_f32_to_bf16_dev(src.ptr, dst.ptr, n_cal, None))
         pm.check(lib.pmetal_hip_sync(None))
-    if not args.no_cpu_baseline and wl["kind"] == "gemv":
-        out["cpu_baseline"] = cpu_baseline_gemv(t, n, k)
+    if not args.no_cpu_baseline:
+        if wl["kind"] == "gemv":
+            out["cpu_baseline"] = cpu_baseline_gemv(t, n, k)
+        elif wl["kind"] == "quantize":
+            out["cpu_baseline"] = cpu_baseline_quantize()
+        elif wl["kind"] == "gemm":
+            out["cpu_baseline"] = cpu_baseline_gemm(wl["type"], wl["m"], wl["n"], wl["k"])
+        else:
+            out["cpu_baseline"] = cpu_baseline_decode(load()[0])
     print(json.dumps(out), flush=True)
 
 
