@@ -126,6 +126,21 @@ def cpu_baseline_quantize(budget_s=12.0):
             "sample": f"{reps} x (786432 elements to Q4_K + 262144 to Q6_K), {dt:.1f} s"}
 
 
+def cpu_baseline_dequantize(budget_s=10.0):
+    """Oracle: the reference's dequantize_q4k, one thread."""
+    from oracle import binding as oracle
+    oracle.build()
+    n = 1 << 22
+    wq = oracle.quantize(Q4K, (np.random.default_rng(9).standard_normal(n) * 0.02).astype(np.float32))
+    reps, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < budget_s:
+        oracle.dequantize(Q4K, wq, [n])
+        reps += 1
+    dt = time.perf_counter() - t0
+    return {"value": round((wq.size + 4.0 * n) * reps / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{reps} x dequantize of {n} Q4_K elements, {dt:.1f} s"}
+
+
 def cpu_baseline_gemm(t, m, n, k, budget_s=12.0):
     """Oracle: reference dequantize + f32 matmul (row by row, sequential dot products), one thread, on a slice."""
     from oracle import binding as oracle
@@ -227,6 +242,37 @@ def bench_gemm(args, m, n, k, t=Q4K):
                      "flops_per_launch": flops, "us_per_launch": round(us, 3)},
         "extra": {"mfma_loop_sustained_TFLOPs": round(sustained, 1), "frac_of_sustained": round(tflops / sustained, 4)},
     }, (t, n, k)
+
+
+def bench_dequantize(args, n, k):
+    """Blocks -> f32 of one 14336 x 4096 tensor per type; rotating over enough tensors to stay out of the last-level cache."""
+    pm, _lib, lib = load()
+    timer = Timer(pm, lib)
+    out = {}
+    for t, name, copies in ((Q4K, "q4k", 2), (Q6K, "q6k", 2), (Q8_0, "q8_0", 2)):
+        ws = [device_weights(pm, lib, t, n * k, 4000 + i) for i in range(copies)]
+        ys = [pm.DeviceBuffer(4 * n * k) for _ in range(copies)]
+        nbytes = lib.pmetal_hip_tensor_size(t, n * k)
+
+        def step():
+            for w, y in zip(ws, ys):
+                pm.check(lib.pmetal_hip_dequantize_dev(t, w.ptr, nbytes, y.ptr, n * k, 0, None), "dequantize")
+
+        ev_ms, wall_ms = timer.run(step, args.steps, args.warmup)
+        us = ev_ms * 1e3 / (args.steps * copies)
+        out[name] = {"us_per_launch": round(us, 2), "GBps": round((nbytes + 4.0 * n * k) / (us * 1e-6) / 1e9, 1),
+                     "bytes_per_launch": nbytes + 4 * n * k, "wall_ms_per_step": wall_ms / args.steps, "ev_ms_per_step": ev_ms / args.steps}
+        for b in ws + ys:
+            b.free()
+    q = out["q4k"]
+    return {
+        "value": q["GBps"], "ms_per_step": q["wall_ms_per_step"], "event_ms_per_step": q["ev_ms_per_step"],
+        "roofline": {"bound": "hbm", "achieved": q["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(q["GBps"] / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "k_dequantize_q4k",
+                     "bytes_per_launch": q["bytes_per_launch"], "us_per_launch": q["us_per_launch"]},
+        "extra": {"q6k": {k2: out["q6k"][k2] for k2 in ("us_per_launch", "GBps")},
+                  "q8_0": {k2: out["q8_0"][k2] for k2 in ("us_per_launch", "GBps")}},
+    }, (Q4K, n, k)
 
 
 def qwen3_06b_linears(pm):
@@ -344,6 +390,8 @@ WORKLOADS["decode_qwen3_0.6b_q4km"] = dict(kind="decode", metric="Q4_K_M decode 
                                            dtype="bf16")
 WORKLOADS["quantize_llama3_8b_q4km"] = dict(kind="quantize", metric="f32->Q4_K_M quantize GB/s of f32 consumed (Llama-3-8B shape)",
                                             unit="GB/s", dtype="f32")
+WORKLOADS["dequantize_14336x4096"] = dict(kind="dequantize", n=14336, k=4096, unit="GB/s", dtype="f32",
+                                          metric="Q4_K dequantize GB/s (blocks read + f32 written) @14336x4096")
 for _m in (16, 64, 128, 512, 2048):
     WORKLOADS[f"gemm_q4k_m{_m}"] = dict(kind="gemm", m=_m, n=14336, k=4096, metric=f"Q4_K GEMM TFLOPS @M={_m},K=4096,N=14336",
                                         unit="TFLOP/s", dtype="f16", type=Q4K)
@@ -371,6 +419,8 @@ def main():
         res, (t, n, k) = bench_decode(args)
     elif wl["kind"] == "quantize":
         res, (t, n, k) = bench_quantize(args)
+    elif wl["kind"] == "dequantize":
+        res, (t, n, k) = bench_dequantize(args, wl["n"], wl["k"])
     else:
         res, (t, n, k) = bench_gemv(args, wl["n"], wl["k"])
     out = {
@@ -383,6 +433,7 @@ def main():
                    "step": {"gemm": "one GEMM launch (activation pre-pass + MFMA kernel)",
                             "gemv": "16 back-to-back GEMVs over 16 distinct weight tensors (528 MB, HBM-resident)",
                             "decode": "all 197 batch-1 projections of one token, back to back on one stream",
+                            "dequantize": "two tensors of 14336 x 4096, blocks resident in HBM",
                             "quantize": "all 226 tensors of the model, f32 resident in HBM"}[wl["kind"]]},
         "roofline": res["roofline"], "extra": res["extra"],
     }
@@ -403,6 +454,8 @@ def main():
             out["cpu_baseline"] = cpu_baseline_quantize()
         elif wl["kind"] == "gemm":
             out["cpu_baseline"] = cpu_baseline_gemm(wl["type"], wl["m"], wl["n"], wl["k"])
+        elif wl["kind"] == "dequantize":
+            out["cpu_baseline"] = cpu_baseline_dequantize()
         else:
             out["cpu_baseline"] = cpu_baseline_decode(load()[0])
     print(json.dumps(out), flush=True)

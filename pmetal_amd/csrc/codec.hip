@@ -136,18 +136,19 @@ __device__ __forceinline__ void scale_min_k4(int j, uint32_t s0, uint32_t s1, ui
 }
 
 // -------------------------------------------------------------------------------------------
-// Q4_K dequantize (k_quants.rs:358-404 + :515-560).  One lane per 4 outputs, one wave per
-// super-block; out = (d*sc) * nibble - (dmin*m), each operation rounded.
+// Q4_K dequantize (k_quants.rs:358-404 + :515-560).  One lane per 4 outputs of a super-block; a wave
+// handles kDeqUnroll consecutive super-blocks and requests the bytes of all of them before it computes, so
+// that a wave has several kilobytes of output per memory round trip.  out = (d*sc) * nibble - (dmin*m),
+// each operation rounded.
 // ORDER 0: the reference's emission order; ORDER 1: inverse of the quantizer's packing.
 // -------------------------------------------------------------------------------------------
+constexpr int kDeqUnroll = 4;
+
 template <int ORDER>
 __global__ __launch_bounds__(256) void k_dequantize_q4k(const uint8_t *__restrict__ src, size_t n,
                                                          float *__restrict__ dst) {
-    const size_t tid = (size_t)blockIdx.x * 256 + threadIdx.x;
-    const size_t e = tid * 4;
-    if (e >= n) return;
-    const uint8_t *blk = src + (tid >> 6) * 144;
-    const int i = (int)(tid & 63);
+    const size_t wave = ((size_t)blockIdx.x * 256 + threadIdx.x) >> 6;
+    const int i = (int)(threadIdx.x & 63);
     const int c = i >> 4;       // 64-element chunk
     const int p = (i & 15) * 4; // position inside the chunk
     int byte, hi, sb;
@@ -160,54 +161,78 @@ __global__ __launch_bounds__(256) void k_dequantize_q4k(const uint8_t *__restric
         hi = p >> 5;
         sb = 2 * c + (p >> 5);
     }
-    const uint4 hdr = *reinterpret_cast<const uint4 *>(blk);
-    const float d = f16_bits_to_f32(hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(hdr.x >> 16);
-    uint32_t sc, m;
-    scale_min_k4(sb, hdr.y, hdr.z, hdr.w, sc, m);
-    const float d1 = d * (float)sc;
-    const float dm1 = dmin * (float)m;
-    uint32_t q = *reinterpret_cast<const uint32_t *>(blk + 16 + byte);
-    q = hi ? (q >> 4) : q;
-    float o[4];
+    uint4 hdr[kDeqUnroll];
+    uint32_t q[kDeqUnroll];
 #pragma unroll
-    for (int t = 0; t < 4; t++) o[t] = d1 * (float)((q >> (8 * t)) & 0xFu) - dm1;
-    if (e + 3 < n) {
-        *reinterpret_cast<float4 *>(dst + e) = make_float4(o[0], o[1], o[2], o[3]);
-    } else {
-        for (int t = 0; t < 4 && e + t < n; t++) dst[e + t] = o[t];
+    for (int u = 0; u < kDeqUnroll; u++) {
+        const size_t blk_i = wave * kDeqUnroll + u;
+        const bool live = blk_i * 256 + (size_t)i * 4 < n;
+        const uint8_t *blk = src + (live ? blk_i : 0) * 144;  // lanes past the end re-read the first block
+        hdr[u] = *reinterpret_cast<const uint4 *>(blk);
+        q[u] = *reinterpret_cast<const uint32_t *>(blk + 16 + byte);
+    }
+#pragma unroll
+    for (int u = 0; u < kDeqUnroll; u++) {
+        const size_t e = (wave * kDeqUnroll + u) * 256 + (size_t)i * 4;
+        if (e >= n) continue;
+        const float d = f16_bits_to_f32(hdr[u].x & 0xFFFFu), dmin = f16_bits_to_f32(hdr[u].x >> 16);
+        uint32_t sc, m;
+        scale_min_k4(sb, hdr[u].y, hdr[u].z, hdr[u].w, sc, m);
+        const float d1 = d * (float)sc;
+        const float dm1 = dmin * (float)m;
+        const uint32_t qq = hi ? (q[u] >> 4) : q[u];
+        float o[4];
+#pragma unroll
+        for (int t = 0; t < 4; t++) o[t] = d1 * (float)((qq >> (8 * t)) & 0xFu) - dm1;
+        if (e + 3 < n) {
+            *reinterpret_cast<float4 *>(dst + e) = make_float4(o[0], o[1], o[2], o[3]);
+        } else {
+            for (int t = 0; t < 4 && e + t < n; t++) dst[e + t] = o[t];
+        }
     }
 }
 
 // -------------------------------------------------------------------------------------------
-// Q6_K dequantize (k_quants.rs:474-496 + :614-660): out = (d * sc) * q, left-associated.
+// Q6_K dequantize (k_quants.rs:474-496 + :614-660): out = (d * sc) * q, left-associated.  Same launch shape.
 // -------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void k_dequantize_q6k(const uint8_t *__restrict__ src, size_t n,
                                                          float *__restrict__ dst) {
-    const size_t tid = (size_t)blockIdx.x * 256 + threadIdx.x;
-    const size_t e = tid * 4;
-    if (e >= n) return;
-    const uint8_t *blk = src + (tid >> 6) * 210;
-    const int i = (int)(tid & 63);
+    const size_t wave = ((size_t)blockIdx.x * 256 + threadIdx.x) >> 6;
+    const int i = (int)(threadIdx.x & 63);
     const int h = i >> 5;         // 128-element half
     const int g = (i >> 3) & 3;   // 32-element group inside the half
     const int l = (i & 7) * 4;    // 0..28
-    const uint32_t qlw = *reinterpret_cast<const u32_a2 *>(blk + 64 * h + 32 * (g & 1) + l);
-    const uint32_t qhw = *reinterpret_cast<const u32_a2 *>(blk + 128 + 32 * h + l);
-    const float sc = (float)(int8_t)blk[192 + 8 * h + 2 * g + (l >> 4)];
-    const float d = f16_bits_to_f32(*reinterpret_cast<const uint16_t *>(blk + 208));
-    const float dsc = d * sc;
-    const uint32_t nib = (g >= 2) ? (qlw >> 4) : qlw;
-    const uint32_t hi2 = qhw >> (2 * g);
-    float o[4];
+    uint32_t qlw[kDeqUnroll], qhw[kDeqUnroll];
+    int scb[kDeqUnroll];
+    uint32_t dh[kDeqUnroll];
 #pragma unroll
-    for (int t = 0; t < 4; t++) {
-        int q = (int)(((nib >> (8 * t)) & 0xFu) | (((hi2 >> (8 * t)) & 3u) << 4)) - 32;
-        o[t] = dsc * (float)q;
+    for (int u = 0; u < kDeqUnroll; u++) {
+        const size_t blk_i = wave * kDeqUnroll + u;
+        const bool live = blk_i * 256 + (size_t)i * 4 < n;
+        const uint8_t *blk = src + (live ? blk_i : 0) * 210;  // lanes past the end re-read the first block
+        qlw[u] = *reinterpret_cast<const u32_a2 *>(blk + 64 * h + 32 * (g & 1) + l);
+        qhw[u] = *reinterpret_cast<const u32_a2 *>(blk + 128 + 32 * h + l);
+        scb[u] = (int)(int8_t)blk[192 + 8 * h + 2 * g + (l >> 4)];
+        dh[u] = *reinterpret_cast<const uint16_t *>(blk + 208);
     }
-    if (e + 3 < n) {
-        *reinterpret_cast<float4 *>(dst + e) = make_float4(o[0], o[1], o[2], o[3]);
-    } else {
-        for (int t = 0; t < 4 && e + t < n; t++) dst[e + t] = o[t];
+#pragma unroll
+    for (int u = 0; u < kDeqUnroll; u++) {
+        const size_t e = (wave * kDeqUnroll + u) * 256 + (size_t)i * 4;
+        if (e >= n) continue;
+        const float dsc = f16_bits_to_f32(dh[u]) * (float)scb[u];
+        const uint32_t nib = (g >= 2) ? (qlw[u] >> 4) : qlw[u];
+        const uint32_t hi2 = qhw[u] >> (2 * g);
+        float o[4];
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            int q = (int)(((nib >> (8 * t)) & 0xFu) | (((hi2 >> (8 * t)) & 3u) << 4)) - 32;
+            o[t] = dsc * (float)q;
+        }
+        if (e + 3 < n) {
+            *reinterpret_cast<float4 *>(dst + e) = make_float4(o[0], o[1], o[2], o[3]);
+        } else {
+            for (int t = 0; t < 4 && e + t < n; t++) dst[e + t] = o[t];
+        }
     }
 }
 
@@ -597,7 +622,7 @@ hipError_t launch_dequantize_q8_0(const uint8_t *src, size_t n, float *dst, hipS
 
 hipError_t launch_dequantize_q4k(const uint8_t *src, size_t n, float *dst, uint32_t order, hipStream_t s) {
     if (n == 0) return hipSuccess;
-    const dim3 grid(grid_for((n + 3) / 4, 256));
+    const dim3 grid(grid_for((n + 4 * kDeqUnroll - 1) / (4 * kDeqUnroll), 256));  // one lane per 4 outputs of kDeqUnroll super-blocks
     if (order == kOrderRef) hipLaunchKernelGGL(k_dequantize_q4k<0>, grid, dim3(256), 0, s, src, n, dst);
     else hipLaunchKernelGGL(k_dequantize_q4k<1>, grid, dim3(256), 0, s, src, n, dst);
     return hipGetLastError();
@@ -605,7 +630,7 @@ hipError_t launch_dequantize_q4k(const uint8_t *src, size_t n, float *dst, uint3
 
 hipError_t launch_dequantize_q6k(const uint8_t *src, size_t n, float *dst, hipStream_t s) {
     if (n == 0) return hipSuccess;
-    hipLaunchKernelGGL(k_dequantize_q6k, dim3(grid_for((n + 3) / 4, 256)), dim3(256), 0, s, src, n, dst);
+    hipLaunchKernelGGL(k_dequantize_q6k, dim3(grid_for((n + 4 * kDeqUnroll - 1) / (4 * kDeqUnroll), 256)), dim3(256), 0, s, src, n, dst);
     return hipGetLastError();
 }
 
