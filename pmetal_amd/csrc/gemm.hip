@@ -270,6 +270,8 @@ __device__ __forceinline__ void rw_half(const uint4 *__restrict__ a_cur, uint4 *
 #pragma unroll
     for (int i = 0; i < Lane<MB, NR, NW>::kARounds; i++)
         if (i * kThreads + L.wave * 64 < kGroups * BM) dma16(xs_nxt + L.a_off[i], a_nxt + i * kThreads + L.wave * 64);
+    // the quant copies must be the newest requests of this half: the barrier at its end waits for all but them
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int rg = 0; rg < NR; rg++)
 #pragma unroll
@@ -569,6 +571,7 @@ __device__ __forceinline__ void rw_half_q6(const uint4 *__restrict__ a_cur, uint
     }
 #pragma unroll
     for (int i = 0; i < LaneQ6<MB>::kARounds; i++) dma16(xs_nxt + L.a_off[i], a_nxt + i * kThreads + L.wave * 64);
+    __builtin_amdgcn_sched_barrier(0);  // the three quant copies stay the newest requests (see barrier_keep)
     // quant pieces two half super-blocks ahead: ql bytes 64 H .., qh bytes 128 + 32 H .. of that super-block
 #pragma unroll
     for (int r = 0; r < 2; r++) dma16(wq_nxt + 64 * H + L.ql_off[r], q_nxt + r * 64);
