@@ -153,8 +153,8 @@ int32_t pmetal_hip_qgemv(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, in
 int32_t pmetal_hip_qgemm(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, int64_t k, const void *x_dev,
                          uint32_t x_dtype, int64_t m, void *y_dev, uint32_t y_dtype, uint32_t order,
                          void *stream);
-/* Dispatch by m: m == 1 -> qgemv (f32 output only), otherwise qgemm (Q4_K, Q6_K).  Q8_0 has a GEMV but no GEMM
- * and runs one GEMV per activation row when m > 1 (f32 output only). */
+/* Dispatch by m: m == 1 -> qgemv (f32 output only), otherwise qgemm (k must be a multiple of 256).  A Q8_0
+ * row that is only a multiple of 32 runs one GEMV per activation row when m > 1 (f32 output only). */
 int32_t pmetal_hip_qlinear(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, int64_t k, const void *x_dev,
                            uint32_t x_dtype, int64_t m, void *y_dev, uint32_t y_dtype, uint32_t order,
                            void *stream);

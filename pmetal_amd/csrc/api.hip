@@ -478,7 +478,7 @@ int32_t pmetal_hip_qgemm(uint32_t t, const uint8_t *w, int64_t n, int64_t k, con
     if (int32_t rc = check_linear(t, w, n, k, x, x_dtype, y, order)) return rc;
     if (y_dtype > PMETAL_HIP_DTYPE_BF16) return fail(PMETAL_HIP_ERR_INVALID_ARG, "y_dtype must be 0 (f32) or 1 (bf16)");
     if (m <= 0 || m > 0x7FFFFFFF) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "m must be in [1, 2^31)");
-    if (t == PMETAL_GGML_TYPE_Q8_0) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "qgemm supports Q4_K and Q6_K weights");
+    if (k % 256 != 0) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qgemm: k=%lld is not a multiple of 256", (long long)k);
     if (!pmh::qgemm_fits(t, m, n, k))
         return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qgemm: m and k must be at most 2^22 (m = %lld, k = %lld)", (long long)m, (long long)k);
     void *ws = nullptr;
@@ -493,8 +493,9 @@ int32_t pmetal_hip_qlinear(uint32_t t, const uint8_t *w, int64_t n, int64_t k, c
                            void *y, uint32_t y_dtype, uint32_t order, void *stream) {
     if (m == 1 && y_dtype == PMETAL_HIP_DTYPE_F32)
         return pmetal_hip_qgemv(t, w, n, k, x, x_dtype, (float *)y, order, stream);
-    if (t == PMETAL_GGML_TYPE_Q8_0 && y_dtype == PMETAL_HIP_DTYPE_F32 && m > 1 && n > 0 && k > 0 && x && y) {
-        // No fused GEMM for Q8_0: one fused GEMV per activation row, back to back on the stream.
+    if (t == PMETAL_GGML_TYPE_Q8_0 && k % 256 != 0 && y_dtype == PMETAL_HIP_DTYPE_F32 && m > 1 && n > 0 && k > 0 && x && y) {
+        // The fused GEMM walks k in steps of 256; a Q8_0 row may be any multiple of 32: one fused GEMV per
+        // activation row then, back to back on the stream.
         const size_t x_row = (size_t)k * (x_dtype == PMETAL_HIP_DTYPE_F32 ? 4 : 2);
         for (int64_t r = 0; r < m; r++) {
             const int32_t rc = pmetal_hip_qgemv(t, w, n, k, (const uint8_t *)x + (size_t)r * x_row, x_dtype,

@@ -1,5 +1,6 @@
-// Dequant-fused Q4_K and Q6_K GEMM  Y[m,n] = sum_k X[m,k] * W[n,k]  on the gfx950 matrix cores, every wave owning
-// its weight rows.  The text below describes Q4_K; the Q6_K kernel further down notes its differences.
+// Dequant-fused Q4_K, Q6_K and Q8_0 GEMM  Y[m,n] = sum_k X[m,k] * W[n,k]  on the gfx950 matrix cores, every wave
+// owning its weight rows.  The text below describes Q4_K; the Q6_K and Q8_0 kernels further down note their
+// differences.
 //
 // W is the packed GGUF stream [n, k] of 144-byte super-blocks; a weight's value is what the reference's
 // dequantize_q4k yields (crates/pmetal-gguf/src/k_quants.rs:358-404; element order REF or GGML as for the
@@ -75,7 +76,8 @@ __device__ __forceinline__ float bf16_to_f32(uint32_t h) { return __builtin_bit_
 // Pre-pass: one workgroup per activation row m < Mp.  rowscale[m] = 2^e with the row maximum * 2^-e in
 // [2^9, 2^10) (bf16 activations are then exact in f16 and block sums stay below 2^15); rows >= M are zero.
 // One thread per operand item: chunk u = 64 elements = sub-blocks 2u, 2u+1 (u = 4 sb + 2 h + g), k-step t.
-// ORDER 0 / 1: Q4_K element orders REF / GGML; ORDER 2: the Q6_K layout (no block sums).
+// ORDER 0 / 1: Q4_K element orders REF / GGML; ORDER 2: the Q6_K layout, ORDER 3: the natural order (Q8_0), both
+// without block sums.
 // ------------------------------------------------------------------------------------------------
 template <bool XF32, int ORDER>
 __global__ __launch_bounds__(256) void k_prep_rw(const void *__restrict__ xg, int64_t k, int M, int Mp,
@@ -120,11 +122,16 @@ __global__ __launch_bounds__(256) void k_prep_rw(const void *__restrict__ xg, in
         // the item's two runs of four elements (lo, hi), its half super-block and its operand group
         int64_t lo, hi, half;
         int t, g;
-        if (ORDER == 2) {  // Q6_K: half = 128 elements; low nibbles at 32 g + 4 t, high nibbles 64 further
+        if (ORDER >= 2) {  // half = 128 elements, 16 items
             half = q >> 4;
             t = (int)(q & 15) >> 1, g = (int)q & 1;
-            lo = 128 * half + 32 * g + 4 * t;
-            hi = lo + 64;
+            if (ORDER == 2) {  // Q6_K: low nibbles at 32 g + 4 t, high nibbles 64 further
+                lo = 128 * half + 32 * g + 4 * t;
+                hi = lo + 64;
+            } else {  // Q8_0: the natural order, 8 consecutive elements
+                lo = 128 * half + 16 * t + 8 * g;
+                hi = lo + 4;
+            }
         } else {
             const int64_t u = q >> 3;
             t = (int)(q & 7), g = (int)u & 1;
@@ -156,7 +163,7 @@ __global__ __launch_bounds__(256) void k_prep_rw(const void *__restrict__ xg, in
         }
         const size_t base = (size_t)(half * kGroups) * Mp + m;
         xs[base + (size_t)(t * 2 + g) * Mp] = __builtin_bit_cast(uint4, h);
-        if (ORDER == 2) continue;  // Q6_K has no min term: no block sums
+        if (ORDER >= 2) continue;  // Q6_K and Q8_0 have no min term: no block sums
         // sums of the two sub-blocks of the chunk over its 8 k-steps (8 consecutive lanes)
         float s0, s1;
         if (ORDER == 0) {  // sub-block 2u: k-steps 0..3 (low and high nibbles), 2u+1: k-steps 4..7
@@ -744,6 +751,174 @@ __global__ __launch_bounds__(512, 1) void k_qgemm_rw_q6(const uint8_t *__restric
         }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Q8_0 (crates/pmetal-gguf/src/quantize.rs:268-300: 34-byte blocks of 32: f16 d, 32 int8; value d * q).  The int8
+// quants are exact in f16, so the B tile is q itself and d, one per 32 elements, multiplies the fp32 partial
+// sum of two k-steps.  That is 16 fp32 FMAs per matrix instruction pair and output block: this kernel is bound
+// by its VALU work, not by the matrix pipe.  A block is 34 bytes, so nothing in a row is aligned to more than
+// 2 bytes: every lane (row n, half g) loads its own 8 quants per k-step and the scales straight from global
+// memory into registers, one half super-block (four blocks) ahead; the activations go through LDS as in the
+// kernels above (natural element order).
+// ------------------------------------------------------------------------------------------------
+struct __attribute__((packed, aligned(2))) q8_u32x2 {
+    uint32_t x, y;
+};
+typedef uint16_t q8_u16 __attribute__((aligned(2)));
+
+struct Q8Half {       // one lane's share of four blocks
+    uint32_t q[4][2][2];  // [block][k-step of the block][dword]
+    uint32_t d[4];        // f16 bits
+};
+
+__device__ __forceinline__ void q8_load(const uint8_t *p, const int g, Q8Half &h) {  // p: the lane's row at the half
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+        h.d[b] = *reinterpret_cast<const q8_u16 *>(p + 34 * b);
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++) {
+            const q8_u32x2 v = *reinterpret_cast<const q8_u32x2 *>(p + 34 * b + 2 + 16 * tt + 8 * g);
+            h.q[b][tt][0] = v.x, h.q[b][tt][1] = v.y;
+        }
+    }
+}
+
+// 8 int8 -> 8 exact f16: q + 128 as an unsigned byte b, 0x6400 | b is the f16 1024 + b, minus 1152.
+__device__ __forceinline__ half8_t q8_operand(const uint32_t w0, const uint32_t w1) {
+    const half2_t m1152 = {(_Float16)-1152.0f, (_Float16)-1152.0f};
+    const uint32_t u0 = w0 ^ 0x80808080u, u1 = w1 ^ 0x80808080u;
+    const half2_t r0 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u0, 0x04010400u)) + m1152;
+    const half2_t r1 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u0, 0x04030402u)) + m1152;
+    const half2_t r2 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u1, 0x04010400u)) + m1152;
+    const half2_t r3 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, u1, 0x04030402u)) + m1152;
+    return half8_t{r0[0], r0[1], r1[0], r1[1], r2[0], r2[1], r3[0], r3[1]};
+}
+
+template <int MB>
+__device__ __forceinline__ void rw_half_q8(const uint4 *__restrict__ a_cur, uint4 *__restrict__ a_nxt,
+                                           const uint4 *__restrict__ xs_nxt, const uint8_t *w_nxt, const Q8Half &cur,
+                                           Q8Half &nxt, const LaneQ6<MB> &L, float16_t (&acc)[MB]) {
+    constexpr int BM = 32 * MB, kThreads = 512;
+    const int col = L.col, g = L.g;
+    // `cur` was requested a whole half super-block ago and is the only thing still outstanding; waiting for it
+    // here, before the new requests go out, keeps that wait from covering them too
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+#pragma unroll
+    for (int i = 0; i < LaneQ6<MB>::kARounds; i++) dma16(xs_nxt + L.a_off[i], a_nxt + i * kThreads + L.wave * 64);
+    __builtin_amdgcn_sched_barrier(0);  // the 12 register loads below stay the newest requests (see barrier_keep)
+    q8_load(w_nxt, g, nxt);
+    __builtin_amdgcn_sched_barrier(0);
+
+    half8_t af[2][MB];
+#pragma unroll
+    for (int i = 0; i < MB; i++) af[0][i] = __builtin_bit_cast(half8_t, a_cur[g * BM + 32 * i + col]);
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+        float16_t part[MB];
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++) {
+            const int t = 2 * b + tt;
+            const half8_t bop = q8_operand(cur.q[b][tt][0], cur.q[b][tt][1]);
+#pragma unroll
+            for (int i = 0; i < MB; i++) {
+                if (tt == 0) {
+                    float16_t z;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) z[r] = 0.0f;
+                    part[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[t & 1][i], bop, z, 0, 0, 0);
+                } else {
+                    part[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[t & 1][i], bop, part[i], 0, 0, 0);
+                }
+                if (i == 0 && t < 7) {  // the next step's fragments, behind the first product of this step
+#pragma unroll
+                    for (int ii = 0; ii < MB; ii++)
+                        af[(t + 1) & 1][ii] = __builtin_bit_cast(half8_t, a_cur[((t + 1) * 2 + g) * BM + 32 * ii + col]);
+                }
+            }
+        }
+        const float d = f16_bits_to_f32(cur.d[b]);
+#pragma unroll
+        for (int i = 0; i < MB; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][r] = __builtin_fmaf(d, part[i][r], acc[i][r]);
+    }
+}
+
+// grid and modes as for k_qgemm_rw; 8 waves = 256 weight rows per workgroup; LDS holds the two activation stages
+template <int MB>
+__global__ __launch_bounds__(512, 1) void k_qgemm_rw_q8(const uint8_t *__restrict__ W, const uint4 *__restrict__ xs,
+                                                         const float *__restrict__ rowscale, void *__restrict__ yg,
+                                                         float *__restrict__ partial, int M, int Mp, int N, int spr, int chunk,
+                                                         int mode) {
+    constexpr int BM = 32 * MB, kThreads = 512;
+    extern __shared__ uint4 smem[];
+    uint4 *a0 = smem, *a1 = a0 + kQ6Groups * BM;
+    const int tid = threadIdx.x;
+    LaneQ6<MB> L;
+    L.wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    L.col = lane & 31, L.g = lane >> 5;
+    const int n0 = blockIdx.x * 256, m0 = blockIdx.y * BM;
+    const int n = n0 + 32 * L.wave + L.col;
+    const int sb0 = blockIdx.z * chunk;
+    const int cnt = spr - sb0 < chunk ? spr - sb0 : chunk;
+    const size_t row_bytes = (size_t)spr * 272;
+    // this lane's row (rows past N repeat the last) at the first block of super-block sb0, and at its last half
+    const uint8_t *wp = W + (size_t)(n < N ? n : N - 1) * row_bytes + (size_t)sb0 * 272;
+    const uint8_t *wlast = W + (size_t)(n < N ? n : N - 1) * row_bytes + (size_t)(spr * 2 - 1) * 136;
+#pragma unroll
+    for (int i = 0; i < LaneQ6<MB>::kARounds; i++) {
+        const int idx = tid + i * kThreads;
+        L.a_off[i] = (uint32_t)((idx / BM) * Mp + idx % BM);
+    }
+    float16_t acc[MB];
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[i][r] = 0.0f;
+
+    Q8Half ha, hb;
+    q8_load(wp, L.g, ha);
+    {
+        const uint4 *xa = xs + (size_t)(sb0 * 2 * kGroups) * Mp + m0;
+#pragma unroll
+        for (int i = 0; i < LaneQ6<MB>::kARounds; i++) dma16(xa + L.a_off[i], a0 + i * kThreads + L.wave * 64);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();
+
+    for (int s = 0; s < cnt; s++) {
+        const int sb = sb0 + s;
+        const int sbn = sb + 1 < spr ? sb + 1 : spr - 1;  // the copies for "the next super-block" stay inside the matrix
+        const uint8_t *w1 = wp + 136, *w2 = wp + 272;
+        rw_half_q8<MB>(a0, a1, xs + (size_t)((sb * 2 + 1) * kGroups) * Mp + m0, w1, ha, hb, L, acc);
+        barrier_keep<12>();
+        rw_half_q8<MB>(a1, a0, xs + (size_t)(sbn * 2 * kGroups) * Mp + m0, w2 < wlast ? w2 : wlast, hb, ha, L, acc);
+        barrier_keep<12>();
+        wp = w2;
+    }
+
+    if (n >= N) return;
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int m = m0 + 32 * i + 8 * (r >> 2) + 4 * L.g + (r & 3);
+            if (m >= M) continue;
+            if (mode == 2) {
+                partial[((size_t)blockIdx.z * Mp + m) * N + n] = acc[i][r];
+            } else {
+                const float v = acc[i][r] * rowscale[m];
+                if (mode == 1) {
+                    uint32_t u = __builtin_bit_cast(uint32_t, v);
+                    u = ((u & 0x7FFFFFFFu) > 0x7F800000u) ? ((u >> 16) | 0x40u) : ((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+                    reinterpret_cast<uint16_t *>(yg)[(size_t)m * N + n] = (uint16_t)u;
+                } else {
+                    reinterpret_cast<float *>(yg)[(size_t)m * N + n] = v;
+                }
+            }
+        }
+}
+
 // y[m][n] = rowscale[m] * (partial[0][m][n] + partial[1][m][n] + ...), added in this order
 template <bool YBF16>
 __global__ __launch_bounds__(256) void k_rw_reduce(const float *__restrict__ partial, int splits, int M, int Mp, int N,
@@ -777,7 +952,7 @@ static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 bool qgemm_fits(uint32_t type, int64_t m, int64_t n, int64_t k) {
     // byte offsets inside a workgroup's rows and item offsets inside the activation copy are 32-bit
-    return (type == kTypeQ4K || type == kTypeQ6K) && m >= 1 && m <= (int64_t)1 << 22 && n >= 1 && k >= 256 && k % 256 == 0 && k <= (int64_t)1 << 22 && n <= 0x7FFFFF00;
+    return (type == kTypeQ4K || type == kTypeQ6K || type == kTypeQ8_0) && m >= 1 && m <= (int64_t)1 << 22 && n >= 1 && k >= 256 && k % 256 == 0 && k <= (int64_t)1 << 22 && n <= 0x7FFFFF00;
 }
 
 GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k) {
@@ -842,6 +1017,20 @@ static hipError_t launch_rw_q6(hipStream_t s, const uint8_t *w, const uint4 *xs,
     return hipGetLastError();
 }
 
+template <int MB>
+static hipError_t launch_rw_q8(hipStream_t s, const uint8_t *w, const uint4 *xs, const float *rowscale, void *y, float *partial,
+                               int64_t m, int64_t n, int spr, const GemmPlan &p, int mode) {
+    auto kern = k_qgemm_rw_q8<MB>;
+    constexpr size_t lds = (size_t)(2 * kQ6Groups * 32 * MB) * 16;
+    if (lds > 64 * 1024) {
+        hipError_t a = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (a != hipSuccess) return a;
+    }
+    const dim3 grid((unsigned)((n + 255) / 256), (unsigned)(p.mp / (32 * MB)), (unsigned)p.splits);
+    hipLaunchKernelGGL(kern, grid, dim3(512), lds, s, w, xs, rowscale, y, partial, (int)m, (int)p.mp, (int)n, spr, p.chunk, mode);
+    return hipGetLastError();
+}
+
 hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype,
                                 int64_t m, void *y, uint32_t y_dtype, uint32_t order, void *workspace, hipStream_t s) {
     if (!qgemm_fits(type, m, n, k)) return hipErrorInvalidValue;
@@ -852,17 +1041,19 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
     const size_t xs_bytes = align256((size_t)spr * 2 * kGroups * p.mp * 16);
     float *rowscale = reinterpret_cast<float *>(ws + xs_bytes);
     float *partial = reinterpret_cast<float *>(ws + xs_bytes + align256((size_t)p.mp * 4));
-    const bool xf32 = x_dtype == kDtypeF32, q6 = type == kTypeQ6K, ref = order == kOrderRef;
-    const int xorder = q6 ? 2 : (ref ? 0 : 1);  // the element order the pre-pass lays the activations out for
+    const bool xf32 = x_dtype == kDtypeF32, q6 = type == kTypeQ6K, q8 = type == kTypeQ8_0, ref = order == kOrderRef;
+    const int xorder = q8 ? 3 : (q6 ? 2 : (ref ? 0 : 1));  // the element order the pre-pass lays the activations out for
 #define PMH_PREP(F, O) hipLaunchKernelGGL((k_prep_rw<F, O>), dim3((unsigned)p.mp), dim3(256), 0, s, x, k, (int)m, (int)p.mp, rowscale, xs)
     if (xf32) {
         if (xorder == 0) PMH_PREP(true, 0);
         else if (xorder == 1) PMH_PREP(true, 1);
-        else PMH_PREP(true, 2);
+        else if (xorder == 2) PMH_PREP(true, 2);
+        else PMH_PREP(true, 3);
     } else {
         if (xorder == 0) PMH_PREP(false, 0);
         else if (xorder == 1) PMH_PREP(false, 1);
-        else PMH_PREP(false, 2);
+        else if (xorder == 2) PMH_PREP(false, 2);
+        else PMH_PREP(false, 3);
     }
 #undef PMH_PREP
     hipError_t e = hipGetLastError();
@@ -870,7 +1061,10 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
     const bool ybf = y_dtype == kDtypeBf16;
     const int mode = p.splits > 1 ? 2 : (ybf ? 1 : 0);
 #define PMH_RW_CASE(O, B, R, NWV) launch_rw<O, B, R, NWV>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
-    if (q6) {
+    if (q8) {
+        e = p.mb == 1 ? launch_rw_q8<1>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
+                      : launch_rw_q8<4>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode);
+    } else if (q6) {
         e = p.mb == 1 ? launch_rw_q6<1>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
                       : launch_rw_q6<4>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode);
     } else if (p.mb == 1) {

@@ -72,7 +72,7 @@ def test_qgemm_bf16_output_and_large_activations(oracle):
         assert np.max(np.abs(got16[row] - want[row])) / scale <= 2.0 ** -8  # bf16 rounding of the output
 
 
-@pytest.mark.parametrize("t", [Q4K, Q6K])
+@pytest.mark.parametrize("t", [Q4K, Q6K, Q8_0])
 @pytest.mark.parametrize("m", [24, 200, 300])
 def test_qgemm_f32_activations(oracle, t, m):
     """f32 activations are rounded once to f16 at the row's power-of-two scale (11 significant bits; a bf16 cast
@@ -147,7 +147,7 @@ def test_qgemm_argument_errors():
     buf = pm.DeviceBuffer(1 << 16)
     assert lib.pmetal_hip_qgemm(Q4K, buf.ptr, 4, 256, buf.ptr, 1, 0, buf.ptr, 0, 0, None) == 6   # m == 0
     assert lib.pmetal_hip_qgemm(Q4K, buf.ptr, 4, 100, buf.ptr, 1, 4, buf.ptr, 0, 0, None) == 6   # k % 256
-    assert lib.pmetal_hip_qgemm(Q8_0, buf.ptr, 4, 256, buf.ptr, 1, 4, buf.ptr, 0, 0, None) == 2  # no Q8_0 GEMM
+    assert lib.pmetal_hip_qgemm(Q8_0, buf.ptr, 4, 96, buf.ptr, 1, 4, buf.ptr, 0, 0, None) == 6   # k % 256 (a valid Q8_0 row)
     assert lib.pmetal_hip_qgemm(Q4K, buf.ptr, 4, 256, buf.ptr, 1, 4, buf.ptr, 7, 0, None) == 1   # y_dtype
 
 
@@ -174,14 +174,30 @@ def test_qgemm_q6k_matches_dequantize_then_matmul(oracle, m, n, k):
         assert elem <= TOL and norm <= TOL
 
 
-@pytest.mark.parametrize("t", [Q8_0])
-def test_qlinear_runs_rowwise_gemv_for_types_without_gemm(oracle, t):
-    n, k, m = 96, 512, 3
-    wq = oracle.quantize(t, weights(51, n * k))
+@pytest.mark.parametrize("m,n,k", [(1, 128, 256), (16, 128, 512), (64, 256, 1024), (128, 384, 4096), (33, 200, 768),
+                                   (130, 129, 256), (512, 512, 2048), (257, 160, 512), (300, 100, 768)])
+def test_qgemm_q8_0_matches_dequantize_then_matmul(oracle, m, n, k):
+    wq = oracle.quantize(Q8_0, weights(700 + m + n, n * k, outliers=1e-3))
+    x = np.random.default_rng(m * 5 + k).standard_normal((m, k)).astype(np.float32)
+    bits = oracle.f32_to_bf16_bits(x.reshape(-1)).reshape(m, k)
+    xr = oracle.bf16_bits_to_f32(bits.reshape(-1)).reshape(m, k)
+    want = reference(oracle, Q8_0, wq, n, k, xr, 0)
+    got = gpu_qgemm(Q8_0, wq, n, k, bits, m)
+    elem, norm = rel_errors(got.reshape(-1), want.reshape(-1))
+    print(f"Q8_0 GEMM m={m} n={n} k={k}: elem {elem:.2e} norm {norm:.2e}")
+    assert elem <= TOL and norm <= TOL
+    got16 = gpu_qgemm(Q8_0, wq, n, k, bits, m, y_dtype=pm.DTYPE_BF16)
+    assert np.max(np.abs(got16 - want)) / np.max(np.abs(want)) <= 2.0 ** -8
+
+
+def test_qlinear_q8_0_rows_that_are_not_a_multiple_of_256(oracle):
+    """Q8_0 rows may be any multiple of 32; the fused GEMM needs 256: qlinear then runs one GEMV per activation row."""
+    n, k, m = 96, 480, 3
+    wq = oracle.quantize(Q8_0, weights(51, n * k))
     x = np.random.default_rng(52).standard_normal((m, k)).astype(np.float32)
     bits = oracle.f32_to_bf16_bits(x.reshape(-1)).reshape(m, k)
-    lin = pm.GgufLinear(t, n, k, wq)
+    lin = pm.GgufLinear(Q8_0, n, k, wq)
     y = lin.forward(pm.DeviceBuffer.from_host(bits), m=m).to_host(np.float32).reshape(m, n)
-    want = reference(oracle, t, wq, n, k, oracle.bf16_bits_to_f32(bits.reshape(-1)).reshape(m, k), 0)
+    want = reference(oracle, Q8_0, wq, n, k, oracle.bf16_bits_to_f32(bits.reshape(-1)).reshape(m, k), 0)
     elem, norm = rel_errors(y.reshape(-1), want.reshape(-1))
     assert elem <= TOL and norm <= TOL
