@@ -142,6 +142,22 @@ def test_qgemm_q4k_k_split_is_deterministic_and_ragged_rows(oracle, m, n, k):
     assert elem <= TOL and norm <= TOL
 
 
+@pytest.mark.parametrize("t", [Q4K, Q6K, Q8_0])
+def test_qgemm_long_rows_with_k_split_above_128_rows(oracle, t):
+    """A down-projection-like shape (few weight rows, long k): more than 128 activation rows and a K split."""
+    m, n, k = 192, 512, 14336
+    wq = oracle.quantize(t, weights(800 + t, n * k))
+    x = np.random.default_rng(801 + t).standard_normal((m, k)).astype(np.float32)
+    bits = oracle.f32_to_bf16_bits(x.reshape(-1)).reshape(m, k)
+    xr = oracle.bf16_bits_to_f32(bits.reshape(-1)).reshape(m, k)
+    want = reference(oracle, t, wq, n, k, xr, 0)
+    got = gpu_qgemm(t, wq, n, k, bits, m)
+    elem, norm = rel_errors(got.reshape(-1), want.reshape(-1))
+    print(f"type {t} GEMM {m}x{n}x{k}: elem {elem:.2e} norm {norm:.2e}")
+    assert elem <= TOL and norm <= TOL
+    assert np.array_equal(got, gpu_qgemm(t, wq, n, k, bits, m))
+
+
 def test_qgemm_argument_errors():
     lib = _lib.load()
     buf = pm.DeviceBuffer(1 << 16)
