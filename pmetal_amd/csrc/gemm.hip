@@ -190,6 +190,73 @@ __global__ __launch_bounds__(256) void k_prep_rw(const void *__restrict__ xg, in
 // ------------------------------------------------------------------------------------------------
 // main kernel
 // ------------------------------------------------------------------------------------------------
+// Epilogue shared by the kernels below: a workgroup's BM x 256 tile of Y goes through LDS so that it leaves as
+// whole rows (16 bytes per lane, 512 bytes or 1 KiB contiguous per row) instead of 2- or 4-byte pieces per lane.
+// Every wave holds 32 columns (lane % 32) of all BM rows: C layout of v_mfma_f32_32x32x*: rows
+// 8 (r / 4) + 4 (lane / 32) + r % 4 of block i.  mode 0: y f32, 1: y bf16 (both scaled by rowscale), 2: fp32
+// partial tile of split z.  Must be reached by all threads of the workgroup, with no copies into LDS in flight.
+constexpr int kTilePad = 16;  // bytes added to an LDS row: rows 4 apart (the two lane halves) then lie in different banks
+template <int MB>
+constexpr size_t tile_lds_bytes() {
+    return (size_t)32 * MB * (256 * 4 + kTilePad);
+}
+
+__device__ __forceinline__ uint32_t bf16_rne_bits(const float v) {
+    const uint32_t u = __builtin_bit_cast(uint32_t, v);
+    return ((u & 0x7FFFFFFFu) > 0x7F800000u) ? ((u >> 16) | 0x40u) : ((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+
+template <int MB>
+__device__ __forceinline__ void store_tile(const float16_t (&acc)[MB], uint4 *smem, const int wave, const int col, const int g,
+                                           const int m0, const int n0, const int M, const int N, const int Mp,
+                                           const float *__restrict__ rowscale, void *__restrict__ yg,
+                                           float *__restrict__ partial, const int mode, const int z) {
+    constexpr int BM = 32 * MB;
+    constexpr int kRowStride = 256 * 4 + kTilePad;  // the LDS tile is fp32, not yet scaled
+    uint8_t *tile = reinterpret_cast<uint8_t *>(smem);
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int ml = 32 * i + 8 * (r >> 2) + 4 * g + (r & 3);
+            *reinterpret_cast<float *>(tile + ml * kRowStride + (32 * wave + col) * 4) = acc[i][r];
+        }
+    __syncthreads();
+    // one 16-byte store per trip and lane: 4 (fp32) or 8 (bf16) consecutive outputs of one row
+    const int per = mode == 1 ? 8 : 4, chunks = 256 / per, esize = mode == 1 ? 2 : 4;
+    uint8_t *out = mode == 2 ? reinterpret_cast<uint8_t *>(partial) + (size_t)z * Mp * N * 4 : reinterpret_cast<uint8_t *>(yg);
+    const bool rows_aligned = ((size_t)N * esize) % 16 == 0;
+    for (int idx = threadIdx.x; idx < BM * chunks; idx += blockDim.x) {
+        const int ml = idx / chunks, c = idx % chunks;
+        const int m = m0 + ml, n = n0 + c * per;
+        if (m >= M || n >= N) continue;
+        const float scale = mode == 2 ? 1.0f : rowscale[m];
+        const float4 *src = reinterpret_cast<const float4 *>(tile + ml * kRowStride + c * per * 4);
+        float v[8];
+        const float4 lo = src[0];
+        v[0] = lo.x * scale, v[1] = lo.y * scale, v[2] = lo.z * scale, v[3] = lo.w * scale;
+        uint4 pack;
+        if (mode == 1) {
+            const float4 hi = src[1];
+            v[4] = hi.x * scale, v[5] = hi.y * scale, v[6] = hi.z * scale, v[7] = hi.w * scale;
+            pack = make_uint4(bf16_rne_bits(v[0]) | (bf16_rne_bits(v[1]) << 16), bf16_rne_bits(v[2]) | (bf16_rne_bits(v[3]) << 16),
+                              bf16_rne_bits(v[4]) | (bf16_rne_bits(v[5]) << 16), bf16_rne_bits(v[6]) | (bf16_rne_bits(v[7]) << 16));
+        } else {
+            pack = make_uint4(__builtin_bit_cast(uint32_t, v[0]), __builtin_bit_cast(uint32_t, v[1]),
+                              __builtin_bit_cast(uint32_t, v[2]), __builtin_bit_cast(uint32_t, v[3]));
+        }
+        uint8_t *dst = out + ((size_t)m * N + n) * esize;
+        if (rows_aligned && n + per <= N) {
+            *reinterpret_cast<uint4 *>(dst) = pack;
+        } else {
+            for (int e = 0; e < per && n + e < N; e++) {
+                if (mode == 1) reinterpret_cast<uint16_t *>(dst)[e] = (uint16_t)bf16_rne_bits(v[e]);
+                else reinterpret_cast<float *>(dst)[e] = v[e];
+            }
+        }
+    }
+}
+
 // per-thread constants of the copy roles; a wave owns NR groups of 32 weight rows
 template <int MB, int NR, int NW>
 struct Lane {
@@ -207,19 +274,9 @@ struct Acc {
     u32x4 hdr[NR];  // headers of the current super-block: d | dmin << 16, then the 12 scale bytes
 };
 
-// 8 quants of one dword (low nibbles, then high nibbles) times their integer scales -> 8 exact f16 values.
-// 0x6400 | q is the f16 1024 + q; (1024 + q) * sc - 1024 * sc is exact in a packed f16 fma.
-__device__ __forceinline__ half8_t dequant8(const uint32_t w, const half2_t sc_lo, const half2_t off_lo, const half2_t sc_hi,
-                                            const half2_t off_hi) {
-    const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
-    const half2_t r0 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, lo, 0x04010400u)), sc_lo, off_lo);
-    const half2_t r1 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, lo, 0x04030402u)), sc_lo, off_lo);
-    const half2_t r2 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, hi, 0x04010400u)), sc_hi, off_hi);
-    const half2_t r3 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, hi, 0x04030402u)), sc_hi, off_hi);
-    return half8_t{r0[0], r0[1], r1[0], r1[1], r2[0], r2[1], r3[0], r3[1]};
-}
-
-// The same in four pieces, so that the pieces can be placed between matrix instructions.  k-step t selects the
+// 8 quants of one dword (low nibbles, then high nibbles) times their integer scales -> 8 exact f16 values:
+// 0x6400 | q is the f16 1024 + q, and (1024 + q) * sc - 1024 * sc is exact in a packed f16 fma.  Built in four
+// pieces, so that the pieces can be placed between matrix instructions.  k-step t selects the
 // scales: GGML order multiplies the low nibbles by the first and the high nibbles by the second sub-block scale,
 // REF order both by the scale of sub-block t / 4.
 struct Dq {
@@ -478,31 +535,11 @@ __global__ __launch_bounds__(64 * NW, MB * NR <= 1 && NW <= 8 ? 2 : 1) void k_qg
         uint4 *t = qc;
         qc = qb, qb = qa, qa = t;
     }
-    // C layout of v_mfma_f32_32x32x*: lane holds column (lane & 31), rows 8 (r / 4) + 4 (lane / 32) + r % 4
-#pragma unroll
-    for (int rg = 0; rg < NR; rg++) {
-        const int n = nw0 + 32 * rg + L.col;
-        if (n >= N) continue;
-#pragma unroll
-        for (int i = 0; i < MB; i++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int m = m0 + 32 * i + 8 * (r >> 2) + 4 * L.g + (r & 3);
-                if (m >= M) continue;
-                if (mode == 2) {
-                    partial[((size_t)blockIdx.z * Mp + m) * N + n] = R.acc[rg][i][r];
-                } else {
-                    const float v = R.acc[rg][i][r] * rowscale[m];
-                    if (mode == 1) {
-                        uint32_t u = __builtin_bit_cast(uint32_t, v);
-                        u = ((u & 0x7FFFFFFFu) > 0x7F800000u) ? ((u >> 16) | 0x40u) : ((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
-                        reinterpret_cast<uint16_t *>(yg)[(size_t)m * N + n] = (uint16_t)u;
-                    } else {
-                        reinterpret_cast<float *>(yg)[(size_t)m * N + n] = v;
-                    }
-                }
-            }
-    }
+    // the last copies (for a half super-block past the end) have landed and every wave is done with the stages
+    static_assert(NR == 1, "the tile store takes one group of weight rows per wave");
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();
+    store_tile<MB>(R.acc[0], smem, L.wave, L.col, L.g, m0, n0, M, N, Mp, rowscale, yg, partial, mode, blockIdx.z);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -728,27 +765,9 @@ __global__ __launch_bounds__(512, 1) void k_qgemm_rw_q6(const uint8_t *__restric
         qc = qb, qb = qa, qa = t;
     }
 
-    const int n = nw0 + L.col;
-    if (n >= N) return;
-#pragma unroll
-    for (int i = 0; i < MB; i++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int m = m0 + 32 * i + 8 * (r >> 2) + 4 * L.g + (r & 3);
-            if (m >= M) continue;
-            if (mode == 2) {
-                partial[((size_t)blockIdx.z * Mp + m) * N + n] = R.acc[i][r];
-            } else {
-                const float v = R.acc[i][r] * rowscale[m];
-                if (mode == 1) {
-                    uint32_t u = __builtin_bit_cast(uint32_t, v);
-                    u = ((u & 0x7FFFFFFFu) > 0x7F800000u) ? ((u >> 16) | 0x40u) : ((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
-                    reinterpret_cast<uint16_t *>(yg)[(size_t)m * N + n] = (uint16_t)u;
-                } else {
-                    reinterpret_cast<float *>(yg)[(size_t)m * N + n] = v;
-                }
-            }
-        }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the last copies (past the end) have landed
+    __syncthreads();
+    store_tile<MB>(R.acc, smem, L.wave, L.col, L.g, m0, n0, M, N, Mp, rowscale, yg, partial, mode, blockIdx.z);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -897,26 +916,9 @@ __global__ __launch_bounds__(512, 1) void k_qgemm_rw_q8(const uint8_t *__restric
         wp = w2;
     }
 
-    if (n >= N) return;
-#pragma unroll
-    for (int i = 0; i < MB; i++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int m = m0 + 32 * i + 8 * (r >> 2) + 4 * L.g + (r & 3);
-            if (m >= M) continue;
-            if (mode == 2) {
-                partial[((size_t)blockIdx.z * Mp + m) * N + n] = acc[i][r];
-            } else {
-                const float v = acc[i][r] * rowscale[m];
-                if (mode == 1) {
-                    uint32_t u = __builtin_bit_cast(uint32_t, v);
-                    u = ((u & 0x7FFFFFFFu) > 0x7F800000u) ? ((u >> 16) | 0x40u) : ((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
-                    reinterpret_cast<uint16_t *>(yg)[(size_t)m * N + n] = (uint16_t)u;
-                } else {
-                    reinterpret_cast<float *>(yg)[(size_t)m * N + n] = v;
-                }
-            }
-        }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the last register loads and copies (past the end) are done
+    __syncthreads();
+    store_tile<MB>(acc, smem, L.wave, L.col, L.g, m0, n0, M, N, Mp, rowscale, yg, partial, mode, blockIdx.z);
 }
 
 // y[m][n] = rowscale[m] * (partial[0][m][n] + partial[1][m][n] + ...), added in this order
@@ -941,7 +943,8 @@ __global__ __launch_bounds__(256) void k_rw_reduce(const float *__restrict__ par
 
 template <int MB, int NR, int NW>
 constexpr size_t rw_lds_bytes() {
-    return (size_t)(2 * kGroups * 32 * MB + NW * NR * (3 * 128 + 64)) * 16;
+    const size_t stages = (size_t)(2 * kGroups * 32 * MB + NW * NR * (3 * 128 + 64)) * 16;
+    return stages > tile_lds_bytes<MB>() ? stages : tile_lds_bytes<MB>();
 }
 
 }  // namespace
@@ -1009,7 +1012,8 @@ template <int MB>
 static hipError_t launch_rw_q6(hipStream_t s, const uint8_t *w, const uint4 *xs, const float *rowscale, void *y, float *partial,
                                int64_t m, int64_t n, int spr, const GemmPlan &p, int mode) {
     auto kern = k_qgemm_rw_q6<MB>;
-    constexpr size_t lds = (size_t)(2 * kQ6Groups * 32 * MB + 8 * (3 * kQ6Stage + 64)) * 16;
+    constexpr size_t stages = (size_t)(2 * kQ6Groups * 32 * MB + 8 * (3 * kQ6Stage + 64)) * 16;
+    constexpr size_t lds = stages > tile_lds_bytes<MB>() ? stages : tile_lds_bytes<MB>();
     hipError_t a = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (a != hipSuccess) return a;
     const dim3 grid((unsigned)((n + 255) / 256), (unsigned)(p.mp / (32 * MB)), (unsigned)p.splits);
@@ -1021,7 +1025,8 @@ template <int MB>
 static hipError_t launch_rw_q8(hipStream_t s, const uint8_t *w, const uint4 *xs, const float *rowscale, void *y, float *partial,
                                int64_t m, int64_t n, int spr, const GemmPlan &p, int mode) {
     auto kern = k_qgemm_rw_q8<MB>;
-    constexpr size_t lds = (size_t)(2 * kQ6Groups * 32 * MB) * 16;
+    constexpr size_t stages = (size_t)(2 * kQ6Groups * 32 * MB) * 16;
+    constexpr size_t lds = stages > tile_lds_bytes<MB>() ? stages : tile_lds_bytes<MB>();
     if (lds > 64 * 1024) {
         hipError_t a = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (a != hipSuccess) return a;
