@@ -73,52 +73,57 @@ __device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
 __device__ __forceinline__ float bf16_to_f32(uint32_t h) { return __builtin_bit_cast(float, h << 16); }
 
 // ------------------------------------------------------------------------------------------------
-// Pre-pass: one workgroup per activation row m < Mp.  rowscale[m] = 2^e with the row maximum * 2^-e in
+// Pre-pass: a workgroup takes R activation rows m < Mp (R = 1: 512 threads on one row, for few rows; R = 4: 256 threads
+// per row with the row index fastest across lanes, so that four lanes write 64 contiguous bytes of every item row).  rowscale[m] = 2^e with the row maximum * 2^-e in
 // [2^9, 2^10) (bf16 activations are then exact in f16 and block sums stay below 2^15); rows >= M are zero.
 // One thread per operand item: chunk u = 64 elements = sub-blocks 2u, 2u+1 (u = 4 sb + 2 h + g), k-step t.
 // ORDER 0 / 1: Q4_K element orders REF / GGML; ORDER 2: the Q6_K layout, ORDER 3: the natural order (Q8_0), both
 // without block sums.
 // ------------------------------------------------------------------------------------------------
-template <bool XF32, int ORDER>
-__global__ __launch_bounds__(256) void k_prep_rw(const void *__restrict__ xg, int64_t k, int M, int Mp,
-                                                  float *__restrict__ rowscale, uint4 *__restrict__ xs) {
-    const int m = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
+template <bool XF32, int ORDER, int R>
+__global__ __launch_bounds__(R == 1 ? 512 : 1024) void k_prep_rw(const void *__restrict__ xg, int64_t k, int M, int Mp,
+                                                                  float *__restrict__ rowscale, uint4 *__restrict__ xs) {
+    constexpr int NT = R == 1 ? 512 : 1024, JN = NT / R, NWV = NT / 64;
+    const int tid = threadIdx.x, lane = tid & 63, r = tid % R, j = tid / R;
+    const int m = blockIdx.x * R + r;
     const bool live = m < M;
-    __shared__ float red[4];
+    __shared__ float red[NWV][R];
     float amax = 0.0f;
     if (live) {
         if (XF32) {
             const float4 *row = reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(xg) + (int64_t)m * k);
-            for (int64_t i = tid; i < k / 4; i += 256) {
+            for (int64_t i = j; i < k / 4; i += JN) {
                 const float4 v = row[i];
                 amax = __builtin_fmaxf(__builtin_fmaxf(amax, __builtin_fmaxf(__builtin_fabsf(v.x), __builtin_fabsf(v.y))),
                                        __builtin_fmaxf(__builtin_fabsf(v.z), __builtin_fabsf(v.w)));
             }
         } else {
             const uint4 *row = reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(xg) + (int64_t)m * k);
-            for (int64_t i = tid; i < k / 8; i += 256) {
+            for (int64_t i = j; i < k / 8; i += JN) {
                 const uint4 v = row[i];
-                const uint32_t r[4] = {v.x, v.y, v.z, v.w};
+                const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
                 for (int q = 0; q < 4; q++)
-                    amax = __builtin_fmaxf(amax, __builtin_fmaxf(__builtin_fabsf(bf16_to_f32(r[q] & 0xFFFFu)),
-                                                                 __builtin_fabsf(bf16_to_f32(r[q] >> 16))));
+                    amax = __builtin_fmaxf(amax, __builtin_fmaxf(__builtin_fabsf(bf16_to_f32(w[q] & 0xFFFFu)),
+                                                                 __builtin_fabsf(bf16_to_f32(w[q] >> 16))));
             }
         }
     }
-    for (int off = 32; off > 0; off >>= 1) amax = __builtin_fmaxf(amax, __shfl_xor(amax, off));
-    if (lane == 0) red[tid >> 6] = amax;
+    for (int off = 32; off >= R; off >>= 1) amax = __builtin_fmaxf(amax, __shfl_xor(amax, off));
+    if (lane < R) red[tid >> 6][lane] = amax;
     __syncthreads();
-    amax = __builtin_fmaxf(__builtin_fmaxf(red[0], red[1]), __builtin_fmaxf(red[2], red[3]));
+    amax = red[0][r];
+#pragma unroll
+    for (int w = 1; w < NWV; w++) amax = __builtin_fmaxf(amax, red[w][r]);
     const int eb = (int)((__builtin_bit_cast(uint32_t, amax) >> 23) & 0xFFu);  // amax in [2^(eb-127), 2^(eb-126))
     int e = eb - 126 - 10;
     e = e < -126 ? -126 : (e > 126 ? 126 : e);
     if (eb == 255) e = 0;  // inf / NaN: let them through
     const float up = __builtin_bit_cast(float, (uint32_t)(127 + e) << 23);
-    if (tid == 0) rowscale[m] = up;
+    if (j == 0) rowscale[m] = up;
     const float down = live ? 1.0f / up : 0.0f;  // exact: a power of two
 
-    for (int64_t q = tid; q < k / 8; q += 256) {
+    for (int64_t q = j; q < k / 8; q += JN) {
         // the item's two runs of four elements (lo, hi), its half super-block and its operand group
         int64_t lo, hi, half;
         int t, g;
@@ -164,18 +169,18 @@ __global__ __launch_bounds__(256) void k_prep_rw(const void *__restrict__ xg, in
         const size_t base = (size_t)(half * kGroups) * Mp + m;
         xs[base + (size_t)(t * 2 + g) * Mp] = __builtin_bit_cast(uint4, h);
         if (ORDER >= 2) continue;  // Q6_K and Q8_0 have no min term: no block sums
-        // sums of the two sub-blocks of the chunk over its 8 k-steps (8 consecutive lanes)
+        // sums of the two sub-blocks of the chunk over its 8 k-steps (8 lanes, R apart)
         float s0, s1;
         if (ORDER == 0) {  // sub-block 2u: k-steps 0..3 (low and high nibbles), 2u+1: k-steps 4..7
             float s = slo + shi;
-            s += __shfl_xor(s, 1);
-            s += __shfl_xor(s, 2);
+            s += __shfl_xor(s, R);
+            s += __shfl_xor(s, 2 * R);
             s0 = s;
-            s1 = __shfl_down(s, 4);
+            s1 = __shfl_down(s, 4 * R);
         } else {  // sub-block 2u: the low nibbles of all k-steps, 2u+1: the high nibbles
-            slo += __shfl_xor(slo, 1), shi += __shfl_xor(shi, 1);
-            slo += __shfl_xor(slo, 2), shi += __shfl_xor(shi, 2);
-            slo += __shfl_xor(slo, 4), shi += __shfl_xor(shi, 4);
+            slo += __shfl_xor(slo, R), shi += __shfl_xor(shi, R);
+            slo += __shfl_xor(slo, 2 * R), shi += __shfl_xor(shi, 2 * R);
+            slo += __shfl_xor(slo, 4 * R), shi += __shfl_xor(shi, 4 * R);
             s0 = slo, s1 = shi;
         }
         if (t == 0) {  // exact head + tail split of each sum; item (H0, L0, H0, L0, H1, L1, H1, L1)
@@ -1048,7 +1053,15 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
     float *partial = reinterpret_cast<float *>(ws + xs_bytes + align256((size_t)p.mp * 4));
     const bool xf32 = x_dtype == kDtypeF32, q6 = type == kTypeQ6K, q8 = type == kTypeQ8_0, ref = order == kOrderRef;
     const int xorder = q8 ? 3 : (q6 ? 2 : (ref ? 0 : 1));  // the element order the pre-pass lays the activations out for
-#define PMH_PREP(F, O) hipLaunchKernelGGL((k_prep_rw<F, O>), dim3((unsigned)p.mp), dim3(256), 0, s, x, k, (int)m, (int)p.mp, rowscale, xs)
+#define PMH_PREP(F, O)                                                                                                       \
+    do {                                                                                                                     \
+        if (p.mp >= 1024)                                                                                                    \
+            hipLaunchKernelGGL((k_prep_rw<F, O, 4>), dim3((unsigned)p.mp / 4), dim3(1024), 0, s, x, k, (int)m, (int)p.mp,    \
+                               rowscale, xs);                                                                                \
+        else                                                                                                                 \
+            hipLaunchKernelGGL((k_prep_rw<F, O, 1>), dim3((unsigned)p.mp), dim3(512), 0, s, x, k, (int)m, (int)p.mp,         \
+                               rowscale, xs);                                                                                \
+    } while (0)
     if (xf32) {
         if (xorder == 0) PMH_PREP(true, 0);
         else if (xorder == 1) PMH_PREP(true, 1);

@@ -158,6 +158,31 @@ def test_qgemm_long_rows_with_k_split_above_128_rows(oracle, t):
     assert np.array_equal(got, gpu_qgemm(t, wq, n, k, bits, m))
 
 
+@pytest.mark.parametrize("t", [Q4K, Q6K, Q8_0])
+@pytest.mark.parametrize("xf32", [False, True])
+def test_qgemm_more_than_1024_activation_rows(oracle, t, xf32):
+    """1100 rows (not a multiple of 128): the activation pre-pass handles four rows per workgroup from 1024 rows on."""
+    m, n, k = 1100, 256, 768
+    wq = oracle.quantize(t, weights(900 + t, n * k, outliers=1e-3))
+    x = np.random.default_rng(901 + t).standard_normal((m, k)).astype(np.float32)
+    x[7] *= 3e4
+    x[1099] *= 2e-5
+    if xf32:  # the kernel rounds f32 activations to f16 at the row's power-of-two scale
+        e = np.floor(np.log2(np.max(np.abs(x), axis=1, keepdims=True))) - 9
+        xr = (np.ldexp(x, (-e).astype(np.int32)).astype(np.float16).astype(np.float32) * np.exp2(e)).astype(np.float32)
+        xin, xd = x, pm.DTYPE_F32
+    else:
+        xin = oracle.f32_to_bf16_bits(x.reshape(-1)).reshape(m, k)
+        xr, xd = oracle.bf16_bits_to_f32(xin.reshape(-1)).reshape(m, k), pm.DTYPE_BF16
+    for order in ((0, 1) if t == Q4K else (0,)):
+        want = reference(oracle, t, wq, n, k, xr, order)
+        got = gpu_qgemm(t, wq, n, k, xin, m, order=order, x_dtype=xd)
+        # per activation row: rows differ by nine orders of magnitude
+        for rows in (slice(0, 7), slice(7, 8), slice(8, 1099), slice(1099, 1100)):
+            elem, norm = rel_errors(got[rows].reshape(-1), want[rows].reshape(-1))
+            assert elem <= TOL and norm <= TOL, (t, order, rows, elem, norm)
+
+
 def test_qgemm_argument_errors():
     lib = _lib.load()
     buf = pm.DeviceBuffer(1 << 16)
