@@ -45,6 +45,27 @@ __device__ __forceinline__ float clamp_round(float v, float lo, float hi) {
     return __builtin_fminf(__builtin_fmaxf(r, lo), hi);
 }
 
+// clamp(nearest_int(v), 0, 15) in three instructions: clamp first (the bounds are integers, so clamping commutes with
+// rounding; NaN -> 0 as `as i32` does), then add the largest float below 0.5 and truncate.  For every w in [0, 15] the
+// rounded sum w + 0.49999997 lies on the same side of each integer as w + 0.5 does exactly (checked over all 2^32
+// floats on the CPU), so this is round-half-away without a compare.
+__device__ __forceinline__ float clamp_round_0_15(float v) {
+    const float w = __builtin_fminf(__builtin_fmaxf(v, 0.0f), 15.0f);
+    return __builtin_truncf(w + 0.49999997f);
+}
+
+// nearest_int(v) = `v.round() as i32` (half away from zero, saturating, NaN -> 0) in three instructions: add the largest
+// float below 0.5 to |v|, put the sign back, convert with truncation (the hardware conversion saturates and maps NaN
+// to 0; the asm keeps that out of the compiler's reach, for which an out-of-range cast is undefined).  Equal to the
+// reference for all 2^32 floats after any clamp to a range inside i32 (checked on the CPU).
+__device__ __forceinline__ int nearest_int_sat(float v) {
+    const float a = __builtin_fabsf(v) + 0.49999997f;
+    int i;
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(i) : "v"(__builtin_copysignf(a, v)));
+    return i;
+}
+__device__ __forceinline__ int clamp_i(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
 // `v as i32` for f32.
 __device__ __forceinline__ int f32_as_i32(float v) {
     if (v != v) return 0;
@@ -265,41 +286,36 @@ __global__ __launch_bounds__(64) void k_quantize_q4k(const float *__restrict__ x
     for (int i = 0; i < 32; i++) xv[i] = xs[lane * kQ4kLdsStride + i];
 
     // ---- make_qkx1_quants(15, 5, xv) ----
-    float mn = xv[0], mx = xv[0];
+    // min_by / max_by with total_cmp: equal keys are identical floats, so integer min / max of the keys will do
+    int kmn = total_key(xv[0]), kmx = kmn;
 #pragma unroll
     for (int i = 1; i < 32; i++) {
-        if (total_key(mn) > total_key(xv[i])) mn = xv[i];
-        if (total_key(mx) <= total_key(xv[i])) mx = xv[i];
+        const int key = total_key(xv[i]);
+        kmn = key < kmn ? key : kmn;
+        kmx = key > kmx ? key : kmx;
     }
+    const float mn = __builtin_bit_cast(float, kmn ^ (int)(((unsigned)(kmn >> 31)) >> 1));
+    const float mx = __builtin_bit_cast(float, kmx ^ (int)(((unsigned)(kmx >> 31)) >> 1));
     float scale = 0.0f, neg_min = 0.0f;  // returned (scale, -min)
     if (!(mx == mn)) {
         float minv = __builtin_fminf(mn, 0.0f);
         float iscale = 15.0f / (mx - minv);
         scale = 1.0f / iscale;
-        uint32_t lp[8] = {0, 0, 0, 0, 0, 0, 0, 0};  // previous quants, 4 per dword
+        float lf[32];  // the quants of the previous try, as floats
+#pragma unroll
+        for (int i = 0; i < 32; i++) lf[i] = 0.0f;
+#pragma unroll  // unrolled so that the quants of try t and t - 1 live in different registers without copies
         for (int t = 0; t < 5; t++) {
-            float lf[32];
-            float sumlx = 0.0f, suml2 = 0.0f;  // suml2 is an integer <= 7200: exact in f32
+            float sumlx = 0.0f, suml2 = 0.0f;  // suml2 is an integer <= 7200: exact in f32, with or without fusing
             bool changed = false;
 #pragma unroll
-            for (int w = 0; w < 8; w++) {
-                uint32_t word = 0;
-#pragma unroll
-                for (int c = 0; c < 4; c++) {
-                    const int i = 4 * w + c;
-                    const float xm = xv[i] - minv;
-                    const float v = iscale * xm;
-                    // clamp(nearest_int(v), 0, 15): for v < 0 any rounding clamps to 0
-                    const float tr = __builtin_truncf(v);
-                    float r = (v - tr >= 0.5f) ? tr + 1.0f : tr;
-                    r = __builtin_fminf(__builtin_fmaxf(r, 0.0f), 15.0f);  // NaN -> 0
-                    lf[i] = r;
-                    sumlx += xm * r;
-                    suml2 += r * r;
-                    word |= (uint32_t)r << (8 * c);
-                }
-                changed |= (word != lp[w]);
-                lp[w] = word;
+            for (int i = 0; i < 32; i++) {
+                const float xm = xv[i] - minv;
+                const float r = clamp_round_0_15(iscale * xm);
+                changed |= (r != lf[i]);
+                lf[i] = r;
+                sumlx += xm * r;
+                suml2 = __builtin_fmaf(r, r, suml2);
             }
             if (suml2 == 0.0f) break;
             scale = sumlx / suml2;
@@ -356,16 +372,33 @@ __global__ __launch_bounds__(64) void k_quantize_q4k(const float *__restrict__ x
     const uint32_t dmin16 = f32_to_f16_bits(max_min / 63.0f);
 
     // ---- requantize with the decoded f16 scales (k_quants.rs:932-943) ----
+    // L = clamp(nearest_int((x + dm) / dq), 0, 15).  Only the integer matters, so the IEEE division (ten instructions)
+    // is replaced by a multiplication with 1 / dq wherever that provably gives the same integer: the product differs
+    // from the correctly rounded quotient by less than 3e-6 for quotients below 16, so if it stays 8e-6 away from every
+    // rounding boundary n + 0.5 both round alike.  A lane that sees a product closer than that (or a dq outside the
+    // range where 1 / dq and the product are normal numbers) redoes its sub-block with the division.
     uint32_t lb[8] = {0, 0, 0, 0, 0, 0, 0, 0};  // 32 quants, one per byte
     const float dq = f16_bits_to_f32(d16) * (float)sc;
     if (dq != 0.0f) {
         const float dm = f16_bits_to_f32(dmin16) * (float)m;
+        const float rinv = 1.0f / dq;
+        bool exact_needed = !(dq > 1e-20f && dq < 1e20f);
 #pragma unroll
         for (int w = 0; w < 8; w++) {
 #pragma unroll
             for (int c = 0; c < 4; c++) {
-                const float r = clamp_round((xv[4 * w + c] + dm) / dq, 0.0f, 15.0f);
+                const float q = __builtin_fminf(__builtin_fmaxf((xv[4 * w + c] + dm) * rinv, 0.0f), 15.0f);
+                const float r = __builtin_truncf(q + 0.49999997f);
+                exact_needed |= !(__builtin_fabsf(__builtin_fabsf(q - r) - 0.5f) >= 8e-6f);
                 lb[w] |= (uint32_t)r << (8 * c);
+            }
+        }
+        if (exact_needed) {
+#pragma unroll
+            for (int w = 0; w < 8; w++) {
+                lb[w] = 0;
+#pragma unroll
+                for (int c = 0; c < 4; c++) lb[w] |= (uint32_t)clamp_round_0_15((xv[4 * w + c] + dm) / dq) << (8 * c);
             }
         }
     }
@@ -448,7 +481,7 @@ __global__ __launch_bounds__(64) void k_quantize_q6k(const float *__restrict__ x
         float sumlx = 0.0f, suml2 = 0.0f;
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            l[i] = clamp_round(iscale0 * xv[i], -32.0f, 31.0f);
+            l[i] = (float)clamp_i(nearest_int_sat(iscale0 * xv[i]), -32, 31);
             sumlx += wx[i] * l[i];
             suml2 += w[i] * (l[i] * l[i]);
         }
@@ -461,7 +494,7 @@ __global__ __launch_bounds__(64) void k_quantize_q6k(const float *__restrict__ x
             float nl[16];
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                nl[i] = clamp_round(isc * xv[i], -32.0f, 31.0f);
+                nl[i] = (float)clamp_i(nearest_int_sat(isc * xv[i]), -32, 31);
                 changed |= (nl[i] != l[i]);
                 slx += wx[i] * nl[i];
                 sl2 += w[i] * (nl[i] * nl[i]);
@@ -474,29 +507,44 @@ __global__ __launch_bounds__(64) void k_quantize_q6k(const float *__restrict__ x
             scale = sumlx / suml2;
             best = scale * sumlx;
         }
+        // Coordinate descent (quantize.rs:813-838), branch-free: every element computes its candidate and the test, and
+        // takes them by select.  The candidate clamp(nearest_int(x sl2 / slx)) comes from a multiplication with an
+        // approximate reciprocal: it differs from the correctly rounded quotient by less than 8e-6 for |quotient| < 33
+        // (one ulp of the reciprocal, half an ulp each for the product and the quotient), so a product that stays
+        // 2e-5 away from every rounding boundary rounds like the quotient; the rare lane closer than that, or with an
+        // slx outside the range where the reciprocal is a normal number, takes the IEEE division.  The returned scale
+        // is sumlx / suml2 of the last accepted change, so one division after the loop replaces one per change.
+        bool any_change = false;
         for (int t = 0; t < 5; t++) {
-            int n_changed = 0;
+            bool changed = false;
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                float slx = sumlx - wx[i] * l[i];
-                if (slx > 0.0f) {
-                    float sl2 = suml2 - w[i] * (l[i] * l[i]);
-                    const float new_l = clamp_round(xv[i] * sl2 / slx, -32.0f, 31.0f);
-                    if (new_l != l[i]) {
-                        slx += wx[i] * new_l;
-                        sl2 += w[i] * (new_l * new_l);
-                        if (sl2 > 0.0f && slx * slx * suml2 > sumlx * sumlx * sl2) {
-                            l[i] = new_l;
-                            sumlx = slx;
-                            suml2 = sl2;
-                            scale = sumlx / suml2;
-                            n_changed++;
-                        }
-                    }
+                const float li = l[i];
+                const float slx = sumlx - wx[i] * li;
+                const float sl2 = suml2 - w[i] * (li * li);
+                const float p = xv[i] * sl2;
+                const bool pos = slx > 0.0f;
+                const float qf = p * __builtin_amdgcn_rcpf(slx);
+                float nl = (float)clamp_i(nearest_int_sat(qf), -32, 31);
+                const bool sure = slx > 1e-30f && slx < 1e30f && __builtin_fabsf(__builtin_fabsf(qf - nl) - 0.5f) >= 2e-5f;
+                if (pos && !sure) nl = (float)clamp_i(nearest_int_sat(p / slx), -32, 31);
+                const bool differs = pos & (nl != li);
+                // from the second sweep on few lanes are still active and a new candidate is rare: skip the test
+                // when no lane has one
+                if (t == 0 || __builtin_amdgcn_ballot_w64(differs) != 0) {
+                    const float slx2 = slx + wx[i] * nl;
+                    const float sl22 = sl2 + w[i] * (nl * nl);
+                    const bool take = differs & (sl22 > 0.0f) & (slx2 * slx2 * suml2 > sumlx * sumlx * sl22);
+                    l[i] = take ? nl : li;
+                    sumlx = take ? slx2 : sumlx;
+                    suml2 = take ? sl22 : suml2;
+                    changed |= take;
                 }
             }
-            if (n_changed == 0) break;
+            if (!changed) break;
+            any_change = true;
         }
+        if (any_change) scale = sumlx / suml2;
     }
 
     // ---- super-block level (k_quants.rs:1082-1102) ----
@@ -519,13 +567,26 @@ __global__ __launch_bounds__(64) void k_quantize_q6k(const float *__restrict__ x
     const int8_t s8 = (int8_t)(uint8_t)(uint32_t)sq;  // `.min(127) as i8` wraps
 
     // ---- requantize (k_quants.rs:1105-1113) ----
+    // clamp(nearest_int(x / dq), -32, 31) by multiplication with 1 / dq where that provably rounds alike (see the Q4_K
+    // kernel), by the division for the lanes that come within 8e-6 of a rounding boundary.
     const float dq = f16_bits_to_f32(d16) * (float)s8;
     uint32_t lw[4] = {0, 0, 0, 0};
     if (dq != 0.0f) {
+        const float rinv = 1.0f / dq;
+        bool exact_needed = !(__builtin_fabsf(dq) > 1e-20f && __builtin_fabsf(dq) < 1e20f);
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            const float ll = clamp_round(xv[i] / dq, -32.0f, 31.0f);
-            lw[i >> 2] |= (uint32_t)(int)(ll + 32.0f) << (8 * (i & 3));
+            const float qf = xv[i] * rinv;
+            const int ll = clamp_i(nearest_int_sat(qf), -32, 31);
+            exact_needed |= !(__builtin_fabsf(__builtin_fabsf(qf - (float)ll) - 0.5f) >= 8e-6f);
+            lw[i >> 2] |= (uint32_t)(ll + 32) << (8 * (i & 3));
+        }
+        if (exact_needed) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) lw[q] = 0;
+#pragma unroll
+            for (int i = 0; i < 16; i++)
+                lw[i >> 2] |= (uint32_t)(clamp_i(nearest_int_sat(xv[i] / dq), -32, 31) + 32) << (8 * (i & 3));
         }
     } else {
 #pragma unroll

@@ -34,7 +34,15 @@ def edge_inputs(block_elems):
         "ragged": weights(6, 256 * 3 + 77),
         "short": weights(7, 5),
         "one_block_plus_one": weights(8, block_elems + 1),
+        # quotients that sit exactly on rounding ties, and scales spread over 35 orders of magnitude
+        "tie_grid": ((rng.integers(-63, 64, 1 << 16) * 0.5) * np.repeat(rng.uniform(0.001, 1, 1 << 8), 256)).astype(np.float32),
+        "scale_spread": (rng.standard_normal(1 << 16) * np.repeat(np.exp(rng.uniform(-40, 40, 1 << 11)), 32)).astype(np.float32),
     }
+    for name, bad in (("with_inf", np.inf), ("with_nan", np.nan)):
+        x = weights(9, 1 << 14)
+        x[rng.integers(0, x.size, 40)] = bad
+        x[rng.integers(0, x.size, 40)] = -bad
+        cases[name] = x
     return cases
 
 
