@@ -195,15 +195,15 @@ __global__ __launch_bounds__(R == 1 ? 512 : 1024) void k_prep_rw(const void *__r
 // ------------------------------------------------------------------------------------------------
 // main kernel
 // ------------------------------------------------------------------------------------------------
-// Epilogue shared by the kernels below: a workgroup's BM x 256 tile of Y goes through LDS so that it leaves as
+// Epilogue shared by the kernels below: a workgroup's BM x 32 NW tile of Y (256 columns for 8 waves) goes through LDS so that it leaves as
 // whole rows (16 bytes per lane, 512 bytes or 1 KiB contiguous per row) instead of 2- or 4-byte pieces per lane.
 // Every wave holds 32 columns (lane % 32) of all BM rows: C layout of v_mfma_f32_32x32x*: rows
 // 8 (r / 4) + 4 (lane / 32) + r % 4 of block i.  mode 0: y f32, 1: y bf16 (both scaled by rowscale), 2: fp32
 // partial tile of split z.  Must be reached by all threads of the workgroup, with no copies into LDS in flight.
 constexpr int kTilePad = 16;  // bytes added to an LDS row: rows 4 apart (the two lane halves) then lie in different banks
-template <int MB>
+template <int MB, int NW = 8>
 constexpr size_t tile_lds_bytes() {
-    return (size_t)32 * MB * (256 * 4 + kTilePad);
+    return (size_t)32 * MB * (32 * NW * 4 + kTilePad);
 }
 
 __device__ __forceinline__ uint32_t bf16_rne_bits(const float v) {
@@ -211,13 +211,14 @@ __device__ __forceinline__ uint32_t bf16_rne_bits(const float v) {
     return ((u & 0x7FFFFFFFu) > 0x7F800000u) ? ((u >> 16) | 0x40u) : ((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
 }
 
-template <int MB>
+template <int MB, int NW = 8>
 __device__ __forceinline__ void store_tile(const float16_t (&acc)[MB], uint4 *smem, const int wave, const int col, const int g,
                                            const int m0, const int n0, const int M, const int N, const int Mp,
                                            const float *__restrict__ rowscale, void *__restrict__ yg,
                                            float *__restrict__ partial, const int mode, const int z) {
     constexpr int BM = 32 * MB;
-    constexpr int kRowStride = 256 * 4 + kTilePad;  // the LDS tile is fp32, not yet scaled
+    constexpr int kCols = 32 * NW;                    // weight rows of the workgroup = columns of its tile of Y
+    constexpr int kRowStride = kCols * 4 + kTilePad;  // the LDS tile is fp32, not yet scaled
     uint8_t *tile = reinterpret_cast<uint8_t *>(smem);
 #pragma unroll
     for (int i = 0; i < MB; i++)
@@ -228,7 +229,7 @@ __device__ __forceinline__ void store_tile(const float16_t (&acc)[MB], uint4 *sm
         }
     __syncthreads();
     // one 16-byte store per trip and lane: 4 (fp32) or 8 (bf16) consecutive outputs of one row
-    const int per = mode == 1 ? 8 : 4, chunks = 256 / per, esize = mode == 1 ? 2 : 4;
+    const int per = mode == 1 ? 8 : 4, chunks = kCols / per, esize = mode == 1 ? 2 : 4;
     uint8_t *out = mode == 2 ? reinterpret_cast<uint8_t *>(partial) + (size_t)z * Mp * N * 4 : reinterpret_cast<uint8_t *>(yg);
     const bool rows_aligned = ((size_t)N * esize) % 16 == 0;
     for (int idx = threadIdx.x; idx < BM * chunks; idx += blockDim.x) {
@@ -544,7 +545,7 @@ __global__ __launch_bounds__(64 * NW, MB * NR <= 1 && NW <= 8 ? 2 : 1) void k_qg
     static_assert(NR == 1, "the tile store takes one group of weight rows per wave");
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();
-    store_tile<MB>(R.acc[0], smem, L.wave, L.col, L.g, m0, n0, M, N, Mp, rowscale, yg, partial, mode, blockIdx.z);
+    store_tile<MB, NW>(R.acc[0], smem, L.wave, L.col, L.g, m0, n0, M, N, Mp, rowscale, yg, partial, mode, blockIdx.z);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -949,7 +950,7 @@ __global__ __launch_bounds__(256) void k_rw_reduce(const float *__restrict__ par
 template <int MB, int NR, int NW>
 constexpr size_t rw_lds_bytes() {
     const size_t stages = (size_t)(2 * kGroups * 32 * MB + NW * NR * (3 * 128 + 64)) * 16;
-    return stages > tile_lds_bytes<MB>() ? stages : tile_lds_bytes<MB>();
+    return stages > tile_lds_bytes<MB, NW>() ? stages : tile_lds_bytes<MB, NW>();
 }
 
 }  // namespace
@@ -965,7 +966,7 @@ bool qgemm_fits(uint32_t type, int64_t m, int64_t n, int64_t k) {
 
 GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k) {
     GemmPlan p;
-    p.mb = m <= 64 ? 1 : 4;  // 32 activation rows per workgroup (more workgroups along M) or 128
+    p.mb = m <= 32 ? 1 : (m <= 64 ? 2 : 4);  // 32, 64 or 128 activation rows per workgroup
     p.mp = (m + 32 * p.mb - 1) / (32 * p.mb) * (32 * p.mb);
     p.nw = 8;
     const int64_t spr = k / 256;
@@ -1080,13 +1081,17 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
     const int mode = p.splits > 1 ? 2 : (ybf ? 1 : 0);
 #define PMH_RW_CASE(O, B, R, NWV) launch_rw<O, B, R, NWV>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
     if (q8) {
-        e = p.mb == 1 ? launch_rw_q8<1>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
-                      : launch_rw_q8<4>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode);
+        e = p.mb == 1   ? launch_rw_q8<1>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
+            : p.mb == 2 ? launch_rw_q8<2>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
+                        : launch_rw_q8<4>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode);
     } else if (q6) {
-        e = p.mb == 1 ? launch_rw_q6<1>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
-                      : launch_rw_q6<4>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode);
+        e = p.mb == 1   ? launch_rw_q6<1>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
+            : p.mb == 2 ? launch_rw_q6<2>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
+                        : launch_rw_q6<4>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode);
     } else if (p.mb == 1) {
         e = ref ? PMH_RW_CASE(0, 1, 1, 8) : PMH_RW_CASE(1, 1, 1, 8);
+    } else if (p.mb == 2) {
+        e = ref ? PMH_RW_CASE(0, 2, 1, 8) : PMH_RW_CASE(1, 2, 1, 8);
     } else {
         e = ref ? PMH_RW_CASE(0, 4, 1, 8) : PMH_RW_CASE(1, 4, 1, 8);
     }

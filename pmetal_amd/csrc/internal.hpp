@@ -36,7 +36,7 @@ hipError_t launch_qgemv_q4k_group(const uint8_t *const *w, const int64_t *n, flo
 
 // ---- gemm.hip: dequant-fused Y = X W^T for Q4_K and Q6_K (every wave owns 32 weight rows) ----
 struct GemmPlan {
-    int mb;      // 32-row activation blocks per workgroup (1 or 4)
+    int mb;      // 32-row activation blocks per workgroup (1, 2 or 4)
     int mp;      // activation rows padded to a multiple of 32 mb
     int nw;      // waves per workgroup
     int splits;  // workgroups along K (more than one: partial tiles plus a reduction kernel)
