@@ -10,6 +10,9 @@
 //   pmetal_gguf::GgmlType::{type_size, block_size, tensor_size}   crates/pmetal-gguf/src/types.rs:102-187
 //   pmetal_gguf::GgufLinear::matmul_from(x, m)    LayerWeight::matmul_from,
 //                                                 crates/pmetal-bridge/src/qwen3_native/weights.rs:66-84
+//   pmetal_gguf::quantize_model_q4_k_m(...)       the quantize-and-write loop of run_quantization,
+//                                                 crates/pmetal/src/commands/quantize.rs:1339-1433
+//   pmetal_gguf::hf_to_gguf_name                  crates/pmetal-models/src/weight_format.rs:389-435
 // A Rust `Result::Err` becomes a thrown exception carrying the library's message.  Everything computes on
 // the GPU; there is no CPU fallback (a missing device throws NoDeviceError).
 #pragma once
@@ -19,12 +22,13 @@
 #include <string>
 #include <vector>
 
+#include "pmetal_gguf_file.hpp"
 #include "pmetal_hip.h"
 
 namespace pmetal_gguf {
 
-enum class GgmlType : uint32_t { F32 = 0, F16 = 1, Q8_0 = 8, Q4K = 12, Q5K = 13, Q6K = 14 };
-
+// GgmlType (all ids of crates/pmetal-gguf/src/types.rs:16-97) comes from pmetal_gguf_file.hpp; the sizes below are the
+// library's own answers for the types it computes with.
 inline size_t type_size(GgmlType t) { return pmetal_hip_type_size((uint32_t)t); }
 inline size_t block_size(GgmlType t) { return pmetal_hip_block_size((uint32_t)t); }
 inline size_t tensor_size(GgmlType t, size_t n_elements) { return pmetal_hip_tensor_size((uint32_t)t, n_elements); }
@@ -155,6 +159,112 @@ class GgufLinear {
 inline bool use_more_bits(size_t layer, size_t n_layers) { return pmetal_hip_use_more_bits(layer, n_layers) != 0; }
 inline GgmlType q4km_tensor_type(const std::string &gguf_name, size_t ndim, size_t n_layers) {
     return (GgmlType)pmetal_hip_q4km_tensor_type(gguf_name.c_str(), ndim, n_layers);
+}
+
+
+// quantize(data, dtype) for every type the Q4_K_M recipe yields: F32 and F16 are conversions on the host
+// (crates/pmetal-gguf/src/quantize.rs:19-30), Q8_0 / Q4K / Q6K run on the GPU, anything else is the reference's
+// "not yet implemented" error.
+inline std::vector<uint8_t> quantize_any(const float *data, size_t n, GgmlType dtype) {
+    if (dtype == GgmlType::F32) {
+        std::vector<uint8_t> out(n * 4);
+        if (n) std::memcpy(out.data(), data, n * 4);
+        return out;
+    }
+    if (dtype == GgmlType::F16) {
+        std::vector<uint8_t> out(n * 2);
+        for (size_t i = 0; i < n; i++) {
+            const uint16_t h = f32_to_f16_bits(data[i]);
+            std::memcpy(out.data() + 2 * i, &h, 2);
+        }
+        return out;
+    }
+    return quantize(data, n, dtype);
+}
+
+// WeightLoader::hf_to_gguf_name (crates/pmetal-models/src/weight_format.rs:389-435)
+inline std::string hf_to_gguf_name(const std::string &hf_name) {
+    if (hf_name == "model.embed_tokens.weight") return "token_embd.weight";
+    if (hf_name == "model.norm.weight") return "output_norm.weight";
+    if (hf_name == "lm_head.weight") return "output.weight";
+    static const std::string prefix = "model.layers.";
+    if (hf_name.compare(0, prefix.size(), prefix) != 0) return hf_name;
+    const std::string rest = hf_name.substr(prefix.size());
+    const size_t dot = rest.find('.');
+    if (dot == std::string::npos) return hf_name;
+    const std::string layer = rest.substr(0, dot), suffix = rest.substr(dot + 1);
+    {  // usize::from_str: decimal digits behind an optional '+', value below 2^64
+        const size_t first = !layer.empty() && layer[0] == '+' ? 1 : 0;
+        if (layer.size() == first) return hf_name;
+        unsigned long long v = 0;
+        for (size_t i = first; i < layer.size(); i++) {
+            if (layer[i] < '0' || layer[i] > '9') return hf_name;
+            const unsigned d = (unsigned)(layer[i] - '0');
+            if (v > (UINT64_MAX - d) / 10) return hf_name;
+            v = v * 10 + d;
+        }
+    }
+    static const std::pair<const char *, const char *> table[] = {
+        {"input_layernorm.weight", "attn_norm.weight"},
+        {"self_attn.q_proj.weight", "attn_q.weight"},
+        {"self_attn.k_proj.weight", "attn_k.weight"},
+        {"self_attn.v_proj.weight", "attn_v.weight"},
+        {"self_attn.o_proj.weight", "attn_output.weight"},
+        {"post_attention_layernorm.weight", "ffn_norm.weight"},
+        {"mlp.gate.weight", "ffn_gate_inp.weight"},
+        {"mlp.router.weight", "ffn_gate_inp.weight"},
+        {"mlp.gate_proj.weight", "ffn_gate.weight"},
+        {"mlp.up_proj.weight", "ffn_up.weight"},
+        {"mlp.down_proj.weight", "ffn_down.weight"},
+        {"mlp.experts.gate_proj.weight", "ffn_gate_exps.weight"},
+        {"mlp.experts.up_proj.weight", "ffn_up_exps.weight"},
+        {"mlp.experts.down_proj.weight", "ffn_down_exps.weight"},
+        {"mlp.shared_expert.gate_proj.weight", "ffn_gate_shexp.weight"},
+        {"mlp.shared_expert.up_proj.weight", "ffn_up_shexp.weight"},
+        {"mlp.shared_expert.down_proj.weight", "ffn_down_shexp.weight"},
+        {"mlp.shared_experts.gate_proj.weight", "ffn_gate_shexp.weight"},
+        {"mlp.shared_experts.up_proj.weight", "ffn_up_shexp.weight"},
+        {"mlp.shared_experts.down_proj.weight", "ffn_down_shexp.weight"},
+        {"mlp.shared_expert_gate.weight", "ffn_gate_inp_shexp.weight"},
+        {"self_attn.q_norm.weight", "attn_q_norm.weight"},
+        {"self_attn.k_norm.weight", "attn_k_norm.weight"},
+    };
+    std::string mapped = suffix;
+    for (const auto &row : table)
+        if (suffix == row.first) mapped = row.second;
+    return "blk." + layer + "." + mapped;
+}
+
+// One f32 tensor of the model to quantize: its Hugging Face name, row-major shape and values (not owned).
+struct SourceTensor {
+    std::string name;
+    std::vector<uint64_t> shape;
+    const float *data;
+};
+
+// The quantize-and-write loop of run_quantization for `--method q4_k_m` over dense tensors
+// (crates/pmetal/src/commands/quantize.rs:1339-1433): tensors in the order of their Hugging Face names, each under
+// its GGUF name, with the type the recipe gives it (norms and 1-D tensors F16, attn_v / ffn_down of the layers that get
+// more bits and the embedding / output matrices Q6_K, the rest Q4_K), quantized by quantize_any.  The builder starts as
+// GgufBuilder::with_model(architecture, "quantized-model"); the caller adds the model's own metadata and writes it.
+inline GgufBuilder quantize_model_q4_k_m(const std::string &architecture, const std::vector<SourceTensor> &weights,
+                                         size_t n_layers) {
+    GgufBuilder builder = GgufBuilder::with_model(architecture, "quantized-model");
+    std::vector<const SourceTensor *> order;
+    for (const SourceTensor &t : weights) order.push_back(&t);
+    std::sort(order.begin(), order.end(), [](const SourceTensor *a, const SourceTensor *b) { return a->name < b->name; });
+    for (const SourceTensor *t : order) {
+        const std::string gguf_name = hf_to_gguf_name(t->name);
+        const GgmlType target = q4km_tensor_type(gguf_name, t->shape.size(), n_layers);
+        size_t n = 1;
+        for (uint64_t d : t->shape) n *= (size_t)d;
+        try {
+            builder.add_raw_tensor(gguf_name, t->shape, target, quantize_any(t->data, n, target));
+        } catch (const Error &e) {
+            throw QuantizationError(e.code, "Quantization error for " + t->name + ": " + e.what());
+        }
+    }
+    return builder;
 }
 
 }  // namespace pmetal_gguf
