@@ -147,7 +147,10 @@ int32_t pmetal_hip_dequantize_dev(uint32_t ggml_type, const uint8_t *src_dev, si
  * with W = reference dequantize of the packed blocks (order as given), fp32 accumulation,
  * max relative error <= 1e-3 against dequantize-then-f32-matmul.
  * W: [n, k] packed row-major, k a multiple of the block size.  x/X: f32 or bf16.
- * y/Y: f32 (qgemv) or f32/bf16 (qgemm), row-major [m, n].                               */
+ * y/Y: f32 (qgemv) or f32/bf16 (qgemm), row-major [m, n].
+ * qgemm keeps scratch memory (converted activations, partial tiles) inside the library, one
+ * buffer per calling thread, device and stream; it grows on demand, which synchronises that
+ * stream once.                                                                           */
 int32_t pmetal_hip_qgemv(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, int64_t k, const void *x_dev,
                          uint32_t x_dtype, float *y_dev, uint32_t order, void *stream);
 int32_t pmetal_hip_qgemm(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, int64_t k, const void *x_dev,

@@ -12,6 +12,7 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <vector>
 
 #include "internal.hpp"
 
@@ -90,28 +91,43 @@ struct DevBuf {
     }
 };
 
-// qgemm scratch, grown on demand and kept per thread so concurrent callers do not share it.
+// qgemm scratch, grown on demand: one buffer per (thread, device, stream), so that neither concurrent callers nor
+// one caller's launches on different streams share it.  Launches on one stream run in order and may.
 struct Workspace {
     void *p = nullptr;
     size_t bytes = 0;
     int device = -1;
+    hipStream_t stream = nullptr;
 };
-thread_local Workspace g_ws;
+struct WorkspaceSet {
+    std::vector<Workspace> items;
+    ~WorkspaceSet() {
+        for (Workspace &w : items)
+            if (w.p) (void)hipFree(w.p);  // at thread exit; fails harmlessly once the runtime is gone
+    }
+};
+thread_local WorkspaceSet g_ws;
 
-int32_t workspace(size_t bytes, void **out) {
+int32_t workspace(size_t bytes, hipStream_t stream, void **out) {
     int dev = 0;
     HIP_TRY(hipGetDevice(&dev));
-    if (g_ws.p && (g_ws.bytes < bytes || g_ws.device != dev)) {
-        HIP_TRY(hipDeviceSynchronize());
-        HIP_TRY(hipFree(g_ws.p));
-        g_ws = Workspace{};
+    Workspace *w = nullptr;
+    for (Workspace &c : g_ws.items)
+        if (c.device == dev && c.stream == stream) w = &c;
+    if (!w) {
+        g_ws.items.push_back(Workspace{nullptr, 0, dev, stream});
+        w = &g_ws.items.back();
     }
-    if (!g_ws.p && bytes) {
-        HIP_TRY(hipMalloc(&g_ws.p, bytes));
-        g_ws.bytes = bytes;
-        g_ws.device = dev;
+    if (w->p && w->bytes < bytes) {
+        HIP_TRY(hipStreamSynchronize(stream));  // earlier launches on this stream may still use the smaller buffer
+        HIP_TRY(hipFree(w->p));
+        w->p = nullptr, w->bytes = 0;
     }
-    *out = g_ws.p;
+    if (!w->p && bytes) {
+        HIP_TRY(hipMalloc(&w->p, bytes));
+        w->bytes = bytes;
+    }
+    *out = w->p;
     return PMETAL_HIP_OK;
 }
 
@@ -482,7 +498,7 @@ int32_t pmetal_hip_qgemm(uint32_t t, const uint8_t *w, int64_t n, int64_t k, con
     if (!pmh::qgemm_fits(t, m, n, k))
         return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qgemm: m and k must be at most 2^22 (m = %lld, k = %lld)", (long long)m, (long long)k);
     void *ws = nullptr;
-    if (int32_t rc = workspace(pmh::qgemm_workspace_bytes(m, n, k), &ws)) return rc;
+    if (int32_t rc = workspace(pmh::qgemm_workspace_bytes(m, n, k), (hipStream_t)stream, &ws)) return rc;
     hipError_t e = pmh::launch_qgemm(t, w, n, k, x, x_dtype, m, y, y_dtype, order, ws, (hipStream_t)stream);
     if (e == hipErrorNotSupported) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "qgemm: configuration not supported");
     if (e != hipSuccess) return hip_fail(e, "qgemm kernel launch");

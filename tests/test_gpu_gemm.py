@@ -242,3 +242,34 @@ def test_qlinear_q8_0_rows_that_are_not_a_multiple_of_256(oracle):
     want = reference(oracle, Q8_0, wq, n, k, oracle.bf16_bits_to_f32(bits.reshape(-1)).reshape(m, k), 0)
     elem, norm = rel_errors(y.reshape(-1), want.reshape(-1))
     assert elem <= TOL and norm <= TOL
+
+
+def test_qgemm_on_two_streams_of_one_thread_keep_separate_scratch(oracle):
+    """Two GEMMs in flight on two streams of the same thread: each stream has its own scratch inside the library, so
+    neither the converted activations nor the partial tiles of one can be overwritten by the other; a later, larger
+    shape on the first stream makes that stream's scratch grow."""
+    lib = _lib.load()
+    s1, s2 = lib.pmetal_hip_stream_create(), lib.pmetal_hip_stream_create()
+    assert s1 and s2
+    try:
+        jobs = []
+        for i, (m, n, k, s) in enumerate([(96, 512, 8192, s1), (200, 768, 1024, s2), (40, 256, 4096, s1), (700, 1024, 2048, s1),
+                                          (17, 300, 2048, s2)]):
+            wq = oracle.quantize(Q4K, weights(950 + i, n * k))
+            x = np.random.default_rng(960 + i).standard_normal((m, k)).astype(np.float32)
+            bits = oracle.f32_to_bf16_bits(x.reshape(-1)).reshape(m, k)
+            xr = oracle.bf16_bits_to_f32(bits.reshape(-1)).reshape(m, k)
+            dw, dx, dy = pm.DeviceBuffer.from_host(wq), pm.DeviceBuffer.from_host(bits), pm.DeviceBuffer(4 * m * n)
+            jobs.append((m, n, k, s, dw, dx, dy, reference(oracle, Q4K, wq, n, k, xr, 0)))
+        for rep in range(3):  # launched back to back, nothing waits in between
+            for m, n, k, s, dw, dx, dy, _ in jobs:
+                pm.check(lib.pmetal_hip_qgemm(Q4K, dw.ptr, n, k, dx.ptr, pm.DTYPE_BF16, m, dy.ptr, pm.DTYPE_F32, 0, s))
+        pm.check(lib.pmetal_hip_sync(s1))
+        pm.check(lib.pmetal_hip_sync(s2))
+        for m, n, k, s, dw, dx, dy, want in jobs:
+            got = dy.to_host(np.float32).reshape(m, n)
+            elem, norm = rel_errors(got.reshape(-1), want.reshape(-1))
+            assert elem <= TOL and norm <= TOL, (m, n, k, elem, norm)
+    finally:
+        lib.pmetal_hip_stream_destroy(s1)
+        lib.pmetal_hip_stream_destroy(s2)
