@@ -213,6 +213,57 @@ def bench_gemv(args, n, k, t=Q4K, copies=16):
     }, (t, n, k)
 
 
+def bench_gemv_q8k(args, n, k, t=Q4K, copies=16):
+    """One step = `copies` x (quantize the f32 activations to Q8_K, integer-dot GEMV), weights rotating through HBM."""
+    pm, _lib, lib = load()
+    timer = Timer(pm, lib)
+    ws = [device_weights(pm, lib, t, n * k, 1000 + i) for i in range(copies)]
+    x = pm.DeviceBuffer.from_host(np.random.default_rng(1).standard_normal(k).astype(np.float32))
+    xq = pm.DeviceBuffer(lib.pmetal_hip_q8k_size(k))
+    ys = [pm.DeviceBuffer(4 * n) for _ in range(copies)]
+
+    def step():
+        for i in range(copies):
+            pm.check(lib.pmetal_hip_quantize_q8k_dev(x.ptr, k, xq.ptr, lib.pmetal_hip_q8k_size(k), None))
+            pm.check(lib.pmetal_hip_qgemv_q8k(t, ws[i].ptr, n, k, xq.ptr, ys[i].ptr, None))
+
+    def gemv_only():
+        for i in range(copies):
+            pm.check(lib.pmetal_hip_qgemv_q8k(t, ws[i].ptr, n, k, xq.ptr, ys[i].ptr, None))
+
+    ev_ms, wall_ms = timer.run(step, args.steps, args.warmup)
+    g_ms, _ = timer.run(gemv_only, args.steps, args.warmup)
+    launches = args.steps * copies
+    bytes_per_launch = pm.GgmlType(t).tensor_size(n * k) + 4 * k + lib.pmetal_hip_q8k_size(k) * 2 + 4 * n
+    us = ev_ms * 1e3 / launches
+    gbs = bytes_per_launch / (us * 1e-6) / 1e9
+    return {
+        "value": gbs, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "k_qgemv_q4k_q8k (+ k_quantize_q8k)" if t == Q4K else "k_qgemv_q6k_q8k (+ k_quantize_q8k)",
+                     "bytes_per_launch": bytes_per_launch, "us_per_launch": round(us, 3)},
+        "extra": {"gemv_only_us_per_launch": round(g_ms * 1e3 / launches, 3), "weight_copies": copies},
+    }, (t, n, k)
+
+
+def cpu_baseline_gemv_q8k(t, n, k, budget_s=12.0):
+    """Oracle: quantize_q8k of the activations + the scalar vec_dot over every row, one thread, on a slice of the rows."""
+    from oracle import binding as oracle
+    oracle.build()
+    rows = min(n, 2048)
+    rng = np.random.default_rng(7)
+    wq = oracle.quantize(t, (rng.standard_normal(rows * k) * 0.02).astype(np.float32))
+    x = rng.standard_normal(k).astype(np.float32)
+    reps, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < budget_s:
+        oracle.qmatvec_q8k(t, wq, rows, k, oracle.quantize_q8k(x))
+        reps += 1
+    dt = time.perf_counter() - t0
+    return {"value": round(reps * wq.size / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{reps} x (quantize_q8k + vec_dot over {rows}x{k} rows of the same shape), {dt:.1f} s"}
+
+
 def bench_gemm(args, m, n, k, t=Q4K):
     pm, _lib, lib = load()
     timer = Timer(pm, lib)
@@ -386,6 +437,10 @@ WORKLOADS = {
     "gemv_q4k_4096x14336": dict(kind="gemv", n=4096, k=14336, metric="Q4_K GEMV GB/s @4096x14336", unit="GB/s",
                                 dtype="bf16"),
 }
+WORKLOADS["gemv_q4k_q8k_14336x4096"] = dict(kind="gemv_q8k", n=14336, k=4096, type=Q4K, unit="GB/s", dtype="i8",
+                                            metric="Q4_K x Q8_K integer-dot GEMV GB/s @14336x4096 (activation quantize included)")
+WORKLOADS["gemv_q6k_q8k_14336x4096"] = dict(kind="gemv_q8k", n=14336, k=4096, type=Q6K, unit="GB/s", dtype="i8",
+                                            metric="Q6_K x Q8_K integer-dot GEMV GB/s @14336x4096 (activation quantize included)")
 WORKLOADS["decode_qwen3_0.6b_q4km"] = dict(kind="decode", metric="Q4_K_M decode linears tokens/s (Qwen3-0.6B shape)", unit="tokens/s",
                                            dtype="bf16")
 WORKLOADS["quantize_llama3_8b_q4km"] = dict(kind="quantize", metric="f32->Q4_K_M quantize GB/s of f32 consumed (Llama-3-8B shape)",
@@ -423,6 +478,8 @@ def main():
         res, (t, n, k) = bench_quantize(args)
     elif wl["kind"] == "dequantize":
         res, (t, n, k) = bench_dequantize(args, wl["n"], wl["k"])
+    elif wl["kind"] == "gemv_q8k":
+        res, (t, n, k) = bench_gemv_q8k(args, wl["n"], wl["k"], wl["type"])
     else:
         res, (t, n, k) = bench_gemv(args, wl["n"], wl["k"])
     out = {
@@ -430,10 +487,12 @@ def main():
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(res["ms_per_step"], 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": wl["dtype"],
         "data": ("synthetic: N(0,0.02) f32 with 0.1% outliers at +-0.5, generated on the device" if wl["kind"] == "quantize"
+                 else "synthetic: N(0,0.02) f32 weights generated and quantized on the device, x ~ N(0,1) f32" if wl["kind"] == "gemv_q8k"
                  else "synthetic: N(0,0.02) f32 weights generated and quantized on the device, x ~ N(0,1) bf16"),
         "config": {"workload": args.workload, "element_order": "REF",
                    "step": {"gemm": "one GEMM launch (activation pre-pass + MFMA kernel)",
                             "gemv": "16 back-to-back GEMVs over 16 distinct weight tensors (528 MB, HBM-resident)",
+                            "gemv_q8k": "16 x (activations f32 -> Q8_K, integer-dot GEMV) over 16 distinct weight tensors",
                             "decode": "all 197 batch-1 projections of one token, back to back on one stream",
                             "dequantize": "two tensors of 14336 x 4096, blocks resident in HBM",
                             "quantize": "all 226 tensors of the model, f32 resident in HBM"}[wl["kind"]]},
@@ -452,6 +511,8 @@ def main():
     if not args.no_cpu_baseline:
         if wl["kind"] == "gemv":
             out["cpu_baseline"] = cpu_baseline_gemv(t, n, k)
+        elif wl["kind"] == "gemv_q8k":
+            out["cpu_baseline"] = cpu_baseline_gemv_q8k(t, n, k)
         elif wl["kind"] == "quantize":
             out["cpu_baseline"] = cpu_baseline_quantize()
         elif wl["kind"] == "gemm":

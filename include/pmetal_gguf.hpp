@@ -155,6 +155,21 @@ class GgufLinear {
     DeviceBuffer w_;
 };
 
+// quantize_q8k (crates/pmetal-gguf/src/k_quants.rs:815-871) of n f32 values on the device: 292-byte BlockQ8K blocks.
+inline DeviceBuffer quantize_q8k(const DeviceBuffer &x, size_t n, void *stream = nullptr) {
+    DeviceBuffer out(pmetal_hip_q8k_size(n) ? pmetal_hip_q8k_size(n) : 16);
+    detail::check(pmetal_hip_quantize_q8k_dev((const float *)x.ptr(), n, (uint8_t *)out.ptr(), pmetal_hip_q8k_size(n), stream), true);
+    return out;
+}
+// y[r] = vec_dot_q4k_q8k / vec_dot_q6k_q8k (row r of w, xq), crates/pmetal-gguf/src/vec_dot.rs:829-851, as the scalar
+// definitions (:617-692) compute them, bit for bit.  w: [n, k] Q4K or Q6K blocks, xq: k / 256 Q8_K blocks, all on the device.
+inline DeviceBuffer qgemv_q8k(GgmlType dtype, const DeviceBuffer &w, int64_t n, int64_t k, const DeviceBuffer &xq,
+                              void *stream = nullptr) {
+    DeviceBuffer y((size_t)(n > 0 ? n : 1) * sizeof(float));
+    detail::check(pmetal_hip_qgemv_q8k((uint32_t)dtype, (const uint8_t *)w.ptr(), n, k, (const uint8_t *)xq.ptr(), (float *)y.ptr(), stream));
+    return y;
+}
+
 // Q4_K_M recipe: crates/pmetal/src/commands/quantize.rs:988-1137
 inline bool use_more_bits(size_t layer, size_t n_layers) { return pmetal_hip_use_more_bits(layer, n_layers) != 0; }
 inline GgmlType q4km_tensor_type(const std::string &gguf_name, size_t ndim, size_t n_layers) {

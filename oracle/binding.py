@@ -77,6 +77,12 @@ def lib() -> C.CDLL:
         L.pmo_qmatmul_f64.argtypes = [C.c_uint32, u8p, C.c_size_t, C.c_size_t, f32p, C.c_size_t, f32p,
                                       C.c_uint32]
         L.pmo_qmatmul_f64.restype = C.c_int32
+        L.pmo_q8k_size.argtypes, L.pmo_q8k_size.restype = [C.c_size_t], C.c_size_t
+        L.pmo_quantize_q8k.argtypes, L.pmo_quantize_q8k.restype = [f32p, C.c_size_t, u8p], None
+        for name in ("pmo_vec_dot_q4k_q8k", "pmo_vec_dot_q6k_q8k"):
+            getattr(L, name).argtypes, getattr(L, name).restype = [u8p, u8p, C.c_size_t], C.c_float
+        L.pmo_qmatvec_q8k.argtypes = [C.c_uint32, u8p, C.c_size_t, C.c_size_t, u8p, f32p]
+        L.pmo_qmatvec_q8k.restype = C.c_int32
         _lib = L
     return _lib
 
@@ -158,6 +164,35 @@ def qmatmul(t: int, w: np.ndarray, n_rows: int, k: int, x: np.ndarray, order: in
     x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, k)
     y = np.empty((x.shape[0], n_rows), dtype=np.float32)
     rc = lib().pmo_qmatmul_f64(t, _u8p(w), n_rows, k, _f32p(x), x.shape[0], _f32p(y), order)
+    if rc != OK:
+        raise ValueError(rc)
+    return y
+
+
+def quantize_q8k(x: np.ndarray) -> np.ndarray:
+    """k_quants.rs:815-871 ``quantize_q8k``: flat f32 -> 292-byte blocks."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+    out = np.zeros(lib().pmo_q8k_size(x.size), dtype=np.uint8)
+    if x.size:
+        lib().pmo_quantize_q8k(_f32p(x), x.size, _u8p(out))
+    return out
+
+
+def vec_dot_q8k(t: int, xs: np.ndarray, ys: np.ndarray, n_blocks: int) -> float:
+    """vec_dot.rs:617-692 (scalar): one row of Q4_K / Q6_K blocks against Q8_K blocks."""
+    xs = np.ascontiguousarray(xs, dtype=np.uint8).reshape(-1)
+    ys = np.ascontiguousarray(ys, dtype=np.uint8).reshape(-1)
+    assert xs.size == n_blocks * tensor_size(t, 256) and ys.size == n_blocks * 292
+    fn = lib().pmo_vec_dot_q4k_q8k if t == TYPE_Q4K else lib().pmo_vec_dot_q6k_q8k
+    return float(fn(_u8p(xs), _u8p(ys), n_blocks))
+
+
+def qmatvec_q8k(t: int, w: np.ndarray, n_rows: int, k: int, xq: np.ndarray) -> np.ndarray:
+    w = np.ascontiguousarray(w, dtype=np.uint8).reshape(-1)
+    xq = np.ascontiguousarray(xq, dtype=np.uint8).reshape(-1)
+    assert w.size == n_rows * tensor_size(t, k) and xq.size == (k // 256) * 292
+    y = np.empty(n_rows, dtype=np.float32)
+    rc = lib().pmo_qmatvec_q8k(t, _u8p(w), n_rows, k, _u8p(xq), _f32p(y))
     if rc != OK:
         raise ValueError(rc)
     return y

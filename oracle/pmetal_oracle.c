@@ -594,6 +594,131 @@ void pmo_dequantize_q6k(const uint8_t *src, size_t n, float *dst) {
 }
 
 /* ------------------------------------------------------------------------- */
+/* Q8_K: k_quants.rs:815-871 quantize_q8k; vec_dot.rs:617-692 (scalar)        */
+/* ------------------------------------------------------------------------- */
+size_t pmo_q8k_size(size_t n) { return (n / 256 + (n % 256 != 0)) * 292; }
+
+/* `v as i8` for f32: saturating, NaN -> 0 */
+static int8_t f32_as_i8(float v) {
+    if (v != v) return 0;
+    if (v >= 127.0f) return 127;
+    if (v <= -128.0f) return -128;
+    return (int8_t)v;
+}
+
+void pmo_quantize_q8k(const float *xs, size_t n, uint8_t *dst) {
+    size_t n_blocks = n / 256 + (n % 256 != 0);
+    memset(dst, 0, n_blocks * 292); /* :818-825; a partial last block is skipped (:829-834) */
+    for (size_t b = 0; b + 1 <= n / 256; b++) {
+        const float *x = xs + b * 256;
+        uint8_t *blk = dst + b * 292;
+        /* :837-844 */
+        float max = 0.0f, amax = 0.0f;
+        for (int i = 0; i < 256; i++) {
+            if (fabsf(x[i]) > amax) {
+                amax = fabsf(x[i]);
+                max = x[i];
+            }
+        }
+        if (amax == 0.0f) continue; /* :846-851 */
+        float iscale = -128.0f / max; /* :853 */
+        int8_t q[256];
+        for (int j = 0; j < 256; j++) { /* :854-857: v.round().min(127.0) as i8; f32::min returns the non-NaN operand */
+            float v = roundf(iscale * x[j]);
+            v = rust_min(v, 127.0f);
+            q[j] = f32_as_i8(v);
+        }
+        memcpy(blk + 4, q, 256);
+        for (int j = 0; j < 16; j++) { /* :860-866 */
+            int32_t sum = 0;
+            for (int ii = 0; ii < 16; ii++) sum += q[j * 16 + ii];
+            int16_t s16 = (int16_t)sum;
+            memcpy(blk + 260 + 2 * j, &s16, 2);
+        }
+        float d = 1.0f / iscale; /* :868 */
+        memcpy(blk, &d, 4);
+    }
+}
+
+/* vec_dot.rs:617-656 */
+float pmo_vec_dot_q4k_q8k(const uint8_t *xs, const uint8_t *ys, size_t n_blocks) {
+    float sum = 0.0f;
+    for (size_t b = 0; b < n_blocks; b++) {
+        const uint8_t *x = xs + b * 144, *y = ys + b * 292;
+        uint16_t d16, dmin16;
+        float yd;
+        memcpy(&d16, x, 2);
+        memcpy(&dmin16, x + 2, 2);
+        memcpy(&yd, y, 4);
+        const uint8_t *scales = x + 4, *qs = x + 16;
+        const int8_t *q8 = (const int8_t *)(y + 4);
+        float d = pmo_f16_to_f32(d16) * yd;       /* :621 */
+        float dmin = pmo_f16_to_f32(dmin16) * yd; /* :622 */
+        int32_t mins_sum = 0;                     /* :625-630 */
+        for (int j = 0; j < 8; j++) {
+            uint8_t sc, m;
+            int16_t b0, b1;
+            pmo_get_scale_min_k4(j, scales, &sc, &m);
+            memcpy(&b0, y + 260 + 2 * (2 * j), 2);
+            memcpy(&b1, y + 260 + 2 * (2 * j + 1), 2);
+            mins_sum += (int32_t)m * ((int32_t)b0 + (int32_t)b1);
+        }
+        sum -= dmin * (float)mins_sum; /* :631 */
+        int32_t sumi = 0;              /* :633-650 */
+        for (int j = 0; j < 4; j++) {
+            uint8_t sc0, sc1, m;
+            pmo_get_scale_min_k4(j * 2, scales, &sc0, &m);
+            pmo_get_scale_min_k4(j * 2 + 1, scales, &sc1, &m);
+            for (int k = 0; k < 32; k++) {
+                int32_t q4l = qs[j * 32 + k] & 0x0F, q4h = qs[j * 32 + k] >> 4;
+                sumi += q4l * (int32_t)q8[j * 64 + k] * (int32_t)sc0;
+                sumi += q4h * (int32_t)q8[j * 64 + k + 32] * (int32_t)sc1;
+            }
+        }
+        sum += d * (float)sumi; /* :652 */
+    }
+    return sum;
+}
+
+/* vec_dot.rs:658-692 */
+float pmo_vec_dot_q6k_q8k(const uint8_t *xs, const uint8_t *ys, size_t n_blocks) {
+    float sum = 0.0f;
+    for (size_t b = 0; b < n_blocks; b++) {
+        const uint8_t *x = xs + b * 210, *y = ys + b * 292;
+        const uint8_t *ql = x, *qh = x + 128;
+        const int8_t *scales = (const int8_t *)(x + 192);
+        const int8_t *q8 = (const int8_t *)(y + 4);
+        uint16_t d16;
+        float yd;
+        memcpy(&d16, x + 208, 2);
+        memcpy(&yd, y, 4);
+        float d = pmo_f16_to_f32(d16) * yd; /* :662 */
+        int32_t sumi = 0;
+        for (int j = 0; j < 16; j++) { /* :665-686 */
+            int32_t scale = scales[j];
+            for (int k = 0; k < 16; k++) {
+                int idx = j * 16 + k;
+                uint8_t lo = (idx % 2 == 0) ? (uint8_t)(ql[idx / 2] & 0x0F) : (uint8_t)(ql[idx / 2] >> 4);
+                uint8_t hi = (uint8_t)((qh[idx / 4] >> ((idx % 4) * 2)) & 0x03);
+                int32_t q6 = (int32_t)(lo | (hi << 4)) - 32;
+                sumi += q6 * (int32_t)q8[idx] * scale;
+            }
+        }
+        sum += d * (float)sumi; /* :688 */
+    }
+    return sum;
+}
+
+int32_t pmo_qmatvec_q8k(uint32_t t, const uint8_t *w, size_t n_rows, size_t k, const uint8_t *xq, float *y) {
+    if (t != PMO_TYPE_Q4K && t != PMO_TYPE_Q6K) return PMO_ERR_UNSUPPORTED_TYPE;
+    if (k % 256 != 0) return PMO_ERR_INVALID_SHAPE;
+    size_t spr = k / 256, row = spr * pmo_type_size(t);
+    for (size_t r = 0; r < n_rows; r++)
+        y[r] = t == PMO_TYPE_Q4K ? pmo_vec_dot_q4k_q8k(w + r * row, xq, spr) : pmo_vec_dot_q6k_q8k(w + r * row, xq, spr);
+    return PMO_OK;
+}
+
+/* ------------------------------------------------------------------------- */
 /* quantize.rs:17-87 and dequant.rs:92-132, :184-216                         */
 /* ------------------------------------------------------------------------- */
 int32_t pmo_quantize(uint32_t t, const float *x, size_t n, uint8_t *dst, size_t dst_len) {

@@ -95,6 +95,16 @@ int32_t pmo_is_quantizable_gguf_tensor(const char *gguf_name, size_t ndim);
  * returns the GgmlType id chosen for the tensor. */
 uint32_t pmo_q4km_tensor_type(const char *gguf_name, size_t ndim, size_t n_layers);
 
+/* Q8_K activation blocks and the integer dot products over them.
+ * k_quants.rs:140-155 BlockQ8K {f32 d; i8 qs[256]; i16 bsums[16]} = 292 bytes; :815-871 quantize_q8k (a trailing
+ * partial block stays all-zero); vec_dot.rs:617-656 scalar vec_dot_q4k_q8k, :658-692 scalar vec_dot_q6k_q8k.
+ * pmo_qmatvec_q8k: y[r] = vec_dot(row r of W, xq) for W of type Q4K or Q6K, k a multiple of 256. */
+size_t pmo_q8k_size(size_t n_elements);
+void pmo_quantize_q8k(const float *x, size_t n, uint8_t *dst);
+float pmo_vec_dot_q4k_q8k(const uint8_t *xs, const uint8_t *ys, size_t n_blocks);
+float pmo_vec_dot_q6k_q8k(const uint8_t *xs, const uint8_t *ys, size_t n_blocks);
+int32_t pmo_qmatvec_q8k(uint32_t ggml_type, const uint8_t *w, size_t n_rows, size_t k, const uint8_t *xq, float *y);
+
 /* Not a reference function: "reference dequantize, then matmul", the definition
  * the fused GEMV/GEMM kernels are checked against.  W is [n_rows, k] quantized
  * row-major; x is f32 [k]; y[n] = sum_k W[n,k]*x[k] accumulated in double and

@@ -30,6 +30,7 @@ EXTRA = {
     "gemv.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
     "gemv_q4k.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
     "gemm.hip": [],
+    "q8k.hip": ["-ffp-contract=off", "-fno-gpu-flush-denormals-to-zero"],
     "util.hip": [],
     "api.hip": [],
 }

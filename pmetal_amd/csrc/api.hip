@@ -597,6 +597,42 @@ int32_t pmetal_hip_f32_to_bf16_dev(const float *src, uint16_t *dst, size_t n, vo
     return ok();
 }
 
+// ---- Q8_K activations ----
+size_t pmetal_hip_q8k_size(size_t n) { return (n / 256 + (n % 256 != 0)) * 292; }
+
+int32_t pmetal_hip_quantize_q8k_dev(const float *src, size_t n, uint8_t *dst, size_t dst_len, void *stream) {
+    const size_t expected = pmetal_hip_q8k_size(n);
+    if (dst_len != expected)
+        return fail(PMETAL_HIP_ERR_INVALID_SIZE, "Invalid data size: expected %zu bytes, got %zu", expected, dst_len);
+    if (n == 0) return ok();
+    if (!src || !dst) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
+    if (!aligned16(src) || !aligned16(dst)) return fail(PMETAL_HIP_ERR_INVALID_ARG, "device pointers must be 16-byte aligned");
+    if (int32_t rc = require_device()) return rc;
+    hipError_t e = pmh::launch_quantize_q8k(src, n, dst, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "quantize_q8k kernel launch");
+    return ok();
+}
+
+int32_t pmetal_hip_qgemv_q8k(uint32_t t, const uint8_t *w, int64_t n, int64_t k, const uint8_t *xq, float *y, void *stream) {
+    if (t != PMETAL_GGML_TYPE_Q4K && t != PMETAL_GGML_TYPE_Q6K)
+        return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "qgemv_q8k: GGML type %u has no Q8_K dot product here", t);
+    if (n < 0 || k < 0 || n > 0x7FFFFFFF) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "n and k must be non-negative, n below 2^31");
+    if (k % 256 != 0) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qgemv_q8k: k=%lld is not a multiple of 256", (long long)k);
+    if (k > 32768) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qgemv_q8k: k=%lld exceeds 32768", (long long)k);
+    if (n == 0) return ok();
+    if (!w || !xq || !y) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
+    if (!aligned16(w) || !aligned16(xq) || !aligned16(y)) return fail(PMETAL_HIP_ERR_INVALID_ARG, "device pointers must be 16-byte aligned");
+    if (int32_t rc = require_device()) return rc;
+    if (k == 0) {  // an empty sum
+        hipError_t z = pmh::launch_zero_bytes(reinterpret_cast<uint8_t *>(y), (size_t)n * 4, (hipStream_t)stream);
+        if (z != hipSuccess) return hip_fail(z, "fill kernel launch");
+        return ok();
+    }
+    hipError_t e = pmh::launch_qgemv_q8k(t, w, n, k, xq, y, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "qgemv_q8k kernel launch");
+    return ok();
+}
+
 // ---- measurement aid ----
 int32_t pmetal_hip_mfma_probe_f16(int32_t iters, int32_t vary, int32_t workgroups, float *sink, void *stream) {
     if (iters < 0 || workgroups < 1 || workgroups > 65536) return fail(PMETAL_HIP_ERR_INVALID_ARG, "iters >= 0, 1 <= workgroups <= 65536");

@@ -49,6 +49,11 @@ size_t qgemm_workspace_bytes(int64_t m, int64_t n, int64_t k);
 hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype,
                         int64_t m, void *y, uint32_t y_dtype, uint32_t order, void *workspace, hipStream_t s);
 
+// ---- q8k.hip: Q8_K activation blocks and the integer dot products over them ----
+hipError_t launch_quantize_q8k(const float *x, size_t n, uint8_t *dst, hipStream_t s);
+// k a multiple of 256 and at most 32768 (the activation blocks live in LDS); type Q4_K or Q6_K
+hipError_t launch_qgemv_q8k(uint32_t type, const uint8_t *w, int64_t n, int64_t k, const uint8_t *xq, float *y, hipStream_t s);
+
 // ---- util.hip ----
 hipError_t launch_fill_normal(float *dst, size_t n, uint64_t seed, float std, float outlier_rate,
                               float outlier_mag, hipStream_t s);

@@ -166,6 +166,29 @@ def _dev_ptr(obj) -> int:
     return int(obj)
 
 
+def q8k_size(n_elements: int) -> int:
+    """Bytes of ``n_elements`` quantized to Q8_K (292 per 256, crates/pmetal-gguf/src/k_quants.rs:140-155)."""
+    return _lib.load().pmetal_hip_q8k_size(n_elements)
+
+
+def quantize_q8k_dev(x, n: int, out=None, stream=None) -> DeviceBuffer:
+    """``quantize_q8k`` (crates/pmetal-gguf/src/k_quants.rs:815-871) of ``n`` f32 values on the device."""
+    lib = _lib.load()
+    if out is None:
+        out = DeviceBuffer(max(q8k_size(n), 16))
+    check(lib.pmetal_hip_quantize_q8k_dev(_dev_ptr(x), n, _dev_ptr(out), q8k_size(n), stream), "quantize")
+    return out
+
+
+def qgemv_q8k(dtype: int, w, n: int, k: int, xq, y=None, stream=None) -> DeviceBuffer:
+    """``y[r] = vec_dot_<dtype>_q8k(row r of w, xq)`` (crates/pmetal-gguf/src/vec_dot.rs:617-692), bit for bit."""
+    lib = _lib.load()
+    if y is None:
+        y = DeviceBuffer(max(4 * n, 16))
+    check(lib.pmetal_hip_qgemv_q8k(int(dtype), _dev_ptr(w), n, k, _dev_ptr(xq), _dev_ptr(y), stream))
+    return y
+
+
 class GgufLinear:
     """A GGUF-quantized weight ``[n, k]`` resident on the device; ``forward`` is ``x @ W^T``.
 
