@@ -178,8 +178,8 @@ inline GgmlType q4km_tensor_type(const std::string &gguf_name, size_t ndim, size
 
 
 // quantize(data, dtype) for every type the Q4_K_M recipe yields: F32 and F16 are conversions on the host
-// (crates/pmetal-gguf/src/quantize.rs:19-30), Q8_0 / Q4K / Q6K run on the GPU, anything else is the reference's
-// "not yet implemented" error.
+// (crates/pmetal-gguf/src/quantize.rs:19-30), Q8_0 / Q4K / Q5K / Q6K run on the GPU, anything else is the
+// reference's "not yet implemented" error.
 inline std::vector<uint8_t> quantize_any(const float *data, size_t n, GgmlType dtype) {
     if (dtype == GgmlType::F32) {
         std::vector<uint8_t> out(n * 4);
@@ -260,7 +260,7 @@ struct SourceTensor {
 // The quantize-and-write loop of run_quantization for `--method q4_k_m` over dense tensors
 // (crates/pmetal/src/commands/quantize.rs:1339-1433): tensors in the order of their Hugging Face names, each under
 // its GGUF name, with the type the recipe gives it (norms and 1-D tensors F16, attn_v / ffn_down of the layers that get
-// more bits and the embedding / output matrices Q6_K, the rest Q4_K), quantized by quantize_any.  The builder starts as
+// more bits and the embedding / output matrices Q6_K, a fused attn_qkv Q5_K, the rest Q4_K), quantized by quantize_any.  The builder starts as
 // GgufBuilder::with_model(architecture, "quantized-model"); the caller adds the model's own metadata and writes it.
 inline GgufBuilder quantize_model_q4_k_m(const std::string &architecture, const std::vector<SourceTensor> &weights,
                                          size_t n_layers) {

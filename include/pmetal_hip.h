@@ -37,7 +37,7 @@ extern "C" {
 #define PMETAL_GGML_TYPE_F16 1u
 #define PMETAL_GGML_TYPE_Q8_0 8u
 #define PMETAL_GGML_TYPE_Q4K 12u
-#define PMETAL_GGML_TYPE_Q5K 13u /* named by the recipe only; no kernels */
+#define PMETAL_GGML_TYPE_Q5K 13u /* quantize / dequantize only (k_quants.rs:960-1051, :407-462); no linear kernels */
 #define PMETAL_GGML_TYPE_Q6K 14u
 
 /* Error classes.  1-3, 6, 7 map onto DequantError (crates/pmetal-gguf/src/dequant.rs:37-70)

@@ -322,6 +322,7 @@ size_t pmo_type_size(uint32_t t) {
     case PMO_TYPE_F16: return 2;
     case PMO_TYPE_Q8_0: return 34;
     case PMO_TYPE_Q4K: return 144;
+    case PMO_TYPE_Q5K: return 176;
     case PMO_TYPE_Q6K: return 210;
     default: return 0;
     }
@@ -333,6 +334,7 @@ size_t pmo_block_size(uint32_t t) {
     case PMO_TYPE_F16: return 1;
     case PMO_TYPE_Q8_0: return 32;
     case PMO_TYPE_Q4K:
+    case PMO_TYPE_Q5K:
     case PMO_TYPE_Q6K: return 256;
     default: return 0;
     }
@@ -594,6 +596,115 @@ void pmo_dequantize_q6k(const uint8_t *src, size_t n, float *dst) {
 }
 
 /* ------------------------------------------------------------------------- */
+/* k_quants.rs:960-1051 quantize_q5k, :407-462 dequantize_q5k                */
+/* ------------------------------------------------------------------------- */
+void pmo_quantize_q5k(const float *xs, size_t n, uint8_t *dst) {
+    size_t n_blocks = n / QK_K + (n % QK_K != 0);
+    memset(dst, 0, n_blocks * 176); /* :962-971; a partial last block is skipped (:975-977) */
+    for (size_t b = 0; b < n / QK_K; b++) {
+        const float *x = xs + b * QK_K;
+        uint8_t *blk = dst + b * 176, *sc_bytes = blk + 4, *qh = blk + 16, *qs = blk + 48;
+        float mins[8], scales[8];
+        for (int j = 0; j < 8; j++) pmo_make_qkx1_quants(31, 5, x + 32 * j, 32, &scales[j], &mins[j]); /* :983-985 */
+        float max_scale = 0.0f, max_min = 0.0f; /* :987-988 fold(0.0, |max, val| val.max(max)) */
+        for (int j = 0; j < 8; j++) {
+            max_scale = rust_max(scales[j], max_scale);
+            max_min = rust_max(mins[j], max_min);
+        }
+        float inv_scale = max_scale > 0.0f ? 63.0f / max_scale : 0.0f; /* :990-995 */
+        float inv_min = max_min > 0.0f ? 63.0f / max_min : 0.0f;
+        for (int j = 0; j < 8; j++) { /* :997-1008 */
+            int32_t a = pmo_nearest_int(inv_scale * scales[j]), c = pmo_nearest_int(inv_min * mins[j]);
+            uint8_t ls = (uint8_t)(a < 63 ? a : 63), lm = (uint8_t)(c < 63 ? c : 63);
+            if (j < 4) {
+                sc_bytes[j] = ls;
+                sc_bytes[j + 4] = lm;
+            } else {
+                sc_bytes[j + 4] = (uint8_t)((ls & 0xF) | ((lm & 0xF) << 4));
+                sc_bytes[j - 4] |= (uint8_t)((ls >> 4) << 6);
+                sc_bytes[j] |= (uint8_t)((lm >> 4) << 6);
+            }
+        }
+        uint16_t d16 = pmo_f32_to_f16(max_scale / 63.0f), dmin16 = pmo_f32_to_f16(max_min / 63.0f); /* :1010-1011 */
+        memcpy(blk, &d16, 2);
+        memcpy(blk + 2, &dmin16, 2);
+        uint8_t l[QK_K];
+        memset(l, 0, sizeof l);
+        for (int j = 0; j < 8; j++) { /* :1013-1024 */
+            uint8_t sc, m;
+            pmo_get_scale_min_k4(j, sc_bytes, &sc, &m);
+            float d = pmo_f16_to_f32(d16) * (float)sc;
+            if (d != 0.0f) {
+                float dm = pmo_f16_to_f32(dmin16) * (float)m;
+                for (int ii = 0; ii < 32; ii++)
+                    l[32 * j + ii] = (uint8_t)clamp_i32(pmo_nearest_int((x[32 * j + ii] + dm) / d), 0, 31);
+            }
+        }
+        uint8_t m1 = 1, m2 = 2; /* :1027-1047 */
+        for (int n0 = 0; n0 < QK_K; n0 += 64) {
+            int offset = (n0 / 64) * 32;
+            for (int j = 0; j < 32; j++) {
+                uint8_t l1 = l[n0 + j], l2 = l[n0 + j + 32];
+                if (l1 > 15) {
+                    l1 -= 16;
+                    qh[j] |= m1;
+                }
+                if (l2 > 15) {
+                    l2 -= 16;
+                    qh[j] |= m2;
+                }
+                qs[offset + j] = (uint8_t)(l1 | (l2 << 4));
+            }
+            m1 = (uint8_t)(m1 << 2);
+            m2 = (uint8_t)(m2 << 2);
+        }
+    }
+}
+
+static void dequantize_q5k_block(const uint8_t *blk, float *out, uint32_t order) {
+    uint16_t d16, dmin16;
+    memcpy(&d16, blk, 2);
+    memcpy(&dmin16, blk + 2, 2);
+    const float d = pmo_f16_to_f32(d16), dmin = pmo_f16_to_f32(dmin16);
+    const uint8_t *scales = blk + 4, *qh = blk + 16, *qs = blk + 48;
+    int idx = 0, is = 0;
+    for (int j = 0; j < QK_K; j += 64) { /* :414-459 */
+        uint8_t sc1, m1, sc2, m2;
+        pmo_get_scale_min_k4(is, scales, &sc1, &m1);
+        pmo_get_scale_min_k4(is + 1, scales, &sc2, &m2);
+        const float d1 = d * (float)sc1, dm1 = dmin * (float)m1, d2 = d * (float)sc2, dm2 = dmin * (float)m2;
+        const int q_start = j / 2, qh_start = j / 8, c = j / 64;
+        for (int half = 0; half < 2; half++) {
+            for (int l = 0; l < 32; l++) {
+                uint8_t nib, bit;
+                if (order == PMO_ORDER_REF) { /* :426-438, :442-455 */
+                    const uint8_t byte = qs[q_start + 16 * half + l / 2];
+                    nib = (l % 2 == 0) ? (uint8_t)(byte & 0xF) : (uint8_t)(byte >> 4);
+                    bit = (uint8_t)((qh[qh_start + 4 * half + l / 8] >> (l % 8)) & 1);
+                } else { /* inverse of :1030-1047 */
+                    const uint8_t byte = qs[32 * c + l];
+                    nib = half ? (uint8_t)(byte >> 4) : (uint8_t)(byte & 0xF);
+                    bit = (uint8_t)((qh[l] >> (2 * c + half)) & 1);
+                }
+                const uint8_t q = (uint8_t)(nib | (bit << 4));
+                out[idx++] = half ? d2 * (float)q - dm2 : d1 * (float)q - dm1;
+            }
+        }
+        is += 2;
+    }
+}
+
+void pmo_dequantize_q5k(const uint8_t *src, size_t n, float *dst, uint32_t order) {
+    size_t n_blocks = n / QK_K + (n % QK_K != 0);
+    float tmp[QK_K];
+    for (size_t b = 0; b < n_blocks; b++) {
+        dequantize_q5k_block(src + b * 176, tmp, order);
+        size_t cnt = n - b * QK_K < QK_K ? n - b * QK_K : QK_K;
+        memcpy(dst + b * QK_K, tmp, cnt * sizeof(float));
+    }
+}
+
+/* ------------------------------------------------------------------------- */
 /* Q8_K: k_quants.rs:815-871 quantize_q8k; vec_dot.rs:617-692 (scalar)        */
 /* ------------------------------------------------------------------------- */
 size_t pmo_q8k_size(size_t n) { return (n / 256 + (n % 256 != 0)) * 292; }
@@ -722,17 +833,18 @@ int32_t pmo_qmatvec_q8k(uint32_t t, const uint8_t *w, size_t n_rows, size_t k, c
 /* quantize.rs:17-87 and dequant.rs:92-132, :184-216                         */
 /* ------------------------------------------------------------------------- */
 int32_t pmo_quantize(uint32_t t, const float *x, size_t n, uint8_t *dst, size_t dst_len) {
-    if (t != PMO_TYPE_Q8_0 && t != PMO_TYPE_Q4K && t != PMO_TYPE_Q6K) return PMO_ERR_UNSUPPORTED_TYPE;
+    if (t != PMO_TYPE_Q8_0 && t != PMO_TYPE_Q4K && t != PMO_TYPE_Q5K && t != PMO_TYPE_Q6K) return PMO_ERR_UNSUPPORTED_TYPE;
     if (dst_len != pmo_tensor_size(t, n)) return PMO_ERR_INVALID_SIZE;
     if (t == PMO_TYPE_Q8_0) pmo_quantize_q8_0(x, n, dst);
     else if (t == PMO_TYPE_Q4K) pmo_quantize_q4k(x, n, dst);
+    else if (t == PMO_TYPE_Q5K) pmo_quantize_q5k(x, n, dst);
     else pmo_quantize_q6k(x, n, dst);
     return PMO_OK;
 }
 
 int32_t pmo_dequantize(uint32_t t, const uint8_t *src, size_t src_len, const int32_t *shape, size_t ndim,
                        float *dst, size_t dst_cap, uint32_t order) {
-    if (t != PMO_TYPE_Q8_0 && t != PMO_TYPE_Q4K && t != PMO_TYPE_Q6K) return PMO_ERR_UNSUPPORTED_TYPE;
+    if (t != PMO_TYPE_Q8_0 && t != PMO_TYPE_Q4K && t != PMO_TYPE_Q5K && t != PMO_TYPE_Q6K) return PMO_ERR_UNSUPPORTED_TYPE;
     /* dequant.rs:193-206 shape_n_elements */
     for (size_t i = 0; i < ndim; i++)
         if (shape[i] < 0) return PMO_ERR_INVALID_SHAPE;
@@ -747,6 +859,7 @@ int32_t pmo_dequantize(uint32_t t, const uint8_t *src, size_t src_len, const int
     if (dst_cap < n) return PMO_ERR_INVALID_SIZE;
     if (t == PMO_TYPE_Q8_0) pmo_dequantize_q8_0(src, n, dst);
     else if (t == PMO_TYPE_Q4K) pmo_dequantize_q4k(src, n, dst, order);
+    else if (t == PMO_TYPE_Q5K) pmo_dequantize_q5k(src, n, dst, order);
     else pmo_dequantize_q6k(src, n, dst);
     return PMO_OK;
 }

@@ -30,6 +30,7 @@ enum {
     PMO_TYPE_F16 = 1,
     PMO_TYPE_Q8_0 = 8,
     PMO_TYPE_Q4K = 12,
+    PMO_TYPE_Q5K = 13, /* quantize / dequantize only */
     PMO_TYPE_Q6K = 14,
 };
 
@@ -74,12 +75,16 @@ size_t pmo_tensor_size(uint32_t ggml_type, size_t n_elements);
 void pmo_quantize_q8_0(const float *x, size_t n, uint8_t *dst);
 void pmo_quantize_q4k(const float *x, size_t n, uint8_t *dst);
 void pmo_quantize_q6k(const float *x, size_t n, uint8_t *dst);
+/* k_quants.rs:960-1051 (176-byte blocks: d, dmin, scales[12], qh[32], qs[128]) */
+void pmo_quantize_q5k(const float *x, size_t n, uint8_t *dst);
 
 /* dequant.rs:466-495, k_quants.rs:358-404 + 515-560, k_quants.rs:474-496 + 614-660.
  * src holds pmo_tensor_size(type, n) bytes; dst receives n floats. */
 void pmo_dequantize_q8_0(const uint8_t *src, size_t n, float *dst);
 void pmo_dequantize_q4k(const uint8_t *src, size_t n, float *dst, uint32_t order);
 void pmo_dequantize_q6k(const uint8_t *src, size_t n, float *dst);
+/* k_quants.rs:407-462 + :663-710; order 0 = the reference's emission order, 1 = the inverse of quantize_q5k's packing */
+void pmo_dequantize_q5k(const uint8_t *src, size_t n, float *dst, uint32_t order);
 
 /* quantize.rs:17-87 (dispatcher) and dequant.rs:92-132 + 184-216 (dispatcher and
  * validation).  Return a PMO_* code. */

@@ -49,9 +49,12 @@ int32_t hip_fail(hipError_t e, const char *what) {
         if (_e != hipSuccess) return hip_fail(_e, #expr);  \
     } while (0)
 
+// types with quantized-linear kernels
 bool path_type(uint32_t t) {
     return t == PMETAL_GGML_TYPE_Q8_0 || t == PMETAL_GGML_TYPE_Q4K || t == PMETAL_GGML_TYPE_Q6K;
 }
+// types with quantize / dequantize kernels: the above and Q5_K (the Q4_K_M recipe gives it to fused attn_qkv tensors)
+bool codec_type(uint32_t t) { return path_type(t) || t == PMETAL_GGML_TYPE_Q5K; }
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -165,6 +168,7 @@ size_t pmetal_hip_type_size(uint32_t t) {
     switch (t) {
     case PMETAL_GGML_TYPE_Q8_0: return 34;
     case PMETAL_GGML_TYPE_Q4K: return 144;
+    case PMETAL_GGML_TYPE_Q5K: return 176;
     case PMETAL_GGML_TYPE_Q6K: return 210;
     default: return 0;
     }
@@ -174,6 +178,7 @@ size_t pmetal_hip_block_size(uint32_t t) {
     switch (t) {
     case PMETAL_GGML_TYPE_Q8_0: return 32;
     case PMETAL_GGML_TYPE_Q4K:
+    case PMETAL_GGML_TYPE_Q5K:
     case PMETAL_GGML_TYPE_Q6K: return 256;
     default: return 0;
     }
@@ -185,11 +190,11 @@ size_t pmetal_hip_tensor_size(uint32_t t, size_t n) {
     return (n / bs + (n % bs != 0)) * pmetal_hip_type_size(t);
 }
 
-int32_t pmetal_hip_is_supported(uint32_t t) { return path_type(t) ? 1 : 0; }
+int32_t pmetal_hip_is_supported(uint32_t t) { return codec_type(t) ? 1 : 0; }
 
 int32_t pmetal_hip_expected_byte_size(uint32_t t, const int32_t *shape, size_t ndim, size_t *out_bytes,
                                       size_t *out_elements) {
-    if (!path_type(t)) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "unsupported GGML type %u", t);
+    if (!codec_type(t)) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "unsupported GGML type %u", t);
     size_t n = 0;
     if (int32_t rc = shape_elements(shape, ndim, &n)) return rc;
     const size_t bs = pmetal_hip_block_size(t), ts = pmetal_hip_type_size(t);
@@ -343,7 +348,7 @@ int32_t pmetal_hip_event_destroy(void *event) {
 
 // ---- quantize ----
 int32_t pmetal_hip_quantize_dev(uint32_t t, const float *src, size_t n, uint8_t *dst, size_t dst_len, void *stream) {
-    if (!path_type(t))
+    if (!codec_type(t))
         return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "Quantization to GGML type %u not yet implemented", t);
     const size_t expected = pmetal_hip_tensor_size(t, n);
     if (dst_len != expected)
@@ -356,13 +361,14 @@ int32_t pmetal_hip_quantize_dev(uint32_t t, const float *src, size_t n, uint8_t 
     hipError_t e;
     if (t == PMETAL_GGML_TYPE_Q8_0) e = pmh::launch_quantize_q8_0(src, n, dst, s);
     else if (t == PMETAL_GGML_TYPE_Q4K) e = pmh::launch_quantize_q4k(src, n, dst, s);
+    else if (t == PMETAL_GGML_TYPE_Q5K) e = pmh::launch_quantize_q5k(src, n, dst, s);
     else e = pmh::launch_quantize_q6k(src, n, dst, s);
     if (e != hipSuccess) return hip_fail(e, "quantize kernel launch");
     return ok();
 }
 
 int32_t pmetal_hip_quantize(uint32_t t, const float *src, size_t n, uint8_t *dst, size_t dst_len) {
-    if (!path_type(t))
+    if (!codec_type(t))
         return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "Quantization to GGML type %u not yet implemented", t);
     const size_t expected = pmetal_hip_tensor_size(t, n);
     if (dst_len != expected)
@@ -382,7 +388,7 @@ int32_t pmetal_hip_quantize(uint32_t t, const float *src, size_t n, uint8_t *dst
 // ---- dequantize ----
 int32_t pmetal_hip_dequantize_dev(uint32_t t, const uint8_t *src, size_t src_len, float *dst, size_t n, uint32_t order,
                                   void *stream) {
-    if (!path_type(t)) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "Unsupported quantization type: %u", t);
+    if (!codec_type(t)) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "Unsupported quantization type: %u", t);
     if (order > PMETAL_HIP_ORDER_GGML) return fail(PMETAL_HIP_ERR_INVALID_ARG, "order must be 0 (REF) or 1 (GGML)");
     const size_t expected = pmetal_hip_tensor_size(t, n);
     if (src_len != expected)
@@ -395,6 +401,7 @@ int32_t pmetal_hip_dequantize_dev(uint32_t t, const uint8_t *src, size_t src_len
     hipError_t e;
     if (t == PMETAL_GGML_TYPE_Q8_0) e = pmh::launch_dequantize_q8_0(src, n, dst, s);
     else if (t == PMETAL_GGML_TYPE_Q4K) e = pmh::launch_dequantize_q4k(src, n, dst, order, s);
+    else if (t == PMETAL_GGML_TYPE_Q5K) e = pmh::launch_dequantize_q5k(src, n, dst, order, s);
     else e = pmh::launch_dequantize_q6k(src, n, dst, s);
     if (e != hipSuccess) return hip_fail(e, "dequantize kernel launch");
     return ok();
@@ -402,7 +409,7 @@ int32_t pmetal_hip_dequantize_dev(uint32_t t, const uint8_t *src, size_t src_len
 
 int32_t pmetal_hip_dequantize(uint32_t t, const uint8_t *src, size_t src_len, const int32_t *shape, size_t ndim,
                               float *dst, size_t dst_len, uint32_t order) {
-    if (!path_type(t)) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "Unsupported quantization type: %u", t);
+    if (!codec_type(t)) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "Unsupported quantization type: %u", t);
     if (order > PMETAL_HIP_ORDER_GGML) return fail(PMETAL_HIP_ERR_INVALID_ARG, "order must be 0 (REF) or 1 (GGML)");
     size_t n = 0;
     if (int32_t rc = shape_elements(shape, ndim, &n)) return rc;

@@ -49,8 +49,9 @@ __device__ __forceinline__ float clamp_round(float v, float lo, float hi) {
 // rounding; NaN -> 0 as `as i32` does), then add the largest float below 0.5 and truncate.  For every w in [0, 15] the
 // rounded sum w + 0.49999997 lies on the same side of each integer as w + 0.5 does exactly (checked over all 2^32
 // floats on the CPU), so this is round-half-away without a compare.
-__device__ __forceinline__ float clamp_round_0_15(float v) {
-    const float w = __builtin_fminf(__builtin_fmaxf(v, 0.0f), 15.0f);
+template <int NMAX = 15>
+__device__ __forceinline__ float clamp_round_0_15(float v) {  // NMAX = 31 for the 5-bit quants of Q5_K
+    const float w = __builtin_fminf(__builtin_fmaxf(v, 0.0f), (float)NMAX);
     return __builtin_truncf(w + 0.49999997f);
 }
 
@@ -214,6 +215,63 @@ __global__ __launch_bounds__(256) void k_dequantize_q4k(const uint8_t *__restric
 }
 
 // -------------------------------------------------------------------------------------------
+// Q5_K dequantize (k_quants.rs:407-462 + :663-710): 176-byte blocks {d, dmin, scales[12], qh[32], qs[128]};
+// out = (d*sc) * q - (dmin*m) with q = nibble | fifth bit << 4.  Same launch shape as Q4_K.
+// ORDER 0: the reference's emission order: output l of the first / second half of chunk c takes nibble l % 2 of
+// qs[32 c + 16 half + l / 2] and bit l % 8 of qh[8 c + 4 half + l / 8].  ORDER 1: the inverse of the quantizer's packing
+// (k_quants.rs:1027-1047): nibble `half` of qs[32 c + l] and bit 2 c + half of qh[l].
+// -------------------------------------------------------------------------------------------
+template <int ORDER>
+__global__ __launch_bounds__(256) void k_dequantize_q5k(const uint8_t *__restrict__ src, size_t n,
+                                                         float *__restrict__ dst) {
+    const size_t wave = ((size_t)blockIdx.x * 256 + threadIdx.x) >> 6;
+    const int i = (int)(threadIdx.x & 63);
+    const int c = i >> 4;        // 64-element chunk
+    const int p = (i & 15) * 4;  // position inside the chunk
+    const int half = p >> 5, l = p & 31;
+    const int sb = 2 * c + half;
+    uint4 hdr[kDeqUnroll];
+    uint32_t q[kDeqUnroll], h[kDeqUnroll];
+#pragma unroll
+    for (int u = 0; u < kDeqUnroll; u++) {
+        const size_t blk_i = wave * kDeqUnroll + u;
+        const bool live = blk_i * 256 + (size_t)i * 4 < n;
+        const uint8_t *blk = src + (live ? blk_i : 0) * 176;  // lanes past the end re-read the first block
+        hdr[u] = *reinterpret_cast<const uint4 *>(blk);
+        if (ORDER == 0) {
+            q[u] = *reinterpret_cast<const uint16_t *>(blk + 48 + 32 * c + 16 * half + (l >> 1));
+            h[u] = (uint32_t)blk[16 + 8 * c + 4 * half + (l >> 3)] >> (l & 7);
+        } else {
+            q[u] = *reinterpret_cast<const uint32_t *>(blk + 48 + 32 * c + l);
+            h[u] = *reinterpret_cast<const uint32_t *>(blk + 16 + l) >> (2 * c + half);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kDeqUnroll; u++) {
+        const size_t e = (wave * kDeqUnroll + u) * 256 + (size_t)i * 4;
+        if (e >= n) continue;
+        const float d = f16_bits_to_f32(hdr[u].x & 0xFFFFu), dmin = f16_bits_to_f32(hdr[u].x >> 16);
+        uint32_t sc, m;
+        scale_min_k4(sb, hdr[u].y, hdr[u].z, hdr[u].w, sc, m);
+        const float d1 = d * (float)sc;
+        const float dm1 = dmin * (float)m;
+        float o[4];
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            uint32_t v;
+            if (ORDER == 0) v = ((q[u] >> (4 * t)) & 0xFu) | (((h[u] >> t) & 1u) << 4);
+            else v = (((half ? q[u] >> 4 : q[u]) >> (8 * t)) & 0xFu) | (((h[u] >> (8 * t)) & 1u) << 4);
+            o[t] = d1 * (float)v - dm1;
+        }
+        if (e + 3 < n) {
+            *reinterpret_cast<float4 *>(dst + e) = make_float4(o[0], o[1], o[2], o[3]);
+        } else {
+            for (int t = 0; t < 4 && e + t < n; t++) dst[e + t] = o[t];
+        }
+    }
+}
+
+// -------------------------------------------------------------------------------------------
 // Q6_K dequantize (k_quants.rs:474-496 + :614-660): out = (d * sc) * q, left-associated.  Same launch shape.
 // -------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void k_dequantize_q6k(const uint8_t *__restrict__ src, size_t n,
@@ -265,8 +323,14 @@ __global__ __launch_bounds__(256) void k_dequantize_q6k(const uint8_t *__restric
 // -------------------------------------------------------------------------------------------
 constexpr int kQ4kLdsStride = 33;  // 32 floats + 1 pad: lanes read column-wise without bank conflicts
 
+// NMAX = 15: Q4_K (k_quants.rs:876-955).  NMAX = 31: Q5_K (k_quants.rs:960-1051), the same search and scale packing with
+// 5-bit quants: 176-byte blocks, the low four bits packed like Q4_K behind 32 bytes qh, where bit j of qh[l] is the
+// fifth bit of element l of sub-block j.
+template <int NMAX>
 __global__ __launch_bounds__(64) void k_quantize_q4k(const float *__restrict__ x, size_t n_sb,
                                                       uint8_t *__restrict__ dst) {
+    constexpr bool Q5 = NMAX == 31;
+    constexpr int kBytes = Q5 ? 176 : 144, kQsOff = Q5 ? 48 : 16;
     __shared__ float xs[64 * kQ4kLdsStride];
     const int lane = threadIdx.x;
     const size_t sb0 = (size_t)blockIdx.x * 8;
@@ -285,7 +349,7 @@ __global__ __launch_bounds__(64) void k_quantize_q4k(const float *__restrict__ x
 #pragma unroll
     for (int i = 0; i < 32; i++) xv[i] = xs[lane * kQ4kLdsStride + i];
 
-    // ---- make_qkx1_quants(15, 5, xv) ----
+    // ---- make_qkx1_quants(NMAX, 5, xv) ----
     // min_by / max_by with total_cmp: equal keys are identical floats, so integer min / max of the keys will do
     int kmn = total_key(xv[0]), kmx = kmn;
 #pragma unroll
@@ -299,19 +363,19 @@ __global__ __launch_bounds__(64) void k_quantize_q4k(const float *__restrict__ x
     float scale = 0.0f, neg_min = 0.0f;  // returned (scale, -min)
     if (!(mx == mn)) {
         float minv = __builtin_fminf(mn, 0.0f);
-        float iscale = 15.0f / (mx - minv);
+        float iscale = (float)NMAX / (mx - minv);
         scale = 1.0f / iscale;
         float lf[32];  // the quants of the previous try, as floats
 #pragma unroll
         for (int i = 0; i < 32; i++) lf[i] = 0.0f;
 #pragma unroll  // unrolled so that the quants of try t and t - 1 live in different registers without copies
         for (int t = 0; t < 5; t++) {
-            float sumlx = 0.0f, suml2 = 0.0f;  // suml2 is an integer <= 7200: exact in f32, with or without fusing
+            float sumlx = 0.0f, suml2 = 0.0f;  // suml2 is an integer <= 32 NMAX^2 < 2^24: exact in f32, with or without fusing
             bool changed = false;
 #pragma unroll
             for (int i = 0; i < 32; i++) {
                 const float xm = xv[i] - minv;
-                const float r = clamp_round_0_15(iscale * xm);
+                const float r = clamp_round_0_15<NMAX>(iscale * xm);
                 changed |= (r != lf[i]);
                 lf[i] = r;
                 sumlx += xm * r;
@@ -374,7 +438,7 @@ __global__ __launch_bounds__(64) void k_quantize_q4k(const float *__restrict__ x
     // ---- requantize with the decoded f16 scales (k_quants.rs:932-943) ----
     // L = clamp(nearest_int((x + dm) / dq), 0, 15).  Only the integer matters, so the IEEE division (ten instructions)
     // is replaced by a multiplication with 1 / dq wherever that provably gives the same integer: the product differs
-    // from the correctly rounded quotient by less than 3e-6 for quotients below 16, so if it stays 8e-6 away from every
+    // from the correctly rounded quotient by less than 3e-6 for quotients below 32, so if it stays 8e-6 away from every
     // rounding boundary n + 0.5 both round alike.  A lane that sees a product closer than that (or a dq outside the
     // range where 1 / dq and the product are normal numbers) redoes its sub-block with the division.
     uint32_t lb[8] = {0, 0, 0, 0, 0, 0, 0, 0};  // 32 quants, one per byte
@@ -387,7 +451,7 @@ __global__ __launch_bounds__(64) void k_quantize_q4k(const float *__restrict__ x
         for (int w = 0; w < 8; w++) {
 #pragma unroll
             for (int c = 0; c < 4; c++) {
-                const float q = __builtin_fminf(__builtin_fmaxf((xv[4 * w + c] + dm) * rinv, 0.0f), 15.0f);
+                const float q = __builtin_fminf(__builtin_fmaxf((xv[4 * w + c] + dm) * rinv, 0.0f), (float)NMAX);
                 const float r = __builtin_truncf(q + 0.49999997f);
                 exact_needed |= !(__builtin_fabsf(__builtin_fabsf(q - r) - 0.5f) >= 8e-6f);
                 lb[w] |= (uint32_t)r << (8 * c);
@@ -398,7 +462,7 @@ __global__ __launch_bounds__(64) void k_quantize_q4k(const float *__restrict__ x
             for (int w = 0; w < 8; w++) {
                 lb[w] = 0;
 #pragma unroll
-                for (int c = 0; c < 4; c++) lb[w] |= (uint32_t)clamp_round_0_15((xv[4 * w + c] + dm) / dq) << (8 * c);
+                for (int c = 0; c < 4; c++) lb[w] |= (uint32_t)clamp_round_0_15<NMAX>((xv[4 * w + c] + dm) / dq) << (8 * c);
             }
         }
     }
@@ -406,6 +470,20 @@ __global__ __launch_bounds__(64) void k_quantize_q4k(const float *__restrict__ x
     // Even sub-block 2c supplies the low nibbles, odd 2c+1 the high ones.  The even lane emits bytes
     // l = 0..15 of the pair, the odd lane bytes 16..31.
     const bool odd = lane & 1;
+    uint32_t qh_word = 0;
+    if (Q5) {
+        // qh[l] |= 1 << j where L_j[l] > 15 (k_quants.rs:1027-1047): this lane's fifth bits at bit j of every byte, ored
+        // over the eight lanes of the super-block; lane j then keeps dword j (bytes 4 j .. 4 j + 3)
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+            uint32_t h = ((lb[w] >> 4) & 0x01010101u) << j;
+            h |= __shfl_xor(h, 1);
+            h |= __shfl_xor(h, 2);
+            h |= __shfl_xor(h, 4);
+            qh_word = j == w ? h : qh_word;
+            lb[w] &= 0x0F0F0F0Fu;
+        }
+    }
     uint32_t outw[4];
 #pragma unroll
     for (int w = 0; w < 4; w++) {
@@ -415,8 +493,9 @@ __global__ __launch_bounds__(64) void k_quantize_q4k(const float *__restrict__ x
     }
     const size_t sb = sb0 + (lane >> 3);
     if (sb < n_sb) {
-        uint8_t *blk = dst + sb * 144;
-        *reinterpret_cast<uint4 *>(blk + 16 + 16 * j) = make_uint4(outw[0], outw[1], outw[2], outw[3]);
+        uint8_t *blk = dst + sb * kBytes;
+        *reinterpret_cast<uint4 *>(blk + kQsOff + 16 * j) = make_uint4(outw[0], outw[1], outw[2], outw[3]);
+        if (Q5) *reinterpret_cast<uint32_t *>(blk + 16 + 4 * j) = qh_word;
         if (j < 4) {
             blk[4 + j] = (uint8_t)byte_a;
             blk[8 + j] = (uint8_t)byte_b;
@@ -660,7 +739,18 @@ hipError_t launch_quantize_q4k(const float *x, size_t n, uint8_t *dst, hipStream
         if (e != hipSuccess) return e;
     }
     if (n_sb == 0) return hipSuccess;
-    hipLaunchKernelGGL(k_quantize_q4k, dim3(grid_for(n_sb, 8)), dim3(64), 0, s, x, n_sb, dst);
+    hipLaunchKernelGGL(k_quantize_q4k<15>, dim3(grid_for(n_sb, 8)), dim3(64), 0, s, x, n_sb, dst);
+    return hipGetLastError();
+}
+
+hipError_t launch_quantize_q5k(const float *x, size_t n, uint8_t *dst, hipStream_t s) {
+    const size_t n_sb = n / 256;  // full super-blocks; a trailing partial one is zero bytes
+    if (n % 256) {
+        hipError_t e = launch_zero_bytes(dst + n_sb * 176, 176, s);
+        if (e != hipSuccess) return e;
+    }
+    if (n_sb == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_quantize_q4k<31>, dim3(grid_for(n_sb, 8)), dim3(64), 0, s, x, n_sb, dst);
     return hipGetLastError();
 }
 
@@ -678,6 +768,14 @@ hipError_t launch_quantize_q6k(const float *x, size_t n, uint8_t *dst, hipStream
 hipError_t launch_dequantize_q8_0(const uint8_t *src, size_t n, float *dst, hipStream_t s) {
     if (n == 0) return hipSuccess;
     hipLaunchKernelGGL(k_dequantize_q8_0, dim3(grid_for((n + 3) / 4, 256)), dim3(256), 0, s, src, n, dst);
+    return hipGetLastError();
+}
+
+hipError_t launch_dequantize_q5k(const uint8_t *src, size_t n, float *dst, uint32_t order, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    const dim3 grid(grid_for((n + 4 * kDeqUnroll - 1) / (4 * kDeqUnroll), 256));
+    if (order == kOrderRef) hipLaunchKernelGGL(k_dequantize_q5k<0>, grid, dim3(256), 0, s, src, n, dst);
+    else hipLaunchKernelGGL(k_dequantize_q5k<1>, grid, dim3(256), 0, s, src, n, dst);
     return hipGetLastError();
 }
 

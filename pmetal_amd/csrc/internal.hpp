@@ -7,16 +7,18 @@
 
 namespace pmh {
 
-constexpr uint32_t kTypeQ8_0 = 8, kTypeQ4K = 12, kTypeQ6K = 14;
+constexpr uint32_t kTypeQ8_0 = 8, kTypeQ4K = 12, kTypeQ5K = 13, kTypeQ6K = 14;
 constexpr uint32_t kOrderRef = 0, kOrderGgml = 1;
 constexpr uint32_t kDtypeF32 = 0, kDtypeBf16 = 1;
 
 // ---- codec.hip: bit-exact quantize / dequantize (compiled without fp contraction) ----
 hipError_t launch_quantize_q8_0(const float *x, size_t n, uint8_t *dst, hipStream_t s);
 hipError_t launch_quantize_q4k(const float *x, size_t n, uint8_t *dst, hipStream_t s);
+hipError_t launch_quantize_q5k(const float *x, size_t n, uint8_t *dst, hipStream_t s);
 hipError_t launch_quantize_q6k(const float *x, size_t n, uint8_t *dst, hipStream_t s);
 hipError_t launch_dequantize_q8_0(const uint8_t *src, size_t n, float *dst, hipStream_t s);
 hipError_t launch_dequantize_q4k(const uint8_t *src, size_t n, float *dst, uint32_t order, hipStream_t s);
+hipError_t launch_dequantize_q5k(const uint8_t *src, size_t n, float *dst, uint32_t order, hipStream_t s);
 hipError_t launch_dequantize_q6k(const uint8_t *src, size_t n, float *dst, hipStream_t s);
 
 // ---- gemv.hip: dequant-fused y = W x ----

@@ -376,7 +376,8 @@ def test_quantize_model_q4_k_m_file_equals_oracle(oracle, tmp_path):
     subprocess.run(["g++", "-std=c++17", "-O1", "-Wall", "-I", os.path.join(ROOT, "include"), SRC, "-o", exe, "-L", LIBDIR,
                     "-lpmetal_hip", f"-Wl,-rpath,{LIBDIR}", "-Wl,-rpath,/opt/rocm/lib"], check=True)
     layers, hidden, inter, kv, vocab = 9, 512, 1280, 256, 1000
-    tensors = [("model.embed_tokens.weight", [vocab, hidden]), ("model.norm.weight", [hidden]), ("lm_head.weight", [vocab, hidden])]
+    tensors = [("model.embed_tokens.weight", [vocab, hidden]), ("model.norm.weight", [hidden]), ("lm_head.weight", [vocab, hidden]),
+               ("blk.1.attn_qkv.weight", [3 * 256, hidden])]  # already GGUF-named, fused: the recipe gives it Q5_K
     for layer in range(layers):
         p = f"model.layers.{layer}."
         tensors += [(p + "input_layernorm.weight", [hidden]), (p + "post_attention_layernorm.weight", [hidden]),
@@ -409,7 +410,7 @@ def test_quantize_model_q4_k_m_file_equals_oracle(oracle, tmp_path):
         types[t] = types.get(t, 0) + 1
     b.add_metadata("qwen3.block_count", ("u32", layers))
     want = b.build_to_bytes()
-    assert set(types) == {1, 12, 14} and types[14] >= 4  # F16 norms, Q4_K, Q6_K on the embedding / output / more-bits layers
+    assert set(types) == {1, 12, 13, 14} and types[14] >= 4  # F16 norms, Q4_K, Q5_K (fused qkv), Q6_K on the embedding / output / more-bits layers
     got = open(out, "rb").read()
     assert len(got) == len(want)
     assert got == want

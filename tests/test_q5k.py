@@ -1,0 +1,140 @@
+"""Q5_K quantize / dequantize (crates/pmetal-gguf/src/k_quants.rs:960-1051, :407-462): the oracle against what pins it,
+the HIP kernels against the oracle bit for bit.  Q5_K is what the Q4_K_M recipe gives a fused attn_qkv tensor."""
+import numpy as np
+import pytest
+
+Q5K = 13
+
+
+def q5k_block(d, dmin, sc, m, L):
+    """A block from its parts, packed as quantize_q5k packs (k_quants.rs:997-1008, :1027-1047)."""
+    scales = np.zeros(12, dtype=np.uint8)
+    for j in range(8):
+        if j < 4:
+            scales[j] |= sc[j] & 63
+            scales[j + 4] |= m[j] & 63
+        else:
+            scales[j + 4] = (sc[j] & 0xF) | ((m[j] & 0xF) << 4)
+            scales[j - 4] |= (sc[j] >> 4) << 6
+            scales[j] |= (m[j] >> 4) << 6
+    L = np.asarray(L, dtype=np.uint8).reshape(4, 2, 32)
+    qs = ((L[:, 0, :] & 15) | ((L[:, 1, :] & 15) << 4)).reshape(-1)
+    qh = np.zeros(32, dtype=np.uint8)
+    for c in range(4):
+        qh |= ((L[c, 0, :] >> 4) << (2 * c)).astype(np.uint8) | ((L[c, 1, :] >> 4) << (2 * c + 1)).astype(np.uint8)
+    return np.frombuffer(np.float16(d).tobytes() + np.float16(dmin).tobytes() + scales.tobytes() + qh.tobytes() + qs.tobytes(),
+                         dtype=np.uint8)
+
+
+def test_q5k_sizes_and_zero_blocks(oracle):
+    assert oracle.tensor_size(Q5K, 256) == 176 and oracle.tensor_size(Q5K, 257) == 352  # k_quants.rs:162, types.rs:115
+    assert not oracle.quantize(Q5K, np.zeros(512, np.float32)).any()
+    assert not oracle.quantize(Q5K, np.full(256, 0.37, np.float32)).any()  # max == min in every sub-block -> (0, 0)
+    blk = oracle.quantize(Q5K, np.ones(300, np.float32))
+    assert blk.size == 352 and not blk[176:].any()  # a partial trailing block stays zero (k_quants.rs:975-977)
+
+
+def test_q5k_exact_grid_block_is_packed_as_derived_by_hand(oracle):
+    """x = 0, 1, ..., 31 in every sub-block: min 0, max 31, iscale 1 -> l = x, scale 1.0, min -0.0 (quantize.rs:583-644).
+    All eight scales are 1.0 -> max_scale 1, ls = 63 each, lm = 0, d = f16(1 / 63); requantizing with the decoded d:
+    d * 63 is 1 to within 2e-4, so L = x again.  The bytes follow from the packing rules."""
+    x = np.tile(np.arange(32, dtype=np.float32), 8)
+    got = oracle.quantize(Q5K, x)
+    want = q5k_block(1.0 / 63.0, 0.0, [63] * 8, [0] * 8, np.tile(np.arange(32), 8))
+    assert np.array_equal(got, want)
+    # qh: elements 16..31 of every sub-block carry the fifth bit: bytes 16..31 of qh are 0xFF, bytes 0..15 are 0
+    assert (got[16:32] == 0).all() and (got[32:48] == 0xFF).all()
+    # and both dequantization orders: the inverse of the packing gives the grid back; the reference's own order does not
+    d = np.float32(np.float16(1.0 / 63.0)) * np.float32(63)
+    back = oracle.dequantize(Q5K, got, [256], order=oracle.ORDER_GGML)
+    assert np.array_equal(back, (d * x).astype(np.float32))
+    ref = oracle.dequantize(Q5K, got, [256], order=oracle.ORDER_REF)
+    assert not np.array_equal(ref, back)
+
+
+def test_q5k_dequantize_single_positions(oracle):
+    """One non-zero quant: where the reference's order (k_quants.rs:414-459) and the packing's inverse put it."""
+    rng = np.random.default_rng(2)
+    for _ in range(300):
+        e = int(rng.integers(256))
+        q = int(rng.integers(1, 32))
+        sc = [int(v) for v in rng.integers(1, 64, 8)]
+        L = np.zeros(256, np.uint8)
+        L[e] = q
+        blk = q5k_block(1.0, 0.0, sc, [0] * 8, L)
+        ggml = oracle.dequantize(Q5K, blk, [256], order=oracle.ORDER_GGML)
+        assert np.count_nonzero(ggml) == 1 and ggml[e] == float(sc[e // 32] * q)
+        # the reference's order: nibble and fifth bit are looked up separately, so one stored quant can surface as a
+        # nibble at one output and as a 16 at another.  Follow the lookups by hand:
+        c, p = e // 64, e % 64
+        byte, hi_nibble = 32 * c + (p % 32), p >= 32          # where the packing put the low four bits
+        half, r = (byte % 32) // 16, byte % 16                 # REF reads qs[32 c + 16 half + l / 2]: l = 2 r (+ 1 for the high nibble)
+        out_nib = 64 * c + 32 * half + 2 * r + (1 if hi_nibble else 0)
+        qh_byte, qh_bit = p % 32, 2 * c + (1 if p >= 32 else 0)  # where the packing put the fifth bit
+        c2, rest = qh_byte // 8, qh_byte % 8                   # REF reads qh[8 c2 + 4 half2 + l / 8] bit l % 8
+        half2, l2 = rest // 4, 8 * (rest % 4) + qh_bit
+        out_bit = 64 * c2 + 32 * half2 + l2
+        want = np.zeros(256, np.float32)
+        if q & 15:
+            want[out_nib] += float(sc[out_nib // 32] * (q & 15))
+        if q >> 4:
+            want[out_bit] += float(sc[out_bit // 32] * 16)
+        ref = oracle.dequantize(Q5K, blk, [256], order=oracle.ORDER_REF)
+        assert np.array_equal(ref, want), (e, q)
+
+
+def test_q5k_round_trip_bounds(oracle):
+    """The reference's round-trip style bound (k_quants.rs:1446-1509 for its siblings), in the packing's order."""
+    x = ((np.arange(256) - 128.0) * 0.01).astype(np.float32)
+    back = oracle.dequantize(Q5K, oracle.quantize(Q5K, x), [256], order=oracle.ORDER_GGML)
+    assert np.sqrt(np.mean((back - x) ** 2)) < 0.05 and np.abs(back - x).max() < 0.15
+    rng = np.random.default_rng(3)
+    x = (rng.standard_normal(256 * 64) * 0.02).astype(np.float32)
+    q = oracle.quantize(Q5K, x)
+    back = oracle.dequantize(Q5K, q, [x.size], order=oracle.ORDER_GGML)
+    rel = np.sqrt(np.mean((back - x) ** 2)) / np.sqrt(np.mean(x ** 2))
+    assert rel < 0.04  # 5 bits: about half the error of Q4_K
+    q4 = oracle.dequantize(12, oracle.quantize(12, x), [x.size], order=oracle.ORDER_GGML)
+    assert rel < 0.7 * np.sqrt(np.mean((q4 - x) ** 2)) / np.sqrt(np.mean(x ** 2))
+
+
+@pytest.mark.gpu
+def test_gpu_q5k_quantize_and_dequantize_bit_exact(oracle):
+    import pmetal_amd as pm
+    from gpu_util import first_mismatch, gpu_dequantize_dev, gpu_quantize_dev, weights
+    from test_gpu_codec import edge_inputs
+    pm.init(0)
+    cases = dict(edge_inputs(256))
+    cases["random"] = weights(55, 1 << 20, outliers=1e-3)
+    cases["grid"] = np.tile(np.arange(32, dtype=np.float32), 64)
+    for name, x in cases.items():
+        want = oracle.quantize(Q5K, x)
+        got = gpu_quantize_dev(Q5K, x)
+        assert np.array_equal(got, want), f"{name}: {first_mismatch(got, want, 176)}"
+        if x.size == 0:
+            continue
+        for order in (0, 1):
+            wd = oracle.dequantize(Q5K, want, [x.size], order=order)
+            gd = gpu_dequantize_dev(Q5K, want, x.size, order=order)
+            nan = np.isnan(wd)
+            assert np.array_equal(np.isnan(gd), nan), (name, order)
+            assert np.array_equal(gd[~nan].view(np.uint32), wd[~nan].view(np.uint32)), (name, order)
+    # every bit pattern of a block, including f16 infinities and NaNs in d / dmin
+    rng = np.random.default_rng(9)
+    raw = rng.integers(0, 256, 176 * 4096, dtype=np.uint8)
+    for order in (0, 1):
+        wd = oracle.dequantize(Q5K, raw, [4096 * 256], order=order)
+        gd = gpu_dequantize_dev(Q5K, raw, 4096 * 256, order=order)
+        nan = np.isnan(wd)
+        assert np.array_equal(np.isnan(gd), nan)
+        assert np.array_equal(gd[~nan].view(np.uint32), wd[~nan].view(np.uint32))
+    # ragged lengths through the host-pointer entry points
+    for n in (1, 255, 257, 1000):
+        x = weights(n, n)
+        assert np.array_equal(pm.quantize(x, Q5K), oracle.quantize(Q5K, x))
+        assert np.array_equal(pm.dequantize(oracle.quantize(Q5K, x), Q5K, [n]), oracle.dequantize(Q5K, oracle.quantize(Q5K, x), [n]))
+    # no linear kernels for Q5_K: the reference's error class, not a crash
+    lib = pm._lib.load()
+    buf = pm.DeviceBuffer(1 << 16)
+    assert lib.pmetal_hip_qgemv(Q5K, buf.ptr, 4, 256, buf.ptr, 1, buf.ptr, 0, None) == 2
+    lib.pmetal_hip_clear_error()
