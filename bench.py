@@ -264,6 +264,59 @@ def cpu_baseline_gemv_q8k(t, n, k, budget_s=12.0):
             "sample": f"{reps} x (quantize_q8k + vec_dot over {rows}x{k} rows of the same shape), {dt:.1f} s"}
 
 
+def bench_calibrate(args, n, k):
+    """One step = the round trips of calibrate_tensor for one resident 14336 x 4096 f32 tensor: for each candidate type
+    with kernels here (Q8_K, Q6_K, Q5_K, Q4_K) quantize, dequantize, score."""
+    pm, _lib, lib = load()
+    timer = Timer(pm, lib)
+    ne = n * k
+    x = pm.DeviceBuffer(4 * ne)
+    pm.check(lib.pmetal_hip_fill_normal_f32(x.ptr, ne, 11, 0.02, 1e-3, 0.5, None))
+    deq = pm.DeviceBuffer(4 * ne)
+    cands = [15, 14, 13, 12]
+    qs = {t: pm.DeviceBuffer(lib.pmetal_hip_tensor_size(t, ne)) for t in cands}
+    scores = {}
+    import ctypes as C
+
+    def step():
+        for t in cands:
+            nb = lib.pmetal_hip_tensor_size(t, ne)
+            pm.check(lib.pmetal_hip_quantize_dev(t, x.ptr, ne, qs[t].ptr, nb, None))
+            pm.check(lib.pmetal_hip_dequantize_dev(t, qs[t].ptr, nb, deq.ptr, ne, 1, None))
+            sc = C.c_double()
+            pm.check(lib.pmetal_hip_kl_divergence_dev(x.ptr, deq.ptr, ne, C.byref(sc), None))
+            scores[t] = sc.value
+
+    steps, warm = max(1, args.steps // 20), max(1, args.warmup // 10)
+    ev_ms, wall_ms = timer.run(step, steps, warm)
+    # per candidate: quantize reads 4n and writes the blocks, dequantize reads them and writes 4n, the metric reads 8n
+    bytes_per_step = sum(4 * ne + 2 * lib.pmetal_hip_tensor_size(t, ne) + 4 * ne + 8 * ne for t in cands)
+    gbs = 4.0 * ne * len(cands) / (wall_ms / steps * 1e-3) / 1e9
+    res = {
+        "value": gbs, "ms_per_step": wall_ms / steps, "event_ms_per_step": ev_ms / steps,
+        "roofline": {"bound": "hbm", "achieved": round(bytes_per_step / (wall_ms / steps * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(bytes_per_step / (wall_ms / steps * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "k_quantize_* / k_dequantize_* / k_kl_sums", "bytes_per_step": bytes_per_step},
+        "extra": {"scores": {str(t): scores[t] for t in cands}, "steps_run": steps},
+    }
+    args.steps, args.warmup = steps, warm
+    return res, (Q4K, n, k)
+
+
+def cpu_baseline_calibrate(budget_elems=1 << 20):
+    """Oracle: calibrate_tensor (quantize, dequantize, score for the same four candidates), one thread, on 2^20 elements."""
+    from oracle import binding as oracle
+    oracle.build()
+    x = (np.random.default_rng(3).standard_normal(budget_elems) * 0.02).astype(np.float32)
+    reps, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < 10.0:
+        oracle.calibrate_tensor("blk.0.ffn_up.weight", x, [budget_elems // 256, 256], candidates=(15, 14, 13, 12), order=1)
+        reps += 1
+    dt = time.perf_counter() - t0
+    return {"value": round(4.0 * budget_elems * 4 * reps / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{reps} x calibrate_tensor over {budget_elems} elements, four candidates, {dt:.1f} s"}
+
+
 def bench_gemm(args, m, n, k, t=Q4K):
     pm, _lib, lib = load()
     timer = Timer(pm, lib)
@@ -441,6 +494,8 @@ WORKLOADS["gemv_q4k_q8k_14336x4096"] = dict(kind="gemv_q8k", n=14336, k=4096, ty
                                             metric="Q4_K x Q8_K integer-dot GEMV GB/s @14336x4096 (activation quantize included)")
 WORKLOADS["gemv_q6k_q8k_14336x4096"] = dict(kind="gemv_q8k", n=14336, k=4096, type=Q6K, unit="GB/s", dtype="i8",
                                             metric="Q6_K x Q8_K integer-dot GEMV GB/s @14336x4096 (activation quantize included)")
+WORKLOADS["calibrate_14336x4096"] = dict(kind="calibrate", n=14336, k=4096, unit="GB/s", dtype="f32",
+                                         metric="KL calibration GB/s of f32 evaluated (4 candidates, quantize + dequantize + score) @14336x4096")
 WORKLOADS["decode_qwen3_0.6b_q4km"] = dict(kind="decode", metric="Q4_K_M decode linears tokens/s (Qwen3-0.6B shape)", unit="tokens/s",
                                            dtype="bf16")
 WORKLOADS["quantize_llama3_8b_q4km"] = dict(kind="quantize", metric="f32->Q4_K_M quantize GB/s of f32 consumed (Llama-3-8B shape)",
@@ -480,6 +535,8 @@ def main():
         res, (t, n, k) = bench_dequantize(args, wl["n"], wl["k"])
     elif wl["kind"] == "gemv_q8k":
         res, (t, n, k) = bench_gemv_q8k(args, wl["n"], wl["k"], wl["type"])
+    elif wl["kind"] == "calibrate":
+        res, (t, n, k) = bench_calibrate(args, wl["n"], wl["k"])
     else:
         res, (t, n, k) = bench_gemv(args, wl["n"], wl["k"])
     out = {
@@ -488,11 +545,13 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": wl["dtype"],
         "data": ("synthetic: N(0,0.02) f32 with 0.1% outliers at +-0.5, generated on the device" if wl["kind"] == "quantize"
                  else "synthetic: N(0,0.02) f32 weights generated and quantized on the device, x ~ N(0,1) f32" if wl["kind"] == "gemv_q8k"
+                 else "synthetic: N(0,0.02) f32 with 0.1% outliers at +-0.5, generated on the device" if wl["kind"] == "calibrate"
                  else "synthetic: N(0,0.02) f32 weights generated and quantized on the device, x ~ N(0,1) bf16"),
-        "config": {"workload": args.workload, "element_order": "REF",
+        "config": {"workload": args.workload, "element_order": "GGML" if wl["kind"] == "calibrate" else "REF",
                    "step": {"gemm": "one GEMM launch (activation pre-pass + MFMA kernel)",
                             "gemv": "16 back-to-back GEMVs over 16 distinct weight tensors (528 MB, HBM-resident)",
                             "gemv_q8k": "16 x (activations f32 -> Q8_K, integer-dot GEMV) over 16 distinct weight tensors",
+                            "calibrate": "one tensor resident in HBM: 4 candidates x (quantize, dequantize, f64 score read back)",
                             "decode": "all 197 batch-1 projections of one token, back to back on one stream",
                             "dequantize": "two tensors of 14336 x 4096, blocks resident in HBM",
                             "quantize": "all 226 tensors of the model, f32 resident in HBM"}[wl["kind"]]},
@@ -513,6 +572,8 @@ def main():
             out["cpu_baseline"] = cpu_baseline_gemv(t, n, k)
         elif wl["kind"] == "gemv_q8k":
             out["cpu_baseline"] = cpu_baseline_gemv_q8k(t, n, k)
+        elif wl["kind"] == "calibrate":
+            out["cpu_baseline"] = cpu_baseline_calibrate()
         elif wl["kind"] == "quantize":
             out["cpu_baseline"] = cpu_baseline_quantize()
         elif wl["kind"] == "gemm":

@@ -170,6 +170,66 @@ inline DeviceBuffer qgemv_q8k(GgmlType dtype, const DeviceBuffer &w, int64_t n, 
     return y;
 }
 
+// DynamicQuantizer::is_critical_layer (crates/pmetal-gguf/src/dynamic.rs:254-268)
+inline bool is_critical_layer(const std::string &name) {
+    for (const char *s : {"lm_head", "output", "token_embd", "embed_tokens", "wte", "final_norm", "ln_f"})
+        if (name.find(s) != std::string::npos) return true;
+    return false;
+}
+
+// KlCalibrationConfig and CalibratedTensor (crates/pmetal-gguf/src/dynamic.rs:80-123, :186-196)
+struct KlCalibrationConfig {
+    std::vector<GgmlType> candidates{GgmlType::Q8K, GgmlType::Q6K, GgmlType::Q5K, GgmlType::Q4K, GgmlType::Q3K, GgmlType::Q2K};
+    double kl_threshold = 0.01;
+    GgmlType fallback_type = GgmlType::Q8K;
+    size_t sample_size = 0;
+    uint32_t order = PMETAL_HIP_ORDER_REF;  // element order of the dequantizer in the round trip (the reference: REF)
+};
+struct CalibratedTensor {
+    GgmlType quant_type;
+    double kl_score;
+    std::vector<std::pair<GgmlType, double>> all_scores;
+};
+
+// DynamicQuantizer::calibrate_tensor (crates/pmetal-gguf/src/dynamic.rs:420-502) with the round trips on the GPU: the
+// tensor is uploaded once; every candidate is quantized, dequantized and scored on the device.  A candidate without
+// kernels here (Q3_K, Q2_K), or a shape whose byte size is not the quantized tensor's, is skipped, as the reference
+// skips a candidate whose quantize or dequantize fails.
+inline CalibratedTensor calibrate_tensor(const std::string &name, const float *data, size_t n, const std::vector<int32_t> &shape,
+                                         const KlCalibrationConfig &cfg = KlCalibrationConfig()) {
+    const double kMax = 1.7976931348623157e308;  // f64::MAX
+    if (is_critical_layer(name)) return {cfg.fallback_type, 0.0, {{cfg.fallback_type, 0.0}}};
+    size_t n_shape = 1;
+    for (int32_t d : shape) n_shape *= (size_t)(d > 0 ? d : 0);
+    const size_t sample = cfg.sample_size > 0 && n > cfg.sample_size ? cfg.sample_size : n;
+    std::vector<std::pair<GgmlType, double>> scores;
+    DeviceBuffer dx((n ? n : 4) * sizeof(float)), ddeq((n ? n : 4) * sizeof(float));
+    if (n) detail::check(pmetal_hip_h2d(dx.ptr(), data, n * sizeof(float)));
+    for (GgmlType t : cfg.candidates) {
+        const size_t nbytes = pmetal_hip_tensor_size((uint32_t)t, n);
+        if (!pmetal_hip_is_supported((uint32_t)t) || n_shape > n || pmetal_hip_tensor_size((uint32_t)t, n_shape) != nbytes) continue;
+        if (n_shape == 0) {
+            scores.emplace_back(t, 0.0);
+            continue;
+        }
+        DeviceBuffer dq(nbytes ? nbytes : 16);
+        detail::check(pmetal_hip_quantize_dev((uint32_t)t, (const float *)dx.ptr(), n, (uint8_t *)dq.ptr(), nbytes, nullptr), true);
+        detail::check(pmetal_hip_dequantize_dev((uint32_t)t, (const uint8_t *)dq.ptr(), nbytes, (float *)ddeq.ptr(), n_shape, cfg.order, nullptr));
+        double score = 0.0;
+        detail::check(pmetal_hip_kl_divergence_dev((const float *)dx.ptr(), (const float *)ddeq.ptr(), sample < n_shape ? sample : n_shape,
+                                                   &score, nullptr));
+        scores.emplace_back(t, score);
+    }
+    if (scores.empty()) return {cfg.fallback_type, kMax, {{cfg.fallback_type, kMax}}};
+    CalibratedTensor out{scores[0].first, scores[0].second, scores};
+    for (auto it = scores.rbegin(); it != scores.rend(); ++it)
+        if (it->second <= cfg.kl_threshold) {
+            out.quant_type = it->first, out.kl_score = it->second;
+            break;
+        }
+    return out;
+}
+
 // Q4_K_M recipe: crates/pmetal/src/commands/quantize.rs:988-1137
 inline bool use_more_bits(size_t layer, size_t n_layers) { return pmetal_hip_use_more_bits(layer, n_layers) != 0; }
 inline GgmlType q4km_tensor_type(const std::string &gguf_name, size_t ndim, size_t n_layers) {

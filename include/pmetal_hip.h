@@ -39,6 +39,7 @@ extern "C" {
 #define PMETAL_GGML_TYPE_Q4K 12u
 #define PMETAL_GGML_TYPE_Q5K 13u /* quantize / dequantize only (k_quants.rs:960-1051, :407-462); no linear kernels */
 #define PMETAL_GGML_TYPE_Q6K 14u
+#define PMETAL_GGML_TYPE_Q8K 15u /* quantize / dequantize (k_quants.rs:815-871, :498-506) and the activation side of qgemv_q8k */
 
 /* Error classes.  1-3, 6, 7 map onto DequantError (crates/pmetal-gguf/src/dequant.rs:37-70)
  * and PMetalError::Quantization (crates/pmetal-core/src/error.rs:50-52). */
@@ -191,6 +192,15 @@ size_t pmetal_hip_q8k_size(size_t n_elements);
 int32_t pmetal_hip_quantize_q8k_dev(const float *src_dev, size_t n, uint8_t *dst_dev, size_t dst_len, void *stream);
 int32_t pmetal_hip_qgemv_q8k(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, int64_t k, const uint8_t *xq_dev,
                              float *y_dev, void *stream);
+
+/* ---- KL calibration metric -------------------------------------------------------------
+ * compute_kl_divergence (crates/pmetal-gguf/src/dynamic.rs:140-180): normalised RMSE plus cosine distance between n
+ * original and n dequantized values, both on the device, accumulated in f64 (in a different order than the
+ * reference's sequential loop: equal to about 1e-13 relative).  Synchronises the stream; *score is host memory.
+ * The quantize -> dequantize -> score loop of calibrate_tensor (dynamic.rs:420-502) is host logic over
+ * pmetal_hip_quantize_dev / _dequantize_dev / this (pmetal_gguf::calibrate_tensor, pmetal_amd.gguf.calibrate_tensor). */
+int32_t pmetal_hip_kl_divergence_dev(const float *original_dev, const float *dequantized_dev, size_t n, double *score,
+                                     void *stream);
 
 /* ---- Q4_K_M recipe (crates/pmetal/src/commands/quantize.rs) --------------------------- */
 int32_t pmetal_hip_use_more_bits(size_t layer, size_t n_layers);                   /* :988-993  */

@@ -15,6 +15,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libpmetal_oracle.so")
 
 TYPE_F32, TYPE_F16, TYPE_Q8_0, TYPE_Q4K, TYPE_Q6K = 0, 1, 8, 12, 14
+TYPE_Q5K, TYPE_Q8K = 13, 15
 ORDER_REF, ORDER_GGML = 0, 1
 OK, ERR_UNSUPPORTED_TYPE, ERR_INVALID_SIZE, ERR_INVALID_SHAPE, ERR_SHAPE_TOO_LARGE = 0, 2, 3, 6, 7
 
@@ -77,6 +78,7 @@ def lib() -> C.CDLL:
         L.pmo_qmatmul_f64.argtypes = [C.c_uint32, u8p, C.c_size_t, C.c_size_t, f32p, C.c_size_t, f32p,
                                       C.c_uint32]
         L.pmo_qmatmul_f64.restype = C.c_int32
+        L.pmo_kl_divergence.argtypes, L.pmo_kl_divergence.restype = [f32p, f32p, C.c_size_t], C.c_double
         L.pmo_q8k_size.argtypes, L.pmo_q8k_size.restype = [C.c_size_t], C.c_size_t
         L.pmo_quantize_q8k.argtypes, L.pmo_quantize_q8k.restype = [f32p, C.c_size_t, u8p], None
         for name in ("pmo_vec_dot_q4k_q8k", "pmo_vec_dot_q6k_q8k"):
@@ -196,6 +198,48 @@ def qmatvec_q8k(t: int, w: np.ndarray, n_rows: int, k: int, xq: np.ndarray) -> n
     if rc != OK:
         raise ValueError(rc)
     return y
+
+
+def kl_divergence(original: np.ndarray, dequantized: np.ndarray) -> float:
+    """dynamic.rs:140-180 ``compute_kl_divergence``."""
+    a = np.ascontiguousarray(original, dtype=np.float32).reshape(-1)
+    b = np.ascontiguousarray(dequantized, dtype=np.float32).reshape(-1)
+    assert a.size == b.size
+    return float(lib().pmo_kl_divergence(_f32p(a), _f32p(b), a.size))
+
+
+def is_critical_layer(name: str) -> bool:
+    """dynamic.rs:254-268"""
+    return any(s in name for s in ("lm_head", "output", "token_embd", "embed_tokens", "wte", "final_norm", "ln_f"))
+
+
+DEFAULT_CANDIDATES = (15, 14, 13, 12, 11, 10)  # Q8K, Q6K, Q5K, Q4K, Q3K, Q2K (dynamic.rs:104-121)
+
+
+def calibrate_tensor(name: str, data: np.ndarray, shape, candidates=DEFAULT_CANDIDATES, kl_threshold: float = 0.01,
+                     fallback_type: int = 15, sample_size: int = 0, order: int = ORDER_REF):
+    """dynamic.rs:420-502 ``calibrate_tensor``: (quant_type, kl_score, all_scores).  A candidate whose quantizer or
+    dequantizer fails is skipped (:456-464), which here is every type the oracle does not restate."""
+    data = np.ascontiguousarray(data, dtype=np.float32).reshape(-1)
+    if is_critical_layer(name):
+        return fallback_type, 0.0, [(fallback_type, 0.0)]
+    sample = data[:sample_size] if 0 < sample_size < data.size else data
+    scores = []
+    for t in candidates:
+        try:
+            deq = dequantize(t, quantize(t, data), shape, order)
+        except ValueError:
+            continue
+        n = min(sample.size, deq.size)
+        scores.append((t, kl_divergence(sample[:n], deq[:n])))
+    if not scores:
+        return fallback_type, float(np.finfo(np.float64).max), [(fallback_type, float(np.finfo(np.float64).max))]
+    best_type, best_score = scores[0]
+    for t, sc in reversed(scores):
+        if sc <= kl_threshold:
+            best_type, best_score = t, sc
+            break
+    return best_type, best_score, scores
 
 
 def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:

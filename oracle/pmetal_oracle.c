@@ -324,6 +324,7 @@ size_t pmo_type_size(uint32_t t) {
     case PMO_TYPE_Q4K: return 144;
     case PMO_TYPE_Q5K: return 176;
     case PMO_TYPE_Q6K: return 210;
+    case PMO_TYPE_Q8K: return 292;
     default: return 0;
     }
 }
@@ -335,7 +336,8 @@ size_t pmo_block_size(uint32_t t) {
     case PMO_TYPE_Q8_0: return 32;
     case PMO_TYPE_Q4K:
     case PMO_TYPE_Q5K:
-    case PMO_TYPE_Q6K: return 256;
+    case PMO_TYPE_Q6K:
+    case PMO_TYPE_Q8K: return 256;
     default: return 0;
     }
 }
@@ -751,6 +753,37 @@ void pmo_quantize_q8k(const float *xs, size_t n, uint8_t *dst) {
     }
 }
 
+/* k_quants.rs:498-506 */
+void pmo_dequantize_q8k(const uint8_t *src, size_t n, float *dst) {
+    for (size_t i = 0; i < n; i++) {
+        const uint8_t *blk = src + (i / 256) * 292;
+        float d;
+        memcpy(&d, blk, 4);
+        dst[i] = d * (float)(int8_t)blk[4 + i % 256];
+    }
+}
+
+/* dynamic.rs:140-180 */
+double pmo_kl_divergence(const float *original, const float *dequantized, size_t n) {
+    if (n == 0) return 0.0;
+    double sq_err_sum = 0.0, sq_orig_sum = 0.0;
+    for (size_t i = 0; i < n; i++) { /* :150-154: the difference is taken in f32, then widened */
+        double diff = (double)(original[i] - dequantized[i]);
+        sq_err_sum += diff * diff;
+        sq_orig_sum += (double)original[i] * (double)original[i];
+    }
+    double nrmse = sq_orig_sum > 0.0 ? sqrt(sq_err_sum / (double)n) / sqrt(sq_orig_sum / (double)n) : 0.0;
+    double dot = 0.0, norm_a = 0.0, norm_b = 0.0;
+    for (size_t i = 0; i < n; i++) { /* :163-169 */
+        double a = (double)original[i], b = (double)dequantized[i];
+        dot += a * b;
+        norm_a += a * a;
+        norm_b += b * b;
+    }
+    double cos_sim = (norm_a > 0.0 && norm_b > 0.0) ? dot / (sqrt(norm_a) * sqrt(norm_b)) : 1.0;
+    return nrmse + (1.0 - cos_sim);
+}
+
 /* vec_dot.rs:617-656 */
 float pmo_vec_dot_q4k_q8k(const uint8_t *xs, const uint8_t *ys, size_t n_blocks) {
     float sum = 0.0f;
@@ -833,9 +866,10 @@ int32_t pmo_qmatvec_q8k(uint32_t t, const uint8_t *w, size_t n_rows, size_t k, c
 /* quantize.rs:17-87 and dequant.rs:92-132, :184-216                         */
 /* ------------------------------------------------------------------------- */
 int32_t pmo_quantize(uint32_t t, const float *x, size_t n, uint8_t *dst, size_t dst_len) {
-    if (t != PMO_TYPE_Q8_0 && t != PMO_TYPE_Q4K && t != PMO_TYPE_Q5K && t != PMO_TYPE_Q6K) return PMO_ERR_UNSUPPORTED_TYPE;
+    if (t != PMO_TYPE_Q8_0 && t != PMO_TYPE_Q4K && t != PMO_TYPE_Q5K && t != PMO_TYPE_Q6K && t != PMO_TYPE_Q8K) return PMO_ERR_UNSUPPORTED_TYPE;
     if (dst_len != pmo_tensor_size(t, n)) return PMO_ERR_INVALID_SIZE;
-    if (t == PMO_TYPE_Q8_0) pmo_quantize_q8_0(x, n, dst);
+    if (t == PMO_TYPE_Q8K) pmo_quantize_q8k(x, n, dst);
+    else if (t == PMO_TYPE_Q8_0) pmo_quantize_q8_0(x, n, dst);
     else if (t == PMO_TYPE_Q4K) pmo_quantize_q4k(x, n, dst);
     else if (t == PMO_TYPE_Q5K) pmo_quantize_q5k(x, n, dst);
     else pmo_quantize_q6k(x, n, dst);
@@ -844,7 +878,7 @@ int32_t pmo_quantize(uint32_t t, const float *x, size_t n, uint8_t *dst, size_t 
 
 int32_t pmo_dequantize(uint32_t t, const uint8_t *src, size_t src_len, const int32_t *shape, size_t ndim,
                        float *dst, size_t dst_cap, uint32_t order) {
-    if (t != PMO_TYPE_Q8_0 && t != PMO_TYPE_Q4K && t != PMO_TYPE_Q5K && t != PMO_TYPE_Q6K) return PMO_ERR_UNSUPPORTED_TYPE;
+    if (t != PMO_TYPE_Q8_0 && t != PMO_TYPE_Q4K && t != PMO_TYPE_Q5K && t != PMO_TYPE_Q6K && t != PMO_TYPE_Q8K) return PMO_ERR_UNSUPPORTED_TYPE;
     /* dequant.rs:193-206 shape_n_elements */
     for (size_t i = 0; i < ndim; i++)
         if (shape[i] < 0) return PMO_ERR_INVALID_SHAPE;
@@ -860,6 +894,7 @@ int32_t pmo_dequantize(uint32_t t, const uint8_t *src, size_t src_len, const int
     if (t == PMO_TYPE_Q8_0) pmo_dequantize_q8_0(src, n, dst);
     else if (t == PMO_TYPE_Q4K) pmo_dequantize_q4k(src, n, dst, order);
     else if (t == PMO_TYPE_Q5K) pmo_dequantize_q5k(src, n, dst, order);
+    else if (t == PMO_TYPE_Q8K) pmo_dequantize_q8k(src, n, dst);
     else pmo_dequantize_q6k(src, n, dst);
     return PMO_OK;
 }

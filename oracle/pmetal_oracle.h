@@ -32,6 +32,7 @@ enum {
     PMO_TYPE_Q4K = 12,
     PMO_TYPE_Q5K = 13, /* quantize / dequantize only */
     PMO_TYPE_Q6K = 14,
+    PMO_TYPE_Q8K = 15, /* quantize / dequantize and the activation side of the integer dot products */
 };
 
 /* Error classes mirroring DequantError (dequant.rs:37-70) and
@@ -105,6 +106,10 @@ uint32_t pmo_q4km_tensor_type(const char *gguf_name, size_t ndim, size_t n_layer
  * partial block stays all-zero); vec_dot.rs:617-656 scalar vec_dot_q4k_q8k, :658-692 scalar vec_dot_q6k_q8k.
  * pmo_qmatvec_q8k: y[r] = vec_dot(row r of W, xq) for W of type Q4K or Q6K, k a multiple of 256. */
 size_t pmo_q8k_size(size_t n_elements);
+/* k_quants.rs:498-506 + :562-610 */
+void pmo_dequantize_q8k(const uint8_t *src, size_t n, float *dst);
+/* dynamic.rs:140-180 compute_kl_divergence: normalised RMSE + cosine distance, sequential f64 sums */
+double pmo_kl_divergence(const float *original, const float *dequantized, size_t n);
 void pmo_quantize_q8k(const float *x, size_t n, uint8_t *dst);
 float pmo_vec_dot_q4k_q8k(const uint8_t *xs, const uint8_t *ys, size_t n_blocks);
 float pmo_vec_dot_q6k_q8k(const uint8_t *xs, const uint8_t *ys, size_t n_blocks);

@@ -7,6 +7,7 @@
 // There is no CPU fallback anywhere in this file: without a HIP device every compute call fails.
 #include "../../include/pmetal_hip.h"
 
+#include <cmath>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -53,8 +54,9 @@ int32_t hip_fail(hipError_t e, const char *what) {
 bool path_type(uint32_t t) {
     return t == PMETAL_GGML_TYPE_Q8_0 || t == PMETAL_GGML_TYPE_Q4K || t == PMETAL_GGML_TYPE_Q6K;
 }
-// types with quantize / dequantize kernels: the above and Q5_K (the Q4_K_M recipe gives it to fused attn_qkv tensors)
-bool codec_type(uint32_t t) { return path_type(t) || t == PMETAL_GGML_TYPE_Q5K; }
+// types with quantize / dequantize kernels: the above, Q5_K (the Q4_K_M recipe gives it to fused attn_qkv tensors) and
+// Q8_K (the activation format of the integer dot products, and the first candidate of the KL calibration)
+bool codec_type(uint32_t t) { return path_type(t) || t == PMETAL_GGML_TYPE_Q5K || t == PMETAL_GGML_TYPE_Q8K; }
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -170,6 +172,7 @@ size_t pmetal_hip_type_size(uint32_t t) {
     case PMETAL_GGML_TYPE_Q4K: return 144;
     case PMETAL_GGML_TYPE_Q5K: return 176;
     case PMETAL_GGML_TYPE_Q6K: return 210;
+    case PMETAL_GGML_TYPE_Q8K: return 292;
     default: return 0;
     }
 }
@@ -179,7 +182,8 @@ size_t pmetal_hip_block_size(uint32_t t) {
     case PMETAL_GGML_TYPE_Q8_0: return 32;
     case PMETAL_GGML_TYPE_Q4K:
     case PMETAL_GGML_TYPE_Q5K:
-    case PMETAL_GGML_TYPE_Q6K: return 256;
+    case PMETAL_GGML_TYPE_Q6K:
+    case PMETAL_GGML_TYPE_Q8K: return 256;
     default: return 0;
     }
 }
@@ -362,6 +366,7 @@ int32_t pmetal_hip_quantize_dev(uint32_t t, const float *src, size_t n, uint8_t 
     if (t == PMETAL_GGML_TYPE_Q8_0) e = pmh::launch_quantize_q8_0(src, n, dst, s);
     else if (t == PMETAL_GGML_TYPE_Q4K) e = pmh::launch_quantize_q4k(src, n, dst, s);
     else if (t == PMETAL_GGML_TYPE_Q5K) e = pmh::launch_quantize_q5k(src, n, dst, s);
+    else if (t == PMETAL_GGML_TYPE_Q8K) e = pmh::launch_quantize_q8k(src, n, dst, s);
     else e = pmh::launch_quantize_q6k(src, n, dst, s);
     if (e != hipSuccess) return hip_fail(e, "quantize kernel launch");
     return ok();
@@ -402,6 +407,7 @@ int32_t pmetal_hip_dequantize_dev(uint32_t t, const uint8_t *src, size_t src_len
     if (t == PMETAL_GGML_TYPE_Q8_0) e = pmh::launch_dequantize_q8_0(src, n, dst, s);
     else if (t == PMETAL_GGML_TYPE_Q4K) e = pmh::launch_dequantize_q4k(src, n, dst, order, s);
     else if (t == PMETAL_GGML_TYPE_Q5K) e = pmh::launch_dequantize_q5k(src, n, dst, order, s);
+    else if (t == PMETAL_GGML_TYPE_Q8K) e = pmh::launch_dequantize_q8k(src, n, dst, s);
     else e = pmh::launch_dequantize_q6k(src, n, dst, s);
     if (e != hipSuccess) return hip_fail(e, "dequantize kernel launch");
     return ok();
@@ -637,6 +643,34 @@ int32_t pmetal_hip_qgemv_q8k(uint32_t t, const uint8_t *w, int64_t n, int64_t k,
     }
     hipError_t e = pmh::launch_qgemv_q8k(t, w, n, k, xq, y, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "qgemv_q8k kernel launch");
+    return ok();
+}
+
+// ---- KL calibration metric ----
+int32_t pmetal_hip_kl_divergence_dev(const float *original, const float *dequantized, size_t n, double *score, void *stream) {
+    if (!score) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
+    if (n == 0) {  // dynamic.rs:143-145
+        *score = 0.0;
+        return ok();
+    }
+    if (!original || !dequantized) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
+    if (!aligned16(original) || !aligned16(dequantized)) return fail(PMETAL_HIP_ERR_INVALID_ARG, "device pointers must be 16-byte aligned");
+    if (int32_t rc = require_device()) return rc;
+    const int groups = pmh::kl_sums_workgroups(n);
+    DevBuf part;
+    HIP_TRY(hipMalloc(&part.p, (size_t)groups * 4 * sizeof(double)));
+    hipError_t e = pmh::launch_kl_sums(original, dequantized, n, (double *)part.p, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "kl sums kernel launch");
+    std::vector<double> host((size_t)groups * 4);
+    HIP_TRY(hipMemcpyAsync(host.data(), part.p, host.size() * sizeof(double), hipMemcpyDeviceToHost, (hipStream_t)stream));
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    double sq_err = 0.0, aa = 0.0, ab = 0.0, bb = 0.0;
+    for (int g = 0; g < groups; g++) sq_err += host[4 * g], aa += host[4 * g + 1], ab += host[4 * g + 2], bb += host[4 * g + 3];
+    // dynamic.rs:155-178
+    const double dn = (double)n;
+    const double nrmse = aa > 0.0 ? std::sqrt(sq_err / dn) / std::sqrt(aa / dn) : 0.0;
+    const double cos_sim = (aa > 0.0 && bb > 0.0) ? ab / (std::sqrt(aa) * std::sqrt(bb)) : 1.0;
+    *score = nrmse + (1.0 - cos_sim);
     return ok();
 }
 

@@ -7,7 +7,7 @@
 
 namespace pmh {
 
-constexpr uint32_t kTypeQ8_0 = 8, kTypeQ4K = 12, kTypeQ5K = 13, kTypeQ6K = 14;
+constexpr uint32_t kTypeQ8_0 = 8, kTypeQ4K = 12, kTypeQ5K = 13, kTypeQ6K = 14, kTypeQ8K = 15;
 constexpr uint32_t kOrderRef = 0, kOrderGgml = 1;
 constexpr uint32_t kDtypeF32 = 0, kDtypeBf16 = 1;
 
@@ -53,6 +53,10 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
 
 // ---- q8k.hip: Q8_K activation blocks and the integer dot products over them ----
 hipError_t launch_quantize_q8k(const float *x, size_t n, uint8_t *dst, hipStream_t s);
+hipError_t launch_dequantize_q8k(const uint8_t *src, size_t n, float *dst, hipStream_t s);
+// four f64 sums per workgroup (sum (a-b)^2, sum a^2, sum a b, sum b^2) into partial[4 * kl_sums_workgroups(n)]
+int kl_sums_workgroups(size_t n);
+hipError_t launch_kl_sums(const float *a, const float *b, size_t n, double *partial, hipStream_t s);
 // k a multiple of 256 and at most 32768 (the activation blocks live in LDS); type Q4_K or Q6_K
 hipError_t launch_qgemv_q8k(uint32_t type, const uint8_t *w, int64_t n, int64_t k, const uint8_t *xq, float *y, hipStream_t s);
 

@@ -76,6 +76,68 @@ __global__ __launch_bounds__(256) void k_quantize_q8k(const float *__restrict__ 
     if (lane == 0) *reinterpret_cast<float *>(out) = 1.0f / iscale;
 }
 
+// dequantize_q8k (crates/pmetal-gguf/src/k_quants.rs:498-506): out = d * q, one rounding.  One lane per 4 outputs.
+__global__ __launch_bounds__(256) void k_dequantize_q8k(const uint8_t *__restrict__ src, size_t n, float *__restrict__ dst) {
+    const size_t e = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (e >= n) return;
+    const uint8_t *blk = src + (e >> 8) * kQ8kBytes;
+    const float d = *reinterpret_cast<const float *>(blk);
+    const uint32_t q = *reinterpret_cast<const uint32_t *>(blk + 4 + (e & 255));
+    float o[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) o[c] = d * (float)(int8_t)(q >> (8 * c));
+    if (e + 3 < n) {
+        *reinterpret_cast<float4 *>(dst + e) = make_float4(o[0], o[1], o[2], o[3]);
+    } else {
+        for (int c = 0; c < 4 && e + c < n; c++) dst[e + c] = o[c];
+    }
+}
+
+// The four f64 sums of compute_kl_divergence (crates/pmetal-gguf/src/dynamic.rs:140-180) over n pairs (original,
+// dequantized): sum (a - b)^2 with the difference taken in f32 as the reference takes it, sum a^2, sum a b, sum b^2.
+// Every workgroup writes its four partial sums; the caller adds the workgroups' sums in order.
+__global__ __launch_bounds__(256) void k_kl_sums(const float *__restrict__ a, const float *__restrict__ b, size_t n,
+                                                  double *__restrict__ partial) {
+    double s_err = 0.0, s_aa = 0.0, s_ab = 0.0, s_bb = 0.0;
+    auto add = [&](float av, float bv) {
+        const double diff = (double)(av - bv), x = (double)av, y = (double)bv;
+        s_err += diff * diff, s_aa += x * x, s_ab += x * y, s_bb += y * y;
+    };
+    // Whole rounds of four float4 pairs per lane (eight loads in flight), then single float4 pairs, then the tail.
+    constexpr int kUnroll = 4;
+    const size_t lanes = (size_t)gridDim.x * 256, me = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t nvec = n / 4, rounds = nvec / (lanes * kUnroll);
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    const f4 *a4 = reinterpret_cast<const f4 *>(a), *b4 = reinterpret_cast<const f4 *>(b);
+    for (size_t r = 0; r < rounds; r++) {
+        f4 x[kUnroll], y[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            const size_t v = (r * kUnroll + u) * lanes + me;
+            x[u] = __builtin_nontemporal_load(a4 + v), y[u] = __builtin_nontemporal_load(b4 + v);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) add(x[u].x, y[u].x), add(x[u].y, y[u].y), add(x[u].z, y[u].z), add(x[u].w, y[u].w);
+    }
+    for (size_t v = rounds * kUnroll * lanes + me; v < nvec; v += lanes) {
+        const f4 x = a4[v], y = b4[v];
+        add(x.x, y.x), add(x.y, y.y), add(x.z, y.z), add(x.w, y.w);
+    }
+    for (size_t e = nvec * 4 + me; e < n; e += lanes) add(a[e], b[e]);
+    __shared__ double red[4][4];
+    double v[4] = {s_err, s_aa, s_ab, s_bb};
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) v[k] += __shfl_xor(v[k], off);
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0)
+        for (int k = 0; k < 4; k++) red[wave][k] = v[k];
+    __syncthreads();
+    if (threadIdx.x < 4) partial[(size_t)blockIdx.x * 4 + threadIdx.x] = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
+}
+
 // ------------------------------------------------------------------------------------------------
 // GEMV over Q8_K activations.  The activation blocks are laid out once per workgroup in LDS (qs 16-byte aligned,
 // then d, then bsums).
@@ -277,6 +339,21 @@ hipError_t launch_quantize_q8k(const float *x, size_t n, uint8_t *dst, hipStream
     const size_t n_blocks = n / 256 + (n % 256 != 0), n_full = n / 256;
     if (n_blocks == 0) return hipSuccess;
     hipLaunchKernelGGL(k_quantize_q8k, dim3((unsigned)((n_blocks + 3) / 4)), dim3(256), 0, s, x, n_full, n_blocks, dst);
+    return hipGetLastError();
+}
+
+hipError_t launch_dequantize_q8k(const uint8_t *src, size_t n, float *dst, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_dequantize_q8k, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, s, src, n, dst);
+    return hipGetLastError();
+}
+
+int kl_sums_workgroups(size_t n) {
+    const size_t want = (n + 4095) / 4096;  // at least four float4 pairs per lane
+    return (int)(want < 1 ? 1 : (want > 2048 ? 2048 : want));
+}
+hipError_t launch_kl_sums(const float *a, const float *b, size_t n, double *partial, hipStream_t s) {
+    hipLaunchKernelGGL(k_kl_sums, dim3((unsigned)kl_sums_workgroups(n)), dim3(256), 0, s, a, b, n, partial);
     return hipGetLastError();
 }
 

@@ -29,6 +29,9 @@ class GgmlType(enum.IntEnum):
     Q4K = 12
     Q5K = 13
     Q6K = 14
+    Q8K = 15
+    Q3K = 11
+    Q2K = 10
 
     def type_size(self) -> int:
         return _lib.load().pmetal_hip_type_size(int(self))
@@ -187,6 +190,64 @@ def qgemv_q8k(dtype: int, w, n: int, k: int, xq, y=None, stream=None) -> DeviceB
         y = DeviceBuffer(max(4 * n, 16))
     check(lib.pmetal_hip_qgemv_q8k(int(dtype), _dev_ptr(w), n, k, _dev_ptr(xq), _dev_ptr(y), stream))
     return y
+
+
+def kl_divergence_dev(original, dequantized, n: int, stream=None) -> float:
+    """``compute_kl_divergence`` (crates/pmetal-gguf/src/dynamic.rs:140-180) of two device arrays of ``n`` f32."""
+    score = C.c_double()
+    check(_lib.load().pmetal_hip_kl_divergence_dev(_dev_ptr(original), _dev_ptr(dequantized), n, C.byref(score), stream))
+    return score.value
+
+
+def is_critical_layer(name: str) -> bool:
+    """``DynamicQuantizer::is_critical_layer`` (crates/pmetal-gguf/src/dynamic.rs:254-268)."""
+    return any(s in name for s in ("lm_head", "output", "token_embd", "embed_tokens", "wte", "final_norm", "ln_f"))
+
+
+#: ``KlCalibrationConfig::default().candidates`` (crates/pmetal-gguf/src/dynamic.rs:104-121), best quality first
+DEFAULT_KL_CANDIDATES = (GgmlType.Q8K, GgmlType.Q6K, GgmlType.Q5K, GgmlType.Q4K, GgmlType.Q3K, GgmlType.Q2K)
+
+
+def calibrate_tensor(name: str, data, shape, candidates=DEFAULT_KL_CANDIDATES, kl_threshold: float = 0.01,
+                     fallback_type: int = GgmlType.Q8K, sample_size: int = 0, order: int = ORDER_REF):
+    """``DynamicQuantizer::calibrate_tensor`` (crates/pmetal-gguf/src/dynamic.rs:420-502) with the round trips on the GPU:
+    the tensor is uploaded once, every candidate is quantized, dequantized (in the reference dequantizer's element order
+    unless ``order`` says otherwise) and scored on the device.  Returns ``(quant_type, kl_score, all_scores)``.  As in
+    the reference, a candidate the quantizer does not implement is skipped (here: Q3_K, Q2_K)."""
+    lib = _lib.load()
+    x = np.ascontiguousarray(data, dtype=np.float32).reshape(-1)
+    if is_critical_layer(name):
+        return int(fallback_type), 0.0, [(int(fallback_type), 0.0)]
+    n = x.size
+    n_shape = int(np.prod([int(d) for d in shape], dtype=np.int64)) if len(shape) else 1
+    sample = sample_size if 0 < sample_size < n else n
+    scores = []
+    if n:
+        dx, ddeq = DeviceBuffer.from_host(x), DeviceBuffer(4 * max(n, 4))
+    for t in candidates:
+        t = int(t)
+        # quantize the whole tensor, dequantize what the shape asks for; a type without kernels, or a shape whose byte
+        # size is not that of the quantized tensor, is an `Err(_) => continue` (dynamic.rs:456-464)
+        nbytes = lib.pmetal_hip_tensor_size(t, n)
+        if not lib.pmetal_hip_is_supported(t) or n_shape > n or lib.pmetal_hip_tensor_size(t, n_shape) != nbytes:
+            continue
+        if n_shape == 0:
+            scores.append((t, 0.0))
+            continue
+        dq = DeviceBuffer(max(nbytes, 16))
+        check(lib.pmetal_hip_quantize_dev(t, dx.ptr, n, dq.ptr, nbytes, None), "quantize")
+        check(lib.pmetal_hip_dequantize_dev(t, dq.ptr, nbytes, ddeq.ptr, n_shape, order, None))
+        scores.append((t, kl_divergence_dev(dx, ddeq, min(sample, n_shape))))
+        dq.free()
+    if not scores:
+        big = float(np.finfo(np.float64).max)
+        return int(fallback_type), big, [(int(fallback_type), big)]
+    best_type, best_score = scores[0]
+    for t, sc in reversed(scores):
+        if sc <= kl_threshold:
+            best_type, best_score = t, sc
+            break
+    return best_type, best_score, scores
 
 
 class GgufLinear:

@@ -3,7 +3,7 @@
 //   crates/pmetal-gguf/src/k_quants.rs:1334-1342 (block sizes), :1368-1383 (Q4K dequantize range),
 //   :1446-1465 and :1490-1509 (Q4K / Q6K round trips), crates/pmetal-gguf/src/dequant.rs:1016-1036 (Q8_0
 //   block structure), :1139-1150 (invalid size / shape), crates/pmetal/src/commands/quantize.rs:1561-1608
-//   (Q4_K_M recipe).
+//   (Q4_K_M recipe), crates/pmetal-gguf/src/dynamic.rs:789-800, :934-1018 (critical layers, KL metric, calibration).
 // Usage: test_reference_suite [--host-only]   (--host-only skips everything that needs a GPU)
 #include <cmath>
 #include <cstdio>
@@ -157,17 +157,52 @@ static void test_linear_matmul_from() {
     CHECK(worst <= 1e-3 * scale);
 }
 
+static void test_critical_layers() {  // dynamic.rs:789-800
+    CHECK(is_critical_layer("lm_head.weight") && is_critical_layer("model.output.weight"));
+    CHECK(is_critical_layer("model.embed_tokens.weight") && is_critical_layer("token_embd.weight"));
+    CHECK(!is_critical_layer("model.layers.0.mlp.weight"));
+    const KlCalibrationConfig cfg;  // dynamic.rs:958-965
+    CHECK(cfg.candidates.size() == 6 && cfg.candidates.front() == GgmlType::Q8K && cfg.candidates.back() == GgmlType::Q2K);
+    CHECK(cfg.sample_size == 0 && std::fabs(cfg.kl_threshold - 0.01) < 1e-9);
+}
+
+static void test_calibration() {  // dynamic.rs:968-1018, :934-956 through the device metric
+    const KlCalibrationConfig cfg;
+    const std::vector<float> ones(1024, 1.0f);
+    const CalibratedTensor crit = calibrate_tensor("model.lm_head.weight", ones.data(), ones.size(), {32, 32}, cfg);
+    CHECK(crit.quant_type == cfg.fallback_type && crit.kl_score == 0.0);
+    std::vector<float> ramp(256);
+    for (int i = 0; i < 256; i++) ramp[i] = (float)i * 0.01f - 1.28f;
+    const CalibratedTensor r = calibrate_tensor("model.layers.0.mlp.gate_proj.weight", ramp.data(), ramp.size(), {1, 256}, cfg);
+    bool member = r.quant_type == cfg.fallback_type;
+    for (GgmlType t : cfg.candidates) member = member || t == r.quant_type;
+    CHECK(member && !r.all_scores.empty());
+    CHECK(r.all_scores.size() == 4 && r.all_scores[0].first == GgmlType::Q8K && r.all_scores[0].second < 0.01);  // Q3_K, Q2_K skipped
+    // compute_kl_divergence: identical -> ~0, perturbed -> small positive, zeros -> 0
+    const float a[8] = {1, 2, 3, 4, 5, 0, 0, 0}, b[8] = {1.1f, 2.1f, 2.9f, 4.2f, 4.8f, 0, 0, 0}, z[8] = {0};
+    DeviceBuffer da(a, sizeof a), db(b, sizeof b), dz(z, sizeof z);
+    double s = -1;
+    detail::check(pmetal_hip_kl_divergence_dev((const float *)da.ptr(), (const float *)da.ptr(), 5, &s, nullptr));
+    CHECK(s >= 0 && s < 1e-10);
+    detail::check(pmetal_hip_kl_divergence_dev((const float *)da.ptr(), (const float *)db.ptr(), 5, &s, nullptr));
+    CHECK(s > 0 && s < 1.0);
+    detail::check(pmetal_hip_kl_divergence_dev((const float *)dz.ptr(), (const float *)dz.ptr(), 8, &s, nullptr));
+    CHECK(s == 0.0);
+}
+
 int main(int argc, char **argv) {
     const bool host_only = argc > 1 && std::strcmp(argv[1], "--host-only") == 0;
     test_block_sizes();
     test_recipe();
     test_invalid_size_and_shape();
+    test_critical_layers();
     if (!host_only) {
         CHECK(pmetal_hip_init(0) == 0);
         test_q8_0_block_structure();
         test_q4k_dequantize_simple();
         test_roundtrips();
         test_linear_matmul_from();
+        test_calibration();
     }
     std::printf(failures ? "%d check(s) failed\n" : "all checks passed\n", failures);
     return failures ? 1 : 0;
