@@ -266,14 +266,14 @@ def cpu_baseline_gemv_q8k(t, n, k, budget_s=12.0):
 
 def bench_calibrate(args, n, k):
     """One step = the round trips of calibrate_tensor for one resident 14336 x 4096 f32 tensor: for each candidate type
-    with kernels here (Q8_K, Q6_K, Q5_K, Q4_K) quantize, dequantize, score."""
+    of the reference's default list (Q8_K, Q6_K, Q5_K, Q4_K, Q3_K, Q2_K) quantize, dequantize, score."""
     pm, _lib, lib = load()
     timer = Timer(pm, lib)
     ne = n * k
     x = pm.DeviceBuffer(4 * ne)
     pm.check(lib.pmetal_hip_fill_normal_f32(x.ptr, ne, 11, 0.02, 1e-3, 0.5, None))
     deq = pm.DeviceBuffer(4 * ne)
-    cands = [15, 14, 13, 12]
+    cands = [15, 14, 13, 12, 11, 10]
     qs = {t: pm.DeviceBuffer(lib.pmetal_hip_tensor_size(t, ne)) for t in cands}
     scores = {}
     import ctypes as C
@@ -304,17 +304,17 @@ def bench_calibrate(args, n, k):
 
 
 def cpu_baseline_calibrate(budget_elems=1 << 20):
-    """Oracle: calibrate_tensor (quantize, dequantize, score for the same four candidates), one thread, on 2^20 elements."""
+    """Oracle: calibrate_tensor (quantize, dequantize, score for the same six candidates), one thread, on 2^20 elements."""
     from oracle import binding as oracle
     oracle.build()
     x = (np.random.default_rng(3).standard_normal(budget_elems) * 0.02).astype(np.float32)
     reps, t0 = 0, time.perf_counter()
     while time.perf_counter() - t0 < 10.0:
-        oracle.calibrate_tensor("blk.0.ffn_up.weight", x, [budget_elems // 256, 256], candidates=(15, 14, 13, 12), order=1)
+        oracle.calibrate_tensor("blk.0.ffn_up.weight", x, [budget_elems // 256, 256], candidates=(15, 14, 13, 12, 11, 10), order=1)
         reps += 1
     dt = time.perf_counter() - t0
-    return {"value": round(4.0 * budget_elems * 4 * reps / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"{reps} x calibrate_tensor over {budget_elems} elements, four candidates, {dt:.1f} s"}
+    return {"value": round(4.0 * budget_elems * 6 * reps / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{reps} x calibrate_tensor over {budget_elems} elements, six candidates, {dt:.1f} s"}
 
 
 def bench_gemm(args, m, n, k, t=Q4K):
@@ -495,7 +495,7 @@ WORKLOADS["gemv_q4k_q8k_14336x4096"] = dict(kind="gemv_q8k", n=14336, k=4096, ty
 WORKLOADS["gemv_q6k_q8k_14336x4096"] = dict(kind="gemv_q8k", n=14336, k=4096, type=Q6K, unit="GB/s", dtype="i8",
                                             metric="Q6_K x Q8_K integer-dot GEMV GB/s @14336x4096 (activation quantize included)")
 WORKLOADS["calibrate_14336x4096"] = dict(kind="calibrate", n=14336, k=4096, unit="GB/s", dtype="f32",
-                                         metric="KL calibration GB/s of f32 evaluated (4 candidates, quantize + dequantize + score) @14336x4096")
+                                         metric="KL calibration GB/s of f32 evaluated (6 candidates, quantize + dequantize + score) @14336x4096")
 WORKLOADS["decode_qwen3_0.6b_q4km"] = dict(kind="decode", metric="Q4_K_M decode linears tokens/s (Qwen3-0.6B shape)", unit="tokens/s",
                                            dtype="bf16")
 WORKLOADS["quantize_llama3_8b_q4km"] = dict(kind="quantize", metric="f32->Q4_K_M quantize GB/s of f32 consumed (Llama-3-8B shape)",
@@ -551,7 +551,7 @@ def main():
                    "step": {"gemm": "one GEMM launch (activation pre-pass + MFMA kernel)",
                             "gemv": "16 back-to-back GEMVs over 16 distinct weight tensors (528 MB, HBM-resident)",
                             "gemv_q8k": "16 x (activations f32 -> Q8_K, integer-dot GEMV) over 16 distinct weight tensors",
-                            "calibrate": "one tensor resident in HBM: 4 candidates x (quantize, dequantize, f64 score read back)",
+                            "calibrate": "one tensor resident in HBM: 6 candidates x (quantize, dequantize, f64 score read back)",
                             "decode": "all 197 batch-1 projections of one token, back to back on one stream",
                             "dequantize": "two tensors of 14336 x 4096, blocks resident in HBM",
                             "quantize": "all 226 tensors of the model, f32 resident in HBM"}[wl["kind"]]},

@@ -193,7 +193,7 @@ struct CalibratedTensor {
 
 // DynamicQuantizer::calibrate_tensor (crates/pmetal-gguf/src/dynamic.rs:420-502) with the round trips on the GPU: the
 // tensor is uploaded once; every candidate is quantized, dequantized and scored on the device.  A candidate without
-// kernels here (Q3_K, Q2_K), or a shape whose byte size is not the quantized tensor's, is skipped, as the reference
+// kernels here, or a shape whose byte size is not the quantized tensor's, is skipped, as the reference
 // skips a candidate whose quantize or dequantize fails.
 inline CalibratedTensor calibrate_tensor(const std::string &name, const float *data, size_t n, const std::vector<int32_t> &shape,
                                          const KlCalibrationConfig &cfg = KlCalibrationConfig()) {
@@ -238,7 +238,7 @@ inline GgmlType q4km_tensor_type(const std::string &gguf_name, size_t ndim, size
 
 
 // quantize(data, dtype) for every type the Q4_K_M recipe yields: F32 and F16 are conversions on the host
-// (crates/pmetal-gguf/src/quantize.rs:19-30), Q8_0 / Q4K / Q5K / Q6K run on the GPU, anything else is the
+// (crates/pmetal-gguf/src/quantize.rs:19-30), Q8_0 and the k-quants run on the GPU, anything else is the
 // reference's "not yet implemented" error.
 inline std::vector<uint8_t> quantize_any(const float *data, size_t n, GgmlType dtype) {
     if (dtype == GgmlType::F32) {

@@ -16,6 +16,7 @@ LIB_PATH = os.path.join(HERE, "libpmetal_oracle.so")
 
 TYPE_F32, TYPE_F16, TYPE_Q8_0, TYPE_Q4K, TYPE_Q6K = 0, 1, 8, 12, 14
 TYPE_Q5K, TYPE_Q8K = 13, 15
+TYPE_Q2K, TYPE_Q3K = 10, 11
 ORDER_REF, ORDER_GGML = 0, 1
 OK, ERR_UNSUPPORTED_TYPE, ERR_INVALID_SIZE, ERR_INVALID_SHAPE, ERR_SHAPE_TOO_LARGE = 0, 2, 3, 6, 7
 
@@ -51,6 +52,8 @@ def lib() -> C.CDLL:
         L.pmo_make_qkx1_quants.restype = None
         L.pmo_make_qx_quants.argtypes = [C.c_int32, C.c_int32, f32p, C.c_int32, i8p]
         L.pmo_make_qx_quants.restype = C.c_float
+        L.pmo_make_q3_quants.argtypes = [f32p, C.c_int32, C.c_int32, C.c_int32, i8p]
+        L.pmo_make_q3_quants.restype = C.c_float
         L.pmo_get_scale_min_k4.argtypes = [C.c_int32, u8p, u8p, u8p]
         L.pmo_get_scale_min_k4.restype = None
         for name in ("pmo_type_size", "pmo_block_size"):
@@ -138,6 +141,14 @@ def make_qx_quants(n: int, nmax: int, x: np.ndarray, rmse_type: int):
     x = np.ascontiguousarray(x, dtype=np.float32)
     ls = np.zeros(n, dtype=np.int8)
     s = lib().pmo_make_qx_quants(n, nmax, _f32p(x), rmse_type, ls.ctypes.data_as(C.POINTER(C.c_int8)))
+    return np.float32(s), ls
+
+
+def make_q3_quants(x: np.ndarray, nmax: int, do_rmse: bool):
+    """quantize.rs:655 ``make_q3_quants``: (scale, quants offset by nmax)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    ls = np.zeros(x.size, dtype=np.int8)
+    s = lib().pmo_make_q3_quants(_f32p(x), x.size, nmax, int(do_rmse), ls.ctypes.data_as(C.POINTER(C.c_int8)))
     return np.float32(s), ls
 
 

@@ -321,6 +321,8 @@ size_t pmo_type_size(uint32_t t) {
     case PMO_TYPE_F32: return 4;
     case PMO_TYPE_F16: return 2;
     case PMO_TYPE_Q8_0: return 34;
+    case PMO_TYPE_Q2K: return 84;
+    case PMO_TYPE_Q3K: return 110;
     case PMO_TYPE_Q4K: return 144;
     case PMO_TYPE_Q5K: return 176;
     case PMO_TYPE_Q6K: return 210;
@@ -334,6 +336,8 @@ size_t pmo_block_size(uint32_t t) {
     case PMO_TYPE_F32:
     case PMO_TYPE_F16: return 1;
     case PMO_TYPE_Q8_0: return 32;
+    case PMO_TYPE_Q2K:
+    case PMO_TYPE_Q3K:
     case PMO_TYPE_Q4K:
     case PMO_TYPE_Q5K:
     case PMO_TYPE_Q6K:
@@ -707,6 +711,242 @@ void pmo_dequantize_q5k(const uint8_t *src, size_t n, float *dst, uint32_t order
 }
 
 /* ------------------------------------------------------------------------- */
+/* k_quants.rs:1242-1321 quantize_q2k, :230-266 dequantize_q2k               */
+/* Block (84 bytes): scales[16] (low nibble scale, high nibble min), qs[64],  */
+/* d f16, dmin f16.                                                           */
+/* ------------------------------------------------------------------------- */
+void pmo_quantize_q2k(const float *xs, size_t n, uint8_t *dst) {
+    size_t n_blocks = n / QK_K + (n % QK_K != 0);
+    memset(dst, 0, n_blocks * 84); /* :1246-1255; a partial last block is skipped (:1259-1261) */
+    for (size_t b = 0; b < n / QK_K; b++) {
+        const float *x = xs + b * QK_K;
+        uint8_t *blk = dst + b * 84, *bscales = blk, *qs = blk + 16;
+        float mins[16], scales[16];
+        for (int j = 0; j < 16; j++) pmo_make_qkx1_quants(3, 5, x + 16 * j, 16, &scales[j], &mins[j]); /* :1267-1271 */
+        float max_scale = 0.0f, max_min = 0.0f; /* :1273-1274 fold(0.0, |max, val| val.max(max)) */
+        for (int j = 0; j < 16; j++) max_scale = rust_max(scales[j], max_scale);
+        for (int j = 0; j < 16; j++) max_min = rust_max(mins[j], max_min);
+        uint16_t d16 = 0, dmin16 = 0;
+        if (max_scale > 0.0f) { /* :1276-1285; `as u8` keeps the low eight bits of the i32 */
+            float iscale = 15.0f / max_scale;
+            for (int j = 0; j < 16; j++) bscales[j] = (uint8_t)(uint32_t)pmo_nearest_int(iscale * scales[j]);
+            d16 = pmo_f32_to_f16(max_scale / 15.0f);
+        }
+        if (max_min > 0.0f) { /* :1287-1296; `l << 4` on a u8 drops the bits shifted out */
+            float iscale = 15.0f / max_min;
+            for (int j = 0; j < 16; j++) {
+                uint8_t l = (uint8_t)(uint32_t)pmo_nearest_int(iscale * mins[j]);
+                bscales[j] |= (uint8_t)(l << 4);
+            }
+            dmin16 = pmo_f32_to_f16(max_min / 15.0f);
+        }
+        memcpy(blk + 80, &d16, 2);
+        memcpy(blk + 82, &dmin16, 2);
+        uint8_t l[QK_K];
+        memset(l, 0, sizeof l);
+        for (int j = 0; j < 16; j++) { /* :1299-1310 */
+            float d = pmo_f16_to_f32(d16) * (float)(bscales[j] & 0xF);
+            if (d == 0.0f) continue;
+            float dm = pmo_f16_to_f32(dmin16) * (float)(bscales[j] >> 4);
+            for (int ii = 0; ii < 16; ii++)
+                l[16 * j + ii] = (uint8_t)clamp_i32(pmo_nearest_int((x[16 * j + ii] + dm) / d), 0, 3);
+        }
+        for (int j = 0; j < QK_K; j += 128) /* :1313-1320 */
+            for (int ll = 0; ll < 32; ll++)
+                qs[j / 4 + ll] = (uint8_t)(l[j + ll] | (l[j + ll + 32] << 2) | (l[j + ll + 64] << 4) | (l[j + ll + 96] << 6));
+    }
+}
+
+static void dequantize_q2k_block(const uint8_t *blk, float *out) {
+    uint16_t d16, dmin16;
+    memcpy(&d16, blk + 80, 2);
+    memcpy(&dmin16, blk + 82, 2);
+    const float d = pmo_f16_to_f32(d16), min = pmo_f16_to_f32(dmin16);
+    const uint8_t *scales = blk;
+    int idx = 0, is = 0;
+    for (int h = 0; h < 2; h++) { /* :237-265 */
+        const uint8_t *qs = blk + 16 + 32 * h;
+        for (int shift = 0; shift < 8; shift += 2) {
+            for (int sub = 0; sub < 2; sub++) {
+                const uint8_t sc = scales[is++];
+                const float dl = d * (float)(sc & 0xF), ml = min * (float)(sc >> 4);
+                for (int i = 0; i < 16; i++) out[idx++] = dl * (float)((qs[16 * sub + i] >> shift) & 3) - ml;
+            }
+        }
+    }
+}
+
+void pmo_dequantize_q2k(const uint8_t *src, size_t n, float *dst) {
+    size_t n_blocks = n / QK_K + (n % QK_K != 0);
+    float tmp[QK_K];
+    for (size_t b = 0; b < n_blocks; b++) {
+        dequantize_q2k_block(src + b * 84, tmp);
+        size_t cnt = n - b * QK_K < QK_K ? n - b * QK_K : QK_K;
+        memcpy(dst + b * QK_K, tmp, cnt * sizeof(float));
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* quantize.rs:655-727 make_q3_quants; k_quants.rs:1139-1237 quantize_q3k,    */
+/* :281-355 dequantize_q3k.  Block (110 bytes): hmask[32], qs[64],            */
+/* scales[12], d f16.                                                         */
+/* ------------------------------------------------------------------------- */
+float pmo_make_q3_quants(const float *x, int32_t n, int32_t nmax, int32_t do_rmse, int8_t *ls) {
+    int8_t l[QK_K];
+    memset(l, 0, sizeof l);
+    float max = 0.0f, amax = 0.0f; /* :659-667 */
+    for (int32_t i = 0; i < n; i++) {
+        float ax = fabsf(x[i]);
+        if (ax > amax) {
+            amax = ax;
+            max = x[i];
+        }
+    }
+    if (amax == 0.0f) { /* :669-671 */
+        if (ls) memset(ls, 0, (size_t)n);
+        return 0.0f;
+    }
+    float iscale = -(float)nmax / max; /* :673 */
+    if (do_rmse) {
+        float sumlx = 0.0f, suml2 = 0.0f; /* :676-685 */
+        for (int32_t i = 0; i < n; i++) {
+            int32_t li = clamp_i32(f32_as_i32(roundf(iscale * x[i])), -nmax, nmax - 1);
+            l[i] = (int8_t)li;
+            float w = x[i] * x[i];
+            sumlx += w * x[i] * (float)li;
+            suml2 += w * (float)(li * li);
+        }
+        for (int sweep = 0; sweep < 5; sweep++) { /* :688-713 */
+            int n_changed = 0;
+            for (int32_t i = 0; i < n; i++) {
+                float w = x[i] * x[i];
+                float slx = sumlx - w * x[i] * (float)l[i];
+                if (slx > 0.0f) {
+                    float sl2 = suml2 - w * (float)((int32_t)l[i] * (int32_t)l[i]);
+                    int32_t new_l = clamp_i32(f32_as_i32(roundf(x[i] * sl2 / slx)), -nmax, nmax - 1);
+                    if (new_l != (int32_t)l[i]) {
+                        slx += w * x[i] * (float)new_l;
+                        sl2 += w * (float)(new_l * new_l);
+                        if (sl2 > 0.0f && slx * slx * suml2 > sumlx * sumlx * sl2) {
+                            l[i] = (int8_t)new_l;
+                            sumlx = slx;
+                            suml2 = sl2;
+                            n_changed++;
+                        }
+                    }
+                }
+            }
+            if (n_changed == 0) break;
+        }
+        if (ls)
+            for (int32_t i = 0; i < n; i++) ls[i] = (int8_t)(l[i] + nmax); /* :715-717 */
+        return sumlx / suml2;
+    }
+    for (int32_t i = 0; i < n; i++) { /* :722-726 */
+        int32_t li = clamp_i32(f32_as_i32(roundf(iscale * x[i])), -nmax, nmax - 1);
+        if (ls) ls[i] = (int8_t)(li + nmax);
+    }
+    return 1.0f / iscale;
+}
+
+void pmo_quantize_q3k(const float *xs, size_t n, uint8_t *dst) {
+    size_t n_blocks = n / QK_K + (n % QK_K != 0);
+    memset(dst, 0, n_blocks * 110); /* :1141-1150; a partial last block is skipped (:1154-1156) */
+    for (size_t b = 0; b < n / QK_K; b++) {
+        const float *x = xs + b * QK_K;
+        uint8_t *blk = dst + b * 110, *hmask = blk, *qs = blk + 32, *bscales = blk + 96;
+        float scales_f[16];
+        for (int j = 0; j < 16; j++) scales_f[j] = pmo_make_q3_quants(x + 16 * j, 16, 4, 1, NULL); /* :1159-1162 */
+        float max_scale = 0.0f; /* :1165-1170 */
+        for (int j = 0; j < 16; j++)
+            if (fabsf(scales_f[j]) > fabsf(max_scale)) max_scale = scales_f[j];
+        uint16_t d16 = pmo_f32_to_f16(0.0f);
+        if (max_scale != 0.0f) { /* :1174-1186 */
+            float iscale = -32.0f / max_scale;
+            for (int j = 0; j < 16; j++) {
+                int32_t l_val = clamp_i32(pmo_nearest_int(iscale * scales_f[j]), -32, 31) + 32;
+                if (j < 8) bscales[j] = (uint8_t)(l_val & 0xF);
+                else bscales[j - 8] |= (uint8_t)((l_val & 0xF) << 4);
+                l_val >>= 4;
+                bscales[j % 4 + 8] |= (uint8_t)(l_val << (2 * (j / 4)));
+            }
+            d16 = pmo_f32_to_f16(1.0f / iscale);
+        }
+        memcpy(blk + 108, &d16, 2);
+        int8_t l[QK_K];
+        memset(l, 0, sizeof l);
+        for (int j = 0; j < 16; j++) { /* :1192-1206 */
+            uint8_t sc = j < 8 ? (uint8_t)(bscales[j] & 0xF) : (uint8_t)(bscales[j - 8] >> 4);
+            int8_t scs = (int8_t)((int8_t)(sc | (((bscales[8 + j % 4] >> (2 * (j / 4))) & 3) << 4)) - 32);
+            float d = pmo_f16_to_f32(d16) * (float)scs;
+            if (d != 0.0f)
+                for (int ii = 0; ii < 16; ii++)
+                    l[16 * j + ii] = (int8_t)(clamp_i32(pmo_nearest_int(x[16 * j + ii] / d), -4, 3) + 4);
+        }
+        int m = 0; /* :1209-1224 */
+        uint8_t hm = 1;
+        for (int i = 0; i < QK_K; i++) {
+            if (l[i] > 3) {
+                hmask[m] |= hm;
+                l[i] = (int8_t)(l[i] - 4);
+            }
+            if (++m == QK_K / 8) {
+                m = 0;
+                hm = (uint8_t)(hm << 1);
+            }
+        }
+        for (int j = 0; j < QK_K; j += 128) /* :1227-1234 */
+            for (int ll = 0; ll < 32; ll++)
+                qs[j / 4 + ll] = (uint8_t)(l[j + ll] | (l[j + ll + 32] << 2) | (l[j + ll + 64] << 4) | (l[j + ll + 96] << 6));
+    }
+}
+
+static void dequantize_q3k_block(const uint8_t *blk, float *out) {
+    uint16_t d16;
+    memcpy(&d16, blk + 108, 2);
+    const float d = pmo_f16_to_f32(d16);
+    const uint8_t *hmask = blk, *bscales = blk + 96;
+    uint32_t aux[4] = {0, 0, 0, 0}; /* :285-314 */
+    for (int i = 0; i < 3; i++)
+        aux[i] = (uint32_t)bscales[4 * i] | (uint32_t)bscales[4 * i + 1] << 8 | (uint32_t)bscales[4 * i + 2] << 16 |
+                 (uint32_t)bscales[4 * i + 3] << 24;
+    const uint32_t k1 = 0x03030303u, k2 = 0x0f0f0f0fu, tmp = aux[2];
+    aux[2] = ((aux[0] >> 4) & k2) | (((tmp >> 4) & k1) << 4);
+    aux[3] = ((aux[1] >> 4) & k2) | (((tmp >> 6) & k1) << 4);
+    aux[0] = (aux[0] & k2) | ((tmp & k1) << 4);
+    aux[1] = (aux[1] & k2) | (((tmp >> 2) & k1) << 4);
+    int8_t scales[16]; /* :317-323 */
+    for (int i = 0; i < 4; i++)
+        for (int j = 0; j < 4; j++) scales[4 * i + j] = (int8_t)((int8_t)(uint8_t)(aux[i] >> (8 * j)) - 32);
+    int is = 0, idx = 0; /* :332-354 */
+    uint8_t m = 1;
+    for (int h = 0; h < 2; h++) {
+        const uint8_t *qs = blk + 32 + 32 * h;
+        for (int shift = 0; shift < 8; shift += 2) {
+            for (int sub = 0; sub < 2; sub++) {
+                const float dl = d * (float)scales[is++];
+                for (int i = 0; i < 16; i++) {
+                    const int qi = i + 16 * sub;
+                    const int8_t q = (int8_t)(((qs[qi] >> shift) & 3) + ((hmask[qi] & m) ? 0 : -4));
+                    out[idx++] = dl * (float)q;
+                }
+            }
+            m = (uint8_t)(m << 1);
+        }
+    }
+}
+
+void pmo_dequantize_q3k(const uint8_t *src, size_t n, float *dst) {
+    size_t n_blocks = n / QK_K + (n % QK_K != 0);
+    float tmp[QK_K];
+    for (size_t b = 0; b < n_blocks; b++) {
+        dequantize_q3k_block(src + b * 110, tmp);
+        size_t cnt = n - b * QK_K < QK_K ? n - b * QK_K : QK_K;
+        memcpy(dst + b * QK_K, tmp, cnt * sizeof(float));
+    }
+}
+
+/* ------------------------------------------------------------------------- */
 /* Q8_K: k_quants.rs:815-871 quantize_q8k; vec_dot.rs:617-692 (scalar)        */
 /* ------------------------------------------------------------------------- */
 size_t pmo_q8k_size(size_t n) { return (n / 256 + (n % 256 != 0)) * 292; }
@@ -866,9 +1106,12 @@ int32_t pmo_qmatvec_q8k(uint32_t t, const uint8_t *w, size_t n_rows, size_t k, c
 /* quantize.rs:17-87 and dequant.rs:92-132, :184-216                         */
 /* ------------------------------------------------------------------------- */
 int32_t pmo_quantize(uint32_t t, const float *x, size_t n, uint8_t *dst, size_t dst_len) {
-    if (t != PMO_TYPE_Q8_0 && t != PMO_TYPE_Q4K && t != PMO_TYPE_Q5K && t != PMO_TYPE_Q6K && t != PMO_TYPE_Q8K) return PMO_ERR_UNSUPPORTED_TYPE;
+    if (t != PMO_TYPE_Q8_0 && t != PMO_TYPE_Q2K && t != PMO_TYPE_Q3K && t != PMO_TYPE_Q4K && t != PMO_TYPE_Q5K && t != PMO_TYPE_Q6K && t != PMO_TYPE_Q8K)
+        return PMO_ERR_UNSUPPORTED_TYPE;
     if (dst_len != pmo_tensor_size(t, n)) return PMO_ERR_INVALID_SIZE;
     if (t == PMO_TYPE_Q8K) pmo_quantize_q8k(x, n, dst);
+    else if (t == PMO_TYPE_Q2K) pmo_quantize_q2k(x, n, dst);
+    else if (t == PMO_TYPE_Q3K) pmo_quantize_q3k(x, n, dst);
     else if (t == PMO_TYPE_Q8_0) pmo_quantize_q8_0(x, n, dst);
     else if (t == PMO_TYPE_Q4K) pmo_quantize_q4k(x, n, dst);
     else if (t == PMO_TYPE_Q5K) pmo_quantize_q5k(x, n, dst);
@@ -878,7 +1121,8 @@ int32_t pmo_quantize(uint32_t t, const float *x, size_t n, uint8_t *dst, size_t 
 
 int32_t pmo_dequantize(uint32_t t, const uint8_t *src, size_t src_len, const int32_t *shape, size_t ndim,
                        float *dst, size_t dst_cap, uint32_t order) {
-    if (t != PMO_TYPE_Q8_0 && t != PMO_TYPE_Q4K && t != PMO_TYPE_Q5K && t != PMO_TYPE_Q6K && t != PMO_TYPE_Q8K) return PMO_ERR_UNSUPPORTED_TYPE;
+    if (t != PMO_TYPE_Q8_0 && t != PMO_TYPE_Q2K && t != PMO_TYPE_Q3K && t != PMO_TYPE_Q4K && t != PMO_TYPE_Q5K && t != PMO_TYPE_Q6K && t != PMO_TYPE_Q8K)
+        return PMO_ERR_UNSUPPORTED_TYPE;
     /* dequant.rs:193-206 shape_n_elements */
     for (size_t i = 0; i < ndim; i++)
         if (shape[i] < 0) return PMO_ERR_INVALID_SHAPE;
@@ -895,6 +1139,8 @@ int32_t pmo_dequantize(uint32_t t, const uint8_t *src, size_t src_len, const int
     else if (t == PMO_TYPE_Q4K) pmo_dequantize_q4k(src, n, dst, order);
     else if (t == PMO_TYPE_Q5K) pmo_dequantize_q5k(src, n, dst, order);
     else if (t == PMO_TYPE_Q8K) pmo_dequantize_q8k(src, n, dst);
+    else if (t == PMO_TYPE_Q2K) pmo_dequantize_q2k(src, n, dst);
+    else if (t == PMO_TYPE_Q3K) pmo_dequantize_q3k(src, n, dst);
     else pmo_dequantize_q6k(src, n, dst);
     return PMO_OK;
 }

@@ -29,6 +29,8 @@ enum {
     PMO_TYPE_F32 = 0,
     PMO_TYPE_F16 = 1,
     PMO_TYPE_Q8_0 = 8,
+    PMO_TYPE_Q2K = 10, /* quantize / dequantize only */
+    PMO_TYPE_Q3K = 11, /* quantize / dequantize only */
     PMO_TYPE_Q4K = 12,
     PMO_TYPE_Q5K = 13, /* quantize / dequantize only */
     PMO_TYPE_Q6K = 14,
@@ -79,6 +81,13 @@ void pmo_quantize_q6k(const float *x, size_t n, uint8_t *dst);
 /* k_quants.rs:960-1051 (176-byte blocks: d, dmin, scales[12], qh[32], qs[128]) */
 void pmo_quantize_q5k(const float *x, size_t n, uint8_t *dst);
 
+/* k_quants.rs:1242-1321 (84-byte blocks: scales[16], qs[64], d, dmin) and :1139-1237 (110-byte blocks: hmask[32],
+ * qs[64], scales[12], d) */
+void pmo_quantize_q2k(const float *x, size_t n, uint8_t *dst);
+void pmo_quantize_q3k(const float *x, size_t n, uint8_t *dst);
+/* quantize.rs:655-727: returns the scale; ls (may be NULL) receives the n quants, offset by nmax */
+float pmo_make_q3_quants(const float *x, int32_t n, int32_t nmax, int32_t do_rmse, int8_t *ls);
+
 /* dequant.rs:466-495, k_quants.rs:358-404 + 515-560, k_quants.rs:474-496 + 614-660.
  * src holds pmo_tensor_size(type, n) bytes; dst receives n floats. */
 void pmo_dequantize_q8_0(const uint8_t *src, size_t n, float *dst);
@@ -86,6 +95,10 @@ void pmo_dequantize_q4k(const uint8_t *src, size_t n, float *dst, uint32_t order
 void pmo_dequantize_q6k(const uint8_t *src, size_t n, float *dst);
 /* k_quants.rs:407-462 + :663-710; order 0 = the reference's emission order, 1 = the inverse of quantize_q5k's packing */
 void pmo_dequantize_q5k(const uint8_t *src, size_t n, float *dst, uint32_t order);
+
+/* k_quants.rs:230-266 + :762-810 and :281-355 + :713-760 (both are the inverses of their quantizers' packing) */
+void pmo_dequantize_q2k(const uint8_t *src, size_t n, float *dst);
+void pmo_dequantize_q3k(const uint8_t *src, size_t n, float *dst);
 
 /* quantize.rs:17-87 (dispatcher) and dequant.rs:92-132 + 184-216 (dispatcher and
  * validation).  Return a PMO_* code. */

@@ -56,7 +56,9 @@ bool path_type(uint32_t t) {
 }
 // types with quantize / dequantize kernels: the above, Q5_K (the Q4_K_M recipe gives it to fused attn_qkv tensors) and
 // Q8_K (the activation format of the integer dot products, and the first candidate of the KL calibration)
-bool codec_type(uint32_t t) { return path_type(t) || t == PMETAL_GGML_TYPE_Q5K || t == PMETAL_GGML_TYPE_Q8K; }
+bool codec_type(uint32_t t) {
+    return path_type(t) || t == PMETAL_GGML_TYPE_Q2K || t == PMETAL_GGML_TYPE_Q3K || t == PMETAL_GGML_TYPE_Q5K || t == PMETAL_GGML_TYPE_Q8K;
+}
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -170,6 +172,8 @@ size_t pmetal_hip_type_size(uint32_t t) {
     switch (t) {
     case PMETAL_GGML_TYPE_Q8_0: return 34;
     case PMETAL_GGML_TYPE_Q4K: return 144;
+    case PMETAL_GGML_TYPE_Q2K: return 84;
+    case PMETAL_GGML_TYPE_Q3K: return 110;
     case PMETAL_GGML_TYPE_Q5K: return 176;
     case PMETAL_GGML_TYPE_Q6K: return 210;
     case PMETAL_GGML_TYPE_Q8K: return 292;
@@ -181,6 +185,8 @@ size_t pmetal_hip_block_size(uint32_t t) {
     switch (t) {
     case PMETAL_GGML_TYPE_Q8_0: return 32;
     case PMETAL_GGML_TYPE_Q4K:
+    case PMETAL_GGML_TYPE_Q2K:
+    case PMETAL_GGML_TYPE_Q3K:
     case PMETAL_GGML_TYPE_Q5K:
     case PMETAL_GGML_TYPE_Q6K:
     case PMETAL_GGML_TYPE_Q8K: return 256;
@@ -367,6 +373,8 @@ int32_t pmetal_hip_quantize_dev(uint32_t t, const float *src, size_t n, uint8_t 
     else if (t == PMETAL_GGML_TYPE_Q4K) e = pmh::launch_quantize_q4k(src, n, dst, s);
     else if (t == PMETAL_GGML_TYPE_Q5K) e = pmh::launch_quantize_q5k(src, n, dst, s);
     else if (t == PMETAL_GGML_TYPE_Q8K) e = pmh::launch_quantize_q8k(src, n, dst, s);
+    else if (t == PMETAL_GGML_TYPE_Q2K) e = pmh::launch_quantize_q2k(src, n, dst, s);
+    else if (t == PMETAL_GGML_TYPE_Q3K) e = pmh::launch_quantize_q3k(src, n, dst, s);
     else e = pmh::launch_quantize_q6k(src, n, dst, s);
     if (e != hipSuccess) return hip_fail(e, "quantize kernel launch");
     return ok();
@@ -408,6 +416,8 @@ int32_t pmetal_hip_dequantize_dev(uint32_t t, const uint8_t *src, size_t src_len
     else if (t == PMETAL_GGML_TYPE_Q4K) e = pmh::launch_dequantize_q4k(src, n, dst, order, s);
     else if (t == PMETAL_GGML_TYPE_Q5K) e = pmh::launch_dequantize_q5k(src, n, dst, order, s);
     else if (t == PMETAL_GGML_TYPE_Q8K) e = pmh::launch_dequantize_q8k(src, n, dst, s);
+    else if (t == PMETAL_GGML_TYPE_Q2K) e = pmh::launch_dequantize_q2k(src, n, dst, s);
+    else if (t == PMETAL_GGML_TYPE_Q3K) e = pmh::launch_dequantize_q3k(src, n, dst, s);
     else e = pmh::launch_dequantize_q6k(src, n, dst, s);
     if (e != hipSuccess) return hip_fail(e, "dequantize kernel launch");
     return ok();

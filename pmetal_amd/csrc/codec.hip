@@ -721,6 +721,322 @@ inline unsigned grid_for(size_t work_items, size_t per_block) {
     return (unsigned)((work_items + per_block - 1) / per_block);
 }
 
+// -------------------------------------------------------------------------------------------
+// Q2_K and Q3_K (quantize / dequantize only).  Both have sixteen 16-element sub-blocks per super-block and pack the
+// low two bits of element e into qs[32 (e / 128) + e % 32] at bit 2 ((e % 128) / 32); both dequantizers are the
+// inverses of that packing, so there is one element order.
+// -------------------------------------------------------------------------------------------
+
+// Q2_K dequantize (k_quants.rs:230-266 + :762-810): out = (d * (sc & 15)) * q - dmin * (sc >> 4).  84-byte blocks:
+// scales[16], qs[64], d, dmin.  One wave per super-block, four outputs per lane.
+__global__ __launch_bounds__(256) void k_dequantize_q2k(const uint8_t *__restrict__ src, size_t n,
+                                                         float *__restrict__ dst) {
+    const size_t wave = ((size_t)blockIdx.x * 256 + threadIdx.x) >> 6;
+    const int i = (int)(threadIdx.x & 63);
+    const int h = i >> 5, p = (i >> 3) & 3, l = (i & 7) * 4;
+    uint32_t qw[kDeqUnroll], scb[kDeqUnroll], dd[kDeqUnroll];
+#pragma unroll
+    for (int u = 0; u < kDeqUnroll; u++) {
+        const size_t blk_i = wave * kDeqUnroll + u;
+        const bool live = blk_i * 256 + (size_t)i * 4 < n;
+        const uint8_t *blk = src + (live ? blk_i : 0) * 84;  // lanes past the end re-read the first block
+        qw[u] = *reinterpret_cast<const uint32_t *>(blk + 16 + 32 * h + l);
+        scb[u] = blk[i >> 2];
+        dd[u] = *reinterpret_cast<const uint32_t *>(blk + 80);
+    }
+#pragma unroll
+    for (int u = 0; u < kDeqUnroll; u++) {
+        const size_t e = (wave * kDeqUnroll + u) * 256 + (size_t)i * 4;
+        if (e >= n) continue;
+        const float dl = f16_bits_to_f32(dd[u] & 0xFFFFu) * (float)(scb[u] & 0xFu);
+        const float ml = f16_bits_to_f32(dd[u] >> 16) * (float)(scb[u] >> 4);
+        float o[4];
+#pragma unroll
+        for (int t = 0; t < 4; t++) o[t] = dl * (float)((qw[u] >> (8 * t + 2 * p)) & 3u) - ml;
+        if (e + 3 < n) {
+            *reinterpret_cast<float4 *>(dst + e) = make_float4(o[0], o[1], o[2], o[3]);
+        } else {
+            for (int t = 0; t < 4 && e + t < n; t++) dst[e + t] = o[t];
+        }
+    }
+}
+
+// Q3_K dequantize (k_quants.rs:281-355 + :713-760): out = (d * (sc6 - 32)) * (q2 - (hbit ? 0 : 4)).  110-byte blocks:
+// hmask[32], qs[64], scales[12], d; the high bit of element e is bit e / 32 of hmask[e % 32]; the sixteen 6-bit
+// scales are four low bits in the nibbles of scales[0..8] and two high bits in scales[8..12].
+__global__ __launch_bounds__(256) void k_dequantize_q3k(const uint8_t *__restrict__ src, size_t n,
+                                                         float *__restrict__ dst) {
+    const size_t wave = ((size_t)blockIdx.x * 256 + threadIdx.x) >> 6;
+    const int i = (int)(threadIdx.x & 63);
+    const int h = i >> 5, p = (i >> 3) & 3, l = (i & 7) * 4, is = i >> 2;
+    uint32_t qw[kDeqUnroll], hw[kDeqUnroll], lo[kDeqUnroll], hi[kDeqUnroll], dd[kDeqUnroll];
+#pragma unroll
+    for (int u = 0; u < kDeqUnroll; u++) {
+        const size_t blk_i = wave * kDeqUnroll + u;
+        const bool live = blk_i * 256 + (size_t)i * 4 < n;
+        const uint8_t *blk = src + (live ? blk_i : 0) * 110;
+        hw[u] = *reinterpret_cast<const u32_a2 *>(blk + l);
+        qw[u] = *reinterpret_cast<const u32_a2 *>(blk + 32 + 32 * h + l);
+        lo[u] = blk[96 + (is & 7)];
+        hi[u] = blk[104 + (is & 3)];
+        dd[u] = *reinterpret_cast<const uint16_t *>(blk + 108);
+    }
+#pragma unroll
+    for (int u = 0; u < kDeqUnroll; u++) {
+        const size_t e = (wave * kDeqUnroll + u) * 256 + (size_t)i * 4;
+        if (e >= n) continue;
+        const uint32_t sc6 = ((is < 8 ? lo[u] : lo[u] >> 4) & 0xFu) | (((hi[u] >> (2 * (is >> 2))) & 3u) << 4);
+        const float dl = f16_bits_to_f32(dd[u]) * (float)((int)sc6 - 32);
+        float o[4];
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const int q = (int)((qw[u] >> (8 * t + 2 * p)) & 3u) - (((hw[u] >> (8 * t + 4 * h + p)) & 1u) ? 0 : 4);
+            o[t] = dl * (float)q;
+        }
+        if (e + 3 < n) {
+            *reinterpret_cast<float4 *>(dst + e) = make_float4(o[0], o[1], o[2], o[3]);
+        } else {
+            for (int t = 0; t < 4 && e + t < n; t++) dst[e + t] = o[t];
+        }
+    }
+}
+
+// The 1024-float tile of four super-blocks, one 16-element sub-block per lane: staged through LDS with a row stride
+// of 17 floats so that the lanes' column-wise reads do not collide.
+constexpr int kSub16Stride = 17;
+__device__ __forceinline__ void load_sub16(const float *__restrict__ x, size_t n_sb, size_t sb0, float *xs, float (&xv)[16]) {
+    const int lane = threadIdx.x;
+    const size_t n_valid = (n_sb - sb0 < 4 ? n_sb - sb0 : 4) * 256;  // floats this wave may read
+    const float *src = x + sb0 * 256;
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int idx = it * 64 + lane;  // float4 index inside the tile
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if ((size_t)idx * 4 < n_valid) v = *reinterpret_cast<const float4 *>(src + idx * 4);
+        float *q = xs + (idx >> 2) * kSub16Stride + (idx & 3) * 4;
+        q[0] = v.x, q[1] = v.y, q[2] = v.z, q[3] = v.w;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 16; i++) xv[i] = xs[lane * kSub16Stride + i];
+}
+
+// Sub-block j = 8 h + 2 p + s of a super-block holds the elements whose low bits go to qs[32 h + 16 s + i] at bit 2 p.
+// The four lanes of one (h, s) or their sixteen bytes together and lane p stores dword p of them.
+__device__ __forceinline__ void store_qs2(const uint32_t (&q)[16], int j, uint8_t *qs) {
+    const int p = (j >> 1) & 3;
+    uint32_t w[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        w[k] = (q[4 * k] | (q[4 * k + 1] << 8) | (q[4 * k + 2] << 16) | (q[4 * k + 3] << 24)) << (2 * p);
+        w[k] |= __shfl_xor(w[k], 2);
+        w[k] |= __shfl_xor(w[k], 4);
+    }
+    const uint32_t mine = p == 0 ? w[0] : (p == 1 ? w[1] : (p == 2 ? w[2] : w[3]));
+    if (qs) *reinterpret_cast<u32_a2 *>(qs + 32 * (j >> 3) + 16 * (j & 1) + 4 * p) = mine;
+}
+
+// Q2_K quantize (k_quants.rs:1242-1321): make_qkx1_quants(3, 5) (quantize.rs:583-644) per 16-element sub-block, 4-bit
+// scales and mins against d = max_scale / 15 and dmin = max_min / 15, requantization with the decoded f16 values.
+__global__ __launch_bounds__(64) void k_quantize_q2k(const float *__restrict__ x, size_t n_sb, uint8_t *__restrict__ dst) {
+    __shared__ float xs[64 * kSub16Stride];
+    const int lane = threadIdx.x, j = lane & 15;
+    const size_t sb0 = (size_t)blockIdx.x * 4;
+    float xv[16];
+    load_sub16(x, n_sb, sb0, xs, xv);
+
+    // ---- make_qkx1_quants(3, 5, xv) ----
+    int kmn = total_key(xv[0]), kmx = kmn;
+#pragma unroll
+    for (int i = 1; i < 16; i++) {
+        const int key = total_key(xv[i]);
+        kmn = key < kmn ? key : kmn;
+        kmx = key > kmx ? key : kmx;
+    }
+    const float mn = __builtin_bit_cast(float, kmn ^ (int)(((unsigned)(kmn >> 31)) >> 1));
+    const float mx = __builtin_bit_cast(float, kmx ^ (int)(((unsigned)(kmx >> 31)) >> 1));
+    float scale = 0.0f, neg_min = 0.0f;
+    if (!(mx == mn)) {
+        float minv = __builtin_fminf(mn, 0.0f);
+        float iscale = 3.0f / (mx - minv);
+        scale = 1.0f / iscale;
+        float lf[16];
+#pragma unroll
+        for (int i = 0; i < 16; i++) lf[i] = 0.0f;
+#pragma unroll
+        for (int t = 0; t < 5; t++) {
+            float sumlx = 0.0f, suml2 = 0.0f;  // suml2 <= 16 * 9: exact in f32
+            bool changed = false;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const float xm = xv[i] - minv;
+                const float r = clamp_round_0_15<3>(iscale * xm);
+                changed |= (r != lf[i]);
+                lf[i] = r;
+                sumlx += xm * r;
+                suml2 = __builtin_fmaf(r, r, suml2);
+            }
+            if (suml2 == 0.0f) break;
+            scale = sumlx / suml2;
+            float sum = -0.0f;  // Iterator::sum::<f32> folds from -0.0
+#pragma unroll
+            for (int i = 0; i < 16; i++) sum += xv[i] - scale * lf[i];
+            minv = sum / 16.0f;
+            if (minv > 0.0f) minv = 0.0f;
+            iscale = 1.0f / scale;
+            if (!changed) break;
+        }
+        neg_min = -minv;
+    }
+
+    // ---- super-block level (k_quants.rs:1273-1296): the 16 lanes of a super-block cooperate ----
+    float max_scale = scale, max_min = neg_min;
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+        max_scale = __builtin_fmaxf(max_scale, __shfl_xor(max_scale, off));
+        max_min = __builtin_fmaxf(max_min, __shfl_xor(max_min, off));
+    }
+    max_scale = __builtin_fmaxf(max_scale, 0.0f);  // fold(0.0, max): NaNs drop out, +0.0 wins over -0.0
+    max_min = __builtin_fmaxf(max_min, 0.0f);
+    uint32_t byte = 0, d16 = 0, dmin16 = 0;
+    if (max_scale > 0.0f) {
+        byte = (uint32_t)f32_as_i32(round_half_away((15.0f / max_scale) * scale)) & 0xFFu;  // `as u8`
+        d16 = f32_to_f16_bits(max_scale / 15.0f);
+    }
+    if (max_min > 0.0f) {
+        const uint32_t lm = (uint32_t)f32_as_i32(round_half_away((15.0f / max_min) * neg_min)) & 0xFFu;
+        byte |= (lm << 4) & 0xFFu;
+        dmin16 = f32_to_f16_bits(max_min / 15.0f);
+    }
+
+    // ---- requantize (k_quants.rs:1299-1310) ----
+    uint32_t q[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) q[i] = 0;
+    const float dq = f16_bits_to_f32(d16) * (float)(byte & 0xFu);
+    if (dq != 0.0f) {
+        const float dm = f16_bits_to_f32(dmin16) * (float)(byte >> 4);
+#pragma unroll
+        for (int i = 0; i < 16; i++) q[i] = (uint32_t)clamp_round_0_15<3>((xv[i] + dm) / dq);
+    }
+    const size_t sb = sb0 + (lane >> 4);
+    uint8_t *blk = sb < n_sb ? dst + sb * 84 : nullptr;
+    store_qs2(q, j, blk ? blk + 16 : nullptr);
+    if (blk) {
+        blk[j] = (uint8_t)byte;
+        if (j == 0) *reinterpret_cast<uint32_t *>(blk + 80) = d16 | (dmin16 << 16);
+    }
+}
+
+// Q3_K quantize (k_quants.rs:1139-1237): make_q3_quants(x, 4, true) (quantize.rs:655-719) per 16-element sub-block,
+// 6-bit signed scales against d = 1 / iscale with iscale = -32 / (the scale of largest magnitude, the first of equals),
+// requantization with the decoded f16 value.
+__global__ __launch_bounds__(64) void k_quantize_q3k(const float *__restrict__ x, size_t n_sb, uint8_t *__restrict__ dst) {
+    __shared__ float xs[64 * kSub16Stride];
+    const int lane = threadIdx.x, j = lane & 15;
+    const size_t sb0 = (size_t)blockIdx.x * 4;
+    float xv[16];
+    load_sub16(x, n_sb, sb0, xs, xv);
+
+    // ---- make_q3_quants(xv, 4, true) ----
+    float maxv = 0.0f, amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const float ax = __builtin_fabsf(xv[i]);
+        if (ax > amax) amax = ax, maxv = xv[i];
+    }
+    float scale = 0.0f;
+    if (amax != 0.0f) {
+        const float iscale = -4.0f / maxv;
+        int l[16];
+        float sumlx = 0.0f, suml2 = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            l[i] = clamp_i(nearest_int_sat(iscale * xv[i]), -4, 3);
+            const float w = xv[i] * xv[i];
+            sumlx += w * xv[i] * (float)l[i];
+            suml2 += w * (float)(l[i] * l[i]);
+        }
+        for (int sweep = 0; sweep < 5; sweep++) {
+            bool any = false;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const float w = xv[i] * xv[i], wx = w * xv[i];
+                float slx = sumlx - wx * (float)l[i];
+                if (slx > 0.0f) {
+                    float sl2 = suml2 - w * (float)(l[i] * l[i]);
+                    const int nl = clamp_i(nearest_int_sat(xv[i] * sl2 / slx), -4, 3);
+                    if (nl != l[i]) {
+                        slx += wx * (float)nl;
+                        sl2 += w * (float)(nl * nl);
+                        if (sl2 > 0.0f && slx * slx * suml2 > sumlx * sumlx * sl2) {
+                            l[i] = nl, sumlx = slx, suml2 = sl2, any = true;
+                        }
+                    }
+                }
+            }
+            if (!any) break;
+        }
+        scale = sumlx / suml2;
+    }
+
+    // ---- super-block level (k_quants.rs:1165-1186) ----
+    // `if scale.abs() > max_scale.abs()` in order: the first of the largest magnitudes; NaN never compares greater
+    const float mag = scale == scale ? __builtin_fabsf(scale) : 0.0f;
+    float big = mag;
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) big = __builtin_fmaxf(big, __shfl_xor(big, off));
+    const unsigned long long hit = __ballot(mag == big);
+    const int first = __builtin_ctzll(((hit >> (lane & 48)) & 0xFFFFull) | 0x10000ull) & 15;
+    const float max_scale = big > 0.0f ? __shfl(scale, (lane & 48) + first) : 0.0f;
+    int lv = 0;
+    uint32_t d16 = 0;
+    if (max_scale != 0.0f) {
+        const float iscale = -32.0f / max_scale;
+        lv = clamp_i(nearest_int_sat(iscale * scale), -32, 31) + 32;
+        d16 = f32_to_f16_bits(1.0f / iscale);
+    }
+    // scales[j] = (l_j & 15) | (l_{j+8} & 15) << 4 for j < 8; scales[8 + i] = sum_k (l_{i+4k} >> 4) << 2k
+    const uint32_t lo = (uint32_t)lv & 0xFu, lo_hi = __shfl_xor(lo, 8);
+    uint32_t top = ((uint32_t)lv >> 4) << (2 * (j >> 2));
+    top |= __shfl_xor(top, 4);
+    top |= __shfl_xor(top, 8);
+
+    // ---- requantize (k_quants.rs:1192-1206), high bits (:1209-1224) ----
+    uint32_t q[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) q[i] = 0;
+    const float dq = f16_bits_to_f32(d16) * (float)(lv - 32);
+    if (max_scale != 0.0f && dq != 0.0f) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) q[i] = (uint32_t)(clamp_i(nearest_int_sat(xv[i] / dq), -4, 3) + 4);
+    }
+    // element 16 j + i has its high bit at bit j / 2 of hmask[16 (j % 2) + i]: the eight lanes of one parity or theirs
+    uint32_t hw[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        hw[k] = ((q[4 * k] >> 2) | ((q[4 * k + 1] >> 2) << 8) | ((q[4 * k + 2] >> 2) << 16) | ((q[4 * k + 3] >> 2) << 24)) << (j >> 1);
+        hw[k] |= __shfl_xor(hw[k], 2);
+        hw[k] |= __shfl_xor(hw[k], 4);
+        hw[k] |= __shfl_xor(hw[k], 8);
+    }
+#pragma unroll
+    for (int i = 0; i < 16; i++) q[i] &= 3u;
+    const size_t sb = sb0 + (lane >> 4);
+    uint8_t *blk = sb < n_sb ? dst + sb * 110 : nullptr;
+    store_qs2(q, j, blk ? blk + 32 : nullptr);
+    if (blk) {
+        const int k = j >> 1;  // lanes 0..7 of a super-block store the hmask dwords: parity j & 1, dword k & 3
+        if (k < 4) {
+            const uint32_t mine = k == 0 ? hw[0] : (k == 1 ? hw[1] : (k == 2 ? hw[2] : hw[3]));
+            *reinterpret_cast<u32_a2 *>(blk + 16 * (j & 1) + 4 * k) = mine;
+        }
+        if (j < 8) blk[96 + j] = (uint8_t)(lo | (lo_hi << 4));
+        if (j < 4) blk[104 + j] = (uint8_t)top;
+        if (j == 0) *reinterpret_cast<uint16_t *>(blk + 108) = (uint16_t)d16;
+    }
+}
+
 }  // namespace
 
 namespace pmh {
@@ -762,6 +1078,40 @@ hipError_t launch_quantize_q6k(const float *x, size_t n, uint8_t *dst, hipStream
     }
     if (n_sb == 0) return hipSuccess;
     hipLaunchKernelGGL(k_quantize_q6k, dim3(grid_for(n_sb, 4)), dim3(64), 0, s, x, n_sb, dst);
+    return hipGetLastError();
+}
+
+hipError_t launch_quantize_q2k(const float *x, size_t n, uint8_t *dst, hipStream_t s) {
+    const size_t n_sb = n / 256;
+    if (n % 256) {
+        hipError_t e = launch_zero_bytes(dst + n_sb * 84, 84, s);
+        if (e != hipSuccess) return e;
+    }
+    if (n_sb == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_quantize_q2k, dim3(grid_for(n_sb, 4)), dim3(64), 0, s, x, n_sb, dst);
+    return hipGetLastError();
+}
+
+hipError_t launch_quantize_q3k(const float *x, size_t n, uint8_t *dst, hipStream_t s) {
+    const size_t n_sb = n / 256;
+    if (n % 256) {
+        hipError_t e = launch_zero_bytes(dst + n_sb * 110, 110, s);
+        if (e != hipSuccess) return e;
+    }
+    if (n_sb == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_quantize_q3k, dim3(grid_for(n_sb, 4)), dim3(64), 0, s, x, n_sb, dst);
+    return hipGetLastError();
+}
+
+hipError_t launch_dequantize_q2k(const uint8_t *src, size_t n, float *dst, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_dequantize_q2k, dim3(grid_for((n + 4 * kDeqUnroll - 1) / (4 * kDeqUnroll), 256)), dim3(256), 0, s, src, n, dst);
+    return hipGetLastError();
+}
+
+hipError_t launch_dequantize_q3k(const uint8_t *src, size_t n, float *dst, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_dequantize_q3k, dim3(grid_for((n + 4 * kDeqUnroll - 1) / (4 * kDeqUnroll), 256)), dim3(256), 0, s, src, n, dst);
     return hipGetLastError();
 }
 

@@ -7,7 +7,7 @@
 
 namespace pmh {
 
-constexpr uint32_t kTypeQ8_0 = 8, kTypeQ4K = 12, kTypeQ5K = 13, kTypeQ6K = 14, kTypeQ8K = 15;
+constexpr uint32_t kTypeQ8_0 = 8, kTypeQ2K = 10, kTypeQ3K = 11, kTypeQ4K = 12, kTypeQ5K = 13, kTypeQ6K = 14, kTypeQ8K = 15;
 constexpr uint32_t kOrderRef = 0, kOrderGgml = 1;
 constexpr uint32_t kDtypeF32 = 0, kDtypeBf16 = 1;
 
@@ -15,10 +15,14 @@ constexpr uint32_t kDtypeF32 = 0, kDtypeBf16 = 1;
 hipError_t launch_quantize_q8_0(const float *x, size_t n, uint8_t *dst, hipStream_t s);
 hipError_t launch_quantize_q4k(const float *x, size_t n, uint8_t *dst, hipStream_t s);
 hipError_t launch_quantize_q5k(const float *x, size_t n, uint8_t *dst, hipStream_t s);
+hipError_t launch_quantize_q2k(const float *x, size_t n, uint8_t *dst, hipStream_t s);
+hipError_t launch_quantize_q3k(const float *x, size_t n, uint8_t *dst, hipStream_t s);
 hipError_t launch_quantize_q6k(const float *x, size_t n, uint8_t *dst, hipStream_t s);
 hipError_t launch_dequantize_q8_0(const uint8_t *src, size_t n, float *dst, hipStream_t s);
 hipError_t launch_dequantize_q4k(const uint8_t *src, size_t n, float *dst, uint32_t order, hipStream_t s);
 hipError_t launch_dequantize_q5k(const uint8_t *src, size_t n, float *dst, uint32_t order, hipStream_t s);
+hipError_t launch_dequantize_q2k(const uint8_t *src, size_t n, float *dst, hipStream_t s);
+hipError_t launch_dequantize_q3k(const uint8_t *src, size_t n, float *dst, hipStream_t s);
 hipError_t launch_dequantize_q6k(const uint8_t *src, size_t n, float *dst, hipStream_t s);
 
 // ---- gemv.hip: dequant-fused y = W x ----

@@ -213,7 +213,7 @@ def calibrate_tensor(name: str, data, shape, candidates=DEFAULT_KL_CANDIDATES, k
     """``DynamicQuantizer::calibrate_tensor`` (crates/pmetal-gguf/src/dynamic.rs:420-502) with the round trips on the GPU:
     the tensor is uploaded once, every candidate is quantized, dequantized (in the reference dequantizer's element order
     unless ``order`` says otherwise) and scored on the device.  Returns ``(quant_type, kl_score, all_scores)``.  As in
-    the reference, a candidate the quantizer does not implement is skipped (here: Q3_K, Q2_K)."""
+    the reference, a candidate the quantizer does not implement is skipped."""
     lib = _lib.load()
     x = np.ascontiguousarray(data, dtype=np.float32).reshape(-1)
     if is_critical_layer(name):

@@ -177,7 +177,7 @@ static void test_calibration() {  // dynamic.rs:968-1018, :934-956 through the d
     bool member = r.quant_type == cfg.fallback_type;
     for (GgmlType t : cfg.candidates) member = member || t == r.quant_type;
     CHECK(member && !r.all_scores.empty());
-    CHECK(r.all_scores.size() == 4 && r.all_scores[0].first == GgmlType::Q8K && r.all_scores[0].second < 0.01);  // Q3_K, Q2_K skipped
+    CHECK(r.all_scores.size() == 6 && r.all_scores[0].first == GgmlType::Q8K && r.all_scores[0].second < 0.01);
     // compute_kl_divergence: identical -> ~0, perturbed -> small positive, zeros -> 0
     const float a[8] = {1, 2, 3, 4, 5, 0, 0, 0}, b[8] = {1.1f, 2.1f, 2.9f, 4.2f, 4.8f, 0, 0, 0}, z[8] = {0};
     DeviceBuffer da(a, sizeof a), db(b, sizeof b), dz(z, sizeof z);

@@ -45,13 +45,13 @@ def test_critical_layers_and_calibration_logic(oracle):
     # dynamic.rs:987-1018: the ramp; the selected type is a candidate, at least one candidate was scored
     data = (np.arange(256) * 0.01 - 1.28).astype(np.float32)
     t, score, scores = oracle.calibrate_tensor("model.layers.0.mlp.gate_proj.weight", data, [1, 256])
-    assert t in oracle.DEFAULT_CANDIDATES and scores and [s[0] for s in scores] == [Q8K, Q6K, Q5K, Q4K]  # Q3_K, Q2_K: not restated
-    assert scores[0][1] < 0.01 and t == max((s for s in scores if s[1] <= 0.01), key=lambda s: [Q8K, Q6K, Q5K, Q4K].index(s[0]))[0]
+    assert t in oracle.DEFAULT_CANDIDATES and scores and [s[0] for s in scores] == [Q8K, Q6K, Q5K, Q4K, Q3K, Q2K]
+    assert scores[0][1] < 0.01 and t == max((s for s in scores if s[1] <= 0.01), key=lambda s: [Q8K, Q6K, Q5K, Q4K, Q3K, Q2K].index(s[0]))[0]
     # the most compressed candidate under the threshold wins; none under it -> the first (highest quality) one
     x = (np.random.default_rng(1).standard_normal(4096) * 0.02).astype(np.float32)
     _, _, scores = oracle.calibrate_tensor("blk.0.ffn_up.weight", x, [16, 256], order=oracle.ORDER_GGML)
     by = dict(scores)
-    assert by[Q8K] < by[Q6K] < by[Q5K] < by[Q4K]  # fewer bits, more loss (in the order that inverts the quantizer)
+    assert by[Q8K] < by[Q6K] < by[Q5K] < by[Q4K] < by[Q3K] < by[Q2K]  # fewer bits, more loss (in the order that inverts the quantizer)
     assert oracle.calibrate_tensor("blk.0.ffn_up.weight", x, [16, 256], kl_threshold=by[Q5K] * 1.01, order=oracle.ORDER_GGML)[0] == Q5K
     assert oracle.calibrate_tensor("blk.0.ffn_up.weight", x, [16, 256], kl_threshold=by[Q4K] * 1.01, order=oracle.ORDER_GGML)[0] == Q4K
     assert oracle.calibrate_tensor("blk.0.ffn_up.weight", x, [16, 256], kl_threshold=1e-9, order=oracle.ORDER_GGML)[0] == Q8K
@@ -64,9 +64,9 @@ def test_critical_layers_and_calibration_logic(oracle):
     assert t == Q8K and score == np.finfo(np.float64).max and len(scores) == 1
     # a shape a few elements short of the data still has the data's byte size: it is scored on the elements it names
     t, score, scores = oracle.calibrate_tensor("blk.0.ffn_up.weight", x, [16, 255])
-    assert len(scores) == 4 and score < 0.01
-    # no candidate the oracle restates
-    assert oracle.calibrate_tensor("blk.0.ffn_up.weight", x, [16, 256], candidates=(Q3K, Q2K))[1] == np.finfo(np.float64).max
+    assert len(scores) == 6 and score < 0.01
+    # no candidate that the quantizer implements (here and in the reference: the i-quants, quantize.rs:82-85)
+    assert oracle.calibrate_tensor("blk.0.ffn_up.weight", x, [16, 256], candidates=(16, 17))[1] == np.finfo(np.float64).max
 
 
 def test_q8k_dequantize_known_answers(oracle):
@@ -120,7 +120,7 @@ def test_gpu_calibrate_tensor_matches_oracle(oracle):
     }
     for name, (x, shape) in tensors.items():
         for kwargs in ({}, {"order": 1}, {"sample_size": 300}, {"kl_threshold": 0.05, "order": 1}, {"kl_threshold": 1e-9},
-                       {"candidates": (Q6K, Q4K), "fallback_type": Q6K, "order": 1}, {"candidates": (Q3K, Q2K)}):
+                       {"candidates": (Q6K, Q4K), "fallback_type": Q6K, "order": 1}, {"candidates": (Q3K, Q2K), "kl_threshold": 0.5}, {"candidates": (16, 17)}):
             wt, ws, wall = oracle.calibrate_tensor(name, x, shape, **kwargs)
             gt, gs, gall = gguf.calibrate_tensor(name, x, shape, **kwargs)
             assert gt == wt and [t for t, _ in gall] == [t for t, _ in wall], (name, kwargs)
@@ -133,4 +133,4 @@ def test_gpu_calibrate_tensor_matches_oracle(oracle):
     t, score, _ = gguf.calibrate_tensor("blk.0.ffn_up.weight", x, [64, 1000])
     assert t == Q8K and score == np.finfo(np.float64).max
     got, want = gguf.calibrate_tensor("blk.0.ffn_up.weight", x, [64, 1023]), oracle.calibrate_tensor("blk.0.ffn_up.weight", x, [64, 1023])
-    assert got[0] == want[0] and got[1] == pytest.approx(want[1], rel=1e-10, abs=1e-14) and len(got[2]) == len(want[2]) == 4
+    assert got[0] == want[0] and got[1] == pytest.approx(want[1], rel=1e-10, abs=1e-14) and len(got[2]) == len(want[2]) == 6
