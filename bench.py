@@ -207,7 +207,7 @@ def bench_gemv(args, n, k, t=Q4K, copies=16):
         "value": gbs, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "k_qgemv_q4k_chunk", "bytes_per_launch": bytes_per_launch,
+                     "kernel": {Q4K: "k_qgemv_q4k_chunk", Q6K: "k_qgemv_q6k", Q8_0: "k_qgemv_q8_0"}[t], "bytes_per_launch": bytes_per_launch,
                      "us_per_launch": round(us_per_launch, 3)},
         "extra": {"cache_resident_GBps": round(cached_gbs, 1), "weight_copies": copies},
     }, (t, n, k)
@@ -490,6 +490,8 @@ WORKLOADS = {
     "gemv_q4k_4096x14336": dict(kind="gemv", n=4096, k=14336, metric="Q4_K GEMV GB/s @4096x14336", unit="GB/s",
                                 dtype="bf16"),
 }
+WORKLOADS["gemv_q6k_14336x4096"] = dict(kind="gemv", n=14336, k=4096, type=Q6K, metric="Q6_K GEMV GB/s @14336x4096", unit="GB/s", dtype="bf16")
+WORKLOADS["gemv_q8_0_14336x4096"] = dict(kind="gemv", n=14336, k=4096, type=Q8_0, metric="Q8_0 GEMV GB/s @14336x4096", unit="GB/s", dtype="bf16")
 WORKLOADS["gemv_q4k_q8k_14336x4096"] = dict(kind="gemv_q8k", n=14336, k=4096, type=Q4K, unit="GB/s", dtype="i8",
                                             metric="Q4_K x Q8_K integer-dot GEMV GB/s @14336x4096 (activation quantize included)")
 WORKLOADS["gemv_q6k_q8k_14336x4096"] = dict(kind="gemv_q8k", n=14336, k=4096, type=Q6K, unit="GB/s", dtype="i8",
@@ -538,7 +540,7 @@ def main():
     elif wl["kind"] == "calibrate":
         res, (t, n, k) = bench_calibrate(args, wl["n"], wl["k"])
     else:
-        res, (t, n, k) = bench_gemv(args, wl["n"], wl["k"])
+        res, (t, n, k) = bench_gemv(args, wl["n"], wl["k"], wl.get("type", Q4K))
     out = {
         "metric": wl["metric"], "value": round(res["value"], 1), "unit": wl["unit"], "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(res["ms_per_step"], 5),
@@ -549,7 +551,7 @@ def main():
                  else "synthetic: N(0,0.02) f32 weights generated and quantized on the device, x ~ N(0,1) bf16"),
         "config": {"workload": args.workload, "element_order": "GGML" if wl["kind"] == "calibrate" else "REF",
                    "step": {"gemm": "one GEMM launch (activation pre-pass + MFMA kernel)",
-                            "gemv": "16 back-to-back GEMVs over 16 distinct weight tensors (528 MB, HBM-resident)",
+                            "gemv": "16 back-to-back GEMVs over 16 distinct weight tensors (HBM-resident: 528 MB for Q4_K)",
                             "gemv_q8k": "16 x (activations f32 -> Q8_K, integer-dot GEMV) over 16 distinct weight tensors",
                             "calibrate": "one tensor resident in HBM: 6 candidates x (quantize, dequantize, f64 score read back)",
                             "decode": "all 197 batch-1 projections of one token, back to back on one stream",

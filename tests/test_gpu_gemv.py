@@ -70,6 +70,52 @@ def test_qgemv_q4k_large_ragged_shapes(oracle, n, k, x_dtype):
         assert elem <= TOL and norm <= TOL
 
 
+# Large Q6_K matrices from random block bytes: ragged row counts, rows of 8 to 64 super-blocks, fewer rows than
+# compute units times waves; activations with large and tiny outliers and a run of zeros.
+Q6K_BIG_CASES = [(6001, 4096), (14336, 4096), (4096, 14336), (30001, 2048), (500, 16384), (1900, 6144)]
+
+
+@pytest.mark.parametrize("n,k", Q6K_BIG_CASES)
+@pytest.mark.parametrize("x_dtype", [pm.DTYPE_BF16, pm.DTYPE_F32])
+def test_qgemv_q6k_large_shapes(oracle, n, k, x_dtype):
+    rng = np.random.default_rng(n + k)
+    raw = rng.integers(0, 256, size=(n * (k // 256), 210), dtype=np.uint8)
+    raw[:, 208:210] = np.frombuffer(np.array([0.001], np.float16).tobytes(), np.uint8)
+    raw = raw.reshape(-1)
+    x = rng.standard_normal(k).astype(np.float32)
+    x[rng.integers(0, k, k // 300)] *= 1000.0
+    x[rng.integers(0, k, k // 300)] *= 1e-6
+    x[5:21] = 0.0
+    if x_dtype == pm.DTYPE_BF16:
+        x_dev = oracle.f32_to_bf16_bits(x)
+        x_ref = oracle.bf16_bits_to_f32(x_dev)
+    else:
+        x_dev = x_ref = x
+    want = oracle.qmatvec(Q6K, raw, n, k, x_ref)
+    got = gpu_qgemv(Q6K, raw, n, k, x_dev, x_dtype, 0)
+    elem, norm = rel_errors(got, want)
+    print(f"Q6_K {n}x{k} x_dtype {x_dtype}: elem {elem:.2e} norm {norm:.2e}")
+    assert elem <= TOL and norm <= TOL
+
+
+def test_qgemv_q6k_large_quantized_weights_and_linearity(oracle):
+    n, k = 7000, 4096
+    wq = pm.quantize(weights(21, n * k, outliers=1e-3), Q6K)
+    rng = np.random.default_rng(22)
+    xa, xb = rng.standard_normal(k).astype(np.float32), rng.standard_normal(k).astype(np.float32)
+    want = oracle.qmatvec(Q6K, wq, n, k, xa)
+    ya = gpu_qgemv(Q6K, wq, n, k, xa, pm.DTYPE_F32, 0)
+    elem, norm = rel_errors(ya, want)
+    assert elem <= TOL and norm <= TOL
+    yb = gpu_qgemv(Q6K, wq, n, k, xb, pm.DTYPE_F32, 0)
+    yab = gpu_qgemv(Q6K, wq, n, k, (xa + xb).astype(np.float32), pm.DTYPE_F32, 0)
+    assert np.abs(yab - (ya + yb)).max() <= 1e-4 * np.abs(yab).max()
+    assert not gpu_qgemv(Q6K, wq, n, k, np.zeros(k, np.float32), pm.DTYPE_F32, 0).any()
+    # an infinity among the activations reaches every output
+    xa[100] = np.inf
+    assert np.isnan(gpu_qgemv(Q6K, wq, n, k, xa, pm.DTYPE_F32, 0)).all()
+
+
 def test_qgemv_config0_q8_0_round_trip_and_gemv(oracle):
     # BASELINE config 0: 3072x1024 N(0, 0.02), Q8_0 round trip, then y = W x with f32 x ~ N(0, 1)
     n, k = 3072, 1024
