@@ -10,7 +10,7 @@ from gpu_util import Q4K, Q6K, first_mismatch, rel_errors
 from pmetal_amd import _lib
 
 pytestmark = pytest.mark.gpu
-BLOCK = {Q4K: 144, Q6K: 210}
+BLOCK = {Q4K: 144, Q6K: 210, 13: 176, 11: 110, 10: 84, 15: 292}
 TOL = 1e-3
 
 
@@ -32,11 +32,18 @@ LLAMA3_8B = [("blk.4.attn_q", 4096, 4096, Q4K), ("blk.4.attn_k", 1024, 4096, Q4K
              ("blk.0.ffn_down", 4096, 14336, Q6K), ("output", 128256, 4096, Q6K)]
 
 
-@pytest.mark.parametrize("name,rows,cols,t", LLAMA3_8B, ids=[x[0] for x in LLAMA3_8B])
+# the fused attn_qkv tensor of the recipe (Q5_K) and the other candidate types of the KL calibration on the 14336 x 4096
+# tensor it is measured on (dynamic.rs:958-965)
+OTHER_TYPES = [("blk.4.attn_qkv", 6144, 4096, 13), ("calibrate.q8k", 14336, 4096, 15), ("calibrate.q5k", 14336, 4096, 13),
+               ("calibrate.q3k", 14336, 4096, 11), ("calibrate.q2k", 14336, 4096, 10)]
+
+
+@pytest.mark.parametrize("name,rows,cols,t", LLAMA3_8B + OTHER_TYPES, ids=[x[0] for x in LLAMA3_8B + OTHER_TYPES])
 def test_quantize_full_size_tensor_sampled(oracle, name, rows, cols, t):
     lib = _lib.load()
     n = rows * cols
-    assert int(pm.q4km_tensor_type(name + ".weight", 2, 32)) == t
+    if not name.startswith("calibrate"):
+        assert int(pm.q4km_tensor_type(name + ".weight", 2, 32)) == t
     x = pm.DeviceBuffer(4 * n)
     # N(0, 0.02^2) with 0.1 % of +-0.5 outliers, generated on the device
     pm.check(lib.pmetal_hip_fill_normal_f32(x.ptr, n, 1234 + rows, 0.02, 1e-3, 0.5, None))
