@@ -266,13 +266,12 @@ def cpu_baseline_gemv_q8k(t, n, k, budget_s=12.0):
 
 def bench_calibrate(args, n, k):
     """One step = the round trips of calibrate_tensor for one resident 14336 x 4096 f32 tensor: for each candidate type
-    of the reference's default list (Q8_K, Q6_K, Q5_K, Q4_K, Q3_K, Q2_K) quantize, dequantize, score."""
+    of the reference's default list (Q8_K, Q6_K, Q5_K, Q4_K, Q3_K, Q2_K) quantize, then dequantize and score in one pass."""
     pm, _lib, lib = load()
     timer = Timer(pm, lib)
     ne = n * k
     x = pm.DeviceBuffer(4 * ne)
     pm.check(lib.pmetal_hip_fill_normal_f32(x.ptr, ne, 11, 0.02, 1e-3, 0.5, None))
-    deq = pm.DeviceBuffer(4 * ne)
     cands = [15, 14, 13, 12, 11, 10]
     qs = {t: pm.DeviceBuffer(lib.pmetal_hip_tensor_size(t, ne)) for t in cands}
     scores = {}
@@ -282,21 +281,20 @@ def bench_calibrate(args, n, k):
         for t in cands:
             nb = lib.pmetal_hip_tensor_size(t, ne)
             pm.check(lib.pmetal_hip_quantize_dev(t, x.ptr, ne, qs[t].ptr, nb, None))
-            pm.check(lib.pmetal_hip_dequantize_dev(t, qs[t].ptr, nb, deq.ptr, ne, 1, None))
             sc = C.c_double()
-            pm.check(lib.pmetal_hip_kl_divergence_dev(x.ptr, deq.ptr, ne, C.byref(sc), None))
+            pm.check(lib.pmetal_hip_kl_divergence_quantized_dev(t, qs[t].ptr, nb, x.ptr, ne, 1, C.byref(sc), None))
             scores[t] = sc.value
 
     steps, warm = max(1, args.steps // 20), max(1, args.warmup // 10)
     ev_ms, wall_ms = timer.run(step, steps, warm)
-    # per candidate: quantize reads 4n and writes the blocks, dequantize reads them and writes 4n, the metric reads 8n
-    bytes_per_step = sum(4 * ne + 2 * lib.pmetal_hip_tensor_size(t, ne) + 4 * ne + 8 * ne for t in cands)
+    # per candidate: quantize reads 4n and writes the blocks, the fused comparison reads the blocks and 4n
+    bytes_per_step = sum(4 * ne + 2 * lib.pmetal_hip_tensor_size(t, ne) + 4 * ne for t in cands)
     gbs = 4.0 * ne * len(cands) / (wall_ms / steps * 1e-3) / 1e9
     res = {
         "value": gbs, "ms_per_step": wall_ms / steps, "event_ms_per_step": ev_ms / steps,
         "roofline": {"bound": "hbm", "achieved": round(bytes_per_step / (wall_ms / steps * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(bytes_per_step / (wall_ms / steps * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "k_quantize_* / k_dequantize_* / k_kl_sums", "bytes_per_step": bytes_per_step},
+                     "kernel": "k_quantize_* / k_kl_sums_kq", "bytes_per_step": bytes_per_step},
         "extra": {"scores": {str(t): scores[t] for t in cands}, "steps_run": steps},
     }
     args.steps, args.warmup = steps, warm
@@ -553,7 +551,7 @@ def main():
                    "step": {"gemm": "one GEMM launch (activation pre-pass + MFMA kernel)",
                             "gemv": "16 back-to-back GEMVs over 16 distinct weight tensors (HBM-resident: 528 MB for Q4_K)",
                             "gemv_q8k": "16 x (activations f32 -> Q8_K, integer-dot GEMV) over 16 distinct weight tensors",
-                            "calibrate": "one tensor resident in HBM: 6 candidates x (quantize, dequantize, f64 score read back)",
+                            "calibrate": "one tensor resident in HBM: 6 candidates x (quantize, fused dequantize-and-score, f64 score read back)",
                             "decode": "all 197 batch-1 projections of one token, back to back on one stream",
                             "dequantize": "two tensors of 14336 x 4096, blocks resident in HBM",
                             "quantize": "all 226 tensors of the model, f32 resident in HBM"}[wl["kind"]]},

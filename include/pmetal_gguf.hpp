@@ -19,6 +19,7 @@
 
 #include <cstdint>
 #include <stdexcept>
+#include <memory>
 #include <string>
 #include <vector>
 
@@ -192,7 +193,7 @@ struct CalibratedTensor {
 };
 
 // DynamicQuantizer::calibrate_tensor (crates/pmetal-gguf/src/dynamic.rs:420-502) with the round trips on the GPU: the
-// tensor is uploaded once; every candidate is quantized, dequantized and scored on the device.  A candidate without
+// tensor is uploaded once; every candidate is quantized and scored on the device (the k-quants without storing the dequantized tensor).  A candidate without
 // kernels here, or a shape whose byte size is not the quantized tensor's, is skipped, as the reference
 // skips a candidate whose quantize or dequantize fails.
 inline CalibratedTensor calibrate_tensor(const std::string &name, const float *data, size_t n, const std::vector<int32_t> &shape,
@@ -203,7 +204,8 @@ inline CalibratedTensor calibrate_tensor(const std::string &name, const float *d
     for (int32_t d : shape) n_shape *= (size_t)(d > 0 ? d : 0);
     const size_t sample = cfg.sample_size > 0 && n > cfg.sample_size ? cfg.sample_size : n;
     std::vector<std::pair<GgmlType, double>> scores;
-    DeviceBuffer dx((n ? n : 4) * sizeof(float)), ddeq((n ? n : 4) * sizeof(float));
+    DeviceBuffer dx((n ? n : 4) * sizeof(float));
+    std::unique_ptr<DeviceBuffer> ddeq;  // only for a type that has no fused comparison
     if (n) detail::check(pmetal_hip_h2d(dx.ptr(), data, n * sizeof(float)));
     for (GgmlType t : cfg.candidates) {
         const size_t nbytes = pmetal_hip_tensor_size((uint32_t)t, n);
@@ -214,10 +216,16 @@ inline CalibratedTensor calibrate_tensor(const std::string &name, const float *d
         }
         DeviceBuffer dq(nbytes ? nbytes : 16);
         detail::check(pmetal_hip_quantize_dev((uint32_t)t, (const float *)dx.ptr(), n, (uint8_t *)dq.ptr(), nbytes, nullptr), true);
-        detail::check(pmetal_hip_dequantize_dev((uint32_t)t, (const uint8_t *)dq.ptr(), nbytes, (float *)ddeq.ptr(), n_shape, cfg.order, nullptr));
+        const size_t cmp_len = sample < n_shape ? sample : n_shape;
         double score = 0.0;
-        detail::check(pmetal_hip_kl_divergence_dev((const float *)dx.ptr(), (const float *)ddeq.ptr(), sample < n_shape ? sample : n_shape,
-                                                   &score, nullptr));
+        if (pmetal_hip_block_size((uint32_t)t) == 256) {  // k-quants: decoded and compared in one pass, nothing stored
+            detail::check(pmetal_hip_kl_divergence_quantized_dev((uint32_t)t, (const uint8_t *)dq.ptr(), nbytes, (const float *)dx.ptr(), cmp_len,
+                                                                 cfg.order, &score, nullptr));
+        } else {
+            if (!ddeq) ddeq.reset(new DeviceBuffer(n * sizeof(float)));
+            detail::check(pmetal_hip_dequantize_dev((uint32_t)t, (const uint8_t *)dq.ptr(), nbytes, (float *)ddeq->ptr(), n_shape, cfg.order, nullptr));
+            detail::check(pmetal_hip_kl_divergence_dev((const float *)dx.ptr(), (const float *)ddeq->ptr(), cmp_len, &score, nullptr));
+        }
         scores.emplace_back(t, score);
     }
     if (scores.empty()) return {cfg.fallback_type, kMax, {{cfg.fallback_type, kMax}}};

@@ -203,6 +203,13 @@ int32_t pmetal_hip_qgemv_q8k(uint32_t ggml_type, const uint8_t *w_dev, int64_t n
  * pmetal_hip_quantize_dev / _dequantize_dev / this (pmetal_gguf::calibrate_tensor, pmetal_amd.gguf.calibrate_tensor). */
 int32_t pmetal_hip_kl_divergence_dev(const float *original_dev, const float *dequantized_dev, size_t n, double *score,
                                      void *stream);
+/* The dequantize and score steps of that loop (dynamic.rs:462-467) in one pass for the k-quant types (Q2_K .. Q6_K,
+ * Q8_K): the first n elements of the blocks are decoded in registers, in the given element order, and compared with
+ * original_dev[0..n) without being stored.  Equal to _dequantize_dev followed by _kl_divergence_dev up to the order of
+ * the f64 sums.  Any other type: PMETAL_HIP_ERR_UNSUPPORTED_TYPE; n beyond what the blocks hold: ..._INVALID_SIZE. */
+int32_t pmetal_hip_kl_divergence_quantized_dev(uint32_t ggml_type, const uint8_t *quantized_dev, size_t quantized_len,
+                                               const float *original_dev, size_t n, uint32_t order, double *score,
+                                               void *stream);
 
 /* ---- Q4_K_M recipe (crates/pmetal/src/commands/quantize.rs) --------------------------- */
 int32_t pmetal_hip_use_more_bits(size_t layer, size_t n_layers);                   /* :988-993  */

@@ -57,6 +57,7 @@ SYMBOLS = [
     ("pmetal_hip_quantize_q8k_dev", _i32, [_vp, _sz, _vp, _sz, _vp]),
     ("pmetal_hip_qgemv_q8k", _i32, [_u32, _vp, _i64, _i64, _vp, _vp, _vp]),
     ("pmetal_hip_kl_divergence_dev", _i32, [_vp, _vp, _sz, C.POINTER(C.c_double), _vp]),
+    ("pmetal_hip_kl_divergence_quantized_dev", _i32, [_u32, _vp, _sz, _vp, _sz, _u32, C.POINTER(C.c_double), _vp]),
     ("pmetal_hip_use_more_bits", _i32, [_sz, _sz]),
     ("pmetal_hip_is_quantizable_gguf_tensor", _i32, [C.c_char_p, _sz]),
     ("pmetal_hip_q4km_tensor_type", _u32, [C.c_char_p, _sz, _sz]),

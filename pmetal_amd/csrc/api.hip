@@ -657,6 +657,22 @@ int32_t pmetal_hip_qgemv_q8k(uint32_t t, const uint8_t *w, int64_t n, int64_t k,
 }
 
 // ---- KL calibration metric ----
+namespace {
+// compute_kl_divergence (dynamic.rs:155-178) from the per-workgroup partial sums, added in workgroup order
+int32_t kl_score_from_partials(const DevBuf &part, int groups, size_t n, double *score, hipStream_t stream) {
+    std::vector<double> host((size_t)groups * 4);
+    HIP_TRY(hipMemcpyAsync(host.data(), part.p, host.size() * sizeof(double), hipMemcpyDeviceToHost, stream));
+    HIP_TRY(hipStreamSynchronize(stream));
+    double sq_err = 0.0, aa = 0.0, ab = 0.0, bb = 0.0;
+    for (int g = 0; g < groups; g++) sq_err += host[4 * g], aa += host[4 * g + 1], ab += host[4 * g + 2], bb += host[4 * g + 3];
+    const double dn = (double)n;
+    const double nrmse = aa > 0.0 ? std::sqrt(sq_err / dn) / std::sqrt(aa / dn) : 0.0;
+    const double cos_sim = (aa > 0.0 && bb > 0.0) ? ab / (std::sqrt(aa) * std::sqrt(bb)) : 1.0;
+    *score = nrmse + (1.0 - cos_sim);
+    return ok();
+}
+}  // namespace
+
 int32_t pmetal_hip_kl_divergence_dev(const float *original, const float *dequantized, size_t n, double *score, void *stream) {
     if (!score) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
     if (n == 0) {  // dynamic.rs:143-145
@@ -671,17 +687,30 @@ int32_t pmetal_hip_kl_divergence_dev(const float *original, const float *dequant
     HIP_TRY(hipMalloc(&part.p, (size_t)groups * 4 * sizeof(double)));
     hipError_t e = pmh::launch_kl_sums(original, dequantized, n, (double *)part.p, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "kl sums kernel launch");
-    std::vector<double> host((size_t)groups * 4);
-    HIP_TRY(hipMemcpyAsync(host.data(), part.p, host.size() * sizeof(double), hipMemcpyDeviceToHost, (hipStream_t)stream));
-    HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
-    double sq_err = 0.0, aa = 0.0, ab = 0.0, bb = 0.0;
-    for (int g = 0; g < groups; g++) sq_err += host[4 * g], aa += host[4 * g + 1], ab += host[4 * g + 2], bb += host[4 * g + 3];
-    // dynamic.rs:155-178
-    const double dn = (double)n;
-    const double nrmse = aa > 0.0 ? std::sqrt(sq_err / dn) / std::sqrt(aa / dn) : 0.0;
-    const double cos_sim = (aa > 0.0 && bb > 0.0) ? ab / (std::sqrt(aa) * std::sqrt(bb)) : 1.0;
-    *score = nrmse + (1.0 - cos_sim);
-    return ok();
+    return kl_score_from_partials(part, groups, n, score, (hipStream_t)stream);
+}
+
+int32_t pmetal_hip_kl_divergence_quantized_dev(uint32_t t, const uint8_t *quantized, size_t quantized_len, const float *original, size_t n,
+                                               uint32_t order, double *score, void *stream) {
+    if (!codec_type(t) || pmetal_hip_block_size(t) != 256)
+        return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "the fused comparison takes the k-quant types only, not GGML type %u", t);
+    if (order > PMETAL_HIP_ORDER_GGML) return fail(PMETAL_HIP_ERR_INVALID_ARG, "invalid element order %u", order);
+    if (!score) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
+    if (quantized_len % pmetal_hip_type_size(t) || n > quantized_len / pmetal_hip_type_size(t) * 256)
+        return fail(PMETAL_HIP_ERR_INVALID_SIZE, "%zu bytes of GGML type %u do not hold %zu elements", quantized_len, t, n);
+    if (n == 0) {  // dynamic.rs:143-145
+        *score = 0.0;
+        return ok();
+    }
+    if (!original || !quantized) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
+    if (!aligned16(original) || !aligned16(quantized)) return fail(PMETAL_HIP_ERR_INVALID_ARG, "device pointers must be 16-byte aligned");
+    if (int32_t rc = require_device()) return rc;
+    const int groups = pmh::kl_sums_quantized_workgroups(n);
+    DevBuf part;
+    HIP_TRY(hipMalloc(&part.p, (size_t)groups * 4 * sizeof(double)));
+    hipError_t e = pmh::launch_kl_sums_quantized(t, quantized, original, n, order, (double *)part.p, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "fused kl sums kernel launch");
+    return kl_score_from_partials(part, groups, n, score, (hipStream_t)stream);
 }
 
 // ---- measurement aid ----

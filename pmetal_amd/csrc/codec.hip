@@ -158,111 +158,204 @@ __device__ __forceinline__ void scale_min_k4(int j, uint32_t s0, uint32_t s1, ui
 }
 
 // -------------------------------------------------------------------------------------------
-// Q4_K dequantize (k_quants.rs:358-404 + :515-560).  One lane per 4 outputs of a super-block; a wave
-// handles kDeqUnroll consecutive super-blocks and requests the bytes of all of them before it computes, so
-// that a wave has several kilobytes of output per memory round trip.  out = (d*sc) * nibble - (dmin*m),
-// each operation rounded.
-// ORDER 0: the reference's emission order; ORDER 1: inverse of the quantizer's packing.
+// Dequantizers of the k-quant formats.  A decoder describes one format: lane i (0..63) of a wave loads its share
+// of a super-block (`load`) and turns it into elements 4 i .. 4 i + 3 (`values`), with every operation rounded as
+// the reference rounds it.  k_dequantize_kq stores the values; k_kl_sums_kq compares them with the original
+// tensor without storing them.  A wave handles kDeqUnroll super-blocks per step and requests the bytes of all of
+// them before it computes, so that it has several kilobytes of output per memory round trip.
+// ORDER 0: the reference dequantizer's emission order; ORDER 1: the inverse of the quantizer's packing (they differ
+// for Q4_K and Q5_K only).
 // -------------------------------------------------------------------------------------------
 constexpr int kDeqUnroll = 4;
 
+// Q4_K (k_quants.rs:358-404 + :515-560): out = (d*sc) * nibble - (dmin*m).
 template <int ORDER>
-__global__ __launch_bounds__(256) void k_dequantize_q4k(const uint8_t *__restrict__ src, size_t n,
-                                                         float *__restrict__ dst) {
-    const size_t wave = ((size_t)blockIdx.x * 256 + threadIdx.x) >> 6;
-    const int i = (int)(threadIdx.x & 63);
-    const int c = i >> 4;       // 64-element chunk
-    const int p = (i & 15) * 4; // position inside the chunk
-    int byte, hi, sb;
-    if (ORDER == 0) {
-        byte = 32 * c + (p & 15) + 16 * (p >> 5);
-        hi = (p >> 4) & 1;
-        sb = 2 * c + (p >> 5);
-    } else {
-        byte = 32 * c + (p & 31);
-        hi = p >> 5;
+struct DecQ4K {
+    static constexpr int kBytes = 144;
+    struct Raw {
+        uint4 hdr;
+        uint32_t q;
+    };
+    static __device__ __forceinline__ void where(int i, int &byte, int &hi, int &sb) {
+        const int c = i >> 4;        // 64-element chunk
+        const int p = (i & 15) * 4;  // position inside the chunk
+        if (ORDER == 0) {
+            byte = 32 * c + (p & 15) + 16 * (p >> 5);
+            hi = (p >> 4) & 1;
+        } else {
+            byte = 32 * c + (p & 31);
+            hi = p >> 5;
+        }
         sb = 2 * c + (p >> 5);
     }
-    uint4 hdr[kDeqUnroll];
-    uint32_t q[kDeqUnroll];
-#pragma unroll
-    for (int u = 0; u < kDeqUnroll; u++) {
-        const size_t blk_i = wave * kDeqUnroll + u;
-        const bool live = blk_i * 256 + (size_t)i * 4 < n;
-        const uint8_t *blk = src + (live ? blk_i : 0) * 144;  // lanes past the end re-read the first block
-        hdr[u] = *reinterpret_cast<const uint4 *>(blk);
-        q[u] = *reinterpret_cast<const uint32_t *>(blk + 16 + byte);
+    static __device__ __forceinline__ Raw load(const uint8_t *blk, int i) {
+        int byte, hi, sb;
+        where(i, byte, hi, sb);
+        return {*reinterpret_cast<const uint4 *>(blk), *reinterpret_cast<const uint32_t *>(blk + 16 + byte)};
     }
-#pragma unroll
-    for (int u = 0; u < kDeqUnroll; u++) {
-        const size_t e = (wave * kDeqUnroll + u) * 256 + (size_t)i * 4;
-        if (e >= n) continue;
-        const float d = f16_bits_to_f32(hdr[u].x & 0xFFFFu), dmin = f16_bits_to_f32(hdr[u].x >> 16);
+    static __device__ __forceinline__ void values(const Raw &r, int i, float (&o)[4]) {
+        int byte, hi, sb;
+        where(i, byte, hi, sb);
+        const float d = f16_bits_to_f32(r.hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(r.hdr.x >> 16);
         uint32_t sc, m;
-        scale_min_k4(sb, hdr[u].y, hdr[u].z, hdr[u].w, sc, m);
+        scale_min_k4(sb, r.hdr.y, r.hdr.z, r.hdr.w, sc, m);
         const float d1 = d * (float)sc;
         const float dm1 = dmin * (float)m;
-        const uint32_t qq = hi ? (q[u] >> 4) : q[u];
-        float o[4];
+        const uint32_t qq = hi ? (r.q >> 4) : r.q;
 #pragma unroll
         for (int t = 0; t < 4; t++) o[t] = d1 * (float)((qq >> (8 * t)) & 0xFu) - dm1;
-        if (e + 3 < n) {
-            *reinterpret_cast<float4 *>(dst + e) = make_float4(o[0], o[1], o[2], o[3]);
-        } else {
-            for (int t = 0; t < 4 && e + t < n; t++) dst[e + t] = o[t];
-        }
     }
-}
+};
 
-// -------------------------------------------------------------------------------------------
-// Q5_K dequantize (k_quants.rs:407-462 + :663-710): 176-byte blocks {d, dmin, scales[12], qh[32], qs[128]};
-// out = (d*sc) * q - (dmin*m) with q = nibble | fifth bit << 4.  Same launch shape as Q4_K.
-// ORDER 0: the reference's emission order: output l of the first / second half of chunk c takes nibble l % 2 of
-// qs[32 c + 16 half + l / 2] and bit l % 8 of qh[8 c + 4 half + l / 8].  ORDER 1: the inverse of the quantizer's packing
-// (k_quants.rs:1027-1047): nibble `half` of qs[32 c + l] and bit 2 c + half of qh[l].
-// -------------------------------------------------------------------------------------------
+// Q5_K (k_quants.rs:407-462 + :663-710): 176-byte blocks {d, dmin, scales[12], qh[32], qs[128]};
+// out = (d*sc) * q - (dmin*m) with q = nibble | fifth bit << 4.
+// ORDER 0: output l of the first / second half of chunk c takes nibble l % 2 of qs[32 c + 16 half + l / 2] and bit
+// l % 8 of qh[8 c + 4 half + l / 8].  ORDER 1 (the inverse of k_quants.rs:1027-1047): nibble `half` of qs[32 c + l] and
+// bit 2 c + half of qh[l].
 template <int ORDER>
-__global__ __launch_bounds__(256) void k_dequantize_q5k(const uint8_t *__restrict__ src, size_t n,
-                                                         float *__restrict__ dst) {
-    const size_t wave = ((size_t)blockIdx.x * 256 + threadIdx.x) >> 6;
-    const int i = (int)(threadIdx.x & 63);
-    const int c = i >> 4;        // 64-element chunk
-    const int p = (i & 15) * 4;  // position inside the chunk
-    const int half = p >> 5, l = p & 31;
-    const int sb = 2 * c + half;
-    uint4 hdr[kDeqUnroll];
-    uint32_t q[kDeqUnroll], h[kDeqUnroll];
-#pragma unroll
-    for (int u = 0; u < kDeqUnroll; u++) {
-        const size_t blk_i = wave * kDeqUnroll + u;
-        const bool live = blk_i * 256 + (size_t)i * 4 < n;
-        const uint8_t *blk = src + (live ? blk_i : 0) * 176;  // lanes past the end re-read the first block
-        hdr[u] = *reinterpret_cast<const uint4 *>(blk);
+struct DecQ5K {
+    static constexpr int kBytes = 176;
+    struct Raw {
+        uint4 hdr;
+        uint32_t q, h;
+    };
+    static __device__ __forceinline__ Raw load(const uint8_t *blk, int i) {
+        const int c = i >> 4, p = (i & 15) * 4, half = p >> 5, l = p & 31;
+        Raw r;
+        r.hdr = *reinterpret_cast<const uint4 *>(blk);
         if (ORDER == 0) {
-            q[u] = *reinterpret_cast<const uint16_t *>(blk + 48 + 32 * c + 16 * half + (l >> 1));
-            h[u] = (uint32_t)blk[16 + 8 * c + 4 * half + (l >> 3)] >> (l & 7);
+            r.q = *reinterpret_cast<const uint16_t *>(blk + 48 + 32 * c + 16 * half + (l >> 1));
+            r.h = (uint32_t)blk[16 + 8 * c + 4 * half + (l >> 3)] >> (l & 7);
         } else {
-            q[u] = *reinterpret_cast<const uint32_t *>(blk + 48 + 32 * c + l);
-            h[u] = *reinterpret_cast<const uint32_t *>(blk + 16 + l) >> (2 * c + half);
+            r.q = *reinterpret_cast<const uint32_t *>(blk + 48 + 32 * c + l);
+            r.h = *reinterpret_cast<const uint32_t *>(blk + 16 + l) >> (2 * c + half);
         }
+        return r;
     }
-#pragma unroll
-    for (int u = 0; u < kDeqUnroll; u++) {
-        const size_t e = (wave * kDeqUnroll + u) * 256 + (size_t)i * 4;
-        if (e >= n) continue;
-        const float d = f16_bits_to_f32(hdr[u].x & 0xFFFFu), dmin = f16_bits_to_f32(hdr[u].x >> 16);
+    static __device__ __forceinline__ void values(const Raw &r, int i, float (&o)[4]) {
+        const int c = i >> 4, p = (i & 15) * 4, half = p >> 5;
+        const float d = f16_bits_to_f32(r.hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(r.hdr.x >> 16);
         uint32_t sc, m;
-        scale_min_k4(sb, hdr[u].y, hdr[u].z, hdr[u].w, sc, m);
+        scale_min_k4(2 * c + half, r.hdr.y, r.hdr.z, r.hdr.w, sc, m);
         const float d1 = d * (float)sc;
         const float dm1 = dmin * (float)m;
-        float o[4];
 #pragma unroll
         for (int t = 0; t < 4; t++) {
             uint32_t v;
-            if (ORDER == 0) v = ((q[u] >> (4 * t)) & 0xFu) | (((h[u] >> t) & 1u) << 4);
-            else v = (((half ? q[u] >> 4 : q[u]) >> (8 * t)) & 0xFu) | (((h[u] >> (8 * t)) & 1u) << 4);
+            if (ORDER == 0) v = ((r.q >> (4 * t)) & 0xFu) | (((r.h >> t) & 1u) << 4);
+            else v = (((half ? r.q >> 4 : r.q) >> (8 * t)) & 0xFu) | (((r.h >> (8 * t)) & 1u) << 4);
             o[t] = d1 * (float)v - dm1;
         }
+    }
+};
+
+// Q6_K (k_quants.rs:474-496 + :614-660): out = (d * sc) * q, left-associated.  Blocks are 2-byte aligned.
+struct DecQ6K {
+    static constexpr int kBytes = 210;
+    struct Raw {
+        uint32_t ql, qh, d;
+        int sc;
+    };
+    static __device__ __forceinline__ Raw load(const uint8_t *blk, int i) {
+        const int h = i >> 5;        // 128-element half
+        const int g = (i >> 3) & 3;  // 32-element group inside the half
+        const int l = (i & 7) * 4;   // 0..28
+        return {*reinterpret_cast<const u32_a2 *>(blk + 64 * h + 32 * (g & 1) + l), *reinterpret_cast<const u32_a2 *>(blk + 128 + 32 * h + l),
+                *reinterpret_cast<const uint16_t *>(blk + 208), (int)(int8_t)blk[192 + 8 * h + 2 * g + (l >> 4)]};
+    }
+    static __device__ __forceinline__ void values(const Raw &r, int i, float (&o)[4]) {
+        const int g = (i >> 3) & 3;
+        const float dsc = f16_bits_to_f32(r.d) * (float)r.sc;
+        const uint32_t nib = (g >= 2) ? (r.ql >> 4) : r.ql;
+        const uint32_t hi2 = r.qh >> (2 * g);
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const int q = (int)(((nib >> (8 * t)) & 0xFu) | (((hi2 >> (8 * t)) & 3u) << 4)) - 32;
+            o[t] = dsc * (float)q;
+        }
+    }
+};
+
+// Q2_K and Q3_K have sixteen 16-element sub-blocks per super-block and pack the low two bits of element e into
+// qs[32 (e / 128) + e % 32] at bit 2 ((e % 128) / 32).
+// Q2_K (k_quants.rs:230-266 + :762-810): out = (d * (sc & 15)) * q - dmin * (sc >> 4).  84-byte blocks: scales[16],
+// qs[64], d, dmin.
+struct DecQ2K {
+    static constexpr int kBytes = 84;
+    struct Raw {
+        uint32_t q, sc, dd;
+    };
+    static __device__ __forceinline__ Raw load(const uint8_t *blk, int i) {
+        const int h = i >> 5, l = (i & 7) * 4;
+        return {*reinterpret_cast<const uint32_t *>(blk + 16 + 32 * h + l), blk[i >> 2], *reinterpret_cast<const uint32_t *>(blk + 80)};
+    }
+    static __device__ __forceinline__ void values(const Raw &r, int i, float (&o)[4]) {
+        const int p = (i >> 3) & 3;
+        const float dl = f16_bits_to_f32(r.dd & 0xFFFFu) * (float)(r.sc & 0xFu);
+        const float ml = f16_bits_to_f32(r.dd >> 16) * (float)(r.sc >> 4);
+#pragma unroll
+        for (int t = 0; t < 4; t++) o[t] = dl * (float)((r.q >> (8 * t + 2 * p)) & 3u) - ml;
+    }
+};
+
+// Q3_K (k_quants.rs:281-355 + :713-760): out = (d * (sc6 - 32)) * (q2 - (hbit ? 0 : 4)).  110-byte blocks: hmask[32],
+// qs[64], scales[12], d; the high bit of element e is bit e / 32 of hmask[e % 32]; the sixteen 6-bit scales are four low
+// bits in the nibbles of scales[0..8] and two high bits in scales[8..12].
+struct DecQ3K {
+    static constexpr int kBytes = 110;
+    struct Raw {
+        uint32_t q, h, lo, hi, d;
+    };
+    static __device__ __forceinline__ Raw load(const uint8_t *blk, int i) {
+        const int h = i >> 5, l = (i & 7) * 4, is = i >> 2;
+        return {*reinterpret_cast<const u32_a2 *>(blk + 32 + 32 * h + l), *reinterpret_cast<const u32_a2 *>(blk + l), blk[96 + (is & 7)],
+                blk[104 + (is & 3)], *reinterpret_cast<const uint16_t *>(blk + 108)};
+    }
+    static __device__ __forceinline__ void values(const Raw &r, int i, float (&o)[4]) {
+        const int h = i >> 5, p = (i >> 3) & 3, is = i >> 2;
+        const uint32_t sc6 = ((is < 8 ? r.lo : r.lo >> 4) & 0xFu) | (((r.hi >> (2 * (is >> 2))) & 3u) << 4);
+        const float dl = f16_bits_to_f32(r.d) * (float)((int)sc6 - 32);
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const int q = (int)((r.q >> (8 * t + 2 * p)) & 3u) - (((r.h >> (8 * t + 4 * h + p)) & 1u) ? 0 : 4);
+            o[t] = dl * (float)q;
+        }
+    }
+};
+
+// Q8_K (k_quants.rs:498-506): out = d * q, one rounding.  292-byte blocks: d f32, qs[256] i8, bsums[16] i16.
+struct DecQ8K {
+    static constexpr int kBytes = 292;
+    struct Raw {
+        float d;
+        uint32_t q;
+    };
+    static __device__ __forceinline__ Raw load(const uint8_t *blk, int i) {
+        return {*reinterpret_cast<const float *>(blk), *reinterpret_cast<const uint32_t *>(blk + 4 + 4 * i)};
+    }
+    static __device__ __forceinline__ void values(const Raw &r, int, float (&o)[4]) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) o[t] = r.d * (float)(int8_t)(r.q >> (8 * t));
+    }
+};
+
+template <class D>
+__global__ __launch_bounds__(256) void k_dequantize_kq(const uint8_t *__restrict__ src, size_t n, float *__restrict__ dst) {
+    const size_t wave = ((size_t)blockIdx.x * 256 + threadIdx.x) >> 6;
+    const int i = (int)(threadIdx.x & 63);
+    typename D::Raw raw[kDeqUnroll];
+#pragma unroll
+    for (int u = 0; u < kDeqUnroll; u++) {
+        const size_t blk_i = wave * kDeqUnroll + u;
+        const bool live = blk_i * 256 + (size_t)i * 4 < n;
+        raw[u] = D::load(src + (live ? blk_i : 0) * D::kBytes, i);  // lanes past the end re-read the first block
+    }
+#pragma unroll
+    for (int u = 0; u < kDeqUnroll; u++) {
+        const size_t e = (wave * kDeqUnroll + u) * 256 + (size_t)i * 4;
+        if (e >= n) continue;
+        float o[4];
+        D::values(raw[u], i, o);
         if (e + 3 < n) {
             *reinterpret_cast<float4 *>(dst + e) = make_float4(o[0], o[1], o[2], o[3]);
         } else {
@@ -271,48 +364,58 @@ __global__ __launch_bounds__(256) void k_dequantize_q5k(const uint8_t *__restric
     }
 }
 
-// -------------------------------------------------------------------------------------------
-// Q6_K dequantize (k_quants.rs:474-496 + :614-660): out = (d * sc) * q, left-associated.  Same launch shape.
-// -------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void k_dequantize_q6k(const uint8_t *__restrict__ src, size_t n,
-                                                         float *__restrict__ dst) {
-    const size_t wave = ((size_t)blockIdx.x * 256 + threadIdx.x) >> 6;
+// The four f64 sums of compute_kl_divergence (crates/pmetal-gguf/src/dynamic.rs:140-180) between the first n elements
+// of the original tensor and of the dequantized blocks, which are decoded in registers and never stored: sum (a - b)^2
+// with the difference taken in f32, sum a^2, sum a b, sum b^2.  Waves walk the super-blocks with a grid stride; every
+// workgroup writes its four partial sums, the caller adds the workgroups' sums in order.
+template <class D>
+__global__ __launch_bounds__(256) void k_kl_sums_kq(const uint8_t *__restrict__ src, const float *__restrict__ a, size_t n,
+                                                    double *__restrict__ partial) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
     const int i = (int)(threadIdx.x & 63);
-    const int h = i >> 5;         // 128-element half
-    const int g = (i >> 3) & 3;   // 32-element group inside the half
-    const int l = (i & 7) * 4;    // 0..28
-    uint32_t qlw[kDeqUnroll], qhw[kDeqUnroll];
-    int scb[kDeqUnroll];
-    uint32_t dh[kDeqUnroll];
+    const size_t n_waves = (size_t)gridDim.x * 4, wave0 = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const size_t n_blocks = (n + 255) / 256;
+    double s_err = 0.0, s_aa = 0.0, s_ab = 0.0, s_bb = 0.0;
+    for (size_t b0 = wave0 * kDeqUnroll; b0 < n_blocks; b0 += n_waves * kDeqUnroll) {
+        typename D::Raw raw[kDeqUnroll];
+        f4 av[kDeqUnroll];
 #pragma unroll
-    for (int u = 0; u < kDeqUnroll; u++) {
-        const size_t blk_i = wave * kDeqUnroll + u;
-        const bool live = blk_i * 256 + (size_t)i * 4 < n;
-        const uint8_t *blk = src + (live ? blk_i : 0) * 210;  // lanes past the end re-read the first block
-        qlw[u] = *reinterpret_cast<const u32_a2 *>(blk + 64 * h + 32 * (g & 1) + l);
-        qhw[u] = *reinterpret_cast<const u32_a2 *>(blk + 128 + 32 * h + l);
-        scb[u] = (int)(int8_t)blk[192 + 8 * h + 2 * g + (l >> 4)];
-        dh[u] = *reinterpret_cast<const uint16_t *>(blk + 208);
-    }
-#pragma unroll
-    for (int u = 0; u < kDeqUnroll; u++) {
-        const size_t e = (wave * kDeqUnroll + u) * 256 + (size_t)i * 4;
-        if (e >= n) continue;
-        const float dsc = f16_bits_to_f32(dh[u]) * (float)scb[u];
-        const uint32_t nib = (g >= 2) ? (qlw[u] >> 4) : qlw[u];
-        const uint32_t hi2 = qhw[u] >> (2 * g);
-        float o[4];
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-            int q = (int)(((nib >> (8 * t)) & 0xFu) | (((hi2 >> (8 * t)) & 3u) << 4)) - 32;
-            o[t] = dsc * (float)q;
+        for (int u = 0; u < kDeqUnroll; u++) {
+            const size_t e = (b0 + u) * 256 + (size_t)i * 4;
+            raw[u] = D::load(src + (e < n ? b0 + u : 0) * D::kBytes, i);
+            av[u] = (f4){0.f, 0.f, 0.f, 0.f};
+            if (e + 3 < n) {
+                av[u] = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(a + e));
+            } else {
+                for (int t = 0; t < 4 && e + t < n; t++) av[u][t] = a[e + t];
+            }
         }
-        if (e + 3 < n) {
-            *reinterpret_cast<float4 *>(dst + e) = make_float4(o[0], o[1], o[2], o[3]);
-        } else {
-            for (int t = 0; t < 4 && e + t < n; t++) dst[e + t] = o[t];
+#pragma unroll
+        for (int u = 0; u < kDeqUnroll; u++) {
+            const size_t e = (b0 + u) * 256 + (size_t)i * 4;
+            float o[4];
+            D::values(raw[u], i, o);
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                if (e + t < n) {
+                    const double diff = (double)(av[u][t] - o[t]), x = (double)av[u][t], y = (double)o[t];
+                    s_err += diff * diff, s_aa += x * x, s_ab += x * y, s_bb += y * y;
+                }
+            }
         }
     }
+    __shared__ double red[4][4];
+    double v[4] = {s_err, s_aa, s_ab, s_bb};
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) v[k] += __shfl_xor(v[k], off);
+    }
+    const int wave = threadIdx.x >> 6;
+    if (i == 0)
+        for (int k = 0; k < 4; k++) red[wave][k] = v[k];
+    __syncthreads();
+    if (threadIdx.x < 4) partial[(size_t)blockIdx.x * 4 + threadIdx.x] = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
 }
 
 // -------------------------------------------------------------------------------------------
@@ -722,84 +825,10 @@ inline unsigned grid_for(size_t work_items, size_t per_block) {
 }
 
 // -------------------------------------------------------------------------------------------
-// Q2_K and Q3_K (quantize / dequantize only).  Both have sixteen 16-element sub-blocks per super-block and pack the
-// low two bits of element e into qs[32 (e / 128) + e % 32] at bit 2 ((e % 128) / 32); both dequantizers are the
-// inverses of that packing, so there is one element order.
+// Q2_K and Q3_K quantizers.  Both formats have sixteen 16-element sub-blocks per super-block and pack the low two bits
+// of element e into qs[32 (e / 128) + e % 32] at bit 2 ((e % 128) / 32); both reference dequantizers are the inverses of
+// that packing, so there is one element order.
 // -------------------------------------------------------------------------------------------
-
-// Q2_K dequantize (k_quants.rs:230-266 + :762-810): out = (d * (sc & 15)) * q - dmin * (sc >> 4).  84-byte blocks:
-// scales[16], qs[64], d, dmin.  One wave per super-block, four outputs per lane.
-__global__ __launch_bounds__(256) void k_dequantize_q2k(const uint8_t *__restrict__ src, size_t n,
-                                                         float *__restrict__ dst) {
-    const size_t wave = ((size_t)blockIdx.x * 256 + threadIdx.x) >> 6;
-    const int i = (int)(threadIdx.x & 63);
-    const int h = i >> 5, p = (i >> 3) & 3, l = (i & 7) * 4;
-    uint32_t qw[kDeqUnroll], scb[kDeqUnroll], dd[kDeqUnroll];
-#pragma unroll
-    for (int u = 0; u < kDeqUnroll; u++) {
-        const size_t blk_i = wave * kDeqUnroll + u;
-        const bool live = blk_i * 256 + (size_t)i * 4 < n;
-        const uint8_t *blk = src + (live ? blk_i : 0) * 84;  // lanes past the end re-read the first block
-        qw[u] = *reinterpret_cast<const uint32_t *>(blk + 16 + 32 * h + l);
-        scb[u] = blk[i >> 2];
-        dd[u] = *reinterpret_cast<const uint32_t *>(blk + 80);
-    }
-#pragma unroll
-    for (int u = 0; u < kDeqUnroll; u++) {
-        const size_t e = (wave * kDeqUnroll + u) * 256 + (size_t)i * 4;
-        if (e >= n) continue;
-        const float dl = f16_bits_to_f32(dd[u] & 0xFFFFu) * (float)(scb[u] & 0xFu);
-        const float ml = f16_bits_to_f32(dd[u] >> 16) * (float)(scb[u] >> 4);
-        float o[4];
-#pragma unroll
-        for (int t = 0; t < 4; t++) o[t] = dl * (float)((qw[u] >> (8 * t + 2 * p)) & 3u) - ml;
-        if (e + 3 < n) {
-            *reinterpret_cast<float4 *>(dst + e) = make_float4(o[0], o[1], o[2], o[3]);
-        } else {
-            for (int t = 0; t < 4 && e + t < n; t++) dst[e + t] = o[t];
-        }
-    }
-}
-
-// Q3_K dequantize (k_quants.rs:281-355 + :713-760): out = (d * (sc6 - 32)) * (q2 - (hbit ? 0 : 4)).  110-byte blocks:
-// hmask[32], qs[64], scales[12], d; the high bit of element e is bit e / 32 of hmask[e % 32]; the sixteen 6-bit
-// scales are four low bits in the nibbles of scales[0..8] and two high bits in scales[8..12].
-__global__ __launch_bounds__(256) void k_dequantize_q3k(const uint8_t *__restrict__ src, size_t n,
-                                                         float *__restrict__ dst) {
-    const size_t wave = ((size_t)blockIdx.x * 256 + threadIdx.x) >> 6;
-    const int i = (int)(threadIdx.x & 63);
-    const int h = i >> 5, p = (i >> 3) & 3, l = (i & 7) * 4, is = i >> 2;
-    uint32_t qw[kDeqUnroll], hw[kDeqUnroll], lo[kDeqUnroll], hi[kDeqUnroll], dd[kDeqUnroll];
-#pragma unroll
-    for (int u = 0; u < kDeqUnroll; u++) {
-        const size_t blk_i = wave * kDeqUnroll + u;
-        const bool live = blk_i * 256 + (size_t)i * 4 < n;
-        const uint8_t *blk = src + (live ? blk_i : 0) * 110;
-        hw[u] = *reinterpret_cast<const u32_a2 *>(blk + l);
-        qw[u] = *reinterpret_cast<const u32_a2 *>(blk + 32 + 32 * h + l);
-        lo[u] = blk[96 + (is & 7)];
-        hi[u] = blk[104 + (is & 3)];
-        dd[u] = *reinterpret_cast<const uint16_t *>(blk + 108);
-    }
-#pragma unroll
-    for (int u = 0; u < kDeqUnroll; u++) {
-        const size_t e = (wave * kDeqUnroll + u) * 256 + (size_t)i * 4;
-        if (e >= n) continue;
-        const uint32_t sc6 = ((is < 8 ? lo[u] : lo[u] >> 4) & 0xFu) | (((hi[u] >> (2 * (is >> 2))) & 3u) << 4);
-        const float dl = f16_bits_to_f32(dd[u]) * (float)((int)sc6 - 32);
-        float o[4];
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-            const int q = (int)((qw[u] >> (8 * t + 2 * p)) & 3u) - (((hw[u] >> (8 * t + 4 * h + p)) & 1u) ? 0 : 4);
-            o[t] = dl * (float)q;
-        }
-        if (e + 3 < n) {
-            *reinterpret_cast<float4 *>(dst + e) = make_float4(o[0], o[1], o[2], o[3]);
-        } else {
-            for (int t = 0; t < 4 && e + t < n; t++) dst[e + t] = o[t];
-        }
-    }
-}
 
 // The 1024-float tile of four super-blocks, one 16-element sub-block per lane: staged through LDS with a row stride
 // of 17 floats so that the lanes' column-wise reads do not collide.
@@ -1105,13 +1134,13 @@ hipError_t launch_quantize_q3k(const float *x, size_t n, uint8_t *dst, hipStream
 
 hipError_t launch_dequantize_q2k(const uint8_t *src, size_t n, float *dst, hipStream_t s) {
     if (n == 0) return hipSuccess;
-    hipLaunchKernelGGL(k_dequantize_q2k, dim3(grid_for((n + 4 * kDeqUnroll - 1) / (4 * kDeqUnroll), 256)), dim3(256), 0, s, src, n, dst);
+    hipLaunchKernelGGL(k_dequantize_kq<DecQ2K>, dim3(grid_for((n + 4 * kDeqUnroll - 1) / (4 * kDeqUnroll), 256)), dim3(256), 0, s, src, n, dst);
     return hipGetLastError();
 }
 
 hipError_t launch_dequantize_q3k(const uint8_t *src, size_t n, float *dst, hipStream_t s) {
     if (n == 0) return hipSuccess;
-    hipLaunchKernelGGL(k_dequantize_q3k, dim3(grid_for((n + 4 * kDeqUnroll - 1) / (4 * kDeqUnroll), 256)), dim3(256), 0, s, src, n, dst);
+    hipLaunchKernelGGL(k_dequantize_kq<DecQ3K>, dim3(grid_for((n + 4 * kDeqUnroll - 1) / (4 * kDeqUnroll), 256)), dim3(256), 0, s, src, n, dst);
     return hipGetLastError();
 }
 
@@ -1123,23 +1152,58 @@ hipError_t launch_dequantize_q8_0(const uint8_t *src, size_t n, float *dst, hipS
 
 hipError_t launch_dequantize_q5k(const uint8_t *src, size_t n, float *dst, uint32_t order, hipStream_t s) {
     if (n == 0) return hipSuccess;
-    const dim3 grid(grid_for((n + 4 * kDeqUnroll - 1) / (4 * kDeqUnroll), 256));
-    if (order == kOrderRef) hipLaunchKernelGGL(k_dequantize_q5k<0>, grid, dim3(256), 0, s, src, n, dst);
-    else hipLaunchKernelGGL(k_dequantize_q5k<1>, grid, dim3(256), 0, s, src, n, dst);
+    const dim3 grid = dim3(grid_for((n + 4 * kDeqUnroll - 1) / (4 * kDeqUnroll), 256));
+    if (order == kOrderRef) hipLaunchKernelGGL(k_dequantize_kq<DecQ5K<0>>, grid, dim3(256), 0, s, src, n, dst);
+    else hipLaunchKernelGGL(k_dequantize_kq<DecQ5K<1>>, grid, dim3(256), 0, s, src, n, dst);
     return hipGetLastError();
 }
 
 hipError_t launch_dequantize_q4k(const uint8_t *src, size_t n, float *dst, uint32_t order, hipStream_t s) {
     if (n == 0) return hipSuccess;
-    const dim3 grid(grid_for((n + 4 * kDeqUnroll - 1) / (4 * kDeqUnroll), 256));  // one lane per 4 outputs of kDeqUnroll super-blocks
-    if (order == kOrderRef) hipLaunchKernelGGL(k_dequantize_q4k<0>, grid, dim3(256), 0, s, src, n, dst);
-    else hipLaunchKernelGGL(k_dequantize_q4k<1>, grid, dim3(256), 0, s, src, n, dst);
+    const dim3 grid = dim3(grid_for((n + 4 * kDeqUnroll - 1) / (4 * kDeqUnroll), 256));  // one lane per 4 outputs of kDeqUnroll super-blocks
+    if (order == kOrderRef) hipLaunchKernelGGL(k_dequantize_kq<DecQ4K<0>>, grid, dim3(256), 0, s, src, n, dst);
+    else hipLaunchKernelGGL(k_dequantize_kq<DecQ4K<1>>, grid, dim3(256), 0, s, src, n, dst);
     return hipGetLastError();
 }
 
 hipError_t launch_dequantize_q6k(const uint8_t *src, size_t n, float *dst, hipStream_t s) {
     if (n == 0) return hipSuccess;
-    hipLaunchKernelGGL(k_dequantize_q6k, dim3(grid_for((n + 4 * kDeqUnroll - 1) / (4 * kDeqUnroll), 256)), dim3(256), 0, s, src, n, dst);
+    hipLaunchKernelGGL(k_dequantize_kq<DecQ6K>, dim3(grid_for((n + 4 * kDeqUnroll - 1) / (4 * kDeqUnroll), 256)), dim3(256), 0, s, src, n, dst);
+    return hipGetLastError();
+}
+
+hipError_t launch_dequantize_q8k(const uint8_t *src, size_t n, float *dst, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_dequantize_kq<DecQ8K>, dim3(grid_for((n + 4 * kDeqUnroll - 1) / (4 * kDeqUnroll), 256)), dim3(256), 0, s, src, n, dst);
+    return hipGetLastError();
+}
+
+// Workgroups of the fused dequantize-and-compare kernel: every wave gets at least two steps of kDeqUnroll super-blocks.
+int kl_sums_quantized_workgroups(size_t n) {
+    const size_t want = (n + 256 * kDeqUnroll * 8 - 1) / (256 * kDeqUnroll * 8);
+    return (int)(want < 1 ? 1 : (want > 2048 ? 2048 : want));
+}
+
+// type: one of the k-quants (Q2_K .. Q6_K, Q8_K); n > 0 elements of `original` against the first n decoded elements.
+hipError_t launch_kl_sums_quantized(uint32_t type, const uint8_t *src, const float *original, size_t n, uint32_t order, double *partial,
+                                    hipStream_t s) {
+    const dim3 grid((unsigned)kl_sums_quantized_workgroups(n)), block(256);
+    const bool ref = order == kOrderRef;
+    switch (type) {
+    case kTypeQ2K: hipLaunchKernelGGL(k_kl_sums_kq<DecQ2K>, grid, block, 0, s, src, original, n, partial); break;
+    case kTypeQ3K: hipLaunchKernelGGL(k_kl_sums_kq<DecQ3K>, grid, block, 0, s, src, original, n, partial); break;
+    case kTypeQ4K:
+        if (ref) hipLaunchKernelGGL(k_kl_sums_kq<DecQ4K<0>>, grid, block, 0, s, src, original, n, partial);
+        else hipLaunchKernelGGL(k_kl_sums_kq<DecQ4K<1>>, grid, block, 0, s, src, original, n, partial);
+        break;
+    case kTypeQ5K:
+        if (ref) hipLaunchKernelGGL(k_kl_sums_kq<DecQ5K<0>>, grid, block, 0, s, src, original, n, partial);
+        else hipLaunchKernelGGL(k_kl_sums_kq<DecQ5K<1>>, grid, block, 0, s, src, original, n, partial);
+        break;
+    case kTypeQ6K: hipLaunchKernelGGL(k_kl_sums_kq<DecQ6K>, grid, block, 0, s, src, original, n, partial); break;
+    case kTypeQ8K: hipLaunchKernelGGL(k_kl_sums_kq<DecQ8K>, grid, block, 0, s, src, original, n, partial); break;
+    default: return hipErrorInvalidValue;
+    }
     return hipGetLastError();
 }
 

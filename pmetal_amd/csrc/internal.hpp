@@ -61,6 +61,11 @@ hipError_t launch_dequantize_q8k(const uint8_t *src, size_t n, float *dst, hipSt
 // four f64 sums per workgroup (sum (a-b)^2, sum a^2, sum a b, sum b^2) into partial[4 * kl_sums_workgroups(n)]
 int kl_sums_workgroups(size_t n);
 hipError_t launch_kl_sums(const float *a, const float *b, size_t n, double *partial, hipStream_t s);
+// the same sums between `original` and the first n elements decoded from k-quant blocks (never stored), into
+// partial[4 * kl_sums_quantized_workgroups(n)]; hipErrorInvalidValue for a type that is not a k-quant
+int kl_sums_quantized_workgroups(size_t n);
+hipError_t launch_kl_sums_quantized(uint32_t type, const uint8_t *src, const float *original, size_t n, uint32_t order, double *partial,
+                                    hipStream_t s);
 // k a multiple of 256 and at most 32768 (the activation blocks live in LDS); type Q4_K or Q6_K
 hipError_t launch_qgemv_q8k(uint32_t type, const uint8_t *w, int64_t n, int64_t k, const uint8_t *xq, float *y, hipStream_t s);
 

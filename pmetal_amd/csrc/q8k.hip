@@ -76,23 +76,6 @@ __global__ __launch_bounds__(256) void k_quantize_q8k(const float *__restrict__ 
     if (lane == 0) *reinterpret_cast<float *>(out) = 1.0f / iscale;
 }
 
-// dequantize_q8k (crates/pmetal-gguf/src/k_quants.rs:498-506): out = d * q, one rounding.  One lane per 4 outputs.
-__global__ __launch_bounds__(256) void k_dequantize_q8k(const uint8_t *__restrict__ src, size_t n, float *__restrict__ dst) {
-    const size_t e = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
-    if (e >= n) return;
-    const uint8_t *blk = src + (e >> 8) * kQ8kBytes;
-    const float d = *reinterpret_cast<const float *>(blk);
-    const uint32_t q = *reinterpret_cast<const uint32_t *>(blk + 4 + (e & 255));
-    float o[4];
-#pragma unroll
-    for (int c = 0; c < 4; c++) o[c] = d * (float)(int8_t)(q >> (8 * c));
-    if (e + 3 < n) {
-        *reinterpret_cast<float4 *>(dst + e) = make_float4(o[0], o[1], o[2], o[3]);
-    } else {
-        for (int c = 0; c < 4 && e + c < n; c++) dst[e + c] = o[c];
-    }
-}
-
 // The four f64 sums of compute_kl_divergence (crates/pmetal-gguf/src/dynamic.rs:140-180) over n pairs (original,
 // dequantized): sum (a - b)^2 with the difference taken in f32 as the reference takes it, sum a^2, sum a b, sum b^2.
 // Every workgroup writes its four partial sums; the caller adds the workgroups' sums in order.
@@ -339,12 +322,6 @@ hipError_t launch_quantize_q8k(const float *x, size_t n, uint8_t *dst, hipStream
     const size_t n_blocks = n / 256 + (n % 256 != 0), n_full = n / 256;
     if (n_blocks == 0) return hipSuccess;
     hipLaunchKernelGGL(k_quantize_q8k, dim3((unsigned)((n_blocks + 3) / 4)), dim3(256), 0, s, x, n_full, n_blocks, dst);
-    return hipGetLastError();
-}
-
-hipError_t launch_dequantize_q8k(const uint8_t *src, size_t n, float *dst, hipStream_t s) {
-    if (n == 0) return hipSuccess;
-    hipLaunchKernelGGL(k_dequantize_q8k, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, s, src, n, dst);
     return hipGetLastError();
 }
 

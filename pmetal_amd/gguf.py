@@ -199,6 +199,14 @@ def kl_divergence_dev(original, dequantized, n: int, stream=None) -> float:
     return score.value
 
 
+def kl_divergence_quantized_dev(dtype, quantized, nbytes: int, original, n: int, order: int = ORDER_REF, stream=None) -> float:
+    """Dequantize-and-score in one pass for the k-quant types: the first ``n`` elements of the blocks against ``original``."""
+    score = C.c_double()
+    check(_lib.load().pmetal_hip_kl_divergence_quantized_dev(int(dtype), _dev_ptr(quantized), nbytes, _dev_ptr(original), n, order,
+                                                             C.byref(score), stream))
+    return score.value
+
+
 def is_critical_layer(name: str) -> bool:
     """``DynamicQuantizer::is_critical_layer`` (crates/pmetal-gguf/src/dynamic.rs:254-268)."""
     return any(s in name for s in ("lm_head", "output", "token_embd", "embed_tokens", "wte", "final_norm", "ln_f"))
@@ -211,8 +219,8 @@ DEFAULT_KL_CANDIDATES = (GgmlType.Q8K, GgmlType.Q6K, GgmlType.Q5K, GgmlType.Q4K,
 def calibrate_tensor(name: str, data, shape, candidates=DEFAULT_KL_CANDIDATES, kl_threshold: float = 0.01,
                      fallback_type: int = GgmlType.Q8K, sample_size: int = 0, order: int = ORDER_REF):
     """``DynamicQuantizer::calibrate_tensor`` (crates/pmetal-gguf/src/dynamic.rs:420-502) with the round trips on the GPU:
-    the tensor is uploaded once, every candidate is quantized, dequantized (in the reference dequantizer's element order
-    unless ``order`` says otherwise) and scored on the device.  Returns ``(quant_type, kl_score, all_scores)``.  As in
+    the tensor is uploaded once, every candidate is quantized and scored on the device against its dequantized values (in
+    the reference dequantizer's element order unless ``order`` says otherwise; the k-quants without storing them).  Returns ``(quant_type, kl_score, all_scores)``.  As in
     the reference, a candidate the quantizer does not implement is skipped."""
     lib = _lib.load()
     x = np.ascontiguousarray(data, dtype=np.float32).reshape(-1)
@@ -223,7 +231,7 @@ def calibrate_tensor(name: str, data, shape, candidates=DEFAULT_KL_CANDIDATES, k
     sample = sample_size if 0 < sample_size < n else n
     scores = []
     if n:
-        dx, ddeq = DeviceBuffer.from_host(x), DeviceBuffer(4 * max(n, 4))
+        dx, ddeq = DeviceBuffer.from_host(x), None
     for t in candidates:
         t = int(t)
         # quantize the whole tensor, dequantize what the shape asks for; a type without kernels, or a shape whose byte
@@ -236,8 +244,12 @@ def calibrate_tensor(name: str, data, shape, candidates=DEFAULT_KL_CANDIDATES, k
             continue
         dq = DeviceBuffer(max(nbytes, 16))
         check(lib.pmetal_hip_quantize_dev(t, dx.ptr, n, dq.ptr, nbytes, None), "quantize")
-        check(lib.pmetal_hip_dequantize_dev(t, dq.ptr, nbytes, ddeq.ptr, n_shape, order, None))
-        scores.append((t, kl_divergence_dev(dx, ddeq, min(sample, n_shape))))
+        if lib.pmetal_hip_block_size(t) == 256:  # k-quants: decoded and compared in one pass, nothing stored
+            scores.append((t, kl_divergence_quantized_dev(t, dq, nbytes, dx, min(sample, n_shape), order)))
+        else:
+            ddeq = ddeq or DeviceBuffer(4 * max(n, 4))
+            check(lib.pmetal_hip_dequantize_dev(t, dq.ptr, nbytes, ddeq.ptr, n_shape, order, None))
+            scores.append((t, kl_divergence_dev(dx, ddeq, min(sample, n_shape))))
         dq.free()
     if not scores:
         big = float(np.finfo(np.float64).max)

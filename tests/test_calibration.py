@@ -134,3 +134,47 @@ def test_gpu_calibrate_tensor_matches_oracle(oracle):
     assert t == Q8K and score == np.finfo(np.float64).max
     got, want = gguf.calibrate_tensor("blk.0.ffn_up.weight", x, [64, 1023]), oracle.calibrate_tensor("blk.0.ffn_up.weight", x, [64, 1023])
     assert got[0] == want[0] and got[1] == pytest.approx(want[1], rel=1e-10, abs=1e-14) and len(got[2]) == len(want[2]) == 6
+
+
+@pytest.mark.gpu
+def test_gpu_fused_dequantize_and_score_equals_the_two_steps(oracle):
+    """pmetal_hip_kl_divergence_quantized_dev against dequantize_dev + kl_divergence_dev and against the oracle, for every
+    k-quant type, both element orders, lengths that end inside a block and inside a float4, random block bytes."""
+    import pmetal_amd as pm
+    from pmetal_amd import _lib, gguf
+    pm.init(0)
+    lib = _lib.load()
+    rng = np.random.default_rng(31)
+    n_full = 256 * 700
+    x = (rng.standard_normal(n_full) * 0.02).astype(np.float32)
+    dx = pm.DeviceBuffer.from_host(x)
+    ddeq = pm.DeviceBuffer(4 * n_full)
+    for t in (Q8K, Q6K, Q5K, Q4K, Q3K, Q2K):
+        q = oracle.quantize(t, x)
+        dq = pm.DeviceBuffer.from_host(q)
+        for order in (0, 1):
+            for n in (n_full, n_full - 1, n_full - 255, 256 * 300 + 7, 5, 1):
+                got = gguf.kl_divergence_quantized_dev(t, dq, q.size, dx, n, order)
+                pm.check(lib.pmetal_hip_dequantize_dev(t, dq.ptr, q.size, ddeq.ptr, n_full, order, None))
+                two = gguf.kl_divergence_dev(dx, ddeq, n)
+                want = oracle.kl_divergence(x[:n], oracle.dequantize(t, q, [n_full], order=order)[:n])
+                assert got == pytest.approx(two, rel=1e-10, abs=1e-14), (t, order, n)
+                assert got == pytest.approx(want, rel=1e-10, abs=1e-14), (t, order, n)
+        # zero elements: 0.0 without touching the device; more elements than the blocks hold: invalid size
+        assert gguf.kl_divergence_quantized_dev(t, dq, q.size, dx, 0) == 0.0
+        sc = __import__("ctypes").c_double()
+        assert lib.pmetal_hip_kl_divergence_quantized_dev(t, dq.ptr, q.size, dx.ptr, n_full + 1, 0, sc, None) == 3
+        assert lib.pmetal_hip_kl_divergence_quantized_dev(t, dq.ptr, q.size - 2, dx.ptr, 16, 0, sc, None) == 3
+        lib.pmetal_hip_clear_error()
+    # a type with 32-element blocks has no fused comparison: the reference's unsupported-type class
+    sc = __import__("ctypes").c_double()
+    assert lib.pmetal_hip_kl_divergence_quantized_dev(Q8_0, dx.ptr, 34, dx.ptr, 32, 0, sc, None) == 2
+    assert lib.pmetal_hip_kl_divergence_quantized_dev(Q4K, dx.ptr, 144, dx.ptr, 32, 7, sc, None) == 1
+    lib.pmetal_hip_clear_error()
+    # NaNs and infinities in random block bytes propagate as in the two-step path
+    raw = rng.integers(0, 256, 176 * 64, dtype=np.uint8)
+    draw = pm.DeviceBuffer.from_host(raw)
+    got = gguf.kl_divergence_quantized_dev(Q5K, draw, raw.size, dx, 64 * 256, 1)
+    pm.check(lib.pmetal_hip_dequantize_dev(Q5K, draw.ptr, raw.size, ddeq.ptr, 64 * 256, 1, None))
+    two = gguf.kl_divergence_dev(dx, ddeq, 64 * 256)
+    assert (np.isnan(got) and np.isnan(two)) or got == pytest.approx(two, rel=1e-10)
