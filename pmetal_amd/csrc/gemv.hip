@@ -398,6 +398,8 @@ hipError_t launch_qgemv(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
                     : launch_q6k<false>(team, grid, lds, s, w, x, y, (int)n, spr);
     }
     if (type == kTypeQ8_0) {
+        hipError_t chunk_err = hipSuccess;
+        if (try_launch_qgemv_q8_0_chunk(w, n, k, x, x_dtype, y, s, &chunk_err)) return chunk_err;
         const int bpr = (int)(k / 32);
         const int team = pow2_divisor(bpr, 64);
         const size_t lds = (size_t)bpr * 128;

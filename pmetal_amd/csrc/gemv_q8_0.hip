@@ -1,0 +1,276 @@
+// Dequant-fused GEMV for large Q8_0 matrices on gfx950: rows staged through LDS, integer dot products.
+//
+// y[n] = sum_k W[n,k] * x[k], W the GGUF Q8_0 block stream (34 bytes per 32 weights: d f16, qs[32] i8; value d * q,
+// dequant.rs:466-495).  A 34-byte block is aligned to two bytes only, and a lane that reads its own block from
+// global memory touches a different cache line than its neighbours with every load.  Here a wave copies 2176
+// contiguous, 16-byte aligned bytes of a row (64 blocks) into LDS with whole-wave 16-byte loads, and each lane then
+// takes its block out of LDS as aligned dwords which one funnel shift per dword puts into place.
+//
+//  * The activations are converted once per workgroup to fixed point: every 32-element group (one block) gets a
+//    power-of-two scale that puts its largest magnitude below 2^22, and the 23-bit signed integers are written as
+//    three balanced base-256 digits in [-128, 127].  sum q x over a block is then 2^e * (65536 dot(q, d2) + 256
+//    dot(q, d1) + dot(q, d0)) with v_dot4_i32_i8 on the quant dwords: integer arithmetic, exact up to the fixed-point
+//    resolution of x (22 bits under the group maximum).
+//  * One workgroup per compute unit; a row is ks = (k / 32) / 64 chunks of 64 blocks.  Wave (g, h) takes chunk h of the
+//    rows of row group g, lane l block 64 h + l, so that a lane's digits (24 registers) never change.  Up to kDepth
+//    rows are in flight per wave; every load is issued unconditionally (rows past the end read the first bytes of
+//    W) so that the number of outstanding loads is known at every wait.  Lane partial sums go to LDS; after a barrier
+//    the workgroup adds up each of its rows and stores y.
+//
+// Smaller matrices, and rows that are not whole chunks, stay with the kernel in gemv.hip.
+#include "gemv_common.hpp"
+#include "internal.hpp"
+
+namespace {
+
+using namespace pmh::gemv;
+
+typedef uint32_t u4v __attribute__((ext_vector_type(4)));  // a 16-byte piece
+
+constexpr int kDepth = 5;  // rows in flight per wave
+constexpr int kPre = 2;    // of which this many are requested before x is converted
+constexpr int kPlanes = 3;
+constexpr int kChunkBytes = 64 * 34;          // 2176 = 136 pieces of 16 bytes
+constexpr int kStageBytes = kChunkBytes + 16;  // the ninth dword of the last lane lies past the chunk
+
+__host__ __device__ constexpr int part_stride(int slots, int red) { return ((slots + 63) / 64) * 64 + (red & 63); }
+
+__device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {
+    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
+}
+
+// Activations -> LDS.  Thread idx converts elements 4 idx .. 4 idx + 3; eight consecutive threads hold one block.
+// xd[(plane * 8 + dword) * slots + block]: four digits; xm[block] = the block's scale.
+template <bool XF32>
+__device__ __forceinline__ void stage_x(const void *__restrict__ xg, int slots, int nthreads, uint32_t *xd, float *xm) {
+    const int total = slots * 8;  // k / 4
+    for (int idx0 = 0; idx0 < total; idx0 += nthreads) {
+        const int idx = idx0 + (int)threadIdx.x;
+        const bool live = idx < total;
+        const int id = live ? idx : total - 1;
+        float v[4];
+        if (XF32) {
+            const float4 f = reinterpret_cast<const float4 *>(xg)[id];
+            v[0] = f.x, v[1] = f.y, v[2] = f.z, v[3] = f.w;
+        } else {
+            const uint2 b = reinterpret_cast<const uint2 *>(xg)[id];
+            v[0] = __builtin_bit_cast(float, b.x << 16), v[1] = __builtin_bit_cast(float, b.x & 0xFFFF0000u);
+            v[2] = __builtin_bit_cast(float, b.y << 16), v[3] = __builtin_bit_cast(float, b.y & 0xFFFF0000u);
+        }
+        // largest magnitude of the block, as bits (the order of non-negative floats is that of their bits)
+        uint32_t mb = 0;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const uint32_t a = __builtin_bit_cast(uint32_t, v[c]) & 0x7FFFFFFFu;
+            mb = a > mb ? a : mb;
+        }
+#pragma unroll
+        for (int off = 1; off < 8; off <<= 1) {
+            const uint32_t o = (uint32_t)__shfl_xor((int)mb, off);
+            mb = o > mb ? o : mb;
+        }
+        int eb = (int)(mb >> 23);    // biased exponent: every |x| of the block is below 2^(eb - 126)
+        const bool bad = eb == 255;  // an infinity or a NaN among the activations: every output becomes NaN
+        eb = eb < 21 ? 21 : eb;
+        const float mult = __builtin_bit_cast(float, (uint32_t)(275 - eb) << 23);  // 2^(148 - eb): |x| * mult < 2^22
+        const float scale = bad ? __builtin_nanf("") : __builtin_bit_cast(float, (uint32_t)(eb - 21) << 23);  // 2^(eb - 148); 0 below 2^-126
+        uint32_t dig[kPlanes] = {0, 0, 0};
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const int xi = bad ? 0 : (int)__builtin_rintf(v[c] * mult);
+            const int d0 = (int)(int8_t)xi, r1 = (xi - d0) >> 8;
+            const int d1 = (int)(int8_t)r1, d2 = (r1 - d1) >> 8;
+            dig[0] |= (uint32_t)(d0 & 0xFF) << (8 * c);
+            dig[1] |= (uint32_t)(d1 & 0xFF) << (8 * c);
+            dig[2] |= (uint32_t)(d2 & 0xFF) << (8 * c);
+        }
+        if (live) {
+            const int blk = id >> 3, dw = id & 7;
+#pragma unroll
+            for (int p = 0; p < kPlanes; p++) xd[(p * 8 + dw) * slots + blk] = dig[p];
+            if (dw == 0) xm[blk] = scale;
+        }
+    }
+}
+
+template <bool XF32, bool SINGLE>
+__global__ __launch_bounds__(1024) void k_qgemv_q8_0_chunk(const uint8_t *__restrict__ W, const void *__restrict__ xg,
+                                                            float *__restrict__ y, int n_rows, int bpr, int rows_per_wg,
+                                                            int rows_per_wave, int n_nominal, int red, int nthreads) {
+    extern __shared__ uint4 smem[];
+    const int slots = bpr;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int n_waves = nthreads >> 6;
+    uint32_t *stage = reinterpret_cast<uint32_t *>(smem) + wave * (kStageBytes / 4);  // this wave's row chunk
+    uint32_t *xd = reinterpret_cast<uint32_t *>(smem) + n_waves * (kStageBytes / 4);  // [kPlanes * 8][slots]
+    float *xm = reinterpret_cast<float *>(xd + kPlanes * 8 * slots);                  // [slots]
+    float *part = xm + slots;                                                         // [group][n_nominal][part_stride]
+    const int ps = part_stride(slots, red);
+    const int ks = bpr >> 6;
+    const int h = wave % ks, g = wave / ks;
+    const int wg_r0 = blockIdx.x * rows_per_wg;
+    const int wg_r1 = wg_r0 + rows_per_wg < n_rows ? wg_r0 + rows_per_wg : n_rows;
+    const int wave_r0 = wg_r0 + g * rows_per_wave;
+    const int wave_r1 = wave_r0 + rows_per_wave < wg_r1 ? wave_r0 + rows_per_wave : wg_r1;
+    const int nt_wave = wave_r1 > wave_r0 ? wave_r1 - wave_r0 : 0;  // real tasks of this wave (wave-uniform)
+
+    const uint32_t rowbytes = (uint32_t)bpr * 34u;
+    const uint32_t off_a = (uint32_t)h * kChunkBytes + 16u * (uint32_t)lane;
+    const uint32_t off_c = (uint32_t)h * kChunkBytes + 2048u + 16u * (uint32_t)(lane & 7);
+    // a wave's 136 pieces of a row chunk: lane l takes pieces l and 64 + l, lanes 0..7 also piece 128 + l
+    auto issue = [&](int i, u4v &a, u4v &b, u4v &c) {
+        const bool real = i < nt_wave;  // wave-uniform
+        const uint32_t ro = real ? (uint32_t)(wave_r0 + i) * rowbytes : 0u;
+        a = *reinterpret_cast<const u4v *>(W + (ro + (real ? off_a : 0u)));
+        b = *reinterpret_cast<const u4v *>(W + (ro + (real ? off_a + 1024u : 0u)));
+        c = *reinterpret_cast<const u4v *>(W + (ro + (real ? off_c : 0u)));
+    };
+
+    u4v ra[kDepth], rb[kDepth], rc[kDepth];
+#pragma unroll
+    for (int i = 0; i < kPre; i++) issue(i, ra[i], rb[i], rc[i]);
+    stage_x<XF32>(xg, slots, nthreads, xd, xm);
+    __syncthreads();
+
+    const int slot = h * 64 + lane;
+    uint32_t xr[kPlanes][8];
+#pragma unroll
+    for (int p = 0; p < kPlanes; p++)
+#pragma unroll
+        for (int k = 0; k < 8; k++) xr[p][k] = xd[(p * 8 + k) * slots + slot];
+    const float xscale = xm[slot];
+
+    // Block `lane` of the chunk starts at byte 34 lane: on a dword boundary for an even lane (the scale is the low half
+    // of that dword, the quants follow two bytes in), two bytes past one for an odd lane (the scale is the high half of
+    // the dword below, the quants start on a dword boundary).
+    const int odd = lane & 1;
+    const uint32_t *sp = stage + ((34 * lane) >> 2);       // the dword that holds the scale
+    const uint32_t *qp = stage + ((34 * lane + 2) >> 2);   // the dword that holds the first quant
+    const uint32_t d_shift = odd ? 16u : 0u, q_shift = odd ? 0u : 16u;
+
+    float *pp = part + (size_t)(g * n_nominal) * ps + slot;
+    auto consume = [&](int i, const u4v a, const u4v b, const u4v c) {
+        if (i < nt_wave) {  // wave-uniform
+        u4v *st4 = reinterpret_cast<u4v *>(stage);
+        st4[lane] = a;
+        st4[64 + lane] = b;
+        if (lane < 8) st4[128 + lane] = c;
+        // LDS executes a wave's instructions in order: the reads below see the writes above, and the next row's writes
+        // come after these reads
+        const uint32_t dw = *sp;
+        uint32_t w[9];
+#pragma unroll
+        for (int k = 0; k < 9; k++) w[k] = qp[k];
+        int acc[kPlanes] = {0, 0, 0};
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const uint32_t q = __builtin_amdgcn_alignbit(w[k + 1], w[k], q_shift);
+#pragma unroll
+            for (int p = 0; p < kPlanes; p++) acc[p] = sdot4(q, xr[p][k], acc[p]);
+        }
+        float f = (float)acc[kPlanes - 1];
+#pragma unroll
+        for (int p = kPlanes - 2; p >= 0; p--) f = __builtin_fmaf(f, 256.0f, (float)acc[p]);
+        pp[(size_t)i * ps] = (f16_bits_to_f32((dw >> d_shift) & 0xFFFFu) * xscale) * f;
+        }
+    };
+
+    int issued = kPre;
+#pragma unroll
+    for (int i = 0; i < kDepth; i++) {
+        consume(i, ra[i], rb[i], rc[i]);
+        const int upto = SINGLE ? (kPre + 2 * (i + 1) < kDepth ? kPre + 2 * (i + 1) : kDepth)
+                                : (kPre + 2 * (i + 1) < kDepth + i + 1 ? kPre + 2 * (i + 1) : kDepth + i + 1);
+#pragma unroll
+        for (; issued < upto; issued++) issue(issued, ra[issued % kDepth], rb[issued % kDepth], rc[issued % kDepth]);
+    }
+    if (!SINGLE) {
+        int base = kDepth;
+        for (; base + kDepth < n_nominal; base += kDepth) {
+#pragma unroll
+            for (int i = 0; i < kDepth; i++) {
+                consume(base + i, ra[i], rb[i], rc[i]);
+                issue(base + kDepth + i, ra[i], rb[i], rc[i]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kDepth; i++) consume(base + i, ra[i], rb[i], rc[i]);
+    }
+    __syncthreads();
+
+    // Row totals: `red` lanes per row (a power of two from 8 to 64 that divides slots), lane p adding every
+    // red-th partial, then a sum over the lanes of the row.
+    const int wg_rows = wg_r1 - wg_r0;
+    const int per_thread = slots / red;
+    const int red_shift = 31 - __builtin_clz(red);
+    for (int idx0 = 0; idx0 < wg_rows * red; idx0 += nthreads) {
+        const int idx = idx0 + (int)threadIdx.x;
+        int rl = idx >> red_shift;
+        const bool ok = rl < wg_rows;
+        rl = ok ? rl : wg_rows - 1;
+        const int grp = rl / rows_per_wave, loc = rl - grp * rows_per_wave;
+        const int p = idx & (red - 1);
+        const float *src = part + (size_t)(grp * n_nominal + loc) * ps + p;
+        float t0 = 0.0f, t1 = 0.0f, t2 = 0.0f, t3 = 0.0f;
+        int i = 0;
+        for (; i + 8 <= per_thread; i += 8) {  // eight reads in flight
+            const float *q = src + (size_t)i * red;
+            const float a0 = q[0], a1 = q[red], a2 = q[2 * red], a3 = q[3 * red];
+            const float a4 = q[4 * red], a5 = q[5 * red], a6 = q[6 * red], a7 = q[7 * red];
+            t0 += a0 + a4, t1 += a1 + a5, t2 += a2 + a6, t3 += a3 + a7;
+        }
+        for (; i < per_thread; i++) t0 += src[(size_t)i * red];
+        const float sum = team_sum_rt((t0 + t1) + (t2 + t3), red);
+        if (ok && p == 0) y[wg_r0 + rl] = sum;
+    }
+}
+
+}  // namespace
+
+namespace pmh {
+
+// Runs the row-staging kernel when the shape suits it and returns true; otherwise leaves *err untouched and returns
+// false (the caller falls back to the general Q8_0 kernel).  Preconditions as for launch_qgemv.
+bool try_launch_qgemv_q8_0_chunk(const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, float *y,
+                                 hipStream_t s, hipError_t *err) {
+    const int bpr = (int)(k / 32);
+    if (bpr % 64) return false;
+    const int ks = bpr / 64;
+    const uint64_t w_bytes = (uint64_t)n * (uint64_t)bpr * 34u;
+    static const int64_t mode = gemv::tuning("PMETAL_HIP_GEMV_Q8_0_KERNEL", 0);  // 0 = choose, 1 = this kernel, 2 = general kernel
+    if (mode == 2 || ks > 16 || w_bytes >= (1ull << 32)) return false;
+    if (mode == 0 && w_bytes < (12ull << 20)) return false;
+    const size_t slots = (size_t)bpr;
+    const int64_t want = gemv::compute_units();
+    int64_t n_wg = n < want ? n : want;
+    const int64_t rows_per_wg = (n + n_wg - 1) / n_wg;
+    n_wg = (n + rows_per_wg - 1) / rows_per_wg;
+    int64_t groups = 16 / ks;
+    if (groups > rows_per_wg) groups = rows_per_wg;
+    const int64_t rows_per_wave = (rows_per_wg + groups - 1) / groups;
+    groups = (rows_per_wg + rows_per_wave - 1) / rows_per_wave;
+    const int64_t n_nominal = rows_per_wave;
+    const int64_t threads = ks * groups * 64;
+    int red = 8;  // lanes per row in the final summation: as many as the workgroup has to spare, at most 64
+    while (red < 64 && rows_per_wg * red * 2 <= threads) red *= 2;
+    const size_t lds = (size_t)(threads / 64) * kStageBytes + slots * 4 * (kPlanes * 8) + slots * 4 +
+                       (size_t)groups * (size_t)n_nominal * part_stride((int)slots, red) * 4;
+    if (lds > 128 * 1024) return false;
+    const bool single = n_nominal <= kDepth;
+    const bool xf32 = x_dtype == kDtypeF32;
+    auto go = [&](auto kern) {
+        if (lds > 64 * 1024) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return e;
+        }
+        hipLaunchKernelGGL(kern, dim3((unsigned)n_wg), dim3((unsigned)threads), lds, s, w, x, y, (int)n, bpr, (int)rows_per_wg,
+                           (int)rows_per_wave, (int)n_nominal, red, (int)threads);
+        return hipGetLastError();
+    };
+    if (xf32) *err = single ? go(k_qgemv_q8_0_chunk<true, true>) : go(k_qgemv_q8_0_chunk<true, false>);
+    else *err = single ? go(k_qgemv_q8_0_chunk<false, true>) : go(k_qgemv_q8_0_chunk<false, false>);
+    return true;
+}
+
+}  // namespace pmh

@@ -116,6 +116,53 @@ def test_qgemv_q6k_large_quantized_weights_and_linearity(oracle):
     assert np.isnan(gpu_qgemv(Q6K, wq, n, k, xa, pm.DTYPE_F32, 0)).all()
 
 
+# Q8_0 matrices of 12 MiB and more whose rows are whole chunks of 64 blocks (k a multiple of 2048) take the kernel that
+# stages rows through LDS: ragged row counts, rows of 1, 2, 7 and 16 chunks, fewer rows than compute units times waves;
+# activations with large and tiny outliers and a run of zeros; quants over the whole int8 range.
+Q8_0_BIG_CASES = [(6001, 4096), (14336, 4096), (4096, 14336), (30001, 2048), (500, 32768), (1900, 6144)]
+
+
+@pytest.mark.parametrize("n,k", Q8_0_BIG_CASES)
+@pytest.mark.parametrize("x_dtype", [pm.DTYPE_BF16, pm.DTYPE_F32])
+def test_qgemv_q8_0_large_shapes(oracle, n, k, x_dtype):
+    rng = np.random.default_rng(n + k + 1)
+    raw = rng.integers(0, 256, size=(n * (k // 32), 34), dtype=np.uint8)
+    scales = (rng.uniform(0.5, 2.0, n * (k // 32)) * 1e-3 * rng.choice([-1.0, 1.0], n * (k // 32))).astype(np.float16)
+    raw[:, 0:2] = scales.view(np.uint8).reshape(-1, 2)
+    raw = raw.reshape(-1)
+    x = rng.standard_normal(k).astype(np.float32)
+    x[rng.integers(0, k, k // 300)] *= 1000.0
+    x[rng.integers(0, k, k // 300)] *= 1e-6
+    x[5:40] = 0.0
+    if x_dtype == pm.DTYPE_BF16:
+        x_dev = oracle.f32_to_bf16_bits(x)
+        x_ref = oracle.bf16_bits_to_f32(x_dev)
+    else:
+        x_dev = x_ref = x
+    want = oracle.qmatvec(Q8_0, raw, n, k, x_ref)
+    got = gpu_qgemv(Q8_0, raw, n, k, x_dev, x_dtype, 0)
+    elem, norm = rel_errors(got, want)
+    print(f"Q8_0 {n}x{k} x_dtype {x_dtype}: elem {elem:.2e} norm {norm:.2e}")
+    assert elem <= TOL and norm <= TOL
+
+
+def test_qgemv_q8_0_large_unit_vectors_and_special_values(oracle):
+    """Every position of a block, in an even and in an odd block, reaches the right activation; zero input gives zero;
+    an infinity among the activations reaches every output."""
+    n, k = 7000, 4096
+    wq = pm.quantize(weights(23, n * k, outliers=1e-3), Q8_0)
+    w = oracle.dequantize(Q8_0, wq, [n, k]).reshape(n, k)
+    for j in list(range(0, 70)) + [2047, 2048, 2049, 4062, 4063, 4095]:
+        x = np.zeros(k, np.float32)
+        x[j] = 1.0
+        got = gpu_qgemv(Q8_0, wq, n, k, x, pm.DTYPE_F32, 0)
+        assert np.array_equal(got, w[:, j]), j
+    assert not gpu_qgemv(Q8_0, wq, n, k, np.zeros(k, np.float32), pm.DTYPE_F32, 0).any()
+    x = np.random.default_rng(5).standard_normal(k).astype(np.float32)
+    x[100] = np.inf
+    assert np.isnan(gpu_qgemv(Q8_0, wq, n, k, x, pm.DTYPE_F32, 0)).all()
+
+
 def test_qgemv_config0_q8_0_round_trip_and_gemv(oracle):
     # BASELINE config 0: 3072x1024 N(0, 0.02), Q8_0 round trip, then y = W x with f32 x ~ N(0, 1)
     n, k = 3072, 1024
