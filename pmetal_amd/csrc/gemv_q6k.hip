@@ -1,0 +1,328 @@
+// Dequant-fused GEMV for large Q6_K matrices on gfx950: integer dot products over the packed bytes.
+//
+// y[n] = sum_k W[n,k] * x[k], W the GGUF Q6_K block stream (210 bytes per 256 weights: ql[128], qh[64],
+// scales[16] i8, d f16; value d * sc * (q - 32) with q = nibble | two high bits << 4, k_quants.rs:474-496).
+//
+//  * The activations are converted once per workgroup to fixed point: every 16-element group (one Q6_K
+//    sub-block) gets a power-of-two scale that puts its largest magnitude below 2^22, and the 23-bit signed
+//    integers are written as three balanced base-256 digits in [-128, 127].  sum q x over a sub-block is then
+//    2^e * (65536 dot(q, d2) + 256 dot(q, d1) + dot(q, d0)) with v_dot4_i32_i8 on four stored 6-bit values per
+//    dword: integer arithmetic, exact up to the fixed-point resolution of x (22 bits under the group maximum).
+//    The stored values are q + 32; the offset is removed with the group's sum of x, computed with the digits.
+//  * One workgroup per compute unit; a row is ks = (k / 256) / 8 chunks of eight super-blocks.  Wave (g, h) takes
+//    chunk h of the rows of row group g: eight lanes per super-block, lane t owning the two sub-blocks that
+//    share the ql bytes 16 (t % 4) .. + 15 of half t / 4, so that a lane's digits (24 registers) never change.
+//  * Blocks are only 2-byte aligned, and dword loads at such addresses are slow.  A wave therefore copies the 1680
+//    contiguous, 16-byte aligned bytes of its chunk of a row into its own piece of LDS with whole-wave 16-byte loads
+//    (up to kDepth rows in flight, every load issued unconditionally so that the number of outstanding loads is known
+//    at every wait; rows past the end read the first bytes of W), and each lane takes its pieces out of LDS as
+//    aligned dwords which one funnel shift per dword puts into place for the odd super-blocks.  LDS executes a
+//    wave's instructions in order, so the copy needs no barrier.
+//  * Lane partial sums go to LDS; after a barrier the workgroup adds up each of its rows and stores y.
+//
+// Smaller or oddly shaped matrices stay with the bf16 kernel in gemv.hip.
+#include "gemv_common.hpp"
+#include "internal.hpp"
+
+namespace {
+
+using namespace pmh::gemv;
+
+typedef uint32_t u4v __attribute__((ext_vector_type(4)));  // a 16-byte piece
+
+constexpr int kDepth = 6;  // tasks in flight per wave
+constexpr int kPre = 2;    // of which this many are requested before x is converted
+constexpr int kPlanes = 3;
+constexpr int kChunkBytes = 8 * 210;           // 1680 = 105 pieces of 16 bytes
+constexpr int kStageBytes = kChunkBytes + 16;  // the shifted reads of the last lanes reach one dword past the chunk
+
+__host__ __device__ constexpr int part_stride(int slots, int red) { return ((slots + 63) / 64) * 64 + (red & 63); }
+
+__device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {
+    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
+}
+
+// Activations -> LDS.  Thread idx converts elements 4 idx .. 4 idx + 3; the four threads of a quad hold one
+// 16-element group.  Element e = 256 sb + 128 hh + 32 g + l belongs to lane t = 4 hh + 2 (g & 1) + l / 16 of its
+// super-block (slot 8 sb + t), sub-block s = g >> 1 of that lane, dword (l % 16) / 4.
+// xd[(plane * 8 + 4 s + dword) * slots + slot]: four digits; xm[slot] = (scale s = 0, scale s = 1, sum s = 0, sum s = 1).
+template <bool XF32>
+__device__ __forceinline__ void stage_x(const void *__restrict__ xg, int slots, int nthreads, uint32_t *xd, float *xm) {
+    const int total = slots * 8;  // quads of four elements: k / 4
+    for (int idx0 = 0; idx0 < total; idx0 += nthreads) {
+        const int idx = idx0 + (int)threadIdx.x;
+        const bool live = idx < total;
+        const int id = live ? idx : total - 1;
+        float v[4];
+        if (XF32) {
+            const float4 f = reinterpret_cast<const float4 *>(xg)[id];
+            v[0] = f.x, v[1] = f.y, v[2] = f.z, v[3] = f.w;
+        } else {
+            const uint2 b = reinterpret_cast<const uint2 *>(xg)[id];
+            v[0] = __builtin_bit_cast(float, b.x << 16), v[1] = __builtin_bit_cast(float, b.x & 0xFFFF0000u);
+            v[2] = __builtin_bit_cast(float, b.y << 16), v[3] = __builtin_bit_cast(float, b.y & 0xFFFF0000u);
+        }
+        // largest magnitude of the 16-element group, as bits (the order of non-negative floats is that of their bits)
+        uint32_t mb = 0;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const uint32_t a = __builtin_bit_cast(uint32_t, v[c]) & 0x7FFFFFFFu;
+            mb = a > mb ? a : mb;
+        }
+        uint32_t o = (uint32_t)__shfl_xor((int)mb, 1);
+        mb = o > mb ? o : mb;
+        o = (uint32_t)__shfl_xor((int)mb, 2);
+        mb = o > mb ? o : mb;
+        int eb = (int)(mb >> 23);  // biased exponent: every |x| of the group is below 2^(eb - 126)
+        const bool bad = eb == 255;  // an infinity or a NaN among the activations: every output becomes NaN
+        eb = eb < 21 ? 21 : eb;
+        const float mult = __builtin_bit_cast(float, (uint32_t)(275 - eb) << 23);  // 2^(148 - eb): |x| * mult < 2^22
+        const float scale = bad ? __builtin_nanf("") : __builtin_bit_cast(float, (uint32_t)(eb - 21) << 23);  // 2^(eb - 148); 0 below 2^-126
+        uint32_t dig[kPlanes] = {0, 0, 0};
+        int sum = 0;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const int xi = bad ? 0 : (int)__builtin_rintf(v[c] * mult);
+            sum += xi;
+            const int d0 = (int)(int8_t)xi, r1 = (xi - d0) >> 8;
+            const int d1 = (int)(int8_t)r1, d2 = (r1 - d1) >> 8;
+            dig[0] |= (uint32_t)(d0 & 0xFF) << (8 * c);
+            dig[1] |= (uint32_t)(d1 & 0xFF) << (8 * c);
+            dig[2] |= (uint32_t)(d2 & 0xFF) << (8 * c);
+        }
+        sum += __shfl_xor(sum, 1);
+        sum += __shfl_xor(sum, 2);
+        if (live) {
+            const int e = id * 4, sb = e >> 8, r = e & 255;
+            const int hh = r >> 7, g = (r >> 5) & 3, l = r & 31;
+            const int slot = sb * 8 + 4 * hh + 2 * (g & 1) + (l >> 4), s = g >> 1, dw = (l & 15) >> 2;
+#pragma unroll
+            for (int p = 0; p < kPlanes; p++) xd[(p * 8 + 4 * s + dw) * slots + slot] = dig[p];
+            if (dw == 0) {
+                xm[slot * 4 + s] = scale;
+                xm[slot * 4 + 2 + s] = (float)sum;
+            }
+        }
+    }
+}
+
+// One lane's share of a super-block, as it lies in memory.
+struct Task {
+    uint32_t ql[4], qh[4], sc[2], d;
+};
+
+// The two sub-blocks of a lane: A = low nibbles (group ga = tq >> 1), B = high nibbles (group ga + 2).
+template <int PLANES>
+__device__ __forceinline__ float lane_dot(const Task &t, const uint32_t (&xr)[kPlanes][8], const float4 xm, int sh_a, int sh_b,
+                                          int sc_up) {
+    const uint32_t(&ql)[4] = t.ql, (&qh)[4] = t.qh;
+    int acc_a[PLANES], acc_b[PLANES];
+#pragma unroll
+    for (int p = 0; p < PLANES; p++) acc_a[p] = acc_b[p] = 0;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const uint32_t va = (ql[k] & 0x0F0F0F0Fu) | ((qh[k] << sh_a) & 0x30303030u);
+        const uint32_t vb = ((ql[k] >> 4) & 0x0F0F0F0Fu) | ((qh[k] >> sh_b) & 0x30303030u);
+#pragma unroll
+        for (int p = 0; p < PLANES; p++) {
+            acc_a[p] = sdot4(va, xr[p][k], acc_a[p]);
+            acc_b[p] = sdot4(vb, xr[p][4 + k], acc_b[p]);
+        }
+    }
+    float fa = (float)acc_a[PLANES - 1], fb = (float)acc_b[PLANES - 1];
+#pragma unroll
+    for (int p = PLANES - 2; p >= 0; p--) {
+        fa = __builtin_fmaf(fa, 256.0f, (float)acc_a[p]);
+        fb = __builtin_fmaf(fb, 256.0f, (float)acc_b[p]);
+    }
+    fa = __builtin_fmaf(-32.0f, xm.z, fa);  // the stored quants are q + 32
+    fb = __builtin_fmaf(-32.0f, xm.w, fb);
+    const float sa = (float)((int)(t.sc[0] << sc_up) >> 24), sb = (float)((int)(t.sc[1] << sc_up) >> 24);  // the lane's two i8 scales
+    return f16_bits_to_f32(t.d) * __builtin_fmaf(sa * xm.x, fa, (sb * xm.y) * fb);
+}
+
+template <bool XF32, bool SINGLE>
+__global__ __launch_bounds__(1024) void k_qgemv_q6k_chunk(const uint8_t *__restrict__ W, const void *__restrict__ xg,
+                                                           float *__restrict__ y, int n_rows, int spr, int rows_per_wg,
+                                                           int rows_per_wave, int n_nominal, int red, int nthreads) {
+    extern __shared__ uint4 smem[];
+    const int slots = spr * 8;
+    const int n_waves = nthreads >> 6;
+    const int wave_id = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    uint32_t *stage = reinterpret_cast<uint32_t *>(smem) + wave_id * (kStageBytes / 4);  // this wave's row chunk
+    uint32_t *xd = reinterpret_cast<uint32_t *>(smem) + n_waves * (kStageBytes / 4);     // [kPlanes * 8][slots]
+    float *xm = reinterpret_cast<float *>(xd + kPlanes * 8 * slots);  // [slots][4]
+    float *part = xm + 4 * slots;                              // [group][n_nominal][part_stride]
+    const int ps = part_stride(slots, red);
+    const int lane = threadIdx.x & 63;
+    const int t = lane & 7, hh = t >> 2, tq = t & 3;
+    const int wave = wave_id;
+    const int ks = spr >> 3;
+    const int h = wave % ks, g = wave / ks;
+    const int wg_r0 = blockIdx.x * rows_per_wg;
+    const int wg_r1 = wg_r0 + rows_per_wg < n_rows ? wg_r0 + rows_per_wg : n_rows;
+    const int wave_r0 = wg_r0 + g * rows_per_wave;
+    const int wave_r1 = wave_r0 + rows_per_wave < wg_r1 ? wave_r0 + rows_per_wave : wg_r1;
+    const int nt_wave = wave_r1 > wave_r0 ? wave_r1 - wave_r0 : 0;  // real tasks of this wave (wave-uniform)
+
+    const uint32_t rowbytes = (uint32_t)spr * 210u;
+    // a wave's 105 pieces of a row chunk: lane l takes piece l, lanes 0..40 also piece 64 + l
+    const uint32_t off_a = (uint32_t)h * kChunkBytes + 16u * (uint32_t)lane;
+    const uint32_t off_b = (uint32_t)h * kChunkBytes + 1024u + 16u * (uint32_t)(lane < 41 ? lane : 40);
+    auto issue = [&](int i, u4v &a, u4v &b) {
+        const bool real = i < nt_wave;  // wave-uniform
+        const uint32_t ro = real ? (uint32_t)(wave_r0 + i) * rowbytes : 0u;
+        a = *reinterpret_cast<const u4v *>(W + (ro + (real ? off_a : 0u)));
+        b = *reinterpret_cast<const u4v *>(W + (ro + (real ? off_b : 0u)));
+    };
+
+    u4v ra[kDepth], rb[kDepth];
+#pragma unroll
+    for (int i = 0; i < kPre; i++) issue(i, ra[i], rb[i]);
+    stage_x<XF32>(xg, slots, nthreads, xd, xm);
+    __syncthreads();
+
+    const int slot = h * 64 + lane;
+    uint32_t xr[kPlanes][8];
+#pragma unroll
+    for (int p = 0; p < kPlanes; p++)
+#pragma unroll
+        for (int k = 0; k < 8; k++) xr[p][k] = xd[(p * 8 + k) * slots + slot];
+    const float4 xmr = *reinterpret_cast<const float4 *>(xm + 4 * slot);
+    const int ga = tq >> 1;
+    const int sh_a = 4 - 2 * ga, sh_b = 2 * ga;      // group ga: bits 2 ga of a qh byte -> bits 4..5; group ga + 2: bits 4 + 2 ga
+    const int sc_up = 24 - 8 * (2 * ga + (tq & 1));  // scale bytes 2 g + l / 16 of the half (word x for A, word y for B): shift to the top byte
+
+    // Super-block sb of the chunk starts at byte 210 sb: on a dword boundary for an even sb, two bytes past one for an
+    // odd sb.  Every piece is read from the dword boundary at or below it and shifted down by `mis` bytes.
+    const uint32_t mis = 2u * ((uint32_t)(lane >> 3) & 1u), sh = 8u * mis;
+    const uint32_t blk = (uint32_t)(lane >> 3) * 210u - mis;
+    const uint32_t *p_ql = stage + ((blk + 64u * hh + 16u * tq) >> 2);
+    const uint32_t *p_qh = stage + ((blk + 128u + 32u * hh + 16u * (tq & 1)) >> 2);
+    const uint32_t *p_sc = stage + ((blk + 192u + 8u * hh) >> 2);
+    const uint32_t *p_d = stage + ((blk + 208u) >> 2);
+
+    float *pp = part + (size_t)(g * n_nominal) * ps + slot;
+    auto consume = [&](int i, const u4v a, const u4v b) {
+        if (i < nt_wave) {  // wave-uniform
+            u4v *st4 = reinterpret_cast<u4v *>(stage);
+            st4[lane] = a;
+            if (lane < 41) st4[64 + lane] = b;
+            // LDS executes a wave's instructions in order: the reads below see the writes above, and the next row's
+            // writes come after these reads
+            uint32_t wl[5], wh[5], ws[3];
+#pragma unroll
+            for (int k = 0; k < 5; k++) wl[k] = p_ql[k], wh[k] = p_qh[k];
+#pragma unroll
+            for (int k = 0; k < 3; k++) ws[k] = p_sc[k];
+            Task tk;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                tk.ql[k] = __builtin_amdgcn_alignbit(wl[k + 1], wl[k], sh);
+                tk.qh[k] = __builtin_amdgcn_alignbit(wh[k + 1], wh[k], sh);
+            }
+            tk.sc[0] = __builtin_amdgcn_alignbit(ws[1], ws[0], sh);
+            tk.sc[1] = __builtin_amdgcn_alignbit(ws[2], ws[1], sh);
+            tk.d = (*p_d >> sh) & 0xFFFFu;
+            pp[(size_t)i * ps] = lane_dot<kPlanes>(tk, xr, xmr, sh_a, sh_b, sc_up);
+        }
+    };
+
+    int issued = kPre;
+#pragma unroll
+    for (int i = 0; i < kDepth; i++) {
+        consume(i, ra[i], rb[i]);
+        const int upto = SINGLE ? (kPre + 2 * (i + 1) < kDepth ? kPre + 2 * (i + 1) : kDepth)
+                                : (kPre + 2 * (i + 1) < kDepth + i + 1 ? kPre + 2 * (i + 1) : kDepth + i + 1);
+#pragma unroll
+        for (; issued < upto; issued++) issue(issued, ra[issued % kDepth], rb[issued % kDepth]);
+    }
+    if (!SINGLE) {
+        int base = kDepth;
+        for (; base + kDepth < n_nominal; base += kDepth) {
+#pragma unroll
+            for (int i = 0; i < kDepth; i++) {
+                consume(base + i, ra[i], rb[i]);
+                issue(base + kDepth + i, ra[i], rb[i]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kDepth; i++) consume(base + i, ra[i], rb[i]);
+    }
+    __syncthreads();
+
+    // Row totals: `red` lanes per row (a power of two from 8 to 64 that divides slots), lane p adding every
+    // red-th partial, then a sum over the lanes of the row.
+    const int wg_rows = wg_r1 - wg_r0;
+    const int per_thread = slots / red;
+    const int red_shift = 31 - __builtin_clz(red);
+    for (int idx0 = 0; idx0 < wg_rows * red; idx0 += nthreads) {
+        const int idx = idx0 + (int)threadIdx.x;
+        int rl = idx >> red_shift;
+        const bool ok = rl < wg_rows;
+        rl = ok ? rl : wg_rows - 1;
+        const int grp = rl / rows_per_wave, loc = rl - grp * rows_per_wave;
+        const int p = idx & (red - 1);
+        const float *src = part + (size_t)(grp * n_nominal + loc) * ps + p;
+        float t0 = 0.0f, t1 = 0.0f, t2 = 0.0f, t3 = 0.0f;
+        int i = 0;
+        for (; i + 8 <= per_thread; i += 8) {  // eight reads in flight
+            const float *q = src + (size_t)i * red;
+            const float a0 = q[0], a1 = q[red], a2 = q[2 * red], a3 = q[3 * red];
+            const float a4 = q[4 * red], a5 = q[5 * red], a6 = q[6 * red], a7 = q[7 * red];
+            t0 += a0 + a4, t1 += a1 + a5, t2 += a2 + a6, t3 += a3 + a7;
+        }
+        for (; i < per_thread; i++) t0 += src[(size_t)i * red];
+        const float sum = team_sum_rt((t0 + t1) + (t2 + t3), red);
+        if (ok && p == 0) y[wg_r0 + rl] = sum;
+    }
+}
+
+}  // namespace
+
+namespace pmh {
+
+// Runs the chunk kernel when the shape suits it and returns true; otherwise leaves *err untouched and returns
+// false (the caller falls back to the general Q6_K kernel).  Preconditions as for launch_qgemv.
+bool try_launch_qgemv_q6k_chunk(const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, float *y,
+                                hipStream_t s, hipError_t *err) {
+    const int spr = (int)(k / 256);
+    if (spr % 8) return false;
+    const int ks = spr / 8;
+    const uint64_t w_bytes = (uint64_t)n * (uint64_t)spr * 210u;
+    static const int64_t mode = gemv::tuning("PMETAL_HIP_GEMV_Q6K_KERNEL", 0);  // 0 = choose, 1 = chunk kernel, 2 = general kernel
+    if (mode == 2 || ks > 16 || w_bytes >= (1ull << 32)) return false;
+    if (mode == 0 && w_bytes < (12ull << 20)) return false;
+    const size_t slots = (size_t)spr * 8;
+    const size_t lds_x = slots * 4 * (kPlanes * 8) + slots * 16;
+    const int64_t want = gemv::compute_units();
+    int64_t n_wg = n < want ? n : want;
+    const int64_t rows_per_wg = (n + n_wg - 1) / n_wg;
+    n_wg = (n + rows_per_wg - 1) / rows_per_wg;
+    int64_t groups = 16 / ks;
+    if (groups > rows_per_wg) groups = rows_per_wg;
+    const int64_t rows_per_wave = (rows_per_wg + groups - 1) / groups;
+    groups = (rows_per_wg + rows_per_wave - 1) / rows_per_wave;
+    const int64_t n_nominal = rows_per_wave;
+    const int64_t threads = ks * groups * 64;
+    int red = 8;  // lanes per row in the final summation: as many as the workgroup has to spare, at most 64
+    while (red < 64 && rows_per_wg * red * 2 <= threads) red *= 2;
+    const size_t lds = (size_t)(threads / 64) * kStageBytes + lds_x + (size_t)groups * (size_t)n_nominal * part_stride((int)slots, red) * 4;
+    if (lds > 128 * 1024) return false;
+    const bool single = n_nominal <= kDepth;
+    const bool xf32 = x_dtype == kDtypeF32;
+    auto go = [&](auto kern) {
+        if (lds > 64 * 1024) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return e;
+        }
+        hipLaunchKernelGGL(kern, dim3((unsigned)n_wg), dim3((unsigned)threads), lds, s, w, x, y, (int)n, spr, (int)rows_per_wg,
+                           (int)rows_per_wave, (int)n_nominal, red, (int)threads);
+        return hipGetLastError();
+    };
+    if (xf32) *err = single ? go(k_qgemv_q6k_chunk<true, true>) : go(k_qgemv_q6k_chunk<true, false>);
+    else *err = single ? go(k_qgemv_q6k_chunk<false, true>) : go(k_qgemv_q6k_chunk<false, false>);
+    return true;
+}
+
+}  // namespace pmh

@@ -70,8 +70,9 @@ def test_qgemv_q4k_large_ragged_shapes(oracle, n, k, x_dtype):
         assert elem <= TOL and norm <= TOL
 
 
-# Large Q6_K matrices from random block bytes: ragged row counts, rows of 8 to 64 super-blocks, fewer rows than
-# compute units times waves; activations with large and tiny outliers and a run of zeros.
+# Q6_K matrices of 12 MiB and more whose rows are whole chunks of eight super-blocks (k a multiple of 2048) take the
+# kernel that stages rows through LDS: ragged row counts, rows of 1 to 8 chunks, fewer rows than compute units times
+# waves; activations with large and tiny outliers and a run of zeros (the fixed-point scale is per 16 elements).
 Q6K_BIG_CASES = [(6001, 4096), (14336, 4096), (4096, 14336), (30001, 2048), (500, 16384), (1900, 6144)]
 
 
