@@ -1,7 +1,7 @@
 // The reference's own unit tests for this path, restated against the C++ host mirror
 // (include/pmetal_gguf.hpp) so that they read like the originals:
 //   crates/pmetal-gguf/src/k_quants.rs:1334-1342 (block sizes), :1368-1383 (Q4K dequantize range),
-//   :1446-1465 and :1490-1509 (Q4K / Q6K round trips), crates/pmetal-gguf/src/dequant.rs:1016-1036 (Q8_0
+//   :1446-1465, :1490-1509, :1512-1553 (Q4K / Q6K / Q3K / Q2K round trips), crates/pmetal-gguf/src/dequant.rs:1016-1036 (Q8_0
 //   block structure), :1139-1150 (invalid size / shape), crates/pmetal/src/commands/quantize.rs:1561-1608
 //   (Q4_K_M recipe), crates/pmetal-gguf/src/dynamic.rs:789-800, :934-1018 (critical layers, KL metric, calibration).
 // Usage: test_reference_suite [--host-only]   (--host-only skips everything that needs a GPU)
@@ -120,6 +120,26 @@ static void test_roundtrips() {  // k_quants.rs:1446-1465, :1490-1509
         CHECK(bytes.size() == 210);
         const auto restored = dequantize(bytes, GgmlType::Q6K, {256});
         CHECK(rmse(original, restored) < 0.1f && max_err(original, restored) < 0.3f);
+    }
+    {  // k_quants.rs:1512-1531
+        const auto bytes = quantize(original, GgmlType::Q3K);
+        CHECK(bytes.size() == 110);
+        const auto restored = dequantize(bytes, GgmlType::Q3K, {256});
+        CHECK(rmse(original, restored) < 1.5f && max_err(original, restored) < 4.0f);
+        CHECK(rmse(original, restored) < 0.2f);  // what the format actually achieves on the ramp
+    }
+    {  // k_quants.rs:1534-1553
+        const auto bytes = quantize(original, GgmlType::Q2K);
+        CHECK(bytes.size() == 84);
+        const auto restored = dequantize(bytes, GgmlType::Q2K, {256});
+        CHECK(rmse(original, restored) < 1.0f && max_err(original, restored) < 2.0f);
+        CHECK(rmse(original, restored) < 0.3f);
+    }
+    {  // the Q5_K sibling of :1446-1465, in the order that inverts the quantizer's packing
+        const auto bytes = quantize(original, GgmlType::Q5K);
+        CHECK(bytes.size() == 176);
+        const auto restored = dequantize(bytes, GgmlType::Q5K, {256}, PMETAL_HIP_ORDER_GGML);
+        CHECK(rmse(original, restored) < 0.05f && max_err(original, restored) < 0.15f);
     }
     {
         const auto bytes = quantize(original, GgmlType::Q8_0);
