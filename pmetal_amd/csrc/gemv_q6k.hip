@@ -20,7 +20,9 @@
 //    wave's instructions in order, so the copy needs no barrier.
 //  * Lane partial sums go to LDS; after a barrier the workgroup adds up each of its rows and stores y.
 //
-// Smaller or oddly shaped matrices stay with the bf16 kernel in gemv.hip.
+//  * Rows of k / 256 super-blocks that are not whole chunks are handled by the RAGGED variant of the kernel (see there).
+//
+// Matrices below 12 MiB and rows shorter than one chunk stay with the bf16 kernel in gemv.hip.
 #include "gemv_common.hpp"
 #include "internal.hpp"
 
@@ -34,7 +36,7 @@ constexpr int kDepth = 6;  // tasks in flight per wave
 constexpr int kPre = 2;    // of which this many are requested before x is converted
 constexpr int kPlanes = 3;
 constexpr int kChunkBytes = 8 * 210;           // 1680 = 105 pieces of 16 bytes
-constexpr int kStageBytes = kChunkBytes + 16;  // the shifted reads of the last lanes reach one dword past the chunk
+constexpr int kStageBytes = kChunkBytes + 32;  // a chunk that starts up to 14 bytes into its first piece, plus one dword for the shifted reads
 
 __host__ __device__ constexpr int part_stride(int slots, int red) { return ((slots + 63) / 64) * 64 + (red & 63); }
 
@@ -46,15 +48,17 @@ __device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {
 // 16-element group.  Element e = 256 sb + 128 hh + 32 g + l belongs to lane t = 4 hh + 2 (g & 1) + l / 16 of its
 // super-block (slot 8 sb + t), sub-block s = g >> 1 of that lane, dword (l % 16) / 4.
 // xd[(plane * 8 + 4 s + dword) * slots + slot]: four digits; xm[slot] = (scale s = 0, scale s = 1, sum s = 0, sum s = 1).
+// Slots past the end of a row (its last chunk may hold fewer than eight super-blocks) get zero digits and a zero scale.
 template <bool XF32>
-__device__ __forceinline__ void stage_x(const void *__restrict__ xg, int slots, int nthreads, uint32_t *xd, float *xm) {
-    const int total = slots * 8;  // quads of four elements: k / 4
+__device__ __forceinline__ void stage_x(const void *__restrict__ xg, int slots, int k_quads, int nthreads, uint32_t *xd, float *xm) {
+    const int total = slots * 8;  // quads of four elements, padded to whole chunks; k_quads = k / 4 of them exist
     for (int idx0 = 0; idx0 < total; idx0 += nthreads) {
         const int idx = idx0 + (int)threadIdx.x;
         const bool live = idx < total;
         const int id = live ? idx : total - 1;
-        float v[4];
-        if (XF32) {
+        float v[4] = {0.f, 0.f, 0.f, 0.f};
+        if (id >= k_quads) {
+        } else if (XF32) {
             const float4 f = reinterpret_cast<const float4 *>(xg)[id];
             v[0] = f.x, v[1] = f.y, v[2] = f.z, v[3] = f.w;
         } else {
@@ -141,12 +145,17 @@ __device__ __forceinline__ float lane_dot(const Task &t, const uint32_t (&xr)[kP
     return f16_bits_to_f32(t.d) * __builtin_fmaf(sa * xm.x, fa, (sb * xm.y) * fb);
 }
 
-template <bool XF32, bool SINGLE>
+// RAGGED: rows that are not whole chunks (k / 256 not a multiple of 8).  Such rows start at any even address, so a
+// chunk starts `delta` bytes into its first 16-byte piece, delta and the odd / even position of the super-blocks
+// change from row to row, the last chunk of a row is short, and the last pieces of the tensor must not be passed.
+template <bool XF32, bool SINGLE, bool RAGGED>
 __global__ __launch_bounds__(1024) void k_qgemv_q6k_chunk(const uint8_t *__restrict__ W, const void *__restrict__ xg,
                                                            float *__restrict__ y, int n_rows, int spr, int rows_per_wg,
-                                                           int rows_per_wave, int n_nominal, int red, int nthreads) {
+                                                           int rows_per_wave, int n_nominal, int red, int nthreads,
+                                                           uint32_t w_last) {
     extern __shared__ uint4 smem[];
-    const int slots = spr * 8;
+    const int ks = (spr + 7) >> 3;
+    const int slots = ks * 64;
     const int n_waves = nthreads >> 6;
     const int wave_id = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     uint32_t *stage = reinterpret_cast<uint32_t *>(smem) + wave_id * (kStageBytes / 4);  // this wave's row chunk
@@ -157,7 +166,6 @@ __global__ __launch_bounds__(1024) void k_qgemv_q6k_chunk(const uint8_t *__restr
     const int lane = threadIdx.x & 63;
     const int t = lane & 7, hh = t >> 2, tq = t & 3;
     const int wave = wave_id;
-    const int ks = spr >> 3;
     const int h = wave % ks, g = wave / ks;
     const int wg_r0 = blockIdx.x * rows_per_wg;
     const int wg_r1 = wg_r0 + rows_per_wg < n_rows ? wg_r0 + rows_per_wg : n_rows;
@@ -166,20 +174,27 @@ __global__ __launch_bounds__(1024) void k_qgemv_q6k_chunk(const uint8_t *__restr
     const int nt_wave = wave_r1 > wave_r0 ? wave_r1 - wave_r0 : 0;  // real tasks of this wave (wave-uniform)
 
     const uint32_t rowbytes = (uint32_t)spr * 210u;
-    // a wave's 105 pieces of a row chunk: lane l takes piece l, lanes 0..40 also piece 64 + l
+    // a wave's 105 pieces of a row chunk (106 when the chunk may start inside a piece): lane l takes piece l, the first
+    // 41 (42) lanes also piece 64 + l
     const uint32_t off_a = (uint32_t)h * kChunkBytes + 16u * (uint32_t)lane;
-    const uint32_t off_b = (uint32_t)h * kChunkBytes + 1024u + 16u * (uint32_t)(lane < 41 ? lane : 40);
+    constexpr int kTail = RAGGED ? 42 : 41;  // lanes that take a second piece
+    const uint32_t off_b = (uint32_t)h * kChunkBytes + 1024u + 16u * (uint32_t)(lane < kTail ? lane : kTail - 1);
     auto issue = [&](int i, u4v &a, u4v &b) {
         const bool real = i < nt_wave;  // wave-uniform
         const uint32_t ro = real ? (uint32_t)(wave_r0 + i) * rowbytes : 0u;
-        a = *reinterpret_cast<const u4v *>(W + (ro + (real ? off_a : 0u)));
-        b = *reinterpret_cast<const u4v *>(W + (ro + (real ? off_b : 0u)));
+        uint32_t pa = ro + (real ? off_a : 0u), pb = ro + (real ? off_b : 0u);
+        if (RAGGED) {  // from the 16-byte boundary below the chunk, never past the piece that holds the tensor's last byte
+            pa = (pa & ~15u) < w_last ? (pa & ~15u) : w_last;
+            pb = (pb & ~15u) < w_last ? (pb & ~15u) : w_last;
+        }
+        a = *reinterpret_cast<const u4v *>(W + pa);
+        b = *reinterpret_cast<const u4v *>(W + pb);
     };
 
     u4v ra[kDepth], rb[kDepth];
 #pragma unroll
     for (int i = 0; i < kPre; i++) issue(i, ra[i], rb[i]);
-    stage_x<XF32>(xg, slots, nthreads, xd, xm);
+    stage_x<XF32>(xg, slots, spr * 64, nthreads, xd, xm);
     __syncthreads();
 
     const int slot = h * 64 + lane;
@@ -193,23 +208,25 @@ __global__ __launch_bounds__(1024) void k_qgemv_q6k_chunk(const uint8_t *__restr
     const int sh_a = 4 - 2 * ga, sh_b = 2 * ga;      // group ga: bits 2 ga of a qh byte -> bits 4..5; group ga + 2: bits 4 + 2 ga
     const int sc_up = 24 - 8 * (2 * ga + (tq & 1));  // scale bytes 2 g + l / 16 of the half (word x for A, word y for B): shift to the top byte
 
-    // Super-block sb of the chunk starts at byte 210 sb: on a dword boundary for an even sb, two bytes past one for an
-    // odd sb.  Every piece is read from the dword boundary at or below it and shifted down by `mis` bytes.
-    const uint32_t mis = 2u * ((uint32_t)(lane >> 3) & 1u), sh = 8u * mis;
-    const uint32_t blk = (uint32_t)(lane >> 3) * 210u - mis;
-    const uint32_t *p_ql = stage + ((blk + 64u * hh + 16u * tq) >> 2);
-    const uint32_t *p_qh = stage + ((blk + 128u + 32u * hh + 16u * (tq & 1)) >> 2);
-    const uint32_t *p_sc = stage + ((blk + 192u + 8u * hh) >> 2);
-    const uint32_t *p_d = stage + ((blk + 208u) >> 2);
+    // Super-block sb of the chunk starts at byte delta + 210 sb of the staged pieces (delta = 0 unless RAGGED): on a dword
+    // boundary or two bytes past one.  Every piece is read from the dword boundary at or below it and shifted down by
+    // `mis` bytes.
+    const uint32_t sb_byte = (uint32_t)(lane >> 3) * 210u;
+    const uint32_t c_ql = 16u * hh + 4u * tq, c_qh = 32u + 8u * hh + 4u * (tq & 1), c_sc = 48u + 2u * hh, c_d = 52u;  // dwords into the block
+    const bool lane_valid = !RAGGED || h * 8 + (lane >> 3) < spr;  // the last chunk of a ragged row is short
 
     float *pp = part + (size_t)(g * n_nominal) * ps + slot;
     auto consume = [&](int i, const u4v a, const u4v b) {
         if (i < nt_wave) {  // wave-uniform
             u4v *st4 = reinterpret_cast<u4v *>(stage);
             st4[lane] = a;
-            if (lane < 41) st4[64 + lane] = b;
+            if (lane < kTail) st4[64 + lane] = b;
             // LDS executes a wave's instructions in order: the reads below see the writes above, and the next row's
             // writes come after these reads
+            const uint32_t delta = RAGGED ? ((uint32_t)(wave_r0 + i) * rowbytes) & 15u : 0u;  // wave-uniform
+            const uint32_t t0 = delta + sb_byte, mis = t0 & 2u, sh = 8u * mis;
+            const uint32_t *blk = stage + ((t0 - mis) >> 2);
+            const uint32_t *p_ql = blk + c_ql, *p_qh = blk + c_qh, *p_sc = blk + c_sc;
             uint32_t wl[5], wh[5], ws[3];
 #pragma unroll
             for (int k = 0; k < 5; k++) wl[k] = p_ql[k], wh[k] = p_qh[k];
@@ -223,8 +240,9 @@ __global__ __launch_bounds__(1024) void k_qgemv_q6k_chunk(const uint8_t *__restr
             }
             tk.sc[0] = __builtin_amdgcn_alignbit(ws[1], ws[0], sh);
             tk.sc[1] = __builtin_amdgcn_alignbit(ws[2], ws[1], sh);
-            tk.d = (*p_d >> sh) & 0xFFFFu;
-            pp[(size_t)i * ps] = lane_dot<kPlanes>(tk, xr, xmr, sh_a, sh_b, sc_up);
+            tk.d = (blk[c_d] >> sh) & 0xFFFFu;
+            const float val = lane_dot<kPlanes>(tk, xr, xmr, sh_a, sh_b, sc_up);
+            pp[(size_t)i * ps] = lane_valid ? val : 0.0f;
         }
     };
 
@@ -287,13 +305,14 @@ namespace pmh {
 bool try_launch_qgemv_q6k_chunk(const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, float *y,
                                 hipStream_t s, hipError_t *err) {
     const int spr = (int)(k / 256);
-    if (spr % 8) return false;
-    const int ks = spr / 8;
+    if (spr < 8) return false;
+    const bool ragged = spr % 8 != 0;
+    const int ks = (spr + 7) / 8;
     const uint64_t w_bytes = (uint64_t)n * (uint64_t)spr * 210u;
     static const int64_t mode = gemv::tuning("PMETAL_HIP_GEMV_Q6K_KERNEL", 0);  // 0 = choose, 1 = chunk kernel, 2 = general kernel
     if (mode == 2 || ks > 16 || w_bytes >= (1ull << 32)) return false;
     if (mode == 0 && w_bytes < (12ull << 20)) return false;
-    const size_t slots = (size_t)spr * 8;
+    const size_t slots = (size_t)ks * 64;
     const size_t lds_x = slots * 4 * (kPlanes * 8) + slots * 16;
     const int64_t want = gemv::compute_units();
     int64_t n_wg = n < want ? n : want;
@@ -317,11 +336,16 @@ bool try_launch_qgemv_q6k_chunk(const uint8_t *w, int64_t n, int64_t k, const vo
             if (e != hipSuccess) return e;
         }
         hipLaunchKernelGGL(kern, dim3((unsigned)n_wg), dim3((unsigned)threads), lds, s, w, x, y, (int)n, spr, (int)rows_per_wg,
-                           (int)rows_per_wave, (int)n_nominal, red, (int)threads);
+                           (int)rows_per_wave, (int)n_nominal, red, (int)threads, (uint32_t)((w_bytes - 1) & ~(uint64_t)15));
         return hipGetLastError();
     };
-    if (xf32) *err = single ? go(k_qgemv_q6k_chunk<true, true>) : go(k_qgemv_q6k_chunk<true, false>);
-    else *err = single ? go(k_qgemv_q6k_chunk<false, true>) : go(k_qgemv_q6k_chunk<false, false>);
+    if (ragged) {
+        if (xf32) *err = single ? go(k_qgemv_q6k_chunk<true, true, true>) : go(k_qgemv_q6k_chunk<true, false, true>);
+        else *err = single ? go(k_qgemv_q6k_chunk<false, true, true>) : go(k_qgemv_q6k_chunk<false, false, true>);
+    } else {
+        if (xf32) *err = single ? go(k_qgemv_q6k_chunk<true, true, false>) : go(k_qgemv_q6k_chunk<true, false, false>);
+        else *err = single ? go(k_qgemv_q6k_chunk<false, true, false>) : go(k_qgemv_q6k_chunk<false, false, false>);
+    }
     return true;
 }
 

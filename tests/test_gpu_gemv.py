@@ -70,10 +70,12 @@ def test_qgemv_q4k_large_ragged_shapes(oracle, n, k, x_dtype):
         assert elem <= TOL and norm <= TOL
 
 
-# Q6_K matrices of 12 MiB and more whose rows are whole chunks of eight super-blocks (k a multiple of 2048) take the
-# kernel that stages rows through LDS: ragged row counts, rows of 1 to 8 chunks, fewer rows than compute units times
+# Q6_K matrices of 12 MiB and more with rows of at least eight super-blocks (k >= 2048) take the kernel that stages
+# rows through LDS: ragged row counts, rows of 1 to 8 chunks, fewer rows than compute units times
 # waves; activations with large and tiny outliers and a run of zeros (the fixed-point scale is per 16 elements).
-Q6K_BIG_CASES = [(6001, 4096), (14336, 4096), (4096, 14336), (30001, 2048), (500, 16384), (1900, 6144)]
+Q6K_BIG_CASES = [(6001, 4096), (14336, 4096), (4096, 14336), (30001, 2048), (500, 16384), (1900, 6144),
+                 # rows that are not whole chunks: 14, 43, 9 and 25 super-blocks (even and odd: rows start at any even address)
+                 (6001, 3584), (3001, 11008), (7001, 2304), (2049, 6400)]
 
 
 @pytest.mark.parametrize("n,k", Q6K_BIG_CASES)
