@@ -17,7 +17,9 @@
 //    W) so that the number of outstanding loads is known at every wait.  Lane partial sums go to LDS; after a barrier
 //    the workgroup adds up each of its rows and stores y.
 //
-// Smaller matrices, and rows that are not whole chunks, stay with the kernel in gemv.hip.
+//  * A row whose last chunk is short (k a multiple of 256 but not of 2048) is handled by the RAGGED variant (see there).
+//
+// Matrices below 12 MiB, rows shorter than one chunk and k that is not a multiple of 256 stay with the kernel in gemv.hip.
 #include "gemv_common.hpp"
 #include "internal.hpp"
 
@@ -41,15 +43,17 @@ __device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {
 
 // Activations -> LDS.  Thread idx converts elements 4 idx .. 4 idx + 3; eight consecutive threads hold one block.
 // xd[(plane * 8 + dword) * slots + block]: four digits; xm[block] = the block's scale.
+// Blocks past the end of a row (its last chunk may hold fewer than 64 blocks) get zero digits and a zero scale.
 template <bool XF32>
-__device__ __forceinline__ void stage_x(const void *__restrict__ xg, int slots, int nthreads, uint32_t *xd, float *xm) {
-    const int total = slots * 8;  // k / 4
+__device__ __forceinline__ void stage_x(const void *__restrict__ xg, int slots, int k_quads, int nthreads, uint32_t *xd, float *xm) {
+    const int total = slots * 8;  // quads of four elements, padded to whole chunks; k_quads = k / 4 of them exist
     for (int idx0 = 0; idx0 < total; idx0 += nthreads) {
         const int idx = idx0 + (int)threadIdx.x;
         const bool live = idx < total;
         const int id = live ? idx : total - 1;
-        float v[4];
-        if (XF32) {
+        float v[4] = {0.f, 0.f, 0.f, 0.f};
+        if (id >= k_quads) {
+        } else if (XF32) {
             const float4 f = reinterpret_cast<const float4 *>(xg)[id];
             v[0] = f.x, v[1] = f.y, v[2] = f.z, v[3] = f.w;
         } else {
@@ -93,12 +97,17 @@ __device__ __forceinline__ void stage_x(const void *__restrict__ xg, int slots, 
     }
 }
 
-template <bool XF32, bool SINGLE>
+// RAGGED: rows whose last chunk is short (k / 32 not a multiple of 64; k is a multiple of 256, so rows and chunks still
+// start on 16-byte boundaries).  The copy must not pass the tensor's last piece, and the lanes without a block
+// contribute zero.
+template <bool XF32, bool SINGLE, bool RAGGED>
 __global__ __launch_bounds__(1024) void k_qgemv_q8_0_chunk(const uint8_t *__restrict__ W, const void *__restrict__ xg,
                                                             float *__restrict__ y, int n_rows, int bpr, int rows_per_wg,
-                                                            int rows_per_wave, int n_nominal, int red, int nthreads) {
+                                                            int rows_per_wave, int n_nominal, int red, int nthreads,
+                                                            uint32_t w_last) {
     extern __shared__ uint4 smem[];
-    const int slots = bpr;
+    const int ks = (bpr + 63) >> 6;
+    const int slots = ks * 64;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int n_waves = nthreads >> 6;
@@ -107,7 +116,6 @@ __global__ __launch_bounds__(1024) void k_qgemv_q8_0_chunk(const uint8_t *__rest
     float *xm = reinterpret_cast<float *>(xd + kPlanes * 8 * slots);                  // [slots]
     float *part = xm + slots;                                                         // [group][n_nominal][part_stride]
     const int ps = part_stride(slots, red);
-    const int ks = bpr >> 6;
     const int h = wave % ks, g = wave / ks;
     const int wg_r0 = blockIdx.x * rows_per_wg;
     const int wg_r1 = wg_r0 + rows_per_wg < n_rows ? wg_r0 + rows_per_wg : n_rows;
@@ -122,15 +130,17 @@ __global__ __launch_bounds__(1024) void k_qgemv_q8_0_chunk(const uint8_t *__rest
     auto issue = [&](int i, u4v &a, u4v &b, u4v &c) {
         const bool real = i < nt_wave;  // wave-uniform
         const uint32_t ro = real ? (uint32_t)(wave_r0 + i) * rowbytes : 0u;
-        a = *reinterpret_cast<const u4v *>(W + (ro + (real ? off_a : 0u)));
-        b = *reinterpret_cast<const u4v *>(W + (ro + (real ? off_a + 1024u : 0u)));
-        c = *reinterpret_cast<const u4v *>(W + (ro + (real ? off_c : 0u)));
+        uint32_t pa = ro + (real ? off_a : 0u), pb = ro + (real ? off_a + 1024u : 0u), pc = ro + (real ? off_c : 0u);
+        if (RAGGED) pa = pa < w_last ? pa : w_last, pb = pb < w_last ? pb : w_last, pc = pc < w_last ? pc : w_last;
+        a = *reinterpret_cast<const u4v *>(W + pa);
+        b = *reinterpret_cast<const u4v *>(W + pb);
+        c = *reinterpret_cast<const u4v *>(W + pc);
     };
 
     u4v ra[kDepth], rb[kDepth], rc[kDepth];
 #pragma unroll
     for (int i = 0; i < kPre; i++) issue(i, ra[i], rb[i], rc[i]);
-    stage_x<XF32>(xg, slots, nthreads, xd, xm);
+    stage_x<XF32>(xg, slots, bpr * 8, nthreads, xd, xm);
     __syncthreads();
 
     const int slot = h * 64 + lane;
@@ -148,6 +158,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q8_0_chunk(const uint8_t *__rest
     const uint32_t *sp = stage + ((34 * lane) >> 2);       // the dword that holds the scale
     const uint32_t *qp = stage + ((34 * lane + 2) >> 2);   // the dword that holds the first quant
     const uint32_t d_shift = odd ? 16u : 0u, q_shift = odd ? 0u : 16u;
+    const bool lane_valid = !RAGGED || slot < bpr;  // the last chunk of a ragged row is short
 
     float *pp = part + (size_t)(g * n_nominal) * ps + slot;
     auto consume = [&](int i, const u4v a, const u4v b, const u4v c) {
@@ -172,7 +183,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q8_0_chunk(const uint8_t *__rest
         float f = (float)acc[kPlanes - 1];
 #pragma unroll
         for (int p = kPlanes - 2; p >= 0; p--) f = __builtin_fmaf(f, 256.0f, (float)acc[p]);
-        pp[(size_t)i * ps] = (f16_bits_to_f32((dw >> d_shift) & 0xFFFFu) * xscale) * f;
+        pp[(size_t)i * ps] = lane_valid ? (f16_bits_to_f32((dw >> d_shift) & 0xFFFFu) * xscale) * f : 0.0f;
         }
     };
 
@@ -235,13 +246,14 @@ namespace pmh {
 bool try_launch_qgemv_q8_0_chunk(const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, float *y,
                                  hipStream_t s, hipError_t *err) {
     const int bpr = (int)(k / 32);
-    if (bpr % 64) return false;
-    const int ks = bpr / 64;
+    if (bpr < 64 || bpr % 8) return false;  // rows of at least one chunk that start on 16-byte boundaries
+    const bool ragged = bpr % 64 != 0;
+    const int ks = (bpr + 63) / 64;
     const uint64_t w_bytes = (uint64_t)n * (uint64_t)bpr * 34u;
     static const int64_t mode = gemv::tuning("PMETAL_HIP_GEMV_Q8_0_KERNEL", 0);  // 0 = choose, 1 = this kernel, 2 = general kernel
     if (mode == 2 || ks > 16 || w_bytes >= (1ull << 32)) return false;
     if (mode == 0 && w_bytes < (12ull << 20)) return false;
-    const size_t slots = (size_t)bpr;
+    const size_t slots = (size_t)ks * 64;
     const int64_t want = gemv::compute_units();
     int64_t n_wg = n < want ? n : want;
     const int64_t rows_per_wg = (n + n_wg - 1) / n_wg;
@@ -265,11 +277,16 @@ bool try_launch_qgemv_q8_0_chunk(const uint8_t *w, int64_t n, int64_t k, const v
             if (e != hipSuccess) return e;
         }
         hipLaunchKernelGGL(kern, dim3((unsigned)n_wg), dim3((unsigned)threads), lds, s, w, x, y, (int)n, bpr, (int)rows_per_wg,
-                           (int)rows_per_wave, (int)n_nominal, red, (int)threads);
+                           (int)rows_per_wave, (int)n_nominal, red, (int)threads, (uint32_t)((w_bytes - 1) & ~(uint64_t)15));
         return hipGetLastError();
     };
-    if (xf32) *err = single ? go(k_qgemv_q8_0_chunk<true, true>) : go(k_qgemv_q8_0_chunk<true, false>);
-    else *err = single ? go(k_qgemv_q8_0_chunk<false, true>) : go(k_qgemv_q8_0_chunk<false, false>);
+    if (ragged) {
+        if (xf32) *err = single ? go(k_qgemv_q8_0_chunk<true, true, true>) : go(k_qgemv_q8_0_chunk<true, false, true>);
+        else *err = single ? go(k_qgemv_q8_0_chunk<false, true, true>) : go(k_qgemv_q8_0_chunk<false, false, true>);
+    } else {
+        if (xf32) *err = single ? go(k_qgemv_q8_0_chunk<true, true, false>) : go(k_qgemv_q8_0_chunk<true, false, false>);
+        else *err = single ? go(k_qgemv_q8_0_chunk<false, true, false>) : go(k_qgemv_q8_0_chunk<false, false, false>);
+    }
     return true;
 }
 

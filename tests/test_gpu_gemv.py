@@ -119,10 +119,12 @@ def test_qgemv_q6k_large_quantized_weights_and_linearity(oracle):
     assert np.isnan(gpu_qgemv(Q6K, wq, n, k, xa, pm.DTYPE_F32, 0)).all()
 
 
-# Q8_0 matrices of 12 MiB and more whose rows are whole chunks of 64 blocks (k a multiple of 2048) take the kernel that
+# Q8_0 matrices of 12 MiB and more with rows of at least 64 blocks (k >= 2048, a multiple of 256) take the kernel that
 # stages rows through LDS: ragged row counts, rows of 1, 2, 7 and 16 chunks, fewer rows than compute units times waves;
 # activations with large and tiny outliers and a run of zeros; quants over the whole int8 range.
-Q8_0_BIG_CASES = [(6001, 4096), (14336, 4096), (4096, 14336), (30001, 2048), (500, 32768), (1900, 6144)]
+Q8_0_BIG_CASES = [(6001, 4096), (14336, 4096), (4096, 14336), (30001, 2048), (500, 32768), (1900, 6144),
+                  # rows whose last chunk is short: 112, 344, 72 and 200 blocks
+                  (6001, 3584), (3001, 11008), (7001, 2304), (2049, 6400)]
 
 
 @pytest.mark.parametrize("n,k", Q8_0_BIG_CASES)
