@@ -39,7 +39,7 @@ extern "C" {
 #define PMETAL_GGML_TYPE_Q2K 10u /* quantize / dequantize only (k_quants.rs:1242-1321, :230-266); no linear kernels */
 #define PMETAL_GGML_TYPE_Q3K 11u /* quantize / dequantize only (k_quants.rs:1139-1237, :281-355); no linear kernels */
 #define PMETAL_GGML_TYPE_Q4K 12u
-#define PMETAL_GGML_TYPE_Q5K 13u /* quantize / dequantize only (k_quants.rs:960-1051, :407-462); no linear kernels */
+#define PMETAL_GGML_TYPE_Q5K 13u /* quantize / dequantize (k_quants.rs:960-1051, :407-462) and the fused GEMV; no fused GEMM */
 #define PMETAL_GGML_TYPE_Q6K 14u
 #define PMETAL_GGML_TYPE_Q8K 15u /* quantize / dequantize (k_quants.rs:815-871, :498-506) and the activation side of qgemv_q8k */
 

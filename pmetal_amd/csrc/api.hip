@@ -450,9 +450,11 @@ int32_t pmetal_hip_dequantize(uint32_t t, const uint8_t *src, size_t src_len, co
 }
 
 // ---- quantized linear ----
+// gemv_only: Q5_K has a fused GEMV but no fused GEMM
 static int32_t check_linear(uint32_t t, const void *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype,
-                            const void *y, uint32_t order) {
-    if (!path_type(t)) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "Unsupported quantization type: %u", t);
+                            const void *y, uint32_t order, bool gemv_only = false) {
+    if (!path_type(t) && !(gemv_only && t == PMETAL_GGML_TYPE_Q5K))
+        return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "Unsupported quantization type: %u", t);
     if (order > PMETAL_HIP_ORDER_GGML) return fail(PMETAL_HIP_ERR_INVALID_ARG, "order must be 0 (REF) or 1 (GGML)");
     if (x_dtype > PMETAL_HIP_DTYPE_BF16) return fail(PMETAL_HIP_ERR_INVALID_ARG, "x_dtype must be 0 (f32) or 1 (bf16)");
     if (n <= 0 || k <= 0) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "n and k must be positive (n=%lld, k=%lld)", (long long)n, (long long)k);
@@ -467,7 +469,7 @@ static int32_t check_linear(uint32_t t, const void *w, int64_t n, int64_t k, con
 
 int32_t pmetal_hip_qgemv(uint32_t t, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, float *y,
                          uint32_t order, void *stream) {
-    if (int32_t rc = check_linear(t, w, n, k, x, x_dtype, y, order)) return rc;
+    if (int32_t rc = check_linear(t, w, n, k, x, x_dtype, y, order, true)) return rc;
     hipError_t e = pmh::launch_qgemv(t, w, n, k, x, x_dtype, y, order, (hipStream_t)stream);
     if (e == hipErrorInvalidValue)
         return fail(PMETAL_HIP_ERR_SHAPE_TOO_LARGE, "k=%lld does not fit the activation staging buffer", (long long)k);
@@ -532,9 +534,10 @@ int32_t pmetal_hip_qlinear(uint32_t t, const uint8_t *w, int64_t n, int64_t k, c
                            void *y, uint32_t y_dtype, uint32_t order, void *stream) {
     if (m == 1 && y_dtype == PMETAL_HIP_DTYPE_F32)
         return pmetal_hip_qgemv(t, w, n, k, x, x_dtype, (float *)y, order, stream);
-    if (t == PMETAL_GGML_TYPE_Q8_0 && k % 256 != 0 && y_dtype == PMETAL_HIP_DTYPE_F32 && m > 1 && n > 0 && k > 0 && x && y) {
-        // The fused GEMM walks k in steps of 256; a Q8_0 row may be any multiple of 32: one fused GEMV per
-        // activation row then, back to back on the stream.
+    if (((t == PMETAL_GGML_TYPE_Q8_0 && k % 256 != 0) || t == PMETAL_GGML_TYPE_Q5K) && y_dtype == PMETAL_HIP_DTYPE_F32 && m > 1 && n > 0 &&
+        k > 0 && x && y) {
+        // The fused GEMM walks k in steps of 256, and a Q8_0 row may be any multiple of 32; Q5_K has no fused GEMM: one
+        // fused GEMV per activation row then, back to back on the stream.
         const size_t x_row = (size_t)k * (x_dtype == PMETAL_HIP_DTYPE_F32 ? 4 : 2);
         for (int64_t r = 0; r < m; r++) {
             const int32_t rc = pmetal_hip_qgemv(t, w, n, k, (const uint8_t *)x + (size_t)r * x_row, x_dtype,

@@ -133,8 +133,67 @@ def test_gpu_q5k_quantize_and_dequantize_bit_exact(oracle):
         x = weights(n, n)
         assert np.array_equal(pm.quantize(x, Q5K), oracle.quantize(Q5K, x))
         assert np.array_equal(pm.dequantize(oracle.quantize(Q5K, x), Q5K, [n]), oracle.dequantize(Q5K, oracle.quantize(Q5K, x), [n]))
-    # no linear kernels for Q5_K: the reference's error class, not a crash
+
+
+Q5K_GEMV_CASES = [(6144, 4096), (3072, 1024), (7, 256), (33, 1792), (1001, 2304), (6001, 3584), (301, 11008), (4096, 14336), (20, 32768)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n,k", Q5K_GEMV_CASES)
+def test_gpu_q5k_gemv_matches_dequantize_then_matmul(oracle, n, k):
+    """Fused Q5_K GEMV against the oracle's dequantize-then-matmul in f64, both element orders and both activation types:
+    the fused attn_qkv shape of an 8B-class model, small and ragged shapes (rows of 1 to 128 super-blocks, short last
+    chunks, fewer rows than compute units), random block bytes."""
+    import pmetal_amd as pm
+    from gpu_util import gpu_qgemv, rel_errors
+    pm.init(0)
+    rng = np.random.default_rng(n * 7 + k)
+    raw = rng.integers(0, 256, size=(n * (k // 256), 176), dtype=np.uint8)
+    raw[:, 0:4] = np.frombuffer(np.array([0.01, 0.02], np.float16).tobytes(), np.uint8)  # d, dmin small and finite
+    raw = raw.reshape(-1)
+    x = rng.standard_normal(k).astype(np.float32)
+    x[rng.integers(0, k, max(1, k // 300))] *= 1000.0
+    x[rng.integers(0, k, max(1, k // 300))] *= 1e-6
+    x[5:21] = 0.0
+    bits = oracle.f32_to_bf16_bits(x)
+    for x_dtype, x_dev, x_ref in ((pm.DTYPE_F32, x, x), (pm.DTYPE_BF16, bits, oracle.bf16_bits_to_f32(bits))):
+        for order in (0, 1):
+            want = oracle.qmatvec(Q5K, raw, n, k, x_ref, order=order)
+            got = gpu_qgemv(Q5K, raw, n, k, x_dev, x_dtype, order)
+            elem, norm = rel_errors(got, want)
+            assert elem <= 1e-3 and norm <= 1e-3, (n, k, x_dtype, order, elem, norm)
+
+
+@pytest.mark.gpu
+def test_gpu_q5k_gemv_unit_vectors_quantized_weights_and_linear(oracle):
+    import pmetal_amd as pm
+    from gpu_util import gpu_qgemv, rel_errors, weights
+    pm.init(0)
+    n, k = 300, 2048
+    wq = pm.quantize(weights(77, n * k, outliers=1e-3), Q5K)
+    for order in (0, 1):
+        w = oracle.dequantize(Q5K, wq, [n, k], order=order).reshape(n, k)
+        for j in list(range(0, 70)) + [255, 256, 511, 1023, 1024, 2047]:
+            x = np.zeros(k, np.float32)
+            x[j] = 1.0
+            got = gpu_qgemv(Q5K, wq, n, k, x, pm.DTYPE_F32, order)
+            assert np.allclose(got, w[:, j], rtol=1e-6, atol=1e-9), (order, j)
+    assert not gpu_qgemv(Q5K, wq, n, k, np.zeros(k, np.float32), pm.DTYPE_F32, 1).any()
+    x = np.random.default_rng(5).standard_normal(k).astype(np.float32)
+    x[100] = np.inf
+    assert np.isnan(gpu_qgemv(Q5K, wq, n, k, x, pm.DTYPE_F32, 1)).all()
+    # qlinear with several activation rows runs one fused GEMV per row (there is no fused Q5_K GEMM)
     lib = pm._lib.load()
-    buf = pm.DeviceBuffer(1 << 16)
-    assert lib.pmetal_hip_qgemv(Q5K, buf.ptr, 4, 256, buf.ptr, 1, buf.ptr, 0, None) == 2
+    m = 3
+    xs = np.random.default_rng(6).standard_normal((m, k)).astype(np.float32)
+    dw, dx, dy = pm.DeviceBuffer.from_host(wq), pm.DeviceBuffer.from_host(xs), pm.DeviceBuffer(4 * m * n)
+    pm.check(lib.pmetal_hip_qlinear(Q5K, dw.ptr, n, k, dx.ptr, pm.DTYPE_F32, m, dy.ptr, pm.DTYPE_F32, 1, None))
+    pm.check(lib.pmetal_hip_sync(None))
+    got = dy.to_host(np.float32).reshape(m, n)
+    for r in range(m):
+        want = oracle.qmatvec(Q5K, wq, n, k, xs[r], order=1)
+        elem, norm = rel_errors(got[r], want)
+        assert elem <= 1e-3 and norm <= 1e-3
+    # no fused GEMM for Q5_K: the reference's error class, not a crash
+    assert lib.pmetal_hip_qgemm(Q5K, dw.ptr, n, k, dx.ptr, pm.DTYPE_F32, m, dy.ptr, pm.DTYPE_F32, 1, None) == 2
     lib.pmetal_hip_clear_error()
