@@ -159,14 +159,17 @@ def cpu_baseline_gemm(t, m, n, k, budget_s=12.0):
             "sample": f"{reps} x (dequantize + matmul) of {mm} x {rows} x {k}, {dt:.1f} s"}
 
 
-def cpu_baseline_decode(pm, budget_s=15.0):
-    """Oracle: dequantize + f32 matvec, one thread, over the projections of the first two layers of the stack."""
+def cpu_baseline_decode(pm, model="qwen3_0.6b", budget_s=15.0):
+    """Oracle: dequantize + f32 matvec, one thread, over the projections of the first two layers of the stack (the first
+    layer's attention projections for the 8B shape, whose single layers take seconds on one core)."""
     from oracle import binding as oracle
     oracle.build()
-    lins = [l for l in qwen3_06b_linears(pm) if l[0].startswith(("blk.0.", "blk.1."))]
+    all_lins = qwen3_06b_linears(pm) if model == "qwen3_0.6b" else llama3_8b_linears(pm)
+    prefixes = ("blk.0.", "blk.1.") if model == "qwen3_0.6b" else ("blk.0.attn",)
+    lins = [l for l in all_lins if l[0].startswith(prefixes)]
     rng = np.random.default_rng(8)
     ws = [(t, oracle.quantize(t, (rng.standard_normal(n * k) * 0.02).astype(np.float32)), n, k) for _, n, k, t in lins]
-    xs = {k: oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(rng.standard_normal(k).astype(np.float32))) for k in (1024, 2048, 3072)}
+    xs = {k: oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(rng.standard_normal(k).astype(np.float32))) for k in sorted({l[2] for l in lins})}
     reps, t0 = 0, time.perf_counter()
     while time.perf_counter() - t0 < budget_s:
         for t, wq, n, k in ws:
@@ -174,9 +177,9 @@ def cpu_baseline_decode(pm, budget_s=15.0):
         reps += 1
     dt = time.perf_counter() - t0
     sample_bytes = sum(gemv_bytes(t, n, k, 2) for t, _, n, k in ws)
-    total_bytes = sum(gemv_bytes(t, n, k, 2) for _, n, k, t in qwen3_06b_linears(pm))
+    total_bytes = sum(gemv_bytes(t, n, k, 2) for _, n, k, t in all_lins)
     return {"value": round(reps / dt * sample_bytes / total_bytes, 4), "unit": "tokens/s", "cores": 1, "kind": "port",
-            "sample": f"{reps} x the 14 projections of layers 0-1 ({sample_bytes} of {total_bytes} weight bytes per token), "
+            "sample": f"{reps} x the {len(ws)} projections {' / '.join(prefixes)}* ({sample_bytes} of {total_bytes} weight bytes per token), "
                       f"scaled by bytes, {dt:.1f} s"}
 
 
@@ -190,8 +193,15 @@ def bench_gemv(args, n, k, t=Q4K, copies=16):
     for i in range(copies):
         descs[i] = _lib.LinearDesc(t, pm.DTYPE_BF16, 0, 0, n, k, ws[i].ptr, x.ptr, ys[i].ptr)
 
+    # One launch per matrix: consecutive descriptors name different (identical) activation buffers, because the batch entry
+    # point sends consecutive matrices that share x two to a launch where the kernel allows it.
+    x2 = pm.DeviceBuffer.from_host(bf16_bits(np.random.default_rng(1).standard_normal(k)))
+    solo = (_lib.LinearDesc * copies)()
+    for i in range(copies):
+        solo[i] = _lib.LinearDesc(t, pm.DTYPE_BF16, 0, 0, n, k, ws[i].ptr, (x if i % 2 == 0 else x2).ptr, ys[i].ptr)
+
     def step():
-        pm.check(lib.pmetal_hip_qgemv_batch(descs, copies, None))
+        pm.check(lib.pmetal_hip_qgemv_batch(solo, copies, None))
 
     ev_ms, wall_ms = timer.run(step, args.steps, args.warmup)
     launches = args.steps * copies
@@ -200,16 +210,21 @@ def bench_gemv(args, n, k, t=Q4K, copies=16):
     gbs = bytes_per_launch / (us_per_launch * 1e-6) / 1e9
 
     # same kernel with one weight tensor re-read from the last-level cache (reported, never `value`)
-    one = (_lib.LinearDesc * copies)(*[descs[0]] * copies)
+    one = (_lib.LinearDesc * copies)()
+    for i in range(copies):
+        one[i] = _lib.LinearDesc(t, pm.DTYPE_BF16, 0, 0, n, k, ws[0].ptr, (x if i % 2 == 0 else x2).ptr, ys[0].ptr)
     c_ms, _ = timer.run(lambda: pm.check(lib.pmetal_hip_qgemv_batch(one, copies, None)), args.steps, args.warmup)
     cached_gbs = bytes_per_launch / (c_ms * 1e-3 / launches) / 1e9
+    # all sixteen sharing one x (as gate / up do): two matrices per launch where the kernel allows it
+    b_ms, _ = timer.run(lambda: pm.check(lib.pmetal_hip_qgemv_batch(descs, copies, None)), args.steps, args.warmup)
     return {
         "value": gbs, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
                      "kernel": {Q4K: "k_qgemv_q4k_chunk", Q6K: "k_qgemv_q6k_chunk", Q8_0: "k_qgemv_q8_0_chunk", 13: "k_qgemv_q5k_chunk"}[t], "bytes_per_launch": bytes_per_launch,
                      "us_per_launch": round(us_per_launch, 3)},
-        "extra": {"cache_resident_GBps": round(cached_gbs, 1), "weight_copies": copies},
+        "extra": {"cache_resident_GBps": round(cached_gbs, 1), "weight_copies": copies,
+                  "batch_entry_us_per_matrix": round(b_ms * 1e3 / launches, 3)},
     }, (t, n, k)
 
 
@@ -403,14 +418,19 @@ def llama3_8b_tensors(pm):
     return out
 
 
-def bench_decode(args):
-    """All batch-1 linear projections of one token of a random-init Qwen3-0.6B-shaped stack (linears only)."""
+def llama3_8b_linears(pm):
+    """(gguf name, n, k, type) of every batch-1 projection of a Llama-3-8B-shaped decoder, Q4_K_M recipe."""
+    return [l for l in llama3_8b_tensors(pm) if l[0] != "token_embd.weight"]
+
+
+def bench_decode(args, model="qwen3_0.6b"):
+    """All batch-1 linear projections of one token of a random-init decoder stack of the given shape (linears only)."""
     pm, _lib, lib = load()
     timer = Timer(pm, lib)
-    lins = qwen3_06b_linears(pm)
+    lins = qwen3_06b_linears(pm) if model == "qwen3_0.6b" else llama3_8b_linears(pm)
     descs = (_lib.LinearDesc * len(lins))()
     keep, total_bytes = [], 0
-    xs = {k: pm.DeviceBuffer.from_host(bf16_bits(np.random.default_rng(k).standard_normal(k))) for k in (1024, 2048, 3072)}
+    xs = {k: pm.DeviceBuffer.from_host(bf16_bits(np.random.default_rng(k).standard_normal(k))) for k in sorted({l[2] for l in lins})}
     for i, (name, n, k, t) in enumerate(lins):
         w = device_weights(pm, lib, t, n * k, 3000 + i)
         y = pm.DeviceBuffer(4 * n)
@@ -438,7 +458,9 @@ def bench_decode(args):
     return {
         "value": tok_s, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "k_qgemv_q4k / k_qgemv_q6k (197 projections in 127 launches)",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "k_qgemv_q4k / k_qgemv_q6k (197 projections in 127 launches)" if model == "qwen3_0.6b"
+                     else "k_qgemv_q4k_chunk / k_qgemv_q6k_chunk (225 projections)",
                      "bytes_per_step": total_bytes},
         "extra": {"launches_per_token": len(lins), "q6k_tensors": sum(1 for l in lins if l[3] == Q6K),
                   "submission": "one recorded sequence per token", "eager_tokens_per_s": round(args.steps / (eager_ms * 1e-3), 1)},
@@ -500,6 +522,8 @@ WORKLOADS["calibrate_14336x4096"] = dict(kind="calibrate", n=14336, k=4096, unit
                                          metric="KL calibration GB/s of f32 evaluated (6 candidates, quantize + dequantize + score) @14336x4096")
 WORKLOADS["decode_qwen3_0.6b_q4km"] = dict(kind="decode", metric="Q4_K_M decode linears tokens/s (Qwen3-0.6B shape)", unit="tokens/s",
                                            dtype="bf16")
+WORKLOADS["decode_llama3_8b_q4km"] = dict(kind="decode", model="llama3_8b", metric="Q4_K_M decode linears tokens/s (Llama-3-8B shape)",
+                                          unit="tokens/s", dtype="bf16")
 WORKLOADS["quantize_llama3_8b_q4km"] = dict(kind="quantize", metric="f32->Q4_K_M quantize GB/s of f32 consumed (Llama-3-8B shape)",
                                             unit="GB/s", dtype="f32")
 WORKLOADS["dequantize_14336x4096"] = dict(kind="dequantize", n=14336, k=4096, unit="GB/s", dtype="f32",
@@ -530,7 +554,7 @@ def main():
     if wl["kind"] == "gemm":
         res, (t, n, k) = bench_gemm(args, wl["m"], wl["n"], wl["k"], wl["type"])
     elif wl["kind"] == "decode":
-        res, (t, n, k) = bench_decode(args)
+        res, (t, n, k) = bench_decode(args, wl.get("model", "qwen3_0.6b"))
     elif wl["kind"] == "quantize":
         res, (t, n, k) = bench_quantize(args)
     elif wl["kind"] == "dequantize":
@@ -551,10 +575,10 @@ def main():
                  else "synthetic: N(0,0.02) f32 weights generated and quantized on the device, x ~ N(0,1) bf16"),
         "config": {"workload": args.workload, "element_order": "GGML" if wl["kind"] == "calibrate" else "REF",
                    "step": {"gemm": "one GEMM launch (activation pre-pass + MFMA kernel)",
-                            "gemv": "16 back-to-back GEMVs over 16 distinct weight tensors (HBM-resident: 528 MB for Q4_K)",
+                            "gemv": "16 back-to-back GEMV launches over 16 distinct weight tensors (HBM-resident: 528 MB for Q4_K)",
                             "gemv_q8k": "16 x (activations f32 -> Q8_K, integer-dot GEMV) over 16 distinct weight tensors",
                             "calibrate": "one tensor resident in HBM: 6 candidates x (quantize, fused dequantize-and-score, f64 score read back)",
-                            "decode": "all 197 batch-1 projections of one token, back to back on one stream",
+                            "decode": "all batch-1 projections of one token (197 for Qwen3-0.6B, 225 for Llama-3-8B), back to back on one stream",
                             "dequantize": "two tensors of 14336 x 4096, blocks resident in HBM",
                             "quantize": "all 226 tensors of the model, f32 resident in HBM"}[wl["kind"]]},
         "roofline": res["roofline"], "extra": res["extra"],
@@ -583,7 +607,7 @@ def main():
         elif wl["kind"] == "dequantize":
             out["cpu_baseline"] = cpu_baseline_dequantize()
         else:
-            out["cpu_baseline"] = cpu_baseline_decode(load()[0])
+            out["cpu_baseline"] = cpu_baseline_decode(load()[0], wl.get("model", "qwen3_0.6b"))
     print(json.dumps(out), flush=True)
 
 

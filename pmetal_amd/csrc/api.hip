@@ -494,6 +494,24 @@ int32_t pmetal_hip_qgemv_batch(const pmetal_hip_linear_desc *descs, size_t count
             }
         }
         if (j - i < 2) {
+            // Two consecutive large Q4_K projections of the same activation vector (gate / up of a large model) share a
+            // launch of the large-matrix kernel.
+            if (i + 1 < count && d.ggml_type == PMETAL_GGML_TYPE_Q4K && d.k > 0 && d.k % 256 == 0 && d.n > 0 &&
+                !pmh::qgemv_q4k_groupable(d.n, d.k)) {
+                const pmetal_hip_linear_desc &e = descs[i + 1];
+                if (e.ggml_type == d.ggml_type && e.k == d.k && e.x_dev == d.x_dev && e.x_dtype == d.x_dtype && e.order == d.order &&
+                    e.n > 0 && !pmh::qgemv_q4k_groupable(e.n, e.k)) {
+                    if (int32_t rc = check_linear(d.ggml_type, d.w_dev, d.n, d.k, d.x_dev, d.x_dtype, d.y_dev, d.order)) return rc;
+                    if (int32_t rc = check_linear(e.ggml_type, e.w_dev, e.n, e.k, e.x_dev, e.x_dtype, e.y_dev, e.order)) return rc;
+                    const hipError_t err = pmh::launch_qgemv_q4k_pair(d.w_dev, d.n, d.y_dev, e.w_dev, e.n, e.y_dev, d.k, d.x_dev, d.x_dtype,
+                                                                      d.order, (hipStream_t)stream);
+                    if (err == hipSuccess) {
+                        i += 2;
+                        continue;
+                    }
+                    if (err != hipErrorNotSupported) return hip_fail(err, "paired qgemv kernel launch");
+                }
+            }
             if (int32_t rc = pmetal_hip_qgemv(d.ggml_type, d.w_dev, d.n, d.k, d.x_dev, d.x_dtype, d.y_dev, d.order, stream))
                 return rc;
             i++;

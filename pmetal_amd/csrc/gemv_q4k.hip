@@ -314,11 +314,21 @@ constexpr int kPre = 2;  // of which this many are requested before x is convert
 // those rows in different banks.
 __host__ __device__ constexpr int part_stride(int slots, int red) { return ((slots + 63) / 64) * 64 + (red & 63); }
 
-template <int ORDER, bool XF32, int T, bool SINGLE>
-__global__ __launch_bounds__(1024) void k_qgemv_q4k_chunk(const uint8_t *__restrict__ W, const void *__restrict__ xg,
-                                                           float *__restrict__ y, int n_rows, int spr,
-                                                           int rows_per_wg, int rows_per_wave, int n_nominal, int red,
-                                                           int nthreads) {
+template <int ORDER, bool XF32, int T, bool SINGLE, bool PAIR>
+__global__ __launch_bounds__(1024) void k_qgemv_q4k_chunk(const uint8_t *__restrict__ W0, const uint8_t *__restrict__ W1,
+                                                           const void *__restrict__ xg, int split_wg, int n_rows0, int n_rows1,
+                                                           int spr, int rows_per_wg, int rows_per_wave, int n_nominal, int red,
+                                                           int nthreads, float *__restrict__ y0, float *__restrict__ y1) {
+    // (the arguments needed before the first weight request come first: the leading 16 dwords of the kernel-argument
+    // segment are preloaded into scalar registers at wave launch)
+    // Two matrices that share k and the activation vector (the gate / up projections) can go through one launch:
+    // workgroups [0, split_wg) belong to the first, the others to the second (PAIR; otherwise W1, y1, n_rows1 and split_wg
+    // are not looked at).
+    const bool second = PAIR && (int)blockIdx.x >= split_wg;  // workgroup-uniform
+    const uint8_t *__restrict__ W = second ? W1 : W0;
+    float *__restrict__ y = second ? y1 : y0;
+    const int n_rows = second ? n_rows1 : n_rows0;
+    const int wg_index = second ? (int)blockIdx.x - split_wg : (int)blockIdx.x;
     constexpr int NDIG = XF32 ? 6 : 5;
     constexpr int SEG = T / 8;   // super-blocks a team covers
     constexpr int RPT = 64 / T;  // rows per task
@@ -333,7 +343,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q4k_chunk(const uint8_t *__restr
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int ks = spr / SEG;
     const int h = wave % ks, g = wave / ks;
-    const int wg_r0 = blockIdx.x * rows_per_wg;
+    const int wg_r0 = wg_index * rows_per_wg;
     const int wg_r1 = wg_r0 + rows_per_wg < n_rows ? wg_r0 + rows_per_wg : n_rows;
     const int wave_r0 = wg_r0 + g * rows_per_wave;
     const int wave_r1 = wave_r0 + rows_per_wave < wg_r1 ? wave_r0 + rows_per_wave : wg_r1;
@@ -554,12 +564,18 @@ hipError_t launch_with_lds(Kern kern, dim3 grid, dim3 block, size_t lds, hipStre
 
 template <int ORDER, bool XF32>
 hipError_t launch_chunk(int T, bool single, dim3 grid, dim3 block, size_t lds, hipStream_t s, const uint8_t *w,
-                        const void *x, float *y, int n, int spr, int rows_per_wg, int rows_per_wave, int n_nominal, int red) {
-#define PMH_GO(TT)                                                                                                  \
-    return single ? launch_with_lds(k_qgemv_q4k_chunk<ORDER, XF32, TT, true>, grid, block, lds, s, w, x, y, n, spr, \
-                                    rows_per_wg, rows_per_wave, n_nominal, red, (int)block.x)                       \
-                  : launch_with_lds(k_qgemv_q4k_chunk<ORDER, XF32, TT, false>, grid, block, lds, s, w, x, y, n, spr, \
-                                    rows_per_wg, rows_per_wave, n_nominal, red, (int)block.x)
+                        const void *x, float *y, int n, int spr, int rows_per_wg, int rows_per_wave, int n_nominal, int red,
+                        const uint8_t *w1, int split_wg, float *y1, int n1) {
+#define PMH_GO(TT)                                                                                                       \
+    if (n1 > 0)                                                                                                                    \
+        return single ? launch_with_lds(k_qgemv_q4k_chunk<ORDER, XF32, TT, true, true>, grid, block, lds, s, w, w1, x, split_wg, n, n1,  \
+                                        spr, rows_per_wg, rows_per_wave, n_nominal, red, (int)block.x, y, y1)                      \
+                      : launch_with_lds(k_qgemv_q4k_chunk<ORDER, XF32, TT, false, true>, grid, block, lds, s, w, w1, x, split_wg, n, n1, \
+                                        spr, rows_per_wg, rows_per_wave, n_nominal, red, (int)block.x, y, y1);                     \
+    return single ? launch_with_lds(k_qgemv_q4k_chunk<ORDER, XF32, TT, true, false>, grid, block, lds, s, w, w1, x, split_wg, n, n1,     \
+                                    spr, rows_per_wg, rows_per_wave, n_nominal, red, (int)block.x, y, y1)                          \
+                  : launch_with_lds(k_qgemv_q4k_chunk<ORDER, XF32, TT, false, false>, grid, block, lds, s, w, w1, x, split_wg, n, n1,    \
+                                    spr, rows_per_wg, rows_per_wave, n_nominal, red, (int)block.x, y, y1)
     switch (T) {
     case 8: PMH_GO(8);
     case 16: PMH_GO(16);
@@ -633,54 +649,76 @@ hipError_t launch_group_general(const uint8_t *const *w, const int64_t *n, float
 
 namespace pmh {
 
+// Kernel A over one matrix (n1 == 0) or two that share k, x and the element order.  hipErrorNotSupported when the shape
+// does not suit it: a row of more than 16 chunks, offsets beyond 32 bits, partial sums that do not fit in LDS.
+static hipError_t launch_kernel_a(const uint8_t *w0, int64_t n0, float *y0, const uint8_t *w1, int64_t n1, float *y1, int64_t k,
+                                  const void *x, bool xf32, uint32_t order, hipStream_t s) {
+    const int spr = (int)(k / 256);
+    const int T = 8 * gemv::pow2_divisor(spr, 8);
+    const size_t slots = (size_t)spr * 8;
+    const size_t lds_x = slots * 16 * (xf32 ? 6 : 5) + slots * 16;
+    // Workgroups own contiguous chunks of rows, one per compute unit (x is staged once per workgroup).
+    const int64_t n = n0 + n1, want = gemv::compute_units();
+    int64_t n_wg = n < want ? n : want;
+    const int64_t rows_per_wg = (n + n_wg - 1) / n_wg;
+    const int64_t wg0 = (n0 + rows_per_wg - 1) / rows_per_wg, wg1 = (n1 + rows_per_wg - 1) / rows_per_wg;
+    const dim3 grid((unsigned)(wg0 + wg1));
+    const int ks = spr / (T / 8), rpt = 64 / T;
+    const uint64_t w_max = (uint64_t)(n0 > n1 ? n0 : n1) * (uint64_t)spr * 144u;
+    if (ks > 16 || w_max >= (1ull << 32)) return hipErrorNotSupported;
+    int64_t groups = 16 / ks;
+    const int64_t max_groups = (rows_per_wg + rpt - 1) / rpt;
+    if (groups > max_groups) groups = max_groups;
+    const int64_t rows_per_wave = (rows_per_wg + groups - 1) / groups;
+    groups = (rows_per_wg + rows_per_wave - 1) / rows_per_wave;
+    const int64_t n_nominal = (rows_per_wave + rpt - 1) / rpt;
+    const int64_t threads = ks * groups * 64;
+    int red = 8;  // lanes per row in the final summation: as many as the workgroup has to spare, at most T
+    while (red < 64 && red * 2 <= T && rows_per_wg * red * 2 <= threads) red *= 2;
+    const size_t lds = lds_x + (size_t)groups * (size_t)n_nominal * rpt * part_stride((int)slots, red) * 4;
+    if (lds > 128 * 1024) return hipErrorNotSupported;
+    const dim3 block((unsigned)threads);
+    const bool single = n_nominal <= kDepth;
+    const int a_n = (int)n0, a_rpw = (int)rows_per_wg, a_rpv = (int)rows_per_wave, a_nn = (int)n_nominal;
+    const uint8_t *b_w = n1 ? w1 : w0;
+    float *b_y = n1 ? y1 : y0;
+    const int b_split = (int)wg0, b_n = (int)n1;
+    if (order == kOrderRef)
+        return xf32 ? launch_chunk<0, true>(T, single, grid, block, lds, s, w0, x, y0, a_n, spr, a_rpw, a_rpv, a_nn, red, b_w, b_split, b_y, b_n)
+                    : launch_chunk<0, false>(T, single, grid, block, lds, s, w0, x, y0, a_n, spr, a_rpw, a_rpv, a_nn, red, b_w, b_split, b_y, b_n);
+    return xf32 ? launch_chunk<1, true>(T, single, grid, block, lds, s, w0, x, y0, a_n, spr, a_rpw, a_rpv, a_nn, red, b_w, b_split, b_y, b_n)
+                : launch_chunk<1, false>(T, single, grid, block, lds, s, w0, x, y0, a_n, spr, a_rpw, a_rpv, a_nn, red, b_w, b_split, b_y, b_n);
+}
+
 // Preconditions as for launch_qgemv.  Returns hipErrorInvalidValue when x does not fit in LDS.
 hipError_t launch_qgemv_q4k(const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, float *y,
                             uint32_t order, hipStream_t s) {
     const bool xf32 = x_dtype == kDtypeF32;
     const int spr = (int)(k / 256);
-    const int T = 8 * gemv::pow2_divisor(spr, 8);
     const size_t slots = (size_t)spr * 8;
     const size_t lds_x = slots * 16 * (xf32 ? 6 : 5) + slots * 16;
     if (lds_x > gemv::kMaxLds) return hipErrorInvalidValue;
-
-    // Workgroups own contiguous chunks of rows, one per compute unit (x is staged once per
-    // workgroup).
-    const int64_t want = gemv::compute_units();
-    int64_t n_wg = n < want ? n : want;
-    const int64_t rows_per_wg = (n + n_wg - 1) / n_wg;
-    n_wg = (n + rows_per_wg - 1) / rows_per_wg;
-    const dim3 grid((unsigned)n_wg);
-
-    // Kernel A when a row is at most 16 chunks, offsets fit 32 bits, the partial sums fit in LDS and there is
-    // enough work per compute unit to pay for its second barrier (measured crossover: about 12 MiB of weights).
-    const int ks = spr / (T / 8), rpt = 64 / T;
+    // Kernel A when there is enough work per compute unit to pay for its second barrier (measured crossover: about
+    // 12 MiB of weights) and the shape suits it.
     const uint64_t w_bytes = (uint64_t)n * (uint64_t)spr * 144u;
     static const int64_t mode = gemv::tuning("PMETAL_HIP_GEMV_KERNEL", 0);  // 0 = choose, 1 = kernel A, 2 = kernel B
-    const bool want_a = mode == 1 || (mode == 0 && w_bytes >= (12ull << 20));
-    if (want_a && ks <= 16 && w_bytes < (1ull << 32)) {
-        int64_t groups = 16 / ks;
-        const int64_t max_groups = (rows_per_wg + rpt - 1) / rpt;
-        if (groups > max_groups) groups = max_groups;
-        const int64_t rows_per_wave = (rows_per_wg + groups - 1) / groups;
-        groups = (rows_per_wg + rows_per_wave - 1) / rows_per_wave;
-        const int64_t n_nominal = (rows_per_wave + rpt - 1) / rpt;
-        const int64_t threads = ks * groups * 64;
-        int red = 8;  // lanes per row in the final summation: as many as the workgroup has to spare, at most T
-        while (red < 64 && red * 2 <= T && rows_per_wg * red * 2 <= threads) red *= 2;
-        const size_t lds = lds_x + (size_t)groups * (size_t)n_nominal * rpt * part_stride((int)slots, red) * 4;
-        if (lds <= 128 * 1024) {
-            const dim3 block((unsigned)threads);
-            const bool single = n_nominal <= kDepth;
-            const int a_n = (int)n, a_rpw = (int)rows_per_wg, a_rpv = (int)rows_per_wave, a_nn = (int)n_nominal;
-            if (order == kOrderRef)
-                return xf32 ? launch_chunk<0, true>(T, single, grid, block, lds, s, w, x, y, a_n, spr, a_rpw, a_rpv, a_nn, red)
-                            : launch_chunk<0, false>(T, single, grid, block, lds, s, w, x, y, a_n, spr, a_rpw, a_rpv, a_nn, red);
-            return xf32 ? launch_chunk<1, true>(T, single, grid, block, lds, s, w, x, y, a_n, spr, a_rpw, a_rpv, a_nn, red)
-                        : launch_chunk<1, false>(T, single, grid, block, lds, s, w, x, y, a_n, spr, a_rpw, a_rpv, a_nn, red);
-        }
+    if (mode == 1 || (mode == 0 && w_bytes >= (12ull << 20))) {
+        const hipError_t e = launch_kernel_a(w, n, y, nullptr, 0, nullptr, k, x, xf32, order, s);
+        if (e != hipErrorNotSupported) return e;
     }
-
     return launch_group_general(&w, &n, &y, 1, k, x, xf32, order, s);
+}
+
+// Two matrices of kernel-A size that share k, x, x_dtype and the element order (the gate / up projections of a large
+// model) in one launch.  hipErrorNotSupported when the pair does not suit kernel A: the caller launches them one by one.
+hipError_t launch_qgemv_q4k_pair(const uint8_t *w0, int64_t n0, float *y0, const uint8_t *w1, int64_t n1, float *y1, int64_t k,
+                                 const void *x, uint32_t x_dtype, uint32_t order, hipStream_t s) {
+    const bool xf32 = x_dtype == kDtypeF32;
+    const size_t slots = (size_t)(k / 256) * 8;
+    if (slots * 16 * (xf32 ? 6 : 5) + slots * 16 > gemv::kMaxLds) return hipErrorNotSupported;
+    static const int64_t mode = gemv::tuning("PMETAL_HIP_GEMV_KERNEL", 0);
+    if (mode == 2) return hipErrorNotSupported;
+    return launch_kernel_a(w0, n0, y0, w1, n1, y1, k, x, xf32, order, s);
 }
 
 // Matrices that kernel A would not take anyway (small ones), sharing k, x, x_dtype and order, in one launch.

@@ -44,6 +44,10 @@ bool try_launch_qgemv_q8_0_chunk(const uint8_t *w, int64_t n, int64_t k, const v
 hipError_t launch_qgemv_q4k(const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, float *y,
                             uint32_t order, hipStream_t s);
 // Several small Q4_K matrices with the same k, x, x_dtype and order in one launch (count <= kMaxGemvGroup);
+// launch_qgemv_q4k_pair: two large matrices (not groupable) that share k, x and the element order in one launch of the
+// large-matrix kernel; hipErrorNotSupported when the pair does not suit it.
+hipError_t launch_qgemv_q4k_pair(const uint8_t *w0, int64_t n0, float *y0, const uint8_t *w1, int64_t n1, float *y1, int64_t k,
+                                 const void *x, uint32_t x_dtype, uint32_t order, hipStream_t s);
 // qgemv_q4k_groupable tells whether a matrix is small enough to go into a group.
 bool qgemv_q4k_groupable(int64_t n, int64_t k);
 hipError_t launch_qgemv_q4k_group(const uint8_t *const *w, const int64_t *n, float *const *y, int count, int64_t k,

@@ -261,6 +261,43 @@ def test_qgemv_batch_groups_projections_of_one_activation(oracle, order):
         assert np.array_equal(dy.to_host(np.float32), single)
 
 
+@pytest.mark.parametrize("order", [0, 1])
+def test_qgemv_batch_pairs_large_projections_of_one_activation(oracle, order):
+    """Two consecutive large Q4_K matrices that share x (gate / up) go through one launch of the large-matrix kernel:
+    the results of one by one launches, also with different and ragged row counts, followed by an unrelated third matrix."""
+    from pmetal_amd import _lib
+    lib = _lib.load()
+    k = 4096
+    rows = [6001, 7301, 6500]
+    rng = np.random.default_rng(17)
+    bits = oracle.f32_to_bf16_bits(rng.standard_normal(k).astype(np.float32))
+    other = oracle.f32_to_bf16_bits(rng.standard_normal(k).astype(np.float32))
+    dx, dx2 = pm.DeviceBuffer.from_host(bits), pm.DeviceBuffer.from_host(other)
+    xs_of = [dx, dx, dx2]
+    descs = (_lib.LinearDesc * len(rows))()
+    keep, singles = [], []
+    for i, n in enumerate(rows):
+        raw = rng.integers(0, 256, size=(n * (k // 256), 144), dtype=np.uint8)
+        raw[:, 0:4] = np.frombuffer(np.array([0.01, 0.02], np.float16).tobytes(), np.uint8)
+        raw = raw.reshape(-1)
+        dw, dy = pm.DeviceBuffer.from_host(raw), pm.DeviceBuffer(4 * n)
+        pm.check(lib.pmetal_hip_memset(dy.ptr, 0xFF, 4 * n, None))
+        keep.append((dw, dy))
+        descs[i] = _lib.LinearDesc(Q4K, pm.DTYPE_BF16, order, 0, n, k, dw.ptr, xs_of[i].ptr, dy.ptr)
+        singles.append(gpu_qgemv(Q4K, raw, n, k, bits if xs_of[i] is dx else other, pm.DTYPE_BF16, order))
+        if i == 0:
+            want = oracle.qmatvec(Q4K, raw, n, k, oracle.bf16_bits_to_f32(bits), order=order)
+            elem, norm = rel_errors(singles[0], want)
+            assert elem <= TOL and norm <= TOL
+    pm.check(lib.pmetal_hip_qgemv_batch(descs, len(rows), None))
+    pm.check(lib.pmetal_hip_sync(None))
+    for (dw, dy), single in zip(keep, singles):
+        # the shared launch divides the rows among workgroups differently, so the lanes that add up a row differ: equal up
+        # to the order of the f32 partial sums
+        got = dy.to_host(np.float32)
+        assert np.abs(got - single).max() <= 2e-6 * np.abs(single).max()
+
+
 def test_qgemv_argument_errors():
     from pmetal_amd import _lib
     lib = _lib.load()
