@@ -13,7 +13,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)
 sys.path.insert(0, ROOT)
 from oracle import binding as ob  # noqa: E402
 
-TYPES = {"q8_0": 8, "q4k": 12, "q6k": 14}
+TYPES = {"q8_0": 8, "q4k": 12, "q6k": 14, "q5k": 13, "q3k": 11, "q2k": 10, "q8k": 15}
+TWO_ORDERS = (12, 13)  # Q4_K and Q5_K: the reference dequantizer's order and the inverse of the packing
 
 
 def inputs():
@@ -37,7 +38,7 @@ def main():
         q = ob.quantize(t, x)
         out[name + "_bytes"] = q
         out[name + "_deq"] = ob.dequantize(t, q, [x.size]).view(np.uint32)
-        if t == 12:
+        if t in TWO_ORDERS:
             out[name + "_deq_ggml"] = ob.dequantize(t, q, [x.size], order=1).view(np.uint32)
     np.savez_compressed(os.path.join(ROOT, "tests", "golden", "blocks.npz"), **out)
     print({k: v.shape for k, v in out.items()})

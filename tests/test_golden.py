@@ -6,7 +6,8 @@ import numpy as np
 import pytest
 
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "blocks.npz")
-TYPES = {"q8_0": 8, "q4k": 12, "q6k": 14}
+TYPES = {"q8_0": 8, "q4k": 12, "q6k": 14, "q5k": 13, "q3k": 11, "q2k": 10, "q8k": 15}
+TWO_ORDERS = (12, 13)
 
 
 @pytest.fixture(scope="module")
@@ -20,9 +21,9 @@ def test_oracle_reproduces_golden(oracle, gold, name):
     q = oracle.quantize(t, gold["x"])
     assert np.array_equal(q, gold[name + "_bytes"])
     assert np.array_equal(oracle.dequantize(t, q, [gold["x"].size]).view(np.uint32), gold[name + "_deq"])
-    if t == 12:
+    if t in TWO_ORDERS:
         got = oracle.dequantize(t, q, [gold["x"].size], order=1).view(np.uint32)
-        assert np.array_equal(got, gold["q4k_deq_ggml"])
+        assert np.array_equal(got, gold[name + "_deq_ggml"])
 
 
 def test_golden_zero_superblock(gold):
@@ -41,5 +42,5 @@ def test_hip_reproduces_golden(gold, name):
     q = gpu_quantize_dev(t, gold["x"])
     assert np.array_equal(q, gold[name + "_bytes"])
     assert np.array_equal(gpu_dequantize_dev(t, q, gold["x"].size).view(np.uint32), gold[name + "_deq"])
-    if t == 12:
-        assert np.array_equal(gpu_dequantize_dev(t, q, gold["x"].size, order=1).view(np.uint32), gold["q4k_deq_ggml"])
+    if t in TWO_ORDERS:
+        assert np.array_equal(gpu_dequantize_dev(t, q, gold["x"].size, order=1).view(np.uint32), gold[name + "_deq_ggml"])
