@@ -84,7 +84,7 @@ def bf16_bits(x):
 
 
 def gemv_bytes(t, n, k, x_bytes):
-    per_block = {Q8_0: (34, 32), Q4K: (144, 256), Q6K: (210, 256), 13: (176, 256)}[t]
+    per_block = {Q8_0: (34, 32), Q4K: (144, 256), Q6K: (210, 256), 13: (176, 256), 11: (110, 256), 10: (84, 256)}[t]
     return n * (k // per_block[1]) * per_block[0] + k * x_bytes + n * 4
 
 
@@ -221,7 +221,7 @@ def bench_gemv(args, n, k, t=Q4K, copies=16):
         "value": gbs, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": {Q4K: "k_qgemv_q4k_chunk", Q6K: "k_qgemv_q6k_chunk", Q8_0: "k_qgemv_q8_0_chunk", 13: "k_qgemv_q5k_chunk"}[t], "bytes_per_launch": bytes_per_launch,
+                     "kernel": {Q4K: "k_qgemv_q4k_chunk", Q6K: "k_qgemv_q6k_chunk", Q8_0: "k_qgemv_q8_0_chunk", 13: "k_qgemv_q5k_chunk", 11: "k_qgemv_q23k_chunk<FormatQ3K>", 10: "k_qgemv_q23k_chunk<FormatQ2K>"}[t], "bytes_per_launch": bytes_per_launch,
                      "us_per_launch": round(us_per_launch, 3)},
         "extra": {"cache_resident_GBps": round(cached_gbs, 1), "weight_copies": copies,
                   "batch_entry_us_per_matrix": round(b_ms * 1e3 / launches, 3)},
@@ -511,6 +511,8 @@ WORKLOADS = {
                                 dtype="bf16"),
 }
 WORKLOADS["gemv_q6k_14336x4096"] = dict(kind="gemv", n=14336, k=4096, type=Q6K, metric="Q6_K GEMV GB/s @14336x4096", unit="GB/s", dtype="bf16")
+WORKLOADS["gemv_q3k_14336x4096"] = dict(kind="gemv", n=14336, k=4096, type=11, metric="Q3_K GEMV GB/s @14336x4096", unit="GB/s", dtype="bf16")
+WORKLOADS["gemv_q2k_14336x4096"] = dict(kind="gemv", n=14336, k=4096, type=10, metric="Q2_K GEMV GB/s @14336x4096", unit="GB/s", dtype="bf16")
 WORKLOADS["gemv_q5k_6144x4096"] = dict(kind="gemv", n=6144, k=4096, type=13, metric="Q5_K GEMV GB/s @6144x4096 (fused attn_qkv)", unit="GB/s", dtype="bf16")
 WORKLOADS["gemv_q6k_18944x3584"] = dict(kind="gemv", n=18944, k=3584, type=Q6K, metric="Q6_K GEMV GB/s @18944x3584", unit="GB/s", dtype="bf16")
 WORKLOADS["gemv_q8_0_14336x4096"] = dict(kind="gemv", n=14336, k=4096, type=Q8_0, metric="Q8_0 GEMV GB/s @14336x4096", unit="GB/s", dtype="bf16")

@@ -14,7 +14,8 @@
  *  - Ownership: the caller owns every buffer it passes and every device allocation
  *    it requested; the library keeps no caller pointer after a call returns.
  *  - Device pointers must be 16-byte aligned (hipMalloc and torch allocations are;
- *    GGUF tensor data is 32-byte aligned in the file).
+ *    GGUF tensor data is 32-byte aligned in the file).  One exception: the output of
+ *    pmetal_hip_qgemv needs 4-byte alignment only, so that it can be a row of an [m, n] matrix.
  *  - `stream` is a hipStream_t passed as void*; NULL is the default stream.  Device
  *    entry points are asynchronous on that stream; host-pointer entry points
  *    synchronise before returning.
@@ -36,8 +37,8 @@ extern "C" {
 #define PMETAL_GGML_TYPE_F32 0u
 #define PMETAL_GGML_TYPE_F16 1u
 #define PMETAL_GGML_TYPE_Q8_0 8u
-#define PMETAL_GGML_TYPE_Q2K 10u /* quantize / dequantize only (k_quants.rs:1242-1321, :230-266); no linear kernels */
-#define PMETAL_GGML_TYPE_Q3K 11u /* quantize / dequantize only (k_quants.rs:1139-1237, :281-355); no linear kernels */
+#define PMETAL_GGML_TYPE_Q2K 10u /* quantize / dequantize (k_quants.rs:1242-1321, :230-266) and the fused GEMV; no fused GEMM */
+#define PMETAL_GGML_TYPE_Q3K 11u /* quantize / dequantize (k_quants.rs:1139-1237, :281-355) and the fused GEMV; no fused GEMM */
 #define PMETAL_GGML_TYPE_Q4K 12u
 #define PMETAL_GGML_TYPE_Q5K 13u /* quantize / dequantize (k_quants.rs:960-1051, :407-462) and the fused GEMV; no fused GEMM */
 #define PMETAL_GGML_TYPE_Q6K 14u

@@ -1224,6 +1224,8 @@ static int32_t dequant_row(uint32_t t, const uint8_t *w, size_t row, size_t k, f
     if (t == PMO_TYPE_Q8_0) pmo_dequantize_q8_0(w + row * row_bytes, k, tmp);
     else if (t == PMO_TYPE_Q4K) pmo_dequantize_q4k(w + row * row_bytes, k, tmp, order);
     else if (t == PMO_TYPE_Q5K) pmo_dequantize_q5k(w + row * row_bytes, k, tmp, order);
+    else if (t == PMO_TYPE_Q2K) pmo_dequantize_q2k(w + row * row_bytes, k, tmp);
+    else if (t == PMO_TYPE_Q3K) pmo_dequantize_q3k(w + row * row_bytes, k, tmp);
     else if (t == PMO_TYPE_Q6K) pmo_dequantize_q6k(w + row * row_bytes, k, tmp);
     else return PMO_ERR_UNSUPPORTED_TYPE;
     return PMO_OK;

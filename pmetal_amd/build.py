@@ -29,6 +29,7 @@ EXTRA = {
     # in front of the first load of these latency-bound kernels)
     "gemv.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
     "gemv_q4k.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
+    "gemv_q23k.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
     "gemv_q5k.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
     "gemv_q6k.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
     "gemv_q8_0.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],

@@ -450,10 +450,12 @@ int32_t pmetal_hip_dequantize(uint32_t t, const uint8_t *src, size_t src_len, co
 }
 
 // ---- quantized linear ----
-// gemv_only: Q5_K has a fused GEMV but no fused GEMM
+// types with a fused GEMV but no fused GEMM
+static bool gemv_only_type(uint32_t t) { return t == PMETAL_GGML_TYPE_Q5K || t == PMETAL_GGML_TYPE_Q3K || t == PMETAL_GGML_TYPE_Q2K; }
+
 static int32_t check_linear(uint32_t t, const void *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype,
                             const void *y, uint32_t order, bool gemv_only = false) {
-    if (!path_type(t) && !(gemv_only && t == PMETAL_GGML_TYPE_Q5K))
+    if (!path_type(t) && !(gemv_only && gemv_only_type(t)))
         return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "Unsupported quantization type: %u", t);
     if (order > PMETAL_HIP_ORDER_GGML) return fail(PMETAL_HIP_ERR_INVALID_ARG, "order must be 0 (REF) or 1 (GGML)");
     if (x_dtype > PMETAL_HIP_DTYPE_BF16) return fail(PMETAL_HIP_ERR_INVALID_ARG, "x_dtype must be 0 (f32) or 1 (bf16)");
@@ -462,7 +464,9 @@ static int32_t check_linear(uint32_t t, const void *w, int64_t n, int64_t k, con
     if (k % bs != 0) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "k=%lld is not a multiple of the block size %lld", (long long)k, (long long)bs);
     if (n > 0x7FFFFFFF || k / bs > 0x7FFFFFF) return fail(PMETAL_HIP_ERR_SHAPE_TOO_LARGE, "n or k too large");
     if (!w || !x || !y) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
-    if (!aligned16(w) || !aligned16(x) || !aligned16(y))
+    // the GEMV kernels store y one float at a time (so that the rows of an [m, n] output can be written one GEMV each);
+    // the GEMM stores 16-byte vectors
+    if (!aligned16(w) || !aligned16(x) || (gemv_only ? (reinterpret_cast<uintptr_t>(y) & 3u) != 0 : !aligned16(y)))
         return fail(PMETAL_HIP_ERR_INVALID_ARG, "device pointers must be 16-byte aligned");
     return require_device();
 }
@@ -552,9 +556,9 @@ int32_t pmetal_hip_qlinear(uint32_t t, const uint8_t *w, int64_t n, int64_t k, c
                            void *y, uint32_t y_dtype, uint32_t order, void *stream) {
     if (m == 1 && y_dtype == PMETAL_HIP_DTYPE_F32)
         return pmetal_hip_qgemv(t, w, n, k, x, x_dtype, (float *)y, order, stream);
-    if (((t == PMETAL_GGML_TYPE_Q8_0 && k % 256 != 0) || t == PMETAL_GGML_TYPE_Q5K) && y_dtype == PMETAL_HIP_DTYPE_F32 && m > 1 && n > 0 &&
+    if (((t == PMETAL_GGML_TYPE_Q8_0 && k % 256 != 0) || gemv_only_type(t)) && y_dtype == PMETAL_HIP_DTYPE_F32 && m > 1 && n > 0 &&
         k > 0 && x && y) {
-        // The fused GEMM walks k in steps of 256, and a Q8_0 row may be any multiple of 32; Q5_K has no fused GEMM: one
+        // The fused GEMM walks k in steps of 256, and a Q8_0 row may be any multiple of 32; Q5_K, Q3_K and Q2_K have no fused GEMM: one
         // fused GEMV per activation row then, back to back on the stream.
         const size_t x_row = (size_t)k * (x_dtype == PMETAL_HIP_DTYPE_F32 ? 4 : 2);
         for (int64_t r = 0; r < m; r++) {

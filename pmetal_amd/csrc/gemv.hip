@@ -389,6 +389,8 @@ hipError_t launch_qgemv(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
     const int planes = xf32 ? 3 : 1;
     if (type == kTypeQ4K) return launch_qgemv_q4k(w, n, k, x, x_dtype, y, order, s);
     if (type == kTypeQ5K) return launch_qgemv_q5k(w, n, k, x, x_dtype, y, order, s);
+    if (type == kTypeQ2K) return launch_qgemv_q2k(w, n, k, x, x_dtype, y, s);
+    if (type == kTypeQ3K) return launch_qgemv_q3k(w, n, k, x, x_dtype, y, s);
     if (type == kTypeQ6K) {
         hipError_t chunk_err = hipSuccess;
         if (try_launch_qgemv_q6k_chunk(w, n, k, x, x_dtype, y, s, &chunk_err)) return chunk_err;

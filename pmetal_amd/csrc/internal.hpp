@@ -35,6 +35,9 @@ constexpr int kMaxGemvGroup = 4;
 // gemv_q5k.hip: the Q5_K GEMV (every shape with k a multiple of 256 that fits; hipErrorInvalidValue otherwise)
 hipError_t launch_qgemv_q5k(const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, float *y, uint32_t order,
                             hipStream_t s);
+// gemv_q23k.hip: the Q2_K and Q3_K GEMVs (every shape with k a multiple of 256 that fits; hipErrorInvalidValue otherwise)
+hipError_t launch_qgemv_q2k(const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, float *y, hipStream_t s);
+hipError_t launch_qgemv_q3k(const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, float *y, hipStream_t s);
 // gemv_q6k.hip: the row-staging integer-dot kernel for large Q6_K matrices; false when the shape does not suit it
 bool try_launch_qgemv_q6k_chunk(const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, float *y,
                                 hipStream_t s, hipError_t *err);

@@ -203,8 +203,70 @@ def test_gpu_q2k_q3k_quantize_and_dequantize_bit_exact(oracle):
             x = weights(n, n)
             assert np.array_equal(pm.quantize(x, t), oracle.quantize(t, x))
             assert np.array_equal(pm.dequantize(oracle.quantize(t, x), t, [n]), oracle.dequantize(t, oracle.quantize(t, x), [n]))
-        # no linear kernels: the reference's error class, not a crash
-        lib = pm._lib.load()
-        buf = pm.DeviceBuffer(1 << 16)
-        assert lib.pmetal_hip_qgemv(t, buf.ptr, 4, 256, buf.ptr, 1, buf.ptr, 0, None) == 2
-        lib.pmetal_hip_clear_error()
+
+
+GEMV_CASES = [(6144, 4096), (3072, 1024), (7, 256), (33, 1792), (1001, 2304), (3001, 3584), (301, 11008), (2048, 14336), (20, 32768),
+              (5, 6400)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("t", [Q2K, Q3K])
+@pytest.mark.parametrize("n,k", GEMV_CASES)
+def test_gpu_q2k_q3k_gemv_matches_dequantize_then_matmul(oracle, t, n, k):
+    """Fused Q2_K / Q3_K GEMV against the oracle's dequantize-then-matmul in f64, both activation types: large, small and
+    ragged shapes (rows of 1 to 128 super-blocks, odd counts so that rows start at every alignment, short last chunks,
+    fewer rows than compute units), random block bytes."""
+    import pmetal_amd as pm
+    from gpu_util import gpu_qgemv, rel_errors
+    pm.init(0)
+    nb = {Q2K: 84, Q3K: 110}[t]
+    rng = np.random.default_rng(n * 7 + k + t)
+    raw = rng.integers(0, 256, size=(n * (k // 256), nb), dtype=np.uint8)
+    if t == Q2K:
+        raw[:, 80:84] = np.frombuffer(np.array([0.01, 0.02], np.float16).tobytes(), np.uint8)  # d, dmin small and finite
+    else:
+        raw[:, 108:110] = np.frombuffer(np.array([0.01], np.float16).tobytes(), np.uint8)
+    raw = raw.reshape(-1)
+    x = rng.standard_normal(k).astype(np.float32)
+    x[rng.integers(0, k, max(1, k // 300))] *= 1000.0
+    x[rng.integers(0, k, max(1, k // 300))] *= 1e-6
+    x[5:21] = 0.0
+    bits = oracle.f32_to_bf16_bits(x)
+    for x_dtype, x_dev, x_ref in ((pm.DTYPE_F32, x, x), (pm.DTYPE_BF16, bits, oracle.bf16_bits_to_f32(bits))):
+        want = oracle.qmatvec(t, raw, n, k, x_ref)
+        got = gpu_qgemv(t, raw, n, k, x_dev, x_dtype, 0)
+        elem, norm = rel_errors(got, want)
+        assert elem <= 1e-3 and norm <= 1e-3, (t, n, k, x_dtype, elem, norm)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("t", [Q2K, Q3K])
+def test_gpu_q2k_q3k_gemv_unit_vectors_and_linear(oracle, t):
+    import pmetal_amd as pm
+    from gpu_util import gpu_qgemv, rel_errors, weights
+    pm.init(0)
+    n, k = 301, 2304  # nine super-blocks per row: rows start at every alignment, the second chunk holds one super-block
+    wq = pm.quantize(weights(78, n * k, outliers=1e-3), t)
+    w = oracle.dequantize(t, wq, [n, k]).reshape(n, k)
+    for j in list(range(0, 140)) + [255, 256, 511, 1023, 1024, 2047, 2048, 2303]:
+        x = np.zeros(k, np.float32)
+        x[j] = 1.0
+        got = gpu_qgemv(t, wq, n, k, x, pm.DTYPE_F32, 0)
+        assert np.allclose(got, w[:, j], rtol=1e-6, atol=1e-9), (t, j)
+    assert not gpu_qgemv(t, wq, n, k, np.zeros(k, np.float32), pm.DTYPE_F32, 0).any()
+    x = np.random.default_rng(5).standard_normal(k).astype(np.float32)
+    x[100] = np.inf
+    assert np.isnan(gpu_qgemv(t, wq, n, k, x, pm.DTYPE_F32, 0)).all()
+    # qlinear with several activation rows runs one fused GEMV per row; there is no fused GEMM for these types
+    lib = pm._lib.load()
+    m = 3
+    xs = np.random.default_rng(6).standard_normal((m, k)).astype(np.float32)
+    dw, dx, dy = pm.DeviceBuffer.from_host(wq), pm.DeviceBuffer.from_host(xs), pm.DeviceBuffer(4 * m * n)
+    pm.check(lib.pmetal_hip_qlinear(t, dw.ptr, n, k, dx.ptr, pm.DTYPE_F32, m, dy.ptr, pm.DTYPE_F32, 0, None))
+    pm.check(lib.pmetal_hip_sync(None))
+    got = dy.to_host(np.float32).reshape(m, n)
+    for r in range(m):
+        elem, norm = rel_errors(got[r], oracle.qmatvec(t, wq, n, k, xs[r]))
+        assert elem <= 1e-3 and norm <= 1e-3
+    assert lib.pmetal_hip_qgemm(t, dw.ptr, n, k, dx.ptr, pm.DTYPE_F32, m, dy.ptr, pm.DTYPE_F32, 0, None) == 2
+    lib.pmetal_hip_clear_error()
