@@ -1,0 +1,124 @@
+// Shared pieces of the row-staging GEMV kernels (gemv_q5k.hip, gemv_q6k.hip, gemv_q8_0.hip, gemv_q23k.hip): one
+// workgroup per compute unit, wave (g, h) = chunk h of the rows of row group g, lane partial sums through LDS.
+#pragma once
+#include "gemv_common.hpp"
+
+namespace pmh {
+namespace gemv {
+
+// Row stride of the partial sums in LDS.  The final summation puts `red` lanes on a row (lane p adds every red-th
+// partial), 64 / red rows side by side in a wave: a stride of `red` floats past a multiple of 64 keeps those rows in
+// different banks.
+__host__ __device__ constexpr int part_stride(int slots, int red) { return ((slots + 63) / 64) * 64 + (red & 63); }
+
+__device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {
+    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
+}
+
+// Fixed point for a group of activations that shares one power-of-two scale.  `mb` is the largest magnitude of the group
+// as float bits; every |x| of the group is then below 2^(eb - 126) with eb the biased exponent.  mult = 2^(148 - eb) puts
+// them below 2^22; scale = 2^(eb - 148) undoes it (0 for groups below 2^-126, NaN when the group holds an infinity or a
+// NaN, so that every output of the GEMV becomes NaN).
+struct GroupScale {
+    float mult, scale;
+    bool bad;
+};
+__device__ __forceinline__ GroupScale group_scale(uint32_t mb) {
+    int eb = (int)(mb >> 23);
+    GroupScale g;
+    g.bad = eb == 255;
+    eb = eb < 21 ? 21 : eb;
+    g.mult = __builtin_bit_cast(float, (uint32_t)(275 - eb) << 23);
+    g.scale = g.bad ? __builtin_nanf("") : __builtin_bit_cast(float, (uint32_t)(eb - 21) << 23);
+    return g;
+}
+
+// Four activations -> one dword per digit plane (three balanced base-256 digits in [-128, 127] per value, value c in
+// byte c); returns the sum of the four fixed-point integers.
+__device__ __forceinline__ int to_digits(const float (&v)[4], const GroupScale &g, uint32_t (&dig)[3]) {
+    dig[0] = dig[1] = dig[2] = 0;
+    int sum = 0;
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        const int xi = g.bad ? 0 : (int)__builtin_rintf(v[c] * g.mult);
+        sum += xi;
+        const int d0 = (int)(int8_t)xi, r1 = (xi - d0) >> 8;
+        const int d1 = (int)(int8_t)r1, d2 = (r1 - d1) >> 8;
+        dig[0] |= (uint32_t)(d0 & 0xFF) << (8 * c);
+        dig[1] |= (uint32_t)(d1 & 0xFF) << (8 * c);
+        dig[2] |= (uint32_t)(d2 & 0xFF) << (8 * c);
+    }
+    return sum;
+}
+
+// largest magnitude of four floats, as bits (the order of non-negative floats is that of their bits)
+__device__ __forceinline__ uint32_t max_magnitude_bits(const float (&v)[4]) {
+    uint32_t mb = 0;
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        const uint32_t a = __builtin_bit_cast(uint32_t, v[c]) & 0x7FFFFFFFu;
+        mb = a > mb ? a : mb;
+    }
+    return mb;
+}
+
+// 65536 acc[2] + 256 acc[1] + acc[0] in f32
+__device__ __forceinline__ float combine_planes(const int (&acc)[3]) {
+    return __builtin_fmaf(__builtin_fmaf((float)acc[2], 256.0f, (float)acc[1]), 256.0f, (float)acc[0]);
+}
+
+// Row totals after the barrier: `red` lanes per row (a power of two from 8 to 64 that divides slots), lane p adding
+// every red-th partial, then a sum over the lanes of the row.  part is [group][n_nominal][ps].
+__device__ __forceinline__ void reduce_rows(const float *part, int ps, int slots, int red, int wg_r0, int wg_rows, int rows_per_wave,
+                                            int n_nominal, int nthreads, float *__restrict__ y) {
+    const int per_thread = slots / red;
+    const int red_shift = 31 - __builtin_clz(red);
+    for (int idx0 = 0; idx0 < wg_rows * red; idx0 += nthreads) {
+        const int idx = idx0 + (int)threadIdx.x;
+        int rl = idx >> red_shift;
+        const bool ok = rl < wg_rows;
+        rl = ok ? rl : wg_rows - 1;
+        const int grp = rl / rows_per_wave, loc = rl - grp * rows_per_wave;
+        const int p = idx & (red - 1);
+        const float *src = part + (size_t)(grp * n_nominal + loc) * ps + p;
+        float t0 = 0.0f, t1 = 0.0f, t2 = 0.0f, t3 = 0.0f;
+        int i = 0;
+        for (; i + 8 <= per_thread; i += 8) {  // eight reads in flight
+            const float *q = src + (size_t)i * red;
+            const float a0 = q[0], a1 = q[red], a2 = q[2 * red], a3 = q[3 * red];
+            const float a4 = q[4 * red], a5 = q[5 * red], a6 = q[6 * red], a7 = q[7 * red];
+            t0 += a0 + a4, t1 += a1 + a5, t2 += a2 + a6, t3 += a3 + a7;
+        }
+        for (; i < per_thread; i++) t0 += src[(size_t)i * red];
+        const float sum = team_sum_rt((t0 + t1) + (t2 + t3), red);
+        if (ok && p == 0) y[wg_r0 + rl] = sum;
+    }
+}
+
+// Launch geometry: rows split evenly over one workgroup per compute unit, the workgroup's rows over 16 / ks row groups.
+struct ChunkPlan {
+    int64_t n_wg, rows_per_wg, rows_per_wave, n_nominal, threads;
+    int red;
+    size_t lds;
+};
+// stage_bytes: LDS of one wave's row chunk; lds_x: LDS of the staged activations (slots = 64 ks lane slots)
+inline ChunkPlan plan_chunks(int64_t n, int ks, size_t stage_bytes, size_t lds_x) {
+    ChunkPlan p;
+    const int64_t want = compute_units();
+    p.n_wg = n < want ? n : want;
+    p.rows_per_wg = (n + p.n_wg - 1) / p.n_wg;
+    p.n_wg = (n + p.rows_per_wg - 1) / p.rows_per_wg;
+    int64_t groups = 16 / ks;
+    if (groups > p.rows_per_wg) groups = p.rows_per_wg;
+    p.rows_per_wave = (p.rows_per_wg + groups - 1) / groups;
+    groups = (p.rows_per_wg + p.rows_per_wave - 1) / p.rows_per_wave;
+    p.n_nominal = p.rows_per_wave;
+    p.threads = ks * groups * 64;
+    p.red = 8;  // lanes per row in the final summation: as many as the workgroup has to spare, at most 64
+    while (p.red < 64 && p.rows_per_wg * p.red * 2 <= p.threads) p.red *= 2;
+    p.lds = (size_t)(p.threads / 64) * stage_bytes + lds_x + (size_t)groups * (size_t)p.n_nominal * part_stride(ks * 64, p.red) * 4;
+    return p;
+}
+
+}  // namespace gemv
+}  // namespace pmh

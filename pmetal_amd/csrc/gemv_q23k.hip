@@ -23,7 +23,7 @@
 //    bytes of W), and each lane takes its pieces out of LDS as aligned dwords, which for Q3_K one funnel shift per
 //    dword puts into place.  LDS executes a wave's instructions in order, so the copy needs no barrier.  Lane partial
 //    sums go to LDS; after a barrier the workgroup adds up each of its rows and stores y.
-#include "gemv_common.hpp"
+#include "gemv_chunk.hpp"
 #include "internal.hpp"
 
 namespace {
@@ -35,12 +35,6 @@ typedef uint32_t u4v __attribute__((ext_vector_type(4)));  // a 16-byte piece
 constexpr int kDepth = 8;  // rows in flight per wave
 constexpr int kPre = 2;    // of which this many are requested before x is converted
 constexpr int kPlanes = 3;
-
-__host__ __device__ constexpr int part_stride(int slots, int red) { return ((slots + 63) / 64) * 64 + (red & 63); }
-
-__device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {
-    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
-}
 
 // Element of group p (0..3), position i (0..7), of lane t of super-block sb.
 __device__ __forceinline__ int element_of(int sb, int t, int p, int i) { return 256 * sb + 128 * (t >> 2) + 32 * p + 8 * (t & 3) + i; }
@@ -66,38 +60,19 @@ __device__ __forceinline__ void stage_x(const void *__restrict__ xg, int slots, 
             else if (XF32) v[cc] = reinterpret_cast<const float *>(xg)[e];
             else v[cc] = __builtin_bit_cast(float, (uint32_t) reinterpret_cast<const uint16_t *>(xg)[e] << 16);
         }
-        uint32_t mb = 0;  // largest magnitude of the group, as bits (the order of non-negative floats is that of their bits)
-#pragma unroll
-        for (int cc = 0; cc < 4; cc++) {
-            const uint32_t a = __builtin_bit_cast(uint32_t, v[cc]) & 0x7FFFFFFFu;
-            mb = a > mb ? a : mb;
-        }
+        uint32_t mb = max_magnitude_bits(v);  // then over the lanes that share the group
         const uint32_t o = (uint32_t)__shfl_xor((int)mb, 1);
         mb = o > mb ? o : mb;
-        int eb = (int)(mb >> 23);    // biased exponent: every |x| of the group is below 2^(eb - 126)
-        const bool bad = eb == 255;  // an infinity or a NaN among the activations: every output becomes NaN
-        eb = eb < 21 ? 21 : eb;
-        const float mult = __builtin_bit_cast(float, (uint32_t)(275 - eb) << 23);  // 2^(148 - eb): |x| * mult < 2^22
-        const float scale = bad ? __builtin_nanf("") : __builtin_bit_cast(float, (uint32_t)(eb - 21) << 23);  // 2^(eb - 148); 0 below 2^-126
-        uint32_t dig[kPlanes] = {0, 0, 0};
-        int sum = 0;
-#pragma unroll
-        for (int cc = 0; cc < 4; cc++) {
-            const int xi = bad ? 0 : (int)__builtin_rintf(v[cc] * mult);
-            sum += xi;
-            const int d0 = (int)(int8_t)xi, r1 = (xi - d0) >> 8;
-            const int d1 = (int)(int8_t)r1, d2 = (r1 - d1) >> 8;
-            dig[0] |= (uint32_t)(d0 & 0xFF) << (8 * cc);
-            dig[1] |= (uint32_t)(d1 & 0xFF) << (8 * cc);
-            dig[2] |= (uint32_t)(d2 & 0xFF) << (8 * cc);
-        }
+        const GroupScale gs = group_scale(mb);
+        uint32_t dig[kPlanes];
+        int sum = to_digits(v, gs, dig);
         sum += __shfl_xor(sum, 1);
         if (live) {
 #pragma unroll
             for (int pl = 0; pl < kPlanes; pl++) xd[(pl * 8 + 2 * p + c) * slots + slot] = dig[pl];
             if (c == 0) {
-                xm[slot * 8 + p] = scale;
-                xm[slot * 8 + 4 + p] = (float)sum * scale;
+                xm[slot * 8 + p] = gs.scale;
+                xm[slot * 8 + 4 + p] = (float)sum * gs.scale;
             }
         }
     }
@@ -267,31 +242,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q23k_chunk(const uint8_t *__rest
     }
     __syncthreads();
 
-    // Row totals: `red` lanes per row (a power of two from 8 to 64 that divides slots), lane p adding every
-    // red-th partial, then a sum over the lanes of the row.
-    const int wg_rows = wg_r1 - wg_r0;
-    const int per_thread = slots / red;
-    const int red_shift = 31 - __builtin_clz(red);
-    for (int idx0 = 0; idx0 < wg_rows * red; idx0 += nthreads) {
-        const int idx = idx0 + (int)threadIdx.x;
-        int rl = idx >> red_shift;
-        const bool ok = rl < wg_rows;
-        rl = ok ? rl : wg_rows - 1;
-        const int grp = rl / rows_per_wave, loc = rl - grp * rows_per_wave;
-        const int p = idx & (red - 1);
-        const float *src = part + (size_t)(grp * n_nominal + loc) * ps + p;
-        float t0 = 0.0f, t1 = 0.0f, t2 = 0.0f, t3 = 0.0f;
-        int i = 0;
-        for (; i + 8 <= per_thread; i += 8) {  // eight reads in flight
-            const float *q = src + (size_t)i * red;
-            const float a0 = q[0], a1 = q[red], a2 = q[2 * red], a3 = q[3 * red];
-            const float a4 = q[4 * red], a5 = q[5 * red], a6 = q[6 * red], a7 = q[7 * red];
-            t0 += a0 + a4, t1 += a1 + a5, t2 += a2 + a6, t3 += a3 + a7;
-        }
-        for (; i < per_thread; i++) t0 += src[(size_t)i * red];
-        const float sum = team_sum_rt((t0 + t1) + (t2 + t3), red);
-        if (ok && p == 0) y[wg_r0 + rl] = sum;
-    }
+    reduce_rows(part, ps, slots, red, wg_r0, wg_r1 - wg_r0, rows_per_wave, n_nominal, nthreads, y);
 }
 
 template <class F>
@@ -302,19 +253,11 @@ hipError_t launch_format(const uint8_t *w, int64_t n, int64_t k, const void *x, 
     if (ks > 16 || w_bytes >= (1ull << 32)) return hipErrorInvalidValue;
     const size_t slots = (size_t)ks * 64;
     const size_t lds_x = slots * 4 * (kPlanes * 8) + slots * 32;
-    const int64_t want = compute_units();
-    int64_t n_wg = n < want ? n : want;
-    const int64_t rows_per_wg = (n + n_wg - 1) / n_wg;
-    n_wg = (n + rows_per_wg - 1) / rows_per_wg;
-    int64_t groups = 16 / ks;
-    if (groups > rows_per_wg) groups = rows_per_wg;
-    const int64_t rows_per_wave = (rows_per_wg + groups - 1) / groups;
-    groups = (rows_per_wg + rows_per_wave - 1) / rows_per_wave;
-    const int64_t n_nominal = rows_per_wave;
-    const int64_t threads = ks * groups * 64;
-    int red = 8;  // lanes per row in the final summation: as many as the workgroup has to spare, at most 64
-    while (red < 64 && rows_per_wg * red * 2 <= threads) red *= 2;
-    const size_t lds = (size_t)(threads / 64) * F::kPieces * 16 + lds_x + (size_t)groups * (size_t)n_nominal * part_stride((int)slots, red) * 4;
+    const ChunkPlan plan = plan_chunks(n, ks, (size_t)F::kPieces * 16, lds_x);
+    const int64_t n_wg = plan.n_wg, rows_per_wg = plan.rows_per_wg, rows_per_wave = plan.rows_per_wave, n_nominal = plan.n_nominal,
+                  threads = plan.threads;
+    const int red = plan.red;
+    const size_t lds = plan.lds;
     if (lds > kMaxLds) return hipErrorInvalidValue;
     const bool single = n_nominal <= kDepth;
     auto go = [&](auto kern) {

@@ -23,7 +23,7 @@
 //  * Rows of k / 256 super-blocks that are not whole chunks are handled by the RAGGED variant of the kernel (see there).
 //
 // Matrices below 12 MiB and rows shorter than one chunk stay with the bf16 kernel in gemv.hip.
-#include "gemv_common.hpp"
+#include "gemv_chunk.hpp"
 #include "internal.hpp"
 
 namespace {
@@ -37,12 +37,6 @@ constexpr int kPre = 2;    // of which this many are requested before x is conve
 constexpr int kPlanes = 3;
 constexpr int kChunkBytes = 8 * 210;           // 1680 = 105 pieces of 16 bytes
 constexpr int kStageBytes = kChunkBytes + 32;  // a chunk that starts up to 14 bytes into its first piece, plus one dword for the shifted reads
-
-__host__ __device__ constexpr int part_stride(int slots, int red) { return ((slots + 63) / 64) * 64 + (red & 63); }
-
-__device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {
-    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
-}
 
 // Activations -> LDS.  Thread idx converts elements 4 idx .. 4 idx + 3; the four threads of a quad hold one
 // 16-element group.  Element e = 256 sb + 128 hh + 32 g + l belongs to lane t = 4 hh + 2 (g & 1) + l / 16 of its
@@ -67,33 +61,14 @@ __device__ __forceinline__ void stage_x(const void *__restrict__ xg, int slots, 
             v[2] = __builtin_bit_cast(float, b.y << 16), v[3] = __builtin_bit_cast(float, b.y & 0xFFFF0000u);
         }
         // largest magnitude of the 16-element group, as bits (the order of non-negative floats is that of their bits)
-        uint32_t mb = 0;
-#pragma unroll
-        for (int c = 0; c < 4; c++) {
-            const uint32_t a = __builtin_bit_cast(uint32_t, v[c]) & 0x7FFFFFFFu;
-            mb = a > mb ? a : mb;
-        }
+        uint32_t mb = max_magnitude_bits(v);  // then over the lanes that share the group
         uint32_t o = (uint32_t)__shfl_xor((int)mb, 1);
         mb = o > mb ? o : mb;
         o = (uint32_t)__shfl_xor((int)mb, 2);
         mb = o > mb ? o : mb;
-        int eb = (int)(mb >> 23);  // biased exponent: every |x| of the group is below 2^(eb - 126)
-        const bool bad = eb == 255;  // an infinity or a NaN among the activations: every output becomes NaN
-        eb = eb < 21 ? 21 : eb;
-        const float mult = __builtin_bit_cast(float, (uint32_t)(275 - eb) << 23);  // 2^(148 - eb): |x| * mult < 2^22
-        const float scale = bad ? __builtin_nanf("") : __builtin_bit_cast(float, (uint32_t)(eb - 21) << 23);  // 2^(eb - 148); 0 below 2^-126
-        uint32_t dig[kPlanes] = {0, 0, 0};
-        int sum = 0;
-#pragma unroll
-        for (int c = 0; c < 4; c++) {
-            const int xi = bad ? 0 : (int)__builtin_rintf(v[c] * mult);
-            sum += xi;
-            const int d0 = (int)(int8_t)xi, r1 = (xi - d0) >> 8;
-            const int d1 = (int)(int8_t)r1, d2 = (r1 - d1) >> 8;
-            dig[0] |= (uint32_t)(d0 & 0xFF) << (8 * c);
-            dig[1] |= (uint32_t)(d1 & 0xFF) << (8 * c);
-            dig[2] |= (uint32_t)(d2 & 0xFF) << (8 * c);
-        }
+        const GroupScale gs = group_scale(mb);
+        uint32_t dig[kPlanes];
+        int sum = to_digits(v, gs, dig);
         sum += __shfl_xor(sum, 1);
         sum += __shfl_xor(sum, 2);
         if (live) {
@@ -103,7 +78,7 @@ __device__ __forceinline__ void stage_x(const void *__restrict__ xg, int slots, 
 #pragma unroll
             for (int p = 0; p < kPlanes; p++) xd[(p * 8 + 4 * s + dw) * slots + slot] = dig[p];
             if (dw == 0) {
-                xm[slot * 4 + s] = scale;
+                xm[slot * 4 + s] = gs.scale;
                 xm[slot * 4 + 2 + s] = (float)sum;
             }
         }
@@ -269,31 +244,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q6k_chunk(const uint8_t *__restr
     }
     __syncthreads();
 
-    // Row totals: `red` lanes per row (a power of two from 8 to 64 that divides slots), lane p adding every
-    // red-th partial, then a sum over the lanes of the row.
-    const int wg_rows = wg_r1 - wg_r0;
-    const int per_thread = slots / red;
-    const int red_shift = 31 - __builtin_clz(red);
-    for (int idx0 = 0; idx0 < wg_rows * red; idx0 += nthreads) {
-        const int idx = idx0 + (int)threadIdx.x;
-        int rl = idx >> red_shift;
-        const bool ok = rl < wg_rows;
-        rl = ok ? rl : wg_rows - 1;
-        const int grp = rl / rows_per_wave, loc = rl - grp * rows_per_wave;
-        const int p = idx & (red - 1);
-        const float *src = part + (size_t)(grp * n_nominal + loc) * ps + p;
-        float t0 = 0.0f, t1 = 0.0f, t2 = 0.0f, t3 = 0.0f;
-        int i = 0;
-        for (; i + 8 <= per_thread; i += 8) {  // eight reads in flight
-            const float *q = src + (size_t)i * red;
-            const float a0 = q[0], a1 = q[red], a2 = q[2 * red], a3 = q[3 * red];
-            const float a4 = q[4 * red], a5 = q[5 * red], a6 = q[6 * red], a7 = q[7 * red];
-            t0 += a0 + a4, t1 += a1 + a5, t2 += a2 + a6, t3 += a3 + a7;
-        }
-        for (; i < per_thread; i++) t0 += src[(size_t)i * red];
-        const float sum = team_sum_rt((t0 + t1) + (t2 + t3), red);
-        if (ok && p == 0) y[wg_r0 + rl] = sum;
-    }
+    reduce_rows(part, ps, slots, red, wg_r0, wg_r1 - wg_r0, rows_per_wave, n_nominal, nthreads, y);
 }
 
 }  // namespace
@@ -314,19 +265,11 @@ bool try_launch_qgemv_q6k_chunk(const uint8_t *w, int64_t n, int64_t k, const vo
     if (mode == 0 && w_bytes < (12ull << 20)) return false;
     const size_t slots = (size_t)ks * 64;
     const size_t lds_x = slots * 4 * (kPlanes * 8) + slots * 16;
-    const int64_t want = gemv::compute_units();
-    int64_t n_wg = n < want ? n : want;
-    const int64_t rows_per_wg = (n + n_wg - 1) / n_wg;
-    n_wg = (n + rows_per_wg - 1) / rows_per_wg;
-    int64_t groups = 16 / ks;
-    if (groups > rows_per_wg) groups = rows_per_wg;
-    const int64_t rows_per_wave = (rows_per_wg + groups - 1) / groups;
-    groups = (rows_per_wg + rows_per_wave - 1) / rows_per_wave;
-    const int64_t n_nominal = rows_per_wave;
-    const int64_t threads = ks * groups * 64;
-    int red = 8;  // lanes per row in the final summation: as many as the workgroup has to spare, at most 64
-    while (red < 64 && rows_per_wg * red * 2 <= threads) red *= 2;
-    const size_t lds = (size_t)(threads / 64) * kStageBytes + lds_x + (size_t)groups * (size_t)n_nominal * part_stride((int)slots, red) * 4;
+    const gemv::ChunkPlan plan = gemv::plan_chunks(n, ks, kStageBytes, lds_x);
+    const int64_t n_wg = plan.n_wg, rows_per_wg = plan.rows_per_wg, rows_per_wave = plan.rows_per_wave, n_nominal = plan.n_nominal,
+                  threads = plan.threads;
+    const int red = plan.red;
+    const size_t lds = plan.lds;
     if (lds > 128 * 1024) return false;
     const bool single = n_nominal <= kDepth;
     const bool xf32 = x_dtype == kDtypeF32;
