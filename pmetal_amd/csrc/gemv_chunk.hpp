@@ -62,11 +62,6 @@ __device__ __forceinline__ uint32_t max_magnitude_bits(const float (&v)[4]) {
     return mb;
 }
 
-// 65536 acc[2] + 256 acc[1] + acc[0] in f32
-__device__ __forceinline__ float combine_planes(const int (&acc)[3]) {
-    return __builtin_fmaf(__builtin_fmaf((float)acc[2], 256.0f, (float)acc[1]), 256.0f, (float)acc[0]);
-}
-
 // Row totals after the barrier: `red` lanes per row (a power of two from 8 to 64 that divides slots), lane p adding
 // every red-th partial, then a sum over the lanes of the row.  part is [group][n_nominal][ps].
 __device__ __forceinline__ void reduce_rows(const float *part, int ps, int slots, int red, int wg_r0, int wg_rows, int rows_per_wave,
