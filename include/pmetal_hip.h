@@ -151,6 +151,8 @@ int32_t pmetal_hip_dequantize_dev(uint32_t ggml_type, const uint8_t *src_dev, si
  * with W = reference dequantize of the packed blocks (order as given), fp32 accumulation,
  * max relative error <= 1e-3 against dequantize-then-f32-matmul.
  * W: [n, k] packed row-major, k a multiple of the block size.  x/X: f32 or bf16.
+ * Types: Q8_0, Q4_K and Q6_K have both kernels; Q5_K, Q3_K and Q2_K the GEMV only (k <= 32768), for which qlinear runs
+ * one GEMV per activation row and qgemm answers PMETAL_HIP_ERR_UNSUPPORTED_TYPE.
  * y/Y: f32 (qgemv) or f32/bf16 (qgemm), row-major [m, n].
  * qgemm keeps scratch memory (converted activations, partial tiles) inside the library, one
  * buffer per calling thread, device and stream; it grows on demand, which synchronises that
