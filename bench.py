@@ -30,7 +30,8 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled against a streaming
 # kernel of known size (summary and commands: profiles/qgemv_q4k_14336x4096.md)
-MEASURED_TRAFFIC = {"gemv_q4k_14336x4096": 33293144}
+MEASURED_TRAFFIC = {"gemv_q4k_14336x4096": 33293144, "gemv_q6k_14336x4096": 48531385,
+                    "gemv_q8_0_14336x4096": 62642111}
 BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16/fp16 MFMA, published
 Q8_0, Q4K, Q6K = 8, 12, 14
 
