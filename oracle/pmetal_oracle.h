@@ -13,6 +13,16 @@
  * quantize_q4k / quantize_q6k on general inputs are therefore pinned by the
  * fidelity of this restatement and the independent twin only, never by running
  * the Rust: "restatement-pinned".
+ *
+ * PARITY UNPINNED (no fixture of the reference and no closed form fixes the
+ * result bit for bit on general input; pinned on exact-grid, zero, partial and
+ * hand-derived blocks, by invariants and by the twin only):
+ *   pmo_make_qkx1_quants, pmo_make_qx_quants, pmo_make_q3_quants and the bytes of
+ *   pmo_quantize_q4k, pmo_quantize_q5k, pmo_quantize_q6k, pmo_quantize_q3k,
+ *   pmo_quantize_q2k.
+ * Pinned by the reference's known answers or by closed forms: everything else
+ * (nearest_int, the 6-bit scale packing, Q8_0 and Q8_K, every dequantizer, the
+ * integer dot products, the calibration score, the recipe, the matrix products).
  */
 #ifndef PMETAL_ORACLE_H
 #define PMETAL_ORACLE_H
