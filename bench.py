@@ -587,6 +587,10 @@ def main():
         "roofline": res["roofline"], "extra": res["extra"],
     }
     out["extra"]["event_ms_per_step"] = round(res["event_ms_per_step"], 5)
+    if wl["kind"] == "gemv":
+        # `dtype` names the activation type handed over; the kernels of these (large) shapes multiply in integers
+        out["config"]["arithmetic"] = ("bf16 activations converted exactly to fixed-point int8 digit planes, v_dot4_i32_i8 against "
+                                       "the quantized weights, f32 block scales and accumulation")
     out["roofline"]["traffic"] = MEASURED_TRAFFIC.get(args.workload)
     if args.calibrate:
         pm, _lib, lib = load()
