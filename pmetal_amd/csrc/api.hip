@@ -450,7 +450,8 @@ int32_t pmetal_hip_dequantize(uint32_t t, const uint8_t *src, size_t src_len, co
 }
 
 // ---- quantized linear ----
-// types with a fused GEMV but no fused GEMM
+constexpr int64_t kRowLoopMax = 8;  // activation rows up to which qlinear sends Q5_K / Q3_K / Q2_K through the GEMV, row by row
+// types with a fused GEMV but no GEMM kernel of their own (their GEMM goes through Q6_K, see qgemm_reblocked)
 static bool gemv_only_type(uint32_t t) { return t == PMETAL_GGML_TYPE_Q5K || t == PMETAL_GGML_TYPE_Q3K || t == PMETAL_GGML_TYPE_Q2K; }
 
 static int32_t check_linear(uint32_t t, const void *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype,
@@ -536,8 +537,50 @@ int32_t pmetal_hip_qgemv_batch(const pmetal_hip_linear_desc *descs, size_t count
     return ok();
 }
 
+// Q5_K, Q3_K and Q2_K have no GEMM kernel of their own: their super-blocks are re-blocked, exactly, into one or two Q6_K
+// tensors in the scratch buffer (W = A + B), which go through the Q6_K GEMM; two partial results are added in f32.
+static int32_t qgemm_reblocked(uint32_t t, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, int64_t m, void *y,
+                               uint32_t y_dtype, uint32_t order, void *stream) {
+    auto up16 = [](size_t v) { return (v + 15) & ~(size_t)15; };
+    hipStream_t s = (hipStream_t)stream;
+    const int parts = pmh::reblock_q6k_parts(t);
+    const size_t n_blocks = (size_t)n * (size_t)(k / 256);
+    if (n_blocks > SIZE_MAX / 512 || (size_t)m > SIZE_MAX / 16 / (size_t)n)
+        return fail(PMETAL_HIP_ERR_SHAPE_TOO_LARGE, "qgemm: shape is too large");
+    const size_t gemm_bytes = up16(pmh::qgemm_workspace_bytes(m, n, k)), w_bytes = up16(n_blocks * 210);
+    const size_t y_elems = (size_t)m * (size_t)n, y_bytes = up16(y_elems * 4);
+    const bool y_f32 = y_dtype == PMETAL_HIP_DTYPE_F32;
+    // scratch: [GEMM scratch][A][B][partial result of B][partial result of A when y is not f32]
+    const size_t total = gemm_bytes + parts * w_bytes + (parts == 2 ? y_bytes * (y_f32 ? 1 : 2) : 0);
+    void *ws = nullptr;
+    if (int32_t rc = workspace(total, s, &ws)) return rc;
+    uint8_t *base = (uint8_t *)ws, *wa = base + gemm_bytes, *wb = wa + w_bytes;
+    float *yb = (float *)(wb + w_bytes), *ya = y_f32 ? (float *)y : (float *)((uint8_t *)yb + y_bytes);
+    hipError_t e = pmh::launch_reblock_q6k(t, w, n_blocks, order, wa, wb, s);
+    if (e != hipSuccess) return hip_fail(e, "re-blocking kernel launch");
+    if (parts == 1) {
+        e = pmh::launch_qgemm(PMETAL_GGML_TYPE_Q6K, wa, n, k, x, x_dtype, m, y, y_dtype, 0, ws, s);
+    } else {
+        e = pmh::launch_qgemm(PMETAL_GGML_TYPE_Q6K, wa, n, k, x, x_dtype, m, ya, PMETAL_HIP_DTYPE_F32, 0, ws, s);
+        if (e == hipSuccess) e = pmh::launch_qgemm(PMETAL_GGML_TYPE_Q6K, wb, n, k, x, x_dtype, m, yb, PMETAL_HIP_DTYPE_F32, 0, ws, s);
+        if (e == hipSuccess) e = pmh::launch_add_store(ya, yb, y_elems, y, !y_f32, s);
+    }
+    if (e == hipErrorNotSupported) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "qgemm: configuration not supported");
+    if (e != hipSuccess) return hip_fail(e, "qgemm kernel launch");
+    return ok();
+}
+
 int32_t pmetal_hip_qgemm(uint32_t t, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, int64_t m,
                          void *y, uint32_t y_dtype, uint32_t order, void *stream) {
+    if (gemv_only_type(t)) {
+        if (int32_t rc = check_linear(t, w, n, k, x, x_dtype, y, order, true)) return rc;
+        if (!aligned16(y)) return fail(PMETAL_HIP_ERR_INVALID_ARG, "device pointers must be 16-byte aligned");
+        if (y_dtype > PMETAL_HIP_DTYPE_BF16) return fail(PMETAL_HIP_ERR_INVALID_ARG, "y_dtype must be 0 (f32) or 1 (bf16)");
+        if (m <= 0 || m > 0x7FFFFFFF) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "m must be in [1, 2^31)");
+        if (!pmh::qgemm_fits(PMETAL_GGML_TYPE_Q6K, m, n, k))
+            return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qgemm: m and k must be at most 2^22 (m = %lld, k = %lld)", (long long)m, (long long)k);
+        return qgemm_reblocked(t, w, n, k, x, x_dtype, m, y, y_dtype, order, stream);
+    }
     if (int32_t rc = check_linear(t, w, n, k, x, x_dtype, y, order)) return rc;
     if (y_dtype > PMETAL_HIP_DTYPE_BF16) return fail(PMETAL_HIP_ERR_INVALID_ARG, "y_dtype must be 0 (f32) or 1 (bf16)");
     if (m <= 0 || m > 0x7FFFFFFF) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "m must be in [1, 2^31)");
@@ -556,10 +599,11 @@ int32_t pmetal_hip_qlinear(uint32_t t, const uint8_t *w, int64_t n, int64_t k, c
                            void *y, uint32_t y_dtype, uint32_t order, void *stream) {
     if (m == 1 && y_dtype == PMETAL_HIP_DTYPE_F32)
         return pmetal_hip_qgemv(t, w, n, k, x, x_dtype, (float *)y, order, stream);
-    if (((t == PMETAL_GGML_TYPE_Q8_0 && k % 256 != 0) || gemv_only_type(t)) && y_dtype == PMETAL_HIP_DTYPE_F32 && m > 1 && n > 0 &&
-        k > 0 && x && y) {
-        // The fused GEMM walks k in steps of 256, and a Q8_0 row may be any multiple of 32; Q5_K, Q3_K and Q2_K have no fused GEMM: one
-        // fused GEMV per activation row then, back to back on the stream.
+    if (((t == PMETAL_GGML_TYPE_Q8_0 && k % 256 != 0) || (gemv_only_type(t) && m <= kRowLoopMax)) && y_dtype == PMETAL_HIP_DTYPE_F32 &&
+        m > 1 && n > 0 && k > 0 && x && y) {
+        // The fused GEMM walks k in steps of 256, and a Q8_0 row may be any multiple of 32: one fused GEMV per activation row
+        // then, back to back on the stream.  Q5_K, Q3_K and Q2_K reach the GEMM through a re-blocking pass over the whole
+        // matrix, which a few rows do not repay.
         const size_t x_row = (size_t)k * (x_dtype == PMETAL_HIP_DTYPE_F32 ? 4 : 2);
         for (int64_t r = 0; r < m; r++) {
             const int32_t rc = pmetal_hip_qgemv(t, w, n, k, (const uint8_t *)x + (size_t)r * x_row, x_dtype,

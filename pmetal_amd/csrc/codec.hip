@@ -247,6 +247,21 @@ struct DecQ5K {
             o[t] = d1 * (float)v - dm1;
         }
     }
+    // the same elements as integers: value = d * sc * q[t] - dmin * m
+    static constexpr bool kHasMin = true;
+    static __device__ __forceinline__ void ints(const Raw &r, int i, int (&q)[4], int &sc_out, int &m_out) {
+        const int c = i >> 4, p = (i & 15) * 4, half = p >> 5;
+        uint32_t sc, m;
+        scale_min_k4(2 * c + half, r.hdr.y, r.hdr.z, r.hdr.w, sc, m);
+        sc_out = (int)sc, m_out = (int)m;
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            if (ORDER == 0) q[t] = (int)(((r.q >> (4 * t)) & 0xFu) | (((r.h >> t) & 1u) << 4));
+            else q[t] = (int)((((half ? r.q >> 4 : r.q) >> (8 * t)) & 0xFu) | (((r.h >> (8 * t)) & 1u) << 4));
+        }
+    }
+    static __device__ __forceinline__ uint32_t d_bits(const uint8_t *blk) { return *reinterpret_cast<const uint16_t *>(blk); }
+    static __device__ __forceinline__ uint32_t dmin_bits(const uint8_t *blk) { return *reinterpret_cast<const uint16_t *>(blk + 2); }
 };
 
 // Q6_K (k_quants.rs:474-496 + :614-660): out = (d * sc) * q, left-associated.  Blocks are 2-byte aligned.
@@ -296,6 +311,15 @@ struct DecQ2K {
 #pragma unroll
         for (int t = 0; t < 4; t++) o[t] = dl * (float)((r.q >> (8 * t + 2 * p)) & 3u) - ml;
     }
+    static constexpr bool kHasMin = true;
+    static __device__ __forceinline__ void ints(const Raw &r, int i, int (&q)[4], int &sc_out, int &m_out) {
+        const int p = (i >> 3) & 3;
+        sc_out = (int)(r.sc & 0xFu), m_out = (int)(r.sc >> 4);
+#pragma unroll
+        for (int t = 0; t < 4; t++) q[t] = (int)((r.q >> (8 * t + 2 * p)) & 3u);
+    }
+    static __device__ __forceinline__ uint32_t d_bits(const uint8_t *blk) { return *reinterpret_cast<const uint16_t *>(blk + 80); }
+    static __device__ __forceinline__ uint32_t dmin_bits(const uint8_t *blk) { return *reinterpret_cast<const uint16_t *>(blk + 82); }
 };
 
 // Q3_K (k_quants.rs:281-355 + :713-760): out = (d * (sc6 - 32)) * (q2 - (hbit ? 0 : 4)).  110-byte blocks: hmask[32],
@@ -321,6 +345,16 @@ struct DecQ3K {
             o[t] = dl * (float)q;
         }
     }
+    static constexpr bool kHasMin = false;
+    static __device__ __forceinline__ void ints(const Raw &r, int i, int (&q)[4], int &sc_out, int &m_out) {
+        const int h = i >> 5, p = (i >> 3) & 3, is = i >> 2;
+        const uint32_t sc6 = ((is < 8 ? r.lo : r.lo >> 4) & 0xFu) | (((r.hi >> (2 * (is >> 2))) & 3u) << 4);
+        sc_out = (int)sc6 - 32, m_out = 0;
+#pragma unroll
+        for (int t = 0; t < 4; t++) q[t] = (int)((r.q >> (8 * t + 2 * p)) & 3u) - (((r.h >> (8 * t + 4 * h + p)) & 1u) ? 0 : 4);
+    }
+    static __device__ __forceinline__ uint32_t d_bits(const uint8_t *blk) { return *reinterpret_cast<const uint16_t *>(blk + 108); }
+    static __device__ __forceinline__ uint32_t dmin_bits(const uint8_t *) { return 0; }
 };
 
 // Q8_K (k_quants.rs:498-506): out = d * q, one rounding.  292-byte blocks: d f32, qs[256] i8, bsums[16] i16.
@@ -361,6 +395,70 @@ __global__ __launch_bounds__(256) void k_dequantize_kq(const uint8_t *__restrict
         } else {
             for (int t = 0; t < 4 && e + t < n; t++) dst[e + t] = o[t];
         }
+    }
+}
+
+// Exact re-blocking of Q5_K, Q3_K and Q2_K super-blocks into Q6_K ones, for the matrix-matrix product: the fused GEMM
+// kernels exist for Q4_K, Q6_K and Q8_0, and Q6_K (value d * sc * (q - 32), sixteen int8 scales, q - 32 in [-32, 31])
+// holds the other formats' elements without loss.  With the decoder's integers (value = d * s * q - dmin * m):
+//   block A: d, scale s per 16 elements, stored quant q + 32      (Q5_K: s <= 63, q <= 31; Q3_K: s in [-32, 31], q in
+//            [-4, 3]; Q2_K: s <= 15, q <= 3)
+//   block B (formats with mins): dmin as d, scale m, stored quant 31, i.e. -1 * dmin * m for every element.
+// W x = A x + B x then, every product exact.  One wave per super-block: lane i decodes elements 4 i .. 4 i + 3 into
+// LDS, then assembles ql bytes 2 i and 2 i + 1 and qh byte i of the Q6_K layout (k_quants.rs:1116-1130).
+template <class D>
+__global__ __launch_bounds__(256) void k_reblock_q6k(const uint8_t *__restrict__ src, size_t n_blocks, uint8_t *__restrict__ dst_a,
+                                                     uint8_t *__restrict__ dst_b) {
+    __shared__ __align__(16) uint8_t quants[4][256];
+    __shared__ int8_t scales[4][2][16];
+    const int w = (int)(threadIdx.x >> 6), i = (int)(threadIdx.x & 63);
+    const size_t blk_i = (size_t)blockIdx.x * 4 + w;
+    const bool live = blk_i < n_blocks;  // wave-uniform
+    const uint8_t *blk = src + (live ? blk_i : 0) * D::kBytes;
+    const typename D::Raw raw = D::load(blk, i);
+    int q[4], sc, m;
+    D::ints(raw, i, q, sc, m);
+    *reinterpret_cast<uint32_t *>(&quants[w][4 * i]) =
+        (uint32_t)(q[0] + 32) | ((uint32_t)(q[1] + 32) << 8) | ((uint32_t)(q[2] + 32) << 16) | ((uint32_t)(q[3] + 32) << 24);
+    if ((i & 3) == 0) scales[w][0][i >> 2] = (int8_t)sc, scales[w][1][i >> 2] = (int8_t)m;
+    __syncthreads();
+    if (!live) return;
+    const uint8_t *qv = quants[w];
+    uint32_t ql = 0;
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const int b = 2 * i + t, lo = 128 * (b >> 6) + (b & 63);  // ql byte b: low nibble of element lo, high of lo + 64
+        ql |= ((uint32_t)(qv[lo] & 15u) | ((uint32_t)(qv[lo + 64] & 15u) << 4)) << (8 * t);
+    }
+    const int e0 = 128 * (i >> 5) + (i & 31);  // qh byte i: bits 2 g .. 2 g + 1 from element e0 + 32 g
+    const uint32_t qh = (uint32_t)(qv[e0] >> 4) | ((uint32_t)(qv[e0 + 32] >> 4) << 2) | ((uint32_t)(qv[e0 + 64] >> 4) << 4) |
+                        ((uint32_t)(qv[e0 + 96] >> 4) << 6);
+    uint8_t *out = dst_a + blk_i * 210;
+    *reinterpret_cast<uint16_t *>(out + 2 * i) = (uint16_t)ql;
+    out[128 + i] = (uint8_t)qh;
+    if (i < 16) out[192 + i] = (uint8_t)scales[w][0][i];
+    if (i == 0) *reinterpret_cast<uint16_t *>(out + 208) = (uint16_t)D::d_bits(blk);
+    if (D::kHasMin) {
+        out = dst_b + blk_i * 210;
+        *reinterpret_cast<uint16_t *>(out + 2 * i) = 0xFFFFu;  // 31 = nibble 15, top bits 01
+        out[128 + i] = 0x55u;
+        if (i < 16) out[192 + i] = (uint8_t)scales[w][1][i];
+        if (i == 0) *reinterpret_cast<uint16_t *>(out + 208) = (uint16_t)D::dmin_bits(blk);
+    }
+}
+
+// y = a + b (f32), stored as f32 or as bf16 rounded to nearest even
+__global__ __launch_bounds__(256) void k_add_store(const float *__restrict__ a, const float *__restrict__ b, size_t n, void *__restrict__ y,
+                                                   int y_bf16) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const float v = a[idx] + b[idx];
+    if (y_bf16) {
+        const uint32_t u = __builtin_bit_cast(uint32_t, v);
+        reinterpret_cast<uint16_t *>(y)[idx] =
+            (uint16_t)(((u & 0x7FFFFFFFu) > 0x7F800000u) ? ((u >> 16) | 0x40u) : ((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16));
+    } else {
+        reinterpret_cast<float *>(y)[idx] = v;
     }
 }
 
@@ -1204,6 +1302,33 @@ hipError_t launch_kl_sums_quantized(uint32_t type, const uint8_t *src, const flo
     case kTypeQ8K: hipLaunchKernelGGL(k_kl_sums_kq<DecQ8K>, grid, block, 0, s, src, original, n, partial); break;
     default: return hipErrorInvalidValue;
     }
+    return hipGetLastError();
+}
+
+int reblock_q6k_parts(uint32_t type) {
+    return type == kTypeQ3K ? 1 : (type == kTypeQ5K || type == kTypeQ2K) ? 2 : 0;
+}
+
+hipError_t launch_reblock_q6k(uint32_t type, const uint8_t *src, size_t n_blocks, uint32_t order, uint8_t *dst_a, uint8_t *dst_b,
+                              hipStream_t s) {
+    if (n_blocks == 0) return hipSuccess;
+    const dim3 grid((unsigned)((n_blocks + 3) / 4)), block(256);
+    if (type == kTypeQ5K) {
+        if (order == kOrderRef) hipLaunchKernelGGL(k_reblock_q6k<DecQ5K<0>>, grid, block, 0, s, src, n_blocks, dst_a, dst_b);
+        else hipLaunchKernelGGL(k_reblock_q6k<DecQ5K<1>>, grid, block, 0, s, src, n_blocks, dst_a, dst_b);
+    } else if (type == kTypeQ3K) {
+        hipLaunchKernelGGL(k_reblock_q6k<DecQ3K>, grid, block, 0, s, src, n_blocks, dst_a, dst_b);
+    } else if (type == kTypeQ2K) {
+        hipLaunchKernelGGL(k_reblock_q6k<DecQ2K>, grid, block, 0, s, src, n_blocks, dst_a, dst_b);
+    } else {
+        return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_add_store(const float *a, const float *b, size_t n, void *y, bool y_bf16, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_add_store, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, a, b, n, y, y_bf16 ? 1 : 0);
     return hipGetLastError();
 }
 

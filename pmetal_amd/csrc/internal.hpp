@@ -78,6 +78,13 @@ hipError_t launch_dequantize_q8k(const uint8_t *src, size_t n, float *dst, hipSt
 int kl_sums_workgroups(size_t n);
 hipError_t launch_kl_sums(const float *a, const float *b, size_t n, double *partial, hipStream_t s);
 // the same sums between `original` and the first n elements decoded from k-quant blocks (never stored), into
+// Exact re-blocking of Q5_K / Q3_K / Q2_K super-blocks into Q6_K ones (210 bytes each): W = A (+ B for the formats with
+// mins).  reblock_q6k_parts: 2, 1, 2; 0 for any other type.  dst_b is not touched when there is one part.
+int reblock_q6k_parts(uint32_t type);
+hipError_t launch_reblock_q6k(uint32_t type, const uint8_t *src, size_t n_blocks, uint32_t order, uint8_t *dst_a, uint8_t *dst_b,
+                              hipStream_t s);
+// y[i] = a[i] + b[i], stored as f32 or bf16
+hipError_t launch_add_store(const float *a, const float *b, size_t n, void *y, bool y_bf16, hipStream_t s);
 // partial[4 * kl_sums_quantized_workgroups(n)]; hipErrorInvalidValue for a type that is not a k-quant
 int kl_sums_quantized_workgroups(size_t n);
 hipError_t launch_kl_sums_quantized(uint32_t type, const uint8_t *src, const float *original, size_t n, uint32_t order, double *partial,

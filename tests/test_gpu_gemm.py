@@ -273,3 +273,68 @@ def test_qgemm_on_two_streams_of_one_thread_keep_separate_scratch(oracle):
     finally:
         lib.pmetal_hip_stream_destroy(s1)
         lib.pmetal_hip_stream_destroy(s2)
+
+
+# Q5_K, Q3_K and Q2_K reach the GEMM through an exact re-blocking into Q6_K super-blocks (one tensor, or two for the formats
+# with mins).  d / dmin offsets inside a block, for random block bytes with finite scales:
+REBLOCKED = {13: (176, (0, 2)), 11: (110, (108,)), 10: (84, (80, 82))}
+
+
+@pytest.mark.parametrize("t", sorted(REBLOCKED))
+@pytest.mark.parametrize("m,n,k", [(9, 128, 256), (16, 128, 512), (33, 200, 768), (130, 129, 256), (300, 512, 2048)])
+def test_qgemm_q5k_q3k_q2k_matches_dequantize_then_matmul(oracle, t, m, n, k):
+    """Random block bytes (every scale, min and quant value; negative Q3_K scales) and quantized weights, both element
+    orders for Q5_K, f32 and bf16 results, against the oracle's dequantize-then-matmul in f64."""
+    size, d_at = REBLOCKED[t]
+    rng = np.random.default_rng(1000 * t + m + n + k)
+    raw = rng.integers(0, 256, size=(n * (k // 256), size), dtype=np.uint8)
+    for j, off in enumerate(d_at):
+        raw[:, off:off + 2] = np.frombuffer(np.array([0.01 * (j + 1)], np.float16).tobytes(), np.uint8)
+    raw[3, d_at[0]:d_at[0] + 2] = np.frombuffer(np.array([-0.03], np.float16).tobytes(), np.uint8)  # a negative d
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    bits = oracle.f32_to_bf16_bits(x.reshape(-1)).reshape(m, k)
+    xb = oracle.bf16_bits_to_f32(bits.reshape(-1)).reshape(m, k)
+    for wq in (raw.reshape(-1), oracle.quantize(t, weights(t + m, n * k, outliers=1e-3))):
+        for order in ((0, 1) if t == 13 else (0,)):
+            want = reference(oracle, t, wq, n, k, xb, order)
+            got = gpu_qgemm(t, wq, n, k, bits, m, order=order)
+            elem, norm = rel_errors(got.reshape(-1), want.reshape(-1))
+            print(f"type {t} GEMM m={m} n={n} k={k} order={order}: elem {elem:.2e} norm {norm:.2e}")
+            assert elem <= TOL and norm <= TOL
+            got16 = gpu_qgemm(t, wq, n, k, bits, m, y_dtype=pm.DTYPE_BF16, order=order)
+            assert np.allclose(got16, got, rtol=2.0 ** -8, atol=1e-30)
+    # f32 activations: the GEMM rounds them to f16 at the row's power-of-two scale (test_qgemm_f32_activations); both
+    # parts of a re-blocked tensor see the same rounded values
+    got = gpu_qgemm(t, raw.reshape(-1), n, k, x, m, x_dtype=pm.DTYPE_F32)
+    want = reference(oracle, t, raw.reshape(-1), n, k, x, 0)
+    e = np.floor(np.log2(np.max(np.abs(x), axis=1, keepdims=True))) - 9
+    xr = (np.ldexp(x, (-e).astype(np.int32)).astype(np.float16).astype(np.float32) * np.exp2(e)).astype(np.float32)
+    want_r = reference(oracle, t, raw.reshape(-1), n, k, xr, 0)
+    for row in range(m):
+        _, norm = rel_errors(got[row], want[row])
+        elem_r, norm_r = rel_errors(got[row], want_r[row])
+        assert norm <= 2 * TOL and elem_r <= TOL and norm_r <= TOL, (row, norm, elem_r, norm_r)
+
+
+@pytest.mark.parametrize("t", sorted(REBLOCKED))
+def test_qlinear_q5k_q3k_q2k_dispatch(oracle, t):
+    """qlinear: up to eight activation rows one fused GEMV each, above that the re-blocked GEMM; both agree with the
+    oracle; a second, smaller call reuses the scratch buffer."""
+    lib = _lib.load()
+    n, k = 320, 1024
+    wq = oracle.quantize(t, weights(t, n * k, outliers=1e-3))
+    dw = pm.DeviceBuffer.from_host(wq)
+    for m in (8, 9, 64, 3):
+        x = np.random.default_rng(m).standard_normal((m, k)).astype(np.float32)
+        x = oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(x.reshape(-1))).reshape(m, k)  # survives the GEMM's f16 rounding
+        dx, dy = pm.DeviceBuffer.from_host(x), pm.DeviceBuffer(4 * m * n)
+        pm.check(lib.pmetal_hip_qlinear(t, dw.ptr, n, k, dx.ptr, pm.DTYPE_F32, m, dy.ptr, pm.DTYPE_F32, 0, None))
+        pm.check(lib.pmetal_hip_sync(None))
+        want = reference(oracle, t, wq, n, k, x, 0)
+        elem, norm = rel_errors(dy.to_host(np.float32), want.reshape(-1))
+        assert elem <= TOL and norm <= TOL, (t, m, elem, norm)
+    # the GEMM's own argument checks
+    assert lib.pmetal_hip_qgemm(t, dw.ptr, n, k, dx.ptr, pm.DTYPE_F32, 0, dy.ptr, pm.DTYPE_F32, 0, None) == 6
+    assert lib.pmetal_hip_qgemm(t, dw.ptr, n, k, dx.ptr, pm.DTYPE_F32, 3, dy.ptr + 4, pm.DTYPE_F32, 0, None) == 1
+    assert lib.pmetal_hip_qgemm(t, dw.ptr, n, k, dx.ptr, pm.DTYPE_F32, 3, dy.ptr, 7, 0, None) == 1
+    lib.pmetal_hip_clear_error()
