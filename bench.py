@@ -356,7 +356,7 @@ def bench_gemm(args, m, n, k, t=Q4K):
         "value": tflops, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / BF16_PEAK_TFLOPS, 4), "traffic": None,
-                     "kernel": {Q4K: "k_qgemm_rw", Q6K: "k_qgemm_rw_q6", Q8_0: "k_qgemm_rw_q8"}[t] + " (+ k_prep_rw, k_rw_reduce when K is split)",
+                     "kernel": {Q4K: "k_qgemm_rw", Q6K: "k_qgemm_rw_q6", Q8_0: "k_qgemm_rw_q8"}.get(t, "k_reblock_q6k + k_qgemm_rw_q6 per part") + " (+ k_prep_rw, k_rw_reduce when K is split)",
                      "flops_per_launch": flops, "us_per_launch": round(us, 3)},
         "extra": {"mfma_loop_sustained_TFLOPs": round(sustained, 1), "frac_of_sustained": round(tflops / sustained, 4)},
     }, (t, n, k)
@@ -538,6 +538,9 @@ WORKLOADS["gemm_q6k_m512"] = dict(kind="gemm", m=512, n=14336, k=4096, metric="Q
                                   unit="TFLOP/s", dtype="f16", type=Q6K)
 WORKLOADS["gemm_q8_0_m512"] = dict(kind="gemm", m=512, n=14336, k=4096, metric="Q8_0 GEMM TFLOPS @M=512,K=4096,N=14336",
                                    unit="TFLOP/s", dtype="f16", type=Q8_0)
+for _name, _t in (("q5k", 13), ("q3k", 11), ("q2k", 10)):  # re-blocked into Q6_K inside the call (two tensors, one, two)
+    WORKLOADS[f"gemm_{_name}_m512"] = dict(kind="gemm", m=512, n=14336, k=4096, unit="TFLOP/s", dtype="f16", type=_t,
+                                           metric=f"{_name.upper().replace('K', '_K')} GEMM TFLOPS (nominal flops) @M=512,K=4096,N=14336")
 
 
 def main():

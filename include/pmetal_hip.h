@@ -37,10 +37,10 @@ extern "C" {
 #define PMETAL_GGML_TYPE_F32 0u
 #define PMETAL_GGML_TYPE_F16 1u
 #define PMETAL_GGML_TYPE_Q8_0 8u
-#define PMETAL_GGML_TYPE_Q2K 10u /* quantize / dequantize (k_quants.rs:1242-1321, :230-266) and the fused GEMV; no fused GEMM */
-#define PMETAL_GGML_TYPE_Q3K 11u /* quantize / dequantize (k_quants.rs:1139-1237, :281-355) and the fused GEMV; no fused GEMM */
+#define PMETAL_GGML_TYPE_Q2K 10u /* quantize / dequantize (k_quants.rs:1242-1321, :230-266) and the fused GEMV; GEMM through Q6_K re-blocking */
+#define PMETAL_GGML_TYPE_Q3K 11u /* quantize / dequantize (k_quants.rs:1139-1237, :281-355) and the fused GEMV; GEMM through Q6_K re-blocking */
 #define PMETAL_GGML_TYPE_Q4K 12u
-#define PMETAL_GGML_TYPE_Q5K 13u /* quantize / dequantize (k_quants.rs:960-1051, :407-462) and the fused GEMV; no fused GEMM */
+#define PMETAL_GGML_TYPE_Q5K 13u /* quantize / dequantize (k_quants.rs:960-1051, :407-462) and the fused GEMV; GEMM through Q6_K re-blocking */
 #define PMETAL_GGML_TYPE_Q6K 14u
 #define PMETAL_GGML_TYPE_Q8K 15u /* quantize / dequantize (k_quants.rs:815-871, :498-506) and the activation side of qgemv_q8k */
 
@@ -151,8 +151,10 @@ int32_t pmetal_hip_dequantize_dev(uint32_t ggml_type, const uint8_t *src_dev, si
  * with W = reference dequantize of the packed blocks (order as given), fp32 accumulation,
  * max relative error <= 1e-3 against dequantize-then-f32-matmul.
  * W: [n, k] packed row-major, k a multiple of the block size.  x/X: f32 or bf16.
- * Types: Q8_0, Q4_K and Q6_K have both kernels; Q5_K, Q3_K and Q2_K the GEMV only (k <= 32768), for which qlinear runs
- * one GEMV per activation row and qgemm answers PMETAL_HIP_ERR_UNSUPPORTED_TYPE.
+ * Types: Q8_0, Q4_K and Q6_K have both kernels.  Q5_K, Q3_K and Q2_K have a GEMV kernel (k <= 32768) and no GEMM
+ * kernel of their own: qgemm re-blocks their super-blocks, without loss, into one (Q3_K) or two (Q5_K, Q2_K: values
+ * and mins) Q6_K tensors in its scratch memory on every call (Q5_K 2.4, Q3_K 1.9, Q2_K 5 times the bytes of W) and runs the Q6_K
+ * GEMM on them; qlinear runs one GEMV per activation row up to m = 8 and qgemm above.
  * y/Y: f32 (qgemv) or f32/bf16 (qgemm), row-major [m, n].
  * qgemm keeps scratch memory (converted activations, partial tiles) inside the library, one
  * buffer per calling thread, device and stream; it grows on demand, which synchronises that
@@ -163,7 +165,8 @@ int32_t pmetal_hip_qgemm(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, in
                          uint32_t x_dtype, int64_t m, void *y_dev, uint32_t y_dtype, uint32_t order,
                          void *stream);
 /* Dispatch by m: m == 1 -> qgemv (f32 output only), otherwise qgemm (k must be a multiple of 256).  A Q8_0
- * row that is only a multiple of 32 runs one GEMV per activation row when m > 1 (f32 output only). */
+ * row that is only a multiple of 32 runs one GEMV per activation row when m > 1 (f32 output only), and so do
+ * Q5_K, Q3_K and Q2_K for 2 <= m <= 8 with f32 output. */
 int32_t pmetal_hip_qlinear(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, int64_t k, const void *x_dev,
                            uint32_t x_dtype, int64_t m, void *y_dev, uint32_t y_dtype, uint32_t order,
                            void *stream);
