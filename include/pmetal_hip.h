@@ -164,6 +164,21 @@ int32_t pmetal_hip_qgemv(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, in
 int32_t pmetal_hip_qgemm(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, int64_t k, const void *x_dev,
                          uint32_t x_dtype, int64_t m, void *y_dev, uint32_t y_dtype, uint32_t order,
                          void *stream);
+/* pmetal_hip_qgemm without any allocation.  No counterpart in the reference (there MLX owns every buffer): it is for
+ * callers that cannot call hipMalloc -- code under HIP graph capture, tight serving loops, harnesses that forbid it.
+ * Same arguments, kernels and results (bit for bit) as pmetal_hip_qgemm for Q8_0, Q4_K and Q6_K; the scratch memory
+ * (converted activations, row scales, partial tiles of a K split) is a fixed array of
+ * PMETAL_HIP_NOALLOC_SCRATCH_BYTES inside the library's code object, one copy per device, held until the process ends.
+ * A shape that needs more (roughly: m * k * 2.25 bytes plus, for few activation rows, splits * m * n * 4) fails with
+ * PMETAL_HIP_ERR_SHAPE_TOO_LARGE before anything is launched; Q5_K / Q3_K / Q2_K (re-blocking needs scratch of the size
+ * of W) fail with PMETAL_HIP_ERR_UNSUPPORTED_TYPE.  Calls no hipMalloc / hipFree and nothing else that allocates.
+ * pmetal_hip_init(device) looks the array's address up; without it the first call on a device does.  All calls on one
+ * device share the array: calls that overlap on one device (two streams, two threads) race; calls on one stream are
+ * ordered and may follow each other without a synchronisation.                                                        */
+#define PMETAL_HIP_NOALLOC_SCRATCH_BYTES ((size_t)32 << 20)
+int32_t pmetal_hip_qgemm_noalloc(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, int64_t k, const void *x_dev,
+                                 uint32_t x_dtype, int64_t m, void *y_dev, uint32_t y_dtype, uint32_t order,
+                                 void *stream);
 /* Dispatch by m: m == 1 -> qgemv (f32 output only), otherwise qgemm (k must be a multiple of 256).  A Q8_0
  * row that is only a multiple of 32 runs one GEMV per activation row when m > 1 (f32 output only), and so do
  * Q5_K, Q3_K and Q2_K for 2 <= m <= 8 with f32 output. */

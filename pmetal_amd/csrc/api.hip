@@ -138,6 +138,33 @@ int32_t workspace(size_t bytes, hipStream_t stream, void **out) {
     return PMETAL_HIP_OK;
 }
 
+
+// ---- scratch memory of the entry point that allocates nothing (pmetal_hip_qgemm_noalloc) ----
+// A fixed array in the code object: every device that loads the library holds its own copy, at its own address, until the
+// process ends.  In host code the name `scratch` is only a handle for hipGetSymbolAddress; kernels and copies get the
+// device address looked up below, once per device.
+constexpr size_t kNoAllocScratchBytes = PMETAL_HIP_NOALLOC_SCRATCH_BYTES;  // 32 MiB
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+constexpr int kMaxScratchDevices = 64;
+void *g_scratch_ptr[kMaxScratchDevices] = {nullptr};
+std::mutex g_scratch_mu;
+
+// Device address of `scratch` on the calling thread's current device (looked up on the first call for that device).
+int32_t scratch_of_current_device(void **out) {
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxScratchDevices) return fail(PMETAL_HIP_ERR_INVALID_ARG, "device %d is beyond the %d devices the library keeps scratch for", dev, kMaxScratchDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fail(PMETAL_HIP_ERR_HIP_RUNTIME, "hipGetSymbolAddress returned no address for the scratch array");
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return PMETAL_HIP_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -160,6 +187,8 @@ int32_t pmetal_hip_init(int32_t device) {
     if (device < 0 || device >= n) return fail(PMETAL_HIP_ERR_INVALID_ARG, "device %d out of range [0, %d)", device, n);
     HIP_TRY(hipSetDevice(device));
     HIP_TRY(hipFree(nullptr));  // forces context creation and code-object load
+    void *sp = nullptr;
+    if (int32_t rc = scratch_of_current_device(&sp)) return rc;  // so that pmetal_hip_qgemm_noalloc has nothing left to set up
     return ok();
 }
 
@@ -589,6 +618,32 @@ int32_t pmetal_hip_qgemm(uint32_t t, const uint8_t *w, int64_t n, int64_t k, con
         return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qgemm: m and k must be at most 2^22 (m = %lld, k = %lld)", (long long)m, (long long)k);
     void *ws = nullptr;
     if (int32_t rc = workspace(pmh::qgemm_workspace_bytes(m, n, k), (hipStream_t)stream, &ws)) return rc;
+    hipError_t e = pmh::launch_qgemm(t, w, n, k, x, x_dtype, m, y, y_dtype, order, ws, (hipStream_t)stream);
+    if (e == hipErrorNotSupported) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "qgemm: configuration not supported");
+    if (e != hipSuccess) return hip_fail(e, "qgemm kernel launch");
+    return ok();
+}
+
+// pmetal_hip_qgemm for callers that cannot allocate: the scratch is the fixed `scratch` array of the current device.
+// Calls no hipMalloc / hipFree and nothing else that allocates.  Every call on a device uses the same array, so calls that
+// overlap on one device race; nothing in it has to start at zero (the pre-pass writes every activation item and row scale
+// the main kernel reads, padding rows included, and a K split writes every partial tile before the reduction reads it).
+int32_t pmetal_hip_qgemm_noalloc(uint32_t t, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, int64_t m,
+                                 void *y, uint32_t y_dtype, uint32_t order, void *stream) {
+    if (gemv_only_type(t))
+        return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "qgemm_noalloc: GGML type %u goes through re-blocking, which needs scratch of the size of W", t);
+    if (int32_t rc = check_linear(t, w, n, k, x, x_dtype, y, order)) return rc;
+    if (y_dtype > PMETAL_HIP_DTYPE_BF16) return fail(PMETAL_HIP_ERR_INVALID_ARG, "y_dtype must be 0 (f32) or 1 (bf16)");
+    if (m <= 0 || m > 0x7FFFFFFF) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "m must be in [1, 2^31)");
+    if (k % 256 != 0) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qgemm: k=%lld is not a multiple of 256", (long long)k);
+    if (!pmh::qgemm_fits(t, m, n, k))
+        return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qgemm: m and k must be at most 2^22 (m = %lld, k = %lld)", (long long)m, (long long)k);
+    const size_t need = pmh::qgemm_workspace_bytes(m, n, k);
+    if (need > kNoAllocScratchBytes)
+        return fail(PMETAL_HIP_ERR_SHAPE_TOO_LARGE, "qgemm_noalloc: m=%lld, n=%lld, k=%lld needs %zu bytes of scratch, the fixed array holds %zu",
+                    (long long)m, (long long)n, (long long)k, need, kNoAllocScratchBytes);
+    void *ws = nullptr;
+    if (int32_t rc = scratch_of_current_device(&ws)) return rc;
     hipError_t e = pmh::launch_qgemm(t, w, n, k, x, x_dtype, m, y, y_dtype, order, ws, (hipStream_t)stream);
     if (e == hipErrorNotSupported) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "qgemm: configuration not supported");
     if (e != hipSuccess) return hip_fail(e, "qgemm kernel launch");
