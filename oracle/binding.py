@@ -88,8 +88,23 @@ def lib() -> C.CDLL:
             getattr(L, name).argtypes, getattr(L, name).restype = [u8p, u8p, C.c_size_t], C.c_float
         L.pmo_qmatvec_q8k.argtypes = [C.c_uint32, u8p, C.c_size_t, C.c_size_t, u8p, f32p]
         L.pmo_qmatvec_q8k.restype = C.c_int32
+        L.pmo_quantize_mt.argtypes = [C.c_uint32, f32p, C.c_size_t, u8p, C.c_size_t, C.c_int32]
+        L.pmo_quantize_mt.restype = C.c_int32
+        L.pmo_qmatvec_mt.argtypes = [C.c_uint32, u8p, C.c_size_t, C.c_size_t, f32p, f32p, C.c_uint32, C.c_int32, C.c_int32]
+        L.pmo_qmatvec_mt.restype = C.c_int32
+        L.pmo_qmatmul_f64_mt.argtypes = [C.c_uint32, u8p, C.c_size_t, C.c_size_t, f32p, C.c_size_t, f32p, C.c_uint32,
+                                         C.c_int32]
+        L.pmo_qmatmul_f64_mt.restype = C.c_int32
         _lib = L
     return _lib
+
+
+def host_threads() -> int:
+    """Threads worth starting on this host: the CPUs this process may run on."""
+    try:
+        return max(1, len(os.sched_getaffinity(0)))
+    except AttributeError:
+        return max(1, os.cpu_count() or 1)
 
 
 def _f32p(a):
@@ -104,11 +119,15 @@ def tensor_size(t: int, n: int) -> int:
     return lib().pmo_tensor_size(t, n)
 
 
-def quantize(t: int, x: np.ndarray) -> np.ndarray:
-    """quantize.rs:17 ``quantize(data, dtype)``: flat f32 -> block bytes."""
+def quantize(t: int, x: np.ndarray, threads: int = 1) -> np.ndarray:
+    """quantize.rs:17 ``quantize(data, dtype)``: flat f32 -> block bytes (``threads`` > 1: the same bytes, block ranges
+    spread over host threads)."""
     x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
     out = np.zeros(tensor_size(t, x.size), dtype=np.uint8)
-    rc = lib().pmo_quantize(t, _f32p(x), x.size, _u8p(out), out.size)
+    if threads > 1:
+        rc = lib().pmo_quantize_mt(t, _f32p(x), x.size, _u8p(out), out.size, threads)
+    else:
+        rc = lib().pmo_quantize(t, _f32p(x), x.size, _u8p(out), out.size)
     if rc != OK:
         raise ValueError(f"oracle quantize failed with code {rc}")
     return out
@@ -160,23 +179,30 @@ def get_scale_min_k4(j: int, q: np.ndarray):
 
 
 def qmatvec(t: int, w: np.ndarray, n_rows: int, k: int, x: np.ndarray, order: int = ORDER_REF,
-            acc: str = "f64") -> np.ndarray:
+            acc: str = "f64", threads: int = 1) -> np.ndarray:
     w = np.ascontiguousarray(w, dtype=np.uint8).reshape(-1)
     x = np.ascontiguousarray(x, dtype=np.float32)
     assert w.size == n_rows * tensor_size(t, k) and x.size == k
     y = np.empty(n_rows, dtype=np.float32)
-    fn = lib().pmo_qmatvec_f64 if acc == "f64" else lib().pmo_qmatvec_f32
-    rc = fn(t, _u8p(w), n_rows, k, _f32p(x), _f32p(y), order)
+    if threads > 1:
+        rc = lib().pmo_qmatvec_mt(t, _u8p(w), n_rows, k, _f32p(x), _f32p(y), order, 1 if acc == "f64" else 0, threads)
+    else:
+        fn = lib().pmo_qmatvec_f64 if acc == "f64" else lib().pmo_qmatvec_f32
+        rc = fn(t, _u8p(w), n_rows, k, _f32p(x), _f32p(y), order)
     if rc != OK:
         raise ValueError(rc)
     return y
 
 
-def qmatmul(t: int, w: np.ndarray, n_rows: int, k: int, x: np.ndarray, order: int = ORDER_REF) -> np.ndarray:
+def qmatmul(t: int, w: np.ndarray, n_rows: int, k: int, x: np.ndarray, order: int = ORDER_REF,
+            threads: int = 1) -> np.ndarray:
     w = np.ascontiguousarray(w, dtype=np.uint8).reshape(-1)
     x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, k)
     y = np.empty((x.shape[0], n_rows), dtype=np.float32)
-    rc = lib().pmo_qmatmul_f64(t, _u8p(w), n_rows, k, _f32p(x), x.shape[0], _f32p(y), order)
+    if threads > 1:
+        rc = lib().pmo_qmatmul_f64_mt(t, _u8p(w), n_rows, k, _f32p(x), x.shape[0], _f32p(y), order, threads)
+    else:
+        rc = lib().pmo_qmatmul_f64(t, _u8p(w), n_rows, k, _f32p(x), x.shape[0], _f32p(y), order)
     if rc != OK:
         raise ValueError(rc)
     return y

@@ -28,6 +28,7 @@
 #include "pmetal_oracle.h"
 
 #include <math.h>
+#include <pthread.h>
 #include <stdlib.h>
 #include <string.h>
 
@@ -1280,4 +1281,109 @@ int32_t pmo_qmatmul_f64(uint32_t t, const uint8_t *w, size_t n_rows, size_t k, c
     }
     free(tmp);
     return PMO_OK;
+}
+
+/* ------------------------------------------------------------------------- */
+/* The same functions over several host threads.  The reference runs this path */
+/* on one thread (no rayon in crates/pmetal-gguf); these exist so that whole    */
+/* tensors can be checked in a test's time budget and so that the benchmark can */
+/* report an all-cores CPU figure beside the single-thread one.  Every thread   */
+/* calls the single-threaded function above on its own range of blocks or rows, */
+/* so the results are the single-threaded ones bit for bit.                     */
+/* ------------------------------------------------------------------------- */
+typedef struct {
+    int kind; /* 0 quantize, 1 matvec f32, 2 matvec f64, 3 matmul f64 */
+    uint32_t t, order;
+    const float *x;
+    const uint8_t *w;
+    uint8_t *dst;
+    float *y;
+    size_t lo, hi, n, k, m_rows, n_rows;
+} mt_job;
+
+static void *mt_run(void *arg) {
+    mt_job *j = (mt_job *)arg;
+    if (j->kind == 0) { /* blocks [lo, hi) of a flat tensor of n elements */
+        size_t bs = pmo_block_size(j->t), ts = pmo_type_size(j->t);
+        size_t e0 = j->lo * bs, e1 = j->hi * bs < j->n ? j->hi * bs : j->n;
+        (void)pmo_quantize(j->t, j->x + e0, e1 - e0, j->dst + j->lo * ts, pmo_tensor_size(j->t, e1 - e0));
+    } else if (j->kind == 1 || j->kind == 2) { /* rows [lo, hi) */
+        size_t row_bytes = pmo_tensor_size(j->t, j->k);
+        if (j->kind == 1) (void)pmo_qmatvec_f32(j->t, j->w + j->lo * row_bytes, j->hi - j->lo, j->k, j->x, j->y + j->lo, j->order);
+        else (void)pmo_qmatvec_f64(j->t, j->w + j->lo * row_bytes, j->hi - j->lo, j->k, j->x, j->y + j->lo, j->order);
+    } else { /* rows [lo, hi) of W against every activation row */
+        float *tmp = (float *)malloc(j->k * sizeof(float));
+        if (!tmp) return NULL;
+        for (size_t r = j->lo; r < j->hi; r++) {
+            dequant_row(j->t, j->w, r, j->k, tmp, j->order);
+            for (size_t m = 0; m < j->m_rows; m++) {
+                const float *xr = j->x + m * j->k;
+                double acc = 0.0;
+                for (size_t i = 0; i < j->k; i++) acc += (double)tmp[i] * (double)xr[i];
+                j->y[m * j->n_rows + r] = (float)acc;
+            }
+        }
+        free(tmp);
+    }
+    return NULL;
+}
+
+static int32_t mt_dispatch(mt_job proto, size_t units, int32_t threads) {
+    if (threads < 1) threads = 1;
+    if ((size_t)threads > units) threads = units ? (int32_t)units : 1;
+    pthread_t *th = (pthread_t *)malloc(sizeof(pthread_t) * (size_t)threads);
+    mt_job *jobs = (mt_job *)malloc(sizeof(mt_job) * (size_t)threads);
+    if (!th || !jobs) {
+        free(th);
+        free(jobs);
+        return PMO_ERR_SHAPE_TOO_LARGE;
+    }
+    int started = 0;
+    for (int i = 0; i < threads; i++) {
+        jobs[i] = proto;
+        jobs[i].lo = units * (size_t)i / (size_t)threads;
+        jobs[i].hi = units * (size_t)(i + 1) / (size_t)threads;
+        if (pthread_create(&th[i], NULL, mt_run, &jobs[i]) != 0) break;
+        started++;
+    }
+    for (int i = started; i < threads; i++) { /* could not start: run the rest here */
+        jobs[i] = proto;
+        jobs[i].lo = units * (size_t)i / (size_t)threads;
+        jobs[i].hi = units * (size_t)(i + 1) / (size_t)threads;
+        mt_run(&jobs[i]);
+    }
+    for (int i = 0; i < started; i++) pthread_join(th[i], NULL);
+    free(th);
+    free(jobs);
+    return PMO_OK;
+}
+
+int32_t pmo_quantize_mt(uint32_t t, const float *x, size_t n, uint8_t *dst, size_t dst_len, int32_t threads) {
+    size_t bs = pmo_block_size(t);
+    if (bs == 0 || t == PMO_TYPE_F32 || t == PMO_TYPE_F16) return PMO_ERR_UNSUPPORTED_TYPE;
+    if (dst_len != pmo_tensor_size(t, n)) return PMO_ERR_INVALID_SIZE;
+    mt_job j;
+    memset(&j, 0, sizeof j);
+    j.kind = 0, j.t = t, j.x = x, j.dst = dst, j.n = n;
+    return mt_dispatch(j, (n + bs - 1) / bs, threads);
+}
+
+int32_t pmo_qmatvec_mt(uint32_t t, const uint8_t *w, size_t n_rows, size_t k, const float *x, float *y, uint32_t order,
+                       int32_t f64_acc, int32_t threads) {
+    size_t bs = pmo_block_size(t);
+    if (bs <= 1 || k % bs != 0) return PMO_ERR_INVALID_SHAPE;
+    mt_job j;
+    memset(&j, 0, sizeof j);
+    j.kind = f64_acc ? 2 : 1, j.t = t, j.order = order, j.w = w, j.x = x, j.y = y, j.k = k;
+    return mt_dispatch(j, n_rows, threads);
+}
+
+int32_t pmo_qmatmul_f64_mt(uint32_t t, const uint8_t *w, size_t n_rows, size_t k, const float *x, size_t m_rows, float *y,
+                           uint32_t order, int32_t threads) {
+    size_t bs = pmo_block_size(t);
+    if (bs <= 1 || k % bs != 0) return PMO_ERR_INVALID_SHAPE;
+    mt_job j;
+    memset(&j, 0, sizeof j);
+    j.kind = 3, j.t = t, j.order = order, j.w = w, j.x = x, j.y = y, j.k = k, j.m_rows = m_rows, j.n_rows = n_rows;
+    return mt_dispatch(j, n_rows, threads);
 }

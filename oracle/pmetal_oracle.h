@@ -152,6 +152,14 @@ int32_t pmo_qmatvec_f32(uint32_t ggml_type, const uint8_t *w, size_t n_rows, siz
 int32_t pmo_qmatmul_f64(uint32_t ggml_type, const uint8_t *w, size_t n_rows, size_t k,
                         const float *x, size_t m_rows, float *y, uint32_t order);
 
+/* The functions above over `threads` host threads (ranges of blocks or of rows; bit-identical to the single-threaded
+ * results).  Not how the reference runs (it is single-threaded): for whole-tensor tests and the all-cores CPU figure. */
+int32_t pmo_quantize_mt(uint32_t ggml_type, const float *x, size_t n, uint8_t *dst, size_t dst_len, int32_t threads);
+int32_t pmo_qmatvec_mt(uint32_t ggml_type, const uint8_t *w, size_t n_rows, size_t k, const float *x, float *y,
+                       uint32_t order, int32_t f64_acc, int32_t threads);
+int32_t pmo_qmatmul_f64_mt(uint32_t ggml_type, const uint8_t *w, size_t n_rows, size_t k, const float *x, size_t m_rows,
+                           float *y, uint32_t order, int32_t threads);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,7 +1,7 @@
-"""GPU parity at the full sizes of the measured configurations, verified on samples the CPU oracle can afford:
-the Llama-3-8B-shaped quantizer input (every distinct tensor shape and type of the Q4_K_M recipe, generated on
-the device, first / middle / last slices compared bit for bit) and the Qwen3-0.6B-shaped decode step (one
-layer of every recipe variant plus the output projection against dequantize-then-matmul)."""
+"""GPU parity at the full sizes of the measured configurations: the Llama-3-8B-shaped quantizer input (every distinct
+tensor shape and type of the Q4_K_M recipe, generated on the device, every super-block compared bit for bit with the
+oracle run on all host threads) and the Qwen3-0.6B-shaped decode step (one layer of every recipe variant plus the output
+projection against dequantize-then-matmul)."""
 import numpy as np
 import pytest
 
@@ -38,10 +38,30 @@ OTHER_TYPES = [("blk.4.attn_qkv", 6144, 4096, 13), ("calibrate.q8k", 14336, 4096
                ("calibrate.q3k", 14336, 4096, 11), ("calibrate.q2k", 14336, 4096, 10)]
 
 
+def _oracle_dequantize_threads(oracle, t, raw, n, threads):
+    """The oracle's dequantizer over ranges of super-blocks on several host threads (ctypes releases the GIL)."""
+    from concurrent.futures import ThreadPoolExecutor
+    sbs = n // 256
+    out = np.empty(n, np.float32)
+    edges = [sbs * i // threads for i in range(threads + 1)]
+
+    def work(i):
+        a, b = edges[i], edges[i + 1]
+        if b > a:
+            out[a * 256:b * 256] = oracle.dequantize(t, raw[a * BLOCK[t]:b * BLOCK[t]], [(b - a) * 256])
+
+    with ThreadPoolExecutor(threads) as pool:
+        list(pool.map(work, range(threads)))
+    return out
+
+
 @pytest.mark.parametrize("name,rows,cols,t", LLAMA3_8B + OTHER_TYPES, ids=[x[0] for x in LLAMA3_8B + OTHER_TYPES])
-def test_quantize_full_size_tensor_sampled(oracle, name, rows, cols, t):
+def test_quantize_full_size_tensor_whole(oracle, name, rows, cols, t):
+    """Every super-block of the tensor: the device's bytes against the oracle's (run on all host threads), then the device's
+    dequantized values of those bytes against the oracle's, bit for bit."""
     lib = _lib.load()
     n = rows * cols
+    threads = min(oracle.host_threads(), 16)
     if not name.startswith("calibrate"):
         assert int(pm.q4km_tensor_type(name + ".weight", 2, 32)) == t
     x = pm.DeviceBuffer(4 * n)
@@ -52,21 +72,17 @@ def test_quantize_full_size_tensor_sampled(oracle, name, rows, cols, t):
     pm.check(lib.pmetal_hip_memset(q.ptr, 0xA5, nbytes, None))
     pm.check(lib.pmetal_hip_quantize_dev(t, x.ptr, n, q.ptr, nbytes, None), "quantize")
     pm.check(lib.pmetal_hip_sync(None))
-    sbs = n // 256
-    span = 1024  # super-blocks per sample
-    for sb0 in (0, (sbs // 2) // 8 * 8 + 3, sbs - span):
-        xin = _d2h(lib, x.ptr, sb0 * 256 * 4, span * 256 * 4, np.float32)
-        got = _d2h(lib, q.ptr, sb0 * BLOCK[t], span * BLOCK[t], np.uint8)
-        want = oracle.quantize(t, xin)
-        assert np.array_equal(got, want), f"{name} super-block {sb0 + first_mismatch(got, want, BLOCK[t])}"
-    # dequantize the whole tensor in place of x and check the same samples
+    xin = _d2h(lib, x.ptr, 0, 4 * n, np.float32)
+    got = _d2h(lib, q.ptr, 0, nbytes, np.uint8)
+    want = oracle.quantize(t, xin, threads=threads)
+    assert np.array_equal(got, want), f"{name}: {first_mismatch(got, want, BLOCK[t])}"
+    del xin, want
+    # dequantize the whole tensor in place of x
     pm.check(lib.pmetal_hip_dequantize_dev(t, q.ptr, nbytes, x.ptr, n, 0, None))
     pm.check(lib.pmetal_hip_sync(None))
-    for sb0 in (0, sbs - span):
-        raw = _d2h(lib, q.ptr, sb0 * BLOCK[t], span * BLOCK[t], np.uint8)
-        got = _d2h(lib, x.ptr, sb0 * 256 * 4, span * 256 * 4, np.float32)
-        want = oracle.dequantize(t, raw, [span * 256])
-        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    deq = _d2h(lib, x.ptr, 0, 4 * n, np.float32)
+    want = _oracle_dequantize_threads(oracle, t, got, n, threads)
+    assert np.array_equal(deq.view(np.uint32), want.view(np.uint32)), name
 
 
 def test_decode_step_projections_against_oracle(oracle):

@@ -94,18 +94,45 @@ def test_qgemm_f32_activations(oracle, t, m):
         assert norm <= TOL and elem_r <= TOL and norm_r <= TOL, (row, norm, elem_r, norm_r)
 
 
-def test_qgemm_config2_full_size(oracle):
-    # BASELINE config 2: M = 512, K = 4096, N = 14336, bf16 activations ~ N(0, 1)
-    m, n, k = 512, 14336, 4096
-    wq = pm.quantize(weights(31, n * k), Q4K)
-    x = np.random.default_rng(32).standard_normal((m, k)).astype(np.float32)
+@pytest.fixture(scope="module")
+def config2_weights(oracle):
+    """The 14336 x 4096 Q4_K weight of the GEMM configuration: quantized on the device, and every byte compared with the
+    oracle's quantizer (run on all host threads) before any product is taken."""
+    n, k = 14336, 4096
+    w = weights(31, n * k)
+    wq = pm.quantize(w, Q4K)
+    want = oracle.quantize(Q4K, w, threads=min(oracle.host_threads(), 16))
+    assert np.array_equal(wq, want)
+    return wq
+
+
+@pytest.mark.parametrize("m", [16, 64, 128, 512, 2048])
+def test_qgemm_config2_full_size(oracle, config2_weights, m):
+    """M = 512 and the sweep 16 / 64 / 128 / 2048 at K = 4096, N = 14336, bf16 activations ~ N(0, 1).  The f64 reference covers
+    every activation row against 1152 weight rows (the first and last 64 and 1024 drawn at random): all of the kernel's
+    code paths for the shape (K split and partial-tile reduction for few rows, 128-row workgroups and the four-row
+    pre-pass for many) contribute to every output column alike."""
+    n, k = 14336, 4096
+    wq = config2_weights
+    x = np.random.default_rng(32 + m).standard_normal((m, k)).astype(np.float32)
     bits = oracle.f32_to_bf16_bits(x.reshape(-1)).reshape(m, k)
     xr = oracle.bf16_bits_to_f32(bits.reshape(-1)).reshape(m, k)
-    want = reference(oracle, Q4K, wq, n, k, xr, 0)
     got = gpu_qgemm(Q4K, wq, n, k, bits, m)
-    elem, norm = rel_errors(got.reshape(-1), want.reshape(-1))
-    print(f"Q4_K GEMM 512x14336x4096: elem {elem:.2e} norm {norm:.2e}")
+    assert np.isfinite(got).all()
+    rows = np.unique(np.concatenate([np.arange(64), np.arange(n - 64, n),
+                                     np.random.default_rng(m).choice(n, 1024, replace=False)]))
+    row_bytes = k // 256 * 144
+    sub = wq.reshape(n, row_bytes)[rows].reshape(-1)
+    want = oracle.qmatmul(Q4K, sub, rows.size, k, xr, threads=min(oracle.host_threads(), 16))
+    elem, norm = rel_errors(got[:, rows].reshape(-1), want.reshape(-1))
+    print(f"Q4_K GEMM {m}x14336x4096: elem {elem:.2e} norm {norm:.2e} over {rows.size} weight rows")
     assert elem <= TOL and norm <= TOL
+    # every column, cheaply: row 0 of the product is the GEMV of activation row 0 (itself checked against the oracle at
+    # this shape in the GEMV tests)
+    from gpu_util import gpu_qgemv
+    y0 = gpu_qgemv(Q4K, wq, n, k, bits[0], pm.DTYPE_BF16)
+    e0, n0 = rel_errors(got[0], y0)
+    assert n0 <= 1e-4, (e0, n0)
 
 
 def test_qgemm_agrees_with_qgemv_and_qlinear_dispatch(oracle):
