@@ -304,20 +304,19 @@ __device__ __forceinline__ void stage_x_finish(const void *xg, int slots, int nt
 // The workgroup has KS * G waves: wave (g, h) takes chunk h of the rows of row group g, 64/T rows per task,
 // so every task of a wave needs the same x digits, which stay in registers.  Up to kDepth tasks are in
 // flight per wave; every load is issued unconditionally (tasks past the end read the first bytes of W, all
-// lanes the same address) so that the number of outstanding loads is known at every wait.  Each lane's
-// partial sum goes to LDS; after a barrier the workgroup adds up the partials of each of its rows.
+// lanes the same address) so that the number of outstanding loads is known at every wait.  A task's lane sums
+// are added up inside the wave (DPP) and the team's last lane drops one float per row and chunk into LDS; after
+// a barrier one thread per row adds the KS chunk sums and the workgroup stores its rows of y with one coalesced
+// store.  (Keeping every lane's partial in LDS and adding them up after the barrier cost 0.5 us per launch at
+// 14336 x 4096; stores inside the streaming loop are worse: on this target they share the loads' counter, and
+// the counted waits degenerate.)
 constexpr int kDepth = 8;  // tasks in flight per wave
-constexpr int kPre = 2;  // of which this many are requested before x is converted
-
-// Row stride of the partial sums in LDS.  The final summation puts `red` lanes on a row (lane p adds every
-// red-th partial), 64 / red rows side by side in a wave: a stride of `red` floats past a multiple of 64 keeps
-// those rows in different banks.
-__host__ __device__ constexpr int part_stride(int slots, int red) { return ((slots + 63) / 64) * 64 + (red & 63); }
+constexpr int kPre = 2;    // of which this many are requested before x is converted
 
 template <int ORDER, bool XF32, int T, bool SINGLE, bool PAIR>
 __global__ __launch_bounds__(1024) void k_qgemv_q4k_chunk(const uint8_t *__restrict__ W0, const uint8_t *__restrict__ W1,
                                                            const void *__restrict__ xg, int split_wg, int n_rows0, int n_rows1,
-                                                           int spr, int rows_per_wg, int rows_per_wave, int n_nominal, int red,
+                                                           int spr, int rows_per_wg, int rows_per_wave, int n_nominal,
                                                            int nthreads, float *__restrict__ y0, float *__restrict__ y1) {
     // (the arguments needed before the first weight request come first: the leading 16 dwords of the kernel-argument
     // segment are preloaded into scalar registers at wave launch)
@@ -336,8 +335,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q4k_chunk(const uint8_t *__restr
     const int slots = spr * 8;
     uint4 *xd = smem;
     float4 *xm = reinterpret_cast<float4 *>(xd + NDIG * slots);
-    float *part = reinterpret_cast<float *>(xm + slots);  // [group][n_nominal * RPT][part_stride(slots)]
-    const int ps = part_stride(slots, red);
+    float *part = reinterpret_cast<float *>(xm + slots);  // [group][n_nominal * RPT][ks]
     const int lane = threadIdx.x & 63;
     const int lt = lane & (T - 1), tm = lane / T, j = lane & 7;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -377,13 +375,16 @@ __global__ __launch_bounds__(1024) void k_qgemv_q4k_chunk(const uint8_t *__restr
     for (int k = 0; k < NDIG; k++) xr[k] = xd[k * slots + h * T + lt];
     const float4 xmr = xm[h * T + lt];
 
-    // partial sums: row (g, t * RPT + tm) of the padded layout, column h * T + lt
+    // chunk sums: row (g, t * RPT + tm) of the padded layout, column h
     const int npad = n_nominal * RPT;
-    float *pp = part + (size_t)(g * npad + tm) * ps + h * T + lt;
-    const int pstride = RPT * ps;  // floats between consecutive tasks
+    float *pp = part + (size_t)(g * npad + tm) * ks + h;
+    const int pstride = RPT * ks;  // floats between consecutive tasks
 
     auto consume = [&](int t, const uint4 &h4, const uint4 &q4) {
-        if (t < nt_wave) pp[(size_t)t * pstride] = lane_dot<ORDER, NDIG>(h4, q4, s0, s1, xr, xmr);
+        if (t < nt_wave) {
+            const float v = team_sum_last<T>(lane_dot<ORDER, NDIG>(h4, q4, s0, s1, xr, xmr));
+            if (lt == T - 1) pp[(size_t)t * pstride] = v;
+        }
     };
 
     // First round: the ring fills up while the first tasks are consumed (two requests per task consumed),
@@ -413,30 +414,14 @@ __global__ __launch_bounds__(1024) void k_qgemv_q4k_chunk(const uint8_t *__restr
     }
     __syncthreads();
 
-    // Row totals: `red` lanes per row (a power of two from 8 to 64 that divides slots), lane p adding every
-    // red-th partial, then a sum over the lanes of the row.
+    // Row totals: one thread per row adds the row's chunk sums in chunk order.
     const int wg_rows = wg_r1 - wg_r0;
-    const int per_thread = slots / red;
-    const int red_shift = 31 - __builtin_clz(red);
-    for (int idx0 = 0; idx0 < wg_rows * red; idx0 += nthreads) {
-        const int idx = idx0 + threadIdx.x;
-        int rl = idx >> red_shift;
-        const bool ok = rl < wg_rows;
-        rl = ok ? rl : wg_rows - 1;
+    for (int rl = (int)threadIdx.x; rl < wg_rows; rl += nthreads) {
         const int grp = rl / rows_per_wave, loc = rl - grp * rows_per_wave;
-        const int p = idx & (red - 1);
-        const float *src = part + (size_t)(grp * npad + loc) * ps + p;
-        float t0 = 0.0f, t1 = 0.0f, t2 = 0.0f, t3 = 0.0f;
-        int i = 0;
-        for (; i + 8 <= per_thread; i += 8) {  // eight reads in flight
-            const float *q = src + (size_t)i * red;
-            const float a0 = q[0], a1 = q[red], a2 = q[2 * red], a3 = q[3 * red];
-            const float a4 = q[4 * red], a5 = q[5 * red], a6 = q[6 * red], a7 = q[7 * red];
-            t0 += a0 + a4, t1 += a1 + a5, t2 += a2 + a6, t3 += a3 + a7;
-        }
-        for (; i < per_thread; i++) t0 += src[(size_t)i * red];
-        const float sum = team_sum_rt((t0 + t1) + (t2 + t3), red);
-        if (ok && p == 0) y[wg_r0 + rl] = sum;
+        const float *src = part + (size_t)(grp * npad + loc) * ks;
+        float sum = src[0];
+        for (int i = 1; i < ks; i++) sum += src[i];
+        y[wg_r0 + rl] = sum;
     }
 }
 
@@ -564,18 +549,18 @@ hipError_t launch_with_lds(Kern kern, dim3 grid, dim3 block, size_t lds, hipStre
 
 template <int ORDER, bool XF32>
 hipError_t launch_chunk(int T, bool single, dim3 grid, dim3 block, size_t lds, hipStream_t s, const uint8_t *w,
-                        const void *x, float *y, int n, int spr, int rows_per_wg, int rows_per_wave, int n_nominal, int red,
+                        const void *x, float *y, int n, int spr, int rows_per_wg, int rows_per_wave, int n_nominal,
                         const uint8_t *w1, int split_wg, float *y1, int n1) {
 #define PMH_GO(TT)                                                                                                       \
     if (n1 > 0)                                                                                                                    \
         return single ? launch_with_lds(k_qgemv_q4k_chunk<ORDER, XF32, TT, true, true>, grid, block, lds, s, w, w1, x, split_wg, n, n1,  \
-                                        spr, rows_per_wg, rows_per_wave, n_nominal, red, (int)block.x, y, y1)                      \
+                                        spr, rows_per_wg, rows_per_wave, n_nominal, (int)block.x, y, y1)                      \
                       : launch_with_lds(k_qgemv_q4k_chunk<ORDER, XF32, TT, false, true>, grid, block, lds, s, w, w1, x, split_wg, n, n1, \
-                                        spr, rows_per_wg, rows_per_wave, n_nominal, red, (int)block.x, y, y1);                     \
+                                        spr, rows_per_wg, rows_per_wave, n_nominal, (int)block.x, y, y1);                     \
     return single ? launch_with_lds(k_qgemv_q4k_chunk<ORDER, XF32, TT, true, false>, grid, block, lds, s, w, w1, x, split_wg, n, n1,     \
-                                    spr, rows_per_wg, rows_per_wave, n_nominal, red, (int)block.x, y, y1)                          \
+                                    spr, rows_per_wg, rows_per_wave, n_nominal, (int)block.x, y, y1)                          \
                   : launch_with_lds(k_qgemv_q4k_chunk<ORDER, XF32, TT, false, false>, grid, block, lds, s, w, w1, x, split_wg, n, n1,    \
-                                    spr, rows_per_wg, rows_per_wave, n_nominal, red, (int)block.x, y, y1)
+                                    spr, rows_per_wg, rows_per_wave, n_nominal, (int)block.x, y, y1)
     switch (T) {
     case 8: PMH_GO(8);
     case 16: PMH_GO(16);
@@ -673,9 +658,7 @@ static hipError_t launch_kernel_a(const uint8_t *w0, int64_t n0, float *y0, cons
     groups = (rows_per_wg + rows_per_wave - 1) / rows_per_wave;
     const int64_t n_nominal = (rows_per_wave + rpt - 1) / rpt;
     const int64_t threads = ks * groups * 64;
-    int red = 8;  // lanes per row in the final summation: as many as the workgroup has to spare, at most T
-    while (red < 64 && red * 2 <= T && rows_per_wg * red * 2 <= threads) red *= 2;
-    const size_t lds = lds_x + (size_t)groups * (size_t)n_nominal * rpt * part_stride((int)slots, red) * 4;
+    const size_t lds = lds_x + (size_t)groups * (size_t)n_nominal * rpt * ks * 4;
     if (lds > 128 * 1024) return hipErrorNotSupported;
     const dim3 block((unsigned)threads);
     const bool single = n_nominal <= kDepth;
@@ -684,10 +667,10 @@ static hipError_t launch_kernel_a(const uint8_t *w0, int64_t n0, float *y0, cons
     float *b_y = n1 ? y1 : y0;
     const int b_split = (int)wg0, b_n = (int)n1;
     if (order == kOrderRef)
-        return xf32 ? launch_chunk<0, true>(T, single, grid, block, lds, s, w0, x, y0, a_n, spr, a_rpw, a_rpv, a_nn, red, b_w, b_split, b_y, b_n)
-                    : launch_chunk<0, false>(T, single, grid, block, lds, s, w0, x, y0, a_n, spr, a_rpw, a_rpv, a_nn, red, b_w, b_split, b_y, b_n);
-    return xf32 ? launch_chunk<1, true>(T, single, grid, block, lds, s, w0, x, y0, a_n, spr, a_rpw, a_rpv, a_nn, red, b_w, b_split, b_y, b_n)
-                : launch_chunk<1, false>(T, single, grid, block, lds, s, w0, x, y0, a_n, spr, a_rpw, a_rpv, a_nn, red, b_w, b_split, b_y, b_n);
+        return xf32 ? launch_chunk<0, true>(T, single, grid, block, lds, s, w0, x, y0, a_n, spr, a_rpw, a_rpv, a_nn, b_w, b_split, b_y, b_n)
+                    : launch_chunk<0, false>(T, single, grid, block, lds, s, w0, x, y0, a_n, spr, a_rpw, a_rpv, a_nn, b_w, b_split, b_y, b_n);
+    return xf32 ? launch_chunk<1, true>(T, single, grid, block, lds, s, w0, x, y0, a_n, spr, a_rpw, a_rpv, a_nn, b_w, b_split, b_y, b_n)
+                : launch_chunk<1, false>(T, single, grid, block, lds, s, w0, x, y0, a_n, spr, a_rpw, a_rpv, a_nn, b_w, b_split, b_y, b_n);
 }
 
 // Preconditions as for launch_qgemv.  Returns hipErrorInvalidValue when x does not fit in LDS.
