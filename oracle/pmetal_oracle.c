@@ -13,14 +13,21 @@
  *   nearest_int ........... reference KATs quantize.rs:862-868.
  *   get_scale_min_k4 ...... reference KATs quantize.rs:1035-1047,
  *                           k_quants.rs:1386-1396; pack/unpack identity.
- *   make_qkx1_quants ...... closed forms (reference tests quantize.rs:998-1017)
- *                           + independent numpy-float32 twin. Restatement-pinned.
- *   make_qx_quants ........ closed forms + invariants + numpy twin.
- *                           Restatement-pinned.
+ *   make_qkx1_quants, make_qx_quants, make_q3_quants
+ *                           a restatement of the same Rust in rational arithmetic
+ *                           (tests/exact_ref.py: fractions.Fraction, one IEEE-754
+ *                           rounding per operation) gives the expected bits for
+ *                           tests/golden/exact_cases.json: inputs whose sums are exact
+ *                           in any order (2, 3, 4 and 5 tries; rescale passes taken
+ *                           and refused; single-element moves taken and refused;
+ *                           every exit) and Gaussian inputs in the reference's order.
+ *                           Also the reference's closed forms (quantize.rs:998-1032).
  *   quantize_q8_0 ......... fully determined by IEEE ops: numpy twin is exact.
- *   quantize_q4k/q6k ...... block sizes, reference round-trip bounds
- *                           (k_quants.rs:1446-1509), invariants, numpy twin.
- *                           Restatement-pinned (bytes never compared with Rust).
+ *   quantize_q4k/q5k/q6k/q3k/q2k
+ *                           whole super-blocks built from those inputs with bytes
+ *                           derived by the rational restatement (same fixture); block
+ *                           sizes, reference round-trip bounds (k_quants.rs:1446-1553).
+ *                           The Rust itself was never run (no toolchain here).
  *   dequantize_* .......... reference KATs (dequant.rs:1016-1036,
  *                           k_quants.rs:1368-1383) + hand-built blocks + numpy.
  *   recipe ................ reference KATs commands/quantize.rs:1561-1608.

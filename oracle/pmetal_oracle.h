@@ -8,21 +8,21 @@
  * Every function follows one function of the reference (Epistates/pmetal,
  * crate pmetal-gguf) and cites it as file:line relative to the reference root.
  * The reference is Rust and cannot be compiled in this environment, so the
- * oracle is pinned by the reference's own known-answer tests, by closed forms
- * and by an independent numpy-float32 re-derivation (see tests/).  The bytes of
- * quantize_q4k / quantize_q6k on general inputs are therefore pinned by the
- * fidelity of this restatement and the independent twin only, never by running
- * the Rust: "restatement-pinned".
- *
- * PARITY UNPINNED (no fixture of the reference and no closed form fixes the
- * result bit for bit on general input; pinned on exact-grid, zero, partial and
- * hand-derived blocks, by invariants and by the twin only):
- *   pmo_make_qkx1_quants, pmo_make_qx_quants, pmo_make_q3_quants and the bytes of
- *   pmo_quantize_q4k, pmo_quantize_q5k, pmo_quantize_q6k, pmo_quantize_q3k,
- *   pmo_quantize_q2k.
- * Pinned by the reference's known answers or by closed forms: everything else
- * (nearest_int, the 6-bit scale packing, Q8_0 and Q8_K, every dequantizer, the
- * integer dot products, the calibration score, the recipe, the matrix products).
+ * oracle is pinned without it: by the reference's own known-answer tests, by
+ * closed forms, and -- for the order-sensitive scale searches and the bytes of
+ * the k-quant quantizers -- by expected values that a second restatement of the
+ * same Rust in rational arithmetic produces (tests/exact_ref.py ->
+ * tests/golden/exact_cases.json, checked in tests/test_exact_pins.py):
+ *   pmo_make_qkx1_quants, pmo_make_qx_quants, pmo_make_q3_quants: inputs whose
+ *     sums are exact in any order, so that the result follows from the algorithm's
+ *     definition (2 to 5 tries, accepted and refused rescale passes and moves,
+ *     every early exit), plus Gaussian inputs with one rounding per operation in
+ *     the reference's order;
+ *   pmo_quantize_q4k / _q5k / _q6k / _q3k / _q2k: whole super-blocks built from
+ *     those inputs.
+ * What stays unpinned in the strict sense: nothing was ever compared with output
+ * of the Rust itself; a misreading of the Rust shared by the C restatement and
+ * the rational one (written separately, from the Rust) would pass.
  */
 #ifndef PMETAL_ORACLE_H
 #define PMETAL_ORACLE_H
