@@ -12,7 +12,11 @@ Timing: HIP events recorded on the stream the kernels are launched on (the null 
 stream synchronisation; inputs are resident in HBM before the timed region.  `roofline.achieved` is
 algorithmic bytes (or flops) per launch divided by the average launch duration over the timed region.
 The CPU baseline is the oracle's restatement of the reference algorithm (dequantize, then an f32
-dot product; single thread, as the reference runs) on a bounded sample of the same workload.
+dot product) on a bounded sample of the same workload: `value` on one thread, as the reference runs
+it, and `all_cores` with the rows / blocks spread over every host thread; `host` names the machine.
+
+The default invocation also times the other two parts of the headline metric (the Q4_K GEMM at M = 512 and
+the f32 -> Q4_K_M quantizer) and a plain read of the same bytes, and reports them under `extra`.
 """
 import argparse
 import ctypes as C
@@ -28,10 +32,11 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled against a streaming
-# kernel of known size (summary and commands: profiles/qgemv_q4k_14336x4096.md)
-MEASURED_TRAFFIC = {"gemv_q4k_14336x4096": 33293144, "gemv_q6k_14336x4096": 48531385,
-                    "gemv_q8_0_14336x4096": 62642111}
+# HBM bytes per launch as recorded from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled against a streaming kernel
+# of known size; constants taken from the profile summaries named here, not measured by this script
+RECORDED_TRAFFIC = {"gemv_q4k_14336x4096": (33293144, "profiles/qgemv_q4k_14336x4096.md"),
+                    "gemv_q6k_14336x4096": (48531385, "profiles/qgemv_q6k_q8_0_14336x4096.md"),
+                    "gemv_q8_0_14336x4096": (62642111, "profiles/qgemv_q6k_q8_0_14336x4096.md")}
 BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16/fp16 MFMA, published
 Q8_0, Q4K, Q6K = 8, 12, 14
 
@@ -89,7 +94,38 @@ def gemv_bytes(t, n, k, x_bytes):
     return n * (k // per_block[1]) * per_block[0] + k * x_bytes + n * 4
 
 
-def cpu_baseline_gemv(t, n, k, budget_s=12.0):
+def host_description():
+    """Logical CPUs of the host, the CPUs this process may use, and the CPU model."""
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count() or 1
+    return {"nproc": os.cpu_count() or 1, "usable_cpus": usable, "cpu_model": model}
+
+
+def baseline_threads():
+    """Threads of the all-cores leg: the CPUs this process may use, at most 64."""
+    return max(1, min(host_description()["usable_cpus"], 64))
+
+
+def timed_reps(fn, budget_s):
+    reps, t0 = 0, time.perf_counter()
+    while reps == 0 or time.perf_counter() - t0 < budget_s:
+        fn()
+        reps += 1
+    return reps, time.perf_counter() - t0
+
+
+def cpu_baseline_gemv(t, n, k, budget_s=6.0):
     """Oracle: reference dequantize + sequential f32 dot, one thread, on whole rows of the same shape."""
     from oracle import binding as oracle
     oracle.build()
@@ -99,17 +135,18 @@ def cpu_baseline_gemv(t, n, k, budget_s=12.0):
     wq = oracle.quantize(t, w)
     x = oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(rng.standard_normal(k).astype(np.float32)))
     oracle.qmatvec(t, wq, rows, k, x, acc="f32")
-    reps, t0 = 0, time.perf_counter()
-    while time.perf_counter() - t0 < budget_s:
-        oracle.qmatvec(t, wq, rows, k, x, acc="f32")
-        reps += 1
-    dt = time.perf_counter() - t0
+    reps, dt = timed_reps(lambda: oracle.qmatvec(t, wq, rows, k, x, acc="f32"), budget_s)
     gbs = gemv_bytes(t, rows, k, 2) * reps / dt / 1e9
+    th = baseline_threads()
+    reps_mt, dt_mt = timed_reps(lambda: oracle.qmatvec(t, wq, rows, k, x, acc="f32", threads=th), budget_s / 2)
     return {"value": round(gbs, 3), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"{reps} x (dequantize + f32 matvec) of {rows}x{k} rows of the same shape, {dt:.1f} s"}
+            "sample": f"{reps} x (dequantize + f32 matvec) of {rows}x{k} rows of the same shape, {dt:.1f} s",
+            "all_cores": {"value": round(gemv_bytes(t, rows, k, 2) * reps_mt / dt_mt / 1e9, 3), "unit": "GB/s", "cores": th,
+                          "sample": f"{reps_mt} x the same rows spread over {th} threads, {dt_mt:.1f} s"},
+            "host": host_description()}
 
 
-def cpu_baseline_quantize(budget_s=12.0):
+def cpu_baseline_quantize(budget_s=6.0):
     """Oracle: the reference's quantizers, one thread, on f32 tensors in the model's Q4_K : Q6_K element ratio."""
     from oracle import binding as oracle
     oracle.build()
@@ -117,14 +154,19 @@ def cpu_baseline_quantize(budget_s=12.0):
     x4 = (rng.standard_normal(3 << 18) * 0.02).astype(np.float32)   # 786432 elements to Q4_K
     x6 = (rng.standard_normal(1 << 18) * 0.02).astype(np.float32)   # 262144 elements to Q6_K (the recipe's 26 %)
     oracle.quantize(Q4K, x4[:4096]), oracle.quantize(Q6K, x6[:4096])
-    reps, t0 = 0, time.perf_counter()
-    while time.perf_counter() - t0 < budget_s:
-        oracle.quantize(Q4K, x4)
-        oracle.quantize(Q6K, x6)
-        reps += 1
-    dt = time.perf_counter() - t0
+
+    def once(threads=1):
+        oracle.quantize(Q4K, x4, threads=threads)
+        oracle.quantize(Q6K, x6, threads=threads)
+
+    reps, dt = timed_reps(once, budget_s)
+    th = baseline_threads()
+    reps_mt, dt_mt = timed_reps(lambda: once(th), budget_s / 2)
     return {"value": round(4.0 * (x4.size + x6.size) * reps / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"{reps} x (786432 elements to Q4_K + 262144 to Q6_K), {dt:.1f} s"}
+            "sample": f"{reps} x (786432 elements to Q4_K + 262144 to Q6_K), {dt:.1f} s",
+            "all_cores": {"value": round(4.0 * (x4.size + x6.size) * reps_mt / dt_mt / 1e9, 4), "unit": "GB/s", "cores": th,
+                          "sample": f"{reps_mt} x the same elements, super-block ranges spread over {th} threads, {dt_mt:.1f} s"},
+            "host": host_description()}
 
 
 def cpu_baseline_dequantize(budget_s=10.0):
@@ -142,7 +184,7 @@ def cpu_baseline_dequantize(budget_s=10.0):
             "sample": f"{reps} x dequantize of {n} Q4_K elements, {dt:.1f} s"}
 
 
-def cpu_baseline_gemm(t, m, n, k, budget_s=12.0):
+def cpu_baseline_gemm(t, m, n, k, budget_s=6.0):
     """Oracle: reference dequantize + f32 matmul (row by row, sequential dot products), one thread, on a slice."""
     from oracle import binding as oracle
     oracle.build()
@@ -151,13 +193,14 @@ def cpu_baseline_gemm(t, m, n, k, budget_s=12.0):
     wq = oracle.quantize(t, (rng.standard_normal(rows * k) * 0.02).astype(np.float32))
     x = oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(rng.standard_normal(mm * k).astype(np.float32))).reshape(mm, k)
     oracle.qmatmul(t, wq, rows, k, x[:1])
-    reps, t0 = 0, time.perf_counter()
-    while time.perf_counter() - t0 < budget_s:
-        oracle.qmatmul(t, wq, rows, k, x)
-        reps += 1
-    dt = time.perf_counter() - t0
+    reps, dt = timed_reps(lambda: oracle.qmatmul(t, wq, rows, k, x), budget_s)
+    th = baseline_threads()
+    reps_mt, dt_mt = timed_reps(lambda: oracle.qmatmul(t, wq, rows, k, x, threads=th), budget_s / 2)
     return {"value": round(2.0 * mm * rows * k * reps / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
-            "sample": f"{reps} x (dequantize + matmul) of {mm} x {rows} x {k}, {dt:.1f} s"}
+            "sample": f"{reps} x (dequantize + matmul) of {mm} x {rows} x {k}, {dt:.1f} s",
+            "all_cores": {"value": round(2.0 * mm * rows * k * reps_mt / dt_mt / 1e12, 6), "unit": "TFLOP/s", "cores": th,
+                          "sample": f"{reps_mt} x the same product, weight rows spread over {th} threads, {dt_mt:.1f} s"},
+            "host": host_description()}
 
 
 def cpu_baseline_decode(pm, model="qwen3_0.6b", budget_s=15.0):
@@ -184,7 +227,8 @@ def cpu_baseline_decode(pm, model="qwen3_0.6b", budget_s=15.0):
                       f"scaled by bytes, {dt:.1f} s"}
 
 
-def bench_gemv(args, n, k, t=Q4K, copies=16):
+def bench_gemv(args, n, k, t=Q4K, copies=16, passes=8):
+    """One step = `passes` sweeps over `copies` distinct weight tensors, one GEMV launch per tensor."""
     pm, _lib, lib = load()
     timer = Timer(pm, lib)
     ws = [device_weights(pm, lib, t, n * k, 1000 + i) for i in range(copies)]
@@ -201,11 +245,14 @@ def bench_gemv(args, n, k, t=Q4K, copies=16):
     for i in range(copies):
         solo[i] = _lib.LinearDesc(t, pm.DTYPE_BF16, 0, 0, n, k, ws[i].ptr, (x if i % 2 == 0 else x2).ptr, ys[i].ptr)
 
-    def step():
-        pm.check(lib.pmetal_hip_qgemv_batch(solo, copies, None))
+    def sweeps(descs_):
+        def run():
+            for _ in range(passes):
+                pm.check(lib.pmetal_hip_qgemv_batch(descs_, copies, None))
+        return run
 
-    ev_ms, wall_ms = timer.run(step, args.steps, args.warmup)
-    launches = args.steps * copies
+    ev_ms, wall_ms = timer.run(sweeps(solo), args.steps, args.warmup)
+    launches = args.steps * copies * passes
     bytes_per_launch = gemv_bytes(t, n, k, 2)
     us_per_launch = ev_ms * 1e3 / launches
     gbs = bytes_per_launch / (us_per_launch * 1e-6) / 1e9
@@ -214,18 +261,37 @@ def bench_gemv(args, n, k, t=Q4K, copies=16):
     one = (_lib.LinearDesc * copies)()
     for i in range(copies):
         one[i] = _lib.LinearDesc(t, pm.DTYPE_BF16, 0, 0, n, k, ws[0].ptr, (x if i % 2 == 0 else x2).ptr, ys[0].ptr)
-    c_ms, _ = timer.run(lambda: pm.check(lib.pmetal_hip_qgemv_batch(one, copies, None)), args.steps, args.warmup)
+    c_ms, _ = timer.run(sweeps(one), args.steps, args.warmup)
     cached_gbs = bytes_per_launch / (c_ms * 1e-3 / launches) / 1e9
     # all sixteen sharing one x (as gate / up do): two matrices per launch where the kernel allows it
-    b_ms, _ = timer.run(lambda: pm.check(lib.pmetal_hip_qgemv_batch(descs, copies, None)), args.steps, args.warmup)
+    b_ms, _ = timer.run(sweeps(descs), args.steps, args.warmup)
+    # what a launch that only reads the same weight bytes takes on this machine, from HBM and from the cache
+    sink = pm.DeviceBuffer(16)
+    w_bytes = lib.pmetal_hip_tensor_size(t, n * k)
+
+    def reads(bufs):
+        def run():
+            for _ in range(passes):
+                for b in bufs:
+                    pm.check(lib.pmetal_hip_read_probe(b.ptr, w_bytes, sink.ptr, None))
+        return run
+
+    r_ms, _ = timer.run(reads(ws), args.steps, args.warmup)
+    rc_ms, _ = timer.run(reads([ws[0]] * copies), args.steps, args.warmup)
+    read_us, read_cached_us = r_ms * 1e3 / launches, rc_ms * 1e3 / launches
     return {
         "value": gbs, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
                      "kernel": {Q4K: "k_qgemv_q4k_chunk", Q6K: "k_qgemv_q6k_chunk", Q8_0: "k_qgemv_q8_0_chunk", 13: "k_qgemv_q5k_chunk", 11: "k_qgemv_q23k_chunk<FormatQ3K>", 10: "k_qgemv_q23k_chunk<FormatQ2K>"}[t], "bytes_per_launch": bytes_per_launch,
                      "us_per_launch": round(us_per_launch, 3)},
-        "extra": {"cache_resident_GBps": round(cached_gbs, 1), "weight_copies": copies,
-                  "batch_entry_us_per_matrix": round(b_ms * 1e3 / launches, 3)},
+        "extra": {"cache_resident_GBps": round(cached_gbs, 1), "cache_resident_us_per_launch": round(c_ms * 1e3 / launches, 3),
+                  "weight_copies": copies, "launches_per_step": copies * passes,
+                  "batch_entry_us_per_matrix": round(b_ms * 1e3 / launches, 3),
+                  "plain_read_us": {"hbm": round(read_us, 3), "cache_resident": round(read_cached_us, 3),
+                                    "bytes": w_bytes, "hbm_GBps": round(w_bytes / (read_us * 1e-6) / 1e9, 1),
+                                    "what": "pmetal_hip_read_probe over the same weight tensors, same launch pattern: a kernel that only reads"},
+                  "gemv_over_plain_read": round(us_per_launch / read_us, 3)},
     }, (t, n, k)
 
 
@@ -543,6 +609,31 @@ for _name, _t in (("q5k", 13), ("q3k", 11), ("q2k", 10)):  # re-blocked into Q6_
                                            metric=f"{_name.upper().replace('K', '_K')} GEMM TFLOPS (nominal flops) @M=512,K=4096,N=14336")
 
 
+def other_parts(args):
+    """The Q4_K GEMM at M = 512 and the Llama-3-8B-shaped f32 -> Q4_K_M quantizer, each with its roofline and CPU baseline."""
+    import copy
+    out = {}
+    a = copy.copy(args)
+    a.steps, a.warmup = max(args.steps, 50), max(args.warmup, 5)
+    res, _ = bench_gemm(a, 512, 14336, 4096, Q4K)
+    wl = WORKLOADS["gemm_q4k_m512"]
+    out["gemm_q4k_m512"] = {"metric": wl["metric"], "value": round(res["value"], 1), "unit": wl["unit"], "dtype": wl["dtype"],
+                            "steps": a.steps, "ms_per_step": round(res["ms_per_step"], 5), "roofline": res["roofline"],
+                            "extra": res["extra"]}
+    if not args.no_cpu_baseline:
+        out["gemm_q4k_m512"]["cpu_baseline"] = cpu_baseline_gemm(Q4K, 512, 14336, 4096, budget_s=3.0)
+    a = copy.copy(args)
+    a.steps, a.warmup = 5, 1
+    res, _ = bench_quantize(a)
+    wl = WORKLOADS["quantize_llama3_8b_q4km"]
+    out["quantize_llama3_8b_q4km"] = {"metric": wl["metric"], "value": round(res["value"], 1), "unit": wl["unit"],
+                                      "dtype": wl["dtype"], "steps": a.steps, "ms_per_step": round(res["ms_per_step"], 5),
+                                      "roofline": res["roofline"], "extra": res["extra"]}
+    if not args.no_cpu_baseline:
+        out["quantize_llama3_8b_q4km"]["cpu_baseline"] = cpu_baseline_quantize(budget_s=3.0)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -550,6 +641,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="gemv_q4k_14336x4096", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra-workloads", action="store_true",
+                    help="default workload only: do not also time the GEMM and quantizer parts of the metric")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain streaming kernel of known size (f32 -> bf16 over 2^24 elements: 64 MiB read, "
                          "32 MiB written) so that profiler byte counters can be scaled against it")
@@ -581,7 +674,7 @@ def main():
                  else "synthetic: N(0,0.02) f32 weights generated and quantized on the device, x ~ N(0,1) bf16"),
         "config": {"workload": args.workload, "element_order": "GGML" if wl["kind"] == "calibrate" else "REF",
                    "step": {"gemm": "one GEMM launch (activation pre-pass + MFMA kernel)",
-                            "gemv": "16 back-to-back GEMV launches over 16 distinct weight tensors (HBM-resident: 528 MB for Q4_K)",
+                            "gemv": "8 sweeps of 16 back-to-back GEMV launches, one per distinct weight tensor (HBM-resident: 528 MB for Q4_K)",
                             "gemv_q8k": "16 x (activations f32 -> Q8_K, integer-dot GEMV) over 16 distinct weight tensors",
                             "calibrate": "one tensor resident in HBM: 6 candidates x (quantize, fused dequantize-and-score, f64 score read back)",
                             "decode": "all batch-1 projections of one token (197 for Qwen3-0.6B, 225 for Llama-3-8B), back to back on one stream",
@@ -594,7 +687,10 @@ def main():
         # `dtype` names the activation type handed over; the kernels of these (large) shapes multiply in integers
         out["config"]["arithmetic"] = ("bf16 activations converted exactly to fixed-point int8 digit planes, v_dot4_i32_i8 against "
                                        "the quantized weights, f32 block scales and accumulation")
-    out["roofline"]["traffic"] = MEASURED_TRAFFIC.get(args.workload)
+    rec = RECORDED_TRAFFIC.get(args.workload)
+    out["roofline"]["traffic"] = rec[0] if rec else None
+    if rec:
+        out["roofline"]["traffic_source"] = f"recorded constant from {rec[1]} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE), not measured in this run"
     if args.calibrate:
         pm, _lib, lib = load()
         n_cal = 1 << 24
@@ -603,6 +699,9 @@ def main():
         for _ in range(5):
             pm.check(lib.pmetal_hip_f32_to_bf16_dev(src.ptr, dst.ptr, n_cal, None))
         pm.check(lib.pmetal_hip_sync(None))
+    if args.workload == "gemv_q4k_14336x4096" and not args.no_extra_workloads:
+        # the other two parts of the headline metric ("Q4_K GEMM TFLOPS; quantize GB/s"), timed in the same run
+        out["extra"]["other_parts_of_the_metric"] = other_parts(args)
     if not args.no_cpu_baseline:
         if wl["kind"] == "gemv":
             out["cpu_baseline"] = cpu_baseline_gemv(t, n, k)

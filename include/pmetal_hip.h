@@ -256,6 +256,12 @@ int32_t pmetal_hip_f32_to_bf16_dev(const float *src_dev, uint16_t *dst_dev, size
  * practice).                                                                                */
 int32_t pmetal_hip_mfma_probe_f16(int32_t iters, int32_t vary, int32_t workgroups, float *sink_dev, void *stream);
 
+/* Launches a kernel that does nothing but read `bytes` (rounded down to 16) from src_dev with 16-byte loads, so that a
+ * caller can time what a single launch over that many bytes costs on this machine when nothing is computed: the floor the
+ * fused GEMV of a tensor of that size is measured against.  `sink_dev` is a 4-byte device buffer (never written in
+ * practice).                                                                                                         */
+int32_t pmetal_hip_read_probe(const void *src_dev, size_t bytes, uint32_t *sink_dev, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

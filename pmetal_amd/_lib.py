@@ -65,6 +65,7 @@ SYMBOLS = [
     ("pmetal_hip_fill_normal_f32", _i32, [_vp, _sz, _u64, _f32, _f32, _f32, _vp]),
     ("pmetal_hip_f32_to_bf16_dev", _i32, [_vp, _vp, _sz, _vp]),
     ("pmetal_hip_mfma_probe_f16", _i32, [_i32, _i32, _i32, _vp, _vp]),
+    ("pmetal_hip_read_probe", _i32, [_vp, _sz, _vp, _vp]),
 ]
 
 _lib = None

@@ -847,4 +847,13 @@ int32_t pmetal_hip_mfma_probe_f16(int32_t iters, int32_t vary, int32_t workgroup
     return ok();
 }
 
+int32_t pmetal_hip_read_probe(const void *src, size_t bytes, uint32_t *sink, void *stream) {
+    if (!src || !sink) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
+    if (!aligned16(src)) return fail(PMETAL_HIP_ERR_INVALID_ARG, "device pointers must be 16-byte aligned");
+    if (int32_t rc = require_device()) return rc;
+    hipError_t e = pmh::launch_read_probe(src, bytes, sink, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "probe kernel launch");
+    return ok();
+}
+
 }  // extern "C"

@@ -98,5 +98,6 @@ hipError_t launch_fill_normal(float *dst, size_t n, uint64_t seed, float std, fl
 hipError_t launch_f32_to_bf16(const float *src, uint16_t *dst, size_t n, hipStream_t s);
 hipError_t launch_zero_bytes(uint8_t *dst, size_t bytes, hipStream_t s);
 hipError_t launch_mfma_probe(int iters, int vary, int workgroups, float *sink, hipStream_t s);
+hipError_t launch_read_probe(const void *src, size_t bytes, uint32_t *sink, hipStream_t s);
 
 }  // namespace pmh

@@ -81,6 +81,19 @@ __global__ __launch_bounds__(512) void k_mfma_probe(int iters, int vary, float *
     if (s == 1.2345f) sink[0] = s;  // keeps the loop alive; practically never true
 }
 
+// Plain streaming read: every thread loads 16 bytes per step of a grid-wide sweep and folds them into a value that is
+// (practically) never stored.  The time of this kernel over n bytes is what the memory system of the machine allows a
+// single launch that does nothing but read them.
+__global__ __launch_bounds__(256) void k_read_probe(const uint4 *__restrict__ p, size_t n16, uint32_t *__restrict__ sink) {
+    const size_t stride = (size_t)gridDim.x * 256;
+    uint32_t acc = 0;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) {
+        const uint4 v = p[i];
+        acc += v.x ^ v.y ^ v.z ^ v.w;
+    }
+    if (acc == 0x12345678u) sink[0] = acc;
+}
+
 inline unsigned capped_grid(size_t items) {
     size_t g = (items + 255) / 256;
     return (unsigned)(g < 1 ? 1 : (g > 65536 ? 65536 : g));
@@ -107,6 +120,15 @@ hipError_t launch_fill_normal(float *dst, size_t n, uint64_t seed, float std, fl
     if (n == 0) return hipSuccess;
     hipLaunchKernelGGL(k_fill_normal, dim3(capped_grid((n + 1) / 2)), dim3(256), 0, s, dst, n, seed, std,
                        outlier_rate, outlier_mag);
+    return hipGetLastError();
+}
+
+hipError_t launch_read_probe(const void *src, size_t bytes, uint32_t *sink, hipStream_t s) {
+    const size_t n16 = bytes / 16;
+    if (n16 == 0) return hipSuccess;
+    size_t grid = (n16 + 255) / 256;
+    if (grid > 2048) grid = 2048;  // eight workgroups per compute unit: the fastest sweep for tensors of tens of MB
+    hipLaunchKernelGGL(k_read_probe, dim3((unsigned)grid), dim3(256), 0, s, reinterpret_cast<const uint4 *>(src), n16, sink);
     return hipGetLastError();
 }
 
