@@ -101,9 +101,14 @@ int32_t pmetal_hip_sync(void *stream);
  * costs more than running them; a recording replays the whole sequence with one submission (a HIP
  * graph).  Between record_begin and record_end every kernel launch issued on `stream` through this
  * library is recorded instead of run.  Record only launch-type calls (qgemv, qgemv_batch,
- * quantize_dev, dequantize_dev, f32_to_bf16_dev, and qgemm / qlinear once a call of the same or a
- * larger shape has run, so that their scratch buffer exists); pmetal_hip_memset refuses to be
- * recorded.  A recording holds the pointers it was recorded with.                            */
+ * quantize_dev, dequantize_dev, f32_to_bf16_dev, qgemm_noalloc, and qgemm / qlinear once a call of
+ * the same or a larger shape has run on that stream: nothing can be allocated while a stream is
+ * being recorded, and a qgemm whose scratch does not exist yet fails with INVALID_ARG);
+ * pmetal_hip_memset refuses to be recorded.  A recording holds the pointers it was recorded
+ * with, the library's scratch buffer of that stream included: that buffer is kept until the
+ * stream is destroyed, whatever runs on the stream later.  pmetal_hip_stream_destroy waits for
+ * the stream and releases the calling thread's scratch for it; recordings made on a destroyed
+ * stream must not be replayed.                                                              */
 void *pmetal_hip_stream_create(void); /* NULL on failure (error slot set) */
 int32_t pmetal_hip_stream_destroy(void *stream);
 int32_t pmetal_hip_record_begin(void *stream); /* `stream` must come from pmetal_hip_stream_create */
@@ -151,7 +156,8 @@ int32_t pmetal_hip_dequantize_dev(uint32_t ggml_type, const uint8_t *src_dev, si
  * with W = reference dequantize of the packed blocks (order as given), fp32 accumulation,
  * max relative error <= 1e-3 against dequantize-then-f32-matmul.
  * W: [n, k] packed row-major, k a multiple of the block size.  x/X: f32 or bf16.
- * Types: Q8_0, Q4_K and Q6_K have both kernels.  Q5_K, Q3_K and Q2_K have a GEMV kernel (k <= 32768) and no GEMM
+ * Types: Q8_0, Q4_K and Q6_K have both kernels.  Q5_K, Q3_K and Q2_K have a GEMV kernel (k <= 32768 and a tensor below
+ * 4 GiB, any number of rows; beyond that qgemv fails with SHAPE_TOO_LARGE and qlinear uses the GEMM) and no GEMM
  * kernel of their own: qgemm re-blocks their super-blocks, without loss, into one (Q3_K) or two (Q5_K, Q2_K: values
  * and mins) Q6_K tensors in its scratch memory on every call (Q5_K 2.4, Q3_K 1.9, Q2_K 5 times the bytes of W) and runs the Q6_K
  * GEMM on them; qlinear runs one GEMV per activation row up to m = 8 and qgemm above.

@@ -98,19 +98,29 @@ struct DevBuf {
     }
 };
 
-// qgemm scratch, grown on demand: one buffer per (thread, device, stream), so that neither concurrent callers nor
+// Library-owned scratch, grown on demand: one buffer per (thread, device, stream), so that neither concurrent callers nor
 // one caller's launches on different streams share it.  Launches on one stream run in order and may.
+//  * A buffer that was handed out while its stream was being recorded is pinned: the recording holds its address, so it is
+//    never freed or replaced before the process ends (a larger request gets a new buffer, the pinned one is kept aside).
+//  * While a stream is being recorded nothing may be allocated or synchronised on it: a request that the current buffer
+//    cannot serve fails with a clear error instead (run the same or a larger shape once before recording).
+//  * pmetal_hip_stream_destroy releases the buffers of that stream (pinned ones included: the recordings made on a
+//    destroyed stream must not be replayed any more).
 struct Workspace {
     void *p = nullptr;
     size_t bytes = 0;
     int device = -1;
     hipStream_t stream = nullptr;
+    bool pinned = false;
 };
 struct WorkspaceSet {
     std::vector<Workspace> items;
+    std::vector<Workspace> retired;  // pinned buffers that a larger one replaced
     ~WorkspaceSet() {
         for (Workspace &w : items)
             if (w.p) (void)hipFree(w.p);  // at thread exit; fails harmlessly once the runtime is gone
+        for (Workspace &w : retired)
+            if (w.p) (void)hipFree(w.p);
     }
 };
 thread_local WorkspaceSet g_ws;
@@ -118,26 +128,55 @@ thread_local WorkspaceSet g_ws;
 int32_t workspace(size_t bytes, hipStream_t stream, void **out) {
     int dev = 0;
     HIP_TRY(hipGetDevice(&dev));
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (stream) HIP_TRY(hipStreamIsCapturing(stream, &cap));
+    const bool recording = cap != hipStreamCaptureStatusNone;
     Workspace *w = nullptr;
     for (Workspace &c : g_ws.items)
         if (c.device == dev && c.stream == stream) w = &c;
     if (!w) {
-        g_ws.items.push_back(Workspace{nullptr, 0, dev, stream});
+        g_ws.items.push_back(Workspace{nullptr, 0, dev, stream, false});
         w = &g_ws.items.back();
     }
-    if (w->p && w->bytes < bytes) {
-        HIP_TRY(hipStreamSynchronize(stream));  // earlier launches on this stream may still use the smaller buffer
-        HIP_TRY(hipFree(w->p));
-        w->p = nullptr, w->bytes = 0;
+    if (w->bytes < bytes) {
+        if (recording)
+            return fail(PMETAL_HIP_ERR_INVALID_ARG,
+                        "this call needs %zu bytes of scratch and the stream's buffer holds %zu: nothing can be allocated while the "
+                        "stream is being recorded (run a call of this or a larger shape on the stream first)", bytes, w->bytes);
+        if (w->p) {
+            if (w->pinned) {
+                g_ws.retired.push_back(*w);  // a recording still names it
+            } else {
+                HIP_TRY(hipStreamSynchronize(stream));  // earlier launches on this stream may still use the smaller buffer
+                HIP_TRY(hipFree(w->p));
+            }
+            w->p = nullptr, w->bytes = 0, w->pinned = false;
+        }
+        if (bytes) {
+            HIP_TRY(hipMalloc(&w->p, bytes));
+            w->bytes = bytes;
+        }
     }
-    if (!w->p && bytes) {
-        HIP_TRY(hipMalloc(&w->p, bytes));
-        w->bytes = bytes;
-    }
+    if (recording) w->pinned = true;
     *out = w->p;
     return PMETAL_HIP_OK;
 }
 
+// Releases what workspace() holds for `stream` on the calling thread.
+void drop_workspaces_of(hipStream_t stream) {
+    auto drop = [&](std::vector<Workspace> &v) {
+        for (size_t i = 0; i < v.size();) {
+            if (v[i].stream == stream) {
+                if (v[i].p) (void)hipFree(v[i].p);
+                v.erase(v.begin() + (long)i);
+            } else {
+                i++;
+            }
+        }
+    };
+    drop(g_ws.items);
+    drop(g_ws.retired);
+}
 
 // ---- scratch memory of the entry point that allocates nothing (pmetal_hip_qgemm_noalloc) ----
 // A fixed array in the code object: every device that loads the library holds its own copy, at its own address, until the
@@ -308,6 +347,8 @@ void *pmetal_hip_stream_create(void) {
 
 int32_t pmetal_hip_stream_destroy(void *stream) {
     if (!stream) return ok();
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    drop_workspaces_of((hipStream_t)stream);  // the calling thread's scratch for this stream (other threads' goes at their exit)
     HIP_TRY(hipStreamDestroy((hipStream_t)stream));
     return ok();
 }
@@ -505,8 +546,10 @@ int32_t pmetal_hip_qgemv(uint32_t t, const uint8_t *w, int64_t n, int64_t k, con
                          uint32_t order, void *stream) {
     if (int32_t rc = check_linear(t, w, n, k, x, x_dtype, y, order, true)) return rc;
     hipError_t e = pmh::launch_qgemv(t, w, n, k, x, x_dtype, y, order, (hipStream_t)stream);
-    if (e == hipErrorInvalidValue)
-        return fail(PMETAL_HIP_ERR_SHAPE_TOO_LARGE, "k=%lld does not fit the activation staging buffer", (long long)k);
+    if (e == hipErrorInvalidValue)  // refused by the launcher before anything ran
+        return fail(PMETAL_HIP_ERR_SHAPE_TOO_LARGE,
+                    "qgemv: n=%lld, k=%lld does not fit the kernel of GGML type %u (the activations of a row must fit in LDS: k <= 32768 "
+                    "for Q5_K / Q3_K / Q2_K; a tensor must stay below 4 GiB)", (long long)n, (long long)k, t);
     if (e != hipSuccess) return hip_fail(e, "qgemv kernel launch");
     return ok();
 }
@@ -652,10 +695,17 @@ int32_t pmetal_hip_qgemm_noalloc(uint32_t t, const uint8_t *w, int64_t n, int64_
 
 int32_t pmetal_hip_qlinear(uint32_t t, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, int64_t m,
                            void *y, uint32_t y_dtype, uint32_t order, void *stream) {
-    if (m == 1 && y_dtype == PMETAL_HIP_DTYPE_F32)
-        return pmetal_hip_qgemv(t, w, n, k, x, x_dtype, (float *)y, order, stream);
-    if (((t == PMETAL_GGML_TYPE_Q8_0 && k % 256 != 0) || (gemv_only_type(t) && m <= kRowLoopMax)) && y_dtype == PMETAL_HIP_DTYPE_F32 &&
-        m > 1 && n > 0 && k > 0 && x && y) {
+    if (m == 1 && y_dtype == PMETAL_HIP_DTYPE_F32) {
+        const int32_t rc = pmetal_hip_qgemv(t, w, n, k, x, x_dtype, (float *)y, order, stream);
+        // a shape the GEMV kernels refuse (a row too long for LDS) still has the GEMM, which takes one activation row
+        if (rc != PMETAL_HIP_ERR_SHAPE_TOO_LARGE || k % 256 != 0) return rc;
+        return pmetal_hip_qgemm(t, w, n, k, x, x_dtype, m, y, y_dtype, order, stream);
+    }
+    const bool q8_ragged = t == PMETAL_GGML_TYPE_Q8_0 && k % 256 != 0;
+    if (q8_ragged && y_dtype != PMETAL_HIP_DTYPE_F32)
+        return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qlinear: a Q8_0 row of k=%lld (not a multiple of 256) runs through the GEMV, whose output is f32 only",
+                    (long long)k);
+    if ((q8_ragged || (gemv_only_type(t) && m <= kRowLoopMax)) && y_dtype == PMETAL_HIP_DTYPE_F32 && m > 1 && n > 0 && k > 0 && x && y) {
         // The fused GEMM walks k in steps of 256, and a Q8_0 row may be any multiple of 32: one fused GEMV per activation row
         // then, back to back on the stream.  Q5_K, Q3_K and Q2_K reach the GEMM through a re-blocking pass over the whole
         // matrix, which a few rows do not repay.
@@ -663,9 +713,10 @@ int32_t pmetal_hip_qlinear(uint32_t t, const uint8_t *w, int64_t n, int64_t k, c
         for (int64_t r = 0; r < m; r++) {
             const int32_t rc = pmetal_hip_qgemv(t, w, n, k, (const uint8_t *)x + (size_t)r * x_row, x_dtype,
                                                 (float *)y + (size_t)r * (size_t)n, order, stream);
+            if (rc == PMETAL_HIP_ERR_SHAPE_TOO_LARGE && r == 0 && !q8_ragged) break;  // the GEMM below takes every shape
             if (rc != PMETAL_HIP_OK) return rc;
+            if (r == m - 1) return ok();
         }
-        return PMETAL_HIP_OK;
     }
     return pmetal_hip_qgemm(t, w, n, k, x, x_dtype, m, y, y_dtype, order, stream);
 }
@@ -783,9 +834,9 @@ int32_t pmetal_hip_qgemv_q8k(uint32_t t, const uint8_t *w, int64_t n, int64_t k,
 // ---- KL calibration metric ----
 namespace {
 // compute_kl_divergence (dynamic.rs:155-178) from the per-workgroup partial sums, added in workgroup order
-int32_t kl_score_from_partials(const DevBuf &part, int groups, size_t n, double *score, hipStream_t stream) {
+int32_t kl_score_from_partials(const void *part, int groups, size_t n, double *score, hipStream_t stream) {
     std::vector<double> host((size_t)groups * 4);
-    HIP_TRY(hipMemcpyAsync(host.data(), part.p, host.size() * sizeof(double), hipMemcpyDeviceToHost, stream));
+    HIP_TRY(hipMemcpyAsync(host.data(), part, host.size() * sizeof(double), hipMemcpyDeviceToHost, stream));
     HIP_TRY(hipStreamSynchronize(stream));
     double sq_err = 0.0, aa = 0.0, ab = 0.0, bb = 0.0;
     for (int g = 0; g < groups; g++) sq_err += host[4 * g], aa += host[4 * g + 1], ab += host[4 * g + 2], bb += host[4 * g + 3];
@@ -807,9 +858,9 @@ int32_t pmetal_hip_kl_divergence_dev(const float *original, const float *dequant
     if (!aligned16(original) || !aligned16(dequantized)) return fail(PMETAL_HIP_ERR_INVALID_ARG, "device pointers must be 16-byte aligned");
     if (int32_t rc = require_device()) return rc;
     const int groups = pmh::kl_sums_workgroups(n);
-    DevBuf part;
-    HIP_TRY(hipMalloc(&part.p, (size_t)groups * 4 * sizeof(double)));
-    hipError_t e = pmh::launch_kl_sums(original, dequantized, n, (double *)part.p, (hipStream_t)stream);
+    void *part = nullptr;  // the stream's scratch (shared with qgemm: calls on one stream run in order, and this one synchronises)
+    if (int32_t rc = workspace((size_t)groups * 4 * sizeof(double), (hipStream_t)stream, &part)) return rc;
+    hipError_t e = pmh::launch_kl_sums(original, dequantized, n, (double *)part, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "kl sums kernel launch");
     return kl_score_from_partials(part, groups, n, score, (hipStream_t)stream);
 }
@@ -830,9 +881,9 @@ int32_t pmetal_hip_kl_divergence_quantized_dev(uint32_t t, const uint8_t *quanti
     if (!aligned16(original) || !aligned16(quantized)) return fail(PMETAL_HIP_ERR_INVALID_ARG, "device pointers must be 16-byte aligned");
     if (int32_t rc = require_device()) return rc;
     const int groups = pmh::kl_sums_quantized_workgroups(n);
-    DevBuf part;
-    HIP_TRY(hipMalloc(&part.p, (size_t)groups * 4 * sizeof(double)));
-    hipError_t e = pmh::launch_kl_sums_quantized(t, quantized, original, n, order, (double *)part.p, (hipStream_t)stream);
+    void *part = nullptr;
+    if (int32_t rc = workspace((size_t)groups * 4 * sizeof(double), (hipStream_t)stream, &part)) return rc;
+    hipError_t e = pmh::launch_kl_sums_quantized(t, quantized, original, n, order, (double *)part, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "fused kl sums kernel launch");
     return kl_score_from_partials(part, groups, n, score, (hipStream_t)stream);
 }

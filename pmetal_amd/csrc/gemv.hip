@@ -316,14 +316,7 @@ __global__ __launch_bounds__(256) void k_qgemv_q8_0(const uint8_t *__restrict__ 
 // ------------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------------
-int rows_per_team() {
-    static const int v = [] {
-        const char *e = std::getenv("PMETAL_HIP_GEMV_ROWS_PER_TEAM");
-        const int r = e ? std::atoi(e) : 0;
-        return r > 0 ? r : 4;
-    }();
-    return v;
-}
+constexpr int rows_per_team() { return 4; }
 
 // Rows per team: rows_per_team() when that still leaves a workgroup for every compute unit, fewer otherwise
 // (a small matrix is spread over the whole chip rather than streamed by a few workgroups).

@@ -1,15 +1,10 @@
 // Shared pieces of the row-staging GEMV kernels (gemv_q5k.hip, gemv_q6k.hip, gemv_q8_0.hip, gemv_q23k.hip): one
-// workgroup per compute unit, wave (g, h) = chunk h of the rows of row group g, lane partial sums through LDS.
+// workgroup per compute unit, wave (g, h) = chunk h of the rows of row group g, one chunk sum per row through LDS.
 #pragma once
 #include "gemv_common.hpp"
 
 namespace pmh {
 namespace gemv {
-
-// Row stride of the partial sums in LDS.  The final summation puts `red` lanes on a row (lane p adds every red-th
-// partial), 64 / red rows side by side in a wave: a stride of `red` floats past a multiple of 64 keeps those rows in
-// different banks.
-__host__ __device__ constexpr int part_stride(int slots, int red) { return ((slots + 63) / 64) * 64 + (red & 63); }
 
 __device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {
     return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
@@ -62,38 +57,28 @@ __device__ __forceinline__ uint32_t max_magnitude_bits(const float (&v)[4]) {
     return mb;
 }
 
-// Row totals after the barrier: `red` lanes per row (a power of two from 8 to 64 that divides slots), lane p adding
-// every red-th partial, then a sum over the lanes of the row.  part is [group][n_nominal][ps].
-__device__ __forceinline__ void reduce_rows(const float *part, int ps, int slots, int red, int wg_r0, int wg_rows, int rows_per_wave,
-                                            int n_nominal, int nthreads, float *__restrict__ y) {
-    const int per_thread = slots / red;
-    const int red_shift = 31 - __builtin_clz(red);
-    for (int idx0 = 0; idx0 < wg_rows * red; idx0 += nthreads) {
-        const int idx = idx0 + (int)threadIdx.x;
-        int rl = idx >> red_shift;
-        const bool ok = rl < wg_rows;
-        rl = ok ? rl : wg_rows - 1;
+// A task's lane values are added up inside the wave (DPP); lane 63 drops the total into part[group][row][chunk].
+__device__ __forceinline__ void store_chunk_sum(float *slot_of_task, float lane_value, int lane) {
+    const float total = team_sum_last<64>(lane_value);
+    if (lane == 63) *slot_of_task = total;
+}
+
+// Row totals after the barrier: one thread per row adds the row's ks chunk sums in chunk order; the workgroup's rows leave
+// with one coalesced store.  part is [group][n_nominal][ks].
+__device__ __forceinline__ void reduce_rows(const float *part, int ks, int wg_r0, int wg_rows, int rows_per_wave, int n_nominal,
+                                            int nthreads, float *__restrict__ y) {
+    for (int rl = (int)threadIdx.x; rl < wg_rows; rl += nthreads) {
         const int grp = rl / rows_per_wave, loc = rl - grp * rows_per_wave;
-        const int p = idx & (red - 1);
-        const float *src = part + (size_t)(grp * n_nominal + loc) * ps + p;
-        float t0 = 0.0f, t1 = 0.0f, t2 = 0.0f, t3 = 0.0f;
-        int i = 0;
-        for (; i + 8 <= per_thread; i += 8) {  // eight reads in flight
-            const float *q = src + (size_t)i * red;
-            const float a0 = q[0], a1 = q[red], a2 = q[2 * red], a3 = q[3 * red];
-            const float a4 = q[4 * red], a5 = q[5 * red], a6 = q[6 * red], a7 = q[7 * red];
-            t0 += a0 + a4, t1 += a1 + a5, t2 += a2 + a6, t3 += a3 + a7;
-        }
-        for (; i < per_thread; i++) t0 += src[(size_t)i * red];
-        const float sum = team_sum_rt((t0 + t1) + (t2 + t3), red);
-        if (ok && p == 0) y[wg_r0 + rl] = sum;
+        const float *src = part + (size_t)(grp * n_nominal + loc) * ks;
+        float sum = src[0];
+        for (int i = 1; i < ks; i++) sum += src[i];
+        y[wg_r0 + rl] = sum;
     }
 }
 
 // Launch geometry: rows split evenly over one workgroup per compute unit, the workgroup's rows over 16 / ks row groups.
 struct ChunkPlan {
     int64_t n_wg, rows_per_wg, rows_per_wave, n_nominal, threads;
-    int red;
     size_t lds;
 };
 // stage_bytes: LDS of one wave's row chunk; lds_x: LDS of the staged activations (slots = 64 ks lane slots)
@@ -109,9 +94,7 @@ inline ChunkPlan plan_chunks(int64_t n, int ks, size_t stage_bytes, size_t lds_x
     groups = (p.rows_per_wg + p.rows_per_wave - 1) / p.rows_per_wave;
     p.n_nominal = p.rows_per_wave;
     p.threads = ks * groups * 64;
-    p.red = 8;  // lanes per row in the final summation: as many as the workgroup has to spare, at most 64
-    while (p.red < 64 && p.rows_per_wg * p.red * 2 <= p.threads) p.red *= 2;
-    p.lds = (size_t)(p.threads / 64) * stage_bytes + lds_x + (size_t)groups * (size_t)p.n_nominal * part_stride(ks * 64, p.red) * 4;
+    p.lds = (size_t)(p.threads / 64) * stage_bytes + lds_x + (size_t)groups * (size_t)p.n_nominal * ks * 4;
     return p;
 }
 

@@ -76,13 +76,6 @@ inline int pow2_divisor(int64_t v, int cap) {
     return t;
 }
 
-// integer tuning knob from the environment (read once per name by the callers' statics)
-inline int64_t tuning(const char *name, int64_t dflt) {
-    const char *e = std::getenv(name);
-    if (!e || !*e) return dflt;
-    return std::atoll(e);
-}
-
 // compute units of the current device (256 on MI355X); falls back to 256 if the query fails
 inline int compute_units() {
     static const int n = [] {

@@ -156,7 +156,7 @@ struct FormatQ3K {
 template <class F, bool XF32, bool SINGLE>
 __global__ __launch_bounds__(1024) void k_qgemv_q23k_chunk(const uint8_t *__restrict__ W, const void *__restrict__ xg,
                                                             float *__restrict__ y, int n_rows, int spr, int rows_per_wg,
-                                                            int rows_per_wave, int n_nominal, int red, int nthreads,
+                                                            int rows_per_wave, int n_nominal, int nthreads,
                                                             uint32_t w_last) {
     constexpr int kStageDwords = F::kPieces * 4;
     extern __shared__ uint4 smem[];
@@ -167,8 +167,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q23k_chunk(const uint8_t *__rest
     uint32_t *stage = reinterpret_cast<uint32_t *>(smem) + wave * kStageDwords;   // this wave's row chunk
     uint32_t *xd = reinterpret_cast<uint32_t *>(smem) + n_waves * kStageDwords;  // [kPlanes * 8][slots]
     float *xm = reinterpret_cast<float *>(xd + kPlanes * 8 * slots);             // [slots][8]
-    float *part = xm + 8 * slots;                                                // [group][n_nominal][part_stride]
-    const int ps = part_stride(slots, red);
+    float *part = xm + 8 * slots;                                                // [group][n_nominal][ks]
     const int lane = threadIdx.x & 63;
     const int t = lane & 7;
     const int h = wave % ks, g = wave / ks;
@@ -205,7 +204,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q23k_chunk(const uint8_t *__rest
     const uint32_t chunk_byte = (uint32_t)h * 8u * (uint32_t)F::kBytes;
     const bool lane_valid = h * 8 + (lane >> 3) < spr;  // the last chunk of a row may be short
 
-    float *pp = part + (size_t)(g * n_nominal) * ps + slot;
+    float *pp = part + (size_t)(g * n_nominal) * ks + h;
     auto consume = [&](int i, const u4v a) {
         if (i < nt_wave) {  // wave-uniform
             u4v *st4 = reinterpret_cast<u4v *>(stage);
@@ -215,7 +214,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q23k_chunk(const uint8_t *__rest
             const uint32_t delta = ((uint32_t)(wave_r0 + i) * rowbytes + chunk_byte) & 15u;  // where the chunk starts in its first piece
             const uint32_t t0 = delta + sb_byte, mis = t0 & 2u;
             const float val = F::lane_value(stage + ((t0 - mis) >> 2), 8u * mis, t, xr, xs, xsum);
-            pp[(size_t)i * ps] = lane_valid ? val : 0.0f;
+            store_chunk_sum(pp + (size_t)i * ks, lane_valid ? val : 0.0f, lane);
         }
     };
 
@@ -242,7 +241,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q23k_chunk(const uint8_t *__rest
     }
     __syncthreads();
 
-    reduce_rows(part, ps, slots, red, wg_r0, wg_r1 - wg_r0, rows_per_wave, n_nominal, nthreads, y);
+    reduce_rows(part, ks, wg_r0, wg_r1 - wg_r0, rows_per_wave, n_nominal, nthreads, y);
 }
 
 template <class F>
@@ -256,7 +255,6 @@ hipError_t launch_format(const uint8_t *w, int64_t n, int64_t k, const void *x, 
     const ChunkPlan plan = plan_chunks(n, ks, (size_t)F::kPieces * 16, lds_x);
     const int64_t n_wg = plan.n_wg, rows_per_wg = plan.rows_per_wg, rows_per_wave = plan.rows_per_wave, n_nominal = plan.n_nominal,
                   threads = plan.threads;
-    const int red = plan.red;
     const size_t lds = plan.lds;
     if (lds > kMaxLds) return hipErrorInvalidValue;
     const bool single = n_nominal <= kDepth;
@@ -266,7 +264,7 @@ hipError_t launch_format(const uint8_t *w, int64_t n, int64_t k, const void *x, 
             if (e != hipSuccess) return e;
         }
         hipLaunchKernelGGL(kern, dim3((unsigned)n_wg), dim3((unsigned)threads), lds, s, w, x, y, (int)n, spr, (int)rows_per_wg,
-                           (int)rows_per_wave, (int)n_nominal, red, (int)threads, (uint32_t)((w_bytes - 1) & ~(uint64_t)15));
+                           (int)rows_per_wave, (int)n_nominal, (int)threads, (uint32_t)((w_bytes - 1) & ~(uint64_t)15));
         return hipGetLastError();
     };
     if (x_dtype == pmh::kDtypeF32) return single ? go(k_qgemv_q23k_chunk<F, true, true>) : go(k_qgemv_q23k_chunk<F, true, false>);

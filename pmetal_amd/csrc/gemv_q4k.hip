@@ -684,8 +684,7 @@ hipError_t launch_qgemv_q4k(const uint8_t *w, int64_t n, int64_t k, const void *
     // Kernel A when there is enough work per compute unit to pay for its second barrier (measured crossover: about
     // 12 MiB of weights) and the shape suits it.
     const uint64_t w_bytes = (uint64_t)n * (uint64_t)spr * 144u;
-    static const int64_t mode = gemv::tuning("PMETAL_HIP_GEMV_KERNEL", 0);  // 0 = choose, 1 = kernel A, 2 = kernel B
-    if (mode == 1 || (mode == 0 && w_bytes >= (12ull << 20))) {
+    if (w_bytes >= (12ull << 20)) {
         const hipError_t e = launch_kernel_a(w, n, y, nullptr, 0, nullptr, k, x, xf32, order, s);
         if (e != hipErrorNotSupported) return e;
     }
@@ -699,8 +698,6 @@ hipError_t launch_qgemv_q4k_pair(const uint8_t *w0, int64_t n0, float *y0, const
     const bool xf32 = x_dtype == kDtypeF32;
     const size_t slots = (size_t)(k / 256) * 8;
     if (slots * 16 * (xf32 ? 6 : 5) + slots * 16 > gemv::kMaxLds) return hipErrorNotSupported;
-    static const int64_t mode = gemv::tuning("PMETAL_HIP_GEMV_KERNEL", 0);
-    if (mode == 2) return hipErrorNotSupported;
     return launch_kernel_a(w0, n0, y0, w1, n1, y1, k, x, xf32, order, s);
 }
 

@@ -102,7 +102,7 @@ __device__ __forceinline__ uint32_t even_bits_to_bytes(uint32_t b) { return ((b 
 template <int ORDER, bool XF32, bool SINGLE>
 __global__ __launch_bounds__(1024) void k_qgemv_q5k_chunk(const uint8_t *__restrict__ W, const void *__restrict__ xg,
                                                            float *__restrict__ y, int n_rows, int spr, int rows_per_wg,
-                                                           int rows_per_wave, int n_nominal, int red, int nthreads,
+                                                           int rows_per_wave, int n_nominal, int nthreads,
                                                            uint32_t w_last) {
     extern __shared__ uint4 smem[];
     const int ks = (spr + 7) >> 3;
@@ -112,8 +112,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q5k_chunk(const uint8_t *__restr
     uint32_t *stage = reinterpret_cast<uint32_t *>(smem) + wave * (kStageBytes / 4);   // this wave's row chunk
     uint32_t *xd = reinterpret_cast<uint32_t *>(smem) + n_waves * (kStageBytes / 4);  // [kPlanes * 8][slots]
     float *xm = reinterpret_cast<float *>(xd + kPlanes * 8 * slots);                  // [slots][4]
-    float *part = xm + 4 * slots;                                                     // [group][n_nominal][part_stride]
-    const int ps = part_stride(slots, red);
+    float *part = xm + 4 * slots;                                                     // [group][n_nominal][ks]
     const int lane = threadIdx.x & 63;
     const int t = lane & 7;
     const int h = wave % ks, g = wave / ks;
@@ -157,7 +156,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q5k_chunk(const uint8_t *__restr
     const int sub_a = ORDER == 0 ? t : c2, sub_b = ORDER == 0 ? t : c2 + 1;
     const bool lane_valid = h * 8 + (lane >> 3) < spr;  // the last chunk of a row may be short
 
-    float *pp = part + (size_t)(g * n_nominal) * ps + slot;
+    float *pp = part + (size_t)(g * n_nominal) * ks + h;
     auto consume = [&](int i, const u4v a, const u4v b) {
         if (i < nt_wave) {  // wave-uniform
             u4v *st4 = reinterpret_cast<u4v *>(stage);
@@ -205,7 +204,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q5k_chunk(const uint8_t *__restr
             scale_min_k4(sub_b, s0, s1, s2, sc_b, m_b);
             const float d = f16_bits_to_f32(hd & 0xFFFFu), dmin = f16_bits_to_f32(hd >> 16);
             const float val = d * __builtin_fmaf(sc_a * xmr.x, fa, (sc_b * xmr.y) * fb) - dmin * __builtin_fmaf(m_a, xmr.z, m_b * xmr.w);
-            pp[(size_t)i * ps] = lane_valid ? val : 0.0f;
+            store_chunk_sum(pp + (size_t)i * ks, lane_valid ? val : 0.0f, lane);
         }
     };
 
@@ -232,7 +231,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q5k_chunk(const uint8_t *__restr
     }
     __syncthreads();
 
-    reduce_rows(part, ps, slots, red, wg_r0, wg_r1 - wg_r0, rows_per_wave, n_nominal, nthreads, y);
+    reduce_rows(part, ks, wg_r0, wg_r1 - wg_r0, rows_per_wave, n_nominal, nthreads, y);
 }
 
 }  // namespace
@@ -252,7 +251,6 @@ hipError_t launch_qgemv_q5k(const uint8_t *w, int64_t n, int64_t k, const void *
     const gemv::ChunkPlan plan = gemv::plan_chunks(n, ks, kStageBytes, lds_x);
     const int64_t n_wg = plan.n_wg, rows_per_wg = plan.rows_per_wg, rows_per_wave = plan.rows_per_wave, n_nominal = plan.n_nominal,
                   threads = plan.threads;
-    const int red = plan.red;
     const size_t lds = plan.lds;
     if (lds > gemv::kMaxLds) return hipErrorInvalidValue;
     const bool single = n_nominal <= kDepth;
@@ -263,7 +261,7 @@ hipError_t launch_qgemv_q5k(const uint8_t *w, int64_t n, int64_t k, const void *
             if (e != hipSuccess) return e;
         }
         hipLaunchKernelGGL(kern, dim3((unsigned)n_wg), dim3((unsigned)threads), lds, s, w, x, y, (int)n, spr, (int)rows_per_wg,
-                           (int)rows_per_wave, (int)n_nominal, red, (int)threads, (uint32_t)((w_bytes - 1) & ~(uint64_t)15));
+                           (int)rows_per_wave, (int)n_nominal, (int)threads, (uint32_t)((w_bytes - 1) & ~(uint64_t)15));
         return hipGetLastError();
     };
     if (order == kOrderRef) {

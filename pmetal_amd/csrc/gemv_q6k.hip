@@ -126,7 +126,7 @@ __device__ __forceinline__ float lane_dot(const Task &t, const uint32_t (&xr)[kP
 template <bool XF32, bool SINGLE, bool RAGGED>
 __global__ __launch_bounds__(1024) void k_qgemv_q6k_chunk(const uint8_t *__restrict__ W, const void *__restrict__ xg,
                                                            float *__restrict__ y, int n_rows, int spr, int rows_per_wg,
-                                                           int rows_per_wave, int n_nominal, int red, int nthreads,
+                                                           int rows_per_wave, int n_nominal, int nthreads,
                                                            uint32_t w_last) {
     extern __shared__ uint4 smem[];
     const int ks = (spr + 7) >> 3;
@@ -136,8 +136,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q6k_chunk(const uint8_t *__restr
     uint32_t *stage = reinterpret_cast<uint32_t *>(smem) + wave_id * (kStageBytes / 4);  // this wave's row chunk
     uint32_t *xd = reinterpret_cast<uint32_t *>(smem) + n_waves * (kStageBytes / 4);     // [kPlanes * 8][slots]
     float *xm = reinterpret_cast<float *>(xd + kPlanes * 8 * slots);  // [slots][4]
-    float *part = xm + 4 * slots;                              // [group][n_nominal][part_stride]
-    const int ps = part_stride(slots, red);
+    float *part = xm + 4 * slots;                              // [group][n_nominal][ks]
     const int lane = threadIdx.x & 63;
     const int t = lane & 7, hh = t >> 2, tq = t & 3;
     const int wave = wave_id;
@@ -190,7 +189,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q6k_chunk(const uint8_t *__restr
     const uint32_t c_ql = 16u * hh + 4u * tq, c_qh = 32u + 8u * hh + 4u * (tq & 1), c_sc = 48u + 2u * hh, c_d = 52u;  // dwords into the block
     const bool lane_valid = !RAGGED || h * 8 + (lane >> 3) < spr;  // the last chunk of a ragged row is short
 
-    float *pp = part + (size_t)(g * n_nominal) * ps + slot;
+    float *pp = part + (size_t)(g * n_nominal) * ks + h;
     auto consume = [&](int i, const u4v a, const u4v b) {
         if (i < nt_wave) {  // wave-uniform
             u4v *st4 = reinterpret_cast<u4v *>(stage);
@@ -217,7 +216,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q6k_chunk(const uint8_t *__restr
             tk.sc[1] = __builtin_amdgcn_alignbit(ws[2], ws[1], sh);
             tk.d = (blk[c_d] >> sh) & 0xFFFFu;
             const float val = lane_dot<kPlanes>(tk, xr, xmr, sh_a, sh_b, sc_up);
-            pp[(size_t)i * ps] = lane_valid ? val : 0.0f;
+            store_chunk_sum(pp + (size_t)i * ks, lane_valid ? val : 0.0f, lane);
         }
     };
 
@@ -244,7 +243,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q6k_chunk(const uint8_t *__restr
     }
     __syncthreads();
 
-    reduce_rows(part, ps, slots, red, wg_r0, wg_r1 - wg_r0, rows_per_wave, n_nominal, nthreads, y);
+    reduce_rows(part, ks, wg_r0, wg_r1 - wg_r0, rows_per_wave, n_nominal, nthreads, y);
 }
 
 }  // namespace
@@ -260,15 +259,13 @@ bool try_launch_qgemv_q6k_chunk(const uint8_t *w, int64_t n, int64_t k, const vo
     const bool ragged = spr % 8 != 0;
     const int ks = (spr + 7) / 8;
     const uint64_t w_bytes = (uint64_t)n * (uint64_t)spr * 210u;
-    static const int64_t mode = gemv::tuning("PMETAL_HIP_GEMV_Q6K_KERNEL", 0);  // 0 = choose, 1 = chunk kernel, 2 = general kernel
-    if (mode == 2 || ks > 16 || w_bytes >= (1ull << 32)) return false;
-    if (mode == 0 && w_bytes < (12ull << 20)) return false;
+    if (ks > 16 || w_bytes >= (1ull << 32)) return false;
+    if (w_bytes < (12ull << 20)) return false;  // measured crossover with the general kernel
     const size_t slots = (size_t)ks * 64;
     const size_t lds_x = slots * 4 * (kPlanes * 8) + slots * 16;
     const gemv::ChunkPlan plan = gemv::plan_chunks(n, ks, kStageBytes, lds_x);
     const int64_t n_wg = plan.n_wg, rows_per_wg = plan.rows_per_wg, rows_per_wave = plan.rows_per_wave, n_nominal = plan.n_nominal,
                   threads = plan.threads;
-    const int red = plan.red;
     const size_t lds = plan.lds;
     if (lds > 128 * 1024) return false;
     const bool single = n_nominal <= kDepth;
@@ -279,7 +276,7 @@ bool try_launch_qgemv_q6k_chunk(const uint8_t *w, int64_t n, int64_t k, const vo
             if (e != hipSuccess) return e;
         }
         hipLaunchKernelGGL(kern, dim3((unsigned)n_wg), dim3((unsigned)threads), lds, s, w, x, y, (int)n, spr, (int)rows_per_wg,
-                           (int)rows_per_wave, (int)n_nominal, red, (int)threads, (uint32_t)((w_bytes - 1) & ~(uint64_t)15));
+                           (int)rows_per_wave, (int)n_nominal, (int)threads, (uint32_t)((w_bytes - 1) & ~(uint64_t)15));
         return hipGetLastError();
     };
     if (ragged) {

@@ -80,7 +80,7 @@ __device__ __forceinline__ void stage_x(const void *__restrict__ xg, int slots, 
 template <bool XF32, bool SINGLE, bool RAGGED>
 __global__ __launch_bounds__(1024) void k_qgemv_q8_0_chunk(const uint8_t *__restrict__ W, const void *__restrict__ xg,
                                                             float *__restrict__ y, int n_rows, int bpr, int rows_per_wg,
-                                                            int rows_per_wave, int n_nominal, int red, int nthreads,
+                                                            int rows_per_wave, int n_nominal, int nthreads,
                                                             uint32_t w_last) {
     extern __shared__ uint4 smem[];
     const int ks = (bpr + 63) >> 6;
@@ -91,8 +91,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q8_0_chunk(const uint8_t *__rest
     uint32_t *stage = reinterpret_cast<uint32_t *>(smem) + wave * (kStageBytes / 4);  // this wave's row chunk
     uint32_t *xd = reinterpret_cast<uint32_t *>(smem) + n_waves * (kStageBytes / 4);  // [kPlanes * 8][slots]
     float *xm = reinterpret_cast<float *>(xd + kPlanes * 8 * slots);                  // [slots]
-    float *part = xm + slots;                                                         // [group][n_nominal][part_stride]
-    const int ps = part_stride(slots, red);
+    float *part = xm + slots;                                                         // [group][n_nominal][ks]
     const int h = wave % ks, g = wave / ks;
     const int wg_r0 = blockIdx.x * rows_per_wg;
     const int wg_r1 = wg_r0 + rows_per_wg < n_rows ? wg_r0 + rows_per_wg : n_rows;
@@ -137,7 +136,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q8_0_chunk(const uint8_t *__rest
     const uint32_t d_shift = odd ? 16u : 0u, q_shift = odd ? 0u : 16u;
     const bool lane_valid = !RAGGED || slot < bpr;  // the last chunk of a ragged row is short
 
-    float *pp = part + (size_t)(g * n_nominal) * ps + slot;
+    float *pp = part + (size_t)(g * n_nominal) * ks + h;
     auto consume = [&](int i, const u4v a, const u4v b, const u4v c) {
         if (i < nt_wave) {  // wave-uniform
         u4v *st4 = reinterpret_cast<u4v *>(stage);
@@ -160,7 +159,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q8_0_chunk(const uint8_t *__rest
         float f = (float)acc[kPlanes - 1];
 #pragma unroll
         for (int p = kPlanes - 2; p >= 0; p--) f = __builtin_fmaf(f, 256.0f, (float)acc[p]);
-        pp[(size_t)i * ps] = lane_valid ? (f16_bits_to_f32((dw >> d_shift) & 0xFFFFu) * xscale) * f : 0.0f;
+        store_chunk_sum(pp + (size_t)i * ks, lane_valid ? (f16_bits_to_f32((dw >> d_shift) & 0xFFFFu) * xscale) * f : 0.0f, lane);
         }
     };
 
@@ -187,7 +186,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q8_0_chunk(const uint8_t *__rest
     }
     __syncthreads();
 
-    reduce_rows(part, ps, slots, red, wg_r0, wg_r1 - wg_r0, rows_per_wave, n_nominal, nthreads, y);
+    reduce_rows(part, ks, wg_r0, wg_r1 - wg_r0, rows_per_wave, n_nominal, nthreads, y);
 }
 
 }  // namespace
@@ -203,14 +202,12 @@ bool try_launch_qgemv_q8_0_chunk(const uint8_t *w, int64_t n, int64_t k, const v
     const bool ragged = bpr % 64 != 0;
     const int ks = (bpr + 63) / 64;
     const uint64_t w_bytes = (uint64_t)n * (uint64_t)bpr * 34u;
-    static const int64_t mode = gemv::tuning("PMETAL_HIP_GEMV_Q8_0_KERNEL", 0);  // 0 = choose, 1 = this kernel, 2 = general kernel
-    if (mode == 2 || ks > 16 || w_bytes >= (1ull << 32)) return false;
-    if (mode == 0 && w_bytes < (12ull << 20)) return false;
+    if (ks > 16 || w_bytes >= (1ull << 32)) return false;
+    if (w_bytes < (12ull << 20)) return false;  // measured crossover with the general kernel
     const size_t slots = (size_t)ks * 64;
     const gemv::ChunkPlan plan = gemv::plan_chunks(n, ks, kStageBytes, slots * 4 * (kPlanes * 8) + slots * 4);
     const int64_t n_wg = plan.n_wg, rows_per_wg = plan.rows_per_wg, rows_per_wave = plan.rows_per_wave, n_nominal = plan.n_nominal,
                   threads = plan.threads;
-    const int red = plan.red;
     const size_t lds = plan.lds;
     if (lds > 128 * 1024) return false;
     const bool single = n_nominal <= kDepth;
@@ -221,7 +218,7 @@ bool try_launch_qgemv_q8_0_chunk(const uint8_t *w, int64_t n, int64_t k, const v
             if (e != hipSuccess) return e;
         }
         hipLaunchKernelGGL(kern, dim3((unsigned)n_wg), dim3((unsigned)threads), lds, s, w, x, y, (int)n, bpr, (int)rows_per_wg,
-                           (int)rows_per_wave, (int)n_nominal, red, (int)threads, (uint32_t)((w_bytes - 1) & ~(uint64_t)15));
+                           (int)rows_per_wave, (int)n_nominal, (int)threads, (uint32_t)((w_bytes - 1) & ~(uint64_t)15));
         return hipGetLastError();
     };
     if (ragged) {

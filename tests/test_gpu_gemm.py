@@ -365,3 +365,30 @@ def test_qlinear_q5k_q3k_q2k_dispatch(oracle, t):
     assert lib.pmetal_hip_qgemm(t, dw.ptr, n, k, dx.ptr, pm.DTYPE_F32, 3, dy.ptr + 4, pm.DTYPE_F32, 0, None) == 1
     assert lib.pmetal_hip_qgemm(t, dw.ptr, n, k, dx.ptr, pm.DTYPE_F32, 3, dy.ptr, 7, 0, None) == 1
     lib.pmetal_hip_clear_error()
+
+
+def test_qlinear_falls_back_to_the_gemm_when_the_gemv_refuses_the_row_length(oracle):
+    """Q5_K rows longer than the GEMV's activation staging (k > 32768): one activation row still has the re-blocked GEMM.
+    A Q8_0 row that is not a multiple of 256 with a bf16 output has no kernel and says so."""
+    lib = _lib.load()
+    n, k = 64, 33024
+    rng = np.random.default_rng(77)
+    wq = oracle.quantize(13, (rng.standard_normal(n * k) * 0.02).astype(np.float32))
+    x = rng.standard_normal(k).astype(np.float32)
+    bits = oracle.f32_to_bf16_bits(x)
+    xr = oracle.bf16_bits_to_f32(bits)
+    dw, dx, dy = pm.DeviceBuffer.from_host(wq), pm.DeviceBuffer.from_host(bits), pm.DeviceBuffer(4 * n)
+    assert lib.pmetal_hip_qgemv(13, dw.ptr, n, k, dx.ptr, pm.DTYPE_BF16, dy.ptr, 0, None) == 7
+    msg = lib.pmetal_hip_last_error_message()
+    assert b"n=64" in msg and b"k=33024" in msg
+    pm.check(lib.pmetal_hip_qlinear(13, dw.ptr, n, k, dx.ptr, pm.DTYPE_BF16, 1, dy.ptr, pm.DTYPE_F32, 0, None))
+    pm.check(lib.pmetal_hip_sync(None))
+    want = oracle.qmatvec(13, wq, n, k, xr)
+    elem, norm = rel_errors(dy.to_host(np.float32), want)
+    assert elem <= TOL and norm <= TOL, (elem, norm)
+    w8 = pm.DeviceBuffer.from_host(oracle.quantize(Q8_0, (rng.standard_normal(64 * 96) * 0.02).astype(np.float32)))
+    y16 = pm.DeviceBuffer(2 * 4 * 64)
+    x8 = pm.DeviceBuffer.from_host(bits[:4 * 96].copy())
+    assert lib.pmetal_hip_qlinear(Q8_0, w8.ptr, 64, 96, x8.ptr, pm.DTYPE_BF16, 4, y16.ptr, pm.DTYPE_BF16, 0, None) == 6
+    assert b"f32 only" in lib.pmetal_hip_last_error_message()
+    lib.pmetal_hip_clear_error()

@@ -72,3 +72,53 @@ def test_record_argument_errors():
     assert lib.pmetal_hip_recording_destroy(None) == 0
     assert lib.pmetal_hip_stream_destroy(None) == 0
     lib.pmetal_hip_clear_error()
+
+
+def test_recorded_qgemm_survives_a_larger_call_on_the_same_stream(oracle):
+    """A recording of the fused GEMM names the library's scratch buffer.  A larger call on the same stream afterwards
+    gets a new buffer, the recorded one stays alive, and the replay reproduces the eager bits; a shape the stream's
+    buffer cannot hold is refused while the stream is being recorded."""
+    lib = _lib.load()
+    n, k, m = 512, 1024, 24
+    w = pm.DeviceBuffer.from_host(oracle.quantize(Q4K, weights(900, n * k)))
+    xb = oracle.f32_to_bf16_bits(np.random.default_rng(901).standard_normal(m * k).astype(np.float32))
+    x = pm.DeviceBuffer.from_host(xb)
+    y = pm.DeviceBuffer(4 * m * n)
+    n2, k2, m2 = 768, 2048, 200
+    w2 = pm.DeviceBuffer.from_host(oracle.quantize(Q4K, weights(902, n2 * k2)))
+    x2 = pm.DeviceBuffer.from_host(oracle.f32_to_bf16_bits(np.random.default_rng(903).standard_normal(m2 * k2).astype(np.float32)))
+    y2 = pm.DeviceBuffer(4 * m2 * n2)
+    stream = lib.pmetal_hip_stream_create()
+    assert stream
+    try:
+        # nothing has run on this stream yet: a recording cannot allocate the scratch
+        pm.check(lib.pmetal_hip_record_begin(stream))
+        rc = lib.pmetal_hip_qgemm(Q4K, w.ptr, n, k, x.ptr, pm.DTYPE_BF16, m, y.ptr, pm.DTYPE_F32, 0, stream)
+        assert rc == 1 and b"recorded" in lib.pmetal_hip_last_error_message()
+        lib.pmetal_hip_clear_error()
+        dead = lib.pmetal_hip_record_end(stream)
+        if dead:
+            pm.check(lib.pmetal_hip_recording_destroy(dead))
+        lib.pmetal_hip_clear_error()
+        # eager run (allocates the stream's scratch), then the recording
+        pm.check(lib.pmetal_hip_qgemm(Q4K, w.ptr, n, k, x.ptr, pm.DTYPE_BF16, m, y.ptr, pm.DTYPE_F32, 0, stream))
+        pm.check(lib.pmetal_hip_sync(stream))
+        eager = y.to_host(np.float32).copy()
+        assert np.isfinite(eager).all()
+        pm.check(lib.pmetal_hip_record_begin(stream))
+        pm.check(lib.pmetal_hip_qgemm(Q4K, w.ptr, n, k, x.ptr, pm.DTYPE_BF16, m, y.ptr, pm.DTYPE_F32, 0, stream))
+        rec = lib.pmetal_hip_record_end(stream)
+        assert rec, lib.pmetal_hip_last_error_message()
+        try:
+            for rep in range(3):
+                # a larger product on the same stream between replays: its scratch must not replace the recorded one
+                pm.check(lib.pmetal_hip_qgemm(Q4K, w2.ptr, n2, k2, x2.ptr, pm.DTYPE_BF16, m2, y2.ptr, pm.DTYPE_F32, 0, stream))
+                pm.check(lib.pmetal_hip_memset(y.ptr, 0xFF, 4 * m * n, None))
+                pm.check(lib.pmetal_hip_sync(None))
+                pm.check(lib.pmetal_hip_replay(rec, stream))
+                pm.check(lib.pmetal_hip_sync(stream))
+                assert np.array_equal(y.to_host(np.float32), eager), rep
+        finally:
+            pm.check(lib.pmetal_hip_recording_destroy(rec))
+    finally:
+        pm.check(lib.pmetal_hip_stream_destroy(stream))

@@ -272,3 +272,28 @@ def test_gpu_q2k_q3k_gemv_unit_vectors_and_linear(oracle, t):
     pm.check(lib.pmetal_hip_qgemm(t, dw.ptr, n, k, dx.ptr, pm.DTYPE_F32, m, dy.ptr, pm.DTYPE_F32, 0, None))
     pm.check(lib.pmetal_hip_sync(None))
     assert np.allclose(dy.to_host(np.float32).reshape(m, n), got, rtol=0, atol=1e-3 * np.abs(got).max())  # f32 activations: f16-rounded in the GEMM
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("t", [Q3K, Q2K, 13])
+def test_gpu_gemv_vocabulary_sized_matrix(oracle, t):
+    """An output projection of 128256 x 4096 (501 rows per workgroup): the row sums go through LDS one float per row and
+    chunk, so the row count of a matrix does not limit the kernel.  Random block bytes; the reference covers the first
+    and last 256 rows and 512 rows drawn at random."""
+    import pmetal_amd as pm
+    from gpu_util import gpu_qgemv, rel_errors
+    n, k = 128256, 4096
+    ts = {Q3K: 110, Q2K: 84, 13: 176}[t]
+    rng = np.random.default_rng(40 + t)
+    raw = rng.integers(0, 256, n * (k // 256) * ts, dtype=np.uint8)
+    blocks = raw.reshape(-1, ts)
+    for off in {Q3K: (109,), Q2K: (81, 83), 13: (1, 3)}[t]:  # keep the f16 scales finite and small
+        blocks[:, off] &= 0x3F
+    x = rng.standard_normal(k).astype(np.float32)
+    got = gpu_qgemv(t, raw, n, k, x, pm.DTYPE_F32)
+    rows = np.unique(np.concatenate([np.arange(256), np.arange(n - 256, n), rng.choice(n, 512, replace=False)]))
+    row_bytes = k // 256 * ts
+    want = oracle.qmatvec(t, raw.reshape(n, row_bytes)[rows].reshape(-1), rows.size, k, x)
+    elem, norm = rel_errors(got[rows], want)
+    assert elem <= 1e-3 and norm <= 1e-3, (elem, norm)
+    assert np.isfinite(got).all()
