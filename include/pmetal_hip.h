@@ -192,6 +192,22 @@ int32_t pmetal_hip_qlinear(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, 
                            uint32_t x_dtype, int64_t m, void *y_dev, uint32_t y_dtype, uint32_t order,
                            void *stream);
 
+/* Re-blocked weights for the GEMM of Q5_K / Q3_K / Q2_K.  The reference brings a weight into the layout its matmul wants
+ * once, when the model is loaded (LayerWeight, crates/pmetal-bridge/src/qwen3_native/weights.rs:29-45: dense weights are
+ * transposed at load time, quantized ones kept as MLX's quantized_matmul reads them); the counterpart here: these three
+ * types have no GEMM kernel of their own, and their super-blocks convert without loss into one (Q3_K) or two (Q5_K, Q2_K:
+ * values and mins) Q6_K tensors.  pmetal_hip_reblock_dev does that conversion once into memory the caller owns
+ * (pmetal_hip_reblock_size bytes: 210 bytes per super-block and part, each part rounded up to 16; 0 for a type or shape
+ * that is not re-blocked); pmetal_hip_qgemm_reblocked multiplies with it: the same result as pmetal_hip_qgemm, which does
+ * both steps on every call (into scratch of that size) when handed the original blocks.  `order` applies to Q5_K only.
+ * The GEMV of these types reads the original blocks; a caller that wants both keeps both.                              */
+size_t pmetal_hip_reblock_size(uint32_t ggml_type, int64_t n, int64_t k);
+int32_t pmetal_hip_reblock_dev(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, int64_t k, uint32_t order,
+                               uint8_t *dst_dev, size_t dst_len, void *stream);
+int32_t pmetal_hip_qgemm_reblocked(uint32_t ggml_type, const uint8_t *reblocked_dev, size_t reblocked_len, int64_t n,
+                                   int64_t k, const void *x_dev, uint32_t x_dtype, int64_t m, void *y_dev, uint32_t y_dtype,
+                                   void *stream);
+
 /* One decode step's worth of batch-1 projections, launched back to back on one stream
  * (the per-token loop over LayerWeight::matmul_from, weights.rs:66-84). */
 typedef struct pmetal_hip_linear_desc {

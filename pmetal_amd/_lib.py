@@ -52,6 +52,9 @@ SYMBOLS = [
     ("pmetal_hip_qgemv", _i32, [_u32, _vp, _i64, _i64, _vp, _u32, _vp, _u32, _vp]),
     ("pmetal_hip_qgemm", _i32, [_u32, _vp, _i64, _i64, _vp, _u32, _i64, _vp, _u32, _u32, _vp]),
     ("pmetal_hip_qgemm_noalloc", _i32, [_u32, _vp, _i64, _i64, _vp, _u32, _i64, _vp, _u32, _u32, _vp]),
+    ("pmetal_hip_reblock_size", _sz, [_u32, _i64, _i64]),
+    ("pmetal_hip_reblock_dev", _i32, [_u32, _vp, _i64, _i64, _u32, _vp, _sz, _vp]),
+    ("pmetal_hip_qgemm_reblocked", _i32, [_u32, _vp, _sz, _i64, _i64, _vp, _u32, _i64, _vp, _u32, _vp]),
     ("pmetal_hip_qlinear", _i32, [_u32, _vp, _i64, _i64, _vp, _u32, _i64, _vp, _u32, _u32, _vp]),
     ("pmetal_hip_qgemv_batch", _i32, [C.POINTER(LinearDesc), _sz, _vp]),
     ("pmetal_hip_q8k_size", _sz, [_sz]),

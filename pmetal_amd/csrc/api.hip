@@ -610,36 +610,99 @@ int32_t pmetal_hip_qgemv_batch(const pmetal_hip_linear_desc *descs, size_t count
 }
 
 // Q5_K, Q3_K and Q2_K have no GEMM kernel of their own: their super-blocks are re-blocked, exactly, into one or two Q6_K
-// tensors in the scratch buffer (W = A + B), which go through the Q6_K GEMM; two partial results are added in f32.
-static int32_t qgemm_reblocked(uint32_t t, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, int64_t m, void *y,
-                               uint32_t y_dtype, uint32_t order, void *stream) {
-    auto up16 = [](size_t v) { return (v + 15) & ~(size_t)15; };
-    hipStream_t s = (hipStream_t)stream;
+// tensors (W = A + B), which go through the Q6_K GEMM; two partial results are added in f32.  The re-blocked tensors are
+// [A][B], each n * (k / 256) * 210 bytes rounded up to 16.
+static size_t up16(size_t v) { return (v + 15) & ~(size_t)15; }
+
+static size_t reblocked_part_bytes(int64_t n, int64_t k) { return up16((size_t)n * (size_t)(k / 256) * 210); }
+
+// The GEMM over re-blocked weights.  scratch: [GEMM scratch][partial result of B][partial result of A when y is not f32].
+static int32_t qgemm_over_reblocked(uint32_t t, const uint8_t *wa, int64_t n, int64_t k, const void *x, uint32_t x_dtype, int64_t m,
+                                    void *y, uint32_t y_dtype, uint8_t *scratch, size_t gemm_bytes, hipStream_t s) {
     const int parts = pmh::reblock_q6k_parts(t);
-    const size_t n_blocks = (size_t)n * (size_t)(k / 256);
-    if (n_blocks > SIZE_MAX / 512 || (size_t)m > SIZE_MAX / 16 / (size_t)n)
-        return fail(PMETAL_HIP_ERR_SHAPE_TOO_LARGE, "qgemm: shape is too large");
-    const size_t gemm_bytes = up16(pmh::qgemm_workspace_bytes(m, n, k)), w_bytes = up16(n_blocks * 210);
     const size_t y_elems = (size_t)m * (size_t)n, y_bytes = up16(y_elems * 4);
     const bool y_f32 = y_dtype == PMETAL_HIP_DTYPE_F32;
-    // scratch: [GEMM scratch][A][B][partial result of B][partial result of A when y is not f32]
-    const size_t total = gemm_bytes + parts * w_bytes + (parts == 2 ? y_bytes * (y_f32 ? 1 : 2) : 0);
-    void *ws = nullptr;
-    if (int32_t rc = workspace(total, s, &ws)) return rc;
-    uint8_t *base = (uint8_t *)ws, *wa = base + gemm_bytes, *wb = wa + w_bytes;
-    float *yb = (float *)(wb + w_bytes), *ya = y_f32 ? (float *)y : (float *)((uint8_t *)yb + y_bytes);
-    hipError_t e = pmh::launch_reblock_q6k(t, w, n_blocks, order, wa, wb, s);
-    if (e != hipSuccess) return hip_fail(e, "re-blocking kernel launch");
+    const uint8_t *wb = wa + reblocked_part_bytes(n, k);
+    float *yb = (float *)(scratch + gemm_bytes), *ya = y_f32 ? (float *)y : (float *)((uint8_t *)yb + y_bytes);
+    hipError_t e;
     if (parts == 1) {
-        e = pmh::launch_qgemm(PMETAL_GGML_TYPE_Q6K, wa, n, k, x, x_dtype, m, y, y_dtype, 0, ws, s);
-    } else {
-        e = pmh::launch_qgemm(PMETAL_GGML_TYPE_Q6K, wa, n, k, x, x_dtype, m, ya, PMETAL_HIP_DTYPE_F32, 0, ws, s);
-        if (e == hipSuccess) e = pmh::launch_qgemm(PMETAL_GGML_TYPE_Q6K, wb, n, k, x, x_dtype, m, yb, PMETAL_HIP_DTYPE_F32, 0, ws, s);
+        e = pmh::launch_qgemm(PMETAL_GGML_TYPE_Q6K, wa, n, k, x, x_dtype, m, y, y_dtype, 0, scratch, s);
+    } else {  // the second product reuses the first one's converted activations
+        e = pmh::launch_qgemm(PMETAL_GGML_TYPE_Q6K, wa, n, k, x, x_dtype, m, ya, PMETAL_HIP_DTYPE_F32, 0, scratch, s);
+        if (e == hipSuccess) e = pmh::launch_qgemm(PMETAL_GGML_TYPE_Q6K, wb, n, k, x, x_dtype, m, yb, PMETAL_HIP_DTYPE_F32, 0, scratch, s, true);
         if (e == hipSuccess) e = pmh::launch_add_store(ya, yb, y_elems, y, !y_f32, s);
     }
     if (e == hipErrorNotSupported) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "qgemm: configuration not supported");
     if (e != hipSuccess) return hip_fail(e, "qgemm kernel launch");
     return ok();
+}
+
+static size_t reblocked_scratch_bytes(uint32_t t, int64_t m, int64_t n, int64_t k, uint32_t y_dtype, size_t *gemm_bytes) {
+    *gemm_bytes = up16(pmh::qgemm_workspace_bytes(m, n, k));
+    const size_t y_bytes = up16((size_t)m * (size_t)n * 4);
+    return *gemm_bytes + (pmh::reblock_q6k_parts(t) == 2 ? y_bytes * (y_dtype == PMETAL_HIP_DTYPE_F32 ? 1 : 2) : 0);
+}
+
+static int32_t check_reblocked_shape(int64_t n, int64_t k, int64_t m) {
+    const size_t n_blocks = (size_t)n * (size_t)(k / 256);
+    if (n_blocks > SIZE_MAX / 512 || (m > 0 && (size_t)m > SIZE_MAX / 16 / (size_t)n))
+        return fail(PMETAL_HIP_ERR_SHAPE_TOO_LARGE, "qgemm: shape is too large");
+    return PMETAL_HIP_OK;
+}
+
+// qgemm for these types when the caller has not re-blocked: re-block into the scratch buffer, then multiply.
+static int32_t qgemm_reblocked(uint32_t t, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, int64_t m, void *y,
+                               uint32_t y_dtype, uint32_t order, void *stream) {
+    hipStream_t s = (hipStream_t)stream;
+    if (int32_t rc = check_reblocked_shape(n, k, m)) return rc;
+    const int parts = pmh::reblock_q6k_parts(t);
+    size_t gemm_bytes = 0;
+    const size_t mul_bytes = reblocked_scratch_bytes(t, m, n, k, y_dtype, &gemm_bytes), w_bytes = reblocked_part_bytes(n, k);
+    void *ws = nullptr;
+    if (int32_t rc = workspace(mul_bytes + parts * w_bytes, s, &ws)) return rc;
+    uint8_t *wa = (uint8_t *)ws + mul_bytes;
+    hipError_t e = pmh::launch_reblock_q6k(t, w, (size_t)n * (size_t)(k / 256), order, wa, wa + w_bytes, s);
+    if (e != hipSuccess) return hip_fail(e, "re-blocking kernel launch");
+    return qgemm_over_reblocked(t, wa, n, k, x, x_dtype, m, y, y_dtype, (uint8_t *)ws, gemm_bytes, s);
+}
+
+size_t pmetal_hip_reblock_size(uint32_t t, int64_t n, int64_t k) {
+    if (!gemv_only_type(t) || n <= 0 || k <= 0 || k % 256 != 0) return 0;
+    return (size_t)pmh::reblock_q6k_parts(t) * reblocked_part_bytes(n, k);
+}
+
+int32_t pmetal_hip_reblock_dev(uint32_t t, const uint8_t *w, int64_t n, int64_t k, uint32_t order, uint8_t *dst, size_t dst_len,
+                               void *stream) {
+    if (!gemv_only_type(t)) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "GGML type %u is not re-blocked (Q5_K, Q3_K and Q2_K are)", t);
+    if (int32_t rc = check_linear(t, w, n, k, w, 0, dst, order, true)) return rc;
+    if (!aligned16(dst)) return fail(PMETAL_HIP_ERR_INVALID_ARG, "device pointers must be 16-byte aligned");
+    if (int32_t rc = check_reblocked_shape(n, k, 0)) return rc;
+    const size_t expected = pmetal_hip_reblock_size(t, n, k);
+    if (dst_len != expected) return fail(PMETAL_HIP_ERR_INVALID_SIZE, "Invalid data size: expected %zu bytes, got %zu", expected, dst_len);
+    const size_t w_bytes = reblocked_part_bytes(n, k);
+    hipError_t e = pmh::launch_reblock_q6k(t, w, (size_t)n * (size_t)(k / 256), order, dst, dst + w_bytes, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "re-blocking kernel launch");
+    return ok();
+}
+
+int32_t pmetal_hip_qgemm_reblocked(uint32_t t, const uint8_t *reblocked, size_t reblocked_len, int64_t n, int64_t k, const void *x,
+                                   uint32_t x_dtype, int64_t m, void *y, uint32_t y_dtype, void *stream) {
+    if (!gemv_only_type(t)) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "GGML type %u is not re-blocked (Q5_K, Q3_K and Q2_K are)", t);
+    if (int32_t rc = check_linear(t, reblocked, n, k, x, x_dtype, y, 0, true)) return rc;
+    if (!aligned16(y)) return fail(PMETAL_HIP_ERR_INVALID_ARG, "device pointers must be 16-byte aligned");
+    if (y_dtype > PMETAL_HIP_DTYPE_BF16) return fail(PMETAL_HIP_ERR_INVALID_ARG, "y_dtype must be 0 (f32) or 1 (bf16)");
+    if (m <= 0 || m > 0x7FFFFFFF) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "m must be in [1, 2^31)");
+    if (!pmh::qgemm_fits(PMETAL_GGML_TYPE_Q6K, m, n, k))
+        return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qgemm: m and k must be at most 2^22 (m = %lld, k = %lld)", (long long)m, (long long)k);
+    if (int32_t rc = check_reblocked_shape(n, k, m)) return rc;
+    const size_t expected = pmetal_hip_reblock_size(t, n, k);
+    if (reblocked_len != expected)
+        return fail(PMETAL_HIP_ERR_INVALID_SIZE, "Invalid data size: expected %zu bytes of re-blocked weights, got %zu", expected, reblocked_len);
+    size_t gemm_bytes = 0;
+    const size_t mul_bytes = reblocked_scratch_bytes(t, m, n, k, y_dtype, &gemm_bytes);
+    void *ws = nullptr;
+    if (int32_t rc = workspace(mul_bytes, (hipStream_t)stream, &ws)) return rc;
+    return qgemm_over_reblocked(t, reblocked, n, k, x, x_dtype, m, y, y_dtype, (uint8_t *)ws, gemm_bytes, (hipStream_t)stream);
 }
 
 int32_t pmetal_hip_qgemm(uint32_t t, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, int64_t m,

@@ -407,13 +407,8 @@ __global__ __launch_bounds__(256) void k_dequantize_kq(const uint8_t *__restrict
 // W x = A x + B x then, every product exact.  One wave per super-block: lane i decodes elements 4 i .. 4 i + 3 into
 // LDS, then assembles ql bytes 2 i and 2 i + 1 and qh byte i of the Q6_K layout (k_quants.rs:1116-1130).
 template <class D>
-__global__ __launch_bounds__(256) void k_reblock_q6k(const uint8_t *__restrict__ src, size_t n_blocks, uint8_t *__restrict__ dst_a,
-                                                     uint8_t *__restrict__ dst_b) {
-    __shared__ __align__(16) uint8_t quants[4][256];
-    __shared__ int8_t scales[4][2][16];
-    const int w = (int)(threadIdx.x >> 6), i = (int)(threadIdx.x & 63);
-    const size_t blk_i = (size_t)blockIdx.x * 4 + w;
-    const bool live = blk_i < n_blocks;  // wave-uniform
+__device__ __forceinline__ void reblock_one(const uint8_t *__restrict__ src, size_t blk_i, bool live, int w, int i, uint8_t (&quants)[4][256],
+                                            int8_t (&scales)[4][2][16], uint8_t (&outbuf)[2][840]) {
     const uint8_t *blk = src + (live ? blk_i : 0) * D::kBytes;
     const typename D::Raw raw = D::load(blk, i);
     int q[4], sc, m;
@@ -433,17 +428,39 @@ __global__ __launch_bounds__(256) void k_reblock_q6k(const uint8_t *__restrict__
     const int e0 = 128 * (i >> 5) + (i & 31);  // qh byte i: bits 2 g .. 2 g + 1 from element e0 + 32 g
     const uint32_t qh = (uint32_t)(qv[e0] >> 4) | ((uint32_t)(qv[e0 + 32] >> 4) << 2) | ((uint32_t)(qv[e0 + 64] >> 4) << 4) |
                         ((uint32_t)(qv[e0 + 96] >> 4) << 6);
-    uint8_t *out = dst_a + blk_i * 210;
-    *reinterpret_cast<uint16_t *>(out + 2 * i) = (uint16_t)ql;
-    out[128 + i] = (uint8_t)qh;
-    if (i < 16) out[192 + i] = (uint8_t)scales[w][0][i];
-    if (i == 0) *reinterpret_cast<uint16_t *>(out + 208) = (uint16_t)D::d_bits(blk);
+    // the four super-blocks of the workgroup are 840 contiguous bytes of the output: assemble them in LDS, store dwords
+    uint8_t *oa = outbuf[0] + w * 210, *ob = outbuf[1] + w * 210;
+    *reinterpret_cast<uint16_t *>(oa + 2 * i) = (uint16_t)ql;
+    oa[128 + i] = (uint8_t)qh;
+    if (i < 16) oa[192 + i] = (uint8_t)scales[w][0][i];
+    if (i == 0) *reinterpret_cast<uint16_t *>(oa + 208) = (uint16_t)D::d_bits(blk);
     if (D::kHasMin) {
-        out = dst_b + blk_i * 210;
-        *reinterpret_cast<uint16_t *>(out + 2 * i) = 0xFFFFu;  // 31 = nibble 15, top bits 01
-        out[128 + i] = 0x55u;
-        if (i < 16) out[192 + i] = (uint8_t)scales[w][1][i];
-        if (i == 0) *reinterpret_cast<uint16_t *>(out + 208) = (uint16_t)D::dmin_bits(blk);
+        *reinterpret_cast<uint16_t *>(ob + 2 * i) = 0xFFFFu;  // 31 = nibble 15, top bits 01
+        ob[128 + i] = 0x55u;
+        if (i < 16) ob[192 + i] = (uint8_t)scales[w][1][i];
+        if (i == 0) *reinterpret_cast<uint16_t *>(ob + 208) = (uint16_t)D::dmin_bits(blk);
+    }
+}
+
+template <class D>
+__global__ __launch_bounds__(256) void k_reblock_q6k(const uint8_t *__restrict__ src, size_t n_blocks, uint8_t *__restrict__ dst_a,
+                                                     uint8_t *__restrict__ dst_b) {
+    __shared__ __align__(16) uint8_t quants[4][256];
+    __shared__ int8_t scales[4][2][16];
+    __shared__ __align__(16) uint8_t outbuf[2][840];
+    const size_t blk0 = (size_t)blockIdx.x * 4;
+    const int w = (int)(threadIdx.x >> 6), i = (int)(threadIdx.x & 63);
+    const bool live = blk0 + w < n_blocks;  // wave-uniform
+    reblock_one<D>(src, blk0 + w, live, w, i, quants, scales, outbuf);
+    __syncthreads();
+    const size_t left = n_blocks - blk0;
+    const unsigned bytes = (unsigned)(left < 4 ? left : 4) * 210u;  // a multiple of 4 except for one or three blocks (then of 2)
+    const unsigned t = threadIdx.x;
+    for (int part = 0; part < (D::kHasMin ? 2 : 1); part++) {
+        uint8_t *dst = (part ? dst_b : dst_a) + blk0 * 210;  // 840 bytes per workgroup: 8-byte aligned
+        const uint8_t *from = outbuf[part];
+        if (4 * t + 4 <= bytes) *reinterpret_cast<uint32_t *>(dst + 4 * t) = *reinterpret_cast<const uint32_t *>(from + 4 * t);
+        else if (4 * t + 2 <= bytes) *reinterpret_cast<uint16_t *>(dst + 4 * t) = *reinterpret_cast<const uint16_t *>(from + 4 * t);
     }
 }
 

@@ -1043,7 +1043,7 @@ static hipError_t launch_rw_q8(hipStream_t s, const uint8_t *w, const uint4 *xs,
 }
 
 hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype,
-                                int64_t m, void *y, uint32_t y_dtype, uint32_t order, void *workspace, hipStream_t s) {
+                                int64_t m, void *y, uint32_t y_dtype, uint32_t order, void *workspace, hipStream_t s, bool reuse_prepass) {
     if (!qgemm_fits(type, m, n, k)) return hipErrorInvalidValue;
     const GemmPlan p = qgemm_plan(m, n, k);
     const int spr = (int)(k / 256);
@@ -1063,7 +1063,9 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
             hipLaunchKernelGGL((k_prep_rw<F, O, 1>), dim3((unsigned)p.mp), dim3(512), 0, s, x, k, (int)m, (int)p.mp,         \
                                rowscale, xs);                                                                                \
     } while (0)
-    if (xf32) {
+    if (reuse_prepass) {
+        // the workspace still holds the converted activations of the previous call (same x, m, k and weight type)
+    } else if (xf32) {
         if (xorder == 0) PMH_PREP(true, 0);
         else if (xorder == 1) PMH_PREP(true, 1);
         else if (xorder == 2) PMH_PREP(true, 2);

@@ -68,8 +68,11 @@ bool qgemm_fits(uint32_t type, int64_t m, int64_t n, int64_t k);
 GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k);
 // Bytes of device workspace qgemm needs for (m, n, k); the caller provides it.
 size_t qgemm_workspace_bytes(int64_t m, int64_t n, int64_t k);
+// reuse_prepass: the workspace still holds the converted activations of the previous launch_qgemm on this stream with the same
+// x, m, k and weight type (two weights that share their activations: the pre-pass runs once)
 hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype,
-                        int64_t m, void *y, uint32_t y_dtype, uint32_t order, void *workspace, hipStream_t s);
+                        int64_t m, void *y, uint32_t y_dtype, uint32_t order, void *workspace, hipStream_t s,
+                        bool reuse_prepass = false);
 
 // ---- q8k.hip: Q8_K activation blocks and the integer dot products over them ----
 hipError_t launch_quantize_q8k(const float *x, size_t n, uint8_t *dst, hipStream_t s);
