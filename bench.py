@@ -418,13 +418,22 @@ def bench_gemm(args, m, n, k, t=Q4K):
     flops = 2.0 * m * n * k
     us = ev_ms * 1e3 / args.steps
     tflops = flops / (us * 1e-6) / 1e12
+    pair_us = None
+    if t in (Q4K, Q6K, Q8_0):  # two weights against the same activations (gate / up): one pre-pass for both
+        w2 = device_weights(pm, lib, t, n * k, 2001)
+        y2 = pm.DeviceBuffer(2 * m * n)
+        descs = (_lib.GemmDesc * 2)(_lib.GemmDesc(t, pm.DTYPE_BF16, 0, 0, n, w.ptr, y.ptr), _lib.GemmDesc(t, pm.DTYPE_BF16, 0, 0, n, w2.ptr, y2.ptr))
+        b_ms, _ = timer.run(lambda: pm.check(lib.pmetal_hip_qgemm_batch(descs, 2, k, x.ptr, pm.DTYPE_BF16, m, None)), args.steps, args.warmup)
+        pair_us = b_ms * 1e3 / args.steps / 2
     return {
         "value": tflops, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / BF16_PEAK_TFLOPS, 4), "traffic": None,
                      "kernel": {Q4K: "k_qgemm_rw", Q6K: "k_qgemm_rw_q6", Q8_0: "k_qgemm_rw_q8"}.get(t, "k_reblock_q6k + k_qgemm_rw_q6 per part") + " (+ k_prep_rw, k_rw_reduce when K is split)",
                      "flops_per_launch": flops, "us_per_launch": round(us, 3)},
-        "extra": {"mfma_loop_sustained_TFLOPs": round(sustained, 1), "frac_of_sustained": round(tflops / sustained, 4)},
+        "extra": {"mfma_loop_sustained_TFLOPs": round(sustained, 1), "frac_of_sustained": round(tflops / sustained, 4),
+                  "two_weights_sharing_x_us_per_weight": None if pair_us is None else round(pair_us, 3),
+                  "two_weights_sharing_x_TFLOPs": None if pair_us is None else round(flops / (pair_us * 1e-6) / 1e12, 1)},
     }, (t, n, k)
 
 

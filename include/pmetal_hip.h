@@ -192,6 +192,22 @@ int32_t pmetal_hip_qlinear(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, 
                            uint32_t x_dtype, int64_t m, void *y_dev, uint32_t y_dtype, uint32_t order,
                            void *stream);
 
+/* Several weights against the same [m, k] activations (the gate / up or q / k / v projections of a prefill: what a layer's
+ * consecutive LayerWeight::matmul_from calls on one input amount to, weights.rs:66-84): the same results as one
+ * pmetal_hip_qgemm per weight, bit for bit, with the activations converted once per element order instead of once per
+ * weight.  Q8_0, Q4_K and Q6_K; the weights may differ in type, n, output type and element order.                       */
+typedef struct pmetal_hip_gemm_desc {
+    uint32_t ggml_type;
+    uint32_t y_dtype;
+    uint32_t order;
+    uint32_t reserved;
+    int64_t n;
+    const uint8_t *w_dev;
+    void *y_dev;
+} pmetal_hip_gemm_desc;
+int32_t pmetal_hip_qgemm_batch(const pmetal_hip_gemm_desc *descs, size_t count, int64_t k, const void *x_dev,
+                               uint32_t x_dtype, int64_t m, void *stream);
+
 /* Re-blocked weights for the GEMM of Q5_K / Q3_K / Q2_K.  The reference brings a weight into the layout its matmul wants
  * once, when the model is loaded (LayerWeight, crates/pmetal-bridge/src/qwen3_native/weights.rs:29-45: dense weights are
  * transposed at load time, quantized ones kept as MLX's quantized_matmul reads them); the counterpart here: these three

@@ -18,6 +18,12 @@ class LinearDesc(C.Structure):
                 ("k", _i64), ("w_dev", _vp), ("x_dev", _vp), ("y_dev", _vp)]
 
 
+class GemmDesc(C.Structure):
+    """``pmetal_hip_gemm_desc``"""
+    _fields_ = [("ggml_type", _u32), ("y_dtype", _u32), ("order", _u32), ("reserved", _u32), ("n", _i64), ("w_dev", _vp),
+                ("y_dev", _vp)]
+
+
 SYMBOLS = [
     ("pmetal_hip_device_count", _i32, []),
     ("pmetal_hip_init", _i32, [_i32]),
@@ -52,6 +58,7 @@ SYMBOLS = [
     ("pmetal_hip_qgemv", _i32, [_u32, _vp, _i64, _i64, _vp, _u32, _vp, _u32, _vp]),
     ("pmetal_hip_qgemm", _i32, [_u32, _vp, _i64, _i64, _vp, _u32, _i64, _vp, _u32, _u32, _vp]),
     ("pmetal_hip_qgemm_noalloc", _i32, [_u32, _vp, _i64, _i64, _vp, _u32, _i64, _vp, _u32, _u32, _vp]),
+    ("pmetal_hip_qgemm_batch", _i32, [C.POINTER(GemmDesc), _sz, _i64, _vp, _u32, _i64, _vp]),
     ("pmetal_hip_reblock_size", _sz, [_u32, _i64, _i64]),
     ("pmetal_hip_reblock_dev", _i32, [_u32, _vp, _i64, _i64, _u32, _vp, _sz, _vp]),
     ("pmetal_hip_qgemm_reblocked", _i32, [_u32, _vp, _sz, _i64, _i64, _vp, _u32, _i64, _vp, _u32, _vp]),

@@ -730,6 +730,45 @@ int32_t pmetal_hip_qgemm(uint32_t t, const uint8_t *w, int64_t n, int64_t k, con
     return ok();
 }
 
+// Several weights against the same activations (gate / up, q / k / v of a prefill): the activation pre-pass runs once per
+// element order instead of once per weight.
+int32_t pmetal_hip_qgemm_batch(const pmetal_hip_gemm_desc *descs, size_t count, int64_t k, const void *x, uint32_t x_dtype, int64_t m,
+                               void *stream) {
+    if (count && !descs) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL descriptor array");
+    size_t need = 0;
+    for (size_t i = 0; i < count; i++) {
+        const pmetal_hip_gemm_desc &d = descs[i];
+        if (gemv_only_type(d.ggml_type))
+            return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "qgemm_batch: GGML type %u goes through re-blocking (use pmetal_hip_qgemm_reblocked)", d.ggml_type);
+        if (int32_t rc = check_linear(d.ggml_type, d.w_dev, d.n, k, x, x_dtype, d.y_dev, d.order)) return rc;
+        if (d.y_dtype > PMETAL_HIP_DTYPE_BF16) return fail(PMETAL_HIP_ERR_INVALID_ARG, "y_dtype must be 0 (f32) or 1 (bf16)");
+        if (m <= 0 || m > 0x7FFFFFFF) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "m must be in [1, 2^31)");
+        if (k % 256 != 0) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qgemm: k=%lld is not a multiple of 256", (long long)k);
+        if (!pmh::qgemm_fits(d.ggml_type, m, d.n, k))
+            return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qgemm: m and k must be at most 2^22 (m = %lld, k = %lld)", (long long)m, (long long)k);
+        const size_t b = pmh::qgemm_workspace_bytes(m, d.n, k);
+        need = b > need ? b : need;
+    }
+    if (count == 0) return ok();
+    void *ws = nullptr;
+    if (int32_t rc = workspace(need, (hipStream_t)stream, &ws)) return rc;
+    // the converted activations depend on the weight type and element order only through the order they are laid out in
+    auto layout = [](const pmetal_hip_gemm_desc &d) {
+        return d.ggml_type == PMETAL_GGML_TYPE_Q8_0 ? 3 : (d.ggml_type == PMETAL_GGML_TYPE_Q6K ? 2 : (d.order == PMETAL_HIP_ORDER_REF ? 0 : 1));
+    };
+    int have = -1;
+    for (size_t i = 0; i < count; i++) {
+        const pmetal_hip_gemm_desc &d = descs[i];
+        const int want = layout(d);
+        hipError_t e = pmh::launch_qgemm(d.ggml_type, d.w_dev, d.n, k, x, x_dtype, m, d.y_dev, d.y_dtype, d.order, ws, (hipStream_t)stream,
+                                         want == have);
+        if (e == hipErrorNotSupported) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "qgemm: configuration not supported");
+        if (e != hipSuccess) return hip_fail(e, "qgemm kernel launch");
+        have = want;
+    }
+    return ok();
+}
+
 // pmetal_hip_qgemm for callers that cannot allocate: the scratch is the fixed `scratch` array of the current device.
 // Calls no hipMalloc / hipFree and nothing else that allocates.  Every call on a device uses the same array, so calls that
 // overlap on one device race; nothing in it has to start at zero (the pre-pass writes every activation item and row scale

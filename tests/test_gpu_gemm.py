@@ -392,3 +392,32 @@ def test_qlinear_falls_back_to_the_gemm_when_the_gemv_refuses_the_row_length(ora
     assert lib.pmetal_hip_qlinear(Q8_0, w8.ptr, 64, 96, x8.ptr, pm.DTYPE_BF16, 4, y16.ptr, pm.DTYPE_BF16, 0, None) == 6
     assert b"f32 only" in lib.pmetal_hip_last_error_message()
     lib.pmetal_hip_clear_error()
+
+
+def test_qgemm_batch_equals_separate_calls(oracle):
+    """Weights that share their activations: pmetal_hip_qgemm_batch gives the bits of one pmetal_hip_qgemm per weight
+    (mixed types, element orders, output types, with and without a K split)."""
+    lib = _lib.load()
+    k = 2048
+    rng = np.random.default_rng(5150)
+    specs = [(Q4K, 768, 0, pm.DTYPE_F32), (Q4K, 512, 0, pm.DTYPE_BF16), (Q4K, 256, 1, pm.DTYPE_F32), (Q6K, 640, 0, pm.DTYPE_F32),
+             (Q6K, 320, 0, pm.DTYPE_BF16), (Q8_0, 384, 0, pm.DTYPE_F32), (Q4K, 1024, 0, pm.DTYPE_F32)]
+    ws = [pm.DeviceBuffer.from_host(oracle.quantize(t, weights(800 + i, n * k))) for i, (t, n, _, _) in enumerate(specs)]
+    for m in (3, 48, 300):
+        xb = oracle.f32_to_bf16_bits(rng.standard_normal(m * k).astype(np.float32))
+        dx = pm.DeviceBuffer.from_host(xb)
+        sizes = [m * n * (4 if yd == pm.DTYPE_F32 else 2) for (_, n, _, yd) in specs]
+        y_one = [pm.DeviceBuffer(sz) for sz in sizes]
+        y_bat = [pm.DeviceBuffer(sz) for sz in sizes]
+        descs = (_lib.GemmDesc * len(specs))()
+        for i, (t, n, order, yd) in enumerate(specs):
+            pm.check(lib.pmetal_hip_memset(y_bat[i].ptr, 0xFF, sizes[i], None))
+            pm.check(lib.pmetal_hip_qgemm(t, ws[i].ptr, n, k, dx.ptr, pm.DTYPE_BF16, m, y_one[i].ptr, yd, order, None))
+            descs[i] = _lib.GemmDesc(t, yd, order, 0, n, ws[i].ptr, y_bat[i].ptr)
+        pm.check(lib.pmetal_hip_qgemm_batch(descs, len(specs), k, dx.ptr, pm.DTYPE_BF16, m, None))
+        pm.check(lib.pmetal_hip_sync(None))
+        for i in range(len(specs)):
+            assert np.array_equal(y_one[i].to_host(np.uint8), y_bat[i].to_host(np.uint8)), (m, specs[i])
+    bad = (_lib.GemmDesc * 1)(_lib.GemmDesc(13, 0, 0, 0, 256, ws[0].ptr, y_bat[0].ptr))
+    assert lib.pmetal_hip_qgemm_batch(bad, 1, k, dx.ptr, pm.DTYPE_BF16, 3, None) == 2
+    lib.pmetal_hip_clear_error()
