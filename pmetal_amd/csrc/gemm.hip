@@ -927,6 +927,163 @@ __global__ __launch_bounds__(512, 1) void k_qgemm_rw_q8(const uint8_t *__restric
     store_tile<MB>(acc, smem, L.wave, L.col, L.g, m0, n0, M, N, Mp, rowscale, yg, partial, mode, blockIdx.z);
 }
 
+// ------------------------------------------------------------------------------------------------
+// Q4_K with at most 16 activation rows (a decode batch, a speculative window) and rows of at most 16 super-blocks: the
+// weights are read once, at the pace of the GEMV, and nothing but the pre-pass runs before or after this kernel.
+//   * v_mfma_f32_16x16x32_f16: 16 activation rows x 16 weight rows x 32 k.  Lane (r = lane % 16, kg = lane / 16) holds
+//     the eight k of k-group kg for activation row r (first operand) resp. weight row r (second operand); the output
+//     tile has column lane % 16 (weight row) and rows 4 (lane / 16) + 0..3 (activation rows).
+//   * A wave owns one or two super-block columns of W (wave w: super-blocks w and w + 8) and walks the row tiles of its
+//     workgroup.  Its activation operands for those super-blocks -- per super-block eight items (k-step t, k-group kg)
+//     and the item of sub-block sums, exactly the items the pre-pass writes -- are loaded once and stay in registers.
+//   * Per row tile and super-block a lane loads the 16-byte header of its weight row and the 32 quant bytes of
+//     sub-blocks 2 kg and 2 kg + 1 (dword t of them is its operand of k-step t), straight from global memory into
+//     registers, a few row tiles ahead (every load unconditional, so the outstanding loads are counted exactly).
+//     Arithmetic as in the large kernel: exact integer tiles sc * q, d on the fp32 sum of a super-block, the min term as
+//     one more matrix instruction over exact head + tail splits.
+//   * The waves' 16 x 16 partial tiles (one per super-block column) are added through LDS in wave order by the first
+//     wave (one barrier per row tile, no partial tiles in global memory, no reduction kernel; the result does not
+//     depend on scheduling) and collected in LDS; the workgroup stores its columns of y after its last row tile, scaled
+//     by the rows' powers of two.  No store and no other load is issued inside the streaming loop: on this target stores
+//     share the loads' counter, and one of them in flight turns every counted wait into a wait for everything.
+// ------------------------------------------------------------------------------------------------
+typedef float float4_t __attribute__((ext_vector_type(4)));
+constexpr int kSmallWaves = 8;  // waves per workgroup (fewer when a row has fewer super-blocks); 16 waves of one super-block each run alike
+constexpr int kSmallDepth = 2;  // row tiles in flight per wave (four are slower: 16.5 against 12.7 us at 14336 x 4096)
+constexpr int kSmallMaxM = 16, kSmallMaxSpr = 16;
+
+template <int NSB>
+struct SmallTile {
+    uint4 h[NSB], qa[NSB], qb[NSB];
+};
+
+template <int ORDER, int NSB>
+__global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t *__restrict__ W, const uint4 *__restrict__ xs,
+                                                                   const float *__restrict__ rowscale, void *__restrict__ yg, int M,
+                                                                   int Mp, int N, int spr, int tiles, int tiles_per_wg, int ybf16) {
+    __shared__ float4_t red[2][kSmallWaves][64];
+    extern __shared__ float4_t out_tiles[];  // [tiles_per_wg rounded up to whole rounds][64]: lane slots of the finished tiles
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int nwaves = (int)(blockDim.x >> 6);
+    const int nl = lane & 15, kg = lane >> 4;
+    const uint32_t low = kg < 2 ? 0xFFFFFFFFu : 0u;
+    int sbi[NSB];
+    bool sbv[NSB];  // wave-uniform
+#pragma unroll
+    for (int i = 0; i < NSB; i++) {
+        sbi[i] = wave + i * nwaves;
+        sbv[i] = sbi[i] < spr;
+        sbi[i] = sbv[i] ? sbi[i] : 0;
+    }
+    // activation operands of this wave's super-blocks: item (2 sb + kg / 2, group 2 t + kg % 2) of row nl, and the sums item
+    half8_t af[NSB][8], asum[NSB];
+#pragma unroll
+    for (int i = 0; i < NSB; i++) {
+        const uint4 *base = xs + (size_t)((2 * sbi[i] + (kg >> 1)) * kGroups) * Mp + nl;
+#pragma unroll
+        for (int t = 0; t < 8; t++) af[i][t] = __builtin_bit_cast(half8_t, base[(size_t)(2 * t + (kg & 1)) * Mp]);
+        asum[i] = __builtin_bit_cast(half8_t, base[(size_t)(16 + (kg & 1)) * Mp]);
+        if (!sbv[i]) {  // a super-block past the end of the row multiplies zeros (no branch in the streaming loop)
+            const half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int t = 0; t < 8; t++) af[i][t] = z;
+            asum[i] = z;
+        }
+    }
+    const int t0 = (int)blockIdx.x * tiles_per_wg;
+    const int t1 = t0 + tiles_per_wg < tiles ? t0 + tiles_per_wg : tiles;  // t1 > t0 by the launch geometry
+    const uint32_t row_bytes = (uint32_t)spr * (uint32_t)kBlockBytes;
+    auto issue = [&](int ti, SmallTile<NSB> &w) {
+        int tile = t0 + ti;
+        tile = tile < t1 ? tile : t1 - 1;  // past the end: the last tile again (loaded, not used)
+        int n = tile * 16 + nl;
+        n = n < N ? n : N - 1;
+        const uint8_t *row = W + (uint32_t)n * row_bytes;  // the tensor is smaller than 4 GiB (checked by the launcher)
+#pragma unroll
+        for (int i = 0; i < NSB; i++) {
+            const uint8_t *blk = row + (uint32_t)sbi[i] * (uint32_t)kBlockBytes;
+            w.h[i] = *reinterpret_cast<const uint4 *>(blk);
+            w.qa[i] = *reinterpret_cast<const uint4 *>(blk + 16 + 32 * kg);
+            w.qb[i] = *reinterpret_cast<const uint4 *>(blk + 32 + 32 * kg);
+        }
+    };
+    auto consume = [&](int ti, const SmallTile<NSB> &w) {
+        float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int i = 0; i < NSB; i++) {
+            const uint4 hdr = w.h[i];
+            // scales and mins of sub-blocks 2 kg and 2 kg + 1 (6-bit fields, crates/pmetal-gguf/src/quantize.rs:844-855)
+            const uint32_t sh = 16u * (uint32_t)(kg & 1);
+            const uint32_t yv = hdr.y >> sh, zv = hdr.z >> sh, wv = hdr.w >> sh;
+            // sub-blocks 0..3 (kg < 2) and 4..7 store them differently; both forms are computed and one is picked by a
+            // per-lane bit mask (a branch here would be taken by half of every wave)
+            const uint32_t sc0 = ((yv & 63u) & low) | (((wv & 0xFu) | ((yv >> 2) & 0x30u)) & ~low);
+            const uint32_t sc1 = (((yv >> 8) & 63u) & low) | ((((wv >> 8) & 0xFu) | ((yv >> 10) & 0x30u)) & ~low);
+            const uint32_t mn0 = ((zv & 63u) & low) | ((((wv >> 4) & 0xFu) | ((zv >> 2) & 0x30u)) & ~low);
+            const uint32_t mn1 = (((zv >> 8) & 63u) & low) | ((((wv >> 12) & 0xFu) | ((zv >> 10) & 0x30u)) & ~low);
+            const _Float16 s0 = (_Float16)(float)sc0, s1 = (_Float16)(float)sc1;
+            const _Float16 o0 = (_Float16)(-1024.0f * (float)sc0), o1 = (_Float16)(-1024.0f * (float)sc1);  // exact: sc <= 63
+            const half2_t sc2[2] = {half2_t{s0, s0}, half2_t{s1, s1}}, off2[2] = {half2_t{o0, o0}, half2_t{o1, o1}};
+            const uint32_t qd[8] = {w.qa[i].x, w.qa[i].y, w.qa[i].z, w.qa[i].w, w.qb[i].x, w.qb[i].y, w.qb[i].z, w.qb[i].w};
+            float4_t part = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                Dq d;
+#pragma unroll
+                for (int c = 0; c < 4; c++) dq_chunk<ORDER>(c, t, qd[t], sc2, off2, d);
+                part = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i][t], d.value(), part, 0, 0, 0);
+            }
+            // (of a super-block past the end of the row only zeros may enter the sums, whatever bytes were loaded for it)
+            const float dmin = sbv[i] ? f16_bits_to_f32(hdr.x >> 16) : 0.0f, dd = sbv[i] ? f16_bits_to_f32(hdr.x & 0xFFFFu) : 0.0f;
+            _Float16 h0, l0, h1, l1;
+            neg_min_split(dmin, mn0, h0, l0);
+            neg_min_split(dmin, mn1, h1, l1);
+            const half8_t br = {h0, h0, l0, l0, h1, h1, l1, l1};
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(asum[i], br, acc, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[r] = __builtin_fmaf(dd, part[r], acc[r]);
+        }
+        const int buf = ti & 1;
+        red[buf][wave][lane] = acc;
+        __syncthreads();  // the next tile writes the other buffer; the one after that comes behind the next barrier
+        if (wave == 0) {
+            float4_t v = red[buf][0][lane];
+            for (int q = 1; q < nwaves; q++) {
+                const float4_t u = red[buf][q][lane];
+#pragma unroll
+                for (int r = 0; r < 4; r++) v[r] += u[r];
+            }
+            out_tiles[ti * 64 + lane] = v;
+        }
+    };
+    SmallTile<NSB> ring[kSmallDepth];
+#pragma unroll
+    for (int i = 0; i < kSmallDepth; i++) issue(i, ring[i]);
+    // Whole rounds of kSmallDepth tiles, with nothing conditional around the loads, so that the outstanding loads are
+    // counted exactly at every wait; the tiles past the workgroup's last one are computed on repeated data and dropped.
+    const int rounds = (tiles_per_wg + kSmallDepth - 1) / kSmallDepth;
+    for (int rd = 0; rd < rounds; rd++) {
+#pragma unroll
+        for (int i = 0; i < kSmallDepth; i++) {
+            consume(rd * kSmallDepth + i, ring[i]);
+            issue((rd + 1) * kSmallDepth + i, ring[i]);
+        }
+    }
+    __syncthreads();
+    // y[m][16 t0 + j] for j over the workgroup's columns: consecutive threads store consecutive columns of one row
+    const int cols = (t1 - t0) * 16;
+    for (int idx = (int)threadIdx.x; idx < M * cols; idx += (int)blockDim.x) {
+        const int m = idx / cols, j = idx - m * cols;
+        const int n = t0 * 16 + j;
+        if (n < N) {
+            const float o = out_tiles[(j >> 4) * 64 + (m >> 2) * 16 + (j & 15)][m & 3] * rowscale[m];
+            if (ybf16) reinterpret_cast<uint16_t *>(yg)[(size_t)m * N + n] = (uint16_t)bf16_rne_bits(o);
+            else reinterpret_cast<float *>(yg)[(size_t)m * N + n] = o;
+        }
+    }
+}
+
 // y[m][n] = rowscale[m] * (partial[0][m][n] + partial[1][m][n] + ...), added in this order
 template <bool YBF16>
 __global__ __launch_bounds__(256) void k_rw_reduce(const float *__restrict__ partial, int splits, int M, int Mp, int N,
@@ -958,6 +1115,21 @@ constexpr size_t rw_lds_bytes() {
 namespace pmh {
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+// The fused kernel for few activation rows takes Q4_K with m <= 16 and rows of at most 16 super-blocks (k <= 4096).
+static bool qgemm_small_applies(uint32_t type, int64_t m, int64_t n, int64_t k) {
+    return type == kTypeQ4K && m <= kSmallMaxM && k / 256 <= kSmallMaxSpr && (uint64_t)n * (uint64_t)(k / 256) * 144u < (1ull << 32);
+}
+
+static int compute_units_gemm() {
+    static const int n = [] {
+        int dev = 0, cu = 0;
+        if (hipGetDevice(&dev) != hipSuccess) return 256;
+        if (hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cu <= 0) return 256;
+        return cu;
+    }();
+    return n;
+}
 
 bool qgemm_fits(uint32_t type, int64_t m, int64_t n, int64_t k) {
     // byte offsets inside a workgroup's rows and item offsets inside the activation copy are 32-bit
@@ -1080,6 +1252,36 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     const bool ybf = y_dtype == kDtypeBf16;
+    if (qgemm_small_applies(type, m, n, k)) {
+        const int nwaves = spr < kSmallWaves ? spr : kSmallWaves;
+        const int tiles = (int)((n + 15) / 16);
+        const int64_t slots = (int64_t)compute_units_gemm() * (kSmallWaves / nwaves);
+        const int n_wg = (int)(tiles < slots ? tiles : slots);
+        int tiles_per_wg = (tiles + n_wg - 1) / n_wg;
+        tiles_per_wg = tiles_per_wg < 96 ? tiles_per_wg : 96;  // the finished tiles wait in LDS: 1 KiB each
+        const dim3 grid((unsigned)((tiles + tiles_per_wg - 1) / tiles_per_wg)), block((unsigned)(64 * nwaves));
+        const size_t lds = (size_t)((tiles_per_wg + kSmallDepth - 1) / kSmallDepth * kSmallDepth) * 1024;
+#define PMH_SMALL(O, S)                                                                                                          \
+    do {                                                                                                                         \
+        if (lds > 48 * 1024) {                                                                                                   \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_qgemm_small<O, S>), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                    (int)lds);                                                                                   \
+            if (e != hipSuccess) return e;                                                                                       \
+        }                                                                                                                        \
+        hipLaunchKernelGGL((k_qgemm_small<O, S>), grid, block, lds, s, w, xs, rowscale, y, (int)m, (int)p.mp, (int)n, spr, tiles, \
+                           tiles_per_wg, ybf ? 1 : 0);                                                                           \
+    } while (0)
+        if (spr > kSmallWaves) {
+            static_assert(2 * kSmallWaves >= kSmallMaxSpr, "two super-blocks per wave must cover the longest row");
+            if (ref) PMH_SMALL(0, 2);
+            else PMH_SMALL(1, 2);
+        } else {
+            if (ref) PMH_SMALL(0, 1);
+            else PMH_SMALL(1, 1);
+        }
+#undef PMH_SMALL
+        return hipGetLastError();
+    }
     const int mode = p.splits > 1 ? 2 : (ybf ? 1 : 0);
 #define PMH_RW_CASE(O, B, R, NWV) launch_rw<O, B, R, NWV>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
     if (q8) {
