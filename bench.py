@@ -34,9 +34,13 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 # HBM bytes per launch as recorded from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled against a streaming kernel
 # of known size; constants taken from the profile summaries named here, not measured by this script
-RECORDED_TRAFFIC = {"gemv_q4k_14336x4096": (33293144, "profiles/qgemv_q4k_14336x4096.md"),
-                    "gemv_q6k_14336x4096": (48531385, "profiles/qgemv_q6k_q8_0_14336x4096.md"),
-                    "gemv_q8_0_14336x4096": (62642111, "profiles/qgemv_q6k_q8_0_14336x4096.md")}
+RECORDED_TRAFFIC = {"gemv_q4k_14336x4096": (33294684, "profiles/qgemv_q4k_14336x4096.md"),
+                    "gemv_q4k_4096x14336": (33416379, "profiles/qgemv_q4k_4096x14336.md"),
+                    "gemv_q6k_14336x4096": (48547409, "profiles/qgemv_other_types.md"),
+                    "gemv_q8_0_14336x4096": (62645025, "profiles/qgemv_other_types.md"),
+                    "gemv_q5k_6144x4096": (17531108, "profiles/qgemv_other_types.md"),
+                    "gemv_q3k_14336x4096": (25572926, "profiles/qgemv_other_types.md"),
+                    "gemv_q2k_14336x4096": (19567272, "profiles/qgemv_other_types.md")}
 BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16/fp16 MFMA, published
 Q8_0, Q4K, Q6K = 8, 12, 14
 
@@ -404,9 +408,20 @@ def bench_gemm(args, m, n, k, t=Q4K):
     x = pm.DeviceBuffer.from_host(bf16_bits(np.random.default_rng(2).standard_normal(m * k)))
     y = pm.DeviceBuffer(2 * m * n)
 
-    def step():
+    def per_call():
         pm.check(lib.pmetal_hip_qgemm(t, w.ptr, n, k, x.ptr, pm.DTYPE_BF16, m, y.ptr, pm.DTYPE_BF16, 0, None))
 
+    step, per_call_us = per_call, None
+    rb_bytes = lib.pmetal_hip_reblock_size(t, n, k)
+    if rb_bytes:  # Q5_K / Q3_K / Q2_K: re-blocked once, as a loader does; the per-call form is timed beside it
+        rb = pm.DeviceBuffer(rb_bytes)
+        pm.check(lib.pmetal_hip_reblock_dev(t, w.ptr, n, k, 0, rb.ptr, rb_bytes, None), "reblock")
+
+        def step():
+            pm.check(lib.pmetal_hip_qgemm_reblocked(t, rb.ptr, rb_bytes, n, k, x.ptr, pm.DTYPE_BF16, m, y.ptr, pm.DTYPE_BF16, None))
+
+        pc_ms, _ = timer.run(per_call, args.steps, args.warmup)
+        per_call_us = pc_ms * 1e3 / args.steps
     ev_ms, wall_ms = timer.run(step, args.steps, args.warmup)
     # what the matrix cores of this machine sustain in a register-only MFMA loop (no memory, no LDS) of about the
     # same length, with operands that vary: the ceiling any kernel here works under (the published peak assumes
@@ -429,11 +444,14 @@ def bench_gemm(args, m, n, k, t=Q4K):
         "value": tflops, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / BF16_PEAK_TFLOPS, 4), "traffic": None,
-                     "kernel": {Q4K: "k_qgemm_rw", Q6K: "k_qgemm_rw_q6", Q8_0: "k_qgemm_rw_q8"}.get(t, "k_reblock_q6k + k_qgemm_rw_q6 per part") + " (+ k_prep_rw, k_rw_reduce when K is split)",
+                     "kernel": {Q4K: "k_qgemm_rw", Q6K: "k_qgemm_rw_q6", Q8_0: "k_qgemm_rw_q8"}.get(t, "k_qgemm_rw_q6 per Q6_K part of the re-blocked weight") + " (+ k_prep_rw, k_rw_reduce when K is split)",
                      "flops_per_launch": flops, "us_per_launch": round(us, 3)},
         "extra": {"mfma_loop_sustained_TFLOPs": round(sustained, 1), "frac_of_sustained": round(tflops / sustained, 4),
                   "two_weights_sharing_x_us_per_weight": None if pair_us is None else round(pair_us, 3),
-                  "two_weights_sharing_x_TFLOPs": None if pair_us is None else round(flops / (pair_us * 1e-6) / 1e12, 1)},
+                  "two_weights_sharing_x_TFLOPs": None if pair_us is None else round(flops / (pair_us * 1e-6) / 1e12, 1),
+                  **({} if per_call_us is None else {"weight": "re-blocked to Q6_K once (pmetal_hip_reblock_dev), then pmetal_hip_qgemm_reblocked per call",
+                                                    "reblocked_bytes": rb_bytes,
+                                                    "reblocking_on_every_call_us": round(per_call_us, 3)})},
     }, (t, n, k)
 
 
