@@ -599,7 +599,15 @@ hipError_t launch_group_general(const uint8_t *const *w, const int64_t *n, float
     for (int i = 0; i < count; i++) total += n[i];
     const int64_t want = compute_units();
     int64_t n_wg = total < want ? total : want;
-    const int64_t rows_per_wg = (total + n_wg - 1) / n_wg;
+    int64_t rows_per_wg = (total + n_wg - 1) / n_wg;
+    // every member rounds its workgroup count up: keep the sum within one workgroup per compute unit (a 257th workgroup
+    // would run alone behind the others and nearly double the launch)
+    for (;;) {
+        int64_t c = 0;
+        for (int i = 0; i < count; i++) c += (n[i] + rows_per_wg - 1) / rows_per_wg;
+        if (c <= want || rows_per_wg >= total) break;
+        rows_per_wg++;
+    }
     GemvGroup grp{};
     int begin = 0;
     for (int i = 0; i < pmh::kMaxGemvGroup; i++) {
