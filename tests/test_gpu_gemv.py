@@ -47,10 +47,13 @@ def test_qgemv_matches_dequantize_then_matmul(oracle, t, n, k, x_dtype):
         assert elem <= TOL and norm <= TOL
 
 
-# Shapes of 12 MiB and more take the chunk-owner kernel: ragged row counts (the last workgroup, wave and task are
-# short), 32-lane teams (k / 256 = 12), a row count below the number of compute units times the waves, and a
-# row of 16 chunks (k = 32768).
-BIG_CASES = [(6001, 4096), (7301, 3072), (3001, 8192), (16385, 1536), (800, 32768)]
+# Shapes of 12 MiB and more take the large-matrix kernels.  Rows of one or two chunks (k = 2048, 4096) with at most
+# eight tasks per wave go to the kernel whose waves own whole rows (6001 x 4096, 12001 x 2048, 32767 x 2048: ragged row
+# counts, so the last workgroup and its waves are short); more rows than that (20000 x 4096, 40001 x 2048) and every
+# other row length go to the chunk-owner kernel: 32-lane teams (k / 256 = 12), a row count below the number of compute
+# units times the waves, and a row of 16 chunks (k = 32768).
+BIG_CASES = [(6001, 4096), (7301, 3072), (3001, 8192), (16385, 1536), (800, 32768), (12001, 2048), (32767, 2048),
+             (20000, 4096), (40001, 2048)]
 
 
 @pytest.mark.parametrize("n,k", BIG_CASES)
