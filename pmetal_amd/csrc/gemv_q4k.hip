@@ -820,13 +820,15 @@ hipError_t launch_qgemv_q4k(const uint8_t *w, int64_t n, int64_t k, const void *
     const size_t slots = (size_t)spr * 8;
     const size_t lds_x = slots * 16 * (xf32 ? 6 : 5) + slots * 16;
     if (lds_x > gemv::kMaxLds) return hipErrorInvalidValue;
-    // Kernel A when there is enough work per compute unit to pay for its second barrier (measured crossover: about
-    // 12 MiB of weights) and the shape suits it.
     const uint64_t w_bytes = (uint64_t)n * (uint64_t)spr * 144u;
-    if (w_bytes >= (12ull << 20)) {
-        hipError_t e = launch_kernel_rows(w, n, y, nullptr, 0, nullptr, k, x, xf32, order, s);
+    // Measured crossovers against kernel B: the row-owner kernel from about 8 MiB (4096 x 4096: 4.21 against 4.28 us,
+    // 5120 x 4096: 4.5 against 5.4; 2048 x 4096: 3.7 against 3.5), kernel A from about 12 MiB.
+    if (w_bytes >= (8ull << 20)) {
+        const hipError_t e = launch_kernel_rows(w, n, y, nullptr, 0, nullptr, k, x, xf32, order, s);
         if (e != hipErrorNotSupported) return e;
-        e = launch_kernel_a(w, n, y, nullptr, 0, nullptr, k, x, xf32, order, s);
+    }
+    if (w_bytes >= (12ull << 20)) {
+        const hipError_t e = launch_kernel_a(w, n, y, nullptr, 0, nullptr, k, x, xf32, order, s);
         if (e != hipErrorNotSupported) return e;
     }
     return launch_group_general(&w, &n, &y, 1, k, x, xf32, order, s);
