@@ -287,7 +287,7 @@ def bench_gemv(args, n, k, t=Q4K, copies=16, passes=8):
         "value": gbs, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": {Q4K: "k_qgemv_q4k_chunk", Q6K: "k_qgemv_q6k_chunk", Q8_0: "k_qgemv_q8_0_chunk", 13: "k_qgemv_q5k_chunk", 11: "k_qgemv_q23k_chunk<FormatQ3K>", 10: "k_qgemv_q23k_chunk<FormatQ2K>"}[t], "bytes_per_launch": bytes_per_launch,
+                     "kernel": {Q4K: "k_qgemv_q4k_rows" if k in (2048, 4096) else "k_qgemv_q4k_chunk", Q6K: "k_qgemv_q6k_chunk", Q8_0: "k_qgemv_q8_0_chunk", 13: "k_qgemv_q5k_chunk", 11: "k_qgemv_q23k_chunk<FormatQ3K>", 10: "k_qgemv_q23k_chunk<FormatQ2K>"}[t], "bytes_per_launch": bytes_per_launch,
                      "us_per_launch": round(us_per_launch, 3)},
         "extra": {"cache_resident_GBps": round(cached_gbs, 1), "cache_resident_us_per_launch": round(c_ms * 1e3 / launches, 3),
                   "weight_copies": copies, "launches_per_step": copies * passes,

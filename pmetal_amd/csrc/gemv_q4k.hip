@@ -754,8 +754,8 @@ static hipError_t launch_kernel_rows(const uint8_t *w0, int64_t n0, float *y0, c
     const int ks = spr / 8;
     const uint64_t w_max = (uint64_t)(n0 > n1 ? n0 : n1) * (uint64_t)spr * 144u;
     if (w_max >= (1ull << 32)) return hipErrorNotSupported;
-    // two workgroups per compute unit
-    const int64_t n = n0 + n1, want = 2 * (int64_t)gemv::compute_units();
+    // two workgroups per compute unit and matrix
+    const int64_t n = n0 + n1, want = (n1 > 0 ? 4 : 2) * (int64_t)gemv::compute_units();
     const int64_t n_wg = n < want ? n : want;
     const int64_t rows_per_wg = (n + n_wg - 1) / n_wg;
     if (((rows_per_wg + kRowsWaves - 1) / kRowsWaves) * ks > kDepth) return hipErrorNotSupported;
