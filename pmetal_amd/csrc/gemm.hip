@@ -972,7 +972,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t 
     bool sbv[NSB];  // wave-uniform
 #pragma unroll
     for (int i = 0; i < NSB; i++) {
-        sbi[i] = wave + i * nwaves;
+        sbi[i] = NSB * wave + i;  // adjacent super-blocks: one contiguous piece of every row per wave
         sbv[i] = sbi[i] < spr;
         sbi[i] = sbv[i] ? sbi[i] : 0;
     }
