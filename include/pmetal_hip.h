@@ -243,12 +243,13 @@ int32_t pmetal_hip_qgemv_batch(const pmetal_hip_linear_desc *descs, size_t count
  * quantize_q8k (crates/pmetal-gguf/src/k_quants.rs:815-871) into BlockQ8K (k_quants.rs:140-155:
  * f32 d, i8 qs[256], i16 bsums[16]; 292 bytes per 256 elements, a trailing partial block all-zero),
  * bytes bit-identical to the reference; dst_len must be pmetal_hip_q8k_size(n).
- * qgemv_q8k: y[r] = vec_dot_q4k_q8k / vec_dot_q6k_q8k (row r of W, xq) as the reference's scalar
- * definitions compute them (crates/pmetal-gguf/src/vec_dot.rs:617-656, :658-692), bit for bit:
- * exact integer sums per super-block, the float sum over the super-blocks in their order.
- * ggml_type Q4K or Q6K; k a multiple of 256, at most 32768; xq_dev holds k / 256 blocks.  For
- * Q4_K the pairing of nibbles and activations is the quantizer's own (GGML) order; for Q6_K it
- * is the linear order of that dot product, which is not the order dequantize_q6k uses.      */
+ * qgemv_q8k: y[r] = vec_dot_q4k_q8k / _q6k_ / _q5k_ / _q3k_ / _q2k_q8k (row r of W, xq) as the reference's scalar
+ * definitions compute them (crates/pmetal-gguf/src/vec_dot.rs:617-656, :658-692, :695-737, :739-777, :779-810), bit for
+ * bit: exact integer sums per super-block, the float sum over the super-blocks in their order.
+ * ggml_type Q4K, Q6K, Q5K, Q3K or Q2K; k a multiple of 256, at most 32768; xq_dev holds k / 256 blocks.  For
+ * Q4_K the pairing of nibbles and activations is the quantizer's own (GGML) order; for the other types it is the order
+ * linear in the element index that each of those dot products uses, which is not the order the dequantizer of the type
+ * uses (and vec_dot_q3k_q8k gives the second half of every super-block a zero scale: reproduced as it is).      */
 size_t pmetal_hip_q8k_size(size_t n_elements);
 int32_t pmetal_hip_quantize_q8k_dev(const float *src_dev, size_t n, uint8_t *dst_dev, size_t dst_len, void *stream);
 int32_t pmetal_hip_qgemv_q8k(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, int64_t k, const uint8_t *xq_dev,

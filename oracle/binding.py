@@ -84,7 +84,7 @@ def lib() -> C.CDLL:
         L.pmo_kl_divergence.argtypes, L.pmo_kl_divergence.restype = [f32p, f32p, C.c_size_t], C.c_double
         L.pmo_q8k_size.argtypes, L.pmo_q8k_size.restype = [C.c_size_t], C.c_size_t
         L.pmo_quantize_q8k.argtypes, L.pmo_quantize_q8k.restype = [f32p, C.c_size_t, u8p], None
-        for name in ("pmo_vec_dot_q4k_q8k", "pmo_vec_dot_q6k_q8k"):
+        for name in ("pmo_vec_dot_q4k_q8k", "pmo_vec_dot_q6k_q8k", "pmo_vec_dot_q5k_q8k", "pmo_vec_dot_q3k_q8k", "pmo_vec_dot_q2k_q8k"):
             getattr(L, name).argtypes, getattr(L, name).restype = [u8p, u8p, C.c_size_t], C.c_float
         L.pmo_qmatvec_q8k.argtypes = [C.c_uint32, u8p, C.c_size_t, C.c_size_t, u8p, f32p]
         L.pmo_qmatvec_q8k.restype = C.c_int32
@@ -218,11 +218,12 @@ def quantize_q8k(x: np.ndarray) -> np.ndarray:
 
 
 def vec_dot_q8k(t: int, xs: np.ndarray, ys: np.ndarray, n_blocks: int) -> float:
-    """vec_dot.rs:617-692 (scalar): one row of Q4_K / Q6_K blocks against Q8_K blocks."""
+    """vec_dot.rs:617-810 (scalar): one row of Q4_K / Q6_K / Q5_K / Q3_K / Q2_K blocks against Q8_K blocks."""
     xs = np.ascontiguousarray(xs, dtype=np.uint8).reshape(-1)
     ys = np.ascontiguousarray(ys, dtype=np.uint8).reshape(-1)
     assert xs.size == n_blocks * tensor_size(t, 256) and ys.size == n_blocks * 292
-    fn = lib().pmo_vec_dot_q4k_q8k if t == TYPE_Q4K else lib().pmo_vec_dot_q6k_q8k
+    fn = {TYPE_Q4K: lib().pmo_vec_dot_q4k_q8k, TYPE_Q6K: lib().pmo_vec_dot_q6k_q8k, TYPE_Q5K: lib().pmo_vec_dot_q5k_q8k,
+          TYPE_Q3K: lib().pmo_vec_dot_q3k_q8k, TYPE_Q2K: lib().pmo_vec_dot_q2k_q8k}[t]
     return float(fn(_u8p(xs), _u8p(ys), n_blocks))
 
 

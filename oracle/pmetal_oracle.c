@@ -1101,12 +1101,115 @@ float pmo_vec_dot_q6k_q8k(const uint8_t *xs, const uint8_t *ys, size_t n_blocks)
     return sum;
 }
 
+/* vec_dot.rs:695-737 (scalar): element j of a super-block takes the low (j even) or high nibble of qs[j / 2], bit j % 8 of
+ * qh[j / 8] and the scale of sub-block j / 32; the min term as for Q4_K. */
+float pmo_vec_dot_q5k_q8k(const uint8_t *xs, const uint8_t *ys, size_t n_blocks) {
+    float sum = 0.0f;
+    for (size_t b = 0; b < n_blocks; b++) {
+        const uint8_t *x = xs + b * 176, *y = ys + b * 292;
+        const uint8_t *scales = x + 4, *qh = x + 16, *qs = x + 48;
+        const int8_t *q8 = (const int8_t *)(y + 4);
+        uint16_t d16, m16;
+        float yd;
+        memcpy(&d16, x, 2);
+        memcpy(&m16, x + 2, 2);
+        memcpy(&yd, y, 4);
+        float d = pmo_f16_to_f32(d16) * yd, dmin = pmo_f16_to_f32(m16) * yd; /* :699-700 */
+        int32_t mins_sum = 0;
+        for (int j = 0; j < 8; j++) { /* :703-708 */
+            uint8_t sc, m;
+            int16_t b0, b1;
+            pmo_get_scale_min_k4(j, scales, &sc, &m);
+            memcpy(&b0, y + 260 + 4 * j, 2);
+            memcpy(&b1, y + 262 + 4 * j, 2);
+            mins_sum += (int32_t)m * ((int32_t)b0 + (int32_t)b1);
+        }
+        sum -= dmin * (float)mins_sum; /* :709 */
+        int32_t sumi = 0;
+        for (int j = 0; j < 256; j++) { /* :712-731 */
+            uint8_t ql = (j % 2 == 0) ? (uint8_t)(qs[j / 2] & 0x0F) : (uint8_t)(qs[j / 2] >> 4);
+            uint8_t hi = (uint8_t)(((qh[j / 8] >> (j % 8)) & 0x01) << 4);
+            int32_t q5 = (int32_t)(ql | hi);
+            uint8_t sc, m;
+            pmo_get_scale_min_k4(j / 32, scales, &sc, &m);
+            sumi += q5 * (int32_t)q8[j] * (int32_t)sc;
+        }
+        sum += d * (float)sumi; /* :733 */
+    }
+    return sum;
+}
+
+/* vec_dot.rs:739-777 (scalar): only the first eight scales are unpacked (the low nibbles of scales[0..4], minus 8); the
+ * scales of sub-blocks 8..15 stay zero, so the second half of every super-block contributes nothing.  Element j takes
+ * bits 2 (j % 4) .. of qs[j / 4] and bit j % 8 of hmask[j / 8] as its third bit, minus 4. */
+float pmo_vec_dot_q3k_q8k(const uint8_t *xs, const uint8_t *ys, size_t n_blocks) {
+    float sum = 0.0f;
+    for (size_t b = 0; b < n_blocks; b++) {
+        const uint8_t *x = xs + b * 110, *y = ys + b * 292;
+        const uint8_t *hmask = x, *qs = x + 32, *sc12 = x + 96;
+        const int8_t *q8 = (const int8_t *)(y + 4);
+        uint16_t d16;
+        float yd;
+        memcpy(&d16, x + 108, 2);
+        memcpy(&yd, y, 4);
+        float d = pmo_f16_to_f32(d16) * yd; /* :743 */
+        int32_t scales[16] = {0};
+        int32_t aux0 = (int32_t)((uint32_t)sc12[0] | ((uint32_t)sc12[1] << 8) | ((uint32_t)sc12[2] << 16) | ((uint32_t)sc12[3] << 24));
+        for (int i = 0; i < 8; i++) scales[i] = (int32_t)(int8_t)((aux0 >> (4 * i)) & 0xF) - 8; /* :747-755 */
+        int32_t sumi = 0;
+        for (int j = 0; j < 256; j++) { /* :757-771 */
+            uint8_t ql = (uint8_t)((qs[j / 4] >> ((j % 4) * 2)) & 0x03);
+            uint8_t hi = (uint8_t)(((hmask[j / 8] >> (j % 8)) & 0x01) << 2);
+            int32_t q3 = (int32_t)(ql | hi) - 4;
+            sumi += q3 * (int32_t)q8[j] * scales[j / 16];
+        }
+        sum += d * (float)sumi; /* :773 */
+    }
+    return sum;
+}
+
+/* vec_dot.rs:779-810 (scalar): element j takes bits 2 (j % 4) .. of qs[j / 4] and the low nibble of scales[j / 16]; the
+ * min term is the high nibble of scales[j] times bsums[j]. */
+float pmo_vec_dot_q2k_q8k(const uint8_t *xs, const uint8_t *ys, size_t n_blocks) {
+    float sum = 0.0f;
+    for (size_t b = 0; b < n_blocks; b++) {
+        const uint8_t *x = xs + b * 84, *y = ys + b * 292;
+        const uint8_t *scales = x, *qs = x + 16;
+        const int8_t *q8 = (const int8_t *)(y + 4);
+        uint16_t d16, m16;
+        float yd;
+        memcpy(&d16, x + 80, 2);
+        memcpy(&m16, x + 82, 2);
+        memcpy(&yd, y, 4);
+        float d = pmo_f16_to_f32(d16) * yd, dmin = pmo_f16_to_f32(m16) * yd; /* :783-784 */
+        int32_t mins_sum = 0;
+        for (int j = 0; j < 16; j++) { /* :787-792 */
+            int16_t bs;
+            memcpy(&bs, y + 260 + 2 * j, 2);
+            mins_sum += (int32_t)(scales[j] >> 4) * (int32_t)bs;
+        }
+        sum -= dmin * (float)mins_sum; /* :793 */
+        int32_t sumi = 0;
+        for (int j = 0; j < 256; j++) { /* :796-803 */
+            int32_t q2 = (int32_t)((qs[j / 4] >> ((j % 4) * 2)) & 0x03);
+            sumi += q2 * (int32_t)q8[j] * (int32_t)(scales[j / 16] & 0x0F);
+        }
+        sum += d * (float)sumi; /* :805 */
+    }
+    return sum;
+}
+
 int32_t pmo_qmatvec_q8k(uint32_t t, const uint8_t *w, size_t n_rows, size_t k, const uint8_t *xq, float *y) {
-    if (t != PMO_TYPE_Q4K && t != PMO_TYPE_Q6K) return PMO_ERR_UNSUPPORTED_TYPE;
+    float (*dot)(const uint8_t *, const uint8_t *, size_t) = t == PMO_TYPE_Q4K   ? pmo_vec_dot_q4k_q8k
+                                                             : t == PMO_TYPE_Q6K ? pmo_vec_dot_q6k_q8k
+                                                             : t == PMO_TYPE_Q5K ? pmo_vec_dot_q5k_q8k
+                                                             : t == PMO_TYPE_Q3K ? pmo_vec_dot_q3k_q8k
+                                                             : t == PMO_TYPE_Q2K ? pmo_vec_dot_q2k_q8k
+                                                                                 : NULL;
+    if (!dot) return PMO_ERR_UNSUPPORTED_TYPE;
     if (k % 256 != 0) return PMO_ERR_INVALID_SHAPE;
     size_t spr = k / 256, row = spr * pmo_type_size(t);
-    for (size_t r = 0; r < n_rows; r++)
-        y[r] = t == PMO_TYPE_Q4K ? pmo_vec_dot_q4k_q8k(w + r * row, xq, spr) : pmo_vec_dot_q6k_q8k(w + r * row, xq, spr);
+    for (size_t r = 0; r < n_rows; r++) y[r] = dot(w + r * row, xq, spr);
     return PMO_OK;
 }
 

@@ -127,7 +127,7 @@ uint32_t pmo_q4km_tensor_type(const char *gguf_name, size_t ndim, size_t n_layer
 /* Q8_K activation blocks and the integer dot products over them.
  * k_quants.rs:140-155 BlockQ8K {f32 d; i8 qs[256]; i16 bsums[16]} = 292 bytes; :815-871 quantize_q8k (a trailing
  * partial block stays all-zero); vec_dot.rs:617-656 scalar vec_dot_q4k_q8k, :658-692 scalar vec_dot_q6k_q8k.
- * pmo_qmatvec_q8k: y[r] = vec_dot(row r of W, xq) for W of type Q4K or Q6K, k a multiple of 256. */
+ * pmo_qmatvec_q8k: y[r] = vec_dot(row r of W, xq) for W of type Q4K, Q6K, Q5K, Q3K or Q2K, k a multiple of 256. */
 size_t pmo_q8k_size(size_t n_elements);
 /* k_quants.rs:498-506 + :562-610 */
 void pmo_dequantize_q8k(const uint8_t *src, size_t n, float *dst);
@@ -136,6 +136,12 @@ double pmo_kl_divergence(const float *original, const float *dequantized, size_t
 void pmo_quantize_q8k(const float *x, size_t n, uint8_t *dst);
 float pmo_vec_dot_q4k_q8k(const uint8_t *xs, const uint8_t *ys, size_t n_blocks);
 float pmo_vec_dot_q6k_q8k(const uint8_t *xs, const uint8_t *ys, size_t n_blocks);
+/* vec_dot.rs:695-737, :739-777, :779-810: the scalar dot products of the other k-quants, each in the element order that
+ * routine itself uses (linear in the element index; not the order the dequantizers of these types use).  Pinned by
+ * tests/test_q8k.py: sums derived by hand, single-position blocks against the index arithmetic above. */
+float pmo_vec_dot_q5k_q8k(const uint8_t *xs, const uint8_t *ys, size_t n_blocks);
+float pmo_vec_dot_q3k_q8k(const uint8_t *xs, const uint8_t *ys, size_t n_blocks);
+float pmo_vec_dot_q2k_q8k(const uint8_t *xs, const uint8_t *ys, size_t n_blocks);
 int32_t pmo_qmatvec_q8k(uint32_t ggml_type, const uint8_t *w, size_t n_rows, size_t k, const uint8_t *xq, float *y);
 
 /* Not a reference function: "reference dequantize, then matmul", the definition

@@ -916,7 +916,8 @@ int32_t pmetal_hip_quantize_q8k_dev(const float *src, size_t n, uint8_t *dst, si
 }
 
 int32_t pmetal_hip_qgemv_q8k(uint32_t t, const uint8_t *w, int64_t n, int64_t k, const uint8_t *xq, float *y, void *stream) {
-    if (t != PMETAL_GGML_TYPE_Q4K && t != PMETAL_GGML_TYPE_Q6K)
+    if (t != PMETAL_GGML_TYPE_Q4K && t != PMETAL_GGML_TYPE_Q6K && t != PMETAL_GGML_TYPE_Q5K && t != PMETAL_GGML_TYPE_Q3K &&
+        t != PMETAL_GGML_TYPE_Q2K)
         return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "qgemv_q8k: GGML type %u has no Q8_K dot product here", t);
     if (n < 0 || k < 0 || n > 0x7FFFFFFF) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "n and k must be non-negative, n below 2^31");
     if (k % 256 != 0) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qgemv_q8k: k=%lld is not a multiple of 256", (long long)k);

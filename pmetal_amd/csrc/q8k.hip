@@ -247,6 +247,99 @@ __device__ __forceinline__ int dot_q6(const TaskQ6 &t, const XqLds &xq, int sb, 
     return scale * (s - 32 * (int)xq.bsum[sb * 16 + g]);
 }
 
+// Byte e of the result = bits 2 e, 2 e + 1 of the byte h: fields 0 and 2 move by 0 and 12 bits, fields 1 and 3 by 6 and 18
+// (the two copies of each product do not overlap, so the multiplications are plain shifts and ors).
+__device__ __forceinline__ uint32_t spread_fields2(uint32_t h) {
+    return (((h & 0x33u) * 0x1001u) & 0x00030003u) | (((h & 0xCCu) * 0x40040u) & 0x03000300u);
+}
+// Byte e of the result = bit e of the nibble b (bit e moves by 7 e; the stray copies fall outside the mask).
+__device__ __forceinline__ uint32_t spread_bits4(uint32_t b) { return (b * 0x00204081u) & 0x01010101u; }
+// Byte e of the result = nibble e of the 16-bit value x.
+__device__ __forceinline__ uint32_t spread_nibbles4(uint32_t x) {
+    x = (x | (x << 8)) & 0x00FF00FFu;
+    return (x | (x << 4)) & 0x0F0F0F0Fu;
+}
+
+// Q5_K in the element order of the reference's dot product (crates/pmetal-gguf/src/vec_dot.rs:695-737): element j takes
+// the low (j even) or high nibble of qs[j / 2], bit j % 8 of qh[j / 8] and the scale of sub-block j / 32.  8 lanes per
+// super-block, lane j holds sub-block j: qs bytes 16 j .. 16 j + 15, qh bytes 4 j .. 4 j + 3; it also takes the min term
+// of sub-block j.
+struct TaskQ5 {
+    uint4 hdr, q;
+    uint32_t qh;
+};
+__device__ __forceinline__ void load_q5(const uint8_t *__restrict__ row, int sb, int j, bool live, TaskQ5 &t) {
+    const uint8_t *blk = row + (size_t)(live ? sb : 0) * 176;
+    t.hdr = *reinterpret_cast<const uint4 *>(blk);
+    t.qh = *reinterpret_cast<const uint32_t *>(blk + 16 + 4 * j);
+    t.q = *reinterpret_cast<const uint4 *>(blk + 48 + 16 * j);
+}
+__device__ __forceinline__ void dot_q5(const TaskQ5 &t, const XqLds &xq, int sb, int j, int &sumi, int &mins) {
+    const uint4 ya = xq.qs[sb * 16 + 2 * j], yb = xq.qs[sb * 16 + 2 * j + 1];
+    const uint32_t y[8] = {ya.x, ya.y, ya.z, ya.w, yb.x, yb.y, yb.z, yb.w};
+    const uint32_t w[4] = {t.q.x, t.q.y, t.q.z, t.q.w};
+    int s = 0;
+#pragma unroll
+    for (int m = 0; m < 8; m++) {  // elements 4 m .. 4 m + 3 of the sub-block: qs bytes 2 m, 2 m + 1, bits 4 m .. of qh
+        const uint32_t nib = spread_nibbles4((w[m >> 1] >> (16 * (m & 1))) & 0xFFFFu);
+        const uint32_t top = spread_bits4((t.qh >> (4 * m)) & 0xFu) << 4;
+        s = dot4(nib | top, y[m], s);
+    }
+    uint32_t scj, mj;
+    scale_min_k4(j, t.hdr.y, t.hdr.z, t.hdr.w, scj, mj);
+    const uint32_t bs = reinterpret_cast<const uint32_t *>(xq.bsum)[sb * 8 + j];  // bsums 2 j and 2 j + 1
+    sumi = (int)scj * s;
+    mins = (int)mj * ((int)(int16_t)(bs & 0xFFFFu) + (int)(int16_t)(bs >> 16));
+}
+
+// Q2_K (crates/pmetal-gguf/src/vec_dot.rs:779-810): element j takes bits 2 (j % 4) .. of qs[j / 4] and the low nibble of
+// scales[j / 16]; the min term is the high nibble of scales[g] times bsums[g].  16 lanes per super-block, lane g holds
+// the 16 elements of group g: qs bytes 4 g .. 4 g + 3.  Blocks are 84 bytes: dwords stay aligned.
+struct TaskQ2 {
+    uint32_t q, sc, hdr;  // sc: scales[g]; hdr: d | dmin << 16
+};
+__device__ __forceinline__ void load_q2(const uint8_t *__restrict__ row, int sb, int g, bool live, TaskQ2 &t) {
+    const uint8_t *blk = row + (size_t)(live ? sb : 0) * 84;
+    t.sc = blk[g];
+    t.q = *reinterpret_cast<const uint32_t *>(blk + 16 + 4 * g);
+    t.hdr = *reinterpret_cast<const uint32_t *>(blk + 80);
+}
+__device__ __forceinline__ void dot_q2(const TaskQ2 &t, const XqLds &xq, int sb, int g, int &sumi, int &mins) {
+    const uint4 q8 = xq.qs[sb * 16 + g];
+    const uint32_t y[4] = {q8.x, q8.y, q8.z, q8.w};
+    int s = 0;
+#pragma unroll
+    for (int m = 0; m < 4; m++) s = dot4(spread_fields2((t.q >> (8 * m)) & 0xFFu), y[m], s);
+    sumi = (int)(t.sc & 0xFu) * s;
+    mins = (int)(t.sc >> 4) * (int)xq.bsum[sb * 16 + g];
+}
+
+// Q3_K (crates/pmetal-gguf/src/vec_dot.rs:739-777): element j takes bits 2 (j % 4) .. of qs[j / 4], bit j % 8 of
+// hmask[j / 8] as its third bit, minus 4; that routine unpacks only the first eight scales (nibble g of the first four
+// scale bytes, minus 8) and leaves the scales of groups 8..15 at zero.  16 lanes per super-block, lane g holds group g:
+// qs bytes 4 g .. 4 g + 3, hmask bytes 2 g, 2 g + 1.  Blocks are 110 bytes: only 2-byte aligned.
+// sum (q - 4) q8 = sum q q8 - 4 bsum[g].
+struct TaskQ3 {
+    uint32_t q, hm, aux0, d;
+};
+__device__ __forceinline__ void load_q3(const uint8_t *__restrict__ row, int sb, int g, bool live, TaskQ3 &t) {
+    const uint8_t *blk = row + (size_t)(live ? sb : 0) * 110;
+    t.hm = *reinterpret_cast<const uint16_t *>(blk + 2 * g);
+    t.q = load_u32_a2(blk + 32 + 4 * g);
+    t.aux0 = load_u32_a2(blk + 96);
+    t.d = *reinterpret_cast<const uint16_t *>(blk + 108);
+}
+__device__ __forceinline__ int dot_q3(const TaskQ3 &t, const XqLds &xq, int sb, int g) {
+    const uint4 q8 = xq.qs[sb * 16 + g];
+    const uint32_t y[4] = {q8.x, q8.y, q8.z, q8.w};
+    int s = 0;
+#pragma unroll
+    for (int m = 0; m < 4; m++)
+        s = dot4(spread_fields2((t.q >> (8 * m)) & 0xFFu) | (spread_bits4((t.hm >> (4 * m)) & 0xFu) << 2), y[m], s);
+    const int scale = g < 8 ? (int)((t.aux0 >> (4 * g)) & 0xFu) - 8 : 0;
+    return scale * (s - 4 * (int)xq.bsum[sb * 16 + g]);
+}
+
 // What the row walker below needs to know about a weight type.
 struct Q4Traits {
     using Task = TaskQ4;
@@ -265,6 +358,33 @@ struct Q6Traits {
         sumi = dot_q6(t, xq, sb, l), mins = 0;
     }
     static __device__ __forceinline__ uint32_t header(const Task &t) { return t.sc_d >> 16;  }  // d
+};
+
+struct Q5Traits {
+    using Task = TaskQ5;
+    static constexpr int kGroup = 8, kBlockBytes = 176;
+    static constexpr bool kHasMin = true;
+    static __device__ __forceinline__ void load(const uint8_t *row, int sb, int l, bool live, Task &t) { load_q5(row, sb, l, live, t); }
+    static __device__ __forceinline__ void dot(const Task &t, const XqLds &xq, int sb, int l, int &sumi, int &mins) { dot_q5(t, xq, sb, l, sumi, mins); }
+    static __device__ __forceinline__ uint32_t header(const Task &t) { return t.hdr.x; }  // d | dmin << 16
+};
+struct Q2Traits {
+    using Task = TaskQ2;
+    static constexpr int kGroup = 16, kBlockBytes = 84;
+    static constexpr bool kHasMin = true;
+    static __device__ __forceinline__ void load(const uint8_t *row, int sb, int l, bool live, Task &t) { load_q2(row, sb, l, live, t); }
+    static __device__ __forceinline__ void dot(const Task &t, const XqLds &xq, int sb, int l, int &sumi, int &mins) { dot_q2(t, xq, sb, l, sumi, mins); }
+    static __device__ __forceinline__ uint32_t header(const Task &t) { return t.hdr; }  // d | dmin << 16
+};
+struct Q3Traits {
+    using Task = TaskQ3;
+    static constexpr int kGroup = 16, kBlockBytes = 110;
+    static constexpr bool kHasMin = false;
+    static __device__ __forceinline__ void load(const uint8_t *row, int sb, int l, bool live, Task &t) { load_q3(row, sb, l, live, t); }
+    static __device__ __forceinline__ void dot(const Task &t, const XqLds &xq, int sb, int l, int &sumi, int &mins) {
+        sumi = dot_q3(t, xq, sb, l), mins = 0;
+    }
+    static __device__ __forceinline__ uint32_t header(const Task &t) { return t.d; }
 };
 
 // A wave multiplies 64 / kGroup rows at once: lane group g walks row g of the wave's rows super-block by
@@ -334,16 +454,25 @@ hipError_t launch_kl_sums(const float *a, const float *b, size_t n, double *part
     return hipGetLastError();
 }
 
-// k must be a multiple of 256 with the activation blocks fitting in LDS (k <= 32768); type Q4_K or Q6_K.
+// k must be a multiple of 256 with the activation blocks fitting in LDS (k <= 32768); type Q4_K, Q6_K, Q5_K, Q3_K or Q2_K.
+template <typename TR>
+static hipError_t launch_q8k_rows(const uint8_t *w, int64_t n, int spr, size_t lds, const uint8_t *xq, float *y, hipStream_t s) {
+    const int rows_per_wg = kWaves * 64 / TR::kGroup;
+    const dim3 grid((unsigned)((n + rows_per_wg - 1) / rows_per_wg)), block(64 * kWaves);
+    hipLaunchKernelGGL(k_qgemv_q8k<TR>, grid, block, lds, s, w, xq, y, (int)n, spr);
+    return hipGetLastError();
+}
 hipError_t launch_qgemv_q8k(uint32_t type, const uint8_t *w, int64_t n, int64_t k, const uint8_t *xq, float *y, hipStream_t s) {
     const int spr = (int)(k / 256);
     const size_t lds = xq_lds_bytes(spr);
     if (lds > 64 * 1024) return hipErrorInvalidValue;
-    const int rows_per_wg = kWaves * 64 / (type == kTypeQ4K ? Q4Traits::kGroup : Q6Traits::kGroup);
-    const dim3 grid((unsigned)((n + rows_per_wg - 1) / rows_per_wg)), block(64 * kWaves);
-    if (type == kTypeQ4K) hipLaunchKernelGGL(k_qgemv_q8k<Q4Traits>, grid, block, lds, s, w, xq, y, (int)n, spr);
-    else hipLaunchKernelGGL(k_qgemv_q8k<Q6Traits>, grid, block, lds, s, w, xq, y, (int)n, spr);
-    return hipGetLastError();
+    switch (type) {
+    case kTypeQ4K: return launch_q8k_rows<Q4Traits>(w, n, spr, lds, xq, y, s);
+    case kTypeQ5K: return launch_q8k_rows<Q5Traits>(w, n, spr, lds, xq, y, s);
+    case kTypeQ3K: return launch_q8k_rows<Q3Traits>(w, n, spr, lds, xq, y, s);
+    case kTypeQ2K: return launch_q8k_rows<Q2Traits>(w, n, spr, lds, xq, y, s);
+    default: return launch_q8k_rows<Q6Traits>(w, n, spr, lds, xq, y, s);
+    }
 }
 
 }  // namespace pmh

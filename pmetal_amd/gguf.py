@@ -184,7 +184,7 @@ def quantize_q8k_dev(x, n: int, out=None, stream=None) -> DeviceBuffer:
 
 
 def qgemv_q8k(dtype: int, w, n: int, k: int, xq, y=None, stream=None) -> DeviceBuffer:
-    """``y[r] = vec_dot_<dtype>_q8k(row r of w, xq)`` (crates/pmetal-gguf/src/vec_dot.rs:617-692), bit for bit."""
+    """``y[r] = vec_dot_<dtype>_q8k(row r of w, xq)`` (crates/pmetal-gguf/src/vec_dot.rs:617-810; Q4_K, Q6_K, Q5_K, Q3_K, Q2_K), bit for bit."""
     lib = _lib.load()
     if y is None:
         y = DeviceBuffer(max(4 * n, 16))

@@ -1,11 +1,12 @@
 """Q8_K activation blocks and the integer dot products over them (crates/pmetal-gguf/src/k_quants.rs:815-871,
-vec_dot.rs:617-692): the oracle against what pins it, then the HIP kernels against the oracle, bit for bit."""
+vec_dot.rs:617-810): the oracle against what pins it, then the HIP kernels against the oracle, bit for bit."""
 import struct
 
 import numpy as np
 import pytest
 
 Q4K, Q6K = 12, 14
+Q2K, Q3K, Q5K = 10, 11, 13
 
 
 # ---------------------------------------------------------------------------------------------------------------------
@@ -156,6 +157,156 @@ def test_vec_dot_q6k_q8k_known_answers(oracle):
     assert np.float32(got) == want
 
 
+def k4_scales(sc, m) -> bytes:
+    """The 12 scale bytes of a Q4_K / Q5_K super-block from 8 scales and 8 mins of 6 bits (k_quants.rs:915-926)."""
+    scales = np.zeros(12, dtype=np.uint8)
+    for j in range(8):
+        if j < 4:
+            scales[j] |= sc[j] & 63
+            scales[j + 4] |= m[j] & 63
+        else:
+            scales[j + 4] = (sc[j] & 0xF) | ((m[j] & 0xF) << 4)
+            scales[j - 4] |= (sc[j] >> 4) << 6
+            scales[j] |= (m[j] >> 4) << 6
+    return scales.tobytes()
+
+
+def q5k_block_linear(d: float, dmin: float, sc, m, q) -> bytes:
+    """A Q5_K super-block (d, dmin, scales[12], qh[32], qs[128]) whose element j, in the order the reference's dot product
+    reads it (vec_dot.rs:712-731), is q[j] (0..31): nibble j % 2 of qs[j / 2], bit j % 8 of qh[j / 8]."""
+    q = np.asarray(q, dtype=np.uint8)
+    qs, qh = np.zeros(128, dtype=np.uint8), np.zeros(32, dtype=np.uint8)
+    for j in range(256):
+        qs[j // 2] |= (q[j] & 0xF) << (4 * (j % 2))
+        qh[j // 8] |= (q[j] >> 4) << (j % 8)
+    return np.float16(d).tobytes() + np.float16(dmin).tobytes() + k4_scales(sc, m) + qh.tobytes() + qs.tobytes()
+
+
+def q2k_block_linear(d: float, dmin: float, sc, m, q) -> bytes:
+    """A Q2_K super-block (scales[16], qs[64], d, dmin) whose element j, in the order of vec_dot.rs:796-803, is q[j]
+    (0..3): bits 2 (j % 4) of qs[j / 4]; scales[g] = sc[g] | m[g] << 4."""
+    q = np.asarray(q, dtype=np.uint8)
+    qs = np.zeros(64, dtype=np.uint8)
+    for j in range(256):
+        qs[j // 4] |= (q[j] & 3) << (2 * (j % 4))
+    scales = np.array([(sc[g] & 0xF) | ((m[g] & 0xF) << 4) for g in range(16)], dtype=np.uint8)
+    return scales.tobytes() + qs.tobytes() + np.float16(d).tobytes() + np.float16(dmin).tobytes()
+
+
+def q3k_block_linear(d: float, scale_bytes, q) -> bytes:
+    """A Q3_K super-block (hmask[32], qs[64], scales[12], d) whose element j, in the order of vec_dot.rs:757-771, is
+    q[j] (0..7, value q - 4): bits 2 (j % 4) of qs[j / 4], bit j % 8 of hmask[j / 8]."""
+    q = np.asarray(q, dtype=np.uint8)
+    qs, hm = np.zeros(64, dtype=np.uint8), np.zeros(32, dtype=np.uint8)
+    for j in range(256):
+        qs[j // 4] |= (q[j] & 3) << (2 * (j % 4))
+        hm[j // 8] |= (q[j] >> 2) << (j % 8)
+    return hm.tobytes() + qs.tobytes() + np.asarray(scale_bytes, dtype=np.uint8).tobytes() + np.float16(d).tobytes()
+
+
+def test_vec_dot_q5k_q8k_known_answers(oracle):
+    ones = np.frombuffer(q8k_block(1.0, [1] * 256), np.uint8)
+    # q = 17 everywhere (fifth bit and low nibble 1), all scales 2, no mins: 256 * 17 * 2
+    blk = q5k_block_linear(1.0, 0.0, [2] * 8, [0] * 8, [17] * 256)
+    assert oracle.vec_dot_q8k(Q5K, np.frombuffer(blk, np.uint8), ones, 1) == 256 * 17 * 2
+    # the min term: m = 5 on sub-blocks 0 and 7 (the two forms of the 6-bit packing), dmin = 0.5 -> minus 0.5 * 5 * 32 * 2
+    blk = q5k_block_linear(1.0, 0.5, [0] * 8, [5, 0, 0, 0, 0, 0, 0, 5], [31] * 256)
+    assert oracle.vec_dot_q8k(Q5K, np.frombuffer(blk, np.uint8), ones, 1) == -160.0
+    rng = np.random.default_rng(5)
+    for _ in range(300):  # a single position: quant, activation and the scale of sub-block e / 32 (scales up to 63)
+        e, f = int(rng.integers(256)), int(rng.integers(256))
+        sc = [int(v) for v in rng.integers(1, 64, 8)]
+        q = np.zeros(256, np.uint8)
+        q[e] = int(rng.integers(1, 32))
+        a = np.zeros(256, np.int8)
+        a[f] = -7
+        blk = q5k_block_linear(2.0, 0.0, sc, [0] * 8, q)
+        got = oracle.vec_dot_q8k(Q5K, np.frombuffer(blk, np.uint8), np.frombuffer(q8k_block(0.5, a), np.uint8), 1)
+        assert got == (2.0 * 0.5 * int(q[e]) * -7 * sc[e // 32] if e == f else 0.0), (e, f)
+    # several blocks, every field random: integer sums per block, then the f32 recurrence of the routine in block order
+    w, x, want = b"", b"", np.float32(0)
+    for b in range(4):
+        sc, m = [int(v) for v in rng.integers(0, 64, 8)], [int(v) for v in rng.integers(0, 64, 8)]
+        q = rng.integers(0, 32, 256).astype(np.uint8)
+        a = rng.integers(-127, 128, 256).astype(np.int8)
+        d, dmin, yd = np.float16(rng.uniform(0.001, 0.01)), np.float16(rng.uniform(0.001, 0.01)), np.float32(rng.uniform(0.01, 0.1))
+        w += q5k_block_linear(float(d), float(dmin), sc, m, q)
+        x += q8k_block(float(yd), a)
+        mins = int((np.array(m, np.int64) * a.astype(np.int64).reshape(8, 32).sum(1)).sum())
+        sumi = int((q.astype(np.int64) * a.astype(np.int64) * np.repeat(sc, 32)).sum())
+        want = np.float32(want - np.float32(np.float32(np.float32(dmin) * yd) * np.float32(mins)))
+        want = np.float32(want + np.float32(np.float32(np.float32(d) * yd) * np.float32(sumi)))
+    assert np.float32(oracle.vec_dot_q8k(Q5K, np.frombuffer(w, np.uint8), np.frombuffer(x, np.uint8), 4)) == want
+
+
+def test_vec_dot_q2k_q8k_known_answers(oracle):
+    ones = np.frombuffer(q8k_block(1.0, [1] * 256), np.uint8)
+    blk = q2k_block_linear(1.0, 0.0, [3] * 16, [0] * 16, [2] * 256)   # 256 * 2 * 3
+    assert oracle.vec_dot_q8k(Q2K, np.frombuffer(blk, np.uint8), ones, 1) == 1536.0
+    blk = q2k_block_linear(1.0, 0.25, [0] * 16, [15] + [0] * 14 + [1], [3] * 256)  # minus 0.25 * (15 * 16 + 1 * 16)
+    assert oracle.vec_dot_q8k(Q2K, np.frombuffer(blk, np.uint8), ones, 1) == -64.0
+    rng = np.random.default_rng(6)
+    for _ in range(300):
+        e, f = int(rng.integers(256)), int(rng.integers(256))
+        sc = [int(v) for v in rng.integers(1, 16, 16)]
+        q = np.zeros(256, np.uint8)
+        q[e] = int(rng.integers(1, 4))
+        a = np.zeros(256, np.int8)
+        a[f] = 11
+        blk = q2k_block_linear(1.0, 0.0, sc, [0] * 16, q)
+        got = oracle.vec_dot_q8k(Q2K, np.frombuffer(blk, np.uint8), np.frombuffer(q8k_block(1.0, a), np.uint8), 1)
+        assert got == (float(int(q[e]) * 11 * sc[e // 16]) if e == f else 0.0), (e, f)
+    w, x, want = b"", b"", np.float32(0)
+    for b in range(4):
+        sc, m = [int(v) for v in rng.integers(0, 16, 16)], [int(v) for v in rng.integers(0, 16, 16)]
+        q = rng.integers(0, 4, 256).astype(np.uint8)
+        a = rng.integers(-127, 128, 256).astype(np.int8)
+        d, dmin, yd = np.float16(rng.uniform(0.001, 0.01)), np.float16(rng.uniform(0.001, 0.01)), np.float32(rng.uniform(0.01, 0.1))
+        w += q2k_block_linear(float(d), float(dmin), sc, m, q)
+        x += q8k_block(float(yd), a)
+        mins = int((np.array(m, np.int64) * a.astype(np.int64).reshape(16, 16).sum(1)).sum())
+        sumi = int((q.astype(np.int64) * a.astype(np.int64) * np.repeat(sc, 16)).sum())
+        want = np.float32(want - np.float32(np.float32(np.float32(dmin) * yd) * np.float32(mins)))
+        want = np.float32(want + np.float32(np.float32(np.float32(d) * yd) * np.float32(sumi)))
+    assert np.float32(oracle.vec_dot_q8k(Q2K, np.frombuffer(w, np.uint8), np.frombuffer(x, np.uint8), 4)) == want
+
+
+def test_vec_dot_q3k_q8k_known_answers(oracle):
+    ones = np.frombuffer(q8k_block(1.0, [1] * 256), np.uint8)
+    # scale nibbles 9 (value +1) in the first four bytes, q = 7 (value 3) everywhere: the first 128 elements count with
+    # scale 1, the last 128 with the zero that the routine leaves there -> 128 * 3
+    blk = q3k_block_linear(1.0, [0x99] * 4 + [0xFF] * 8, [7] * 256)
+    assert oracle.vec_dot_q8k(Q3K, np.frombuffer(blk, np.uint8), ones, 1) == 384.0
+    # nibble 0 is scale -8; q = 0 is value -4: 128 * (-4) * (-8)
+    blk = q3k_block_linear(0.5, [0x00] * 12, [0] * 256)
+    assert oracle.vec_dot_q8k(Q3K, np.frombuffer(blk, np.uint8), ones, 1) == 0.5 * 128 * 32
+    rng = np.random.default_rng(7)
+    for _ in range(300):  # a single position: every other quant is 4 (value 0)
+        e, f = int(rng.integers(256)), int(rng.integers(256))
+        sb = [int(v) for v in rng.integers(0, 256, 12)]
+        q = np.full(256, 4, np.uint8)
+        q[e] = int(rng.integers(0, 8))
+        a = np.zeros(256, np.int8)
+        a[f] = 13
+        blk = q3k_block_linear(1.0, sb, q)
+        got = oracle.vec_dot_q8k(Q3K, np.frombuffer(blk, np.uint8), np.frombuffer(q8k_block(1.0, a), np.uint8), 1)
+        g = e // 16
+        scale = (((sb[g // 2] >> (4 * (g % 2))) & 0xF) - 8) if g < 8 else 0
+        assert got == (float((int(q[e]) - 4) * 13 * scale) if e == f else 0.0), (e, f, g)
+    w, x, want = b"", b"", np.float32(0)
+    for b in range(4):
+        sb = [int(v) for v in rng.integers(0, 256, 12)]
+        q = rng.integers(0, 8, 256).astype(np.uint8)
+        a = rng.integers(-127, 128, 256).astype(np.int8)
+        d, yd = np.float16(rng.uniform(0.001, 0.01)), np.float32(rng.uniform(0.01, 0.1))
+        w += q3k_block_linear(float(d), sb, q)
+        x += q8k_block(float(yd), a)
+        scales = np.array([(((sb[g // 2] >> (4 * (g % 2))) & 0xF) - 8) if g < 8 else 0 for g in range(16)], np.int64)
+        sumi = int(((q.astype(np.int64) - 4) * a.astype(np.int64) * np.repeat(scales, 16)).sum())
+        want = np.float32(want + np.float32(np.float32(np.float32(d) * yd) * np.float32(sumi)))
+    assert np.float32(oracle.vec_dot_q8k(Q3K, np.frombuffer(w, np.uint8), np.frombuffer(x, np.uint8), 4)) == want
+
+
 # ---------------------------------------------------------------------------------------------------------------------
 # HIP kernels against the oracle (GPU)
 # ---------------------------------------------------------------------------------------------------------------------
@@ -209,7 +360,7 @@ def test_gpu_quantize_q8k_bit_exact(oracle):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("t", [Q4K, Q6K])
+@pytest.mark.parametrize("t", [Q4K, Q6K, Q5K, Q3K, Q2K])
 @pytest.mark.parametrize("n,k", [(1, 256), (7, 512), (300, 1024), (64, 4096), (1000, 2048), (4096, 4096), (33, 32768), (513, 2304)])
 def test_gpu_qgemv_q8k_bit_exact(oracle, t, n, k):
     import pmetal_amd as pm
@@ -237,12 +388,40 @@ def test_gpu_qgemv_q8k_bit_exact(oracle, t, n, k):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("t,block,d_at", [(Q5K, 176, (0, 2)), (Q3K, 110, (108,)), (Q2K, 84, (80, 82))])
+def test_gpu_qgemv_q8k_random_block_bytes(oracle, t, block, d_at):
+    """Every scale, min, quant and high-bit pattern: random block bytes with finite d / dmin of both signs, rows that start
+    at every alignment the block size allows (odd numbers of super-blocks), activations over the whole int8 range."""
+    import pmetal_amd as pm
+    from pmetal_amd import gguf
+    pm.init(0)
+    rng = np.random.default_rng(t)
+    for n, k in ((37, 256 * 3), (260, 256 * 7), (1025, 2048)):
+        spr = k // 256
+        raw = rng.integers(0, 256, size=(n * spr, block), dtype=np.uint8)
+        for off in d_at:
+            vals = (rng.uniform(0.001, 0.05, n * spr) * rng.choice([-1.0, 1.0], n * spr)).astype(np.float16)
+            raw[:, off:off + 2] = vals.view(np.uint8).reshape(-1, 2)
+        raw = raw.reshape(-1)
+        xq = np.concatenate([np.frombuffer(q8k_block(float(rng.uniform(0.01, 0.1)), rng.integers(-128, 128, 256).astype(np.int8)), np.uint8)
+                             for _ in range(spr)])
+        want = oracle.qmatvec_q8k(t, raw, n, k, xq)
+        dw, dxq, dy = pm.DeviceBuffer.from_host(raw), pm.DeviceBuffer.from_host(xq), pm.DeviceBuffer(max(4 * n, 16))
+        gguf.qgemv_q8k(t, dw, n, k, dxq, dy)
+        pm.check(pm._lib.load().pmetal_hip_sync(None))
+        got = dy.to_host(np.float32, n)
+        bad = np.nonzero(got.view(np.uint32) != want.view(np.uint32))[0]
+        assert bad.size == 0, (t, n, k, bad[:5], got[bad[:5]], want[bad[:5]])
+
+
+@pytest.mark.gpu
 def test_gpu_qgemv_q8k_argument_errors():
     import pmetal_amd as pm
     pm.init(0)
     lib = pm._lib.load()
     buf = pm.DeviceBuffer(1 << 16)
     assert lib.pmetal_hip_qgemv_q8k(8, buf.ptr, 4, 256, buf.ptr, buf.ptr, None) == 2      # Q8_0 weights: no such product
+    assert lib.pmetal_hip_qgemv_q8k(15, buf.ptr, 4, 256, buf.ptr, buf.ptr, None) == 2     # nor Q8_K against Q8_K
     assert lib.pmetal_hip_qgemv_q8k(Q4K, buf.ptr, 4, 300, buf.ptr, buf.ptr, None) == 6    # k not a multiple of 256
     assert lib.pmetal_hip_qgemv_q8k(Q4K, buf.ptr, 4, 65536, buf.ptr, buf.ptr, None) == 6  # k too long for LDS
     assert lib.pmetal_hip_qgemv_q8k(Q4K, None, 4, 256, buf.ptr, buf.ptr, None) == 1
