@@ -437,16 +437,22 @@ __global__ __launch_bounds__(1024) void k_qgemv_q4k_chunk(const uint8_t *__restr
 constexpr int kRowsWaves = 8;         // waves per workgroup
 constexpr int kRowsPerWaveMax = 8;    // row totals a wave keeps in LDS (kDepth tasks of one chunk each)
 
-template <int ORDER, bool XF32, int KS, bool PAIR>
-__global__ __launch_bounds__(64 * kRowsWaves) void k_qgemv_q4k_rows(const uint8_t *__restrict__ W0, const uint8_t *__restrict__ W1,
-                                                                     const void *__restrict__ xg, int split_wg, int n_rows0, int n_rows1,
-                                                                     int spr, int rows_per_wg, float *__restrict__ y0,
-                                                                     float *__restrict__ y1) {
-    const bool second = PAIR && (int)blockIdx.x >= split_wg;  // workgroup-uniform
-    const uint8_t *__restrict__ W = second ? W1 : W0;
-    float *__restrict__ y = second ? y1 : y0;
-    const int n_rows = second ? n_rows1 : n_rows0;
-    const int wg_index = second ? (int)blockIdx.x - split_wg : (int)blockIdx.x;
+template <int ORDER, bool XF32, int KS, bool MULTI>
+__global__ __launch_bounds__(64 * kRowsWaves) void k_qgemv_q4k_rows(const void *__restrict__ xg, const uint8_t *__restrict__ w0,
+                                                                     const uint8_t *__restrict__ w1, const uint8_t *__restrict__ w2,
+                                                                     const uint8_t *__restrict__ w3, int wg_b1, int wg_b2, int wg_b3,
+                                                                     int spr, int rows_per_wg, int n0, int n1, int n2, int n3,
+                                                                     float *__restrict__ y0, float *__restrict__ y1,
+                                                                     float *__restrict__ y2, float *__restrict__ y3) {
+    // Up to four matrices that share k and the activation vector go through one launch (MULTI): workgroups
+    // [wg_b(g), wg_b(g + 1)) belong to matrix g (workgroup-uniform selects); otherwise only w0, n0, y0 are looked at.
+    static_assert(pmh::kMaxGemvGroup == 4, "the argument list spells out four group members");
+    const int bx = (int)blockIdx.x;
+    const int g = MULTI ? (bx >= wg_b1 ? 1 : 0) + (bx >= wg_b2 ? 1 : 0) + (bx >= wg_b3 ? 1 : 0) : 0;
+    const uint8_t *__restrict__ W = g == 0 ? w0 : g == 1 ? w1 : g == 2 ? w2 : w3;
+    float *__restrict__ y = g == 0 ? y0 : g == 1 ? y1 : g == 2 ? y2 : y3;
+    const int n_rows = g == 0 ? n0 : g == 1 ? n1 : g == 2 ? n2 : n3;
+    const int wg_index = bx - (g == 0 ? 0 : g == 1 ? wg_b1 : g == 2 ? wg_b2 : wg_b3);
     constexpr int NDIG = XF32 ? 6 : 5;
     constexpr int T = 64, nthreads = 64 * kRowsWaves;
     extern __shared__ uint4 smem[];
@@ -733,44 +739,67 @@ hipError_t launch_group_general(const uint8_t *const *w, const int64_t *n, float
 
 namespace pmh {
 
-// Kernel R over one matrix (n1 == 0) or two that share k, x and the element order.  hipErrorNotSupported when the shape does
-// not suit it (rows of more than two chunks or not whole chunks, more rows per wave than the ring holds tasks, offsets
-// beyond 32 bits): the caller goes on to kernel A.
+// Kernel R over one to four matrices that share k, x and the element order.  hipErrorNotSupported when the shapes do not
+// suit it (rows of more than two chunks or not whole chunks, more rows per wave than the ring holds tasks, offsets beyond
+// 32 bits): the caller goes on to another kernel.
 template <int ORDER, bool XF32>
-static hipError_t launch_rows_kernel(int ks, bool pair, dim3 grid, size_t lds, hipStream_t s, const uint8_t *w0, const uint8_t *w1,
-                                     const void *x, int split_wg, int n0, int n1, int spr, int rows_per_wg, float *y0, float *y1) {
+static hipError_t launch_rows_kernel(int ks, bool multi, dim3 grid, size_t lds, hipStream_t s, const GemvGroup &grp, const void *x, int spr,
+                                     int rows_per_wg) {
     const dim3 block(64 * kRowsWaves);
-    if (ks == 2)
-        return pair ? launch_with_lds(k_qgemv_q4k_rows<ORDER, XF32, 2, true>, grid, block, lds, s, w0, w1, x, split_wg, n0, n1, spr, rows_per_wg, y0, y1)
-                    : launch_with_lds(k_qgemv_q4k_rows<ORDER, XF32, 2, false>, grid, block, lds, s, w0, w1, x, split_wg, n0, n1, spr, rows_per_wg, y0, y1);
-    return pair ? launch_with_lds(k_qgemv_q4k_rows<ORDER, XF32, 1, true>, grid, block, lds, s, w0, w1, x, split_wg, n0, n1, spr, rows_per_wg, y0, y1)
-                : launch_with_lds(k_qgemv_q4k_rows<ORDER, XF32, 1, false>, grid, block, lds, s, w0, w1, x, split_wg, n0, n1, spr, rows_per_wg, y0, y1);
+    auto go = [&](auto kern) {
+        return launch_with_lds(kern, grid, block, lds, s, x, grp.w[0], grp.w[1], grp.w[2], grp.w[3], grp.wg_begin[1], grp.wg_begin[2],
+                               grp.wg_begin[3], spr, rows_per_wg, grp.n[0], grp.n[1], grp.n[2], grp.n[3], grp.y[0], grp.y[1], grp.y[2],
+                               grp.y[3]);
+    };
+    if (ks == 2) return multi ? go(k_qgemv_q4k_rows<ORDER, XF32, 2, true>) : go(k_qgemv_q4k_rows<ORDER, XF32, 2, false>);
+    return multi ? go(k_qgemv_q4k_rows<ORDER, XF32, 1, true>) : go(k_qgemv_q4k_rows<ORDER, XF32, 1, false>);
 }
 
-static hipError_t launch_kernel_rows(const uint8_t *w0, int64_t n0, float *y0, const uint8_t *w1, int64_t n1, float *y1, int64_t k,
-                                     const void *x, bool xf32, uint32_t order, hipStream_t s) {
+static hipError_t launch_kernel_rows(const uint8_t *const *w, const int64_t *n, float *const *y, int count, int64_t k, const void *x,
+                                     bool xf32, uint32_t order, hipStream_t s) {
     const int spr = (int)(k / 256);
-    if (spr % 8 != 0 || spr / 8 > 2) return hipErrorNotSupported;
+    if (spr % 8 != 0 || spr / 8 > 2 || count < 1 || count > kMaxGemvGroup) return hipErrorNotSupported;
     const int ks = spr / 8;
-    const uint64_t w_max = (uint64_t)(n0 > n1 ? n0 : n1) * (uint64_t)spr * 144u;
-    if (w_max >= (1ull << 32)) return hipErrorNotSupported;
-    // two workgroups per compute unit and matrix
-    const int64_t n = n0 + n1, want = (n1 > 0 ? 4 : 2) * (int64_t)gemv::compute_units();
-    const int64_t n_wg = n < want ? n : want;
-    const int64_t rows_per_wg = (n + n_wg - 1) / n_wg;
-    if (((rows_per_wg + kRowsWaves - 1) / kRowsWaves) * ks > kDepth) return hipErrorNotSupported;
-    const int64_t wg0 = (n0 + rows_per_wg - 1) / rows_per_wg, wg1 = (n1 + rows_per_wg - 1) / rows_per_wg;
+    int64_t total = 0, n_max = 0;
+    for (int i = 0; i < count; i++) total += n[i], n_max = n[i] > n_max ? n[i] : n_max;
+    if ((uint64_t)n_max * (uint64_t)spr * 144u >= (1ull << 32)) return hipErrorNotSupported;
+    // Two workgroups per compute unit; a launch of several matrices that would leave a wave more tasks than the ring holds
+    // takes four per compute unit instead (two rounds, and the end of one workgroup overlaps the start of the next).
+    const int64_t cus = gemv::compute_units();
+    const int64_t max_rows_per_wg = (int64_t)kRowsWaves * (kDepth / ks);
+    int64_t want = 2 * cus;
+    if (count > 1 && (total + want - 1) / want > max_rows_per_wg) want = 4 * cus;
+    int64_t n_wg = total < want ? total : want;
+    int64_t rows_per_wg = (total + n_wg - 1) / n_wg;
+    // every member rounds its workgroup count up: keep the sum within the intended number of workgroups
+    for (;;) {
+        int64_t c = 0;
+        for (int i = 0; i < count; i++) c += (n[i] + rows_per_wg - 1) / rows_per_wg;
+        if (c <= want || rows_per_wg >= total) break;
+        rows_per_wg++;
+    }
+    if (rows_per_wg > max_rows_per_wg) return hipErrorNotSupported;
+    GemvGroup grp{};
+    int begin = 0;
+    for (int i = 0; i < kMaxGemvGroup; i++) {
+        grp.wg_begin[i] = begin;
+        if (i < count) {
+            grp.w[i] = w[i], grp.y[i] = y[i], grp.n[i] = (int)n[i];
+            begin += (int)((n[i] + rows_per_wg - 1) / rows_per_wg);
+        } else {
+            grp.w[i] = w[0], grp.y[i] = y[0], grp.n[i] = 0;
+        }
+    }
+    grp.wg_begin[kMaxGemvGroup] = begin;
     const size_t slots = (size_t)spr * 8;
     const size_t lds = slots * 16 * (xf32 ? 6 : 5) + slots * 16 + (size_t)kRowsWaves * kRowsPerWaveMax * 4;
-    const dim3 grid((unsigned)(wg0 + wg1));
-    const uint8_t *b_w = n1 ? w1 : w0;
-    float *b_y = n1 ? y1 : y0;
-    const bool pair = n1 > 0;
+    const dim3 grid((unsigned)begin);
+    const bool multi = count > 1;
     if (order == kOrderRef)
-        return xf32 ? launch_rows_kernel<0, true>(ks, pair, grid, lds, s, w0, b_w, x, (int)wg0, (int)n0, (int)n1, spr, (int)rows_per_wg, y0, b_y)
-                    : launch_rows_kernel<0, false>(ks, pair, grid, lds, s, w0, b_w, x, (int)wg0, (int)n0, (int)n1, spr, (int)rows_per_wg, y0, b_y);
-    return xf32 ? launch_rows_kernel<1, true>(ks, pair, grid, lds, s, w0, b_w, x, (int)wg0, (int)n0, (int)n1, spr, (int)rows_per_wg, y0, b_y)
-                : launch_rows_kernel<1, false>(ks, pair, grid, lds, s, w0, b_w, x, (int)wg0, (int)n0, (int)n1, spr, (int)rows_per_wg, y0, b_y);
+        return xf32 ? launch_rows_kernel<0, true>(ks, multi, grid, lds, s, grp, x, spr, (int)rows_per_wg)
+                    : launch_rows_kernel<0, false>(ks, multi, grid, lds, s, grp, x, spr, (int)rows_per_wg);
+    return xf32 ? launch_rows_kernel<1, true>(ks, multi, grid, lds, s, grp, x, spr, (int)rows_per_wg)
+                : launch_rows_kernel<1, false>(ks, multi, grid, lds, s, grp, x, spr, (int)rows_per_wg);
 }
 
 // Kernel A over one matrix (n1 == 0) or two that share k, x and the element order.  hipErrorNotSupported when the shape
@@ -824,7 +853,7 @@ hipError_t launch_qgemv_q4k(const uint8_t *w, int64_t n, int64_t k, const void *
     // Measured crossovers against kernel B: the row-owner kernel from about 8 MiB (4096 x 4096: 4.21 against 4.28 us,
     // 5120 x 4096: 4.5 against 5.4; 2048 x 4096: 3.7 against 3.5), kernel A from about 12 MiB.
     if (w_bytes >= (8ull << 20)) {
-        const hipError_t e = launch_kernel_rows(w, n, y, nullptr, 0, nullptr, k, x, xf32, order, s);
+        const hipError_t e = launch_kernel_rows(&w, &n, &y, 1, k, x, xf32, order, s);
         if (e != hipErrorNotSupported) return e;
     }
     if (w_bytes >= (12ull << 20)) {
@@ -841,7 +870,10 @@ hipError_t launch_qgemv_q4k_pair(const uint8_t *w0, int64_t n0, float *y0, const
     const bool xf32 = x_dtype == kDtypeF32;
     const size_t slots = (size_t)(k / 256) * 8;
     if (slots * 16 * (xf32 ? 6 : 5) + slots * 16 > gemv::kMaxLds) return hipErrorNotSupported;
-    const hipError_t e = launch_kernel_rows(w0, n0, y0, w1, n1, y1, k, x, xf32, order, s);
+    const uint8_t *ws[2] = {w0, w1};
+    const int64_t ns[2] = {n0, n1};
+    float *ys[2] = {y0, y1};
+    const hipError_t e = launch_kernel_rows(ws, ns, ys, 2, k, x, xf32, order, s);
     if (e != hipErrorNotSupported) return e;
     return launch_kernel_a(w0, n0, y0, w1, n1, y1, k, x, xf32, order, s);
 }
@@ -852,7 +884,16 @@ bool qgemv_q4k_groupable(int64_t n, int64_t k) { return (uint64_t)n * (uint64_t)
 hipError_t launch_qgemv_q4k_group(const uint8_t *const *w, const int64_t *n, float *const *y, int count, int64_t k,
                                   const void *x, uint32_t x_dtype, uint32_t order, hipStream_t s) {
     if (count < 1 || count > kMaxGemvGroup) return hipErrorInvalidValue;
-    return launch_group_general(w, n, y, count, k, x, x_dtype == kDtypeF32, order, s);
+    // a group that is large as a whole (q / k / v of an 8B-class model: 14 MB) streams like one large matrix
+    uint64_t bytes = 0;
+    for (int i = 0; i < count; i++) bytes += (uint64_t)n[i] * (uint64_t)(k / 256) * 144u;
+    const size_t slots = (size_t)(k / 256) * 8;
+    const bool xf32 = x_dtype == kDtypeF32;
+    if (bytes >= (8ull << 20) && slots * 16 * (xf32 ? 6 : 5) + slots * 16 <= gemv::kMaxLds) {
+        const hipError_t e = launch_kernel_rows(w, n, y, count, k, x, xf32, order, s);
+        if (e != hipErrorNotSupported) return e;
+    }
+    return launch_group_general(w, n, y, count, k, x, xf32, order, s);
 }
 
 }  // namespace pmh

@@ -264,6 +264,42 @@ def test_qgemv_batch_groups_projections_of_one_activation(oracle, order):
         assert np.array_equal(dy.to_host(np.float32), single)
 
 
+@pytest.mark.parametrize("k,x_dtype", [(4096, pm.DTYPE_BF16), (2048, pm.DTYPE_F32)])
+@pytest.mark.parametrize("order", [0, 1])
+def test_qgemv_batch_groups_that_are_large_as_a_whole(oracle, order, k, x_dtype):
+    """q / k / v of an 8B-class model: each below the large-matrix threshold, 14 MB together.  The group streams through
+    the row-owner kernel as one launch; every member against the oracle and against its own launch (ragged row counts,
+    a fourth small member, then a matrix with another x)."""
+    from pmetal_amd import _lib
+    lib = _lib.load()
+    rows = [4096, 1024, 1031, 517, 700]
+    rng = np.random.default_rng(k + order)
+    xa, xa_ref = activations(oracle, 5, k, x_dtype)
+    xb, xb_ref = activations(oracle, 6, k, x_dtype)
+    dx, dx2 = pm.DeviceBuffer.from_host(xa), pm.DeviceBuffer.from_host(xb)
+    xs_of = [dx, dx, dx, dx, dx2]
+    descs = (_lib.LinearDesc * len(rows))()
+    keep = []
+    for i, n in enumerate(rows):
+        raw = rng.integers(0, 256, size=(n * (k // 256), 144), dtype=np.uint8)
+        raw[:, 0:4] = np.frombuffer(np.array([0.01, 0.02], np.float16).tobytes(), np.uint8)
+        raw = raw.reshape(-1)
+        dw, dy = pm.DeviceBuffer.from_host(raw), pm.DeviceBuffer(4 * n)
+        pm.check(lib.pmetal_hip_memset(dy.ptr, 0xFF, 4 * n, None))
+        x_dev, x_ref = (xa, xa_ref) if xs_of[i] is dx else (xb, xb_ref)
+        keep.append((dw, dy, raw, n, x_dev, x_ref))
+        descs[i] = _lib.LinearDesc(Q4K, x_dtype, order, 0, n, k, dw.ptr, xs_of[i].ptr, dy.ptr)
+    pm.check(lib.pmetal_hip_qgemv_batch(descs, len(rows), None))
+    pm.check(lib.pmetal_hip_sync(None))
+    for dw, dy, raw, n, x_dev, x_ref in keep:
+        got = dy.to_host(np.float32)
+        want = oracle.qmatvec(Q4K, raw, n, k, x_ref, order=order)
+        elem, norm = rel_errors(got, want)
+        assert elem <= TOL and norm <= TOL, (n, elem, norm)
+        single = gpu_qgemv(Q4K, raw, n, k, x_dev, x_dtype, order)
+        assert np.abs(got - single).max() <= 2e-6 * np.abs(single).max()
+
+
 @pytest.mark.parametrize("order", [0, 1])
 def test_qgemv_batch_pairs_large_projections_of_one_activation(oracle, order):
     """Two consecutive large Q4_K matrices that share x (gate / up) go through one launch of the large-matrix kernel:
