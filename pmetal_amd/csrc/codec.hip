@@ -1060,8 +1060,21 @@ __global__ __launch_bounds__(64) void k_quantize_q2k(const float *__restrict__ x
     const float dq = f16_bits_to_f32(d16) * (float)(byte & 0xFu);
     if (dq != 0.0f) {
         const float dm = f16_bits_to_f32(dmin16) * (float)(byte >> 4);
+        // by multiplication with 1 / dq where that provably rounds like the division (see the Q4_K kernel), by the division
+        // for the lanes that come within 8e-6 of a rounding boundary
+        const float rinv = 1.0f / dq;
+        bool exact_needed = !(dq > 1e-20f && dq < 1e20f);
 #pragma unroll
-        for (int i = 0; i < 16; i++) q[i] = (uint32_t)clamp_round_0_15<3>((xv[i] + dm) / dq);
+        for (int i = 0; i < 16; i++) {
+            const float qf = __builtin_fminf(__builtin_fmaxf((xv[i] + dm) * rinv, 0.0f), 3.0f);
+            const float r = __builtin_truncf(qf + 0.49999997f);
+            exact_needed |= !(__builtin_fabsf(__builtin_fabsf(qf - r) - 0.5f) >= 8e-6f);
+            q[i] = (uint32_t)r;
+        }
+        if (exact_needed) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) q[i] = (uint32_t)clamp_round_0_15<3>((xv[i] + dm) / dq);
+        }
     }
     const size_t sb = sb0 + (lane >> 4);
     uint8_t *blk = sb < n_sb ? dst + sb * 84 : nullptr;
@@ -1092,31 +1105,42 @@ __global__ __launch_bounds__(64) void k_quantize_q3k(const float *__restrict__ x
     float scale = 0.0f;
     if (amax != 0.0f) {
         const float iscale = -4.0f / maxv;
-        int l[16];
+        float l[16], w[16], wx[16];  // the quants as floats: small integers, every product with them as in integer form
         float sumlx = 0.0f, suml2 = 0.0f;
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            l[i] = clamp_i(nearest_int_sat(iscale * xv[i]), -4, 3);
-            const float w = xv[i] * xv[i];
-            sumlx += w * xv[i] * (float)l[i];
-            suml2 += w * (float)(l[i] * l[i]);
+            l[i] = (float)clamp_i(nearest_int_sat(iscale * xv[i]), -4, 3);
+            w[i] = xv[i] * xv[i];
+            wx[i] = w[i] * xv[i];
+            sumlx += wx[i] * l[i];
+            suml2 += w[i] * (l[i] * l[i]);
         }
+        // The sweeps (quantize.rs:680-713), branch-free as in the Q6_K kernel: every element computes its candidate and the
+        // test and takes them by select; the candidate clamp(nearest_int(x sl2 / slx)) comes from a multiplication with an
+        // approximate reciprocal where that provably rounds like the quotient (within 8e-6 of it for |quotient| < 33, so
+        // 2e-5 away from every rounding boundary is safe), from the IEEE division otherwise.
         for (int sweep = 0; sweep < 5; sweep++) {
             bool any = false;
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                const float w = xv[i] * xv[i], wx = w * xv[i];
-                float slx = sumlx - wx * (float)l[i];
-                if (slx > 0.0f) {
-                    float sl2 = suml2 - w * (float)(l[i] * l[i]);
-                    const int nl = clamp_i(nearest_int_sat(xv[i] * sl2 / slx), -4, 3);
-                    if (nl != l[i]) {
-                        slx += wx * (float)nl;
-                        sl2 += w * (float)(nl * nl);
-                        if (sl2 > 0.0f && slx * slx * suml2 > sumlx * sumlx * sl2) {
-                            l[i] = nl, sumlx = slx, suml2 = sl2, any = true;
-                        }
-                    }
+                const float li = l[i];
+                const float slx = sumlx - wx[i] * li;
+                const float sl2 = suml2 - w[i] * (li * li);
+                const float p = xv[i] * sl2;
+                const bool pos = slx > 0.0f;
+                const float qf = p * __builtin_amdgcn_rcpf(slx);
+                float nl = (float)clamp_i(nearest_int_sat(qf), -4, 3);
+                const bool sure = slx > 1e-30f && slx < 1e30f && __builtin_fabsf(__builtin_fabsf(qf - nl) - 0.5f) >= 2e-5f;
+                if (pos && !sure) nl = (float)clamp_i(nearest_int_sat(p / slx), -4, 3);
+                const bool differs = pos & (nl != li);
+                if (sweep == 0 || __builtin_amdgcn_ballot_w64(differs) != 0) {  // later sweeps: rarely a candidate anywhere
+                    const float slx2 = slx + wx[i] * nl;
+                    const float sl22 = sl2 + w[i] * (nl * nl);
+                    const bool take = differs & (sl22 > 0.0f) & (slx2 * slx2 * suml2 > sumlx * sumlx * sl22);
+                    l[i] = take ? nl : li;
+                    sumlx = take ? slx2 : sumlx;
+                    suml2 = take ? sl22 : suml2;
+                    any |= take;
                 }
             }
             if (!any) break;
@@ -1152,8 +1176,19 @@ __global__ __launch_bounds__(64) void k_quantize_q3k(const float *__restrict__ x
     for (int i = 0; i < 16; i++) q[i] = 0;
     const float dq = f16_bits_to_f32(d16) * (float)(lv - 32);
     if (max_scale != 0.0f && dq != 0.0f) {
+        const float rinv = 1.0f / dq;
+        bool exact_needed = !(__builtin_fabsf(dq) > 1e-20f && __builtin_fabsf(dq) < 1e20f);
 #pragma unroll
-        for (int i = 0; i < 16; i++) q[i] = (uint32_t)(clamp_i(nearest_int_sat(xv[i] / dq), -4, 3) + 4);
+        for (int i = 0; i < 16; i++) {
+            const float qf = xv[i] * rinv;
+            const int ll = clamp_i(nearest_int_sat(qf), -4, 3);
+            exact_needed |= !(__builtin_fabsf(__builtin_fabsf(qf - (float)ll) - 0.5f) >= 8e-6f);
+            q[i] = (uint32_t)(ll + 4);
+        }
+        if (exact_needed) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) q[i] = (uint32_t)(clamp_i(nearest_int_sat(xv[i] / dq), -4, 3) + 4);
+        }
     }
     // element 16 j + i has its high bit at bit j / 2 of hmask[16 (j % 2) + i]: the eight lanes of one parity or theirs
     uint32_t hw[4];
