@@ -566,7 +566,7 @@ def bench_decode(args, model="qwen3_0.6b"):
         "value": tok_s, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "k_qgemv_q4k / k_qgemv_q6k (197 projections in 127 launches)" if model == "qwen3_0.6b"
+                     "kernel": "k_qgemv_q4k / k_qgemv_q6k (197 projections in 113 launches)" if model == "qwen3_0.6b"
                      else "k_qgemv_q4k_chunk / k_qgemv_q6k_chunk (225 projections)",
                      "bytes_per_step": total_bytes},
         "extra": {"launches_per_token": len(lins), "q6k_tensors": sum(1 for l in lins if l[3] == Q6K),

@@ -570,6 +570,31 @@ int32_t pmetal_hip_qgemv_batch(const pmetal_hip_linear_desc *descs, size_t count
                 j++;
             }
         }
+        // A Q6_K projection of the same activations right after such a group (the v of a Q4_K_M layer whose q and k are
+        // Q4_K) joins its launch when the shapes suit it.
+        if (j > i && j < count && j - i < (size_t)pmh::kMaxGemvGroup && d.ggml_type == PMETAL_GGML_TYPE_Q4K && d.k > 0 && d.k % 256 == 0 &&
+            d.n > 0 && pmh::qgemv_q4k_groupable(d.n, d.k)) {
+            const pmetal_hip_linear_desc &v = descs[j];
+            if (v.ggml_type == PMETAL_GGML_TYPE_Q6K && v.k == d.k && v.x_dev == d.x_dev && v.x_dtype == d.x_dtype && v.order == d.order &&
+                v.n > 0) {
+                const uint8_t *w[pmh::kMaxGemvGroup];
+                float *y[pmh::kMaxGemvGroup];
+                int64_t n[pmh::kMaxGemvGroup];
+                for (size_t g = i; g < j; g++) {
+                    const pmetal_hip_linear_desc &e = descs[g];
+                    if (int32_t rc = check_linear(e.ggml_type, e.w_dev, e.n, e.k, e.x_dev, e.x_dtype, e.y_dev, e.order)) return rc;
+                    w[g - i] = e.w_dev, y[g - i] = e.y_dev, n[g - i] = e.n;
+                }
+                if (int32_t rc = check_linear(v.ggml_type, v.w_dev, v.n, v.k, v.x_dev, v.x_dtype, v.y_dev, v.order)) return rc;
+                const hipError_t err = pmh::launch_qgemv_q4k_q6k_group(w, n, y, (int)(j - i), v.w_dev, v.n, v.y_dev, d.k, d.x_dev, d.x_dtype,
+                                                                       d.order, (hipStream_t)stream);
+                if (err == hipSuccess) {
+                    i = j + 1;
+                    continue;
+                }
+                if (err != hipErrorNotSupported) return hip_fail(err, "mixed grouped qgemv kernel launch");
+            }
+        }
         if (j - i < 2) {
             // Two consecutive large Q4_K projections of the same activation vector (gate / up of a large model) share a
             // launch of the large-matrix kernel.

@@ -26,7 +26,7 @@
 //  * At the end of a row the team's partial sums are reduced with DPP only (quad_perm, row_half_mirror,
 //    row_mirror inside a 16-lane row, row_bcast:15 / row_bcast:31 across rows); the last lane of the
 //    team stores y[row].
-#include "gemv_common.hpp"
+#include "gemv_q6k_small.hpp"
 
 namespace {
 
@@ -540,15 +540,22 @@ struct GemvGroup {
 // The arguments come as scalars, the ones needed first up front: the leading 16 dwords of the kernel-argument
 // segment are preloaded into scalar registers at wave launch (the translation unit is built with
 // -amdgpu-kernarg-preload-count=16), so the first weight request does not wait for an argument fetch.
-template <int ORDER, bool XF32, int T>
+// Q6LAST: the fourth member is a Q6_K matrix (the v projection of a layer whose q and k are Q4_K): the workgroups from
+// wg_b3 on run the small-matrix Q6_K GEMV over it, with q6_teams teams of T lanes each taking rows.
+template <int ORDER, bool XF32, int T, bool Q6LAST>
 __global__ __launch_bounds__(1024) void k_qgemv_q4k(const void *__restrict__ xg, const uint8_t *__restrict__ w0,
                                                      const uint8_t *__restrict__ w1, const uint8_t *__restrict__ w2,
                                                      const uint8_t *__restrict__ w3, int wg_b1, int wg_b2, int wg_b3,
                                                      int spr, int rows_per_wg, int per_team, int n0, int n1, int n2,
                                                      int n3, float *__restrict__ y0, float *__restrict__ y1,
-                                                     float *__restrict__ y2, float *__restrict__ y3, int nthreads) {
+                                                     float *__restrict__ y2, float *__restrict__ y3, int nthreads, int q6_teams) {
     static_assert(pmh::kMaxGemvGroup == 4, "the argument list spells out four group members");
     const int bx = (int)blockIdx.x;
+    if (Q6LAST && bx >= wg_b3) {  // workgroup-uniform
+        extern __shared__ uint4 smem6[];
+        q6k_small_body<T, XF32>(w3, xg, y3, n3, spr, bx - wg_b3, (int)gridDim.x - wg_b3, q6_teams, smem6);
+        return;
+    }
     const int g = (bx >= wg_b1 ? 1 : 0) + (bx >= wg_b2 ? 1 : 0) + (bx >= wg_b3 ? 1 : 0);
     const uint8_t *__restrict__ W = g == 0 ? w0 : g == 1 ? w1 : g == 2 ? w2 : w3;
     float *__restrict__ y = g == 0 ? y0 : g == 1 ? y1 : g == 2 ? y2 : y3;
@@ -669,18 +676,87 @@ hipError_t launch_chunk(int T, bool single, dim3 grid, dim3 block, size_t lds, h
 
 template <int ORDER, bool XF32>
 hipError_t launch_general(int T, dim3 grid, dim3 block, size_t lds, hipStream_t s, const GemvGroup &grp, const void *x,
-                          int spr, int rows_per_wg, int per_team) {
+                          int spr, int rows_per_wg, int per_team, int q6_teams = 0) {
     auto go = [&](auto kern) {
         return launch_with_lds(kern, grid, block, lds, s, x, grp.w[0], grp.w[1], grp.w[2], grp.w[3], grp.wg_begin[1],
                                grp.wg_begin[2], grp.wg_begin[3], spr, rows_per_wg, per_team, grp.n[0], grp.n[1], grp.n[2],
-                               grp.n[3], grp.y[0], grp.y[1], grp.y[2], grp.y[3], (int)block.x);
+                               grp.n[3], grp.y[0], grp.y[1], grp.y[2], grp.y[3], (int)block.x, q6_teams);
     };
-    switch (T) {
-    case 8: return go(k_qgemv_q4k<ORDER, XF32, 8>);
-    case 16: return go(k_qgemv_q4k<ORDER, XF32, 16>);
-    case 32: return go(k_qgemv_q4k<ORDER, XF32, 32>);
-    default: return go(k_qgemv_q4k<ORDER, XF32, 64>);
+    if (q6_teams > 0) {
+        switch (T) {
+        case 8: return go(k_qgemv_q4k<ORDER, XF32, 8, true>);
+        case 16: return go(k_qgemv_q4k<ORDER, XF32, 16, true>);
+        case 32: return go(k_qgemv_q4k<ORDER, XF32, 32, true>);
+        default: return go(k_qgemv_q4k<ORDER, XF32, 64, true>);
+        }
     }
+    switch (T) {
+    case 8: return go(k_qgemv_q4k<ORDER, XF32, 8, false>);
+    case 16: return go(k_qgemv_q4k<ORDER, XF32, 16, false>);
+    case 32: return go(k_qgemv_q4k<ORDER, XF32, 32, false>);
+    default: return go(k_qgemv_q4k<ORDER, XF32, 64, false>);
+    }
+}
+
+// One to three small Q4_K matrices and one small Q6_K matrix that share k and x in one launch of kernel B: the workgroups
+// are divided between the two kinds by their bytes.
+hipError_t launch_group_mixed(const uint8_t *const *w, const int64_t *n, float *const *y, int count, const uint8_t *w6, int64_t n6,
+                              float *y6, int64_t k, const void *x, bool xf32, uint32_t order, hipStream_t s) {
+    const int spr = (int)(k / 256);
+    const int T = 8 * pow2_divisor(spr, 8);
+    const size_t slots = (size_t)spr * 8;
+    const size_t lds4 = slots * 16 * (xf32 ? 6 : 5) + slots * 16, lds6 = slots * 64 * (xf32 ? 3 : 1) + slots * 16;
+    const size_t lds = lds4 > lds6 ? lds4 : lds6;
+    if (lds > kMaxLds || count < 1 || count > pmh::kMaxGemvGroup - 1) return hipErrorNotSupported;
+    int64_t total = 0;
+    for (int i = 0; i < count; i++) total += n[i];
+    const int64_t cus = compute_units();
+    if (total + n6 < 2 * cus) return hipErrorNotSupported;  // too small to divide
+    // a Q6_K byte costs more instructions than a Q4_K byte: its share is weighted by 1.3 (measured flat from 1.15 to 1.8)
+    const double b4 = (double)total * spr * 144.0, b6 = (double)n6 * spr * 210.0 * 1.3;
+    int64_t wgs6 = (int64_t)((double)cus * b6 / (b4 + b6) + 0.5);
+    wgs6 = wgs6 < 1 ? 1 : (wgs6 > cus - count ? cus - count : wgs6);
+    const int64_t wgs4 = cus - wgs6;
+    int64_t rows_per_wg = (total + wgs4 - 1) / wgs4;
+    for (;;) {
+        int64_t c = 0;
+        for (int i = 0; i < count; i++) c += (n[i] + rows_per_wg - 1) / rows_per_wg;
+        if (c <= wgs4 || rows_per_wg >= total) break;
+        rows_per_wg++;
+    }
+    GemvGroup grp{};
+    int begin = 0;
+    for (int i = 0; i < pmh::kMaxGemvGroup - 1; i++) {
+        grp.wg_begin[i] = begin;
+        if (i < count) {
+            grp.w[i] = w[i], grp.y[i] = y[i], grp.n[i] = (int)n[i];
+            begin += (int)((n[i] + rows_per_wg - 1) / rows_per_wg);
+        } else {
+            grp.w[i] = w[0], grp.y[i] = y[0], grp.n[i] = 0;
+        }
+    }
+    grp.wg_begin[3] = begin;  // the Q6_K member starts here
+    grp.w[3] = w6, grp.y[3] = y6, grp.n[3] = (int)n6;
+    const dim3 grid((unsigned)(begin + wgs6));
+    const int teams_per_wave = 64 / T;
+    const int64_t rows6 = (n6 + wgs6 - 1) / wgs6;                 // rows of a Q6_K workgroup: two per team at a time
+    int64_t q6_teams = (rows6 + 1) / 2;
+    int best_waves = 16;
+    int64_t best_cost = INT64_MAX;
+    for (int waves = 16; waves >= 1; waves--) {  // as in launch_group_general
+        const int64_t teams = (int64_t)waves * teams_per_wave;
+        const int64_t per_team = (rows_per_wg + teams - 1) / teams;
+        if (per_team < best_cost) best_cost = per_team, best_waves = waves;
+    }
+    const int64_t teams_avail = (int64_t)best_waves * teams_per_wave;
+    q6_teams = q6_teams < 1 ? 1 : (q6_teams > teams_avail ? teams_avail : q6_teams);
+    const int per_team = (int)((rows_per_wg + teams_avail - 1) / teams_avail);
+    const dim3 block((unsigned)best_waves * 64);
+    if (order == pmh::kOrderRef)
+        return xf32 ? launch_general<0, true>(T, grid, block, lds, s, grp, x, spr, (int)rows_per_wg, per_team, (int)q6_teams)
+                    : launch_general<0, false>(T, grid, block, lds, s, grp, x, spr, (int)rows_per_wg, per_team, (int)q6_teams);
+    return xf32 ? launch_general<1, true>(T, grid, block, lds, s, grp, x, spr, (int)rows_per_wg, per_team, (int)q6_teams)
+                : launch_general<1, false>(T, grid, block, lds, s, grp, x, spr, (int)rows_per_wg, per_team, (int)q6_teams);
 }
 
 // Kernel B over a group of matrices: up to 16 waves; the wave count is the largest that keeps the busiest
@@ -880,6 +956,16 @@ hipError_t launch_qgemv_q4k_pair(const uint8_t *w0, int64_t n0, float *y0, const
 
 // Matrices that kernel A would not take anyway (small ones), sharing k, x, x_dtype and order, in one launch.
 bool qgemv_q4k_groupable(int64_t n, int64_t k) { return (uint64_t)n * (uint64_t)(k / 256) * 144u < (12ull << 20); }
+
+// A group of small Q4_K matrices followed by one small Q6_K matrix over the same activations (q, k and a Q6_K v): one
+// launch.  hipErrorNotSupported when the shapes do not suit it; the caller launches the two kinds one after the other.
+hipError_t launch_qgemv_q4k_q6k_group(const uint8_t *const *w, const int64_t *n, float *const *y, int count, const uint8_t *w6, int64_t n6,
+                                      float *y6, int64_t k, const void *x, uint32_t x_dtype, uint32_t order, hipStream_t s) {
+    uint64_t bytes = (uint64_t)n6 * (uint64_t)(k / 256) * 210u;
+    for (int i = 0; i < count; i++) bytes += (uint64_t)n[i] * (uint64_t)(k / 256) * 144u;
+    if (bytes >= (8ull << 20)) return hipErrorNotSupported;  // large groups stream through the row-owner kernels
+    return launch_group_mixed(w, n, y, count, w6, n6, y6, k, x, x_dtype == kDtypeF32, order, s);
+}
 
 hipError_t launch_qgemv_q4k_group(const uint8_t *const *w, const int64_t *n, float *const *y, int count, int64_t k,
                                   const void *x, uint32_t x_dtype, uint32_t order, hipStream_t s) {

@@ -53,6 +53,8 @@ hipError_t launch_qgemv_q4k_pair(const uint8_t *w0, int64_t n0, float *y0, const
                                  const void *x, uint32_t x_dtype, uint32_t order, hipStream_t s);
 // qgemv_q4k_groupable tells whether a matrix is small enough to go into a group.
 bool qgemv_q4k_groupable(int64_t n, int64_t k);
+hipError_t launch_qgemv_q4k_q6k_group(const uint8_t *const *w, const int64_t *n, float *const *y, int count, const uint8_t *w6, int64_t n6,
+                                      float *y6, int64_t k, const void *x, uint32_t x_dtype, uint32_t order, hipStream_t s);
 hipError_t launch_qgemv_q4k_group(const uint8_t *const *w, const int64_t *n, float *const *y, int count, int64_t k,
                                   const void *x, uint32_t x_dtype, uint32_t order, hipStream_t s);
 

@@ -300,6 +300,47 @@ def test_qgemv_batch_groups_that_are_large_as_a_whole(oracle, order, k, x_dtype)
         assert np.abs(got - single).max() <= 2e-6 * np.abs(single).max()
 
 
+@pytest.mark.parametrize("k,x_dtype", [(1024, pm.DTYPE_BF16), (2048, pm.DTYPE_F32), (768, pm.DTYPE_BF16)])
+@pytest.mark.parametrize("rows", [[2048, 1024, 1024], [517, 300], [1024, 1000, 37, 96], [2048, 1024, 1024, 1024]])
+@pytest.mark.parametrize("order", [0, 1])
+def test_qgemv_batch_takes_a_q6k_projection_into_a_q4k_group(oracle, order, rows, k, x_dtype):
+    """q and k in Q4_K followed by v in Q6_K over the same x (a Q4_K_M layer): one launch.  The last of `rows` is the
+    Q6_K matrix; every member against the oracle and against its own launch.  With four Q4_K members before it the
+    Q6_K matrix does not fit the group and runs on its own."""
+    from pmetal_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(k + order + len(rows))
+    xa, xa_ref = activations(oracle, 9, k, x_dtype)
+    dx = pm.DeviceBuffer.from_host(xa)
+    if len(rows) == 4 and rows[0] == 2048:
+        rows = rows + [600]
+    descs = (_lib.LinearDesc * len(rows))()
+    keep = []
+    for i, n in enumerate(rows):
+        t = Q6K if i == len(rows) - 1 else Q4K
+        bs = 210 if t == Q6K else 144
+        raw = rng.integers(0, 256, size=(n * (k // 256), bs), dtype=np.uint8)
+        half = np.frombuffer(np.array([0.01, 0.02], np.float16).tobytes(), np.uint8)
+        if t == Q6K:
+            raw[:, 208:210] = half[:2]
+        else:
+            raw[:, 0:4] = half
+        raw = raw.reshape(-1)
+        dw, dy = pm.DeviceBuffer.from_host(raw), pm.DeviceBuffer(4 * n)
+        pm.check(lib.pmetal_hip_memset(dy.ptr, 0xFF, 4 * n, None))
+        keep.append((t, dw, dy, raw, n))
+        descs[i] = _lib.LinearDesc(t, x_dtype, order, 0, n, k, dw.ptr, dx.ptr, dy.ptr)
+    pm.check(lib.pmetal_hip_qgemv_batch(descs, len(rows), None))
+    pm.check(lib.pmetal_hip_sync(None))
+    for t, dw, dy, raw, n in keep:
+        got = dy.to_host(np.float32)
+        want = oracle.qmatvec(t, raw, n, k, xa_ref, order=order)
+        elem, norm = rel_errors(got, want)
+        assert elem <= TOL and norm <= TOL, (t, n, elem, norm)
+        single = gpu_qgemv(t, raw, n, k, xa, x_dtype, order)
+        assert np.abs(got - single).max() <= 2e-6 * np.abs(single).max()
+
+
 @pytest.mark.parametrize("order", [0, 1])
 def test_qgemv_batch_pairs_large_projections_of_one_activation(oracle, order):
     """Two consecutive large Q4_K matrices that share x (gate / up) go through one launch of the large-matrix kernel:
