@@ -1104,6 +1104,35 @@ __global__ __launch_bounds__(256) void k_rw_reduce(const float *__restrict__ par
     }
 }
 
+// The same over eight consecutive outputs of one row per thread (N a multiple of 8): 16-byte loads and stores.
+template <bool YBF16>
+__global__ __launch_bounds__(256) void k_rw_reduce8(const float *__restrict__ partial, int splits, int M, int Mp, int N,
+                                                     const float *__restrict__ rowscale, void *__restrict__ yg) {
+    const size_t idx = ((size_t)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (idx >= (size_t)M * N) return;
+    const int m = (int)(idx / N);
+    const size_t plane = (size_t)Mp * N;
+    const float4 *p = reinterpret_cast<const float4 *>(partial + idx);
+    float4 a = p[0], b = p[1];
+    for (int z = 1; z < splits; z++) {
+        const float4 *q = reinterpret_cast<const float4 *>(partial + (size_t)z * plane + idx);
+        const float4 c = q[0], d = q[1];
+        a.x += c.x, a.y += c.y, a.z += c.z, a.w += c.w;
+        b.x += d.x, b.y += d.y, b.z += d.z, b.w += d.w;
+    }
+    const float sc = rowscale[m];
+    const float v[8] = {a.x * sc, a.y * sc, a.z * sc, a.w * sc, b.x * sc, b.y * sc, b.z * sc, b.w * sc};
+    if (YBF16) {
+        *reinterpret_cast<uint4 *>(reinterpret_cast<uint16_t *>(yg) + idx) =
+            make_uint4(bf16_rne_bits(v[0]) | (bf16_rne_bits(v[1]) << 16), bf16_rne_bits(v[2]) | (bf16_rne_bits(v[3]) << 16),
+                       bf16_rne_bits(v[4]) | (bf16_rne_bits(v[5]) << 16), bf16_rne_bits(v[6]) | (bf16_rne_bits(v[7]) << 16));
+    } else {
+        float4 *o = reinterpret_cast<float4 *>(reinterpret_cast<float *>(yg) + idx);
+        o[0] = make_float4(v[0], v[1], v[2], v[3]);
+        o[1] = make_float4(v[4], v[5], v[6], v[7]);
+    }
+}
+
 template <int MB, int NR, int NW>
 constexpr size_t rw_lds_bytes() {
     const size_t stages = (size_t)(2 * kGroups * 32 * MB + NW * NR * (3 * 128 + 64)) * 16;
@@ -1302,6 +1331,12 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
 #undef PMH_RW_CASE
     if (e != hipSuccess || p.splits == 1) return e;
     const size_t total = (size_t)m * n;
+    if (n % 8 == 0) {
+        const dim3 grid8((unsigned)((total / 8 + 255) / 256));
+        if (ybf) hipLaunchKernelGGL(k_rw_reduce8<true>, grid8, dim3(256), 0, s, partial, p.splits, (int)m, (int)p.mp, (int)n, rowscale, y);
+        else hipLaunchKernelGGL(k_rw_reduce8<false>, grid8, dim3(256), 0, s, partial, p.splits, (int)m, (int)p.mp, (int)n, rowscale, y);
+        return hipGetLastError();
+    }
     const dim3 rgrid((unsigned)((total + 255) / 256));
     if (ybf) hipLaunchKernelGGL(k_rw_reduce<true>, rgrid, dim3(256), 0, s, partial, p.splits, (int)m, (int)p.mp, (int)n, rowscale, y);
     else hipLaunchKernelGGL(k_rw_reduce<false>, rgrid, dim3(256), 0, s, partial, p.splits, (int)m, (int)p.mp, (int)n, rowscale, y);
