@@ -1167,7 +1167,9 @@ bool qgemm_fits(uint32_t type, int64_t m, int64_t n, int64_t k) {
 
 GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k) {
     GemmPlan p;
-    p.mb = m <= 32 ? 1 : (m <= 64 ? 2 : 4);  // 32, 64 or 128 activation rows per workgroup
+    // 32, 64 or 128 activation rows per workgroup; up to 128 rows two 64-row blocks beat one 128-row block (half the
+    // K splits for the same number of workgroups: 36.9 against 38.3 us at 14336x4096)
+    p.mb = m <= 32 ? 1 : (m <= 128 ? 2 : 4);
     p.mp = (m + 32 * p.mb - 1) / (32 * p.mb) * (32 * p.mb);
     p.nw = 8;
     const int64_t spr = k / 256;
