@@ -1167,9 +1167,10 @@ bool qgemm_fits(uint32_t type, int64_t m, int64_t n, int64_t k) {
 
 GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k) {
     GemmPlan p;
-    // 32, 64 or 128 activation rows per workgroup; up to 128 rows two 64-row blocks beat one 128-row block (half the
-    // K splits for the same number of workgroups: 36.9 against 38.3 us at 14336x4096)
-    p.mb = m <= 32 ? 1 : (m <= 128 ? 2 : 4);
+    // 32, 64 or 128 activation rows per workgroup; up to 192 rows 64-row blocks beat 128-row blocks (fewer K splits
+    // for the same number of workgroups: 36.9 against 38.3 us at M = 128, 51.7 against 53.8 at M = 192, 14336x4096;
+    // equal at 256, and from 320 rows on the larger block wins)
+    p.mb = m <= 32 ? 1 : (m <= 192 ? 2 : 4);
     p.mp = (m + 32 * p.mb - 1) / (32 * p.mb) * (32 * p.mb);
     p.nw = 8;
     const int64_t spr = k / 256;

@@ -73,7 +73,7 @@ def test_qgemm_bf16_output_and_large_activations(oracle):
 
 
 @pytest.mark.parametrize("t", [Q4K, Q6K, Q8_0])
-@pytest.mark.parametrize("m", [24, 200, 300])
+@pytest.mark.parametrize("m", [24, 150, 192, 200, 300])
 def test_qgemm_f32_activations(oracle, t, m):
     """f32 activations are rounded once to f16 at the row's power-of-two scale (11 significant bits; a bf16 cast
     would keep 8): against the unrounded reference the result holds the 1e-3 bound norm-wise, and element-wise
