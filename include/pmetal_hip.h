@@ -128,8 +128,8 @@ int32_t pmetal_hip_event_destroy(void *event);
  * Output bytes are bit-identical to the reference CPU path.  dst_len must equal
  * pmetal_hip_tensor_size(type, n).  A trailing partial 256-super-block is emitted as
  * zero bytes (k_quants.rs:890-892); Q8_0 zero-pads inside its last block.
- * The host variants (here and of dequantize) are synchronous; tensors of 8 Mi elements
- * or more stream through pinned staging buffers that the library keeps (3 x 37 MiB of
+ * The host variants (here and of dequantize) are synchronous; tensors of 256 Ki elements
+ * or more stream through pinned staging buffers that the library keeps (3 x 21 MiB of
  * pinned host and of device memory per device, made on first use), and such calls take
  * turns across threads.                                                                */
 int32_t pmetal_hip_quantize(uint32_t ggml_type, const float *src_host, size_t n, uint8_t *dst_host,

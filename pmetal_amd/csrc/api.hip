@@ -207,13 +207,15 @@ int32_t scratch_of_current_device(void **out) {
 }
 
 // ---- host-to-host codec calls on large tensors ----
-// A tensor in pageable host memory goes through chunks of kPipeElems elements: a few host threads copy a chunk into a
+// A tensor of at least kPipeMinElems elements in pageable host memory goes through chunks (a quarter of the tensor, at
+// most kPipeElems elements; smaller tensors take one allocate-copy-run-copy round): a few host threads copy a chunk into a
 // pinned staging buffer, a copy engine moves it, the kernel runs, and the result comes back the same way, each chunk on
 // the stream of its slot, so that the host copies, both transfer directions and the kernels of neighbouring chunks
 // overlap.  The slots (pinned and device buffers, streams, events) are made on first use, per device, and kept until
 // the process ends; calls take turns (one mutex).
 constexpr size_t kPipeElems = (size_t)4 << 20;  // 16 MiB of f32; a multiple of every block size
 constexpr size_t kPipeQBytes = kPipeElems / 256 * 292;  // the largest encoded chunk (Q8_K)
+constexpr size_t kPipeGrain = 8192, kPipeMinElems = (size_t)256 << 10;  // chunks are multiples of the grain, at least 1 MiB of f32
 constexpr int kPipeSlots = 3, kCopyThreads = 4;  // measured: 26 / 38 / 41 / 41 GB/s with 1 / 2 / 4 / 8 copy threads
 
 struct PipeSlot {
@@ -523,7 +525,7 @@ int32_t pmetal_hip_quantize(uint32_t t, const float *src, size_t n, uint8_t *dst
     if (n == 0) return ok();
     if (!src || !dst) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
     if (int32_t rc = require_device()) return rc;
-    if (n >= 2 * kPipeElems) return codec_pipelined(true, t, const_cast<float *>(src), dst, n, 0);
+    if (n >= kPipeMinElems) return codec_pipelined(true, t, const_cast<float *>(src), dst, n, 0);
     DevBuf din, dout;
     HIP_TRY(hipMalloc(&din.p, n * sizeof(float)));
     HIP_TRY(hipMalloc(&dout.p, expected));
@@ -574,7 +576,7 @@ int32_t pmetal_hip_dequantize(uint32_t t, const uint8_t *src, size_t src_len, co
     if (n == 0) return ok();
     if (!src || !dst) return fail(PMETAL_HIP_ERR_INVALID_ARG, "NULL pointer");
     if (int32_t rc = require_device()) return rc;
-    if (n >= 2 * kPipeElems) return codec_pipelined(false, t, dst, const_cast<uint8_t *>(src), n, order);
+    if (n >= kPipeMinElems) return codec_pipelined(false, t, dst, const_cast<uint8_t *>(src), n, order);
     DevBuf din, dout;
     HIP_TRY(hipMalloc(&din.p, expected));
     HIP_TRY(hipMalloc(&dout.p, n * sizeof(float)));
@@ -592,21 +594,24 @@ int32_t codec_pipelined(bool quantize, uint32_t t, float *plain, uint8_t *packed
     std::lock_guard<std::mutex> lock(g_pipe_mutex);
     HostPipe *p = nullptr;
     if (int32_t rc = host_pipe(&p)) return rc;
-    const size_t chunks = (n + kPipeElems - 1) / kPipeElems, q_chunk = pmetal_hip_tensor_size(t, kPipeElems);
-    auto elems_of = [&](size_t i) { return i + 1 < chunks ? kPipeElems : n - i * kPipeElems; };
+    // chunk: a quarter of the tensor (so that the stages of neighbouring chunks overlap), at most what a slot holds
+    size_t chunk = ((n / 4 + kPipeGrain - 1) / kPipeGrain) * kPipeGrain;
+    chunk = chunk < kPipeMinElems ? kPipeMinElems : (chunk > kPipeElems ? kPipeElems : chunk);
+    const size_t chunks = (n + chunk - 1) / chunk, q_chunk = pmetal_hip_tensor_size(t, chunk);
+    auto elems_of = [&](size_t i) { return i + 1 < chunks ? chunk : n - i * chunk; };
     int32_t rc = PMETAL_HIP_OK;
     auto retire = [&](size_t i) -> int32_t {  // chunk i's result: staging buffer -> caller's memory
         PipeSlot &sl = p->slot[i % kPipeSlots];
         HIP_TRY(hipEventSynchronize(sl.done));
         if (quantize) par_copy(packed + i * q_chunk, sl.h_q, pmetal_hip_tensor_size(t, elems_of(i)));
-        else par_copy(plain + i * kPipeElems, sl.h_f32, elems_of(i) * sizeof(float));
+        else par_copy(plain + i * chunk, sl.h_f32, elems_of(i) * sizeof(float));
         return PMETAL_HIP_OK;
     };
     auto submit = [&](size_t i) -> int32_t {
         PipeSlot &sl = p->slot[i % kPipeSlots];
         const size_t elems = elems_of(i), qb = pmetal_hip_tensor_size(t, elems);
         if (quantize) {
-            par_copy(sl.h_f32, plain + i * kPipeElems, elems * sizeof(float));
+            par_copy(sl.h_f32, plain + i * chunk, elems * sizeof(float));
             HIP_TRY(hipMemcpyAsync(sl.d_f32, sl.h_f32, elems * sizeof(float), hipMemcpyHostToDevice, sl.st));
             if (int32_t r = pmetal_hip_quantize_dev(t, sl.d_f32, elems, sl.d_q, qb, sl.st)) return r;
             HIP_TRY(hipMemcpyAsync(sl.h_q, sl.d_q, qb, hipMemcpyDeviceToHost, sl.st));

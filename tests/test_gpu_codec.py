@@ -75,18 +75,19 @@ def test_quantize_host_pointer_entry_point(oracle, t):
     assert np.array_equal(pm.quantize(x, t), oracle.quantize(t, x))
 
 
+@pytest.mark.parametrize("n", [11_000_000 + 123, 20_000_000 + 7, 1_500_000 + 31, 262_144])
 @pytest.mark.parametrize("t", [Q8_0, Q4K, Q6K, 13, 11, 10, 15])
-def test_host_pointer_entry_points_on_a_tensor_of_several_staging_chunks(oracle, t):
-    """Large host tensors go through pinned staging chunks of 4 Mi elements.  11 M elements with a ragged tail: the bytes
-    equal those of the one-launch device path, and the super-blocks on both sides of every chunk boundary, the first and
-    the last ones equal the oracle's; the same for the way back."""
-    n = 11_000_000 + 123
+def test_host_pointer_entry_points_on_a_tensor_of_several_staging_chunks(oracle, t, n):
+    """Host tensors of 256 Ki elements or more go through pinned staging chunks (a quarter of the tensor rounded up to
+    8192 elements, between 256 Ki and 4 Mi elements).  Ragged tails: the bytes equal those of the one-launch device
+    path, and the super-blocks on both sides of chunk boundaries, the first and the last ones equal the oracle's; the
+    same for the way back."""
     x = weights(500 + t, n)
     got = pm.quantize(x, t)
     assert np.array_equal(got, gpu_quantize_dev(t, x))
     bs, ts = (32, 34) if t == Q8_0 else (256, {Q4K: 144, Q6K: 210, 13: 176, 11: 110, 10: 84, 15: 292}[t])
-    chunk = 4 << 20
-    spots = [0, chunk - 2 * bs, 2 * chunk - 2 * bs, (n // bs - 3) * bs]
+    chunk = min(max((n // 4 + 8191) // 8192 * 8192, 256 << 10), 4 << 20)
+    spots = [0] + [c * chunk - 2 * bs for c in (1, 2) if c * chunk + 2 * bs < n] + [(n // bs - 3) * bs]
     for e0 in spots:
         e1 = min(n, e0 + 4 * bs)
         want = oracle.quantize(t, x[e0:e1])
@@ -96,7 +97,7 @@ def test_host_pointer_entry_points_on_a_tensor_of_several_staging_chunks(oracle,
     back = pm.dequantize(whole, t, (n_out,))
     assert back.size == n_out
     assert np.array_equal(back.view(np.uint32), gpu_dequantize_dev(t, whole, n // bs * bs)[:n_out].view(np.uint32))
-    for e0 in spots[:3]:
+    for e0 in spots[:-1]:
         want = oracle.dequantize(t, got[e0 // bs * ts:(e0 // bs + 4) * ts], (4 * bs,))
         assert np.array_equal(back[e0:e0 + 4 * bs].view(np.uint32), want.view(np.uint32)), e0
 
