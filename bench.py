@@ -725,8 +725,12 @@ def main():
     out["extra"]["event_ms_per_step"] = round(res["event_ms_per_step"], 5)
     if wl["kind"] == "gemv":
         # `dtype` names the activation type handed over; the kernels of these (large) shapes multiply in integers
-        out["config"]["arithmetic"] = ("bf16 activations converted exactly to fixed-point int8 digit planes, v_dot4_i32_i8 against "
-                                       "the quantized weights, f32 block scales and accumulation")
+        if "_q4k_" in args.workload:
+            out["config"]["arithmetic"] = ("bf16 activations converted to 20-bit fixed point per 32-element block, five 4-bit digit planes, "
+                                           "v_dot8_u32_u4 against the packed nibbles, f32 block scales and accumulation")
+        else:
+            out["config"]["arithmetic"] = ("bf16 activations converted exactly to fixed-point int8 digit planes, v_dot4_i32_i8 against "
+                                           "the quantized weights, f32 block scales and accumulation")
     rec = RECORDED_TRAFFIC.get(args.workload)
     out["roofline"]["traffic"] = rec[0] if rec else None
     if rec:
