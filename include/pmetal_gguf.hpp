@@ -13,12 +13,15 @@
 //   pmetal_gguf::quantize_model_q4_k_m(...)       the quantize-and-write loop of run_quantization,
 //                                                 crates/pmetal/src/commands/quantize.rs:1339-1433
 //   pmetal_gguf::hf_to_gguf_name                  crates/pmetal-models/src/weight_format.rs:389-435
+//   pmetal_gguf::gguf_to_hf_name, load_gguf       WeightLoader::gguf_to_hf_name / load_gguf,
+//                                                 crates/pmetal-models/src/weight_format.rs:332-386, :258-313
 // A Rust `Result::Err` becomes a thrown exception carrying the library's message.  Everything computes on
 // the GPU; there is no CPU fallback (a missing device throws NoDeviceError).
 #pragma once
 
 #include <cstdint>
 #include <stdexcept>
+#include <map>
 #include <memory>
 #include <string>
 #include <vector>
@@ -333,6 +336,114 @@ inline std::string hf_to_gguf_name(const std::string &hf_name) {
     for (const auto &row : table)
         if (suffix == row.first) mapped = row.second;
     return "blk." + layer + "." + mapped;
+}
+
+// WeightLoader::gguf_to_hf_name (crates/pmetal-models/src/weight_format.rs:332-386): the three top-level tensors, then
+// blk.N.<tensor> -> model.layers.N.<tensor>; N is taken as written (it is not parsed), unknown names pass through.
+inline std::string gguf_to_hf_name(const std::string &gguf_name) {
+    if (gguf_name == "token_embd.weight") return "model.embed_tokens.weight";
+    if (gguf_name == "output_norm.weight") return "model.norm.weight";
+    if (gguf_name == "output.weight") return "lm_head.weight";
+    if (gguf_name.compare(0, 4, "blk.") != 0) return gguf_name;
+    // splitn(3, '.'): "blk", the block number, the rest; fewer than three parts pass through
+    const size_t d1 = gguf_name.find('.', 4);
+    if (d1 == std::string::npos) return gguf_name;
+    const std::string block = gguf_name.substr(4, d1 - 4), rest = gguf_name.substr(d1 + 1);
+    static const std::pair<const char *, const char *> table[] = {
+        {"attn_norm.weight", "input_layernorm.weight"},
+        {"attn_q.weight", "self_attn.q_proj.weight"},
+        {"attn_k.weight", "self_attn.k_proj.weight"},
+        {"attn_v.weight", "self_attn.v_proj.weight"},
+        {"attn_output.weight", "self_attn.o_proj.weight"},
+        {"ffn_norm.weight", "post_attention_layernorm.weight"},
+        {"ffn_gate.weight", "mlp.gate_proj.weight"},
+        {"ffn_up.weight", "mlp.up_proj.weight"},
+        {"ffn_down.weight", "mlp.down_proj.weight"},
+        {"ffn_gate_inp.weight", "mlp.gate.weight"},
+        {"ffn_gate_exps.weight", "mlp.experts.gate_proj.weight"},
+        {"ffn_up_exps.weight", "mlp.experts.up_proj.weight"},
+        {"ffn_down_exps.weight", "mlp.experts.down_proj.weight"},
+        {"ffn_gate_shexp.weight", "mlp.shared_expert.gate_proj.weight"},
+        {"ffn_up_shexp.weight", "mlp.shared_expert.up_proj.weight"},
+        {"ffn_down_shexp.weight", "mlp.shared_expert.down_proj.weight"},
+        {"ffn_gate_inp_shexp.weight", "mlp.shared_expert_gate.weight"},
+        {"attn_q_norm.weight", "self_attn.q_norm.weight"},
+        {"attn_k_norm.weight", "self_attn.k_norm.weight"},
+    };
+    std::string mapped = rest;
+    for (const auto &row : table)
+        if (rest == row.first) mapped = row.second;
+    return "model.layers." + block + "." + mapped;
+}
+
+// dequantize(data, dtype, shape) for every type this build decodes: F32 / F16 / BF16 are conversions on the host
+// (crates/pmetal-gguf/src/dequant.rs:219-258, sizes validated as there), Q8_0 and the k-quants run on the GPU.
+inline bool load_supported(GgmlType dtype) {
+    return dtype == GgmlType::F32 || dtype == GgmlType::F16 || dtype == GgmlType::Bf16 || pmetal_hip_is_supported((uint32_t)dtype) != 0;
+}
+inline std::vector<float> dequantize_any(const uint8_t *data, size_t len, GgmlType dtype, const std::vector<int32_t> &shape) {
+    if (dtype != GgmlType::F32 && dtype != GgmlType::F16 && dtype != GgmlType::Bf16) return dequantize(data, len, dtype, shape);
+    size_t n = 1;
+    for (int32_t d : shape) {
+        if (d < 0) throw DequantError(PMETAL_HIP_ERR_INVALID_SHAPE, "dimensions must be non-negative");
+        if (d != 0 && n > SIZE_MAX / (size_t)d) throw DequantError(PMETAL_HIP_ERR_SHAPE_TOO_LARGE, "shape is too large");
+        n *= (size_t)d;
+    }
+    const size_t width = dtype == GgmlType::F32 ? 4 : 2;
+    if (n > SIZE_MAX / width) throw DequantError(PMETAL_HIP_ERR_SHAPE_TOO_LARGE, "shape is too large");
+    if (len != n * width)
+        throw DequantError(PMETAL_HIP_ERR_INVALID_SIZE,
+                           "Invalid data size: expected " + std::to_string(n * width) + " bytes, got " + std::to_string(len));
+    std::vector<float> out(n);
+    for (size_t i = 0; i < n; i++) {
+        if (dtype == GgmlType::F32) {
+            std::memcpy(&out[i], data + 4 * i, 4);
+        } else {
+            uint16_t h;
+            std::memcpy(&h, data + 2 * i, 2);
+            if (dtype == GgmlType::F16) {
+                out[i] = f16_bits_to_f32(h);
+            } else {
+                const uint32_t u = (uint32_t)h << 16;
+                std::memcpy(&out[i], &u, 4);
+            }
+        }
+    }
+    return out;
+}
+
+// One tensor as WeightLoader::load_gguf returns it: f32 values, row-major, with the shape the file gives.
+struct LoadedTensor {
+    std::vector<int32_t> shape;
+    std::vector<float> data;
+};
+
+// WeightLoader::load_gguf (crates/pmetal-models/src/weight_format.rs:258-313): every tensor of the file whose type can be
+// decoded, dequantized to f32 under its Hugging Face name; tensors of other types are skipped (the reference logs a
+// warning), a dimension beyond i32 is an error (:142-153).  Here "can be decoded" means load_supported(): the plain
+// types and the block types with kernels in this library; `skipped`, when given, receives the names left out.
+inline std::map<std::string, LoadedTensor> load_gguf(const std::string &path, std::vector<std::string> *skipped = nullptr) {
+    const GgufContent content = GgufContent::from_file(path);
+    std::map<std::string, LoadedTensor> weights;
+    for (const std::string &name : content.tensor_order) {
+        const TensorInfo *info = content.get_tensor_info(name);
+        if (!info) throw Error(PMETAL_HIP_ERR_INVALID_ARG, "Tensor not found: " + name);
+        if (!load_supported(info->dtype)) {
+            if (skipped) skipped->push_back(name);
+            continue;
+        }
+        LoadedTensor t;
+        for (uint64_t d : info->dimensions) {
+            if (d > (uint64_t)INT32_MAX)
+                throw Error(PMETAL_HIP_ERR_SHAPE_TOO_LARGE,
+                            "Tensor " + name + " dimension " + std::to_string(d) + " exceeds MLX i32 shape limits");
+            t.shape.push_back((int32_t)d);
+        }
+        const std::vector<uint8_t> raw = content.read_tensor_data_from_file(path, name);
+        t.data = dequantize_any(raw.data(), raw.size(), info->dtype, t.shape);
+        weights[gguf_to_hf_name(name)] = std::move(t);
+    }
+    return weights;
 }
 
 // One f32 tensor of the model to quantize: its Hugging Face name, row-major shape and values (not owned).

@@ -228,6 +228,27 @@ inline uint16_t f32_to_f16_bits(float f) {
     return (uint16_t)(sign | out);
 }
 
+// half::f16::to_f32 on the host: exact (every f16 value, subnormals included, is an f32 value; NaN keeps its payload).
+inline float f16_bits_to_f32(uint16_t h) {
+    const uint32_t sign = ((uint32_t)h & 0x8000u) << 16, exp = (h >> 10) & 0x1Fu, man = h & 0x3FFu;
+    uint32_t x;
+    if (exp == 0x1F) {
+        x = sign | 0x7F800000u | (man << 13);
+    } else if (exp != 0) {
+        x = sign | ((exp + 112u) << 23) | (man << 13);
+    } else if (man == 0) {
+        x = sign;
+    } else {  // subnormal half: man * 2^-24, normalised
+        int shift = 0;
+        uint32_t m = man;
+        while (!(m & 0x400u)) m <<= 1, shift++;
+        x = sign | ((uint32_t)(113 - shift) << 23) | ((m & 0x3FFu) << 13);
+    }
+    float f;
+    std::memcpy(&f, &x, 4);
+    return f;
+}
+
 // align_offset (writer.rs:609-611, test helper in the reference)
 inline uint64_t align_offset(uint64_t offset, uint64_t alignment) {
     uint64_t out;

@@ -354,3 +354,48 @@ def hf_to_gguf_name(hf_name: str) -> str:
     if not digits or not all("0" <= ch <= "9" for ch in digits) or int(digits) >= 1 << 64:
         return hf_name
     return f"blk.{layer}.{_HF_SUFFIX.get(suffix, suffix)}"
+
+
+# crates/pmetal-models/src/weight_format.rs:332-386
+_GGUF_SUFFIX = {
+    "attn_norm.weight": "input_layernorm.weight", "attn_q.weight": "self_attn.q_proj.weight",
+    "attn_k.weight": "self_attn.k_proj.weight", "attn_v.weight": "self_attn.v_proj.weight",
+    "attn_output.weight": "self_attn.o_proj.weight", "ffn_norm.weight": "post_attention_layernorm.weight",
+    "ffn_gate.weight": "mlp.gate_proj.weight", "ffn_up.weight": "mlp.up_proj.weight", "ffn_down.weight": "mlp.down_proj.weight",
+    "ffn_gate_inp.weight": "mlp.gate.weight", "ffn_gate_exps.weight": "mlp.experts.gate_proj.weight",
+    "ffn_up_exps.weight": "mlp.experts.up_proj.weight", "ffn_down_exps.weight": "mlp.experts.down_proj.weight",
+    "ffn_gate_shexp.weight": "mlp.shared_expert.gate_proj.weight", "ffn_up_shexp.weight": "mlp.shared_expert.up_proj.weight",
+    "ffn_down_shexp.weight": "mlp.shared_expert.down_proj.weight", "ffn_gate_inp_shexp.weight": "mlp.shared_expert_gate.weight",
+    "attn_q_norm.weight": "self_attn.q_norm.weight", "attn_k_norm.weight": "self_attn.k_norm.weight",
+}
+
+
+def gguf_to_hf_name(gguf_name: str) -> str:
+    top = {"token_embd.weight": "model.embed_tokens.weight", "output_norm.weight": "model.norm.weight",
+           "output.weight": "lm_head.weight"}
+    if gguf_name in top:
+        return top[gguf_name]
+    if gguf_name.startswith("blk."):
+        parts = gguf_name.split(".", 2)  # splitn(3, '.')
+        if len(parts) >= 3:
+            return f"model.layers.{parts[1]}.{_GGUF_SUFFIX.get(parts[2], parts[2])}"
+    return gguf_name
+
+
+def load_gguf(data: bytes, dequantize, supported):
+    """WeightLoader::load_gguf (weight_format.rs:258-313) over a file image: {hugging face name: (shape, f32 values)} of
+    every tensor whose type ``supported(dtype)`` accepts, decoded by ``dequantize(raw bytes, dtype, shape)``; a dimension
+    beyond i32 is an error (:142-153).  Returns the dict and the names skipped."""
+    content = GgufContent.read(data)
+    weights, skipped = {}, []
+    for name in content.tensor_order:
+        info = content.tensor_infos[name]
+        if not supported(info["dtype"]):
+            skipped.append(name)
+            continue
+        for d in info["dimensions"]:
+            if d > 2**31 - 1:
+                raise ValueError(f"Tensor {name} dimension {d} exceeds MLX i32 shape limits")
+        shape = list(info["dimensions"])
+        weights[gguf_to_hf_name(name)] = (shape, dequantize(content.read_tensor_data(data, name), info["dtype"], shape))
+    return weights, skipped

@@ -8,6 +8,9 @@
 //   test_gguf_file --read-error IN              print the kind of GgufReadError reading IN raises ("none" if none)
 //   test_gguf_file --f16 IN OUT                 raw f32 values -> raw f16 bit patterns (f32_to_f16_bits)
 //   test_gguf_file --quantize-model SPEC OUT    (GPU) synthetic f32 model -> quantize_model_q4_k_m -> OUT
+//   test_gguf_file --f16-to-f32 IN OUT          raw f16 bit patterns -> raw f32 values (f16_bits_to_f32)
+//   test_gguf_file --load-model IN OUT          (GPU) load_gguf: tensor names and shapes to stdout, f32 values to OUT
+//   test_gguf_file --names IN                   (GPU build) gguf_to_hf_name and hf_to_gguf_name of every hex-encoded name in IN
 //
 // Spec grammar (whitespace-separated tokens; strings are hex-encoded so that they may hold anything):
 //   align N | meta KEYHEX VALUE | tensor NAMEHEX DTYPE NDIMS DIM... SEED
@@ -272,6 +275,22 @@ static int cmd_quantize_model(const std::string &spec, const std::string &out) {
                 b.num_tensors(), f32_bytes / 1e9, q, f32_bytes / 1e9 / q, w);
     return 0;
 }
+
+// load_gguf: per tensor, in the order of the Hugging Face names, a line `hexname ndim dims... dtype-independent count`;
+// the f32 values of all tensors follow each other in OUT in the same order.
+static int cmd_load_model(const std::string &file, const std::string &out) {
+    std::vector<std::string> skipped;
+    const auto weights = load_gguf(file, &skipped);
+    std::ofstream o(out, std::ios::binary);
+    for (const auto &kv : weights) {
+        std::printf("%s %zu", hex(kv.first).c_str(), kv.second.shape.size());
+        for (int32_t d : kv.second.shape) std::printf(" %d", d);
+        std::printf(" %zu\n", kv.second.data.size());
+        o.write(reinterpret_cast<const char *>(kv.second.data.data()), (std::streamsize)(kv.second.data.size() * 4));
+    }
+    for (const std::string &s : skipped) std::printf("skipped %s\n", hex(s).c_str());
+    return 0;
+}
 #endif
 
 static void put32(std::vector<uint8_t> &b, uint32_t v) { detail::put_le<uint32_t>(b, v); }
@@ -410,8 +429,29 @@ int main(int argc, char **argv) {
             std::ofstream(argv[3], std::ios::binary).write(reinterpret_cast<const char *>(out.data()), (std::streamsize)(out.size() * 2));
             return 0;
         }
+        if (cmd == "--f16-to-f32" && argc == 4) {
+            const std::vector<uint8_t> in = slurp(argv[2]);
+            std::vector<float> out(in.size() / 2);
+            for (size_t i = 0; i < out.size(); i++) {
+                uint16_t h;
+                std::memcpy(&h, in.data() + 2 * i, 2);
+                out[i] = f16_bits_to_f32(h);
+            }
+            std::ofstream(argv[3], std::ios::binary).write(reinterpret_cast<const char *>(out.data()), (std::streamsize)(out.size() * 4));
+            return 0;
+        }
 #ifndef PMETAL_TEST_HOST_ONLY
         if (cmd == "--quantize-model" && argc == 4) return cmd_quantize_model(argv[2], argv[3]);
+        if (cmd == "--load-model" && argc == 4) return cmd_load_model(argv[2], argv[3]);
+        if (cmd == "--names" && argc == 3) {  // one hex-encoded name per line: both mappings of it
+            std::ifstream in(argv[2]);
+            std::string word;
+            while (in >> word) {
+                const std::string name = unhex(word);
+                std::printf("%s %s\n", hex(gguf_to_hf_name(name)).c_str(), hex(hf_to_gguf_name(name)).c_str());
+            }
+            return 0;
+        }
 #endif
     } catch (const std::exception &e) {
         std::printf("exception: %s\n", e.what());

@@ -354,6 +354,55 @@ def test_hf_to_gguf_name_examples():
     assert f("visual.blocks.0.attn.qkv.weight") == "visual.blocks.0.attn.qkv.weight"
 
 
+def test_gguf_to_hf_name_reference_examples():
+    """The reference's own examples, weight_format.rs:668-786, and the pass-through cases its code implies."""
+    f = og.gguf_to_hf_name
+    assert f("token_embd.weight") == "model.embed_tokens.weight"
+    assert f("output_norm.weight") == "model.norm.weight"
+    assert f("output.weight") == "lm_head.weight"
+    assert f("blk.0.attn_q.weight") == "model.layers.0.self_attn.q_proj.weight"
+    assert f("blk.15.attn_k.weight") == "model.layers.15.self_attn.k_proj.weight"
+    assert f("blk.7.attn_v.weight") == "model.layers.7.self_attn.v_proj.weight"
+    assert f("blk.0.attn_output.weight") == "model.layers.0.self_attn.o_proj.weight"
+    assert f("blk.0.ffn_gate.weight") == "model.layers.0.mlp.gate_proj.weight"
+    assert f("blk.0.ffn_up.weight") == "model.layers.0.mlp.up_proj.weight"
+    assert f("blk.0.ffn_down.weight") == "model.layers.0.mlp.down_proj.weight"
+    assert f("blk.0.attn_norm.weight") == "model.layers.0.input_layernorm.weight"
+    assert f("blk.0.ffn_norm.weight") == "model.layers.0.post_attention_layernorm.weight"
+    assert f("blk.0.attn_q_norm.weight") == "model.layers.0.self_attn.q_norm.weight"
+    assert f("blk.0.attn_k_norm.weight") == "model.layers.0.self_attn.k_norm.weight"
+    for name in ROUND_TRIP_NAMES:  # test_hf_to_gguf_name_round_trip_core_tensors
+        assert f(og.hf_to_gguf_name(name)) == name
+    assert og.hf_to_gguf_name("model.layers.0.mlp.gate.weight") == "blk.0.ffn_gate_inp.weight"  # test_hf_to_gguf_name_moe_tensors
+    assert og.hf_to_gguf_name("model.layers.0.mlp.experts.gate_proj.weight") == "blk.0.ffn_gate_exps.weight"
+    assert og.hf_to_gguf_name("model.layers.0.mlp.shared_expert.up_proj.weight") == "blk.0.ffn_up_shexp.weight"
+    # unknown tensors and names that are not blk.N.rest pass through; the block number is not parsed
+    assert f("blk.3.attn_rot_embd") == "model.layers.3.attn_rot_embd"
+    assert f("blk.5") == "blk.5" and f("blk.x.ffn_up.weight") == "model.layers.x.mlp.up_proj.weight"
+    assert f("rope_freqs.weight") == "rope_freqs.weight" and f("blk..attn_q.weight") == "model.layers..self_attn.q_proj.weight"
+
+
+ROUND_TRIP_NAMES = ["model.embed_tokens.weight", "model.norm.weight", "lm_head.weight", "model.layers.0.self_attn.q_proj.weight",
+                    "model.layers.1.self_attn.k_proj.weight", "model.layers.2.self_attn.v_proj.weight",
+                    "model.layers.3.self_attn.o_proj.weight", "model.layers.4.input_layernorm.weight",
+                    "model.layers.5.post_attention_layernorm.weight", "model.layers.6.mlp.gate_proj.weight",
+                    "model.layers.7.mlp.up_proj.weight", "model.layers.8.mlp.down_proj.weight",
+                    "model.layers.9.self_attn.q_norm.weight", "model.layers.10.self_attn.k_norm.weight"]
+
+
+def test_host_f16_to_f32_is_exact(host_exe, tmp_path):
+    """f16_bits_to_f32 (the F16 tensors of a file that is loaded) on all 65536 bit patterns against numpy."""
+    bits = np.arange(65536, dtype=np.uint16)
+    src, dst = str(tmp_path / "f16.bin"), str(tmp_path / "f32.bin")
+    bits.tofile(src)
+    subprocess.run([host_exe, "--f16-to-f32", src, dst], check=True)
+    got = np.fromfile(dst, dtype=np.float32)
+    want = bits.view(np.float16).astype(np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+    assert np.isnan(got[nan]).all() and np.array_equal(got[nan].view(np.uint32) >> 31, want[nan].view(np.uint32) >> 31)
+
+
 # ---------------------------------------------------------------------------------------------------------------------
 # GPU: the Q4_K_M model driver end to end
 # ---------------------------------------------------------------------------------------------------------------------
@@ -417,3 +466,42 @@ def test_quantize_model_q4_k_m_file_equals_oracle(oracle, tmp_path):
     # and the file reads back: the C++ reader's view of it equals the oracle's
     r = subprocess.run([exe, "--dump", out], capture_output=True, text=True)
     assert r.stdout == oracle_dump(want)
+
+    # the way back, WeightLoader::load_gguf (weight_format.rs:258-313): every tensor dequantized to f32 under its Hugging
+    # Face name, bit for bit what the oracle's dequantizers give for the same bytes (F16 by numpy)
+    vals = str(tmp_path / "loaded.bin")
+    r = subprocess.run([exe, "--load-model", out, vals], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+
+    def oracle_dequantize(raw, dtype, shape):
+        raw = np.frombuffer(raw, dtype=np.uint8)
+        if dtype == 1:
+            return raw.view(np.float16).astype(np.float32)
+        return oracle.dequantize(dtype, raw, shape)
+
+    loaded, skipped = og.load_gguf(want, oracle_dequantize, lambda dt: dt in (0, 1, 30, 8, 10, 11, 12, 13, 14, 15))
+    assert not skipped and len(loaded) == len(tensors)
+    flat = np.fromfile(vals, dtype=np.float32)
+    lines = r.stdout.strip().split("\n")
+    assert len(lines) == len(loaded)
+    pos = 0
+    for line, name in zip(lines, sorted(loaded, key=lambda s: s.encode())):
+        f = line.split()
+        assert bytes.fromhex(f[0]).decode() == name
+        shape, values = loaded[name]
+        assert [int(v) for v in f[2:2 + int(f[1])]] == shape and int(f[-1]) == values.size
+        assert np.array_equal(flat[pos:pos + values.size].view(np.uint32), values.view(np.uint32)), name
+        pos += values.size
+    assert pos == flat.size
+    # the loaded names are the Hugging Face names the model was given (the fused tensor keeps its GGUF-style name under
+    # model.layers.N.)
+    assert set(loaded) == {n if not n.startswith("blk.") else og.gguf_to_hf_name(n) for n, _ in tensors}
+    # both name mappings of the C++ mirror against the oracle's, over the reference's examples and some odd names
+    names = ROUND_TRIP_NAMES + [og.hf_to_gguf_name(n) for n in ROUND_TRIP_NAMES] + [
+        "blk.3.attn_rot_embd", "blk.5", "blk.x.ffn_up.weight", "rope_freqs.weight", "blk..attn_q.weight", "model.layers.7",
+        "model.layers.+3.mlp.up_proj.weight", "model.layers.0.mlp.shared_experts.down_proj.weight", "blk.2.ffn_gate_inp_shexp.weight"]
+    listing = str(tmp_path / "names.txt")
+    open(listing, "w").write("\n".join(hx(n) for n in names) + "\n")
+    r = subprocess.run([exe, "--names", listing], capture_output=True, text=True)
+    got_names = [tuple(bytes.fromhex(h).decode() for h in l.split()) for l in r.stdout.strip().split("\n")]
+    assert got_names == [(og.gguf_to_hf_name(n), og.hf_to_gguf_name(n)) for n in names]
