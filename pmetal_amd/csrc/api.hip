@@ -712,10 +712,10 @@ int32_t pmetal_hip_qgemv_batch(const pmetal_hip_linear_desc *descs, size_t count
                 int64_t n[pmh::kMaxGemvGroup];
                 for (size_t g = i; g < j; g++) {
                     const pmetal_hip_linear_desc &e = descs[g];
-                    if (int32_t rc = check_linear(e.ggml_type, e.w_dev, e.n, e.k, e.x_dev, e.x_dtype, e.y_dev, e.order)) return rc;
+                    if (int32_t rc = check_linear(e.ggml_type, e.w_dev, e.n, e.k, e.x_dev, e.x_dtype, e.y_dev, e.order, true)) return rc;
                     w[g - i] = e.w_dev, y[g - i] = e.y_dev, n[g - i] = e.n;
                 }
-                if (int32_t rc = check_linear(v.ggml_type, v.w_dev, v.n, v.k, v.x_dev, v.x_dtype, v.y_dev, v.order)) return rc;
+                if (int32_t rc = check_linear(v.ggml_type, v.w_dev, v.n, v.k, v.x_dev, v.x_dtype, v.y_dev, v.order, true)) return rc;
                 const hipError_t err = pmh::launch_qgemv_q4k_q6k_group(w, n, y, (int)(j - i), v.w_dev, v.n, v.y_dev, d.k, d.x_dev, d.x_dtype,
                                                                        d.order, (hipStream_t)stream);
                 if (err == hipSuccess) {
@@ -733,8 +733,8 @@ int32_t pmetal_hip_qgemv_batch(const pmetal_hip_linear_desc *descs, size_t count
                 const pmetal_hip_linear_desc &e = descs[i + 1];
                 if (e.ggml_type == d.ggml_type && e.k == d.k && e.x_dev == d.x_dev && e.x_dtype == d.x_dtype && e.order == d.order &&
                     e.n > 0 && !pmh::qgemv_q4k_groupable(e.n, e.k)) {
-                    if (int32_t rc = check_linear(d.ggml_type, d.w_dev, d.n, d.k, d.x_dev, d.x_dtype, d.y_dev, d.order)) return rc;
-                    if (int32_t rc = check_linear(e.ggml_type, e.w_dev, e.n, e.k, e.x_dev, e.x_dtype, e.y_dev, e.order)) return rc;
+                    if (int32_t rc = check_linear(d.ggml_type, d.w_dev, d.n, d.k, d.x_dev, d.x_dtype, d.y_dev, d.order, true)) return rc;
+                    if (int32_t rc = check_linear(e.ggml_type, e.w_dev, e.n, e.k, e.x_dev, e.x_dtype, e.y_dev, e.order, true)) return rc;
                     const hipError_t err = pmh::launch_qgemv_q4k_pair(d.w_dev, d.n, d.y_dev, e.w_dev, e.n, e.y_dev, d.k, d.x_dev, d.x_dtype,
                                                                       d.order, (hipStream_t)stream);
                     if (err == hipSuccess) {
@@ -754,7 +754,7 @@ int32_t pmetal_hip_qgemv_batch(const pmetal_hip_linear_desc *descs, size_t count
         int64_t n[pmh::kMaxGemvGroup];
         for (size_t g = i; g < j; g++) {
             const pmetal_hip_linear_desc &e = descs[g];
-            if (int32_t rc = check_linear(e.ggml_type, e.w_dev, e.n, e.k, e.x_dev, e.x_dtype, e.y_dev, e.order)) return rc;
+            if (int32_t rc = check_linear(e.ggml_type, e.w_dev, e.n, e.k, e.x_dev, e.x_dtype, e.y_dev, e.order, true)) return rc;
             w[g - i] = e.w_dev, y[g - i] = e.y_dev, n[g - i] = e.n;
         }
         hipError_t err = pmh::launch_qgemv_q4k_group(w, n, y, (int)(j - i), d.k, d.x_dev, d.x_dtype, d.order, (hipStream_t)stream);

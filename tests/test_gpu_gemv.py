@@ -326,14 +326,18 @@ def test_qgemv_batch_takes_a_q6k_projection_into_a_q4k_group(oracle, order, rows
         else:
             raw[:, 0:4] = half
         raw = raw.reshape(-1)
-        dw, dy = pm.DeviceBuffer.from_host(raw), pm.DeviceBuffer(4 * n)
-        pm.check(lib.pmetal_hip_memset(dy.ptr, 0xFF, 4 * n, None))
-        keep.append((t, dw, dy, raw, n))
-        descs[i] = _lib.LinearDesc(t, x_dtype, order, 0, n, k, dw.ptr, dx.ptr, dy.ptr)
+        # y needs 4-byte alignment only, in a shared launch as in a launch of its own: every other member sits one float in
+        shift = i % 2
+        dw, dy = pm.DeviceBuffer.from_host(raw), pm.DeviceBuffer(4 * (n + 4))
+        pm.check(lib.pmetal_hip_memset(dy.ptr, 0xFF, 4 * (n + 4), None))
+        keep.append((t, dw, dy, raw, n, shift))
+        descs[i] = _lib.LinearDesc(t, x_dtype, order, 0, n, k, dw.ptr, dx.ptr, dy.ptr + 4 * shift)
     pm.check(lib.pmetal_hip_qgemv_batch(descs, len(rows), None))
     pm.check(lib.pmetal_hip_sync(None))
-    for t, dw, dy, raw, n in keep:
-        got = dy.to_host(np.float32)
+    for t, dw, dy, raw, n, shift in keep:
+        whole = dy.to_host(np.float32)
+        got = whole[shift:shift + n]
+        assert np.isnan(whole[shift + n:]).all() and np.isnan(whole[:shift]).all()  # nothing written outside
         want = oracle.qmatvec(t, raw, n, k, xa_ref, order=order)
         elem, norm = rel_errors(got, want)
         assert elem <= TOL and norm <= TOL, (t, n, elem, norm)
