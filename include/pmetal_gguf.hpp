@@ -266,7 +266,7 @@ inline GgmlType q4km_tensor_type(const std::string &gguf_name, size_t ndim, size
 
 
 // quantize(data, dtype) for every type the Q4_K_M recipe yields: F32 and F16 are conversions on the host
-// (crates/pmetal-gguf/src/quantize.rs:19-30), Q8_0 and the k-quants run on the GPU, anything else is the
+// (crates/pmetal-gguf/src/quantize.rs:19-30), the 32-element formats and the k-quants run on the GPU, anything else is the
 // reference's "not yet implemented" error.
 inline std::vector<uint8_t> quantize_any(const float *data, size_t n, GgmlType dtype) {
     if (dtype == GgmlType::F32) {
@@ -377,7 +377,7 @@ inline std::string gguf_to_hf_name(const std::string &gguf_name) {
 }
 
 // dequantize(data, dtype, shape) for every type this build decodes: F32 / F16 / BF16 are conversions on the host
-// (crates/pmetal-gguf/src/dequant.rs:219-258, sizes validated as there), Q8_0 and the k-quants run on the GPU.
+// (crates/pmetal-gguf/src/dequant.rs:219-258, sizes validated as there), the 32-element formats and the k-quants run on the GPU.
 inline bool load_supported(GgmlType dtype) {
     return dtype == GgmlType::F32 || dtype == GgmlType::F16 || dtype == GgmlType::Bf16 || pmetal_hip_is_supported((uint32_t)dtype) != 0;
 }

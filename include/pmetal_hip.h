@@ -36,7 +36,13 @@ extern "C" {
 /* GgmlType ids: crates/pmetal-gguf/src/types.rs:16-97. */
 #define PMETAL_GGML_TYPE_F32 0u
 #define PMETAL_GGML_TYPE_F16 1u
+/* the 32-element formats beside Q8_0: quantize (quantize.rs:93-230, :302-359) and dequantize (dequant.rs:300-463, :505-528) only */
+#define PMETAL_GGML_TYPE_Q4_0 2u
+#define PMETAL_GGML_TYPE_Q4_1 3u
+#define PMETAL_GGML_TYPE_Q5_0 6u
+#define PMETAL_GGML_TYPE_Q5_1 7u
 #define PMETAL_GGML_TYPE_Q8_0 8u
+#define PMETAL_GGML_TYPE_Q8_1 9u
 #define PMETAL_GGML_TYPE_Q2K 10u /* quantize / dequantize (k_quants.rs:1242-1321, :230-266) and the fused GEMV; GEMM through Q6_K re-blocking */
 #define PMETAL_GGML_TYPE_Q3K 11u /* quantize / dequantize (k_quants.rs:1139-1237, :281-355) and the fused GEMV; GEMM through Q6_K re-blocking */
 #define PMETAL_GGML_TYPE_Q4K 12u

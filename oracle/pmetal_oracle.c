@@ -30,6 +30,11 @@
  *                           The Rust itself was never run (no toolchain here).
  *   dequantize_* .......... reference KATs (dequant.rs:1016-1036,
  *                           k_quants.rs:1368-1383) + hand-built blocks + numpy.
+ *   quantize_q4_0/q4_1/q5_0/q5_1/q8_1, dequantize_legacy
+ *                           the reference's block tests (dequant.rs:935-1053), every code
+ *                           at every position of hand-written blocks, and quantized bytes
+ *                           derived by hand for inputs on power-of-two grids (no operation
+ *                           rounds), zero / short / non-finite blocks: tests/test_legacy32.py.
  *   recipe ................ reference KATs commands/quantize.rs:1561-1608.
  */
 #include "pmetal_oracle.h"
@@ -328,7 +333,12 @@ size_t pmo_type_size(uint32_t t) {
     switch (t) {
     case PMO_TYPE_F32: return 4;
     case PMO_TYPE_F16: return 2;
+    case PMO_TYPE_Q4_0: return 18;
+    case PMO_TYPE_Q4_1: return 20;
+    case PMO_TYPE_Q5_0: return 22;
+    case PMO_TYPE_Q5_1: return 24;
     case PMO_TYPE_Q8_0: return 34;
+    case PMO_TYPE_Q8_1: return 36;
     case PMO_TYPE_Q2K: return 84;
     case PMO_TYPE_Q3K: return 110;
     case PMO_TYPE_Q4K: return 144;
@@ -343,6 +353,11 @@ size_t pmo_block_size(uint32_t t) {
     switch (t) {
     case PMO_TYPE_F32:
     case PMO_TYPE_F16: return 1;
+    case PMO_TYPE_Q4_0:
+    case PMO_TYPE_Q4_1:
+    case PMO_TYPE_Q5_0:
+    case PMO_TYPE_Q5_1:
+    case PMO_TYPE_Q8_1:
     case PMO_TYPE_Q8_0: return 32;
     case PMO_TYPE_Q2K:
     case PMO_TYPE_Q3K:
@@ -382,6 +397,193 @@ void pmo_quantize_q8_0(const float *x, size_t n, uint8_t *dst) {
             if (start + i < end) v = (int8_t)clamp_i32(pmo_nearest_int(x[start + i] * iscale), -127, 127);
             out[2 + i] = (uint8_t)v;
         }
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* The 32-element formats beside Q8_0: quantize.rs:93-230, :302-359 and      */
+/* dequant.rs:300-463, :505-528.  A short last block is quantized over the   */
+/* elements it has (its minimum / maximum are taken over those only) with    */
+/* 0.0 standing in for the missing ones.                                     */
+/* ------------------------------------------------------------------------- */
+static int is_finite_f32(float v) { return (f32_bits(v) & 0x7F800000u) != 0x7F800000u; }
+
+/* quantize.rs:332-342 */
+static float signed_absmax(const float *x, size_t n) {
+    float s = 0.0f, absmax = 0.0f;
+    for (size_t i = 0; i < n; i++)
+        if (is_finite_f32(x[i]) && fabsf(x[i]) > absmax) absmax = fabsf(x[i]), s = x[i];
+    return s;
+}
+
+/* quantize.rs:344-359; f32::min / f32::max over finite values only, so no NaN reaches them */
+static void block_min_max(const float *x, size_t n, float *mn, float *mx) {
+    float lo = INFINITY, hi = -INFINITY;
+    *mn = *mx = 0.0f;
+    if (n == 0) return;
+    for (size_t i = 0; i < n; i++) {
+        if (!is_finite_f32(x[i])) continue;
+        /* equal values of opposite-signed zeros: f32::min keeps -0.0 over +0.0 and f32::max +0.0 over -0.0 on the
+           reference's targets; only the value matters below (min is encoded as f16, where -0.0 and +0.0 differ) */
+        if (x[i] < lo || (x[i] == lo && (f32_bits(x[i]) >> 31))) lo = x[i];
+        if (x[i] > hi || (x[i] == hi && !(f32_bits(x[i]) >> 31))) hi = x[i];
+    }
+    if (is_finite_f32(lo) && is_finite_f32(hi)) *mn = lo, *mx = hi;
+}
+
+static void put_f16(uint8_t *p, float v) {
+    uint16_t h = pmo_f32_to_f16(v);
+    p[0] = (uint8_t)(h & 0xFF), p[1] = (uint8_t)(h >> 8);
+}
+static float get_f16(const uint8_t *p) { return pmo_f16_to_f32((uint16_t)(p[0] | (p[1] << 8))); }
+static float at_or_zero(const float *x, size_t len, size_t i) { return i < len ? x[i] : 0.0f; }
+
+/* quantize.rs:93-128 */
+void pmo_quantize_q4_0(const float *x, size_t n, uint8_t *dst) {
+    size_t n_blocks = n / 32 + (n % 32 != 0);
+    for (size_t b = 0; b < n_blocks; b++) {
+        const float *blk = x + b * 32;
+        size_t len = n - b * 32 < 32 ? n - b * 32 : 32;
+        float max = 0.0f, amax = 0.0f;
+        for (size_t i = 0; i < len; i++) {
+            float ax = fabsf(blk[i]);
+            if (ax > amax) amax = ax, max = blk[i];
+        }
+        float scale = max / -8.0f;
+        float iscale = scale == 0.0f ? 0.0f : 1.0f / scale;
+        uint8_t *out = dst + b * 18;
+        put_f16(out, scale);
+        for (size_t i = 0; i < 16; i++) {
+            int32_t q0 = clamp_i32(pmo_nearest_int(at_or_zero(blk, len, i) * iscale + 8.5f), 0, 15);
+            int32_t q1 = clamp_i32(pmo_nearest_int(at_or_zero(blk, len, i + 16) * iscale + 8.5f), 0, 15);
+            out[2 + i] = (uint8_t)(q0 | (q1 << 4));
+        }
+    }
+}
+
+/* quantize.rs:130-157 */
+void pmo_quantize_q4_1(const float *x, size_t n, uint8_t *dst) {
+    size_t n_blocks = n / 32 + (n % 32 != 0);
+    for (size_t b = 0; b < n_blocks; b++) {
+        const float *blk = x + b * 32;
+        size_t len = n - b * 32 < 32 ? n - b * 32 : 32;
+        float mn, mx;
+        block_min_max(blk, len, &mn, &mx);
+        float scale = (mx - mn) / 15.0f;
+        float iscale = scale == 0.0f ? 0.0f : 1.0f / scale;
+        uint8_t *out = dst + b * 20;
+        put_f16(out, scale);
+        put_f16(out + 2, mn);
+        for (size_t i = 0; i < 16; i++) {
+            int32_t q0 = clamp_i32(pmo_nearest_int((at_or_zero(blk, len, i) - mn) * iscale), 0, 15);
+            int32_t q1 = clamp_i32(pmo_nearest_int((at_or_zero(blk, len, i + 16) - mn) * iscale), 0, 15);
+            out[4 + i] = (uint8_t)(q0 | (q1 << 4));
+        }
+    }
+}
+
+/* quantize.rs:159-191 (Q5_0) and :193-230 (Q5_1) */
+static void quantize_q5(const float *x, size_t n, uint8_t *dst, int with_min) {
+    size_t n_blocks = n / 32 + (n % 32 != 0), bytes = with_min ? 24 : 22;
+    for (size_t b = 0; b < n_blocks; b++) {
+        const float *blk = x + b * 32;
+        size_t len = n - b * 32 < 32 ? n - b * 32 : 32;
+        float mn = 0.0f, mx = 0.0f, scale;
+        if (with_min) {
+            block_min_max(blk, len, &mn, &mx);
+            scale = (mx - mn) / 31.0f;
+        } else {
+            scale = signed_absmax(blk, len) / -16.0f;
+        }
+        float iscale = scale == 0.0f ? 0.0f : 1.0f / scale;
+        uint32_t qh = 0;
+        uint8_t qs[16];
+        for (size_t i = 0; i < 16; i++) {
+            float x0 = at_or_zero(blk, len, i), x1 = at_or_zero(blk, len, i + 16);
+            int32_t q0, q1;
+            if (with_min) {
+                q0 = clamp_i32(pmo_nearest_int((x0 - mn) * iscale), 0, 31);
+                q1 = clamp_i32(pmo_nearest_int((x1 - mn) * iscale), 0, 31);
+            } else {
+                q0 = clamp_i32(pmo_nearest_int(x0 * iscale + 16.5f), 0, 31);
+                q1 = clamp_i32(pmo_nearest_int(x1 * iscale + 16.5f), 0, 31);
+            }
+            qs[i] = (uint8_t)((q0 & 0x0F) | ((q1 & 0x0F) << 4));
+            qh |= (uint32_t)((q0 & 0x10) >> 4) << i;
+            qh |= (uint32_t)((q1 & 0x10) >> 4) << (i + 16);
+        }
+        uint8_t *out = dst + b * bytes;
+        put_f16(out, scale);
+        out += 2;
+        if (with_min) put_f16(out, mn), out += 2;
+        out[0] = (uint8_t)qh, out[1] = (uint8_t)(qh >> 8), out[2] = (uint8_t)(qh >> 16), out[3] = (uint8_t)(qh >> 24);
+        memcpy(out + 4, qs, 16);
+    }
+}
+void pmo_quantize_q5_0(const float *x, size_t n, uint8_t *dst) { quantize_q5(x, n, dst, 0); }
+void pmo_quantize_q5_1(const float *x, size_t n, uint8_t *dst) { quantize_q5(x, n, dst, 1); }
+
+/* quantize.rs:302-330 */
+void pmo_quantize_q8_1(const float *x, size_t n, uint8_t *dst) {
+    size_t n_blocks = n / 32 + (n % 32 != 0);
+    for (size_t b = 0; b < n_blocks; b++) {
+        const float *blk = x + b * 32;
+        size_t len = n - b * 32 < 32 ? n - b * 32 : 32;
+        float amax = 0.0f;
+        for (size_t i = 0; i < len; i++) amax = rust_max(amax, fabsf(blk[i]));
+        float scale = amax / 127.0f;
+        float iscale = amax == 0.0f ? 0.0f : 127.0f / amax;
+        uint8_t *out = dst + b * 36;
+        int32_t sum = 0;
+        for (size_t i = 0; i < 32; i++) {
+            int32_t q = clamp_i32(pmo_nearest_int(at_or_zero(blk, len, i) * iscale), -127, 127);
+            out[4 + i] = (uint8_t)(int8_t)q;
+            sum += q;
+        }
+        put_f16(out, scale);
+        put_f16(out + 2, (float)sum * scale);
+    }
+}
+
+/* dequant.rs:300-334 (Q4_0), :344-371 (Q4_1), :382-414 (Q5_0), :425-463 (Q5_1), :505-528 (Q8_1) */
+void pmo_dequantize_legacy(uint32_t t, const uint8_t *src, size_t n, float *dst) {
+    size_t n_blocks = n / 32 + (n % 32 != 0), bytes = pmo_type_size(t);
+    for (size_t b = 0; b < n_blocks; b++) {
+        const uint8_t *blk = src + b * bytes;
+        float v[32];
+        float scale = get_f16(blk);
+        if (t == PMO_TYPE_Q8_1) {
+            for (int i = 0; i < 32; i++) v[i] = (float)(int8_t)blk[4 + i] * scale;
+        } else if (t == PMO_TYPE_Q4_0) {
+            for (int i = 0; i < 16; i++) {
+                v[i] = (float)(int8_t)((int8_t)(blk[2 + i] & 0x0F) - 8) * scale;
+                v[i + 16] = (float)(int8_t)((int8_t)(blk[2 + i] >> 4) - 8) * scale;
+            }
+        } else if (t == PMO_TYPE_Q4_1) {
+            float mn = get_f16(blk + 2);
+            for (int i = 0; i < 16; i++) {
+                v[i] = (float)(blk[4 + i] & 0x0F) * scale + mn;
+                v[i + 16] = (float)(blk[4 + i] >> 4) * scale + mn;
+            }
+        } else {
+            int with_min = t == PMO_TYPE_Q5_1;
+            float mn = with_min ? get_f16(blk + 2) : 0.0f;
+            const uint8_t *p = blk + (with_min ? 4 : 2);
+            uint32_t qh = (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
+            const uint8_t *qs = p + 4;
+            for (int i = 0; i < 16; i++) {
+                int32_t q_lo = (int32_t)(qs[i] & 0x0F) | (int32_t)(((qh >> i) & 1u) << 4);
+                int32_t q_hi = (int32_t)(qs[i] >> 4) | (int32_t)(((qh >> (i + 16)) & 1u) << 4);
+                if (with_min) {
+                    v[i] = (float)q_lo * scale + mn;
+                    v[i + 16] = (float)q_hi * scale + mn;
+                } else {
+                    v[i] = (float)(q_lo - 16) * scale;
+                    v[i + 16] = (float)(q_hi - 16) * scale;
+                }
+            }
+        }
+        for (size_t i = 0; i < 32 && b * 32 + i < n; i++) dst[b * 32 + i] = v[i];
     }
 }
 
@@ -1217,9 +1419,15 @@ int32_t pmo_qmatvec_q8k(uint32_t t, const uint8_t *w, size_t n_rows, size_t k, c
 /* quantize.rs:17-87 and dequant.rs:92-132, :184-216                         */
 /* ------------------------------------------------------------------------- */
 int32_t pmo_quantize(uint32_t t, const float *x, size_t n, uint8_t *dst, size_t dst_len) {
-    if (t != PMO_TYPE_Q8_0 && t != PMO_TYPE_Q2K && t != PMO_TYPE_Q3K && t != PMO_TYPE_Q4K && t != PMO_TYPE_Q5K && t != PMO_TYPE_Q6K && t != PMO_TYPE_Q8K)
+    int legacy = t == PMO_TYPE_Q4_0 || t == PMO_TYPE_Q4_1 || t == PMO_TYPE_Q5_0 || t == PMO_TYPE_Q5_1 || t == PMO_TYPE_Q8_1;
+    if (!legacy && t != PMO_TYPE_Q8_0 && t != PMO_TYPE_Q2K && t != PMO_TYPE_Q3K && t != PMO_TYPE_Q4K && t != PMO_TYPE_Q5K && t != PMO_TYPE_Q6K && t != PMO_TYPE_Q8K)
         return PMO_ERR_UNSUPPORTED_TYPE;
     if (dst_len != pmo_tensor_size(t, n)) return PMO_ERR_INVALID_SIZE;
+    if (t == PMO_TYPE_Q4_0) return pmo_quantize_q4_0(x, n, dst), PMO_OK;
+    if (t == PMO_TYPE_Q4_1) return pmo_quantize_q4_1(x, n, dst), PMO_OK;
+    if (t == PMO_TYPE_Q5_0) return pmo_quantize_q5_0(x, n, dst), PMO_OK;
+    if (t == PMO_TYPE_Q5_1) return pmo_quantize_q5_1(x, n, dst), PMO_OK;
+    if (t == PMO_TYPE_Q8_1) return pmo_quantize_q8_1(x, n, dst), PMO_OK;
     if (t == PMO_TYPE_Q8K) pmo_quantize_q8k(x, n, dst);
     else if (t == PMO_TYPE_Q2K) pmo_quantize_q2k(x, n, dst);
     else if (t == PMO_TYPE_Q3K) pmo_quantize_q3k(x, n, dst);
@@ -1232,7 +1440,8 @@ int32_t pmo_quantize(uint32_t t, const float *x, size_t n, uint8_t *dst, size_t 
 
 int32_t pmo_dequantize(uint32_t t, const uint8_t *src, size_t src_len, const int32_t *shape, size_t ndim,
                        float *dst, size_t dst_cap, uint32_t order) {
-    if (t != PMO_TYPE_Q8_0 && t != PMO_TYPE_Q2K && t != PMO_TYPE_Q3K && t != PMO_TYPE_Q4K && t != PMO_TYPE_Q5K && t != PMO_TYPE_Q6K && t != PMO_TYPE_Q8K)
+    int legacy = t == PMO_TYPE_Q4_0 || t == PMO_TYPE_Q4_1 || t == PMO_TYPE_Q5_0 || t == PMO_TYPE_Q5_1 || t == PMO_TYPE_Q8_1;
+    if (!legacy && t != PMO_TYPE_Q8_0 && t != PMO_TYPE_Q2K && t != PMO_TYPE_Q3K && t != PMO_TYPE_Q4K && t != PMO_TYPE_Q5K && t != PMO_TYPE_Q6K && t != PMO_TYPE_Q8K)
         return PMO_ERR_UNSUPPORTED_TYPE;
     /* dequant.rs:193-206 shape_n_elements */
     for (size_t i = 0; i < ndim; i++)
@@ -1246,7 +1455,8 @@ int32_t pmo_dequantize(uint32_t t, const uint8_t *src, size_t src_len, const int
     /* dequant.rs:208-216 validate_data_size */
     if (src_len != pmo_tensor_size(t, n)) return PMO_ERR_INVALID_SIZE;
     if (dst_cap < n) return PMO_ERR_INVALID_SIZE;
-    if (t == PMO_TYPE_Q8_0) pmo_dequantize_q8_0(src, n, dst);
+    if (legacy) pmo_dequantize_legacy(t, src, n, dst);
+    else if (t == PMO_TYPE_Q8_0) pmo_dequantize_q8_0(src, n, dst);
     else if (t == PMO_TYPE_Q4K) pmo_dequantize_q4k(src, n, dst, order);
     else if (t == PMO_TYPE_Q5K) pmo_dequantize_q5k(src, n, dst, order);
     else if (t == PMO_TYPE_Q8K) pmo_dequantize_q8k(src, n, dst);

@@ -38,7 +38,12 @@ extern "C" {
 enum {
     PMO_TYPE_F32 = 0,
     PMO_TYPE_F16 = 1,
+    PMO_TYPE_Q4_0 = 2, /* the 32-element formats beside Q8_0: quantize / dequantize only */
+    PMO_TYPE_Q4_1 = 3,
+    PMO_TYPE_Q5_0 = 6,
+    PMO_TYPE_Q5_1 = 7,
     PMO_TYPE_Q8_0 = 8,
+    PMO_TYPE_Q8_1 = 9,
     PMO_TYPE_Q2K = 10, /* quantize / dequantize only */
     PMO_TYPE_Q3K = 11, /* quantize / dequantize only */
     PMO_TYPE_Q4K = 12,
@@ -112,6 +117,12 @@ void pmo_dequantize_q3k(const uint8_t *src, size_t n, float *dst);
 
 /* quantize.rs:17-87 (dispatcher) and dequant.rs:92-132 + 184-216 (dispatcher and
  * validation).  Return a PMO_* code. */
+void pmo_quantize_q4_0(const float *x, size_t n, uint8_t *dst); /* quantize.rs:93-128 */
+void pmo_quantize_q4_1(const float *x, size_t n, uint8_t *dst); /* :130-157 */
+void pmo_quantize_q5_0(const float *x, size_t n, uint8_t *dst); /* :159-191 */
+void pmo_quantize_q5_1(const float *x, size_t n, uint8_t *dst); /* :193-230 */
+void pmo_quantize_q8_1(const float *x, size_t n, uint8_t *dst); /* :302-330 */
+void pmo_dequantize_legacy(uint32_t ggml_type, const uint8_t *src, size_t n, float *dst); /* dequant.rs:300-463, :505-528 */
 int32_t pmo_quantize(uint32_t ggml_type, const float *x, size_t n, uint8_t *dst, size_t dst_len);
 int32_t pmo_dequantize(uint32_t ggml_type, const uint8_t *src, size_t src_len, const int32_t *shape,
                        size_t ndim, float *dst, size_t dst_cap, uint32_t order);

@@ -58,8 +58,14 @@ bool path_type(uint32_t t) {
 }
 // types with quantize / dequantize kernels: the above, Q5_K (the Q4_K_M recipe gives it to fused attn_qkv tensors) and
 // Q8_K (the activation format of the integer dot products, and the first candidate of the KL calibration)
+// the 32-element formats beside Q8_0: quantize / dequantize only
+bool legacy32_type(uint32_t t) {
+    return t == PMETAL_GGML_TYPE_Q4_0 || t == PMETAL_GGML_TYPE_Q4_1 || t == PMETAL_GGML_TYPE_Q5_0 || t == PMETAL_GGML_TYPE_Q5_1 ||
+           t == PMETAL_GGML_TYPE_Q8_1;
+}
 bool codec_type(uint32_t t) {
-    return path_type(t) || t == PMETAL_GGML_TYPE_Q2K || t == PMETAL_GGML_TYPE_Q3K || t == PMETAL_GGML_TYPE_Q5K || t == PMETAL_GGML_TYPE_Q8K;
+    return path_type(t) || legacy32_type(t) || t == PMETAL_GGML_TYPE_Q2K || t == PMETAL_GGML_TYPE_Q3K || t == PMETAL_GGML_TYPE_Q5K ||
+           t == PMETAL_GGML_TYPE_Q8K;
 }
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -304,6 +310,11 @@ void pmetal_hip_clear_error(void) { ok(); }
 // ---- sizes: types.rs:102-187 ----
 size_t pmetal_hip_type_size(uint32_t t) {
     switch (t) {
+    case PMETAL_GGML_TYPE_Q4_0: return 18;
+    case PMETAL_GGML_TYPE_Q4_1: return 20;
+    case PMETAL_GGML_TYPE_Q5_0: return 22;
+    case PMETAL_GGML_TYPE_Q5_1: return 24;
+    case PMETAL_GGML_TYPE_Q8_1: return 36;
     case PMETAL_GGML_TYPE_Q8_0: return 34;
     case PMETAL_GGML_TYPE_Q4K: return 144;
     case PMETAL_GGML_TYPE_Q2K: return 84;
@@ -317,6 +328,11 @@ size_t pmetal_hip_type_size(uint32_t t) {
 
 size_t pmetal_hip_block_size(uint32_t t) {
     switch (t) {
+    case PMETAL_GGML_TYPE_Q4_0:
+    case PMETAL_GGML_TYPE_Q4_1:
+    case PMETAL_GGML_TYPE_Q5_0:
+    case PMETAL_GGML_TYPE_Q5_1:
+    case PMETAL_GGML_TYPE_Q8_1:
     case PMETAL_GGML_TYPE_Q8_0: return 32;
     case PMETAL_GGML_TYPE_Q4K:
     case PMETAL_GGML_TYPE_Q2K:
@@ -505,7 +521,8 @@ int32_t pmetal_hip_quantize_dev(uint32_t t, const float *src, size_t n, uint8_t 
     if (int32_t rc = require_device()) return rc;
     hipStream_t s = (hipStream_t)stream;
     hipError_t e;
-    if (t == PMETAL_GGML_TYPE_Q8_0) e = pmh::launch_quantize_q8_0(src, n, dst, s);
+    if (legacy32_type(t)) e = pmh::launch_quantize_legacy32(t, src, n, dst, s);
+    else if (t == PMETAL_GGML_TYPE_Q8_0) e = pmh::launch_quantize_q8_0(src, n, dst, s);
     else if (t == PMETAL_GGML_TYPE_Q4K) e = pmh::launch_quantize_q4k(src, n, dst, s);
     else if (t == PMETAL_GGML_TYPE_Q5K) e = pmh::launch_quantize_q5k(src, n, dst, s);
     else if (t == PMETAL_GGML_TYPE_Q8K) e = pmh::launch_quantize_q8k(src, n, dst, s);
@@ -549,7 +566,8 @@ int32_t pmetal_hip_dequantize_dev(uint32_t t, const uint8_t *src, size_t src_len
     if (int32_t rc = require_device()) return rc;
     hipStream_t s = (hipStream_t)stream;
     hipError_t e;
-    if (t == PMETAL_GGML_TYPE_Q8_0) e = pmh::launch_dequantize_q8_0(src, n, dst, s);
+    if (legacy32_type(t)) e = pmh::launch_dequantize_legacy32(t, src, n, dst, s);
+    else if (t == PMETAL_GGML_TYPE_Q8_0) e = pmh::launch_dequantize_q8_0(src, n, dst, s);
     else if (t == PMETAL_GGML_TYPE_Q4K) e = pmh::launch_dequantize_q4k(src, n, dst, order, s);
     else if (t == PMETAL_GGML_TYPE_Q5K) e = pmh::launch_dequantize_q5k(src, n, dst, order, s);
     else if (t == PMETAL_GGML_TYPE_Q8K) e = pmh::launch_dequantize_q8k(src, n, dst, s);

@@ -143,6 +143,171 @@ __global__ __launch_bounds__(256) void k_dequantize_q8_0(const uint8_t *__restri
     }
 }
 
+// -------------------------------------------------------------------------------------------
+// The 32-element formats beside Q8_0 (FMT = GGML type id): Q4_0 (2: d, 16 bytes of nibbles), Q4_1 (3: d, m, nibbles),
+// Q5_0 (6: d, qh, nibbles), Q5_1 (7: d, m, qh, nibbles), Q8_1 (9: d, s, 32 int8).  Low nibbles are elements 0..15, high
+// nibbles 16..31; bit i of qh is the fifth bit of element i.  quantize.rs:93-230, :302-359; dequant.rs:300-463, :505-528.
+// Eight lanes per block, lane j holding elements 4 j .. 4 j + 3, as in the Q8_0 kernels.
+// -------------------------------------------------------------------------------------------
+template <int FMT>
+struct Legacy32 {
+    static constexpr bool kMin = FMT == 3 || FMT == 7, kHigh = FMT == 6 || FMT == 7, kInt8 = FMT == 9;
+    static constexpr int kBytes = FMT == 2 ? 18 : FMT == 3 ? 20 : FMT == 6 ? 22 : FMT == 7 ? 24 : 36;
+    static constexpr int kQhOff = kMin ? 4 : 2, kQsOff = kInt8 ? 4 : 2 + (kMin ? 2 : 0) + (kHigh ? 4 : 0);
+    static constexpr int kMaxQ = kHigh ? 31 : 15;
+};
+
+__device__ __forceinline__ bool finite_f32(float v) { return (__builtin_bit_cast(uint32_t, v) & 0x7F800000u) != 0x7F800000u; }
+
+template <int FMT>
+__global__ __launch_bounds__(256) void k_quantize_b32(const float *__restrict__ x, size_t n, uint8_t *__restrict__ dst,
+                                                       size_t n_blocks) {
+    using F = Legacy32<FMT>;
+    const size_t tid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t blk = tid >> 3;
+    const int j = (int)(tid & 7);
+    const size_t e = tid * 4;
+    float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // an element past the end of the tensor counts as 0.0 when it is quantized ...
+    bool have[4];                           // ... but takes no part in the block's minimum / maximum
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        have[c] = e + c < n;
+        if (have[c]) v[c] = x[e + c];
+    }
+    float scale, mn = 0.0f;
+    if (F::kInt8) {  // amax = fold(0.0, max(|x|)), NaN ignored
+        float a = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v[0]), __builtin_fabsf(v[1])),
+                                  __builtin_fmaxf(__builtin_fabsf(v[2]), __builtin_fabsf(v[3])));
+        a = __builtin_fmaxf(a, 0.0f);
+        a = __builtin_fmaxf(a, __shfl_xor(a, 1));
+        a = __builtin_fmaxf(a, __shfl_xor(a, 2));
+        a = __builtin_fmaxf(a, __shfl_xor(a, 4));
+        scale = a / 127.0f;
+        const float iscale = (a == 0.0f) ? 0.0f : 127.0f / a;
+        uint32_t packed = 0;
+        int sum = 0;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const int q = (int)clamp_round(v[c] * iscale, -127.0f, 127.0f);
+            sum += q;
+            packed |= ((uint32_t)q & 0xFFu) << (8 * c);
+        }
+        sum += __shfl_xor(sum, 1);
+        sum += __shfl_xor(sum, 2);
+        sum += __shfl_xor(sum, 4);
+        if (blk < n_blocks) {
+            uint8_t *out = dst + blk * F::kBytes;
+            *reinterpret_cast<uint32_t *>(out + 4 + 4 * j) = packed;  // 36-byte blocks: dwords stay aligned
+            if (j == 0) {
+                *reinterpret_cast<uint16_t *>(out) = (uint16_t)f32_to_f16_bits(scale);
+                *reinterpret_cast<uint16_t *>(out + 2) = (uint16_t)f32_to_f16_bits((float)sum * scale);
+            }
+        }
+        return;
+    }
+    float q[4];
+    if (F::kMin) {
+        // block_min_max: over the finite elements; (0, 0) if there is none.  Total-order keys, so that of equal zeros the
+        // negative one is the minimum and the positive one the maximum.
+        int klo = 0x7FFFFFFF, khi = (int)0x80000000;
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+            if (have[c] && finite_f32(v[c])) {
+                const int key = total_key(v[c]);
+                klo = key < klo ? key : klo;
+                khi = key > khi ? key : khi;
+            }
+#pragma unroll
+        for (int off = 1; off < 8; off <<= 1) {
+            const int ol = __shfl_xor(klo, off), oh = __shfl_xor(khi, off);
+            klo = ol < klo ? ol : klo;
+            khi = oh > khi ? oh : khi;
+        }
+        float mx = 0.0f;
+        if (klo <= khi) {  // at least one finite element
+            mn = __builtin_bit_cast(float, klo ^ (int)(((unsigned)(klo >> 31)) >> 1));
+            mx = __builtin_bit_cast(float, khi ^ (int)(((unsigned)(khi >> 31)) >> 1));
+        }
+        scale = (mx - mn) / (float)F::kMaxQ;
+        const float iscale = scale == 0.0f ? 0.0f : 1.0f / scale;
+#pragma unroll
+        for (int c = 0; c < 4; c++) q[c] = clamp_round((v[c] - mn) * iscale, 0.0f, (float)F::kMaxQ);
+    } else {
+        // the element of largest magnitude, the first one among equals (Q5_0: among the finite ones), with its sign
+        float amax = 0.0f, smax = 0.0f;
+        int idx = 0;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const float ax = __builtin_fabsf(v[c]);
+            if (have[c] && (FMT == 2 || finite_f32(v[c])) && ax > amax) amax = ax, smax = v[c], idx = 4 * j + c;
+        }
+#pragma unroll
+        for (int off = 1; off < 8; off <<= 1) {
+            const float oa = __shfl_xor(amax, off), os = __shfl_xor(smax, off);
+            const int oi = __shfl_xor(idx, off);
+            if (oa > amax || (oa == amax && oa > 0.0f && oi < idx)) amax = oa, smax = os, idx = oi;
+        }
+        scale = smax / (FMT == 2 ? -8.0f : -16.0f);
+        const float iscale = scale == 0.0f ? 0.0f : 1.0f / scale;
+        const float half_up = FMT == 2 ? 8.5f : 16.5f;
+#pragma unroll
+        for (int c = 0; c < 4; c++) q[c] = clamp_round(v[c] * iscale + half_up, 0.0f, (float)F::kMaxQ);
+    }
+    uint32_t nib = 0, hi = 0;
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        const uint32_t qi = (uint32_t)q[c];
+        nib |= (qi & 0xFu) << (8 * c);
+        hi |= (qi >> 4) << (4 * j + c);
+    }
+    const uint32_t other = (uint32_t)__shfl_xor((int)nib, 4);  // lanes 0..3 hold the low, lanes 4..7 the high nibbles
+    if (F::kHigh) {
+        hi |= (uint32_t)__shfl_xor((int)hi, 1);
+        hi |= (uint32_t)__shfl_xor((int)hi, 2);
+        hi |= (uint32_t)__shfl_xor((int)hi, 4);
+    }
+    if (blk < n_blocks) {
+        uint8_t *out = dst + blk * F::kBytes;
+        if (j < 4) *reinterpret_cast<u32_a2 *>(out + F::kQsOff + 4 * j) = nib | (other << 4);
+        if (j == 4) *reinterpret_cast<uint16_t *>(out) = (uint16_t)f32_to_f16_bits(scale);
+        if (F::kMin && j == 5) *reinterpret_cast<uint16_t *>(out + 2) = (uint16_t)f32_to_f16_bits(mn);
+        if (F::kHigh && j == 6) *reinterpret_cast<u32_a2 *>(out + F::kQhOff) = hi;
+    }
+}
+
+// One lane per 4 outputs: lane j of a block decodes elements 4 j .. 4 j + 3.
+template <int FMT>
+__global__ __launch_bounds__(256) void k_dequantize_b32(const uint8_t *__restrict__ src, size_t n, float *__restrict__ dst) {
+    using F = Legacy32<FMT>;
+    const size_t tid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t e = tid * 4;
+    if (e >= n) return;
+    const uint8_t *blk = src + (tid >> 3) * F::kBytes;
+    const int j = (int)(tid & 7);
+    const float d = f16_bits_to_f32(*reinterpret_cast<const uint16_t *>(blk));
+    float o[4];
+    if (F::kInt8) {
+        const uint32_t q = *reinterpret_cast<const uint32_t *>(blk + 4 + 4 * j);
+#pragma unroll
+        for (int c = 0; c < 4; c++) o[c] = (float)(int8_t)(q >> (8 * c)) * d;
+    } else {
+        const float m = F::kMin ? f16_bits_to_f32(*reinterpret_cast<const uint16_t *>(blk + 2)) : 0.0f;
+        const uint32_t qs = *reinterpret_cast<const u32_a2 *>(blk + F::kQsOff + 4 * (j & 3)) >> (4 * (j >> 2));
+        const uint32_t qh = F::kHigh ? *reinterpret_cast<const u32_a2 *>(blk + F::kQhOff) >> (4 * j) : 0u;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const int q = (int)((qs >> (8 * c)) & 0xFu) | (int)(((qh >> c) & 1u) << 4);
+            if (F::kMin) o[c] = (float)q * d + m;
+            else o[c] = (float)(q - (F::kHigh ? 16 : 8)) * d;
+        }
+    }
+    if (e + 3 < n) {
+        *reinterpret_cast<float4 *>(dst + e) = make_float4(o[0], o[1], o[2], o[3]);
+    } else {
+        for (int c = 0; c < 4 && e + c < n; c++) dst[e + c] = o[c];
+    }
+}
+
 // get_scale_min_k4 (quantize.rs:844-855) on the 12 scale bytes held as three dwords.
 __device__ __forceinline__ void scale_min_k4(int j, uint32_t s0, uint32_t s1, uint32_t s2, uint32_t &sc,
                                              uint32_t &m) {
@@ -1224,6 +1389,35 @@ hipError_t launch_quantize_q8_0(const float *x, size_t n, uint8_t *dst, hipStrea
     const size_t n_blocks = (n + 31) / 32;
     if (n_blocks == 0) return hipSuccess;
     hipLaunchKernelGGL(k_quantize_q8_0, dim3(grid_for(n_blocks * 8, 256)), dim3(256), 0, s, x, n, dst, n_blocks);
+    return hipGetLastError();
+}
+
+// Q4_0, Q4_1, Q5_0, Q5_1, Q8_1 (GGML type ids 2, 3, 6, 7, 9)
+hipError_t launch_quantize_legacy32(uint32_t type, const float *x, size_t n, uint8_t *dst, hipStream_t s) {
+    const size_t n_blocks = (n + 31) / 32;
+    if (n_blocks == 0) return hipSuccess;
+    const dim3 grid(grid_for(n_blocks * 8, 256)), block(256);
+    switch (type) {
+    case 2: hipLaunchKernelGGL(k_quantize_b32<2>, grid, block, 0, s, x, n, dst, n_blocks); break;
+    case 3: hipLaunchKernelGGL(k_quantize_b32<3>, grid, block, 0, s, x, n, dst, n_blocks); break;
+    case 6: hipLaunchKernelGGL(k_quantize_b32<6>, grid, block, 0, s, x, n, dst, n_blocks); break;
+    case 7: hipLaunchKernelGGL(k_quantize_b32<7>, grid, block, 0, s, x, n, dst, n_blocks); break;
+    case 9: hipLaunchKernelGGL(k_quantize_b32<9>, grid, block, 0, s, x, n, dst, n_blocks); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+hipError_t launch_dequantize_legacy32(uint32_t type, const uint8_t *src, size_t n, float *dst, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    const dim3 grid(grid_for((n + 3) / 4, 256)), block(256);
+    switch (type) {
+    case 2: hipLaunchKernelGGL(k_dequantize_b32<2>, grid, block, 0, s, src, n, dst); break;
+    case 3: hipLaunchKernelGGL(k_dequantize_b32<3>, grid, block, 0, s, src, n, dst); break;
+    case 6: hipLaunchKernelGGL(k_dequantize_b32<6>, grid, block, 0, s, src, n, dst); break;
+    case 7: hipLaunchKernelGGL(k_dequantize_b32<7>, grid, block, 0, s, src, n, dst); break;
+    case 9: hipLaunchKernelGGL(k_dequantize_b32<9>, grid, block, 0, s, src, n, dst); break;
+    default: return hipErrorInvalidValue;
+    }
     return hipGetLastError();
 }
 

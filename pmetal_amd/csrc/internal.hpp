@@ -13,6 +13,8 @@ constexpr uint32_t kDtypeF32 = 0, kDtypeBf16 = 1;
 
 // ---- codec.hip: bit-exact quantize / dequantize (compiled without fp contraction) ----
 hipError_t launch_quantize_q8_0(const float *x, size_t n, uint8_t *dst, hipStream_t s);
+hipError_t launch_quantize_legacy32(uint32_t type, const float *x, size_t n, uint8_t *dst, hipStream_t s);
+hipError_t launch_dequantize_legacy32(uint32_t type, const uint8_t *src, size_t n, float *dst, hipStream_t s);
 hipError_t launch_quantize_q4k(const float *x, size_t n, uint8_t *dst, hipStream_t s);
 hipError_t launch_quantize_q5k(const float *x, size_t n, uint8_t *dst, hipStream_t s);
 hipError_t launch_quantize_q2k(const float *x, size_t n, uint8_t *dst, hipStream_t s);

@@ -25,7 +25,12 @@ from . import _lib
 class GgmlType(enum.IntEnum):
     F32 = 0
     F16 = 1
+    Q4_0 = 2
+    Q4_1 = 3
+    Q5_0 = 6
+    Q5_1 = 7
     Q8_0 = 8
+    Q8_1 = 9
     Q4K = 12
     Q5K = 13
     Q6K = 14

@@ -73,7 +73,7 @@ static void test_invalid_size_and_shape() {  // dequant.rs:1139-1150
     CHECK(caught);
     caught = false;
     try {
-        quantize(std::vector<float>(32), (GgmlType)2);  // Q4_0 is outside this path
+        quantize(std::vector<float>(256), (GgmlType)16);  // IQ2_XXS is outside this path
     } catch (const QuantizationError &) {
         caught = true;
     }

@@ -66,7 +66,7 @@ def test_validation_order_and_error_slot(lib):
     one = (C.c_int32 * 1)(256)
     assert lib.pmetal_hip_dequantize(Q4K, raw.ctypes.data, 10, one, 1, None, 0, 0) == 3
     assert b"expected 144 bytes, got 10" in lib.pmetal_hip_last_error_message()
-    assert lib.pmetal_hip_quantize(2, None, 32, None, 18) == 2
+    assert lib.pmetal_hip_quantize(16, None, 256, None, 66) == 2  # IQ2_XXS: no kernel here
     assert lib.pmetal_hip_quantize(Q4K, None, 256, None, 100) == 3
     lib.pmetal_hip_clear_error()
     assert lib.pmetal_hip_last_error_code() == 0

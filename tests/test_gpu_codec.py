@@ -154,5 +154,5 @@ def test_errors_match_reference_classes():
         pm.dequantize(np.zeros(0, np.uint8), 99, [0])
     assert e.value.kind == "UnsupportedType"
     with pytest.raises(pm.QuantizationError):
-        pm.quantize(np.zeros(32, np.float32), 2)  # Q4_0: outside this path
+        pm.quantize(np.zeros(256, np.float32), 16)  # IQ2_XXS: outside this path
     assert pm.dequantize(np.zeros(0, np.uint8), Q6K, [0, 7]).size == 0
