@@ -38,7 +38,10 @@ def test_sizes_match_types_rs(lib):
     assert lib.pmetal_hip_tensor_size(Q4K, 14336 * 4096) == 33030144
     assert lib.pmetal_hip_tensor_size(Q8_0, 33) == 68
     assert lib.pmetal_hip_tensor_size(99, 1000) == 0 and lib.pmetal_hip_type_size(0) == 0
-    assert [lib.pmetal_hip_is_supported(t) for t in (Q8_0, Q4K, Q6K, 2, 13, 15, 11, 10, 16)] == [1, 1, 1, 0, 1, 1, 1, 1, 0]
+    assert [lib.pmetal_hip_is_supported(t) for t in (Q8_0, Q4K, Q6K, 2, 13, 15, 11, 10, 16, 41)] == [1, 1, 1, 1, 1, 1, 1, 1, 0, 0]
+    # the 32-element formats beside Q8_0 (types.rs:106-111, :150)
+    assert [lib.pmetal_hip_type_size(t) for t in (2, 3, 6, 7, 9)] == [18, 20, 22, 24, 36]
+    assert [lib.pmetal_hip_block_size(t) for t in (2, 3, 6, 7, 9)] == [32] * 5
     assert lib.pmetal_hip_type_size(13) == 176 and lib.pmetal_hip_block_size(13) == 256  # Q5_K: quantize / dequantize only
     assert lib.pmetal_hip_type_size(15) == 292 and lib.pmetal_hip_block_size(15) == 256  # Q8_K likewise
 
