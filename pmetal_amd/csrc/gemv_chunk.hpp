@@ -30,19 +30,30 @@ __device__ __forceinline__ GroupScale group_scale(uint32_t mb) {
 
 // Four activations -> one dword per digit plane (three balanced base-256 digits in [-128, 127] per value, value c in
 // byte c); returns the sum of the four fixed-point integers.
+//  * |v * mult| < 2^22, so adding 1.5 * 2^23 rounds to the integer grid (nearest even, as rintf does) and leaves the
+//    integer xi in the low bits of the float.
+//  * xi + 0x808080 = sum (d_k + 128) 256^k with every d_k + 128 in [0, 255]: the bytes of the biased value, each with its
+//    top bit flipped, are the balanced digits.  The three bytes of the four values are transposed into the three planes
+//    with byte permutes.
 __device__ __forceinline__ int to_digits(const float (&v)[4], const GroupScale &g, uint32_t (&dig)[3]) {
-    dig[0] = dig[1] = dig[2] = 0;
+    constexpr float kMagic = 12582912.0f;                       // 0x4B400000
+    constexpr uint32_t kUnbias = 0x4B400000u - 0x00808080u;     // float bits -> xi + 0x808080
+    uint32_t u[4];
     int sum = 0;
 #pragma unroll
     for (int c = 0; c < 4; c++) {
-        const int xi = g.bad ? 0 : (int)__builtin_rintf(v[c] * g.mult);
-        sum += xi;
-        const int d0 = (int)(int8_t)xi, r1 = (xi - d0) >> 8;
-        const int d1 = (int)(int8_t)r1, d2 = (r1 - d1) >> 8;
-        dig[0] |= (uint32_t)(d0 & 0xFF) << (8 * c);
-        dig[1] |= (uint32_t)(d1 & 0xFF) << (8 * c);
-        dig[2] |= (uint32_t)(d2 & 0xFF) << (8 * c);
+        u[c] = __builtin_bit_cast(uint32_t, __builtin_fmaf(v[c], g.mult, kMagic)) - kUnbias;
+        sum += (int)u[c];
     }
+    sum -= 4 * 0x00808080;
+    const uint32_t t01 = __builtin_amdgcn_perm(u[1], u[0], 0x05010400u);  // u0.b0 u1.b0 u0.b1 u1.b1
+    const uint32_t t23 = __builtin_amdgcn_perm(u[3], u[2], 0x05010400u);
+    const uint32_t h01 = __builtin_amdgcn_perm(u[1], u[0], 0x0C0C0602u);  // u0.b2 u1.b2 0 0
+    const uint32_t h23 = __builtin_amdgcn_perm(u[3], u[2], 0x0C0C0602u);
+    dig[0] = __builtin_amdgcn_perm(t23, t01, 0x05040100u) ^ 0x80808080u;
+    dig[1] = __builtin_amdgcn_perm(t23, t01, 0x07060302u) ^ 0x80808080u;
+    dig[2] = (h01 | (h23 << 16)) ^ 0x80808080u;
+    if (g.bad) dig[0] = dig[1] = dig[2] = 0, sum = 0;  // the group's scale is NaN: its digits only have to be finite work
     return sum;
 }
 
