@@ -38,50 +38,58 @@ constexpr int kPlanes = 3;
 constexpr int kChunkBytes = 8 * 210;           // 1680 = 105 pieces of 16 bytes
 constexpr int kStageBytes = kChunkBytes + 32;  // a chunk that starts up to 14 bytes into its first piece, plus one dword for the shifted reads
 
-// Activations -> LDS.  Thread idx converts elements 4 idx .. 4 idx + 3; the four threads of a quad hold one
-// 16-element group.  Element e = 256 sb + 128 hh + 32 g + l belongs to lane t = 4 hh + 2 (g & 1) + l / 16 of its
-// super-block (slot 8 sb + t), sub-block s = g >> 1 of that lane, dword (l % 16) / 4.
+// Activations -> LDS.  A thread converts one 16-element group (one Q6_K sub-block): the group's largest magnitude and
+// the sum of its fixed-point values stay inside the thread, and the index arithmetic is done once per group.
+// Element e = 256 sb + 128 hh + 32 g + l belongs to lane t = 4 hh + 2 (g & 1) + l / 16 of its super-block
+// (slot 8 sb + t), sub-block s = g >> 1 of that lane, dword (l % 16) / 4.
 // xd[(plane * 8 + 4 s + dword) * slots + slot]: four digits; xm[slot] = (scale s = 0, scale s = 1, sum s = 0, sum s = 1).
 // Slots past the end of a row (its last chunk may hold fewer than eight super-blocks) get zero digits and a zero scale.
 template <bool XF32>
 __device__ __forceinline__ void stage_x(const void *__restrict__ xg, int slots, int k_quads, int nthreads, uint32_t *xd, float *xm) {
-    const int total = slots * 8;  // quads of four elements, padded to whole chunks; k_quads = k / 4 of them exist
-    for (int idx0 = 0; idx0 < total; idx0 += nthreads) {
-        const int idx = idx0 + (int)threadIdx.x;
-        const bool live = idx < total;
-        const int id = live ? idx : total - 1;
-        float v[4] = {0.f, 0.f, 0.f, 0.f};
-        if (id >= k_quads) {
-        } else if (XF32) {
-            const float4 f = reinterpret_cast<const float4 *>(xg)[id];
-            v[0] = f.x, v[1] = f.y, v[2] = f.z, v[3] = f.w;
-        } else {
-            const uint2 b = reinterpret_cast<const uint2 *>(xg)[id];
-            v[0] = __builtin_bit_cast(float, b.x << 16), v[1] = __builtin_bit_cast(float, b.x & 0xFFFF0000u);
-            v[2] = __builtin_bit_cast(float, b.y << 16), v[3] = __builtin_bit_cast(float, b.y & 0xFFFF0000u);
-        }
-        // largest magnitude of the 16-element group, as bits (the order of non-negative floats is that of their bits)
-        uint32_t mb = max_magnitude_bits(v);  // then over the lanes that share the group
-        uint32_t o = (uint32_t)__shfl_xor((int)mb, 1);
-        mb = o > mb ? o : mb;
-        o = (uint32_t)__shfl_xor((int)mb, 2);
-        mb = o > mb ? o : mb;
-        const GroupScale gs = group_scale(mb);
-        uint32_t dig[kPlanes];
-        int sum = to_digits(v, gs, dig);
-        sum += __shfl_xor(sum, 1);
-        sum += __shfl_xor(sum, 2);
-        if (live) {
-            const int e = id * 4, sb = e >> 8, r = e & 255;
-            const int hh = r >> 7, g = (r >> 5) & 3, l = r & 31;
-            const int slot = sb * 8 + 4 * hh + 2 * (g & 1) + (l >> 4), s = g >> 1, dw = (l & 15) >> 2;
+    const int total = slots * 2, k_groups = k_quads >> 2;  // groups, padded to whole chunks; k_groups of them exist
+    for (int grp = (int)threadIdx.x; grp < total; grp += nthreads) {
+        float v[4][4];
+        if (grp >= k_groups) {
 #pragma unroll
-            for (int p = 0; p < kPlanes; p++) xd[(p * 8 + 4 * s + dw) * slots + slot] = dig[p];
-            if (dw == 0) {
-                xm[slot * 4 + s] = gs.scale;
-                xm[slot * 4 + 2 + s] = (float)sum;
+            for (int q = 0; q < 4; q++) v[q][0] = v[q][1] = v[q][2] = v[q][3] = 0.f;
+        } else if (XF32) {
+            const float4 *src = reinterpret_cast<const float4 *>(xg) + (size_t)grp * 4;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const float4 f = src[q];
+                v[q][0] = f.x, v[q][1] = f.y, v[q][2] = f.z, v[q][3] = f.w;
+            }
+        } else {
+            const uint4 *src = reinterpret_cast<const uint4 *>(xg) + (size_t)grp * 2;
+            const uint4 a = src[0], b = src[1];
+            const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                v[q][0] = __builtin_bit_cast(float, w[2 * q] << 16), v[q][1] = __builtin_bit_cast(float, w[2 * q] & 0xFFFF0000u);
+                v[q][2] = __builtin_bit_cast(float, w[2 * q + 1] << 16), v[q][3] = __builtin_bit_cast(float, w[2 * q + 1] & 0xFFFF0000u);
             }
         }
+        // largest magnitude of the group, as bits (the order of non-negative floats is that of their bits)
+        uint32_t mb = 0;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const uint32_t o = max_magnitude_bits(v[q]);
+            mb = o > mb ? o : mb;
+        }
+        const GroupScale gs = group_scale(mb);
+        const int e = grp * 16, sb = e >> 8, r = e & 255;
+        const int hh = r >> 7, g = (r >> 5) & 3;
+        const int slot = sb * 8 + 4 * hh + 2 * (g & 1) + ((r >> 4) & 1), s = g >> 1;
+        int sum = 0;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            uint32_t dig[kPlanes];
+            sum += to_digits(v[q], gs, dig);
+#pragma unroll
+            for (int p = 0; p < kPlanes; p++) xd[(p * 8 + 4 * s + q) * slots + slot] = dig[p];
+        }
+        xm[slot * 4 + s] = gs.scale;
+        xm[slot * 4 + 2 + s] = (float)sum;
     }
 }
 

@@ -35,42 +35,60 @@ constexpr int kPlanes = 3;
 constexpr int kChunkBytes = 64 * 34;          // 2176 = 136 pieces of 16 bytes
 constexpr int kStageBytes = kChunkBytes + 16;  // the ninth dword of the last lane lies past the chunk
 
-// Activations -> LDS.  Thread idx converts elements 4 idx .. 4 idx + 3; eight consecutive threads hold one block.
+// Activations -> LDS.  Thread idx converts elements 16 idx .. 16 idx + 15; two consecutive threads hold one block.
 // xd[(plane * 8 + dword) * slots + block]: four digits; xm[block] = the block's scale.
 // Blocks past the end of a row (its last chunk may hold fewer than 64 blocks) get zero digits and a zero scale.
 template <bool XF32>
 __device__ __forceinline__ void stage_x(const void *__restrict__ xg, int slots, int k_quads, int nthreads, uint32_t *xd, float *xm) {
-    const int total = slots * 8;  // quads of four elements, padded to whole chunks; k_quads = k / 4 of them exist
+    // a thread converts half a block (16 elements: dwords 4 hf .. 4 hf + 3 of the block's digits); the two threads of a
+    // block are neighbours in a wave and exchange their largest magnitudes
+    const int total = slots * 2, k_halves = k_quads >> 2;  // half blocks, padded to whole chunks; k_halves of them exist
     for (int idx0 = 0; idx0 < total; idx0 += nthreads) {
         const int idx = idx0 + (int)threadIdx.x;
         const bool live = idx < total;
         const int id = live ? idx : total - 1;
-        float v[4] = {0.f, 0.f, 0.f, 0.f};
-        if (id >= k_quads) {
+        float v[4][4];
+        if (id >= k_halves) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) v[q][0] = v[q][1] = v[q][2] = v[q][3] = 0.f;
         } else if (XF32) {
-            const float4 f = reinterpret_cast<const float4 *>(xg)[id];
-            v[0] = f.x, v[1] = f.y, v[2] = f.z, v[3] = f.w;
+            const float4 *src = reinterpret_cast<const float4 *>(xg) + (size_t)id * 4;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const float4 f = src[q];
+                v[q][0] = f.x, v[q][1] = f.y, v[q][2] = f.z, v[q][3] = f.w;
+            }
         } else {
-            const uint2 b = reinterpret_cast<const uint2 *>(xg)[id];
-            v[0] = __builtin_bit_cast(float, b.x << 16), v[1] = __builtin_bit_cast(float, b.x & 0xFFFF0000u);
-            v[2] = __builtin_bit_cast(float, b.y << 16), v[3] = __builtin_bit_cast(float, b.y & 0xFFFF0000u);
+            const uint4 *src = reinterpret_cast<const uint4 *>(xg) + (size_t)id * 2;
+            const uint4 a = src[0], b = src[1];
+            const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                v[q][0] = __builtin_bit_cast(float, w[2 * q] << 16), v[q][1] = __builtin_bit_cast(float, w[2 * q] & 0xFFFF0000u);
+                v[q][2] = __builtin_bit_cast(float, w[2 * q + 1] << 16), v[q][3] = __builtin_bit_cast(float, w[2 * q + 1] & 0xFFFF0000u);
+            }
         }
         // largest magnitude of the block, as bits (the order of non-negative floats is that of their bits)
-        uint32_t mb = max_magnitude_bits(v);  // then over the lanes that share the group
+        uint32_t mb = 0;
 #pragma unroll
-        for (int off = 1; off < 8; off <<= 1) {
-            const uint32_t o = (uint32_t)__shfl_xor((int)mb, off);
+        for (int q = 0; q < 4; q++) {
+            const uint32_t o = max_magnitude_bits(v[q]);
             mb = o > mb ? o : mb;
         }
+        const uint32_t o = (uint32_t)__shfl_xor((int)mb, 1);
+        mb = o > mb ? o : mb;
         const GroupScale gs = group_scale(mb);
-        uint32_t dig[kPlanes];
-        to_digits(v, gs, dig);
-        if (live) {
-            const int blk = id >> 3, dw = id & 7;
+        const int blk = id >> 1, hf = id & 1;
 #pragma unroll
-            for (int p = 0; p < kPlanes; p++) xd[(p * 8 + dw) * slots + blk] = dig[p];
-            if (dw == 0) xm[blk] = gs.scale;
+        for (int q = 0; q < 4; q++) {
+            uint32_t dig[kPlanes];
+            to_digits(v[q], gs, dig);
+            if (live) {
+#pragma unroll
+                for (int p = 0; p < kPlanes; p++) xd[(p * 8 + 4 * hf + q) * slots + blk] = dig[p];
+            }
         }
+        if (live && hf == 0) xm[blk] = gs.scale;
     }
 }
 
