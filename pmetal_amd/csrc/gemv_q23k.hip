@@ -39,42 +39,49 @@ constexpr int kPlanes = 3;
 // Element of group p (0..3), position i (0..7), of lane t of super-block sb.
 __device__ __forceinline__ int element_of(int sb, int t, int p, int i) { return 256 * sb + 128 * (t >> 2) + 32 * p + 8 * (t & 3) + i; }
 
-// Activations -> LDS, two threads per 8-element group (thread c of the pair converts positions 4 c .. 4 c + 3, i.e. digit
-// dword c).  Groups past the end of a row (its last chunk may hold fewer than eight super-blocks) get zero digits, scale
-// and sum.
+// Activations -> LDS.  A thread converts one group of eight consecutive elements (digit dwords 0 and 1 of the group): the
+// group's largest magnitude and the sum of its fixed-point values stay inside the thread.  Groups past the end of a row
+// (its last chunk may hold fewer than eight super-blocks) get zero digits, scale and sum.
 // xd[(plane * 8 + 2 p + dword) * slots + slot]: four digits; xm[slot * 8 + p] = scale of group p, xm[slot * 8 + 4 + p] = its
 // sum of x.
 template <bool XF32>
 __device__ __forceinline__ void stage_x(const void *__restrict__ xg, int slots, int spr, int nthreads, uint32_t *xd, float *xm) {
-    const int total = slots * 8;  // quads of four positions
-    for (int idx0 = 0; idx0 < total; idx0 += nthreads) {
-        const int idx = idx0 + (int)threadIdx.x;
-        const bool live = idx < total;
-        const int id = live ? idx : total - 1;
-        const int c = id & 1, p = (id >> 1) & 3, slot = id >> 3, sb = slot >> 3, t = slot & 7;
-        float v[4];
+    const int total = slots * 4;
+    for (int grp = (int)threadIdx.x; grp < total; grp += nthreads) {
+        const int p = grp & 3, slot = grp >> 2, sb = slot >> 3, t = slot & 7;
+        const int first = element_of(sb, t, p, 0);
+        float v[2][4];
+        if (sb >= spr) {
 #pragma unroll
-        for (int cc = 0; cc < 4; cc++) {
-            const int e = element_of(sb, t, p, 4 * c + cc);
-            if (sb >= spr) v[cc] = 0.0f;
-            else if (XF32) v[cc] = reinterpret_cast<const float *>(xg)[e];
-            else v[cc] = __builtin_bit_cast(float, (uint32_t) reinterpret_cast<const uint16_t *>(xg)[e] << 16);
-        }
-        uint32_t mb = max_magnitude_bits(v);  // then over the lanes that share the group
-        const uint32_t o = (uint32_t)__shfl_xor((int)mb, 1);
-        mb = o > mb ? o : mb;
-        const GroupScale gs = group_scale(mb);
-        uint32_t dig[kPlanes];
-        int sum = to_digits(v, gs, dig);
-        sum += __shfl_xor(sum, 1);
-        if (live) {
+            for (int c = 0; c < 2; c++) v[c][0] = v[c][1] = v[c][2] = v[c][3] = 0.f;
+        } else if (XF32) {
+            const float4 *src = reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(xg) + first);
 #pragma unroll
-            for (int pl = 0; pl < kPlanes; pl++) xd[(pl * 8 + 2 * p + c) * slots + slot] = dig[pl];
-            if (c == 0) {
-                xm[slot * 8 + p] = gs.scale;
-                xm[slot * 8 + 4 + p] = (float)sum * gs.scale;
+            for (int c = 0; c < 2; c++) {
+                const float4 f = src[c];
+                v[c][0] = f.x, v[c][1] = f.y, v[c][2] = f.z, v[c][3] = f.w;
+            }
+        } else {
+            const uint4 a = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(xg) + first);
+            const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                v[c][0] = __builtin_bit_cast(float, w[2 * c] << 16), v[c][1] = __builtin_bit_cast(float, w[2 * c] & 0xFFFF0000u);
+                v[c][2] = __builtin_bit_cast(float, w[2 * c + 1] << 16), v[c][3] = __builtin_bit_cast(float, w[2 * c + 1] & 0xFFFF0000u);
             }
         }
+        const uint32_t m0 = max_magnitude_bits(v[0]), m1 = max_magnitude_bits(v[1]);
+        const GroupScale gs = group_scale(m0 > m1 ? m0 : m1);
+        int sum = 0;
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            uint32_t dig[kPlanes];
+            sum += to_digits(v[c], gs, dig);
+#pragma unroll
+            for (int pl = 0; pl < kPlanes; pl++) xd[(pl * 8 + 2 * p + c) * slots + slot] = dig[pl];
+        }
+        xm[slot * 8 + p] = gs.scale;
+        xm[slot * 8 + 4 + p] = (float)sum * gs.scale;
     }
 }
 

@@ -32,7 +32,8 @@ using namespace pmh::gemv;
 
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));  // a 16-byte piece
 
-constexpr int kDepth = 6;  // rows in flight per wave
+constexpr int kDepth = 6;      // rows in flight per wave
+constexpr int kDepthLong = 8;  // ... for the variant that holds all of a wave's seven or eight rows at once (DEEP)
 constexpr int kPre = 2;    // of which this many are requested before x is converted
 constexpr int kPlanes = 3;
 constexpr int kChunkBytes = 8 * 176;  // 1408 = 88 pieces of 16 bytes
@@ -45,44 +46,76 @@ __device__ __forceinline__ int element_of(int sb, int t, int s, int i) {
     return 256 * sb + 64 * (t >> 1) + 32 * s + 16 * (t & 1) + i;
 }
 
-// Activations -> LDS, four threads per 16-element group (thread c of the quad converts positions 4 c .. 4 c + 3, i.e.
-// digit dword c).  Groups past the end of a row (its last chunk may hold fewer than eight super-blocks) get zero digits,
-// scale and sum.
+// Activations -> LDS.  A thread converts one 16-element group: the group's largest magnitude and the sum of its
+// fixed-point values stay inside the thread.  In REF order the two groups of a lane are the even and the odd elements of
+// its 32-element sub-block (the two halves of a dword of bf16 activations); in GGML order a group is 16 consecutive
+// elements.  Groups past the end of a row (its last chunk may hold fewer than eight super-blocks) get zero digits, scale
+// and sum.
 // xd[(plane * 8 + 4 s + dword) * slots + slot]: four digits; xm[slot] = (scale A, scale B, sum of x over A, over B).
 template <int ORDER, bool XF32>
 __device__ __forceinline__ void stage_x(const void *__restrict__ xg, int slots, int spr, int nthreads, uint32_t *xd, float *xm) {
-    const int total = slots * 8;  // quads of four positions
-    for (int idx0 = 0; idx0 < total; idx0 += nthreads) {
-        const int idx = idx0 + (int)threadIdx.x;
-        const bool live = idx < total;
-        const int id = live ? idx : total - 1;
-        const int c = id & 3, s = (id >> 2) & 1, slot = id >> 3, sb = slot >> 3, t = slot & 7;
-        float v[4];
+    const int total = slots * 2;
+    for (int grp = (int)threadIdx.x; grp < total; grp += nthreads) {
+        const int s = grp & 1, slot = grp >> 1, sb = slot >> 3, t = slot & 7;
+        const int first = element_of<ORDER>(sb, t, s, 0);
+        float v[4][4];
+        if (sb >= spr) {
 #pragma unroll
-        for (int cc = 0; cc < 4; cc++) {
-            const int e = element_of<ORDER>(sb, t, s, 4 * c + cc);
-            if (sb >= spr) v[cc] = 0.0f;
-            else if (XF32) v[cc] = reinterpret_cast<const float *>(xg)[e];
-            else v[cc] = __builtin_bit_cast(float, (uint32_t) reinterpret_cast<const uint16_t *>(xg)[e] << 16);
-        }
-        uint32_t mb = max_magnitude_bits(v);  // then over the lanes that share the group
-        uint32_t o = (uint32_t)__shfl_xor((int)mb, 1);
-        mb = o > mb ? o : mb;
-        o = (uint32_t)__shfl_xor((int)mb, 2);
-        mb = o > mb ? o : mb;
-        const GroupScale gs = group_scale(mb);
-        uint32_t dig[kPlanes];
-        int sum = to_digits(v, gs, dig);
-        sum += __shfl_xor(sum, 1);
-        sum += __shfl_xor(sum, 2);
-        if (live) {
+            for (int q = 0; q < 4; q++) v[q][0] = v[q][1] = v[q][2] = v[q][3] = 0.f;
+        } else if (ORDER == 0) {
+            if (XF32) {
+                const float2 *src = reinterpret_cast<const float2 *>(reinterpret_cast<const float *>(xg) + (first - s));
 #pragma unroll
-            for (int p = 0; p < kPlanes; p++) xd[(p * 8 + 4 * s + c) * slots + slot] = dig[p];
-            if (c == 0) {
-                xm[slot * 4 + s] = gs.scale;
-                xm[slot * 4 + 2 + s] = (float)sum * gs.scale;
+                for (int q = 0; q < 4; q++)
+#pragma unroll
+                    for (int c = 0; c < 4; c++) {
+                        const float2 f = src[4 * q + c];
+                        v[q][c] = s ? f.y : f.x;
+                    }
+            } else {
+                const uint4 *src = reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(xg) + (first - s));
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const uint4 a = src[q];
+                    const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+                    for (int c = 0; c < 4; c++) v[q][c] = __builtin_bit_cast(float, s ? (w[c] & 0xFFFF0000u) : (w[c] << 16));
+                }
+            }
+        } else if (XF32) {
+            const float4 *src = reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(xg) + first);
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const float4 f = src[q];
+                v[q][0] = f.x, v[q][1] = f.y, v[q][2] = f.z, v[q][3] = f.w;
+            }
+        } else {
+            const uint4 *src = reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(xg) + first);
+            const uint4 a = src[0], b = src[1];
+            const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                v[q][0] = __builtin_bit_cast(float, w[2 * q] << 16), v[q][1] = __builtin_bit_cast(float, w[2 * q] & 0xFFFF0000u);
+                v[q][2] = __builtin_bit_cast(float, w[2 * q + 1] << 16), v[q][3] = __builtin_bit_cast(float, w[2 * q + 1] & 0xFFFF0000u);
             }
         }
+        uint32_t mb = 0;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const uint32_t o = max_magnitude_bits(v[q]);
+            mb = o > mb ? o : mb;
+        }
+        const GroupScale gs = group_scale(mb);
+        int sum = 0;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            uint32_t dig[kPlanes];
+            sum += to_digits(v[q], gs, dig);
+#pragma unroll
+            for (int p = 0; p < kPlanes; p++) xd[(p * 8 + 4 * s + q) * slots + slot] = dig[p];
+        }
+        xm[slot * 4 + s] = gs.scale;
+        xm[slot * 4 + 2 + s] = (float)sum * gs.scale;
     }
 }
 
@@ -99,11 +132,12 @@ __device__ __forceinline__ void scale_min_k4(int j, uint32_t s0, uint32_t s1, ui
 // byte that the multiplication adds up overlap in single bit positions whose carries end in unused bits.
 __device__ __forceinline__ uint32_t even_bits_to_bytes(uint32_t b) { return ((b & 0x55u) * 0x41041u) & 0x01010101u; }
 
-template <int ORDER, bool XF32, bool SINGLE>
+template <int ORDER, bool XF32, bool SINGLE, bool DEEP = false>
 __global__ __launch_bounds__(1024) void k_qgemv_q5k_chunk(const uint8_t *__restrict__ W, const void *__restrict__ xg,
                                                            float *__restrict__ y, int n_rows, int spr, int rows_per_wg,
                                                            int rows_per_wave, int n_nominal, int nthreads,
                                                            uint32_t w_last) {
+    constexpr int kDepth = DEEP ? kDepthLong : ::kDepth;
     extern __shared__ uint4 smem[];
     const int ks = (spr + 7) >> 3;
     const int slots = ks * 64;
@@ -253,6 +287,7 @@ hipError_t launch_qgemv_q5k(const uint8_t *w, int64_t n, int64_t k, const void *
                   threads = plan.threads;
     const size_t lds = plan.lds;
     if (lds > gemv::kMaxLds) return hipErrorInvalidValue;
+    const bool deep = n_nominal > kDepth && n_nominal <= kDepthLong;  // seven or eight rows per wave: all in flight at once
     const bool single = n_nominal <= kDepth;
     const bool xf32 = x_dtype == kDtypeF32;
     auto go = [&](auto kern) {
@@ -264,12 +299,10 @@ hipError_t launch_qgemv_q5k(const uint8_t *w, int64_t n, int64_t k, const void *
                            (int)rows_per_wave, (int)n_nominal, (int)threads, (uint32_t)((w_bytes - 1) & ~(uint64_t)15));
         return hipGetLastError();
     };
-    if (order == kOrderRef) {
-        if (xf32) return single ? go(k_qgemv_q5k_chunk<0, true, true>) : go(k_qgemv_q5k_chunk<0, true, false>);
-        return single ? go(k_qgemv_q5k_chunk<0, false, true>) : go(k_qgemv_q5k_chunk<0, false, false>);
-    }
-    if (xf32) return single ? go(k_qgemv_q5k_chunk<1, true, true>) : go(k_qgemv_q5k_chunk<1, true, false>);
-    return single ? go(k_qgemv_q5k_chunk<1, false, true>) : go(k_qgemv_q5k_chunk<1, false, false>);
+#define PMH_Q5K(O, F) (deep ? go(k_qgemv_q5k_chunk<O, F, true, true>) : single ? go(k_qgemv_q5k_chunk<O, F, true>) : go(k_qgemv_q5k_chunk<O, F, false>))
+    if (order == kOrderRef) return xf32 ? PMH_Q5K(0, true) : PMH_Q5K(0, false);
+    return xf32 ? PMH_Q5K(1, true) : PMH_Q5K(1, false);
+#undef PMH_Q5K
 }
 
 }  // namespace pmh
