@@ -437,7 +437,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q4k_chunk(const uint8_t *__restr
 constexpr int kRowsWaves = 8;         // waves per workgroup
 constexpr int kRowsPerWaveMax = 8;    // row totals a wave keeps in LDS (kDepth tasks of one chunk each)
 
-template <int ORDER, bool XF32, int KS, bool MULTI>
+template <int ORDER, bool XF32, int KS, bool MULTI, bool Q6LAST = false>
 __global__ __launch_bounds__(64 * kRowsWaves) void k_qgemv_q4k_rows(const void *__restrict__ xg, const uint8_t *__restrict__ w0,
                                                                      const uint8_t *__restrict__ w1, const uint8_t *__restrict__ w2,
                                                                      const uint8_t *__restrict__ w3, int wg_b1, int wg_b2, int wg_b3,
@@ -447,7 +447,15 @@ __global__ __launch_bounds__(64 * kRowsWaves) void k_qgemv_q4k_rows(const void *
     // Up to four matrices that share k and the activation vector go through one launch (MULTI): workgroups
     // [wg_b(g), wg_b(g + 1)) belong to matrix g (workgroup-uniform selects); otherwise only w0, n0, y0 are looked at.
     static_assert(pmh::kMaxGemvGroup == 4, "the argument list spells out four group members");
+    static_assert(MULTI || !Q6LAST, "the Q6_K member is the fourth of a group");
     const int bx = (int)blockIdx.x;
+    extern __shared__ uint4 smem[];
+    if (Q6LAST && bx >= wg_b3) {
+        // Q6LAST: the fourth member is a small Q6_K matrix over the same activations (an attention v projection beside
+        // q and k); its workgroups run the small-matrix Q6_K kernel's body, one team per wave
+        q6k_small_body<64, XF32>(w3, xg, y3, n3, spr, bx - wg_b3, (int)gridDim.x - wg_b3, kRowsWaves, smem);
+        return;
+    }
     const int g = MULTI ? (bx >= wg_b1 ? 1 : 0) + (bx >= wg_b2 ? 1 : 0) + (bx >= wg_b3 ? 1 : 0) : 0;
     const uint8_t *__restrict__ W = g == 0 ? w0 : g == 1 ? w1 : g == 2 ? w2 : w3;
     float *__restrict__ y = g == 0 ? y0 : g == 1 ? y1 : g == 2 ? y2 : y3;
@@ -455,7 +463,6 @@ __global__ __launch_bounds__(64 * kRowsWaves) void k_qgemv_q4k_rows(const void *
     const int wg_index = bx - (g == 0 ? 0 : g == 1 ? wg_b1 : g == 2 ? wg_b2 : wg_b3);
     constexpr int NDIG = XF32 ? 6 : 5;
     constexpr int T = 64, nthreads = 64 * kRowsWaves;
-    extern __shared__ uint4 smem[];
     const int slots = spr * 8;
     uint4 *xd = smem;
     float4 *xm = reinterpret_cast<float4 *>(xd + NDIG * slots);
@@ -819,22 +826,26 @@ namespace pmh {
 // suit it (rows of more than two chunks or not whole chunks, more rows per wave than the ring holds tasks, offsets beyond
 // 32 bits): the caller goes on to another kernel.
 template <int ORDER, bool XF32>
-static hipError_t launch_rows_kernel(int ks, bool multi, dim3 grid, size_t lds, hipStream_t s, const GemvGroup &grp, const void *x, int spr,
-                                     int rows_per_wg) {
+static hipError_t launch_rows_kernel(int ks, bool multi, bool q6last, dim3 grid, size_t lds, hipStream_t s, const GemvGroup &grp,
+                                     const void *x, int spr, int rows_per_wg) {
     const dim3 block(64 * kRowsWaves);
     auto go = [&](auto kern) {
         return launch_with_lds(kern, grid, block, lds, s, x, grp.w[0], grp.w[1], grp.w[2], grp.w[3], grp.wg_begin[1], grp.wg_begin[2],
                                grp.wg_begin[3], spr, rows_per_wg, grp.n[0], grp.n[1], grp.n[2], grp.n[3], grp.y[0], grp.y[1], grp.y[2],
                                grp.y[3]);
     };
+    if (q6last) return ks == 2 ? go(k_qgemv_q4k_rows<ORDER, XF32, 2, true, true>) : go(k_qgemv_q4k_rows<ORDER, XF32, 1, true, true>);
     if (ks == 2) return multi ? go(k_qgemv_q4k_rows<ORDER, XF32, 2, true>) : go(k_qgemv_q4k_rows<ORDER, XF32, 2, false>);
     return multi ? go(k_qgemv_q4k_rows<ORDER, XF32, 1, true>) : go(k_qgemv_q4k_rows<ORDER, XF32, 1, false>);
 }
 
+// w6 / n6 / y6: a small Q6_K matrix over the same activations that rides along as the fourth member (n6 == 0: none); its
+// workgroups come on top of the Q4_K members' share.
 static hipError_t launch_kernel_rows(const uint8_t *const *w, const int64_t *n, float *const *y, int count, int64_t k, const void *x,
-                                     bool xf32, uint32_t order, hipStream_t s) {
+                                     bool xf32, uint32_t order, hipStream_t s, const uint8_t *w6 = nullptr, int64_t n6 = 0,
+                                     float *y6 = nullptr) {
     const int spr = (int)(k / 256);
-    if (spr % 8 != 0 || spr / 8 > 2 || count < 1 || count > kMaxGemvGroup) return hipErrorNotSupported;
+    if (spr % 8 != 0 || spr / 8 > 2 || count < 1 || count > kMaxGemvGroup - (n6 > 0 ? 1 : 0)) return hipErrorNotSupported;
     const int ks = spr / 8;
     int64_t total = 0, n_max = 0;
     for (int i = 0; i < count; i++) total += n[i], n_max = n[i] > n_max ? n[i] : n_max;
@@ -845,6 +856,14 @@ static hipError_t launch_kernel_rows(const uint8_t *const *w, const int64_t *n, 
     const int64_t max_rows_per_wg = (int64_t)kRowsWaves * (kDepth / ks);
     int64_t want = 2 * cus;
     if (count > 1 && (total + want - 1) / want > max_rows_per_wg) want = 4 * cus;
+    // the Q6_K member: a team (one wave) walks two rows at a time, so one workgroup per 16 rows, at most half of all
+    int64_t wgs6 = 0;
+    if (n6 > 0) {
+        if ((uint64_t)n6 * (uint64_t)spr * 210u >= (1ull << 31)) return hipErrorNotSupported;
+        wgs6 = (n6 + 2 * kRowsWaves - 1) / (2 * kRowsWaves);
+        wgs6 = wgs6 > want / 2 ? want / 2 : wgs6;
+        want -= wgs6;
+    }
     int64_t n_wg = total < want ? total : want;
     int64_t rows_per_wg = (total + n_wg - 1) / n_wg;
     // every member rounds its workgroup count up: keep the sum within the intended number of workgroups
@@ -868,14 +887,20 @@ static hipError_t launch_kernel_rows(const uint8_t *const *w, const int64_t *n, 
     }
     grp.wg_begin[kMaxGemvGroup] = begin;
     const size_t slots = (size_t)spr * 8;
-    const size_t lds = slots * 16 * (xf32 ? 6 : 5) + slots * 16 + (size_t)kRowsWaves * kRowsPerWaveMax * 4;
-    const dim3 grid((unsigned)begin);
-    const bool multi = count > 1;
+    size_t lds = slots * 16 * (xf32 ? 6 : 5) + slots * 16 + (size_t)kRowsWaves * kRowsPerWaveMax * 4;
+    const bool q6last = n6 > 0;
+    if (q6last) {  // (the unused members before it hold no workgroups: wg_begin[count .. 3] are all `begin`)
+        grp.w[kMaxGemvGroup - 1] = w6, grp.y[kMaxGemvGroup - 1] = y6, grp.n[kMaxGemvGroup - 1] = (int)n6;
+        const size_t lds6 = slots * 64 * (xf32 ? 3 : 1) + slots * 16;
+        lds = lds6 > lds ? lds6 : lds;
+    }
+    const dim3 grid((unsigned)(begin + wgs6));
+    const bool multi = count > 1 || q6last;
     if (order == kOrderRef)
-        return xf32 ? launch_rows_kernel<0, true>(ks, multi, grid, lds, s, grp, x, spr, (int)rows_per_wg)
-                    : launch_rows_kernel<0, false>(ks, multi, grid, lds, s, grp, x, spr, (int)rows_per_wg);
-    return xf32 ? launch_rows_kernel<1, true>(ks, multi, grid, lds, s, grp, x, spr, (int)rows_per_wg)
-                : launch_rows_kernel<1, false>(ks, multi, grid, lds, s, grp, x, spr, (int)rows_per_wg);
+        return xf32 ? launch_rows_kernel<0, true>(ks, multi, q6last, grid, lds, s, grp, x, spr, (int)rows_per_wg)
+                    : launch_rows_kernel<0, false>(ks, multi, q6last, grid, lds, s, grp, x, spr, (int)rows_per_wg);
+    return xf32 ? launch_rows_kernel<1, true>(ks, multi, q6last, grid, lds, s, grp, x, spr, (int)rows_per_wg)
+                : launch_rows_kernel<1, false>(ks, multi, q6last, grid, lds, s, grp, x, spr, (int)rows_per_wg);
 }
 
 // Kernel A over one matrix (n1 == 0) or two that share k, x and the element order.  hipErrorNotSupported when the shape
@@ -963,8 +988,13 @@ hipError_t launch_qgemv_q4k_q6k_group(const uint8_t *const *w, const int64_t *n,
                                       float *y6, int64_t k, const void *x, uint32_t x_dtype, uint32_t order, hipStream_t s) {
     uint64_t bytes = (uint64_t)n6 * (uint64_t)(k / 256) * 210u;
     for (int i = 0; i < count; i++) bytes += (uint64_t)n[i] * (uint64_t)(k / 256) * 144u;
-    if (bytes >= (8ull << 20)) return hipErrorNotSupported;  // large groups stream through the row-owner kernels
-    return launch_group_mixed(w, n, y, count, w6, n6, y6, k, x, x_dtype == kDtypeF32, order, s);
+    const bool xf32 = x_dtype == kDtypeF32;
+    if (bytes >= (8ull << 20)) {  // a large group streams through the row-owner kernel, the Q6_K member as its fourth
+        const size_t slots = (size_t)(k / 256) * 8;
+        if (slots * 16 * (xf32 ? 6 : 5) + slots * 16 > gemv::kMaxLds) return hipErrorNotSupported;
+        return launch_kernel_rows(w, n, y, count, k, x, xf32, order, s, w6, n6, y6);
+    }
+    return launch_group_mixed(w, n, y, count, w6, n6, y6, k, x, xf32, order, s);
 }
 
 hipError_t launch_qgemv_q4k_group(const uint8_t *const *w, const int64_t *n, float *const *y, int count, int64_t k,

@@ -307,6 +307,21 @@ def test_qgemv_batch_takes_a_q6k_projection_into_a_q4k_group(oracle, order, rows
     """q and k in Q4_K followed by v in Q6_K over the same x (a Q4_K_M layer): one launch.  The last of `rows` is the
     Q6_K matrix; every member against the oracle and against its own launch.  With four Q4_K members before it the
     Q6_K matrix does not fit the group and runs on its own."""
+    mixed_group_case(oracle, order, rows, k, x_dtype)
+
+
+@pytest.mark.parametrize("rows,k,x_dtype", [([4096, 1024, 1024], 4096, pm.DTYPE_BF16), ([4096, 1024, 1024], 4096, pm.DTYPE_F32),
+                                            ([8192, 2100, 517], 2048, pm.DTYPE_BF16), ([5120, 3001], 4096, pm.DTYPE_BF16),
+                                            ([3000, 1000, 1000, 4100], 4096, pm.DTYPE_BF16)])
+@pytest.mark.parametrize("order", [0, 1])
+def test_qgemv_batch_takes_a_q6k_projection_into_a_large_q4k_group(oracle, order, rows, k, x_dtype):
+    """The same with the shapes of an 8B-class model (q 4096 x 4096, k and a Q6_K v 1024 x 4096: the group streams
+    through the kernel for large matrices, the Q6_K member as its fourth), with ragged row counts, with rows of one
+    chunk, and with a Q6_K member that is larger than any Q4_K member."""
+    mixed_group_case(oracle, order, rows, k, x_dtype)
+
+
+def mixed_group_case(oracle, order, rows, k, x_dtype):
     from pmetal_amd import _lib
     lib = _lib.load()
     rng = np.random.default_rng(k + order + len(rows))
