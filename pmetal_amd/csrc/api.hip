@@ -242,13 +242,13 @@ int32_t host_pipe(HostPipe **out) {  // caller holds g_pipe_mutex
     HIP_TRY(hipGetDevice(&dev));
     HostPipe &p = g_pipes[dev];
     if (!p.ready) {
-        for (PipeSlot &sl : p.slot) {
-            HIP_TRY(hipHostMalloc((void **)&sl.h_f32, kPipeElems * sizeof(float), hipHostMallocDefault));
-            HIP_TRY(hipHostMalloc((void **)&sl.h_q, kPipeQBytes, hipHostMallocDefault));
-            HIP_TRY(hipMalloc((void **)&sl.d_f32, kPipeElems * sizeof(float)));
-            HIP_TRY(hipMalloc((void **)&sl.d_q, kPipeQBytes));
-            HIP_TRY(hipStreamCreateWithFlags(&sl.st, hipStreamNonBlocking));
-            HIP_TRY(hipEventCreateWithFlags(&sl.done, hipEventDisableTiming));
+        for (PipeSlot &sl : p.slot) {  // (a call that failed half way left what it had: only the missing pieces are made)
+            if (!sl.h_f32) HIP_TRY(hipHostMalloc((void **)&sl.h_f32, kPipeElems * sizeof(float), hipHostMallocDefault));
+            if (!sl.h_q) HIP_TRY(hipHostMalloc((void **)&sl.h_q, kPipeQBytes, hipHostMallocDefault));
+            if (!sl.d_f32) HIP_TRY(hipMalloc((void **)&sl.d_f32, kPipeElems * sizeof(float)));
+            if (!sl.d_q) HIP_TRY(hipMalloc((void **)&sl.d_q, kPipeQBytes));
+            if (!sl.st) HIP_TRY(hipStreamCreateWithFlags(&sl.st, hipStreamNonBlocking));
+            if (!sl.done) HIP_TRY(hipEventCreateWithFlags(&sl.done, hipEventDisableTiming));
         }
         p.ready = true;
     }
