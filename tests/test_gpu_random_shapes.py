@@ -212,3 +212,27 @@ def test_codec_random_lengths(oracle, t, seed):
         got = gpu_dequantize_dev(t, want_q, n, order)
         assert same_floats(got, want), (t, n, kind, order)
     assert same_floats(pm.dequantize(want_q, t, (n,)), oracle.dequantize(t, want_q, [n]))
+
+
+@pytest.mark.parametrize("t", [Q4K, Q6K, Q5K, Q3K, Q2K])
+@pytest.mark.parametrize("seed", range(8))
+def test_qgemv_q8k_random_shapes(oracle, t, seed):
+    """The integer-dot GEMV over Q8_K activations at drawn shapes: bit-identical to the reference's scalar dot products."""
+    from pmetal_amd import gguf
+    lib = pm._lib.load()
+    rng = np.random.default_rng(12000 + 40 * t + seed)
+    for _ in range(2):
+        n, k = random_shape(rng, t, 24 << 20)
+        raw = random_blocks(rng, t, n, k)
+        act = (rng.standard_normal(k) * np.repeat(np.exp(rng.uniform(-3, 3, k // 256)), 256)).astype(np.float32)
+        xq = oracle.quantize_q8k(act)
+        print(f"type {t} {n}x{k}", flush=True)
+        want = oracle.qmatvec_q8k(t, raw, n, k, xq)
+        dw, dxq = pm.DeviceBuffer.from_host(raw), pm.DeviceBuffer.from_host(xq)
+        dy = pm.DeviceBuffer(max(4 * n, 16))
+        pm.check(lib.pmetal_hip_memset(dy.ptr, 0xFF, max(4 * n, 16), None))
+        gguf.qgemv_q8k(t, dw, n, k, dxq, dy)
+        pm.check(lib.pmetal_hip_sync(None))
+        got = dy.to_host(np.float32, n)
+        bad = np.nonzero(got.view(np.uint32) != want.view(np.uint32))[0]
+        assert bad.size == 0, (t, n, k, bad[:5], got[bad[:5]], want[bad[:5]])
