@@ -260,14 +260,16 @@ __device__ __forceinline__ float lane_dot(const uint4 hdr, const uint4 qv, const
 // passes a long row needs).  All threads of the workgroup take part; the caller places the barrier.
 constexpr int kStagePre = 2;  // passes of activation loads requested up front
 
+// `live` slots hold activations (8 per super-block of a row); the slots from there to `slots` (the padding of a short last
+// chunk) are converted from zeros and read nothing.
 template <int ORDER, bool XF32>
 __device__ __forceinline__ void stage_x_begin(const void *xg, int slots, int nthreads, uint4 (&r_lo)[kStagePre],
-                                              uint4 (&r_hi)[kStagePre]) {
+                                              uint4 (&r_hi)[kStagePre], int live) {
 #pragma unroll
     for (int ps = 0; ps < kStagePre; ps++) {
         r_lo[ps] = r_hi[ps] = make_uint4(0u, 0u, 0u, 0u);
         const int idx = threadIdx.x + ps * nthreads;
-        if (idx < slots * 4) {
+        if (idx < live * 4) {
             size_t e_lo, e_hi;
             stage_offsets<ORDER>(idx, e_lo, e_hi);
             r_lo[ps] = load_x4_raw<XF32>(xg, e_lo);
@@ -278,7 +280,7 @@ __device__ __forceinline__ void stage_x_begin(const void *xg, int slots, int nth
 
 template <int ORDER, int NDIG, bool XF32>
 __device__ __forceinline__ void stage_x_finish(const void *xg, int slots, int nthreads, const uint4 (&r_lo)[kStagePre],
-                                               const uint4 (&r_hi)[kStagePre], uint4 *xd, float4 *xm) {
+                                               const uint4 (&r_hi)[kStagePre], uint4 *xd, float4 *xm, int live) {
     const int stage_total = slots * 4;
     float x_lo[4], x_hi[4];
 #pragma unroll
@@ -291,10 +293,14 @@ __device__ __forceinline__ void stage_x_finish(const void *xg, int slots, int nt
         }
     }
     for (int idx = threadIdx.x + kStagePre * nthreads; idx < stage_total; idx += nthreads) {
-        size_t e_lo, e_hi;
-        stage_offsets<ORDER>(idx, e_lo, e_hi);
-        unpack_x4<XF32>(load_x4_raw<XF32>(xg, e_lo), x_lo);
-        unpack_x4<XF32>(load_x4_raw<XF32>(xg, e_hi), x_hi);
+        uint4 a = make_uint4(0u, 0u, 0u, 0u), b = a;
+        if (idx < live * 4) {
+            size_t e_lo, e_hi;
+            stage_offsets<ORDER>(idx, e_lo, e_hi);
+            a = load_x4_raw<XF32>(xg, e_lo), b = load_x4_raw<XF32>(xg, e_hi);
+        }
+        unpack_x4<XF32>(a, x_lo);
+        unpack_x4<XF32>(b, x_hi);
         stage_convert<NDIG, XF32>(idx, x_lo, x_hi, slots, xd, xm);
     }
 }
@@ -311,9 +317,13 @@ __device__ __forceinline__ void stage_x_finish(const void *xg, int slots, int nt
 // 14336 x 4096; stores inside the streaming loop are worse: on this target they share the loads' counter, and
 // the counted waits degenerate.)
 constexpr int kDepth = 8;  // tasks in flight per wave
-constexpr int kPre = 2;    // of which this many are requested before x is converted
+constexpr int kPre = 2;    // of which this many are requested before x is converted (the row-owner kernel)
+// Kernel A requests three tasks before x is converted (against two: 4096 x 14336 9.9 -> 9.6 us, other shapes unchanged;
+// four: 9.7; the row-owner kernel is fastest at two) and then two more per task consumed until the ring is full.
+constexpr int kPreA = 3, kFillA = 2;
+static_assert(kPreA + kFillA * kDepth >= 2 * kDepth, "after the first round every task of the second is requested");
 
-template <int ORDER, bool XF32, int T, bool SINGLE, bool PAIR>
+template <int ORDER, bool XF32, int T, bool SINGLE, bool PAIR, bool RAGGED = false>
 __global__ __launch_bounds__(1024) void k_qgemv_q4k_chunk(const uint8_t *__restrict__ W0, const uint8_t *__restrict__ W1,
                                                            const void *__restrict__ xg, int split_wg, int n_rows0, int n_rows1,
                                                            int spr, int rows_per_wg, int rows_per_wave, int n_nominal,
@@ -331,15 +341,19 @@ __global__ __launch_bounds__(1024) void k_qgemv_q4k_chunk(const uint8_t *__restr
     constexpr int NDIG = XF32 ? 6 : 5;
     constexpr int SEG = T / 8;   // super-blocks a team covers
     constexpr int RPT = 64 / T;  // rows per task
+    // RAGGED (T = 64 only): rows that are not whole chunks of eight super-blocks and have too many of them for a
+    // narrower team (k = 11008, 13824, 18944, ...).  The last chunk of a row is short: its missing super-blocks get zero
+    // activations, their lanes read the row's first block and contribute nothing.
+    static_assert(!RAGGED || T == 64, "short last chunks exist for whole-wave teams only");
     extern __shared__ uint4 smem[];
-    const int slots = spr * 8;
+    const int ks = RAGGED ? (spr + SEG - 1) / SEG : spr / SEG;
+    const int slots = RAGGED ? ks * 64 : spr * 8;
     uint4 *xd = smem;
     float4 *xm = reinterpret_cast<float4 *>(xd + NDIG * slots);
     float *part = reinterpret_cast<float *>(xm + slots);  // [group][n_nominal * RPT][ks]
     const int lane = threadIdx.x & 63;
     const int lt = lane & (T - 1), tm = lane / T, j = lane & 7;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const int ks = spr / SEG;
     const int h = wave % ks, g = wave / ks;
     const int wg_r0 = wg_index * rows_per_wg;
     const int wg_r1 = wg_r0 + rows_per_wg < n_rows ? wg_r0 + rows_per_wg : n_rows;
@@ -349,7 +363,8 @@ __global__ __launch_bounds__(1024) void k_qgemv_q4k_chunk(const uint8_t *__restr
     const int nt_wave = (rows_here + RPT - 1) / RPT;  // real tasks of this wave (wave-uniform)
 
     const uint32_t rowbytes = (uint32_t)spr * 144u;
-    const uint32_t chunk_off = (uint32_t)(h * SEG + (lt >> 3)) * 144u;
+    const bool lane_valid = !RAGGED || h * SEG + (lt >> 3) < spr;
+    const uint32_t chunk_off = lane_valid ? (uint32_t)(h * SEG + (lt >> 3)) * 144u : 0u;
     const uint32_t chunk_qoff = chunk_off + 16u + 16u * (uint32_t)j;
     auto issue = [&](int t, uint4 &h4, uint4 &q4) {
         const bool real = t < nt_wave;  // wave-uniform
@@ -361,11 +376,11 @@ __global__ __launch_bounds__(1024) void k_qgemv_q4k_chunk(const uint8_t *__restr
     };
 
     uint4 x_lo[kStagePre], x_hi[kStagePre];
-    stage_x_begin<ORDER, XF32>(xg, slots, nthreads, x_lo, x_hi);
+    stage_x_begin<ORDER, XF32>(xg, slots, nthreads, x_lo, x_hi, spr * 8);
     uint4 bh[kDepth], bq[kDepth];
 #pragma unroll
-    for (int i = 0; i < kPre; i++) issue(i, bh[i], bq[i]);
-    stage_x_finish<ORDER, NDIG, XF32>(xg, slots, nthreads, x_lo, x_hi, xd, xm);
+    for (int i = 0; i < kPreA; i++) issue(i, bh[i], bq[i]);
+    stage_x_finish<ORDER, NDIG, XF32>(xg, slots, nthreads, x_lo, x_hi, xd, xm, spr * 8);
     __syncthreads();
 
     const ScaleSel s0 = scale_sel(ORDER == 0 ? j : 2 * (j >> 1));
@@ -382,19 +397,20 @@ __global__ __launch_bounds__(1024) void k_qgemv_q4k_chunk(const uint8_t *__restr
 
     auto consume = [&](int t, const uint4 &h4, const uint4 &q4) {
         if (t < nt_wave) {
-            const float v = team_sum_last<T>(lane_dot<ORDER, NDIG>(h4, q4, s0, s1, xr, xmr));
+            const float mine = lane_dot<ORDER, NDIG>(h4, q4, s0, s1, xr, xmr);
+            const float v = team_sum_last<T>(RAGGED && !lane_valid ? 0.0f : mine);
             if (lt == T - 1) pp[(size_t)t * pstride] = v;
         }
     };
 
-    // First round: the ring fills up while the first tasks are consumed (two requests per task consumed),
+    // First round: the ring fills up while the first tasks are consumed (kFillA more requests per task consumed),
     // so no wave sits in front of the load unit with nothing to compute.
-    int issued = kPre;
+    int issued = kPreA;
 #pragma unroll
     for (int i = 0; i < kDepth; i++) {
         consume(i, bh[i], bq[i]);
-        const int upto = SINGLE ? (kPre + 2 * (i + 1) < kDepth ? kPre + 2 * (i + 1) : kDepth)
-                                : (kPre + 2 * (i + 1) < kDepth + i + 1 ? kPre + 2 * (i + 1) : kDepth + i + 1);
+        const int upto = SINGLE ? (kPreA + kFillA * (i + 1) < kDepth ? kPreA + kFillA * (i + 1) : kDepth)
+                                : (kPreA + kFillA * (i + 1) < kDepth + i + 1 ? kPreA + kFillA * (i + 1) : kDepth + i + 1);
 #pragma unroll
         for (; issued < upto; issued++) issue(issued, bh[issued % kDepth], bq[issued % kDepth]);
     }
@@ -489,11 +505,11 @@ __global__ __launch_bounds__(64 * kRowsWaves) void k_qgemv_q4k_rows(const void *
         q4 = *reinterpret_cast<const uint4 *>(W + (ro + (real ? 16u + 16u * (uint32_t)j : 0u)));
     };
     uint4 x_lo[kStagePre], x_hi[kStagePre];
-    stage_x_begin<ORDER, XF32>(xg, slots, nthreads, x_lo, x_hi);
+    stage_x_begin<ORDER, XF32>(xg, slots, nthreads, x_lo, x_hi, slots);
     uint4 bh[kDepth], bq[kDepth];
 #pragma unroll
     for (int i = 0; i < kPre; i++) issue(i, bh[i], bq[i]);
-    stage_x_finish<ORDER, NDIG, XF32>(xg, slots, nthreads, x_lo, x_hi, xd, xm);
+    stage_x_finish<ORDER, NDIG, XF32>(xg, slots, nthreads, x_lo, x_hi, xd, xm, slots);
     __syncthreads();
     const ScaleSel s0 = scale_sel(ORDER == 0 ? j : 2 * (j >> 1));
     const ScaleSel s1 = scale_sel(ORDER == 0 ? j : 2 * (j >> 1) + 1);
@@ -600,7 +616,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q4k(const void *__restrict__ xg,
     // kRing tasks are in flight per team.  They are requested before x is converted, so the memory system
     // streams while the staging runs, and each buffer is refilled as soon as it has been consumed.
     uint4 x_lo[kStagePre], x_hi[kStagePre];
-    stage_x_begin<ORDER, XF32>(xg, slots, nthreads, x_lo, x_hi);
+    stage_x_begin<ORDER, XF32>(xg, slots, nthreads, x_lo, x_hi, slots);
     uint4 bh[kRing], bq[kRing];
 #pragma unroll
     for (int i = 0; i < kRing; i++) {
@@ -609,7 +625,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q4k(const void *__restrict__ xg,
             bq[i] = *reinterpret_cast<const uint4 *>(pq + i * STRIDE);
         }
     }
-    stage_x_finish<ORDER, NDIG, XF32>(xg, slots, nthreads, x_lo, x_hi, xd, xm);
+    stage_x_finish<ORDER, NDIG, XF32>(xg, slots, nthreads, x_lo, x_hi, xd, xm, slots);
     __syncthreads();
 
     const ScaleSel s0 = scale_sel(ORDER == 0 ? j : 2 * (j >> 1));
@@ -661,7 +677,18 @@ hipError_t launch_with_lds(Kern kern, dim3 grid, dim3 block, size_t lds, hipStre
 template <int ORDER, bool XF32>
 hipError_t launch_chunk(int T, bool single, dim3 grid, dim3 block, size_t lds, hipStream_t s, const uint8_t *w,
                         const void *x, float *y, int n, int spr, int rows_per_wg, int rows_per_wave, int n_nominal,
-                        const uint8_t *w1, int split_wg, float *y1, int n1) {
+                        const uint8_t *w1, int split_wg, float *y1, int n1, bool ragged) {
+    if (ragged) {
+        if (n1 > 0)
+            return single ? launch_with_lds(k_qgemv_q4k_chunk<ORDER, XF32, 64, true, true, true>, grid, block, lds, s, w, w1, x, split_wg, n,
+                                            n1, spr, rows_per_wg, rows_per_wave, n_nominal, (int)block.x, y, y1)
+                          : launch_with_lds(k_qgemv_q4k_chunk<ORDER, XF32, 64, false, true, true>, grid, block, lds, s, w, w1, x, split_wg, n,
+                                            n1, spr, rows_per_wg, rows_per_wave, n_nominal, (int)block.x, y, y1);
+        return single ? launch_with_lds(k_qgemv_q4k_chunk<ORDER, XF32, 64, true, false, true>, grid, block, lds, s, w, w1, x, split_wg, n, n1,
+                                        spr, rows_per_wg, rows_per_wave, n_nominal, (int)block.x, y, y1)
+                      : launch_with_lds(k_qgemv_q4k_chunk<ORDER, XF32, 64, false, false, true>, grid, block, lds, s, w, w1, x, split_wg, n, n1,
+                                        spr, rows_per_wg, rows_per_wave, n_nominal, (int)block.x, y, y1);
+    }
 #define PMH_GO(TT)                                                                                                       \
     if (n1 > 0)                                                                                                                    \
         return single ? launch_with_lds(k_qgemv_q4k_chunk<ORDER, XF32, TT, true, true>, grid, block, lds, s, w, w1, x, split_wg, n, n1,  \
@@ -908,16 +935,20 @@ static hipError_t launch_kernel_rows(const uint8_t *const *w, const int64_t *n, 
 static hipError_t launch_kernel_a(const uint8_t *w0, int64_t n0, float *y0, const uint8_t *w1, int64_t n1, float *y1, int64_t k,
                                   const void *x, bool xf32, uint32_t order, hipStream_t s) {
     const int spr = (int)(k / 256);
-    const int T = 8 * gemv::pow2_divisor(spr, 8);
-    const size_t slots = (size_t)spr * 8;
+    int T = 8 * gemv::pow2_divisor(spr, 8);
+    // rows that a narrower team would cut into more than 16 chunks: whole-wave teams with a short last chunk
+    const bool ragged = T < 64 && spr / (T / 8) > 16 && (spr + 7) / 8 <= 16;
+    if (ragged) T = 64;
+    const size_t slots = ragged ? (size_t)((spr + 7) / 8) * 64 : (size_t)spr * 8;
     const size_t lds_x = slots * 16 * (xf32 ? 6 : 5) + slots * 16;
+    if (lds_x > gemv::kMaxLds) return hipErrorNotSupported;
     // Workgroups own contiguous chunks of rows, one per compute unit (x is staged once per workgroup).
     const int64_t n = n0 + n1, want = gemv::compute_units();
     int64_t n_wg = n < want ? n : want;
     const int64_t rows_per_wg = (n + n_wg - 1) / n_wg;
     const int64_t wg0 = (n0 + rows_per_wg - 1) / rows_per_wg, wg1 = (n1 + rows_per_wg - 1) / rows_per_wg;
     const dim3 grid((unsigned)(wg0 + wg1));
-    const int ks = spr / (T / 8), rpt = 64 / T;
+    const int ks = ragged ? (spr + 7) / 8 : spr / (T / 8), rpt = 64 / T;
     const uint64_t w_max = (uint64_t)(n0 > n1 ? n0 : n1) * (uint64_t)spr * 144u;
     if (ks > 16 || w_max >= (1ull << 32)) return hipErrorNotSupported;
     int64_t groups = 16 / ks;
@@ -936,10 +967,10 @@ static hipError_t launch_kernel_a(const uint8_t *w0, int64_t n0, float *y0, cons
     float *b_y = n1 ? y1 : y0;
     const int b_split = (int)wg0, b_n = (int)n1;
     if (order == kOrderRef)
-        return xf32 ? launch_chunk<0, true>(T, single, grid, block, lds, s, w0, x, y0, a_n, spr, a_rpw, a_rpv, a_nn, b_w, b_split, b_y, b_n)
-                    : launch_chunk<0, false>(T, single, grid, block, lds, s, w0, x, y0, a_n, spr, a_rpw, a_rpv, a_nn, b_w, b_split, b_y, b_n);
-    return xf32 ? launch_chunk<1, true>(T, single, grid, block, lds, s, w0, x, y0, a_n, spr, a_rpw, a_rpv, a_nn, b_w, b_split, b_y, b_n)
-                : launch_chunk<1, false>(T, single, grid, block, lds, s, w0, x, y0, a_n, spr, a_rpw, a_rpv, a_nn, b_w, b_split, b_y, b_n);
+        return xf32 ? launch_chunk<0, true>(T, single, grid, block, lds, s, w0, x, y0, a_n, spr, a_rpw, a_rpv, a_nn, b_w, b_split, b_y, b_n, ragged)
+                    : launch_chunk<0, false>(T, single, grid, block, lds, s, w0, x, y0, a_n, spr, a_rpw, a_rpv, a_nn, b_w, b_split, b_y, b_n, ragged);
+    return xf32 ? launch_chunk<1, true>(T, single, grid, block, lds, s, w0, x, y0, a_n, spr, a_rpw, a_rpv, a_nn, b_w, b_split, b_y, b_n, ragged)
+                : launch_chunk<1, false>(T, single, grid, block, lds, s, w0, x, y0, a_n, spr, a_rpw, a_rpv, a_nn, b_w, b_split, b_y, b_n, ragged);
 }
 
 // Preconditions as for launch_qgemv.  Returns hipErrorInvalidValue when x does not fit in LDS.

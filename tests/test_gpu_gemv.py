@@ -53,7 +53,9 @@ def test_qgemv_matches_dequantize_then_matmul(oracle, t, n, k, x_dtype):
 # other row length go to the chunk-owner kernel: 32-lane teams (k / 256 = 12), a row count below the number of compute
 # units times the waves, and a row of 16 chunks (k = 32768).
 BIG_CASES = [(6001, 4096), (7301, 3072), (3001, 8192), (16385, 1536), (800, 32768), (12001, 2048), (32767, 2048),
-             (20000, 4096), (40001, 2048)]
+             (20000, 4096), (40001, 2048),
+             # rows of 43, 54, 74, 17 and 34 super-blocks: whole-wave teams with a short last chunk
+             (4096, 11008), (3001, 13824), (2500, 18944), (5003, 4352), (3001, 8704)]
 
 
 @pytest.mark.parametrize("n,k", BIG_CASES)
