@@ -1171,6 +1171,9 @@ GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k) {
     // for the same number of workgroups: 36.9 against 38.3 us at M = 128, 51.7 against 53.8 at M = 192, 14336x4096;
     // equal at 256, and from 320 rows on the larger block wins)
     p.mb = m <= 32 ? 1 : (m <= 192 ? 2 : 4);
+    // few tiles (a narrow weight: k / v projections of 1024 or 2048 rows): 64-row blocks double them and halve the K
+    // splits (M = 512: 1024 x 4096 28.7 -> 25.3 us, 2048 x 4096 33.8 -> 30.5; equal from 64 tiles on)
+    if (p.mb == 4 && ((n + 255) / 256) * ((m + 127) / 128) <= 32) p.mb = 2;
     p.mp = (m + 32 * p.mb - 1) / (32 * p.mb) * (32 * p.mb);
     p.nw = 8;
     const int64_t spr = k / 256;
