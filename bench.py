@@ -644,6 +644,10 @@ WORKLOADS["gemm_q6k_m512"] = dict(kind="gemm", m=512, n=14336, k=4096, metric="Q
                                   unit="TFLOP/s", dtype="f16", type=Q6K)
 WORKLOADS["gemm_q8_0_m512"] = dict(kind="gemm", m=512, n=14336, k=4096, metric="Q8_0 GEMM TFLOPS @M=512,K=4096,N=14336",
                                    unit="TFLOP/s", dtype="f16", type=Q8_0)
+WORKLOADS["gemm_q8_0_m16"] = dict(kind="gemm", m=16, n=14336, k=4096, metric="Q8_0 GEMM TFLOPS @M=16,K=4096,N=14336",
+                                  unit="TFLOP/s", dtype="f16", type=Q8_0)
+WORKLOADS["gemm_q6k_m16"] = dict(kind="gemm", m=16, n=14336, k=4096, metric="Q6_K GEMM TFLOPS @M=16,K=4096,N=14336",
+                                 unit="TFLOP/s", dtype="f16", type=Q6K)
 for _name, _t in (("q5k", 13), ("q3k", 11), ("q2k", 10)):  # re-blocked into Q6_K inside the call (two tensors, one, two)
     WORKLOADS[f"gemm_{_name}_m512"] = dict(kind="gemm", m=512, n=14336, k=4096, unit="TFLOP/s", dtype="f16", type=_t,
                                            metric=f"{_name.upper().replace('K', '_K')} GEMM TFLOPS (nominal flops) @M=512,K=4096,N=14336")

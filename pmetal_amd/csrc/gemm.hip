@@ -1084,6 +1084,153 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t 
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// The same for Q8_0 (34-byte blocks: f16 d, 32 int8).  A k-step of v_mfma_f32_16x16x32_f16 is one block: lane (r, kg)
+// holds the eight quants 8 kg .. 8 kg + 7 of the block of weight row r, exact in f16, and the block's d multiplies the
+// fp32 product tile of that one k-step.  A wave owns one or two runs of eight blocks (256 elements = 272 bytes) of every
+// row, as the Q4_K kernel owns super-blocks.  Nothing in a row of 34-byte blocks is aligned to more than two bytes, and
+// loads at such addresses are slow, so the wave copies the 16 x 272 bytes of a row tile's run -- 16-byte aligned at both
+// ends -- through registers into its own piece of LDS with whole-wave 16-byte loads (the ring holds these pieces) and
+// every lane takes its quants and scales out of LDS: aligned dwords, those of the even blocks shifted by two bytes.  LDS
+// executes a wave's instructions in order, so the copy needs no barrier.  Ring, reduction over the waves and epilogue
+// as above.
+// ------------------------------------------------------------------------------------------------
+constexpr int kQ8RunBytes = 272, kQ8TileRunPieces = 16 * kQ8RunBytes / 16;  // 272 pieces of 16 bytes: 4.25 per lane
+
+// (one run's pieces: a tile of two runs is two of these, kept apart so that each stays in registers)
+struct SmallRunQ8 {
+    u32x4 piece[5];  // (a vector type: copies of it are loads and stores that stay in registers)
+};
+
+template <int NSB>
+__global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q8(const uint8_t *__restrict__ W, const uint4 *__restrict__ xs,
+                                                                      const float *__restrict__ rowscale, void *__restrict__ yg, int M,
+                                                                      int Mp, int N, int spr, int tiles, int tiles_per_wg, int ybf16) {
+    __shared__ float4_t red[2][kSmallWaves][64];
+    extern __shared__ float4_t dyn[];  // out_tiles [tiles_per_wg rounded up to whole rounds][64], then the waves' stages
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int nwaves = (int)(blockDim.x >> 6);
+    const int nl = lane & 15, kg = lane >> 4;
+    const int rounds = (tiles_per_wg + kSmallDepth - 1) / kSmallDepth;
+    float4_t *out_tiles = dyn;
+    u32x4 *stage = reinterpret_cast<u32x4 *>(dyn + rounds * kSmallDepth * 64) + wave * (NSB * kQ8TileRunPieces);
+    int sbi[NSB];
+    bool sbv[NSB];  // wave-uniform
+#pragma unroll
+    for (int i = 0; i < NSB; i++) {
+        sbi[i] = NSB * wave + i;
+        sbv[i] = sbi[i] < spr;
+        sbi[i] = sbv[i] ? sbi[i] : 0;
+    }
+    // activation operands: block b of run sb holds elements 256 sb + 32 b ..; the item of its k-group kg is item
+    // 4 (b % 4) + kg of half 2 sb + b / 4 (the pre-pass writes 16 items of eight consecutive elements per 128)
+    half8_t af[NSB][8];
+#pragma unroll
+    for (int i = 0; i < NSB; i++) {
+#pragma unroll
+        for (int b = 0; b < 8; b++) {
+            const uint4 *item = xs + (size_t)((2 * sbi[i] + (b >> 2)) * kGroups + 4 * (b & 3) + kg) * Mp + nl;
+            af[i][b] = __builtin_bit_cast(half8_t, *item);
+            if (!sbv[i]) af[i][b] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        }
+    }
+    const int t0 = (int)blockIdx.x * tiles_per_wg;
+    const int t1 = t0 + tiles_per_wg < tiles ? t0 + tiles_per_wg : tiles;
+    const uint32_t row_bytes = (uint32_t)spr * (uint32_t)kQ8RunBytes;
+    // piece j of this lane: index lane + 64 j of the tile's 272 (the fifth exists for the first 16 lanes; the others load
+    // the last piece again and drop it)
+    uint32_t piece_row[5], piece_off[5];
+#pragma unroll
+    for (int j = 0; j < 5; j++) {
+        int idx = lane + 64 * j;
+        idx = idx < kQ8TileRunPieces ? idx : kQ8TileRunPieces - 1;
+        piece_row[j] = (uint32_t)(idx / 17), piece_off[j] = 16u * (uint32_t)(idx % 17);
+    }
+    auto issue = [&](int ti, SmallRunQ8 &wa, SmallRunQ8 &wb) __attribute__((always_inline)) {
+        int tile = t0 + ti;
+        tile = tile < t1 ? tile : t1 - 1;  // past the end: the last tile again (loaded, not used)
+#pragma unroll
+        for (int j = 0; j < 5; j++) {
+            int n = tile * 16 + (int)piece_row[j];
+            n = n < N ? n : N - 1;
+            const uint8_t *p = W + ((uint32_t)n * row_bytes + piece_off[j]);  // the tensor is smaller than 4 GiB (checked by the launcher)
+#pragma unroll
+            for (int i = 0; i < NSB; i++) (i == 0 ? wa : wb).piece[j] = *reinterpret_cast<const u32x4 *>(p + (uint32_t)sbi[i] * (uint32_t)kQ8RunBytes);
+        }
+    };
+    const uint32_t *mine = reinterpret_cast<const uint32_t *>(stage) + nl * (kQ8RunBytes / 4);  // this lane's weight row in the stage
+    auto consume = [&](int ti, const SmallRunQ8 &wa, const SmallRunQ8 &wb) __attribute__((always_inline)) {
+        float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        const float4_t none = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int i = 0; i < NSB; i++) {
+            u32x4 *st = stage + i * kQ8TileRunPieces;
+            const SmallRunQ8 &w = i == 0 ? wa : wb;
+#pragma unroll
+            for (int j = 0; j < 4; j++) st[lane + 64 * j] = w.piece[j];
+            if (lane < kQ8TileRunPieces - 256) st[lane + 256] = w.piece[4];
+            // LDS executes a wave's instructions in order: the reads below see the writes above, and the next tile's
+            // writes come after these reads
+            const uint32_t *row = mine + i * (kQ8TileRunPieces * 4);
+#pragma unroll
+            for (int b = 0; b < 8; b++) {
+                // block b starts at byte 34 b of the run: on a dword boundary for even b (d in the low half of that dword,
+                // the quants from its high half on), two bytes past one for odd b (d in the high half of the dword below)
+                uint32_t q0, q1, dbits;
+                if ((b & 1) == 0) {
+                    const uint32_t *p = row + (34 * b) / 4 + 2 * kg;
+                    const uint32_t w0 = p[0], w1 = p[1], w2 = p[2];
+                    q0 = __builtin_amdgcn_alignbit(w1, w0, 16), q1 = __builtin_amdgcn_alignbit(w2, w1, 16);
+                    dbits = row[(34 * b) / 4] & 0xFFFFu;
+                } else {
+                    const uint32_t *p = row + (34 * b + 2) / 4 + 2 * kg;
+                    q0 = p[0], q1 = p[1];
+                    dbits = row[(34 * b - 2) / 4] >> 16;
+                }
+                // (of a run past the end of the row only zeros may enter the sums, whatever bytes were loaded for it)
+                const float d = sbv[i] ? f16_bits_to_f32(dbits) : 0.0f;
+                const float4_t part = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i][b], q8_operand(q0, q1), none, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 4; r++) acc[r] = __builtin_fmaf(d, part[r], acc[r]);
+            }
+        }
+        const int buf = ti & 1;
+        red[buf][wave][lane] = acc;
+        __syncthreads();  // the next tile writes the other buffer; the one after that comes behind the next barrier
+        if (wave == 0) {
+            float4_t v = red[buf][0][lane];
+            for (int q = 1; q < nwaves; q++) {
+                const float4_t u = red[buf][q][lane];
+#pragma unroll
+                for (int r = 0; r < 4; r++) v[r] += u[r];
+            }
+            out_tiles[ti * 64 + lane] = v;
+        }
+    };
+    static_assert(kSmallDepth == 2, "the ring is written out as two tiles");
+    SmallRunQ8 ring0a, ring0b, ring1a, ring1b;  // (the b halves are unused with one run per wave)
+    issue(0, ring0a, ring0b);
+    issue(1, ring1a, ring1b);
+    for (int rd = 0; rd < rounds; rd++) {
+        consume(2 * rd, ring0a, ring0b);
+        issue(2 * rd + 2, ring0a, ring0b);
+        consume(2 * rd + 1, ring1a, ring1b);
+        issue(2 * rd + 3, ring1a, ring1b);
+    }
+    __syncthreads();
+    const int cols = (t1 - t0) * 16;
+    for (int idx = (int)threadIdx.x; idx < M * cols; idx += (int)blockDim.x) {
+        const int m = idx / cols, j = idx - m * cols;
+        const int n = t0 * 16 + j;
+        if (n < N) {
+            const float o = out_tiles[(j >> 4) * 64 + (m >> 2) * 16 + (j & 15)][m & 3] * rowscale[m];
+            if (ybf16) reinterpret_cast<uint16_t *>(yg)[(size_t)m * N + n] = (uint16_t)bf16_rne_bits(o);
+            else reinterpret_cast<float *>(yg)[(size_t)m * N + n] = o;
+        }
+    }
+}
+
 // y[m][n] = rowscale[m] * (partial[0][m][n] + partial[1][m][n] + ...), added in this order
 template <bool YBF16>
 __global__ __launch_bounds__(256) void k_rw_reduce(const float *__restrict__ partial, int splits, int M, int Mp, int N,
@@ -1147,7 +1294,9 @@ static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 // The fused kernel for few activation rows takes Q4_K with m <= 16 and rows of at most 16 super-blocks (k <= 4096).
 static bool qgemm_small_applies(uint32_t type, int64_t m, int64_t n, int64_t k) {
-    return type == kTypeQ4K && m <= kSmallMaxM && k / 256 <= kSmallMaxSpr && (uint64_t)n * (uint64_t)(k / 256) * 144u < (1ull << 32);
+    const uint64_t run_bytes = type == kTypeQ4K ? 144u : 272u;  // bytes of 256 weights
+    return (type == kTypeQ4K || type == kTypeQ8_0) && m <= kSmallMaxM && k / 256 <= kSmallMaxSpr &&
+           (uint64_t)n * (uint64_t)(k / 256) * run_bytes < (1ull << 32);
 }
 
 static int compute_units_gemm() {
@@ -1306,7 +1455,23 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
         hipLaunchKernelGGL((k_qgemm_small<O, S>), grid, block, lds, s, w, xs, rowscale, y, (int)m, (int)p.mp, (int)n, spr, tiles, \
                            tiles_per_wg, ybf ? 1 : 0);                                                                           \
     } while (0)
-        if (spr > kSmallWaves) {
+        if (q8) {
+            const int nsb = spr > kSmallWaves ? 2 : 1;
+            const size_t lds8 = lds + (size_t)nwaves * nsb * kQ8TileRunPieces * 16;  // the waves' stages behind the finished tiles
+#define PMH_SMALL_Q8(S)                                                                                                          \
+    do {                                                                                                                         \
+        if (lds8 > 48 * 1024) {                                                                                                  \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_qgemm_small_q8<S>), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                    (int)lds8);                                                                                  \
+            if (e != hipSuccess) return e;                                                                                       \
+        }                                                                                                                        \
+        hipLaunchKernelGGL((k_qgemm_small_q8<S>), grid, block, lds8, s, w, xs, rowscale, y, (int)m, (int)p.mp, (int)n, spr, tiles, \
+                           tiles_per_wg, ybf ? 1 : 0);                                                                           \
+    } while (0)
+            if (nsb == 2) PMH_SMALL_Q8(2);
+            else PMH_SMALL_Q8(1);
+#undef PMH_SMALL_Q8
+        } else if (spr > kSmallWaves) {
             static_assert(2 * kSmallWaves >= kSmallMaxSpr, "two super-blocks per wave must cover the longest row");
             if (ref) PMH_SMALL(0, 2);
             else PMH_SMALL(1, 2);
