@@ -1231,6 +1231,170 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q8(const uint8
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// The same for Q6_K (210-byte super-blocks: ql[128], qh[64], 16 int8 scales, f16 d; value d sc (q - 32),
+// crates/pmetal-gguf/src/k_quants.rs:474-496), for rows of 8 or 16 super-blocks (k = 2048, 4096: rows then start on
+// 16-byte boundaries).  A k-step of v_mfma_f32_16x16x16_f16 is one sub-block of 16 elements: lane (r, kg) holds the
+// four quants 4 kg .. 4 kg + 3 of the sub-block of weight row r as exact f16 (q - 32), and d sc of the sub-block
+// multiplies the fp32 product tile of that step.  Sub-block (hh, g, lh) -- elements 128 hh + 32 g + 16 lh .. of the
+// super-block -- takes the low (g < 2) or high nibbles of the ql dword at 64 hh + 32 (g % 2) + 16 lh + 4 kg, bits 2 g of
+// the qh dword at 32 hh + 16 lh + 4 kg and scale 8 hh + 2 g + lh; its activation operand is one half of the pre-pass
+// item (t = 4 lh + kg, g % 2) of half hh, which holds elements 32 (g % 2) + 4 t .. and those 64 further.
+// A wave owns one or two adjacent super-blocks of every row.  Their bytes start (210 NSB wave) % 16 bytes into a
+// 16-byte piece: the wave copies the pieces that cover them, row by row, through registers into its own LDS with
+// whole-wave 16-byte loads (never past the piece that holds the tensor's last byte), and the lanes read aligned dwords;
+// the fields of a super-block sit a wave-uniform 0 or 2 bytes off a dword boundary and are shifted into place.
+// ------------------------------------------------------------------------------------------------
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+template <int NSB>
+struct SmallQ6 {
+    static constexpr int kRowPieces = NSB == 2 ? 27 : 14;             // 16-byte pieces that cover 210 NSB bytes from any even start
+    static constexpr int kLoads = (16 * kRowPieces + 63) / 64;        // pieces per lane and row tile: 7 or 4
+    static constexpr int kStageDwords = 16 * kRowPieces * 4 + 4;      // (+ one piece: the shifted reads look one dword ahead)
+};
+template <int NSB>
+struct SmallRunQ6 {
+    u32x4 piece[SmallQ6<NSB>::kLoads];  // (a vector type: copies of it are loads and stores that stay in registers)
+};
+
+template <int NSB>
+__global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q6(const uint8_t *__restrict__ W, const uint4 *__restrict__ xs,
+                                                                      const float *__restrict__ rowscale, void *__restrict__ yg, int M,
+                                                                      int Mp, int N, int spr, int tiles, int tiles_per_wg, int ybf16,
+                                                                      uint32_t w_last) {
+    constexpr int P = SmallQ6<NSB>::kRowPieces, kLoads = SmallQ6<NSB>::kLoads;
+    __shared__ float4_t red[2][kSmallWaves][64];
+    extern __shared__ float4_t dyn[];  // out_tiles [tiles_per_wg rounded up to whole rounds][64], then the waves' stages
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int nwaves = (int)(blockDim.x >> 6);
+    const int nl = lane & 15, kg = lane >> 4;
+    const int rounds = (tiles_per_wg + kSmallDepth - 1) / kSmallDepth;
+    float4_t *out_tiles = dyn;
+    uint32_t *stage = reinterpret_cast<uint32_t *>(dyn + rounds * kSmallDepth * 64) + wave * SmallQ6<NSB>::kStageDwords;
+    // this wave's super-blocks NSB wave .. (all of them exist: the launcher gives a wave per NSB super-blocks of the row)
+    const uint32_t run_start = 210u * (uint32_t)(NSB * wave), delta = run_start & 15u;
+    // activation operands: item (t = 4 lh + kg, gp) of half 2 sb + hh; index [hh][lh][gp]
+    half8_t af[NSB][2][2][2];
+#pragma unroll
+    for (int i = 0; i < NSB; i++)
+#pragma unroll
+        for (int hh = 0; hh < 2; hh++)
+#pragma unroll
+            for (int lh = 0; lh < 2; lh++)
+#pragma unroll
+                for (int gp = 0; gp < 2; gp++) {
+                    const uint4 *item = xs + (size_t)((2 * (NSB * wave + i) + hh) * kGroups + 2 * (4 * lh + kg) + gp) * Mp + nl;
+                    af[i][hh][lh][gp] = __builtin_bit_cast(half8_t, *item);
+                }
+    const int t0 = (int)blockIdx.x * tiles_per_wg;
+    const int t1 = t0 + tiles_per_wg < tiles ? t0 + tiles_per_wg : tiles;
+    const uint32_t row_bytes = (uint32_t)spr * 210u;
+    uint32_t piece_row[kLoads], piece_off[kLoads];
+#pragma unroll
+    for (int j = 0; j < kLoads; j++) {
+        int idx = lane + 64 * j;
+        idx = idx < 16 * P ? idx : 16 * P - 1;  // (the last load of a lane may not exist: it repeats the last piece and is dropped)
+        piece_row[j] = (uint32_t)(idx / P), piece_off[j] = (run_start & ~15u) + 16u * (uint32_t)(idx % P);
+    }
+    auto issue = [&](int ti, SmallRunQ6<NSB> &w) __attribute__((always_inline)) {
+        int tile = t0 + ti;
+        tile = tile < t1 ? tile : t1 - 1;  // past the end: the last tile again (loaded, not used)
+#pragma unroll
+        for (int j = 0; j < kLoads; j++) {
+            int n = tile * 16 + (int)piece_row[j];
+            n = n < N ? n : N - 1;
+            uint32_t a = (uint32_t)n * row_bytes + piece_off[j];  // the tensor is smaller than 4 GiB (checked by the launcher)
+            a = a < w_last ? a : w_last;  // a piece past the one with the tensor's last byte holds nothing of this run
+            w.piece[j] = *reinterpret_cast<const u32x4 *>(W + a);
+        }
+    };
+    const uint32_t *mine = stage + nl * (P * 4);  // this lane's weight row in the stage (dwords)
+    auto consume = [&](int ti, const SmallRunQ6<NSB> &w) __attribute__((always_inline)) {
+        float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        const float4_t none = {0.0f, 0.0f, 0.0f, 0.0f};
+        u32x4 *st = reinterpret_cast<u32x4 *>(stage);
+#pragma unroll
+        for (int j = 0; j < kLoads; j++)
+            if (lane + 64 * j < 16 * P) st[lane + 64 * j] = w.piece[j];
+        // LDS executes a wave's instructions in order: the reads below see the writes above, and the next tile's
+        // writes come after these reads
+#pragma unroll
+        for (int i = 0; i < NSB; i++) {
+            const uint32_t at = delta + 210u * (uint32_t)i;  // byte of the super-block in the lane's staged row: wave-uniform
+            const uint32_t sh = 8u * (at & 2u);
+            const uint32_t *blk = mine + (at >> 2);
+            auto field = [&](int dword) -> uint32_t {  // the dword at byte 4 * dword of the super-block
+                return __builtin_amdgcn_alignbit(blk[dword + 1], blk[dword], sh);
+            };
+            uint32_t sc[4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) sc[q] = field(48 + q);
+            const float d = f16_bits_to_f32(field(52) & 0xFFFFu);
+#pragma unroll
+            for (int hh = 0; hh < 2; hh++)
+#pragma unroll
+                for (int lh = 0; lh < 2; lh++) {
+                    const uint32_t qh = field(32 + 8 * hh + 4 * lh + kg);
+#pragma unroll
+                    for (int gp = 0; gp < 2; gp++) {
+                        const uint32_t ql = field(16 * hh + 8 * gp + 4 * lh + kg);
+                        const half8_t a8 = af[i][hh][lh][gp];
+#pragma unroll
+                        for (int up = 0; up < 2; up++) {  // group g = gp + 2 up: the low, then the high nibbles
+                            const int g = gp + 2 * up;
+                            const uint32_t v = ((ql >> (4 * up)) & 0x0F0F0F0Fu) | (((qh >> (2 * g)) & 0x03030303u) << 4);
+                            // 0x6400 | q is the f16 1024 + q; minus 1056 leaves q - 32, exact
+                            const half2_t m1056 = {(_Float16)-1056.0f, (_Float16)-1056.0f};
+                            const half2_t b01 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, v, 0x04010400u)) + m1056;
+                            const half2_t b23 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, v, 0x04030402u)) + m1056;
+                            const half4_t b4 = {b01[0], b01[1], b23[0], b23[1]};
+                            const half4_t a4 = up ? half4_t{a8[4], a8[5], a8[6], a8[7]} : half4_t{a8[0], a8[1], a8[2], a8[3]};
+                            const float4_t part = __builtin_amdgcn_mfma_f32_16x16x16f16(a4, b4, none, 0, 0, 0);
+                            const int si = 8 * hh + 2 * g + lh;  // the sub-block's scale byte
+                            const float s = d * (float)((int)(sc[si >> 2] << (24 - 8 * (si & 3))) >> 24);
+#pragma unroll
+                            for (int r = 0; r < 4; r++) acc[r] = __builtin_fmaf(s, part[r], acc[r]);
+                        }
+                    }
+                }
+        }
+        const int buf = ti & 1;
+        red[buf][wave][lane] = acc;
+        __syncthreads();  // the next tile writes the other buffer; the one after that comes behind the next barrier
+        if (wave == 0) {
+            float4_t v = red[buf][0][lane];
+            for (int q = 1; q < nwaves; q++) {
+                const float4_t u = red[buf][q][lane];
+#pragma unroll
+                for (int r = 0; r < 4; r++) v[r] += u[r];
+            }
+            out_tiles[ti * 64 + lane] = v;
+        }
+    };
+    static_assert(kSmallDepth == 2, "the ring is written out as two tiles");
+    SmallRunQ6<NSB> ring0, ring1;
+    issue(0, ring0);
+    issue(1, ring1);
+    for (int rd = 0; rd < rounds; rd++) {
+        consume(2 * rd, ring0);
+        issue(2 * rd + 2, ring0);
+        consume(2 * rd + 1, ring1);
+        issue(2 * rd + 3, ring1);
+    }
+    __syncthreads();
+    const int cols = (t1 - t0) * 16;
+    for (int idx = (int)threadIdx.x; idx < M * cols; idx += (int)blockDim.x) {
+        const int m = idx / cols, j = idx - m * cols;
+        const int n = t0 * 16 + j;
+        if (n < N) {
+            const float o = out_tiles[(j >> 4) * 64 + (m >> 2) * 16 + (j & 15)][m & 3] * rowscale[m];
+            if (ybf16) reinterpret_cast<uint16_t *>(yg)[(size_t)m * N + n] = (uint16_t)bf16_rne_bits(o);
+            else reinterpret_cast<float *>(yg)[(size_t)m * N + n] = o;
+        }
+    }
+}
+
 // y[m][n] = rowscale[m] * (partial[0][m][n] + partial[1][m][n] + ...), added in this order
 template <bool YBF16>
 __global__ __launch_bounds__(256) void k_rw_reduce(const float *__restrict__ partial, int splits, int M, int Mp, int N,
@@ -1294,9 +1458,13 @@ static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 // The fused kernel for few activation rows takes Q4_K with m <= 16 and rows of at most 16 super-blocks (k <= 4096).
 static bool qgemm_small_applies(uint32_t type, int64_t m, int64_t n, int64_t k) {
-    const uint64_t run_bytes = type == kTypeQ4K ? 144u : 272u;  // bytes of 256 weights
-    return (type == kTypeQ4K || type == kTypeQ8_0) && m <= kSmallMaxM && k / 256 <= kSmallMaxSpr &&
-           (uint64_t)n * (uint64_t)(k / 256) * run_bytes < (1ull << 32);
+    const int64_t spr = k / 256;
+    if (m > kSmallMaxM || spr > kSmallMaxSpr) return false;
+    if (type == kTypeQ4K) return (uint64_t)n * (uint64_t)spr * 144u < (1ull << 32);
+    if (type == kTypeQ8_0) return (uint64_t)n * (uint64_t)spr * 272u < (1ull << 32);
+    // Q6_K: rows of 8 or 16 super-blocks (they start on 16-byte boundaries and divide among eight waves)
+    if (type == kTypeQ6K) return (spr == 8 || spr == 16) && (uint64_t)n * (uint64_t)spr * 210u < (1ull << 32);
+    return false;
 }
 
 static int compute_units_gemm() {
@@ -1455,7 +1623,25 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
         hipLaunchKernelGGL((k_qgemm_small<O, S>), grid, block, lds, s, w, xs, rowscale, y, (int)m, (int)p.mp, (int)n, spr, tiles, \
                            tiles_per_wg, ybf ? 1 : 0);                                                                           \
     } while (0)
-        if (q8) {
+        if (q6) {
+            const int nsb = spr > kSmallWaves ? 2 : 1;
+            const size_t stage = (size_t)(nsb == 2 ? SmallQ6<2>::kStageDwords : SmallQ6<1>::kStageDwords) * 4;
+            const size_t lds6 = lds + (size_t)nwaves * stage;  // the waves' stages behind the finished tiles
+            const uint32_t w_last = (uint32_t)(((uint64_t)n * (uint64_t)spr * 210u - 1) & ~(uint64_t)15);
+#define PMH_SMALL_Q6(S)                                                                                                          \
+    do {                                                                                                                         \
+        if (lds6 > 48 * 1024) {                                                                                                  \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_qgemm_small_q6<S>), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                    (int)lds6);                                                                                  \
+            if (e != hipSuccess) return e;                                                                                       \
+        }                                                                                                                        \
+        hipLaunchKernelGGL((k_qgemm_small_q6<S>), grid, block, lds6, s, w, xs, rowscale, y, (int)m, (int)p.mp, (int)n, spr, tiles, \
+                           tiles_per_wg, ybf ? 1 : 0, w_last);                                                                   \
+    } while (0)
+            if (nsb == 2) PMH_SMALL_Q6(2);
+            else PMH_SMALL_Q6(1);
+#undef PMH_SMALL_Q6
+        } else if (q8) {
             const int nsb = spr > kSmallWaves ? 2 : 1;
             const size_t lds8 = lds + (size_t)nwaves * nsb * kQ8TileRunPieces * 16;  // the waves' stages behind the finished tiles
 #define PMH_SMALL_Q8(S)                                                                                                          \

@@ -421,3 +421,49 @@ def test_qgemm_batch_equals_separate_calls(oracle):
     bad = (_lib.GemmDesc * 1)(_lib.GemmDesc(13, 0, 0, 0, 256, ws[0].ptr, y_bat[0].ptr))
     assert lib.pmetal_hip_qgemm_batch(bad, 1, k, dx.ptr, pm.DTYPE_BF16, 3, None) == 2
     lib.pmetal_hip_clear_error()
+
+
+@pytest.mark.parametrize("t", [Q4K, Q6K, Q8_0])
+@pytest.mark.parametrize("m", [1, 2, 5, 9, 16])
+@pytest.mark.parametrize("n,k", [(700, 2048), (333, 4096), (16, 2048), (4099, 4096), (40, 1024)])
+def test_qgemm_short_batches(oracle, t, m, n, k):
+    """At most 16 activation rows: the fused kernels that read the weights once (rows of up to 16 super-blocks; Q6_K:
+    of 8 or 16).  Random block bytes (every scale, min and quant pattern), row counts that are no multiple of the 16-row
+    tiles, one full tile, more tiles than workgroups take in one round; bf16 and f32 activations, f32 and bf16 outputs;
+    unit activations that pick single weights out of the matrix."""
+    rng = np.random.default_rng(1000 * t + 31 * m + n + k)
+    block = {Q4K: 144, Q6K: 210, Q8_0: 34}[t]
+    per = 32 if t == Q8_0 else 256
+    raw = rng.integers(0, 256, size=(n * (k // per), block), dtype=np.uint8)
+    half = np.frombuffer(np.array([0.01, 0.02], np.float16).tobytes(), np.uint8)
+    if t == Q4K:
+        raw[:, 0:4] = half
+    elif t == Q6K:
+        raw[:, 208:210] = half[:2]
+    else:
+        raw[:, 0:2] = (rng.uniform(0.5, 2.0, raw.shape[0]) * 0.01 * rng.choice([-1.0, 1.0], raw.shape[0])).astype(np.float16).view(np.uint8).reshape(-1, 2)
+    raw = raw.reshape(-1)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    bits = oracle.f32_to_bf16_bits(x.reshape(-1)).reshape(m, k)
+    xr = oracle.bf16_bits_to_f32(bits.reshape(-1)).reshape(m, k)
+    want = reference(oracle, t, raw, n, k, xr, 0)
+    got = gpu_qgemm(t, raw, n, k, bits, m)
+    elem, norm = rel_errors(got.reshape(-1), want.reshape(-1))
+    assert elem <= TOL and norm <= TOL, (elem, norm)
+    got16 = gpu_qgemm(t, raw, n, k, bits, m, y_dtype=pm.DTYPE_BF16)
+    assert np.max(np.abs(got16 - want)) / np.max(np.abs(want)) <= 2.0 ** -8
+    # f32 activations that are exact in f16 at the row's scale: small integers
+    xi = rng.integers(-8, 9, size=(m, k)).astype(np.float32)
+    got = gpu_qgemm(t, raw, n, k, xi, m, x_dtype=pm.DTYPE_F32)
+    elem, norm = rel_errors(got.reshape(-1), reference(oracle, t, raw, n, k, xi, 0).reshape(-1))
+    assert elem <= TOL and norm <= TOL, (elem, norm)
+    # unit vectors: row r of the activations picks column (r * 97 + 5) % k of the dequantized weight, bit for bit where
+    # the weight is exact in the output
+    xu = np.zeros((m, k), np.float32)
+    cols = [(r * 97 + 5 + 13 * m) % k for r in range(m)]
+    for r, c in enumerate(cols):
+        xu[r, c] = 1.0
+    got = gpu_qgemm(t, raw, n, k, oracle.f32_to_bf16_bits(xu.reshape(-1)).reshape(m, k), m)
+    w = oracle.dequantize(t, raw, [n, k]).reshape(n, k)
+    for r, c in enumerate(cols):
+        assert np.allclose(got[r], w[:, c], rtol=1e-6, atol=0), (r, c)
