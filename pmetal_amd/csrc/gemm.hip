@@ -965,7 +965,8 @@ struct SmallRun {
 template <int ORDER, int NSB>
 __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t *__restrict__ W, const uint4 *__restrict__ xs,
                                                                    const float *__restrict__ rowscale, void *__restrict__ yg, int M,
-                                                                   int Mp, int N, int spr, int tiles, int tiles_per_wg, int ybf16) {
+                                                                   int Mp, int N, int spr, int tiles, int tiles_per_wg, int ybf16,
+                                                                   float *__restrict__ partial) {
     __shared__ float4_t red[2][kSmallWaves][64];
     extern __shared__ float4_t dyn[];  // out_tiles [tiles_per_wg rounded up to whole rounds][64]: lane slots of the finished tiles; then the waves' stages
     const int lane = threadIdx.x & 63;
@@ -980,7 +981,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t 
     bool sbv[NSB];  // wave-uniform
 #pragma unroll
     for (int i = 0; i < NSB; i++) {
-        sbi[i] = NSB * wave + i;  // adjacent super-blocks: one contiguous piece of every row per wave
+        sbi[i] = (int)blockIdx.y * (NSB * nwaves) + NSB * wave + i;  // adjacent super-blocks: one contiguous piece of every row per wave; workgroup row blockIdx.y of the grid takes the blockIdx.y-th run of NSB * waves super-blocks of a long row
         sbv[i] = sbi[i] < spr;
         sbi[i] = sbv[i] ? sbi[i] : 0;
     }
@@ -1099,8 +1100,11 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t 
         const int m = idx / cols, j = idx - m * cols;
         const int n = t0 * 16 + j;
         if (n < N) {
-            const float o = out_tiles[(j >> 4) * 64 + (m >> 2) * 16 + (j & 15)][m & 3] * rowscale[m];
-            if (ybf16) reinterpret_cast<uint16_t *>(yg)[(size_t)m * N + n] = (uint16_t)bf16_rne_bits(o);
+            const float sum = out_tiles[(j >> 4) * 64 + (m >> 2) * 16 + (j & 15)][m & 3];
+            const float o = sum * rowscale[m];
+            // a long row is cut into runs over gridDim.y workgroup rows: fp32 partial tiles, not yet scaled, for k_rw_reduce
+            if (partial) partial[((size_t)blockIdx.y * Mp + m) * N + n] = sum;
+            else if (ybf16) reinterpret_cast<uint16_t *>(yg)[(size_t)m * N + n] = (uint16_t)bf16_rne_bits(o);
             else reinterpret_cast<float *>(yg)[(size_t)m * N + n] = o;
         }
     }
@@ -1127,7 +1131,8 @@ struct SmallRunQ8 {
 template <int NSB>
 __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q8(const uint8_t *__restrict__ W, const uint4 *__restrict__ xs,
                                                                       const float *__restrict__ rowscale, void *__restrict__ yg, int M,
-                                                                      int Mp, int N, int spr, int tiles, int tiles_per_wg, int ybf16) {
+                                                                      int Mp, int N, int spr, int tiles, int tiles_per_wg, int ybf16,
+                                                                   float *__restrict__ partial) {
     __shared__ float4_t red[2][kSmallWaves][64];
     extern __shared__ float4_t dyn[];  // out_tiles [tiles_per_wg rounded up to whole rounds][64], then the waves' stages
     const int lane = threadIdx.x & 63;
@@ -1141,7 +1146,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q8(const uint8
     bool sbv[NSB];  // wave-uniform
 #pragma unroll
     for (int i = 0; i < NSB; i++) {
-        sbi[i] = NSB * wave + i;
+        sbi[i] = (int)blockIdx.y * (NSB * nwaves) + NSB * wave + i;
         sbv[i] = sbi[i] < spr;
         sbi[i] = sbv[i] ? sbi[i] : 0;
     }
@@ -1246,8 +1251,11 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q8(const uint8
         const int m = idx / cols, j = idx - m * cols;
         const int n = t0 * 16 + j;
         if (n < N) {
-            const float o = out_tiles[(j >> 4) * 64 + (m >> 2) * 16 + (j & 15)][m & 3] * rowscale[m];
-            if (ybf16) reinterpret_cast<uint16_t *>(yg)[(size_t)m * N + n] = (uint16_t)bf16_rne_bits(o);
+            const float sum = out_tiles[(j >> 4) * 64 + (m >> 2) * 16 + (j & 15)][m & 3];
+            const float o = sum * rowscale[m];
+            // a long row is cut into runs over gridDim.y workgroup rows: fp32 partial tiles, not yet scaled, for k_rw_reduce
+            if (partial) partial[((size_t)blockIdx.y * Mp + m) * N + n] = sum;
+            else if (ybf16) reinterpret_cast<uint16_t *>(yg)[(size_t)m * N + n] = (uint16_t)bf16_rne_bits(o);
             else reinterpret_cast<float *>(yg)[(size_t)m * N + n] = o;
         }
     }
@@ -1283,7 +1291,7 @@ template <int NSB>
 __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q6(const uint8_t *__restrict__ W, const uint4 *__restrict__ xs,
                                                                       const float *__restrict__ rowscale, void *__restrict__ yg, int M,
                                                                       int Mp, int N, int spr, int tiles, int tiles_per_wg, int ybf16,
-                                                                      uint32_t w_last) {
+                                                                      uint32_t w_last, float *__restrict__ partial) {
     constexpr int P = SmallQ6<NSB>::kRowPieces, kLoads = SmallQ6<NSB>::kLoads;
     __shared__ float4_t red[2][kSmallWaves][64];
     extern __shared__ float4_t dyn[];  // out_tiles [tiles_per_wg rounded up to whole rounds][64], then the waves' stages
@@ -1294,8 +1302,13 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q6(const uint8
     const int rounds = (tiles_per_wg + kSmallDepth - 1) / kSmallDepth;
     float4_t *out_tiles = dyn;
     uint32_t *stage = reinterpret_cast<uint32_t *>(dyn + rounds * kSmallDepth * 64) + wave * SmallQ6<NSB>::kStageDwords;
-    // this wave's super-blocks NSB wave .. (all of them exist: the launcher gives a wave per NSB super-blocks of the row)
-    const uint32_t run_start = 210u * (uint32_t)(NSB * wave), delta = run_start & 15u;
+    // this wave's super-blocks sb0 .. sb0 + NSB - 1 (rows are whole multiples of eight super-blocks, so the NSB of a wave
+    // exist together or not at all; a wave past the end of a long row's last run works on the row's first super-blocks
+    // with zero activations and zero scales)
+    const int sb_here = (int)blockIdx.y * (NSB * nwaves) + NSB * wave;
+    const bool run_valid = sb_here + NSB <= spr;  // wave-uniform
+    const int sb0 = run_valid ? sb_here : 0;
+    const uint32_t run_start = 210u * (uint32_t)sb0, delta = run_start & 15u;
     // activation operands: item (t = 4 lh + kg, gp) of half 2 sb + hh; index [hh][lh][gp]
     half8_t af[NSB][2][2][2];
 #pragma unroll
@@ -1306,8 +1319,9 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q6(const uint8
             for (int lh = 0; lh < 2; lh++)
 #pragma unroll
                 for (int gp = 0; gp < 2; gp++) {
-                    const uint4 *item = xs + (size_t)((2 * (NSB * wave + i) + hh) * kGroups + 2 * (4 * lh + kg) + gp) * Mp + nl;
+                    const uint4 *item = xs + (size_t)((2 * (sb0 + i) + hh) * kGroups + 2 * (4 * lh + kg) + gp) * Mp + nl;
                     af[i][hh][lh][gp] = __builtin_bit_cast(half8_t, *item);
+                    if (!run_valid) af[i][hh][lh][gp] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
                 }
     const int t0 = (int)blockIdx.x * tiles_per_wg;
     const int t1 = t0 + tiles_per_wg < tiles ? t0 + tiles_per_wg : tiles;
@@ -1352,7 +1366,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q6(const uint8
             uint32_t sc[4];
 #pragma unroll
             for (int q = 0; q < 4; q++) sc[q] = field(48 + q);
-            const float d = f16_bits_to_f32(field(52) & 0xFFFFu);
+            const float d = run_valid ? f16_bits_to_f32(field(52) & 0xFFFFu) : 0.0f;
 #pragma unroll
             for (int hh = 0; hh < 2; hh++)
 #pragma unroll
@@ -1410,8 +1424,11 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q6(const uint8
         const int m = idx / cols, j = idx - m * cols;
         const int n = t0 * 16 + j;
         if (n < N) {
-            const float o = out_tiles[(j >> 4) * 64 + (m >> 2) * 16 + (j & 15)][m & 3] * rowscale[m];
-            if (ybf16) reinterpret_cast<uint16_t *>(yg)[(size_t)m * N + n] = (uint16_t)bf16_rne_bits(o);
+            const float sum = out_tiles[(j >> 4) * 64 + (m >> 2) * 16 + (j & 15)][m & 3];
+            const float o = sum * rowscale[m];
+            // a long row is cut into runs over gridDim.y workgroup rows: fp32 partial tiles, not yet scaled, for k_rw_reduce
+            if (partial) partial[((size_t)blockIdx.y * Mp + m) * N + n] = sum;
+            else if (ybf16) reinterpret_cast<uint16_t *>(yg)[(size_t)m * N + n] = (uint16_t)bf16_rne_bits(o);
             else reinterpret_cast<float *>(yg)[(size_t)m * N + n] = o;
         }
     }
@@ -1479,13 +1496,16 @@ namespace pmh {
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 // The fused kernel for few activation rows takes Q4_K with m <= 16 and rows of at most 16 super-blocks (k <= 4096).
+// The fused kernels for at most 16 activation rows.  Rows of more than 16 super-blocks are cut into runs of 16, one
+// workgroup row of the grid each, whose partial tiles k_rw_reduce adds (qgemm_plan sets splits and chunk to match).
+constexpr int kSmallMaxRuns = 8;  // k <= 32768
 static bool qgemm_small_applies(uint32_t type, int64_t m, int64_t n, int64_t k) {
     const int64_t spr = k / 256;
-    if (m > kSmallMaxM || spr > kSmallMaxSpr) return false;
+    if (m > kSmallMaxM || spr > kSmallMaxSpr * kSmallMaxRuns) return false;
     if (type == kTypeQ4K) return (uint64_t)n * (uint64_t)spr * 144u < (1ull << 32);
     if (type == kTypeQ8_0) return (uint64_t)n * (uint64_t)spr * 272u < (1ull << 32);
-    // Q6_K: rows of 8 or 16 super-blocks (they start on 16-byte boundaries and divide among eight waves)
-    if (type == kTypeQ6K) return (spr == 8 || spr == 16) && (uint64_t)n * (uint64_t)spr * 210u < (1ull << 32);
+    // Q6_K: rows of a multiple of eight super-blocks (they start on 16-byte boundaries and divide among eight waves)
+    if (type == kTypeQ6K) return spr % 8 == 0 && (uint64_t)n * (uint64_t)spr * 210u < (1ull << 32);
     return false;
 }
 
@@ -1535,6 +1555,9 @@ GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k) {
                          (splits > 1 ? (double)splits * (double)m * (double)n * 8.0 / 4.0e12 + 3.0e-6 : 0.0);
         if (want == 1 || t < best) best = t, p.splits = (int)splits, p.chunk = (int)chunk;
     }
+    // at most 16 activation rows against long rows: runs of 16 super-blocks (the fused kernels' K split; the large kernel
+    // takes the same split when a shape falls back to it)
+    if (m <= kSmallMaxM && spr > kSmallMaxSpr) p.chunk = kSmallMaxSpr, p.splits = (int)((spr + kSmallMaxSpr - 1) / kSmallMaxSpr);
     return p;
 }
 
@@ -1629,11 +1652,20 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
     if (qgemm_small_applies(type, m, n, k)) {
         const int nwaves = spr < kSmallWaves ? spr : kSmallWaves;
         const int tiles = (int)((n + 15) / 16);
-        const int64_t slots = (int64_t)compute_units_gemm() * (kSmallWaves / nwaves);
+        // one workgroup per compute unit over all runs of a long row: each then walks several row tiles with its activation
+        // operands in registers (one tile per workgroup and four times the workgroups: 35 against 27 us at M = 16, 4096 x 14336)
+        const int runs_of_row = spr > kSmallMaxSpr ? p.splits : 1;
+        int64_t slots = (int64_t)compute_units_gemm() * (kSmallWaves / nwaves) / runs_of_row;
+        slots = slots < 1 ? 1 : slots;
         const int n_wg = (int)(tiles < slots ? tiles : slots);
         int tiles_per_wg = (tiles + n_wg - 1) / n_wg;
         tiles_per_wg = tiles_per_wg < 96 ? tiles_per_wg : 96;  // the finished tiles wait in LDS: 1 KiB each
-        const dim3 grid((unsigned)((tiles + tiles_per_wg - 1) / tiles_per_wg)), block((unsigned)(64 * nwaves));
+        // a long row: p.splits runs of 16 super-blocks, one workgroup row of the grid each, partial tiles for k_rw_reduce
+        // (for rows of up to 16 super-blocks the plan's split belongs to the large kernel and is not used here)
+        const int runs = runs_of_row;
+        float *const part_out = runs > 1 ? partial : nullptr;
+        const int nsb = spr > kSmallWaves ? 2 : 1;
+        const dim3 grid((unsigned)((tiles + tiles_per_wg - 1) / tiles_per_wg), (unsigned)runs), block((unsigned)(64 * nwaves));
         const size_t lds = (size_t)((tiles_per_wg + kSmallDepth - 1) / kSmallDepth * kSmallDepth) * 1024;
 #define PMH_SMALL(O, S)                                                                                                          \
     do {                                                                                                                         \
@@ -1644,10 +1676,9 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
             if (e != hipSuccess) return e;                                                                                       \
         }                                                                                                                        \
         hipLaunchKernelGGL((k_qgemm_small<O, S>), grid, block, lds4, s, w, xs, rowscale, y, (int)m, (int)p.mp, (int)n, spr, tiles, \
-                           tiles_per_wg, ybf ? 1 : 0);                                                                           \
+                           tiles_per_wg, ybf ? 1 : 0, part_out);                                                                           \
     } while (0)
         if (q6) {
-            const int nsb = spr > kSmallWaves ? 2 : 1;
             const size_t stage = (size_t)(nsb == 2 ? SmallQ6<2>::kStageDwords : SmallQ6<1>::kStageDwords) * 4;
             const size_t lds6 = lds + (size_t)nwaves * stage;  // the waves' stages behind the finished tiles
             const uint32_t w_last = (uint32_t)(((uint64_t)n * (uint64_t)spr * 210u - 1) & ~(uint64_t)15);
@@ -1659,13 +1690,12 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
             if (e != hipSuccess) return e;                                                                                       \
         }                                                                                                                        \
         hipLaunchKernelGGL((k_qgemm_small_q6<S>), grid, block, lds6, s, w, xs, rowscale, y, (int)m, (int)p.mp, (int)n, spr, tiles, \
-                           tiles_per_wg, ybf ? 1 : 0, w_last);                                                                   \
+                           tiles_per_wg, ybf ? 1 : 0, w_last, part_out);                                                                   \
     } while (0)
             if (nsb == 2) PMH_SMALL_Q6(2);
             else PMH_SMALL_Q6(1);
 #undef PMH_SMALL_Q6
         } else if (q8) {
-            const int nsb = spr > kSmallWaves ? 2 : 1;
             const size_t lds8 = lds + (size_t)nwaves * nsb * kQ8TileRunPieces * 16;  // the waves' stages behind the finished tiles
 #define PMH_SMALL_Q8(S)                                                                                                          \
     do {                                                                                                                         \
@@ -1675,7 +1705,7 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
             if (e != hipSuccess) return e;                                                                                       \
         }                                                                                                                        \
         hipLaunchKernelGGL((k_qgemm_small_q8<S>), grid, block, lds8, s, w, xs, rowscale, y, (int)m, (int)p.mp, (int)n, spr, tiles, \
-                           tiles_per_wg, ybf ? 1 : 0);                                                                           \
+                           tiles_per_wg, ybf ? 1 : 0, part_out);                                                                           \
     } while (0)
             if (nsb == 2) PMH_SMALL_Q8(2);
             else PMH_SMALL_Q8(1);
@@ -1689,8 +1719,9 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
             else PMH_SMALL(1, 1);
         }
 #undef PMH_SMALL
-        return hipGetLastError();
-    }
+        e = hipGetLastError();
+        if (e != hipSuccess || runs == 1) return e;
+    } else {
     const int mode = p.splits > 1 ? 2 : (ybf ? 1 : 0);
 #define PMH_RW_CASE(O, B, R, NWV) launch_rw<O, B, R, NWV>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
     if (q8) {
@@ -1710,6 +1741,8 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
     }
 #undef PMH_RW_CASE
     if (e != hipSuccess || p.splits == 1) return e;
+    }
+    // the partial tiles of a K split (of the large kernels or of the short-batch kernels' runs), added in split order
     const size_t total = (size_t)m * n;
     if (n % 8 == 0) {
         const dim3 grid8((unsigned)((total / 8 + 255) / 256));

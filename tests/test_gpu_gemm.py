@@ -425,7 +425,9 @@ def test_qgemm_batch_equals_separate_calls(oracle):
 
 @pytest.mark.parametrize("t", [Q4K, Q6K, Q8_0])
 @pytest.mark.parametrize("m", [1, 2, 5, 9, 16])
-@pytest.mark.parametrize("n,k", [(700, 2048), (333, 4096), (16, 2048), (4099, 4096), (40, 1024)])
+@pytest.mark.parametrize("n,k", [(700, 2048), (333, 4096), (16, 2048), (4099, 4096), (40, 1024),
+                                 # rows of more than 16 super-blocks: runs of 16, partial tiles added in a second kernel
+                                 (500, 14336), (130, 6144), (77, 11008), (64, 32768)])
 def test_qgemm_short_batches(oracle, t, m, n, k):
     """At most 16 activation rows: the fused kernels that read the weights once (rows of up to 16 super-blocks; Q6_K:
     of 8 or 16).  Random block bytes (every scale, min and quant pattern), row counts that are no multiple of the 16-row
