@@ -1659,7 +1659,9 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
         slots = slots < 1 ? 1 : slots;
         const int n_wg = (int)(tiles < slots ? tiles : slots);
         int tiles_per_wg = (tiles + n_wg - 1) / n_wg;
-        tiles_per_wg = tiles_per_wg < 96 ? tiles_per_wg : 96;  // the finished tiles wait in LDS: 1 KiB each
+        // the finished tiles wait in LDS, 1 KiB each, beside the waves' stages (at most 70 KiB, Q8_0) and the 16 KiB of the
+        // reduction buffers: 64 of them keep the workgroup within 160 KiB for every type
+        tiles_per_wg = tiles_per_wg < 64 ? tiles_per_wg : 64;
         // a long row: p.splits runs of 16 super-blocks, one workgroup row of the grid each, partial tiles for k_rw_reduce
         // (for rows of up to 16 super-blocks the plan's split belongs to the large kernel and is not used here)
         const int runs = runs_of_row;

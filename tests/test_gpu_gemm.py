@@ -469,3 +469,30 @@ def test_qgemm_short_batches(oracle, t, m, n, k):
     w = oracle.dequantize(t, raw, [n, k]).reshape(n, k)
     for r, c in enumerate(cols):
         assert np.allclose(got[r], w[:, c], rtol=1e-6, atol=0), (r, c)
+
+
+@pytest.mark.parametrize("t", [Q4K, Q6K, Q8_0])
+def test_qgemm_short_batch_very_tall_weight(oracle, t):
+    """300 000 weight rows against 9 activation rows: more row tiles per workgroup than its LDS holds finished tiles for,
+    so the grid has more workgroups than compute units.  The first 2000 and the last 3000 rows against the oracle."""
+    n, k, m = 300000, 2048, 9
+    rng = np.random.default_rng(t)
+    block = {Q4K: 144, Q6K: 210, Q8_0: 34}[t]
+    per = 32 if t == Q8_0 else 256
+    raw = rng.integers(0, 256, size=(n * (k // per), block), dtype=np.uint8)
+    half = np.frombuffer(np.array([0.01, 0.02], np.float16).tobytes(), np.uint8)
+    if t == Q4K:
+        raw[:, 0:4] = half
+    elif t == Q6K:
+        raw[:, 208:210] = half[:2]
+    else:
+        raw[:, 0:2] = half[:2]
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    bits = oracle.f32_to_bf16_bits(x.reshape(-1)).reshape(m, k)
+    xr = oracle.bf16_bits_to_f32(bits.reshape(-1)).reshape(m, k)
+    got = gpu_qgemm(t, raw.reshape(-1), n, k, bits, m)
+    rows = np.r_[0:2000, n - 3000:n]
+    sub = raw.reshape(n, -1)[rows].reshape(-1)
+    want = reference(oracle, t, sub, len(rows), k, xr, 0)
+    elem, norm = rel_errors(got[:, rows].reshape(-1), want.reshape(-1))
+    assert elem <= TOL and norm <= TOL, (elem, norm)
