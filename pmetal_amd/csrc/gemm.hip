@@ -955,6 +955,46 @@ constexpr int kSmallWaves = 8;  // waves per workgroup (fewer when a row has few
 constexpr int kSmallDepth = 2;  // row tiles in flight per wave (four are slower: 16.5 against 12.7 us at 14336 x 4096)
 constexpr int kSmallMaxM = 16, kSmallMaxSpr = 16;
 
+// The two steps the short-batch kernels share.  A row tile's 16 x 16 partial tiles, one per wave: every wave leaves its
+// own in LDS, and after one barrier the first wave adds them in wave order and keeps the sum as finished tile `ti` (the
+// next tile writes the other buffer; the one after that comes behind the next barrier).
+__device__ __forceinline__ void small_add_waves(float4_t (&red)[2][kSmallWaves][64], int ti, int wave, int nwaves, int lane,
+                                                const float4_t acc, float4_t *out_tiles) {
+    const int buf = ti & 1;
+    red[buf][wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0) {
+        float4_t v = red[buf][0][lane];
+        for (int q = 1; q < nwaves; q++) {
+            const float4_t u = red[buf][q][lane];
+#pragma unroll
+            for (int r = 0; r < 4; r++) v[r] += u[r];
+        }
+        out_tiles[ti * 64 + lane] = v;
+    }
+}
+
+// After the last tile: y[m][16 t0 + j] for j over the workgroup's columns (consecutive threads store consecutive columns of
+// one row), scaled by the rows' powers of two; or, when a long row is cut into runs over the grid's second dimension,
+// the fp32 partial tile of this run, not yet scaled, for k_rw_reduce.
+__device__ __forceinline__ void small_store(const float4_t *out_tiles, int t0, int t1, int M, int Mp, int N,
+                                            const float *__restrict__ rowscale, void *__restrict__ yg, int ybf16,
+                                            float *__restrict__ partial) {
+    __syncthreads();
+    const int cols = (t1 - t0) * 16;
+    for (int idx = (int)threadIdx.x; idx < M * cols; idx += (int)blockDim.x) {
+        const int m = idx / cols, j = idx - m * cols;
+        const int n = t0 * 16 + j;
+        if (n < N) {
+            const float sum = out_tiles[(j >> 4) * 64 + (m >> 2) * 16 + (j & 15)][m & 3];
+            const float o = sum * rowscale[m];
+            if (partial) partial[((size_t)blockIdx.y * Mp + m) * N + n] = sum;
+            else if (ybf16) reinterpret_cast<uint16_t *>(yg)[(size_t)m * N + n] = (uint16_t)bf16_rne_bits(o);
+            else reinterpret_cast<float *>(yg)[(size_t)m * N + n] = o;
+        }
+    }
+}
+
 template <int NSB>
 struct SmallRun {
     static constexpr int kPieces = 16 * 9 * NSB;        // 16-byte pieces of a row tile's NSB super-blocks (144 bytes each)
@@ -1068,18 +1108,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t 
 #pragma unroll
             for (int r = 0; r < 4; r++) acc[r] = __builtin_fmaf(dd, part[r], acc[r]);
         }
-        const int buf = ti & 1;
-        red[buf][wave][lane] = acc;
-        __syncthreads();  // the next tile writes the other buffer; the one after that comes behind the next barrier
-        if (wave == 0) {
-            float4_t v = red[buf][0][lane];
-            for (int q = 1; q < nwaves; q++) {
-                const float4_t u = red[buf][q][lane];
-#pragma unroll
-                for (int r = 0; r < 4; r++) v[r] += u[r];
-            }
-            out_tiles[ti * 64 + lane] = v;
-        }
+        small_add_waves(red, ti, wave, nwaves, lane, acc, out_tiles);
     };
     static_assert(kSmallDepth == 2, "the ring is written out as two tiles");
     SmallRun<NSB> ring0, ring1;
@@ -1093,21 +1122,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t 
         consume(2 * rd + 1, ring1);
         issue(2 * rd + 3, ring1);
     }
-    __syncthreads();
-    // y[m][16 t0 + j] for j over the workgroup's columns: consecutive threads store consecutive columns of one row
-    const int cols = (t1 - t0) * 16;
-    for (int idx = (int)threadIdx.x; idx < M * cols; idx += (int)blockDim.x) {
-        const int m = idx / cols, j = idx - m * cols;
-        const int n = t0 * 16 + j;
-        if (n < N) {
-            const float sum = out_tiles[(j >> 4) * 64 + (m >> 2) * 16 + (j & 15)][m & 3];
-            const float o = sum * rowscale[m];
-            // a long row is cut into runs over gridDim.y workgroup rows: fp32 partial tiles, not yet scaled, for k_rw_reduce
-            if (partial) partial[((size_t)blockIdx.y * Mp + m) * N + n] = sum;
-            else if (ybf16) reinterpret_cast<uint16_t *>(yg)[(size_t)m * N + n] = (uint16_t)bf16_rne_bits(o);
-            else reinterpret_cast<float *>(yg)[(size_t)m * N + n] = o;
-        }
-    }
+    small_store(out_tiles, t0, t1, M, Mp, N, rowscale, yg, ybf16, partial);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1222,18 +1237,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q8(const uint8
                 for (int r = 0; r < 4; r++) acc[r] = __builtin_fmaf(d, part[r], acc[r]);
             }
         }
-        const int buf = ti & 1;
-        red[buf][wave][lane] = acc;
-        __syncthreads();  // the next tile writes the other buffer; the one after that comes behind the next barrier
-        if (wave == 0) {
-            float4_t v = red[buf][0][lane];
-            for (int q = 1; q < nwaves; q++) {
-                const float4_t u = red[buf][q][lane];
-#pragma unroll
-                for (int r = 0; r < 4; r++) v[r] += u[r];
-            }
-            out_tiles[ti * 64 + lane] = v;
-        }
+        small_add_waves(red, ti, wave, nwaves, lane, acc, out_tiles);
     };
     static_assert(kSmallDepth == 2, "the ring is written out as two tiles");
     SmallRunQ8 ring0a, ring0b, ring1a, ring1b;  // (the b halves are unused with one run per wave)
@@ -1245,20 +1249,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q8(const uint8
         consume(2 * rd + 1, ring1a, ring1b);
         issue(2 * rd + 3, ring1a, ring1b);
     }
-    __syncthreads();
-    const int cols = (t1 - t0) * 16;
-    for (int idx = (int)threadIdx.x; idx < M * cols; idx += (int)blockDim.x) {
-        const int m = idx / cols, j = idx - m * cols;
-        const int n = t0 * 16 + j;
-        if (n < N) {
-            const float sum = out_tiles[(j >> 4) * 64 + (m >> 2) * 16 + (j & 15)][m & 3];
-            const float o = sum * rowscale[m];
-            // a long row is cut into runs over gridDim.y workgroup rows: fp32 partial tiles, not yet scaled, for k_rw_reduce
-            if (partial) partial[((size_t)blockIdx.y * Mp + m) * N + n] = sum;
-            else if (ybf16) reinterpret_cast<uint16_t *>(yg)[(size_t)m * N + n] = (uint16_t)bf16_rne_bits(o);
-            else reinterpret_cast<float *>(yg)[(size_t)m * N + n] = o;
-        }
-    }
+    small_store(out_tiles, t0, t1, M, Mp, N, rowscale, yg, ybf16, partial);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1395,18 +1386,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q6(const uint8
                     }
                 }
         }
-        const int buf = ti & 1;
-        red[buf][wave][lane] = acc;
-        __syncthreads();  // the next tile writes the other buffer; the one after that comes behind the next barrier
-        if (wave == 0) {
-            float4_t v = red[buf][0][lane];
-            for (int q = 1; q < nwaves; q++) {
-                const float4_t u = red[buf][q][lane];
-#pragma unroll
-                for (int r = 0; r < 4; r++) v[r] += u[r];
-            }
-            out_tiles[ti * 64 + lane] = v;
-        }
+        small_add_waves(red, ti, wave, nwaves, lane, acc, out_tiles);
     };
     static_assert(kSmallDepth == 2, "the ring is written out as two tiles");
     SmallRunQ6<NSB> ring0, ring1;
@@ -1418,20 +1398,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q6(const uint8
         consume(2 * rd + 1, ring1);
         issue(2 * rd + 3, ring1);
     }
-    __syncthreads();
-    const int cols = (t1 - t0) * 16;
-    for (int idx = (int)threadIdx.x; idx < M * cols; idx += (int)blockDim.x) {
-        const int m = idx / cols, j = idx - m * cols;
-        const int n = t0 * 16 + j;
-        if (n < N) {
-            const float sum = out_tiles[(j >> 4) * 64 + (m >> 2) * 16 + (j & 15)][m & 3];
-            const float o = sum * rowscale[m];
-            // a long row is cut into runs over gridDim.y workgroup rows: fp32 partial tiles, not yet scaled, for k_rw_reduce
-            if (partial) partial[((size_t)blockIdx.y * Mp + m) * N + n] = sum;
-            else if (ybf16) reinterpret_cast<uint16_t *>(yg)[(size_t)m * N + n] = (uint16_t)bf16_rne_bits(o);
-            else reinterpret_cast<float *>(yg)[(size_t)m * N + n] = o;
-        }
-    }
+    small_store(out_tiles, t0, t1, M, Mp, N, rowscale, yg, ybf16, partial);
 }
 
 // y[m][n] = rowscale[m] * (partial[0][m][n] + partial[1][m][n] + ...), added in this order
