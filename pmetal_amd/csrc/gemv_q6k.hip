@@ -22,7 +22,9 @@
 //
 //  * Rows of k / 256 super-blocks that are not whole chunks are handled by the RAGGED variant of the kernel (see there).
 //
-// Matrices below 12 MiB and rows shorter than one chunk stay with the bf16 kernel in gemv.hip.
+//  * Rows shorter than a chunk (k < 2048) are handled by the FOLD variant: a wave's task is 8 / (k / 256) whole rows.
+//
+// Matrices below 12 MiB stay with the bf16 kernel in gemv.hip.
 #include "gemv_chunk.hpp"
 #include "internal.hpp"
 
@@ -135,11 +137,17 @@ __device__ __forceinline__ float lane_dot(const Task &t, const uint32_t (&xr)[kP
 // DEEP: a ring of kDepthLong tasks for waves with seven or eight rows, all of which are then in flight at once (measured
 // against the ring of six, same machine: 4096 x 14336 13.98 -> 13.24 us, 14336 x 4096 12.08 -> 11.72, 8192 x 8192 14.1 ->
 // 13.4; waves with more rows, or fewer, are better off with six: 18944 x 3584 15.3 against 15.7, 4096 x 4096 6.15 against 6.25).
-template <bool XF32, bool SINGLE, bool RAGGED, bool DEEP = false>
+// FOLD (with RAGGED): rows of fold_spr < 8 super-blocks.  Rows follow one another in memory, so rpc = 8 / fold_spr of them
+// are one task: the kernel sees a matrix of ceil(n_real / rpc) rows of spr = rpc * fold_spr super-blocks, every lane
+// group takes the activations of its super-block's place in its own row, and the lane sums are added per row inside
+// the wave and stored straight to y (a task's rows past the end of the matrix are loaded from clamped addresses and
+// dropped).
+template <bool XF32, bool SINGLE, bool RAGGED, bool DEEP = false, bool FOLD = false>
 __global__ __launch_bounds__(1024) void k_qgemv_q6k_chunk(const uint8_t *__restrict__ W, const void *__restrict__ xg,
                                                            float *__restrict__ y, int n_rows, int spr, int rows_per_wg,
                                                            int rows_per_wave, int n_nominal, int nthreads,
-                                                           uint32_t w_last) {
+                                                           uint32_t w_last, int fold_spr, int n_real) {
+    static_assert(!FOLD || RAGGED, "folded rows start at any even address");
     constexpr int kDepth = DEEP ? kDepthLong : ::kDepth;
     extern __shared__ uint4 smem[];
     const int ks = (spr + 7) >> 3;
@@ -181,10 +189,12 @@ __global__ __launch_bounds__(1024) void k_qgemv_q6k_chunk(const uint8_t *__restr
     u4v ra[kDepth], rb[kDepth];
 #pragma unroll
     for (int i = 0; i < kPre; i++) issue(i, ra[i], rb[i]);
-    stage_x<XF32>(xg, slots, spr * 64, nthreads, xd, xm);
+    stage_x<XF32>(xg, slots, (FOLD ? fold_spr : spr) * 64, nthreads, xd, xm);
     __syncthreads();
 
-    const int slot = h * 64 + lane;
+    const int row_lanes = FOLD ? fold_spr * 8 : 64;   // lanes that share a row of the matrix
+    const int row_in_task = FOLD ? lane / row_lanes : 0;
+    const int slot = FOLD ? lane - row_in_task * row_lanes : h * 64 + lane;
     uint32_t xr[kPlanes][8];
 #pragma unroll
     for (int p = 0; p < kPlanes; p++)
@@ -229,7 +239,20 @@ __global__ __launch_bounds__(1024) void k_qgemv_q6k_chunk(const uint8_t *__restr
             tk.sc[1] = __builtin_amdgcn_alignbit(ws[2], ws[1], sh);
             tk.d = (blk[c_d] >> sh) & 0xFFFFu;
             const float val = lane_dot<kPlanes>(tk, xr, xmr, sh_a, sh_b, sc_up);
-            store_chunk_sum(pp + (size_t)i * ks, lane_valid ? val : 0.0f, lane);
+            if (FOLD) {
+                float tot;
+                if ((fold_spr & (fold_spr - 1)) == 0) {
+                    tot = team_sum_rt(val, row_lanes);
+                } else {  // 3, 5, 6 or 7 lane groups: the group totals, then the row's groups one by one
+                    const float grp = team_sum<8>(val);
+                    tot = grp;
+                    for (int j = 1; j < fold_spr; j++) tot += __shfl(grp, (lane + 8 * j) & 63);
+                }
+                const int row = (wave_r0 + i) * (spr / fold_spr) + row_in_task;
+                if (lane_valid && lane == row_in_task * row_lanes && row < n_real) y[row] = tot;
+            } else {
+                store_chunk_sum(pp + (size_t)i * ks, lane_valid ? val : 0.0f, lane);
+            }
         }
     };
 
@@ -254,6 +277,7 @@ __global__ __launch_bounds__(1024) void k_qgemv_q6k_chunk(const uint8_t *__restr
 #pragma unroll
         for (int i = 0; i < kDepth; i++) consume(base + i, ra[i], rb[i]);
     }
+    if (FOLD) return;
     __syncthreads();
 
     reduce_rows(part, ks, wg_r0, wg_r1 - wg_r0, rows_per_wave, n_nominal, nthreads, y);
@@ -267,11 +291,19 @@ namespace pmh {
 // false (the caller falls back to the general Q6_K kernel).  Preconditions as for launch_qgemv.
 bool try_launch_qgemv_q6k_chunk(const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, float *y,
                                 hipStream_t s, hipError_t *err) {
-    const int spr = (int)(k / 256);
-    if (spr < 8) return false;
-    const bool ragged = spr % 8 != 0;
+    const int spr_real = (int)(k / 256);
+    // Short rows: 8 / spr_real of them are one row of the kernel.  Rows of 5 or 6 super-blocks would leave three or two
+    // of a wave's eight lane groups idle and are faster in the general kernel (128256 x 1536: 40.9 against 48.9 us), as are
+    // matrices below 24 MiB (16000 x 1024: 6.1 against 7.0 us; 32000 x 1024: 10.0 against 9.6).
+    const bool fold = spr_real < 8;
+    if (fold && (spr_real == 5 || spr_real == 6 || (uint64_t)n * (uint64_t)spr_real * 210u < (24ull << 20))) return false;
+    const int rpc = fold ? 8 / spr_real : 1;
+    const int spr = spr_real * rpc;
+    const int64_t n_real = n;
+    if (fold) n = (n + rpc - 1) / rpc;
+    const bool ragged = fold || spr % 8 != 0;
     const int ks = (spr + 7) / 8;
-    const uint64_t w_bytes = (uint64_t)n * (uint64_t)spr * 210u;
+    const uint64_t w_bytes = (uint64_t)n_real * (uint64_t)spr_real * 210u;
     if (ks > 16 || w_bytes >= (1ull << 32)) return false;
     if (w_bytes < (12ull << 20)) return false;  // measured crossover with the general kernel
     const size_t slots = (size_t)ks * 64;
@@ -290,10 +322,14 @@ bool try_launch_qgemv_q6k_chunk(const uint8_t *w, int64_t n, int64_t k, const vo
             if (e != hipSuccess) return e;
         }
         hipLaunchKernelGGL(kern, dim3((unsigned)n_wg), dim3((unsigned)threads), lds, s, w, x, y, (int)n, spr, (int)rows_per_wg,
-                           (int)rows_per_wave, (int)n_nominal, (int)threads, (uint32_t)((w_bytes - 1) & ~(uint64_t)15));
+                           (int)rows_per_wave, (int)n_nominal, (int)threads, (uint32_t)((w_bytes - 1) & ~(uint64_t)15), spr_real, (int)n_real);
         return hipGetLastError();
     };
-    if (deep) {  // all tasks of a wave fit the longer ring: the SINGLE form of it
+    if (fold) {
+        if (deep) *err = xf32 ? go(k_qgemv_q6k_chunk<true, true, true, true, true>) : go(k_qgemv_q6k_chunk<false, true, true, true, true>);
+        else if (xf32) *err = single ? go(k_qgemv_q6k_chunk<true, true, true, false, true>) : go(k_qgemv_q6k_chunk<true, false, true, false, true>);
+        else *err = single ? go(k_qgemv_q6k_chunk<false, true, true, false, true>) : go(k_qgemv_q6k_chunk<false, false, true, false, true>);
+    } else if (deep) {  // all tasks of a wave fit the longer ring: the SINGLE form of it
         if (ragged) *err = xf32 ? go(k_qgemv_q6k_chunk<true, true, true, true>) : go(k_qgemv_q6k_chunk<false, true, true, true>);
         else *err = xf32 ? go(k_qgemv_q6k_chunk<true, true, false, true>) : go(k_qgemv_q6k_chunk<false, true, false, true>);
     } else if (ragged) {

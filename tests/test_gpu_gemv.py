@@ -75,12 +75,16 @@ def test_qgemv_q4k_large_ragged_shapes(oracle, n, k, x_dtype):
         assert elem <= TOL and norm <= TOL
 
 
-# Q6_K matrices of 12 MiB and more with rows of at least eight super-blocks (k >= 2048) take the kernel that stages
-# rows through LDS: ragged row counts, rows of 1 to 8 chunks, fewer rows than compute units times
+# Q6_K matrices of 12 MiB and more take the kernel that stages rows through LDS: ragged row counts, rows of 1 to 8 chunks, fewer rows than compute units times
 # waves; activations with large and tiny outliers and a run of zeros (the fixed-point scale is per 16 elements).
 Q6K_BIG_CASES = [(6001, 4096), (14336, 4096), (4096, 14336), (30001, 2048), (500, 16384), (1900, 6144),
                  # rows that are not whole chunks: 14, 43, 9 and 25 super-blocks (even and odd: rows start at any even address)
-                 (6001, 3584), (3001, 11008), (7001, 2304), (2049, 6400)]
+                 (6001, 3584), (3001, 11008), (7001, 2304), (2049, 6400),
+                 # rows shorter than a chunk (1 to 7 super-blocks): several whole rows are one task of a wave; row counts
+                 # that leave the last task short
+                 # (from 24 MiB on; rows of 5 or 6 super-blocks and smaller matrices stay with the general kernel)
+                 (32001, 1024), (151936, 1024), (62003, 512), (121003, 256), (40002, 768), (18002, 1792), (24001, 1280),
+                 (20001, 1536), (15001, 1024)]
 
 
 @pytest.mark.parametrize("n,k", Q6K_BIG_CASES)
@@ -129,7 +133,12 @@ def test_qgemv_q6k_large_quantized_weights_and_linearity(oracle):
 # activations with large and tiny outliers and a run of zeros; quants over the whole int8 range.
 Q8_0_BIG_CASES = [(6001, 4096), (14336, 4096), (4096, 14336), (30001, 2048), (500, 32768), (1900, 6144),
                   # rows whose last chunk is short: 112, 344, 72 and 200 blocks
-                  (6001, 3584), (3001, 11008), (7001, 2304), (2049, 6400)]
+                  (6001, 3584), (3001, 11008), (7001, 2304), (2049, 6400),
+                 # rows shorter than a chunk (1 to 7 super-blocks): several whole rows are one task of a wave; row counts
+                 # that leave the last task short
+                 # (from 24 MiB on; rows of 5 or 6 super-blocks and smaller matrices stay with the general kernel)
+                 (32001, 1024), (151936, 1024), (62003, 512), (121003, 256), (40002, 768), (18002, 1792), (24001, 1280),
+                 (20001, 1536), (15001, 1024)]
 
 
 @pytest.mark.parametrize("n,k", Q8_0_BIG_CASES)
