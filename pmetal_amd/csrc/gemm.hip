@@ -958,8 +958,17 @@ constexpr int kSmallMaxM = 16, kSmallMaxSpr = 16;
 // The two steps the short-batch kernels share.  A row tile's 16 x 16 partial tiles, one per wave: every wave leaves its
 // own in LDS, and after one barrier the first wave adds them in wave order and keeps the sum as finished tile `ti` (the
 // next tile writes the other buffer; the one after that comes behind the next barrier).
-__device__ __forceinline__ void small_add_waves(float4_t (&red)[2][kSmallWaves][64], int ti, int wave, int nwaves, int lane,
-                                                const float4_t acc, float4_t *out_tiles) {
+//
+// A workgroup with few tiles (at most kSmallKeepTiles) keeps every wave's partial tile of every row tile instead
+// (`keep`, [tile][wave][lane]) and adds them after the last one, in the same wave order: its waves then meet at one
+// barrier, not at one per tile.
+constexpr int kSmallKeepTiles = 8;
+__device__ __forceinline__ void small_add_waves(float4_t (&red)[2][kSmallWaves][64], float4_t *keep, int ti, int wave, int nwaves,
+                                                int lane, const float4_t acc, float4_t *out_tiles) {
+    if (keep) {  // workgroup-uniform
+        keep[(ti * nwaves + wave) * 64 + lane] = acc;
+        return;
+    }
     const int buf = ti & 1;
     red[buf][wave][lane] = acc;
     __syncthreads();
@@ -967,6 +976,20 @@ __device__ __forceinline__ void small_add_waves(float4_t (&red)[2][kSmallWaves][
         float4_t v = red[buf][0][lane];
         for (int q = 1; q < nwaves; q++) {
             const float4_t u = red[buf][q][lane];
+#pragma unroll
+            for (int r = 0; r < 4; r++) v[r] += u[r];
+        }
+        out_tiles[ti * 64 + lane] = v;
+    }
+}
+
+__device__ __forceinline__ void small_add_kept(const float4_t *keep, int n_tiles, int wave, int nwaves, int lane, float4_t *out_tiles) {
+    if (!keep) return;
+    __syncthreads();
+    for (int ti = wave; ti < n_tiles; ti += nwaves) {
+        float4_t v = keep[(ti * nwaves) * 64 + lane];
+        for (int q = 1; q < nwaves; q++) {
+            const float4_t u = keep[(ti * nwaves + q) * 64 + lane];
 #pragma unroll
             for (int r = 0; r < 4; r++) v[r] += u[r];
         }
@@ -1016,7 +1039,8 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t 
     const uint32_t low = kg < 2 ? 0xFFFFFFFFu : 0u;
     const int rounds = (tiles_per_wg + kSmallDepth - 1) / kSmallDepth;
     float4_t *out_tiles = dyn;
-    u32x4 *stage = reinterpret_cast<u32x4 *>(dyn + rounds * kSmallDepth * 64) + wave * SmallRun<NSB>::kPieces;
+    float4_t *keep = tiles_per_wg <= kSmallKeepTiles ? dyn + rounds * kSmallDepth * 64 : nullptr;
+    u32x4 *stage = reinterpret_cast<u32x4 *>(dyn + rounds * kSmallDepth * 64 * (keep ? 1 + nwaves : 1)) + wave * SmallRun<NSB>::kPieces;
     int sbi[NSB];
     bool sbv[NSB];  // wave-uniform
 #pragma unroll
@@ -1108,7 +1132,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t 
 #pragma unroll
             for (int r = 0; r < 4; r++) acc[r] = __builtin_fmaf(dd, part[r], acc[r]);
         }
-        small_add_waves(red, ti, wave, nwaves, lane, acc, out_tiles);
+        small_add_waves(red, keep, ti, wave, nwaves, lane, acc, out_tiles);
     };
     static_assert(kSmallDepth == 2, "the ring is written out as two tiles");
     SmallRun<NSB> ring0, ring1;
@@ -1122,6 +1146,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t 
         consume(2 * rd + 1, ring1);
         issue(2 * rd + 3, ring1);
     }
+    small_add_kept(keep, rounds * kSmallDepth, wave, nwaves, lane, out_tiles);
     small_store(out_tiles, t0, t1, M, Mp, N, rowscale, yg, ybf16, partial);
 }
 
@@ -1156,7 +1181,8 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q8(const uint8
     const int nl = lane & 15, kg = lane >> 4;
     const int rounds = (tiles_per_wg + kSmallDepth - 1) / kSmallDepth;
     float4_t *out_tiles = dyn;
-    u32x4 *stage = reinterpret_cast<u32x4 *>(dyn + rounds * kSmallDepth * 64) + wave * (NSB * kQ8TileRunPieces);
+    float4_t *keep = tiles_per_wg <= kSmallKeepTiles ? dyn + rounds * kSmallDepth * 64 : nullptr;
+    u32x4 *stage = reinterpret_cast<u32x4 *>(dyn + rounds * kSmallDepth * 64 * (keep ? 1 + nwaves : 1)) + wave * (NSB * kQ8TileRunPieces);
     int sbi[NSB];
     bool sbv[NSB];  // wave-uniform
 #pragma unroll
@@ -1237,7 +1263,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q8(const uint8
                 for (int r = 0; r < 4; r++) acc[r] = __builtin_fmaf(d, part[r], acc[r]);
             }
         }
-        small_add_waves(red, ti, wave, nwaves, lane, acc, out_tiles);
+        small_add_waves(red, keep, ti, wave, nwaves, lane, acc, out_tiles);
     };
     static_assert(kSmallDepth == 2, "the ring is written out as two tiles");
     SmallRunQ8 ring0a, ring0b, ring1a, ring1b;  // (the b halves are unused with one run per wave)
@@ -1249,6 +1275,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q8(const uint8
         consume(2 * rd + 1, ring1a, ring1b);
         issue(2 * rd + 3, ring1a, ring1b);
     }
+    small_add_kept(keep, rounds * kSmallDepth, wave, nwaves, lane, out_tiles);
     small_store(out_tiles, t0, t1, M, Mp, N, rowscale, yg, ybf16, partial);
 }
 
@@ -1292,7 +1319,8 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q6(const uint8
     const int nl = lane & 15, kg = lane >> 4;
     const int rounds = (tiles_per_wg + kSmallDepth - 1) / kSmallDepth;
     float4_t *out_tiles = dyn;
-    uint32_t *stage = reinterpret_cast<uint32_t *>(dyn + rounds * kSmallDepth * 64) + wave * SmallQ6<NSB>::kStageDwords;
+    float4_t *keep = tiles_per_wg <= kSmallKeepTiles ? dyn + rounds * kSmallDepth * 64 : nullptr;
+    uint32_t *stage = reinterpret_cast<uint32_t *>(dyn + rounds * kSmallDepth * 64 * (keep ? 1 + nwaves : 1)) + wave * SmallQ6<NSB>::kStageDwords;
     // this wave's super-blocks sb0 .. sb0 + NSB - 1 (rows are whole multiples of eight super-blocks, so the NSB of a wave
     // exist together or not at all; a wave past the end of a long row's last run works on the row's first super-blocks
     // with zero activations and zero scales)
@@ -1386,7 +1414,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q6(const uint8
                     }
                 }
         }
-        small_add_waves(red, ti, wave, nwaves, lane, acc, out_tiles);
+        small_add_waves(red, keep, ti, wave, nwaves, lane, acc, out_tiles);
     };
     static_assert(kSmallDepth == 2, "the ring is written out as two tiles");
     SmallRunQ6<NSB> ring0, ring1;
@@ -1398,6 +1426,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q6(const uint8
         consume(2 * rd + 1, ring1);
         issue(2 * rd + 3, ring1);
     }
+    small_add_kept(keep, rounds * kSmallDepth, wave, nwaves, lane, out_tiles);
     small_store(out_tiles, t0, t1, M, Mp, N, rowscale, yg, ybf16, partial);
 }
 
@@ -1635,7 +1664,9 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
         float *const part_out = runs > 1 ? partial : nullptr;
         const int nsb = spr > kSmallWaves ? 2 : 1;
         const dim3 grid((unsigned)((tiles + tiles_per_wg - 1) / tiles_per_wg), (unsigned)runs), block((unsigned)(64 * nwaves));
-        const size_t lds = (size_t)((tiles_per_wg + kSmallDepth - 1) / kSmallDepth * kSmallDepth) * 1024;
+        // (a workgroup of few tiles also keeps every wave's partial tile of each until the end)
+        const size_t lds = (size_t)((tiles_per_wg + kSmallDepth - 1) / kSmallDepth * kSmallDepth) * 1024 *
+                           (tiles_per_wg <= kSmallKeepTiles ? 1 + nwaves : 1);
 #define PMH_SMALL(O, S)                                                                                                          \
     do {                                                                                                                         \
         const size_t lds4 = lds + (size_t)nwaves * SmallRun<S>::kPieces * 16; /* the waves' stages behind the finished tiles */ \
