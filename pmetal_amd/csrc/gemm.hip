@@ -1281,8 +1281,8 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q8(const uint8
 
 // ------------------------------------------------------------------------------------------------
 // The same for Q6_K (210-byte super-blocks: ql[128], qh[64], 16 int8 scales, f16 d; value d sc (q - 32),
-// crates/pmetal-gguf/src/k_quants.rs:474-496), for rows of 8 or 16 super-blocks (k = 2048, 4096: rows then start on
-// 16-byte boundaries).  A k-step of v_mfma_f32_16x16x16_f16 is one sub-block of 16 elements: lane (r, kg) holds the
+// crates/pmetal-gguf/src/k_quants.rs:474-496); first for rows of a multiple of eight super-blocks, which start on
+// 16-byte boundaries.  A k-step of v_mfma_f32_16x16x16_f16 is one sub-block of 16 elements: lane (r, kg) holds the
 // four quants 4 kg .. 4 kg + 3 of the sub-block of weight row r as exact f16 (q - 32), and d sc of the sub-block
 // multiplies the fp32 product tile of that step.  Sub-block (hh, g, lh) -- elements 128 hh + 32 g + 16 lh .. of the
 // super-block -- takes the low (g < 2) or high nibbles of the ql dword at 64 hh + 32 (g % 2) + 16 lh + 4 kg, bits 2 g of
@@ -1294,23 +1294,29 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q8(const uint8
 // the fields of a super-block sit a wave-uniform 0 or 2 bytes off a dword boundary and are shifted into place.
 // ------------------------------------------------------------------------------------------------
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
-template <int NSB>
+template <int NSB, bool ANY = false>
 struct SmallQ6 {
-    static constexpr int kRowPieces = NSB == 2 ? 27 : 14;             // 16-byte pieces that cover 210 NSB bytes from any even start
+    // 16-byte pieces that cover 210 NSB bytes from where a wave's super-blocks start in their piece: any even byte for one
+    // super-block per wave or rows of any length (ANY), a multiple of four for pairs of super-blocks in rows that start
+    // on 16-byte boundaries
+    static constexpr int kRowPieces = NSB == 2 ? (ANY ? 28 : 27) : 14;
     static constexpr int kLoads = (16 * kRowPieces + 63) / 64;        // pieces per lane and row tile: 7 or 4
     static constexpr int kStageDwords = 16 * kRowPieces * 4 + 4;      // (+ one piece: the shifted reads look one dword ahead)
 };
 template <int NSB>
 struct SmallRunQ6 {
-    u32x4 piece[SmallQ6<NSB>::kLoads];  // (a vector type: copies of it are loads and stores that stay in registers)
+    u32x4 piece[SmallQ6<NSB>::kLoads];  static_assert(SmallQ6<NSB, true>::kLoads == SmallQ6<NSB, false>::kLoads, "one ring for both forms");  // (a vector type: copies of it are loads and stores that stay in registers)
 };
 
-template <int NSB>
+// ANY: rows of any number of super-blocks.  A row then starts at any even address, so where a wave's super-blocks lie in
+// their first piece, and whether their fields sit two bytes off a dword boundary, differs from row to row (per lane); the
+// last wave with work may own one super-block where the others own two.
+template <int NSB, bool ANY>
 __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q6(const uint8_t *__restrict__ W, const uint4 *__restrict__ xs,
                                                                       const float *__restrict__ rowscale, void *__restrict__ yg, int M,
                                                                       int Mp, int N, int spr, int tiles, int tiles_per_wg, int ybf16,
                                                                       uint32_t w_last, float *__restrict__ partial) {
-    constexpr int P = SmallQ6<NSB>::kRowPieces, kLoads = SmallQ6<NSB>::kLoads;
+    constexpr int P = SmallQ6<NSB, ANY>::kRowPieces, kLoads = SmallQ6<NSB, ANY>::kLoads;
     __shared__ float4_t red[2][kSmallWaves][64];
     extern __shared__ float4_t dyn[];  // out_tiles [tiles_per_wg rounded up to whole rounds][64], then the waves' stages
     const int lane = threadIdx.x & 63;
@@ -1320,13 +1326,15 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q6(const uint8
     const int rounds = (tiles_per_wg + kSmallDepth - 1) / kSmallDepth;
     float4_t *out_tiles = dyn;
     float4_t *keep = tiles_per_wg <= kSmallKeepTiles ? dyn + rounds * kSmallDepth * 64 : nullptr;
-    uint32_t *stage = reinterpret_cast<uint32_t *>(dyn + rounds * kSmallDepth * 64 * (keep ? 1 + nwaves : 1)) + wave * SmallQ6<NSB>::kStageDwords;
+    uint32_t *stage = reinterpret_cast<uint32_t *>(dyn + rounds * kSmallDepth * 64 * (keep ? 1 + nwaves : 1)) + wave * SmallQ6<NSB, ANY>::kStageDwords;
     // this wave's super-blocks sb0 .. sb0 + NSB - 1 (rows are whole multiples of eight super-blocks, so the NSB of a wave
     // exist together or not at all; a wave past the end of a long row's last run works on the row's first super-blocks
     // with zero activations and zero scales)
     const int sb_here = (int)blockIdx.y * (NSB * nwaves) + NSB * wave;
-    const bool run_valid = sb_here + NSB <= spr;  // wave-uniform
-    const int sb0 = run_valid ? sb_here : 0;
+    bool sbv[NSB];  // wave-uniform; without ANY all of a wave's super-blocks exist or none
+#pragma unroll
+    for (int i = 0; i < NSB; i++) sbv[i] = sb_here + i < spr;
+    const int sb0 = sbv[0] ? sb_here : 0;
     const uint32_t run_start = 210u * (uint32_t)sb0, delta = run_start & 15u;
     // activation operands: item (t = 4 lh + kg, gp) of half 2 sb + hh; index [hh][lh][gp]
     half8_t af[NSB][2][2][2];
@@ -1338,9 +1346,9 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q6(const uint8
             for (int lh = 0; lh < 2; lh++)
 #pragma unroll
                 for (int gp = 0; gp < 2; gp++) {
-                    const uint4 *item = xs + (size_t)((2 * (sb0 + i) + hh) * kGroups + 2 * (4 * lh + kg) + gp) * Mp + nl;
+                    const uint4 *item = xs + (size_t)((2 * (sbv[i] ? sb0 + i : 0) + hh) * kGroups + 2 * (4 * lh + kg) + gp) * Mp + nl;
                     af[i][hh][lh][gp] = __builtin_bit_cast(half8_t, *item);
-                    if (!run_valid) af[i][hh][lh][gp] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+                    if (!sbv[i]) af[i][hh][lh][gp] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
                 }
     const int t0 = (int)blockIdx.x * tiles_per_wg;
     const int t1 = t0 + tiles_per_wg < tiles ? t0 + tiles_per_wg : tiles;
@@ -1350,7 +1358,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q6(const uint8
     for (int j = 0; j < kLoads; j++) {
         int idx = lane + 64 * j;
         idx = idx < 16 * P ? idx : 16 * P - 1;  // (the last load of a lane may not exist: it repeats the last piece and is dropped)
-        piece_row[j] = (uint32_t)(idx / P), piece_off[j] = (run_start & ~15u) + 16u * (uint32_t)(idx % P);
+        piece_row[j] = (uint32_t)(idx / P), piece_off[j] = (ANY ? 0u : run_start & ~15u) + 16u * (uint32_t)(idx % P);
     }
     auto issue = [&](int ti, SmallRunQ6<NSB> &w) __attribute__((always_inline)) {
         int tile = t0 + ti;
@@ -1360,6 +1368,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q6(const uint8
             int n = tile * 16 + (int)piece_row[j];
             n = n < N ? n : N - 1;
             uint32_t a = (uint32_t)n * row_bytes + piece_off[j];  // the tensor is smaller than 4 GiB (checked by the launcher)
+            if (ANY) a = (((uint32_t)n * row_bytes + run_start) & ~15u) + piece_off[j];  // from the piece that holds the run's first byte in this row
             a = a < w_last ? a : w_last;  // a piece past the one with the tensor's last byte holds nothing of this run
             w.piece[j] = *reinterpret_cast<const u32x4 *>(W + a);
         }
@@ -1374,9 +1383,17 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q6(const uint8
             if (lane + 64 * j < 16 * P) st[lane + 64 * j] = w.piece[j];
         // LDS executes a wave's instructions in order: the reads below see the writes above, and the next tile's
         // writes come after these reads
+        uint32_t delta_row = delta;
+        if (ANY) {  // of the row this lane reads, as issue() took it
+            int tile = t0 + ti;
+            tile = tile < t1 ? tile : t1 - 1;
+            int n = tile * 16 + nl;
+            n = n < N ? n : N - 1;
+            delta_row = ((uint32_t)n * row_bytes + run_start) & 15u;
+        }
 #pragma unroll
         for (int i = 0; i < NSB; i++) {
-            const uint32_t at = delta + 210u * (uint32_t)i;  // byte of the super-block in the lane's staged row: wave-uniform
+            const uint32_t at = delta_row + 210u * (uint32_t)i;  // byte of the super-block in the lane's staged row (wave-uniform without ANY)
             const uint32_t sh = 8u * (at & 2u);
             const uint32_t *blk = mine + (at >> 2);
             auto field = [&](int dword) -> uint32_t {  // the dword at byte 4 * dword of the super-block
@@ -1385,7 +1402,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q6(const uint8
             uint32_t sc[4];
 #pragma unroll
             for (int q = 0; q < 4; q++) sc[q] = field(48 + q);
-            const float d = run_valid ? f16_bits_to_f32(field(52) & 0xFFFFu) : 0.0f;
+            const float d = sbv[i] ? f16_bits_to_f32(field(52) & 0xFFFFu) : 0.0f;
 #pragma unroll
             for (int hh = 0; hh < 2; hh++)
 #pragma unroll
@@ -1500,8 +1517,7 @@ static bool qgemm_small_applies(uint32_t type, int64_t m, int64_t n, int64_t k) 
     if (m > kSmallMaxM || spr > kSmallMaxSpr * kSmallMaxRuns) return false;
     if (type == kTypeQ4K) return (uint64_t)n * (uint64_t)spr * 144u < (1ull << 32);
     if (type == kTypeQ8_0) return (uint64_t)n * (uint64_t)spr * 272u < (1ull << 32);
-    // Q6_K: rows of a multiple of eight super-blocks (they start on 16-byte boundaries and divide among eight waves)
-    if (type == kTypeQ6K) return spr % 8 == 0 && (uint64_t)n * (uint64_t)spr * 210u < (1ull << 32);
+    if (type == kTypeQ6K) return (uint64_t)n * (uint64_t)spr * 210u < (1ull << 32);
     return false;
 }
 
@@ -1679,21 +1695,24 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
                            tiles_per_wg, ybf ? 1 : 0, part_out);                                                                           \
     } while (0)
         if (q6) {
-            const size_t stage = (size_t)(nsb == 2 ? SmallQ6<2>::kStageDwords : SmallQ6<1>::kStageDwords) * 4;
+            const bool any = spr % 8 != 0;  // rows that do not start on 16-byte boundaries
+            const size_t stage = (size_t)(nsb == 2 ? SmallQ6<2, true>::kStageDwords : SmallQ6<1>::kStageDwords) * 4;
             const size_t lds6 = lds + (size_t)nwaves * stage;  // the waves' stages behind the finished tiles
             const uint32_t w_last = (uint32_t)(((uint64_t)n * (uint64_t)spr * 210u - 1) & ~(uint64_t)15);
-#define PMH_SMALL_Q6(S)                                                                                                          \
+#define PMH_SMALL_Q6(S, A)                                                                                                        \
     do {                                                                                                                         \
         if (lds6 > 48 * 1024) {                                                                                                  \
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_qgemm_small_q6<S>), hipFuncAttributeMaxDynamicSharedMemorySize, \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_qgemm_small_q6<S, A>), hipFuncAttributeMaxDynamicSharedMemorySize, \
                                     (int)lds6);                                                                                  \
             if (e != hipSuccess) return e;                                                                                       \
         }                                                                                                                        \
-        hipLaunchKernelGGL((k_qgemm_small_q6<S>), grid, block, lds6, s, w, xs, rowscale, y, (int)m, (int)p.mp, (int)n, spr, tiles, \
+        hipLaunchKernelGGL((k_qgemm_small_q6<S, A>), grid, block, lds6, s, w, xs, rowscale, y, (int)m, (int)p.mp, (int)n, spr, tiles, \
                            tiles_per_wg, ybf ? 1 : 0, w_last, part_out);                                                                   \
     } while (0)
-            if (nsb == 2) PMH_SMALL_Q6(2);
-            else PMH_SMALL_Q6(1);
+            if (nsb == 2 && any) PMH_SMALL_Q6(2, true);
+            else if (nsb == 2) PMH_SMALL_Q6(2, false);
+            else if (any) PMH_SMALL_Q6(1, true);
+            else PMH_SMALL_Q6(1, false);
 #undef PMH_SMALL_Q6
         } else if (q8) {
             const size_t lds8 = lds + (size_t)nwaves * nsb * kQ8TileRunPieces * 16;  // the waves' stages behind the finished tiles

@@ -427,10 +427,12 @@ def test_qgemm_batch_equals_separate_calls(oracle):
 @pytest.mark.parametrize("m", [1, 2, 5, 9, 16])
 @pytest.mark.parametrize("n,k", [(700, 2048), (333, 4096), (16, 2048), (4099, 4096), (40, 1024),
                                  # rows of more than 16 super-blocks: runs of 16, partial tiles added in a second kernel
-                                 (500, 14336), (130, 6144), (77, 11008), (64, 32768)])
+                                 (500, 14336), (130, 6144), (77, 11008), (64, 32768),
+                                 # rows of 11, 1, 3, 20 and 13 super-blocks: Q6_K rows then start at any even address, the last
+                                 # wave with work owns one super-block where the others own two, a second run holds four
+                                 (333, 2816), (1001, 256), (250, 768), (123, 5120), (47, 3328)])
 def test_qgemm_short_batches(oracle, t, m, n, k):
-    """At most 16 activation rows: the fused kernels that read the weights once (rows of up to 16 super-blocks; Q6_K:
-    of 8 or 16).  Random block bytes (every scale, min and quant pattern), row counts that are no multiple of the 16-row
+    """At most 16 activation rows: the fused kernels that read the weights once (rows of any number of super-blocks, in runs of 16).  Random block bytes (every scale, min and quant pattern), row counts that are no multiple of the 16-row
     tiles, one full tile, more tiles than workgroups take in one round; bf16 and f32 activations, f32 and bf16 outputs;
     unit activations that pick single weights out of the matrix."""
     rng = np.random.default_rng(1000 * t + 31 * m + n + k)
