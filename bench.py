@@ -34,13 +34,13 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 # HBM bytes per launch as recorded from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled against a streaming kernel
 # of known size; constants taken from the profile summaries named here, not measured by this script
-RECORDED_TRAFFIC = {"gemv_q4k_14336x4096": (33287333, "profiles/qgemv_q4k_14336x4096.md"),
-                    "gemv_q4k_4096x14336": (33414126, "profiles/qgemv_q4k_4096x14336.md"),
-                    "gemv_q6k_14336x4096": (48547094, "profiles/qgemv_other_types.md"),
-                    "gemv_q8_0_14336x4096": (62653146, "profiles/qgemv_other_types.md"),
-                    "gemv_q5k_6144x4096": (17530055, "profiles/qgemv_other_types.md"),
-                    "gemv_q3k_14336x4096": (25568828, "profiles/qgemv_other_types.md"),
-                    "gemv_q2k_14336x4096": (19580724, "profiles/qgemv_other_types.md")}
+RECORDED_TRAFFIC = {"gemv_q4k_14336x4096": (33287193, "profiles/qgemv_q4k_14336x4096.md"),
+                    "gemv_q4k_4096x14336": (33414162, "profiles/qgemv_q4k_4096x14336.md"),
+                    "gemv_q6k_14336x4096": (48532488, "profiles/qgemv_other_types.md"),
+                    "gemv_q8_0_14336x4096": (62653287, "profiles/qgemv_other_types.md"),
+                    "gemv_q5k_6144x4096": (17530063, "profiles/qgemv_other_types.md"),
+                    "gemv_q3k_14336x4096": (25568799, "profiles/qgemv_other_types.md"),
+                    "gemv_q2k_14336x4096": (19580687, "profiles/qgemv_other_types.md")}
 BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16/fp16 MFMA, published
 Q8_0, Q4K, Q6K = 8, 12, 14
 
