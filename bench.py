@@ -622,6 +622,7 @@ WORKLOADS["gemv_q3k_14336x4096"] = dict(kind="gemv", n=14336, k=4096, type=11, m
 WORKLOADS["gemv_q2k_14336x4096"] = dict(kind="gemv", n=14336, k=4096, type=10, metric="Q2_K GEMV GB/s @14336x4096", unit="GB/s", dtype="bf16")
 WORKLOADS["gemv_q5k_6144x4096"] = dict(kind="gemv", n=6144, k=4096, type=13, metric="Q5_K GEMV GB/s @6144x4096 (fused attn_qkv)", unit="GB/s", dtype="bf16")
 WORKLOADS["gemv_q6k_18944x3584"] = dict(kind="gemv", n=18944, k=3584, type=Q6K, metric="Q6_K GEMV GB/s @18944x3584", unit="GB/s", dtype="bf16")
+WORKLOADS["gemv_q6k_151936x1024"] = dict(kind="gemv", n=151936, k=1024, type=Q6K, metric="Q6_K GEMV GB/s @151936x1024 (output projection of a small model)", unit="GB/s", dtype="bf16")
 WORKLOADS["gemv_q8_0_14336x4096"] = dict(kind="gemv", n=14336, k=4096, type=Q8_0, metric="Q8_0 GEMV GB/s @14336x4096", unit="GB/s", dtype="bf16")
 WORKLOADS["gemv_q4k_q8k_14336x4096"] = dict(kind="gemv_q8k", n=14336, k=4096, type=Q4K, unit="GB/s", dtype="i8",
                                             metric="Q4_K x Q8_K integer-dot GEMV GB/s @14336x4096 (activation quantize included)")
