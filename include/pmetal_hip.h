@@ -60,6 +60,7 @@ extern "C" {
 #define PMETAL_HIP_ERR_NO_DEVICE 5
 #define PMETAL_HIP_ERR_INVALID_SHAPE 6   /* DequantError::InvalidShape                   */
 #define PMETAL_HIP_ERR_SHAPE_TOO_LARGE 7 /* DequantError::ShapeTooLarge                  */
+#define PMETAL_HIP_ERR_BUSY 8            /* a shared resource of the library is in use by another call */
 
 /* Q4_K element order for dequantize / GEMV / GEMM.
  *  REF : the order the reference's dequantize_q4k emits (k_quants.rs:365-403); default,
@@ -189,8 +190,11 @@ int32_t pmetal_hip_qgemm(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, in
  * PMETAL_HIP_ERR_SHAPE_TOO_LARGE before anything is launched; Q5_K / Q3_K / Q2_K (re-blocking needs scratch of the size
  * of W) fail with PMETAL_HIP_ERR_UNSUPPORTED_TYPE.  Calls no hipMalloc / hipFree and nothing else that allocates.
  * pmetal_hip_init(device) looks the array's address up; without it the first call on a device does.  All calls on one
- * device share the array: calls that overlap on one device (two streams, two threads) race; calls on one stream are
- * ordered and may follow each other without a synchronisation.                                                        */
+ * device share the array: calls on one stream are ordered and may follow each other without a synchronisation; a call
+ * that would overlap another one on the same device -- issued on a different stream before the previous call's kernels
+ * have finished, or from a second thread while a call is being issued -- is refused with PMETAL_HIP_ERR_BUSY and launches
+ * nothing.  Calls issued while their stream is being recorded cannot be checked this way: keeping replays of such
+ * recordings from overlapping each other, and other calls, stays with the caller.                                     */
 #define PMETAL_HIP_NOALLOC_SCRATCH_BYTES ((size_t)32 << 20)
 int32_t pmetal_hip_qgemm_noalloc(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, int64_t k, const void *x_dev,
                                  uint32_t x_dtype, int64_t m, void *y_dev, uint32_t y_dtype, uint32_t order,

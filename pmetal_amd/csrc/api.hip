@@ -7,6 +7,7 @@
 // There is no CPU fallback anywhere in this file: without a HIP device every compute call fails.
 #include "../../include/pmetal_hip.h"
 
+#include <atomic>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -108,30 +109,45 @@ struct DevBuf {
 
 // Library-owned scratch, grown on demand: one buffer per (thread, device, stream), so that neither concurrent callers nor
 // one caller's launches on different streams share it.  Launches on one stream run in order and may.
+//  * The buffers live in one process-wide list behind a mutex; an entry carries the thread that asked for it.
 //  * A buffer that was handed out while its stream was being recorded is pinned: the recording holds its address, so it is
-//    never freed or replaced before the process ends (a larger request gets a new buffer, the pinned one is kept aside).
+//    neither freed nor replaced while the stream lives -- not when a larger request comes (that one gets a new buffer, the
+//    pinned one is kept aside), and not when the thread that recorded ends (a recording may be replayed from any thread).
 //  * While a stream is being recorded nothing may be allocated or synchronised on it: a request that the current buffer
 //    cannot serve fails with a clear error instead (run the same or a larger shape once before recording).
-//  * pmetal_hip_stream_destroy releases the buffers of that stream (pinned ones included: the recordings made on a
-//    destroyed stream must not be replayed any more).
+//  * pmetal_hip_stream_destroy releases every buffer of that stream, whichever thread asked for it, pinned ones included
+//    (the recordings made on a destroyed stream must not be replayed any more), so a later stream that happens to get the
+//    same handle value starts without entries.
+//  * A thread that ends releases its unpinned buffers.
 struct Workspace {
     void *p = nullptr;
     size_t bytes = 0;
     int device = -1;
     hipStream_t stream = nullptr;
     bool pinned = false;
+    bool retired = false;  // a pinned buffer that a larger one replaced: kept for the recordings that name it
+    uint64_t owner = 0;    // token of the thread that asked for it
 };
-struct WorkspaceSet {
-    std::vector<Workspace> items;
-    std::vector<Workspace> retired;  // pinned buffers that a larger one replaced
-    ~WorkspaceSet() {
-        for (Workspace &w : items)
-            if (w.p) (void)hipFree(w.p);  // at thread exit; fails harmlessly once the runtime is gone
-        for (Workspace &w : retired)
-            if (w.p) (void)hipFree(w.p);
+std::mutex g_ws_mu;
+std::vector<Workspace> g_ws_all;  // guarded by g_ws_mu
+std::atomic<uint64_t> g_ws_next_owner{1};
+
+struct WorkspaceOwner {
+    const uint64_t token = g_ws_next_owner.fetch_add(1);
+    ~WorkspaceOwner() {  // at thread exit; hipFree fails harmlessly once the runtime is gone
+        std::lock_guard<std::mutex> lock(g_ws_mu);
+        for (size_t i = 0; i < g_ws_all.size();) {
+            Workspace &w = g_ws_all[i];
+            if (w.owner == token && !w.pinned) {
+                if (w.p) (void)hipFree(w.p);
+                g_ws_all.erase(g_ws_all.begin() + (long)i);
+            } else {
+                i++;
+            }
+        }
     }
 };
-thread_local WorkspaceSet g_ws;
+thread_local WorkspaceOwner g_ws_owner;
 
 int32_t workspace(size_t bytes, hipStream_t stream, void **out) {
     int dev = 0;
@@ -139,51 +155,55 @@ int32_t workspace(size_t bytes, hipStream_t stream, void **out) {
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (stream) HIP_TRY(hipStreamIsCapturing(stream, &cap));
     const bool recording = cap != hipStreamCaptureStatusNone;
-    Workspace *w = nullptr;
-    for (Workspace &c : g_ws.items)
-        if (c.device == dev && c.stream == stream) w = &c;
-    if (!w) {
-        g_ws.items.push_back(Workspace{nullptr, 0, dev, stream, false});
-        w = &g_ws.items.back();
+    const uint64_t me = g_ws_owner.token;
+    std::lock_guard<std::mutex> lock(g_ws_mu);
+    size_t at = g_ws_all.size();
+    for (size_t i = 0; i < g_ws_all.size(); i++) {
+        const Workspace &c = g_ws_all[i];
+        if (c.owner == me && c.device == dev && c.stream == stream && !c.retired) at = i;
     }
-    if (w->bytes < bytes) {
+    if (at == g_ws_all.size()) {
+        Workspace fresh;
+        fresh.device = dev, fresh.stream = stream, fresh.owner = me;
+        g_ws_all.push_back(fresh);
+    }
+    if (g_ws_all[at].bytes < bytes) {
         if (recording)
             return fail(PMETAL_HIP_ERR_INVALID_ARG,
                         "this call needs %zu bytes of scratch and the stream's buffer holds %zu: nothing can be allocated while the "
-                        "stream is being recorded (run a call of this or a larger shape on the stream first)", bytes, w->bytes);
-        if (w->p) {
-            if (w->pinned) {
-                g_ws.retired.push_back(*w);  // a recording still names it
+                        "stream is being recorded (run a call of this or a larger shape on the stream first)", bytes, g_ws_all[at].bytes);
+        if (g_ws_all[at].p) {
+            if (g_ws_all[at].pinned) {
+                Workspace old = g_ws_all[at];  // a recording still names it
+                old.retired = true;
+                g_ws_all.push_back(old);
             } else {
                 HIP_TRY(hipStreamSynchronize(stream));  // earlier launches on this stream may still use the smaller buffer
-                HIP_TRY(hipFree(w->p));
+                HIP_TRY(hipFree(g_ws_all[at].p));
             }
-            w->p = nullptr, w->bytes = 0, w->pinned = false;
+            g_ws_all[at].p = nullptr, g_ws_all[at].bytes = 0, g_ws_all[at].pinned = false;
         }
         if (bytes) {
-            HIP_TRY(hipMalloc(&w->p, bytes));
-            w->bytes = bytes;
+            HIP_TRY(hipMalloc(&g_ws_all[at].p, bytes));
+            g_ws_all[at].bytes = bytes;
         }
     }
-    if (recording) w->pinned = true;
-    *out = w->p;
+    if (recording) g_ws_all[at].pinned = true;
+    *out = g_ws_all[at].p;
     return PMETAL_HIP_OK;
 }
 
-// Releases what workspace() holds for `stream` on the calling thread.
+// Releases what workspace() holds for `stream`, for every thread.
 void drop_workspaces_of(hipStream_t stream) {
-    auto drop = [&](std::vector<Workspace> &v) {
-        for (size_t i = 0; i < v.size();) {
-            if (v[i].stream == stream) {
-                if (v[i].p) (void)hipFree(v[i].p);
-                v.erase(v.begin() + (long)i);
-            } else {
-                i++;
-            }
+    std::lock_guard<std::mutex> lock(g_ws_mu);
+    for (size_t i = 0; i < g_ws_all.size();) {
+        if (g_ws_all[i].stream == stream) {
+            if (g_ws_all[i].p) (void)hipFree(g_ws_all[i].p);
+            g_ws_all.erase(g_ws_all.begin() + (long)i);
+        } else {
+            i++;
         }
-    };
-    drop(g_ws.items);
-    drop(g_ws.retired);
+    }
 }
 
 // ---- scratch memory of the entry point that allocates nothing (pmetal_hip_qgemm_noalloc) ----
@@ -193,22 +213,37 @@ void drop_workspaces_of(hipStream_t stream) {
 constexpr size_t kNoAllocScratchBytes = PMETAL_HIP_NOALLOC_SCRATCH_BYTES;  // 32 MiB
 static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
 constexpr int kMaxScratchDevices = 64;
-void *g_scratch_ptr[kMaxScratchDevices] = {nullptr};
+// Per device: the array's address, and what tells a second user of the array from the first.  Launches on one stream run
+// in order and may follow one another; a call on another stream while the previous call's kernels have not finished (the
+// event recorded behind them is not reached), or from another thread while a call is being issued, would overwrite
+// scratch that is still being read: such a call is refused.  Calls made while a stream is being recorded cannot be told
+// apart this way (an event recorded there belongs to the recording) and stay the caller's to keep apart.
+struct NoAllocScratch {
+    void *ptr = nullptr;
+    hipEvent_t done = nullptr;      // recorded behind the kernels of the last call that was not being recorded
+    hipStream_t last = nullptr;     // the stream of that call
+    bool pending = false;           // `done` has been recorded and not yet been seen reached
+    std::atomic<bool> busy{false};  // a thread is inside the entry point for this device
+};
+NoAllocScratch g_scratch[kMaxScratchDevices];
 std::mutex g_scratch_mu;
 
-// Device address of `scratch` on the calling thread's current device (looked up on the first call for that device).
-int32_t scratch_of_current_device(void **out) {
+// Looks the array's device address up for the calling thread's current device and makes that device's event: set-up, once
+// per device (from pmetal_hip_init, else on the first call for that device).
+int32_t scratch_of_current_device(NoAllocScratch **out) {
     int dev = 0;
     HIP_TRY(hipGetDevice(&dev));
     if (dev < 0 || dev >= kMaxScratchDevices) return fail(PMETAL_HIP_ERR_INVALID_ARG, "device %d is beyond the %d devices the library keeps scratch for", dev, kMaxScratchDevices);
     std::lock_guard<std::mutex> lock(g_scratch_mu);
-    if (!g_scratch_ptr[dev]) {
+    NoAllocScratch &sc = g_scratch[dev];
+    if (!sc.ptr) {
         void *p = nullptr;
         HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
         if (!p) return fail(PMETAL_HIP_ERR_HIP_RUNTIME, "hipGetSymbolAddress returned no address for the scratch array");
-        g_scratch_ptr[dev] = p;
+        HIP_TRY(hipEventCreateWithFlags(&sc.done, hipEventDisableTiming));
+        sc.ptr = p;
     }
-    *out = g_scratch_ptr[dev];
+    *out = &sc;
     return PMETAL_HIP_OK;
 }
 
@@ -298,7 +333,7 @@ int32_t pmetal_hip_init(int32_t device) {
     if (device < 0 || device >= n) return fail(PMETAL_HIP_ERR_INVALID_ARG, "device %d out of range [0, %d)", device, n);
     HIP_TRY(hipSetDevice(device));
     HIP_TRY(hipFree(nullptr));  // forces context creation and code-object load
-    void *sp = nullptr;
+    NoAllocScratch *sp = nullptr;
     if (int32_t rc = scratch_of_current_device(&sp)) return rc;  // so that pmetal_hip_qgemm_noalloc has nothing left to set up
     return ok();
 }
@@ -430,7 +465,7 @@ void *pmetal_hip_stream_create(void) {
 int32_t pmetal_hip_stream_destroy(void *stream) {
     if (!stream) return ok();
     HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
-    drop_workspaces_of((hipStream_t)stream);  // the calling thread's scratch for this stream (other threads' goes at their exit)
+    drop_workspaces_of((hipStream_t)stream);  // every thread's scratch for this stream, pinned buffers included
     HIP_TRY(hipStreamDestroy((hipStream_t)stream));
     return ok();
 }
@@ -811,7 +846,7 @@ static int32_t qgemm_over_reblocked(uint32_t t, const uint8_t *wa, int64_t n, in
 }
 
 static size_t reblocked_scratch_bytes(uint32_t t, int64_t m, int64_t n, int64_t k, uint32_t y_dtype, size_t *gemm_bytes) {
-    *gemm_bytes = up16(pmh::qgemm_workspace_bytes(m, n, k));
+    *gemm_bytes = up16(pmh::qgemm_workspace_bytes(PMETAL_GGML_TYPE_Q6K, m, n, k));
     const size_t y_bytes = up16((size_t)m * (size_t)n * 4);
     return *gemm_bytes + (pmh::reblock_q6k_parts(t) == 2 ? y_bytes * (y_dtype == PMETAL_HIP_DTYPE_F32 ? 1 : 2) : 0);
 }
@@ -896,7 +931,7 @@ int32_t pmetal_hip_qgemm(uint32_t t, const uint8_t *w, int64_t n, int64_t k, con
     if (!pmh::qgemm_fits(t, m, n, k))
         return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qgemm: m and k must be at most 2^22 (m = %lld, k = %lld)", (long long)m, (long long)k);
     void *ws = nullptr;
-    if (int32_t rc = workspace(pmh::qgemm_workspace_bytes(m, n, k), (hipStream_t)stream, &ws)) return rc;
+    if (int32_t rc = workspace(pmh::qgemm_workspace_bytes(t, m, n, k), (hipStream_t)stream, &ws)) return rc;
     hipError_t e = pmh::launch_qgemm(t, w, n, k, x, x_dtype, m, y, y_dtype, order, ws, (hipStream_t)stream);
     if (e == hipErrorNotSupported) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "qgemm: configuration not supported");
     if (e != hipSuccess) return hip_fail(e, "qgemm kernel launch");
@@ -919,7 +954,7 @@ int32_t pmetal_hip_qgemm_batch(const pmetal_hip_gemm_desc *descs, size_t count, 
         if (k % 256 != 0) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qgemm: k=%lld is not a multiple of 256", (long long)k);
         if (!pmh::qgemm_fits(d.ggml_type, m, d.n, k))
             return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qgemm: m and k must be at most 2^22 (m = %lld, k = %lld)", (long long)m, (long long)k);
-        const size_t b = pmh::qgemm_workspace_bytes(m, d.n, k);
+        const size_t b = pmh::qgemm_workspace_bytes(d.ggml_type, m, d.n, k);
         need = b > need ? b : need;
     }
     if (count == 0) return ok();
@@ -929,15 +964,17 @@ int32_t pmetal_hip_qgemm_batch(const pmetal_hip_gemm_desc *descs, size_t count, 
     auto layout = [](const pmetal_hip_gemm_desc &d) {
         return d.ggml_type == PMETAL_GGML_TYPE_Q8_0 ? 3 : (d.ggml_type == PMETAL_GGML_TYPE_Q6K ? 2 : (d.order == PMETAL_HIP_ORDER_REF ? 0 : 1));
     };
-    int have = -1;
+    // ... and through the padded row count of the launch plan, which follows n: the item stride and the place of the row
+    // scales behind the items change with it, so a narrow weight behind a wide one gets a pre-pass of its own
+    int have = -1, have_mp = -1;
     for (size_t i = 0; i < count; i++) {
         const pmetal_hip_gemm_desc &d = descs[i];
-        const int want = layout(d);
+        const int want = layout(d), want_mp = pmh::qgemm_plan(m, d.n, k).mp;
         hipError_t e = pmh::launch_qgemm(d.ggml_type, d.w_dev, d.n, k, x, x_dtype, m, d.y_dev, d.y_dtype, d.order, ws, (hipStream_t)stream,
-                                         want == have);
+                                         want == have && want_mp == have_mp);
         if (e == hipErrorNotSupported) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "qgemm: configuration not supported");
         if (e != hipSuccess) return hip_fail(e, "qgemm kernel launch");
-        have = want;
+        have = want, have_mp = want_mp;
     }
     return ok();
 }
@@ -956,15 +993,41 @@ int32_t pmetal_hip_qgemm_noalloc(uint32_t t, const uint8_t *w, int64_t n, int64_
     if (k % 256 != 0) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qgemm: k=%lld is not a multiple of 256", (long long)k);
     if (!pmh::qgemm_fits(t, m, n, k))
         return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qgemm: m and k must be at most 2^22 (m = %lld, k = %lld)", (long long)m, (long long)k);
-    const size_t need = pmh::qgemm_workspace_bytes(m, n, k);
+    const size_t need = pmh::qgemm_workspace_bytes(t, m, n, k);
     if (need > kNoAllocScratchBytes)
         return fail(PMETAL_HIP_ERR_SHAPE_TOO_LARGE, "qgemm_noalloc: m=%lld, n=%lld, k=%lld needs %zu bytes of scratch, the fixed array holds %zu",
                     (long long)m, (long long)n, (long long)k, need, kNoAllocScratchBytes);
-    void *ws = nullptr;
-    if (int32_t rc = scratch_of_current_device(&ws)) return rc;
-    hipError_t e = pmh::launch_qgemm(t, w, n, k, x, x_dtype, m, y, y_dtype, order, ws, (hipStream_t)stream);
+    NoAllocScratch *sc = nullptr;
+    if (int32_t rc = scratch_of_current_device(&sc)) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (s) HIP_TRY(hipStreamIsCapturing(s, &cap));
+    const bool recording = cap != hipStreamCaptureStatusNone;
+    if (sc->busy.exchange(true))
+        return fail(PMETAL_HIP_ERR_BUSY, "qgemm_noalloc: another thread is issuing a call on this device, and all calls share one scratch array");
+    struct Release {
+        std::atomic<bool> &flag;
+        ~Release() { flag.store(false); }
+    } release{sc->busy};
+    if (!recording && sc->pending) {
+        if (sc->last == s) {
+            // same stream: this call's kernels run behind the previous call's
+        } else {
+            const hipError_t q = hipEventQuery(sc->done);
+            if (q == hipErrorNotReady)
+                return fail(PMETAL_HIP_ERR_BUSY, "qgemm_noalloc: the previous call on this device, on another stream, has not finished and "
+                                                 "all calls share one scratch array (wait for that stream, or use one stream)");
+            if (q != hipSuccess) return hip_fail(q, "hipEventQuery");
+            sc->pending = false;
+        }
+    }
+    hipError_t e = pmh::launch_qgemm(t, w, n, k, x, x_dtype, m, y, y_dtype, order, sc->ptr, s);
     if (e == hipErrorNotSupported) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "qgemm: configuration not supported");
     if (e != hipSuccess) return hip_fail(e, "qgemm kernel launch");
+    if (!recording) {
+        HIP_TRY(hipEventRecord(sc->done, s));
+        sc->last = s, sc->pending = true;
+    }
     return ok();
 }
 

@@ -1573,10 +1573,12 @@ GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k) {
     return p;
 }
 
-size_t qgemm_workspace_bytes(int64_t m, int64_t n, int64_t k) {
+size_t qgemm_workspace_bytes(uint32_t type, int64_t m, int64_t n, int64_t k) {
     const GemmPlan p = qgemm_plan(m, n, k);
     const size_t xs = align256((size_t)(k / 256) * 2 * kGroups * p.mp * 16);
-    const size_t part = p.splits > 1 ? align256((size_t)p.splits * p.mp * n * 4) : 0;
+    // the short-batch kernels take a row of up to kSmallMaxSpr super-blocks whole: the plan's K split is not used there
+    const bool unsplit = qgemm_small_applies(type, m, n, k) && k / 256 <= kSmallMaxSpr;
+    const size_t part = p.splits > 1 && !unsplit ? align256((size_t)p.splits * p.mp * n * 4) : 0;
     return xs + align256((size_t)p.mp * 4) + part;
 }
 

@@ -70,8 +70,8 @@ struct GemmPlan {
 };
 bool qgemm_fits(uint32_t type, int64_t m, int64_t n, int64_t k);
 GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k);
-// Bytes of device workspace qgemm needs for (m, n, k); the caller provides it.
-size_t qgemm_workspace_bytes(int64_t m, int64_t n, int64_t k);
+// Bytes of device workspace qgemm needs for a weight of `type` at (m, n, k); the caller provides it.
+size_t qgemm_workspace_bytes(uint32_t type, int64_t m, int64_t n, int64_t k);
 // reuse_prepass: the workspace still holds the converted activations of the previous launch_qgemm on this stream with the same
 // x, m, k and weight type (two weights that share their activations: the pre-pass runs once)
 hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype,

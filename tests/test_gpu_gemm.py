@@ -424,6 +424,38 @@ def test_qgemm_batch_equals_separate_calls(oracle):
 
 
 @pytest.mark.parametrize("t", [Q4K, Q6K, Q8_0])
+@pytest.mark.parametrize("m", [300, 200, 516])
+def test_qgemm_batch_wide_and_narrow_weights_share_x(oracle, t, m):
+    """A wide and a narrow weight of one type and element order behind each other (q_proj / k_proj of a prefill): the launch plan
+    pads the activation rows differently for the two (m = 300: 384 rows for n = 4096, 320 for n = 1024), so the converted
+    activations of the first must not serve the second.  Both orders of the descriptors, bit for bit against separate calls."""
+    lib = _lib.load()
+    k = 4096
+    rng = np.random.default_rng(977 + m + t)
+    ns = (4096, 1024)
+    ws = [pm.DeviceBuffer.from_host(oracle.quantize(t, weights(4100 + n, n * k))) for n in ns]
+    xb = oracle.f32_to_bf16_bits(rng.standard_normal(m * k).astype(np.float32))
+    dx = pm.DeviceBuffer.from_host(xb)
+    y_one = []
+    for w, n in zip(ws, ns):
+        y = pm.DeviceBuffer(m * n * 4)
+        pm.check(lib.pmetal_hip_qgemm(t, w.ptr, n, k, dx.ptr, pm.DTYPE_BF16, m, y.ptr, pm.DTYPE_F32, 0, None))
+        pm.check(lib.pmetal_hip_sync(None))
+        y_one.append(y.to_host(np.uint8))
+    for first in (0, 1):
+        idx = (first, 1 - first)
+        y_bat = [pm.DeviceBuffer(m * ns[i] * 4) for i in idx]
+        descs = (_lib.GemmDesc * 2)()
+        for j, i in enumerate(idx):
+            pm.check(lib.pmetal_hip_memset(y_bat[j].ptr, 0xFF, m * ns[i] * 4, None))
+            descs[j] = _lib.GemmDesc(t, pm.DTYPE_F32, 0, 0, ns[i], ws[i].ptr, y_bat[j].ptr)
+        pm.check(lib.pmetal_hip_qgemm_batch(descs, 2, k, dx.ptr, pm.DTYPE_BF16, m, None))
+        pm.check(lib.pmetal_hip_sync(None))
+        for j, i in enumerate(idx):
+            assert np.array_equal(y_one[i], y_bat[j].to_host(np.uint8)), (m, first, ns[i])
+
+
+@pytest.mark.parametrize("t", [Q4K, Q6K, Q8_0])
 @pytest.mark.parametrize("m", [1, 2, 5, 9, 16])
 @pytest.mark.parametrize("n,k", [(700, 2048), (333, 4096), (16, 2048), (4099, 4096), (40, 1024),
                                  # rows of more than 16 super-blocks: runs of 16, partial tiles added in a second kernel
