@@ -22,13 +22,27 @@
  *                           and refused; single-element moves taken and refused;
  *                           every exit) and Gaussian inputs in the reference's order.
  *                           Also the reference's closed forms (quantize.rs:998-1032).
- *   quantize_q8_0 ......... fully determined by IEEE ops: numpy twin is exact.
+ *   quantize_q8_0 ......... rational expected bytes (same fixture): a short last block, a
+ *                           zero block, a negative maximum, blocks where 127 / amax and
+ *                           1 / (amax / 127) round an element differently; numpy twin.
  *   quantize_q4k/q5k/q6k/q3k/q2k
  *                           whole super-blocks built from those inputs with bytes
- *                           derived by the rational restatement (same fixture); block
- *                           sizes, reference round-trip bounds (k_quants.rs:1446-1553).
- *                           The Rust itself was never run (no toolchain here).
- *   dequantize_* .......... reference KATs (dequant.rs:1016-1036,
+ *                           derived by the rational restatement (same fixture), and
+ *                           blocks that single out one step each: max_min folded from
+ *                           +0.0, two scales of equal magnitude and opposite sign, a
+ *                           scale code of 128, scale code 0, all-zero blocks, Gaussian
+ *                           blocks whose bytes change when d / dmin are not the decoded
+ *                           f16 values or the quotient is not an IEEE division, tensors
+ *                           with a partial last super-block; block sizes, reference
+ *                           round-trip bounds (k_quants.rs:1446-1553).
+ *                           tests/test_oracle_mutations.py edits this file one line at a
+ *                           time (one edit or more per item of the bit-exactness checklist)
+ *                           and checks that the fixture alone notices each edit.
+ *                           These are two restatements of the Rust by reading, pinned
+ *                           against each other; the Rust itself was never run (no
+ *                           toolchain here).
+ *   dequantize_* .......... rational expected values for random block bytes (same fixture);
+ *                           reference KATs (dequant.rs:1016-1036,
  *                           k_quants.rs:1368-1383) + hand-built blocks + numpy.
  *   quantize_q4_0/q4_1/q5_0/q5_1/q8_1, dequantize_legacy
  *                           the reference's block tests (dequant.rs:935-1053), every code

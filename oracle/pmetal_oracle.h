@@ -19,8 +19,14 @@
  *     every early exit), plus Gaussian inputs with one rounding per operation in
  *     the reference's order;
  *   pmo_quantize_q4k / _q5k / _q6k / _q3k / _q2k: whole super-blocks built from
- *     those inputs.
- * What stays unpinned in the strict sense: nothing was ever compared with output
+ *     those inputs, blocks that single out one super-block step each (decoded f16
+ *     d / dmin in the requantization, IEEE division, the fold from +0.0, the first
+ *     of equal scale magnitudes, the scale code 128, scale code 0, all-zero and
+ *     partial blocks), pmo_quantize_q8_0 and the dequantizers likewise;
+ *   tests/test_oracle_mutations.py edits pmetal_oracle.c one line at a time and
+ *     checks that the fixture alone notices every edit.
+ * The oracle is thus pinned by two independent restatements of the Rust, not by
+ * the reference itself.  What stays unpinned in the strict sense: nothing was ever compared with output
  * of the Rust itself; a misreading of the Rust shared by the C restatement and
  * the rational one (written separately, from the Rust) would pass.
  */

@@ -422,6 +422,8 @@ def make_qx_quants(n: int, nmax: int, x, rmse_type: int):
             break
         if slx * slx <= best * sl2:
             _T.hit(f"qx:rescale{p + 1}:rejected")
+            if slx * slx == best * sl2:
+                _T.hit("qx:rescale:tie_rejected")
             break
         _T.hit(f"qx:rescale{p + 1}:accepted")
         for i in range(n):           # :802-805
@@ -453,6 +455,8 @@ def make_qx_quants(n: int, nmax: int, x, rmse_type: int):
                         _T.hit(f"qx:descent{sweep + 1}:rejected")
             else:
                 _T.hit("qx:descent:slx<=0")
+                if slx == ZERO:
+                    _T.hit("qx:descent:slx==0")
         if n_changed == 0:           # :835
             _T.hit(f"qx:descent:stop_after_sweep_{sweep + 1}")
             break
@@ -714,3 +718,97 @@ def quantize_q2k_block(x):  # k_quants.rs:1242-1323
 
 BLOCK_QUANTIZERS = {12: quantize_q4k_block, 13: quantize_q5k_block, 14: quantize_q6k_block,
                     11: quantize_q3k_block, 10: quantize_q2k_block}
+
+
+# ------------------------------------------------------------------------------------------------
+# whole tensors: a trailing partial super-block is emitted as zeros (k_quants.rs:890-892, :1070-1072)
+# ------------------------------------------------------------------------------------------------
+BLOCK_BYTES = {12: 144, 13: 176, 14: 210, 11: 110, 10: 84}
+
+
+def quantize_tensor(t: int, x) -> bytes:
+    if t == 8:
+        return quantize_q8_0(x)
+    out = b""
+    for b in range((len(x) + 255) // 256):
+        blk = x[256 * b:256 * b + 256]
+        out += BLOCK_QUANTIZERS[t](blk) if len(blk) == 256 else bytes(BLOCK_BYTES[t])
+    return out
+
+
+def quantize_q8_0(x) -> bytes:  # quantize.rs:268-300
+    out = []
+    for b in range((len(x) + 31) // 32):
+        blk = x[32 * b:32 * b + 32]
+        amax = ZERO
+        for v in blk:                # fold(0.0, |acc, x| acc.max(x.abs()))
+            amax = rust_max(amax, v.abs())
+        scale = amax / F32.of(127)
+        iscale = ZERO if amax == ZERO else F32.of(127) / amax
+        out += _u16le(f32_to_f16_bits(scale))
+        for i in range(32):
+            out.append(clamp(nearest_int(blk[i] * iscale), -127, 127) & 0xFF if i < len(blk) else 0)
+    return bytes(out)
+
+
+# ------------------------------------------------------------------------------------------------
+# dequantizers: every product and difference is rounded on its own
+# ------------------------------------------------------------------------------------------------
+def dequantize_q8_0(raw: bytes, n: int):  # dequant.rs:466-495
+    y = []
+    for b in range(len(raw) // 34):
+        blk = raw[34 * b:34 * b + 34]
+        scale = f16_bits_to_f32(blk[0] | (blk[1] << 8))
+        for i in range(32):
+            q = blk[2 + i] - 256 if blk[2 + i] >= 128 else blk[2 + i]
+            y.append(F32.of(q) * scale)
+    return y[:n]
+
+
+def dequantize_q4k(raw: bytes, n: int, ggml_order: bool = False):
+    """k_quants.rs:358-404 (the reference's order).  ggml_order: the inverse of quantize_q4k's packing (:946-951) instead."""
+    y = []
+    for b in range(len(raw) // 144):
+        blk = raw[144 * b:144 * b + 144]
+        d, dmin = f16_bits_to_f32(blk[0] | (blk[1] << 8)), f16_bits_to_f32(blk[2] | (blk[3] << 8))
+        sc, qs = list(blk[4:16]), blk[16:]
+        is_ = 0
+        for j in range(0, 256, 64):
+            s1, m1 = get_scale_min_k4(is_, sc)
+            s2, m2 = get_scale_min_k4(is_ + 1, sc)
+            d1, dm1 = d * F32.of(s1), dmin * F32.of(m1)
+            d2, dm2 = d * F32.of(s2), dmin * F32.of(m2)
+            q = qs[j // 2:j // 2 + 32]
+            if ggml_order:
+                y += [d1 * F32.of(q[l] & 0xF) - dm1 for l in range(32)]
+                y += [d2 * F32.of(q[l] >> 4) - dm2 for l in range(32)]
+            else:
+                y += [d1 * F32.of(q[l] & 0xF) - dm1 for l in range(16)]
+                y += [d1 * F32.of(q[l] >> 4) - dm1 for l in range(16)]
+                y += [d2 * F32.of(q[16 + l] & 0xF) - dm2 for l in range(16)]
+                y += [d2 * F32.of(q[16 + l] >> 4) - dm2 for l in range(16)]
+            is_ += 2
+    return y[:n]
+
+
+def dequantize_q6k(raw: bytes, n: int):  # k_quants.rs:474-496
+    y = []
+    for b in range(len(raw) // 210):
+        blk = raw[210 * b:210 * b + 210]
+        d = f16_bits_to_f32(blk[208] | (blk[209] << 8))
+        out = [None] * 256
+        for c in range(2):
+            ql, qh = blk[64 * c:], blk[128 + 32 * c:]
+            sc = [v - 256 if v >= 128 else v for v in blk[192 + 8 * c:192 + 8 * c + 8]]
+            for l in range(32):
+                is_ = l // 16
+                q1 = ((ql[l] & 0xF) | ((qh[l] & 3) << 4)) - 32
+                q2 = ((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32
+                q3 = ((ql[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32
+                q4 = ((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32
+                out[128 * c + l] = d * F32.of(sc[is_]) * F32.of(q1)
+                out[128 * c + l + 32] = d * F32.of(sc[is_ + 2]) * F32.of(q2)
+                out[128 * c + l + 64] = d * F32.of(sc[is_ + 4]) * F32.of(q3)
+                out[128 * c + l + 96] = d * F32.of(sc[is_ + 6]) * F32.of(q4)
+        y += out
+    return y[:n]

@@ -83,6 +83,41 @@ QX_INPUTS = [
     # the largest magnitude twice with both signs: the first one (positive) decides, the other is clamped to 31
     [24.0, -24.0, 3.0, -5.0, 7.0, 1.0, 0.0, 2.0, -9.0, 11.0, 4.0, -6.0, 8.0, -2.0, 5.0, -1.0],
 ]
+# the new quants of a rescale pass differ from the old ones and slx^2 == best * sl2 exactly (quantize.rs:798 refuses the pass on a
+# tie); found by a search over sub-blocks of small integers and half-integers
+QX_TIE_INPUTS = [
+    [-19.0, -21.0, -16.0, 19.0, -3.0, 13.0, 0.0, 22.0, 14.0, 6.0, -14.0, -23.0, -5.0, -14.0, 4.0, -2.0],
+    [11.0, 11.0, -13.0, -11.0, 23.0, 13.0, 5.0, -1.0, -9.0, -13.0, -21.0, -21.0, 10.0, -7.0, -23.0, 4.0],
+    [17.0, 8.0, -24.0, 22.0, 4.0, 24.0, 5.0, 10.0, 7.0, -3.0, -10.0, 13.0, -2.0, -14.0, 19.0, -4.0],
+    [12.0, -1.5, -3.0, 2.5, 6.0, -1.0, -4.5, -0.5, 1.5, 3.0, -6.5, 0.0, -12.0, -9.5, -10.0, -9.5],
+    [10.5, -11.5, -1.5, 11.0, 7.0, -11.5, -1.0, 8.0, 6.5, 3.5, -4.5, 11.5, -4.0, 0.5, 2.0, 8.5],
+]
+# one element carries the whole of sumlx (every other quant is 0): slx == 0 exactly for it (quantize.rs:819), both signs
+QX_SLX_ZERO_INPUTS = [
+    [-32.0, 0.25, -0.25, 0.125, 0.0, 0.375, -0.125, 0.25, 0.0, 0.0, 0.125, -0.375, 0.25, 0.0, -0.25, 0.125],
+    [0.125, 0.125, 16.0, -0.125, 0.0, 0.0, 0.125, -0.125, 0.0, 0.125, 0.0, 0.0, -0.125, 0.0, 0.125, 0.0],
+]
+# Gaussian super-blocks (block `index` of gaussian(default_rng(seed), blocks * elements)) whose bytes change when a step of the
+# block quantizer is done differently; found by a search, kept as (type, blocks in the stream, seed, index, what they pin)
+GAUSS_PICKS = [
+    (12, 64, 7000, 3, "requantize with the decoded f16 d / dmin (k_quants.rs:935-937)"),
+    (12, 64, 7000, 4, "requantize with the decoded f16 d / dmin (k_quants.rs:935-937)"),
+    (13, 64, 7000, 0, "requantize with the decoded f16 d / dmin (k_quants.rs:1016-1018)"),
+    (13, 64, 7000, 1, "requantize with the decoded f16 d / dmin (k_quants.rs:1016-1018)"),
+    (10, 64, 7000, 19, "requantize with the decoded f16 d / dmin (k_quants.rs:1300-1304)"),
+    (10, 64, 7000, 43, "requantize with the decoded f16 d / dmin (k_quants.rs:1300-1304)"),
+    (11, 64, 7000, 42, "requantize with the decoded f16 d (k_quants.rs:1199)"),
+    (11, 64, 7001, 26, "requantize with the decoded f16 d (k_quants.rs:1199)"),
+    (14, 64, 7000, 1, "requantize with the decoded f16 d (k_quants.rs:1106)"),
+    (14, 64, 7000, 3, "requantize with the decoded f16 d (k_quants.rs:1106)"),
+    (12, 20000, 7000, 7616, "(x + dm) / d is a division, not a product with 1 / d (k_quants.rs:939)"),
+    (12, 20000, 7001, 6501, "(x + dm) / d is a division, not a product with 1 / d (k_quants.rs:939)"),
+    (14, 20000, 7000, 15395, "x / d is a division, not a product with 1 / d (k_quants.rs:1109)"),
+    (14, 20000, 7000, 17017, "x / d is a division, not a product with 1 / d (k_quants.rs:1109)"),
+    (8, 100000, 7000, 54099, "iscale = 127 / amax, not 1 / (amax / 127) (quantize.rs:282)"),
+    (8, 100000, 7001, 58597, "iscale = 127 / amax, not 1 / (amax / 127) (quantize.rs:282)"),
+    (8, 100000, 7001, 86130, "iscale = 127 / amax, not 1 / (amax / 127) (quantize.rs:282)"),
+]
 Q3_INPUTS = [
     [27.0, -19.0, -32.0, -16.0, -7.0, 25.0, -4.0, -33.0, -13.0, 8.0, 25.0, 19.0, 40.0, -25.0, 31.0, -36.0],
     [-1.0, 32.0, -5.0, 9.0, -34.0, 27.0, -5.0, 0.0, -33.0, 16.0, 11.0, -13.0, 22.0, 2.0, -36.0, -23.0],
@@ -155,7 +190,7 @@ def block_case(name, t, xs, family, parts):
 
 
 def main():
-    out = {"qkx1": [], "qx": [], "q3": [], "blocks": []}
+    out = {"qkx1": [], "qx": [], "q3": [], "blocks": [], "tensors": [], "dequant": []}
     rng = np.random.default_rng(20240607)
 
     # ---- make_qkx1_quants ----
@@ -193,6 +228,14 @@ def main():
         assert c["order_free"], c["name"]
         out["qx"].append(c)
         qsubs.append((c["name"], xs))
+    for i, pat in enumerate(QX_TIE_INPUTS):
+        c = case_qx(f"qx_rescale_tie_{i}", [f32(v) for v in pat], "order_free")
+        assert c["order_free"] and "qx:rescale:tie_rejected" in c["branches"], c["name"]
+        out["qx"].append(c)
+    for i, pat in enumerate(QX_SLX_ZERO_INPUTS):
+        c = case_qx(f"qx_slx_zero_{i}", [f32(v) for v in pat], "order_free")
+        assert c["order_free"] and "qx:descent:slx==0" in c["branches"], c["name"]
+        out["qx"].append(c)
     out["qx"].append(case_qx("qx_all_zero", [f32(0)] * 16, "special"))
     out["qx"].append(case_qx("qx_rmse_type_0", [f32(v) for v in QX_INPUTS[0]], "order_free", rmse_type=0))
     for i in range(24):
@@ -247,6 +290,93 @@ def main():
             if i == 1:  # the benchmark's outliers
                 xs[17], xs[200] = f32(0.5), f32(-0.5)
             out["blocks"].append(block_case(f"block_type{t}_gauss_{i}", t, xs, "ordered", []))
+
+    # ---- super-blocks that single out one step of the block quantizers ----
+    # Q4_K / Q5_K / Q2_K with every element positive: each sub-block returns the min -0.0, and max_min folds from +0.0
+    # (k_quants.rs:904-905), so dmin is 0x0000 and not 0x8000
+    pos15 = [xs for name, xs in subs[15] if all(x.q > 0 for x in xs)]
+    pos3 = [xs for name, xs in subs[3] if all(x.q > 0 for x in xs)]
+    assert pos15 and pos3
+    allpos32 = sum((scaled(pos15[0], -(j % 3) - 4) for j in range(8)), [])
+    allpos16 = sum((scaled(pos3[0], -(j % 3) - 4) for j in range(16)), [])
+    for t, xs in ((12, allpos32), (13, allpos32), (10, allpos16)):
+        c = block_case(f"block_type{t}_all_positive", t, xs, "order_free", ["all-positive sub-blocks"])
+        raw = bytes.fromhex(c["bytes"])
+        assert (raw[2:4] if t != 10 else raw[82:84]) == bytes(2), "dmin must be +0.0"
+        out["blocks"].append(c)
+    # Q6_K: two sub-blocks whose scales are +1 and -1 exactly (an exact grid and its mirror image), the others smaller: the
+    # first of the two decides the sign of d (k_quants.rs:1090), and the other one's scale code 128 is cut to 127 (:1101)
+    grid = [f32(v) for v in QX_INPUTS[15]]
+    assert case_qx("", grid, "order_free")["scale_bits"] == f32(1).bits()
+    mirror = [-x for x in grid]
+    assert case_qx("", mirror, "order_free")["scale_bits"] == f32(-1).bits()
+    small = [scaled(qsubs[(3 * j) % 15][1], -7 - j % 4) for j in range(14)]
+    for name, first, second in (("plus_first", grid, mirror), ("minus_first", mirror, grid)):
+        xs = sum(small[:5], []) + first + sum(small[5:9], []) + second + sum(small[9:], [])
+        c = block_case(f"block_type14_equal_scales_{name}", 14, xs, "order_free", ["scales +1 and -1"])
+        raw = bytes.fromhex(c["bytes"])
+        codes = sorted(v - 256 if v > 127 else v for v in (raw[192 + 5], raw[192 + 10]))
+        assert codes == [-128, 127], codes
+        out["blocks"].append(c)
+    # a sub-block far below the largest one gets the scale code 0 and keeps its quants: all 0 in Q4_K (k_quants.rs:936), the ones
+    # make_qx_quants left in Q6_K (:1107)
+    tiny4 = sum((scaled(subs[15][j % len(subs[15])][1], -3 if j != 2 else -20) for j in range(8)), [])
+    tiny6 = sum((scaled(qsubs[j % len(qsubs)][1], -5 if j != 4 else -24) for j in range(16)), [])
+    out["blocks"].append(block_case("block_type12_scale_code_zero", 12, tiny4, "order_free", ["sub-block 2 at 2^-17 of the others"]))
+    out["blocks"].append(block_case("block_type14_scale_code_zero", 14, tiny6, "order_free", ["sub-block 4 at 2^-19 of the others"]))
+    # all-zero super-blocks: Q4_K / Q5_K / Q3_K / Q2_K all-zero bytes, Q6_K d = f16(-0.0) = 0x8000 (k_quants.rs:1096-1097)
+    for t in (12, 13, 14, 11, 10):
+        c = block_case(f"block_type{t}_all_zero", t, [f32(0)] * 256, "special", [])
+        assert (bytes.fromhex(c["bytes"])[208:210] == bytes([0, 0x80])) if t == 14 else not any(bytes.fromhex(c["bytes"]))
+        out["blocks"].append(c)
+    # the Gaussian picks
+    for t, nblocks, seed, index, why in GAUSS_PICKS:
+        el = 32 if t == 8 else 256
+        stream = (np.random.default_rng(seed).standard_normal(nblocks * el) * 0.02).astype(np.float32)
+        xs = [E.F32.from_bits(int(u)) for u in stream[index * el:(index + 1) * el].view(np.uint32)]
+        E.new_trace()
+        c = {"name": f"pick_type{t}_seed{seed}_{index}", "family": "ordered", "type": t, "x_bits": bits_of(xs),
+             "bytes": E.quantize_tensor(t, xs).hex(), "pins": why}
+        out["blocks" if t != 8 else "tensors"].append(c)
+
+    # ---- whole tensors: ragged lengths and Q8_0 ----
+    def tensor_case(name, t, xs, family):
+        E.new_trace()
+        return {"name": name, "family": family, "type": t, "x_bits": bits_of(xs), "bytes": E.quantize_tensor(t, xs).hex()}
+
+    tail = [f32(Fraction(v, 8)) for v in range(-22, 22)]  # 44 elements past the last whole super-block: emitted as zeros
+    for t, blk in ((12, tiny4), (13, allpos32), (14, tiny6), (11, sum((scaled(q3subs[j % len(q3subs)][1], -5) for j in range(16)), [])),
+                   (10, allpos16)):
+        c = tensor_case(f"tensor_type{t}_300_elements", t, blk + tail, "order_free")
+        assert len(c["bytes"]) == 4 * E.BLOCK_BYTES[t] and not any(bytes.fromhex(c["bytes"])[E.BLOCK_BYTES[t]:])
+        out["tensors"].append(c)
+    ramp = [f32(Fraction(v - 16, 8)) for v in range(40)]  # Q8_0: a whole block and 8 elements of a second one
+    out["tensors"].append(tensor_case("tensor_q8_0_40_elements", 8, ramp, "order_free"))
+    out["tensors"].append(tensor_case("tensor_q8_0_zero_block", 8, [f32(0)] * 32, "special"))
+    neg = [f32(-127)] + [f32(v) for v in range(-15, 16)]  # the largest magnitude is negative: amax = |x|, codes reach -127
+    out["tensors"].append(tensor_case("tensor_q8_0_negative_maximum", 8, neg, "order_free"))
+    out["tensors"].append(tensor_case("tensor_q8_0_gauss", 8, gaussian(rng, 96), "ordered"))
+
+    # ---- dequantizers: block bytes -> values, every product and difference rounded on its own ----
+    def dequant_case(name, t, raw, n, order):
+        fn = {8: lambda: E.dequantize_q8_0(raw, n), 12: lambda: E.dequantize_q4k(raw, n, order == 1), 14: lambda: E.dequantize_q6k(raw, n)}[t]
+        E.new_trace()
+        return {"name": name, "type": t, "order": order, "n": n, "bytes": raw.hex(), "y_bits": [y.bits() for y in fn()]}
+
+    drng = np.random.default_rng(4242)
+    for t, size in ((12, 144), (14, 210), (8, 34)):
+        nblk = 2 if t != 8 else 5
+        raw = bytearray(drng.integers(0, 256, nblk * size, dtype=np.uint8).tobytes())
+        for b in range(nblk):  # finite f16 scales (clear the top exponent bit)
+            for off in {12: (1, 3), 14: (209,), 8: (1,)}[t]:
+                raw[b * size + off] &= 0xBF
+        n = nblk * (32 if t == 8 else 256) - 7  # the output is cut to n elements
+        for order in ((0, 1) if t == 12 else (0,)):
+            out["dequant"].append(dequant_case(f"dequant_type{t}_order{order}_random_bytes", t, bytes(raw), n, order))
+    for c in out["blocks"]:  # and what the quantizers wrote for the Gaussian blocks
+        if c["name"] in ("block_type12_gauss_0", "block_type14_gauss_0"):
+            for order in ((0, 1) if c["type"] == 12 else (0,)):
+                out["dequant"].append(dequant_case(f"dequant_{c['name']}_order{order}", c["type"], bytes.fromhex(c["bytes"]), 256, order))
 
     path = os.path.join(HERE, "exact_cases.json")
     with open(path, "w") as f:

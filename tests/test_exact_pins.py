@@ -38,9 +38,26 @@ Which order-free case reaches which lines of the reference (asserted by ``test_o
   quantize.rs:693       slx <= 0 skips the element                         q3:descent:slx<=0
   quantize.rs:700-705   move accepted / rejected in sweeps 1 .. 5          q3:descent1..5:accepted, q3:descent1..5:rejected
   quantize.rs:709-711   1 .. 5 sweeps, and five sweeps that all change     q3:descent:stop_after_sweep_1 .. _5, q3:descent:five_sweeps_changed
+  quantize.rs:798       slx^2 == best * sl2 exactly with changed quants: refused    qx:rescale:tie_rejected  (qx_rescale_tie_0 .. _4)
+  quantize.rs:819       slx == 0 exactly                                   qx:descent:slx==0        (qx_slx_zero_0, _1)
 Whole super-blocks (``blocks``): 8 or 16 of the order-free sub-blocks above, each scaled by its own power of two (exact), so
 that the super-block steps (largest scale, 6-bit / 4-bit / signed scale codes, f16 d and dmin, requantization with the
-decoded scales, bit packing) run on known sub-block results; those steps hold no sums, only single operations.
+decoded scales, bit packing) run on known sub-block results; those steps hold no sums, only single operations.  Blocks that
+single out one step each:
+  k_quants.rs:904-905   max_min folds from +0.0 (all sub-blocks return -0.0)         block_type12/13/10_all_positive
+  k_quants.rs:1090      the first of two scales of equal magnitude decides d's sign  block_type14_equal_scales_plus_first, _minus_first
+  k_quants.rs:1101      a scale code of 128 is cut to 127 before `as i8`             the same two blocks
+  k_quants.rs:936,1107  `if d != 0.0`: a sub-block with scale code 0 keeps its quants block_type12/14_scale_code_zero
+  k_quants.rs:1096-97   all-zero Q6_K block: d = f16(-0.0) = 0x8000                  block_type14_all_zero (and the other types' zero blocks)
+  k_quants.rs:935-937, :1016-1018, :1106, :1199, :1300-1304   requantization with the decoded f16 d / dmin: Gaussian blocks whose
+                        bytes differ if the unrounded value is used                  pick_type12/13/14/11/10_seed7000_*
+  k_quants.rs:939,1109  the quotient is an IEEE division (blocks with a quotient next to a rounding boundary)   pick_type12/14_seed700x_*
+Whole tensors (``tensors``): a trailing partial super-block is emitted as zeros (k_quants.rs:890-892 and the like; 300 elements
+of every k-quant type), Q8_0 (quantize.rs:268-300) with a short last block, a zero block, a negative maximum, and Gaussian
+blocks where round(x * (127 / amax)) differs from round(x * (1 / (amax / 127))) (:282, pick_type8_*).
+Dequantizers (``dequant``): random block bytes and quantized Gaussian blocks -> values in rational arithmetic, both element
+orders for Q4_K, the output cut to n elements.
+``tests/test_oracle_mutations.py`` edits the oracle one line at a time and checks that these cases notice.
 """
 import json
 import os
@@ -69,6 +86,7 @@ REQUIRED_ORDER_FREE = {
     "q3:descent:stop_after_sweep_1",
     "q3:descent:stop_after_sweep_2", "q3:descent:stop_after_sweep_3", "q3:descent:stop_after_sweep_4",
     "q3:descent:stop_after_sweep_5", "q3:descent:five_sweeps_changed",
+    "qx:rescale:tie_rejected", "qx:descent:slx==0",
 }
 
 
@@ -206,6 +224,31 @@ def test_oracle_block_bytes(oracle, case):
     assert np.array_equal(got, want), np.nonzero(got != want)[0][:8]
 
 
+@pytest.mark.parametrize("case", CASES["tensors"], ids=[c["name"] for c in CASES["tensors"]])
+def test_oracle_tensor_bytes(oracle, case):
+    got = oracle.quantize(case["type"], f32_from_bits(case["x_bits"]))
+    assert got.tobytes().hex() == case["bytes"]
+
+
+@pytest.mark.parametrize("case", CASES["dequant"], ids=[c["name"] for c in CASES["dequant"]])
+def test_oracle_dequantized_bits(oracle, case):
+    raw = np.frombuffer(bytes.fromhex(case["bytes"]), dtype=np.uint8)
+    got = oracle.dequantize(case["type"], raw, [case["n"]], order=case["order"])
+    assert [int(v) for v in got.view(np.uint32)] == case["y_bits"]
+
+
+def test_fixture_tensor_and_dequant_cases_reproduce_from_the_rational_reference():
+    for c in CASES["tensors"]:
+        E.new_trace()
+        assert E.quantize_tensor(c["type"], _xs(c)).hex() == c["bytes"], c["name"]
+    for c in CASES["dequant"][:3]:
+        raw = bytes.fromhex(c["bytes"])
+        fn = {8: lambda: E.dequantize_q8_0(raw, c["n"]), 12: lambda: E.dequantize_q4k(raw, c["n"], c["order"] == 1),
+              14: lambda: E.dequantize_q6k(raw, c["n"])}[c["type"]]
+        E.new_trace()
+        assert [y.bits() for y in fn()] == c["y_bits"], c["name"]
+
+
 # ---- the HIP quantizers against the fixture (not against the oracle) ------------------------------------------------------
 @pytest.mark.gpu
 def test_gpu_block_bytes_equal_the_rational_reference():
@@ -222,3 +265,18 @@ def test_gpu_block_bytes_equal_the_rational_reference():
         for c in cases:  # and one block at a time (a tensor of a single super-block)
             one = pm.quantize(f32_from_bits(c["x_bits"]), pm.GgmlType(t))
             assert np.array_equal(one, np.frombuffer(bytes.fromhex(c["bytes"]), dtype=np.uint8)), c["name"]
+
+
+@pytest.mark.gpu
+def test_gpu_tensor_bytes_and_dequantized_bits_equal_the_rational_reference():
+    """Ragged tensors, Q8_0 and the dequantizers through the HIP library against the rational fixture."""
+    import pmetal_amd as pm
+
+    pm.init(0)
+    for c in CASES["tensors"]:
+        got = pm.quantize(f32_from_bits(c["x_bits"]), pm.GgmlType(c["type"]))
+        assert got.tobytes().hex() == c["bytes"], c["name"]
+    for c in CASES["dequant"]:
+        raw = np.frombuffer(bytes.fromhex(c["bytes"]), dtype=np.uint8)
+        got = pm.dequantize(raw, pm.GgmlType(c["type"]), [c["n"]], order=c["order"])
+        assert [int(v) for v in got.view(np.uint32)] == c["y_bits"], c["name"]
