@@ -8,7 +8,8 @@ Q4_K batch-1 decode GEMV, W 14336x4096, x bf16, fp32 accumulate.  A step is one 
 over a batch of 16 distinct weight tensors (16 same-shaped layers of a decode step): 16 x 33 MB is
 larger than the 256 MB last-level cache, so every step streams its weights from HBM.
 
-Timing: HIP events recorded on the stream the kernels are launched on (the null stream), bracketed by
+Timing: HIP events recorded on the stream the kernels are launched on (the null stream, or the stream of a recorded
+launch sequence that is replayed), bracketed by
 stream synchronisation; inputs are resident in HBM before the timed region.  `roofline.achieved` is
 algorithmic bytes (or flops) per launch divided by the average launch duration over the timed region.
 The CPU baseline is the oracle's restatement of the reference algorithm (dequantize, then an f32
@@ -255,8 +256,20 @@ def bench_gemv(args, n, k, t=Q4K, copies=16, passes=8):
                 pm.check(lib.pmetal_hip_qgemv_batch(descs_, copies, None))
         return run
 
-    ev_ms, wall_ms = timer.run(sweeps(solo), args.steps, args.warmup)
+    eager_ms, _ = timer.run(sweeps(solo), args.steps, args.warmup)
     launches = args.steps * copies * passes
+    # the same launches recorded once (a HIP graph) and replayed with one submission per step: what a decoder does
+    stream = lib.pmetal_hip_stream_create()
+    pm.check(lib.pmetal_hip_record_begin(stream))
+    for _ in range(passes):
+        pm.check(lib.pmetal_hip_qgemv_batch(solo, copies, stream))
+    rec = lib.pmetal_hip_record_end(stream)
+    if not rec:
+        raise RuntimeError(lib.pmetal_hip_last_error_message())
+    timer.stream = stream
+    ev_ms, wall_ms = timer.run(lambda: pm.check(lib.pmetal_hip_replay(rec, stream)), args.steps, args.warmup)
+    timer.stream = None
+    pm.check(lib.pmetal_hip_recording_destroy(rec))
     bytes_per_launch = gemv_bytes(t, n, k, 2)
     us_per_launch = ev_ms * 1e3 / launches
     gbs = bytes_per_launch / (us_per_launch * 1e-6) / 1e9
@@ -289,7 +302,9 @@ def bench_gemv(args, n, k, t=Q4K, copies=16, passes=8):
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
                      "kernel": {Q4K: "k_qgemv_q4k_rows" if k in (2048, 4096) else "k_qgemv_q4k_chunk", Q6K: "k_qgemv_q6k_chunk", Q8_0: "k_qgemv_q8_0_chunk", 13: "k_qgemv_q5k_chunk", 11: "k_qgemv_q23k_chunk<FormatQ3K>", 10: "k_qgemv_q23k_chunk<FormatQ2K>"}[t], "bytes_per_launch": bytes_per_launch,
                      "us_per_launch": round(us_per_launch, 3)},
-        "extra": {"cache_resident_GBps": round(cached_gbs, 1), "cache_resident_us_per_launch": round(c_ms * 1e3 / launches, 3),
+        "extra": {"submission": "the step's 128 launches recorded once and replayed (one submission per step)",
+                  "eager_us_per_launch": round(eager_ms * 1e3 / launches, 3),
+                  "cache_resident_GBps": round(cached_gbs, 1), "cache_resident_us_per_launch": round(c_ms * 1e3 / launches, 3),
                   "weight_copies": copies, "launches_per_step": copies * passes,
                   "batch_entry_us_per_matrix": round(b_ms * 1e3 / launches, 3),
                   "plain_read_us": {"hbm": round(read_us, 3), "cache_resident": round(read_cached_us, 3),
@@ -438,6 +453,7 @@ def bench_gemm(args, m, n, k, t=Q4K):
     flops = 2.0 * m * n * k
     us = ev_ms * 1e3 / (args.steps * copies)
     tflops = flops / (us * 1e-6) / 1e12
+    dense = dense_library_tflops(m, n, k) if args.dense_library else None
     pair_us = None
     if t in (Q4K, Q6K, Q8_0):  # two weights against the same activations (gate / up): one pre-pass for both
         if copies == 1:
@@ -460,12 +476,47 @@ def bench_gemm(args, m, n, k, t=Q4K):
                      "flops_per_launch": flops, "us_per_launch": round(us, 3)},
         "extra": {"calls_per_step": copies, "weights": f"{copies} tensor(s) in turn" + (" (from HBM)" if copies > 1 else " (33 MB: stays in the last-level cache)"),
                   "mfma_loop_sustained_TFLOPs": round(sustained, 1), "frac_of_sustained": round(tflops / sustained, 4),
+                  "dense_library_TFLOPs": dense,
                   "two_weights_sharing_x_us_per_weight": None if pair_us is None else round(pair_us, 3),
                   "two_weights_sharing_x_TFLOPs": None if pair_us is None else round(flops / (pair_us * 1e-6) / 1e12, 1),
                   **({} if per_call_us is None else {"weight": "re-blocked to Q6_K once (pmetal_hip_reblock_dev), then pmetal_hip_qgemm_reblocked per call",
                                                     "reblocked_bytes": rb_bytes,
                                                     "reblocking_on_every_call_us": round(per_call_us, 3)})},
     }, (t, n, k)
+
+
+_DENSE_SCRIPT = """
+import sys, torch
+m, n, k, reps = (int(a) for a in sys.argv[1:5])
+x = torch.randn(m, k, device="cuda", dtype=torch.float16)
+w = (torch.randn(n, k, device="cuda", dtype=torch.float32) * 0.02).to(torch.float16)
+for _ in range(5):
+    y = x @ w.t()
+torch.cuda.synchronize()
+e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+e0.record()
+for _ in range(reps):
+    y = x @ w.t()
+e1.record()
+torch.cuda.synchronize()
+print("TFLOPS", 2.0 * m * n * k * reps / (e0.elapsed_time(e1) * 1e-3) / 1e12)
+"""
+
+
+def dense_library_tflops(m, n, k, reps=50):
+    """A yardstick beside the kernel, never part of it: the f16 product of the same shape (X[m,k] W[n,k]^T, dense, already
+    dequantized) through torch.matmul, i.e. the vendor's GEMM library, timed with torch's own events on this machine.  It
+    runs in a child process: torch brings its own HIP runtime, which cannot share a process with the one this library loads."""
+    import subprocess
+    try:
+        r = subprocess.run([sys.executable, "-c", _DENSE_SCRIPT, str(m), str(n), str(k), str(reps)], capture_output=True, text=True,
+                           timeout=240)
+    except (OSError, subprocess.TimeoutExpired):
+        return None
+    for line in r.stdout.splitlines():
+        if line.startswith("TFLOPS"):
+            return round(float(line.split()[1]), 1)
+    return None
 
 
 def bench_dequantize(args, n, k):
@@ -655,11 +706,13 @@ for _name, _t in (("q5k", 13), ("q3k", 11), ("q2k", 10)):  # re-blocked into Q6_
 
 
 def other_parts(args):
-    """The Q4_K GEMM at M = 512 and the Llama-3-8B-shaped f32 -> Q4_K_M quantizer, each with its roofline and CPU baseline."""
+    """The other parts of the metric and of its configurations: the Q4_K GEMM at M = 512 (with the sweep over M), the
+    Llama-3-8B-shaped f32 -> Q4_K_M quantizer, the GEMV's second shape and the decode step of the small model."""
     import copy
     out = {}
     a = copy.copy(args)
     a.steps, a.warmup = max(args.steps, 50), max(args.warmup, 5)
+    a.dense_library = True
     res, _ = bench_gemm(a, 512, 14336, 4096, Q4K)
     wl = WORKLOADS["gemm_q4k_m512"]
     out["gemm_q4k_m512"] = {"metric": wl["metric"], "value": round(res["value"], 1), "unit": wl["unit"], "dtype": wl["dtype"],
@@ -667,6 +720,37 @@ def other_parts(args):
                             "extra": res["extra"]}
     if not args.no_cpu_baseline:
         out["gemm_q4k_m512"]["cpu_baseline"] = cpu_baseline_gemm(Q4K, 512, 14336, 4096, budget_s=3.0)
+    # the sweep of the prefill configuration: the crossover from the GEMV to the matrix cores
+    a.dense_library = False
+    for m in (16, 64, 128, 2048):
+        a.steps, a.warmup = (50, 5) if m <= 128 else (20, 3)
+        res, _ = bench_gemm(a, m, 14336, 4096, Q4K)
+        wl = WORKLOADS[f"gemm_q4k_m{m}"]
+        hbm = None
+        if m <= 128:  # short batches are bound by reading the weights
+            gb = (14336 * 16 * 144 + 2 * m * 4096 + 2 * m * 14336) / (res["roofline"]["us_per_launch"] * 1e-6) / 1e9
+            hbm = {"bound": "hbm", "achieved": round(gb, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gb / HBM_PEAK_GBS, 4)}
+        out[f"gemm_q4k_m{m}"] = {"metric": wl["metric"], "value": round(res["value"], 1), "unit": wl["unit"], "dtype": wl["dtype"],
+                                 "steps": a.steps, "us_per_call": res["roofline"]["us_per_launch"], "roofline": res["roofline"],
+                                 **({"roofline_hbm": hbm} if hbm else {}), "weights": res["extra"]["weights"]}
+    # the second shape of the decode configuration (the down projection)
+    a = copy.copy(args)
+    a.steps, a.warmup = max(args.steps // 4, 10), max(args.warmup // 4, 2)
+    res, _ = bench_gemv(a, 4096, 14336, Q4K)
+    wl = WORKLOADS["gemv_q4k_4096x14336"]
+    rec = RECORDED_TRAFFIC.get("gemv_q4k_4096x14336")
+    res["roofline"]["traffic"] = rec[0] if rec else None
+    out["gemv_q4k_4096x14336"] = {"metric": wl["metric"], "value": round(res["value"], 1), "unit": wl["unit"], "dtype": wl["dtype"],
+                                  "steps": a.steps, "ms_per_step": round(res["ms_per_step"], 5), "roofline": res["roofline"],
+                                  "extra": res["extra"]}
+    # the decode step of the small model (tokens/s over its linear projections)
+    a = copy.copy(args)
+    a.steps, a.warmup = max(args.steps, 100), max(args.warmup, 10)
+    res, _ = bench_decode(a, "qwen3_0.6b")
+    wl = WORKLOADS["decode_qwen3_0.6b_q4km"]
+    out["decode_qwen3_0.6b_q4km"] = {"metric": wl["metric"], "value": round(res["value"], 1), "unit": wl["unit"], "dtype": wl["dtype"],
+                                     "steps": a.steps, "ms_per_step": round(res["ms_per_step"], 5), "roofline": res["roofline"],
+                                     "extra": res["extra"]}
     a = copy.copy(args)
     a.steps, a.warmup = 5, 1
     res, _ = bench_quantize(a)
@@ -688,6 +772,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra-workloads", action="store_true",
                     help="default workload only: do not also time the GEMM and quantizer parts of the metric")
+    ap.add_argument("--dense-library", action="store_true",
+                    help="GEMM workloads: also time torch.matmul (f16, same shape) as a yardstick; the default run does so for M = 512")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain streaming kernel of known size (f32 -> bf16 over 2^24 elements: 64 MiB read, "
                          "32 MiB written) so that profiler byte counters can be scaled against it")
@@ -719,7 +805,7 @@ def main():
                  else "synthetic: N(0,0.02) f32 weights generated and quantized on the device, x ~ N(0,1) bf16"),
         "config": {"workload": args.workload, "element_order": "GGML" if wl["kind"] == "calibrate" else "REF",
                    "step": {"gemm": "one GEMM launch (activation pre-pass + MFMA kernel)",
-                            "gemv": "8 sweeps of 16 back-to-back GEMV launches, one per distinct weight tensor (HBM-resident: 528 MB for Q4_K)",
+                            "gemv": "8 sweeps of 16 back-to-back GEMV launches, one per distinct weight tensor (HBM-resident: 528 MB for Q4_K), replayed from a recorded launch sequence",
                             "gemv_q8k": "16 x (activations f32 -> Q8_K, integer-dot GEMV) over 16 distinct weight tensors",
                             "calibrate": "one tensor resident in HBM: 6 candidates x (quantize, fused dequantize-and-score, f64 score read back)",
                             "decode": "all batch-1 projections of one token (197 for Qwen3-0.6B, 225 for Llama-3-8B), back to back on one stream",

@@ -54,10 +54,13 @@ __global__ __launch_bounds__(256) void k_fill_normal(float *__restrict__ dst, si
 }
 
 // Register-only loop of v_mfma_f32_32x32x16_f16: 8 waves per workgroup (two per SIMD), four independent
-// accumulators per wave, no memory traffic.  With `vary` the operands differ per lane and one of them changes sign
-// every trip (one extra VALU instruction per four matrix instructions); without it they are all 1.0.
+// accumulators per wave, no memory traffic.  With `vary` the operands differ per lane and one register of an operand changes
+// sign after every four matrix instructions (one v_xor with a compile-time register index: the loop body is eight such
+// groups written out, so nothing is selected at run time); without it they are all 1.0.  `iters` counts groups of four
+// matrix instructions and is rounded down to a multiple of eight.
 typedef _Float16 probe_half8 __attribute__((ext_vector_type(8)));
 typedef float probe_float16 __attribute__((ext_vector_type(16)));
+typedef uint32_t probe_u32x4 __attribute__((ext_vector_type(4)));
 __global__ __launch_bounds__(512) void k_mfma_probe(int iters, int vary, float *__restrict__ sink) {
     probe_half8 a, b;
 #pragma unroll
@@ -65,15 +68,20 @@ __global__ __launch_bounds__(512) void k_mfma_probe(int iters, int vary, float *
         a[i] = (_Float16)(vary ? (float)((threadIdx.x * 37 + i * 11) % 97) * 0.37f - 17.0f : 1.0f);
         b[i] = (_Float16)(vary ? (float)((threadIdx.x * 13 + i * 7) % 89) * 0.21f - 9.0f : 1.0f);
     }
+    const uint32_t flip = vary ? 0x80008000u : 0u;  // the sign bits of the two halves of a register
     probe_float16 c0, c1, c2, c3;
 #pragma unroll
     for (int i = 0; i < 16; i++) c0[i] = 0.0f, c1[i] = 0.0f, c2[i] = 0.0f, c3[i] = 0.0f;
-    for (int i = 0; i < iters; i++) {
-        c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c0, 0, 0, 0);
-        c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c1, 0, 0, 0);
-        c2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c2, 0, 0, 0);
-        c3 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c3, 0, 0, 0);
-        if (vary) a[i & 7] = -a[i & 7];
+    for (int i = 0; i < iters / 8; i++) {
+#pragma unroll
+        for (int g = 0; g < 8; g++) {
+            c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c0, 0, 0, 0);
+            c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c1, 0, 0, 0);
+            c2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c2, 0, 0, 0);
+            c3 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c3, 0, 0, 0);
+            probe_u32x4 &bits = reinterpret_cast<probe_u32x4 &>((g & 1) ? b : a);
+            bits[g >> 1] ^= flip;
+        }
     }
     float s = 0.0f;
 #pragma unroll
