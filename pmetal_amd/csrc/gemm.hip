@@ -253,7 +253,10 @@ __device__ __forceinline__ void store_tile(const float16_t (&acc)[MB], uint4 *sm
         }
         uint8_t *dst = out + ((size_t)m * N + n) * esize;
         if (rows_aligned && n + per <= N) {
-            *reinterpret_cast<uint4 *>(dst) = pack;
+            // Y is not read again by this launch: a streaming store keeps it from pushing the activation items and the
+            // other row blocks' weights out of the caches (a partial tile is read back by the reduction: an ordinary store)
+            if (mode == 2) *reinterpret_cast<uint4 *>(dst) = pack;
+            else __builtin_nontemporal_store(u32x4{pack.x, pack.y, pack.z, pack.w}, reinterpret_cast<u32x4 *>(dst));
         } else {
             for (int e = 0; e < per && n + e < N; e++) {
                 if (mode == 1) reinterpret_cast<uint16_t *>(dst)[e] = (uint16_t)bf16_rne_bits(v[e]);
