@@ -41,7 +41,11 @@ RECORDED_TRAFFIC = {"gemv_q4k_14336x4096": (33287193, "profiles/qgemv_q4k_14336x
                     "gemv_q8_0_14336x4096": (62653287, "profiles/qgemv_other_types.md"),
                     "gemv_q5k_6144x4096": (17530063, "profiles/qgemv_other_types.md"),
                     "gemv_q3k_14336x4096": (25568799, "profiles/qgemv_other_types.md"),
-                    "gemv_q2k_14336x4096": (19580687, "profiles/qgemv_other_types.md")}
+                    "gemv_q2k_14336x4096": (19580687, "profiles/qgemv_other_types.md"),
+                    # per call: pre-pass + matrix kernel; per step: all 226 tensors; per tensor
+                    "gemm_q4k_m512": (99287040, "profiles/qgemm_q4k_m512.md"),
+                    "quantize_llama3_8b_q4km": (37284068260, "profiles/quantize_q4km_llama3_8b.md"),
+                    "dequantize_14336x4096": (268075008, "profiles/dequantize_14336x4096.md")}
 BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16/fp16 MFMA, published
 Q8_0, Q4K, Q6K = 8, 12, 14
 
@@ -705,6 +709,13 @@ for _name, _t in (("q5k", 13), ("q3k", 11), ("q2k", 10)):  # re-blocked into Q6_
                                            metric=f"{_name.upper().replace('K', '_K')} GEMM TFLOPS (nominal flops) @M=512,K=4096,N=14336")
 
 
+def set_recorded_traffic(roofline, workload):
+    rec = RECORDED_TRAFFIC.get(workload)
+    roofline["traffic"] = rec[0] if rec else None
+    if rec:
+        roofline["traffic_source"] = f"recorded constant from {rec[1]} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE), not measured in this run"
+
+
 def other_parts(args):
     """The other parts of the metric and of its configurations: the Q4_K GEMM at M = 512 (with the sweep over M), the
     Llama-3-8B-shaped f32 -> Q4_K_M quantizer, the GEMV's second shape and the decode step of the small model."""
@@ -715,6 +726,7 @@ def other_parts(args):
     a.dense_library = True
     res, _ = bench_gemm(a, 512, 14336, 4096, Q4K)
     wl = WORKLOADS["gemm_q4k_m512"]
+    set_recorded_traffic(res["roofline"], "gemm_q4k_m512")
     out["gemm_q4k_m512"] = {"metric": wl["metric"], "value": round(res["value"], 1), "unit": wl["unit"], "dtype": wl["dtype"],
                             "steps": a.steps, "ms_per_step": round(res["ms_per_step"], 5), "roofline": res["roofline"],
                             "extra": res["extra"]}
@@ -738,8 +750,7 @@ def other_parts(args):
     a.steps, a.warmup = max(args.steps // 4, 10), max(args.warmup // 4, 2)
     res, _ = bench_gemv(a, 4096, 14336, Q4K)
     wl = WORKLOADS["gemv_q4k_4096x14336"]
-    rec = RECORDED_TRAFFIC.get("gemv_q4k_4096x14336")
-    res["roofline"]["traffic"] = rec[0] if rec else None
+    set_recorded_traffic(res["roofline"], "gemv_q4k_4096x14336")
     out["gemv_q4k_4096x14336"] = {"metric": wl["metric"], "value": round(res["value"], 1), "unit": wl["unit"], "dtype": wl["dtype"],
                                   "steps": a.steps, "ms_per_step": round(res["ms_per_step"], 5), "roofline": res["roofline"],
                                   "extra": res["extra"]}
@@ -755,6 +766,7 @@ def other_parts(args):
     a.steps, a.warmup = 5, 1
     res, _ = bench_quantize(a)
     wl = WORKLOADS["quantize_llama3_8b_q4km"]
+    set_recorded_traffic(res["roofline"], "quantize_llama3_8b_q4km")
     out["quantize_llama3_8b_q4km"] = {"metric": wl["metric"], "value": round(res["value"], 1), "unit": wl["unit"],
                                       "dtype": wl["dtype"], "steps": a.steps, "ms_per_step": round(res["ms_per_step"], 5),
                                       "roofline": res["roofline"], "extra": res["extra"]}
@@ -822,10 +834,7 @@ def main():
         else:
             out["config"]["arithmetic"] = ("bf16 activations converted exactly to fixed-point int8 digit planes, v_dot4_i32_i8 against "
                                            "the quantized weights, f32 block scales and accumulation")
-    rec = RECORDED_TRAFFIC.get(args.workload)
-    out["roofline"]["traffic"] = rec[0] if rec else None
-    if rec:
-        out["roofline"]["traffic_source"] = f"recorded constant from {rec[1]} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE), not measured in this run"
+    set_recorded_traffic(out["roofline"], args.workload)
     if args.calibrate:
         pm, _lib, lib = load()
         n_cal = 1 << 24
