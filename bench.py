@@ -435,9 +435,16 @@ def bench_gemm(args, m, n, k, t=Q4K):
         for wi in wl:
             pm.check(lib.pmetal_hip_qgemm(t, wi.ptr, n, k, x.ptr, pm.DTYPE_BF16, m, y.ptr, pm.DTYPE_BF16, 0, None))
 
-    step, per_call_us = per_call, None
+    step, per_call_us, reblocked_us = per_call, None, None
     rb_bytes = lib.pmetal_hip_reblock_size(t, n, k)
-    if rb_bytes:  # Q5_K / Q3_K / Q2_K: re-blocked once, as a loader does; the per-call form is timed beside it
+    if rb_bytes and t == 13:  # Q5_K has a matrix kernel of its own; its re-blocked form (two Q6_K tensors) is timed beside it
+        rb = pm.DeviceBuffer(rb_bytes)
+        pm.check(lib.pmetal_hip_reblock_dev(t, w.ptr, n, k, 0, rb.ptr, rb_bytes, None), "reblock")
+        rb_ms, _ = timer.run(lambda: pm.check(lib.pmetal_hip_qgemm_reblocked(t, rb.ptr, rb_bytes, n, k, x.ptr, pm.DTYPE_BF16, m, y.ptr, pm.DTYPE_BF16, None)),
+                             args.steps, args.warmup)
+        reblocked_us = rb_ms * 1e3 / args.steps
+        rb.free()
+    elif rb_bytes:  # Q3_K / Q2_K: re-blocked once, as a loader does; the per-call form is timed beside it
         rb = pm.DeviceBuffer(rb_bytes)
         pm.check(lib.pmetal_hip_reblock_dev(t, w.ptr, n, k, 0, rb.ptr, rb_bytes, None), "reblock")
 
@@ -459,7 +466,7 @@ def bench_gemm(args, m, n, k, t=Q4K):
     tflops = flops / (us * 1e-6) / 1e12
     dense = dense_library_tflops(m, n, k) if args.dense_library else None
     pair_us = None
-    if t in (Q4K, Q6K, Q8_0):  # two weights against the same activations (gate / up): one pre-pass for both
+    if t in (Q4K, Q6K, Q8_0, 13):  # two weights against the same activations (gate / up): one pre-pass for both
         if copies == 1:
             wl.append(device_weights(pm, lib, t, n * k, 2001))
         y2 = pm.DeviceBuffer(2 * m * n)
@@ -476,13 +483,14 @@ def bench_gemm(args, m, n, k, t=Q4K):
         "value": tflops, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / BF16_PEAK_TFLOPS, 4), "traffic": None,
-                     "kernel": {Q4K: "k_qgemm_rw", Q6K: "k_qgemm_rw_q6", Q8_0: "k_qgemm_rw_q8"}.get(t, "k_qgemm_rw_q6 per Q6_K part of the re-blocked weight") + " (+ k_prep_rw, k_rw_reduce when K is split)",
+                     "kernel": {Q4K: "k_qgemm_rw", 13: "k_qgemm_rw<FMT = 1>", Q6K: "k_qgemm_rw_q6", Q8_0: "k_qgemm_rw_q8"}.get(t, "k_qgemm_rw_q6 per Q6_K part of the re-blocked weight") + " (+ k_prep_rw, k_rw_reduce when K is split)",
                      "flops_per_launch": flops, "us_per_launch": round(us, 3)},
         "extra": {"calls_per_step": copies, "weights": f"{copies} tensor(s) in turn" + (" (from HBM)" if copies > 1 else " (33 MB: stays in the last-level cache)"),
                   "mfma_loop_sustained_TFLOPs": round(sustained, 1), "frac_of_sustained": round(tflops / sustained, 4),
                   "dense_library_TFLOPs": dense,
                   "two_weights_sharing_x_us_per_weight": None if pair_us is None else round(pair_us, 3),
                   "two_weights_sharing_x_TFLOPs": None if pair_us is None else round(flops / (pair_us * 1e-6) / 1e12, 1),
+                  **({} if reblocked_us is None else {"reblocked_form_us": round(reblocked_us, 3), "reblocked_bytes": rb_bytes}),
                   **({} if per_call_us is None else {"weight": "re-blocked to Q6_K once (pmetal_hip_reblock_dev), then pmetal_hip_qgemm_reblocked per call",
                                                     "reblocked_bytes": rb_bytes,
                                                     "reblocking_on_every_call_us": round(per_call_us, 3)})},
@@ -704,7 +712,7 @@ WORKLOADS["gemm_q8_0_m16"] = dict(kind="gemm", m=16, n=14336, k=4096, metric="Q8
                                   unit="TFLOP/s", dtype="f16", type=Q8_0)
 WORKLOADS["gemm_q6k_m16"] = dict(kind="gemm", m=16, n=14336, k=4096, metric="Q6_K GEMM TFLOPS @M=16,K=4096,N=14336",
                                  unit="TFLOP/s", dtype="f16", type=Q6K)
-for _name, _t in (("q5k", 13), ("q3k", 11), ("q2k", 10)):  # re-blocked into Q6_K inside the call (two tensors, one, two)
+for _name, _t in (("q5k", 13), ("q3k", 11), ("q2k", 10)):  # Q5_K: its own kernel; Q3_K / Q2_K: re-blocked into Q6_K (one tensor, two)
     WORKLOADS[f"gemm_{_name}_m512"] = dict(kind="gemm", m=512, n=14336, k=4096, unit="TFLOP/s", dtype="f16", type=_t,
                                            metric=f"{_name.upper().replace('K', '_K')} GEMM TFLOPS (nominal flops) @M=512,K=4096,N=14336")
 

@@ -129,12 +129,13 @@ class DeviceBuffer {
 // A GGUF-quantized weight [n, k] resident on the device; the counterpart of LayerWeight for GGUF types.
 class GgufLinear {
    public:
-    // prepare_gemm: re-block a Q5_K / Q3_K / Q2_K weight once into the Q6_K form its GEMM multiplies with, as the reference
-    // brings a weight into its matmul's layout when the model is loaded (weights.rs:29-45); the original blocks stay for the GEMV
+    // prepare_gemm: re-block a Q3_K / Q2_K weight once into the Q6_K form its GEMM multiplies with, as the reference
+    // brings a weight into its matmul's layout when the model is loaded (weights.rs:29-45); the original blocks stay for the
+    // GEMV.  (Q5_K has a matrix kernel that reads its blocks as they are: nothing is prepared for it.)
     GgufLinear(GgmlType dtype, int64_t n, int64_t k, const std::vector<uint8_t> &packed,
                uint32_t order = PMETAL_HIP_ORDER_REF, bool prepare_gemm = false)
         : dtype_(dtype), n_(n), k_(k), order_(order), w_(check_size(dtype, n, k, packed), packed.size()) {
-        if (prepare_gemm) {
+        if (prepare_gemm && dtype_ != GgmlType::Q5K) {
             const size_t len = pmetal_hip_reblock_size((uint32_t)dtype_, n_, k_);
             if (len) {
                 reblocked_.reset(new DeviceBuffer(len));

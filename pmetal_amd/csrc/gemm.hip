@@ -1,6 +1,6 @@
-// Dequant-fused Q4_K, Q6_K and Q8_0 GEMM  Y[m,n] = sum_k X[m,k] * W[n,k]  on the gfx950 matrix cores, every wave
-// owning its weight rows.  The text below describes Q4_K; the Q6_K and Q8_0 kernels further down note their
-// differences.
+// Dequant-fused Q4_K, Q5_K, Q6_K and Q8_0 GEMM  Y[m,n] = sum_k X[m,k] * W[n,k]  on the gfx950 matrix cores, every wave
+// owning its weight rows.  The text below describes Q4_K (Q5_K is the same kernel with the fifth bit of every quant
+// taken from the block's qh bytes: FMT = 1); the Q6_K and Q8_0 kernels further down note their differences.
 //
 // W is the packed GGUF stream [n, k] of 144-byte super-blocks; a weight's value is what the reference's
 // dequantize_q4k yields (crates/pmetal-gguf/src/k_quants.rs:358-404; element order REF or GGML as for the
@@ -47,6 +47,12 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kGroups = 18;    // 16-byte items per activation row and half super-block
 constexpr int kBlockBytes = 144;
+// FMT 0: Q4_K (144 bytes: d, dmin, 12 scale bytes, 128 quant bytes); FMT 1: Q5_K (176 bytes: the same header, then 32 bytes
+// qh with the fifth bits, then the 128 quant bytes; crates/pmetal-gguf/src/k_quants.rs:407-462)
+template <int FMT>
+struct BlockFmt {
+    static constexpr int kBytes = FMT ? 176 : 144, kQs = FMT ? 48 : 16;
+};
 
 #define PMH_GPTR(p) ((const __attribute__((address_space(1))) void *)(p))
 #define PMH_LPTR(p) ((__attribute__((address_space(3))) void *)(p))
@@ -77,8 +83,9 @@ __device__ __forceinline__ float bf16_to_f32(uint32_t h) { return __builtin_bit_
 // per row with the row index fastest across lanes, so that four lanes write 64 contiguous bytes of every item row).  rowscale[m] = 2^e with the row maximum * 2^-e in
 // [2^9, 2^10) (bf16 activations are then exact in f16 and block sums stay below 2^15); rows >= M are zero.
 // One thread per operand item: chunk u = 64 elements = sub-blocks 2u, 2u+1 (u = 4 sb + 2 h + g), k-step t.
-// ORDER 0 / 1: Q4_K element orders REF / GGML; ORDER 2: the Q6_K layout, ORDER 3: the natural order (Q8_0), both
-// without block sums.
+// ORDER 0 / 1: Q4_K element orders REF / GGML (1 is also Q5_K's GGML order); ORDER 2: the Q6_K layout, ORDER 3: the
+// natural order (Q8_0), both without block sums; ORDER 4: Q5_K's REF order, whose sub-block j holds its 32 elements as
+// consecutive nibbles of 16 bytes, so k-step t of a chunk is elements 8 t .. 8 t + 7, the even ones (low nibbles) first.
 // ------------------------------------------------------------------------------------------------
 template <bool XF32, int ORDER, int R>
 __global__ __launch_bounds__(R == 1 ? 512 : 1024) void k_prep_rw(const void *__restrict__ xg, int64_t k, int M, int Mp,
@@ -127,7 +134,7 @@ __global__ __launch_bounds__(R == 1 ? 512 : 1024) void k_prep_rw(const void *__r
         // the item's two runs of four elements (lo, hi), its half super-block and its operand group
         int64_t lo, hi, half;
         int t, g;
-        if (ORDER >= 2) {  // half = 128 elements, 16 items
+        if (ORDER == 2 || ORDER == 3) {  // half = 128 elements, 16 items
             half = q >> 4;
             t = (int)(q & 15) >> 1, g = (int)q & 1;
             if (ORDER == 2) {  // Q6_K: low nibbles at 32 g + 4 t, high nibbles 64 further
@@ -141,8 +148,8 @@ __global__ __launch_bounds__(R == 1 ? 512 : 1024) void k_prep_rw(const void *__r
             const int64_t u = q >> 3;
             t = (int)(q & 7), g = (int)u & 1;
             half = u >> 1;
-            lo = ORDER == 0 ? 64 * u + 32 * (t >> 2) + 4 * (t & 3) : 64 * u + 4 * t;
-            hi = lo + (ORDER == 0 ? 16 : 32);
+            lo = ORDER == 4 ? 64 * u + 8 * t : (ORDER == 0 ? 64 * u + 32 * (t >> 2) + 4 * (t & 3) : 64 * u + 4 * t);
+            hi = lo + (ORDER == 4 ? 4 : (ORDER == 0 ? 16 : 32));
         }
         float v[8];
         if (!live) {
@@ -158,6 +165,11 @@ __global__ __launch_bounds__(R == 1 ? 512 : 1024) void k_prep_rw(const void *__r
             v[0] = bf16_to_f32(a.x & 0xFFFFu), v[1] = bf16_to_f32(a.x >> 16), v[2] = bf16_to_f32(a.y & 0xFFFFu), v[3] = bf16_to_f32(a.y >> 16);
             v[4] = bf16_to_f32(b.x & 0xFFFFu), v[5] = bf16_to_f32(b.x >> 16), v[6] = bf16_to_f32(b.y & 0xFFFFu), v[7] = bf16_to_f32(b.y >> 16);
         }
+        if (ORDER == 4) {  // eight consecutive elements: the even ones, then the odd ones
+            const float e[8] = {v[0], v[2], v[4], v[6], v[1], v[3], v[5], v[7]};
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[i] = e[i];
+        }
         half8_t h;
         float slo = 0.0f, shi = 0.0f;
 #pragma unroll
@@ -168,10 +180,10 @@ __global__ __launch_bounds__(R == 1 ? 512 : 1024) void k_prep_rw(const void *__r
         }
         const size_t base = (size_t)(half * kGroups) * Mp + m;
         xs[base + (size_t)(t * 2 + g) * Mp] = __builtin_bit_cast(uint4, h);
-        if (ORDER >= 2) continue;  // Q6_K and Q8_0 have no min term: no block sums
+        if (ORDER == 2 || ORDER == 3) continue;  // Q6_K and Q8_0 have no min term: no block sums
         // sums of the two sub-blocks of the chunk over its 8 k-steps (8 lanes, R apart)
         float s0, s1;
-        if (ORDER == 0) {  // sub-block 2u: k-steps 0..3 (low and high nibbles), 2u+1: k-steps 4..7
+        if (ORDER == 0 || ORDER == 4) {  // sub-block 2u: k-steps 0..3 (low and high nibbles), 2u+1: k-steps 4..7
             float s = slo + shi;
             s += __shfl_xor(s, R);
             s += __shfl_xor(s, 2 * R);
@@ -274,6 +286,7 @@ struct Lane {
     int wave, col, g;
     uint32_t q_off[NR][2];     // byte offset of this lane's quant piece of round r from the workgroup's first row
     uint32_t h_off[NR];        // ... of this lane's header
+    uint32_t qh_off[NR];       // ... of this lane's piece of the fifth bits (Q5_K: row lane / 2, piece lane % 2)
     uint32_t a_off[kARounds];  // item offset of this lane's activation item of round i from (group 0, row m0)
 };
 
@@ -281,6 +294,7 @@ template <int MB, int NR>
 struct Acc {
     float16_t acc[NR][MB], part[NR][MB];
     u32x4 hdr[NR];  // headers of the current super-block: d | dmin << 16, then the 12 scale bytes
+    uint32_t qh[NR][8];  // Q5_K: the 32 qh bytes of the current super-block of this lane's row
 };
 
 // 8 quants of one dword (low nibbles, then high nibbles) times their integer scales -> 8 exact f16 values:
@@ -293,10 +307,25 @@ struct Dq {
     half2_t r[4];
     __device__ __forceinline__ half8_t value() const { return half8_t{r[0][0], r[0][1], r[1][0], r[1][1], r[2][0], r[2][1], r[3][0], r[3][1]}; }
 };
-template <int ORDER>
-__device__ __forceinline__ void dq_chunk(const int c, const int t, const uint32_t w, const half2_t (&sc2)[2], const half2_t (&off2)[2], Dq &d) {
+// Q5_K (FMT 1): bit 4 of every quant comes from `hq`.  GGML order: hq is the qh dword of the same four bytes, shifted so
+// that bits 0 and 1 of each of its bytes belong to the low and the high nibble of the quant byte at the same place.  REF
+// order: hq is the one qh byte whose bits 0..7 belong to the eight consecutive elements of this k-step (even elements =
+// low nibbles): a multiplication spreads bits 0, 2, 4, 6 to bit 4 of bytes 0..3 (bit 2 i lands on 2 i + 4 + 6 i; the
+// other partial products meet at most in pairs on bits that the mask drops, and their carries stop there).  Values up to
+// 31 times scales up to 63 stay below 2048: exact in f16 like Q4_K's.
+template <int ORDER, int FMT = 0>
+__device__ __forceinline__ void dq_chunk(const int c, const int t, const uint32_t w, const half2_t (&sc2)[2], const half2_t (&off2)[2], Dq &d,
+                                         const uint32_t hq = 0) {
     const int lo_s = ORDER == 0 ? (t >> 2) : 0, hi_s = ORDER == 0 ? (t >> 2) : 1;
-    if (c == 0) {
+    if (FMT == 1 && c == 0) {
+        const uint32_t bit = ORDER == 0 ? ((hq & 0x55u) * 0x00410410u) & 0x10101010u : (hq & 0x01010101u) << 4;
+        d.lo = (w & 0x0F0F0F0Fu) | bit;
+        d.r[0] = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, d.lo, 0x04010400u)), sc2[lo_s], off2[lo_s]);
+    } else if (FMT == 1 && c == 1) {
+        d.r[1] = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, d.lo, 0x04030402u)), sc2[lo_s], off2[lo_s]);
+        const uint32_t bit = ORDER == 0 ? (((hq >> 1) & 0x55u) * 0x00410410u) & 0x10101010u : (hq & 0x02020202u) << 3;
+        d.hi = ((w >> 4) & 0x0F0F0F0Fu) | bit;
+    } else if (c == 0) {
         d.lo = w & 0x0F0F0F0Fu;
         d.r[0] = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, d.lo, 0x04010400u)), sc2[lo_s], off2[lo_s]);
     } else if (c == 1) {
@@ -319,13 +348,13 @@ __device__ __forceinline__ void neg_min_split(const float dmin, const uint32_t m
 // One half super-block H of one wave.  The restrict qualifiers say what the copies in flight cannot touch:
 // operand reads from a_cur / q_cur need not wait for the direct loads into a_nxt / q_nxt / hb.
 //   a_cur / a_nxt: activation stages (18 x BM items)      q_cur / q_nxt: this wave's quant pieces (NR x 128 items)
-//   hb: this wave's headers (NR x 64 items)
+//   hb: this wave's headers (NR x 64 items)       qhs: Q5_K, this wave's fifth bits (NR x 32 rows x 2 items)
 //   xs_nxt: item (group 0, row m0) of the next half super-block    wq_nxt / wh_nxt: first row of the workgroup at
 //   the next half's quant bytes / the next super-block's header
-template <int ORDER, int MB, int NR, int NW, int H>
+template <int ORDER, int MB, int NR, int NW, int H, int FMT>
 __device__ __forceinline__ void rw_half(const uint4 *__restrict__ a_cur, uint4 *__restrict__ a_nxt,
                                         const uint4 *__restrict__ q_cur, uint4 *__restrict__ q_nxt, uint4 *__restrict__ hb,
-                                        const uint4 *__restrict__ xs_nxt, const uint8_t *__restrict__ wq_nxt,
+                                        uint4 *__restrict__ qhs, const uint4 *__restrict__ xs_nxt, const uint8_t *__restrict__ wq_nxt,
                                         const uint8_t *__restrict__ wh_nxt, const Lane<MB, NR, NW> &L, Acc<MB, NR> &R) {
     constexpr int BM = 32 * MB, kThreads = 64 * NW;
     const int col = L.col, g = L.g;
@@ -334,10 +363,18 @@ __device__ __forceinline__ void rw_half(const uint4 *__restrict__ a_cur, uint4 *
         for (int rg = 0; rg < NR; rg++) {
             const uint4 hv = hb[rg * 64 + col];
             R.hdr[rg] = u32x4{hv.x, hv.y, hv.z, hv.w};
+            if (FMT == 1) {  // both halves of the super-block take their fifth bits from these registers
+                const uint4 ha = qhs[rg * 64 + 2 * col], hb2 = qhs[rg * 64 + 2 * col + 1];
+                R.qh[rg][0] = ha.x, R.qh[rg][1] = ha.y, R.qh[rg][2] = ha.z, R.qh[rg][3] = ha.w;
+                R.qh[rg][4] = hb2.x, R.qh[rg][5] = hb2.y, R.qh[rg][6] = hb2.z, R.qh[rg][7] = hb2.w;
+            }
         }
         __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the headers are in registers before their buffer is refilled
 #pragma unroll
-        for (int rg = 0; rg < NR; rg++) dma16(wh_nxt + L.h_off[rg], hb + rg * 64);
+        for (int rg = 0; rg < NR; rg++) {
+            dma16(wh_nxt + L.h_off[rg], hb + rg * 64);
+            if (FMT == 1) dma16(wh_nxt + L.qh_off[rg], qhs + rg * 64);
+        }
     }
     // copies for the next half super-block
 #pragma unroll
@@ -380,6 +417,15 @@ __device__ __forceinline__ void rw_half(const uint4 *__restrict__ a_cur, uint4 *
         off2[rg][0] = half2_t{o0, o0}, off2[rg][1] = half2_t{o1, o1};
     }
 
+    // Q5_K: where k-step t finds its fifth bits.  GGML order: qh dword t (the same four bytes as quant dword t), bits
+    // j0 = 4 H + 2 g (low nibbles) and j0 + 1 (high nibbles) of every byte.  REF order: byte 4 j0 + t of qh.
+    auto fifth = [&](int rg, int t) -> uint32_t {
+        if (FMT == 0) return 0u;
+        if (ORDER == 1) return R.qh[rg][t] >> (uint32_t)(4 * H + 2 * g);
+        const uint32_t dw = g ? R.qh[rg][4 * H + 2 + (t >> 2)] : R.qh[rg][4 * H + (t >> 2)];
+        return dw >> (8 * (t & 3));  // (the decoder masks the byte)
+    };
+
     // min term of sub-blocks j0, j0 + 1: (-h, -h, -l, -l) against the activations' (H, L, H, L): all four cross
     // products of the exact head + tail splits, straight into the accumulators (after the eight k-steps)
     half8_t br[NR];
@@ -403,7 +449,7 @@ __device__ __forceinline__ void rw_half(const uint4 *__restrict__ a_cur, uint4 *
 #pragma unroll
     for (int rg = 0; rg < NR; rg++)
 #pragma unroll
-        for (int c = 0; c < 4; c++) dq_chunk<ORDER>(c, 0, qd[rg][0], sc2[rg], off2[rg], dq[rg]);
+        for (int c = 0; c < 4; c++) dq_chunk<ORDER, FMT>(c, 0, qd[rg][0], sc2[rg], off2[rg], dq[rg], fifth(rg, 0));
 #pragma unroll
     for (int t = 0; t < 8; t++) {
         half8_t b[NR];
@@ -427,7 +473,7 @@ __device__ __forceinline__ void rw_half(const uint4 *__restrict__ a_cur, uint4 *
                     const int slot = i * NR + rg;
 #pragma unroll
                     for (int ch = slot * kChunks / kSlots; ch < (slot + 1) * kChunks / kSlots; ch++)
-                        dq_chunk<ORDER>(ch % 4, t + 1, qd[ch / 4][t + 1], sc2[ch / 4], off2[ch / 4], dq[ch / 4]);
+                        dq_chunk<ORDER, FMT>(ch % 4, t + 1, qd[ch / 4][t + 1], sc2[ch / 4], off2[ch / 4], dq[ch / 4], fifth(ch / 4, t + 1));
                 }
                 if (i == 0 && rg == 0) {
                     // the next step's fragments are requested behind the first product of this step: the wait in
@@ -463,13 +509,15 @@ __device__ __forceinline__ void rw_half(const uint4 *__restrict__ a_cur, uint4 *
 // the next two (they come from HBM): three quant stages per wave, rotated.  Within a half super-block the
 // activation copies are requested before the quant copies, so waiting until only the 2 NR newest requests are
 // outstanding leaves exactly the quant copies for the half after next in flight.
-template <int ORDER, int MB, int NR, int NW>
+template <int ORDER, int MB, int NR, int NW, int FMT = 0>
 __global__ __launch_bounds__(64 * NW, MB * NR <= 1 && NW <= 8 ? 2 : 1) void k_qgemm_rw(
     const uint8_t *__restrict__ W, const uint4 *__restrict__ xs, const float *__restrict__ rowscale, void *__restrict__ yg,
     float *__restrict__ partial, int M, int Mp, int N, int spr, int chunk, int mode) {
     constexpr int BM = 32 * MB, kThreads = 64 * NW, kRows = 32 * NR * NW;
+    constexpr int kBlockBytes = BlockFmt<FMT>::kBytes, kQs = BlockFmt<FMT>::kQs;
     extern __shared__ uint4 smem[];
     uint4 *a0 = smem, *a1 = a0 + kGroups * BM, *qbase = a1 + kGroups * BM, *hb = qbase + 3 * NW * NR * 128;
+    uint4 *qhb = hb + NW * NR * 64;  // Q5_K only
     const int tid = threadIdx.x;
     Lane<MB, NR, NW> L;
     L.wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -493,6 +541,7 @@ __global__ __launch_bounds__(64 * NW, MB * NR <= 1 && NW <= 8 ? 2 : 1) void k_qg
             L.q_off[rg][r] = row_off(32 * rg + row) + 16u * (uint32_t)((lane & 3) ^ ((row >> 2) & 3));
         }
         L.h_off[rg] = row_off(32 * rg + (lane & 31));
+        L.qh_off[rg] = row_off(32 * rg + (lane >> 1)) + 16u + 16u * (uint32_t)(lane & 1);
     }
 #pragma unroll
     for (int i = 0; i < Lane<MB, NR, NW>::kARounds; i++) {
@@ -501,7 +550,7 @@ __global__ __launch_bounds__(64 * NW, MB * NR <= 1 && NW <= 8 ? 2 : 1) void k_qg
     }
     // this wave's three quant stages (rotated: qa is read, qb is next, qc receives the copies) and its headers
     uint4 *qa = qbase + L.wave * (NR * 128), *qb = qa + NW * NR * 128, *qc = qb + NW * NR * 128;
-    uint4 *hw = hb + L.wave * (NR * 64);
+    uint4 *hw = hb + L.wave * (NR * 64), *qhw = qhb + L.wave * (NR * 64);
     const uint8_t *wblk = W + (size_t)n0 * row_bytes;
 
     Acc<MB, NR> R;
@@ -518,10 +567,11 @@ __global__ __launch_bounds__(64 * NW, MB * NR <= 1 && NW <= 8 ? 2 : 1) void k_qg
 #pragma unroll
         for (int rg = 0; rg < NR; rg++) {
             dma16(blk + L.h_off[rg], hw + rg * 64);
+            if (FMT == 1) dma16(blk + L.qh_off[rg], qhw + rg * 64);
 #pragma unroll
             for (int r = 0; r < 2; r++) {
-                dma16(blk + 16 + L.q_off[rg][r], qa + rg * 128 + r * 64);
-                dma16(blk + 16 + 64 + L.q_off[rg][r], qb + rg * 128 + r * 64);
+                dma16(blk + kQs + L.q_off[rg][r], qa + rg * 128 + r * 64);
+                dma16(blk + kQs + 64 + L.q_off[rg][r], qb + rg * 128 + r * 64);
             }
         }
         const uint4 *xa = xs + (size_t)(sb0 * 2 * kGroups) * Mp + m0;
@@ -536,9 +586,9 @@ __global__ __launch_bounds__(64 * NW, MB * NR <= 1 && NW <= 8 ? 2 : 1) void k_qg
         const int sb = sb0 + s;
         const int sbn = sb + 1 < spr ? sb + 1 : spr - 1;  // the copies for "the next super-block" stay inside the matrix
         const uint8_t *blkn = wblk + (size_t)sbn * kBlockBytes;
-        rw_half<ORDER, MB, NR, NW, 0>(a0, a1, qa, qc, hw, xs + (size_t)((sb * 2 + 1) * kGroups) * Mp + m0, blkn + 16, blkn, L, R);
+        rw_half<ORDER, MB, NR, NW, 0, FMT>(a0, a1, qa, qc, hw, qhw, xs + (size_t)((sb * 2 + 1) * kGroups) * Mp + m0, blkn + kQs, blkn, L, R);
         barrier_keep<2 * NR>();
-        rw_half<ORDER, MB, NR, NW, 1>(a1, a0, qb, qa, hw, xs + (size_t)(sbn * 2 * kGroups) * Mp + m0, blkn + 16 + 64, nullptr, L, R);
+        rw_half<ORDER, MB, NR, NW, 1, FMT>(a1, a0, qb, qa, hw, qhw, xs + (size_t)(sbn * 2 * kGroups) * Mp + m0, blkn + kQs + 64, nullptr, L, R);
         barrier_keep<2 * NR>();
         // two half super-blocks on: (qa, qb, qc) <- (qc, qa, qb)
         uint4 *t = qc;
@@ -1499,9 +1549,9 @@ __global__ __launch_bounds__(256) void k_rw_reduce8(const float *__restrict__ pa
     }
 }
 
-template <int MB, int NR, int NW>
+template <int MB, int NR, int NW, int FMT = 0>
 constexpr size_t rw_lds_bytes() {
-    const size_t stages = (size_t)(2 * kGroups * 32 * MB + NW * NR * (3 * 128 + 64)) * 16;
+    const size_t stages = (size_t)(2 * kGroups * 32 * MB + NW * NR * (3 * 128 + 64 + (FMT ? 64 : 0))) * 16;
     return stages > tile_lds_bytes<MB, NW>() ? stages : tile_lds_bytes<MB, NW>();
 }
 
@@ -1536,10 +1586,10 @@ static int compute_units_gemm() {
 
 bool qgemm_fits(uint32_t type, int64_t m, int64_t n, int64_t k) {
     // byte offsets inside a workgroup's rows and item offsets inside the activation copy are 32-bit
-    return (type == kTypeQ4K || type == kTypeQ6K || type == kTypeQ8_0) && m >= 1 && m <= (int64_t)1 << 22 && n >= 1 && k >= 256 && k % 256 == 0 && k <= (int64_t)1 << 22 && n <= 0x7FFFFF00;
+    return (type == kTypeQ4K || type == kTypeQ5K || type == kTypeQ6K || type == kTypeQ8_0) && m >= 1 && m <= (int64_t)1 << 22 && n >= 1 && k >= 256 && k % 256 == 0 && k <= (int64_t)1 << 22 && n <= 0x7FFFFF00;
 }
 
-GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k) {
+GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k, uint32_t type) {
     GemmPlan p;
     // 32, 64 or 128 activation rows per workgroup; up to 192 rows 64-row blocks beat 128-row blocks (fewer K splits
     // for the same number of workgroups: 36.9 against 38.3 us at M = 128, 51.7 against 53.8 at M = 192, 14336x4096;
@@ -1572,12 +1622,13 @@ GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k) {
     }
     // at most 16 activation rows against long rows: runs of 16 super-blocks (the fused kernels' K split; the large kernel
     // takes the same split when a shape falls back to it)
-    if (m <= kSmallMaxM && spr > kSmallMaxSpr) p.chunk = kSmallMaxSpr, p.splits = (int)((spr + kSmallMaxSpr - 1) / kSmallMaxSpr);
+    // (a type without such kernels keeps the split chosen above)
+    if (m <= kSmallMaxM && spr > kSmallMaxSpr && type != kTypeQ5K) p.chunk = kSmallMaxSpr, p.splits = (int)((spr + kSmallMaxSpr - 1) / kSmallMaxSpr);
     return p;
 }
 
 size_t qgemm_workspace_bytes(uint32_t type, int64_t m, int64_t n, int64_t k) {
-    const GemmPlan p = qgemm_plan(m, n, k);
+    const GemmPlan p = qgemm_plan(m, n, k, type);
     const size_t xs = align256((size_t)(k / 256) * 2 * kGroups * p.mp * 16);
     // the short-batch kernels take a row of up to kSmallMaxSpr super-blocks whole: the plan's K split is not used there
     const bool unsplit = qgemm_small_applies(type, m, n, k) && k / 256 <= kSmallMaxSpr;
@@ -1585,11 +1636,11 @@ size_t qgemm_workspace_bytes(uint32_t type, int64_t m, int64_t n, int64_t k) {
     return xs + align256((size_t)p.mp * 4) + part;
 }
 
-template <int ORDER, int MB, int NR, int NW>
+template <int ORDER, int MB, int NR, int NW, int FMT = 0>
 static hipError_t launch_rw(hipStream_t s, const uint8_t *w, const uint4 *xs, const float *rowscale, void *y, float *partial,
                             int64_t m, int64_t n, int spr, const GemmPlan &p, int mode) {
-    auto kern = k_qgemm_rw<ORDER, MB, NR, NW>;
-    constexpr size_t lds = rw_lds_bytes<MB, NR, NW>();
+    auto kern = k_qgemm_rw<ORDER, MB, NR, NW, FMT>;
+    constexpr size_t lds = rw_lds_bytes<MB, NR, NW, FMT>();
     constexpr int kRows = 32 * NR * NW;
     if (lds > 64 * 1024) {
         hipError_t a = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -1631,15 +1682,15 @@ static hipError_t launch_rw_q8(hipStream_t s, const uint8_t *w, const uint4 *xs,
 hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype,
                                 int64_t m, void *y, uint32_t y_dtype, uint32_t order, void *workspace, hipStream_t s, bool reuse_prepass) {
     if (!qgemm_fits(type, m, n, k)) return hipErrorInvalidValue;
-    const GemmPlan p = qgemm_plan(m, n, k);
+    const GemmPlan p = qgemm_plan(m, n, k, type);
     const int spr = (int)(k / 256);
     uint8_t *ws = reinterpret_cast<uint8_t *>(workspace);
     uint4 *xs = reinterpret_cast<uint4 *>(ws);
     const size_t xs_bytes = align256((size_t)spr * 2 * kGroups * p.mp * 16);
     float *rowscale = reinterpret_cast<float *>(ws + xs_bytes);
     float *partial = reinterpret_cast<float *>(ws + xs_bytes + align256((size_t)p.mp * 4));
-    const bool xf32 = x_dtype == kDtypeF32, q6 = type == kTypeQ6K, q8 = type == kTypeQ8_0, ref = order == kOrderRef;
-    const int xorder = q8 ? 3 : (q6 ? 2 : (ref ? 0 : 1));  // the element order the pre-pass lays the activations out for
+    const bool xf32 = x_dtype == kDtypeF32, q6 = type == kTypeQ6K, q8 = type == kTypeQ8_0, q5 = type == kTypeQ5K, ref = order == kOrderRef;
+    const int xorder = q8 ? 3 : (q6 ? 2 : (ref ? (q5 ? 4 : 0) : 1));  // the element order the pre-pass lays the activations out for
 #define PMH_PREP(F, O)                                                                                                       \
     do {                                                                                                                     \
         if (p.mp >= 1024)                                                                                                    \
@@ -1655,12 +1706,14 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
         if (xorder == 0) PMH_PREP(true, 0);
         else if (xorder == 1) PMH_PREP(true, 1);
         else if (xorder == 2) PMH_PREP(true, 2);
-        else PMH_PREP(true, 3);
+        else if (xorder == 3) PMH_PREP(true, 3);
+        else PMH_PREP(true, 4);
     } else {
         if (xorder == 0) PMH_PREP(false, 0);
         else if (xorder == 1) PMH_PREP(false, 1);
         else if (xorder == 2) PMH_PREP(false, 2);
-        else PMH_PREP(false, 3);
+        else if (xorder == 3) PMH_PREP(false, 3);
+        else PMH_PREP(false, 4);
     }
 #undef PMH_PREP
     hipError_t e = hipGetLastError();
@@ -1756,6 +1809,12 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
         e = p.mb == 1   ? launch_rw_q6<1>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
             : p.mb == 2 ? launch_rw_q6<2>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
                         : launch_rw_q6<4>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode);
+    } else if (q5) {
+#define PMH_RW5_CASE(O, B) launch_rw<O, B, 1, 8, 1>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
+        e = p.mb == 1   ? (ref ? PMH_RW5_CASE(0, 1) : PMH_RW5_CASE(1, 1))
+            : p.mb == 2 ? (ref ? PMH_RW5_CASE(0, 2) : PMH_RW5_CASE(1, 2))
+                        : (ref ? PMH_RW5_CASE(0, 4) : PMH_RW5_CASE(1, 4));
+#undef PMH_RW5_CASE
     } else if (p.mb == 1) {
         e = ref ? PMH_RW_CASE(0, 1, 1, 8) : PMH_RW_CASE(1, 1, 1, 8);
     } else if (p.mb == 2) {

@@ -69,7 +69,8 @@ struct GemmPlan {
     int chunk;   // super-blocks per split
 };
 bool qgemm_fits(uint32_t type, int64_t m, int64_t n, int64_t k);
-GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k);
+// (the padded row count mp does not depend on the type; the K split does)
+GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k, uint32_t type = kTypeQ4K);
 // Bytes of device workspace qgemm needs for a weight of `type` at (m, n, k); the caller provides it.
 size_t qgemm_workspace_bytes(uint32_t type, int64_t m, int64_t n, int64_t k);
 // reuse_prepass: the workspace still holds the converted activations of the previous launch_qgemm on this stream with the same

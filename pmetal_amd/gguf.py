@@ -273,8 +273,9 @@ class GgufLinear:
     Mirrors ``LayerWeight::matmul_from`` (crates/pmetal-bridge/src/qwen3_native/weights.rs:66-84): one token goes through
     the fused GEMV, several through the fused GEMM.  ``w`` are the packed block bytes (host array or device buffer).
     As the reference brings a weight into its matmul's layout when the model is loaded (weights.rs:29-45),
-    ``prepare_gemm=True`` re-blocks a Q5_K / Q3_K / Q2_K weight once into the Q6_K form their GEMM multiplies with
-    (the original blocks stay for the GEMV); without it the GEMM of those types re-blocks on every call."""
+    ``prepare_gemm=True`` re-blocks a Q3_K / Q2_K weight once into the Q6_K form their GEMM multiplies with
+    (the original blocks stay for the GEMV); without it the GEMM of those types re-blocks on every call.  Q5_K has a
+    matrix kernel that reads its blocks as they are, so nothing is prepared for it."""
 
     ROW_LOOP_MAX = 8  # up to this many activation rows Q5_K / Q3_K / Q2_K run one fused GEMV per row
 
@@ -287,7 +288,7 @@ class GgufLinear:
             w = DeviceBuffer.from_host(np.ascontiguousarray(w, dtype=np.uint8))
         self.w = w
         self.reblocked, self.reblocked_len = None, 0
-        if prepare_gemm:
+        if prepare_gemm and int(self.dtype) != 13:
             lib = _lib.load()
             self.reblocked_len = lib.pmetal_hip_reblock_size(int(self.dtype), self.n, self.k)
             if self.reblocked_len:

@@ -343,6 +343,39 @@ def test_qgemm_q5k_q3k_q2k_matches_dequantize_then_matmul(oracle, t, m, n, k):
         assert norm <= 2 * TOL and elem_r <= TOL and norm_r <= TOL, (row, norm, elem_r, norm_r)
 
 
+@pytest.mark.parametrize("order", [0, 1])
+@pytest.mark.parametrize("m,n,k", [(7, 96, 512), (40, 300, 1024), (130, 257, 768), (300, 64, 2048)])
+def test_qgemm_q5k_unit_activations_pick_single_weights(oracle, order, m, n, k):
+    """The Q5_K matrix kernel (the Q4_K kernel with the fifth bits from qh): with unit activations row r of the result is
+    column c_r of the dequantized weight, bit for bit -- every quant value, both element orders, every k-step and lane
+    position over the rows -- and the re-blocked form of the same weight gives the same numbers to the f32 summation order."""
+    lib = _lib.load()
+    rng = np.random.default_rng(77 * m + n + k + order)
+    raw = rng.integers(0, 256, size=(n * (k // 256), 176), dtype=np.uint8)
+    raw[:, 0:4] = np.frombuffer(np.array([0.01, 0.02], np.float16).tobytes(), np.uint8)
+    raw = raw.reshape(-1)
+    w = oracle.dequantize(13, raw, [n, k], order=order).reshape(n, k)
+    for rep in range(3):
+        cols = (np.arange(m) * (29 + 2 * rep) + 31 * rep + 3) % k
+        xu = np.zeros((m, k), np.float32)
+        xu[np.arange(m), cols] = 1.0
+        got = gpu_qgemm(13, raw, n, k, oracle.f32_to_bf16_bits(xu.reshape(-1)).reshape(m, k), m, order=order)
+        for r, c in enumerate(cols):
+            assert np.array_equal(got[r], w[:, c]), (rep, r, c)
+    # against the re-blocked form (two Q6_K tensors) on random activations
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    bits = oracle.f32_to_bf16_bits(x.reshape(-1)).reshape(m, k)
+    got = gpu_qgemm(13, raw, n, k, bits, m, order=order)
+    dw = pm.DeviceBuffer.from_host(raw)
+    size = lib.pmetal_hip_reblock_size(13, n, k)
+    dr, dx, dy = pm.DeviceBuffer(size), pm.DeviceBuffer.from_host(bits), pm.DeviceBuffer(4 * m * n)
+    pm.check(lib.pmetal_hip_reblock_dev(13, dw.ptr, n, k, order, dr.ptr, size, None))
+    pm.check(lib.pmetal_hip_qgemm_reblocked(13, dr.ptr, size, n, k, dx.ptr, pm.DTYPE_BF16, m, dy.ptr, pm.DTYPE_F32, None))
+    pm.check(lib.pmetal_hip_sync(None))
+    other = dy.to_host(np.float32).reshape(m, n)
+    assert np.max(np.abs(got - other)) <= 1e-5 * np.max(np.abs(other))
+
+
 @pytest.mark.parametrize("t", sorted(REBLOCKED))
 def test_qlinear_q5k_q3k_q2k_dispatch(oracle, t):
     """qlinear: up to eight activation rows one fused GEMV each, above that the re-blocked GEMM; both agree with the
@@ -351,7 +384,7 @@ def test_qlinear_q5k_q3k_q2k_dispatch(oracle, t):
     n, k = 320, 1024
     wq = oracle.quantize(t, weights(t, n * k, outliers=1e-3))
     dw = pm.DeviceBuffer.from_host(wq)
-    for m in (8, 9, 64, 3):
+    for m in (8, 9, 64, 3, 2):
         x = np.random.default_rng(m).standard_normal((m, k)).astype(np.float32)
         x = oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(x.reshape(-1))).reshape(m, k)  # survives the GEMM's f16 rounding
         dx, dy = pm.DeviceBuffer.from_host(x), pm.DeviceBuffer(4 * m * n)
@@ -368,7 +401,7 @@ def test_qlinear_q5k_q3k_q2k_dispatch(oracle, t):
 
 
 def test_qlinear_falls_back_to_the_gemm_when_the_gemv_refuses_the_row_length(oracle):
-    """Q5_K rows longer than the GEMV's activation staging (k > 32768): one activation row still has the re-blocked GEMM.
+    """Q5_K rows longer than the GEMV's activation staging (k > 32768): one activation row still has the GEMM.
     A Q8_0 row that is not a multiple of 256 with a bf16 output has no kernel and says so."""
     lib = _lib.load()
     n, k = 64, 33024
@@ -400,8 +433,10 @@ def test_qgemm_batch_equals_separate_calls(oracle):
     lib = _lib.load()
     k = 2048
     rng = np.random.default_rng(5150)
-    specs = [(Q4K, 768, 0, pm.DTYPE_F32), (Q4K, 512, 0, pm.DTYPE_BF16), (Q4K, 256, 1, pm.DTYPE_F32), (Q6K, 640, 0, pm.DTYPE_F32),
-             (Q6K, 320, 0, pm.DTYPE_BF16), (Q8_0, 384, 0, pm.DTYPE_F32), (Q4K, 1024, 0, pm.DTYPE_F32)]
+    # (Q5_K behind Q4_K in the GGML order shares its converted activations; in the REF order it has a layout of its own)
+    specs = [(Q4K, 768, 0, pm.DTYPE_F32), (Q4K, 512, 0, pm.DTYPE_BF16), (Q4K, 256, 1, pm.DTYPE_F32), (13, 512, 1, pm.DTYPE_F32),
+             (13, 384, 0, pm.DTYPE_BF16), (Q6K, 640, 0, pm.DTYPE_F32),
+             (Q6K, 320, 0, pm.DTYPE_BF16), (Q8_0, 384, 0, pm.DTYPE_F32), (Q4K, 1024, 0, pm.DTYPE_F32), (13, 256, 0, pm.DTYPE_F32)]
     ws = [pm.DeviceBuffer.from_host(oracle.quantize(t, weights(800 + i, n * k))) for i, (t, n, _, _) in enumerate(specs)]
     for m in (3, 48, 300):
         xb = oracle.f32_to_bf16_bits(rng.standard_normal(m * k).astype(np.float32))
@@ -418,7 +453,7 @@ def test_qgemm_batch_equals_separate_calls(oracle):
         pm.check(lib.pmetal_hip_sync(None))
         for i in range(len(specs)):
             assert np.array_equal(y_one[i].to_host(np.uint8), y_bat[i].to_host(np.uint8)), (m, specs[i])
-    bad = (_lib.GemmDesc * 1)(_lib.GemmDesc(13, 0, 0, 0, 256, ws[0].ptr, y_bat[0].ptr))
+    bad = (_lib.GemmDesc * 1)(_lib.GemmDesc(11, 0, 0, 0, 256, ws[0].ptr, y_bat[0].ptr))  # Q3_K: only through re-blocking
     assert lib.pmetal_hip_qgemm_batch(bad, 1, k, dx.ptr, pm.DTYPE_BF16, 3, None) == 2
     lib.pmetal_hip_clear_error()
 
