@@ -716,74 +716,13 @@ constexpr int kQ4kLdsStride = 33;  // 32 floats + 1 pad: lanes read column-wise 
 // NMAX = 15: Q4_K (k_quants.rs:876-955).  NMAX = 31: Q5_K (k_quants.rs:960-1051), the same search and scale packing with
 // 5-bit quants: 176-byte blocks, the low four bits packed like Q4_K behind 32 bytes qh, where bit j of qh[l] is the
 // fifth bit of element l of sub-block j.
+// The super-block part of quantize_q4k / quantize_q5k for the 8 super-blocks from sb0 on: lane L holds the 32 elements of
+// sub-block L and make_qkx1_quants' (scale, -min) for it.
 template <int NMAX>
-__global__ __launch_bounds__(64) void k_quantize_q4k(const float *__restrict__ x, size_t n_sb,
-                                                      uint8_t *__restrict__ dst) {
+__device__ __forceinline__ void q4k_finish(const float (&xv)[32], const float scale, const float neg_min, const int lane, const size_t sb0,
+                                           const size_t n_sb, uint8_t *__restrict__ dst) {
     constexpr bool Q5 = NMAX == 31;
     constexpr int kBytes = Q5 ? 176 : 144, kQsOff = Q5 ? 48 : 16;
-    __shared__ float xs[64 * kQ4kLdsStride];
-    const int lane = threadIdx.x;
-    const size_t sb0 = (size_t)blockIdx.x * 8;
-    const size_t n_valid = (n_sb - sb0 < 8 ? n_sb - sb0 : 8) * 256;  // floats this wave may read
-    const float *src = x + sb0 * 256;
-#pragma unroll
-    for (int it = 0; it < 8; it++) {
-        const int idx = it * 64 + lane;  // float4 index inside the 2048-float tile
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if ((size_t)idx * 4 < n_valid) v = *reinterpret_cast<const float4 *>(src + idx * 4);
-        float *p = xs + (idx >> 3) * kQ4kLdsStride + (idx & 7) * 4;
-        p[0] = v.x, p[1] = v.y, p[2] = v.z, p[3] = v.w;
-    }
-    __syncthreads();
-    float xv[32];
-#pragma unroll
-    for (int i = 0; i < 32; i++) xv[i] = xs[lane * kQ4kLdsStride + i];
-
-    // ---- make_qkx1_quants(NMAX, 5, xv) ----
-    // min_by / max_by with total_cmp: equal keys are identical floats, so integer min / max of the keys will do
-    int kmn = total_key(xv[0]), kmx = kmn;
-#pragma unroll
-    for (int i = 1; i < 32; i++) {
-        const int key = total_key(xv[i]);
-        kmn = key < kmn ? key : kmn;
-        kmx = key > kmx ? key : kmx;
-    }
-    const float mn = __builtin_bit_cast(float, kmn ^ (int)(((unsigned)(kmn >> 31)) >> 1));
-    const float mx = __builtin_bit_cast(float, kmx ^ (int)(((unsigned)(kmx >> 31)) >> 1));
-    float scale = 0.0f, neg_min = 0.0f;  // returned (scale, -min)
-    if (!(mx == mn)) {
-        float minv = __builtin_fminf(mn, 0.0f);
-        float iscale = (float)NMAX / (mx - minv);
-        scale = 1.0f / iscale;
-        float lf[32];  // the quants of the previous try, as floats
-#pragma unroll
-        for (int i = 0; i < 32; i++) lf[i] = 0.0f;
-#pragma unroll  // unrolled so that the quants of try t and t - 1 live in different registers without copies
-        for (int t = 0; t < 5; t++) {
-            float sumlx = 0.0f, suml2 = 0.0f;  // suml2 is an integer <= 32 NMAX^2 < 2^24: exact in f32, with or without fusing
-            bool changed = false;
-#pragma unroll
-            for (int i = 0; i < 32; i++) {
-                const float xm = xv[i] - minv;
-                const float r = clamp_round_0_15<NMAX>(iscale * xm);
-                changed |= (r != lf[i]);
-                lf[i] = r;
-                sumlx += xm * r;
-                suml2 = __builtin_fmaf(r, r, suml2);
-            }
-            if (suml2 == 0.0f) break;
-            scale = sumlx / suml2;
-            float sum = -0.0f;  // Iterator::sum::<f32> folds from -0.0
-#pragma unroll
-            for (int i = 0; i < 32; i++) sum += xv[i] - scale * lf[i];
-            minv = sum / 32.0f;
-            if (minv > 0.0f) minv = 0.0f;
-            iscale = 1.0f / scale;
-            if (!changed) break;
-        }
-        neg_min = -minv;
-    }
-
     // ---- super-block level (k_quants.rs:904-929): the 8 lanes of a super-block cooperate ----
     float max_scale = scale, max_min = neg_min;
 #pragma unroll
@@ -894,6 +833,82 @@ __global__ __launch_bounds__(64) void k_quantize_q4k(const float *__restrict__ x
         }
         if (j == 0) *reinterpret_cast<uint32_t *>(blk) = d16 | (dmin16 << 16);
     }
+}
+
+template <int NMAX>
+__global__ __launch_bounds__(64) void k_quantize_q4k(const float *__restrict__ x, size_t n_sb,
+                                                      uint8_t *__restrict__ dst) {
+    __shared__ float xs[64 * kQ4kLdsStride];
+    const int lane = threadIdx.x;
+    const size_t sb0 = (size_t)blockIdx.x * 8;
+    const size_t n_valid = (n_sb - sb0 < 8 ? n_sb - sb0 : 8) * 256;  // floats this wave may read
+    const float *src = x + sb0 * 256;
+#pragma unroll
+    for (int it = 0; it < 8; it++) {
+        const int idx = it * 64 + lane;  // float4 index inside the 2048-float tile
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if ((size_t)idx * 4 < n_valid) v = *reinterpret_cast<const float4 *>(src + idx * 4);
+        float *p = xs + (idx >> 3) * kQ4kLdsStride + (idx & 7) * 4;
+        p[0] = v.x, p[1] = v.y, p[2] = v.z, p[3] = v.w;
+    }
+    __syncthreads();
+    float xv[32];
+#pragma unroll
+    for (int i = 0; i < 32; i++) xv[i] = xs[lane * kQ4kLdsStride + i];
+
+    // ---- make_qkx1_quants(NMAX, 5, xv) ----
+    // min_by / max_by with total_cmp: equal keys are identical floats, so integer min / max of the keys will do
+    int kmn = total_key(xv[0]), kmx = kmn;
+#pragma unroll
+    for (int i = 1; i < 32; i++) {
+        const int key = total_key(xv[i]);
+        kmn = key < kmn ? key : kmn;
+        kmx = key > kmx ? key : kmx;
+    }
+    const float mn = __builtin_bit_cast(float, kmn ^ (int)(((unsigned)(kmn >> 31)) >> 1));
+    const float mx = __builtin_bit_cast(float, kmx ^ (int)(((unsigned)(kmx >> 31)) >> 1));
+    float scale = 0.0f, neg_min = 0.0f;  // returned (scale, -min)
+    if (!(mx == mn)) {
+        float minv = __builtin_fminf(mn, 0.0f);
+        float iscale = (float)NMAX / (mx - minv);
+        scale = 1.0f / iscale;
+        // Of the previous try's quants only whether any of them changes is asked: they are kept one per byte and compared
+        // four at a time (a conversion that packs in place of a move, 8 comparisons per try instead of 32).
+        float lf[32];
+        uint32_t lp[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int t = 0; t < 5; t++) {
+            float sumlx = 0.0f, suml2 = 0.0f;  // suml2 is an integer <= 32 NMAX^2 < 2^24: exact in f32, with or without fusing
+            bool changed = false;
+            uint32_t np[8];
+#pragma unroll
+            for (int i = 0; i < 32; i++) {
+                const float xm = xv[i] - minv;
+                const float r = clamp_round_0_15<NMAX>(iscale * xm);
+                np[i >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(r, i & 3, (i & 3) ? np[i >> 2] : 0u);
+                lf[i] = r;
+                sumlx += xm * r;
+                suml2 = __builtin_fmaf(r, r, suml2);
+            }
+#pragma unroll
+            for (int w = 0; w < 8; w++) {
+                changed |= np[w] != lp[w];
+                lp[w] = np[w];
+            }
+            if (suml2 == 0.0f) break;
+            scale = sumlx / suml2;
+            float sum = -0.0f;  // Iterator::sum::<f32> folds from -0.0
+#pragma unroll
+            for (int i = 0; i < 32; i++) sum += xv[i] - scale * lf[i];
+            minv = sum / 32.0f;
+            if (minv > 0.0f) minv = 0.0f;
+            iscale = 1.0f / scale;
+            if (!changed) break;
+        }
+        neg_min = -minv;
+    }
+
+    q4k_finish<NMAX>(xv, scale, neg_min, lane, sb0, n_sb, dst);
 }
 
 // -------------------------------------------------------------------------------------------
@@ -1177,20 +1192,25 @@ __global__ __launch_bounds__(64) void k_quantize_q2k(const float *__restrict__ x
         float iscale = 3.0f / (mx - minv);
         scale = 1.0f / iscale;
         float lf[16];
-#pragma unroll
-        for (int i = 0; i < 16; i++) lf[i] = 0.0f;
+        uint32_t lp[4] = {0, 0, 0, 0};  // the previous try's quants, one per byte (as in the Q4_K kernel)
 #pragma unroll
         for (int t = 0; t < 5; t++) {
             float sumlx = 0.0f, suml2 = 0.0f;  // suml2 <= 16 * 9: exact in f32
             bool changed = false;
+            uint32_t np[4];
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 const float xm = xv[i] - minv;
                 const float r = clamp_round_0_15<3>(iscale * xm);
-                changed |= (r != lf[i]);
+                np[i >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(r, i & 3, (i & 3) ? np[i >> 2] : 0u);
                 lf[i] = r;
                 sumlx += xm * r;
                 suml2 = __builtin_fmaf(r, r, suml2);
+            }
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                changed |= np[w] != lp[w];
+                lp[w] = np[w];
             }
             if (suml2 == 0.0f) break;
             scale = sumlx / suml2;
