@@ -783,7 +783,7 @@ __device__ __forceinline__ void q4k_finish(const float (&xv)[32], const float sc
                 const float q = __builtin_fminf(__builtin_fmaxf((xv[4 * w + c] + dm) * rinv, 0.0f), (float)NMAX);
                 const float r = __builtin_truncf(q + 0.49999997f);
                 exact_needed |= !(__builtin_fabsf(__builtin_fabsf(q - r) - 0.5f) >= 8e-6f);
-                lb[w] |= (uint32_t)r << (8 * c);
+                lb[w] = __builtin_amdgcn_cvt_pk_u8_f32(r, c, lb[w]);  // r is an integer in [0, NMAX]
             }
         }
         if (exact_needed) {
@@ -1008,21 +1008,30 @@ __global__ __launch_bounds__(64) void k_quantize_q6k(const float *__restrict__ x
                 const float sl2 = suml2 - w[i] * (li * li);
                 const float p = xv[i] * sl2;
                 const bool pos = slx > 0.0f;
-                const float qf = p * __builtin_amdgcn_rcpf(slx);
-                float nl = (float)clamp_i(nearest_int_sat(qf), -32, 31);
-                const bool sure = slx > 1e-30f && slx < 1e30f && __builtin_fabsf(__builtin_fabsf(qf - nl) - 0.5f) >= 2e-5f;
-                if (pos && !sure) nl = (float)clamp_i(nearest_int_sat(p / slx), -32, 31);
-                const bool differs = pos & (nl != li);
-                // from the second sweep on few lanes are still active and a new candidate is rare: skip the test
-                // when no lane has one
-                if (t == 0 || __builtin_amdgcn_ballot_w64(differs) != 0) {
-                    const float slx2 = slx + wx[i] * nl;
-                    const float sl22 = sl2 + w[i] * (nl * nl);
-                    const bool take = differs & (sl22 > 0.0f) & (slx2 * slx2 * suml2 > sumlx * sumlx * sl22);
-                    l[i] = take ? nl : li;
-                    sumlx = take ? slx2 : sumlx;
-                    suml2 = take ? sl22 : suml2;
-                    changed |= take;
+                // The candidate is the current quant whenever the quotient lies within 0.5 of it, i.e. |x sl2 - l slx| < slx / 2:
+                // two products and a difference, each correctly rounded, put that difference within 6e-6 slx of its exact
+                // value for |quotient| < 33, and the reference's rounded quotient lies within 4e-6 of the exact one, so a
+                // difference below 0.49998 slx settles it.  98 % of the elements that reach this point are settled this
+                // way; the others (and every slx outside the range where the products are normal numbers) take the
+                // quotient -- a whole wave, when one of its lanes has such an element.
+                const float dd = p - li * slx;
+                const bool same = slx > 1e-30f && slx < 1e30f && __builtin_fabsf(dd) < 0.49998f * slx;
+                if (__builtin_amdgcn_ballot_w64(pos && !same) != 0) {
+                    const float qf = p * __builtin_amdgcn_rcpf(slx);
+                    float nl = (float)clamp_i(nearest_int_sat(qf), -32, 31);
+                    const bool sure = slx > 1e-30f && slx < 1e30f && __builtin_fabsf(__builtin_fabsf(qf - nl) - 0.5f) >= 2e-5f;
+                    if (pos && !sure) nl = (float)clamp_i(nearest_int_sat(p / slx), -32, 31);
+                    const bool differs = pos & (nl != li);
+                    // a new candidate is rare: skip the test when no lane has one
+                    if (__builtin_amdgcn_ballot_w64(differs) != 0) {
+                        const float slx2 = slx + wx[i] * nl;
+                        const float sl22 = sl2 + w[i] * (nl * nl);
+                        const bool take = differs & (sl22 > 0.0f) & (slx2 * slx2 * suml2 > sumlx * sumlx * sl22);
+                        l[i] = take ? nl : li;
+                        sumlx = take ? slx2 : sumlx;
+                        suml2 = take ? sl22 : suml2;
+                        changed |= take;
+                    }
                 }
             }
             if (!changed) break;
