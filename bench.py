@@ -753,6 +753,15 @@ def other_parts(args):
         out[f"gemm_q4k_m{m}"] = {"metric": wl["metric"], "value": round(res["value"], 1), "unit": wl["unit"], "dtype": wl["dtype"],
                                  "steps": a.steps, "us_per_call": res["roofline"]["us_per_launch"], "roofline": res["roofline"],
                                  **({"roofline_hbm": hbm} if hbm else {}), "weights": res["extra"]["weights"]}
+    # the other block types of the recipe's files at the prefill shape (Q6_K: attn_v / ffn_down of half the layers and the
+    # output matrix; Q5_K: a fused attn_qkv)
+    for name, t in (("gemm_q6k_m512", Q6K), ("gemm_q5k_m512", 13)):
+        a.steps, a.warmup = 30, 5
+        res, _ = bench_gemm(a, 512, 14336, 4096, t)
+        wl = WORKLOADS[name]
+        out[name] = {"metric": wl["metric"], "value": round(res["value"], 1), "unit": wl["unit"], "dtype": wl["dtype"],
+                     "steps": a.steps, "us_per_call": res["roofline"]["us_per_launch"], "roofline": res["roofline"],
+                     "two_weights_sharing_x_us_per_weight": res["extra"]["two_weights_sharing_x_us_per_weight"]}
     # the second shape of the decode configuration (the down projection)
     a = copy.copy(args)
     a.steps, a.warmup = max(args.steps // 4, 10), max(args.warmup // 4, 2)
