@@ -435,27 +435,18 @@ def bench_gemm(args, m, n, k, t=Q4K):
         for wi in wl:
             pm.check(lib.pmetal_hip_qgemm(t, wi.ptr, n, k, x.ptr, pm.DTYPE_BF16, m, y.ptr, pm.DTYPE_BF16, 0, None))
 
-    step, per_call_us, reblocked_us = per_call, None, None
+    step, reblocked_us = per_call, None
     rb_bytes = lib.pmetal_hip_reblock_size(t, n, k)
-    if rb_bytes and t == 13:  # Q5_K has a matrix kernel of its own; its re-blocked form (two Q6_K tensors) is timed beside it
+    if rb_bytes:  # Q5_K / Q3_K / Q2_K have matrix kernels of their own; the re-blocked form (one or two Q6_K tensors) is timed beside them
         rb = pm.DeviceBuffer(rb_bytes)
         pm.check(lib.pmetal_hip_reblock_dev(t, w.ptr, n, k, 0, rb.ptr, rb_bytes, None), "reblock")
         rb_ms, _ = timer.run(lambda: pm.check(lib.pmetal_hip_qgemm_reblocked(t, rb.ptr, rb_bytes, n, k, x.ptr, pm.DTYPE_BF16, m, y.ptr, pm.DTYPE_BF16, None)),
                              args.steps, args.warmup)
         reblocked_us = rb_ms * 1e3 / args.steps
         rb.free()
-    elif rb_bytes:  # Q3_K / Q2_K: re-blocked once, as a loader does; the per-call form is timed beside it
-        rb = pm.DeviceBuffer(rb_bytes)
-        pm.check(lib.pmetal_hip_reblock_dev(t, w.ptr, n, k, 0, rb.ptr, rb_bytes, None), "reblock")
-
-        def step():
-            pm.check(lib.pmetal_hip_qgemm_reblocked(t, rb.ptr, rb_bytes, n, k, x.ptr, pm.DTYPE_BF16, m, y.ptr, pm.DTYPE_BF16, None))
-
-        pc_ms, _ = timer.run(per_call, args.steps, args.warmup)
-        per_call_us = pc_ms * 1e3 / args.steps
     ev_ms, wall_ms = timer.run(step, args.steps, args.warmup)
     eager_us = ev_ms * 1e3 / (args.steps * copies)
-    submission = "one call after the other (eager launches)"
+    submission, replay_us = "one call after the other (eager launches)", None
     if step is per_call:
         # the same calls recorded once (a HIP graph of eight passes) and replayed with one submission per step, as a prefill
         # that runs its projections from a recording submits them; the eager figure stays in `extra`
@@ -477,8 +468,10 @@ def bench_gemm(args, m, n, k, t=Q4K):
         timer.stream = None
         pm.check(lib.pmetal_hip_recording_destroy(rec))
         pm.check(lib.pmetal_hip_stream_destroy(stream))
-        ev_ms, wall_ms = r_ev * args.steps / (r_steps * reps), r_wall * args.steps / (r_steps * reps)
-        submission = f"{reps} passes over the weights recorded once and replayed (one submission per {reps * copies} calls)"
+        replay_us = r_ev * 1e3 / (r_steps * reps * copies)
+        if replay_us < eager_us:  # (`value` is the faster of the two ways to submit the same calls; both figures are in `extra`)
+            ev_ms, wall_ms = r_ev * args.steps / (r_steps * reps), r_wall * args.steps / (r_steps * reps)
+            submission = f"{reps} passes over the weights recorded once and replayed (one submission per {reps * copies} calls)"
     # what the matrix cores of this machine sustain in a register-only MFMA loop (no memory, no LDS) of about the
     # same length, with operands that vary: the ceiling any kernel here works under (the published peak assumes
     # the top clock, which a matrix loop does not hold)
@@ -491,7 +484,7 @@ def bench_gemm(args, m, n, k, t=Q4K):
     tflops = flops / (us * 1e-6) / 1e12
     dense = dense_library_tflops(m, n, k) if args.dense_library else None
     pair_us = None
-    if t in (Q4K, Q6K, Q8_0, 13):  # two weights against the same activations (gate / up): one pre-pass for both
+    if t in (Q4K, Q6K, Q8_0, 13, 11, 10):  # two weights against the same activations (gate / up): one pre-pass for both
         if copies == 1:
             wl.append(device_weights(pm, lib, t, n * k, 2001))
         y2 = pm.DeviceBuffer(2 * m * n)
@@ -508,17 +501,15 @@ def bench_gemm(args, m, n, k, t=Q4K):
         "value": tflops, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / BF16_PEAK_TFLOPS, 4), "traffic": None,
-                     "kernel": {Q4K: "k_qgemm_rw", 13: "k_qgemm_rw<FMT = 1>", Q6K: "k_qgemm_rw_q6", Q8_0: "k_qgemm_rw_q8"}.get(t, "k_qgemm_rw_q6 per Q6_K part of the re-blocked weight") + " (+ k_prep_rw, k_rw_reduce when K is split)",
+                     "kernel": {Q4K: "k_qgemm_rw", 13: "k_qgemm_rw<FMT = 1>", Q6K: "k_qgemm_rw_q6", Q8_0: "k_qgemm_rw_q8", 11: "k_qgemm_rw16<Q3_K>", 10: "k_qgemm_rw16<Q2_K>"}[t] + " (+ k_prep_rw, k_rw_reduce when K is split)",
                      "flops_per_launch": flops, "us_per_launch": round(us, 3)},
-        "extra": {"calls_per_step": copies, "submission": submission, "eager_us_per_call": round(eager_us, 3), "weights": f"{copies} tensor(s) in turn" + (" (from HBM)" if copies > 1 else " (33 MB: stays in the last-level cache)"),
+        "extra": {"calls_per_step": copies, "submission": submission, "eager_us_per_call": round(eager_us, 3),
+                  "replayed_us_per_call": None if replay_us is None else round(replay_us, 3), "weights": f"{copies} tensor(s) in turn" + (" (from HBM)" if copies > 1 else " (33 MB: stays in the last-level cache)"),
                   "mfma_loop_sustained_TFLOPs": round(sustained, 1), "frac_of_sustained": round(tflops / sustained, 4),
                   "dense_library_TFLOPs": dense,
                   "two_weights_sharing_x_us_per_weight": None if pair_us is None else round(pair_us, 3),
                   "two_weights_sharing_x_TFLOPs": None if pair_us is None else round(flops / (pair_us * 1e-6) / 1e12, 1),
-                  **({} if reblocked_us is None else {"reblocked_form_us": round(reblocked_us, 3), "reblocked_bytes": rb_bytes}),
-                  **({} if per_call_us is None else {"weight": "re-blocked to Q6_K once (pmetal_hip_reblock_dev), then pmetal_hip_qgemm_reblocked per call",
-                                                    "reblocked_bytes": rb_bytes,
-                                                    "reblocking_on_every_call_us": round(per_call_us, 3)})},
+                  **({} if reblocked_us is None else {"reblocked_form_us": round(reblocked_us, 3), "reblocked_bytes": rb_bytes})},
     }, (t, n, k)
 
 
@@ -737,7 +728,7 @@ WORKLOADS["gemm_q8_0_m16"] = dict(kind="gemm", m=16, n=14336, k=4096, metric="Q8
                                   unit="TFLOP/s", dtype="f16", type=Q8_0)
 WORKLOADS["gemm_q6k_m16"] = dict(kind="gemm", m=16, n=14336, k=4096, metric="Q6_K GEMM TFLOPS @M=16,K=4096,N=14336",
                                  unit="TFLOP/s", dtype="f16", type=Q6K)
-for _name, _t in (("q5k", 13), ("q3k", 11), ("q2k", 10)):  # Q5_K: its own kernel; Q3_K / Q2_K: re-blocked into Q6_K (one tensor, two)
+for _name, _t in (("q5k", 13), ("q3k", 11), ("q2k", 10)):  # (their own kernels; the form re-blocked into Q6_K is timed beside them)
     WORKLOADS[f"gemm_{_name}_m512"] = dict(kind="gemm", m=512, n=14336, k=4096, unit="TFLOP/s", dtype="f16", type=_t,
                                            metric=f"{_name.upper().replace('K', '_K')} GEMM TFLOPS (nominal flops) @M=512,K=4096,N=14336")
 

@@ -129,21 +129,12 @@ class DeviceBuffer {
 // A GGUF-quantized weight [n, k] resident on the device; the counterpart of LayerWeight for GGUF types.
 class GgufLinear {
    public:
-    // prepare_gemm: re-block a Q3_K / Q2_K weight once into the Q6_K form its GEMM multiplies with, as the reference
-    // brings a weight into its matmul's layout when the model is loaded (weights.rs:29-45); the original blocks stay for the
-    // GEMV.  (Q5_K has a matrix kernel that reads its blocks as they are: nothing is prepared for it.)
+    // prepare_gemm: accepted and ignored.  Every type has matrix kernels that read its blocks as they are, so nothing is
+    // laid out again at load time (the reference does that for its matmul, weights.rs:29-45).
     GgufLinear(GgmlType dtype, int64_t n, int64_t k, const std::vector<uint8_t> &packed,
                uint32_t order = PMETAL_HIP_ORDER_REF, bool prepare_gemm = false)
         : dtype_(dtype), n_(n), k_(k), order_(order), w_(check_size(dtype, n, k, packed), packed.size()) {
-        if (prepare_gemm && dtype_ != GgmlType::Q5K) {
-            const size_t len = pmetal_hip_reblock_size((uint32_t)dtype_, n_, k_);
-            if (len) {
-                reblocked_.reset(new DeviceBuffer(len));
-                detail::check(pmetal_hip_reblock_dev((uint32_t)dtype_, (const uint8_t *)w_.ptr(), n_, k_, order_,
-                                                     (uint8_t *)reblocked_->ptr(), len, nullptr));
-                detail::check(pmetal_hip_sync(nullptr));
-            }
-        }
+        (void)prepare_gemm;
     }
 
     // x: [m, k] activations on the device (bf16 unless x_dtype says f32); returns [m, n] f32 on the device.
@@ -151,11 +142,7 @@ class GgufLinear {
     DeviceBuffer matmul_from(const DeviceBuffer &x, int64_t m = 1, uint32_t x_dtype = PMETAL_HIP_DTYPE_BF16,
                              void *stream = nullptr) const {
         DeviceBuffer y((size_t)m * (size_t)n_ * sizeof(float));
-        if (reblocked_ && m > 8)  // up to eight activation rows these types run one fused GEMV per row
-            detail::check(pmetal_hip_qgemm_reblocked((uint32_t)dtype_, (const uint8_t *)reblocked_->ptr(), reblocked_->bytes(), n_, k_,
-                                                     x.ptr(), x_dtype, m, y.ptr(), PMETAL_HIP_DTYPE_F32, stream));
-        else
-            detail::check(pmetal_hip_qlinear((uint32_t)dtype_, (const uint8_t *)w_.ptr(), n_, k_, x.ptr(), x_dtype, m, y.ptr(),
+        detail::check(pmetal_hip_qlinear((uint32_t)dtype_, (const uint8_t *)w_.ptr(), n_, k_, x.ptr(), x_dtype, m, y.ptr(),
                                              PMETAL_HIP_DTYPE_F32, order_, stream));
         return y;
     }
@@ -174,7 +161,6 @@ class GgufLinear {
     int64_t n_, k_;
     uint32_t order_;
     DeviceBuffer w_;
-    std::unique_ptr<DeviceBuffer> reblocked_;
 };
 
 // quantize_q8k (crates/pmetal-gguf/src/k_quants.rs:815-871) of n f32 values on the device: 292-byte BlockQ8K blocks.

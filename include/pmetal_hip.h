@@ -43,8 +43,8 @@ extern "C" {
 #define PMETAL_GGML_TYPE_Q5_1 7u
 #define PMETAL_GGML_TYPE_Q8_0 8u
 #define PMETAL_GGML_TYPE_Q8_1 9u
-#define PMETAL_GGML_TYPE_Q2K 10u /* quantize / dequantize (k_quants.rs:1242-1321, :230-266) and the fused GEMV; GEMM through Q6_K re-blocking */
-#define PMETAL_GGML_TYPE_Q3K 11u /* quantize / dequantize (k_quants.rs:1139-1237, :281-355) and the fused GEMV; GEMM through Q6_K re-blocking */
+#define PMETAL_GGML_TYPE_Q2K 10u /* quantize / dequantize (k_quants.rs:1242-1321, :230-266), the fused GEMV and the fused GEMM */
+#define PMETAL_GGML_TYPE_Q3K 11u /* quantize / dequantize (k_quants.rs:1139-1237, :281-355), the fused GEMV and the fused GEMM */
 #define PMETAL_GGML_TYPE_Q4K 12u
 #define PMETAL_GGML_TYPE_Q5K 13u /* quantize / dequantize (k_quants.rs:960-1051, :407-462), the fused GEMV and the fused GEMM */
 #define PMETAL_GGML_TYPE_Q6K 14u
@@ -167,12 +167,10 @@ int32_t pmetal_hip_dequantize_dev(uint32_t ggml_type, const uint8_t *src_dev, si
  * with W = reference dequantize of the packed blocks (order as given), fp32 accumulation,
  * max relative error <= 1e-3 against dequantize-then-f32-matmul.
  * W: [n, k] packed row-major, k a multiple of the block size.  x/X: f32 or bf16.
- * Types: Q8_0, Q4_K, Q5_K and Q6_K have both kernels (the Q5_K GEMM is the Q4_K kernel with the fifth bit of every quant
- * taken from the block's qh bytes).  Q5_K, Q3_K and Q2_K have a GEMV kernel for k <= 32768 and a tensor below
- * 4 GiB, any number of rows; beyond that qgemv fails with SHAPE_TOO_LARGE and qlinear uses the GEMM.  Q3_K and Q2_K have no GEMM
- * kernel of their own: qgemm re-blocks their super-blocks, without loss, into one (Q3_K) or two (Q2_K: values
- * and mins) Q6_K tensors in its scratch memory on every call (Q3_K 1.9, Q2_K 5 times the bytes of W) and runs the Q6_K
- * GEMM on them; qlinear runs one GEMV per activation row up to m = 8 for Q3_K and Q2_K (m = 2 for Q5_K) and qgemm above.
+ * Types: every type has both kernels (the Q5_K GEMM is the Q4_K kernel with the fifth bit of every quant taken from the
+ * block's qh bytes; Q3_K and Q2_K share a kernel for sixteen 16-element sub-blocks).  The GEMV of Q5_K, Q3_K and Q2_K takes
+ * k <= 32768 and a tensor below 4 GiB, any number of rows; beyond that qgemv fails with SHAPE_TOO_LARGE and qlinear uses the
+ * GEMM.  For these three types qlinear runs two activation rows as two GEMVs and three or more as one GEMM.
  * y/Y: f32 (qgemv) or f32/bf16 (qgemm), row-major [m, n].
  * qgemm keeps scratch memory (converted activations, partial tiles) inside the library, one
  * buffer per calling thread, device and stream; it grows on demand, which synchronises that
@@ -184,12 +182,11 @@ int32_t pmetal_hip_qgemm(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, in
                          void *stream);
 /* pmetal_hip_qgemm without any allocation.  No counterpart in the reference (there MLX owns every buffer): it is for
  * callers that cannot call hipMalloc -- code under HIP graph capture, tight serving loops, harnesses that forbid it.
- * Same arguments, kernels and results (bit for bit) as pmetal_hip_qgemm for Q8_0, Q4_K, Q5_K and Q6_K; the scratch memory
+ * Same arguments, kernels and results (bit for bit) as pmetal_hip_qgemm; the scratch memory
  * (converted activations, row scales, partial tiles of a K split) is a fixed array of
  * PMETAL_HIP_NOALLOC_SCRATCH_BYTES inside the library's code object, one copy per device, held until the process ends.
  * A shape that needs more (roughly: m * k * 2.25 bytes plus, for few activation rows, splits * m * n * 4) fails with
- * PMETAL_HIP_ERR_SHAPE_TOO_LARGE before anything is launched; Q3_K / Q2_K (re-blocking needs scratch of the size
- * of W) fail with PMETAL_HIP_ERR_UNSUPPORTED_TYPE.  Calls no hipMalloc / hipFree and nothing else that allocates.
+ * PMETAL_HIP_ERR_SHAPE_TOO_LARGE before anything is launched.  Calls no hipMalloc / hipFree and nothing else that allocates.
  * pmetal_hip_init(device) looks the array's address up; without it the first call on a device does.  All calls on one
  * device share the array: calls on one stream are ordered and may follow each other without a synchronisation; a call
  * that would overlap another one on the same device -- issued on a different stream before the previous call's kernels
@@ -202,7 +199,7 @@ int32_t pmetal_hip_qgemm_noalloc(uint32_t ggml_type, const uint8_t *w_dev, int64
                                  void *stream);
 /* Dispatch by m: m == 1 -> qgemv (f32 output only), otherwise qgemm (k must be a multiple of 256).  A Q8_0
  * row that is only a multiple of 32 runs one GEMV per activation row when m > 1 (f32 output only), and so do
- * Q3_K and Q2_K for 2 <= m <= 8 and Q5_K for m = 2, with f32 output. */
+ * Q5_K, Q3_K and Q2_K for m = 2, with f32 output. */
 int32_t pmetal_hip_qlinear(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, int64_t k, const void *x_dev,
                            uint32_t x_dtype, int64_t m, void *y_dev, uint32_t y_dtype, uint32_t order,
                            void *stream);
@@ -210,8 +207,8 @@ int32_t pmetal_hip_qlinear(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, 
 /* Several weights against the same [m, k] activations (the gate / up or q / k / v projections of a prefill: what a layer's
  * consecutive LayerWeight::matmul_from calls on one input amount to, weights.rs:66-84): the same results as one
  * pmetal_hip_qgemm per weight, bit for bit, with the activations converted once per element order instead of once per
- * weight.  Q8_0, Q4_K, Q5_K and Q6_K; the weights may differ in type, n, output type and element order (Q4_K and Q5_K
- * weights in the GGML order share one conversion).                                                                      */
+ * weight.  The weights may differ in type, n, output type and element order (Q4_K and Q5_K weights in the GGML order share
+ * one conversion, Q3_K and Q2_K weights another).                                                                       */
 typedef struct pmetal_hip_gemm_desc {
     uint32_t ggml_type;
     uint32_t y_dtype;
@@ -224,16 +221,15 @@ typedef struct pmetal_hip_gemm_desc {
 int32_t pmetal_hip_qgemm_batch(const pmetal_hip_gemm_desc *descs, size_t count, int64_t k, const void *x_dev,
                                uint32_t x_dtype, int64_t m, void *stream);
 
-/* Re-blocked weights for the GEMM of Q3_K / Q2_K (and of Q5_K, for callers that prepared one before its kernel existed:
- * pmetal_hip_qgemm on the original Q5_K blocks is the faster way).  The reference brings a weight into the layout its matmul wants
- * once, when the model is loaded (LayerWeight, crates/pmetal-bridge/src/qwen3_native/weights.rs:29-45: dense weights are
- * transposed at load time, quantized ones kept as MLX's quantized_matmul reads them); the counterpart here: Q3_K and Q2_K
- * have no GEMM kernel of their own, and their super-blocks convert without loss into one (Q3_K) or two (Q5_K, Q2_K:
- * values and mins) Q6_K tensors.  pmetal_hip_reblock_dev does that conversion once into memory the caller owns
+/* Re-blocked weights for the GEMM of Q5_K / Q3_K / Q2_K: the form these types multiplied in before they had matrix kernels of
+ * their own, kept for callers that prepared one (pmetal_hip_qgemm on the original blocks is the faster way and needs no copy).
+ * The reference brings a weight into the layout its matmul wants once, when the model is loaded (LayerWeight,
+ * crates/pmetal-bridge/src/qwen3_native/weights.rs:29-45: dense weights are transposed at load time, quantized ones kept as
+ * MLX's quantized_matmul reads them); the counterpart here: the super-blocks convert without loss into one (Q3_K) or two
+ * (Q5_K, Q2_K: values and mins) Q6_K tensors.  pmetal_hip_reblock_dev does that conversion once into memory the caller owns
  * (pmetal_hip_reblock_size bytes: 210 bytes per super-block and part, each part rounded up to 16; 0 for a type or shape
- * that is not re-blocked); pmetal_hip_qgemm_reblocked multiplies with it: the same result as pmetal_hip_qgemm, which for
- * Q3_K and Q2_K does both steps on every call (into scratch of that size) when handed the original blocks (for Q5_K: the
- * same numbers to the order of the f32 sums).  `order` applies to Q5_K only.
+ * that is not re-blocked); pmetal_hip_qgemm_reblocked multiplies with it: the same numbers as pmetal_hip_qgemm on the
+ * original blocks, to the order of the f32 sums.  `order` applies to Q5_K only.
  * The GEMV of these types reads the original blocks; a caller that wants both keeps both.                              */
 size_t pmetal_hip_reblock_size(uint32_t ggml_type, int64_t n, int64_t k);
 int32_t pmetal_hip_reblock_dev(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, int64_t k, uint32_t order,

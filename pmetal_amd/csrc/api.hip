@@ -703,13 +703,12 @@ int32_t codec_pipelined(bool quantize, uint32_t t, float *plain, uint8_t *packed
 extern "C" {
 
 // ---- quantized linear ----
-constexpr int64_t kRowLoopMax = 8;  // activation rows up to which qlinear sends Q5_K / Q3_K / Q2_K through the GEMV, row by row
+constexpr int64_t kRowLoopMax = 2;  // activation rows up to which qlinear sends Q5_K / Q3_K / Q2_K through the GEMV, row by row
 // types with a fused GEMV but no GEMM kernel of their own (their GEMM goes through Q6_K, see qgemm_reblocked)
 static bool gemv_only_type(uint32_t t) { return t == PMETAL_GGML_TYPE_Q5K || t == PMETAL_GGML_TYPE_Q3K || t == PMETAL_GGML_TYPE_Q2K; }
-// Of these, Q3_K and Q2_K reach the matrix cores only through re-blocking; Q5_K has a matrix kernel of its own (the Q4_K
-// kernel with the fifth bits), and its re-blocked form is kept for callers that prepared one.
-static bool reblocked_gemm_type(uint32_t t) { return t == PMETAL_GGML_TYPE_Q3K || t == PMETAL_GGML_TYPE_Q2K; }
-// check_linear for a GEMM entry point: Q5_K is accepted beside the path types, and y must take 16-byte stores
+// (These got their GEMV kernels first and reached the matrix cores through re-blocking into Q6_K; each has a matrix kernel of
+// its own now, and the re-blocked form is kept for callers that prepared one.)
+// check_linear for a GEMM entry point: they are accepted beside the path types, and y must take 16-byte stores
 static int32_t check_gemm(uint32_t t, const void *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, const void *y, uint32_t order);
 
 static int32_t check_linear(uint32_t t, const void *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype,
@@ -731,7 +730,7 @@ static int32_t check_linear(uint32_t t, const void *w, int64_t n, int64_t k, con
 }
 
 static int32_t check_gemm(uint32_t t, const void *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, const void *y, uint32_t order) {
-    if (int32_t rc = check_linear(t, w, n, k, x, x_dtype, y, order, t == PMETAL_GGML_TYPE_Q5K)) return rc;
+    if (int32_t rc = check_linear(t, w, n, k, x, x_dtype, y, order, gemv_only_type(t))) return rc;
     if (!aligned16(y)) return fail(PMETAL_HIP_ERR_INVALID_ARG, "device pointers must be 16-byte aligned");
     return PMETAL_HIP_OK;
 }
@@ -870,22 +869,6 @@ static int32_t check_reblocked_shape(int64_t n, int64_t k, int64_t m) {
     return PMETAL_HIP_OK;
 }
 
-// qgemm for these types when the caller has not re-blocked: re-block into the scratch buffer, then multiply.
-static int32_t qgemm_reblocked(uint32_t t, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, int64_t m, void *y,
-                               uint32_t y_dtype, uint32_t order, void *stream) {
-    hipStream_t s = (hipStream_t)stream;
-    if (int32_t rc = check_reblocked_shape(n, k, m)) return rc;
-    const int parts = pmh::reblock_q6k_parts(t);
-    size_t gemm_bytes = 0;
-    const size_t mul_bytes = reblocked_scratch_bytes(t, m, n, k, y_dtype, &gemm_bytes), w_bytes = reblocked_part_bytes(n, k);
-    void *ws = nullptr;
-    if (int32_t rc = workspace(mul_bytes + parts * w_bytes, s, &ws)) return rc;
-    uint8_t *wa = (uint8_t *)ws + mul_bytes;
-    hipError_t e = pmh::launch_reblock_q6k(t, w, (size_t)n * (size_t)(k / 256), order, wa, wa + w_bytes, s);
-    if (e != hipSuccess) return hip_fail(e, "re-blocking kernel launch");
-    return qgemm_over_reblocked(t, wa, n, k, x, x_dtype, m, y, y_dtype, (uint8_t *)ws, gemm_bytes, s);
-}
-
 size_t pmetal_hip_reblock_size(uint32_t t, int64_t n, int64_t k) {
     if (!gemv_only_type(t) || n <= 0 || k <= 0 || k % 256 != 0) return 0;
     return (size_t)pmh::reblock_q6k_parts(t) * reblocked_part_bytes(n, k);
@@ -927,15 +910,6 @@ int32_t pmetal_hip_qgemm_reblocked(uint32_t t, const uint8_t *reblocked, size_t 
 
 int32_t pmetal_hip_qgemm(uint32_t t, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, int64_t m,
                          void *y, uint32_t y_dtype, uint32_t order, void *stream) {
-    if (reblocked_gemm_type(t)) {
-        if (int32_t rc = check_linear(t, w, n, k, x, x_dtype, y, order, true)) return rc;
-        if (!aligned16(y)) return fail(PMETAL_HIP_ERR_INVALID_ARG, "device pointers must be 16-byte aligned");
-        if (y_dtype > PMETAL_HIP_DTYPE_BF16) return fail(PMETAL_HIP_ERR_INVALID_ARG, "y_dtype must be 0 (f32) or 1 (bf16)");
-        if (m <= 0 || m > 0x7FFFFFFF) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "m must be in [1, 2^31)");
-        if (!pmh::qgemm_fits(PMETAL_GGML_TYPE_Q6K, m, n, k))
-            return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qgemm: m and k must be at most 2^22 (m = %lld, k = %lld)", (long long)m, (long long)k);
-        return qgemm_reblocked(t, w, n, k, x, x_dtype, m, y, y_dtype, order, stream);
-    }
     if (int32_t rc = check_gemm(t, w, n, k, x, x_dtype, y, order)) return rc;
     if (y_dtype > PMETAL_HIP_DTYPE_BF16) return fail(PMETAL_HIP_ERR_INVALID_ARG, "y_dtype must be 0 (f32) or 1 (bf16)");
     if (m <= 0 || m > 0x7FFFFFFF) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "m must be in [1, 2^31)");
@@ -958,8 +932,6 @@ int32_t pmetal_hip_qgemm_batch(const pmetal_hip_gemm_desc *descs, size_t count, 
     size_t need = 0;
     for (size_t i = 0; i < count; i++) {
         const pmetal_hip_gemm_desc &d = descs[i];
-        if (reblocked_gemm_type(d.ggml_type))
-            return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "qgemm_batch: GGML type %u goes through re-blocking (use pmetal_hip_qgemm_reblocked)", d.ggml_type);
         if (int32_t rc = check_gemm(d.ggml_type, d.w_dev, d.n, k, x, x_dtype, d.y_dev, d.order)) return rc;
         if (d.y_dtype > PMETAL_HIP_DTYPE_BF16) return fail(PMETAL_HIP_ERR_INVALID_ARG, "y_dtype must be 0 (f32) or 1 (bf16)");
         if (m <= 0 || m > 0x7FFFFFFF) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "m must be in [1, 2^31)");
@@ -976,6 +948,7 @@ int32_t pmetal_hip_qgemm_batch(const pmetal_hip_gemm_desc *descs, size_t count, 
     auto layout = [](const pmetal_hip_gemm_desc &d) {
         if (d.ggml_type == PMETAL_GGML_TYPE_Q8_0) return 3;
         if (d.ggml_type == PMETAL_GGML_TYPE_Q6K) return 2;
+        if (d.ggml_type == PMETAL_GGML_TYPE_Q3K || d.ggml_type == PMETAL_GGML_TYPE_Q2K) return 5;  // (one element order)
         if (d.order != PMETAL_HIP_ORDER_REF) return 1;  // Q4_K and Q5_K agree in the GGML order
         return d.ggml_type == PMETAL_GGML_TYPE_Q5K ? 4 : 0;
     };
@@ -1000,8 +973,6 @@ int32_t pmetal_hip_qgemm_batch(const pmetal_hip_gemm_desc *descs, size_t count, 
 // the main kernel reads, padding rows included, and a K split writes every partial tile before the reduction reads it).
 int32_t pmetal_hip_qgemm_noalloc(uint32_t t, const uint8_t *w, int64_t n, int64_t k, const void *x, uint32_t x_dtype, int64_t m,
                                  void *y, uint32_t y_dtype, uint32_t order, void *stream) {
-    if (reblocked_gemm_type(t))
-        return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "qgemm_noalloc: GGML type %u goes through re-blocking, which needs scratch of the size of W", t);
     if (int32_t rc = check_gemm(t, w, n, k, x, x_dtype, y, order)) return rc;
     if (y_dtype > PMETAL_HIP_DTYPE_BF16) return fail(PMETAL_HIP_ERR_INVALID_ARG, "y_dtype must be 0 (f32) or 1 (bf16)");
     if (m <= 0 || m > 0x7FFFFFFF) return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "m must be in [1, 2^31)");
@@ -1059,13 +1030,12 @@ int32_t pmetal_hip_qlinear(uint32_t t, const uint8_t *w, int64_t n, int64_t k, c
         return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qlinear: a Q8_0 row of k=%lld (not a multiple of 256) runs through the GEMV, whose output is f32 only",
                     (long long)k);
     const bool q4k_pair = t == PMETAL_GGML_TYPE_Q4K && m == 2;
-    // (Q5_K has a matrix kernel of its own: two rows are two GEMVs -- 22.7 against 23.1 us at 14336 x 4096, 12.8 against 16.6 at
-    // 6144 x 4096 --, three rows are one GEMM: 33.7 against 23.0 and 18.7 against 16.5)
-    const bool row_loop_type = t == PMETAL_GGML_TYPE_Q5K ? m <= 2 : (gemv_only_type(t) && m <= kRowLoopMax);
+    // (Q5_K, Q3_K and Q2_K have no short-batch kernel: two rows are two GEMVs -- Q5_K 22.7 against 23.1 us at 14336 x 4096, 12.8
+    // against 16.6 at 6144 x 4096 --, three rows are one GEMM: 33.7 against 23.0 and 18.7 against 16.5)
+    const bool row_loop_type = gemv_only_type(t) && m <= kRowLoopMax;
     if ((q8_ragged || q4k_pair || row_loop_type) && y_dtype == PMETAL_HIP_DTYPE_F32 && m > 1 && n > 0 && k > 0 && x && y) {
         // The fused GEMM walks k in steps of 256, and a Q8_0 row may be any multiple of 32: one fused GEMV per activation row
-        // then, back to back on the stream.  Q3_K and Q2_K reach the GEMM through a re-blocking pass over the whole
-        // matrix, which a few rows do not repay.  Two Q4_K rows are two GEMVs: 13.7 against 16.1 us at 14336 x 4096
+        // then, back to back on the stream.  Two Q4_K rows are two GEMVs: 13.7 against 16.1 us at 14336 x 4096
         // (three rows: 19.6 against 16.4).
         const size_t x_row = (size_t)k * (x_dtype == PMETAL_HIP_DTYPE_F32 ? 4 : 2);
         for (int64_t r = 0; r < m; r++) {

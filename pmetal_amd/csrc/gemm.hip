@@ -85,12 +85,16 @@ __device__ __forceinline__ float bf16_to_f32(uint32_t h) { return __builtin_bit_
 // One thread per operand item: chunk u = 64 elements = sub-blocks 2u, 2u+1 (u = 4 sb + 2 h + g), k-step t.
 // ORDER 0 / 1: Q4_K element orders REF / GGML (1 is also Q5_K's GGML order); ORDER 2: the Q6_K layout, ORDER 3: the
 // natural order (Q8_0), both without block sums; ORDER 4: Q5_K's REF order, whose sub-block j holds its 32 elements as
-// consecutive nibbles of 16 bytes, so k-step t of a chunk is elements 8 t .. 8 t + 7, the even ones (low nibbles) first.
+// consecutive nibbles of 16 bytes, so k-step t of a chunk is elements 8 t .. 8 t + 7, the even ones (low nibbles) first;
+// ORDER 5: Q2_K / Q3_K, whose qs byte 32 h + l holds elements 128 h + l + 32 s at bit 2 s: k-step t of lane half g is dword
+// t / 2 of the bytes 16 g .. 16 g + 15 of a half with the shifts s = 2 (t % 2) (first run) and 2 (t % 2) + 1 (second run), and
+// the sums are those of the four 16-element sub-blocks 4 (t % 2) + 2 (run) + g of the half: 20 items per half.
 // ------------------------------------------------------------------------------------------------
 template <bool XF32, int ORDER, int R>
 __global__ __launch_bounds__(R == 1 ? 512 : 1024) void k_prep_rw(const void *__restrict__ xg, int64_t k, int M, int Mp,
                                                                   float *__restrict__ rowscale, uint4 *__restrict__ xs) {
     constexpr int NT = R == 1 ? 512 : 1024, JN = NT / R, NWV = NT / 64;
+    constexpr int kGroups = ORDER == 5 ? 20 : 18;  // items per half super-block and row (shadows the Q4_K constant)
     const int tid = threadIdx.x, lane = tid & 63, r = tid % R, j = tid / R;
     const int m = blockIdx.x * R + r;
     const bool live = m < M;
@@ -148,7 +152,9 @@ __global__ __launch_bounds__(R == 1 ? 512 : 1024) void k_prep_rw(const void *__r
             const int64_t u = q >> 3;
             t = (int)(q & 7), g = (int)u & 1;
             half = u >> 1;
-            lo = ORDER == 4 ? 64 * u + 8 * t : (ORDER == 0 ? 64 * u + 32 * (t >> 2) + 4 * (t & 3) : 64 * u + 4 * t);
+            lo = ORDER == 5   ? 128 * half + 64 * (t & 1) + 16 * g + 4 * (t >> 1)
+                 : ORDER == 4 ? 64 * u + 8 * t
+                              : (ORDER == 0 ? 64 * u + 32 * (t >> 2) + 4 * (t & 3) : 64 * u + 4 * t);
             hi = lo + (ORDER == 4 ? 4 : (ORDER == 0 ? 16 : 32));
         }
         float v[8];
@@ -183,6 +189,19 @@ __global__ __launch_bounds__(R == 1 ? 512 : 1024) void k_prep_rw(const void *__r
         if (ORDER == 2 || ORDER == 3) continue;  // Q6_K and Q8_0 have no min term: no block sums
         // sums of the two sub-blocks of the chunk over its 8 k-steps (8 lanes, R apart)
         float s0, s1;
+        if (ORDER == 5) {
+            // the first runs of the k-steps of one parity are one 16-element sub-block, their second runs another:
+            // k-step 0 ends up with the sums for t % 2 == 0 (item 16 + g), k-step 1 with those for t % 2 == 1 (item 18 + g)
+            slo += __shfl_xor(slo, 2 * R), shi += __shfl_xor(shi, 2 * R);
+            slo += __shfl_xor(slo, 4 * R), shi += __shfl_xor(shi, 4 * R);
+            if (t < 2) {
+                const _Float16 h0 = (_Float16)slo, h1 = (_Float16)shi;
+                const _Float16 l0 = (_Float16)(slo - (float)h0), l1 = (_Float16)(shi - (float)h1);
+                const half8_t item = {h0, l0, h0, l0, h1, l1, h1, l1};
+                xs[base + (size_t)(16 + 2 * t + g) * Mp] = __builtin_bit_cast(uint4, item);
+            }
+            continue;
+        }
         if (ORDER == 0 || ORDER == 4) {  // sub-block 2u: k-steps 0..3 (low and high nibbles), 2u+1: k-steps 4..7
             float s = slo + shi;
             s += __shfl_xor(s, R);
@@ -599,6 +618,249 @@ __global__ __launch_bounds__(64 * NW, MB * NR <= 1 && NW <= 8 ? 2 : 1) void k_qg
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();
     store_tile<MB, NW>(R.acc[0], smem, L.wave, L.col, L.g, m0, n0, M, N, Mp, rowscale, yg, partial, mode, blockIdx.z);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Q2_K and Q3_K (crates/pmetal-gguf/src/k_quants.rs:230-266, :281-355): sixteen 16-element sub-blocks per super-block,
+// two-bit quants, qs byte 32 h + l = elements 128 h + l + 32 s at bit 2 s.  The Q4_K kernel's structure with these
+// differences:
+//   * a half super-block of a row is 32 bytes of qs: lane (n, g) takes bytes 16 g .. 16 g + 15; dword t / 2 of them gives
+//     k-step t its eight values, four at shift 4 (t % 2) (sub-block 8 h + 4 (t % 2) + g) and four at 4 (t % 2) + 2
+//     (sub-block 8 h + 4 (t % 2) + 2 + g): four scales per lane and half, one quant copy per wave and half;
+//   * Q2_K: value d (sc & 15) q - dmin (sc >> 4), q in 0..3: the B tile is (sc & 15) q, and the min terms of the lane's
+//     four sub-blocks are two K = 16 products of exact head + tail splits (activation items 16 + g and 18 + g);
+//   * Q3_K: value d s' (q3 - 4) with s' = sc6 - 32 and q3 = q | hbit << 2, hbit = bit 4 h + s of hmask[l]: the B tile is
+//     s' q3 = (1024 + q3) s' - 1024 s' (1028 s' would not be an f16 number), and the - 4 d s' of every element leaves with the
+//     sub-block sums of the activations, exactly as Q2_K's mins do (coefficient 4 d s' in place of dmin m);
+//   * blocks are 84 / 110 bytes, so rows start at 4- / 2-byte aligned addresses (the direct-to-LDS loads take them); the
+//     header pieces of a row are Q2_K: bytes 0..15 (scales) and 68..83 (d, dmin in the last dword); Q3_K: 0..31 (hmask) and
+//     94..109 (scales in bytes 2..13 of the piece, d in 14..15).
+// ------------------------------------------------------------------------------------------------
+constexpr int kGroups16 = 20;  // activation items per row and half super-block: 16 operands and four of sub-block sums
+template <int FMT>
+struct Block16 {  // FMT 2: Q3_K, 3: Q2_K
+    static constexpr int kBytes = FMT == 3 ? 84 : 110, kQs = FMT == 3 ? 16 : 32;
+    static constexpr int kHdrPieces = FMT == 3 ? 2 : 3;           // per row and super-block
+    static constexpr int kHdrRounds = (32 * kHdrPieces + 63) / 64;  // whole-wave copies
+    static constexpr int kHdrStage = 64 * kHdrRounds;              // items of a wave's header stage
+    static __device__ __forceinline__ uint32_t piece_off(int p) { return FMT == 3 ? (p == 0 ? 0u : 68u) : (p == 2 ? 94u : 16u * (uint32_t)p); }
+};
+
+template <int FMT, int MB, int H>
+__device__ __forceinline__ void rw16_half(const uint4 *__restrict__ a_cur, uint4 *__restrict__ a_nxt, const uint4 *__restrict__ q_cur,
+                                          uint4 *__restrict__ q_nxt, uint4 *__restrict__ hs, const uint4 *__restrict__ xs_nxt,
+                                          const uint8_t *__restrict__ wq_nxt, const uint8_t *__restrict__ wh_nxt, const int wave,
+                                          const int col, const int g, const uint32_t q_off, const uint32_t (&h_off)[Block16<FMT>::kHdrRounds],
+                                          const uint32_t *a_off, float16_t (&acc)[MB], float16_t (&part)[MB], uint32_t (&hdr)[8],
+                                          uint32_t (&hm)[4], uint32_t &dbits) {
+    using B = Block16<FMT>;
+    constexpr int BM = 32 * MB, kThreads = 512, kARounds = (kGroups16 * BM + kThreads - 1) / kThreads;
+    if (H == 0) {
+        // this row's header pieces into registers, then their stage is refilled with the next super-block's
+        if (FMT == 3) {
+            const uint4 sc = hs[col * 2], dd = hs[col * 2 + 1];
+            hdr[0] = sc.x, hdr[1] = sc.y, hdr[2] = sc.z, hdr[3] = sc.w;
+            dbits = dd.w;  // d | dmin << 16
+        } else {
+            const uint4 m0 = hs[col * 3], m1 = hs[col * 3 + 1], sd = hs[col * 3 + 2];
+            // the lane's hmask bytes 16 g + 4 dw .. + 3 (both halves of the super-block use them)
+            hm[0] = g ? m1.x : m0.x, hm[1] = g ? m1.y : m0.y, hm[2] = g ? m1.z : m0.z, hm[3] = g ? m1.w : m0.w;
+            // the twelve scale bytes as three dwords (they start two bytes into the piece), d behind them
+            hdr[0] = __builtin_amdgcn_alignbit(sd.y, sd.x, 16), hdr[1] = __builtin_amdgcn_alignbit(sd.z, sd.y, 16);
+            hdr[2] = __builtin_amdgcn_alignbit(sd.w, sd.z, 16);
+            dbits = sd.w >> 16;
+        }
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+#pragma unroll
+        for (int r = 0; r < B::kHdrRounds; r++) dma16(wh_nxt + h_off[r], hs + 64 * r);
+    }
+#pragma unroll
+    for (int i = 0; i < kARounds; i++)
+        if (i * kThreads + wave * 64 < kGroups16 * BM) dma16(xs_nxt + a_off[i], a_nxt + i * kThreads + wave * 64);
+    // the quant copy must be the newest request of this half: the barrier at its end waits for all but it
+    __builtin_amdgcn_sched_barrier(0);
+    dma16(wq_nxt + q_off, q_nxt);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // this lane's 16 quant bytes: piece g of row col
+    const uint4 qv = q_cur[col * 2 + g];
+    const uint32_t qd[4] = {qv.x, qv.y, qv.z, qv.w};
+    // scales (and mins) of the lane's four sub-blocks j = 8 H + 4 sp + 2 lh + g, index 2 sp + lh
+    half2_t sc2[4], off2[4];
+    float nm[4];  // what a sub-block subtracts per unit of its activation sum, negated: -dmin m (Q2_K), -4 d s' (Q3_K); exact in fp32
+#pragma unroll
+    for (int sp = 0; sp < 2; sp++)
+#pragma unroll
+        for (int lh = 0; lh < 2; lh++) {
+            float scf;
+            if (FMT == 3) {  // byte j of the sixteen: low nibble scale, high nibble min
+                const uint32_t b = (hdr[2 * H + sp] >> (8u * (uint32_t)g + 16u * lh)) & 0xFFu;
+                scf = (float)(b & 15u);
+                nm[2 * sp + lh] = -(f16_bits_to_f32(dbits >> 16) * (float)(b >> 4));
+            } else {
+                // sc6 of sub-block j: low nibble (j < 8) or high nibble (j >= 8) of byte j % 8, bits 4..5 = bits
+                // 2 (j / 4) of byte 8 + j % 4
+                const uint32_t lo4 = (hdr[sp] >> (8u * (uint32_t)g + 16u * lh + 4u * H)) & 15u;
+                const uint32_t hi2 = (hdr[2] >> (8u * (uint32_t)g + 16u * lh + 2u * (2 * H + sp))) & 3u;
+                scf = (float)((int)(lo4 | (hi2 << 4)) - 32);
+                nm[2 * sp + lh] = -(f16_bits_to_f32(dbits & 0xFFFFu) * (4.0f * scf));
+            }
+            const _Float16 sh = (_Float16)scf, oh = (_Float16)(-1024.0f * scf);  // exact: |sc| <= 32
+            sc2[2 * sp + lh] = half2_t{sh, sh}, off2[2 * sp + lh] = half2_t{oh, oh};
+        }
+    // operand of k-step t: dword t / 2, the two-bit fields at 4 (t % 2) and 4 (t % 2) + 2 (Q3_K: bit 2 from hmask)
+    auto operand = [&](int t) -> half8_t {
+        const int dw = t >> 1, sp = t & 1;
+        uint32_t lo = (qd[dw] >> (4 * sp)) & 0x03030303u, hi = (qd[dw] >> (4 * sp + 2)) & 0x03030303u;
+        if (FMT == 2) {
+            const uint32_t m = hm[dw] >> (4 * H + 2 * sp);
+            lo |= (m & 0x01010101u) << 2, hi |= (m & 0x02020202u) << 1;
+        }
+        const half2_t r0 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, lo, 0x04010400u)), sc2[2 * sp], off2[2 * sp]);
+        const half2_t r1 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, lo, 0x04030402u)), sc2[2 * sp], off2[2 * sp]);
+        const half2_t r2 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, hi, 0x04010400u)), sc2[2 * sp + 1], off2[2 * sp + 1]);
+        const half2_t r3 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, hi, 0x04030402u)), sc2[2 * sp + 1], off2[2 * sp + 1]);
+        return half8_t{r0[0], r0[1], r1[0], r1[1], r2[0], r2[1], r3[0], r3[1]};
+    };
+    half8_t af[2][MB];
+#pragma unroll
+    for (int i = 0; i < MB; i++) af[0][i] = __builtin_bit_cast(half8_t, a_cur[g * BM + 32 * i + col]);
+    half8_t b = operand(0);
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+        const half8_t bt = b;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < MB; i++) {
+            const half8_t a = af[t & 1][i];
+            if (H == 0 && t == 0) {  // first product of a super-block starts from zero
+                float16_t z;
+#pragma unroll
+                for (int r = 0; r < 16; r++) z[r] = 0.0f;
+                part[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bt, z, 0, 0, 0);
+            } else {
+                part[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bt, part[i], 0, 0, 0);
+            }
+            if (i == 0) {
+                // the next step's fragments (after the last step: the first sums item) and its operand
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int ii = 0; ii < MB; ii++)
+                    af[(t + 1) & 1][ii] = __builtin_bit_cast(half8_t, a_cur[(t < 7 ? (t + 1) * 2 + g : 16 + g) * BM + 32 * ii + col]);
+                if (t < 7) b = operand(t + 1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    {
+        // sum terms of the lane's four sub-blocks: exact head + tail splits (h, h, l, l) against the sums' (H, L, H, L), pairs
+        // (sp, 0), (sp, 1)
+#pragma unroll
+        for (int sp = 0; sp < 2; sp++) {
+            const _Float16 h0 = (_Float16)nm[2 * sp], h1 = (_Float16)nm[2 * sp + 1];
+            const _Float16 l0 = (_Float16)(nm[2 * sp] - (float)h0), l1 = (_Float16)(nm[2 * sp + 1] - (float)h1);
+            const half8_t br = half8_t{h0, h0, l0, l0, h1, h1, l1, l1};
+#pragma unroll
+            for (int i = 0; i < MB; i++) {
+                const half8_t a = sp == 0 ? af[0][i] : __builtin_bit_cast(half8_t, a_cur[(18 + g) * BM + 32 * i + col]);
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, br, acc[i], 0, 0, 0);
+            }
+        }
+    }
+    if (H == 1) {
+        const float d = f16_bits_to_f32(dbits & 0xFFFFu);
+#pragma unroll
+        for (int i = 0; i < MB; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][r] = __builtin_fmaf(d, part[i][r], acc[i][r]);
+    }
+}
+
+// grid and modes as k_qgemm_rw; eight waves of 32 weight rows
+template <int FMT, int MB>
+__global__ __launch_bounds__(512, MB <= 1 ? 2 : 1) void k_qgemm_rw16(const uint8_t *__restrict__ W, const uint4 *__restrict__ xs,
+                                                                      const float *__restrict__ rowscale, void *__restrict__ yg,
+                                                                      float *__restrict__ partial, int M, int Mp, int N, int spr, int chunk,
+                                                                      int mode) {
+    using B = Block16<FMT>;
+    constexpr int BM = 32 * MB, NW = 8, kThreads = 512, kRows = 256, kARounds = (kGroups16 * BM + kThreads - 1) / kThreads;
+    extern __shared__ uint4 smem[];
+    uint4 *a0 = smem, *a1 = a0 + kGroups16 * BM, *qbase = a1 + kGroups16 * BM, *hb = qbase + 3 * NW * 64;
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63, col = lane & 31, g = lane >> 5;
+    const int n0 = blockIdx.x * kRows, m0 = blockIdx.y * BM;
+    const int nw0 = n0 + 32 * wave;  // first weight row of this wave
+    const int sb0 = blockIdx.z * chunk;
+    const int cnt = spr - sb0 < chunk ? spr - sb0 : chunk;
+    const uint32_t row_bytes = (uint32_t)spr * B::kBytes;
+    auto row_off = [&](int row) {  // byte offset of a row of this wave from the workgroup's first row; rows past N repeat the last
+        int n = nw0 + row;
+        n = n < N ? n : N - 1;
+        return (uint32_t)(n - n0) * row_bytes;
+    };
+    // quant copy: lane -> (row lane / 2, piece lane % 2); header copies: item lane + 64 r -> (row item / P, piece item % P)
+    const uint32_t q_off = row_off(lane >> 1) + 16u * (uint32_t)(lane & 1);
+    uint32_t h_off[B::kHdrRounds];
+#pragma unroll
+    for (int r = 0; r < B::kHdrRounds; r++) {
+        int item = lane + 64 * r;
+        item = item < 32 * B::kHdrPieces ? item : 32 * B::kHdrPieces - 1;  // (the copies past the last item repeat it into the stage's padding)
+        h_off[r] = row_off(item / B::kHdrPieces) + B::piece_off(item % B::kHdrPieces);
+    }
+    uint32_t a_off[kARounds];
+#pragma unroll
+    for (int i = 0; i < kARounds; i++) {
+        const int idx = tid + i * kThreads;
+        a_off[i] = (uint32_t)((idx / BM) * Mp + idx % BM);
+    }
+    uint4 *qa = qbase + wave * 64, *qb = qa + NW * 64, *qc = qb + NW * 64;
+    uint4 *hw = hb + wave * B::kHdrStage;
+    const uint8_t *wblk = W + (size_t)n0 * row_bytes;
+
+    float16_t acc[MB], part[MB];
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[i][r] = 0.0f, part[i][r] = 0.0f;
+    uint32_t hdr[8] = {0, 0, 0, 0, 0, 0, 0, 0}, hm[4] = {0, 0, 0, 0}, dbits = 0;
+
+    {  // prologue: headers, both halves' quant pieces and the first activation stage of super-block sb0
+        const uint8_t *blk = wblk + (size_t)sb0 * B::kBytes;
+#pragma unroll
+        for (int r = 0; r < B::kHdrRounds; r++) dma16(blk + h_off[r], hw + 64 * r);
+        dma16(blk + B::kQs + q_off, qa);
+        dma16(blk + B::kQs + 32 + q_off, qb);
+        const uint4 *xa = xs + (size_t)(sb0 * 2 * kGroups16) * Mp + m0;
+#pragma unroll
+        for (int i = 0; i < kARounds; i++)
+            if (i * kThreads + wave * 64 < kGroups16 * BM) dma16(xa + a_off[i], a0 + i * kThreads + wave * 64);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();
+
+    for (int s = 0; s < cnt; s++) {
+        const int sb = sb0 + s;
+        const int sbn = sb + 1 < spr ? sb + 1 : spr - 1;  // the copies for "the next super-block" stay inside the matrix
+        const uint8_t *blkn = wblk + (size_t)sbn * B::kBytes;
+        rw16_half<FMT, MB, 0>(a0, a1, qa, qc, hw, xs + (size_t)((sb * 2 + 1) * kGroups16) * Mp + m0, blkn + B::kQs, blkn, wave, col, g, q_off,
+                              h_off, a_off, acc, part, hdr, hm, dbits);
+        barrier_keep<1>();
+        rw16_half<FMT, MB, 1>(a1, a0, qb, qa, hw, xs + (size_t)(sbn * 2 * kGroups16) * Mp + m0, blkn + B::kQs + 32, nullptr, wave, col, g, q_off,
+                              h_off, a_off, acc, part, hdr, hm, dbits);
+        barrier_keep<1>();
+        uint4 *t = qc;  // two half super-blocks on: (qa, qb, qc) <- (qc, qa, qb)
+        qc = qb, qb = qa, qa = t;
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();
+    store_tile<MB, NW>(acc, smem, wave, col, g, m0, n0, M, N, Mp, rowscale, yg, partial, mode, blockIdx.z);
+}
+
+template <int FMT, int MB>
+constexpr size_t rw16_lds_bytes() {
+    const size_t stages = (size_t)(2 * kGroups16 * 32 * MB + 8 * (3 * 64 + Block16<FMT>::kHdrStage)) * 16;
+    return stages > tile_lds_bytes<MB, 8>() ? stages : tile_lds_bytes<MB, 8>();
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1586,7 +1848,7 @@ static int compute_units_gemm() {
 
 bool qgemm_fits(uint32_t type, int64_t m, int64_t n, int64_t k) {
     // byte offsets inside a workgroup's rows and item offsets inside the activation copy are 32-bit
-    return (type == kTypeQ4K || type == kTypeQ5K || type == kTypeQ6K || type == kTypeQ8_0) && m >= 1 && m <= (int64_t)1 << 22 && n >= 1 && k >= 256 && k % 256 == 0 && k <= (int64_t)1 << 22 && n <= 0x7FFFFF00;
+    return (type == kTypeQ4K || type == kTypeQ5K || type == kTypeQ6K || type == kTypeQ8_0 || type == kTypeQ3K || type == kTypeQ2K) && m >= 1 && m <= (int64_t)1 << 22 && n >= 1 && k >= 256 && k % 256 == 0 && k <= (int64_t)1 << 22 && n <= 0x7FFFFF00;
 }
 
 GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k, uint32_t type) {
@@ -1623,13 +1885,13 @@ GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k, uint32_t type) {
     // at most 16 activation rows against long rows: runs of 16 super-blocks (the fused kernels' K split; the large kernel
     // takes the same split when a shape falls back to it)
     // (a type without such kernels keeps the split chosen above)
-    if (m <= kSmallMaxM && spr > kSmallMaxSpr && type != kTypeQ5K) p.chunk = kSmallMaxSpr, p.splits = (int)((spr + kSmallMaxSpr - 1) / kSmallMaxSpr);
+    if (m <= kSmallMaxM && spr > kSmallMaxSpr && (type == kTypeQ4K || type == kTypeQ6K || type == kTypeQ8_0)) p.chunk = kSmallMaxSpr, p.splits = (int)((spr + kSmallMaxSpr - 1) / kSmallMaxSpr);
     return p;
 }
 
 size_t qgemm_workspace_bytes(uint32_t type, int64_t m, int64_t n, int64_t k) {
     const GemmPlan p = qgemm_plan(m, n, k, type);
-    const size_t xs = align256((size_t)(k / 256) * 2 * kGroups * p.mp * 16);
+    const size_t xs = align256((size_t)(k / 256) * 2 * (type == kTypeQ3K || type == kTypeQ2K ? kGroups16 : kGroups) * p.mp * 16);
     // the short-batch kernels take a row of up to kSmallMaxSpr super-blocks whole: the plan's K split is not used there
     const bool unsplit = qgemm_small_applies(type, m, n, k) && k / 256 <= kSmallMaxSpr;
     const size_t part = p.splits > 1 && !unsplit ? align256((size_t)p.splits * p.mp * n * 4) : 0;
@@ -1648,6 +1910,20 @@ static hipError_t launch_rw(hipStream_t s, const uint8_t *w, const uint4 *xs, co
     }
     const dim3 grid((unsigned)((n + kRows - 1) / kRows), (unsigned)(p.mp / (32 * MB)), (unsigned)p.splits);
     hipLaunchKernelGGL(kern, grid, dim3(64 * NW), lds, s, w, xs, rowscale, y, partial, (int)m, (int)p.mp, (int)n, spr, p.chunk, mode);
+    return hipGetLastError();
+}
+
+template <int FMT, int MB>
+static hipError_t launch_rw16(hipStream_t s, const uint8_t *w, const uint4 *xs, const float *rowscale, void *y, float *partial, int64_t m,
+                              int64_t n, int spr, const GemmPlan &p, int mode) {
+    auto kern = k_qgemm_rw16<FMT, MB>;
+    constexpr size_t lds = rw16_lds_bytes<FMT, MB>();
+    if (lds > 64 * 1024) {
+        hipError_t a = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (a != hipSuccess) return a;
+    }
+    const dim3 grid((unsigned)((n + 255) / 256), (unsigned)(p.mp / (32 * MB)), (unsigned)p.splits);
+    hipLaunchKernelGGL(kern, grid, dim3(512), lds, s, w, xs, rowscale, y, partial, (int)m, (int)p.mp, (int)n, spr, p.chunk, mode);
     return hipGetLastError();
 }
 
@@ -1686,11 +1962,12 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
     const int spr = (int)(k / 256);
     uint8_t *ws = reinterpret_cast<uint8_t *>(workspace);
     uint4 *xs = reinterpret_cast<uint4 *>(ws);
-    const size_t xs_bytes = align256((size_t)spr * 2 * kGroups * p.mp * 16);
+    const bool q23 = type == kTypeQ3K || type == kTypeQ2K;
+    const size_t xs_bytes = align256((size_t)spr * 2 * (q23 ? kGroups16 : kGroups) * p.mp * 16);
     float *rowscale = reinterpret_cast<float *>(ws + xs_bytes);
     float *partial = reinterpret_cast<float *>(ws + xs_bytes + align256((size_t)p.mp * 4));
     const bool xf32 = x_dtype == kDtypeF32, q6 = type == kTypeQ6K, q8 = type == kTypeQ8_0, q5 = type == kTypeQ5K, ref = order == kOrderRef;
-    const int xorder = q8 ? 3 : (q6 ? 2 : (ref ? (q5 ? 4 : 0) : 1));  // the element order the pre-pass lays the activations out for
+    const int xorder = q23 ? 5 : (q8 ? 3 : (q6 ? 2 : (ref ? (q5 ? 4 : 0) : 1)));  // the element order the pre-pass lays the activations out for
 #define PMH_PREP(F, O)                                                                                                       \
     do {                                                                                                                     \
         if (p.mp >= 1024)                                                                                                    \
@@ -1707,13 +1984,15 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
         else if (xorder == 1) PMH_PREP(true, 1);
         else if (xorder == 2) PMH_PREP(true, 2);
         else if (xorder == 3) PMH_PREP(true, 3);
-        else PMH_PREP(true, 4);
+        else if (xorder == 4) PMH_PREP(true, 4);
+        else PMH_PREP(true, 5);
     } else {
         if (xorder == 0) PMH_PREP(false, 0);
         else if (xorder == 1) PMH_PREP(false, 1);
         else if (xorder == 2) PMH_PREP(false, 2);
         else if (xorder == 3) PMH_PREP(false, 3);
-        else PMH_PREP(false, 4);
+        else if (xorder == 4) PMH_PREP(false, 4);
+        else PMH_PREP(false, 5);
     }
 #undef PMH_PREP
     hipError_t e = hipGetLastError();
@@ -1809,6 +2088,13 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
         e = p.mb == 1   ? launch_rw_q6<1>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
             : p.mb == 2 ? launch_rw_q6<2>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
                         : launch_rw_q6<4>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode);
+    } else if (q23) {
+        e = type == kTypeQ2K ? (p.mb == 1   ? launch_rw16<3, 1>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
+                                : p.mb == 2 ? launch_rw16<3, 2>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
+                                            : launch_rw16<3, 4>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode))
+                             : (p.mb == 1   ? launch_rw16<2, 1>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
+                                : p.mb == 2 ? launch_rw16<2, 2>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
+                                            : launch_rw16<2, 4>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode));
     } else if (q5) {
 #define PMH_RW5_CASE(O, B) launch_rw<O, B, 1, 8, 1>(s, w, xs, rowscale, y, partial, m, n, spr, p, mode)
         e = p.mb == 1   ? (ref ? PMH_RW5_CASE(0, 1) : PMH_RW5_CASE(1, 1))

@@ -273,11 +273,9 @@ class GgufLinear:
     Mirrors ``LayerWeight::matmul_from`` (crates/pmetal-bridge/src/qwen3_native/weights.rs:66-84): one token goes through
     the fused GEMV, several through the fused GEMM.  ``w`` are the packed block bytes (host array or device buffer).
     As the reference brings a weight into its matmul's layout when the model is loaded (weights.rs:29-45),
-    ``prepare_gemm=True`` re-blocks a Q3_K / Q2_K weight once into the Q6_K form their GEMM multiplies with
-    (the original blocks stay for the GEMV); without it the GEMM of those types re-blocks on every call.  Q5_K has a
-    matrix kernel that reads its blocks as they are, so nothing is prepared for it."""
-
-    ROW_LOOP_MAX = 8  # up to this many activation rows Q5_K / Q3_K / Q2_K run one fused GEMV per row
+    Every type has matrix kernels that read its blocks as they are, so nothing is prepared at load time; ``prepare_gemm``
+    is accepted and ignored (it used to re-block Q5_K / Q3_K / Q2_K weights into the Q6_K form their GEMM then multiplied
+    with: ``pmetal_hip_reblock_dev`` / ``pmetal_hip_qgemm_reblocked`` still do that for callers who ask)."""
 
     def __init__(self, dtype: int, n: int, k: int, w, order: int = ORDER_REF, prepare_gemm: bool = False):
         self.dtype, self.n, self.k, self.order = GgmlType(dtype), int(n), int(k), order
@@ -287,24 +285,13 @@ class GgufLinear:
                 raise DequantError(3, f"Invalid data size: expected {expected} bytes, got {w.size}")
             w = DeviceBuffer.from_host(np.ascontiguousarray(w, dtype=np.uint8))
         self.w = w
-        self.reblocked, self.reblocked_len = None, 0
-        if prepare_gemm and int(self.dtype) != 13:
-            lib = _lib.load()
-            self.reblocked_len = lib.pmetal_hip_reblock_size(int(self.dtype), self.n, self.k)
-            if self.reblocked_len:
-                self.reblocked = DeviceBuffer(self.reblocked_len)
-                check(lib.pmetal_hip_reblock_dev(int(self.dtype), _dev_ptr(self.w), self.n, self.k, self.order,
-                                                 self.reblocked.ptr, self.reblocked_len, None))
+        self.reblocked, self.reblocked_len = None, 0  # (kept for callers that look at them)
 
     def forward(self, x, m: int = 1, x_dtype: int = DTYPE_BF16, y=None, y_dtype: int = DTYPE_F32, stream=None):
         """``x``: device buffer of ``[m, k]`` activations; returns the device buffer of ``[m, n]`` outputs."""
         lib = _lib.load()
         if y is None:
             y = DeviceBuffer(m * self.n * (4 if y_dtype == DTYPE_F32 else 2))
-        if self.reblocked is not None and (m > self.ROW_LOOP_MAX or y_dtype != DTYPE_F32):
-            check(lib.pmetal_hip_qgemm_reblocked(int(self.dtype), self.reblocked.ptr, self.reblocked_len, self.n, self.k,
-                                                 _dev_ptr(x), x_dtype, m, _dev_ptr(y), y_dtype, stream))
-            return y
         check(lib.pmetal_hip_qlinear(int(self.dtype), _dev_ptr(self.w), self.n, self.k, _dev_ptr(x), x_dtype, m,
                                      _dev_ptr(y), y_dtype, self.order, stream))
         return y

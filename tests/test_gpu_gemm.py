@@ -302,8 +302,9 @@ def test_qgemm_on_two_streams_of_one_thread_keep_separate_scratch(oracle):
         lib.pmetal_hip_stream_destroy(s2)
 
 
-# Q5_K, Q3_K and Q2_K reach the GEMM through an exact re-blocking into Q6_K super-blocks (one tensor, or two for the formats
-# with mins).  d / dmin offsets inside a block, for random block bytes with finite scales:
+# Q5_K, Q3_K and Q2_K: matrix kernels of their own (and, for weights prepared that way, an exact re-blocking into Q6_K
+# super-blocks: one tensor, or two for the formats with mins).  d / dmin offsets inside a block, for random block bytes with
+# finite scales:
 REBLOCKED = {13: (176, (0, 2)), 11: (110, (108,)), 10: (84, (80, 82))}
 
 
@@ -343,34 +344,38 @@ def test_qgemm_q5k_q3k_q2k_matches_dequantize_then_matmul(oracle, t, m, n, k):
         assert norm <= 2 * TOL and elem_r <= TOL and norm_r <= TOL, (row, norm, elem_r, norm_r)
 
 
-@pytest.mark.parametrize("order", [0, 1])
+@pytest.mark.parametrize("t,order", [(13, 0), (13, 1), (11, 0), (10, 0)])
 @pytest.mark.parametrize("m,n,k", [(7, 96, 512), (40, 300, 1024), (130, 257, 768), (300, 64, 2048)])
-def test_qgemm_q5k_unit_activations_pick_single_weights(oracle, order, m, n, k):
-    """The Q5_K matrix kernel (the Q4_K kernel with the fifth bits from qh): with unit activations row r of the result is
-    column c_r of the dequantized weight, bit for bit -- every quant value, both element orders, every k-step and lane
-    position over the rows -- and the re-blocked form of the same weight gives the same numbers to the f32 summation order."""
+def test_qgemm_q5k_q3k_q2k_unit_activations_pick_single_weights(oracle, t, order, m, n, k):
+    """The matrix kernels of Q5_K (the Q4_K kernel with the fifth bits from qh) and of Q3_K / Q2_K (sixteen 16-element
+    sub-blocks): with unit activations row r of the result is column c_r of the dequantized weight, bit for bit -- every
+    quant value, scale and min, both element orders of Q5_K, every k-step and lane position over the rows, rows that start
+    at 2- and 4-byte aligned addresses -- and the re-blocked form of the same weight gives the same numbers to the f32
+    summation order."""
     lib = _lib.load()
-    rng = np.random.default_rng(77 * m + n + k + order)
-    raw = rng.integers(0, 256, size=(n * (k // 256), 176), dtype=np.uint8)
-    raw[:, 0:4] = np.frombuffer(np.array([0.01, 0.02], np.float16).tobytes(), np.uint8)
+    size, d_at = REBLOCKED[t]
+    rng = np.random.default_rng(77 * m + n + k + order + t)
+    raw = rng.integers(0, 256, size=(n * (k // 256), size), dtype=np.uint8)
+    for j, off in enumerate(d_at):
+        raw[:, off:off + 2] = np.frombuffer(np.array([0.01 * (j + 1)], np.float16).tobytes(), np.uint8)
     raw = raw.reshape(-1)
-    w = oracle.dequantize(13, raw, [n, k], order=order).reshape(n, k)
+    w = oracle.dequantize(t, raw, [n, k], order=order).reshape(n, k)
     for rep in range(3):
         cols = (np.arange(m) * (29 + 2 * rep) + 31 * rep + 3) % k
         xu = np.zeros((m, k), np.float32)
         xu[np.arange(m), cols] = 1.0
-        got = gpu_qgemm(13, raw, n, k, oracle.f32_to_bf16_bits(xu.reshape(-1)).reshape(m, k), m, order=order)
+        got = gpu_qgemm(t, raw, n, k, oracle.f32_to_bf16_bits(xu.reshape(-1)).reshape(m, k), m, order=order)
         for r, c in enumerate(cols):
             assert np.array_equal(got[r], w[:, c]), (rep, r, c)
     # against the re-blocked form (two Q6_K tensors) on random activations
     x = rng.standard_normal((m, k)).astype(np.float32)
     bits = oracle.f32_to_bf16_bits(x.reshape(-1)).reshape(m, k)
-    got = gpu_qgemm(13, raw, n, k, bits, m, order=order)
+    got = gpu_qgemm(t, raw, n, k, bits, m, order=order)
     dw = pm.DeviceBuffer.from_host(raw)
-    size = lib.pmetal_hip_reblock_size(13, n, k)
+    size = lib.pmetal_hip_reblock_size(t, n, k)
     dr, dx, dy = pm.DeviceBuffer(size), pm.DeviceBuffer.from_host(bits), pm.DeviceBuffer(4 * m * n)
-    pm.check(lib.pmetal_hip_reblock_dev(13, dw.ptr, n, k, order, dr.ptr, size, None))
-    pm.check(lib.pmetal_hip_qgemm_reblocked(13, dr.ptr, size, n, k, dx.ptr, pm.DTYPE_BF16, m, dy.ptr, pm.DTYPE_F32, None))
+    pm.check(lib.pmetal_hip_reblock_dev(t, dw.ptr, n, k, order, dr.ptr, size, None))
+    pm.check(lib.pmetal_hip_qgemm_reblocked(t, dr.ptr, size, n, k, dx.ptr, pm.DTYPE_BF16, m, dy.ptr, pm.DTYPE_F32, None))
     pm.check(lib.pmetal_hip_sync(None))
     other = dy.to_host(np.float32).reshape(m, n)
     assert np.max(np.abs(got - other)) <= 1e-5 * np.max(np.abs(other))
@@ -433,9 +438,10 @@ def test_qgemm_batch_equals_separate_calls(oracle):
     lib = _lib.load()
     k = 2048
     rng = np.random.default_rng(5150)
-    # (Q5_K behind Q4_K in the GGML order shares its converted activations; in the REF order it has a layout of its own)
+    # (Q5_K behind Q4_K in the GGML order shares its converted activations; in the REF order it has a layout of its own; Q3_K and
+    # Q2_K share theirs)
     specs = [(Q4K, 768, 0, pm.DTYPE_F32), (Q4K, 512, 0, pm.DTYPE_BF16), (Q4K, 256, 1, pm.DTYPE_F32), (13, 512, 1, pm.DTYPE_F32),
-             (13, 384, 0, pm.DTYPE_BF16), (Q6K, 640, 0, pm.DTYPE_F32),
+             (13, 384, 0, pm.DTYPE_BF16), (11, 300, 0, pm.DTYPE_F32), (10, 520, 0, pm.DTYPE_BF16), (Q6K, 640, 0, pm.DTYPE_F32),
              (Q6K, 320, 0, pm.DTYPE_BF16), (Q8_0, 384, 0, pm.DTYPE_F32), (Q4K, 1024, 0, pm.DTYPE_F32), (13, 256, 0, pm.DTYPE_F32)]
     ws = [pm.DeviceBuffer.from_host(oracle.quantize(t, weights(800 + i, n * k))) for i, (t, n, _, _) in enumerate(specs)]
     for m in (3, 48, 300):
@@ -453,7 +459,7 @@ def test_qgemm_batch_equals_separate_calls(oracle):
         pm.check(lib.pmetal_hip_sync(None))
         for i in range(len(specs)):
             assert np.array_equal(y_one[i].to_host(np.uint8), y_bat[i].to_host(np.uint8)), (m, specs[i])
-    bad = (_lib.GemmDesc * 1)(_lib.GemmDesc(11, 0, 0, 0, 256, ws[0].ptr, y_bat[0].ptr))  # Q3_K: only through re-blocking
+    bad = (_lib.GemmDesc * 1)(_lib.GemmDesc(15, 0, 0, 0, 256, ws[0].ptr, y_bat[0].ptr))  # Q8_K: activations only
     assert lib.pmetal_hip_qgemm_batch(bad, 1, k, dx.ptr, pm.DTYPE_BF16, 3, None) == 2
     lib.pmetal_hip_clear_error()
 

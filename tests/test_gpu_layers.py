@@ -92,9 +92,8 @@ def _forward(oracle, layers, x, project):
 def test_two_layer_stack_of_gguf_linears(oracle, m):
     layers = _layers(oracle)
     lin = [{nm: pm.GgufLinear(t, n, k, raw, prepare_gemm=True) for nm, (t, n, k, raw) in layer.items()} for layer in layers]
-    # (Q3_K and Q2_K are re-blocked for the GEMM; Q5_K and the path types multiply their blocks as they are)
-    assert lin[1]["ffn_up"].reblocked is not None and lin[1]["ffn_gate"].reblocked is not None
-    assert lin[1]["attn_qkv"].reblocked is None and lin[0]["attn_q"].reblocked is None
+    # (every type multiplies its blocks as they are: nothing is prepared)
+    assert all(l.reblocked is None for layer in lin for l in layer.values())
     threads = min(oracle.host_threads(), 16)
     worst = [0.0]
 
@@ -129,8 +128,8 @@ def test_two_layer_stack_of_gguf_linears(oracle, m):
 
 @pytest.mark.parametrize("t", [13, 11, 10])
 def test_reblocked_gemm_equals_qgemm_and_rejects_bad_sizes(oracle, t):
-    """pmetal_hip_qgemm_reblocked over weights re-blocked once gives the bits pmetal_hip_qgemm gives (which re-blocks per call);
-    for Q5_K, whose pmetal_hip_qgemm is a matrix kernel of its own, the same numbers to the f32 summation order."""
+    """pmetal_hip_qgemm_reblocked over weights re-blocked once gives what pmetal_hip_qgemm gives on the original blocks (a
+    matrix kernel of the type's own), to the f32 summation order."""
     from pmetal_amd import _lib
     lib = _lib.load()
     n, k, m = 384, 2048, 40
@@ -146,9 +145,7 @@ def test_reblocked_gemm_equals_qgemm_and_rejects_bad_sizes(oracle, t):
         pm.check(lib.pmetal_hip_qgemm(t, dw.ptr, n, k, dx.ptr, pm.DTYPE_BF16, m, y1.ptr, y_dtype, 0, None))
         pm.check(lib.pmetal_hip_qgemm_reblocked(t, rb.ptr, size, n, k, dx.ptr, pm.DTYPE_BF16, m, y2.ptr, y_dtype, None))
         pm.check(lib.pmetal_hip_sync(None))
-        if t != 13:
-            assert np.array_equal(y1.to_host(np.uint8), y2.to_host(np.uint8))
-        elif y_dtype == pm.DTYPE_F32:
+        if y_dtype == pm.DTYPE_F32:
             a, b = y1.to_host(np.float32), y2.to_host(np.float32)
             assert np.max(np.abs(a - b)) <= 1e-5 * np.max(np.abs(b))
         else:

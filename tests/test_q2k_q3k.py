@@ -257,9 +257,9 @@ def test_gpu_q2k_q3k_gemv_unit_vectors_and_linear(oracle, t):
     x = np.random.default_rng(5).standard_normal(k).astype(np.float32)
     x[100] = np.inf
     assert np.isnan(gpu_qgemv(t, wq, n, k, x, pm.DTYPE_F32, 0)).all()
-    # qlinear with a few activation rows runs one fused GEMV per row
+    # qlinear with two activation rows runs one fused GEMV per row (from three rows on: the matrix kernel)
     lib = pm._lib.load()
-    m = 3
+    m = 2
     xs = np.random.default_rng(6).standard_normal((m, k)).astype(np.float32)
     dw, dx, dy = pm.DeviceBuffer.from_host(wq), pm.DeviceBuffer.from_host(xs), pm.DeviceBuffer(4 * m * n)
     pm.check(lib.pmetal_hip_qlinear(t, dw.ptr, n, k, dx.ptr, pm.DTYPE_F32, m, dy.ptr, pm.DTYPE_F32, 0, None))
@@ -268,7 +268,7 @@ def test_gpu_q2k_q3k_gemv_unit_vectors_and_linear(oracle, t):
     for r in range(m):
         elem, norm = rel_errors(got[r], oracle.qmatvec(t, wq, n, k, xs[r]))
         assert elem <= 1e-3 and norm <= 1e-3
-    # the GEMM entry point takes these types too (through Q6_K re-blocking, tests/test_gpu_gemm.py) and agrees with the row loop
+    # the GEMM entry point takes these types too (tests/test_gpu_gemm.py) and agrees with the row loop
     pm.check(lib.pmetal_hip_qgemm(t, dw.ptr, n, k, dx.ptr, pm.DTYPE_F32, m, dy.ptr, pm.DTYPE_F32, 0, None))
     pm.check(lib.pmetal_hip_sync(None))
     assert np.allclose(dy.to_host(np.float32).reshape(m, n), got, rtol=0, atol=1e-3 * np.abs(got).max())  # f32 activations: f16-rounded in the GEMM

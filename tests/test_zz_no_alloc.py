@@ -66,7 +66,7 @@ def test_noalloc_rejects_what_does_not_fit():
     # 2048 activation rows of k = 8192 need 75 MB of converted activations: refused before anything is launched
     assert fn(Q4K, d.ptr, 14336, 8192, d.ptr, 1, 2048, d.ptr, 0, 0, None) == 7
     assert b"scratch" in lib.pmetal_hip_last_error_message()
-    assert fn(11, d.ptr, 256, 256, d.ptr, 1, 16, d.ptr, 0, 0, None) == 2  # Q3_K goes through re-blocking
+    assert fn(15, d.ptr, 256, 256, d.ptr, 1, 16, d.ptr, 0, 0, None) == 2  # Q8_K: activations only, no GEMM
     assert fn(Q4K, d.ptr, 256, 256, None, 1, 16, d.ptr, 0, 0, None) == 1
 
 
