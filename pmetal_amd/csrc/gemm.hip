@@ -1333,14 +1333,17 @@ __device__ __forceinline__ void small_store(const float4_t *out_tiles, int t0, i
     }
 }
 
-template <int NSB>
+template <int NSB, int FMT = 0>
 struct SmallRun {
-    static constexpr int kPieces = 16 * 9 * NSB;        // 16-byte pieces of a row tile's NSB super-blocks (144 bytes each)
-    static constexpr int kLoads = (kPieces + 63) / 64;  // per lane: 5 or 3
+    static constexpr int kPerSb = BlockFmt<FMT>::kBytes / 16;  // 16-byte pieces of a super-block: 9 (Q4_K) or 11 (Q5_K)
+    static constexpr int kPieces = 16 * kPerSb * NSB;          // ... of a row tile's NSB super-blocks
+    static constexpr int kLoads = (kPieces + 63) / 64;         // per lane: 5 or 3 (Q5_K: 6 or 3)
     u32x4 piece[kLoads];  // (a vector type: copies of it are loads and stores that stay in registers)
 };
 
-template <int ORDER, int NSB>
+// FMT 1: Q5_K -- eleven pieces per super-block (header, two of qh, eight of quants); a lane takes the qh bytes of its two
+// sub-blocks out of its stage as well and ors the fifth bits into the quant dwords as in the large kernel.
+template <int ORDER, int NSB, int FMT = 0>
 __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t *__restrict__ W, const uint4 *__restrict__ xs,
                                                                    const float *__restrict__ rowscale, void *__restrict__ yg, int M,
                                                                    int Mp, int N, int spr, int tiles, int tiles_per_wg, int ybf16,
@@ -1355,7 +1358,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t 
     const int rounds = (tiles_per_wg + kSmallDepth - 1) / kSmallDepth;
     float4_t *out_tiles = dyn;
     float4_t *keep = tiles_per_wg <= kSmallKeepTiles ? dyn + rounds * kSmallDepth * 64 : nullptr;
-    u32x4 *stage = reinterpret_cast<u32x4 *>(dyn + rounds * kSmallDepth * 64 * (keep ? 1 + nwaves : 1)) + wave * SmallRun<NSB>::kPieces;
+    u32x4 *stage = reinterpret_cast<u32x4 *>(dyn + rounds * kSmallDepth * 64 * (keep ? 1 + nwaves : 1)) + wave * SmallRun<NSB, FMT>::kPieces;
     int sbi[NSB];
     bool sbv[NSB];  // wave-uniform
 #pragma unroll
@@ -1381,20 +1384,21 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t 
     }
     const int t0 = (int)blockIdx.x * tiles_per_wg;
     const int t1 = t0 + tiles_per_wg < tiles ? t0 + tiles_per_wg : tiles;  // t1 > t0 by the launch geometry
+    constexpr int kPerSb = SmallRun<NSB, FMT>::kPerSb, kBlockBytes = BlockFmt<FMT>::kBytes, kQ0 = FMT ? 3 : 1;  // kQ0: first quant piece
     const uint32_t row_bytes = (uint32_t)spr * (uint32_t)kBlockBytes;
     // piece j of this lane: index lane + 64 j of the tile's 16 rows x 9 NSB pieces (a load past the last piece repeats it
     // and is dropped); a super-block past the end of the row is replaced by the row's first
-    constexpr int kLoads = SmallRun<NSB>::kLoads, kPieces = SmallRun<NSB>::kPieces;
+    constexpr int kLoads = SmallRun<NSB, FMT>::kLoads, kPieces = SmallRun<NSB, FMT>::kPieces;
     uint32_t piece_row[kLoads], piece_off[kLoads];
 #pragma unroll
     for (int j = 0; j < kLoads; j++) {
         int idx = lane + 64 * j;
         idx = idx < kPieces ? idx : kPieces - 1;
-        const int p = idx % (9 * NSB);
-        piece_row[j] = (uint32_t)(idx / (9 * NSB));
-        piece_off[j] = (uint32_t)(NSB == 2 && p >= 9 ? sbi[NSB - 1] : sbi[0]) * (uint32_t)kBlockBytes + 16u * (uint32_t)(p % 9);
+        const int p = idx % (kPerSb * NSB);
+        piece_row[j] = (uint32_t)(idx / (kPerSb * NSB));
+        piece_off[j] = (uint32_t)(NSB == 2 && p >= kPerSb ? sbi[NSB - 1] : sbi[0]) * (uint32_t)kBlockBytes + 16u * (uint32_t)(p % kPerSb);
     }
-    auto issue = [&](int ti, SmallRun<NSB> &w) __attribute__((always_inline)) {
+    auto issue = [&](int ti, SmallRun<NSB, FMT> &w) __attribute__((always_inline)) {
         int tile = t0 + ti;
         tile = tile < t1 ? tile : t1 - 1;  // past the end: the last tile again (loaded, not used)
 #pragma unroll
@@ -1404,8 +1408,8 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t 
             w.piece[j] = *reinterpret_cast<const u32x4 *>(W + ((uint32_t)n * row_bytes + piece_off[j]));  // the tensor is smaller than 4 GiB (checked by the launcher)
         }
     };
-    const u32x4 *mine = stage + nl * (9 * NSB);  // this lane's weight row in the stage
-    auto consume = [&](int ti, const SmallRun<NSB> &w) __attribute__((always_inline)) {
+    const u32x4 *mine = stage + nl * (kPerSb * NSB);  // this lane's weight row in the stage
+    auto consume = [&](int ti, const SmallRun<NSB, FMT> &w) __attribute__((always_inline)) {
         float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int j = 0; j < kLoads; j++)
@@ -1414,7 +1418,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t 
         // writes come after these reads
 #pragma unroll
         for (int i = 0; i < NSB; i++) {
-            const u32x4 hv = mine[9 * i], qav = mine[9 * i + 1 + 2 * kg], qbv = mine[9 * i + 2 + 2 * kg];
+            const u32x4 hv = mine[kPerSb * i], qav = mine[kPerSb * i + kQ0 + 2 * kg], qbv = mine[kPerSb * i + kQ0 + 1 + 2 * kg];
             const uint4 hdr = make_uint4(hv.x, hv.y, hv.z, hv.w);
             // scales and mins of sub-blocks 2 kg and 2 kg + 1 (6-bit fields, crates/pmetal-gguf/src/quantize.rs:844-855)
             const uint32_t sh = 16u * (uint32_t)(kg & 1);
@@ -1429,12 +1433,27 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t 
             const _Float16 o0 = (_Float16)(-1024.0f * (float)sc0), o1 = (_Float16)(-1024.0f * (float)sc1);  // exact: sc <= 63
             const half2_t sc2[2] = {half2_t{s0, s0}, half2_t{s1, s1}}, off2[2] = {half2_t{o0, o0}, half2_t{o1, o1}};
             const uint32_t qd[8] = {qav.x, qav.y, qav.z, qav.w, qbv.x, qbv.y, qbv.z, qbv.w};
+            // Q5_K: the fifth bits of k-step t.  GGML order: qh dword t (the same four bytes as quant dword t), bits 2 kg and
+            // 2 kg + 1 of every byte.  REF order: byte 4 (2 kg + t / 4) + t % 4 of qh, i.e. of the lane's two qh dwords.
+            uint32_t qh[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (FMT == 1) {
+                if (ORDER == 1) {
+                    const u32x4 ha = mine[kPerSb * i + 1], hb = mine[kPerSb * i + 2];
+                    const uint32_t h8[8] = {ha.x, ha.y, ha.z, ha.w, hb.x, hb.y, hb.z, hb.w};
+#pragma unroll
+                    for (int t = 0; t < 8; t++) qh[t] = h8[t] >> (2 * kg);
+                } else {
+                    const uint2 hp = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint8_t *>(mine + kPerSb * i + 1) + 8 * kg);
+#pragma unroll
+                    for (int t = 0; t < 8; t++) qh[t] = (t < 4 ? hp.x : hp.y) >> (8 * (t & 3));
+                }
+            }
             float4_t part = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int t = 0; t < 8; t++) {
                 Dq d;
 #pragma unroll
-                for (int c = 0; c < 4; c++) dq_chunk<ORDER>(c, t, qd[t], sc2, off2, d);
+                for (int c = 0; c < 4; c++) dq_chunk<ORDER, FMT>(c, t, qd[t], sc2, off2, d, qh[t]);
                 part = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i][t], d.value(), part, 0, 0, 0);
             }
             // (of a super-block past the end of the row only zeros may enter the sums, whatever bytes were loaded for it)
@@ -1450,7 +1469,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t 
         small_add_waves(red, keep, ti, wave, nwaves, lane, acc, out_tiles);
     };
     static_assert(kSmallDepth == 2, "the ring is written out as two tiles");
-    SmallRun<NSB> ring0, ring1;
+    SmallRun<NSB, FMT> ring0, ring1;
     issue(0, ring0);
     issue(1, ring1);
     // Whole rounds of two tiles, with nothing conditional around the loads, so that the outstanding loads are counted
@@ -1831,6 +1850,7 @@ static bool qgemm_small_applies(uint32_t type, int64_t m, int64_t n, int64_t k) 
     const int64_t spr = k / 256;
     if (m > kSmallMaxM || spr > kSmallMaxSpr * kSmallMaxRuns) return false;
     if (type == kTypeQ4K) return (uint64_t)n * (uint64_t)spr * 144u < (1ull << 32);
+    if (type == kTypeQ5K) return (uint64_t)n * (uint64_t)spr * 176u < (1ull << 32);
     if (type == kTypeQ8_0) return (uint64_t)n * (uint64_t)spr * 272u < (1ull << 32);
     if (type == kTypeQ6K) return (uint64_t)n * (uint64_t)spr * 210u < (1ull << 32);
     return false;
@@ -1885,7 +1905,7 @@ GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k, uint32_t type) {
     // at most 16 activation rows against long rows: runs of 16 super-blocks (the fused kernels' K split; the large kernel
     // takes the same split when a shape falls back to it)
     // (a type without such kernels keeps the split chosen above)
-    if (m <= kSmallMaxM && spr > kSmallMaxSpr && (type == kTypeQ4K || type == kTypeQ6K || type == kTypeQ8_0)) p.chunk = kSmallMaxSpr, p.splits = (int)((spr + kSmallMaxSpr - 1) / kSmallMaxSpr);
+    if (m <= kSmallMaxM && spr > kSmallMaxSpr && (type == kTypeQ4K || type == kTypeQ5K || type == kTypeQ6K || type == kTypeQ8_0)) p.chunk = kSmallMaxSpr, p.splits = (int)((spr + kSmallMaxSpr - 1) / kSmallMaxSpr);
     return p;
 }
 
@@ -2020,16 +2040,21 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
         // (a workgroup of few tiles also keeps every wave's partial tile of each until the end)
         const size_t lds = (size_t)((tiles_per_wg + kSmallDepth - 1) / kSmallDepth * kSmallDepth) * 1024 *
                            (tiles_per_wg <= kSmallKeepTiles ? 1 + nwaves : 1);
-#define PMH_SMALL(O, S)                                                                                                          \
+#define PMH_SMALL_F(O, S, F)                                                                                                     \
     do {                                                                                                                         \
-        const size_t lds4 = lds + (size_t)nwaves * SmallRun<S>::kPieces * 16; /* the waves' stages behind the finished tiles */ \
+        const size_t lds4 = lds + (size_t)nwaves * SmallRun<S, F>::kPieces * 16; /* the waves' stages behind the finished tiles */ \
         if (lds4 > 48 * 1024) {                                                                                                   \
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_qgemm_small<O, S>), hipFuncAttributeMaxDynamicSharedMemorySize, \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_qgemm_small<O, S, F>), hipFuncAttributeMaxDynamicSharedMemorySize, \
                                     (int)lds4);                                                                                   \
             if (e != hipSuccess) return e;                                                                                       \
         }                                                                                                                        \
-        hipLaunchKernelGGL((k_qgemm_small<O, S>), grid, block, lds4, s, w, xs, rowscale, y, (int)m, (int)p.mp, (int)n, spr, tiles, \
+        hipLaunchKernelGGL((k_qgemm_small<O, S, F>), grid, block, lds4, s, w, xs, rowscale, y, (int)m, (int)p.mp, (int)n, spr, tiles, \
                            tiles_per_wg, ybf ? 1 : 0, part_out);                                                                           \
+    } while (0)
+#define PMH_SMALL(O, S)         \
+    do {                        \
+        if (q5) PMH_SMALL_F(O, S, 1); \
+        else PMH_SMALL_F(O, S, 0);    \
     } while (0)
         if (q6) {
             const bool any = spr % 8 != 0;  // rows that do not start on 16-byte boundaries
@@ -2075,6 +2100,7 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
             else PMH_SMALL(1, 1);
         }
 #undef PMH_SMALL
+#undef PMH_SMALL_F
         e = hipGetLastError();
         if (e != hipSuccess || runs == 1) return e;
     } else {
