@@ -957,7 +957,7 @@ int32_t pmetal_hip_qgemm_batch(const pmetal_hip_gemm_desc *descs, size_t count, 
     int have = -1, have_mp = -1;
     for (size_t i = 0; i < count; i++) {
         const pmetal_hip_gemm_desc &d = descs[i];
-        const int want = layout(d), want_mp = pmh::qgemm_plan(m, d.n, k).mp;
+        const int want = layout(d), want_mp = pmh::qgemm_plan(m, d.n, k, d.ggml_type).mp;
         hipError_t e = pmh::launch_qgemm(d.ggml_type, d.w_dev, d.n, k, x, x_dtype, m, d.y_dev, d.y_dtype, d.order, ws, (hipStream_t)stream,
                                          want == have && want_mp == have_mp);
         if (e == hipErrorNotSupported) return fail(PMETAL_HIP_ERR_UNSUPPORTED_TYPE, "qgemm: configuration not supported");
