@@ -54,6 +54,27 @@ def test_quantize_edge_cases_bit_exact(oracle, t):
         assert np.array_equal(got, want), f"{name}: {first_mismatch(got, want, BLOCK[t])}"
 
 
+def test_quantize_q4k_corner_cases_inside_a_large_tensor(oracle):
+    """The corner cases above, Gaussian data with outliers and runs of constants, laid end to end to 32768 + 5
+    super-blocks and a ragged tail: sub-blocks that need one, two or all five passes of the search side by side in one
+    wave, in a tensor of many workgroups."""
+    rng = np.random.default_rng(4)
+    parts, total, want_n = [], 0, (32768 + 5) * 256 + 77
+    cases = list(edge_inputs(256).values())
+    i = 0
+    while total < want_n:
+        c = cases[i % len(cases)] if i % 3 == 0 else weights(500 + i, int(rng.integers(1, 40)) * 1024 + int(rng.integers(0, 256)), outliers=1e-3 * (i % 2))
+        if i % 7 == 3:
+            c = np.full(int(rng.integers(1, 9)) * 32, np.float32(rng.standard_normal()), np.float32)
+        parts.append(c)
+        total += c.size
+        i += 1
+    x = np.concatenate(parts)[:want_n].astype(np.float32)
+    want = oracle.quantize(Q4K, x)
+    got = gpu_quantize_dev(Q4K, x)
+    assert np.array_equal(got, want), first_mismatch(got, want, BLOCK[Q4K])
+
+
 @pytest.mark.parametrize("t", [Q8_0, Q4K, Q6K])
 def test_quantize_empty(oracle, t):
     assert gpu_quantize_dev(t, np.zeros(0, np.float32)).size == 0
