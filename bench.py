@@ -501,8 +501,9 @@ def bench_gemm(args, m, n, k, t=Q4K):
         "value": tflops, "ms_per_step": wall_ms / args.steps, "event_ms_per_step": ev_ms / args.steps,
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / BF16_PEAK_TFLOPS, 4), "traffic": None,
-                     "kernel": ({Q4K: "k_qgemm_small", 13: "k_qgemm_small<FMT = 1>", Q6K: "k_qgemm_small_q6", Q8_0: "k_qgemm_small_q8"}[t] + " (+ k_prep_rw)"
-                                if m <= 16 and t in (Q4K, 13, Q6K, Q8_0) else
+                     "kernel": ({Q4K: "k_qgemm_small", 13: "k_qgemm_small<FMT = 1>", Q6K: "k_qgemm_small_q6", Q8_0: "k_qgemm_small_q8",
+                                 11: "k_qgemm_small16<Q3_K>", 10: "k_qgemm_small16<Q2_K>"}[t] + " (+ k_prep_rw)"
+                                if m <= 16 else
                                 {Q4K: "k_qgemm_rw", 13: "k_qgemm_rw<FMT = 1>", Q6K: "k_qgemm_rw_q6", Q8_0: "k_qgemm_rw_q8", 11: "k_qgemm_rw16<Q3_K>", 10: "k_qgemm_rw16<Q2_K>"}[t]
                                 + " (+ k_prep_rw, k_rw_reduce when K is split)"),
                      "flops_per_launch": flops, "us_per_launch": round(us, 3)},
@@ -731,8 +732,9 @@ WORKLOADS["gemm_q8_0_m16"] = dict(kind="gemm", m=16, n=14336, k=4096, metric="Q8
                                   unit="TFLOP/s", dtype="f16", type=Q8_0)
 WORKLOADS["gemm_q6k_m16"] = dict(kind="gemm", m=16, n=14336, k=4096, metric="Q6_K GEMM TFLOPS @M=16,K=4096,N=14336",
                                  unit="TFLOP/s", dtype="f16", type=Q6K)
-WORKLOADS["gemm_q5k_m16"] = dict(kind="gemm", m=16, n=14336, k=4096, metric="Q5_K GEMM TFLOPS @M=16,K=4096,N=14336",
-                                 unit="TFLOP/s", dtype="f16", type=13)
+for _name, _t in (("q5k", 13), ("q3k", 11), ("q2k", 10)):
+    WORKLOADS[f"gemm_{_name}_m16"] = dict(kind="gemm", m=16, n=14336, k=4096, unit="TFLOP/s", dtype="f16", type=_t,
+                                          metric=f"{_name.upper().replace('K', '_K')} GEMM TFLOPS @M=16,K=4096,N=14336")
 for _name, _t in (("q5k", 13), ("q3k", 11), ("q2k", 10)):  # (their own kernels; the form re-blocked into Q6_K is timed beside them)
     WORKLOADS[f"gemm_{_name}_m512"] = dict(kind="gemm", m=512, n=14336, k=4096, unit="TFLOP/s", dtype="f16", type=_t,
                                            metric=f"{_name.upper().replace('K', '_K')} GEMM TFLOPS (nominal flops) @M=512,K=4096,N=14336")

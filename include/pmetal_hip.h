@@ -170,8 +170,8 @@ int32_t pmetal_hip_dequantize_dev(uint32_t ggml_type, const uint8_t *src_dev, si
  * Types: every type has both kernels (the Q5_K GEMM is the Q4_K kernel with the fifth bit of every quant taken from the
  * block's qh bytes; Q3_K and Q2_K share a kernel for sixteen 16-element sub-blocks).  The GEMV of Q5_K, Q3_K and Q2_K takes
  * k <= 32768 and a tensor below 4 GiB, any number of rows; beyond that qgemv fails with SHAPE_TOO_LARGE and qlinear uses the
- * GEMM.  Q4_K, Q5_K, Q6_K and Q8_0 have a second GEMM kernel for m <= 16 that reads the weights once; qlinear runs two
- * activation rows of Q3_K and Q2_K (and of a Q5_K weight of at most 2^23 elements) as two GEMVs, three or more as one GEMM.
+ * GEMM.  Every type has a second GEMM kernel for m <= 16 that reads the weights once; qlinear runs two activation rows of a
+ * Q5_K, Q3_K or Q2_K weight of at most 2^23 elements as two GEMVs, and a larger weight or more rows as one GEMM.
  * y/Y: f32 (qgemv) or f32/bf16 (qgemm), row-major [m, n].
  * qgemm keeps scratch memory (converted activations, partial tiles) inside the library, one
  * buffer per calling thread, device and stream; it grows on demand, which synchronises that
@@ -200,7 +200,7 @@ int32_t pmetal_hip_qgemm_noalloc(uint32_t ggml_type, const uint8_t *w_dev, int64
                                  void *stream);
 /* Dispatch by m: m == 1 -> qgemv (f32 output only), otherwise qgemm (k must be a multiple of 256).  A Q8_0
  * row that is only a multiple of 32 runs one GEMV per activation row when m > 1 (f32 output only), and so do
- * Q3_K, Q2_K and small Q5_K weights for m = 2, with f32 output. */
+ * Q5_K, Q3_K and Q2_K weights of at most 2^23 elements for m = 2, with f32 output. */
 int32_t pmetal_hip_qlinear(uint32_t ggml_type, const uint8_t *w_dev, int64_t n, int64_t k, const void *x_dev,
                            uint32_t x_dtype, int64_t m, void *y_dev, uint32_t y_dtype, uint32_t order,
                            void *stream);

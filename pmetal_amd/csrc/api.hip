@@ -703,7 +703,7 @@ int32_t codec_pipelined(bool quantize, uint32_t t, float *plain, uint8_t *packed
 extern "C" {
 
 // ---- quantized linear ----
-constexpr int64_t kRowLoopMax = 2;  // activation rows up to which qlinear sends Q3_K / Q2_K (and a small Q5_K weight) through the GEMV, row by row
+constexpr int64_t kRowLoopMax = 2;  // activation rows up to which qlinear sends a small Q5_K / Q3_K / Q2_K weight through the GEMV, row by row
 // types with a fused GEMV but no GEMM kernel of their own (their GEMM goes through Q6_K, see qgemm_reblocked)
 static bool gemv_only_type(uint32_t t) { return t == PMETAL_GGML_TYPE_Q5K || t == PMETAL_GGML_TYPE_Q3K || t == PMETAL_GGML_TYPE_Q2K; }
 // (These got their GEMV kernels first and reached the matrix cores through re-blocking into Q6_K; each has a matrix kernel of
@@ -1030,11 +1030,10 @@ int32_t pmetal_hip_qlinear(uint32_t t, const uint8_t *w, int64_t n, int64_t k, c
         return fail(PMETAL_HIP_ERR_INVALID_SHAPE, "qlinear: a Q8_0 row of k=%lld (not a multiple of 256) runs through the GEMV, whose output is f32 only",
                     (long long)k);
     const bool q4k_pair = t == PMETAL_GGML_TYPE_Q4K && m == 2;
-    // Q3_K and Q2_K have no short-batch kernel: two rows are two GEMVs, three rows are one GEMM.  Q5_K has one, and two rows
-    // through it beat two GEMVs (17.3 against 23.1 us at 14336 x 4096, 11.6 against 12.9 at 6144 x 4096) except on a small
-    // weight, where its two launches cost more than they save (10.7 against 7.5 us at 1024 x 4096).
-    const bool q5k_small = t == PMETAL_GGML_TYPE_Q5K && n * k > (int64_t(1) << 23);
-    const bool row_loop_type = gemv_only_type(t) && m <= kRowLoopMax && !q5k_small;
+    // Two rows of Q5_K, Q3_K or Q2_K through the short-batch GEMM beat two GEMVs (Q5_K: 17.3 against 23.1 us at 14336 x 4096,
+    // 11.6 against 12.9 at 6144 x 4096; Q2_K 14.6 against 19.2, Q3_K 17.1 against 22) except on a small weight, where the
+    // GEMM's two launches cost more than they save (Q5_K: 10.7 against 7.5 us at 1024 x 4096).
+    const bool row_loop_type = gemv_only_type(t) && m <= kRowLoopMax && n * k <= (int64_t(1) << 23);
     if ((q8_ragged || q4k_pair || row_loop_type) && y_dtype == PMETAL_HIP_DTYPE_F32 && m > 1 && n > 0 && k > 0 && x && y) {
         // The fused GEMM walks k in steps of 256, and a Q8_0 row may be any multiple of 32: one fused GEMV per activation row
         // then, back to back on the stream.  Two Q4_K rows are two GEMVs: 13.7 against 16.1 us at 14336 x 4096

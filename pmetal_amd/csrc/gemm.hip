@@ -1836,13 +1836,196 @@ constexpr size_t rw_lds_bytes() {
     return stages > tile_lds_bytes<MB, NW>() ? stages : tile_lds_bytes<MB, NW>();
 }
 
+// ------------------------------------------------------------------------------------------------
+// The same for Q3_K and Q2_K (sixteen 16-element sub-blocks).  Lane (r, kg) of v_mfma_f32_16x16x32_f16 stands where lane
+// (n, g) of half h stands in the large kernel, with h = kg / 2 and g = kg % 2: the 16 bytes 16 kg .. of the 64 quant bytes
+// of weight row r, whose dword t / 2 gives k-step t its eight values, against the pre-pass's item (2 sb + h, 2 t + g); four
+// scales per lane; the sub-block sums of the activations (items 16 + g and 18 + g of the half) against the negated min
+// coefficients in two further matrix instructions.  Blocks are 84 / 110 bytes and a lane needs few of them, so every lane
+// loads its own: Q2_K rows start at multiples of four bytes, the quant piece, the scale bytes of its half and the d / dmin
+// dword are plain loads; Q3_K blocks start at any even address, so a lane loads the aligned dwords that cover its pieces
+// (quants and hmask: five; scales and d: four -- every one of them holds bytes of the block, none lies wholly past it) and
+// shifts them by the block's 0 or 16 bits.  Ring, reduction over the waves and epilogue as above.
+// ------------------------------------------------------------------------------------------------
+struct __attribute__((packed, aligned(4))) u32x4_a4 {  // sixteen bytes at a 4-byte aligned address
+    uint32_t x, y, z, w;
+};
+struct __attribute__((packed, aligned(4))) u32x2_a4 {
+    uint32_t x, y;
+};
+__device__ __forceinline__ u32x4 load16_a4(const uint8_t *p) {
+    const u32x4_a4 v = *reinterpret_cast<const u32x4_a4 *>(p);
+    return u32x4{v.x, v.y, v.z, v.w};
+}
+
+template <int FMT, int NSB>
+struct SmallRun16 {  // what a lane holds of a row tile
+    u32x4 q[NSB];          // quant piece (Q3_K: from the dword boundary below it)
+    uint32_t qx[NSB];      // Q3_K: the dword behind it
+    u32x4 hm[NSB];         // Q3_K: hmask bytes 16 g ..
+    uint32_t hmx[NSB];
+    u32x4 sc[NSB];         // Q3_K: scales and d; Q2_K: x, y = scale bytes 8 h .., z = d | dmin << 16
+};
+
+template <int FMT, int NSB>
+__global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small16(const uint8_t *__restrict__ W, const uint4 *__restrict__ xs,
+                                                                     const float *__restrict__ rowscale, void *__restrict__ yg, int M,
+                                                                     int Mp, int N, int spr, int tiles, int tiles_per_wg, int ybf16,
+                                                                     float *__restrict__ partial) {
+    using B = Block16<FMT>;
+    __shared__ float4_t red[2][kSmallWaves][64];
+    extern __shared__ float4_t dyn[];  // out_tiles [tiles_per_wg rounded up to whole rounds][64], then the kept partial tiles
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int nwaves = (int)(blockDim.x >> 6);
+    const int nl = lane & 15, kg = lane >> 4;
+    const uint32_t h = (uint32_t)(kg >> 1), g = (uint32_t)(kg & 1);
+    const int rounds = (tiles_per_wg + kSmallDepth - 1) / kSmallDepth;
+    float4_t *out_tiles = dyn;
+    float4_t *keep = tiles_per_wg <= kSmallKeepTiles ? dyn + rounds * kSmallDepth * 64 : nullptr;
+    int sbi[NSB];
+    bool sbv[NSB];  // wave-uniform
+#pragma unroll
+    for (int i = 0; i < NSB; i++) {
+        sbi[i] = (int)blockIdx.y * (NSB * nwaves) + NSB * wave + i;
+        sbv[i] = sbi[i] < spr;
+        sbi[i] = sbv[i] ? sbi[i] : 0;
+    }
+    half8_t af[NSB][8], asum[NSB][2];
+#pragma unroll
+    for (int i = 0; i < NSB; i++) {
+        const uint4 *base = xs + (size_t)((2 * sbi[i] + (int)h) * kGroups16) * Mp + nl;
+#pragma unroll
+        for (int t = 0; t < 8; t++) af[i][t] = __builtin_bit_cast(half8_t, base[(size_t)(2 * t + (int)g) * Mp]);
+        asum[i][0] = __builtin_bit_cast(half8_t, base[(size_t)(16 + (int)g) * Mp]);
+        asum[i][1] = __builtin_bit_cast(half8_t, base[(size_t)(18 + (int)g) * Mp]);
+        if (!sbv[i]) {  // a super-block past the end of the row multiplies zeros (no branch in the streaming loop)
+            const half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int t = 0; t < 8; t++) af[i][t] = z;
+            asum[i][0] = z, asum[i][1] = z;
+        }
+    }
+    const int t0 = (int)blockIdx.x * tiles_per_wg;
+    const int t1 = t0 + tiles_per_wg < tiles ? t0 + tiles_per_wg : tiles;  // t1 > t0 by the launch geometry
+    const uint32_t row_bytes = (uint32_t)spr * (uint32_t)B::kBytes;
+    auto block_at = [&](int ti, int i) -> uint32_t {  // byte offset of super-block sbi[i] of this lane's row of tile ti (the tensor is smaller than 4 GiB)
+        int tile = t0 + ti;
+        tile = tile < t1 ? tile : t1 - 1;  // past the end: the last tile again (loaded, not used)
+        int n = tile * 16 + nl;
+        n = n < N ? n : N - 1;
+        return (uint32_t)n * row_bytes + (uint32_t)sbi[i] * (uint32_t)B::kBytes;
+    };
+    auto issue = [&](int ti, SmallRun16<FMT, NSB> &w) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NSB; i++) {
+            const uint32_t blk = block_at(ti, i);
+            if (FMT == 3) {
+                w.q[i] = load16_a4(W + (blk + 16u + 16u * (uint32_t)kg));
+                const u32x2_a4 s2 = *reinterpret_cast<const u32x2_a4 *>(W + (blk + 8u * h));
+                const uint32_t dd = *reinterpret_cast<const uint32_t *>(W + (blk + 80u));
+                w.sc[i] = u32x4{s2.x, s2.y, dd, 0u};
+            } else {
+                const uint32_t lo = blk & ~3u;  // (the pieces' offsets inside the block are multiples of four)
+                w.q[i] = load16_a4(W + (lo + 32u + 16u * (uint32_t)kg));
+                w.qx[i] = *reinterpret_cast<const uint32_t *>(W + (lo + 48u + 16u * (uint32_t)kg));
+                w.hm[i] = load16_a4(W + (lo + 16u * g));
+                w.hmx[i] = *reinterpret_cast<const uint32_t *>(W + (lo + 16u + 16u * g));
+                w.sc[i] = load16_a4(W + (lo + 96u));
+            }
+        }
+    };
+    auto consume = [&](int ti, const SmallRun16<FMT, NSB> &w) __attribute__((always_inline)) {
+        float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int i = 0; i < NSB; i++) {
+            uint32_t qd[4], hm[4] = {0, 0, 0, 0}, s8[3], dbits;
+            if (FMT == 3) {
+                qd[0] = w.q[i][0], qd[1] = w.q[i][1], qd[2] = w.q[i][2], qd[3] = w.q[i][3];
+                s8[0] = w.sc[i][0], s8[1] = w.sc[i][1], s8[2] = 0;
+                dbits = w.sc[i][2];  // d | dmin << 16
+            } else {
+                const uint32_t sh = (block_at(ti, i) & 2u) * 8u;  // the block starts two bytes past a dword boundary, or on one
+                qd[0] = __builtin_amdgcn_alignbit(w.q[i][1], w.q[i][0], sh), qd[1] = __builtin_amdgcn_alignbit(w.q[i][2], w.q[i][1], sh);
+                qd[2] = __builtin_amdgcn_alignbit(w.q[i][3], w.q[i][2], sh), qd[3] = __builtin_amdgcn_alignbit(w.qx[i], w.q[i][3], sh);
+                hm[0] = __builtin_amdgcn_alignbit(w.hm[i][1], w.hm[i][0], sh), hm[1] = __builtin_amdgcn_alignbit(w.hm[i][2], w.hm[i][1], sh);
+                hm[2] = __builtin_amdgcn_alignbit(w.hm[i][3], w.hm[i][2], sh), hm[3] = __builtin_amdgcn_alignbit(w.hmx[i], w.hm[i][3], sh);
+                s8[0] = __builtin_amdgcn_alignbit(w.sc[i][1], w.sc[i][0], sh), s8[1] = __builtin_amdgcn_alignbit(w.sc[i][2], w.sc[i][1], sh);
+                s8[2] = __builtin_amdgcn_alignbit(w.sc[i][3], w.sc[i][2], sh);
+                dbits = (w.sc[i][3] >> sh) & 0xFFFFu;
+            }
+            // (of a super-block past the end of the row only zeros may enter the sums, whatever bytes were loaded for it)
+            const float d = sbv[i] ? f16_bits_to_f32(dbits & 0xFFFFu) : 0.0f;
+            const float dmin = sbv[i] ? f16_bits_to_f32(dbits >> 16) : 0.0f;
+            // scales (and mins) of the lane's four sub-blocks j = 8 h + 4 sp + 2 lh + g, index 2 sp + lh
+            half2_t sc2[4], off2[4];
+            float nm[4];
+#pragma unroll
+            for (int sp = 0; sp < 2; sp++)
+#pragma unroll
+                for (int lh = 0; lh < 2; lh++) {
+                    float scf;
+                    if (FMT == 3) {  // s8[sp]: bytes 8 h + 4 sp .. of the sixteen; low nibble scale, high nibble min
+                        const uint32_t b = (s8[sp] >> (8u * g + 16u * lh)) & 0xFFu;
+                        scf = (float)(b & 15u);
+                        nm[2 * sp + lh] = -(dmin * (float)(b >> 4));
+                    } else {
+                        const uint32_t lo4 = (s8[sp] >> (8u * g + 16u * lh + 4u * h)) & 15u;
+                        const uint32_t hi2 = (s8[2] >> (8u * g + 16u * lh + 2u * (2u * h + sp))) & 3u;
+                        scf = (float)((int)(lo4 | (hi2 << 4)) - 32);
+                        nm[2 * sp + lh] = -(d * (4.0f * scf));
+                    }
+                    const _Float16 s16 = (_Float16)scf, o16 = (_Float16)(-1024.0f * scf);  // exact: |sc| <= 32
+                    sc2[2 * sp + lh] = half2_t{s16, s16}, off2[2 * sp + lh] = half2_t{o16, o16};
+                }
+            float4_t part = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                const int dw = t >> 1, sp = t & 1;
+                uint32_t lo = (qd[dw] >> (4 * sp)) & 0x03030303u, hi = (qd[dw] >> (4 * sp + 2)) & 0x03030303u;
+                if (FMT == 2) {
+                    const uint32_t m = hm[dw] >> (4u * h + 2u * sp);
+                    lo |= (m & 0x01010101u) << 2, hi |= (m & 0x02020202u) << 1;
+                }
+                const half2_t r0 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, lo, 0x04010400u)), sc2[2 * sp], off2[2 * sp]);
+                const half2_t r1 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, lo, 0x04030402u)), sc2[2 * sp], off2[2 * sp]);
+                const half2_t r2 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, hi, 0x04010400u)), sc2[2 * sp + 1], off2[2 * sp + 1]);
+                const half2_t r3 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, hi, 0x04030402u)), sc2[2 * sp + 1], off2[2 * sp + 1]);
+                const half8_t b = half8_t{r0[0], r0[1], r1[0], r1[1], r2[0], r2[1], r3[0], r3[1]};
+                part = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i][t], b, part, 0, 0, 0);
+            }
+#pragma unroll
+            for (int sp = 0; sp < 2; sp++) {
+                const _Float16 h0 = (_Float16)nm[2 * sp], h1 = (_Float16)nm[2 * sp + 1];
+                const _Float16 l0 = (_Float16)(nm[2 * sp] - (float)h0), l1 = (_Float16)(nm[2 * sp + 1] - (float)h1);
+                const half8_t br = half8_t{h0, h0, l0, l0, h1, h1, l1, l1};
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(asum[i][sp], br, acc, 0, 0, 0);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[r] = __builtin_fmaf(d, part[r], acc[r]);
+        }
+        small_add_waves(red, keep, ti, wave, nwaves, lane, acc, out_tiles);
+    };
+    static_assert(kSmallDepth == 2, "the ring is written out as two tiles");
+    SmallRun16<FMT, NSB> ring0, ring1;
+    issue(0, ring0);
+    issue(1, ring1);
+    for (int rd = 0; rd < rounds; rd++) {  // whole rounds of two tiles, nothing conditional around the loads
+        consume(2 * rd, ring0);
+        issue(2 * rd + 2, ring0);
+        consume(2 * rd + 1, ring1);
+        issue(2 * rd + 3, ring1);
+    }
+    small_add_kept(keep, rounds * kSmallDepth, wave, nwaves, lane, out_tiles);
+    small_store(out_tiles, t0, t1, M, Mp, N, rowscale, yg, ybf16, partial);
+}
+
 }  // namespace
 
 namespace pmh {
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
-// The fused kernel for few activation rows takes Q4_K with m <= 16 and rows of at most 16 super-blocks (k <= 4096).
 // The fused kernels for at most 16 activation rows.  Rows of more than 16 super-blocks are cut into runs of 16, one
 // workgroup row of the grid each, whose partial tiles k_rw_reduce adds (qgemm_plan sets splits and chunk to match).
 constexpr int kSmallMaxRuns = 8;  // k <= 32768
@@ -1853,6 +2036,8 @@ static bool qgemm_small_applies(uint32_t type, int64_t m, int64_t n, int64_t k) 
     if (type == kTypeQ5K) return (uint64_t)n * (uint64_t)spr * 176u < (1ull << 32);
     if (type == kTypeQ8_0) return (uint64_t)n * (uint64_t)spr * 272u < (1ull << 32);
     if (type == kTypeQ6K) return (uint64_t)n * (uint64_t)spr * 210u < (1ull << 32);
+    if (type == kTypeQ3K) return (uint64_t)n * (uint64_t)spr * 110u < (1ull << 32);
+    if (type == kTypeQ2K) return (uint64_t)n * (uint64_t)spr * 84u < (1ull << 32);
     return false;
 }
 
@@ -1904,8 +2089,7 @@ GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k, uint32_t type) {
     }
     // at most 16 activation rows against long rows: runs of 16 super-blocks (the fused kernels' K split; the large kernel
     // takes the same split when a shape falls back to it)
-    // (a type without such kernels keeps the split chosen above)
-    if (m <= kSmallMaxM && spr > kSmallMaxSpr && (type == kTypeQ4K || type == kTypeQ5K || type == kTypeQ6K || type == kTypeQ8_0)) p.chunk = kSmallMaxSpr, p.splits = (int)((spr + kSmallMaxSpr - 1) / kSmallMaxSpr);
+    if (m <= kSmallMaxM && spr > kSmallMaxSpr) p.chunk = kSmallMaxSpr, p.splits = (int)((spr + kSmallMaxSpr - 1) / kSmallMaxSpr);
     return p;
 }
 
@@ -2056,7 +2240,26 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
         if (q5) PMH_SMALL_F(O, S, 1); \
         else PMH_SMALL_F(O, S, 0);    \
     } while (0)
-        if (q6) {
+        if (q23) {
+#define PMH_SMALL16(F, S)                                                                                                        \
+    do {                                                                                                                         \
+        if (lds > 48 * 1024) {                                                                                                   \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_qgemm_small16<F, S>), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                    (int)lds);                                                                                   \
+            if (e != hipSuccess) return e;                                                                                       \
+        }                                                                                                                        \
+        hipLaunchKernelGGL((k_qgemm_small16<F, S>), grid, block, lds, s, w, xs, rowscale, y, (int)m, (int)p.mp, (int)n, spr, tiles, \
+                           tiles_per_wg, ybf ? 1 : 0, part_out);                                                                 \
+    } while (0)
+            if (type == kTypeQ2K) {
+                if (nsb == 2) PMH_SMALL16(3, 2);
+                else PMH_SMALL16(3, 1);
+            } else {
+                if (nsb == 2) PMH_SMALL16(2, 2);
+                else PMH_SMALL16(2, 1);
+            }
+#undef PMH_SMALL16
+        } else if (q6) {
             const bool any = spr % 8 != 0;  // rows that do not start on 16-byte boundaries
             const size_t stage = (size_t)(nsb == 2 ? SmallQ6<2, true>::kStageDwords : SmallQ6<1>::kStageDwords) * 4;
             const size_t lds6 = lds + (size_t)nwaves * stage;  // the waves' stages behind the finished tiles

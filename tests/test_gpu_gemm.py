@@ -383,11 +383,11 @@ def test_qgemm_q5k_q3k_q2k_unit_activations_pick_single_weights(oracle, t, order
 
 @pytest.mark.parametrize("t", sorted(REBLOCKED))
 def test_qlinear_q5k_q3k_q2k_dispatch(oracle, t):
-    """qlinear: two activation rows one fused GEMV each (Q5_K: on a weight of at most 2^23 elements; a larger one takes
-    its short-batch GEMM), above that the GEMM; both agree with the oracle; a second, smaller call reuses the scratch
+    """qlinear: two activation rows one fused GEMV each on a weight of at most 2^23 elements (a larger one takes its
+    short-batch GEMM), above that the GEMM; both agree with the oracle; a second, smaller call reuses the scratch
     buffer."""
     lib = _lib.load()
-    if t == 13:
+    if True:
         n, k = 2080, 4096  # above 2^23 elements: two rows are one GEMM
         wq = oracle.quantize(t, weights(t, n * k, outliers=1e-3))
         dw = pm.DeviceBuffer.from_host(wq)
@@ -508,7 +508,7 @@ def test_qgemm_batch_wide_and_narrow_weights_share_x(oracle, t, m):
             assert np.array_equal(y_one[i], y_bat[j].to_host(np.uint8)), (m, first, ns[i])
 
 
-@pytest.mark.parametrize("t", [Q4K, Q6K, Q8_0, 13])
+@pytest.mark.parametrize("t", [Q4K, Q6K, Q8_0, 13, 11, 10])
 @pytest.mark.parametrize("m", [1, 2, 5, 9, 16])
 @pytest.mark.parametrize("n,k", [(700, 2048), (333, 4096), (16, 2048), (4099, 4096), (40, 1024),
                                  # rows of more than 16 super-blocks: runs of 16, partial tiles added in a second kernel
@@ -521,7 +521,7 @@ def test_qgemm_short_batches(oracle, t, m, n, k):
     tiles, one full tile, more tiles than workgroups take in one round; bf16 and f32 activations, f32 and bf16 outputs;
     unit activations that pick single weights out of the matrix."""
     rng = np.random.default_rng(1000 * t + 31 * m + n + k)
-    block = {Q4K: 144, Q6K: 210, Q8_0: 34, 13: 176}[t]
+    block = {Q4K: 144, Q6K: 210, Q8_0: 34, 13: 176, 11: 110, 10: 84}[t]
     per = 32 if t == Q8_0 else 256
     raw = rng.integers(0, 256, size=(n * (k // per), block), dtype=np.uint8)
     half = np.frombuffer(np.array([0.01, 0.02], np.float16).tobytes(), np.uint8)
@@ -529,6 +529,10 @@ def test_qgemm_short_batches(oracle, t, m, n, k):
         raw[:, 0:4] = half
     elif t == Q6K:
         raw[:, 208:210] = half[:2]
+    elif t == 11:
+        raw[:, 108:110] = half[:2]
+    elif t == 10:
+        raw[:, 80:84] = half
     else:
         raw[:, 0:2] = (rng.uniform(0.5, 2.0, raw.shape[0]) * 0.01 * rng.choice([-1.0, 1.0], raw.shape[0])).astype(np.float16).view(np.uint8).reshape(-1, 2)
     raw = raw.reshape(-1)
@@ -558,13 +562,13 @@ def test_qgemm_short_batches(oracle, t, m, n, k):
         assert np.allclose(got[r], w[:, c], rtol=1e-6, atol=0), (r, c)
 
 
-@pytest.mark.parametrize("t", [Q4K, Q6K, Q8_0, 13])
+@pytest.mark.parametrize("t", [Q4K, Q6K, Q8_0, 13, 11, 10])
 def test_qgemm_short_batch_very_tall_weight(oracle, t):
     """300 000 weight rows against 9 activation rows: more row tiles per workgroup than its LDS holds finished tiles for,
     so the grid has more workgroups than compute units.  The first 2000 and the last 3000 rows against the oracle."""
     n, k, m = 300000, 2048, 9
     rng = np.random.default_rng(t)
-    block = {Q4K: 144, Q6K: 210, Q8_0: 34, 13: 176}[t]
+    block = {Q4K: 144, Q6K: 210, Q8_0: 34, 13: 176, 11: 110, 10: 84}[t]
     per = 32 if t == Q8_0 else 256
     raw = rng.integers(0, 256, size=(n * (k // per), block), dtype=np.uint8)
     half = np.frombuffer(np.array([0.01, 0.02], np.float16).tobytes(), np.uint8)
@@ -572,6 +576,10 @@ def test_qgemm_short_batch_very_tall_weight(oracle, t):
         raw[:, 0:4] = half
     elif t == Q6K:
         raw[:, 208:210] = half[:2]
+    elif t == 11:
+        raw[:, 108:110] = half[:2]
+    elif t == 10:
+        raw[:, 80:84] = half
     else:
         raw[:, 0:2] = half[:2]
     x = rng.standard_normal((m, k)).astype(np.float32)
