@@ -1,6 +1,7 @@
 /*
  * pmetal_hip.h -- C ABI of libpmetal_hip.so: PMetal's GGUF block-quantized weight
- * path (Q8_0, Q4_K, Q6_K) as hand-written HIP kernels for MI355X (gfx950).
+ * path (Q8_0, Q4_K and Q6_K first; Q5_K, Q3_K, Q2_K, Q8_K and the other 32-element
+ * formats beside them) as hand-written HIP kernels for MI355X (gfx950).
  *
  * This is the surface a Rust `-sys` crate binds (plain pointers and sizes, no
  * C++ or framework types).  Every entry point names the reference interface it
