@@ -26,7 +26,7 @@ def _both(lib, fn, t, n, k, m, seed, y_dtype=0, order=0, x_dtype=1):
     # keep every f16 scale field finite: clear the top exponent bit of d (and dmin)
     ts = lib.pmetal_hip_type_size(t)
     blocks = w.reshape(-1, ts)
-    for off in {Q4K: (1, 3), Q6K: (209,), Q8_0: (1,)}[t]:
+    for off in {Q4K: (1, 3), Q6K: (209,), Q8_0: (1,), 13: (1, 3), 11: (109,), 10: (81, 83)}[t]:
         blocks[:, off] &= 0x3F
     x = rng.standard_normal(m * k).astype(np.float32)
     if x_dtype == 1:
@@ -52,7 +52,12 @@ def test_noalloc_equals_qgemm_two_calls_in_a_row():
     # first a call with a K split (partial tiles in the scratch), then a smaller one over the same array
     for (t, n, k, m, y_dtype, order, x_dtype) in ((Q4K, 1024, 4096, 48, 0, 0, 1), (Q4K, 512, 1024, 5, 1, 1, 1),
                                                   (Q6K, 768, 2048, 33, 0, 0, 0), (Q6K, 256, 512, 1, 1, 0, 1),
-                                                  (Q8_0, 512, 2048, 130, 0, 0, 1), (Q8_0, 256, 256, 7, 0, 0, 0)):
+                                                  (Q8_0, 512, 2048, 130, 0, 0, 1), (Q8_0, 256, 256, 7, 0, 0, 0),
+                                                  # Q5_K, Q3_K, Q2_K: the matrix kernels with a K split, then the short-batch
+                                                  # kernels (rows of 32 and 24 super-blocks go in runs with partial tiles)
+                                                  (13, 1024, 4096, 48, 0, 0, 1), (13, 512, 8192, 9, 1, 1, 1),
+                                                  (11, 640, 2048, 40, 0, 0, 1), (11, 333, 6144, 4, 0, 0, 0),
+                                                  (10, 512, 2048, 100, 1, 0, 1), (10, 250, 4096, 16, 0, 0, 1)):
         a, b = _both(lib, fn, t, n, k, m, seed=n + m, y_dtype=y_dtype, order=order, x_dtype=x_dtype)
         assert np.array_equal(a, b), (t, n, k, m)
         assert not np.all(a == 0xFF)
