@@ -144,6 +144,23 @@ int32_t pmetal_hip_quantize(uint32_t ggml_type, const float *src_host, size_t n,
                             size_t dst_len);
 int32_t pmetal_hip_quantize_dev(uint32_t ggml_type, const float *src_dev, size_t n, uint8_t *dst_dev,
                                 size_t dst_len, void *stream);
+/* The tensor loop of a model (run_quantization, crates/pmetal/src/commands/quantize.rs:1378-1428: one quantize call
+ * per tensor) in one call: the bytes of one pmetal_hip_quantize_dev per descriptor.  The tensors are independent, so the
+ * library spreads them over `stream` and a second stream of its own (per calling thread, default priority): one kernel's
+ * last workgroups overlap the next kernel's first (a batch of one k-quant tensor of 2^24 elements or more is cut in two for
+ * the same reason).  Asynchronous like the single call: the batch starts behind what
+ * `stream` holds, and work given to `stream` afterwards runs behind every tensor of the batch.  All descriptors are checked
+ * before anything is launched.  The second stream is made on the thread's first batch outside a recording; a batch
+ * recorded before that runs on `stream` alone.                                                                        */
+typedef struct pmetal_hip_quantize_desc {
+    uint32_t ggml_type;
+    uint32_t reserved;
+    const float *src_dev;
+    size_t n;
+    uint8_t *dst_dev;
+    size_t dst_len;
+} pmetal_hip_quantize_desc;
+int32_t pmetal_hip_quantize_batch_dev(const pmetal_hip_quantize_desc *descs, size_t count, void *stream);
 
 /* ---- dequantize: pmetal_gguf::dequant::dequantize(data, dtype, shape) -> Vec<f32> ----
  * crates/pmetal-gguf/src/dequant.rs:92-132 with its validation (:184-216); kernels follow

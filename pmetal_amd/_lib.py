@@ -24,6 +24,11 @@ class GemmDesc(C.Structure):
                 ("y_dev", _vp)]
 
 
+class QuantizeDesc(C.Structure):
+    """``pmetal_hip_quantize_desc``"""
+    _fields_ = [("ggml_type", _u32), ("reserved", _u32), ("src_dev", _vp), ("n", _sz), ("dst_dev", _vp), ("dst_len", _sz)]
+
+
 SYMBOLS = [
     ("pmetal_hip_device_count", _i32, []),
     ("pmetal_hip_init", _i32, [_i32]),
@@ -53,6 +58,7 @@ SYMBOLS = [
     ("pmetal_hip_event_destroy", _i32, [_vp]),
     ("pmetal_hip_quantize", _i32, [_u32, _vp, _sz, _vp, _sz]),
     ("pmetal_hip_quantize_dev", _i32, [_u32, _vp, _sz, _vp, _sz, _vp]),
+    ("pmetal_hip_quantize_batch_dev", _i32, [C.POINTER(QuantizeDesc), _sz, _vp]),
     ("pmetal_hip_dequantize", _i32, [_u32, _vp, _sz, C.POINTER(_i32), _sz, _vp, _sz, _u32]),
     ("pmetal_hip_dequantize_dev", _i32, [_u32, _vp, _sz, _vp, _sz, _u32, _vp]),
     ("pmetal_hip_qgemv", _i32, [_u32, _vp, _i64, _i64, _vp, _u32, _vp, _u32, _vp]),

@@ -75,6 +75,118 @@ def test_quantize_q4k_corner_cases_inside_a_large_tensor(oracle):
     assert np.array_equal(got, want), first_mismatch(got, want, BLOCK[Q4K])
 
 
+def _batch_case(seed):
+    """Tensors of a model-like mix: types, sizes from a few blocks to millions of elements, ragged tails, an empty one."""
+    rng = np.random.default_rng(seed)
+    specs = [(Q4K, 3 << 20), (Q6K, (1 << 20) + 77), (Q4K, 1000), (Q8_0, 0), (Q8_0, 3072 * 1024), (13, 2 << 20), (Q4K, 4 << 20),
+             (10, (1 << 19) + 5), (11, 1 << 19), (Q6K, 5 << 19), (2, 4096), (Q4K, 256), (Q4K, 1 << 22)]
+    order = rng.permutation(len(specs))
+    return [(specs[i][0], weights(900 + seed * 31 + int(i), specs[i][1], outliers=1e-3 * (int(i) % 2))) for i in order]
+
+
+@pytest.mark.parametrize("stream_kind", ["default", "created"])
+def test_quantize_batch_equals_separate_calls(oracle, stream_kind):
+    """pmetal_hip_quantize_batch_dev: the bytes of one pmetal_hip_quantize_dev per tensor (and of the oracle), with the
+    batch spread over two streams inside the library; what the caller's stream held before the batch (here: the fill of
+    one source tensor) is done before any tensor is read, and what it is given afterwards (a dequantize of the last
+    output) runs after every tensor."""
+    from pmetal_amd import _lib
+    lib = _lib.load()
+    stream = lib.pmetal_hip_stream_create() if stream_kind == "created" else None
+    for seed in (1, 2):
+        case = _batch_case(seed)
+        src = [pm.DeviceBuffer.from_host(x) if x.size else pm.DeviceBuffer(16) for _, x in case]
+        sizes = [lib.pmetal_hip_tensor_size(t, x.size) for t, x in case]
+        dst = [pm.DeviceBuffer(max(b, 16)) for b in sizes]
+        for d, b in zip(dst, sizes):
+            pm.check(lib.pmetal_hip_memset(d.ptr, 0xA5, max(b, 16), None))
+        pm.check(lib.pmetal_hip_sync(None))
+        # one source is produced on the caller's stream right before the batch
+        big = max(range(len(case)), key=lambda i: case[i][1].size)
+        pm.check(lib.pmetal_hip_fill_normal_f32(src[big].ptr, case[big][1].size, 4242 + seed, 0.02, 1e-3, 0.5, stream))
+        descs = (_lib.QuantizeDesc * len(case))()
+        for i, (t, x) in enumerate(case):
+            descs[i] = _lib.QuantizeDesc(t, 0, src[i].ptr, x.size, dst[i].ptr, sizes[i])
+        pm.check(lib.pmetal_hip_quantize_batch_dev(descs, len(case), stream))
+        last = len(case) - 1 if case[-1][1].size else len(case) - 2
+        back = pm.DeviceBuffer(4 * case[last][1].size)
+        pm.check(lib.pmetal_hip_dequantize_dev(case[last][0], dst[last].ptr, sizes[last], back.ptr, case[last][1].size, 0, stream))
+        pm.check(lib.pmetal_hip_sync(stream))
+        filled = src[big].to_host(np.float32, case[big][1].size)
+        for i, (t, x) in enumerate(case):
+            want = oracle.quantize(t, filled if i == big else x)
+            got = dst[i].to_host(np.uint8, sizes[i])
+            assert np.array_equal(got, want), (seed, i, t, x.size)
+        want_back = oracle.dequantize(case[last][0], dst[last].to_host(np.uint8, sizes[last]), [case[last][1].size])
+        assert np.array_equal(back.to_host(np.float32, case[last][1].size).view(np.uint32), want_back.view(np.uint32))
+    if stream:
+        pm.check(lib.pmetal_hip_stream_destroy(stream))
+
+
+@pytest.mark.parametrize("t", [Q4K, Q6K])
+def test_quantize_batch_of_one_large_tensor(oracle, t):
+    """A batch of a single large tensor is cut in two inside the library: the bytes of the whole tensor, ragged tail included."""
+    from pmetal_amd import _lib
+    lib = _lib.load()
+    x = weights(333 + t, (1 << 24) + 3 * 2048 + 77, outliers=1e-3)
+    nbytes = lib.pmetal_hip_tensor_size(t, x.size)
+    dx, dq = pm.DeviceBuffer.from_host(x), pm.DeviceBuffer(nbytes)
+    pm.check(lib.pmetal_hip_memset(dq.ptr, 0xA5, nbytes, None))
+    descs = (_lib.QuantizeDesc * 1)(_lib.QuantizeDesc(t, 0, dx.ptr, x.size, dq.ptr, nbytes))
+    pm.check(lib.pmetal_hip_quantize_batch_dev(descs, 1, None))
+    pm.check(lib.pmetal_hip_sync(None))
+    want = oracle.quantize(t, x)
+    got = dq.to_host(np.uint8, nbytes)
+    assert np.array_equal(got, want), first_mismatch(got, want, BLOCK[t])
+
+
+def test_quantize_batch_checks_every_descriptor_first_and_can_be_recorded(oracle):
+    from pmetal_amd import _lib
+    lib = _lib.load()
+    xs = [weights(70 + i, n) for i, n in enumerate((1 << 20, 1 << 19, 3 << 18))]
+    types = [Q4K, Q6K, Q4K]
+    src = [pm.DeviceBuffer.from_host(x) for x in xs]
+    sizes = [lib.pmetal_hip_tensor_size(t, x.size) for t, x in zip(types, xs)]
+    dst = [pm.DeviceBuffer(b) for b in sizes]
+    for d, b in zip(dst, sizes):
+        pm.check(lib.pmetal_hip_memset(d.ptr, 0xA5, b, None))
+    descs = (_lib.QuantizeDesc * 3)()
+    for i in range(3):
+        descs[i] = _lib.QuantizeDesc(types[i], 0, src[i].ptr, xs[i].size, dst[i].ptr, sizes[i])
+    # a wrong size in the last descriptor: nothing is launched
+    descs[2].dst_len = sizes[2] - 144
+    assert lib.pmetal_hip_quantize_batch_dev(descs, 3, None) == 3
+    assert b"tensor 2" in lib.pmetal_hip_last_error_message()
+    descs[2].dst_len = sizes[2]
+    descs[1].ggml_type = 16
+    assert lib.pmetal_hip_quantize_batch_dev(descs, 3, None) == 2
+    descs[1].ggml_type = Q6K
+    assert lib.pmetal_hip_quantize_batch_dev(None, 3, None) == 1
+    lib.pmetal_hip_clear_error()
+    pm.check(lib.pmetal_hip_sync(None))
+    assert all(np.all(d.to_host(np.uint8, b) == 0xA5) for d, b in zip(dst, sizes))
+    assert lib.pmetal_hip_quantize_batch_dev(descs, 0, None) == 0
+    # recorded on a created stream (the library's second stream exists after a first batch) and replayed twice
+    stream = lib.pmetal_hip_stream_create()
+    pm.check(lib.pmetal_hip_quantize_batch_dev(descs, 3, stream))
+    pm.check(lib.pmetal_hip_sync(stream))
+    want = [oracle.quantize(t, x) for t, x in zip(types, xs)]
+    pm.check(lib.pmetal_hip_record_begin(stream))
+    pm.check(lib.pmetal_hip_quantize_batch_dev(descs, 3, stream))
+    rec = lib.pmetal_hip_record_end(stream)
+    assert rec, lib.pmetal_hip_last_error_message()
+    for rep in range(2):
+        for d, b in zip(dst, sizes):
+            pm.check(lib.pmetal_hip_memset(d.ptr, 0x5A, b, None))
+        pm.check(lib.pmetal_hip_sync(None))
+        pm.check(lib.pmetal_hip_replay(rec, stream))
+        pm.check(lib.pmetal_hip_sync(stream))
+        for i in range(3):
+            assert np.array_equal(dst[i].to_host(np.uint8, sizes[i]), want[i]), (rep, i)
+    pm.check(lib.pmetal_hip_recording_destroy(rec))
+    pm.check(lib.pmetal_hip_stream_destroy(stream))
+
+
 @pytest.mark.parametrize("t", [Q8_0, Q4K, Q6K])
 def test_quantize_empty(oracle, t):
     assert gpu_quantize_dev(t, np.zeros(0, np.float32)).size == 0
