@@ -150,8 +150,7 @@ int32_t pmetal_hip_quantize_dev(uint32_t ggml_type, const float *src_dev, size_t
  * last workgroups overlap the next kernel's first (a batch of one k-quant tensor of 2^24 elements or more is cut in two for
  * the same reason).  Asynchronous like the single call: the batch starts behind what
  * `stream` holds, and work given to `stream` afterwards runs behind every tensor of the batch.  All descriptors are checked
- * before anything is launched.  The second stream is made on the thread's first batch outside a recording; a batch
- * recorded before that runs on `stream` alone.                                                                        */
+ * before anything is launched.  A batch issued while `stream` is being recorded runs on `stream` alone.               */
 typedef struct pmetal_hip_quantize_desc {
     uint32_t ggml_type;
     uint32_t reserved;

@@ -585,19 +585,21 @@ struct SideStream {
 };
 thread_local SideStream g_side;
 
-// The side stream of the current device, or NULL (no error) when it does not exist yet and cannot be made now: while the
-// caller's stream is being recorded nothing is created.
-int32_t side_stream(bool recording, SideStream **out) {
+// The side stream of the current device for a batch on `s`, or NULL (no error) while `s` is being recorded: a stream that
+// joins a recording belongs to it until the recording ends, and this one serves every stream of the thread, so it never
+// joins one -- a recorded batch runs on the caller's stream alone.
+int32_t side_stream(hipStream_t s, SideStream **out) {
     *out = nullptr;
     int dev = 0;
     HIP_TRY(hipGetDevice(&dev));
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (s) HIP_TRY(hipStreamIsCapturing(s, &cap));
+    if (cap != hipStreamCaptureStatusNone) return PMETAL_HIP_OK;
     if (g_side.s && g_side.device != dev) {
-        if (recording) return PMETAL_HIP_OK;
         (void)hipStreamSynchronize(g_side.s);
         g_side.release();
     }
     if (!g_side.s) {
-        if (recording) return PMETAL_HIP_OK;
         HIP_TRY(hipStreamCreateWithFlags(&g_side.s, hipStreamNonBlocking));  // default priority
         HIP_TRY(hipEventCreateWithFlags(&g_side.fork, hipEventDisableTiming));
         HIP_TRY(hipEventCreateWithFlags(&g_side.join, hipEventDisableTiming));
@@ -626,15 +628,13 @@ int32_t pmetal_hip_quantize_batch_dev(const pmetal_hip_quantize_desc *descs, siz
     if (work == 0) return ok();
     if (int32_t rc = require_device()) return rc;
     hipStream_t s = (hipStream_t)stream;
-    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    if (s) HIP_TRY(hipStreamIsCapturing(s, &cap));
     // a single large tensor of a k-quant type is cut in two for the same reason (its super-blocks are independent; Q4_K at
     // 14336 x 4096: 122 -> 114 us, Q6_K 171 -> 149)
     constexpr size_t kSplitMin = (size_t)1 << 24;
     const bool split = work == 1 && descs[only].n >= kSplitMin && pmetal_hip_block_size(descs[only].ggml_type) == 256;
     SideStream *side = nullptr;
     if (work >= 2 || split)
-        if (int32_t rc = side_stream(cap != hipStreamCaptureStatusNone, &side)) return rc;
+        if (int32_t rc = side_stream(s, &side)) return rc;
     if (side) {
         HIP_TRY(hipEventRecord(side->fork, s));
         HIP_TRY(hipStreamWaitEvent(side->s, side->fork, 0));

@@ -166,15 +166,24 @@ def test_quantize_batch_checks_every_descriptor_first_and_can_be_recorded(oracle
     pm.check(lib.pmetal_hip_sync(None))
     assert all(np.all(d.to_host(np.uint8, b) == 0xA5) for d, b in zip(dst, sizes))
     assert lib.pmetal_hip_quantize_batch_dev(descs, 0, None) == 0
-    # recorded on a created stream (the library's second stream exists after a first batch) and replayed twice
+    # recorded on a created stream and replayed twice
     stream = lib.pmetal_hip_stream_create()
     pm.check(lib.pmetal_hip_quantize_batch_dev(descs, 3, stream))
     pm.check(lib.pmetal_hip_sync(stream))
     want = [oracle.quantize(t, x) for t, x in zip(types, xs)]
     pm.check(lib.pmetal_hip_record_begin(stream))
     pm.check(lib.pmetal_hip_quantize_batch_dev(descs, 3, stream))
+    # (a recorded batch stays on its stream; the library's second stream is free for a batch run on another stream meanwhile)
+    other = lib.pmetal_hip_stream_create()
+    for d, b in zip(dst, sizes):
+        pm.check(lib.pmetal_hip_memset(d.ptr, 0x33, b, other))
+    pm.check(lib.pmetal_hip_quantize_batch_dev(descs, 3, other))
     rec = lib.pmetal_hip_record_end(stream)
     assert rec, lib.pmetal_hip_last_error_message()
+    pm.check(lib.pmetal_hip_sync(other))  # (the thread that records may not wait for a stream before the recording ends)
+    for i in range(3):
+        assert np.array_equal(dst[i].to_host(np.uint8, sizes[i]), want[i]), i
+    pm.check(lib.pmetal_hip_stream_destroy(other))
     for rep in range(2):
         for d, b in zip(dst, sizes):
             pm.check(lib.pmetal_hip_memset(d.ptr, 0x5A, b, None))
