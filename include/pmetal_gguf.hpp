@@ -163,6 +163,27 @@ class GgufLinear {
     DeviceBuffer w_;
 };
 
+// The tensor loop of run_quantization (crates/pmetal/src/commands/quantize.rs:1378-1428) over tensors that are already on
+// the device: one DeviceBuffer of blocks per (dtype, src, n), the bytes of one quantize() per tensor, through one
+// pmetal_hip_quantize_batch_dev call (the independent tensors spread over two streams inside the library).
+struct DeviceTensorF32 {
+    GgmlType dtype;
+    const float *src_dev;
+    size_t n;
+};
+inline std::vector<DeviceBuffer> quantize_tensors_dev(const std::vector<DeviceTensorF32> &tensors, void *stream = nullptr) {
+    std::vector<DeviceBuffer> outs;
+    std::vector<pmetal_hip_quantize_desc> descs;
+    outs.reserve(tensors.size());
+    for (const DeviceTensorF32 &t : tensors) {
+        const size_t bytes = pmetal_hip_tensor_size((uint32_t)t.dtype, t.n);
+        outs.emplace_back(bytes ? bytes : 16);
+        descs.push_back(pmetal_hip_quantize_desc{(uint32_t)t.dtype, 0u, t.src_dev, t.n, (uint8_t *)outs.back().ptr(), bytes});
+    }
+    detail::check(pmetal_hip_quantize_batch_dev(descs.data(), descs.size(), stream), true);
+    return outs;
+}
+
 // quantize_q8k (crates/pmetal-gguf/src/k_quants.rs:815-871) of n f32 values on the device: 292-byte BlockQ8K blocks.
 inline DeviceBuffer quantize_q8k(const DeviceBuffer &x, size_t n, void *stream = nullptr) {
     DeviceBuffer out(pmetal_hip_q8k_size(n) ? pmetal_hip_q8k_size(n) : 16);

@@ -174,6 +174,22 @@ def _dev_ptr(obj) -> int:
     return int(obj)
 
 
+def quantize_tensors_dev(tensors, stream=None):
+    """The tensor loop of ``run_quantization`` (crates/pmetal/src/commands/quantize.rs:1378-1428) over tensors that are
+    already on the device: ``tensors`` is a sequence of ``(dtype, src, n)`` (``src`` a device buffer or torch tensor of
+    ``n`` f32 values); returns one ``DeviceBuffer`` of blocks per tensor.  One ``pmetal_hip_quantize_batch_dev`` call: the
+    bytes of one ``quantize`` per tensor, the independent tensors spread over two streams inside the library."""
+    lib = _lib.load()
+    tensors = [(int(t), src, int(n)) for t, src, n in tensors]
+    sizes = [lib.pmetal_hip_tensor_size(t, n) for t, _, n in tensors]
+    outs = [DeviceBuffer(max(b, 16)) for b in sizes]
+    descs = (_lib.QuantizeDesc * max(len(tensors), 1))()
+    for i, (t, src, n) in enumerate(tensors):
+        descs[i] = _lib.QuantizeDesc(t, 0, _dev_ptr(src) if n else None, n, outs[i].ptr, sizes[i])
+    check(lib.pmetal_hip_quantize_batch_dev(descs, len(tensors), stream), "quantize")
+    return outs
+
+
 def q8k_size(n_elements: int) -> int:
     """Bytes of ``n_elements`` quantized to Q8_K (292 per 256, crates/pmetal-gguf/src/k_quants.rs:140-155)."""
     return _lib.load().pmetal_hip_q8k_size(n_elements)

@@ -210,6 +210,29 @@ static void test_calibration() {  // dynamic.rs:968-1018, :934-956 through the d
     CHECK(s == 0.0);
 }
 
+// the tensor loop of run_quantization (commands/quantize.rs:1378-1428) over device-resident tensors: the bytes of quantize()
+static void test_quantize_tensors_dev() {
+    const GgmlType types[3] = {GgmlType::Q4K, GgmlType::Q6K, GgmlType::Q8_0};
+    const size_t sizes[3] = {256 * 900, 256 * 500 + 17, 32 * 1000};
+    std::vector<std::vector<float>> host(3);
+    std::vector<DeviceBuffer> src;
+    std::vector<DeviceTensorF32> list;
+    for (int i = 0; i < 3; i++) {
+        host[i].resize(sizes[i]);
+        for (size_t j = 0; j < sizes[i]; j++) host[i][j] = 0.02f * std::sin(0.37f * (float)j + (float)i) + (j % 97 == 0 ? 0.4f : 0.0f);
+        src.emplace_back(host[i].data(), sizes[i] * sizeof(float));
+        list.push_back(DeviceTensorF32{types[i], (const float *)src.back().ptr(), sizes[i]});
+    }
+    std::vector<DeviceBuffer> outs = quantize_tensors_dev(list);
+    detail::check(pmetal_hip_sync(nullptr));
+    for (int i = 0; i < 3; i++) {
+        const std::vector<uint8_t> want = quantize(host[i].data(), sizes[i], types[i]);
+        std::vector<uint8_t> got(want.size());
+        outs[i].to_host(got.data(), got.size());
+        CHECK(got == want);
+    }
+}
+
 int main(int argc, char **argv) {
     const bool host_only = argc > 1 && std::strcmp(argv[1], "--host-only") == 0;
     test_block_sizes();
@@ -223,6 +246,7 @@ int main(int argc, char **argv) {
         test_roundtrips();
         test_linear_matmul_from();
         test_calibration();
+        test_quantize_tensors_dev();
     }
     std::printf(failures ? "%d check(s) failed\n" : "all checks passed\n", failures);
     return failures ? 1 : 0;

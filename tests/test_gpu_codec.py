@@ -123,6 +123,22 @@ def test_quantize_batch_equals_separate_calls(oracle, stream_kind):
         pm.check(lib.pmetal_hip_stream_destroy(stream))
 
 
+def test_mirror_quantize_tensors_dev(oracle):
+    """pmetal_amd.gguf.quantize_tensors_dev: a list of device-resident tensors, one buffer of blocks each (an empty one included)."""
+    xs = [(Q4K, weights(41, 5 << 18)), (Q6K, weights(42, (3 << 18) + 100)), (Q8_0, weights(43, 0)), (13, weights(44, 1 << 18))]
+    src = [pm.DeviceBuffer.from_host(x) if x.size else pm.DeviceBuffer(16) for _, x in xs]
+    outs = pm.gguf.quantize_tensors_dev([(t, b, x.size) for (t, x), b in zip(xs, src)])
+    pm.check(_lib_sync())
+    for (t, x), out in zip(xs, outs):
+        want = oracle.quantize(t, x)
+        assert np.array_equal(out.to_host(np.uint8, want.size), want), t
+
+
+def _lib_sync():
+    from pmetal_amd import _lib
+    return _lib.load().pmetal_hip_sync(None)
+
+
 @pytest.mark.parametrize("t", [Q4K, Q6K])
 def test_quantize_batch_of_one_large_tensor(oracle, t):
     """A batch of a single large tensor is cut in two inside the library: the bytes of the whole tensor, ragged tail included."""
