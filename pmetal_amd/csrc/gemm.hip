@@ -1269,6 +1269,7 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 constexpr int kSmallWaves = 8;  // waves per workgroup (fewer when a row has fewer super-blocks); 16 waves of one super-block each run alike
 constexpr int kSmallDepth = 2;  // row tiles in flight per wave (four are slower: 16.5 against 12.7 us at 14336 x 4096)
 constexpr int kSmallMaxM = 16, kSmallMaxSpr = 16;
+constexpr int kSmallMaxM2 = 32;  // Q4_K and Q5_K: two 16-row blocks of activations per weight operand
 
 // The two steps the short-batch kernels share.  A row tile's 16 x 16 partial tiles, one per wave: every wave leaves its
 // own in LDS, and after one barrier the first wave adds them in wave order and keeps the sum as finished tile `ti` (the
@@ -1315,16 +1316,17 @@ __device__ __forceinline__ void small_add_kept(const float4_t *keep, int n_tiles
 // After the last tile: y[m][16 t0 + j] for j over the workgroup's columns (consecutive threads store consecutive columns of
 // one row), scaled by the rows' powers of two; or, when a long row is cut into runs over the grid's second dimension,
 // the fp32 partial tile of this run, not yet scaled, for k_rw_reduce.
+// (mt: 16-row blocks of activations per row tile of weights; the finished tile of block b of row tile ti is slot ti * mt + b)
 __device__ __forceinline__ void small_store(const float4_t *out_tiles, int t0, int t1, int M, int Mp, int N,
                                             const float *__restrict__ rowscale, void *__restrict__ yg, int ybf16,
-                                            float *__restrict__ partial) {
+                                            float *__restrict__ partial, const int mt = 1) {
     __syncthreads();
     const int cols = (t1 - t0) * 16;
     for (int idx = (int)threadIdx.x; idx < M * cols; idx += (int)blockDim.x) {
         const int m = idx / cols, j = idx - m * cols;
         const int n = t0 * 16 + j;
         if (n < N) {
-            const float sum = out_tiles[(j >> 4) * 64 + (m >> 2) * 16 + (j & 15)][m & 3];
+            const float sum = out_tiles[((j >> 4) * mt + (m >> 4)) * 64 + ((m & 15) >> 2) * 16 + (j & 15)][m & 3];
             const float o = sum * rowscale[m];
             if (partial) partial[((size_t)blockIdx.y * Mp + m) * N + n] = sum;
             else if (ybf16) reinterpret_cast<uint16_t *>(yg)[(size_t)m * N + n] = (uint16_t)bf16_rne_bits(o);
@@ -1343,7 +1345,8 @@ struct SmallRun {
 
 // FMT 1: Q5_K -- eleven pieces per super-block (header, two of qh, eight of quants); a lane takes the qh bytes of its two
 // sub-blocks out of its stage as well and ors the fifth bits into the quant dwords as in the large kernel.
-template <int ORDER, int NSB, int FMT = 0>
+// MT: 16-row blocks of activations (1: at most 16 rows, 2: at most 32); a weight operand then feeds MT matrix instructions.
+template <int ORDER, int NSB, int FMT = 0, int MT = 1>
 __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t *__restrict__ W, const uint4 *__restrict__ xs,
                                                                    const float *__restrict__ rowscale, void *__restrict__ yg, int M,
                                                                    int Mp, int N, int spr, int tiles, int tiles_per_wg, int ybf16,
@@ -1357,8 +1360,8 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t 
     const uint32_t low = kg < 2 ? 0xFFFFFFFFu : 0u;
     const int rounds = (tiles_per_wg + kSmallDepth - 1) / kSmallDepth;
     float4_t *out_tiles = dyn;
-    float4_t *keep = tiles_per_wg <= kSmallKeepTiles ? dyn + rounds * kSmallDepth * 64 : nullptr;
-    u32x4 *stage = reinterpret_cast<u32x4 *>(dyn + rounds * kSmallDepth * 64 * (keep ? 1 + nwaves : 1)) + wave * SmallRun<NSB, FMT>::kPieces;
+    float4_t *keep = tiles_per_wg * MT <= kSmallKeepTiles ? dyn + rounds * kSmallDepth * MT * 64 : nullptr;
+    u32x4 *stage = reinterpret_cast<u32x4 *>(dyn + rounds * kSmallDepth * MT * 64 * (keep ? 1 + nwaves : 1)) + wave * SmallRun<NSB, FMT>::kPieces;
     int sbi[NSB];
     bool sbv[NSB];  // wave-uniform
 #pragma unroll
@@ -1367,21 +1370,23 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t 
         sbv[i] = sbi[i] < spr;
         sbi[i] = sbv[i] ? sbi[i] : 0;
     }
-    // activation operands of this wave's super-blocks: item (2 sb + kg / 2, group 2 t + kg % 2) of row nl, and the sums item
-    half8_t af[NSB][8], asum[NSB];
+    // activation operands of this wave's super-blocks: item (2 sb + kg / 2, group 2 t + kg % 2) of rows nl (and 16 + nl), and the sums item
+    half8_t af[NSB][MT][8], asum[NSB][MT];
 #pragma unroll
-    for (int i = 0; i < NSB; i++) {
-        const uint4 *base = xs + (size_t)((2 * sbi[i] + (kg >> 1)) * kGroups) * Mp + nl;
+    for (int i = 0; i < NSB; i++)
 #pragma unroll
-        for (int t = 0; t < 8; t++) af[i][t] = __builtin_bit_cast(half8_t, base[(size_t)(2 * t + (kg & 1)) * Mp]);
-        asum[i] = __builtin_bit_cast(half8_t, base[(size_t)(16 + (kg & 1)) * Mp]);
-        if (!sbv[i]) {  // a super-block past the end of the row multiplies zeros (no branch in the streaming loop)
-            const half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (int b = 0; b < MT; b++) {
+            const uint4 *base = xs + (size_t)((2 * sbi[i] + (kg >> 1)) * kGroups) * Mp + 16 * b + nl;
 #pragma unroll
-            for (int t = 0; t < 8; t++) af[i][t] = z;
-            asum[i] = z;
+            for (int t = 0; t < 8; t++) af[i][b][t] = __builtin_bit_cast(half8_t, base[(size_t)(2 * t + (kg & 1)) * Mp]);
+            asum[i][b] = __builtin_bit_cast(half8_t, base[(size_t)(16 + (kg & 1)) * Mp]);
+            if (!sbv[i]) {  // a super-block past the end of the row multiplies zeros (no branch in the streaming loop)
+                const half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+                for (int t = 0; t < 8; t++) af[i][b][t] = z;
+                asum[i][b] = z;
+            }
         }
-    }
     const int t0 = (int)blockIdx.x * tiles_per_wg;
     const int t1 = t0 + tiles_per_wg < tiles ? t0 + tiles_per_wg : tiles;  // t1 > t0 by the launch geometry
     constexpr int kPerSb = SmallRun<NSB, FMT>::kPerSb, kBlockBytes = BlockFmt<FMT>::kBytes, kQ0 = FMT ? 3 : 1;  // kQ0: first quant piece
@@ -1410,7 +1415,9 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t 
     };
     const u32x4 *mine = stage + nl * (kPerSb * NSB);  // this lane's weight row in the stage
     auto consume = [&](int ti, const SmallRun<NSB, FMT> &w) __attribute__((always_inline)) {
-        float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        float4_t acc[MT];
+#pragma unroll
+        for (int b = 0; b < MT; b++) acc[b] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int j = 0; j < kLoads; j++)
             if (lane + 64 * j < kPieces) stage[lane + 64 * j] = w.piece[j];
@@ -1448,13 +1455,17 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t 
                     for (int t = 0; t < 8; t++) qh[t] = (t < 4 ? hp.x : hp.y) >> (8 * (t & 3));
                 }
             }
-            float4_t part = {0.0f, 0.0f, 0.0f, 0.0f};
+            float4_t part[MT];
+#pragma unroll
+            for (int b = 0; b < MT; b++) part[b] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int t = 0; t < 8; t++) {
                 Dq d;
 #pragma unroll
                 for (int c = 0; c < 4; c++) dq_chunk<ORDER, FMT>(c, t, qd[t], sc2, off2, d, qh[t]);
-                part = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i][t], d.value(), part, 0, 0, 0);
+                const half8_t bv = d.value();
+#pragma unroll
+                for (int b = 0; b < MT; b++) part[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i][b][t], bv, part[b], 0, 0, 0);
             }
             // (of a super-block past the end of the row only zeros may enter the sums, whatever bytes were loaded for it)
             const float dmin = sbv[i] ? f16_bits_to_f32(hdr.x >> 16) : 0.0f, dd = sbv[i] ? f16_bits_to_f32(hdr.x & 0xFFFFu) : 0.0f;
@@ -1462,11 +1473,15 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t 
             neg_min_split(dmin, mn0, h0, l0);
             neg_min_split(dmin, mn1, h1, l1);
             const half8_t br = {h0, h0, l0, l0, h1, h1, l1, l1};
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(asum[i], br, acc, 0, 0, 0);
 #pragma unroll
-            for (int r = 0; r < 4; r++) acc[r] = __builtin_fmaf(dd, part[r], acc[r]);
+            for (int b = 0; b < MT; b++) {
+                acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(asum[i][b], br, acc[b], 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 4; r++) acc[b][r] = __builtin_fmaf(dd, part[b][r], acc[b][r]);
+            }
         }
-        small_add_waves(red, keep, ti, wave, nwaves, lane, acc, out_tiles);
+#pragma unroll
+        for (int b = 0; b < MT; b++) small_add_waves(red, keep, ti * MT + b, wave, nwaves, lane, acc[b], out_tiles);
     };
     static_assert(kSmallDepth == 2, "the ring is written out as two tiles");
     SmallRun<NSB, FMT> ring0, ring1;
@@ -1480,8 +1495,8 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small(const uint8_t 
         consume(2 * rd + 1, ring1);
         issue(2 * rd + 3, ring1);
     }
-    small_add_kept(keep, rounds * kSmallDepth, wave, nwaves, lane, out_tiles);
-    small_store(out_tiles, t0, t1, M, Mp, N, rowscale, yg, ybf16, partial);
+    small_add_kept(keep, rounds * kSmallDepth * MT, wave, nwaves, lane, out_tiles);
+    small_store(out_tiles, t0, t1, M, Mp, N, rowscale, yg, ybf16, partial, MT);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -2031,9 +2046,10 @@ static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 constexpr int kSmallMaxRuns = 8;  // k <= 32768
 static bool qgemm_small_applies(uint32_t type, int64_t m, int64_t n, int64_t k) {
     const int64_t spr = k / 256;
-    if (m > kSmallMaxM || spr > kSmallMaxSpr * kSmallMaxRuns) return false;
-    if (type == kTypeQ4K) return (uint64_t)n * (uint64_t)spr * 144u < (1ull << 32);
-    if (type == kTypeQ5K) return (uint64_t)n * (uint64_t)spr * 176u < (1ull << 32);
+    if (spr > kSmallMaxSpr * kSmallMaxRuns) return false;
+    if (type == kTypeQ4K && m <= kSmallMaxM2) return (uint64_t)n * (uint64_t)spr * 144u < (1ull << 32);
+    if (type == kTypeQ5K && m <= kSmallMaxM2) return (uint64_t)n * (uint64_t)spr * 176u < (1ull << 32);
+    if (m > kSmallMaxM) return false;
     if (type == kTypeQ8_0) return (uint64_t)n * (uint64_t)spr * 272u < (1ull << 32);
     if (type == kTypeQ6K) return (uint64_t)n * (uint64_t)spr * 210u < (1ull << 32);
     if (type == kTypeQ3K) return (uint64_t)n * (uint64_t)spr * 110u < (1ull << 32);
@@ -2089,7 +2105,7 @@ GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k, uint32_t type) {
     }
     // at most 16 activation rows against long rows: runs of 16 super-blocks (the fused kernels' K split; the large kernel
     // takes the same split when a shape falls back to it)
-    if (m <= kSmallMaxM && spr > kSmallMaxSpr) p.chunk = kSmallMaxSpr, p.splits = (int)((spr + kSmallMaxSpr - 1) / kSmallMaxSpr);
+    if ((m <= kSmallMaxM || (m <= kSmallMaxM2 && (type == kTypeQ4K || type == kTypeQ5K))) && spr > kSmallMaxSpr) p.chunk = kSmallMaxSpr, p.splits = (int)((spr + kSmallMaxSpr - 1) / kSmallMaxSpr);
     return p;
 }
 
@@ -2212,9 +2228,10 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
         slots = slots < 1 ? 1 : slots;
         const int n_wg = (int)(tiles < slots ? tiles : slots);
         int tiles_per_wg = (tiles + n_wg - 1) / n_wg;
+        const int mt = m > kSmallMaxM ? 2 : 1;  // 16-row blocks of activations (two: Q4_K and Q5_K only)
         // the finished tiles wait in LDS, 1 KiB each, beside the waves' stages (at most 70 KiB, Q8_0) and the 16 KiB of the
         // reduction buffers: 64 of them keep the workgroup within 160 KiB for every type
-        tiles_per_wg = tiles_per_wg < 64 ? tiles_per_wg : 64;
+        tiles_per_wg = tiles_per_wg < 64 / mt ? tiles_per_wg : 64 / mt;
         // a long row: p.splits runs of 16 super-blocks, one workgroup row of the grid each, partial tiles for k_rw_reduce
         // (for rows of up to 16 super-blocks the plan's split belongs to the large kernel and is not used here)
         const int runs = runs_of_row;
@@ -2222,18 +2239,23 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
         const int nsb = spr > kSmallWaves ? 2 : 1;
         const dim3 grid((unsigned)((tiles + tiles_per_wg - 1) / tiles_per_wg), (unsigned)runs), block((unsigned)(64 * nwaves));
         // (a workgroup of few tiles also keeps every wave's partial tile of each until the end)
-        const size_t lds = (size_t)((tiles_per_wg + kSmallDepth - 1) / kSmallDepth * kSmallDepth) * 1024 *
-                           (tiles_per_wg <= kSmallKeepTiles ? 1 + nwaves : 1);
-#define PMH_SMALL_F(O, S, F)                                                                                                     \
+        const size_t lds = (size_t)((tiles_per_wg + kSmallDepth - 1) / kSmallDepth * kSmallDepth) * mt * 1024 *
+                           (tiles_per_wg * mt <= kSmallKeepTiles ? 1 + nwaves : 1);
+#define PMH_SMALL_FM(O, S, F, T)                                                                                                 \
     do {                                                                                                                         \
         const size_t lds4 = lds + (size_t)nwaves * SmallRun<S, F>::kPieces * 16; /* the waves' stages behind the finished tiles */ \
         if (lds4 > 48 * 1024) {                                                                                                   \
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_qgemm_small<O, S, F>), hipFuncAttributeMaxDynamicSharedMemorySize, \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_qgemm_small<O, S, F, T>), hipFuncAttributeMaxDynamicSharedMemorySize, \
                                     (int)lds4);                                                                                   \
             if (e != hipSuccess) return e;                                                                                       \
         }                                                                                                                        \
-        hipLaunchKernelGGL((k_qgemm_small<O, S, F>), grid, block, lds4, s, w, xs, rowscale, y, (int)m, (int)p.mp, (int)n, spr, tiles, \
+        hipLaunchKernelGGL((k_qgemm_small<O, S, F, T>), grid, block, lds4, s, w, xs, rowscale, y, (int)m, (int)p.mp, (int)n, spr, tiles, \
                            tiles_per_wg, ybf ? 1 : 0, part_out);                                                                           \
+    } while (0)
+#define PMH_SMALL_F(O, S, F)               \
+    do {                                   \
+        if (mt == 2) PMH_SMALL_FM(O, S, F, 2); \
+        else PMH_SMALL_FM(O, S, F, 1);         \
     } while (0)
 #define PMH_SMALL(O, S)         \
     do {                        \
@@ -2304,6 +2326,7 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
         }
 #undef PMH_SMALL
 #undef PMH_SMALL_F
+#undef PMH_SMALL_FM
         e = hipGetLastError();
         if (e != hipSuccess || runs == 1) return e;
     } else {

@@ -345,7 +345,7 @@ def test_qgemm_q5k_q3k_q2k_matches_dequantize_then_matmul(oracle, t, m, n, k):
 
 
 @pytest.mark.parametrize("t,order", [(13, 0), (13, 1), (11, 0), (10, 0)])
-@pytest.mark.parametrize("m,n,k", [(7, 96, 512), (40, 300, 1024), (130, 257, 768), (300, 64, 2048)])
+@pytest.mark.parametrize("m,n,k", [(7, 96, 512), (23, 200, 2048), (40, 300, 1024), (130, 257, 768), (300, 64, 2048)])
 def test_qgemm_q5k_q3k_q2k_unit_activations_pick_single_weights(oracle, t, order, m, n, k):
     """The matrix kernels of Q5_K (the Q4_K kernel with the fifth bits from qh) and of Q3_K / Q2_K (sixteen 16-element
     sub-blocks): with unit activations row r of the result is column c_r of the dequantized weight, bit for bit -- every
@@ -509,7 +509,7 @@ def test_qgemm_batch_wide_and_narrow_weights_share_x(oracle, t, m):
 
 
 @pytest.mark.parametrize("t", [Q4K, Q6K, Q8_0, 13, 11, 10])
-@pytest.mark.parametrize("m", [1, 2, 5, 9, 16])
+@pytest.mark.parametrize("m", [1, 2, 5, 9, 16, 17, 25, 32])
 @pytest.mark.parametrize("n,k", [(700, 2048), (333, 4096), (16, 2048), (4099, 4096), (40, 1024),
                                  # rows of more than 16 super-blocks: runs of 16, partial tiles added in a second kernel
                                  (500, 14336), (130, 6144), (77, 11008), (64, 32768),
@@ -517,7 +517,7 @@ def test_qgemm_batch_wide_and_narrow_weights_share_x(oracle, t, m):
                                  # wave with work owns one super-block where the others own two, a second run holds four
                                  (333, 2816), (1001, 256), (250, 768), (123, 5120), (47, 3328)])
 def test_qgemm_short_batches(oracle, t, m, n, k):
-    """At most 16 activation rows: the fused kernels that read the weights once (rows of any number of super-blocks, in runs of 16).  Random block bytes (every scale, min and quant pattern), row counts that are no multiple of the 16-row
+    """At most 16 activation rows (Q4_K and Q5_K: at most 32, two 16-row blocks per weight operand): the fused kernels that read the weights once (rows of any number of super-blocks, in runs of 16).  Random block bytes (every scale, min and quant pattern), row counts that are no multiple of the 16-row
     tiles, one full tile, more tiles than workgroups take in one round; bf16 and f32 activations, f32 and bf16 outputs;
     unit activations that pick single weights out of the matrix."""
     rng = np.random.default_rng(1000 * t + 31 * m + n + k)
@@ -563,11 +563,12 @@ def test_qgemm_short_batches(oracle, t, m, n, k):
 
 
 @pytest.mark.parametrize("t", [Q4K, Q6K, Q8_0, 13, 11, 10])
-def test_qgemm_short_batch_very_tall_weight(oracle, t):
-    """300 000 weight rows against 9 activation rows: more row tiles per workgroup than its LDS holds finished tiles for,
+@pytest.mark.parametrize("m", [9, 29])
+def test_qgemm_short_batch_very_tall_weight(oracle, t, m):
+    """300 000 weight rows against 9 (29) activation rows: more row tiles per workgroup than its LDS holds finished tiles for,
     so the grid has more workgroups than compute units.  The first 2000 and the last 3000 rows against the oracle."""
-    n, k, m = 300000, 2048, 9
-    rng = np.random.default_rng(t)
+    n, k = 300000, 2048
+    rng = np.random.default_rng(t + m)
     block = {Q4K: 144, Q6K: 210, Q8_0: 34, 13: 176, 11: 110, 10: 84}[t]
     per = 32 if t == Q8_0 else 256
     raw = rng.integers(0, 256, size=(n * (k // per), block), dtype=np.uint8)

@@ -55,6 +55,7 @@ def test_noalloc_equals_qgemm_two_calls_in_a_row():
                                                   (Q8_0, 512, 2048, 130, 0, 0, 1), (Q8_0, 256, 256, 7, 0, 0, 0),
                                                   # Q5_K, Q3_K, Q2_K: the matrix kernels with a K split, then the short-batch
                                                   # kernels (rows of 32 and 24 super-blocks go in runs with partial tiles)
+                                                  (Q4K, 900, 4096, 27, 0, 1, 1), (13, 640, 8192, 20, 0, 0, 1),
                                                   (13, 1024, 4096, 48, 0, 0, 1), (13, 512, 8192, 9, 1, 1, 1),
                                                   (11, 640, 2048, 40, 0, 0, 1), (11, 333, 6144, 4, 0, 0, 0),
                                                   (10, 512, 2048, 100, 1, 0, 1), (10, 250, 4096, 16, 0, 0, 1)):
