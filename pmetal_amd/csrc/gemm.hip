@@ -1517,7 +1517,7 @@ struct SmallRunQ8 {
     u32x4 piece[5];  // (a vector type: copies of it are loads and stores that stay in registers)
 };
 
-template <int NSB>
+template <int NSB, int MT = 1>
 __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q8(const uint8_t *__restrict__ W, const uint4 *__restrict__ xs,
                                                                       const float *__restrict__ rowscale, void *__restrict__ yg, int M,
                                                                       int Mp, int N, int spr, int tiles, int tiles_per_wg, int ybf16,
@@ -1530,8 +1530,8 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q8(const uint8
     const int nl = lane & 15, kg = lane >> 4;
     const int rounds = (tiles_per_wg + kSmallDepth - 1) / kSmallDepth;
     float4_t *out_tiles = dyn;
-    float4_t *keep = tiles_per_wg <= kSmallKeepTiles ? dyn + rounds * kSmallDepth * 64 : nullptr;
-    u32x4 *stage = reinterpret_cast<u32x4 *>(dyn + rounds * kSmallDepth * 64 * (keep ? 1 + nwaves : 1)) + wave * (NSB * kQ8TileRunPieces);
+    float4_t *keep = tiles_per_wg * MT <= kSmallKeepTiles ? dyn + rounds * kSmallDepth * MT * 64 : nullptr;
+    u32x4 *stage = reinterpret_cast<u32x4 *>(dyn + rounds * kSmallDepth * MT * 64 * (keep ? 1 + nwaves : 1)) + wave * (NSB * kQ8TileRunPieces);
     int sbi[NSB];
     bool sbv[NSB];  // wave-uniform
 #pragma unroll
@@ -1542,16 +1542,17 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q8(const uint8
     }
     // activation operands: block b of run sb holds elements 256 sb + 32 b ..; the item of its k-group kg is item
     // 4 (b % 4) + kg of half 2 sb + b / 4 (the pre-pass writes 16 items of eight consecutive elements per 128)
-    half8_t af[NSB][8];
+    half8_t af[NSB][MT][8];  // (MT 16-row blocks of activations: rows nl, 16 + nl)
 #pragma unroll
-    for (int i = 0; i < NSB; i++) {
+    for (int i = 0; i < NSB; i++)
 #pragma unroll
-        for (int b = 0; b < 8; b++) {
-            const uint4 *item = xs + (size_t)((2 * sbi[i] + (b >> 2)) * kGroups + 4 * (b & 3) + kg) * Mp + nl;
-            af[i][b] = __builtin_bit_cast(half8_t, *item);
-            if (!sbv[i]) af[i][b] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-        }
-    }
+        for (int mb = 0; mb < MT; mb++)
+#pragma unroll
+            for (int b = 0; b < 8; b++) {
+                const uint4 *item = xs + (size_t)((2 * sbi[i] + (b >> 2)) * kGroups + 4 * (b & 3) + kg) * Mp + 16 * mb + nl;
+                af[i][mb][b] = __builtin_bit_cast(half8_t, *item);
+                if (!sbv[i]) af[i][mb][b] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+            }
     const int t0 = (int)blockIdx.x * tiles_per_wg;
     const int t1 = t0 + tiles_per_wg < tiles ? t0 + tiles_per_wg : tiles;
     const uint32_t row_bytes = (uint32_t)spr * (uint32_t)kQ8RunBytes;
@@ -1578,7 +1579,9 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q8(const uint8
     };
     const uint32_t *mine = reinterpret_cast<const uint32_t *>(stage) + nl * (kQ8RunBytes / 4);  // this lane's weight row in the stage
     auto consume = [&](int ti, const SmallRunQ8 &wa, const SmallRunQ8 &wb) __attribute__((always_inline)) {
-        float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        float4_t acc[MT];
+#pragma unroll
+        for (int mb = 0; mb < MT; mb++) acc[mb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
         const float4_t none = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int i = 0; i < NSB; i++) {
@@ -1607,12 +1610,17 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q8(const uint8
                 }
                 // (of a run past the end of the row only zeros may enter the sums, whatever bytes were loaded for it)
                 const float d = sbv[i] ? f16_bits_to_f32(dbits) : 0.0f;
-                const float4_t part = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i][b], q8_operand(q0, q1), none, 0, 0, 0);
+                const half8_t bv = q8_operand(q0, q1);
 #pragma unroll
-                for (int r = 0; r < 4; r++) acc[r] = __builtin_fmaf(d, part[r], acc[r]);
+                for (int mb = 0; mb < MT; mb++) {
+                    const float4_t part = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i][mb][b], bv, none, 0, 0, 0);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) acc[mb][r] = __builtin_fmaf(d, part[r], acc[mb][r]);
+                }
             }
         }
-        small_add_waves(red, keep, ti, wave, nwaves, lane, acc, out_tiles);
+#pragma unroll
+        for (int mb = 0; mb < MT; mb++) small_add_waves(red, keep, ti * MT + mb, wave, nwaves, lane, acc[mb], out_tiles);
     };
     static_assert(kSmallDepth == 2, "the ring is written out as two tiles");
     SmallRunQ8 ring0a, ring0b, ring1a, ring1b;  // (the b halves are unused with one run per wave)
@@ -1624,8 +1632,8 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small_q8(const uint8
         consume(2 * rd + 1, ring1a, ring1b);
         issue(2 * rd + 3, ring1a, ring1b);
     }
-    small_add_kept(keep, rounds * kSmallDepth, wave, nwaves, lane, out_tiles);
-    small_store(out_tiles, t0, t1, M, Mp, N, rowscale, yg, ybf16, partial);
+    small_add_kept(keep, rounds * kSmallDepth * MT, wave, nwaves, lane, out_tiles);
+    small_store(out_tiles, t0, t1, M, Mp, N, rowscale, yg, ybf16, partial, MT);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -2044,12 +2052,24 @@ static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 // The fused kernels for at most 16 activation rows.  Rows of more than 16 super-blocks are cut into runs of 16, one
 // workgroup row of the grid each, whose partial tiles k_rw_reduce adds (qgemm_plan sets splits and chunk to match).
 constexpr int kSmallMaxRuns = 8;  // k <= 32768
+// Super-blocks of a row that one short-batch workgroup takes (a longer row goes in runs of that many); 0: no such kernel.
+// Up to 16 rows: eight waves of two super-blocks.  17 to 32 rows (two 16-row blocks of activations per weight operand): the
+// Q4_K / Q5_K kernel still holds two super-blocks' activations per wave, the Q8_0 kernel one (43.4 -> 27.1 us at 14336 x 4096);
+// the Q6_K kernel in that form, with its rows in runs of eight, is no faster than the large kernel (32.2 against 29.9 us).
+static int small_run_spr(uint32_t type, int64_t m) {
+    const bool any = type == kTypeQ4K || type == kTypeQ5K || type == kTypeQ6K || type == kTypeQ8_0 || type == kTypeQ3K || type == kTypeQ2K;
+    if (m <= kSmallMaxM) return any ? kSmallMaxSpr : 0;
+    if (m > kSmallMaxM2) return 0;
+    if (type == kTypeQ4K || type == kTypeQ5K) return kSmallMaxSpr;
+    if (type == kTypeQ8_0) return kSmallWaves;
+    return 0;
+}
 static bool qgemm_small_applies(uint32_t type, int64_t m, int64_t n, int64_t k) {
     const int64_t spr = k / 256;
-    if (spr > kSmallMaxSpr * kSmallMaxRuns) return false;
-    if (type == kTypeQ4K && m <= kSmallMaxM2) return (uint64_t)n * (uint64_t)spr * 144u < (1ull << 32);
-    if (type == kTypeQ5K && m <= kSmallMaxM2) return (uint64_t)n * (uint64_t)spr * 176u < (1ull << 32);
-    if (m > kSmallMaxM) return false;
+    const int run = small_run_spr(type, m);
+    if (run == 0 || spr > (int64_t)run * kSmallMaxRuns) return false;
+    if (type == kTypeQ4K) return (uint64_t)n * (uint64_t)spr * 144u < (1ull << 32);
+    if (type == kTypeQ5K) return (uint64_t)n * (uint64_t)spr * 176u < (1ull << 32);
     if (type == kTypeQ8_0) return (uint64_t)n * (uint64_t)spr * 272u < (1ull << 32);
     if (type == kTypeQ6K) return (uint64_t)n * (uint64_t)spr * 210u < (1ull << 32);
     if (type == kTypeQ3K) return (uint64_t)n * (uint64_t)spr * 110u < (1ull << 32);
@@ -2103,9 +2123,10 @@ GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k, uint32_t type) {
                          (splits > 1 ? (double)splits * (double)m * (double)n * 8.0 / 4.0e12 + 3.0e-6 : 0.0);
         if (want == 1 || t < best) best = t, p.splits = (int)splits, p.chunk = (int)chunk;
     }
-    // at most 16 activation rows against long rows: runs of 16 super-blocks (the fused kernels' K split; the large kernel
-    // takes the same split when a shape falls back to it)
-    if ((m <= kSmallMaxM || (m <= kSmallMaxM2 && (type == kTypeQ4K || type == kTypeQ5K))) && spr > kSmallMaxSpr) p.chunk = kSmallMaxSpr, p.splits = (int)((spr + kSmallMaxSpr - 1) / kSmallMaxSpr);
+    // short batches against long rows: runs of 16 (or 8) super-blocks (the fused kernels' K split; the large kernel takes the
+    // same split when a shape falls back to it)
+    const int run = small_run_spr(type, m);
+    if (run && spr > run) p.chunk = run, p.splits = (int)((spr + run - 1) / run);
     return p;
 }
 
@@ -2113,7 +2134,7 @@ size_t qgemm_workspace_bytes(uint32_t type, int64_t m, int64_t n, int64_t k) {
     const GemmPlan p = qgemm_plan(m, n, k, type);
     const size_t xs = align256((size_t)(k / 256) * 2 * (type == kTypeQ3K || type == kTypeQ2K ? kGroups16 : kGroups) * p.mp * 16);
     // the short-batch kernels take a row of up to kSmallMaxSpr super-blocks whole: the plan's K split is not used there
-    const bool unsplit = qgemm_small_applies(type, m, n, k) && k / 256 <= kSmallMaxSpr;
+    const bool unsplit = qgemm_small_applies(type, m, n, k) && k / 256 <= small_run_spr(type, m);
     const size_t part = p.splits > 1 && !unsplit ? align256((size_t)p.splits * p.mp * n * 4) : 0;
     return xs + align256((size_t)p.mp * 4) + part;
 }
@@ -2223,12 +2244,13 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
         const int tiles = (int)((n + 15) / 16);
         // one workgroup per compute unit over all runs of a long row: each then walks several row tiles with its activation
         // operands in registers (one tile per workgroup and four times the workgroups: 35 against 27 us at M = 16, 4096 x 14336)
-        const int runs_of_row = spr > kSmallMaxSpr ? p.splits : 1;
+        const int run = small_run_spr(type, m);
+        const int runs_of_row = spr > run ? p.splits : 1;
         int64_t slots = (int64_t)compute_units_gemm() * (kSmallWaves / nwaves) / runs_of_row;
         slots = slots < 1 ? 1 : slots;
         const int n_wg = (int)(tiles < slots ? tiles : slots);
         int tiles_per_wg = (tiles + n_wg - 1) / n_wg;
-        const int mt = m > kSmallMaxM ? 2 : 1;  // 16-row blocks of activations (two: Q4_K and Q5_K only)
+        const int mt = m > kSmallMaxM ? 2 : 1;  // 16-row blocks of activations
         // the finished tiles wait in LDS, 1 KiB each, beside the waves' stages (at most 70 KiB, Q8_0) and the 16 KiB of the
         // reduction buffers: 64 of them keep the workgroup within 160 KiB for every type
         tiles_per_wg = tiles_per_wg < 64 / mt ? tiles_per_wg : 64 / mt;
@@ -2236,7 +2258,7 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
         // (for rows of up to 16 super-blocks the plan's split belongs to the large kernel and is not used here)
         const int runs = runs_of_row;
         float *const part_out = runs > 1 ? partial : nullptr;
-        const int nsb = spr > kSmallWaves ? 2 : 1;
+        const int nsb = run > kSmallWaves && spr > kSmallWaves ? 2 : 1;
         const dim3 grid((unsigned)((tiles + tiles_per_wg - 1) / tiles_per_wg), (unsigned)runs), block((unsigned)(64 * nwaves));
         // (a workgroup of few tiles also keeps every wave's partial tile of each until the end)
         const size_t lds = (size_t)((tiles_per_wg + kSmallDepth - 1) / kSmallDepth * kSmallDepth) * mt * 1024 *
@@ -2303,18 +2325,19 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
 #undef PMH_SMALL_Q6
         } else if (q8) {
             const size_t lds8 = lds + (size_t)nwaves * nsb * kQ8TileRunPieces * 16;  // the waves' stages behind the finished tiles
-#define PMH_SMALL_Q8(S)                                                                                                          \
+#define PMH_SMALL_Q8(S, T)                                                                                                       \
     do {                                                                                                                         \
         if (lds8 > 48 * 1024) {                                                                                                  \
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_qgemm_small_q8<S>), hipFuncAttributeMaxDynamicSharedMemorySize, \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_qgemm_small_q8<S, T>), hipFuncAttributeMaxDynamicSharedMemorySize, \
                                     (int)lds8);                                                                                  \
             if (e != hipSuccess) return e;                                                                                       \
         }                                                                                                                        \
-        hipLaunchKernelGGL((k_qgemm_small_q8<S>), grid, block, lds8, s, w, xs, rowscale, y, (int)m, (int)p.mp, (int)n, spr, tiles, \
+        hipLaunchKernelGGL((k_qgemm_small_q8<S, T>), grid, block, lds8, s, w, xs, rowscale, y, (int)m, (int)p.mp, (int)n, spr, tiles, \
                            tiles_per_wg, ybf ? 1 : 0, part_out);                                                                           \
     } while (0)
-            if (nsb == 2) PMH_SMALL_Q8(2);
-            else PMH_SMALL_Q8(1);
+            if (mt == 2) PMH_SMALL_Q8(1, 2);  // (two blocks of activations: one run of eight blocks per wave)
+            else if (nsb == 2) PMH_SMALL_Q8(2, 1);
+            else PMH_SMALL_Q8(1, 1);
 #undef PMH_SMALL_Q8
         } else if (spr > kSmallWaves) {
             static_assert(2 * kSmallWaves >= kSmallMaxSpr, "two super-blocks per wave must cover the longest row");
