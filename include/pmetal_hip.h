@@ -187,7 +187,7 @@ int32_t pmetal_hip_dequantize_dev(uint32_t ggml_type, const uint8_t *src_dev, si
  * Types: every type has both kernels (the Q5_K GEMM is the Q4_K kernel with the fifth bit of every quant taken from the
  * block's qh bytes; Q3_K and Q2_K share a kernel for sixteen 16-element sub-blocks).  The GEMV of Q5_K, Q3_K and Q2_K takes
  * k <= 32768 and a tensor below 4 GiB, any number of rows; beyond that qgemv fails with SHAPE_TOO_LARGE and qlinear uses the
- * GEMM.  Every type has a second GEMM kernel for m <= 16 (Q4_K, Q5_K and Q8_0: m <= 32) that reads the weights once; qlinear runs two activation rows of a
+ * GEMM.  Every type has a second GEMM kernel for m <= 16 (Q4_K, Q5_K, Q8_0 and Q2_K: m <= 32) that reads the weights once; qlinear runs two activation rows of a
  * Q5_K, Q3_K or Q2_K weight of at most 2^23 elements as two GEMVs, and a larger weight or more rows as one GEMM.
  * y/Y: f32 (qgemv) or f32/bf16 (qgemm), row-major [m, n].
  * qgemm keeps scratch memory (converted activations, partial tiles) inside the library, one

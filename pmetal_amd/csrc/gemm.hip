@@ -1890,7 +1890,7 @@ struct SmallRun16 {  // what a lane holds of a row tile
     u32x4 sc[NSB];         // Q3_K: scales and d; Q2_K: x, y = scale bytes 8 h .., z = d | dmin << 16
 };
 
-template <int FMT, int NSB>
+template <int FMT, int NSB, int MT = 1>
 __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small16(const uint8_t *__restrict__ W, const uint4 *__restrict__ xs,
                                                                      const float *__restrict__ rowscale, void *__restrict__ yg, int M,
                                                                      int Mp, int N, int spr, int tiles, int tiles_per_wg, int ybf16,
@@ -1905,7 +1905,7 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small16(const uint8_
     const uint32_t h = (uint32_t)(kg >> 1), g = (uint32_t)(kg & 1);
     const int rounds = (tiles_per_wg + kSmallDepth - 1) / kSmallDepth;
     float4_t *out_tiles = dyn;
-    float4_t *keep = tiles_per_wg <= kSmallKeepTiles ? dyn + rounds * kSmallDepth * 64 : nullptr;
+    float4_t *keep = tiles_per_wg * MT <= kSmallKeepTiles ? dyn + rounds * kSmallDepth * MT * 64 : nullptr;
     int sbi[NSB];
     bool sbv[NSB];  // wave-uniform
 #pragma unroll
@@ -1914,21 +1914,23 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small16(const uint8_
         sbv[i] = sbi[i] < spr;
         sbi[i] = sbv[i] ? sbi[i] : 0;
     }
-    half8_t af[NSB][8], asum[NSB][2];
+    half8_t af[NSB][MT][8], asum[NSB][MT][2];  // (MT 16-row blocks of activations: rows nl, 16 + nl)
 #pragma unroll
-    for (int i = 0; i < NSB; i++) {
-        const uint4 *base = xs + (size_t)((2 * sbi[i] + (int)h) * kGroups16) * Mp + nl;
+    for (int i = 0; i < NSB; i++)
 #pragma unroll
-        for (int t = 0; t < 8; t++) af[i][t] = __builtin_bit_cast(half8_t, base[(size_t)(2 * t + (int)g) * Mp]);
-        asum[i][0] = __builtin_bit_cast(half8_t, base[(size_t)(16 + (int)g) * Mp]);
-        asum[i][1] = __builtin_bit_cast(half8_t, base[(size_t)(18 + (int)g) * Mp]);
-        if (!sbv[i]) {  // a super-block past the end of the row multiplies zeros (no branch in the streaming loop)
-            const half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (int mb = 0; mb < MT; mb++) {
+            const uint4 *base = xs + (size_t)((2 * sbi[i] + (int)h) * kGroups16) * Mp + 16 * mb + nl;
 #pragma unroll
-            for (int t = 0; t < 8; t++) af[i][t] = z;
-            asum[i][0] = z, asum[i][1] = z;
+            for (int t = 0; t < 8; t++) af[i][mb][t] = __builtin_bit_cast(half8_t, base[(size_t)(2 * t + (int)g) * Mp]);
+            asum[i][mb][0] = __builtin_bit_cast(half8_t, base[(size_t)(16 + (int)g) * Mp]);
+            asum[i][mb][1] = __builtin_bit_cast(half8_t, base[(size_t)(18 + (int)g) * Mp]);
+            if (!sbv[i]) {  // a super-block past the end of the row multiplies zeros (no branch in the streaming loop)
+                const half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+                for (int t = 0; t < 8; t++) af[i][mb][t] = z;
+                asum[i][mb][0] = z, asum[i][mb][1] = z;
+            }
         }
-    }
     const int t0 = (int)blockIdx.x * tiles_per_wg;
     const int t1 = t0 + tiles_per_wg < tiles ? t0 + tiles_per_wg : tiles;  // t1 > t0 by the launch geometry
     const uint32_t row_bytes = (uint32_t)spr * (uint32_t)B::kBytes;
@@ -1959,7 +1961,9 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small16(const uint8_
         }
     };
     auto consume = [&](int ti, const SmallRun16<FMT, NSB> &w) __attribute__((always_inline)) {
-        float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        float4_t acc[MT];
+#pragma unroll
+        for (int mb = 0; mb < MT; mb++) acc[mb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int i = 0; i < NSB; i++) {
             uint32_t qd[4], hm[4] = {0, 0, 0, 0}, s8[3], dbits;
@@ -2001,7 +2005,9 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small16(const uint8_
                     const _Float16 s16 = (_Float16)scf, o16 = (_Float16)(-1024.0f * scf);  // exact: |sc| <= 32
                     sc2[2 * sp + lh] = half2_t{s16, s16}, off2[2 * sp + lh] = half2_t{o16, o16};
                 }
-            float4_t part = {0.0f, 0.0f, 0.0f, 0.0f};
+            float4_t part[MT];
+#pragma unroll
+            for (int mb = 0; mb < MT; mb++) part[mb] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int t = 0; t < 8; t++) {
                 const int dw = t >> 1, sp = t & 1;
@@ -2015,19 +2021,24 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small16(const uint8_
                 const half2_t r2 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, hi, 0x04010400u)), sc2[2 * sp + 1], off2[2 * sp + 1]);
                 const half2_t r3 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, hi, 0x04030402u)), sc2[2 * sp + 1], off2[2 * sp + 1]);
                 const half8_t b = half8_t{r0[0], r0[1], r1[0], r1[1], r2[0], r2[1], r3[0], r3[1]};
-                part = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i][t], b, part, 0, 0, 0);
+#pragma unroll
+                for (int mb = 0; mb < MT; mb++) part[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i][mb][t], b, part[mb], 0, 0, 0);
             }
 #pragma unroll
             for (int sp = 0; sp < 2; sp++) {
                 const _Float16 h0 = (_Float16)nm[2 * sp], h1 = (_Float16)nm[2 * sp + 1];
                 const _Float16 l0 = (_Float16)(nm[2 * sp] - (float)h0), l1 = (_Float16)(nm[2 * sp + 1] - (float)h1);
                 const half8_t br = half8_t{h0, h0, l0, l0, h1, h1, l1, l1};
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(asum[i][sp], br, acc, 0, 0, 0);
+#pragma unroll
+                for (int mb = 0; mb < MT; mb++) acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(asum[i][mb][sp], br, acc[mb], 0, 0, 0);
             }
 #pragma unroll
-            for (int r = 0; r < 4; r++) acc[r] = __builtin_fmaf(d, part[r], acc[r]);
+            for (int mb = 0; mb < MT; mb++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) acc[mb][r] = __builtin_fmaf(d, part[mb][r], acc[mb][r]);
         }
-        small_add_waves(red, keep, ti, wave, nwaves, lane, acc, out_tiles);
+#pragma unroll
+        for (int mb = 0; mb < MT; mb++) small_add_waves(red, keep, ti * MT + mb, wave, nwaves, lane, acc[mb], out_tiles);
     };
     static_assert(kSmallDepth == 2, "the ring is written out as two tiles");
     SmallRun16<FMT, NSB> ring0, ring1;
@@ -2039,8 +2050,8 @@ __global__ __launch_bounds__(64 * kSmallWaves) void k_qgemm_small16(const uint8_
         consume(2 * rd + 1, ring1);
         issue(2 * rd + 3, ring1);
     }
-    small_add_kept(keep, rounds * kSmallDepth, wave, nwaves, lane, out_tiles);
-    small_store(out_tiles, t0, t1, M, Mp, N, rowscale, yg, ybf16, partial);
+    small_add_kept(keep, rounds * kSmallDepth * MT, wave, nwaves, lane, out_tiles);
+    small_store(out_tiles, t0, t1, M, Mp, N, rowscale, yg, ybf16, partial, MT);
 }
 
 }  // namespace
@@ -2054,13 +2065,13 @@ static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 constexpr int kSmallMaxRuns = 8;  // k <= 32768
 // Super-blocks of a row that one short-batch workgroup takes (a longer row goes in runs of that many); 0: no such kernel.
 // Up to 16 rows: eight waves of two super-blocks.  17 to 32 rows (two 16-row blocks of activations per weight operand): the
-// Q4_K / Q5_K kernel still holds two super-blocks' activations per wave, the Q8_0 kernel one (43.4 -> 27.1 us at 14336 x 4096);
+// Q4_K / Q5_K and Q2_K kernels still hold two super-blocks' activations per wave, the Q8_0 kernel one (43.4 -> 27.1 us at 14336 x 4096);
 // the Q6_K kernel in that form, with its rows in runs of eight, is no faster than the large kernel (32.2 against 29.9 us).
 static int small_run_spr(uint32_t type, int64_t m) {
     const bool any = type == kTypeQ4K || type == kTypeQ5K || type == kTypeQ6K || type == kTypeQ8_0 || type == kTypeQ3K || type == kTypeQ2K;
     if (m <= kSmallMaxM) return any ? kSmallMaxSpr : 0;
     if (m > kSmallMaxM2) return 0;
-    if (type == kTypeQ4K || type == kTypeQ5K) return kSmallMaxSpr;
+    if (type == kTypeQ4K || type == kTypeQ5K || type == kTypeQ2K) return kSmallMaxSpr;
     if (type == kTypeQ8_0) return kSmallWaves;
     return 0;
 }
@@ -2285,22 +2296,24 @@ hipError_t launch_qgemm(uint32_t type, const uint8_t *w, int64_t n, int64_t k, c
         else PMH_SMALL_F(O, S, 0);    \
     } while (0)
         if (q23) {
-#define PMH_SMALL16(F, S)                                                                                                        \
+#define PMH_SMALL16(F, S, T)                                                                                                     \
     do {                                                                                                                         \
         if (lds > 48 * 1024) {                                                                                                   \
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_qgemm_small16<F, S>), hipFuncAttributeMaxDynamicSharedMemorySize, \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_qgemm_small16<F, S, T>), hipFuncAttributeMaxDynamicSharedMemorySize, \
                                     (int)lds);                                                                                   \
             if (e != hipSuccess) return e;                                                                                       \
         }                                                                                                                        \
-        hipLaunchKernelGGL((k_qgemm_small16<F, S>), grid, block, lds, s, w, xs, rowscale, y, (int)m, (int)p.mp, (int)n, spr, tiles, \
+        hipLaunchKernelGGL((k_qgemm_small16<F, S, T>), grid, block, lds, s, w, xs, rowscale, y, (int)m, (int)p.mp, (int)n, spr, tiles, \
                            tiles_per_wg, ybf ? 1 : 0, part_out);                                                                 \
     } while (0)
             if (type == kTypeQ2K) {
-                if (nsb == 2) PMH_SMALL16(3, 2);
-                else PMH_SMALL16(3, 1);
+                if (mt == 2 && nsb == 2) PMH_SMALL16(3, 2, 2);
+                else if (mt == 2) PMH_SMALL16(3, 1, 2);
+                else if (nsb == 2) PMH_SMALL16(3, 2, 1);
+                else PMH_SMALL16(3, 1, 1);
             } else {
-                if (nsb == 2) PMH_SMALL16(2, 2);
-                else PMH_SMALL16(2, 1);
+                if (nsb == 2) PMH_SMALL16(2, 2, 1);
+                else PMH_SMALL16(2, 1, 1);
             }
 #undef PMH_SMALL16
         } else if (q6) {

@@ -517,7 +517,7 @@ def test_qgemm_batch_wide_and_narrow_weights_share_x(oracle, t, m):
                                  # wave with work owns one super-block where the others own two, a second run holds four
                                  (333, 2816), (1001, 256), (250, 768), (123, 5120), (47, 3328)])
 def test_qgemm_short_batches(oracle, t, m, n, k):
-    """At most 16 activation rows (Q4_K, Q5_K and Q8_0: at most 32, two 16-row blocks per weight operand): the fused kernels that read the weights once (rows of any number of super-blocks, in runs of 16).  Random block bytes (every scale, min and quant pattern), row counts that are no multiple of the 16-row
+    """At most 16 activation rows (Q4_K, Q5_K, Q8_0 and Q2_K: at most 32, two 16-row blocks per weight operand): the fused kernels that read the weights once (rows of any number of super-blocks, in runs of 16).  Random block bytes (every scale, min and quant pattern), row counts that are no multiple of the 16-row
     tiles, one full tile, more tiles than workgroups take in one round; bf16 and f32 activations, f32 and bf16 outputs;
     unit activations that pick single weights out of the matrix."""
     rng = np.random.default_rng(1000 * t + 31 * m + n + k)
