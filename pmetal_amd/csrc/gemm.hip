@@ -2134,10 +2134,10 @@ GemmPlan qgemm_plan(int64_t m, int64_t n, int64_t k, uint32_t type) {
                          (splits > 1 ? (double)splits * (double)m * (double)n * 8.0 / 4.0e12 + 3.0e-6 : 0.0);
         if (want == 1 || t < best) best = t, p.splits = (int)splits, p.chunk = (int)chunk;
     }
-    // short batches against long rows: runs of 16 (or 8) super-blocks (the fused kernels' K split; the large kernel takes the
-    // same split when a shape falls back to it)
+    // short batches against long rows: runs of 16 (or 8) super-blocks, the fused kernels' K split (a shape they do not take
+    // keeps the split chosen above)
     const int run = small_run_spr(type, m);
-    if (run && spr > run) p.chunk = run, p.splits = (int)((spr + run - 1) / run);
+    if (run && spr > run && qgemm_small_applies(type, m, n, k)) p.chunk = run, p.splits = (int)((spr + run - 1) / run);
     return p;
 }
 
