@@ -515,7 +515,10 @@ def test_qgemm_batch_wide_and_narrow_weights_share_x(oracle, t, m):
                                  (500, 14336), (130, 6144), (77, 11008), (64, 32768),
                                  # rows of 11, 1, 3, 20 and 13 super-blocks: Q6_K rows then start at any even address, the last
                                  # wave with work owns one super-block where the others own two, a second run holds four
-                                 (333, 2816), (1001, 256), (250, 768), (123, 5120), (47, 3328)])
+                                 (333, 2816), (1001, 256), (250, 768), (123, 5120), (47, 3328),
+                                 # rows of 72 and 136 super-blocks: more runs than the fused kernels take (Q8_0 with two blocks of
+                                 # activations: eight runs of 8; the others: eight runs of 16), so the large kernel with its own K split
+                                 (40, 18432), (24, 34816)])
 def test_qgemm_short_batches(oracle, t, m, n, k):
     """At most 16 activation rows (Q4_K, Q5_K, Q8_0 and Q2_K: at most 32, two 16-row blocks per weight operand): the fused kernels that read the weights once (rows of any number of super-blocks, in runs of 16).  Random block bytes (every scale, min and quant pattern), row counts that are no multiple of the 16-row
     tiles, one full tile, more tiles than workgroups take in one round; bf16 and f32 activations, f32 and bf16 outputs;
